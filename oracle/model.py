@@ -1,0 +1,237 @@
+"""Float64 NumPy model of the reference's semantics (TEST INFRASTRUCTURE ONLY).
+
+Restates *what* the reference computes (not its kernels): MLX affine dequantisation,
+dequantize-then-matmul, top-k routing, stable expert grouping, SwiGLU expert FFN and the
+weighted combine.  File:line citations are relative to the reference checkout.
+"""
+import numpy as np
+
+# --------------------------------------------------------------------------------------
+# Packing (bit-exact)
+# --------------------------------------------------------------------------------------
+
+
+def pack_u32(q, bits):
+    """Value i of a row sits in word i // (32/bits) at bit offset bits * (i % (32/bits)).
+
+    Follows `word |= q << (k * bits)` (crates/rmlx-nn/src/attention.rs:4853-4862) and
+    `extract_bits` (crates/rmlx-core/src/ops/quantized.rs:206-208).
+    Pinned by: 0x76543210 / 0x04030201 known answers (safetensors_loader.rs:838-866), the
+    0x11111111 rows (quantized.rs:12069-12095) and exhaustive per-slot round trips in tests/.
+    """
+    q = np.asarray(q, dtype=np.uint32)
+    per = 32 // bits
+    assert q.shape[-1] % per == 0
+    qq = q.reshape(q.shape[:-1] + (q.shape[-1] // per, per))
+    shifts = (np.arange(per, dtype=np.uint32) * np.uint32(bits))
+    return np.bitwise_or.reduce(qq << shifts, axis=-1).astype(np.uint32)
+
+
+def unpack_u32(words, bits):
+    """Inverse of `pack_u32`: returns uint8 values, last axis expanded by 32/bits."""
+    words = np.asarray(words, dtype=np.uint32)
+    per = 32 // bits
+    shifts = (np.arange(per, dtype=np.uint32) * np.uint32(bits))
+    vals = (words[..., None] >> shifts) & np.uint32((1 << bits) - 1)
+    return vals.reshape(words.shape[:-1] + (words.shape[-1] * per,)).astype(np.uint8)
+
+
+def words_to_bytes(words):
+    """Byte image the reference's CPU path consumes: for Q4 low nibble = even k, for Q8 one
+    byte per value; equal to the little-endian bytes of the u32 words
+    (crates/rmlx-nn/src/safetensors_loader.rs:562-628)."""
+    w = np.ascontiguousarray(words, dtype="<u4")
+    return w.view(np.uint8).reshape(w.shape[:-1] + (w.shape[-1] * 4,))
+
+
+def bytes_to_words(b):
+    b = np.ascontiguousarray(b, dtype=np.uint8)
+    return b.view("<u4").reshape(b.shape[:-1] + (b.shape[-1] // 4,))
+
+
+# --------------------------------------------------------------------------------------
+# bf16 helpers (NumPy has no bfloat16)
+# --------------------------------------------------------------------------------------
+
+
+def f32_to_bf16_bits(x):
+    """Round-to-nearest-even f32 -> bf16 bit pattern (uint16)."""
+    u = np.ascontiguousarray(x, dtype=np.float32).view(np.uint32)
+    rounded = u + np.uint32(0x7FFF) + ((u >> np.uint32(16)) & np.uint32(1))
+    return (rounded >> np.uint32(16)).astype(np.uint16)
+
+
+def bf16_bits_to_f32(b):
+    return (np.asarray(b, dtype=np.uint16).astype(np.uint32) << np.uint32(16)).view(np.float32)
+
+
+# --------------------------------------------------------------------------------------
+# Dequantize-then-matmul (tolerance oracle)
+# --------------------------------------------------------------------------------------
+
+
+def dequantize(words, scales, biases, group_size, bits):
+    """w[n,k] = scale[n,k//gs] * q[n,k] + bias[n,k//gs], evaluated exactly in float64.
+
+    Semantics of `dequantize_q4_row` (crates/rmlx-core/src/ops/quantized.rs:2602-2622) and of
+    the QuantizedWeight doc (`w_i = scale_g * q_i + bias_g`, :69-77).  Pinned by the
+    [3,5,10,1] -> [6.5,10.5,20.5,2.5] known answer (:10601-10624) and by agreement with the C
+    restatement of `dequantize_q4_row`.
+    """
+    q = unpack_u32(words, bits).astype(np.float64)
+    s = np.repeat(np.asarray(scales, dtype=np.float64), group_size, axis=-1)
+    b = np.repeat(np.asarray(biases, dtype=np.float64), group_size, axis=-1)
+    return s * q + b
+
+
+def qmm(x, words, scales, biases, group_size, bits):
+    """out[m,n] = sum_k x[m,k] * dequant(W)[n,k] in float64 (the reference's
+    `naive_matmul_with_dequant`, quantized.rs:10681-10719, with exact arithmetic).
+    Pinned by: equal-nibble closed forms 224/96/192/448/512 (:10922, :11575, :11784, :12088),
+    agreement with the C restatement of `affine_qmm` (1e-4 relative, the bar the reference
+    itself uses at :10794-10808)."""
+    w = dequantize(words, scales, biases, group_size, bits)
+    return np.asarray(x, dtype=np.float64) @ w.T
+
+
+def gather_qmm(x, words, scales, biases, indices, group_size, bits=4):
+    """out[b] = x[b] @ dequant(W[indices[b]])^T for stacked expert weights [E,N,K*bits/32]
+    (crates/rmlx-core/src/ops/quantized.rs:9279-9290, 9300-9368).  x is [batch, M_b, K] or
+    [batch, K]."""
+    x = np.asarray(x, dtype=np.float64)
+    outs = []
+    for b, e in enumerate(np.asarray(indices)):
+        outs.append(qmm(np.atleast_2d(x[b]), words[e], scales[e], biases[e], group_size, bits))
+    out = np.stack(outs) if outs else np.zeros((0, 1, words.shape[1]))
+    return out if x.ndim == 3 else out[:, 0, :]
+
+
+def tolerance(ref):
+    """The acceptance bar: max|err| <= 1e-2 * RMS(reference output)."""
+    ref = np.asarray(ref, dtype=np.float64)
+    return 1e-2 * float(np.sqrt(np.mean(ref * ref)))
+
+
+# --------------------------------------------------------------------------------------
+# Routing
+# --------------------------------------------------------------------------------------
+
+
+def topk_route(logits, top_k, bias=None, renormalize=True, rank_by="logit"):
+    """softmax over E -> top-k by repeated argmax (strict >, ties -> lowest index) ->
+    weights / sum(top-k) -> histogram -> exclusive scan.
+
+    Restates `moe_topk_route_f32` + `moe_prefix_scan_u32`
+    (crates/rmlx-core/src/ops/topk_route.rs:212-388).  Softmax is evaluated in f32 like the
+    kernel (max-subtracted, multiplied by 1/sum).  `rank_by="softmax"` ranks the f32 softmax
+    values as the kernel does; `rank_by="logit"` ranks the (biased) logits, which is the same
+    order unless two distinct logits collapse to one float after exp.
+    Pinned by the reference's behavioural tests (:674-751, :764-783, :815-840) and by a
+    brute-force stable argsort in tests/.
+    Returns (indices u32 [T*K], weights f32 [T*K], counts u32 [E], offsets u32 [E+1]).
+    """
+    lg = np.asarray(logits, dtype=np.float32)
+    T, E = lg.shape
+    if bias is not None:
+        lg = (lg + np.asarray(bias, dtype=np.float32)[None, :]).astype(np.float32)
+    idx = np.zeros((T, top_k), np.uint32)
+    wts = np.zeros((T, top_k), np.float32)
+    for t in range(T):
+        row = lg[t]
+        mx = np.float32(row.max()) if E else np.float32(0)
+        ex = np.exp((row - mx).astype(np.float32)).astype(np.float32)
+        inv = np.float32(1.0) / np.float32(ex.sum(dtype=np.float32))
+        sm = (ex * inv).astype(np.float32)
+        key = sm if rank_by == "softmax" else row
+        taken = np.zeros(E, bool)
+        for k in range(top_k):
+            best, best_i = None, 0
+            for i in range(E):
+                if taken[i]:
+                    continue
+                if best is None or key[i] > best:
+                    best, best_i = key[i], i
+            taken[best_i] = True
+            idx[t, k] = best_i
+            wts[t, k] = sm[best_i]
+        if renormalize:
+            ssum = np.float32(0)
+            for k in range(top_k):
+                ssum = np.float32(ssum + wts[t, k])
+            invw = np.float32(1.0) / ssum if ssum > 0 else np.float32(0)
+            wts[t] = (wts[t] * invw).astype(np.float32)
+    counts = np.bincount(idx.reshape(-1), minlength=E).astype(np.uint32)
+    offsets = np.concatenate([[0], np.cumsum(counts)]).astype(np.uint32)
+    return idx.reshape(-1), wts.reshape(-1), counts, offsets
+
+
+def expert_dispatch(indices, weights, seq_len, top_k, num_experts):
+    """`expert_dispatch[e] = [(tok, w), ...]` in (tok, k) order
+    (crates/rmlx-nn/src/moe.rs:1439-1447), as plain loops."""
+    disp = [[] for _ in range(num_experts)]
+    for tok in range(seq_len):
+        for k in range(top_k):
+            flat = tok * top_k + k
+            disp[int(indices[flat])].append((tok, float(weights[flat])))
+    return disp
+
+
+def moe_sort(indices, num_experts):
+    """Stable sort of flat assignment ids (tok*K+k) by expert id.  Returns
+    (sorted_assign u32 [A], offsets u32 [E+1]); segment e of sorted_assign lists the flat
+    ids routed to expert e in ascending order -- the same order `expert_dispatch` produces."""
+    indices = np.asarray(indices, dtype=np.uint32)
+    order = np.argsort(indices, kind="stable").astype(np.uint32)
+    counts = np.bincount(indices, minlength=num_experts).astype(np.uint32)
+    offsets = np.concatenate([[0], np.cumsum(counts)]).astype(np.uint32)
+    return order, offsets
+
+
+# --------------------------------------------------------------------------------------
+# Expert FFN + combine
+# --------------------------------------------------------------------------------------
+
+
+def silu(x):
+    x = np.asarray(x, dtype=np.float64)
+    return x / (1.0 + np.exp(-x))
+
+
+def moe_forward(x, indices, weights, gate, up, down, group_size, top_k, round_h=np.float16):
+    """out[t] = sum_k w[t,k] * down_e( silu(gate_e x_t) * up_e x_t ), e = indices[t,k].
+
+    Composition of `ExpertGroup::grouped_forward` (crates/rmlx-nn/src/expert_group.rs:445-524:
+    gate GEMM, up GEMM, silu_gate, down GEMM) and the weighted scatter-add
+    (crates/rmlx-nn/src/moe.rs:1851-1932; `scatter_weighted_add`,
+    crates/rmlx-core/src/ops/moe_kernels.rs:306-363), with expert weights in the stacked Q4
+    layout of `gather_qmv_fast_f16_q4` (quantized.rs:9605-9620).  The hidden activation is
+    rounded to `round_h` (the reference stores it in the input dtype, expert_group.rs:380-383);
+    everything else is float64.  `gate`, `up`, `down` are (words, scales, biases) triples with a
+    leading expert axis.  Pinned by the scatter known answer (moe_kernels.rs:420-450) and by
+    equality with a per-expert loop on small shapes in tests/.
+    """
+    x = np.asarray(x, dtype=np.float64)
+    T, D = x.shape
+    out = np.zeros((T, D), np.float64)
+    idx = np.asarray(indices).reshape(T, top_k)
+    wts = np.asarray(weights, dtype=np.float64).reshape(T, top_k)
+    cache = {}
+
+    def deq(trip, e):
+        key = (id(trip[0]), int(e))
+        if key not in cache:
+            cache[key] = dequantize(trip[0][e], trip[1][e], trip[2][e], group_size, 4)
+        return cache[key]
+
+    for e in np.unique(idx):
+        toks, ks = np.nonzero(idx == e)
+        xe = x[toks]
+        g = xe @ deq(gate, e).T
+        u = xe @ deq(up, e).T
+        h = silu(g) * u
+        if round_h is not None:
+            h = h.astype(round_h).astype(np.float64)
+        y = h @ deq(down, e).T
+        np.add.at(out, toks, wts[toks, ks][:, None] * y)
+        cache.clear()
+    return out
