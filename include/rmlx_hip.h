@@ -1,0 +1,225 @@
+/*
+ * rmlx_hip.h -- C ABI of the MI355X (gfx950) quantized-matmul engine.
+ *
+ * Drop-in boundary for the quantized-matmul hot path of RMLX (`rmlx_core::ops::quantized`,
+ * `ops::topk_route`, `ops::moe_kernels`, and the `rmlx-nn` callers `QuantizedLinear`,
+ * `ExpertGroup::grouped_forward`, `MoeLayer::forward_grouped`).  A Rust `extern "C"` crate
+ * binds exactly these symbols in place of the rmlx-metal dispatch for this path; every entry
+ * point names the reference interface it replaces (paths relative to the reference checkout).
+ *
+ * Conventions (they mirror the reference's):
+ *   - every pointer named `*_dev`, every `rmlx_array::data` and every weight buffer is a DEVICE
+ *     pointer owned by the caller; no function takes ownership of caller memory;
+ *   - outputs are caller-allocated (the caller plays the role of `Array::uninit`,
+ *     crates/rmlx-core/src/array.rs:238); every output of a matmul is f16, row-major;
+ *   - functions return 0 on success, RMLX_INVALID_SHAPE / RMLX_NOT_FOUND (the two
+ *     `KernelError` variants used on this path, crates/rmlx-core/src/kernels/mod.rs:29-42) or
+ *     RMLX_RUNTIME_ERROR for a failing HIP call; the message is kept per thread and read
+ *     with rmlx_hip_last_error();
+ *   - `stream == NULL` means synchronous: the call returns after the GPU has finished
+ *     (`ExecMode::Sync`, crates/rmlx-core/src/ops/mod.rs:182-206).  With a stream the work is
+ *     only enqueued (the `_into_cb` twins, crates/rmlx-core/src/ops/quantized.rs:7797-7802)
+ *     and the caller synchronises;
+ *   - all sizes are checked to fit in u32 (`checked_u32`, crates/rmlx-core/src/ops/mod.rs:71-74).
+ */
+#ifndef RMLX_HIP_H
+#define RMLX_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ---- status / dtype ------------------------------------------------------------------ */
+
+enum {
+  RMLX_OK = 0,
+  RMLX_INVALID_SHAPE = 1, /* KernelError::InvalidShape */
+  RMLX_NOT_FOUND = 2,     /* KernelError::NotFound     */
+  RMLX_RUNTIME_ERROR = 3  /* a HIP runtime call failed */
+};
+
+/* Subset of `DType` (crates/rmlx-core/src/dtype.rs:34-52) that appears on this path. */
+enum {
+  RMLX_DTYPE_F32 = 0,
+  RMLX_DTYPE_F16 = 1,
+  RMLX_DTYPE_BF16 = 2,
+  RMLX_DTYPE_U32 = 3,
+  RMLX_DTYPE_U8 = 4
+};
+
+/* View of an `Array` (crates/rmlx-core/src/array.rs:137-144): `data` already includes the
+ * array's byte offset; the array must be row-contiguous. */
+typedef struct rmlx_array {
+  void* data;
+  int32_t dtype;
+  int32_t ndim;
+  size_t shape[4];
+} rmlx_array;
+
+typedef void* rmlx_stream;            /* a hipStream_t */
+typedef void* rmlx_event;             /* a hipEvent_t  */
+typedef struct rmlx_qweight rmlx_qweight; /* `QuantizedWeight`, opaque */
+
+/* Message of the last failing call on this thread ("" if none). */
+const char* rmlx_hip_last_error(void);
+
+/* ---- runtime shim (replaces the rmlx-metal device/queue/buffer calls this path makes) ---- */
+
+/* Select `device`, verify it is a gfx950 part and load the kernels.  Fails loudly (no CPU
+ * fallback exists in this library). */
+int32_t rmlx_hip_init(int32_t device);
+/* Fills: [0] compute units, [1] wavefront size, [2] LDS bytes per workgroup, [3] total
+ * global memory in MiB, [4] max engine clock kHz, [5] memory clock kHz, [6] bus width bits,
+ * [7] L2 bytes. */
+int32_t rmlx_hip_device_info(int64_t out[8]);
+int32_t rmlx_hip_malloc(void** dev_ptr, size_t bytes);
+int32_t rmlx_hip_free(void* dev_ptr);
+int32_t rmlx_hip_memset(void* dev_ptr, int32_t value, size_t bytes, rmlx_stream stream);
+int32_t rmlx_hip_memcpy_h2d(void* dst_dev, const void* src_host, size_t bytes, rmlx_stream stream);
+int32_t rmlx_hip_memcpy_d2h(void* dst_host, const void* src_dev, size_t bytes, rmlx_stream stream);
+int32_t rmlx_hip_memcpy_d2d(void* dst_dev, const void* src_dev, size_t bytes, rmlx_stream stream);
+int32_t rmlx_hip_stream_create(rmlx_stream* out);
+int32_t rmlx_hip_stream_sync(rmlx_stream stream);
+int32_t rmlx_hip_stream_destroy(rmlx_stream stream);
+int32_t rmlx_hip_event_create(rmlx_event* out);
+int32_t rmlx_hip_event_record(rmlx_event ev, rmlx_stream stream);
+int32_t rmlx_hip_event_sync(rmlx_event ev);
+int32_t rmlx_hip_event_elapsed_ms(rmlx_event start, rmlx_event stop, float* ms);
+int32_t rmlx_hip_event_destroy(rmlx_event ev);
+
+/* ---- QuantizedWeight ------------------------------------------------------------------
+ * `QuantizedWeight::new` (crates/rmlx-core/src/ops/quantized.rs:97-160).  MLX affine layout:
+ * weights u32 [out_features, in_features*bits/32] (value i of a row in word i/(32/bits) at
+ * bit bits*(i%(32/bits))), scales and biases f16 [out_features, in_features/group_size],
+ * w = scale*q + bias.  Same validation and messages: bits in {2,3,4,6,8}, group_size in
+ * {32,64,128}, in_features % group_size == 0, the three byte lengths large enough.
+ * `n_experts` > 1 declares the stacked layout [n_experts, out_features, ...] that
+ * `gather_qmm` / `gather_qmv_fast_f16_q4` consume (quantized.rs:9279-9290, 9605-9620);
+ * pass 1 for a plain linear weight. */
+int32_t rmlx_hip_qweight_create(const void* weights_dev, size_t weights_bytes,
+                                const void* scales_dev, size_t scales_bytes,
+                                const void* biases_dev, size_t biases_bytes,
+                                uint32_t group_size, uint32_t bits,
+                                size_t out_features, size_t in_features, size_t n_experts,
+                                rmlx_qweight** out);
+int32_t rmlx_hip_qweight_destroy(rmlx_qweight* qw);
+
+/* ---- qmv: `affine_quantized_matmul` (quantized.rs:1309-1411) ----------------------------
+ * vec: 1-D (or any shape) with numel == in_features, f16 / f32 (bf16 also accepted and used
+ * natively); out: f16 [out_features].  Q4 and Q8. */
+int32_t rmlx_hip_affine_quantized_matmul(const rmlx_qweight* qw, const rmlx_array* vec,
+                                         void* out_f16_dev, size_t out_bytes, rmlx_stream stream);
+
+/* ---- qmm: `affine_quantized_matmul_batched` (quantized.rs:7149-7782) -----------------------
+ * x: 2-D [M, in_features], f16 / f32 / bf16; out: f16 [M, out_features].  Chooses the kernel
+ * by M (the reference's dispatch ladder, re-tuned for this chip): streaming MFMA GEMV for
+ * small M, LDS-staged dequant + MFMA GEMM above. */
+int32_t rmlx_hip_affine_quantized_matmul_batched(const rmlx_qweight* qw, const rmlx_array* x,
+                                                 void* out_f16_dev, size_t out_bytes,
+                                                 rmlx_stream stream);
+
+/* Same contract as the batched entry point but forces one kernel family (the reference
+ * exposes its kernels individually too, e.g. `affine_qmv_batched_f16_q4` quantized.rs:1675,
+ * `affine_quantized_matmul_nax` :8517).  kernel: 0 = auto, 1 = streaming GEMV (qmv),
+ * 2 = MFMA GEMM (qmm), 3 = portable scalar kernel (any bits/group size the type admits). */
+int32_t rmlx_hip_qmm_select(const rmlx_qweight* qw, const rmlx_array* x, int32_t kernel,
+                            void* out_f16_dev, size_t out_bytes, rmlx_stream stream);
+
+/* ---- `QuantizedLinear::forward` / `Linear::forward` call shape ------------------------------
+ * (crates/rmlx-nn/src/quantized_linear.rs:153-201, crates/rmlx-nn/src/linear.rs:98-191)
+ * x 1-D [in] is treated as [1,in]; 2-D [batch,in] -> [batch,out]; other ranks are rejected;
+ * batch == 1 takes the qmv path.  `bias_f16_dev` (nullable, [out]) is the broadcast bias
+ * `Linear` adds. */
+int32_t rmlx_hip_quantized_linear_forward(const rmlx_qweight* qw, const rmlx_array* x,
+                                          const void* bias_f16_dev, void* out_f16_dev,
+                                          size_t out_bytes, rmlx_stream stream);
+
+/* ---- gather_qmm (quantized.rs:9404-9599) and gather_qmv_fast_f16_q4 (:10061-10236) ---------
+ * out[b] = x[b] @ dequant(W[indices[b]])^T.  x: [batch, m_per_batch, k] f16 or f32;
+ * w/s/b: stacked [n_experts, n, ...] buffers with their byte lengths; indices: u32 [batch];
+ * out: f16 [batch, m_per_batch, n].  Validation as the reference (non-zero dims, even k,
+ * k % group_size, buffer lengths, indices dtype/length, every index < n_experts; batch == 0
+ * returns an empty result).  The index range check reads the indices back and therefore
+ * only runs when stream == NULL; with a stream, rows whose index is out of range are
+ * written as zeros. */
+int32_t rmlx_hip_gather_qmm(const rmlx_array* x, const void* w_packed_dev, size_t w_bytes,
+                            const void* scales_dev, size_t scales_bytes,
+                            const void* biases_dev, size_t biases_bytes,
+                            const rmlx_array* indices, size_t batch, size_t m_per_batch,
+                            size_t n, size_t k, size_t n_experts, uint32_t group_size,
+                            void* out_f16_dev, size_t out_bytes, rmlx_stream stream);
+
+/* ---- gpu_topk_route (crates/rmlx-core/src/ops/topk_route.rs:433-650) -----------------------
+ * gate_logits [T,E] f32 or f16 -> expert_indices u32 [T*K] (descending, ties to the lower
+ * index), expert_weights f32 [T*K] (softmax, renormalised over the K picks unless
+ * renormalize == 0), expert_counts u32 [E], dispatch_offsets u32 [E+1].  1 <= K <= 8,
+ * K <= E <= 256; expert_bias (nullable) is 1-D [E] f32 or f16. */
+int32_t rmlx_hip_topk_route(const rmlx_array* gate_logits, size_t top_k,
+                            const rmlx_array* expert_bias, int32_t renormalize,
+                            uint32_t* expert_indices_dev, float* expert_weights_dev,
+                            uint32_t* expert_counts_dev, uint32_t* dispatch_offsets_dev,
+                            rmlx_stream stream);
+
+/* ---- token -> expert grouping (crates/rmlx-nn/src/moe.rs:1439-1447) --------------------------
+ * On-device replacement of the host-side `expert_dispatch` build: a stable counting sort of
+ * the flat assignment ids (tok*K + k) by expert.  sorted_assign u32 [n_assign]: segment
+ * [offsets[e], offsets[e+1]) lists the ids routed to expert e in ascending order;
+ * offsets u32 [n_experts+1]. */
+int32_t rmlx_hip_moe_sort(const uint32_t* expert_indices_dev, size_t n_assign, size_t n_experts,
+                          uint32_t* sorted_assign_dev, uint32_t* offsets_dev, rmlx_stream stream);
+
+/* ---- index_gather / scatter_weighted_add (crates/rmlx-core/src/ops/moe_kernels.rs:239-363) --
+ * dst[i,:] = src[idx[i],:]            (f16 rows of width d)
+ * dst[tok[i],:] += w[i] * src[i,:]    (f32 accumulation, deterministic: assignments of a
+ *                                      token are added in ascending i) */
+int32_t rmlx_hip_index_gather(const void* src_f16_dev, size_t src_rows, size_t d,
+                              const uint32_t* idx_dev, size_t n, void* dst_f16_dev,
+                              rmlx_stream stream);
+int32_t rmlx_hip_scatter_weighted_add(const void* src_f16_dev, size_t n, size_t d,
+                                      const uint32_t* tok_dev, const float* w_dev,
+                                      void* dst_f16_dev, size_t dst_rows, rmlx_stream stream);
+
+/* ---- silu_gate (crates/rmlx-core/src/ops/silu.rs:142-166) -----------------------------------
+ * out = silu(gate_in) * up_in, f16, sigmoid evaluated in f32. */
+int32_t rmlx_hip_silu_gate(const void* gate_in_f16_dev, const void* up_in_f16_dev,
+                           void* out_f16_dev, size_t numel, rmlx_stream stream);
+
+/* ---- ExpertGroup::grouped_forward (crates/rmlx-nn/src/expert_group.rs:308-533) --------------
+ * Literal contract: `n_items` (expert_idx, input [batch_i, D]) pairs, inputs packed one
+ * after another in x ([sum batch_i, D] f16); out receives the per-item outputs in the same
+ * packing.  Per item: y = (silu(x Wg^T) * (x Wu^T)) Wd^T with Q4 stacked expert weights
+ * gate/up [E, I, D] and down [E, D, I].  `up` may be NULL when `gate` holds the fused
+ * [E, 2I, D] layout (gate rows first).  expert_idx and batch_sizes are HOST arrays.
+ * Validation as the reference: idx < E, n_items == 0 -> nothing to do. */
+int32_t rmlx_hip_expert_group_grouped_forward(const rmlx_qweight* gate, const rmlx_qweight* up,
+                                              const rmlx_qweight* down, size_t n_items,
+                                              const uint32_t* expert_idx_host,
+                                              const uint32_t* batch_sizes_host,
+                                              const rmlx_array* x, void* out_f16_dev,
+                                              size_t out_bytes, rmlx_stream stream);
+
+/* ---- MoeLayer::forward_grouped (crates/rmlx-nn/src/moe.rs:1391-1508) ------------------------
+ * The whole routed-expert block with no host round trip:
+ * route (given) -> on-device sort -> gate/up gather_qmm + SwiGLU -> down gather_qmm ->
+ * f32 weighted combine -> f16 out [T, D].  expert_indices / expert_weights are the [T*K]
+ * outputs of rmlx_hip_topk_route (device). */
+int32_t rmlx_hip_moe_forward_grouped(const rmlx_qweight* gate, const rmlx_qweight* up,
+                                     const rmlx_qweight* down, const rmlx_array* x,
+                                     const uint32_t* expert_indices_dev,
+                                     const float* expert_weights_dev, size_t top_k,
+                                     void* out_f16_dev, size_t out_bytes, rmlx_stream stream);
+
+/* Routing + the block above in one call: gate_logits [T,E] (the router's output). */
+int32_t rmlx_hip_moe_forward(const rmlx_qweight* gate, const rmlx_qweight* up,
+                             const rmlx_qweight* down, const rmlx_array* x,
+                             const rmlx_array* gate_logits, size_t top_k,
+                             const rmlx_array* expert_bias, void* out_f16_dev, size_t out_bytes,
+                             rmlx_stream stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* RMLX_HIP_H */

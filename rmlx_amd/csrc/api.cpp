@@ -1,0 +1,764 @@
+// Host side of the C ABI: validation (same rules and messages as the reference's Rust entry
+// points), the dispatch ladder, and the composition of the MoE block.  No arithmetic happens
+// here and there is no CPU fallback: every path ends in a HIP kernel launch or an error.
+#include <cinttypes>
+#include <cstring>
+#include <vector>
+
+#include "common.hpp"
+
+namespace rmlx {
+
+std::string& last_error() {
+  thread_local std::string e;
+  return e;
+}
+
+int32_t fail(int32_t code, const char* fmt, ...) {
+  char buf[1024];
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(buf, sizeof buf, fmt, ap);
+  va_end(ap);
+  last_error() = buf;
+  return code;
+}
+
+int32_t checked_u32(size_t v, const char* name, uint32_t* out) {
+  if (v > 0xFFFFFFFFull) return fail(RMLX_INVALID_SHAPE, "%s (%zu) exceeds u32::MAX", name, v);
+  *out = (uint32_t)v;
+  return RMLX_OK;
+}
+
+const char* dtype_name(int32_t dt) {
+  switch (dt) {
+    case RMLX_DTYPE_F32: return "Float32";
+    case RMLX_DTYPE_F16: return "Float16";
+    case RMLX_DTYPE_BF16: return "Bfloat16";
+    case RMLX_DTYPE_U32: return "UInt32";
+    case RMLX_DTYPE_U8: return "UInt8";
+    default: return "Unknown";
+  }
+}
+
+DeviceCtx& ctx() {
+  static DeviceCtx c;
+  return c;
+}
+
+int32_t require_init() {
+  if (!ctx().ready) return fail(RMLX_RUNTIME_ERROR, "rmlx_hip_init() has not been called (no GPU context)");
+  return RMLX_OK;
+}
+
+int32_t finish(hipStream_t stream) {
+  if (stream == nullptr) RMLX_HIP_CHECK(hipStreamSynchronize(nullptr));
+  return RMLX_OK;
+}
+
+int32_t Scratch::alloc(size_t bytes, hipStream_t s) {
+  release();
+  stream = s;
+  if (bytes == 0) bytes = 16;
+  RMLX_HIP_CHECK(hipMallocAsync(&ptr, bytes, s));
+  return RMLX_OK;
+}
+
+void Scratch::release() {
+  if (ptr != nullptr) {
+    (void)hipFreeAsync(ptr, stream);
+    ptr = nullptr;
+  }
+}
+
+namespace {
+
+bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+// ---- the dispatch ladder --------------------------------------------------------------------
+// The reference picks by M: QMV for M=1, batched QMV up to a per-chip limit, split-K Steel for
+// 32 <= M < 128 and NAX above (crates/rmlx-core/src/ops/quantized.rs:7200-7256).  Here: the
+// streaming MFMA GEMV (weights read once for up to 8 rows) up to 16 rows, the LDS-staged MFMA
+// GEMM above, the portable kernel for every shape the fast kernels do not take.
+enum { KERNEL_AUTO = 0, KERNEL_QMV = 1, KERNEL_QMM = 2, KERNEL_GENERIC = 3 };
+constexpr uint32_t kQmvMaxM = 16;
+
+int32_t run_matmul(const rmlx_qweight* qw, const void* x, int32_t x_dtype, uint32_t M, __half* out,
+                   int32_t kernel, hipStream_t stream) {
+  uint32_t N, K;
+  RMLX_TRY(checked_u32(qw->out_features, "out_features", &N));
+  RMLX_TRY(checked_u32(qw->in_features, "in_features", &K));
+  if (M == 0) return RMLX_OK;
+  const bool ptr_ok = aligned16(qw->w) && aligned16(qw->s) && aligned16(qw->b) && aligned16(x);
+  const bool can_qmv = qw->bits == 4 && ptr_ok && qmv_q4_supported(N, K, qw->group_size);
+  const bool can_qmm = ptr_ok && qmm_supported(N, K, qw->group_size, qw->bits);
+
+  if (kernel == KERNEL_AUTO) {
+    if (can_qmv && M <= kQmvMaxM) kernel = KERNEL_QMV;
+    else if (can_qmm) kernel = KERNEL_QMM;
+    else if (can_qmv) kernel = KERNEL_QMV;
+    else kernel = KERNEL_GENERIC;
+  } else if (kernel == KERNEL_QMV && !can_qmv) {
+    return fail(RMLX_INVALID_SHAPE,
+                "qmv kernel requires bits=4, group_size=64, N %% 16 == 0, K %% 512 == 0 and 16-byte aligned "
+                "buffers (N=%u K=%u bits=%u group_size=%u)", N, K, qw->bits, qw->group_size);
+  } else if (kernel == KERNEL_QMM && !can_qmm) {
+    return fail(RMLX_INVALID_SHAPE,
+                "qmm kernel requires bits in {4,8}, group_size=64, N %% 64 == 0, K %% 64 == 0 and 16-byte aligned "
+                "buffers (N=%u K=%u bits=%u group_size=%u)", N, K, qw->bits, qw->group_size);
+  } else if (kernel < 0 || kernel > KERNEL_GENERIC) {
+    return fail(RMLX_NOT_FOUND, "unknown kernel selector %d", kernel);
+  }
+
+  // Activations: f16 is native everywhere; bf16 is native only in the Q8 MFMA GEMM.
+  const bool native_bf16 = x_dtype == RMLX_DTYPE_BF16 && kernel == KERNEL_QMM && qw->bits == 8;
+  Scratch cast;
+  const void* xk = x;
+  if (x_dtype != RMLX_DTYPE_F16 && !native_bf16) {
+    RMLX_TRY(cast.alloc((size_t)M * K * sizeof(__half), stream));
+    RMLX_TRY(launch_cast_to_f16(x, x_dtype, static_cast<__half*>(cast.ptr), (size_t)M * K, stream));
+    xk = cast.ptr;
+  }
+
+  if (kernel == KERNEL_QMV) {
+    QmvArgs a{};
+    a.w0 = qw->w; a.s0 = qw->s; a.b0 = qw->b;
+    a.N = N; a.K = K;
+    a.x = static_cast<const __half*>(xk);
+    a.out = out; a.ld_out = N; a.M = M;
+    return launch_qmv_q4(a, stream);
+  }
+  if (kernel == KERNEL_QMM) {
+    QmmArgs a{qw->w, qw->s, qw->b, xk, out, M, N, K, qw->bits, native_bf16 ? 1 : 0};
+    return launch_qmm(a, stream);
+  }
+  GenericArgs g{qw->w, qw->s, qw->b, static_cast<const __half*>(xk), out, nullptr, 0, M, N, K,
+                qw->group_size, qw->bits, 1};
+  return launch_generic(g, stream);
+}
+
+int32_t check_x_dtype(const char* who, int32_t dt) {
+  if (dt != RMLX_DTYPE_F32 && dt != RMLX_DTYPE_F16 && dt != RMLX_DTYPE_BF16)
+    return fail(RMLX_INVALID_SHAPE, "%s requires Float16 or Float32 input, got %s", who, dtype_name(dt));
+  return RMLX_OK;
+}
+
+int32_t check_out(const char* who, size_t have, size_t need) {
+  if (have < need) return fail(RMLX_INVALID_SHAPE, "%s: output buffer too small: %zu bytes < expected %zu bytes", who, have, need);
+  return RMLX_OK;
+}
+
+struct ExpertShapes {
+  uint32_t E, D, I;
+  bool fused;
+};
+
+int32_t check_expert_weights(const char* who, const rmlx_qweight* gate, const rmlx_qweight* up,
+                             const rmlx_qweight* down, ExpertShapes* sh) {
+  if (gate == nullptr || down == nullptr) return fail(RMLX_INVALID_SHAPE, "%s: gate and down weights are required", who);
+  const bool fused = up == nullptr;
+  size_t E = gate->n_experts, D = gate->in_features, I = fused ? gate->out_features / 2 : gate->out_features;
+  if (fused && gate->out_features % 2 != 0) return fail(RMLX_INVALID_SHAPE, "%s: fused gate/up weight needs an even row count", who);
+  if (!fused && (up->n_experts != E || up->in_features != D || up->out_features != I))
+    return fail(RMLX_INVALID_SHAPE, "%s: up weight shape mismatch", who);
+  if (down->n_experts != E || down->in_features != I || down->out_features != D)
+    return fail(RMLX_INVALID_SHAPE, "%s: down weight must be [%zu, %zu, %zu], got [%zu, %zu, %zu]", who, E, D, I,
+                down->n_experts, down->out_features, down->in_features);
+  const rmlx_qweight* all[3] = {gate, up, down};
+  for (const rmlx_qweight* q : all) {
+    if (q == nullptr) continue;
+    if (q->bits != 4 || q->group_size != 64)
+      return fail(RMLX_NOT_FOUND, "%s: expert weights must be Q4 with group_size 64 (got bits=%u group_size=%u)",
+                  who, q->bits, q->group_size);
+    if (!aligned16(q->w) || !aligned16(q->s) || !aligned16(q->b))
+      return fail(RMLX_INVALID_SHAPE, "%s: expert weight buffers must be 16-byte aligned", who);
+  }
+  RMLX_TRY(checked_u32(E, "num_experts", &sh->E));
+  RMLX_TRY(checked_u32(D, "hidden_dim", &sh->D));
+  RMLX_TRY(checked_u32(I, "intermediate_dim", &sh->I));
+  if (!qmv_q4_supported(sh->I, sh->D, 64) || !qmv_q4_supported(sh->D, sh->I, 64))
+    return fail(RMLX_NOT_FOUND, "%s: no kernel for hidden_dim=%u intermediate_dim=%u (both must be multiples of 512)",
+                who, sh->D, sh->I);
+  sh->fused = fused;
+  return RMLX_OK;
+}
+
+// gate/up + SwiGLU then down, over a device chunk table.  h: f16 [positions, I] scratch.
+int32_t run_expert_ffn(const rmlx_qweight* gate, const rmlx_qweight* up, const rmlx_qweight* down,
+                       const ExpertShapes& sh, const __half* x, const uint32_t* row_map, uint32_t row_div,
+                       const uint32_t* chunk_tab, const uint32_t* n_chunks, uint32_t max_chunks, __half* h,
+                       void* y, int y_f32, hipStream_t stream) {
+  QmvArgs a{};
+  a.w0 = gate->w; a.s0 = gate->s; a.b0 = gate->b;
+  if (sh.fused) {
+    a.w1 = gate->w + (size_t)sh.I * (sh.D / 8);
+    a.s1 = gate->s + (size_t)sh.I * (sh.D / 64);
+    a.b1 = gate->b + (size_t)sh.I * (sh.D / 64);
+  } else {
+    a.w1 = up->w; a.s1 = up->s; a.b1 = up->b;
+  }
+  const size_t rows_per_expert = sh.fused ? 2 * (size_t)sh.I : sh.I;
+  a.N = sh.I; a.K = sh.D;
+  a.expert_stride_w = rows_per_expert * (sh.D / 8);
+  a.expert_stride_s = rows_per_expert * (sh.D / 64);
+  a.x = x; a.row_map = row_map; a.row_div = row_div;
+  a.out = h; a.ld_out = sh.I; a.out_f32 = 0; a.dual = 1;
+  a.chunk_tab = chunk_tab; a.n_chunks_dev = n_chunks; a.max_chunks = max_chunks; a.mr = 8;
+  RMLX_TRY(launch_qmv_q4(a, stream));
+
+  QmvArgs d{};
+  d.w0 = down->w; d.s0 = down->s; d.b0 = down->b;
+  d.N = sh.D; d.K = sh.I;
+  d.expert_stride_w = (size_t)sh.D * (sh.I / 8);
+  d.expert_stride_s = (size_t)sh.D * (sh.I / 64);
+  d.x = h; d.row_map = nullptr; d.row_div = 1;
+  d.out = y; d.ld_out = sh.D; d.out_f32 = y_f32; d.dual = 0;
+  d.chunk_tab = chunk_tab; d.n_chunks_dev = n_chunks; d.max_chunks = max_chunks; d.mr = 8;
+  return launch_qmv_q4(d, stream);
+}
+
+}  // namespace
+}  // namespace rmlx
+
+using namespace rmlx;
+
+extern "C" {
+
+const char* rmlx_hip_last_error(void) { return last_error().c_str(); }
+
+// ---- runtime shim ---------------------------------------------------------------------------
+
+int32_t rmlx_hip_init(int32_t device) {
+  int count = 0;
+  RMLX_HIP_CHECK(hipGetDeviceCount(&count));
+  if (device < 0 || device >= count)
+    return fail(RMLX_RUNTIME_ERROR, "device %d not available (%d HIP devices visible)", device, count);
+  RMLX_HIP_CHECK(hipSetDevice(device));
+  hipDeviceProp_t prop;
+  RMLX_HIP_CHECK(hipGetDeviceProperties(&prop, device));
+  if (std::strncmp(prop.gcnArchName, "gfx950", 6) != 0)
+    return fail(RMLX_RUNTIME_ERROR, "device %d is %s; this library only contains gfx950 code", device, prop.gcnArchName);
+  ctx().device = device;
+  ctx().num_cus = prop.multiProcessorCount;
+  ctx().ready = true;
+  return RMLX_OK;
+}
+
+int32_t rmlx_hip_device_info(int64_t out[8]) {
+  RMLX_TRY(require_init());
+  hipDeviceProp_t prop;
+  RMLX_HIP_CHECK(hipGetDeviceProperties(&prop, ctx().device));
+  out[0] = prop.multiProcessorCount;
+  out[1] = prop.warpSize;
+  out[2] = (int64_t)prop.sharedMemPerBlock;
+  out[3] = (int64_t)(prop.totalGlobalMem >> 20);
+  out[4] = prop.clockRate;
+  out[5] = prop.memoryClockRate;
+  out[6] = prop.memoryBusWidth;
+  out[7] = prop.l2CacheSize;
+  return RMLX_OK;
+}
+
+int32_t rmlx_hip_malloc(void** dev_ptr, size_t bytes) {
+  RMLX_TRY(require_init());
+  RMLX_HIP_CHECK(hipMalloc(dev_ptr, bytes == 0 ? 16 : bytes));
+  return RMLX_OK;
+}
+int32_t rmlx_hip_free(void* dev_ptr) {
+  RMLX_HIP_CHECK(hipFree(dev_ptr));
+  return RMLX_OK;
+}
+int32_t rmlx_hip_memset(void* dev_ptr, int32_t value, size_t bytes, rmlx_stream stream) {
+  RMLX_HIP_CHECK(hipMemsetAsync(dev_ptr, value, bytes, (hipStream_t)stream));
+  return finish((hipStream_t)stream);
+}
+int32_t rmlx_hip_memcpy_h2d(void* dst, const void* src, size_t bytes, rmlx_stream stream) {
+  if (bytes == 0) return RMLX_OK;
+  if (stream == nullptr) RMLX_HIP_CHECK(hipMemcpy(dst, src, bytes, hipMemcpyHostToDevice));
+  else RMLX_HIP_CHECK(hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, (hipStream_t)stream));
+  return RMLX_OK;
+}
+int32_t rmlx_hip_memcpy_d2h(void* dst, const void* src, size_t bytes, rmlx_stream stream) {
+  if (bytes == 0) return RMLX_OK;
+  if (stream == nullptr) RMLX_HIP_CHECK(hipMemcpy(dst, src, bytes, hipMemcpyDeviceToHost));
+  else RMLX_HIP_CHECK(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, (hipStream_t)stream));
+  return RMLX_OK;
+}
+int32_t rmlx_hip_memcpy_d2d(void* dst, const void* src, size_t bytes, rmlx_stream stream) {
+  if (bytes == 0) return RMLX_OK;
+  RMLX_HIP_CHECK(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, (hipStream_t)stream));
+  return finish((hipStream_t)stream);
+}
+int32_t rmlx_hip_stream_create(rmlx_stream* out) {
+  RMLX_TRY(require_init());
+  hipStream_t s;
+  RMLX_HIP_CHECK(hipStreamCreateWithFlags(&s, hipStreamNonBlocking));
+  *out = s;
+  return RMLX_OK;
+}
+int32_t rmlx_hip_stream_sync(rmlx_stream stream) {
+  RMLX_HIP_CHECK(hipStreamSynchronize((hipStream_t)stream));
+  return RMLX_OK;
+}
+int32_t rmlx_hip_stream_destroy(rmlx_stream stream) {
+  RMLX_HIP_CHECK(hipStreamDestroy((hipStream_t)stream));
+  return RMLX_OK;
+}
+int32_t rmlx_hip_event_create(rmlx_event* out) {
+  RMLX_TRY(require_init());
+  hipEvent_t e;
+  RMLX_HIP_CHECK(hipEventCreate(&e));
+  *out = e;
+  return RMLX_OK;
+}
+int32_t rmlx_hip_event_record(rmlx_event ev, rmlx_stream stream) {
+  RMLX_HIP_CHECK(hipEventRecord((hipEvent_t)ev, (hipStream_t)stream));
+  return RMLX_OK;
+}
+int32_t rmlx_hip_event_sync(rmlx_event ev) {
+  RMLX_HIP_CHECK(hipEventSynchronize((hipEvent_t)ev));
+  return RMLX_OK;
+}
+int32_t rmlx_hip_event_elapsed_ms(rmlx_event start, rmlx_event stop, float* ms) {
+  RMLX_HIP_CHECK(hipEventElapsedTime(ms, (hipEvent_t)start, (hipEvent_t)stop));
+  return RMLX_OK;
+}
+int32_t rmlx_hip_event_destroy(rmlx_event ev) {
+  RMLX_HIP_CHECK(hipEventDestroy((hipEvent_t)ev));
+  return RMLX_OK;
+}
+
+// ---- QuantizedWeight --------------------------------------------------------------------------
+
+int32_t rmlx_hip_qweight_create(const void* weights_dev, size_t weights_bytes, const void* scales_dev,
+                                size_t scales_bytes, const void* biases_dev, size_t biases_bytes,
+                                uint32_t group_size, uint32_t bits, size_t out_features, size_t in_features,
+                                size_t n_experts, rmlx_qweight** out) {
+  if (out == nullptr) return fail(RMLX_INVALID_SHAPE, "qweight_create: out handle pointer is null");
+  *out = nullptr;
+  if (bits != 2 && bits != 3 && bits != 4 && bits != 6 && bits != 8)
+    return fail(RMLX_INVALID_SHAPE, "unsupported bit width %u; must be one of [2, 3, 4, 6, 8]", bits);
+  if (group_size != 32 && group_size != 64 && group_size != 128)
+    return fail(RMLX_INVALID_SHAPE, "unsupported group_size %u; must be one of [32, 64, 128]", group_size);
+  if (in_features % group_size != 0)
+    return fail(RMLX_INVALID_SHAPE, "in_features (%zu) must be a multiple of group_size (%u)", in_features, group_size);
+  if (n_experts == 0) return fail(RMLX_INVALID_SHAPE, "n_experts must be non-zero");
+  const size_t total = n_experts * out_features * in_features;
+  const size_t per = 32 / bits;
+  const size_t expected_w = ((total + per - 1) / per) * 4;
+  if (weights_bytes < expected_w)
+    return fail(RMLX_INVALID_SHAPE, "weights_buf too small: %zu bytes < expected %zu bytes for [%zu, %zu] at %u bits",
+                weights_bytes, expected_w, out_features, in_features, bits);
+  const size_t groups = total / group_size;
+  const size_t expected_s = groups * 2;
+  if (scales_bytes < expected_s)
+    return fail(RMLX_INVALID_SHAPE, "scales_buf too small: %zu bytes < expected %zu bytes (%zu groups)", scales_bytes,
+                expected_s, groups);
+  if (biases_bytes < expected_s)
+    return fail(RMLX_INVALID_SHAPE, "biases_buf too small: %zu bytes < expected %zu bytes (%zu groups)", biases_bytes,
+                expected_s, groups);
+  if (total != 0 && (weights_dev == nullptr || scales_dev == nullptr || biases_dev == nullptr))
+    return fail(RMLX_INVALID_SHAPE, "qweight_create: null device buffer");
+  rmlx_qweight* q = new rmlx_qweight;
+  q->w = static_cast<const uint32_t*>(weights_dev);
+  q->s = static_cast<const __half*>(scales_dev);
+  q->b = static_cast<const __half*>(biases_dev);
+  q->group_size = group_size;
+  q->bits = bits;
+  q->out_features = out_features;
+  q->in_features = in_features;
+  q->n_experts = n_experts;
+  *out = q;
+  return RMLX_OK;
+}
+
+int32_t rmlx_hip_qweight_destroy(rmlx_qweight* qw) {
+  delete qw;
+  return RMLX_OK;
+}
+
+// ---- qmv / qmm ------------------------------------------------------------------------------------
+
+int32_t rmlx_hip_affine_quantized_matmul(const rmlx_qweight* qw, const rmlx_array* vec, void* out_f16_dev,
+                                         size_t out_bytes, rmlx_stream stream) {
+  RMLX_TRY(require_init());
+  if (qw == nullptr || vec == nullptr) return fail(RMLX_INVALID_SHAPE, "affine_quantized_matmul: null argument");
+  if (vec->dtype != RMLX_DTYPE_F32 && vec->dtype != RMLX_DTYPE_F16 && vec->dtype != RMLX_DTYPE_BF16)
+    return fail(RMLX_INVALID_SHAPE, "affine_quantized_matmul requires Float16 or Float32 input vec, got %s",
+                dtype_name(vec->dtype));
+  if (numel(vec) != qw->in_features)
+    return fail(RMLX_INVALID_SHAPE, "vec.numel() (%zu) != in_features (%zu)", numel(vec), qw->in_features);
+  if (qw->n_experts != 1) return fail(RMLX_INVALID_SHAPE, "affine_quantized_matmul: weight is a stacked expert weight");
+  RMLX_TRY(check_out("affine_quantized_matmul", out_bytes, qw->out_features * 2));
+  RMLX_TRY(run_matmul(qw, vec->data, vec->dtype, 1, static_cast<__half*>(out_f16_dev), KERNEL_AUTO, (hipStream_t)stream));
+  return finish((hipStream_t)stream);
+}
+
+int32_t rmlx_hip_qmm_select(const rmlx_qweight* qw, const rmlx_array* x, int32_t kernel, void* out_f16_dev,
+                            size_t out_bytes, rmlx_stream stream) {
+  RMLX_TRY(require_init());
+  if (qw == nullptr || x == nullptr) return fail(RMLX_INVALID_SHAPE, "affine_quantized_matmul_batched: null argument");
+  RMLX_TRY(check_x_dtype("affine_quantized_matmul_batched", x->dtype));
+  if (x->ndim != 2)
+    return fail(RMLX_INVALID_SHAPE, "affine_quantized_matmul_batched requires 2D input x, got %dD", x->ndim);
+  if (x->shape[1] != qw->in_features)
+    return fail(RMLX_INVALID_SHAPE, "x.shape[1] (%zu) != in_features (%zu)", x->shape[1], qw->in_features);
+  if (qw->bits != 4 && qw->bits != 8 && kernel != KERNEL_GENERIC)
+    return fail(RMLX_INVALID_SHAPE, "affine_quantized_matmul_batched requires bits==4 or bits==8, got %u", qw->bits);
+  if (qw->n_experts != 1) return fail(RMLX_INVALID_SHAPE, "affine_quantized_matmul_batched: weight is a stacked expert weight");
+  uint32_t M;
+  RMLX_TRY(checked_u32(x->shape[0], "M", &M));
+  RMLX_TRY(check_out("affine_quantized_matmul_batched", out_bytes, (size_t)M * qw->out_features * 2));
+  RMLX_TRY(run_matmul(qw, x->data, x->dtype, M, static_cast<__half*>(out_f16_dev), kernel, (hipStream_t)stream));
+  return finish((hipStream_t)stream);
+}
+
+int32_t rmlx_hip_affine_quantized_matmul_batched(const rmlx_qweight* qw, const rmlx_array* x, void* out_f16_dev,
+                                                 size_t out_bytes, rmlx_stream stream) {
+  return rmlx_hip_qmm_select(qw, x, KERNEL_AUTO, out_f16_dev, out_bytes, stream);
+}
+
+int32_t rmlx_hip_quantized_linear_forward(const rmlx_qweight* qw, const rmlx_array* x, const void* bias_f16_dev,
+                                          void* out_f16_dev, size_t out_bytes, rmlx_stream stream) {
+  RMLX_TRY(require_init());
+  if (qw == nullptr || x == nullptr) return fail(RMLX_INVALID_SHAPE, "QuantizedLinear: null argument");
+  size_t batch, feat;
+  if (x->ndim == 1) { batch = 1; feat = x->shape[0]; }
+  else if (x->ndim == 2) { batch = x->shape[0]; feat = x->shape[1]; }
+  else return fail(RMLX_INVALID_SHAPE, "QuantizedLinear: input must be 1D or 2D, got %dD", x->ndim);
+  if (dtype_size(x->dtype) == 0 || x->dtype == RMLX_DTYPE_U32 || x->dtype == RMLX_DTYPE_U8)
+    return fail(RMLX_INVALID_SHAPE, "QuantizedLinear: unsupported input dtype %s", dtype_name(x->dtype));
+  if (feat != qw->in_features)
+    return fail(RMLX_INVALID_SHAPE, "QuantizedLinear: input features mismatch: %zu vs %zu", feat, qw->in_features);
+  if (qw->bits != 4 && qw->bits != 8)
+    return fail(RMLX_INVALID_SHAPE, "QuantizedLinear: bits must be 4 or 8, got %u", qw->bits);
+  uint32_t M, N;
+  RMLX_TRY(checked_u32(batch, "batch", &M));
+  RMLX_TRY(checked_u32(qw->out_features, "out_features", &N));
+  RMLX_TRY(check_out("QuantizedLinear", out_bytes, (size_t)M * N * 2));
+  hipStream_t s = (hipStream_t)stream;
+  RMLX_TRY(run_matmul(qw, x->data, x->dtype, M, static_cast<__half*>(out_f16_dev), KERNEL_AUTO, s));
+  if (bias_f16_dev != nullptr)
+    RMLX_TRY(launch_add_bias_rows(static_cast<__half*>(out_f16_dev), static_cast<const __half*>(bias_f16_dev), M, N, s));
+  return finish(s);
+}
+
+// ---- gather_qmm -----------------------------------------------------------------------------------
+
+int32_t rmlx_hip_gather_qmm(const rmlx_array* x, const void* w_packed_dev, size_t w_bytes, const void* scales_dev,
+                            size_t scales_bytes, const void* biases_dev, size_t biases_bytes,
+                            const rmlx_array* indices, size_t batch, size_t m_per_batch, size_t n, size_t k,
+                            size_t n_experts, uint32_t group_size, void* out_f16_dev, size_t out_bytes,
+                            rmlx_stream stream) {
+  RMLX_TRY(require_init());
+  if (x == nullptr || indices == nullptr) return fail(RMLX_INVALID_SHAPE, "gather_qmm: null argument");
+  if (x->dtype != RMLX_DTYPE_F32 && x->dtype != RMLX_DTYPE_F16)
+    return fail(RMLX_INVALID_SHAPE, "gather_qmm requires Float32 or Float16 input x, got %s", dtype_name(x->dtype));
+  if (indices->dtype != RMLX_DTYPE_U32)
+    return fail(RMLX_INVALID_SHAPE, "gather_qmm: indices must be UInt32, got %s", dtype_name(indices->dtype));
+  if (k == 0 || n == 0 || m_per_batch == 0)
+    return fail(RMLX_INVALID_SHAPE, "gather_qmm: dimensions must be non-zero (k=%zu, n=%zu, m_per_batch=%zu)", k, n, m_per_batch);
+  if (n_experts == 0) return fail(RMLX_INVALID_SHAPE, "gather_qmm: n_experts must be non-zero");
+  const size_t expected_x = batch * m_per_batch * k;
+  if (numel(x) != expected_x)
+    return fail(RMLX_INVALID_SHAPE, "gather_qmm: x has %zu elements but expected batch(%zu) * m_per_batch(%zu) * k(%zu) = %zu",
+                numel(x), batch, m_per_batch, k, expected_x);
+  if (numel(indices) != batch)
+    return fail(RMLX_INVALID_SHAPE, "gather_qmm: indices length %zu != batch %zu", numel(indices), batch);
+  if (group_size == 0) return fail(RMLX_INVALID_SHAPE, "gather_qmm: group_size must be non-zero");
+  if (k % 2 != 0) return fail(RMLX_INVALID_SHAPE, "gather_qmm: K (%zu) must be even for Q4 packing", k);
+  if (k % group_size != 0)
+    return fail(RMLX_INVALID_SHAPE, "gather_qmm: K (%zu) must be a multiple of group_size (%u)", k, group_size);
+  if (k % 8 != 0) return fail(RMLX_INVALID_SHAPE, "gather_qmm: K (%zu) must be a multiple of pack_factor (8)", k);
+  const size_t half_k = k / 2, gpr = k / group_size;
+  const size_t expected_w = n_experts * n * half_k;
+  if (w_bytes < expected_w)
+    return fail(RMLX_INVALID_SHAPE, "gather_qmm: w_packed_buf too small: %zu bytes < expected %zu bytes (n_experts=%zu, N=%zu, K/2=%zu)",
+                w_bytes, expected_w, n_experts, n, half_k);
+  const size_t expected_s = n_experts * n * gpr * 2;
+  if (scales_bytes < expected_s)
+    return fail(RMLX_INVALID_SHAPE, "gather_qmm: scales_buf too small: %zu bytes < expected %zu bytes (n_experts=%zu, N=%zu, groups_per_row=%zu)",
+                scales_bytes, expected_s, n_experts, n, gpr);
+  if (biases_bytes < expected_s)
+    return fail(RMLX_INVALID_SHAPE, "gather_qmm: biases_buf too small: %zu bytes < expected %zu bytes (n_experts=%zu, N=%zu, groups_per_row=%zu)",
+                biases_bytes, expected_s, n_experts, n, gpr);
+  uint32_t B32, M32, N32, K32, E32;
+  RMLX_TRY(checked_u32(batch, "batch", &B32));
+  RMLX_TRY(checked_u32(m_per_batch, "M_per_batch", &M32));
+  RMLX_TRY(checked_u32(n, "N", &N32));
+  RMLX_TRY(checked_u32(k, "K", &K32));
+  RMLX_TRY(checked_u32(n_experts, "n_experts", &E32));
+  RMLX_TRY(checked_u32(batch * m_per_batch, "batch * M_per_batch", &M32));
+  RMLX_TRY(check_out("gather_qmm", out_bytes, batch * m_per_batch * n * 2));
+  if (batch == 0) return RMLX_OK;  // empty result
+
+  hipStream_t s = (hipStream_t)stream;
+  const uint32_t* idx = static_cast<const uint32_t*>(indices->data);
+  if (stream == nullptr) {  // the reference validates every index on the host (quantized.rs:9514-9524)
+    std::vector<uint32_t> host(batch);
+    RMLX_HIP_CHECK(hipMemcpy(host.data(), idx, batch * 4, hipMemcpyDeviceToHost));
+    for (size_t i = 0; i < batch; ++i)
+      if (host[i] >= n_experts)
+        return fail(RMLX_INVALID_SHAPE, "gather_qmm: index[%zu]=%u out of range [0, %zu)", i, host[i], n_experts);
+  }
+
+  const uint32_t rows = B32 * (uint32_t)m_per_batch;
+  Scratch cast;
+  const __half* xk = static_cast<const __half*>(x->data);
+  if (x->dtype != RMLX_DTYPE_F16) {
+    RMLX_TRY(cast.alloc((size_t)rows * k * 2, s));
+    RMLX_TRY(launch_cast_to_f16(x->data, x->dtype, static_cast<__half*>(cast.ptr), (size_t)rows * k, s));
+    xk = static_cast<const __half*>(cast.ptr);
+  }
+  const uint32_t* w = static_cast<const uint32_t*>(w_packed_dev);
+  const __half* sc = static_cast<const __half*>(scales_dev);
+  const __half* bi = static_cast<const __half*>(biases_dev);
+  const bool fast = group_size == 64 && qmv_q4_supported(N32, K32, 64) && aligned16(w) && aligned16(sc) &&
+                    aligned16(bi) && aligned16(xk);
+  if (fast) {
+    const uint32_t per = ((uint32_t)m_per_batch + 7) / 8, n_chunks = B32 * per;
+    if (n_chunks > 65535) return fail(RMLX_INVALID_SHAPE, "gather_qmm: too many row chunks (%u)", n_chunks);
+    Scratch tab;
+    RMLX_TRY(tab.alloc((size_t)n_chunks * 12, s));
+    RMLX_TRY(launch_build_gather_chunks(idx, B32, (uint32_t)m_per_batch, E32, static_cast<uint32_t*>(tab.ptr), s));
+    QmvArgs a{};
+    a.w0 = w; a.s0 = sc; a.b0 = bi;
+    a.N = N32; a.K = K32;
+    a.expert_stride_w = (uint64_t)n * (k / 8);
+    a.expert_stride_s = (uint64_t)n * gpr;
+    a.x = xk; a.out = out_f16_dev; a.ld_out = N32;
+    a.chunk_tab = static_cast<const uint32_t*>(tab.ptr); a.max_chunks = n_chunks;
+    a.mr = m_per_batch >= 5 ? 8 : (m_per_batch >= 3 ? 4 : (m_per_batch == 2 ? 2 : 1));
+    RMLX_TRY(launch_qmv_q4(a, s));
+  } else {
+    GenericArgs g{w, sc, bi, xk, static_cast<__half*>(out_f16_dev), idx, (uint32_t)m_per_batch, rows, N32, K32,
+                  group_size, 4, E32};
+    RMLX_TRY(launch_generic(g, s));
+  }
+  return finish(s);
+}
+
+// ---- routing / grouping / data movement ----------------------------------------------------------------
+
+int32_t rmlx_hip_topk_route(const rmlx_array* gate_logits, size_t top_k, const rmlx_array* expert_bias,
+                            int32_t renormalize, uint32_t* expert_indices_dev, float* expert_weights_dev,
+                            uint32_t* expert_counts_dev, uint32_t* dispatch_offsets_dev, rmlx_stream stream) {
+  RMLX_TRY(require_init());
+  if (gate_logits == nullptr) return fail(RMLX_INVALID_SHAPE, "gpu_topk_route: null gate_logits");
+  if (gate_logits->ndim != 2)
+    return fail(RMLX_INVALID_SHAPE, "gpu_topk_route: gate_logits must be 2D [N, E], got %dD", gate_logits->ndim);
+  if (gate_logits->dtype != RMLX_DTYPE_F32 && gate_logits->dtype != RMLX_DTYPE_F16)
+    return fail(RMLX_INVALID_SHAPE, "gpu_topk_route: gate_logits must be Float16 or Float32, got %s",
+                dtype_name(gate_logits->dtype));
+  if (top_k == 0 || top_k > 8) return fail(RMLX_INVALID_SHAPE, "gpu_topk_route: top_k must be in [1, 8], got %zu", top_k);
+  const size_t T = gate_logits->shape[0], E = gate_logits->shape[1];
+  if (top_k > E) return fail(RMLX_INVALID_SHAPE, "gpu_topk_route: top_k (%zu) > num_experts (%zu)", top_k, E);
+  if (E > 256) return fail(RMLX_INVALID_SHAPE, "gpu_topk_route: num_experts (%zu) exceeds maximum 256", E);
+  if (expert_bias != nullptr) {
+    if (expert_bias->ndim != 1)
+      return fail(RMLX_INVALID_SHAPE, "gpu_topk_route: expert_bias must be 1D [E], got %dD", expert_bias->ndim);
+    if (expert_bias->shape[0] != E)
+      return fail(RMLX_INVALID_SHAPE, "gpu_topk_route: expert_bias length %zu != num_experts %zu", expert_bias->shape[0], E);
+    if (expert_bias->dtype != RMLX_DTYPE_F32 && expert_bias->dtype != RMLX_DTYPE_F16)
+      return fail(RMLX_INVALID_SHAPE, "gpu_topk_route: expert_bias must be Float16 or Float32, got %s",
+                  dtype_name(expert_bias->dtype));
+  }
+  uint32_t T32, A32;
+  RMLX_TRY(checked_u32(T, "seq_len", &T32));
+  RMLX_TRY(checked_u32(T * top_k, "seq_len * top_k", &A32));
+  hipStream_t s = (hipStream_t)stream;
+  // f16 inputs are widened to f32 first, as the reference does (topk_route.rs:474-483).
+  Scratch lg32, bias32;
+  const float* lg = static_cast<const float*>(gate_logits->data);
+  if (gate_logits->dtype == RMLX_DTYPE_F16) {
+    RMLX_TRY(lg32.alloc(T * E * 4, s));
+    RMLX_TRY(launch_cast_f16_to_f32(static_cast<const __half*>(gate_logits->data), static_cast<float*>(lg32.ptr), T * E, s));
+    lg = static_cast<const float*>(lg32.ptr);
+  }
+  const float* bias = nullptr;
+  if (expert_bias != nullptr) {
+    bias = static_cast<const float*>(expert_bias->data);
+    if (expert_bias->dtype == RMLX_DTYPE_F16) {
+      RMLX_TRY(bias32.alloc(E * 4, s));
+      RMLX_TRY(launch_cast_f16_to_f32(static_cast<const __half*>(expert_bias->data), static_cast<float*>(bias32.ptr), E, s));
+      bias = static_cast<const float*>(bias32.ptr);
+    }
+  }
+  RMLX_TRY(launch_topk_route(lg, bias, T32, (uint32_t)E, (uint32_t)top_k, renormalize, expert_indices_dev,
+                             expert_weights_dev, expert_counts_dev, dispatch_offsets_dev, s));
+  return finish(s);
+}
+
+int32_t rmlx_hip_moe_sort(const uint32_t* expert_indices_dev, size_t n_assign, size_t n_experts,
+                          uint32_t* sorted_assign_dev, uint32_t* offsets_dev, rmlx_stream stream) {
+  RMLX_TRY(require_init());
+  uint32_t A, E;
+  RMLX_TRY(checked_u32(n_assign, "n_assign", &A));
+  RMLX_TRY(checked_u32(n_experts, "n_experts", &E));
+  if (E == 0) return fail(RMLX_INVALID_SHAPE, "moe_sort: n_experts must be non-zero");
+  hipStream_t s = (hipStream_t)stream;
+  RMLX_TRY(launch_moe_sort(expert_indices_dev, A, E, sorted_assign_dev, nullptr, nullptr, offsets_dev, nullptr, nullptr, s));
+  return finish(s);
+}
+
+int32_t rmlx_hip_index_gather(const void* src_f16_dev, size_t src_rows, size_t d, const uint32_t* idx_dev, size_t n,
+                              void* dst_f16_dev, rmlx_stream stream) {
+  RMLX_TRY(require_init());
+  uint32_t R, D, N;
+  RMLX_TRY(checked_u32(src_rows, "src_rows", &R));
+  RMLX_TRY(checked_u32(d, "d", &D));
+  RMLX_TRY(checked_u32(n, "n", &N));
+  hipStream_t s = (hipStream_t)stream;
+  RMLX_TRY(launch_index_gather(static_cast<const __half*>(src_f16_dev), D, idx_dev, N, R, static_cast<__half*>(dst_f16_dev), s));
+  return finish(s);
+}
+
+int32_t rmlx_hip_scatter_weighted_add(const void* src_f16_dev, size_t n, size_t d, const uint32_t* tok_dev,
+                                      const float* w_dev, void* dst_f16_dev, size_t dst_rows, rmlx_stream stream) {
+  RMLX_TRY(require_init());
+  uint32_t N, D, R;
+  RMLX_TRY(checked_u32(n, "n", &N));
+  RMLX_TRY(checked_u32(d, "d", &D));
+  RMLX_TRY(checked_u32(dst_rows, "dst_rows", &R));
+  hipStream_t s = (hipStream_t)stream;
+  RMLX_TRY(launch_scatter_weighted_add(static_cast<const __half*>(src_f16_dev), N, D, tok_dev, w_dev,
+                                       static_cast<__half*>(dst_f16_dev), R, s));
+  return finish(s);
+}
+
+int32_t rmlx_hip_silu_gate(const void* gate_in_f16_dev, const void* up_in_f16_dev, void* out_f16_dev, size_t numel_,
+                           rmlx_stream stream) {
+  RMLX_TRY(require_init());
+  hipStream_t s = (hipStream_t)stream;
+  RMLX_TRY(launch_silu_gate(static_cast<const __half*>(gate_in_f16_dev), static_cast<const __half*>(up_in_f16_dev),
+                            static_cast<__half*>(out_f16_dev), numel_, s));
+  return finish(s);
+}
+
+// ---- expert FFN -------------------------------------------------------------------------------------
+
+int32_t rmlx_hip_expert_group_grouped_forward(const rmlx_qweight* gate, const rmlx_qweight* up,
+                                              const rmlx_qweight* down, size_t n_items,
+                                              const uint32_t* expert_idx_host, const uint32_t* batch_sizes_host,
+                                              const rmlx_array* x, void* out_f16_dev, size_t out_bytes,
+                                              rmlx_stream stream) {
+  RMLX_TRY(require_init());
+  if (n_items == 0) return RMLX_OK;  // empty in -> empty out (expert_group.rs:314-316)
+  ExpertShapes sh;
+  RMLX_TRY(check_expert_weights("ExpertGroup", gate, up, down, &sh));
+  if (x == nullptr || expert_idx_host == nullptr || batch_sizes_host == nullptr)
+    return fail(RMLX_INVALID_SHAPE, "ExpertGroup: null argument");
+  size_t total = 0;
+  std::vector<uint32_t> tab;
+  for (size_t i = 0; i < n_items; ++i) {
+    if (expert_idx_host[i] >= sh.E)
+      return fail(RMLX_INVALID_SHAPE, "ExpertGroup: expert_idx %u >= num_experts %u", expert_idx_host[i], sh.E);
+    for (uint32_t r = 0; r < batch_sizes_host[i]; r += 8) {
+      tab.push_back(expert_idx_host[i]);
+      tab.push_back((uint32_t)(total + r));
+      tab.push_back(batch_sizes_host[i] - r < 8u ? batch_sizes_host[i] - r : 8u);
+    }
+    total += batch_sizes_host[i];
+  }
+  if (x->ndim != 2) return fail(RMLX_INVALID_SHAPE, "ExpertGroup: input must be 2D [batch, D], got %dD", x->ndim);
+  if (x->shape[1] != sh.D) return fail(RMLX_INVALID_SHAPE, "ExpertGroup: input dim %zu != hidden_dim %u", x->shape[1], sh.D);
+  if (x->shape[0] != total)
+    return fail(RMLX_INVALID_SHAPE, "ExpertGroup: packed input has %zu rows but the batch sizes sum to %zu", x->shape[0], total);
+  if (x->dtype != RMLX_DTYPE_F16 && x->dtype != RMLX_DTYPE_F32 && x->dtype != RMLX_DTYPE_BF16)
+    return fail(RMLX_INVALID_SHAPE, "ExpertGroup: unsupported dtype %s for SiLU", dtype_name(x->dtype));
+  uint32_t rows;
+  RMLX_TRY(checked_u32(total, "total_tokens", &rows));
+  RMLX_TRY(check_out("ExpertGroup", out_bytes, total * sh.D * 2));
+  if (total == 0) return RMLX_OK;
+  const uint32_t n_chunks = (uint32_t)(tab.size() / 3);
+  if (n_chunks > 65535) return fail(RMLX_INVALID_SHAPE, "ExpertGroup: too many row chunks (%u)", n_chunks);
+
+  hipStream_t s = (hipStream_t)stream;
+  Scratch cast, dtab, h;
+  const __half* xk = static_cast<const __half*>(x->data);
+  if (x->dtype != RMLX_DTYPE_F16) {
+    RMLX_TRY(cast.alloc(total * sh.D * 2, s));
+    RMLX_TRY(launch_cast_to_f16(x->data, x->dtype, static_cast<__half*>(cast.ptr), total * sh.D, s));
+    xk = static_cast<const __half*>(cast.ptr);
+  }
+  if (!aligned16(xk)) return fail(RMLX_INVALID_SHAPE, "ExpertGroup: input must be 16-byte aligned");
+  RMLX_TRY(dtab.alloc(tab.size() * 4, s));
+  RMLX_HIP_CHECK(hipMemcpyAsync(dtab.ptr, tab.data(), tab.size() * 4, hipMemcpyHostToDevice, s));
+  RMLX_HIP_CHECK(hipStreamSynchronize(s));  // `tab` is pageable host memory owned by this call
+  RMLX_TRY(h.alloc(total * sh.I * 2, s));
+  RMLX_TRY(run_expert_ffn(gate, up, down, sh, xk, nullptr, 1, static_cast<const uint32_t*>(dtab.ptr), nullptr, n_chunks,
+                          static_cast<__half*>(h.ptr), out_f16_dev, 0, s));
+  return finish(s);
+}
+
+int32_t rmlx_hip_moe_forward_grouped(const rmlx_qweight* gate, const rmlx_qweight* up, const rmlx_qweight* down,
+                                     const rmlx_array* x, const uint32_t* expert_indices_dev,
+                                     const float* expert_weights_dev, size_t top_k, void* out_f16_dev, size_t out_bytes,
+                                     rmlx_stream stream) {
+  RMLX_TRY(require_init());
+  ExpertShapes sh;
+  RMLX_TRY(check_expert_weights("MoeLayer", gate, up, down, &sh));
+  if (x == nullptr) return fail(RMLX_INVALID_SHAPE, "MoeLayer: null input");
+  if (x->ndim != 2) return fail(RMLX_INVALID_SHAPE, "MoeLayer: input must be 2D [seq_len, hidden_dim], got %dD", x->ndim);
+  if (x->shape[1] != sh.D) return fail(RMLX_INVALID_SHAPE, "MoeLayer: input dim %zu != hidden_dim %u", x->shape[1], sh.D);
+  if (x->dtype != RMLX_DTYPE_F16 && x->dtype != RMLX_DTYPE_F32 && x->dtype != RMLX_DTYPE_BF16)
+    return fail(RMLX_INVALID_SHAPE, "MoeLayer: unsupported input dtype %s", dtype_name(x->dtype));
+  if (top_k == 0 || top_k > 8) return fail(RMLX_INVALID_SHAPE, "MoeLayer: top_k must be in [1, 8], got %zu", top_k);
+  const size_t T = x->shape[0];
+  uint32_t T32, A;
+  RMLX_TRY(checked_u32(T, "seq_len", &T32));
+  RMLX_TRY(checked_u32(T * top_k, "seq_len * top_k", &A));
+  RMLX_TRY(check_out("MoeLayer", out_bytes, T * sh.D * 2));
+  if (T == 0) return RMLX_OK;
+  const uint32_t max_chunks = A / 8 + (A < sh.E ? A : sh.E);
+  if (max_chunks > 65535) return fail(RMLX_INVALID_SHAPE, "MoeLayer: too many row chunks (%u); split the batch", max_chunks);
+
+  hipStream_t s = (hipStream_t)stream;
+  Scratch cast, meta, h, y;
+  const __half* xk = static_cast<const __half*>(x->data);
+  if (x->dtype != RMLX_DTYPE_F16) {
+    RMLX_TRY(cast.alloc(T * sh.D * 2, s));
+    RMLX_TRY(launch_cast_to_f16(x->data, x->dtype, static_cast<__half*>(cast.ptr), T * sh.D, s));
+    xk = static_cast<const __half*>(cast.ptr);
+  }
+  if (!aligned16(xk)) return fail(RMLX_INVALID_SHAPE, "MoeLayer: input must be 16-byte aligned");
+  // meta: sorted[A] | inv[A] | chunk_tab[3*max_chunks] | n_chunks[1]
+  RMLX_TRY(meta.alloc(((size_t)2 * A + 3 * (size_t)max_chunks + 4) * 4, s));
+  uint32_t* sorted = static_cast<uint32_t*>(meta.ptr);
+  uint32_t* inv = sorted + A;
+  uint32_t* chunk_tab = inv + A;
+  uint32_t* n_chunks = chunk_tab + 3 * (size_t)max_chunks;
+  RMLX_TRY(launch_moe_sort(expert_indices_dev, A, sh.E, sorted, inv, nullptr, nullptr, chunk_tab, n_chunks, s));
+  RMLX_TRY(h.alloc((size_t)A * sh.I * 2, s));
+  RMLX_TRY(y.alloc((size_t)A * sh.D * 4, s));
+  RMLX_TRY(run_expert_ffn(gate, up, down, sh, xk, sorted, (uint32_t)top_k, chunk_tab, n_chunks, max_chunks,
+                          static_cast<__half*>(h.ptr), y.ptr, 1, s));
+  RMLX_TRY(launch_moe_combine(static_cast<const float*>(y.ptr), inv, expert_weights_dev, T32, (uint32_t)top_k, sh.D,
+                              static_cast<__half*>(out_f16_dev), s));
+  return finish(s);
+}
+
+int32_t rmlx_hip_moe_forward(const rmlx_qweight* gate, const rmlx_qweight* up, const rmlx_qweight* down,
+                             const rmlx_array* x, const rmlx_array* gate_logits, size_t top_k,
+                             const rmlx_array* expert_bias, void* out_f16_dev, size_t out_bytes, rmlx_stream stream) {
+  RMLX_TRY(require_init());
+  if (x == nullptr || gate_logits == nullptr) return fail(RMLX_INVALID_SHAPE, "MoeLayer: null argument");
+  if (gate_logits->ndim != 2 || x->ndim != 2 || gate_logits->shape[0] != x->shape[0])
+    return fail(RMLX_INVALID_SHAPE, "MoeLayer: gate_logits must be [seq_len, num_experts] matching x");
+  if (gate != nullptr && gate_logits->shape[1] != gate->n_experts)
+    return fail(RMLX_INVALID_SHAPE, "MoeLayer: gate_logits has %zu experts but the weights hold %zu",
+                gate_logits->shape[1], gate->n_experts);
+  const size_t T = x->shape[0];
+  if (top_k == 0 || top_k > 8) return fail(RMLX_INVALID_SHAPE, "gpu_topk_route: top_k must be in [1, 8], got %zu", top_k);
+  hipStream_t s = (hipStream_t)stream;
+  Scratch route;
+  RMLX_TRY(route.alloc(T * top_k * 8 + 16, s));
+  uint32_t* idx = static_cast<uint32_t*>(route.ptr);
+  float* wts = reinterpret_cast<float*>(idx + T * top_k);
+  // Asynchronous inner calls need a real stream handle: the null stream means "synchronous".
+  RMLX_TRY(rmlx_hip_topk_route(gate_logits, top_k, expert_bias, 1, idx, wts, nullptr, nullptr, stream));
+  RMLX_TRY(rmlx_hip_moe_forward_grouped(gate, up, down, x, idx, wts, top_k, out_f16_dev, out_bytes, stream));
+  return finish(s);
+}
+
+}  // extern "C"

@@ -1,0 +1,163 @@
+// Internal definitions shared by the host-side entry points and the kernel launchers.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <hip/hip_fp16.h>
+#include <cstdarg>
+#include <cstdint>
+#include <cstdio>
+#include <string>
+
+#include "../../include/rmlx_hip.h"
+
+namespace rmlx {
+
+// ---- error channel ---------------------------------------------------------------------
+std::string& last_error();
+int32_t fail(int32_t code, const char* fmt, ...) __attribute__((format(printf, 2, 3)));
+
+#define RMLX_HIP_CHECK(expr)                                                                  \
+  do {                                                                                        \
+    hipError_t _e = (expr);                                                                   \
+    if (_e != hipSuccess)                                                                     \
+      return ::rmlx::fail(RMLX_RUNTIME_ERROR, "%s failed: %s (%s:%d)", #expr,                \
+                          hipGetErrorString(_e), __FILE__, __LINE__);                         \
+  } while (0)
+
+#define RMLX_TRY(expr)                 \
+  do {                                 \
+    int32_t _s = (expr);               \
+    if (_s != RMLX_OK) return _s;      \
+  } while (0)
+
+// `checked_u32` of the reference (crates/rmlx-core/src/ops/mod.rs:71-74).
+int32_t checked_u32(size_t v, const char* name, uint32_t* out);
+
+inline size_t dtype_size(int32_t dt) {
+  switch (dt) {
+    case RMLX_DTYPE_F32: case RMLX_DTYPE_U32: return 4;
+    case RMLX_DTYPE_F16: case RMLX_DTYPE_BF16: return 2;
+    case RMLX_DTYPE_U8: return 1;
+    default: return 0;
+  }
+}
+const char* dtype_name(int32_t dt);
+inline size_t numel(const rmlx_array* a) {
+  size_t n = 1;
+  for (int i = 0; i < a->ndim; ++i) n *= a->shape[i];
+  return n;
+}
+
+struct DeviceCtx {
+  bool ready = false;
+  int device = -1;
+  int num_cus = 0;
+};
+DeviceCtx& ctx();
+int32_t require_init();
+
+// Finishes a call: synchronous when the caller passed no stream.
+int32_t finish(hipStream_t stream);
+
+// Stream-ordered scratch (freed with release()).  Used only for dtype casts of the
+// activations and for the MoE intermediates, never on the f16 fast paths of qmv / qmm.
+struct Scratch {
+  void* ptr = nullptr;
+  hipStream_t stream = nullptr;
+  int32_t alloc(size_t bytes, hipStream_t s);
+  void release();
+  ~Scratch() { release(); }
+};
+
+}  // namespace rmlx
+
+// Opaque handle behind rmlx_qweight.
+struct rmlx_qweight {
+  const uint32_t* w;
+  const __half* s;
+  const __half* b;
+  uint32_t group_size;
+  uint32_t bits;
+  size_t out_features;  // N (per expert)
+  size_t in_features;   // K
+  size_t n_experts;     // 1 for a plain linear weight
+};
+
+namespace rmlx {
+
+// ---- kernel launchers (one translation unit per family) ------------------------------------
+
+// Activation cast to f16 (f32 / bf16 -> f16) or bf16 -> kept; n elements.
+int32_t launch_cast_to_f16(const void* src, int32_t src_dtype, __half* dst, size_t n, hipStream_t s);
+int32_t launch_cast_f16_to_f32(const __half* src, float* dst, size_t n, hipStream_t s);
+
+// Portable scalar kernel: any bits in {2,3,4,6,8}, any group size; x f16 [M,K] -> out f16 [M,N].
+// Optional per-row expert lookup (gather): W/S/B of row-batch b start at expert indices[b].
+struct GenericArgs {
+  const uint32_t* w; const __half* s; const __half* b;
+  const __half* x; __half* out;
+  const uint32_t* indices;  // nullable; one expert per `rows_per_index` consecutive x rows
+  uint32_t rows_per_index;
+  uint32_t M, N, K, group_size, bits, n_experts;
+};
+int32_t launch_generic(const GenericArgs& a, hipStream_t s);
+
+// Streaming GEMV family (qmv, gather_qmm, MoE expert projections).  Rows are processed in
+// chunks of at most 8; `chunk_tab` on the device lists (expert, first row position, row count)
+// triples (bit 31 of the count: write zeros instead of computing).
+struct QmvArgs {
+  const uint32_t* w0; const __half* s0; const __half* b0;  // tile set 0
+  const uint32_t* w1; const __half* s1; const __half* b1;  // tile set 1 (fused gate/up only)
+  uint32_t N;                // weight rows per expert covered by this launch (multiple of 16)
+  uint32_t K;                // multiple of 512
+  uint64_t expert_stride_w;  // u32 words per expert
+  uint64_t expert_stride_s;  // halves per expert
+  const __half* x;           // [x_rows, K] f16
+  const uint32_t* row_map;   // nullable: source row of position p is row_map[p] / row_div
+  uint32_t row_div;
+  void* out;                 // f16 [positions, ld_out] (f32 when out_f32)
+  uint32_t ld_out;
+  int out_f32;
+  int dual;                  // 1: out = silu(tile0 . x) * (tile1 . x)
+  const uint32_t* chunk_tab; // nullable -> expert 0, rows [0,M) in chunks of 8
+  const uint32_t* n_chunks_dev;  // nullable -> every chunk of the grid is valid
+  uint32_t max_chunks;       // grid.y when chunk_tab != null
+  uint32_t M;                // used when chunk_tab == null
+  uint32_t mr;               // rows staged per chunk (1,2,4,8); 0 -> derive from M
+};
+int32_t launch_qmv_q4(const QmvArgs& a, hipStream_t s);
+bool qmv_q4_supported(uint32_t N, uint32_t K, uint32_t group_size);
+// chunk table for gather_qmm: batch b owns rows [b*mpb, (b+1)*mpb) and expert indices[b]
+int32_t launch_build_gather_chunks(const uint32_t* indices, uint32_t batch, uint32_t mpb, uint32_t n_experts,
+                                   uint32_t* chunk_tab, hipStream_t s);
+
+struct QmmArgs {
+  const uint32_t* w; const __half* s; const __half* b;
+  const void* x;  // f16 or bf16 [M,K]
+  __half* out;    // [M,N]
+  uint32_t M, N, K, bits;
+  int x_bf16;
+};
+bool qmm_supported(uint32_t N, uint32_t K, uint32_t group_size, uint32_t bits);
+int32_t launch_qmm(const QmmArgs& a, hipStream_t s);
+
+// MoE helpers
+int32_t launch_topk_route(const float* logits, const float* bias, uint32_t T, uint32_t E, uint32_t K,
+                          int renorm, uint32_t* idx, float* w, uint32_t* counts, uint32_t* offsets,
+                          hipStream_t s);
+// Stable counting sort; also emits the chunk table used by the GEMV family
+// (chunk_tab: 3 u32 per chunk; n_chunks: 1 u32).  chunk_tab / n_chunks may be null.
+int32_t launch_moe_sort(const uint32_t* idx, uint32_t n_assign, uint32_t E, uint32_t* sorted, uint32_t* inv,
+                        uint32_t* counts, uint32_t* offsets, uint32_t* chunk_tab, uint32_t* n_chunks,
+                        hipStream_t s);
+int32_t launch_index_gather(const __half* src, uint32_t d, const uint32_t* idx, uint32_t n, uint32_t src_rows,
+                            __half* dst, hipStream_t s);
+int32_t launch_scatter_weighted_add(const __half* src, uint32_t n, uint32_t d, const uint32_t* tok,
+                                    const float* w, __half* dst, uint32_t dst_rows, hipStream_t s);
+int32_t launch_silu_gate(const __half* g, const __half* u, __half* out, size_t n, hipStream_t s);
+// out[t,:] = sum_k w[t*K+k] * y[inv[t*K+k],:]  (y f32 rows at sorted positions)
+int32_t launch_moe_combine(const float* y, const uint32_t* inv, const float* weights, uint32_t T,
+                           uint32_t top_k, uint32_t D, __half* out, hipStream_t s);
+int32_t launch_add_bias_rows(__half* out, const __half* bias, uint32_t M, uint32_t N, hipStream_t s);
+int32_t launch_check_indices(const uint32_t* idx, uint32_t n, uint32_t limit, uint32_t* flag, hipStream_t s);
+
+}  // namespace rmlx

@@ -1,0 +1,265 @@
+// MoE routing and data-movement kernels for gfx950.
+//
+//   topk_route_kernel   -- moe_topk_route_f32 (crates/rmlx-core/src/ops/topk_route.rs:212-359)
+//   moe_sort_kernel     -- histogram + exclusive scan (moe_prefix_scan_u32, topk_route.rs:373-388)
+//                          + the stable token->expert grouping the reference builds on the host
+//                          (crates/rmlx-nn/src/moe.rs:1439-1447), done on the device
+//   index_gather / scatter_weighted_add / silu_gate / combine
+//                       -- crates/rmlx-core/src/ops/moe_kernels.rs:46-223, ops/silu.rs:142-166
+#include "common.hpp"
+
+namespace rmlx {
+namespace {
+
+constexpr int kMaxExperts = 1024;  // LDS histogram capacity of the sort kernel
+
+// ---- routing: one wave per token -----------------------------------------------------------
+// Each lane owns experts lane, lane+64, lane+128, lane+192 (E <= 256).  Ranking uses the biased
+// logit with ties broken towards the lower expert index, which is the order of the softmax
+// values the reference ranks (exp is monotonic), made independent of the exp implementation.
+__global__ __launch_bounds__(64) void topk_route_kernel(const float* __restrict__ logits,
+                                                        const float* __restrict__ bias, uint32_t E,
+                                                        uint32_t K, int renorm, uint32_t* __restrict__ out_idx,
+                                                        float* __restrict__ out_w) {
+  const uint32_t row = blockIdx.x;
+  const uint32_t lane = threadIdx.x;
+  const float NEG_INF = -__builtin_inff();
+  float v[4], sm[4];
+  bool taken[4];
+  float mx = NEG_INF;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const uint32_t e = lane + 64 * j;
+    v[j] = NEG_INF;
+    taken[j] = e >= E;
+    if (e < E) {
+      v[j] = logits[(size_t)row * E + e];
+      if (bias != nullptr) v[j] += bias[e];
+    }
+    mx = fmaxf(mx, v[j]);
+  }
+  for (int off = 32; off > 0; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off, 64));
+  float sum = 0.f;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    sm[j] = (lane + 64 * j < E) ? expf(v[j] - mx) : 0.f;
+    sum += sm[j];
+  }
+  for (int off = 32; off > 0; off >>= 1) sum += __shfl_xor(sum, off, 64);
+  const float inv = 1.0f / sum;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) sm[j] *= inv;
+
+  float wsel[8];
+  uint32_t isel[8];
+  for (uint32_t k = 0; k < K; ++k) {
+    float bv = NEG_INF;
+    uint32_t bi = 0xFFFFFFFFu;
+    float bw = 0.f;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {  // ascending expert index inside the lane: strict > keeps the lower one
+      if (!taken[j] && (bi == 0xFFFFFFFFu || v[j] > bv)) { bv = v[j]; bi = lane + 64 * j; bw = sm[j]; }
+    }
+    for (int off = 32; off > 0; off >>= 1) {
+      const float ov = __shfl_xor(bv, off, 64);
+      const uint32_t oi = __shfl_xor(bi, off, 64);
+      const float ow = __shfl_xor(bw, off, 64);
+      const bool other_better = (oi != 0xFFFFFFFFu) && (bi == 0xFFFFFFFFu || ov > bv || (ov == bv && oi < bi));
+      if (other_better) { bv = ov; bi = oi; bw = ow; }
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      if (bi == lane + 64 * j) taken[j] = true;
+    isel[k] = bi;
+    wsel[k] = bw;
+  }
+  if (lane == 0) {
+    float scale = 1.0f;
+    if (renorm) {
+      float ws = 0.f;
+      for (uint32_t k = 0; k < K; ++k) ws += wsel[k];
+      scale = ws > 0.f ? 1.0f / ws : 0.f;
+    }
+    for (uint32_t k = 0; k < K; ++k) {
+      out_idx[(size_t)row * K + k] = isel[k];
+      out_w[(size_t)row * K + k] = wsel[k] * scale;
+    }
+  }
+}
+
+// ---- histogram + scan + stable counting sort, one workgroup --------------------------------
+// Deterministic by construction: thread e owns expert e and walks each block of 1024
+// assignments in ascending order, so ids of one expert keep their original order.
+__global__ __launch_bounds__(1024) void moe_sort_kernel(const uint32_t* __restrict__ idx, uint32_t n_assign,
+                                                        uint32_t E, uint32_t* __restrict__ sorted,
+                                                        uint32_t* __restrict__ inv, uint32_t* __restrict__ counts,
+                                                        uint32_t* __restrict__ offsets,
+                                                        uint32_t* __restrict__ chunk_tab,
+                                                        uint32_t* __restrict__ n_chunks) {
+  __shared__ uint32_t cnt[kMaxExperts];
+  __shared__ uint32_t off[kMaxExperts + 1];
+  __shared__ uint32_t ids[1024];
+  __shared__ uint32_t pos[1024];
+  const uint32_t tid = threadIdx.x;
+  for (uint32_t e = tid; e < E; e += 1024) cnt[e] = 0;
+  __syncthreads();
+  for (uint32_t i = tid; i < n_assign; i += 1024) {
+    const uint32_t e = idx[i];
+    if (e < E) atomicAdd(&cnt[e], 1u);
+  }
+  __syncthreads();
+  if (tid == 0) {
+    uint32_t run = 0, nc = 0;
+    for (uint32_t e = 0; e < E; ++e) {
+      off[e] = run;
+      if (chunk_tab != nullptr) {
+        for (uint32_t r = 0; r < cnt[e]; r += 8) {
+          chunk_tab[3 * nc + 0] = e;
+          chunk_tab[3 * nc + 1] = run + r;
+          chunk_tab[3 * nc + 2] = cnt[e] - r < 8u ? cnt[e] - r : 8u;
+          ++nc;
+        }
+      }
+      run += cnt[e];
+    }
+    off[E] = run;
+    if (n_chunks != nullptr) *n_chunks = nc;
+  }
+  __syncthreads();
+  for (uint32_t e = tid; e <= E; e += 1024) {
+    if (offsets != nullptr) offsets[e] = off[e];
+    if (counts != nullptr && e < E) counts[e] = cnt[e];
+  }
+  if (sorted == nullptr) return;
+
+  uint32_t cursor = tid < E ? off[tid] : 0;  // thread e places the ids of expert e
+  for (uint32_t base = 0; base < n_assign; base += 1024) {
+    const uint32_t nb = n_assign - base < 1024u ? n_assign - base : 1024u;
+    __syncthreads();
+    if (tid < nb) ids[tid] = idx[base + tid];
+    __syncthreads();
+    if (tid < E) {
+      for (uint32_t i = 0; i < nb; ++i)
+        if (ids[i] == tid) pos[i] = cursor++;
+    }
+    __syncthreads();
+    if (tid < nb && ids[tid] < E) {
+      sorted[pos[tid]] = base + tid;
+      if (inv != nullptr) inv[base + tid] = pos[tid];
+    }
+  }
+}
+
+__global__ void index_gather_kernel(const __half* __restrict__ src, uint32_t d, const uint32_t* __restrict__ idx,
+                                    uint32_t src_rows, __half* __restrict__ dst) {
+  const uint32_t i = blockIdx.x;
+  const uint32_t r = idx[i];
+  for (uint32_t c = threadIdx.x; c < d; c += blockDim.x)
+    dst[(size_t)i * d + c] = r < src_rows ? src[(size_t)r * d + c] : __float2half(0.f);
+}
+
+// One workgroup per destination row: assignments are visited in ascending order, so the f32
+// sum of a row is reproducible.
+__global__ void scatter_weighted_add_kernel(const __half* __restrict__ src, uint32_t n, uint32_t d,
+                                            const uint32_t* __restrict__ tok, const float* __restrict__ w,
+                                            __half* __restrict__ dst) {
+  const uint32_t t = blockIdx.x;
+  for (uint32_t c = threadIdx.x; c < d; c += blockDim.x) {
+    float acc = __half2float(dst[(size_t)t * d + c]);
+    for (uint32_t i = 0; i < n; ++i)
+      if (tok[i] == t) acc += w[i] * __half2float(src[(size_t)i * d + c]);
+    dst[(size_t)t * d + c] = __float2half(acc);
+  }
+}
+
+__global__ void silu_gate_kernel(const __half* __restrict__ g, const __half* __restrict__ u,
+                                 __half* __restrict__ out, size_t n) {
+  size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const size_t stride = (size_t)gridDim.x * blockDim.x;
+  for (; i < n; i += stride) {
+    const float x = __half2float(g[i]);
+    out[i] = __float2half(x / (1.0f + __expf(-x)) * __half2float(u[i]));
+  }
+}
+
+// out[t,:] = sum_k w[t*K+k] * y[inv[t*K+k],:], k ascending, f32.
+__global__ __launch_bounds__(256) void moe_combine_kernel(const float* __restrict__ y,
+                                                          const uint32_t* __restrict__ inv,
+                                                          const float* __restrict__ weights, uint32_t top_k,
+                                                          uint32_t D, __half* __restrict__ out) {
+  const uint32_t t = blockIdx.x;
+  for (uint32_t c = threadIdx.x * 4; c < D; c += blockDim.x * 4) {
+    float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+    for (uint32_t k = 0; k < top_k; ++k) {
+      const float w = weights[(size_t)t * top_k + k];
+      const float4 v = *reinterpret_cast<const float4*>(y + (size_t)inv[(size_t)t * top_k + k] * D + c);
+      acc.x += w * v.x; acc.y += w * v.y; acc.z += w * v.z; acc.w += w * v.w;
+    }
+    __half* o = out + (size_t)t * D + c;
+    o[0] = __float2half(acc.x); o[1] = __float2half(acc.y);
+    o[2] = __float2half(acc.z); o[3] = __float2half(acc.w);
+  }
+}
+
+}  // namespace
+
+int32_t launch_topk_route(const float* logits, const float* bias, uint32_t T, uint32_t E, uint32_t K,
+                          int renorm, uint32_t* idx, float* w, uint32_t* counts, uint32_t* offsets,
+                          hipStream_t s) {
+  if (T > 0) {
+    hipLaunchKernelGGL(topk_route_kernel, dim3(T), dim3(64), 0, s, logits, bias, E, K, renorm, idx, w);
+    RMLX_HIP_CHECK(hipGetLastError());
+  }
+  if (counts != nullptr || offsets != nullptr) {
+    hipLaunchKernelGGL(moe_sort_kernel, dim3(1), dim3(1024), 0, s, idx, T * K, E, (uint32_t*)nullptr,
+                       (uint32_t*)nullptr, counts, offsets, (uint32_t*)nullptr, (uint32_t*)nullptr);
+    RMLX_HIP_CHECK(hipGetLastError());
+  }
+  return RMLX_OK;
+}
+
+int32_t launch_moe_sort(const uint32_t* idx, uint32_t n_assign, uint32_t E, uint32_t* sorted, uint32_t* inv,
+                        uint32_t* counts, uint32_t* offsets, uint32_t* chunk_tab, uint32_t* n_chunks,
+                        hipStream_t s) {
+  if (E > (uint32_t)kMaxExperts)
+    return fail(RMLX_INVALID_SHAPE, "moe_sort: n_experts (%u) exceeds maximum %d", E, kMaxExperts);
+  hipLaunchKernelGGL(moe_sort_kernel, dim3(1), dim3(1024), 0, s, idx, n_assign, E, sorted, inv, counts, offsets,
+                     chunk_tab, n_chunks);
+  RMLX_HIP_CHECK(hipGetLastError());
+  return RMLX_OK;
+}
+
+int32_t launch_index_gather(const __half* src, uint32_t d, const uint32_t* idx, uint32_t n, uint32_t src_rows,
+                            __half* dst, hipStream_t s) {
+  if (n == 0 || d == 0) return RMLX_OK;
+  hipLaunchKernelGGL(index_gather_kernel, dim3(n), dim3(256), 0, s, src, d, idx, src_rows, dst);
+  RMLX_HIP_CHECK(hipGetLastError());
+  return RMLX_OK;
+}
+
+int32_t launch_scatter_weighted_add(const __half* src, uint32_t n, uint32_t d, const uint32_t* tok,
+                                    const float* w, __half* dst, uint32_t dst_rows, hipStream_t s) {
+  if (n == 0 || d == 0 || dst_rows == 0) return RMLX_OK;
+  hipLaunchKernelGGL(scatter_weighted_add_kernel, dim3(dst_rows), dim3(256), 0, s, src, n, d, tok, w, dst);
+  RMLX_HIP_CHECK(hipGetLastError());
+  return RMLX_OK;
+}
+
+int32_t launch_silu_gate(const __half* g, const __half* u, __half* out, size_t n, hipStream_t s) {
+  if (n == 0) return RMLX_OK;
+  size_t blocks = (n + 255) / 256;
+  if (blocks > 8192) blocks = 8192;
+  hipLaunchKernelGGL(silu_gate_kernel, dim3((unsigned)blocks), dim3(256), 0, s, g, u, out, n);
+  RMLX_HIP_CHECK(hipGetLastError());
+  return RMLX_OK;
+}
+
+int32_t launch_moe_combine(const float* y, const uint32_t* inv, const float* weights, uint32_t T, uint32_t top_k,
+                           uint32_t D, __half* out, hipStream_t s) {
+  if (T == 0) return RMLX_OK;
+  hipLaunchKernelGGL(moe_combine_kernel, dim3(T), dim3(256), 0, s, y, inv, weights, top_k, D, out);
+  RMLX_HIP_CHECK(hipGetLastError());
+  return RMLX_OK;
+}
+
+}  // namespace rmlx

@@ -1,0 +1,249 @@
+// Quantized GEMM for gfx950 (prefill, M > 16): dequantize weight tiles into LDS, f16 / bf16
+// MFMA with f32 accumulation, f16 output.
+//
+// Replaces the reference's affine_qmm_nax_q4 / affine_qmm_steel4sg_splitk_q4 /
+// affine_qmm_mma_q8 (crates/rmlx-core/src/ops/quantized.rs:3331-3565, 4572-4786, 5838-5971).
+//
+// Tile BM x BN x 64, 256 threads = 4 waves in a 2x2 grid, v_mfma_f32_16x16x32_{f16,bf16}.
+// Per 64-wide k step every thread dequantizes 16 weights once for the whole workgroup
+// (w = scale*q + bias evaluated in packed f16 after an exact magic-number int->f16 conversion;
+// in f32 for the bf16 variant), writes them to LDS in natural k order next to the raw
+// activation tile, and the four waves read MFMA fragments from there.  Global loads of step
+// t+1 are issued before the MFMAs of step t (register-staged double buffering, two LDS
+// buffers, one barrier per step).  Workgroup ids are remapped so that the tiles sharing a
+// weight panel run on the same XCD (shared L2).
+#include "common.hpp"
+
+namespace rmlx {
+namespace {
+
+typedef _Float16 h8 __attribute__((ext_vector_type(8)));
+typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+typedef __bf16 b8 __attribute__((ext_vector_type(8)));
+typedef float f4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u2 __attribute__((ext_vector_type(2)));
+
+constexpr int kThreads = 256;
+constexpr int BK = 64;
+constexpr int LDK = BK + 8;  // padded LDS row (halves)
+
+struct QmmParams {
+  const uint32_t* w; const __half* s; const __half* b;
+  const uint16_t* x;  // f16 or bf16 bits
+  __half* out;
+  uint32_t M, N, K;
+};
+
+__device__ __forceinline__ uint32_t h2bits(h2 v) { return __builtin_bit_cast(uint32_t, v); }
+
+// 8 Q4 values of one word -> 8 f16 weights (natural k order), w = s*q + b.
+__device__ __forceinline__ u4 dequant_q4_word_f16(uint32_t w, h2 s2, h2 b2) {
+  const uint32_t t = w >> 8;
+  const h2 k1024 = {(_Float16)1024.0f, (_Float16)1024.0f}, k64 = {(_Float16)64.0f, (_Float16)64.0f};
+  h2 p0 = __builtin_bit_cast(h2, (w & 0x000F000Fu) | 0x64006400u) - k1024;  // q0, q4
+  h2 p1 = __builtin_bit_cast(h2, (w & 0x00F000F0u) | 0x54005400u) - k64;    // q1, q5
+  h2 p2 = __builtin_bit_cast(h2, (t & 0x000F000Fu) | 0x64006400u) - k1024;  // q2, q6
+  h2 p3 = __builtin_bit_cast(h2, (t & 0x00F000F0u) | 0x54005400u) - k64;    // q3, q7
+  const uint32_t f0 = h2bits(p0 * s2 + b2), f1 = h2bits(p1 * s2 + b2);
+  const uint32_t f2 = h2bits(p2 * s2 + b2), f3 = h2bits(p3 * s2 + b2);
+  u4 o;
+  o.x = __builtin_amdgcn_perm(f1, f0, 0x05040100u);  // w0, w1
+  o.y = __builtin_amdgcn_perm(f3, f2, 0x05040100u);  // w2, w3
+  o.z = __builtin_amdgcn_perm(f1, f0, 0x07060302u);  // w4, w5
+  o.w = __builtin_amdgcn_perm(f3, f2, 0x07060302u);  // w6, w7
+  return o;
+}
+
+// 4 Q8 values of one word -> 4 f16 weights.
+__device__ __forceinline__ u2 dequant_q8_word_f16(uint32_t w, h2 s2, h2 b2) {
+  const h2 k1024 = {(_Float16)1024.0f, (_Float16)1024.0f};
+  h2 p0 = __builtin_bit_cast(h2, __builtin_amdgcn_perm(0x64646464u, w, 0x04010400u)) - k1024;  // q0, q1
+  h2 p1 = __builtin_bit_cast(h2, __builtin_amdgcn_perm(0x64646464u, w, 0x04030402u)) - k1024;  // q2, q3
+  u2 o;
+  o.x = h2bits(p0 * s2 + b2);
+  o.y = h2bits(p1 * s2 + b2);
+  return o;
+}
+
+__device__ __forceinline__ uint32_t pack_bf16(float a, float b) {
+  typedef __bf16 bf2 __attribute__((ext_vector_type(2)));
+  bf2 v = {(__bf16)a, (__bf16)b};
+  return __builtin_bit_cast(uint32_t, v);
+}
+
+// 4 Q8 values -> 4 bf16 weights, arithmetic in f32.
+__device__ __forceinline__ u2 dequant_q8_word_bf16(uint32_t w, float s, float b) {
+  const float q0 = (float)(w & 0xFFu), q1 = (float)((w >> 8) & 0xFFu);
+  const float q2 = (float)((w >> 16) & 0xFFu), q3 = (float)(w >> 24);
+  u2 o;
+  o.x = pack_bf16(s * q0 + b, s * q1 + b);
+  o.y = pack_bf16(s * q2 + b, s * q3 + b);
+  return o;
+}
+
+template <int BM, int BN, int BITS, bool XBF16>
+__global__ __launch_bounds__(kThreads) void qmm_kernel(QmmParams p) {
+  constexpr int WM = BM / 2, WN = BN / 2;      // wave tile
+  constexpr int TI = WM / 16, TJ = WN / 16;    // 16x16 MFMA tiles per wave
+  constexpr int A_UNITS = BM * BK / 8 / kThreads;  // 16-byte units of the activation tile per thread
+  constexpr int WPT = BN * BK * BITS / 32 / kThreads;  // weight words per thread per step
+  static_assert(BN == 64, "weight staging assumes 4 threads per weight row");
+  static_assert(WPT == (BITS == 4 ? 2 : 4), "16 weights per thread per step");
+
+  __shared__ __attribute__((aligned(16))) uint16_t As[2][BM * LDK];
+  __shared__ __attribute__((aligned(16))) uint16_t Bs[2][BN * LDK];
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+  const int r16 = lane & 15, g = lane >> 4;
+
+  // ---- tile assignment: consecutive ids go to different XCDs; give each XCD whole weight panels
+  const uint32_t tiles_m = (p.M + BM - 1) / BM, tiles_n = p.N / BN;
+  const uint32_t total = tiles_m * tiles_n;
+  uint32_t id = blockIdx.x;
+  if (total % 8 == 0) id = (id % 8) * (total / 8) + id / 8;
+  const uint32_t m0 = (id % tiles_m) * BM, n0 = (id / tiles_m) * BN;
+
+  const uint32_t K = p.K, gpr = K >> 6;
+  const int steps = K / BK;
+
+  // staging coordinates
+  const int brow = tid >> 2, bq = tid & 3;  // weight row in tile, 16-value quarter of the 64-k step
+  const uint32_t* wptr = p.w + (uint64_t)(n0 + brow) * (K * BITS / 32) + bq * WPT;
+  const __half* sptr = p.s + (uint64_t)(n0 + brow) * gpr;
+  const __half* bptr = p.b + (uint64_t)(n0 + brow) * gpr;
+
+  u4 areg[A_UNITS];
+  uint32_t wreg[WPT];
+  __half sreg, breg;
+
+  auto load_global = [&](int step) {
+#pragma unroll
+    for (int i = 0; i < A_UNITS; ++i) {
+      const int u = tid + i * kThreads, row = u >> 3, c8 = u & 7;
+      areg[i] = (u4){0u, 0u, 0u, 0u};
+      if (m0 + row < p.M)
+        areg[i] = *reinterpret_cast<const u4*>(p.x + (uint64_t)(m0 + row) * K + step * BK + c8 * 8);
+    }
+    if (BITS == 4) {
+      const u2 v = *reinterpret_cast<const u2*>(wptr + step * (BK * BITS / 32));
+      wreg[0] = v.x; wreg[1] = v.y;
+    } else {
+      const u4 v = *reinterpret_cast<const u4*>(wptr + step * (BK * BITS / 32));
+      wreg[0] = v.x; wreg[1] = v.y; wreg[WPT - 2] = v.z; wreg[WPT - 1] = v.w;
+    }
+    sreg = sptr[step];
+    breg = bptr[step];
+  };
+
+  auto store_lds = [&](int buf) {
+#pragma unroll
+    for (int i = 0; i < A_UNITS; ++i) {
+      const int u = tid + i * kThreads, row = u >> 3, c8 = u & 7;
+      *reinterpret_cast<u4*>(&As[buf][row * LDK + c8 * 8]) = areg[i];
+    }
+    uint16_t* dst = &Bs[buf][brow * LDK + bq * 16];
+    if (XBF16) {
+      const float s = __half2float(sreg), b = __half2float(breg);
+      const u2 lo = dequant_q8_word_bf16(wreg[0], s, b), l2 = dequant_q8_word_bf16(wreg[1], s, b);
+      const u2 h1 = dequant_q8_word_bf16(wreg[WPT - 2], s, b), h2v = dequant_q8_word_bf16(wreg[WPT - 1], s, b);
+      *reinterpret_cast<u4*>(dst) = (u4){lo.x, lo.y, l2.x, l2.y};
+      *reinterpret_cast<u4*>(dst + 8) = (u4){h1.x, h1.y, h2v.x, h2v.y};
+    } else {
+      const _Float16 sh = __builtin_bit_cast(_Float16, sreg), bh = __builtin_bit_cast(_Float16, breg);
+      const h2 s2 = {sh, sh}, b2 = {bh, bh};
+      if (BITS == 4) {
+        *reinterpret_cast<u4*>(dst) = dequant_q4_word_f16(wreg[0], s2, b2);
+        *reinterpret_cast<u4*>(dst + 8) = dequant_q4_word_f16(wreg[1], s2, b2);
+      } else {
+        const u2 a0 = dequant_q8_word_f16(wreg[0], s2, b2), a1 = dequant_q8_word_f16(wreg[1], s2, b2);
+        const u2 a2 = dequant_q8_word_f16(wreg[WPT - 2], s2, b2), a3 = dequant_q8_word_f16(wreg[WPT - 1], s2, b2);
+        *reinterpret_cast<u4*>(dst) = (u4){a0.x, a0.y, a1.x, a1.y};
+        *reinterpret_cast<u4*>(dst + 8) = (u4){a2.x, a2.y, a3.x, a3.y};
+      }
+    }
+  };
+
+  f4 acc[TI][TJ];
+#pragma unroll
+  for (int i = 0; i < TI; ++i)
+#pragma unroll
+    for (int j = 0; j < TJ; ++j) acc[i][j] = (f4){0.f, 0.f, 0.f, 0.f};
+
+  load_global(0);
+  store_lds(0);
+  __syncthreads();
+
+  for (int step = 0; step < steps; ++step) {
+    const int cur = step & 1;
+    if (step + 1 < steps) load_global(step + 1);
+#pragma unroll
+    for (int kk = 0; kk < BK / 32; ++kk) {
+      u4 af[TI], bf[TJ];
+#pragma unroll
+      for (int i = 0; i < TI; ++i)
+        af[i] = *reinterpret_cast<const u4*>(&As[cur][(wm * WM + i * 16 + r16) * LDK + kk * 32 + g * 8]);
+#pragma unroll
+      for (int j = 0; j < TJ; ++j)
+        bf[j] = *reinterpret_cast<const u4*>(&Bs[cur][(wn * WN + j * 16 + r16) * LDK + kk * 32 + g * 8]);
+#pragma unroll
+      for (int i = 0; i < TI; ++i)
+#pragma unroll
+        for (int j = 0; j < TJ; ++j) {
+          if (XBF16)
+            acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(b8, af[i]),
+                                                                __builtin_bit_cast(b8, bf[j]), acc[i][j], 0, 0, 0);
+          else
+            acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h8, af[i]),
+                                                               __builtin_bit_cast(h8, bf[j]), acc[i][j], 0, 0, 0);
+        }
+    }
+    if (step + 1 < steps) store_lds(cur ^ 1);
+    __syncthreads();
+  }
+
+  // accumulator lane (r16, g) holds column n = r16 and rows 4g..4g+3 of each 16x16 tile
+#pragma unroll
+  for (int i = 0; i < TI; ++i)
+#pragma unroll
+    for (int j = 0; j < TJ; ++j)
+#pragma unroll
+      for (int v = 0; v < 4; ++v) {
+        const uint32_t m = m0 + wm * WM + i * 16 + g * 4 + v;
+        const uint32_t nn = n0 + wn * WN + j * 16 + r16;
+        if (m < p.M) p.out[(uint64_t)m * p.N + nn] = __float2half(acc[i][j][v]);
+      }
+}
+
+template <int BM, int BITS, bool XBF16>
+void launch_t(const QmmParams& p, hipStream_t s) {
+  const uint32_t tiles = ((p.M + BM - 1) / BM) * (p.N / 64);
+  hipLaunchKernelGGL((qmm_kernel<BM, 64, BITS, XBF16>), dim3(tiles), dim3(kThreads), 0, s, p);
+}
+
+}  // namespace
+
+bool qmm_supported(uint32_t N, uint32_t K, uint32_t group_size, uint32_t bits) {
+  return group_size == 64 && (bits == 4 || bits == 8) && N % 64 == 0 && K % 64 == 0 && N > 0 && K > 0;
+}
+
+int32_t launch_qmm(const QmmArgs& a, hipStream_t s) {
+  if (!qmm_supported(a.N, a.K, 64, a.bits))
+    return fail(RMLX_INVALID_SHAPE, "qmm: unsupported shape N=%u K=%u bits=%u", a.N, a.K, a.bits);
+  if (a.M == 0) return RMLX_OK;
+  QmmParams p{a.w, a.s, a.b, reinterpret_cast<const uint16_t*>(a.x), a.out, a.M, a.N, a.K};
+  const bool big = a.M > 64;
+  if (a.bits == 4) {
+    if (a.x_bf16) return fail(RMLX_INVALID_SHAPE, "qmm: Q4 takes f16 activations (bf16 is cast by the caller)");
+    if (big) launch_t<128, 4, false>(p, s); else launch_t<64, 4, false>(p, s);
+  } else if (a.x_bf16) {
+    if (big) launch_t<128, 8, true>(p, s); else launch_t<64, 8, true>(p, s);
+  } else {
+    if (big) launch_t<128, 8, false>(p, s); else launch_t<64, 8, false>(p, s);
+  }
+  RMLX_HIP_CHECK(hipGetLastError());
+  return RMLX_OK;
+}
+
+}  // namespace rmlx

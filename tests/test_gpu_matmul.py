@@ -1,0 +1,270 @@
+"""GPU parity of qmv / qmm against the float64 dequantize-then-matmul oracle, through the C ABI.
+
+Tolerance everywhere: max|err| <= 1e-2 * RMS(oracle output) on f16 outputs (stated in
+helpers.assert_close).  Shapes follow the benchmark configurations plus ragged / edge cases.
+"""
+import numpy as np
+import pytest
+
+from oracle import model, refpath
+from tests.helpers import assert_close, make_weight, make_x, x_as_f64
+
+pytestmark = pytest.mark.gpu
+
+
+def _dev(hip, x, dtype):
+    from rmlx_amd.runtime import BF16, DeviceBuffer
+    return DeviceBuffer.from_numpy(x, BF16) if dtype == "bf16" else DeviceBuffer.from_numpy(x)
+
+
+def _run(hip, words, scales, biases, x, bits, gs=64, dtype="f16", kernel=0, qmv_entry=False):
+    from rmlx_amd import ops
+    qw = ops.QuantizedWeight.from_numpy(words, scales, biases, gs, bits)
+    xd = _dev(hip, x, dtype)
+    if qmv_entry:
+        return ops.affine_quantized_matmul(qw, xd).numpy()[None, :]
+    return ops.affine_quantized_matmul_batched(xd, qw, kernel=kernel).numpy()
+
+
+# ---- closed forms from the reference's tests, on the GPU ------------------------------------------
+
+def test_equal_nibble_closed_forms(hip):
+    from rmlx_amd import runtime as rt
+    # all nibbles c, scale 1, bias 0, x = 1 (row 0) / 2 (row 1): out = c*K, 2*c*K
+    # (quantized.rs:10895-10931, 11541-11591, 12069-12095 scaled to kernel-sized K)
+    for kernel, n, k in [(rt.KERNEL_GENERIC, 8, 64), (rt.KERNEL_QMV, 16, 512), (rt.KERNEL_QMM, 64, 512)]:
+        for c in (1, 3, 7):
+            words = np.full((n, k // 8), c * 0x11111111, np.uint32)
+            s = np.ones((n, k // 64), np.float16)
+            b = np.zeros((n, k // 64), np.float16)
+            x = np.concatenate([np.ones((1, k)), 2 * np.ones((1, k))]).astype(np.float16)
+            out = _run(hip, words, s, b, x, 4, kernel=kernel)
+            assert np.array_equal(out[0], np.full(n, c * k, np.float16)), (kernel, c, out[0][:4])
+            assert np.array_equal(out[1], np.full(n, 2 * c * k, np.float16))
+    # Q8: all bytes 7 -> 7*K (quantized.rs:11752-11800)
+    n, k = 64, 256
+    words = np.full((n, k // 4), 0x07070707, np.uint32)
+    x = np.ones((2, k), np.float16)
+    for kernel in (rt.KERNEL_GENERIC, rt.KERNEL_QMM):
+        out = _run(hip, words, np.ones((n, k // 64), np.float16), np.zeros((n, k // 64), np.float16), x, 8, kernel=kernel)
+        assert np.array_equal(out, np.full((2, n), 7 * k, np.float16))
+
+
+def test_distinct_positions_are_not_mixed_up(hip):
+    """One-hot activations pick out single weights: catches any k / row permutation mistake."""
+    from rmlx_amd import runtime as rt
+    rng = np.random.default_rng(5)
+    n, k = 64, 1024
+    words, s, b = make_weight(rng, n, k, 4)
+    s[:] = 1.0
+    b[:] = 0.0
+    q = model.unpack_u32(words, 4).astype(np.float64)
+    ks = np.array([0, 1, 2, 3, 4, 5, 6, 7, 8, 31, 32, 63, 64, 65, 127, 128, 511, 512, 1000, 1023])
+    for m0 in range(0, len(ks), 8):
+        sel = ks[m0:m0 + 8]
+        x = np.zeros((len(sel), k), np.float16)
+        x[np.arange(len(sel)), sel] = 1.0
+        for kernel in (rt.KERNEL_QMV, rt.KERNEL_QMM, rt.KERNEL_GENERIC):
+            out = _run(hip, words, s, b, x, 4, kernel=kernel)
+            assert np.array_equal(out.astype(np.float64), q[:, sel].T), (kernel, sel)
+
+
+# ---- configuration shapes ----------------------------------------------------------------------
+
+def test_config1_q4_qmv_4096(hip):
+    rng = np.random.default_rng(1001)
+    n = k = 4096
+    words, s, b = make_weight(rng, n, k, 4)
+    x = make_x(rng, 1, k)
+    ref = model.qmm(x_as_f64(x, "f16"), words, s, b, 64, 4)
+    out = _run(hip, words, s, b, x[0], 4, qmv_entry=True)
+    assert_close(out, ref, "config1 qmv")
+    # the CPU reference path (plumbing): C restatement of affine_qmm on the same inputs
+    cpu = refpath.affine_qmm(x.astype(np.float32), model.words_to_bytes(words), s.astype(np.float32),
+                             b.astype(np.float32), 1, n, k, 64)
+    assert_close(cpu, ref, "config1 cpu reference path")
+
+
+@pytest.mark.parametrize("m", [1, 4, 8])
+def test_config2_q4_qmv_qkv(hip, m):
+    rng = np.random.default_rng(1002)
+    n, k = 9216, 4096
+    words, s, b = make_weight(rng, n, k, 4)
+    x = make_x(rng, m, k)
+    ref = model.qmm(x_as_f64(x, "f16"), words, s, b, 64, 4)
+    assert_close(_run(hip, words, s, b, x, 4), ref, f"config2 M={m}")
+
+
+@pytest.mark.parametrize("m", [128, 512])
+def test_config3_q4_qmm(hip, m):
+    rng = np.random.default_rng(1003)
+    n = k = 4096
+    words, s, b = make_weight(rng, n, k, 4)
+    x = make_x(rng, m, k)
+    ref = model.qmm(x_as_f64(x, "f16"), words, s, b, 64, 4)
+    assert_close(_run(hip, words, s, b, x, 4), ref, f"config3 M={m}")
+
+
+def test_config4_q8_qmm_bf16(hip):
+    rng = np.random.default_rng(1004)
+    m, n, k = 128, 12288, 4096
+    words, s, b = make_weight(rng, n, k, 8)
+    x = make_x(rng, m, k, "bf16")
+    ref = model.qmm(x_as_f64(x, "bf16"), words, s, b, 64, 8)
+    assert_close(_run(hip, words, s, b, x, 8, dtype="bf16"), ref, "config4")
+
+
+# ---- kernel families agree, ragged M, dtypes, other group sizes --------------------------------------
+
+@pytest.mark.parametrize("m", [1, 2, 3, 5, 8, 9, 16, 17, 31, 64, 65, 130])
+def test_ragged_m_all_kernels(hip, m):
+    from rmlx_amd import runtime as rt
+    rng = np.random.default_rng(100 + m)
+    n, k = 128, 1024
+    words, s, b = make_weight(rng, n, k, 4)
+    x = make_x(rng, m, k)
+    ref = model.qmm(x_as_f64(x, "f16"), words, s, b, 64, 4)
+    for kernel in (rt.KERNEL_AUTO, rt.KERNEL_QMV, rt.KERNEL_QMM, rt.KERNEL_GENERIC):
+        assert_close(_run(hip, words, s, b, x, 4, kernel=kernel), ref, f"M={m} kernel={kernel}")
+
+
+@pytest.mark.parametrize("k", [512, 1536, 2048, 4608, 8192, 14336])
+def test_qmv_k_sweep(hip, k):
+    rng = np.random.default_rng(k)
+    n, m = 48, 3
+    words, s, b = make_weight(rng, n, k, 4)
+    x = make_x(rng, m, k)
+    ref = model.qmm(x_as_f64(x, "f16"), words, s, b, 64, 4)
+    assert_close(_run(hip, words, s, b, x, 4, kernel=1), ref, f"qmv K={k}")
+
+
+@pytest.mark.parametrize("bits", [4, 8])
+@pytest.mark.parametrize("dtype", ["f16", "f32", "bf16"])
+def test_input_dtypes(hip, bits, dtype):
+    rng = np.random.default_rng(7)
+    n, k = 128, 512
+    words, s, b = make_weight(rng, n, k, bits)
+    for m in (1, 40):
+        x = make_x(rng, m, k, dtype)
+        ref = model.qmm(x_as_f64(x, dtype), words, s, b, 64, bits)
+        assert_close(_run(hip, words, s, b, x, bits, dtype=dtype), ref, f"bits={bits} {dtype} M={m}")
+
+
+@pytest.mark.parametrize("bits", [2, 4, 8])
+@pytest.mark.parametrize("gs", [32, 64, 128])
+def test_group_sizes_and_odd_shapes_portable_kernel(hip, bits, gs):
+    rng = np.random.default_rng(gs + bits)
+    n, k, m = 24, 384, 5  # N not a multiple of 16, K not a multiple of 512 -> portable kernel
+    words, s, b = make_weight(rng, n, k, bits, gs)
+    x = make_x(rng, m, k)
+    ref = model.qmm(x_as_f64(x, "f16"), words, s, b, gs, bits)
+    assert_close(_run(hip, words, s, b, x, bits, gs=gs), ref, f"bits={bits} gs={gs}")
+
+
+def test_qmv_entry_equals_batched_m1(hip):
+    """M=1 qmm == qmv (quantized.rs:10895-10931), bit for bit on the same kernel."""
+    rng = np.random.default_rng(11)
+    n, k = 256, 2048
+    words, s, b = make_weight(rng, n, k, 4)
+    x = make_x(rng, 1, k)
+    a = _run(hip, words, s, b, x[0], 4, qmv_entry=True)
+    bb = _run(hip, words, s, b, x, 4)
+    assert np.array_equal(a, bb)
+
+
+def test_linearity_and_row_independence_full_size(hip):
+    """Size-independent properties at the full 4096^2 shape."""
+    rng = np.random.default_rng(12)
+    n = k = 4096
+    words, s, b = make_weight(rng, n, k, 4)
+    x1 = make_x(rng, 1, k).astype(np.float32)
+    x2 = make_x(rng, 1, k).astype(np.float32)
+    xs = np.concatenate([x1, x2, (x1 + x2)]).astype(np.float16)
+    out = _run(hip, words, s, b, xs, 4).astype(np.float64)
+    exact_sum = xs[2].astype(np.float64) - (xs[0].astype(np.float64) + xs[1].astype(np.float64))
+    assert np.max(np.abs(exact_sum)) < 0.01  # f16 rounding of the sum only
+    tol = 1e-2 * np.sqrt(np.mean(out[2] ** 2))
+    assert np.max(np.abs(out[2] - out[0] - out[1])) < 2 * tol
+    # rows of W are independent: a sub-block of rows gives the same values
+    sub = _run(hip, words[1024:1280], s[1024:1280], b[1024:1280], xs, 4)
+    assert np.array_equal(sub, _run(hip, words, s, b, xs, 4)[:, 1024:1280])
+
+
+def test_quantized_linear_forward(hip):
+    from rmlx_amd import ops
+    from rmlx_amd.runtime import DeviceBuffer
+    rng = np.random.default_rng(13)
+    n, k = 256, 1024
+    for bits in (4, 8):
+        words, s, b = make_weight(rng, n, k, bits)
+        layer = ops.QuantizedLinear(model.words_to_bytes(words), s.astype(np.float32), b.astype(np.float32), k, n, 64, bits)
+        x = make_x(rng, 6, k)
+        ref = model.qmm(x_as_f64(x, "f16"), words, s, b, 64, bits)
+        assert_close(layer.forward(DeviceBuffer.from_numpy(x)).numpy(), ref, "2D")
+        out1 = layer.forward(DeviceBuffer.from_numpy(x[0])).numpy()  # 1-D -> [1, out]
+        assert out1.shape == (1, n)
+        assert_close(out1, ref[:1], "1D")
+        bias = rng.standard_normal(n).astype(np.float16)
+        outb = layer.forward(DeviceBuffer.from_numpy(x), bias=DeviceBuffer.from_numpy(bias)).numpy()
+        assert_close(outb, ref + bias.astype(np.float64)[None, :], "bias")
+        with pytest.raises(ops.KernelError, match="1D or 2D"):
+            layer.forward(DeviceBuffer.from_numpy(np.zeros((2, 3, k), np.float16)))
+        with pytest.raises(ops.KernelError, match="features mismatch"):
+            layer.forward(DeviceBuffer.from_numpy(np.zeros((2, k + 64), np.float16)))
+
+
+def test_async_stream_matches_sync(hip):
+    from rmlx_amd import ops
+    from rmlx_amd.runtime import DeviceBuffer, Stream
+    rng = np.random.default_rng(14)
+    n, k = 512, 1024
+    words, s, b = make_weight(rng, n, k, 4)
+    qw = ops.QuantizedWeight.from_numpy(words, s, b, 64, 4)
+    st = Stream()
+    for m in (1, 7, 96):
+        x = DeviceBuffer.from_numpy(make_x(rng, m, k))
+        sync = ops.affine_quantized_matmul_batched(x, qw).numpy()
+        out = ops.affine_quantized_matmul_batched(x, qw, stream=st)
+        st.sync()
+        assert np.array_equal(out.numpy(), sync)
+
+
+# ---- validation (reference error sites) -------------------------------------------------------------
+
+def test_validation_errors(hip):
+    from rmlx_amd import ops
+    from rmlx_amd.runtime import DeviceBuffer, U32
+    rng = np.random.default_rng(15)
+    n, k = 64, 512
+    words, s, b = make_weight(rng, n, k, 4)
+    wb, sb, bb = DeviceBuffer.from_numpy(words), DeviceBuffer.from_numpy(s), DeviceBuffer.from_numpy(b)
+    with pytest.raises(ops.KernelError, match="unsupported bit width 5"):
+        ops.QuantizedWeight(wb, sb, bb, 64, 5, n, k)
+    with pytest.raises(ops.KernelError, match="unsupported group_size 48"):
+        ops.QuantizedWeight(wb, sb, bb, 48, 4, n, k)
+    with pytest.raises(ops.KernelError, match="multiple of group_size"):
+        ops.QuantizedWeight(wb, sb, bb, 128, 4, n, k + 64)
+    with pytest.raises(ops.KernelError, match="weights_buf too small"):
+        ops.QuantizedWeight(wb, sb, bb, 64, 4, n * 2, k)
+    with pytest.raises(ops.KernelError, match="scales_buf too small"):
+        ops.QuantizedWeight(wb, DeviceBuffer.from_numpy(s[:10]), bb, 64, 4, n, k)
+    with pytest.raises(ops.KernelError, match="biases_buf too small"):
+        ops.QuantizedWeight(wb, sb, DeviceBuffer.from_numpy(b[:10]), 64, 4, n, k)
+    qw = ops.QuantizedWeight(wb, sb, bb, 64, 4, n, k)
+    with pytest.raises(ops.KernelError, match="requires 2D input"):
+        ops.affine_quantized_matmul_batched(DeviceBuffer.from_numpy(np.zeros(k, np.float16)), qw)
+    with pytest.raises(ops.KernelError, match=r"x.shape\[1\]"):
+        ops.affine_quantized_matmul_batched(DeviceBuffer.from_numpy(np.zeros((2, k * 2), np.float16)), qw)
+    with pytest.raises(ops.KernelError, match="Float16 or Float32"):
+        ops.affine_quantized_matmul_batched(DeviceBuffer((2, k), U32), qw)
+    with pytest.raises(ops.KernelError, match=r"vec.numel\(\)"):
+        ops.affine_quantized_matmul(qw, DeviceBuffer.from_numpy(np.zeros(k + 1, np.float16)))
+    e = None
+    try:
+        ops.affine_quantized_matmul_batched(DeviceBuffer.from_numpy(np.zeros((2, 3), np.float16)), qw)
+    except ops.KernelError as err:
+        e = err
+    assert e is not None and e.kind == "InvalidShape"
+    # M = 0 is legal and returns an empty result
+    out = ops.affine_quantized_matmul_batched(DeviceBuffer((0, k), 1), qw)
+    assert out.shape == (0, n)
