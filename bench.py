@@ -1,0 +1,224 @@
+#!/usr/bin/env python3
+"""Benchmark of the quantized-matmul hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--quick]
+
+Headline (`value`): Q4 qmv at M=1, K=N=4096 (group 64, f16) in GB/s of algorithmic bytes.  A step
+is one launch of the qmv kernel; weights are cycled over enough distinct sets (> 1 GiB) that
+every launch streams from HBM instead of the L2 / Infinity Cache.  All inputs are resident in
+HBM before the timed region.  The other benchmark configurations (qmv at N=9216, Q4 qmm at
+M=128/512, Q8 bf16 qmm, the MoE block) are timed the same way and reported under "extra".
+One JSON line is printed on stdout.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0      # MI355X HBM3E
+MFMA_F16_PEAK_TF = 2500.0  # dense f16 / bf16 MFMA
+
+
+def matmul_bytes(m, n, k, bits, gs=64, act_bytes=2):
+    """Algorithmic bytes of one quantized matmul: packed weights + f16 scales and biases +
+    activations in + f16 out."""
+    return n * k * bits // 8 + 2 * (n * k // gs) * 2 + m * k * act_bytes + m * n * 2
+
+
+def make_weight(rng, n, k, bits, lead=()):
+    lo, hi = (0.005, 0.02) if bits == 4 else (0.0005, 0.002)
+    words = rng.integers(0, 2**32, size=tuple(lead) + (n, k * bits // 32), dtype=np.uint32)
+    s = rng.uniform(lo, hi, size=tuple(lead) + (n, k // 64)).astype(np.float16)
+    b = (-(2.0 ** (bits - 1)) * s.astype(np.float32)).astype(np.float16)
+    return words, s, b
+
+
+class Timer:
+    """HIP events on the stream the kernels are launched on."""
+
+    def __init__(self, rt):
+        self.rt = rt
+        self.stream = rt.Stream()
+        self.e0, self.e1 = rt.Event(), rt.Event()
+
+    def run(self, fn, steps, warmup):
+        fn(warmup)
+        self.stream.sync()
+        self.e0.record(self.stream)
+        fn(steps)
+        self.e1.record(self.stream)
+        self.e1.sync()
+        self.stream.sync()
+        return self.e0.elapsed_ms(self.e1) / steps  # ms per step
+
+
+def bench_matmul(ops, rt, timer, rng, m, n, k, bits, x_dtype, steps, warmup, min_total_bytes, check=True):
+    from oracle import model
+    wbytes = n * k * bits // 8 + 4 * (n * k // 64)
+    n_sets = max(1, -(-min_total_bytes // wbytes))
+    base = make_weight(rng, n, k, bits)
+    qws = [ops.QuantizedWeight.from_numpy(*base, 64, bits)]
+    for i in range(1, n_sets):  # distinct buffers; contents rolled so that sets differ
+        qws.append(ops.QuantizedWeight.from_numpy(np.roll(base[0], i, axis=0), np.roll(base[1], i, axis=0),
+                                                  np.roll(base[2], i, axis=0), 64, bits))
+    xf = rng.standard_normal((m, k)).astype(np.float32)
+    if x_dtype == "bf16":
+        xh = model.f32_to_bf16_bits(xf)
+        xd = rt.DeviceBuffer.from_numpy(xh, rt.BF16)
+        x64 = model.bf16_bits_to_f32(xh).astype(np.float64)
+    else:
+        xh = xf.astype(np.float16)
+        xd = rt.DeviceBuffer.from_numpy(xh)
+        x64 = xh.astype(np.float64)
+    outs = [rt.DeviceBuffer((m, n), rt.F16) for _ in range(min(n_sets, 8))]
+    ms = timer.run(lambda c: ops.qmm_encode_many(qws, xd, outs, c, stream=timer.stream), steps, warmup)
+    res = {"us": ms * 1e3, "n_weight_sets": n_sets,
+           "bytes": matmul_bytes(m, n, k, bits, act_bytes=2), "flops": 2 * m * n * k}
+    res["gbs"] = res["bytes"] / (ms * 1e-3) / 1e9
+    res["tflops"] = res["flops"] / (ms * 1e-3) / 1e12
+    if check:  # parity of the timed configuration against the oracle, on weight set 0
+        ops.qmm_encode_many(qws[:1], xd, outs[:1], 1, stream=timer.stream)
+        timer.stream.sync()
+        ref = model.qmm(x64, *base, 64, bits)
+        err = float(np.abs(outs[0].numpy().astype(np.float64) - ref).max())
+        res["max_err"], res["tol"] = err, model.tolerance(ref)
+        res["pass"] = bool(err <= res["tol"])
+    return res
+
+
+def bench_moe(ops, rt, timer, rng, T, steps, warmup, experts):
+    from oracle import model
+    gate_up, down, gh, dh = experts
+    x = rng.standard_normal((T, 4096)).astype(np.float16)
+    logits = rng.standard_normal((T, 128)).astype(np.float32)
+    xd, ld = rt.DeviceBuffer.from_numpy(x), rt.DeviceBuffer.from_numpy(logits)
+    out = rt.DeviceBuffer((T, 4096), rt.F16)
+
+    def run(c):
+        for _ in range(c):
+            ops.moe_forward(gh, None, dh, xd, ld, 8, stream=timer.stream, out=out)
+
+    ms = timer.run(run, steps, warmup)
+    idx, w, _, _ = model.topk_route(logits, 8)
+    distinct = len(np.unique(idx))
+    nbytes = distinct * 10616832 + T * 4096 * 2 * 2 + T * 128 * 4
+    res = {"us": ms * 1e3, "distinct_experts": distinct, "bytes": nbytes, "gbs": nbytes / (ms * 1e-3) / 1e9,
+           "flops": 2 * 8 * T * (4096 * 3072 + 1536 * 4096)}
+    toks = np.arange(min(T, 2))
+    sel = (toks[:, None] * 8 + np.arange(8)[None, :]).reshape(-1)
+    gate = tuple(a[:, :1536] for a in gate_up)
+    up = tuple(a[:, 1536:] for a in gate_up)
+    ref = model.moe_forward(x[toks], idx[sel], w[sel], gate, up, down, 64, 8)
+    err = float(np.abs(out.numpy()[toks].astype(np.float64) - ref).max())
+    res["max_err"], res["tol"], res["pass"] = err, model.tolerance(ref), bool(err <= model.tolerance(ref))
+    return res
+
+
+def cpu_baseline(rng, budget_s=10.0):
+    """The C restatement of the reference's scalar `affine_qmm` (oracle/affine_qmm_ref.c) on the
+    headline configuration (M=1, K=N=4096), one host thread, repeated for about `budget_s`."""
+    from oracle import model, refpath
+    n = k = 4096
+    words, s, b = make_weight(rng, n, k, 4)
+    x = rng.standard_normal((1, k)).astype(np.float16).astype(np.float32)
+    wb, s32, b32 = model.words_to_bytes(words), s.astype(np.float32), b.astype(np.float32)
+    refpath.affine_qmm(x, wb, s32, b32, 1, n, k, 64)  # warm
+    reps, t0 = 0, time.perf_counter()
+    while True:
+        refpath.affine_qmm(x, wb, s32, b32, 1, n, k, 64)
+        reps += 1
+        el = time.perf_counter() - t0
+        if el >= budget_s:
+            break
+    per = el / reps
+    return {"value": matmul_bytes(1, n, k, 4) / per / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
+            "sample": f"{reps} repetitions of the full M=1 K=N=4096 Q4 matmul ({el:.1f} s, {per * 1e3:.2f} ms each)",
+            "us_per_matmul": per * 1e6, "host_cores_available": os.cpu_count()}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=2000)
+    ap.add_argument("--warmup", type=int, default=200)
+    ap.add_argument("--quick", action="store_true", help="headline configuration only, short CPU baseline")
+    ap.add_argument("--no-cpu", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)")
+
+    from rmlx_amd import ops, runtime as rt
+    rt.init(0)
+    info = rt.device_info()
+    timer = Timer(rt)
+    rng = np.random.default_rng(1001)
+    GiB = 1 << 30
+
+    # ---- headline: Q4 qmv M=1 K=N=4096, weights cycled through > 1 GiB ---------------------------------
+    head = bench_matmul(ops, rt, timer, rng, 1, 4096, 4096, 4, "f16", args.steps, args.warmup, GiB + GiB // 8)
+    extra = {"device": info, "q4_qmv_m1_4096": head}
+    if not args.quick:
+        small = max(20, args.steps // 20)
+        extra["q4_qmv_m1_4096_cache_resident"] = bench_matmul(ops, rt, timer, rng, 1, 4096, 4096, 4, "f16",
+                                                              args.steps, args.warmup, 0, check=False)
+        for m in (1, 4, 8):
+            extra[f"q4_qmv_m{m}_n9216"] = bench_matmul(ops, rt, timer, rng, m, 9216, 4096, 4, "f16", args.steps,
+                                                       args.warmup, GiB + GiB // 8, check=(m == 8))
+        for m in (128, 512):
+            r = bench_matmul(ops, rt, timer, rng, m, 4096, 4096, 4, "f16", small, 10, 4 * 9437184)
+            r["mfma_frac"] = r["tflops"] / MFMA_F16_PEAK_TF
+            extra[f"q4_qmm_m{m}_4096"] = r
+        r = bench_matmul(ops, rt, timer, rng, 128, 12288, 4096, 8, "bf16", small, 10, 4 * 53477376)
+        r["mfma_frac"] = r["tflops"] / MFMA_F16_PEAK_TF
+        r["hbm_frac"] = r["gbs"] / HBM_PEAK_GBS
+        extra["q8_qmm_bf16_m128_n12288"] = r
+        gate_up = make_weight(rng, 3072, 4096, 4, lead=(128,))
+        down = make_weight(rng, 4096, 1536, 4, lead=(128,))
+        experts = (gate_up, down, ops.QuantizedWeight.from_numpy(*gate_up, 64, 4),
+                   ops.QuantizedWeight.from_numpy(*down, 64, 4))
+        for T in (4, 32, 128):
+            r = bench_moe(ops, rt, timer, rng, T, max(10, small // 2), 5, experts)
+            r["hbm_frac"] = r["gbs"] / HBM_PEAK_GBS
+            extra[f"moe_q4_T{T}"] = r
+
+    line = {
+        "metric": "Q4 qmv HBM GB/s (M=1, K=N=4096)",
+        "value": head["gbs"],
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": head["us"] / 1e3,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f16",
+        "data": "synthetic",
+        "config": {"workload": "Q4 qmv M=1 K=4096 N=4096 group_size=64 f16 activations, "
+                               f"{head['n_weight_sets']} distinct weight sets cycled (HBM-resident, > 1 GiB)",
+                   "parity_max_err": head.get("max_err"), "parity_tol": head.get("tol")},
+        "roofline": {"bound": "hbm", "achieved": head["gbs"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": head["gbs"] / HBM_PEAK_GBS, "traffic": None,
+                     "kernel": "qmv_q4_kernel<1,1>", "bytes_per_launch": head["bytes"],
+                     "avg_launch_us": head["us"]},
+    }
+    if not args.quick and "q4_qmm_m512_4096" in extra:
+        q = extra["q4_qmm_m512_4096"]
+        line["secondary"] = {"metric": "Q4 qmm TFLOPS (M=512, K=N=4096)", "value": q["tflops"], "unit": "TFLOP/s",
+                             "roofline": {"bound": "mfma", "achieved": q["tflops"], "peak": MFMA_F16_PEAK_TF,
+                                          "unit": "TFLOP/s", "frac": q["mfma_frac"], "traffic": None,
+                                          "kernel": "qmm_kernel<128,64,4,false>", "avg_launch_us": q["us"]}}
+    if not args.no_cpu:
+        line["cpu_baseline"] = cpu_baseline(np.random.default_rng(1001), 3.0 if args.quick else 10.0)
+    line["extra"] = extra
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

@@ -128,6 +128,16 @@ int32_t rmlx_hip_affine_quantized_matmul_batched(const rmlx_qweight* qw, const r
 int32_t rmlx_hip_qmm_select(const rmlx_qweight* qw, const rmlx_array* x, int32_t kernel,
                             void* out_f16_dev, size_t out_bytes, rmlx_stream stream);
 
+/* Encode `count` batched matmuls back to back on `stream` with no synchronisation in between:
+ * the `_into_cb` usage of the reference, which encodes every QMM of a decoder stack into one
+ * command buffer (`affine_quantized_matmul_batched_into_cb`, quantized.rs:7797-7802;
+ * crates/rmlx-core/benches/qmm_pipeline_bench.rs:249-304).  Matmul i multiplies x by
+ * qws[i % n_qw] and writes outs[i % n_out] (each f16 [M, out_features], out_bytes long).
+ * All weights must have the same shape.  stream == NULL synchronises once at the end. */
+int32_t rmlx_hip_qmm_encode_many(const rmlx_qweight* const* qws, size_t n_qw, const rmlx_array* x,
+                                 void* const* outs_f16_dev, size_t n_out, size_t out_bytes,
+                                 size_t count, int32_t kernel, rmlx_stream stream);
+
 /* ---- `QuantizedLinear::forward` / `Linear::forward` call shape ------------------------------
  * (crates/rmlx-nn/src/quantized_linear.rs:153-201, crates/rmlx-nn/src/linear.rs:98-191)
  * x 1-D [in] is treated as [1,in]; 2-D [batch,in] -> [batch,out]; other ranks are rejected;

@@ -418,6 +418,32 @@ int32_t rmlx_hip_affine_quantized_matmul_batched(const rmlx_qweight* qw, const r
   return rmlx_hip_qmm_select(qw, x, KERNEL_AUTO, out_f16_dev, out_bytes, stream);
 }
 
+int32_t rmlx_hip_qmm_encode_many(const rmlx_qweight* const* qws, size_t n_qw, const rmlx_array* x,
+                                 void* const* outs_f16_dev, size_t n_out, size_t out_bytes, size_t count,
+                                 int32_t kernel, rmlx_stream stream) {
+  RMLX_TRY(require_init());
+  if (qws == nullptr || outs_f16_dev == nullptr || x == nullptr || n_qw == 0 || n_out == 0)
+    return fail(RMLX_INVALID_SHAPE, "qmm_encode_many: null or empty argument");
+  RMLX_TRY(check_x_dtype("affine_quantized_matmul_batched", x->dtype));
+  if (x->ndim != 2) return fail(RMLX_INVALID_SHAPE, "affine_quantized_matmul_batched requires 2D input x, got %dD", x->ndim);
+  for (size_t i = 0; i < n_qw; ++i) {
+    if (qws[i] == nullptr || qws[i]->n_experts != 1 || qws[i]->in_features != qws[0]->in_features ||
+        qws[i]->out_features != qws[0]->out_features)
+      return fail(RMLX_INVALID_SHAPE, "qmm_encode_many: weight %zu does not match weight 0", i);
+    if (qws[i]->bits != 4 && qws[i]->bits != 8)
+      return fail(RMLX_INVALID_SHAPE, "affine_quantized_matmul_batched requires bits==4 or bits==8, got %u", qws[i]->bits);
+  }
+  if (x->shape[1] != qws[0]->in_features)
+    return fail(RMLX_INVALID_SHAPE, "x.shape[1] (%zu) != in_features (%zu)", x->shape[1], qws[0]->in_features);
+  uint32_t M;
+  RMLX_TRY(checked_u32(x->shape[0], "M", &M));
+  RMLX_TRY(check_out("qmm_encode_many", out_bytes, (size_t)M * qws[0]->out_features * 2));
+  hipStream_t s = (hipStream_t)stream;
+  for (size_t i = 0; i < count; ++i)
+    RMLX_TRY(run_matmul(qws[i % n_qw], x->data, x->dtype, M, static_cast<__half*>(outs_f16_dev[i % n_out]), kernel, s));
+  return finish(s);
+}
+
 int32_t rmlx_hip_quantized_linear_forward(const rmlx_qweight* qw, const rmlx_array* x, const void* bias_f16_dev,
                                           void* out_f16_dev, size_t out_bytes, rmlx_stream stream) {
   RMLX_TRY(require_init());

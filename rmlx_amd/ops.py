@@ -69,6 +69,15 @@ def affine_quantized_matmul_batched(x, qw, stream=None, kernel=rt.KERNEL_AUTO, o
     return out
 
 
+def qmm_encode_many(qws, x, outs, count, stream=None, kernel=rt.KERNEL_AUTO):
+    """Encode `count` matmuls back to back (weights and outputs are cycled) -- see rmlx_hip_qmm_encode_many."""
+    qarr = (ctypes.c_void_p * len(qws))(*[q.handle for q in qws])
+    oarr = (ctypes.c_void_p * len(outs))(*[o.ptr for o in outs])
+    a = x.array()
+    rt.check(rt.lib().rmlx_hip_qmm_encode_many(qarr, len(qws), ctypes.byref(a), oarr, len(outs), outs[0].nbytes,
+                                               count, kernel, _h(stream)))
+
+
 class QuantizedLinear:
     """`QuantizedLinear` (crates/rmlx-nn/src/quantized_linear.rs:52-201) with the weights
     uploaded once at construction instead of on every forward."""

@@ -158,7 +158,13 @@ def test_group_sizes_and_odd_shapes_portable_kernel(hip, bits, gs):
     words, s, b = make_weight(rng, n, k, bits, gs)
     x = make_x(rng, m, k)
     ref = model.qmm(x_as_f64(x, "f16"), words, s, b, gs, bits)
-    assert_close(_run(hip, words, s, b, x, bits, gs=gs), ref, f"bits={bits} gs={gs}")
+    # the batched entry point only admits 4 and 8 bits (quantized.rs:7175); 2-bit goes to the portable kernel
+    kernel = 3 if bits == 2 else 0
+    assert_close(_run(hip, words, s, b, x, bits, gs=gs, kernel=kernel), ref, f"bits={bits} gs={gs}")
+    if bits == 2:
+        from rmlx_amd import ops
+        with pytest.raises(ops.KernelError, match="requires bits==4 or bits==8, got 2"):
+            _run(hip, words, s, b, x, bits, gs=gs)
 
 
 def test_qmv_entry_equals_batched_m1(hip):

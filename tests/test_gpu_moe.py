@@ -266,9 +266,14 @@ def test_moe_forward_small(hip, fused, T, E, K, D, I):
     ref = model.moe_forward(x, idx, w, gate, up, down, 64, K)
     out = ops.moe_forward(gh, uh, dh, DeviceBuffer.from_numpy(x), DeviceBuffer.from_numpy(logits), K).numpy()
     assert_close(out, ref, "moe_forward")
-    out2 = ops.moe_forward_grouped(gh, uh, dh, DeviceBuffer.from_numpy(x), DeviceBuffer.from_numpy(idx),
-                                   DeviceBuffer.from_numpy(w), K).numpy()
+    # routing on the device followed by the grouped block == the one-call entry point, bit for bit
+    r = ops.gpu_topk_route(DeviceBuffer.from_numpy(logits), K)
+    assert np.array_equal(r.expert_indices.numpy(), idx)
+    out2 = ops.moe_forward_grouped(gh, uh, dh, DeviceBuffer.from_numpy(x), r.expert_indices, r.expert_weights, K).numpy()
     assert np.array_equal(out, out2)
+    out3 = ops.moe_forward_grouped(gh, uh, dh, DeviceBuffer.from_numpy(x), DeviceBuffer.from_numpy(idx),
+                                   DeviceBuffer.from_numpy(w), K).numpy()
+    assert_close(out3, ref, "moe_forward_grouped with host routing")
 
 
 def test_grouped_forward_equals_per_expert_loop(hip):
