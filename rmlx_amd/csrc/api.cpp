@@ -185,7 +185,7 @@ int32_t check_expert_weights(const char* who, const rmlx_qweight* gate, const rm
 
 // gate/up + SwiGLU then down, over a device chunk table.  h: f16 [positions, I] scratch.
 int32_t run_expert_ffn(const rmlx_qweight* gate, const rmlx_qweight* up, const rmlx_qweight* down,
-                       const ExpertShapes& sh, const __half* x, const uint32_t* row_map, uint32_t row_div,
+                       const ExpertShapes& sh, const __half* x, const uint32_t* row_map,
                        const uint32_t* chunk_tab, const uint32_t* n_chunks, uint32_t max_chunks, __half* h,
                        void* y, int y_f32, hipStream_t stream) {
   QmvArgs a{};
@@ -201,7 +201,7 @@ int32_t run_expert_ffn(const rmlx_qweight* gate, const rmlx_qweight* up, const r
   a.N = sh.I; a.K = sh.D;
   a.expert_stride_w = rows_per_expert * (sh.D / 8);
   a.expert_stride_s = rows_per_expert * (sh.D / 64);
-  a.x = x; a.row_map = row_map; a.row_div = row_div;
+  a.x = x; a.row_map = row_map;
   a.out = h; a.ld_out = sh.I; a.out_f32 = 0; a.dual = 1;
   a.chunk_tab = chunk_tab; a.n_chunks_dev = n_chunks; a.max_chunks = max_chunks; a.mr = 8;
   RMLX_TRY(launch_qmv_q4(a, stream));
@@ -211,7 +211,7 @@ int32_t run_expert_ffn(const rmlx_qweight* gate, const rmlx_qweight* up, const r
   d.N = sh.D; d.K = sh.I;
   d.expert_stride_w = (size_t)sh.D * (sh.I / 8);
   d.expert_stride_s = (size_t)sh.D * (sh.I / 64);
-  d.x = h; d.row_map = nullptr; d.row_div = 1;
+  d.x = h; d.row_map = nullptr;
   d.out = y; d.ld_out = sh.D; d.out_f32 = y_f32; d.dual = 0;
   d.chunk_tab = chunk_tab; d.n_chunks_dev = n_chunks; d.max_chunks = max_chunks; d.mr = 8;
   return launch_qmv_q4(d, stream);
@@ -623,7 +623,7 @@ int32_t rmlx_hip_moe_sort(const uint32_t* expert_indices_dev, size_t n_assign, s
   RMLX_TRY(checked_u32(n_experts, "n_experts", &E));
   if (E == 0) return fail(RMLX_INVALID_SHAPE, "moe_sort: n_experts must be non-zero");
   hipStream_t s = (hipStream_t)stream;
-  RMLX_TRY(launch_moe_sort(expert_indices_dev, A, E, sorted_assign_dev, nullptr, nullptr, offsets_dev, nullptr, nullptr, s));
+  RMLX_TRY(launch_moe_sort(expert_indices_dev, A, E, 1, sorted_assign_dev, nullptr, nullptr, nullptr, offsets_dev, nullptr, nullptr, s));
   return finish(s);
 }
 
@@ -712,7 +712,7 @@ int32_t rmlx_hip_expert_group_grouped_forward(const rmlx_qweight* gate, const rm
   RMLX_HIP_CHECK(hipMemcpyAsync(dtab.ptr, tab.data(), tab.size() * 4, hipMemcpyHostToDevice, s));
   RMLX_HIP_CHECK(hipStreamSynchronize(s));  // `tab` is pageable host memory owned by this call
   RMLX_TRY(h.alloc(total * sh.I * 2, s));
-  RMLX_TRY(run_expert_ffn(gate, up, down, sh, xk, nullptr, 1, static_cast<const uint32_t*>(dtab.ptr), nullptr, n_chunks,
+  RMLX_TRY(run_expert_ffn(gate, up, down, sh, xk, nullptr, static_cast<const uint32_t*>(dtab.ptr), nullptr, n_chunks,
                           static_cast<__half*>(h.ptr), out_f16_dev, 0, s));
   return finish(s);
 }
@@ -748,16 +748,17 @@ int32_t rmlx_hip_moe_forward_grouped(const rmlx_qweight* gate, const rmlx_qweigh
     xk = static_cast<const __half*>(cast.ptr);
   }
   if (!aligned16(xk)) return fail(RMLX_INVALID_SHAPE, "MoeLayer: input must be 16-byte aligned");
-  // meta: sorted[A] | inv[A] | chunk_tab[3*max_chunks] | n_chunks[1]
-  RMLX_TRY(meta.alloc(((size_t)2 * A + 3 * (size_t)max_chunks + 4) * 4, s));
+  // meta: sorted[A] | sorted_tok[A] | inv[A] | chunk_tab[3*max_chunks] | n_chunks[1]
+  RMLX_TRY(meta.alloc(((size_t)3 * A + 3 * (size_t)max_chunks + 4) * 4, s));
   uint32_t* sorted = static_cast<uint32_t*>(meta.ptr);
-  uint32_t* inv = sorted + A;
+  uint32_t* sorted_tok = sorted + A;
+  uint32_t* inv = sorted_tok + A;
   uint32_t* chunk_tab = inv + A;
   uint32_t* n_chunks = chunk_tab + 3 * (size_t)max_chunks;
-  RMLX_TRY(launch_moe_sort(expert_indices_dev, A, sh.E, sorted, inv, nullptr, nullptr, chunk_tab, n_chunks, s));
+  RMLX_TRY(launch_moe_sort(expert_indices_dev, A, sh.E, (uint32_t)top_k, sorted, sorted_tok, inv, nullptr, nullptr, chunk_tab, n_chunks, s));
   RMLX_TRY(h.alloc((size_t)A * sh.I * 2, s));
   RMLX_TRY(y.alloc((size_t)A * sh.D * 4, s));
-  RMLX_TRY(run_expert_ffn(gate, up, down, sh, xk, sorted, (uint32_t)top_k, chunk_tab, n_chunks, max_chunks,
+  RMLX_TRY(run_expert_ffn(gate, up, down, sh, xk, sorted_tok, chunk_tab, n_chunks, max_chunks,
                           static_cast<__half*>(h.ptr), y.ptr, 1, s));
   RMLX_TRY(launch_moe_combine(static_cast<const float*>(y.ptr), inv, expert_weights_dev, T32, (uint32_t)top_k, sh.D,
                               static_cast<__half*>(out_f16_dev), s));

@@ -112,8 +112,7 @@ struct QmvArgs {
   uint64_t expert_stride_w;  // u32 words per expert
   uint64_t expert_stride_s;  // halves per expert
   const __half* x;           // [x_rows, K] f16
-  const uint32_t* row_map;   // nullable: source row of position p is row_map[p] / row_div
-  uint32_t row_div;
+  const uint32_t* row_map;   // nullable: source row of position p is row_map[p]
   void* out;                 // f16 [positions, ld_out] (f32 when out_f32)
   uint32_t ld_out;
   int out_f32;
@@ -146,9 +145,10 @@ int32_t launch_topk_route(const float* logits, const float* bias, uint32_t T, ui
                           hipStream_t s);
 // Stable counting sort; also emits the chunk table used by the GEMV family
 // (chunk_tab: 3 u32 per chunk; n_chunks: 1 u32).  chunk_tab / n_chunks may be null.
-int32_t launch_moe_sort(const uint32_t* idx, uint32_t n_assign, uint32_t E, uint32_t* sorted, uint32_t* inv,
-                        uint32_t* counts, uint32_t* offsets, uint32_t* chunk_tab, uint32_t* n_chunks,
-                        hipStream_t s);
+// sorted_tok (nullable): token of each sorted position, sorted[p] / top_k.
+int32_t launch_moe_sort(const uint32_t* idx, uint32_t n_assign, uint32_t E, uint32_t top_k, uint32_t* sorted,
+                        uint32_t* sorted_tok, uint32_t* inv, uint32_t* counts, uint32_t* offsets,
+                        uint32_t* chunk_tab, uint32_t* n_chunks, hipStream_t s);
 int32_t launch_index_gather(const __half* src, uint32_t d, const uint32_t* idx, uint32_t n, uint32_t src_rows,
                             __half* dst, hipStream_t s);
 int32_t launch_scatter_weighted_add(const __half* src, uint32_t n, uint32_t d, const uint32_t* tok,

@@ -91,7 +91,8 @@ __global__ __launch_bounds__(64) void topk_route_kernel(const float* __restrict_
 // Deterministic by construction: thread e owns expert e and walks each block of 1024
 // assignments in ascending order, so ids of one expert keep their original order.
 __global__ __launch_bounds__(1024) void moe_sort_kernel(const uint32_t* __restrict__ idx, uint32_t n_assign,
-                                                        uint32_t E, uint32_t* __restrict__ sorted,
+                                                        uint32_t E, uint32_t top_k, uint32_t* __restrict__ sorted,
+                                                        uint32_t* __restrict__ sorted_tok,
                                                         uint32_t* __restrict__ inv, uint32_t* __restrict__ counts,
                                                         uint32_t* __restrict__ offsets,
                                                         uint32_t* __restrict__ chunk_tab,
@@ -145,6 +146,7 @@ __global__ __launch_bounds__(1024) void moe_sort_kernel(const uint32_t* __restri
     __syncthreads();
     if (tid < nb && ids[tid] < E) {
       sorted[pos[tid]] = base + tid;
+      if (sorted_tok != nullptr) sorted_tok[pos[tid]] = (base + tid) / top_k;
       if (inv != nullptr) inv[base + tid] = pos[tid];
     }
   }
@@ -211,20 +213,21 @@ int32_t launch_topk_route(const float* logits, const float* bias, uint32_t T, ui
     RMLX_HIP_CHECK(hipGetLastError());
   }
   if (counts != nullptr || offsets != nullptr) {
-    hipLaunchKernelGGL(moe_sort_kernel, dim3(1), dim3(1024), 0, s, idx, T * K, E, (uint32_t*)nullptr,
-                       (uint32_t*)nullptr, counts, offsets, (uint32_t*)nullptr, (uint32_t*)nullptr);
+    hipLaunchKernelGGL(moe_sort_kernel, dim3(1), dim3(1024), 0, s, idx, T * K, E, K, (uint32_t*)nullptr,
+                       (uint32_t*)nullptr, (uint32_t*)nullptr, counts, offsets, (uint32_t*)nullptr,
+                       (uint32_t*)nullptr);
     RMLX_HIP_CHECK(hipGetLastError());
   }
   return RMLX_OK;
 }
 
-int32_t launch_moe_sort(const uint32_t* idx, uint32_t n_assign, uint32_t E, uint32_t* sorted, uint32_t* inv,
-                        uint32_t* counts, uint32_t* offsets, uint32_t* chunk_tab, uint32_t* n_chunks,
-                        hipStream_t s) {
+int32_t launch_moe_sort(const uint32_t* idx, uint32_t n_assign, uint32_t E, uint32_t top_k, uint32_t* sorted,
+                        uint32_t* sorted_tok, uint32_t* inv, uint32_t* counts, uint32_t* offsets,
+                        uint32_t* chunk_tab, uint32_t* n_chunks, hipStream_t s) {
   if (E > (uint32_t)kMaxExperts)
     return fail(RMLX_INVALID_SHAPE, "moe_sort: n_experts (%u) exceeds maximum %d", E, kMaxExperts);
-  hipLaunchKernelGGL(moe_sort_kernel, dim3(1), dim3(1024), 0, s, idx, n_assign, E, sorted, inv, counts, offsets,
-                     chunk_tab, n_chunks);
+  hipLaunchKernelGGL(moe_sort_kernel, dim3(1), dim3(1024), 0, s, idx, n_assign, E, top_k ? top_k : 1u, sorted,
+                     sorted_tok, inv, counts, offsets, chunk_tab, n_chunks);
   RMLX_HIP_CHECK(hipGetLastError());
   return RMLX_OK;
 }

@@ -5,8 +5,8 @@
 // gather_qmv_fast_f16_q4 (crates/rmlx-core/src/ops/quantized.rs:798-979, 9752-9842).
 //
 // Design (wave64, MFMA):
-//   * One workgroup = 4 waves = one tile of 16 weight rows; the K range is split across the
-//     4 waves.  Every lane issues all of its 128-bit weight loads before anything else, so a
+//   * One workgroup = 8 waves = one tile of 16 weight rows; the K range is split across the
+//     8 waves.  Every lane issues all of its 128-bit weight loads before anything else, so a
 //     whole [16 x 4096] tile (32 KB) is in flight per workgroup.
 //   * A "slab" is 16 rows x 128 k.  Lane (n = lane%16, g = lane/16) loads the 16 bytes holding
 //     k in [32g, 32g+32) of row n; its four u32 words feed four v_mfma_f32_16x16x32_f16
@@ -21,8 +21,9 @@
 //     rows 8-15 the same x restricted to the second group (the other half of the A operand is
 //     zero), so one accumulator tile yields both per-group integer dot products.  Each is then
 //     folded into the f32 result with  acc += scale * dot + bias * xsum.
-//   * The per-(row, group) sums  sum(x)  and  sum(off*x)  come from the same MFMA with a
-//     constant B operand, computed while the weight loads are in flight.
+//   * The per-(row, group) sums  sum(x)  and  sum(off*x)  are formed by the threads that stage x
+//     (8 consecutive threads hold one group) and parked in LDS; all of the x-side work happens
+//     while the weight loads are in flight.
 #include "common.hpp"
 
 namespace rmlx {
@@ -32,24 +33,42 @@ typedef _Float16 h8 __attribute__((ext_vector_type(8)));
 typedef float f4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u4 __attribute__((ext_vector_type(4)));
 
-constexpr int kThreads = 256;
-constexpr int kWaves = 4;
+constexpr int kThreads = 512;
+constexpr int kWaves = 8;
 constexpr int kChunkSlabs = 32;  // slabs of 128 k staged per pass (4096 k)
-constexpr int kSpwMax = 8;       // slabs per wave per pass
+constexpr int kSpwMax = 4;       // slabs per wave per pass
 constexpr int kSbStride = 65;    // dwords per row of the scale/bias image (64 groups + pad)
 
+// Field order matters: the first 16 dwords are preloaded into SGPRs at wave launch
+// (-amdgpu-kernarg-preload-count), so everything the plain qmv path needs comes first.
 struct KParams {
-  const uint32_t* w[2];
-  const __half* s[2];
-  const __half* b[2];
+  const uint32_t* w0;
+  const __half* s0;
+  const __half* b0;
   const __half* x;
+  void* out;
+  uint32_t K, ld_out, M, out_f32;
+  const uint32_t* w1;
+  const __half* s1;
+  const __half* b1;
   const uint32_t* row_map;
   const uint32_t* chunk_tab;
   const uint32_t* n_chunks;
-  void* out;
   uint64_t estride_w, estride_s;
-  uint32_t K, row_div, ld_out, M, out_f32;
+#ifdef QMV_TRACE
+  unsigned long long* trace;  // development only: per-phase shader clock of workgroup 0 / each wave
+#endif
 };
+
+#ifdef QMV_TRACE
+#define QMV_MARK(p, i)                                                                   \
+  do {                                                                                   \
+    if ((p).trace != nullptr && blockIdx.x == 0 && blockIdx.y == 0 && (threadIdx.x & 63) == 0) \
+      (p).trace[(threadIdx.x >> 6) * 16 + (i)] = __builtin_readcyclecounter();           \
+  } while (0)
+#else
+#define QMV_MARK(p, i) do {} while (0)
+#endif
 
 __device__ __forceinline__ h8 unpack_q4_word(uint32_t w) {
   uint32_t t = w >> 8;
@@ -73,8 +92,198 @@ __device__ __forceinline__ u4 permute_x8(u4 d) {
 
 __device__ __forceinline__ float silu_f(float v) { return v / (1.0f + __expf(-v)); }
 
+__device__ __forceinline__ uint32_t swap16(uint32_t v) {  // value of lane ^ 16
+  return (uint32_t)__builtin_amdgcn_ds_swizzle((int)v, 0x401F);
+}
+
+// One pass over up to 4096 k.
+// FULLP: every wave owns exactly kSpwMax slabs.  Then the k range a wave consumes (512 k) is
+// exactly the range its own 64 threads stage, so the activation image and the sums are
+// wave-private and the pass needs no workgroup barrier; scales and biases come straight from
+// global memory (8 consecutive groups = one aligned 16-byte load per lane, scales in the lanes
+// with even g, biases in the lanes with odd g, exchanged with one swizzle per word).
+// !FULLP (K not a multiple of 4096): slabs are dealt to the waves evenly, everything is
+// staged through LDS for the whole workgroup with barriers.
+template <int MR, int TILES, bool TAB, bool FULLP>
+__device__ __forceinline__ void qmv_pass(const KParams& p, char* xs, float* sums, uint32_t* sbs,
+                                         const u4* const (&wrow)[TILES], f4 (&F)[TILES], uint32_t kc, int nsl,
+                                         uint32_t expert, uint32_t row0, uint32_t rows, uint32_t tile_row,
+                                         bool first_pass) {
+  constexpr int kSlots = 4 * MR;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int n = lane & 15, g = lane >> 4, par = g >> 1;
+  const uint32_t K = p.K, groups_per_row = K >> 6;
+  const int spw = (nsl + kWaves - 1) / kWaves;
+  const int s0 = wave * spw;
+  int my = nsl - s0;
+  my = my < 0 ? 0 : (my > spw ? spw : my);
+
+  // ---- 1. issue every global load of this pass up front.  The few activation / scale loads go
+  //         first: the memory counter retires in order, so they can then be consumed while the
+  //         weight loads (the bulk of the traffic) are still in flight. -----------------------
+  constexpr int kXU = MR;  // 16-byte activation units per thread (kChunkSlabs*16*MR / kThreads)
+  static_assert(kChunkSlabs * 16 == kThreads, "one activation unit per thread and row");
+  const int ngr = nsl * 2;  // quantisation groups in this pass
+  u4 xv[kXU];
+  {
+    uint32_t srcs[kXU];
+#pragma unroll
+    for (int m = 0; m < kXU; ++m) {
+      srcs[m] = row0 + m;
+      if (TAB && p.row_map != nullptr && (uint32_t)m < rows) srcs[m] = p.row_map[row0 + m];  // wave-uniform
+    }
+#pragma unroll
+    for (int m = 0; m < kXU; ++m) {
+      xv[m] = (u4){0u, 0u, 0u, 0u};
+      if ((uint32_t)m < rows && tid < nsl * 16)
+        xv[m] = *reinterpret_cast<const u4*>(p.x + (uint64_t)srcs[m] * K + kc + tid * 8);
+    }
+  }
+  u4 sbv[TILES];
+  const int st = tid / 128, sr = (tid % 128) / 8, sc8 = tid % 8;  // tile, row, 8-group block
+  const bool s_active = !FULLP && tid < TILES * 128 && sc8 * 8 < ngr;
+  u4 sv0 = (u4){0u, 0u, 0u, 0u}, bv0 = (u4){0u, 0u, 0u, 0u};
+  if (FULLP) {
+#pragma unroll
+    for (int t = 0; t < TILES; ++t) {
+      const uint64_t off = (TAB ? expert * p.estride_s : 0) + (uint64_t)(tile_row + n) * groups_per_row + (kc >> 6) + s0 * 2;
+      const __half* sp_ = t == 0 ? p.s0 : p.s1;
+      const __half* bp_ = t == 0 ? p.b0 : p.b1;
+      sbv[t] = *reinterpret_cast<const u4*>(((g & 1) ? bp_ : sp_) + off);
+    }
+  } else if (s_active) {
+    const uint64_t off = (TAB ? expert * p.estride_s : 0) + (uint64_t)(tile_row + sr) * groups_per_row + (kc >> 6) + sc8 * 8;
+    sv0 = *reinterpret_cast<const u4*>((st == 0 ? p.s0 : p.s1) + off);
+    bv0 = *reinterpret_cast<const u4*>((st == 0 ? p.b0 : p.b1) + off);
+  }
+  // every wave has queued its small loads before any wave queues the bulk loads
+  if (FULLP) __builtin_amdgcn_s_barrier();
+  u4 wreg[TILES][kSpwMax];
+#pragma unroll
+  for (int it = 0; it < kSpwMax; ++it) {
+    if (FULLP || it < my) {
+#pragma unroll
+      for (int t = 0; t < TILES; ++t) wreg[t][it] = *(wrow[t] + (kc >> 5) + (s0 + it) * 4);
+    }
+  }
+  QMV_MARK(p, 1);
+
+  if (!FULLP && !first_pass) __syncthreads();  // previous pass finished reading xs / sums / sbs
+
+  // ---- 2. activations -> LDS in operand order; per-(row, group) sums -> LDS -------------------
+  if (!FULLP && s_active) {
+    uint32_t* dst = sbs + (st * 16 + sr) * kSbStride + sc8 * 8;
+    const uint32_t sw[4] = {sv0.x, sv0.y, sv0.z, sv0.w}, bw[4] = {bv0.x, bv0.y, bv0.z, bv0.w};
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      dst[2 * q] = (sw[q] & 0xFFFFu) | (bw[q] << 16);
+      dst[2 * q + 1] = (sw[q] >> 16) | (bw[q] & 0xFFFF0000u);
+    }
+  }
+  {
+    const int c = tid, slab = c >> 4, gg = (c >> 2) & 3, j = c & 3;
+#pragma unroll
+    for (int m = 0; m < kXU; ++m) {
+      if (c < nsl * 16)
+        *reinterpret_cast<u4*>(xs + ((slab * 4 + j) * kSlots + gg * MR + m) * 16) = permute_x8(xv[m]);
+      // this thread's 8 activations: plain sum and sum weighted by the unpack offsets
+      // (even k -> 1024, odd k -> 64); 8 consecutive threads make up one group of 64
+      const h8 hv = __builtin_bit_cast(h8, xv[m]);
+      float xs8 = 0.f, xo8 = 0.f;
+#pragma unroll
+      for (int e = 0; e < 8; e += 2) {
+        xs8 += (float)hv[e] + (float)hv[e + 1];
+        xo8 += 1024.0f * (float)hv[e] + 64.0f * (float)hv[e + 1];
+      }
+#pragma unroll
+      for (int off = 1; off < 8; off <<= 1) {
+        xs8 += __shfl_xor(xs8, off, 64);
+        xo8 += __shfl_xor(xo8, off, 64);
+      }
+      if ((c & 7) == 0) {  // sums[group][m] = (-sum(off*x), sum(x)); rows >= MR stay unused
+        sums[((c >> 3) * 8 + m) * 2 + 0] = -xo8;
+        sums[((c >> 3) * 8 + m) * 2 + 1] = xs8;
+      }
+    }
+  }
+  QMV_MARK(p, 2);
+  if (!FULLP) __syncthreads();
+  QMV_MARK(p, 3);
+
+  // ---- 3. weights: integer dot per group via MFMA, independent slabs interleaved -------------
+  // A-operand activity: accumulator rows 0-7 take group 0 (g<2), rows 8-15 group 1 (g>=2).
+  const int am = n & 7;
+  const bool a_active = ((n < 8) == (g < 2)) && (am < MR);
+  const int a_slot_off = (g * MR + am) * 16;
+  f4 c[TILES][kSpwMax];
+#pragma unroll
+  for (int it = 0; it < kSpwMax; ++it)
+#pragma unroll
+    for (int t = 0; t < TILES; ++t) c[t][it] = (f4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    h8 av[kSpwMax];
+#pragma unroll
+    for (int it = 0; it < kSpwMax; ++it) {
+      av[it] = (h8){0, 0, 0, 0, 0, 0, 0, 0};
+      if ((FULLP || it < my) && a_active)
+        av[it] = *reinterpret_cast<const h8*>(xs + (((s0 + it) * 4 + j) * kSlots) * 16 + a_slot_off);
+    }
+#pragma unroll
+    for (int it = 0; it < kSpwMax; ++it) {
+      if (FULLP || it < my) {
+#pragma unroll
+        for (int t = 0; t < TILES; ++t) {
+          const uint32_t wd = j == 0 ? wreg[t][it].x : (j == 1 ? wreg[t][it].y : (j == 2 ? wreg[t][it].z : wreg[t][it].w));
+          c[t][it] = __builtin_amdgcn_mfma_f32_16x16x32_f16(av[it], unpack_q4_word(wd), c[t][it], 0, 0, 0);
+        }
+      }
+    }
+  }
+  QMV_MARK(p, 4);
+
+  // ---- 4. acc += scale * (dot - sum(off*x)) + bias * sum(x), f32 -------------------------------
+  u4 sv[TILES], bv[TILES];
+  if (FULLP) {
+#pragma unroll
+    for (int t = 0; t < TILES; ++t) {
+      const u4 other = (u4){swap16(sbv[t].x), swap16(sbv[t].y), swap16(sbv[t].z), swap16(sbv[t].w)};
+      sv[t] = (g & 1) ? other : sbv[t];
+      bv[t] = (g & 1) ? sbv[t] : other;
+    }
+  }
+#pragma unroll
+  for (int it = 0; it < kSpwMax; ++it) {
+    if (FULLP || it < my) {
+      const float* sp = sums + (((s0 + it) * 2 + par) * 8 + (g & 1) * 4) * 2;
+      const f4 c01 = *reinterpret_cast<const f4*>(sp);      // (-xoff, xsum) of accumulator rows 4g, 4g+1
+      const f4 c23 = *reinterpret_cast<const f4*>(sp + 4);  // rows 4g+2, 4g+3
+#pragma unroll
+      for (int t = 0; t < TILES; ++t) {
+        uint32_t sbits, bbits;
+        if (FULLP) {  // group 2*it + par of the 8 loaded ones: word `it`, half `par`
+          const uint32_t swd = it == 0 ? sv[t].x : (it == 1 ? sv[t].y : (it == 2 ? sv[t].z : sv[t].w));
+          const uint32_t bwd = it == 0 ? bv[t].x : (it == 1 ? bv[t].y : (it == 2 ? bv[t].z : bv[t].w));
+          sbits = par ? swd >> 16 : swd & 0xFFFFu;
+          bbits = par ? bwd >> 16 : bwd & 0xFFFFu;
+        } else {
+          const uint32_t sb = sbs[(t * 16 + n) * kSbStride + (s0 + it) * 2 + par];
+          sbits = sb & 0xFFFFu;
+          bbits = sb >> 16;
+        }
+        const float sc = __half2float(__ushort_as_half((unsigned short)sbits));
+        const float bi = __half2float(__ushort_as_half((unsigned short)bbits));
+        F[t][0] += sc * (c[t][it][0] + c01[0]) + bi * c01[1];
+        F[t][1] += sc * (c[t][it][1] + c01[2]) + bi * c01[3];
+        F[t][2] += sc * (c[t][it][2] + c23[0]) + bi * c23[1];
+        F[t][3] += sc * (c[t][it][3] + c23[2]) + bi * c23[3];
+      }
+    }
+  }
+}
+
 // MR = activation rows staged per pass (1, 2, 4 or 8); TILES = 1, or 2 for fused gate/up.
-template <int MR, int TILES>
+template <int MR, int TILES, bool TAB>
 __global__ __launch_bounds__(kThreads) void qmv_q4_kernel(KParams p) {
   constexpr int kSlots = 4 * MR;                              // 16-byte slots per (slab, j)
   constexpr int kXsBytes = kChunkSlabs * 4 * kSlots * 16;     // activation image
@@ -82,19 +291,18 @@ __global__ __launch_bounds__(kThreads) void qmv_q4_kernel(KParams p) {
   constexpr int kXsAlloc = kXsBytes > kRedBytes ? kXsBytes : kRedBytes;
   __shared__ __attribute__((aligned(16))) char xs[kXsAlloc];
   __shared__ uint32_t sbs[TILES * 16 * kSbStride];
-  __shared__ __attribute__((aligned(16))) float corr[kWaves * kSpwMax * 4 * 4 * 2];
+  __shared__ __attribute__((aligned(16))) float sums[kChunkSlabs * 2 * 8 * 2];  // [group][row 0..7][-xoff, xsum]
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;
   const int n = lane & 15;   // weight row within the tile / accumulator column
   const int g = lane >> 4;   // k sub-block of the slab / accumulator row group
-  const int par = g >> 1;    // which of the slab's two quantisation groups this lane scales
 
   // ---- which rows -----------------------------------------------------------------------
   uint32_t expert = 0, row0 = blockIdx.y * 8, rows;
   bool write_zeros = false;
-  if (p.chunk_tab != nullptr) {
+  if (TAB) {
     if (p.n_chunks != nullptr && blockIdx.y >= *p.n_chunks) return;
     expert = p.chunk_tab[3 * blockIdx.y + 0];
     row0 = p.chunk_tab[3 * blockIdx.y + 1];
@@ -108,148 +316,38 @@ __global__ __launch_bounds__(kThreads) void qmv_q4_kernel(KParams p) {
 
   const uint32_t K = p.K;
   const uint32_t words_per_row = K >> 3;
-  const uint32_t groups_per_row = K >> 6;
   const uint32_t tile_row = blockIdx.x * 16;
 
   const u4* wrow[TILES];
 #pragma unroll
   for (int t = 0; t < TILES; ++t)
-    wrow[t] = reinterpret_cast<const u4*>(p.w[t] + expert * p.estride_w +
+    wrow[t] = reinterpret_cast<const u4*>((t == 0 ? p.w0 : p.w1) + (TAB ? expert * p.estride_w : 0) +
                                           (uint64_t)(tile_row + n) * words_per_row) + g;
-
-  // A-operand activity: accumulator rows 0-7 take group 0 (g<2), rows 8-15 group 1 (g>=2).
-  const int mslot = n;
-  const int am = mslot & 7;
-  const bool a_active = ((mslot < 8) == (g < 2)) && (am < MR);
-  const int a_slot_off = (g * MR + am) * 16;
-
-  // constant B operand for the x-side sums: column 0 = offsets, column 1 = ones
-  h8 bconst;
-  {
-    const _Float16 o0 = (_Float16)1024.0f, o1 = (_Float16)64.0f, one = (_Float16)1.0f, z = (_Float16)0.0f;
-    h8 offs = {o0, o0, o1, o1, o0, o0, o1, o1};
-    h8 ones = {one, one, one, one, one, one, one, one};
-    h8 zero = {z, z, z, z, z, z, z, z};
-    bconst = n == 0 ? offs : (n == 1 ? ones : zero);
-  }
 
   f4 F[TILES];
 #pragma unroll
   for (int t = 0; t < TILES; ++t) F[t] = (f4){0.f, 0.f, 0.f, 0.f};
+  QMV_MARK(p, 0);
 
   for (uint32_t kc = 0; kc < K; kc += kChunkSlabs * 128) {
-    const int nsl = (K - kc) / 128 < (uint32_t)kChunkSlabs ? (int)((K - kc) / 128) : kChunkSlabs;
-    const int spw = (nsl + kWaves - 1) / kWaves;
-    const int s0 = wave * spw;
-    int my = nsl - s0;
-    my = my < 0 ? 0 : (my > spw ? spw : my);
-
-    // ---- 1. all weight loads of this pass, before anything else ----------------------------
-    u4 wreg[TILES][kSpwMax];
-#pragma unroll
-    for (int it = 0; it < kSpwMax; ++it) {
-      if (it < my) {
-#pragma unroll
-        for (int t = 0; t < TILES; ++t)
-          wreg[t][it] = __builtin_nontemporal_load(wrow[t] + (kc >> 5) + (s0 + it) * 4);
-      }
-    }
-
-    if (kc != 0) __syncthreads();  // previous pass finished reading xs / sbs
-
-    // ---- 2. stage scales+biases (as half2 pairs) and the permuted activations ---------------
-    {
-      const int ngr = nsl * 2;  // groups in this pass
-      for (int u = tid; u < TILES * 16 * 8; u += kThreads) {
-        const int t = u / 128, r = (u % 128) / 8, c8 = u % 8;  // 8 groups per 16 B
-        if (c8 * 8 < ngr) {
-          const uint64_t off = expert * p.estride_s + (uint64_t)(tile_row + r) * groups_per_row + (kc >> 6) + c8 * 8;
-          const u4 sv = *reinterpret_cast<const u4*>(p.s[t] + off);
-          const u4 bv = *reinterpret_cast<const u4*>(p.b[t] + off);
-          uint32_t* dst = sbs + (t * 16 + r) * kSbStride + c8 * 8;
-          const uint32_t sw[4] = {sv.x, sv.y, sv.z, sv.w}, bw[4] = {bv.x, bv.y, bv.z, bv.w};
-#pragma unroll
-          for (int q = 0; q < 4; ++q) {
-            dst[2 * q] = (sw[q] & 0xFFFFu) | (bw[q] << 16);
-            dst[2 * q + 1] = (sw[q] >> 16) | (bw[q] & 0xFFFF0000u);
-          }
-        }
-      }
-      const int units = nsl * 16 * MR;  // 16-byte units (8 halves) of this pass
-      for (int u = tid; u < units; u += kThreads) {
-        const int m = u % MR, c = u / MR;
-        u4 v = (u4){0u, 0u, 0u, 0u};
-        if ((uint32_t)m < rows) {
-          uint32_t src = row0 + m;
-          if (p.row_map != nullptr) src = p.row_map[src] / p.row_div;
-          v = *reinterpret_cast<const u4*>(p.x + (uint64_t)src * K + kc + c * 8);
-        }
-        const int slab = c >> 4, gg = (c >> 2) & 3, j = c & 3;
-        *reinterpret_cast<u4*>(xs + ((slab * 4 + j) * kSlots + gg * MR + m) * 16) = permute_x8(v);
-      }
-    }
-    __syncthreads();
-
-    // ---- 3. x-side sums per (row, group) of this wave's slabs (wave-private LDS) -----------
-    float* mycorr = corr + wave * (kSpwMax * 32);
-#pragma unroll
-    for (int it = 0; it < kSpwMax; ++it) {
-      if (it < my) {
-        f4 c2 = (f4){0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          h8 av = {0, 0, 0, 0, 0, 0, 0, 0};
-          if (a_active) av = *reinterpret_cast<const h8*>(xs + (((s0 + it) * 4 + j) * kSlots) * 16 + a_slot_off);
-          c2 = __builtin_amdgcn_mfma_f32_16x16x32_f16(av, bconst, c2, 0, 0, 0);
-        }
-        if (n < 2) {
-          const float sgn = n == 0 ? -1.0f : 1.0f;  // store -sum(off*x) and +sum(x)
-#pragma unroll
-          for (int i = 0; i < 4; ++i) mycorr[it * 32 + g * 8 + i * 2 + n] = sgn * c2[i];
-        }
-      }
-    }
-
-    // ---- 4. main loop: integer dot per group via MFMA, then scale/bias in f32 ---------------
-#pragma unroll
-    for (int it = 0; it < kSpwMax; ++it) {
-      if (it < my) {
-        const f4 c01 = *reinterpret_cast<const f4*>(mycorr + it * 32 + g * 8);      // (-xoff0,xsum0,-xoff1,xsum1)
-        const f4 c23 = *reinterpret_cast<const f4*>(mycorr + it * 32 + g * 8 + 4);  // rows 2,3
-        h8 av[4];
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          av[j] = (h8){0, 0, 0, 0, 0, 0, 0, 0};
-          if (a_active) av[j] = *reinterpret_cast<const h8*>(xs + (((s0 + it) * 4 + j) * kSlots) * 16 + a_slot_off);
-        }
-#pragma unroll
-        for (int t = 0; t < TILES; ++t) {
-          f4 c = (f4){c01[0], c01[2], c23[0], c23[2]};
-          const u4 wv = wreg[t][it];
-          c = __builtin_amdgcn_mfma_f32_16x16x32_f16(av[0], unpack_q4_word(wv.x), c, 0, 0, 0);
-          c = __builtin_amdgcn_mfma_f32_16x16x32_f16(av[1], unpack_q4_word(wv.y), c, 0, 0, 0);
-          c = __builtin_amdgcn_mfma_f32_16x16x32_f16(av[2], unpack_q4_word(wv.z), c, 0, 0, 0);
-          c = __builtin_amdgcn_mfma_f32_16x16x32_f16(av[3], unpack_q4_word(wv.w), c, 0, 0, 0);
-          const uint32_t sb = sbs[(t * 16 + n) * kSbStride + (s0 + it) * 2 + par];
-          const float sc = __half2float(__ushort_as_half((unsigned short)(sb & 0xFFFFu)));
-          const float bi = __half2float(__ushort_as_half((unsigned short)(sb >> 16)));
-          F[t][0] += sc * c[0] + bi * c01[1];
-          F[t][1] += sc * c[1] + bi * c01[3];
-          F[t][2] += sc * c[2] + bi * c23[1];
-          F[t][3] += sc * c[3] + bi * c23[3];
-        }
-      }
-    }
+    const uint32_t left = (K - kc) / 128;
+    if (left >= (uint32_t)kChunkSlabs)
+      qmv_pass<MR, TILES, TAB, true>(p, xs, sums, sbs, wrow, F, kc, kChunkSlabs, expert, row0, rows, tile_row, kc == 0);
+    else
+      qmv_pass<MR, TILES, TAB, false>(p, xs, sums, sbs, wrow, F, kc, (int)left, expert, row0, rows, tile_row, kc == 0);
   }
 
   // ---- 5. reduce over waves and over the two group halves, write out ---------------------------
+  QMV_MARK(p, 5);
   __syncthreads();  // everyone is done with xs
+  QMV_MARK(p, 6);
   float* red = reinterpret_cast<float*>(xs);
 #pragma unroll
   for (int t = 0; t < TILES; ++t)
 #pragma unroll
     for (int i = 0; i < 4; ++i) red[((wave * TILES + t) * 16 + g * 4 + i) * 16 + n] = F[t][i];
   __syncthreads();
+  QMV_MARK(p, 7);
   if (tid < 128) {
     const int m = tid >> 4, nn = tid & 15;
     if ((uint32_t)m < rows) {
@@ -270,11 +368,13 @@ __global__ __launch_bounds__(kThreads) void qmv_q4_kernel(KParams p) {
       else reinterpret_cast<__half*>(p.out)[o] = __float2half(r);
     }
   }
+  QMV_MARK(p, 8);
 }
 
 template <int MR, int TILES>
-void launch_t(const KParams& p, dim3 grid, hipStream_t s) {
-  hipLaunchKernelGGL((qmv_q4_kernel<MR, TILES>), grid, dim3(kThreads), 0, s, p);
+void launch_t(const KParams& p, bool tab, dim3 grid, hipStream_t s) {
+  if (tab) hipLaunchKernelGGL((qmv_q4_kernel<MR, TILES, true>), grid, dim3(kThreads), 0, s, p);
+  else hipLaunchKernelGGL((qmv_q4_kernel<MR, TILES, false>), grid, dim3(kThreads), 0, s, p);
 }
 
 __global__ void build_gather_chunks_kernel(const uint32_t* indices, uint32_t batch, uint32_t mpb,
@@ -302,36 +402,44 @@ int32_t launch_build_gather_chunks(const uint32_t* indices, uint32_t batch, uint
   return RMLX_OK;
 }
 
+#ifdef QMV_TRACE
+unsigned long long* g_qmv_trace = nullptr;
+#endif
+
 bool qmv_q4_supported(uint32_t N, uint32_t K, uint32_t group_size) {
   return group_size == 64 && N % 16 == 0 && K % 512 == 0 && N > 0 && K > 0;
 }
 
 int32_t launch_qmv_q4(const QmvArgs& a, hipStream_t s) {
   if (!qmv_q4_supported(a.N, a.K, 64)) return fail(RMLX_INVALID_SHAPE, "qmv_q4: N %% 16 and K %% 512 required (N=%u K=%u)", a.N, a.K);
-  KParams p;
-  p.w[0] = a.w0; p.s[0] = a.s0; p.b[0] = a.b0;
-  p.w[1] = a.dual ? a.w1 : a.w0; p.s[1] = a.dual ? a.s1 : a.s0; p.b[1] = a.dual ? a.b1 : a.b0;
+  KParams p{};
+  p.w0 = a.w0; p.s0 = a.s0; p.b0 = a.b0;
+  p.w1 = a.dual ? a.w1 : a.w0; p.s1 = a.dual ? a.s1 : a.s0; p.b1 = a.dual ? a.b1 : a.b0;
   p.x = a.x; p.row_map = a.row_map; p.chunk_tab = a.chunk_tab; p.n_chunks = a.n_chunks_dev;
   p.out = a.out; p.estride_w = a.expert_stride_w; p.estride_s = a.expert_stride_s;
-  p.K = a.K; p.row_div = a.row_div ? a.row_div : 1; p.ld_out = a.ld_out; p.M = a.M; p.out_f32 = a.out_f32;
-  uint32_t chunks = a.chunk_tab ? a.max_chunks : (a.M + 7) / 8;
+  p.K = a.K; p.ld_out = a.ld_out; p.M = a.M; p.out_f32 = a.out_f32;
+#ifdef QMV_TRACE
+  p.trace = g_qmv_trace;
+#endif
+  const bool tab = a.chunk_tab != nullptr;
+  uint32_t chunks = tab ? a.max_chunks : (a.M + 7) / 8;
   if (chunks == 0) return RMLX_OK;
   dim3 grid(a.N / 16, chunks);
   int mr = a.mr;
-  if (mr == 0) mr = a.chunk_tab ? 8 : (a.M >= 5 ? 8 : (a.M >= 3 ? 4 : (a.M == 2 ? 2 : 1)));
+  if (mr == 0) mr = tab ? 8 : (a.M >= 5 ? 8 : (a.M >= 3 ? 4 : (a.M == 2 ? 2 : 1)));
   if (a.dual) {
     switch (mr) {
-      case 1: launch_t<1, 2>(p, grid, s); break;
-      case 2: launch_t<2, 2>(p, grid, s); break;
-      case 4: launch_t<4, 2>(p, grid, s); break;
-      default: launch_t<8, 2>(p, grid, s); break;
+      case 1: launch_t<1, 2>(p, tab, grid, s); break;
+      case 2: launch_t<2, 2>(p, tab, grid, s); break;
+      case 4: launch_t<4, 2>(p, tab, grid, s); break;
+      default: launch_t<8, 2>(p, tab, grid, s); break;
     }
   } else {
     switch (mr) {
-      case 1: launch_t<1, 1>(p, grid, s); break;
-      case 2: launch_t<2, 1>(p, grid, s); break;
-      case 4: launch_t<4, 1>(p, grid, s); break;
-      default: launch_t<8, 1>(p, grid, s); break;
+      case 1: launch_t<1, 1>(p, tab, grid, s); break;
+      case 2: launch_t<2, 1>(p, tab, grid, s); break;
+      case 4: launch_t<4, 1>(p, tab, grid, s); break;
+      default: launch_t<8, 1>(p, tab, grid, s); break;
     }
   }
   RMLX_HIP_CHECK(hipGetLastError());
