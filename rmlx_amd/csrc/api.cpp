@@ -104,7 +104,7 @@ int32_t run_matmul(const rmlx_qweight* qw, const void* x, int32_t x_dtype, uint3
                 "buffers (N=%u K=%u bits=%u group_size=%u)", N, K, qw->bits, qw->group_size);
   } else if (kernel == KERNEL_QMM && !can_qmm) {
     return fail(RMLX_INVALID_SHAPE,
-                "qmm kernel requires bits in {4,8}, group_size=64, N %% 64 == 0, K %% 64 == 0 and 16-byte aligned "
+                "qmm kernel requires bits in {4,8}, group_size=64, N %% 64 == 0, K %% 256 == 0 and 16-byte aligned "
                 "buffers (N=%u K=%u bits=%u group_size=%u)", N, K, qw->bits, qw->group_size);
   } else if (kernel < 0 || kernel > KERNEL_GENERIC) {
     return fail(RMLX_NOT_FOUND, "unknown kernel selector %d", kernel);

@@ -4,13 +4,14 @@
 // Replaces the reference's affine_qmm_nax_q4 / affine_qmm_steel4sg_splitk_q4 /
 // affine_qmm_mma_q8 (crates/rmlx-core/src/ops/quantized.rs:3331-3565, 4572-4786, 5838-5971).
 //
-// Tile BM x BN x 64, 256 threads = 4 waves in a 2x2 grid, v_mfma_f32_16x16x32_{f16,bf16}.
+// Tile BM x 64 x 64, 256 threads = 4 waves stacked along M, v_mfma_f32_16x16x32_{f16,bf16}.
 // Per 64-wide k step every thread dequantizes 16 weights once for the whole workgroup
 // (w = scale*q + bias evaluated in packed f16 after an exact magic-number int->f16 conversion;
-// in f32 for the bf16 variant), writes them to LDS in natural k order next to the raw
-// activation tile, and the four waves read MFMA fragments from there.  Global loads of step
-// t+1 are issued before the MFMAs of step t (register-staged double buffering, two LDS
-// buffers, one barrier per step).  Workgroup ids are remapped so that the tiles sharing a
+// in f32 for the bf16 variant) and writes them to LDS in natural k order; the four waves read
+// the weight fragments from there.  Activations never touch LDS: each wave loads its own rows
+// from global memory directly in MFMA operand layout (LDS bandwidth is the scarce resource
+// here).  Global loads run kDepth steps ahead in a register ring; LDS is double-buffered with
+// one barrier per step.  Workgroup ids are remapped so that the tiles sharing a
 // weight panel run on the same XCD (shared L2).
 #include "common.hpp"
 
@@ -27,13 +28,27 @@ typedef uint32_t u2 __attribute__((ext_vector_type(2)));
 constexpr int kThreads = 256;
 constexpr int BK = 64;
 constexpr int LDK = BK + 8;  // padded LDS row (halves)
+constexpr int kDepth = 4;    // global-load prefetch distance in k-steps (must be even)
 
 struct QmmParams {
   const uint32_t* w; const __half* s; const __half* b;
   const uint16_t* x;  // f16 or bf16 bits
   __half* out;
   uint32_t M, N, K;
+#ifdef QMM_TRACE
+  unsigned long long* trace;  // development only: shader clock at a few points of the first steps
+#endif
 };
+
+#ifdef QMM_TRACE
+#define QMM_MARK(p, step, i)                                                                     \
+  do {                                                                                           \
+    if ((p).trace != nullptr && blockIdx.x == 0 && (threadIdx.x & 63) == 0 && (step) >= 8 && (step) < 12) \
+      (p).trace[((threadIdx.x >> 6) * 4 + ((step) - 8)) * 8 + (i)] = __builtin_readcyclecounter(); \
+  } while (0)
+#else
+#define QMM_MARK(p, step, i) do {} while (0)
+#endif
 
 __device__ __forceinline__ uint32_t h2bits(h2 v) { return __builtin_bit_cast(uint32_t, v); }
 
@@ -84,18 +99,19 @@ __device__ __forceinline__ u2 dequant_q8_word_bf16(uint32_t w, float s, float b)
 
 template <int BM, int BN, int BITS, bool XBF16>
 __global__ __launch_bounds__(kThreads) void qmm_kernel(QmmParams p) {
-  constexpr int WM = BM / 2, WN = BN / 2;      // wave tile
-  constexpr int TI = WM / 16, TJ = WN / 16;    // 16x16 MFMA tiles per wave
-  constexpr int A_UNITS = BM * BK / 8 / kThreads;  // 16-byte units of the activation tile per thread
+  constexpr int WM = BM / 4;                   // rows per wave: the 4 waves are stacked along M
+  constexpr int TI = WM / 16, TJ = BN / 16;    // 16x16 MFMA tiles per wave
+  constexpr int KK = BK / 32;                  // MFMA k-substeps per step
+  constexpr int kValuPerMfma = (BITS == 4 ? 48 : 40) / (KK * TI * TJ) + 1;  // staging VALU ops slotted after each MFMA
   constexpr int WPT = BN * BK * BITS / 32 / kThreads;  // weight words per thread per step
   static_assert(BN == 64, "weight staging assumes 4 threads per weight row");
   static_assert(WPT == (BITS == 4 ? 2 : 4), "16 weights per thread per step");
 
-  __shared__ __attribute__((aligned(16))) uint16_t As[2][BM * LDK];
+  // Only the dequantized weight tile goes through LDS (it is shared by the four waves).  Each
+  // wave reads its own activation rows straight from global memory in MFMA operand layout.
   __shared__ __attribute__((aligned(16))) uint16_t Bs[2][BN * LDK];
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int wm = wave >> 1, wn = wave & 1;
   const int r16 = lane & 15, g = lane >> 4;
 
   // ---- tile assignment: consecutive ids go to different XCDs; give each XCD whole weight panels
@@ -108,57 +124,61 @@ __global__ __launch_bounds__(kThreads) void qmm_kernel(QmmParams p) {
   const uint32_t K = p.K, gpr = K >> 6;
   const int steps = K / BK;
 
-  // staging coordinates
+  // weight staging coordinates
   const int brow = tid >> 2, bq = tid & 3;  // weight row in tile, 16-value quarter of the 64-k step
   const uint32_t* wptr = p.w + (uint64_t)(n0 + brow) * (K * BITS / 32) + bq * WPT;
   const __half* sptr = p.s + (uint64_t)(n0 + brow) * gpr;
   const __half* bptr = p.b + (uint64_t)(n0 + brow) * gpr;
 
-  u4 areg[A_UNITS];
-  uint32_t wreg[WPT];
-  __half sreg, breg;
-
-  auto load_global = [&](int step) {
+  // activation fragment pointers: lane (r16, g) holds k = 8g..8g+7 of row r16 of each 16-row tile.
+  // Rows past M re-read row M-1 (their results are never stored); unconditional loads keep the
+  // number of outstanding loads known to the compiler, i.e. exact s_waitcnt vmcnt counts.
+  const uint16_t* aptr[TI];
 #pragma unroll
-    for (int i = 0; i < A_UNITS; ++i) {
-      const int u = tid + i * kThreads, row = u >> 3, c8 = u & 7;
-      areg[i] = (u4){0u, 0u, 0u, 0u};
-      if (m0 + row < p.M)
-        areg[i] = *reinterpret_cast<const u4*>(p.x + (uint64_t)(m0 + row) * K + step * BK + c8 * 8);
-    }
+  for (int i = 0; i < TI; ++i) {
+    const uint32_t row = m0 + wave * WM + i * 16 + r16;
+    aptr[i] = p.x + (uint64_t)(row < p.M ? row : p.M - 1) * K + g * 8;
+  }
+
+  // Register ring of kDepth k-steps: global loads run kDepth steps ahead of the MFMAs.
+  u4 areg[kDepth][KK][TI];
+  uint32_t wreg[kDepth][WPT];
+  __half sreg[kDepth], breg[kDepth];
+
+  auto load_global = [&](int step, int slot) {
+#pragma unroll
+    for (int kk = 0; kk < KK; ++kk)
+#pragma unroll
+      for (int i = 0; i < TI; ++i)
+        areg[slot][kk][i] = *reinterpret_cast<const u4*>(aptr[i] + step * BK + kk * 32);
     if (BITS == 4) {
       const u2 v = *reinterpret_cast<const u2*>(wptr + step * (BK * BITS / 32));
-      wreg[0] = v.x; wreg[1] = v.y;
+      wreg[slot][0] = v.x; wreg[slot][1] = v.y;
     } else {
       const u4 v = *reinterpret_cast<const u4*>(wptr + step * (BK * BITS / 32));
-      wreg[0] = v.x; wreg[1] = v.y; wreg[WPT - 2] = v.z; wreg[WPT - 1] = v.w;
+      wreg[slot][0] = v.x; wreg[slot][1] = v.y; wreg[slot][WPT - 2] = v.z; wreg[slot][WPT - 1] = v.w;
     }
-    sreg = sptr[step];
-    breg = bptr[step];
+    sreg[slot] = sptr[step];
+    breg[slot] = bptr[step];
   };
 
-  auto store_lds = [&](int buf) {
-#pragma unroll
-    for (int i = 0; i < A_UNITS; ++i) {
-      const int u = tid + i * kThreads, row = u >> 3, c8 = u & 7;
-      *reinterpret_cast<u4*>(&As[buf][row * LDK + c8 * 8]) = areg[i];
-    }
+  auto store_lds = [&](int buf, int slot) {
     uint16_t* dst = &Bs[buf][brow * LDK + bq * 16];
     if (XBF16) {
-      const float s = __half2float(sreg), b = __half2float(breg);
-      const u2 lo = dequant_q8_word_bf16(wreg[0], s, b), l2 = dequant_q8_word_bf16(wreg[1], s, b);
-      const u2 h1 = dequant_q8_word_bf16(wreg[WPT - 2], s, b), h2v = dequant_q8_word_bf16(wreg[WPT - 1], s, b);
+      const float s = __half2float(sreg[slot]), b = __half2float(breg[slot]);
+      const u2 lo = dequant_q8_word_bf16(wreg[slot][0], s, b), l2 = dequant_q8_word_bf16(wreg[slot][1], s, b);
+      const u2 h1 = dequant_q8_word_bf16(wreg[slot][WPT - 2], s, b), h2v = dequant_q8_word_bf16(wreg[slot][WPT - 1], s, b);
       *reinterpret_cast<u4*>(dst) = (u4){lo.x, lo.y, l2.x, l2.y};
       *reinterpret_cast<u4*>(dst + 8) = (u4){h1.x, h1.y, h2v.x, h2v.y};
     } else {
-      const _Float16 sh = __builtin_bit_cast(_Float16, sreg), bh = __builtin_bit_cast(_Float16, breg);
+      const _Float16 sh = __builtin_bit_cast(_Float16, sreg[slot]), bh = __builtin_bit_cast(_Float16, breg[slot]);
       const h2 s2 = {sh, sh}, b2 = {bh, bh};
       if (BITS == 4) {
-        *reinterpret_cast<u4*>(dst) = dequant_q4_word_f16(wreg[0], s2, b2);
-        *reinterpret_cast<u4*>(dst + 8) = dequant_q4_word_f16(wreg[1], s2, b2);
+        *reinterpret_cast<u4*>(dst) = dequant_q4_word_f16(wreg[slot][0], s2, b2);
+        *reinterpret_cast<u4*>(dst + 8) = dequant_q4_word_f16(wreg[slot][1], s2, b2);
       } else {
-        const u2 a0 = dequant_q8_word_f16(wreg[0], s2, b2), a1 = dequant_q8_word_f16(wreg[1], s2, b2);
-        const u2 a2 = dequant_q8_word_f16(wreg[WPT - 2], s2, b2), a3 = dequant_q8_word_f16(wreg[WPT - 1], s2, b2);
+        const u2 a0 = dequant_q8_word_f16(wreg[slot][0], s2, b2), a1 = dequant_q8_word_f16(wreg[slot][1], s2, b2);
+        const u2 a2 = dequant_q8_word_f16(wreg[slot][WPT - 2], s2, b2), a3 = dequant_q8_word_f16(wreg[slot][WPT - 1], s2, b2);
         *reinterpret_cast<u4*>(dst) = (u4){a0.x, a0.y, a1.x, a1.y};
         *reinterpret_cast<u4*>(dst + 8) = (u4){a2.x, a2.y, a3.x, a3.y};
       }
@@ -171,36 +191,60 @@ __global__ __launch_bounds__(kThreads) void qmm_kernel(QmmParams p) {
 #pragma unroll
     for (int j = 0; j < TJ; ++j) acc[i][j] = (f4){0.f, 0.f, 0.f, 0.f};
 
-  load_global(0);
-  store_lds(0);
+  const int last = steps - 1;
+#pragma unroll
+  for (int d = 0; d < kDepth; ++d) load_global(d < last ? d : last, d);
+  store_lds(0, 0);
   __syncthreads();
 
-  for (int step = 0; step < steps; ++step) {
-    const int cur = step & 1;
-    if (step + 1 < steps) load_global(step + 1);
+  // steps is a multiple of kDepth (the host checks K % (64 * kDepth) == 0), so the body below is
+  // branch-free: one scheduling region per step, with an explicit interleaving recipe.
+  for (int step0 = 0; step0 < steps; step0 += kDepth) {
 #pragma unroll
-    for (int kk = 0; kk < BK / 32; ++kk) {
-      u4 af[TI], bf[TJ];
+    for (int d = 0; d < kDepth; ++d) {
+      const int step = step0 + d;
+      const int cur = step & 1;
+      QMM_MARK(p, step, 0);
+      // weight fragments of the current tile (all four waves read the whole 64-row tile)
+      u4 bf[KK][TJ];
 #pragma unroll
-      for (int i = 0; i < TI; ++i)
-        af[i] = *reinterpret_cast<const u4*>(&As[cur][(wm * WM + i * 16 + r16) * LDK + kk * 32 + g * 8]);
+      for (int kk = 0; kk < KK; ++kk)
 #pragma unroll
-      for (int j = 0; j < TJ; ++j)
-        bf[j] = *reinterpret_cast<const u4*>(&Bs[cur][(wn * WN + j * 16 + r16) * LDK + kk * 32 + g * 8]);
+        for (int j = 0; j < TJ; ++j)
+          bf[kk][j] = *reinterpret_cast<const u4*>(&Bs[cur][(j * 16 + r16) * LDK + kk * 32 + g * 8]);
+      // next step's weights: dequantize into the other LDS buffer (independent of the MFMAs, so
+      // the matrix pipe works in the shadow of this VALU / LDS work)
+      store_lds(cur ^ 1, (d + 1) % kDepth);
 #pragma unroll
-      for (int i = 0; i < TI; ++i)
+      for (int kk = 0; kk < KK; ++kk)
 #pragma unroll
-        for (int j = 0; j < TJ; ++j) {
-          if (XBF16)
-            acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(b8, af[i]),
-                                                                __builtin_bit_cast(b8, bf[j]), acc[i][j], 0, 0, 0);
-          else
-            acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h8, af[i]),
-                                                               __builtin_bit_cast(h8, bf[j]), acc[i][j], 0, 0, 0);
-        }
+        for (int i = 0; i < TI; ++i)
+#pragma unroll
+          for (int j = 0; j < TJ; ++j) {
+            if (XBF16)
+              acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(b8, areg[d][kk][i]),
+                                                                  __builtin_bit_cast(b8, bf[kk][j]), acc[i][j], 0, 0, 0);
+            else
+              acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h8, areg[d][kk][i]),
+                                                                 __builtin_bit_cast(h8, bf[kk][j]), acc[i][j], 0, 0, 0);
+          }
+      // slot d is consumed: refill it kDepth steps ahead (the tail re-reads the last step
+      // instead of branching around the loads)
+      load_global(step + kDepth < last ? step + kDepth : last, d);
+      // recipe: all LDS reads up front, then each MFMA followed by a few staging VALU ops; the
+      // two LDS writes and the global loads are spread over the second half
+      __builtin_amdgcn_sched_group_barrier(0x100, KK * TJ, 0);
+#pragma unroll
+      for (int q = 0; q < KK * TI * TJ; ++q) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x002, kValuPerMfma, 0);
+        if (q >= KK * TI * TJ / 2) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+        if (q == KK * TI * TJ / 2 || q == KK * TI * TJ / 2 + 1) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
+      }
+      QMM_MARK(p, step, 3);
+      __syncthreads();
+      QMM_MARK(p, step, 4);
     }
-    if (step + 1 < steps) store_lds(cur ^ 1);
-    __syncthreads();
   }
 
   // accumulator lane (r16, g) holds column n = r16 and rows 4g..4g+3 of each 16x16 tile
@@ -210,8 +254,8 @@ __global__ __launch_bounds__(kThreads) void qmm_kernel(QmmParams p) {
     for (int j = 0; j < TJ; ++j)
 #pragma unroll
       for (int v = 0; v < 4; ++v) {
-        const uint32_t m = m0 + wm * WM + i * 16 + g * 4 + v;
-        const uint32_t nn = n0 + wn * WN + j * 16 + r16;
+        const uint32_t m = m0 + wave * WM + i * 16 + g * 4 + v;
+        const uint32_t nn = n0 + j * 16 + r16;
         if (m < p.M) p.out[(uint64_t)m * p.N + nn] = __float2half(acc[i][j][v]);
       }
 }
@@ -224,8 +268,12 @@ void launch_t(const QmmParams& p, hipStream_t s) {
 
 }  // namespace
 
+#ifdef QMM_TRACE
+unsigned long long* g_qmm_trace = nullptr;
+#endif
+
 bool qmm_supported(uint32_t N, uint32_t K, uint32_t group_size, uint32_t bits) {
-  return group_size == 64 && (bits == 4 || bits == 8) && N % 64 == 0 && K % 64 == 0 && N > 0 && K > 0;
+  return group_size == 64 && (bits == 4 || bits == 8) && N % 64 == 0 && K % (BK * kDepth) == 0 && N > 0 && K > 0;
 }
 
 int32_t launch_qmm(const QmmArgs& a, hipStream_t s) {
@@ -233,6 +281,9 @@ int32_t launch_qmm(const QmmArgs& a, hipStream_t s) {
     return fail(RMLX_INVALID_SHAPE, "qmm: unsupported shape N=%u K=%u bits=%u", a.N, a.K, a.bits);
   if (a.M == 0) return RMLX_OK;
   QmmParams p{a.w, a.s, a.b, reinterpret_cast<const uint16_t*>(a.x), a.out, a.M, a.N, a.K};
+#ifdef QMM_TRACE
+  p.trace = g_qmm_trace;
+#endif
   const bool big = a.M > 64;
   if (a.bits == 4) {
     if (a.x_bf16) return fail(RMLX_INVALID_SHAPE, "qmm: Q4 takes f16 activations (bf16 is cast by the caller)");
