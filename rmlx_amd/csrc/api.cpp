@@ -3,6 +3,8 @@
 // here and there is no CPU fallback: every path ends in a HIP kernel launch or an error.
 #include <cinttypes>
 #include <cstring>
+#include <map>
+#include <mutex>
 #include <vector>
 
 #include "common.hpp"
@@ -56,17 +58,43 @@ int32_t finish(hipStream_t stream) {
   return RMLX_OK;
 }
 
+// Scratch blocks are pooled per stream and never handed back to the driver while the library is
+// loaded: every use is ordered on the owning stream, so a block released by one call can be
+// reused by the next call on that stream without synchronisation, and steady-state calls make
+// no allocator calls at all.
+namespace {
+struct Block { void* ptr; size_t bytes; };
+std::mutex g_pool_mutex;
+std::map<hipStream_t, std::vector<Block>> g_pool;
+}  // namespace
+
 int32_t Scratch::alloc(size_t bytes, hipStream_t s) {
   release();
   stream = s;
   if (bytes == 0) bytes = 16;
-  RMLX_HIP_CHECK(hipMallocAsync(&ptr, bytes, s));
+  {
+    std::lock_guard<std::mutex> lock(g_pool_mutex);
+    std::vector<Block>& free_list = g_pool[s];
+    size_t best = free_list.size();
+    for (size_t i = 0; i < free_list.size(); ++i)
+      if (free_list[i].bytes >= bytes && (best == free_list.size() || free_list[i].bytes < free_list[best].bytes)) best = i;
+    if (best != free_list.size()) {
+      ptr = free_list[best].ptr;
+      size = free_list[best].bytes;
+      free_list.erase(free_list.begin() + (long)best);
+      return RMLX_OK;
+    }
+  }
+  const size_t rounded = (bytes + 0xFFFFF) & ~(size_t)0xFFFFF;  // 1 MiB granularity
+  RMLX_HIP_CHECK(hipMalloc(&ptr, rounded));
+  size = rounded;
   return RMLX_OK;
 }
 
 void Scratch::release() {
   if (ptr != nullptr) {
-    (void)hipFreeAsync(ptr, stream);
+    std::lock_guard<std::mutex> lock(g_pool_mutex);
+    g_pool[stream].push_back(Block{ptr, size});
     ptr = nullptr;
   }
 }
@@ -110,11 +138,19 @@ int32_t run_matmul(const rmlx_qweight* qw, const void* x, int32_t x_dtype, uint3
     return fail(RMLX_NOT_FOUND, "unknown kernel selector %d", kernel);
   }
 
-  // Activations: f16 is native everywhere; bf16 is native only in the Q8 MFMA GEMM.
-  const bool native_bf16 = x_dtype == RMLX_DTYPE_BF16 && kernel == KERNEL_QMM && qw->bits == 8;
+  if (kernel == KERNEL_QMM) {
+    // The GEMM re-lays the activations out in MFMA operand order first (dtype cast fused in;
+    // bf16 stays bf16 for Q8 weights, everything else becomes f16).
+    Scratch ws;
+    RMLX_TRY(ws.alloc(qmm_workspace_bytes(M, K), stream));
+    QmmArgs a{qw->w, qw->s, qw->b, x, x_dtype, out, M, N, K, qw->bits, ws.ptr};
+    return launch_qmm(a, stream);
+  }
+
+  // Activations of the other kernels: f16 (f32 / bf16 are cast first).
   Scratch cast;
   const void* xk = x;
-  if (x_dtype != RMLX_DTYPE_F16 && !native_bf16) {
+  if (x_dtype != RMLX_DTYPE_F16) {
     RMLX_TRY(cast.alloc((size_t)M * K * sizeof(__half), stream));
     RMLX_TRY(launch_cast_to_f16(x, x_dtype, static_cast<__half*>(cast.ptr), (size_t)M * K, stream));
     xk = cast.ptr;
@@ -127,10 +163,6 @@ int32_t run_matmul(const rmlx_qweight* qw, const void* x, int32_t x_dtype, uint3
     a.x = static_cast<const __half*>(xk);
     a.out = out; a.ld_out = N; a.M = M;
     return launch_qmv_q4(a, stream);
-  }
-  if (kernel == KERNEL_QMM) {
-    QmmArgs a{qw->w, qw->s, qw->b, xk, out, M, N, K, qw->bits, native_bf16 ? 1 : 0};
-    return launch_qmm(a, stream);
   }
   GenericArgs g{qw->w, qw->s, qw->b, static_cast<const __half*>(xk), out, nullptr, 0, M, N, K,
                 qw->group_size, qw->bits, 1};

@@ -58,10 +58,11 @@ int32_t require_init();
 // Finishes a call: synchronous when the caller passed no stream.
 int32_t finish(hipStream_t stream);
 
-// Stream-ordered scratch (freed with release()).  Used only for dtype casts of the
-// activations and for the MoE intermediates, never on the f16 fast paths of qmv / qmm.
+// Stream-ordered scratch from a per-stream pool (see api.cpp).  Used for dtype casts, the
+// re-laid-out activations of the GEMM and the MoE intermediates; the f16 qmv path needs none.
 struct Scratch {
   void* ptr = nullptr;
+  size_t size = 0;
   hipStream_t stream = nullptr;
   int32_t alloc(size_t bytes, hipStream_t s);
   void release();
@@ -131,11 +132,13 @@ int32_t launch_build_gather_chunks(const uint32_t* indices, uint32_t batch, uint
 
 struct QmmArgs {
   const uint32_t* w; const __half* s; const __half* b;
-  const void* x;  // f16 or bf16 [M,K]
-  __half* out;    // [M,N]
+  const void* x;      // [M,K] row-major, f16 / bf16 / f32 (cast fused into the re-layout pass)
+  int32_t x_dtype;
+  __half* out;        // [M,N]
   uint32_t M, N, K, bits;
-  int x_bf16;
+  void* workspace;    // qmm_workspace_bytes(M, K) bytes of device scratch (fragment-major activations)
 };
+size_t qmm_workspace_bytes(uint32_t M, uint32_t K);
 bool qmm_supported(uint32_t N, uint32_t K, uint32_t group_size, uint32_t bits);
 int32_t launch_qmm(const QmmArgs& a, hipStream_t s);
 

@@ -32,7 +32,7 @@ constexpr int kDepth = 4;    // global-load prefetch distance in k-steps (must b
 
 struct QmmParams {
   const uint32_t* w; const __half* s; const __half* b;
-  const uint16_t* x;  // f16 or bf16 bits
+  const uint16_t* x;  // f16 or bf16 bits in fragment-major layout (see relayout_a_kernel)
   __half* out;
   uint32_t M, N, K;
 #ifdef QMM_TRACE
@@ -109,7 +109,10 @@ __global__ __launch_bounds__(kThreads) void qmm_kernel(QmmParams p) {
 
   // Only the dequantized weight tile goes through LDS (it is shared by the four waves).  Each
   // wave reads its own activation rows straight from global memory in MFMA operand layout.
-  __shared__ __attribute__((aligned(16))) uint16_t Bs[2][BN * LDK];
+  // Four LDS buffers: step s multiplies out of registers filled from buffer s%4 one step earlier,
+  // prefetches the fragments of step s+1 from buffer (s+1)%4 and writes the tile of step s+2.
+  __shared__ __attribute__((aligned(16))) uint16_t Bs[4][BN * LDK];
+  static_assert(kDepth == 4, "buffer indices below are derived from the unrolled step index");
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int r16 = lane & 15, g = lane >> 4;
@@ -122,7 +125,7 @@ __global__ __launch_bounds__(kThreads) void qmm_kernel(QmmParams p) {
   const uint32_t m0 = (id % tiles_m) * BM, n0 = (id / tiles_m) * BN;
 
   const uint32_t K = p.K, gpr = K >> 6;
-  const int steps = K / BK;
+  const int steps = K / BK;  // a multiple of kDepth (checked on the host)
 
   // weight staging coordinates
   const int brow = tid >> 2, bq = tid & 3;  // weight row in tile, 16-value quarter of the 64-k step
@@ -130,27 +133,32 @@ __global__ __launch_bounds__(kThreads) void qmm_kernel(QmmParams p) {
   const __half* sptr = p.s + (uint64_t)(n0 + brow) * gpr;
   const __half* bptr = p.b + (uint64_t)(n0 + brow) * gpr;
 
-  // activation fragment pointers: lane (r16, g) holds k = 8g..8g+7 of row r16 of each 16-row tile.
-  // Rows past M re-read row M-1 (their results are never stored); unconditional loads keep the
-  // number of outstanding loads known to the compiler, i.e. exact s_waitcnt vmcnt counts.
-  const uint16_t* aptr[TI];
+  // activation fragments: block (16-row tile, 32-wide k chunk) = 64 lanes x 16 bytes, contiguous,
+  // already in MFMA operand order.  Tiles past the last one re-read the last tile (their results
+  // are never stored); unconditional loads keep the number of outstanding loads known to the
+  // compiler, i.e. exact s_waitcnt vmcnt counts.
+  const u4* aptr[TI];
+  const uint32_t mt_last = (p.M + 15) / 16 - 1;
 #pragma unroll
   for (int i = 0; i < TI; ++i) {
-    const uint32_t row = m0 + wave * WM + i * 16 + r16;
-    aptr[i] = p.x + (uint64_t)(row < p.M ? row : p.M - 1) * K + g * 8;
+    const uint32_t mt = (m0 + wave * WM) / 16 + i;
+    aptr[i] = reinterpret_cast<const u4*>(p.x) + (uint64_t)(mt < mt_last ? mt : mt_last) * (K / 32) * 64 + lane;
   }
 
-  // Register ring of kDepth k-steps: global loads run kDepth steps ahead of the MFMAs.
+  // Register ring of kDepth k-steps: global loads run kDepth steps ahead of the MFMAs.  Scales
+  // and biases are fetched four groups (one unrolled iteration) at a time.
   u4 areg[kDepth][KK][TI];
   uint32_t wreg[kDepth][WPT];
-  __half sreg[kDepth], breg[kDepth];
+  u2 sb_cur[2], sb_next[2];  // [0] scales, [1] biases of 4 consecutive groups
 
-  auto load_global = [&](int step, int slot) {
+  auto load_a = [&](int step, int slot) {
 #pragma unroll
     for (int kk = 0; kk < KK; ++kk)
 #pragma unroll
       for (int i = 0; i < TI; ++i)
-        areg[slot][kk][i] = *reinterpret_cast<const u4*>(aptr[i] + step * BK + kk * 32);
+        areg[slot][kk][i] = aptr[i][(step * KK + kk) * 64];
+  };
+  auto load_w = [&](int step, int slot) {
     if (BITS == 4) {
       const u2 v = *reinterpret_cast<const u2*>(wptr + step * (BK * BITS / 32));
       wreg[slot][0] = v.x; wreg[slot][1] = v.y;
@@ -158,20 +166,27 @@ __global__ __launch_bounds__(kThreads) void qmm_kernel(QmmParams p) {
       const u4 v = *reinterpret_cast<const u4*>(wptr + step * (BK * BITS / 32));
       wreg[slot][0] = v.x; wreg[slot][1] = v.y; wreg[slot][WPT - 2] = v.z; wreg[slot][WPT - 1] = v.w;
     }
-    sreg[slot] = sptr[step];
-    breg[slot] = bptr[step];
+  };
+  auto load_sb = [&](int group0, u2 (&dst)[2]) {
+    dst[0] = *reinterpret_cast<const u2*>(sptr + group0);
+    dst[1] = *reinterpret_cast<const u2*>(bptr + group0);
+  };
+  auto pick16 = [](const u2& v, int e) -> uint16_t {  // element e (0..3) of four packed halves
+    const uint32_t wd = e < 2 ? v.x : v.y;
+    return (uint16_t)((e & 1) ? wd >> 16 : wd & 0xFFFFu);
   };
 
-  auto store_lds = [&](int buf, int slot) {
+  // dequantize the weights held in ring slot `slot` (scale / bias bits given) into LDS buffer `buf`
+  auto store_lds = [&](int buf, int slot, uint16_t sbits, uint16_t bbits) {
     uint16_t* dst = &Bs[buf][brow * LDK + bq * 16];
     if (XBF16) {
-      const float s = __half2float(sreg[slot]), b = __half2float(breg[slot]);
+      const float s = __half2float(__ushort_as_half(sbits)), b = __half2float(__ushort_as_half(bbits));
       const u2 lo = dequant_q8_word_bf16(wreg[slot][0], s, b), l2 = dequant_q8_word_bf16(wreg[slot][1], s, b);
       const u2 h1 = dequant_q8_word_bf16(wreg[slot][WPT - 2], s, b), h2v = dequant_q8_word_bf16(wreg[slot][WPT - 1], s, b);
       *reinterpret_cast<u4*>(dst) = (u4){lo.x, lo.y, l2.x, l2.y};
       *reinterpret_cast<u4*>(dst + 8) = (u4){h1.x, h1.y, h2v.x, h2v.y};
     } else {
-      const _Float16 sh = __builtin_bit_cast(_Float16, sreg[slot]), bh = __builtin_bit_cast(_Float16, breg[slot]);
+      const _Float16 sh = __builtin_bit_cast(_Float16, sbits), bh = __builtin_bit_cast(_Float16, bbits);
       const h2 s2 = {sh, sh}, b2 = {bh, bh};
       if (BITS == 4) {
         *reinterpret_cast<u4*>(dst) = dequant_q4_word_f16(wreg[slot][0], s2, b2);
@@ -184,6 +199,13 @@ __global__ __launch_bounds__(kThreads) void qmm_kernel(QmmParams p) {
       }
     }
   };
+  auto read_frags = [&](int buf, u4 (&bf)[KK][TJ]) {
+#pragma unroll
+    for (int kk = 0; kk < KK; ++kk)
+#pragma unroll
+      for (int j = 0; j < TJ; ++j)
+        bf[kk][j] = *reinterpret_cast<const u4*>(&Bs[buf][(j * 16 + r16) * LDK + kk * 32 + g * 8]);
+  };
 
   f4 acc[TI][TJ];
 #pragma unroll
@@ -191,30 +213,38 @@ __global__ __launch_bounds__(kThreads) void qmm_kernel(QmmParams p) {
 #pragma unroll
     for (int j = 0; j < TJ; ++j) acc[i][j] = (f4){0.f, 0.f, 0.f, 0.f};
 
+  // ---- prologue: fill the ring, stage tiles 0 and 1, fetch the fragments of step 0 ------------------
   const int last = steps - 1;
+  load_sb(0, sb_cur);
+  load_sb(steps > 4 ? 4 : 0, sb_next);
 #pragma unroll
-  for (int d = 0; d < kDepth; ++d) load_global(d < last ? d : last, d);
-  store_lds(0, 0);
+  for (int d = 0; d < kDepth; ++d) { load_a(d, d); load_w(d, d); }
+  store_lds(0, 0, pick16(sb_cur[0], 0), pick16(sb_cur[1], 0));
+  store_lds(1, 1, pick16(sb_cur[0], 1), pick16(sb_cur[1], 1));
+  // weight slots 0 and 1 are consumed: refill them with steps 4 and 5
+  load_w(4 < last ? 4 : last, 0);
+  load_w(5 < last ? 5 : last, 1);
   __syncthreads();
+  u4 bf[2][KK][TJ];
+  read_frags(0, bf[0]);
 
-  // steps is a multiple of kDepth (the host checks K % (64 * kDepth) == 0), so the body below is
-  // branch-free: one scheduling region per step, with an explicit interleaving recipe.
   for (int step0 = 0; step0 < steps; step0 += kDepth) {
+    // scales / biases of groups step0+8 .. step0+11 (needed two iterations from now)
+    u2 sb_nn[2];
+    load_sb(step0 + 8 < steps ? step0 + 8 : 0, sb_nn);
 #pragma unroll
     for (int d = 0; d < kDepth; ++d) {
       const int step = step0 + d;
-      const int cur = step & 1;
       QMM_MARK(p, step, 0);
-      // weight fragments of the current tile (all four waves read the whole 64-row tile)
-      u4 bf[KK][TJ];
-#pragma unroll
-      for (int kk = 0; kk < KK; ++kk)
-#pragma unroll
-        for (int j = 0; j < TJ; ++j)
-          bf[kk][j] = *reinterpret_cast<const u4*>(&Bs[cur][(j * 16 + r16) * LDK + kk * 32 + g * 8]);
-      // next step's weights: dequantize into the other LDS buffer (independent of the MFMAs, so
-      // the matrix pipe works in the shadow of this VALU / LDS work)
-      store_lds(cur ^ 1, (d + 1) % kDepth);
+      // fragments of the next step (its tile was written during the previous step)
+      read_frags((d + 1) & 3, bf[(d + 1) & 1]);
+      // tile of step+2: weights sit in ring slot (d+2)&3, their group is step+2
+      {
+        const int e = (d + 2) & 3;
+        const u2& sv = d < 2 ? sb_cur[0] : sb_next[0];
+        const u2& bv = d < 2 ? sb_cur[1] : sb_next[1];
+        store_lds((d + 2) & 3, e, pick16(sv, e), pick16(bv, e));
+      }
 #pragma unroll
       for (int kk = 0; kk < KK; ++kk)
 #pragma unroll
@@ -223,16 +253,17 @@ __global__ __launch_bounds__(kThreads) void qmm_kernel(QmmParams p) {
           for (int j = 0; j < TJ; ++j) {
             if (XBF16)
               acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(b8, areg[d][kk][i]),
-                                                                  __builtin_bit_cast(b8, bf[kk][j]), acc[i][j], 0, 0, 0);
+                                                                  __builtin_bit_cast(b8, bf[d & 1][kk][j]), acc[i][j], 0, 0, 0);
             else
               acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h8, areg[d][kk][i]),
-                                                                 __builtin_bit_cast(h8, bf[kk][j]), acc[i][j], 0, 0, 0);
+                                                                 __builtin_bit_cast(h8, bf[d & 1][kk][j]), acc[i][j], 0, 0, 0);
           }
-      // slot d is consumed: refill it kDepth steps ahead (the tail re-reads the last step
-      // instead of branching around the loads)
-      load_global(step + kDepth < last ? step + kDepth : last, d);
-      // recipe: all LDS reads up front, then each MFMA followed by a few staging VALU ops; the
-      // two LDS writes and the global loads are spread over the second half
+      // refill: activations of step+4 into slot d, weights of step+6 into slot (d+2)&3 (both just
+      // consumed); the tail re-reads the last step instead of branching around the loads
+      load_a(step + 4 < last ? step + 4 : last, d);
+      load_w(step + 6 < last ? step + 6 : last, (d + 2) & 3);
+      // recipe: LDS reads first, then each MFMA followed by a few staging VALU ops; the two LDS
+      // writes and the global loads are spread over the second half
       __builtin_amdgcn_sched_group_barrier(0x100, KK * TJ, 0);
 #pragma unroll
       for (int q = 0; q < KK * TI * TJ; ++q) {
@@ -245,6 +276,8 @@ __global__ __launch_bounds__(kThreads) void qmm_kernel(QmmParams p) {
       __syncthreads();
       QMM_MARK(p, step, 4);
     }
+    sb_cur[0] = sb_next[0]; sb_cur[1] = sb_next[1];
+    sb_next[0] = sb_nn[0]; sb_next[1] = sb_nn[1];
   }
 
   // accumulator lane (r16, g) holds column n = r16 and rows 4g..4g+3 of each 16x16 tile
@@ -258,6 +291,65 @@ __global__ __launch_bounds__(kThreads) void qmm_kernel(QmmParams p) {
         const uint32_t nn = n0 + j * 16 + r16;
         if (m < p.M) p.out[(uint64_t)m * p.N + nn] = __float2half(acc[i][j][v]);
       }
+}
+
+// Activations [M,K] (f16 / bf16 / f32, row-major) -> fragment-major f16 or bf16: for every
+// 16-row tile and 32-wide k chunk, 64 consecutive 16-byte units, unit (r + 16 g) = row r of the
+// tile, k = 8g..8g+7 of the chunk -- exactly what lane r+16g feeds to the MFMA.  A fragment load
+// in the GEMM is then one fully coalesced 1 KB access instead of 16 half-used cache lines.
+// The dtype cast is fused in.
+__global__ __launch_bounds__(256) void relayout_a_kernel(const void* __restrict__ src, int src_dtype,
+                                                         u4* __restrict__ dst, uint32_t M, uint32_t K,
+                                                         int to_bf16) {
+  const uint32_t kchunks = K / 32;
+  const uint64_t units = (uint64_t)((M + 15) / 16) * kchunks * 64;
+  for (uint64_t u = (uint64_t)blockIdx.x * 256 + threadIdx.x; u < units; u += (uint64_t)gridDim.x * 256) {
+    const uint32_t lane = (uint32_t)(u & 63);
+    const uint64_t blk = u >> 6;
+    const uint32_t mt = (uint32_t)(blk / kchunks), kc = (uint32_t)(blk % kchunks);
+    uint32_t row = mt * 16 + (lane & 15);
+    if (row >= M) row = M - 1;
+    const uint64_t off = (uint64_t)row * K + kc * 32 + (lane >> 4) * 8;
+    u4 o;
+    if (src_dtype == RMLX_DTYPE_F32) {
+      const float* f = reinterpret_cast<const float*>(src) + off;
+      uint32_t w[4];
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        if (to_bf16) w[q] = pack_bf16(f[2 * q], f[2 * q + 1]);
+        else {
+          const h2 v = {(_Float16)f[2 * q], (_Float16)f[2 * q + 1]};
+          w[q] = h2bits(v);
+        }
+      }
+      o = (u4){w[0], w[1], w[2], w[3]};
+    } else {
+      o = *reinterpret_cast<const u4*>(reinterpret_cast<const uint16_t*>(src) + off);
+      const bool is_bf16 = src_dtype == RMLX_DTYPE_BF16;
+      if (is_bf16 != (to_bf16 != 0)) {  // bf16 <-> f16 through f32
+        uint32_t w[4] = {o.x, o.y, o.z, o.w};
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          float lo, hi;
+          if (is_bf16) {
+            lo = __uint_as_float(w[q] << 16);
+            hi = __uint_as_float(w[q] & 0xFFFF0000u);
+          } else {
+            const h2 v = __builtin_bit_cast(h2, w[q]);
+            lo = (float)v[0];
+            hi = (float)v[1];
+          }
+          if (to_bf16) w[q] = pack_bf16(lo, hi);
+          else {
+            const h2 v = {(_Float16)lo, (_Float16)hi};
+            w[q] = h2bits(v);
+          }
+        }
+        o = (u4){w[0], w[1], w[2], w[3]};
+      }
+    }
+    dst[u] = o;
+  }
 }
 
 template <int BM, int BITS, bool XBF16>
@@ -276,19 +368,31 @@ bool qmm_supported(uint32_t N, uint32_t K, uint32_t group_size, uint32_t bits) {
   return group_size == 64 && (bits == 4 || bits == 8) && N % 64 == 0 && K % (BK * kDepth) == 0 && N > 0 && K > 0;
 }
 
+size_t qmm_workspace_bytes(uint32_t M, uint32_t K) { return (size_t)((M + 15) / 16) * 16 * K * 2; }
+
 int32_t launch_qmm(const QmmArgs& a, hipStream_t s) {
   if (!qmm_supported(a.N, a.K, 64, a.bits))
     return fail(RMLX_INVALID_SHAPE, "qmm: unsupported shape N=%u K=%u bits=%u", a.N, a.K, a.bits);
   if (a.M == 0) return RMLX_OK;
-  QmmParams p{a.w, a.s, a.b, reinterpret_cast<const uint16_t*>(a.x), a.out, a.M, a.N, a.K};
+  if (a.workspace == nullptr) return fail(RMLX_RUNTIME_ERROR, "qmm: missing activation workspace");
+  const bool want_bf16 = a.bits == 8 && a.x_dtype == RMLX_DTYPE_BF16;
+  {
+    const uint64_t units = (uint64_t)((a.M + 15) / 16) * (a.K / 32) * 64;
+    uint64_t blocks = (units + 255) / 256;
+    if (blocks > 4096) blocks = 4096;
+    hipLaunchKernelGGL(relayout_a_kernel, dim3((unsigned)blocks), dim3(256), 0, s, a.x, a.x_dtype,
+                       reinterpret_cast<u4*>(a.workspace), a.M, a.K, want_bf16 ? 1 : 0);
+  }
+  QmmParams p{a.w, a.s, a.b, reinterpret_cast<const uint16_t*>(a.workspace), a.out, a.M, a.N, a.K};
 #ifdef QMM_TRACE
   p.trace = g_qmm_trace;
 #endif
-  const bool big = a.M > 64;
+  // 128-row tiles only when they still give (most of) the CUs a workgroup
+  const uint32_t tiles128 = ((a.M + 127) / 128) * (a.N / 64);
+  const bool big = a.M > 64 && tiles128 * 4 >= (uint32_t)ctx().num_cus * 3;
   if (a.bits == 4) {
-    if (a.x_bf16) return fail(RMLX_INVALID_SHAPE, "qmm: Q4 takes f16 activations (bf16 is cast by the caller)");
     if (big) launch_t<128, 4, false>(p, s); else launch_t<64, 4, false>(p, s);
-  } else if (a.x_bf16) {
+  } else if (want_bf16) {
     if (big) launch_t<128, 8, true>(p, s); else launch_t<64, 8, true>(p, s);
   } else {
     if (big) launch_t<128, 8, false>(p, s); else launch_t<64, 8, false>(p, s);
