@@ -58,7 +58,7 @@ class Timer:
         return self.e0.elapsed_ms(self.e1) / steps  # ms per step
 
 
-def bench_matmul(ops, rt, timer, rng, m, n, k, bits, x_dtype, steps, warmup, min_total_bytes, check=True):
+def bench_matmul(ops, rt, timer, rng, m, n, k, bits, x_dtype, steps, warmup, min_total_bytes, check=True, kernel=0):
     from oracle import model
     wbytes = n * k * bits // 8 + 4 * (n * k // 64)
     n_sets = max(1, -(-min_total_bytes // wbytes))
@@ -77,13 +77,13 @@ def bench_matmul(ops, rt, timer, rng, m, n, k, bits, x_dtype, steps, warmup, min
         xd = rt.DeviceBuffer.from_numpy(xh)
         x64 = xh.astype(np.float64)
     outs = [rt.DeviceBuffer((m, n), rt.F16) for _ in range(min(n_sets, 8))]
-    ms = timer.run(lambda c: ops.qmm_encode_many(qws, xd, outs, c, stream=timer.stream), steps, warmup)
+    ms = timer.run(lambda c: ops.qmm_encode_many(qws, xd, outs, c, stream=timer.stream, kernel=kernel), steps, warmup)
     res = {"us": ms * 1e3, "n_weight_sets": n_sets,
            "bytes": matmul_bytes(m, n, k, bits, act_bytes=2), "flops": 2 * m * n * k}
     res["gbs"] = res["bytes"] / (ms * 1e-3) / 1e9
     res["tflops"] = res["flops"] / (ms * 1e-3) / 1e12
     if check:  # parity of the timed configuration against the oracle, on weight set 0
-        ops.qmm_encode_many(qws[:1], xd, outs[:1], 1, stream=timer.stream)
+        ops.qmm_encode_many(qws[:1], xd, outs[:1], 1, stream=timer.stream, kernel=kernel)
         timer.stream.sync()
         ref = model.qmm(x64, *base, 64, bits)
         err = float(np.abs(outs[0].numpy().astype(np.float64) - ref).max())
@@ -174,10 +174,11 @@ def main():
             r = bench_matmul(ops, rt, timer, rng, m, 4096, 4096, 4, "f16", small, 10, 4 * 9437184)
             r["mfma_frac"] = r["tflops"] / MFMA_F16_PEAK_TF
             extra[f"q4_qmm_m{m}_4096"] = r
-        r = bench_matmul(ops, rt, timer, rng, 128, 12288, 4096, 8, "bf16", small, 10, 4 * 53477376)
-        r["mfma_frac"] = r["tflops"] / MFMA_F16_PEAK_TF
-        r["hbm_frac"] = r["gbs"] / HBM_PEAK_GBS
-        extra["q8_qmm_bf16_m128_n12288"] = r
+        for name, kern in (("q8_qmm_bf16_m128_n12288", rt.KERNEL_AUTO), ("q8_qmm_bf16_m128_n12288_bf16_mfma", rt.KERNEL_QMM_BF16)):
+            r = bench_matmul(ops, rt, timer, rng, 128, 12288, 4096, 8, "bf16", small, 10, 4 * 53477376, kernel=kern)
+            r["mfma_frac"] = r["tflops"] / MFMA_F16_PEAK_TF
+            r["hbm_frac"] = r["gbs"] / HBM_PEAK_GBS
+            extra[name] = r
         gate_up = make_weight(rng, 3072, 4096, 4, lead=(128,))
         down = make_weight(rng, 4096, 1536, 4, lead=(128,))
         experts = (gate_up, down, ops.QuantizedWeight.from_numpy(*gate_up, 64, 4),
@@ -205,7 +206,7 @@ def main():
                    "parity_max_err": head.get("max_err"), "parity_tol": head.get("tol")},
         "roofline": {"bound": "hbm", "achieved": head["gbs"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": head["gbs"] / HBM_PEAK_GBS, "traffic": None,
-                     "kernel": "qmv_q4_kernel<1,1>", "bytes_per_launch": head["bytes"],
+                     "kernel": "qmv_q4_kernel<1,1,false,true>", "bytes_per_launch": head["bytes"],
                      "avg_launch_us": head["us"]},
     }
     if not args.quick and "q4_qmm_m512_4096" in extra:
@@ -213,7 +214,7 @@ def main():
         line["secondary"] = {"metric": "Q4 qmm TFLOPS (M=512, K=N=4096)", "value": q["tflops"], "unit": "TFLOP/s",
                              "roofline": {"bound": "mfma", "achieved": q["tflops"], "peak": MFMA_F16_PEAK_TF,
                                           "unit": "TFLOP/s", "frac": q["mfma_frac"], "traffic": None,
-                                          "kernel": "qmm_kernel<128,64,4,false>", "avg_launch_us": q["us"]}}
+                                          "kernel": "qmm_kernel<128,64,4,false> (+ relayout_a_kernel)", "avg_launch_us": q["us"]}}
     if not args.no_cpu:
         line["cpu_baseline"] = cpu_baseline(np.random.default_rng(1001), 3.0 if args.quick else 10.0)
     line["extra"] = extra

@@ -108,7 +108,7 @@ bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) ==
 // 32 <= M < 128 and NAX above (crates/rmlx-core/src/ops/quantized.rs:7200-7256).  Here: the
 // streaming MFMA GEMV (weights read once for up to 8 rows) up to 16 rows, the LDS-staged MFMA
 // GEMM above, the portable kernel for every shape the fast kernels do not take.
-enum { KERNEL_AUTO = 0, KERNEL_QMV = 1, KERNEL_QMM = 2, KERNEL_GENERIC = 3 };
+enum { KERNEL_AUTO = 0, KERNEL_QMV = 1, KERNEL_QMM = 2, KERNEL_GENERIC = 3, KERNEL_QMM_BF16 = 4 };
 constexpr uint32_t kQmvMaxM = 16;
 
 int32_t run_matmul(const rmlx_qweight* qw, const void* x, int32_t x_dtype, uint32_t M, __half* out,
@@ -134,16 +134,21 @@ int32_t run_matmul(const rmlx_qweight* qw, const void* x, int32_t x_dtype, uint3
     return fail(RMLX_INVALID_SHAPE,
                 "qmm kernel requires bits in {4,8}, group_size=64, N %% 64 == 0, K %% 256 == 0 and 16-byte aligned "
                 "buffers (N=%u K=%u bits=%u group_size=%u)", N, K, qw->bits, qw->group_size);
-  } else if (kernel < 0 || kernel > KERNEL_GENERIC) {
+  } else if (kernel == KERNEL_QMM_BF16 && !(can_qmm && qw->bits == 8 && x_dtype == RMLX_DTYPE_BF16)) {
+    return fail(RMLX_INVALID_SHAPE, "the bf16 MFMA GEMM takes Bfloat16 activations and 8-bit weights (got %s, bits=%u)",
+                dtype_name(x_dtype), qw->bits);
+  } else if (kernel < 0 || kernel > KERNEL_QMM_BF16) {
     return fail(RMLX_NOT_FOUND, "unknown kernel selector %d", kernel);
   }
 
-  if (kernel == KERNEL_QMM) {
-    // The GEMM re-lays the activations out in MFMA operand order first (dtype cast fused in;
-    // bf16 stays bf16 for Q8 weights, everything else becomes f16).
+  if (kernel == KERNEL_QMM || kernel == KERNEL_QMM_BF16) {
+    // The GEMM re-lays the activations out in MFMA operand order first (dtype cast fused in).
+    // By default everything is multiplied in f16: bf16 -> f16 is exact for normal-range values and
+    // f16 weights keep 11 significant bits.  The bf16 MFMA variant (weights rounded to 8 bits)
+    // passes the tolerance with little margin, so it has to be asked for explicitly.
     Scratch ws;
     RMLX_TRY(ws.alloc(qmm_workspace_bytes(M, K), stream));
-    QmmArgs a{qw->w, qw->s, qw->b, x, x_dtype, out, M, N, K, qw->bits, ws.ptr};
+    QmmArgs a{qw->w, qw->s, qw->b, x, x_dtype, out, M, N, K, qw->bits, ws.ptr, kernel == KERNEL_QMM_BF16 ? 1 : 0};
     return launch_qmm(a, stream);
   }
 

@@ -137,6 +137,7 @@ struct QmmArgs {
   __half* out;        // [M,N]
   uint32_t M, N, K, bits;
   void* workspace;    // qmm_workspace_bytes(M, K) bytes of device scratch (fragment-major activations)
+  int bf16_mfma;      // 1: bf16 activations x Q8 weights on the bf16 MFMA (weights rounded to bf16)
 };
 size_t qmm_workspace_bytes(uint32_t M, uint32_t K);
 bool qmm_supported(uint32_t N, uint32_t K, uint32_t group_size, uint32_t bits);

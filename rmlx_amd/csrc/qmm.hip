@@ -375,7 +375,7 @@ int32_t launch_qmm(const QmmArgs& a, hipStream_t s) {
     return fail(RMLX_INVALID_SHAPE, "qmm: unsupported shape N=%u K=%u bits=%u", a.N, a.K, a.bits);
   if (a.M == 0) return RMLX_OK;
   if (a.workspace == nullptr) return fail(RMLX_RUNTIME_ERROR, "qmm: missing activation workspace");
-  const bool want_bf16 = a.bits == 8 && a.x_dtype == RMLX_DTYPE_BF16;
+  const bool want_bf16 = a.bf16_mfma && a.bits == 8 && a.x_dtype == RMLX_DTYPE_BF16;
   {
     const uint64_t units = (uint64_t)((a.M + 15) / 16) * (a.K / 32) * 64;
     uint64_t blocks = (units + 255) / 256;

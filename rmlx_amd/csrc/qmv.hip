@@ -210,60 +210,51 @@ __device__ __forceinline__ void qmv_pass(const KParams& p, char* xs, float* sums
   if (!FULLP) __syncthreads();
   QMV_MARK(p, 3);
 
-  // ---- 3. weights: integer dot per group via MFMA, independent slabs interleaved -------------
+  // ---- 3. weights: integer dot per group via MFMA (independent slabs interleaved), then
+  //         acc += scale * (dot - sum(off*x)) + bias * sum(x) in f32; one tile set at a time to
+  //         keep the register footprint at two workgroups per CU ----------------------------------
   // A-operand activity: accumulator rows 0-7 take group 0 (g<2), rows 8-15 group 1 (g>=2).
   const int am = n & 7;
   const bool a_active = ((n < 8) == (g < 2)) && (am < MR);
   const int a_slot_off = (g * MR + am) * 16;
-  f4 c[TILES][kSpwMax];
 #pragma unroll
-  for (int it = 0; it < kSpwMax; ++it)
+  for (int t = 0; t < TILES; ++t) {
+    f4 c[kSpwMax];
 #pragma unroll
-    for (int t = 0; t < TILES; ++t) c[t][it] = (f4){0.f, 0.f, 0.f, 0.f};
+    for (int it = 0; it < kSpwMax; ++it) c[it] = (f4){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    h8 av[kSpwMax];
+    for (int j = 0; j < 4; ++j) {
+      h8 av[kSpwMax];
 #pragma unroll
-    for (int it = 0; it < kSpwMax; ++it) {
-      av[it] = (h8){0, 0, 0, 0, 0, 0, 0, 0};
-      if ((FULLP || it < my) && a_active)
-        av[it] = *reinterpret_cast<const h8*>(xs + (((s0 + it) * 4 + j) * kSlots) * 16 + a_slot_off);
+      for (int it = 0; it < kSpwMax; ++it) {
+        av[it] = (h8){0, 0, 0, 0, 0, 0, 0, 0};
+        if ((FULLP || it < my) && a_active)
+          av[it] = *reinterpret_cast<const h8*>(xs + (((s0 + it) * 4 + j) * kSlots) * 16 + a_slot_off);
+      }
+#pragma unroll
+      for (int it = 0; it < kSpwMax; ++it) {
+        if (FULLP || it < my) {
+          const uint32_t wd = j == 0 ? wreg[t][it].x : (j == 1 ? wreg[t][it].y : (j == 2 ? wreg[t][it].z : wreg[t][it].w));
+          c[it] = __builtin_amdgcn_mfma_f32_16x16x32_f16(av[it], unpack_q4_word(wd), c[it], 0, 0, 0);
+        }
+      }
+    }
+    u4 sv, bv;
+    if (FULLP) {
+      const u4 other = (u4){swap16(sbv[t].x), swap16(sbv[t].y), swap16(sbv[t].z), swap16(sbv[t].w)};
+      sv = (g & 1) ? other : sbv[t];
+      bv = (g & 1) ? sbv[t] : other;
     }
 #pragma unroll
     for (int it = 0; it < kSpwMax; ++it) {
       if (FULLP || it < my) {
-#pragma unroll
-        for (int t = 0; t < TILES; ++t) {
-          const uint32_t wd = j == 0 ? wreg[t][it].x : (j == 1 ? wreg[t][it].y : (j == 2 ? wreg[t][it].z : wreg[t][it].w));
-          c[t][it] = __builtin_amdgcn_mfma_f32_16x16x32_f16(av[it], unpack_q4_word(wd), c[t][it], 0, 0, 0);
-        }
-      }
-    }
-  }
-  QMV_MARK(p, 4);
-
-  // ---- 4. acc += scale * (dot - sum(off*x)) + bias * sum(x), f32 -------------------------------
-  u4 sv[TILES], bv[TILES];
-  if (FULLP) {
-#pragma unroll
-    for (int t = 0; t < TILES; ++t) {
-      const u4 other = (u4){swap16(sbv[t].x), swap16(sbv[t].y), swap16(sbv[t].z), swap16(sbv[t].w)};
-      sv[t] = (g & 1) ? other : sbv[t];
-      bv[t] = (g & 1) ? sbv[t] : other;
-    }
-  }
-#pragma unroll
-  for (int it = 0; it < kSpwMax; ++it) {
-    if (FULLP || it < my) {
-      const float* sp = sums + (((s0 + it) * 2 + par) * 8 + (g & 1) * 4) * 2;
-      const f4 c01 = *reinterpret_cast<const f4*>(sp);      // (-xoff, xsum) of accumulator rows 4g, 4g+1
-      const f4 c23 = *reinterpret_cast<const f4*>(sp + 4);  // rows 4g+2, 4g+3
-#pragma unroll
-      for (int t = 0; t < TILES; ++t) {
+        const float* sp = sums + (((s0 + it) * 2 + par) * 8 + (g & 1) * 4) * 2;
+        const f4 c01 = *reinterpret_cast<const f4*>(sp);      // (-xoff, xsum) of accumulator rows 4g, 4g+1
+        const f4 c23 = *reinterpret_cast<const f4*>(sp + 4);  // rows 4g+2, 4g+3
         uint32_t sbits, bbits;
         if (FULLP) {  // group 2*it + par of the 8 loaded ones: word `it`, half `par`
-          const uint32_t swd = it == 0 ? sv[t].x : (it == 1 ? sv[t].y : (it == 2 ? sv[t].z : sv[t].w));
-          const uint32_t bwd = it == 0 ? bv[t].x : (it == 1 ? bv[t].y : (it == 2 ? bv[t].z : bv[t].w));
+          const uint32_t swd = it == 0 ? sv.x : (it == 1 ? sv.y : (it == 2 ? sv.z : sv.w));
+          const uint32_t bwd = it == 0 ? bv.x : (it == 1 ? bv.y : (it == 2 ? bv.z : bv.w));
           sbits = par ? swd >> 16 : swd & 0xFFFFu;
           bbits = par ? bwd >> 16 : bwd & 0xFFFFu;
         } else {
@@ -273,17 +264,21 @@ __device__ __forceinline__ void qmv_pass(const KParams& p, char* xs, float* sums
         }
         const float sc = __half2float(__ushort_as_half((unsigned short)sbits));
         const float bi = __half2float(__ushort_as_half((unsigned short)bbits));
-        F[t][0] += sc * (c[t][it][0] + c01[0]) + bi * c01[1];
-        F[t][1] += sc * (c[t][it][1] + c01[2]) + bi * c01[3];
-        F[t][2] += sc * (c[t][it][2] + c23[0]) + bi * c23[1];
-        F[t][3] += sc * (c[t][it][3] + c23[2]) + bi * c23[3];
+        F[t][0] += sc * (c[it][0] + c01[0]) + bi * c01[1];
+        F[t][1] += sc * (c[it][1] + c01[2]) + bi * c01[3];
+        F[t][2] += sc * (c[it][2] + c23[0]) + bi * c23[1];
+        F[t][3] += sc * (c[it][3] + c23[2]) + bi * c23[3];
       }
     }
+    if (TILES > 1) __builtin_amdgcn_sched_barrier(0);  // finish one tile set before the next (registers)
   }
+  QMV_MARK(p, 4);
 }
 
 // MR = activation rows staged per pass (1, 2, 4 or 8); TILES = 1, or 2 for fused gate/up.
-template <int MR, int TILES, bool TAB>
+// ALLFULL: K is a multiple of 4096, the partial-pass code is not instantiated (fewer registers:
+// two workgroups fit on a CU).
+template <int MR, int TILES, bool TAB, bool ALLFULL>
 __global__ __launch_bounds__(kThreads) void qmv_q4_kernel(KParams p) {
   constexpr int kSlots = 4 * MR;                              // 16-byte slots per (slab, j)
   constexpr int kXsBytes = kChunkSlabs * 4 * kSlots * 16;     // activation image
@@ -331,9 +326,9 @@ __global__ __launch_bounds__(kThreads) void qmv_q4_kernel(KParams p) {
 
   for (uint32_t kc = 0; kc < K; kc += kChunkSlabs * 128) {
     const uint32_t left = (K - kc) / 128;
-    if (left >= (uint32_t)kChunkSlabs)
+    if (ALLFULL || left >= (uint32_t)kChunkSlabs)
       qmv_pass<MR, TILES, TAB, true>(p, xs, sums, sbs, wrow, F, kc, kChunkSlabs, expert, row0, rows, tile_row, kc == 0);
-    else
+    else if (!ALLFULL)
       qmv_pass<MR, TILES, TAB, false>(p, xs, sums, sbs, wrow, F, kc, (int)left, expert, row0, rows, tile_row, kc == 0);
   }
 
@@ -373,8 +368,14 @@ __global__ __launch_bounds__(kThreads) void qmv_q4_kernel(KParams p) {
 
 template <int MR, int TILES>
 void launch_t(const KParams& p, bool tab, dim3 grid, hipStream_t s) {
-  if (tab) hipLaunchKernelGGL((qmv_q4_kernel<MR, TILES, true>), grid, dim3(kThreads), 0, s, p);
-  else hipLaunchKernelGGL((qmv_q4_kernel<MR, TILES, false>), grid, dim3(kThreads), 0, s, p);
+  const bool allfull = p.K % (kChunkSlabs * 128) == 0;
+  if (tab) {
+    if (allfull) hipLaunchKernelGGL((qmv_q4_kernel<MR, TILES, true, true>), grid, dim3(kThreads), 0, s, p);
+    else hipLaunchKernelGGL((qmv_q4_kernel<MR, TILES, true, false>), grid, dim3(kThreads), 0, s, p);
+  } else {
+    if (allfull) hipLaunchKernelGGL((qmv_q4_kernel<MR, TILES, false, true>), grid, dim3(kThreads), 0, s, p);
+    else hipLaunchKernelGGL((qmv_q4_kernel<MR, TILES, false, false>), grid, dim3(kThreads), 0, s, p);
+  }
 }
 
 __global__ void build_gather_chunks_kernel(const uint32_t* indices, uint32_t batch, uint32_t mpb,

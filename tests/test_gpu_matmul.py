@@ -111,7 +111,21 @@ def test_config4_q8_qmm_bf16(hip):
     words, s, b = make_weight(rng, n, k, 8)
     x = make_x(rng, m, k, "bf16")
     ref = model.qmm(x_as_f64(x, "bf16"), words, s, b, 64, 8)
-    assert_close(_run(hip, words, s, b, x, 8, dtype="bf16"), ref, "config4")
+    err_auto, tol = assert_close(_run(hip, words, s, b, x, 8, dtype="bf16"), ref, "config4 (f16 MFMA, default)")
+    # the bf16 matrix-instruction variant: weights rounded to 8 significant bits, still inside the bar
+    err_bf16, _ = assert_close(_run(hip, words, s, b, x, 8, dtype="bf16", kernel=4), ref, "config4 (bf16 MFMA)")
+    assert err_auto < err_bf16
+
+
+def test_bf16_mfma_variant_is_only_for_q8_bf16(hip):
+    from rmlx_amd import ops
+    rng = np.random.default_rng(16)
+    words, s, b = make_weight(rng, 64, 256, 8)
+    with pytest.raises(ops.KernelError, match="bf16 MFMA GEMM takes Bfloat16"):
+        _run(hip, words, s, b, make_x(rng, 32, 256), 8, kernel=4)
+    words, s, b = make_weight(rng, 64, 256, 4)
+    with pytest.raises(ops.KernelError, match="bf16 MFMA GEMM takes Bfloat16"):
+        _run(hip, words, s, b, make_x(rng, 32, 256, "bf16"), 4, dtype="bf16", kernel=4)
 
 
 # ---- kernel families agree, ragged M, dtypes, other group sizes --------------------------------------
