@@ -24,6 +24,12 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0      # MI355X HBM3E
 MFMA_F16_PEAK_TF = 2500.0  # dense f16 / bf16 MFMA
 
+# HBM-side bytes per launch of the two roofline kernels, from rocprofv3 counter runs of this script
+# (FETCH_SIZE and WRITE_SIZE, each scaled by what it reads for the plain copy below); the runs and
+# the scaling are recorded in profiles/bench_all_configs_hbm_traffic_pmc.txt.  Counters cannot be
+# read from inside this process, so the figures are carried here and re-measured with the kernels.
+MEASURED_TRAFFIC_BYTES = {"qmv_q4_m1_4096": 9509664, "qmm_q4_m512_4096": 46988000}
+
 
 def matmul_bytes(m, n, k, bits, gs=64, act_bytes=2):
     """Algorithmic bytes of one quantized matmul: packed weights + f16 scales and biases +
@@ -163,6 +169,16 @@ def main():
     # ---- headline: Q4 qmv M=1 K=N=4096, weights cycled through > 1 GiB ---------------------------------
     head = bench_matmul(ops, rt, timer, rng, 1, 4096, 4096, 4, "f16", args.steps, args.warmup, GiB + GiB // 8)
     extra = {"device": info, "q4_qmv_m1_4096": head}
+    # A plain copy of known size (identity `index_gather`, 128 MiB in, 128 MiB out) so that a counter
+    # run of this same command can scale FETCH_SIZE / WRITE_SIZE by what they read for it.
+    rows = 16384
+    src = rt.DeviceBuffer((rows, 4096), rt.F16)
+    ident = rt.DeviceBuffer.from_numpy(np.arange(rows, dtype=np.uint32))
+    ops.index_gather(src, ident, stream=timer.stream)
+    timer.stream.sync()
+    extra["copy_calibration"] = {"kernel": "index_gather_kernel", "read_bytes": rows * 4096 * 2 + rows * 4,
+                                 "write_bytes": rows * 4096 * 2}
+    del src, ident
     if not args.quick:
         small = max(20, args.steps // 20)
         extra["q4_qmv_m1_4096_cache_resident"] = bench_matmul(ops, rt, timer, rng, 1, 4096, 4096, 4, "f16",
@@ -205,15 +221,16 @@ def main():
                                f"{head['n_weight_sets']} distinct weight sets cycled (HBM-resident, > 1 GiB)",
                    "parity_max_err": head.get("max_err"), "parity_tol": head.get("tol")},
         "roofline": {"bound": "hbm", "achieved": head["gbs"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": head["gbs"] / HBM_PEAK_GBS, "traffic": None,
-                     "kernel": "qmv_q4_kernel<1,1,false,true>", "bytes_per_launch": head["bytes"],
+                     "frac": head["gbs"] / HBM_PEAK_GBS, "traffic": MEASURED_TRAFFIC_BYTES["qmv_q4_m1_4096"],
+                     "kernel": "qmv_q4_kernel<1,1,false,4>", "bytes_per_launch": head["bytes"],
                      "avg_launch_us": head["us"]},
     }
     if not args.quick and "q4_qmm_m512_4096" in extra:
         q = extra["q4_qmm_m512_4096"]
         line["secondary"] = {"metric": "Q4 qmm TFLOPS (M=512, K=N=4096)", "value": q["tflops"], "unit": "TFLOP/s",
                              "roofline": {"bound": "mfma", "achieved": q["tflops"], "peak": MFMA_F16_PEAK_TF,
-                                          "unit": "TFLOP/s", "frac": q["mfma_frac"], "traffic": None,
+                                          "unit": "TFLOP/s", "frac": q["mfma_frac"],
+                                          "traffic": MEASURED_TRAFFIC_BYTES["qmm_q4_m512_4096"],
                                           "kernel": "qmm_kernel<128,64,4,false> (+ relayout_a_kernel)", "avg_launch_us": q["us"]}}
     if not args.no_cpu:
         line["cpu_baseline"] = cpu_baseline(np.random.default_rng(1001), 3.0 if args.quick else 10.0)
