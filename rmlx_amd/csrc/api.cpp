@@ -108,7 +108,7 @@ bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) ==
 // 32 <= M < 128 and NAX above (crates/rmlx-core/src/ops/quantized.rs:7200-7256).  Here: the
 // streaming MFMA GEMV (weights read once for up to 8 rows) up to 16 rows, the LDS-staged MFMA
 // GEMM above, the portable kernel for every shape the fast kernels do not take.
-enum { KERNEL_AUTO = 0, KERNEL_QMV = 1, KERNEL_QMM = 2, KERNEL_GENERIC = 3, KERNEL_QMM_BF16 = 4 };
+enum { KERNEL_AUTO = 0, KERNEL_QMV = 1, KERNEL_QMM = 2, KERNEL_GENERIC = 3, KERNEL_QMM_BF16 = 4, KERNEL_QMM_LDS = 5 };
 constexpr uint32_t kQmvMaxM = 16;
 
 int32_t run_matmul(const rmlx_qweight* qw, const void* x, int32_t x_dtype, uint32_t M, __half* out,
@@ -119,7 +119,9 @@ int32_t run_matmul(const rmlx_qweight* qw, const void* x, int32_t x_dtype, uint3
   if (M == 0) return RMLX_OK;
   const bool ptr_ok = aligned16(qw->w) && aligned16(qw->s) && aligned16(qw->b) && aligned16(x);
   const bool can_qmv = qw->bits == 4 && ptr_ok && qmv_q4_supported(N, K, qw->group_size);
-  const bool can_qmm = ptr_ok && qmm_supported(N, K, qw->group_size, qw->bits);
+  const bool can_qmm_lds = ptr_ok && qmm_supported(N, K, qw->group_size, qw->bits);
+  const bool can_qmm_rw = ptr_ok && qmm_rw_supported(N, K, qw->group_size, qw->bits);
+  const bool can_qmm = can_qmm_lds || can_qmm_rw;
 
   if (kernel == KERNEL_AUTO) {
     if (can_qmv && M <= kQmvMaxM) kernel = KERNEL_QMV;
@@ -134,15 +136,32 @@ int32_t run_matmul(const rmlx_qweight* qw, const void* x, int32_t x_dtype, uint3
     return fail(RMLX_INVALID_SHAPE,
                 "qmm kernel requires bits in {4,8}, group_size=64, N %% 64 == 0, K %% 256 == 0 and 16-byte aligned "
                 "buffers (N=%u K=%u bits=%u group_size=%u)", N, K, qw->bits, qw->group_size);
-  } else if (kernel == KERNEL_QMM_BF16 && !(can_qmm && qw->bits == 8 && x_dtype == RMLX_DTYPE_BF16)) {
+  } else if (kernel == KERNEL_QMM_LDS && !can_qmm_lds) {
+    return fail(RMLX_INVALID_SHAPE,
+                "the LDS-staged qmm kernel requires bits in {4,8}, group_size=64, N %% 64 == 0, K %% 256 == 0 and "
+                "16-byte aligned buffers (N=%u K=%u bits=%u group_size=%u)", N, K, qw->bits, qw->group_size);
+  } else if (kernel == KERNEL_QMM_BF16 && !(can_qmm_lds && qw->bits == 8 && x_dtype == RMLX_DTYPE_BF16)) {
     return fail(RMLX_INVALID_SHAPE, "the bf16 MFMA GEMM takes Bfloat16 activations and 8-bit weights (got %s, bits=%u)",
                 dtype_name(x_dtype), qw->bits);
-  } else if (kernel < 0 || kernel > KERNEL_QMM_BF16) {
+  } else if (kernel < 0 || kernel > KERNEL_QMM_LDS) {
     return fail(RMLX_NOT_FOUND, "unknown kernel selector %d", kernel);
   }
 
-  if (kernel == KERNEL_QMM || kernel == KERNEL_QMM_BF16) {
-    // The GEMM re-lays the activations out in MFMA operand order first (dtype cast fused in).
+  if (kernel == KERNEL_QMM && can_qmm_rw) {
+    // Register-weights GEMM: f16 activations straight from the row-major matrix, no workspace.
+    // bf16 -> f16 is exact for normal-range values and f16 weights keep 11 significant bits.
+    Scratch cast;
+    const void* xk = x;
+    if (x_dtype != RMLX_DTYPE_F16) {
+      RMLX_TRY(cast.alloc((size_t)M * K * sizeof(__half), stream));
+      RMLX_TRY(launch_cast_to_f16(x, x_dtype, static_cast<__half*>(cast.ptr), (size_t)M * K, stream));
+      xk = cast.ptr;
+    }
+    QmmArgs a{qw->w, qw->s, qw->b, xk, RMLX_DTYPE_F16, out, M, N, K, qw->bits, nullptr, 0};
+    return launch_qmm_rw(a, qw->group_size, stream);
+  }
+  if (kernel == KERNEL_QMM || kernel == KERNEL_QMM_BF16 || kernel == KERNEL_QMM_LDS) {
+    // The LDS-staged GEMM re-lays the activations out in MFMA operand order first (dtype cast fused in).
     // By default everything is multiplied in f16: bf16 -> f16 is exact for normal-range values and
     // f16 weights keep 11 significant bits.  The bf16 MFMA variant (weights rounded to 8 bits)
     // passes the tolerance with little margin, so it has to be asked for explicitly.

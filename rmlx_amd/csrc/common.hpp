@@ -142,6 +142,9 @@ struct QmmArgs {
 size_t qmm_workspace_bytes(uint32_t M, uint32_t K);
 bool qmm_supported(uint32_t N, uint32_t K, uint32_t group_size, uint32_t bits);
 int32_t launch_qmm(const QmmArgs& a, hipStream_t s);
+// Register-weights GEMM (qmm_rw.hip): f16 activations only, no workspace.
+bool qmm_rw_supported(uint32_t N, uint32_t K, uint32_t group_size, uint32_t bits);
+int32_t launch_qmm_rw(const QmmArgs& a, uint32_t group_size, hipStream_t s);
 
 // MoE helpers
 int32_t launch_topk_route(const float* logits, const float* bias, uint32_t T, uint32_t E, uint32_t K,

@@ -1,0 +1,402 @@
+// Quantized GEMM for gfx950 (prefill, M > 16) with the weights kept in registers.
+//
+// Replaces the reference's affine_qmm_nax_q4 / affine_qmm_steel4sg_splitk_q4 /
+// affine_qmm_mma_q8 (crates/rmlx-core/src/ops/quantized.rs:3331-3565, 4572-4786, 5838-5971).
+//
+// Design (wave64, v_mfma_f32_16x16x32_f16, f32 accumulation, f16 output):
+//   * Weights never touch LDS.  Lane (n = lane%16, g = lane/16) of a wave loads 16 bytes of
+//     weight row n: the 32 (Q4) or 16 (Q8) values of its lane group inside a 128-wide k block.
+//     Word j of that load is dequantized in registers straight into the MFMA operand of product
+//     j of the block (exact magic-number int -> f16 conversion, then w = s*q + b in packed f16),
+//     so product j multiplies a k set that is not a contiguous run; the activation operand is
+//     laid out to match.  With group size 64 all values of a lane belong to one quantisation
+//     group, so a lane needs a single (scale, bias) pair per load; the pairs of four iterations
+//     come in one 16-byte load per weight row.
+//   * The waves of a workgroup (4 or 8) split the N extent of the tile: every weight is loaded
+//     and dequantized by exactly one wave.
+//   * Activations are shared by the waves and go through LDS.  They are read from the row-major
+//     [M,K] matrix with coalesced 16-byte loads (16 lanes per 256-byte row piece), permuted to
+//     the slot order of the nibble unpacking and written to an xor-swizzled operand layout, so
+//     both the writes and the 16-byte operand reads are bank-conflict free.  No prepass, no
+//     workspace.
+//   * Register rings keep global loads four 128-wide k blocks ahead (weights) and the LDS copy two
+//     blocks ahead (4-stage LDS ring); one barrier per block.  Every step of a block (the MFMAs
+//     of one weight fragment and product) carries its share of the block's LDS writes and global
+//     loads and unpacks the next weight operand, so memory instructions, VALU work and MFMAs
+//     alternate in the instruction stream instead of arriving in bursts.
+//   * Workgroup ids are remapped so that the tiles sharing a weight panel run on one XCD (one L2).
+#include "common.hpp"
+
+namespace rmlx {
+namespace {
+
+typedef _Float16 h8 __attribute__((ext_vector_type(8)));
+typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+typedef float f4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u2 __attribute__((ext_vector_type(2)));
+
+constexpr int kBlockK = 128;  // k extent of one main-loop iteration
+constexpr int kStages = 4;
+constexpr int kUnroll = 4;   // main-loop unrolling = depth of the weight register ring
+
+struct RwParams {
+  const uint32_t* w; const __half* s; const __half* b;
+  const __half* x;   // [M,K] f16 row-major
+  __half* out;
+  uint32_t M, N, K;
+  uint32_t tiles_m, tiles_n;
+#ifdef QMM_RW_TRACE
+  unsigned long long* trace;
+#endif
+};
+
+#ifdef QMM_RW_TRACE
+#ifndef RW_TRACE_WG
+#define RW_TRACE_WG 0
+#endif
+#define RW_MARK(p, it, i)                                                                          \
+  do {                                                                                             \
+    if ((p).trace != nullptr && blockIdx.x == RW_TRACE_WG && (threadIdx.x & 63) == 0 && (it) >= 8 && (it) < 12) \
+      (p).trace[((threadIdx.x >> 6) * 4 + ((it) - 8)) * 8 + (i)] = __builtin_readcyclecounter();    \
+  } while (0)
+#define RW_MARK_ALL(p, i)                                                              \
+  do {                                                                                 \
+    if ((p).trace != nullptr && threadIdx.x == 0)                                      \
+      (p).trace[1024 + blockIdx.x * 2 + (i)] = __builtin_readcyclecounter();            \
+  } while (0)
+#else
+#define RW_MARK(p, it, i) do {} while (0)
+#define RW_MARK_ALL(p, i) do {} while (0)
+#endif
+
+__device__ __forceinline__ uint32_t h2bits(h2 v) { return __builtin_bit_cast(uint32_t, v); }
+
+// 8 Q4 values of one word -> 8 f16 weights in slot order (k0,k4,k1,k5,k2,k6,k3,k7), w = s*q + b.
+// The int -> f16 conversion is exact: (w & 0x000F000F) | 0x64006400 is the pair (1024+q0, 1024+q4),
+// (w & 0x00F000F0) | 0x54005400 is (64+q1, 64+q5); the offsets are subtracted before scaling.
+struct DqConst { uint32_t m0, m1, k0, k1; };
+__device__ __forceinline__ h8 dequant_q4_word(uint32_t w, h2 s2, h2 b2, const DqConst& c) {
+  const uint32_t t = w >> 8;
+  const h2 k1024 = {(_Float16)1024.0f, (_Float16)1024.0f}, k64 = {(_Float16)64.0f, (_Float16)64.0f};
+  const h2 p0 = __builtin_bit_cast(h2, (w & c.m0) | c.k0) - k1024;
+  const h2 p1 = __builtin_bit_cast(h2, (w & c.m1) | c.k1) - k64;
+  const h2 p2 = __builtin_bit_cast(h2, (t & c.m0) | c.k0) - k1024;
+  const h2 p3 = __builtin_bit_cast(h2, (t & c.m1) | c.k1) - k64;
+  u4 o;
+  o.x = h2bits(p0 * s2 + b2);
+  o.y = h2bits(p1 * s2 + b2);
+  o.z = h2bits(p2 * s2 + b2);
+  o.w = h2bits(p3 * s2 + b2);
+  return __builtin_bit_cast(h8, o);
+}
+
+// 8 Q8 values of two words -> 8 f16 weights in natural order.
+__device__ __forceinline__ h8 dequant_q8_pair(uint32_t w0, uint32_t w1, h2 s2, h2 b2) {
+  const h2 k1024 = {(_Float16)1024.0f, (_Float16)1024.0f};
+  const h2 p0 = __builtin_bit_cast(h2, __builtin_amdgcn_perm(0x64646464u, w0, 0x04010400u)) - k1024;
+  const h2 p1 = __builtin_bit_cast(h2, __builtin_amdgcn_perm(0x64646464u, w0, 0x04030402u)) - k1024;
+  const h2 p2 = __builtin_bit_cast(h2, __builtin_amdgcn_perm(0x64646464u, w1, 0x04010400u)) - k1024;
+  const h2 p3 = __builtin_bit_cast(h2, __builtin_amdgcn_perm(0x64646464u, w1, 0x04030402u)) - k1024;
+  u4 o;
+  o.x = h2bits(p0 * s2 + b2);
+  o.y = h2bits(p1 * s2 + b2);
+  o.z = h2bits(p2 * s2 + b2);
+  o.w = h2bits(p3 * s2 + b2);
+  return __builtin_bit_cast(h8, o);
+}
+
+// MF = 16-row activation fragments per workgroup (tile rows = 16*MF), NF = 16-row weight fragments
+// per wave (tile columns = 64*NF), BITS = 4 or 8.
+template <int MF, int NF, int BITS, int NW>
+__global__ __launch_bounds__(64 * NW) void qmm_rw_kernel(RwParams p) {
+  constexpr int kThreads = 64 * NW;
+  constexpr int AL = MF * 256 / kThreads;      // 16-byte activation loads per thread and chunk
+  static_assert(AL * kThreads == MF * 256, "chunk must divide over the workgroup");
+  constexpr int kChunk = MF * 4 * 64;          // 16-byte units of one activation chunk
+  constexpr int WL = BITS == 4 ? 1 : 2;        // 16-byte weight loads per lane, fragment and iteration
+  __shared__ u4 a_lds[kStages * kChunk];
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int n = lane & 15, g = lane >> 4;
+  RW_MARK(p, 8, 6);
+  RW_MARK_ALL(p, 0);
+
+  // Workgroups that share a weight panel get ids that are congruent mod 8 apart, i.e. run on one XCD.
+  uint32_t wg = blockIdx.x;
+  const uint32_t total = p.tiles_m * p.tiles_n;
+  if (total % 8 == 0) wg = (wg % 8) * (total / 8) + wg / 8;
+  const uint32_t mt = wg % p.tiles_m, nt = wg / p.tiles_m;
+
+  const uint32_t K = p.K, S = K / kBlockK, G = K / 64;
+  const uint32_t row_base = nt * (NW * 16 * NF) + wave * (16 * NF) + n;
+
+  const u4* wptr[NF];
+  const __half* sptr[NF];
+  const __half* bptr[NF];
+#pragma unroll
+  for (int f = 0; f < NF; ++f) {
+    const uint64_t row = row_base + f * 16;
+    wptr[f] = reinterpret_cast<const u4*>(p.w + row * (K * BITS / 32)) + g;
+    sptr[f] = p.s + row * G;
+    bptr[f] = p.b + row * G;
+  }
+  // Activation chunk of an iteration: 16*MF rows x 128 k = 16 sixteen-byte segments per row.  Unit
+  // q*kThreads + tid -> (row, segment): 16 consecutive lanes read one row's 256 contiguous bytes.
+  // Segment seg holds k offsets 8*seg..8*seg+7, i.e. product j / lane group gq of the operand
+  // layout; inside LDS the 16-byte slot of (fragment i, product j, lane gq*16 + r) is
+  // (i*4 + j)*64 + gq*16 + (r ^ (4*j + gq)): the xor spreads the 16 lanes of a row over all banks
+  // on the write and stays a permutation of a product's 64 slots on the read.
+  const __half* xsrc[AL];
+  uint32_t lds_w[AL];
+#pragma unroll
+  for (int q = 0; q < AL; ++q) {
+    const uint32_t unit = q * kThreads + tid, r = unit >> 4, seg = unit & 15;
+    uint32_t row = mt * (16 * MF) + r;
+    if (row >= p.M) row = p.M - 1;  // rows past M are computed on stale data and never stored
+    xsrc[q] = p.x + (uint64_t)row * K + seg * 8;
+    const uint32_t j = BITS == 4 ? (seg & 3) : (2 * (seg >> 3) + (seg & 1));
+    const uint32_t gq = BITS == 4 ? (seg >> 2) : ((seg >> 1) & 3);
+    lds_w[q] = ((r >> 4) * 4 + j) * 64 + gq * 16 + ((r & 15) ^ (4 * j + gq));
+  }
+  uint32_t lds_r[4];  // read slot of this lane for product j (fragment i adds 256)
+#pragma unroll
+  for (int j = 0; j < 4; ++j) lds_r[j] = j * 64 + g * 16 + (n ^ (4 * j + g));
+
+  f4 acc[MF][NF];
+#pragma unroll
+  for (int i = 0; i < MF; ++i)
+#pragma unroll
+    for (int f = 0; f < NF; ++f) acc[i][f] = (f4){0.f, 0.f, 0.f, 0.f};
+
+  // Register rings: activation chunks travel global -> registers -> LDS (two sets: a chunk is loaded
+  // three iterations before it is used and written to LDS one iteration before); weights are
+  // loaded four iterations ahead (set = iteration % 4); the scales and biases of four iterations
+  // (eight groups = 16 bytes per row) come in one load per fragment, one block of four ahead.
+  // The loop is unrolled by four so that every ring index is a compile-time constant.
+  u4 ra[2][AL];
+  u4 wq[kUnroll][NF][WL];
+  u4 s_cur[NF], b_cur[NF], s_nxt[NF], b_nxt[NF];
+
+  // Q4: halves (k0..k7) -> slots (k0,k4,k1,k5,k2,k6,k3,k7), the order the nibble unpacking produces
+  auto to_slot_order = [&](u4 v) {
+    if (BITS != 4) return v;
+    u4 o;
+    o.x = __builtin_amdgcn_perm(v.z, v.x, 0x05040100u);
+    o.y = __builtin_amdgcn_perm(v.z, v.x, 0x07060302u);
+    o.z = __builtin_amdgcn_perm(v.w, v.y, 0x05040100u);
+    o.w = __builtin_amdgcn_perm(v.w, v.y, 0x07060302u);
+    return o;
+  };
+  auto load_a = [&](uint32_t it, u4 (&dst)[AL]) {
+#pragma unroll
+    for (int q = 0; q < AL; ++q) {
+      dst[q] = *reinterpret_cast<const u4*>(xsrc[q] + (uint64_t)it * kBlockK);
+    }
+  };
+  auto store_a = [&](uint32_t stage, const u4 (&src)[AL]) {
+#pragma unroll
+    for (int q = 0; q < AL; ++q) a_lds[stage * kChunk + lds_w[q]] = to_slot_order(src[q]);
+  };
+  auto load_sb = [&](uint32_t blk, u4 (&ds)[NF], u4 (&db)[NF]) {
+#pragma unroll
+    for (int f = 0; f < NF; ++f) {
+      ds[f] = reinterpret_cast<const u4*>(sptr[f])[blk];
+      db[f] = reinterpret_cast<const u4*>(bptr[f])[blk];
+    }
+  };
+  auto load_w = [&](uint32_t it, u4 (&dst)[NF][WL]) {
+#pragma unroll
+    for (int f = 0; f < NF; ++f)
+#pragma unroll
+      for (int h = 0; h < WL; ++h) {
+        dst[f][h] = wptr[f][(uint64_t)it * (4 * WL) + h * 4];
+      }
+  };
+  const uint32_t last = S - 1, last_blk = S / kUnroll - 1;
+  auto clampi = [&](uint32_t it) { return it < last ? it : last; };
+
+  // Constants of the unpacking kept in registers so that and+or is one instruction.
+  DqConst dq;
+  dq.m0 = 0x000F000Fu; dq.m1 = 0x00F000F0u; dq.k0 = 0x64006400u; dq.k1 = 0x54005400u;
+  asm volatile("" : "+s"(dq.m0), "+s"(dq.m1), "+v"(dq.k0), "+v"(dq.k1));
+  // Q4: the lane's group within a 128-wide block is g/2 -> which half of the f16 pair it scales with
+  const uint32_t sel_lane = (g >> 1) ? 0x03020302u : 0x01000100u;
+
+  // scale / bias operand pairs of iteration slot u of the current block (u == kUnroll: first
+  // iteration of the next block)
+  auto scale_pair = [&](int u, int f, int h, h2& s2, h2& b2) {
+    const u4 sv = u < kUnroll ? s_cur[f] : s_nxt[f], bv = u < kUnroll ? b_cur[f] : b_nxt[f];
+    const int w = u % kUnroll;
+    const uint32_t sw = w == 0 ? sv.x : (w == 1 ? sv.y : (w == 2 ? sv.z : sv.w));
+    const uint32_t bw = w == 0 ? bv.x : (w == 1 ? bv.y : (w == 2 ? bv.z : bv.w));
+    const uint32_t sel = BITS == 4 ? sel_lane : (h ? 0x03020302u : 0x01000100u);
+    s2 = __builtin_bit_cast(h2, __builtin_amdgcn_perm(sw, sw, sel));
+    b2 = __builtin_bit_cast(h2, __builtin_amdgcn_perm(bw, bw, sel));
+  };
+  // weight operand of step (j, f) of iteration slot u (u == kUnroll: slot 0 of the next block)
+  auto weight_operand = [&](int u, int j, int f) -> h8 {
+    h2 s2, b2;
+    if (BITS == 4) {
+      const u4 q = wq[u % kUnroll][f][0];
+      const uint32_t word = j == 0 ? q.x : (j == 1 ? q.y : (j == 2 ? q.z : q.w));
+      scale_pair(u, f, 0, s2, b2);
+      return dequant_q4_word(word, s2, b2, dq);
+    } else {
+      constexpr int hmax = WL - 1;
+      const int h = (j >> 1) < hmax ? (j >> 1) : hmax;
+      const u4 q = wq[u % kUnroll][f][h];
+      const uint32_t w0 = (j & 1) ? q.z : q.x, w1 = (j & 1) ? q.w : q.y;
+      scale_pair(u, f, h, s2, b2);
+      return dequant_q8_pair(w0, w1, s2, b2);
+    }
+  };
+
+  // ---- prologue: chunks 0 and 1 go to LDS, chunks 2 and 3 wait in the register sets ---------------
+  load_a(0, ra[0]);
+  load_a(clampi(1), ra[1]);
+  load_sb(0, s_cur, b_cur);
+#pragma unroll
+  for (int u = 0; u < kUnroll; ++u) load_w(clampi(u), wq[u]);
+  store_a(0, ra[0]);
+  store_a(1, ra[1]);
+  load_a(clampi(2), ra[0]);
+  load_a(clampi(3), ra[1]);
+  __syncthreads();
+
+  constexpr int NS = 4 * NF;  // steps of an iteration: (product j, fragment f), MF MFMAs each
+  h8 a_cur[MF], a_nxt[MF];
+#pragma unroll
+  for (int i = 0; i < MF; ++i) a_cur[i] = __builtin_bit_cast(h8, a_lds[i * 256 + lds_r[0]]);
+  h8 wv_cur = weight_operand(0, 0, 0), wv_nxt;
+
+  for (uint32_t it0 = 0; it0 < S; it0 += kUnroll) {
+    const uint32_t blk = it0 / kUnroll;
+    load_sb(blk < last_blk ? blk + 1 : last_blk, s_nxt, b_nxt);
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) {
+      const uint32_t it = it0 + u;
+      RW_MARK(p, it, 0);
+      const u4* a_stage = a_lds + (it % kStages) * kChunk;
+      const u4* a_stage_next = a_lds + ((it + 1) % kStages) * kChunk;
+      u4* a_stage_write = a_lds + ((it + 2) % kStages) * kChunk;
+#pragma unroll
+      for (int s = 0; s < NS; ++s) {
+        const int j = s / NF, f = s % NF;
+        // operands of the next product (of the next iteration after the last one: that chunk was
+        // written two iterations ago, so it is visible before this iteration's barrier)
+        if (f == 0) {
+#pragma unroll
+          for (int i = 0; i < MF; ++i)
+            a_nxt[i] = __builtin_bit_cast(h8, j < 3 ? a_stage[i * 256 + lds_r[j < 3 ? j + 1 : 0]] : a_stage_next[i * 256 + lds_r[0]]);
+        }
+        // this step's share of the ring traffic: LDS writes of chunk it+2 in the first half, the
+        // global loads of chunk it+4 into the same registers in the second half, weights last
+#pragma unroll
+        for (int q = 0; q < AL; ++q) {
+          if (s == q * NS / (2 * AL)) a_stage_write[lds_w[q]] = to_slot_order(ra[u % 2][q]);
+          if (s == NS / 2 + q * NS / (2 * AL)) {
+            ra[u % 2][q] = *reinterpret_cast<const u4*>(xsrc[q] + (uint64_t)clampi(it + 4) * kBlockK);
+          }
+        }
+        // next weight operand (the one of the first step of the next iteration after the last step)
+        if (s + 1 < NS) wv_nxt = weight_operand(u, (s + 1) / NF, (s + 1) % NF);
+        else wv_nxt = weight_operand(u + 1, 0, 0);
+#pragma unroll
+        for (int i = 0; i < MF; ++i)
+          acc[i][f] = __builtin_amdgcn_mfma_f32_16x16x32_f16(wv_cur, a_cur[i], acc[i][f], 0, 0, 0);
+        if (s == NS - 1) load_w(clampi(it + kUnroll), wq[u]);  // every word of wq[u] has been unpacked
+        if (f == NF - 1) {
+#pragma unroll
+          for (int i = 0; i < MF; ++i) a_cur[i] = a_nxt[i];
+        }
+        wv_cur = wv_nxt;
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      RW_MARK(p, it, 4);
+      __syncthreads();
+      RW_MARK(p, it, 5);
+    }
+#pragma unroll
+    for (int f = 0; f < NF; ++f) { s_cur[f] = s_nxt[f]; b_cur[f] = b_nxt[f]; }
+  }
+
+  // ---- epilogue: lane holds row m = lane%16 of fragment i, columns 4g..4g+3 of fragment f ------
+#pragma unroll
+  for (int i = 0; i < MF; ++i) {
+    const uint32_t m = mt * (16 * MF) + i * 16 + n;
+    if (m < p.M) {
+#pragma unroll
+      for (int f = 0; f < NF; ++f) {
+        const uint32_t col = nt * (NW * 16 * NF) + wave * (16 * NF) + f * 16 + 4 * g;
+        const h2 lo = {(_Float16)acc[i][f][0], (_Float16)acc[i][f][1]};
+        const h2 hi = {(_Float16)acc[i][f][2], (_Float16)acc[i][f][3]};
+        *reinterpret_cast<u2*>(p.out + (uint64_t)m * p.N + col) = (u2){h2bits(lo), h2bits(hi)};
+      }
+    }
+  }
+  RW_MARK(p, 8, 7);
+  RW_MARK_ALL(p, 1);
+}
+
+template <int MF, int NF, int BITS, int NW>
+void launch_rw(RwParams p, hipStream_t s) {
+  p.tiles_m = (p.M + 16 * MF - 1) / (16 * MF);
+  p.tiles_n = p.N / (NW * 16 * NF);
+  hipLaunchKernelGGL((qmm_rw_kernel<MF, NF, BITS, NW>), dim3(p.tiles_m * p.tiles_n), dim3(64 * NW), 0, s, p);
+}
+
+}  // namespace
+
+#ifdef QMM_RW_TRACE
+unsigned long long* g_qmm_rw_trace = nullptr;
+int g_qmm_rw_force_mf = 0, g_qmm_rw_force_nf = 0, g_qmm_rw_force_nw = 4;
+#endif
+
+bool qmm_rw_supported(uint32_t N, uint32_t K, uint32_t group_size, uint32_t bits) {
+  return group_size == 64 && (bits == 4 || bits == 8) && N > 0 && K > 0 && N % 64 == 0 &&
+         K % (kBlockK * kUnroll) == 0;
+}
+
+
+int32_t launch_qmm_rw(const QmmArgs& a, uint32_t group_size, hipStream_t s) {
+  if (!qmm_rw_supported(a.N, a.K, group_size, a.bits))
+    return fail(RMLX_INVALID_SHAPE, "qmm: unsupported shape N=%u K=%u bits=%u group_size=%u", a.N, a.K, a.bits, group_size);
+  if (a.M == 0) return RMLX_OK;
+  if (a.x_dtype != RMLX_DTYPE_F16) return fail(RMLX_RUNTIME_ERROR, "qmm: activations must be cast to f16 first");
+
+  // Tile choice {MF, NF, NW} (tile rows 16*MF, tile columns 16*NF*NW): least estimated time =
+  // rounds of workgroups over the CUs x work per tile / measured relative efficiency of the tile.
+  const uint32_t cus = (uint32_t)ctx().num_cus;
+  static const struct { int mf, nf, nw; float eff; } cand[] = {
+      {4, 2, 8, 1.0f}, {4, 2, 4, 0.9f}, {4, 1, 8, 0.8f}, {2, 2, 4, 0.65f}, {2, 1, 8, 0.6f}, {2, 1, 4, 0.5f}};
+  int mf = 2, nf = 1, nw = 4;
+  float best = 0.f;
+  for (const auto& c : cand) {
+    const uint32_t bn = 16 * c.nf * c.nw;
+    if (a.N % bn != 0) continue;
+    const uint32_t wgs = ((a.M + 16 * c.mf - 1) / (16 * c.mf)) * (a.N / bn);
+    const float cost = (float)((wgs + cus - 1) / cus) * (float)(c.mf * c.nf * c.nw) / c.eff;
+    if (best == 0.f || cost < best) { best = cost; mf = c.mf; nf = c.nf; nw = c.nw; }
+  }
+#ifdef QMM_RW_TRACE
+  if (g_qmm_rw_force_mf) { mf = g_qmm_rw_force_mf; nf = g_qmm_rw_force_nf; nw = g_qmm_rw_force_nw; }
+#endif
+  RwParams p{};
+  p.w = a.w; p.s = a.s; p.b = a.b;
+  p.x = static_cast<const __half*>(a.x);
+  p.out = a.out; p.M = a.M; p.N = a.N; p.K = a.K;
+#ifdef QMM_RW_TRACE
+  p.trace = g_qmm_rw_trace;
+#endif
+#define RW_CASE(MFV, NFV, NWV)                                                                 \
+  if (mf == MFV && nf == NFV && nw == NWV) {                                                   \
+    if (a.bits == 4) launch_rw<MFV, NFV, 4, NWV>(p, s); else launch_rw<MFV, NFV, 8, NWV>(p, s); \
+  }
+  RW_CASE(4, 2, 8) RW_CASE(4, 1, 8) RW_CASE(2, 1, 8) RW_CASE(2, 1, 4) RW_CASE(4, 2, 4) RW_CASE(2, 2, 4)
+#undef RW_CASE
+  RMLX_HIP_CHECK(hipGetLastError());
+  return RMLX_OK;
+}
+
+}  // namespace rmlx

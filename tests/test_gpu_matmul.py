@@ -32,7 +32,8 @@ def test_equal_nibble_closed_forms(hip):
     from rmlx_amd import runtime as rt
     # all nibbles c, scale 1, bias 0, x = 1 (row 0) / 2 (row 1): out = c*K, 2*c*K
     # (quantized.rs:10895-10931, 11541-11591, 12069-12095 scaled to kernel-sized K)
-    for kernel, n, k in [(rt.KERNEL_GENERIC, 8, 64), (rt.KERNEL_QMV, 16, 512), (rt.KERNEL_QMM, 64, 512)]:
+    for kernel, n, k in [(rt.KERNEL_GENERIC, 8, 64), (rt.KERNEL_QMV, 16, 512), (rt.KERNEL_QMM, 64, 512),
+                         (rt.KERNEL_QMM_LDS, 64, 512), (rt.KERNEL_QMM, 64, 256)]:
         for c in (1, 3, 7):
             words = np.full((n, k // 8), c * 0x11111111, np.uint32)
             s = np.ones((n, k // 64), np.float16)
@@ -42,12 +43,13 @@ def test_equal_nibble_closed_forms(hip):
             assert np.array_equal(out[0], np.full(n, c * k, np.float16)), (kernel, c, out[0][:4])
             assert np.array_equal(out[1], np.full(n, 2 * c * k, np.float16))
     # Q8: all bytes 7 -> 7*K (quantized.rs:11752-11800)
-    n, k = 64, 256
-    words = np.full((n, k // 4), 0x07070707, np.uint32)
-    x = np.ones((2, k), np.float16)
-    for kernel in (rt.KERNEL_GENERIC, rt.KERNEL_QMM):
-        out = _run(hip, words, np.ones((n, k // 64), np.float16), np.zeros((n, k // 64), np.float16), x, 8, kernel=kernel)
-        assert np.array_equal(out, np.full((2, n), 7 * k, np.float16))
+    for n, k, kernels in [(64, 256, (rt.KERNEL_GENERIC, rt.KERNEL_QMM, rt.KERNEL_QMM_LDS)),
+                          (64, 512, (rt.KERNEL_QMM, rt.KERNEL_QMM_LDS))]:
+        words = np.full((n, k // 4), 0x07070707, np.uint32)
+        x = np.ones((2, k), np.float16)
+        for kernel in kernels:
+            out = _run(hip, words, np.ones((n, k // 64), np.float16), np.zeros((n, k // 64), np.float16), x, 8, kernel=kernel)
+            assert np.array_equal(out, np.full((2, n), 7 * k, np.float16)), (kernel, k)
 
 
 def test_distinct_positions_are_not_mixed_up(hip):
@@ -64,7 +66,7 @@ def test_distinct_positions_are_not_mixed_up(hip):
         sel = ks[m0:m0 + 8]
         x = np.zeros((len(sel), k), np.float16)
         x[np.arange(len(sel)), sel] = 1.0
-        for kernel in (rt.KERNEL_QMV, rt.KERNEL_QMM, rt.KERNEL_GENERIC):
+        for kernel in (rt.KERNEL_QMV, rt.KERNEL_QMM, rt.KERNEL_QMM_LDS, rt.KERNEL_GENERIC):
             out = _run(hip, words, s, b, x, 4, kernel=kernel)
             assert np.array_equal(out.astype(np.float64), q[:, sel].T), (kernel, sel)
 
@@ -103,6 +105,7 @@ def test_config3_q4_qmm(hip, m):
     x = make_x(rng, m, k)
     ref = model.qmm(x_as_f64(x, "f16"), words, s, b, 64, 4)
     assert_close(_run(hip, words, s, b, x, 4), ref, f"config3 M={m}")
+    assert_close(_run(hip, words, s, b, x, 4, kernel=5), ref, f"config3 M={m} (LDS-staged kernel)")
 
 
 def test_config4_q8_qmm_bf16(hip):
@@ -115,6 +118,18 @@ def test_config4_q8_qmm_bf16(hip):
     # the bf16 matrix-instruction variant: weights rounded to 8 significant bits, still inside the bar
     err_bf16, _ = assert_close(_run(hip, words, s, b, x, 8, dtype="bf16", kernel=4), ref, "config4 (bf16 MFMA)")
     assert err_auto < err_bf16
+    assert_close(_run(hip, words, s, b, x, 8, dtype="bf16", kernel=5), ref, "config4 (LDS-staged kernel)")
+
+
+@pytest.mark.parametrize("m,n,k,bits", [(33, 64, 512, 4), (100, 128, 1024, 8), (200, 256, 512, 4), (513, 4096, 512, 4),
+                                        (64, 2048, 1536, 4), (17, 192, 512, 8), (300, 1024, 2048, 8), (1100, 512, 512, 4)])
+def test_qmm_tile_shapes(hip, m, n, k, bits):
+    """Shapes that walk through the tile variants of the register-weights GEMM (ragged M, every N step)."""
+    rng = np.random.default_rng(m + n + k + bits)
+    words, s, b = make_weight(rng, n, k, bits)
+    x = make_x(rng, m, k)
+    ref = model.qmm(x_as_f64(x, "f16"), words, s, b, 64, bits)
+    assert_close(_run(hip, words, s, b, x, bits, kernel=2), ref, f"qmm M={m} N={n} K={k} bits={bits}")
 
 
 def test_bf16_mfma_variant_is_only_for_q8_bf16(hip):
@@ -138,7 +153,7 @@ def test_ragged_m_all_kernels(hip, m):
     words, s, b = make_weight(rng, n, k, 4)
     x = make_x(rng, m, k)
     ref = model.qmm(x_as_f64(x, "f16"), words, s, b, 64, 4)
-    for kernel in (rt.KERNEL_AUTO, rt.KERNEL_QMV, rt.KERNEL_QMM, rt.KERNEL_GENERIC):
+    for kernel in (rt.KERNEL_AUTO, rt.KERNEL_QMV, rt.KERNEL_QMM, rt.KERNEL_QMM_LDS, rt.KERNEL_GENERIC):
         assert_close(_run(hip, words, s, b, x, 4, kernel=kernel), ref, f"M={m} kernel={kernel}")
 
 
