@@ -369,7 +369,7 @@ int32_t launch_qmm_rw(const QmmArgs& a, uint32_t group_size, hipStream_t s) {
   // rounds of workgroups over the CUs x work per tile / measured relative efficiency of the tile.
   const uint32_t cus = (uint32_t)ctx().num_cus;
   static const struct { int mf, nf, nw; float eff; } cand[] = {
-      {4, 2, 8, 1.0f}, {4, 2, 4, 0.9f}, {4, 1, 8, 0.8f}, {2, 2, 4, 0.65f}, {2, 1, 8, 0.6f}, {2, 1, 4, 0.5f}};
+      {8, 1, 8, 1.03f}, {4, 2, 8, 1.0f}, {4, 2, 4, 0.9f}, {4, 1, 8, 0.8f}, {2, 2, 4, 0.65f}, {2, 1, 8, 0.6f}, {2, 1, 4, 0.5f}};
   int mf = 2, nf = 1, nw = 4;
   float best = 0.f;
   for (const auto& c : cand) {
@@ -394,6 +394,7 @@ int32_t launch_qmm_rw(const QmmArgs& a, uint32_t group_size, hipStream_t s) {
     if (a.bits == 4) launch_rw<MFV, NFV, 4, NWV>(p, s); else launch_rw<MFV, NFV, 8, NWV>(p, s); \
   }
   RW_CASE(4, 2, 8) RW_CASE(4, 1, 8) RW_CASE(2, 1, 8) RW_CASE(2, 1, 4) RW_CASE(4, 2, 4) RW_CASE(2, 2, 4)
+  RW_CASE(8, 1, 8)
 #undef RW_CASE
   RMLX_HIP_CHECK(hipGetLastError());
   return RMLX_OK;
