@@ -26,8 +26,9 @@
 //     rows 8-15 the same x restricted to the second group (the other half of the A operand is
 //     zero), so one accumulator tile yields both per-group integer dot products.  Each is then
 //     folded into the f32 result with  acc += scale * (dot - sum(off*x)) + bias * sum(x).
-//   * Each wave stages exactly the activations it consumes (wave-private LDS, no barrier) and
-//     forms the per-(row, group) sums while doing so (8 consecutive lanes hold one group).
+//   * Each wave stages exactly the activations it consumes (wave-private LDS, no barrier).  The
+//     per-(row, group) sums sum(x) and sum(off*x) come from the matrix unit too: one extra MFMA per
+//     product against a constant operand, issued while the weights are still in flight.
 #include "common.hpp"
 
 namespace rmlx {
@@ -100,6 +101,10 @@ __device__ __forceinline__ uint32_t swap16(uint32_t v) {  // value of lane ^ 16
   return (uint32_t)__builtin_amdgcn_ds_swizzle((int)v, 0x401F);
 }
 
+__device__ __forceinline__ float swap8(float v) {  // value of lane ^ 8
+  return __builtin_bit_cast(float, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, v), 0x201F));
+}
+
 struct __attribute__((packed, aligned(4))) U4Unaligned { uint32_t v[4]; };
 
 // MR = activation rows staged per pass (1, 2, 4 or 8); TILES = 1, or 2 for fused gate/up;
@@ -114,14 +119,17 @@ __global__ __launch_bounds__(kThreads) void qmv_q4_kernel(KParams p) {
   constexpr int kXsBytes = kWaves * kXsWave;
   constexpr int kXsAlloc = kXsBytes > kRedBytes ? kXsBytes : kRedBytes;
   __shared__ __attribute__((aligned(16))) char xs_all[kXsAlloc];
-  __shared__ __attribute__((aligned(16))) float sums_all[kWaves * kSpwMax * 2 * 8 * 2];  // [wave][group][row][-xoff, xsum]
+  // Activation sums per (row, group): on the matrix unit for 8 rows (see 2b), with lane shuffles
+  // while staging for fewer rows (cheaper there: the extra MFMAs would outweigh ~45 VALU per row).
+  constexpr bool kMfmaSums = MR == 8;
+  __shared__ __attribute__((aligned(16))) float sums_all[kMfmaSums ? 4 : kWaves * kSpwMax * 2 * 8 * 2];  // [wave][group][row][-xoff, xsum]
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int n = lane & 15;   // weight row within the tile / accumulator column
   const int g = lane >> 4;   // k sub-block of the slab / accumulator row group
   const int par = g >> 1;    // which of the slab's two quantisation groups this lane scales
   char* xs = xs_all + wave * kXsWave;
-  float* sums = sums_all + wave * (kSpwMax * 2 * 8 * 2);
+  float* sums = sums_all + (kMfmaSums ? 0 : wave * (kSpwMax * 2 * 8 * 2));
 
   // ---- which rows -----------------------------------------------------------------------
   uint32_t expert = 0, row0 = blockIdx.y * 8, rows;
@@ -165,6 +173,11 @@ __global__ __launch_bounds__(kThreads) void qmv_q4_kernel(KParams p) {
   const int am = n & 7;
   const bool a_active = ((n < 8) == (g < 2)) && (am < MR);
   const int a_slot_off = (g * MR + am) * 16;
+
+  // constant B operand of the activation sums (see 2b)
+  const u4 bconst_bits = n < 8 ? (u4){0x64006400u, 0x54005400u, 0x64006400u, 0x54005400u}
+                               : (u4){0x3C003C00u, 0x3C003C00u, 0x3C003C00u, 0x3C003C00u};
+  const h8 bconst = __builtin_bit_cast(h8, bconst_bits);
 
   f4 F[TILES];
 #pragma unroll
@@ -211,33 +224,61 @@ __global__ __launch_bounds__(kThreads) void qmv_q4_kernel(KParams p) {
     }
     QMV_MARK(p, 1);
 
-    // ---- 2. this wave's activations -> its LDS image in operand order; sums per (row, group) --
-    {
-      const int ls = lane >> 4, gg = (lane >> 2) & 3, j = lane & 3;
+    if constexpr (kMfmaSums) {
+      // ---- 2. this wave's activations -> its LDS image in operand order ------------------------
+      {
+        const int ls = lane >> 4, gg = (lane >> 2) & 3, j = lane & 3;
 #pragma unroll
-      for (int m = 0; m < MR; ++m) {
-        *reinterpret_cast<u4*>(xs + ((ls * 4 + j) * kSlots + gg * MR + m) * 16) = permute_x8(xv[m]);
-        // this lane's 8 activations: plain sum and sum weighted by the unpack offsets
-        // (even k -> 1024, odd k -> 64); 8 consecutive lanes make up one group of 64
-        const h8 hv = __builtin_bit_cast(h8, xv[m]);
-        float xs8 = 0.f, xo8 = 0.f;
+        for (int m = 0; m < MR; ++m)
+          *reinterpret_cast<u4*>(xs + ((ls * 4 + j) * kSlots + gg * MR + m) * 16) = permute_x8(xv[m]);
+      }
+    } else {
+      // ---- 2. this wave's activations -> its LDS image in operand order; sums per (row, group) --
+      {
+        const int ls = lane >> 4, gg = (lane >> 2) & 3, j = lane & 3;
 #pragma unroll
-        for (int e = 0; e < 8; e += 2) {
-          xs8 += (float)hv[e] + (float)hv[e + 1];
-          xo8 += 1024.0f * (float)hv[e] + 64.0f * (float)hv[e + 1];
-        }
+        for (int m = 0; m < MR; ++m) {
+          *reinterpret_cast<u4*>(xs + ((ls * 4 + j) * kSlots + gg * MR + m) * 16) = permute_x8(xv[m]);
+          // this lane's 8 activations: plain sum and sum weighted by the unpack offsets
+          // (even k -> 1024, odd k -> 64); 8 consecutive lanes make up one group of 64
+          const h8 hv = __builtin_bit_cast(h8, xv[m]);
+          float xs8 = 0.f, xo8 = 0.f;
 #pragma unroll
-        for (int off = 1; off < 8; off <<= 1) {
-          xs8 += __shfl_xor(xs8, off, 64);
-          xo8 += __shfl_xor(xo8, off, 64);
-        }
-        if ((lane & 7) == 0) {  // sums[group][m] = (-sum(off*x), sum(x)); rows >= MR stay unused
-          sums[((lane >> 3) * 8 + m) * 2 + 0] = -xo8;
-          sums[((lane >> 3) * 8 + m) * 2 + 1] = xs8;
+          for (int e = 0; e < 8; e += 2) {
+            xs8 += (float)hv[e] + (float)hv[e + 1];
+            xo8 += 1024.0f * (float)hv[e] + 64.0f * (float)hv[e + 1];
+          }
+#pragma unroll
+          for (int off = 1; off < 8; off <<= 1) {
+            xs8 += __shfl_xor(xs8, off, 64);
+            xo8 += __shfl_xor(xo8, off, 64);
+          }
+          if ((lane & 7) == 0) {  // sums[group][m] = (-sum(off*x), sum(x)); rows >= MR stay unused
+            sums[((lane >> 3) * 8 + m) * 2 + 0] = -xo8;
+            sums[((lane >> 3) * 8 + m) * 2 + 1] = xs8;
+          }
         }
       }
     }
     QMV_MARK(p, 2);
+
+    // ---- 2b. per (row, group) sums of the activations, on the matrix unit while the weights are
+    //          still in flight: columns 0-7 of a constant B operand hold the unpack offsets
+    //          (1024 for even k, 64 for odd k, in slot order), columns 8-15 hold ones, so
+    //          accumulator column n < 8 receives sum(off*x) and column n >= 8 sum(x) of its rows.
+    f4 xsums[kSpwMax];
+#pragma unroll
+    for (int it = 0; it < kSpwMax; ++it) {
+      xsums[it] = (f4){0.f, 0.f, 0.f, 0.f};
+      if (kMfmaSums && it < my) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          h8 av = (h8){0, 0, 0, 0, 0, 0, 0, 0};
+          if (a_active) av = *reinterpret_cast<const h8*>(xs + ((it * 4 + j) * kSlots) * 16 + a_slot_off);
+          xsums[it] = __builtin_amdgcn_mfma_f32_16x16x32_f16(av, bconst, xsums[it], 0, 0, 0);
+        }
+      }
+    }
 
     // ---- 3. weights: integer dot per group via MFMA (independent slabs interleaved), then
     //         acc += scale * (dot - sum(off*x)) + bias * sum(x) in f32 ------------------------
@@ -269,17 +310,28 @@ __global__ __launch_bounds__(kThreads) void qmv_q4_kernel(KParams p) {
 #pragma unroll
       for (int it = 0; it < kSpwMax; ++it) {
         if (it < my) {
-          const float* sp = sums + ((it * 2 + par) * 8 + (g & 1) * 4) * 2;
-          const f4 c01 = *reinterpret_cast<const f4*>(sp);      // (-xoff, xsum) of accumulator rows 4g, 4g+1
-          const f4 c23 = *reinterpret_cast<const f4*>(sp + 4);  // rows 4g+2, 4g+3
           const uint32_t swd = it == 0 ? sv.x : (it == 1 ? sv.y : (it == 2 ? sv.z : sv.w));
           const uint32_t bwd = it == 0 ? bv.x : (it == 1 ? bv.y : (it == 2 ? bv.z : bv.w));
           const float sc = __half2float(__ushort_as_half((unsigned short)(par ? swd >> 16 : swd & 0xFFFFu)));
           const float bi = __half2float(__ushort_as_half((unsigned short)(par ? bwd >> 16 : bwd & 0xFFFFu)));
-          F[t][0] += sc * (c[it][0] + c01[0]) + bi * c01[1];
-          F[t][1] += sc * (c[it][1] + c01[2]) + bi * c01[3];
-          F[t][2] += sc * (c[it][2] + c23[0]) + bi * c23[1];
-          F[t][3] += sc * (c[it][3] + c23[2]) + bi * c23[3];
+          if constexpr (kMfmaSums) {
+            // own column holds sum(off*x) (n < 8) or sum(x) (n >= 8) of rows 4g..4g+3, lane n^8 the other
+            const float ce = n < 8 ? -sc : bi, co = n < 8 ? bi : -sc;
+            const f4 own = xsums[it];
+            const float o0 = swap8(own.x), o1 = swap8(own.y), o2 = swap8(own.z), o3 = swap8(own.w);
+            F[t][0] += sc * c[it][0] + ce * own.x + co * o0;
+            F[t][1] += sc * c[it][1] + ce * own.y + co * o1;
+            F[t][2] += sc * c[it][2] + ce * own.z + co * o2;
+            F[t][3] += sc * c[it][3] + ce * own.w + co * o3;
+          } else {
+            const float* sp = sums + ((it * 2 + par) * 8 + (g & 1) * 4) * 2;
+            const f4 c01 = *reinterpret_cast<const f4*>(sp);      // (-xoff, xsum) of accumulator rows 4g, 4g+1
+            const f4 c23 = *reinterpret_cast<const f4*>(sp + 4);  // rows 4g+2, 4g+3
+            F[t][0] += sc * (c[it][0] + c01[0]) + bi * c01[1];
+            F[t][1] += sc * (c[it][1] + c01[2]) + bi * c01[3];
+            F[t][2] += sc * (c[it][2] + c23[0]) + bi * c23[1];
+            F[t][3] += sc * (c[it][3] + c23[2]) + bi * c23[3];
+          }
         }
       }
     }
