@@ -112,7 +112,9 @@ struct __attribute__((packed, aligned(4))) U4Unaligned { uint32_t v[4]; };
 // every wave of every pass owns the same number (3 or 4: no guards, fewer registers, two
 // workgroups per CU), 0 = decided at run time.
 template <int MR, int TILES, bool TAB, int SPW>
-__global__ __launch_bounds__(kThreads) void qmv_q4_kernel(KParams p) {
+__global__ __launch_bounds__(kThreads)
+__attribute__((amdgpu_waves_per_eu(MR == 8 && TILES == 2 && SPW == 4 ? 4 : 1, 8)))
+void qmv_q4_kernel(KParams p) {
   constexpr int kSlots = 4 * MR;                       // 16-byte slots per (slab, j)
   constexpr int kXsWave = kSpwMax * 4 * kSlots * 16;   // bytes of activation image per wave
   constexpr int kRedBytes = kWaves * TILES * 256 * 4;
