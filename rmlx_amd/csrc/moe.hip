@@ -88,8 +88,32 @@ __global__ __launch_bounds__(64) void topk_route_kernel(const float* __restrict_
 }
 
 // ---- histogram + scan + stable counting sort, one workgroup --------------------------------
-// Deterministic by construction: thread e owns expert e and walks each block of 1024
-// assignments in ascending order, so ids of one expert keep their original order.
+// Deterministic by construction.  Offsets and the chunk table come from block-wide exclusive scans
+// of the per-expert counts.  Placement walks the assignments in blocks of 1024: every wave ranks
+// its 64 consecutive assignments among themselves (lane l counts the lanes below it with the same
+// expert), then the waves take turns, in order, to add the running cursor of their experts, so
+// ids of one expert keep their original order (numpy.argsort(kind="stable")).
+__device__ __forceinline__ uint32_t block_exclusive_scan_1024(uint32_t v, uint32_t* wave_tot, uint32_t* total) {
+  const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  uint32_t inc = v;
+#pragma unroll
+  for (int o = 1; o < 64; o <<= 1) {
+    const uint32_t t = __shfl_up(inc, o, 64);
+    if ((int)lane >= o) inc += t;
+  }
+  __syncthreads();  // wave_tot may still be read by a previous scan
+  if (lane == 63) wave_tot[wave] = inc;
+  __syncthreads();
+  uint32_t base = 0, all = 0;
+  for (uint32_t w = 0; w < 16; ++w) {
+    const uint32_t t = wave_tot[w];
+    if (w < wave) base += t;
+    all += t;
+  }
+  *total = all;
+  return base + inc - v;
+}
+
 __global__ __launch_bounds__(1024) void moe_sort_kernel(const uint32_t* __restrict__ idx, uint32_t n_assign,
                                                         uint32_t E, uint32_t top_k, uint32_t* __restrict__ sorted,
                                                         uint32_t* __restrict__ sorted_tok,
@@ -98,57 +122,69 @@ __global__ __launch_bounds__(1024) void moe_sort_kernel(const uint32_t* __restri
                                                         uint32_t* __restrict__ chunk_tab,
                                                         uint32_t* __restrict__ n_chunks) {
   __shared__ uint32_t cnt[kMaxExperts];
-  __shared__ uint32_t off[kMaxExperts + 1];
-  __shared__ uint32_t ids[1024];
-  __shared__ uint32_t pos[1024];
-  const uint32_t tid = threadIdx.x;
-  for (uint32_t e = tid; e < E; e += 1024) cnt[e] = 0;
+  __shared__ uint32_t cur[kMaxExperts];  // running cursor of every expert
+  __shared__ uint32_t wave_tot[16];
+  const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  cnt[tid] = 0;  // kMaxExperts == blockDim.x
   __syncthreads();
   for (uint32_t i = tid; i < n_assign; i += 1024) {
     const uint32_t e = idx[i];
     if (e < E) atomicAdd(&cnt[e], 1u);
   }
   __syncthreads();
-  if (tid == 0) {
-    uint32_t run = 0, nc = 0;
-    for (uint32_t e = 0; e < E; ++e) {
-      off[e] = run;
-      if (chunk_tab != nullptr) {
-        for (uint32_t r = 0; r < cnt[e]; r += 8) {
-          chunk_tab[3 * nc + 0] = e;
-          chunk_tab[3 * nc + 1] = run + r;
-          chunk_tab[3 * nc + 2] = cnt[e] - r < 8u ? cnt[e] - r : 8u;
-          ++nc;
-        }
+  // thread e owns expert e: offsets, counts, its chunks of at most 8 rows
+  const uint32_t my_cnt = tid < E ? cnt[tid] : 0u;
+  uint32_t total_rows, total_chunks;
+  const uint32_t my_off = block_exclusive_scan_1024(my_cnt, wave_tot, &total_rows);
+  const uint32_t my_chunks = (my_cnt + 7) / 8;
+  const uint32_t my_chunk0 = block_exclusive_scan_1024(my_chunks, wave_tot, &total_chunks);
+  cur[tid] = my_off;
+  if (tid < E) {
+    if (offsets != nullptr) offsets[tid] = my_off;
+    if (counts != nullptr) counts[tid] = my_cnt;
+    if (chunk_tab != nullptr) {
+      for (uint32_t c = 0; c < my_chunks; ++c) {
+        chunk_tab[3 * (my_chunk0 + c) + 0] = tid;
+        chunk_tab[3 * (my_chunk0 + c) + 1] = my_off + 8 * c;
+        chunk_tab[3 * (my_chunk0 + c) + 2] = my_cnt - 8 * c < 8u ? my_cnt - 8 * c : 8u;
       }
-      run += cnt[e];
     }
-    off[E] = run;
-    if (n_chunks != nullptr) *n_chunks = nc;
   }
-  __syncthreads();
-  for (uint32_t e = tid; e <= E; e += 1024) {
-    if (offsets != nullptr) offsets[e] = off[e];
-    if (counts != nullptr && e < E) counts[e] = cnt[e];
+  if (tid == 0) {
+    if (offsets != nullptr) offsets[E] = total_rows;
+    if (n_chunks != nullptr) *n_chunks = total_chunks;
   }
   if (sorted == nullptr) return;
 
-  uint32_t cursor = tid < E ? off[tid] : 0;  // thread e places the ids of expert e
   for (uint32_t base = 0; base < n_assign; base += 1024) {
     const uint32_t nb = n_assign - base < 1024u ? n_assign - base : 1024u;
-    __syncthreads();
-    if (tid < nb) ids[tid] = idx[base + tid];
-    __syncthreads();
-    if (tid < E) {
-      for (uint32_t i = 0; i < nb; ++i)
-        if (ids[i] == tid) pos[i] = cursor++;
+    const uint32_t e = tid < nb ? idx[base + tid] : 0xFFFFFFFFu;
+    const bool valid = e < E;
+    // rank among the wave's 64 assignments, and how many of them share the expert
+    uint32_t rank = 0, same_total = 0;
+    for (int j = 0; j < 64; ++j) {
+      const uint32_t ej = (uint32_t)__builtin_amdgcn_readlane((int)e, j);
+      const uint32_t same = ej == e ? 1u : 0u;
+      same_total += same;
+      rank += (j < (int)lane) ? same : 0u;
+    }
+    const uint32_t n_waves = (nb + 63) / 64;
+    uint32_t pos = 0;
+    for (uint32_t w = 0; w < n_waves; ++w) {
+      __syncthreads();  // cursor updates of wave w-1 (and of the previous block) are visible
+      uint32_t c0 = 0;
+      if (wave == w && valid) c0 = cur[e];
+      if (wave == w && valid) {
+        pos = c0 + rank;
+        if (rank + 1 == same_total) cur[e] = c0 + same_total;  // the last one of its expert moves the cursor
+      }
+    }
+    if (valid) {
+      sorted[pos] = base + tid;
+      if (sorted_tok != nullptr) sorted_tok[pos] = (base + tid) / top_k;
+      if (inv != nullptr) inv[base + tid] = pos;
     }
     __syncthreads();
-    if (tid < nb && ids[tid] < E) {
-      sorted[pos[tid]] = base + tid;
-      if (sorted_tok != nullptr) sorted_tok[pos[tid]] = (base + tid) / top_k;
-      if (inv != nullptr) inv[base + tid] = pos[tid];
-    }
   }
 }
 
