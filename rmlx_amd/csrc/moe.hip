@@ -220,23 +220,36 @@ __global__ void silu_gate_kernel(const __half* __restrict__ g, const __half* __r
   }
 }
 
-// out[t,:] = sum_k w[t*K+k] * y[inv[t*K+k],:], k ascending, f32.
+// out[t,:] = sum_k w[t*K+k] * y[inv[t*K+k],:], k ascending, f32.  grid = (T, column blocks of 1024):
+// every thread owns four columns, loads its rows of all top_k experts first and sums in order.
 __global__ __launch_bounds__(256) void moe_combine_kernel(const float* __restrict__ y,
                                                           const uint32_t* __restrict__ inv,
                                                           const float* __restrict__ weights, uint32_t top_k,
                                                           uint32_t D, __half* __restrict__ out) {
   const uint32_t t = blockIdx.x;
-  for (uint32_t c = threadIdx.x * 4; c < D; c += blockDim.x * 4) {
-    float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
-    for (uint32_t k = 0; k < top_k; ++k) {
-      const float w = weights[(size_t)t * top_k + k];
-      const float4 v = *reinterpret_cast<const float4*>(y + (size_t)inv[(size_t)t * top_k + k] * D + c);
-      acc.x += w * v.x; acc.y += w * v.y; acc.z += w * v.z; acc.w += w * v.w;
+  const uint32_t c = (blockIdx.y * 256 + threadIdx.x) * 4;
+  if (c >= D) return;
+  float w[8];
+  float4 v[8];
+#pragma unroll
+  for (uint32_t k = 0; k < 8; ++k) {
+    w[k] = 0.f;
+    v[k] = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (k < top_k) {
+      w[k] = weights[(size_t)t * top_k + k];
+      v[k] = *reinterpret_cast<const float4*>(y + (size_t)inv[(size_t)t * top_k + k] * D + c);
     }
-    __half* o = out + (size_t)t * D + c;
-    o[0] = __float2half(acc.x); o[1] = __float2half(acc.y);
-    o[2] = __float2half(acc.z); o[3] = __float2half(acc.w);
   }
+  float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+  for (uint32_t k = 0; k < 8; ++k) {
+    if (k < top_k) { acc.x += w[k] * v[k].x; acc.y += w[k] * v[k].y; acc.z += w[k] * v[k].z; acc.w += w[k] * v[k].w; }
+  }
+  const __half2 lo = __floats2half2_rn(acc.x, acc.y), hi = __floats2half2_rn(acc.z, acc.w);
+  uint2 o;
+  o.x = *reinterpret_cast<const uint32_t*>(&lo);
+  o.y = *reinterpret_cast<const uint32_t*>(&hi);
+  *reinterpret_cast<uint2*>(out + (size_t)t * D + c) = o;
 }
 
 }  // namespace
@@ -296,7 +309,8 @@ int32_t launch_silu_gate(const __half* g, const __half* u, __half* out, size_t n
 int32_t launch_moe_combine(const float* y, const uint32_t* inv, const float* weights, uint32_t T, uint32_t top_k,
                            uint32_t D, __half* out, hipStream_t s) {
   if (T == 0) return RMLX_OK;
-  hipLaunchKernelGGL(moe_combine_kernel, dim3(T), dim3(256), 0, s, y, inv, weights, top_k, D, out);
+  if (top_k > 8 || D % 4 != 0) return fail(RMLX_INVALID_SHAPE, "moe_combine: top_k <= 8 and D %% 4 == 0 required (top_k=%u D=%u)", top_k, D);
+  hipLaunchKernelGGL(moe_combine_kernel, dim3(T, (D + 1023) / 1024), dim3(256), 0, s, y, inv, weights, top_k, D, out);
   RMLX_HIP_CHECK(hipGetLastError());
   return RMLX_OK;
 }
