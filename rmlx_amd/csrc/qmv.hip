@@ -52,7 +52,7 @@ struct KParams {
   void* out;
   uint32_t K, ld_out, M, out_f32;
   uint32_t ks;  // k-parts per pass (1, 2, 4 or 8); tiles per workgroup = 8 / ks
-  uint32_t pad_;
+  uint32_t pair;  // TILES == 2 only: 1 = the two tiles are rows r and r+16 of one matrix (plain outputs), 0 = gate/up
   const uint32_t* w1;
   const __half* s1;
   const __half* b1;
@@ -107,7 +107,8 @@ __device__ __forceinline__ float swap8(float v) {  // value of lane ^ 8
 
 struct __attribute__((packed, aligned(4))) U4Unaligned { uint32_t v[4]; };
 
-// MR = activation rows staged per pass (1, 2, 4 or 8); TILES = 1, or 2 for fused gate/up;
+// MR = activation rows staged per pass (1, 2, 4 or 8); TILES = 1, or 2 (fused gate/up, or two
+// 16-row tiles of one matrix sharing the staged activations: KParams::pair);
 // TAB = rows come from a device chunk table (gather_qmm, MoE); SPW = slabs per wave and pass when
 // every wave of every pass owns the same number (3 or 4: no guards, fewer registers, two
 // workgroups per CU), 0 = decided at run time.
@@ -152,17 +153,21 @@ void qmv_q4_kernel(KParams p) {
   const uint32_t K = p.K, KS = p.ks, NT = kWaves / KS;
   const uint32_t kp = wave % KS, tw = wave / KS;
   const uint32_t words_per_row = K >> 3, groups_per_row = K >> 6, slabs_total = K >> 7;
-  const uint32_t tile_row = (blockIdx.x * NT + tw) * 16;
+  const bool pair = TILES == 2 && p.pair != 0;
+  const uint32_t rows_per_slot = pair ? 32u : 16u;  // weight rows (of one matrix) per wave tile slot
+  const uint32_t tile_row = (blockIdx.x * NT + tw) * rows_per_slot;
 
   const u4* wrow[TILES];
   const __half* sbrow[TILES];
 #pragma unroll
   for (int t = 0; t < TILES; ++t) {
     const uint64_t e_w = TAB ? expert * p.estride_w : 0, e_s = TAB ? expert * p.estride_s : 0;
-    wrow[t] = reinterpret_cast<const u4*>((t == 0 ? p.w0 : p.w1) + e_w + (uint64_t)(tile_row + n) * words_per_row) + g;
+    const bool first = t == 0 || pair;                       // which matrix
+    const uint32_t wr = tile_row + n + (pair ? 16 * t : 0);  // which row of it
+    wrow[t] = reinterpret_cast<const u4*>((first ? p.w0 : p.w1) + e_w + (uint64_t)wr * words_per_row) + g;
     // scales live in the lanes with even g, biases in the lanes with odd g (exchanged later)
-    const __half* sb = (g & 1) ? (t == 0 ? p.b0 : p.b1) : (t == 0 ? p.s0 : p.s1);
-    sbrow[t] = sb + e_s + (uint64_t)(tile_row + n) * groups_per_row;
+    const __half* sb = (g & 1) ? (first ? p.b0 : p.b1) : (first ? p.s0 : p.s1);
+    sbrow[t] = sb + e_s + (uint64_t)wr * groups_per_row;
   }
   uint32_t srcs[MR];  // source rows of the activations (wave-uniform)
 #pragma unroll
@@ -364,12 +369,16 @@ void qmv_q4_kernel(KParams p) {
         }
         v[t] = acc;
       }
-      float r = v[0];
-      if (TILES == 2) r = silu_f(v[0]) * v[TILES - 1];
-      if (write_zeros) r = 0.f;
-      const uint64_t oidx = (uint64_t)(row0 + m) * p.ld_out + (blockIdx.x * NT + otw) * 16 + nn;
-      if (p.out_f32) reinterpret_cast<float*>(p.out)[oidx] = r;
-      else reinterpret_cast<__half*>(p.out)[oidx] = __float2half(r);
+      const uint64_t obase = (uint64_t)(row0 + m) * p.ld_out + (blockIdx.x * NT + otw) * rows_per_slot + nn;
+      if (TILES == 2 && !pair) v[0] = silu_f(v[0]) * v[TILES - 1];
+#pragma unroll
+      for (int t = 0; t < TILES; ++t) {
+        if (t == 0 || pair) {
+          const float r = write_zeros ? 0.f : v[t];
+          if (p.out_f32) reinterpret_cast<float*>(p.out)[obase + 16 * t] = r;
+          else reinterpret_cast<__half*>(p.out)[obase + 16 * t] = __float2half(r);
+        }
+      }
     }
   }
   QMV_MARK(p, 8);
@@ -450,10 +459,17 @@ int32_t launch_qmv_q4(const QmvArgs& a, hipStream_t s) {
     while (ks < 8 && a.N % (16 * (8 / ks)) != 0) ks *= 2;
   }
   p.ks = ks;
-  dim3 grid(a.N / (16 * (8 / ks)), chunks);
   int mr = a.mr;
   if (mr == 0) mr = tab ? 8 : (a.M >= 5 ? 8 : (a.M >= 3 ? 4 : (a.M == 2 ? 2 : 1)));
-  if (a.dual) {
+  // With 8 rows every wave takes two tiles (rows r and r+16) for the same staged activations when
+  // that still leaves at least four workgroups per CU: the activation traffic and staging work per
+  // weight byte halve.
+  const uint32_t nt = 8 / ks;
+  const bool pair = !a.dual && mr == 8 && a.N % (32 * nt) == 0 &&
+                    (uint64_t)(a.N / (32 * nt)) * chunks >= 4ull * (uint32_t)ctx().num_cus;
+  p.pair = pair ? 1u : 0u;
+  dim3 grid(a.N / (16 * nt * (pair ? 2 : 1)), chunks);
+  if (a.dual || pair) {
     switch (mr) {
       case 1: launch_t<1, 2>(p, tab, grid, s); break;
       case 2: launch_t<2, 2>(p, tab, grid, s); break;
