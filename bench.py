@@ -231,7 +231,7 @@ def main():
                              "roofline": {"bound": "mfma", "achieved": q["tflops"], "peak": MFMA_F16_PEAK_TF,
                                           "unit": "TFLOP/s", "frac": q["mfma_frac"],
                                           "traffic": MEASURED_TRAFFIC_BYTES["qmm_q4_m512_4096"],
-                                          "kernel": "qmm_kernel<128,64,4,false> (+ relayout_a_kernel)", "avg_launch_us": q["us"]}}
+                                          "kernel": "qmm_rw_kernel<4,2,4,4>", "avg_launch_us": q["us"]}}
     if not args.no_cpu:
         line["cpu_baseline"] = cpu_baseline(np.random.default_rng(1001), 3.0 if args.quick else 10.0)
     line["extra"] = extra

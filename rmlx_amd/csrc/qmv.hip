@@ -52,7 +52,7 @@ struct KParams {
   void* out;
   uint32_t K, ld_out, M, out_f32;
   uint32_t ks;  // k-parts per pass (1, 2, 4 or 8); tiles per workgroup = 8 / ks
-  uint32_t pair;  // TILES == 2 only: 1 = the two tiles are rows r and r+16 of one matrix (plain outputs), 0 = gate/up
+  uint32_t pad_;
   const uint32_t* w1;
   const __half* s1;
   const __half* b1;
@@ -108,14 +108,13 @@ __device__ __forceinline__ float swap8(float v) {  // value of lane ^ 8
 struct __attribute__((packed, aligned(4))) U4Unaligned { uint32_t v[4]; };
 
 // MR = activation rows staged per pass (1, 2, 4 or 8); TILES = 1, or 2 (fused gate/up, or two
-// 16-row tiles of one matrix sharing the staged activations: KParams::pair);
+// 16-row tiles of one matrix sharing the staged activations: PAIR);
 // TAB = rows come from a device chunk table (gather_qmm, MoE); SPW = slabs per wave and pass when
 // every wave of every pass owns the same number (3 or 4: no guards, fewer registers, two
 // workgroups per CU), 0 = decided at run time.
-template <int MR, int TILES, bool TAB, int SPW>
-__global__ __launch_bounds__(kThreads)
-__attribute__((amdgpu_waves_per_eu(MR == 8 && TILES == 2 && SPW == 4 ? 4 : 1, 8)))
-void qmv_q4_kernel(KParams p) {
+template <int MR, int TILES, bool TAB, int SPW, bool PAIR>
+__global__ __launch_bounds__(kThreads) void qmv_q4_kernel(KParams p) {
+  static_assert(!PAIR || TILES == 2, "paired tiles need two tile slots");
   constexpr int kSlots = 4 * MR;                       // 16-byte slots per (slab, j)
   constexpr int kXsWave = kSpwMax * 4 * kSlots * 16;   // bytes of activation image per wave
   constexpr int kRedBytes = kWaves * TILES * 256 * 4;
@@ -153,7 +152,7 @@ void qmv_q4_kernel(KParams p) {
   const uint32_t K = p.K, KS = p.ks, NT = kWaves / KS;
   const uint32_t kp = wave % KS, tw = wave / KS;
   const uint32_t words_per_row = K >> 3, groups_per_row = K >> 6, slabs_total = K >> 7;
-  const bool pair = TILES == 2 && p.pair != 0;
+  constexpr bool pair = PAIR;
   const uint32_t rows_per_slot = pair ? 32u : 16u;  // weight rows (of one matrix) per wave tile slot
   const uint32_t tile_row = (blockIdx.x * NT + tw) * rows_per_slot;
 
@@ -384,22 +383,22 @@ void qmv_q4_kernel(KParams p) {
   QMV_MARK(p, 8);
 }
 
-template <int MR, int TILES, int SPW>
+template <int MR, int TILES, int SPW, bool PAIR>
 void launch_s(const KParams& p, bool tab, dim3 grid, hipStream_t s) {
-  if (tab) hipLaunchKernelGGL((qmv_q4_kernel<MR, TILES, true, SPW>), grid, dim3(kThreads), 0, s, p);
-  else hipLaunchKernelGGL((qmv_q4_kernel<MR, TILES, false, SPW>), grid, dim3(kThreads), 0, s, p);
+  if (tab) hipLaunchKernelGGL((qmv_q4_kernel<MR, TILES, true, SPW, PAIR>), grid, dim3(kThreads), 0, s, p);
+  else hipLaunchKernelGGL((qmv_q4_kernel<MR, TILES, false, SPW, PAIR>), grid, dim3(kThreads), 0, s, p);
 }
 
-template <int MR, int TILES>
+template <int MR, int TILES, bool PAIR = false>
 void launch_t(const KParams& p, bool tab, dim3 grid, hipStream_t s) {
   // uniform slab count per wave and pass?
   const uint32_t slabs = p.K / 128, per_pass = p.ks * kSpwMax;
   int spw = 0;
   if (slabs % per_pass == 0) spw = 4;
   else if (slabs < per_pass && slabs % p.ks == 0 && slabs / p.ks == 3) spw = 3;
-  if (spw == 4) launch_s<MR, TILES, 4>(p, tab, grid, s);
-  else if (spw == 3) launch_s<MR, TILES, 3>(p, tab, grid, s);
-  else launch_s<MR, TILES, 0>(p, tab, grid, s);
+  if (spw == 4) launch_s<MR, TILES, 4, PAIR>(p, tab, grid, s);
+  else if (spw == 3) launch_s<MR, TILES, 3, PAIR>(p, tab, grid, s);
+  else launch_s<MR, TILES, 0, PAIR>(p, tab, grid, s);
 }
 
 __global__ void build_gather_chunks_kernel(const uint32_t* indices, uint32_t batch, uint32_t mpb,
@@ -467,9 +466,10 @@ int32_t launch_qmv_q4(const QmvArgs& a, hipStream_t s) {
   const uint32_t nt = 8 / ks;
   const bool pair = !a.dual && mr == 8 && a.N % (32 * nt) == 0 &&
                     (uint64_t)(a.N / (32 * nt)) * chunks >= 4ull * (uint32_t)ctx().num_cus;
-  p.pair = pair ? 1u : 0u;
   dim3 grid(a.N / (16 * nt * (pair ? 2 : 1)), chunks);
-  if (a.dual || pair) {
+  if (pair) {
+    launch_t<8, 2, true>(p, tab, grid, s);
+  } else if (a.dual) {
     switch (mr) {
       case 1: launch_t<1, 2>(p, tab, grid, s); break;
       case 2: launch_t<2, 2>(p, tab, grid, s); break;
