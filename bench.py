@@ -186,6 +186,8 @@ def main():
         for m in (1, 4, 8):
             extra[f"q4_qmv_m{m}_n9216"] = bench_matmul(ops, rt, timer, rng, m, 9216, 4096, 4, "f16", args.steps,
                                                        args.warmup, GiB + GiB // 8, check=(m == 8))
+        extra["q8_qmv_m1_4096"] = bench_matmul(ops, rt, timer, rng, 1, 4096, 4096, 8, "f16", args.steps, args.warmup,
+                                               GiB + GiB // 8)
         for m in (128, 512):
             r = bench_matmul(ops, rt, timer, rng, m, 4096, 4096, 4, "f16", small, 10, 4 * 9437184)
             r["mfma_frac"] = r["tflops"] / MFMA_F16_PEAK_TF

@@ -118,7 +118,8 @@ int32_t run_matmul(const rmlx_qweight* qw, const void* x, int32_t x_dtype, uint3
   RMLX_TRY(checked_u32(qw->in_features, "in_features", &K));
   if (M == 0) return RMLX_OK;
   const bool ptr_ok = aligned16(qw->w) && aligned16(qw->s) && aligned16(qw->b) && aligned16(x);
-  const bool can_qmv = qw->bits == 4 && ptr_ok && qmv_q4_supported(N, K, qw->group_size);
+  const bool can_qmv = ptr_ok && ((qw->bits == 4 && qmv_q4_supported(N, K, qw->group_size)) ||
+                                  (qw->bits == 8 && qmv_q8_supported(N, K, qw->group_size)));
   const bool can_qmm_lds = ptr_ok && qmm_supported(N, K, qw->group_size, qw->bits);
   const bool can_qmm_rw = ptr_ok && qmm_rw_supported(N, K, qw->group_size, qw->bits);
   const bool can_qmm = can_qmm_lds || can_qmm_rw;
@@ -130,8 +131,9 @@ int32_t run_matmul(const rmlx_qweight* qw, const void* x, int32_t x_dtype, uint3
     else kernel = KERNEL_GENERIC;
   } else if (kernel == KERNEL_QMV && !can_qmv) {
     return fail(RMLX_INVALID_SHAPE,
-                "qmv kernel requires bits=4, group_size=64, N %% 16 == 0, K %% 512 == 0 and 16-byte aligned "
-                "buffers (N=%u K=%u bits=%u group_size=%u)", N, K, qw->bits, qw->group_size);
+                "qmv kernel requires bits in {4,8}, group_size=64, N %% 16 == 0, K %% 512 == 0 (4-bit) or "
+                "K %% 2048 == 0 (8-bit) and 16-byte aligned buffers (N=%u K=%u bits=%u group_size=%u)",
+                N, K, qw->bits, qw->group_size);
   } else if (kernel == KERNEL_QMM && !can_qmm) {
     return fail(RMLX_INVALID_SHAPE,
                 "qmm kernel requires bits in {4,8}, group_size=64, N %% 64 == 0, K %% 256 == 0 and 16-byte aligned "
@@ -180,6 +182,8 @@ int32_t run_matmul(const rmlx_qweight* qw, const void* x, int32_t x_dtype, uint3
     xk = cast.ptr;
   }
 
+  if (kernel == KERNEL_QMV && qw->bits == 8)
+    return launch_qmv_q8(qw->w, qw->s, qw->b, static_cast<const __half*>(xk), out, M, N, K, stream);
   if (kernel == KERNEL_QMV) {
     QmvArgs a{};
     a.w0 = qw->w; a.s0 = qw->s; a.b0 = qw->b;

@@ -126,6 +126,10 @@ struct QmvArgs {
 };
 int32_t launch_qmv_q4(const QmvArgs& a, hipStream_t s);
 bool qmv_q4_supported(uint32_t N, uint32_t K, uint32_t group_size);
+// 8-bit streaming GEMV (qmv_q8.hip): f16 activations [M,K], chunks of 16 rows.
+bool qmv_q8_supported(uint32_t N, uint32_t K, uint32_t group_size);
+int32_t launch_qmv_q8(const uint32_t* w, const __half* s, const __half* b, const __half* x, __half* out, uint32_t M,
+                      uint32_t N, uint32_t K, hipStream_t stream);
 // chunk table for gather_qmm: batch b owns rows [b*mpb, (b+1)*mpb) and expert indices[b]
 int32_t launch_build_gather_chunks(const uint32_t* indices, uint32_t batch, uint32_t mpb, uint32_t n_experts,
                                    uint32_t* chunk_tab, hipStream_t s);

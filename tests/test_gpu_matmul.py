@@ -303,3 +303,38 @@ def test_validation_errors(hip):
     # M = 0 is legal and returns an empty result
     out = ops.affine_quantized_matmul_batched(DeviceBuffer((0, k), 1), qw)
     assert out.shape == (0, n)
+
+
+# ---- 8-bit streaming GEMV (affine_qmv_fast_q8, quantized.rs:620-695) -----------------------------------
+
+@pytest.mark.parametrize("m", [1, 2, 7, 16, 17, 40])
+@pytest.mark.parametrize("n,k", [(64, 2048), (48, 4096)])
+def test_q8_qmv_matches_oracle(hip, m, n, k):
+    from rmlx_amd import runtime as rt
+    rng = np.random.default_rng(m * 7 + n + k)
+    words, s, b = make_weight(rng, n, k, 8)
+    x = make_x(rng, m, k)
+    ref = model.qmm(x_as_f64(x, "f16"), words, s, b, 64, 8)
+    assert_close(_run(hip, words, s, b, x, 8, kernel=rt.KERNEL_QMV), ref, f"q8 qmv M={m} N={n} K={k}")
+    if m <= 16:  # the ladder sends small M there by itself
+        assert_close(_run(hip, words, s, b, x, 8), ref, f"q8 auto M={m}")
+
+
+def test_q8_qmv_closed_form_and_positions(hip):
+    from rmlx_amd import runtime as rt
+    n, k = 32, 2048
+    words = np.full((n, k // 4), 0x07070707, np.uint32)  # all bytes 7, scale 1, bias 0, x = 1 -> 7*K (quantized.rs:11752-11800)
+    out = _run(hip, words, np.ones((n, k // 64), np.float16), np.zeros((n, k // 64), np.float16),
+               np.ones((3, k), np.float16), 8, kernel=rt.KERNEL_QMV)
+    assert np.array_equal(out, np.full((3, n), 7 * k, np.float16))
+    # one-hot activations pick out single weights
+    rng = np.random.default_rng(8)
+    words, s, b = make_weight(rng, n, k, 8)
+    s[:] = 1.0
+    b[:] = 0.0
+    q = model.unpack_u32(words, 8).astype(np.float64)
+    ks = np.array([0, 1, 3, 4, 7, 8, 15, 16, 63, 64, 65, 511, 512, 1023, 2047])
+    x = np.zeros((len(ks), k), np.float16)
+    x[np.arange(len(ks)), ks] = 1.0
+    out = _run(hip, words, s, b, x, 8, kernel=rt.KERNEL_QMV)
+    assert np.array_equal(out.astype(np.float64), q[:, ks].T)
