@@ -133,6 +133,18 @@ int32_t rmlx_hip_affine_quantized_matmul_batched(const rmlx_qweight* qw, const r
 int32_t rmlx_hip_qmm_select(const rmlx_qweight* qw, const rmlx_array* x, int32_t kernel,
                             void* out_f16_dev, size_t out_bytes, rmlx_stream stream);
 
+/* Fused store epilogues of the batched matmul (`qmm_add_residual_into_cb` quantized.rs:8227-8340,
+ * `qmm_swiglu_into_cb` :8345-8452): out = x @ dequant(W)^T + residual, resp.
+ * out = silu(gate_result) * (x @ dequant(W)^T).  residual / gate_result: [M, out_features],
+ * Float16 or Float32 (the reference's are Float32), same validation message as the reference
+ * ("... shape must be [M, N]"); out is f16.  Evaluated in f32 on the accumulator with one rounding
+ * in the GEMM kernel; after the GEMV / portable kernels as a separate elementwise pass.  Unlike the
+ * reference (Q4, M > 32 only) every shape the batched entry point takes is accepted. */
+int32_t rmlx_hip_qmm_add_residual(const rmlx_qweight* qw, const rmlx_array* x, const rmlx_array* residual,
+                                  void* out_f16_dev, size_t out_bytes, rmlx_stream stream);
+int32_t rmlx_hip_qmm_swiglu(const rmlx_qweight* qw, const rmlx_array* x, const rmlx_array* gate_result,
+                            void* out_f16_dev, size_t out_bytes, rmlx_stream stream);
+
 /* Encode `count` batched matmuls back to back on `stream` with no synchronisation in between:
  * the `_into_cb` usage of the reference, which encodes every QMM of a decoder stack into one
  * command buffer (`affine_quantized_matmul_batched_into_cb`, quantized.rs:7797-7802;

@@ -111,8 +111,24 @@ bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) ==
 enum { KERNEL_AUTO = 0, KERNEL_QMV = 1, KERNEL_QMM = 2, KERNEL_GENERIC = 3, KERNEL_QMM_BF16 = 4, KERNEL_QMM_LDS = 5 };
 constexpr uint32_t kQmvMaxM = 16;
 
+struct Epilogue { int kind = EPI_NONE; const void* ptr = nullptr; int32_t dtype = RMLX_DTYPE_F16; };
+
+int32_t run_matmul_plain(const rmlx_qweight* qw, const void* x, int32_t x_dtype, uint32_t M, __half* out,
+                         int32_t kernel, hipStream_t stream, const Epilogue& epi, bool* epi_done);
+
+// Matmul plus optional store epilogue: fused in the register-weights GEMM, a separate elementwise
+// pass after every other kernel.
 int32_t run_matmul(const rmlx_qweight* qw, const void* x, int32_t x_dtype, uint32_t M, __half* out,
-                   int32_t kernel, hipStream_t stream) {
+                   int32_t kernel, hipStream_t stream, const Epilogue& epi = Epilogue()) {
+  bool done = false;
+  RMLX_TRY(run_matmul_plain(qw, x, x_dtype, M, out, kernel, stream, epi, &done));
+  if (epi.kind != EPI_NONE && !done)
+    RMLX_TRY(launch_epilogue(out, epi.kind, epi.ptr, epi.dtype, (size_t)M * qw->out_features, stream));
+  return RMLX_OK;
+}
+
+int32_t run_matmul_plain(const rmlx_qweight* qw, const void* x, int32_t x_dtype, uint32_t M, __half* out,
+                         int32_t kernel, hipStream_t stream, const Epilogue& epi, bool* epi_done) {
   uint32_t N, K;
   RMLX_TRY(checked_u32(qw->out_features, "out_features", &N));
   RMLX_TRY(checked_u32(qw->in_features, "in_features", &K));
@@ -159,7 +175,8 @@ int32_t run_matmul(const rmlx_qweight* qw, const void* x, int32_t x_dtype, uint3
       RMLX_TRY(launch_cast_to_f16(x, x_dtype, static_cast<__half*>(cast.ptr), (size_t)M * K, stream));
       xk = cast.ptr;
     }
-    QmmArgs a{qw->w, qw->s, qw->b, xk, RMLX_DTYPE_F16, out, M, N, K, qw->bits, nullptr, 0};
+    QmmArgs a{qw->w, qw->s, qw->b, xk, RMLX_DTYPE_F16, out, M, N, K, qw->bits, nullptr, 0, epi.kind, epi.ptr, epi.dtype};
+    *epi_done = true;
     return launch_qmm_rw(a, qw->group_size, stream);
   }
   if (kernel == KERNEL_QMM || kernel == KERNEL_QMM_BF16 || kernel == KERNEL_QMM_LDS) {
@@ -476,6 +493,41 @@ int32_t rmlx_hip_qmm_select(const rmlx_qweight* qw, const rmlx_array* x, int32_t
 int32_t rmlx_hip_affine_quantized_matmul_batched(const rmlx_qweight* qw, const rmlx_array* x, void* out_f16_dev,
                                                  size_t out_bytes, rmlx_stream stream) {
   return rmlx_hip_qmm_select(qw, x, KERNEL_AUTO, out_f16_dev, out_bytes, stream);
+}
+
+namespace {
+int32_t qmm_with_epilogue(const char* what, const char* operand, int kind, const rmlx_qweight* qw, const rmlx_array* x,
+                          const rmlx_array* e, void* out_f16_dev, size_t out_bytes, rmlx_stream stream) {
+  RMLX_TRY(require_init());
+  if (qw == nullptr || x == nullptr || e == nullptr) return fail(RMLX_INVALID_SHAPE, "%s: null argument", what);
+  RMLX_TRY(check_x_dtype(what, x->dtype));
+  if (x->ndim != 2) return fail(RMLX_INVALID_SHAPE, "%s requires 2D input x, got %dD", what, x->ndim);
+  if (x->shape[1] != qw->in_features)
+    return fail(RMLX_INVALID_SHAPE, "x.shape[1] (%zu) != in_features (%zu)", x->shape[1], qw->in_features);
+  if (qw->bits != 4 && qw->bits != 8) return fail(RMLX_INVALID_SHAPE, "%s requires bits==4 or bits==8, got %u", what, qw->bits);
+  if (qw->n_experts != 1) return fail(RMLX_INVALID_SHAPE, "%s: weight is a stacked expert weight", what);
+  if (e->ndim != 2 || e->shape[0] != x->shape[0] || e->shape[1] != qw->out_features)
+    return fail(RMLX_INVALID_SHAPE, "%s: %s shape must be [%zu, %zu]", what, operand, x->shape[0], qw->out_features);
+  if (e->dtype != RMLX_DTYPE_F16 && e->dtype != RMLX_DTYPE_F32)
+    return fail(RMLX_INVALID_SHAPE, "%s: %s must be Float16 or Float32, got %s", what, operand, dtype_name(e->dtype));
+  uint32_t M;
+  RMLX_TRY(checked_u32(x->shape[0], "M", &M));
+  RMLX_TRY(check_out(what, out_bytes, (size_t)M * qw->out_features * 2));
+  Epilogue epi;
+  epi.kind = kind; epi.ptr = e->data; epi.dtype = e->dtype;
+  RMLX_TRY(run_matmul(qw, x->data, x->dtype, M, static_cast<__half*>(out_f16_dev), KERNEL_AUTO, (hipStream_t)stream, epi));
+  return finish((hipStream_t)stream);
+}
+}  // namespace
+
+int32_t rmlx_hip_qmm_add_residual(const rmlx_qweight* qw, const rmlx_array* x, const rmlx_array* residual,
+                                  void* out_f16_dev, size_t out_bytes, rmlx_stream stream) {
+  return qmm_with_epilogue("qmm_add_residual_into_cb", "residual", EPI_RESIDUAL, qw, x, residual, out_f16_dev, out_bytes, stream);
+}
+
+int32_t rmlx_hip_qmm_swiglu(const rmlx_qweight* qw, const rmlx_array* x, const rmlx_array* gate_result,
+                            void* out_f16_dev, size_t out_bytes, rmlx_stream stream) {
+  return qmm_with_epilogue("qmm_swiglu_into_cb", "gate_result", EPI_SWIGLU, qw, x, gate_result, out_f16_dev, out_bytes, stream);
 }
 
 int32_t rmlx_hip_qmm_encode_many(const rmlx_qweight* const* qws, size_t n_qw, const rmlx_array* x,

@@ -142,7 +142,14 @@ struct QmmArgs {
   uint32_t M, N, K, bits;
   void* workspace;    // qmm_workspace_bytes(M, K) bytes of device scratch (fragment-major activations)
   int bf16_mfma;      // 1: bf16 activations x Q8 weights on the bf16 MFMA (weights rounded to bf16)
+  // fused store epilogue (register-weights GEMM only): 0 none, 1 out = acc + e, 2 out = silu(e) * acc
+  int epi_kind;
+  const void* epi;    // [M,N] f16 or f32
+  int32_t epi_dtype;
 };
+enum { EPI_NONE = 0, EPI_RESIDUAL = 1, EPI_SWIGLU = 2 };
+// out[i] = out[i] + e[i]  /  silu(e[i]) * out[i], in place on f16 out (kernels without a fused epilogue)
+int32_t launch_epilogue(__half* out, int kind, const void* e, int32_t e_dtype, size_t n, hipStream_t s);
 size_t qmm_workspace_bytes(uint32_t M, uint32_t K);
 bool qmm_supported(uint32_t N, uint32_t K, uint32_t group_size, uint32_t bits);
 int32_t launch_qmm(const QmmArgs& a, hipStream_t s);

@@ -139,4 +139,24 @@ int32_t launch_check_indices(const uint32_t* idx, uint32_t n, uint32_t limit, ui
   return RMLX_OK;
 }
 
+namespace {
+__global__ void epilogue_kernel(__half* __restrict__ out, int kind, const void* __restrict__ e, int32_t e_dtype, size_t n) {
+  const size_t stride = (size_t)gridDim.x * blockDim.x;
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) {
+    const float ev = e_dtype == RMLX_DTYPE_F32 ? static_cast<const float*>(e)[i] : __half2float(static_cast<const __half*>(e)[i]);
+    const float v = __half2float(out[i]);
+    out[i] = __float2half(kind == EPI_RESIDUAL ? v + ev : ev / (1.0f + __expf(-ev)) * v);
+  }
+}
+}  // namespace
+
+int32_t launch_epilogue(__half* out, int kind, const void* e, int32_t e_dtype, size_t n, hipStream_t s) {
+  if (n == 0 || kind == EPI_NONE) return RMLX_OK;
+  size_t blocks = (n + 255) / 256;
+  if (blocks > 4096) blocks = 4096;
+  hipLaunchKernelGGL(epilogue_kernel, dim3((unsigned)blocks), dim3(256), 0, s, out, kind, e, e_dtype, n);
+  RMLX_HIP_CHECK(hipGetLastError());
+  return RMLX_OK;
+}
+
 }  // namespace rmlx

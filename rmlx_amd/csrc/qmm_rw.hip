@@ -46,6 +46,8 @@ struct RwParams {
   __half* out;
   uint32_t M, N, K;
   uint32_t tiles_m, tiles_n;
+  int32_t epi_kind, epi_dtype;  // fused store epilogue: EPI_RESIDUAL / EPI_SWIGLU with an [M,N] f16 / f32 operand
+  const void* epi;
 #ifdef QMM_RW_TRACE
   unsigned long long* trace;
 #endif
@@ -329,8 +331,24 @@ __global__ __launch_bounds__(64 * NW) void qmm_rw_kernel(RwParams p) {
 #pragma unroll
       for (int f = 0; f < NF; ++f) {
         const uint32_t col = nt * (NW * 16 * NF) + wave * (16 * NF) + f * 16 + 4 * g;
-        const h2 lo = {(_Float16)acc[i][f][0], (_Float16)acc[i][f][1]};
-        const h2 hi = {(_Float16)acc[i][f][2], (_Float16)acc[i][f][3]};
+        f4 v = acc[i][f];
+        if (p.epi_kind != EPI_NONE) {  // residual add / SwiGLU gate in f32, one rounding (quantized.rs:3206-3246)
+          f4 e;
+          if (p.epi_dtype == RMLX_DTYPE_F32) {
+            e = *reinterpret_cast<const f4*>(static_cast<const float*>(p.epi) + (uint64_t)m * p.N + col);
+          } else {
+            const u2 eb = *reinterpret_cast<const u2*>(static_cast<const __half*>(p.epi) + (uint64_t)m * p.N + col);
+            // (copy the elements to scalars first: __builtin_bit_cast applied to a vector element
+            // expression reads element 0 with this compiler)
+            const uint32_t ex = eb.x, ey = eb.y;
+            const h2 e0 = __builtin_bit_cast(h2, ex), e1 = __builtin_bit_cast(h2, ey);
+            e = (f4){(float)e0[0], (float)e0[1], (float)e1[0], (float)e1[1]};
+          }
+#pragma unroll
+          for (int q = 0; q < 4; ++q) v[q] = p.epi_kind == EPI_RESIDUAL ? v[q] + e[q] : e[q] / (1.0f + __expf(-e[q])) * v[q];
+        }
+        const h2 lo = {(_Float16)v[0], (_Float16)v[1]};
+        const h2 hi = {(_Float16)v[2], (_Float16)v[3]};
         *reinterpret_cast<u2*>(p.out + (uint64_t)m * p.N + col) = (u2){h2bits(lo), h2bits(hi)};
       }
     }
@@ -386,6 +404,7 @@ int32_t launch_qmm_rw(const QmmArgs& a, uint32_t group_size, hipStream_t s) {
   p.w = a.w; p.s = a.s; p.b = a.b;
   p.x = static_cast<const __half*>(a.x);
   p.out = a.out; p.M = a.M; p.N = a.N; p.K = a.K;
+  p.epi_kind = a.epi_kind; p.epi = a.epi; p.epi_dtype = a.epi_dtype;
 #ifdef QMM_RW_TRACE
   p.trace = g_qmm_rw_trace;
 #endif

@@ -69,6 +69,22 @@ def affine_quantized_matmul_batched(x, qw, stream=None, kernel=rt.KERNEL_AUTO, o
     return out
 
 
+def qmm_add_residual(x, qw, residual, stream=None):
+    """`qmm_add_residual_into_cb` (quantized.rs:8227-8340): QMM(x, qw) + residual, f16 out."""
+    out = DeviceBuffer((x.shape[0] if len(x.shape) == 2 else 0, qw.out_features), F16)
+    a, r = x.array(), residual.array()
+    rt.check(rt.lib().rmlx_hip_qmm_add_residual(qw.handle, ctypes.byref(a), ctypes.byref(r), out.ptr, out.nbytes, _h(stream)))
+    return out
+
+
+def qmm_swiglu(x, qw, gate_result, stream=None):
+    """`qmm_swiglu_into_cb` (quantized.rs:8345-8452): silu(gate_result) * QMM(x, qw), f16 out."""
+    out = DeviceBuffer((x.shape[0] if len(x.shape) == 2 else 0, qw.out_features), F16)
+    a, g = x.array(), gate_result.array()
+    rt.check(rt.lib().rmlx_hip_qmm_swiglu(qw.handle, ctypes.byref(a), ctypes.byref(g), out.ptr, out.nbytes, _h(stream)))
+    return out
+
+
 def qmm_encode_many(qws, x, outs, count, stream=None, kernel=rt.KERNEL_AUTO):
     """Encode `count` matmuls back to back (weights and outputs are cycled) -- see rmlx_hip_qmm_encode_many."""
     qarr = (ctypes.c_void_p * len(qws))(*[q.handle for q in qws])

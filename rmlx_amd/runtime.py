@@ -37,7 +37,7 @@ EXPORTS = [
     "rmlx_hip_stream_create", "rmlx_hip_stream_sync", "rmlx_hip_stream_destroy", "rmlx_hip_event_create",
     "rmlx_hip_event_record", "rmlx_hip_event_sync", "rmlx_hip_event_elapsed_ms", "rmlx_hip_event_destroy",
     "rmlx_hip_qweight_create", "rmlx_hip_qweight_destroy", "rmlx_hip_affine_quantized_matmul",
-    "rmlx_hip_affine_quantized_matmul_batched", "rmlx_hip_qmm_select", "rmlx_hip_qmm_encode_many", "rmlx_hip_quantized_linear_forward",
+    "rmlx_hip_affine_quantized_matmul_batched", "rmlx_hip_qmm_select", "rmlx_hip_qmm_add_residual", "rmlx_hip_qmm_swiglu", "rmlx_hip_qmm_encode_many", "rmlx_hip_quantized_linear_forward",
     "rmlx_hip_gather_qmm", "rmlx_hip_topk_route", "rmlx_hip_moe_sort", "rmlx_hip_index_gather",
     "rmlx_hip_scatter_weighted_add", "rmlx_hip_silu_gate", "rmlx_hip_expert_group_grouped_forward",
     "rmlx_hip_moe_forward_grouped", "rmlx_hip_moe_forward",
@@ -81,6 +81,8 @@ def lib():
         "rmlx_hip_affine_quantized_matmul": [vp, arr, vp, sz, vp],
         "rmlx_hip_affine_quantized_matmul_batched": [vp, arr, vp, sz, vp],
         "rmlx_hip_qmm_select": [vp, arr, i32, vp, sz, vp],
+        "rmlx_hip_qmm_add_residual": [vp, arr, arr, vp, sz, vp],
+        "rmlx_hip_qmm_swiglu": [vp, arr, arr, vp, sz, vp],
         "rmlx_hip_qmm_encode_many": [ctypes.POINTER(vp), sz, arr, ctypes.POINTER(vp), sz, sz, sz, i32, vp],
         "rmlx_hip_quantized_linear_forward": [vp, arr, vp, vp, sz, vp],
         "rmlx_hip_gather_qmm": [arr, vp, sz, vp, sz, vp, sz, arr, sz, sz, sz, sz, sz, u32, vp, sz, vp],

@@ -338,3 +338,38 @@ def test_q8_qmv_closed_form_and_positions(hip):
     x[np.arange(len(ks)), ks] = 1.0
     out = _run(hip, words, s, b, x, 8, kernel=rt.KERNEL_QMV)
     assert np.array_equal(out.astype(np.float64), q[:, ks].T)
+
+
+# ---- fused store epilogues (qmm_add_residual_into_cb / qmm_swiglu_into_cb, quantized.rs:8227-8452) -------
+
+@pytest.mark.parametrize("m,n,k,bits", [(64, 256, 512, 4), (130, 128, 1024, 4), (40, 128, 512, 8), (4, 64, 512, 4), (9, 24, 128, 4)])
+@pytest.mark.parametrize("edtype", ["f16", "f32"])
+def test_fused_epilogues(hip, m, n, k, bits, edtype):
+    """GEMM (fused), GEMV and portable (separate pass) kernels against the f64 composition."""
+    from rmlx_amd import ops
+    from rmlx_amd.runtime import DeviceBuffer
+    rng = np.random.default_rng(m + n + k + bits)
+    words, s, b = make_weight(rng, n, k, bits)
+    x = make_x(rng, m, k)
+    e = rng.standard_normal((m, n)).astype(np.float16 if edtype == "f16" else np.float32)
+    qw = ops.QuantizedWeight.from_numpy(words, s, b, 64, bits)
+    base = model.qmm(x_as_f64(x, "f16"), words, s, b, 64, bits)
+    e64 = e.astype(np.float64)
+    xd, ed = DeviceBuffer.from_numpy(x), DeviceBuffer.from_numpy(e)
+    assert_close(ops.qmm_add_residual(xd, qw, ed).numpy(), base + e64, "qmm_add_residual")
+    assert_close(ops.qmm_swiglu(xd, qw, ed).numpy(), model.silu(e64) * base, "qmm_swiglu")
+
+
+def test_fused_epilogue_validation(hip):
+    from rmlx_amd import ops
+    from rmlx_amd.runtime import DeviceBuffer
+    rng = np.random.default_rng(3)
+    words, s, b = make_weight(rng, 64, 512, 4)
+    qw = ops.QuantizedWeight.from_numpy(words, s, b, 64, 4)
+    xd = DeviceBuffer.from_numpy(make_x(rng, 8, 512))
+    with pytest.raises(ops.KernelError, match=r"qmm_add_residual_into_cb: residual shape must be \[8, 64\]"):
+        ops.qmm_add_residual(xd, qw, DeviceBuffer.from_numpy(np.zeros((8, 32), np.float16)))
+    with pytest.raises(ops.KernelError, match=r"qmm_swiglu_into_cb: gate_result shape must be \[8, 64\]"):
+        ops.qmm_swiglu(xd, qw, DeviceBuffer.from_numpy(np.zeros((4, 64), np.float32)))
+    with pytest.raises(ops.KernelError, match="gate_result must be Float16 or Float32"):
+        ops.qmm_swiglu(xd, qw, DeviceBuffer.from_numpy(np.zeros((8, 64), np.uint32)))
