@@ -124,11 +124,21 @@ __global__ __launch_bounds__(64 * NW) void qmm_rw_kernel(RwParams p) {
   RW_MARK(p, 8, 6);
   RW_MARK_ALL(p, 0);
 
-  // Workgroups that share a weight panel get ids that are congruent mod 8 apart, i.e. run on one XCD.
-  uint32_t wg = blockIdx.x;
+  // Workgroup -> tile.  Consecutive workgroup ids go round-robin over the 8 XCDs (one L2 each), so
+  // XCD x = id % 8 runs the ids congruent to x.  Give every XCD a compact block of tiles, half of
+  // the row tiles x a quarter of the column tiles when those divide, so that what its L2 has to
+  // fetch (its activation rows + its weight panels) is smallest; else whole weight panels per XCD.
+  uint32_t wg = blockIdx.x, mt, nt;
   const uint32_t total = p.tiles_m * p.tiles_n;
-  if (total % 8 == 0) wg = (wg % 8) * (total / 8) + wg / 8;
-  const uint32_t mt = wg % p.tiles_m, nt = wg / p.tiles_m;
+  if (total % 8 == 0 && p.tiles_m % 2 == 0 && p.tiles_n % 4 == 0) {
+    const uint32_t xcd = wg % 8, local = wg / 8, bm = p.tiles_m / 2, bn = p.tiles_n / 4;
+    mt = (xcd % 2) * bm + local % bm;
+    nt = (xcd / 2) * bn + local / bm;
+  } else {
+    if (total % 8 == 0) wg = (wg % 8) * (total / 8) + wg / 8;
+    mt = wg % p.tiles_m;
+    nt = wg / p.tiles_m;
+  }
 
   const uint32_t K = p.K, S = K / kBlockK, G = K / 64;
   const uint32_t row_base = nt * (NW * 16 * NF) + wave * (16 * NF) + n;
