@@ -166,16 +166,19 @@ int32_t run_matmul_plain(const rmlx_qweight* qw, const void* x, int32_t x_dtype,
   }
 
   if (kernel == KERNEL_QMM && can_qmm_rw) {
-    // Register-weights GEMM: f16 activations straight from the row-major matrix, no workspace.
-    // bf16 -> f16 is exact for normal-range values and f16 weights keep 11 significant bits.
+    // Register-weights GEMM: f16 / bf16 activations straight from the row-major matrix, no workspace
+    // (bf16 -> f16 inside the kernel: exact for normal-range values, and f16 weights keep 11
+    // significant bits); f32 activations are cast first.
     Scratch cast;
     const void* xk = x;
-    if (x_dtype != RMLX_DTYPE_F16) {
+    int32_t xk_dtype = x_dtype;
+    if (x_dtype == RMLX_DTYPE_F32) {
+      xk_dtype = RMLX_DTYPE_F16;
       RMLX_TRY(cast.alloc((size_t)M * K * sizeof(__half), stream));
       RMLX_TRY(launch_cast_to_f16(x, x_dtype, static_cast<__half*>(cast.ptr), (size_t)M * K, stream));
       xk = cast.ptr;
     }
-    QmmArgs a{qw->w, qw->s, qw->b, xk, RMLX_DTYPE_F16, out, M, N, K, qw->bits, nullptr, 0, epi.kind, epi.ptr, epi.dtype};
+    QmmArgs a{qw->w, qw->s, qw->b, xk, xk_dtype, out, M, N, K, qw->bits, nullptr, 0, epi.kind, epi.ptr, epi.dtype};
     *epi_done = true;
     return launch_qmm_rw(a, qw->group_size, stream);
   }

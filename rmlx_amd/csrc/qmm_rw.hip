@@ -15,7 +15,8 @@
 //   * The waves of a workgroup (4 or 8) split the N extent of the tile: every weight is loaded
 //     and dequantized by exactly one wave.
 //   * Activations are shared by the waves and go through LDS.  They are read from the row-major
-//     [M,K] matrix with coalesced 16-byte loads (16 lanes per 256-byte row piece), permuted to
+//     [M,K] matrix (f16, or bf16 converted on the way) with coalesced 16-byte loads (16 lanes
+//     per 256-byte row piece), permuted to
 //     the slot order of the nibble unpacking and written to an xor-swizzled operand layout, so
 //     both the writes and the 16-byte operand reads are bank-conflict free.  No prepass, no
 //     workspace.
@@ -42,7 +43,7 @@ constexpr int kUnroll = 4;   // main-loop unrolling = depth of the weight regist
 
 struct RwParams {
   const uint32_t* w; const __half* s; const __half* b;
-  const __half* x;   // [M,K] f16 row-major
+  const __half* x;   // [M,K] row-major, f16 (or bf16 bits when XBF16)
   __half* out;
   uint32_t M, N, K;
   uint32_t tiles_m, tiles_n;
@@ -110,7 +111,7 @@ __device__ __forceinline__ h8 dequant_q8_pair(uint32_t w0, uint32_t w1, h2 s2, h
 
 // MF = 16-row activation fragments per workgroup (tile rows = 16*MF), NF = 16-row weight fragments
 // per wave (tile columns = 64*NF), BITS = 4 or 8.
-template <int MF, int NF, int BITS, int NW>
+template <int MF, int NF, int BITS, int NW, bool XBF16>
 __global__ __launch_bounds__(64 * NW) void qmm_rw_kernel(RwParams p) {
   constexpr int kThreads = 64 * NW;
   constexpr int AL = MF * 256 / kThreads;      // 16-byte activation loads per thread and chunk
@@ -192,6 +193,15 @@ __global__ __launch_bounds__(64 * NW) void qmm_rw_kernel(RwParams p) {
 
   // Q4: halves (k0..k7) -> slots (k0,k4,k1,k5,k2,k6,k3,k7), the order the nibble unpacking produces
   auto to_slot_order = [&](u4 v) {
+    if (XBF16) {  // bf16 activations: to f16 through f32 (exact for normal-range values), round to nearest even
+      uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const float lo = __uint_as_float(w[e] << 16), hi = __uint_as_float(w[e] & 0xFFFF0000u);
+        w[e] = h2bits((h2){(_Float16)lo, (_Float16)hi});
+      }
+      v = (u4){w[0], w[1], w[2], w[3]};
+    }
     if (BITS != 4) return v;
     u4 o;
     o.x = __builtin_amdgcn_perm(v.z, v.x, 0x05040100u);
@@ -368,10 +378,12 @@ __global__ __launch_bounds__(64 * NW) void qmm_rw_kernel(RwParams p) {
 }
 
 template <int MF, int NF, int BITS, int NW>
-void launch_rw(RwParams p, hipStream_t s) {
+void launch_rw(RwParams p, bool x_bf16, hipStream_t s) {
   p.tiles_m = (p.M + 16 * MF - 1) / (16 * MF);
   p.tiles_n = p.N / (NW * 16 * NF);
-  hipLaunchKernelGGL((qmm_rw_kernel<MF, NF, BITS, NW>), dim3(p.tiles_m * p.tiles_n), dim3(64 * NW), 0, s, p);
+  const dim3 grid(p.tiles_m * p.tiles_n), block(64 * NW);
+  if (x_bf16) hipLaunchKernelGGL((qmm_rw_kernel<MF, NF, BITS, NW, true>), grid, block, 0, s, p);
+  else hipLaunchKernelGGL((qmm_rw_kernel<MF, NF, BITS, NW, false>), grid, block, 0, s, p);
 }
 
 }  // namespace
@@ -391,7 +403,9 @@ int32_t launch_qmm_rw(const QmmArgs& a, uint32_t group_size, hipStream_t s) {
   if (!qmm_rw_supported(a.N, a.K, group_size, a.bits))
     return fail(RMLX_INVALID_SHAPE, "qmm: unsupported shape N=%u K=%u bits=%u group_size=%u", a.N, a.K, a.bits, group_size);
   if (a.M == 0) return RMLX_OK;
-  if (a.x_dtype != RMLX_DTYPE_F16) return fail(RMLX_RUNTIME_ERROR, "qmm: activations must be cast to f16 first");
+  if (a.x_dtype != RMLX_DTYPE_F16 && a.x_dtype != RMLX_DTYPE_BF16)
+    return fail(RMLX_RUNTIME_ERROR, "qmm: f32 activations must be cast to f16 first");
+  const bool x_bf16 = a.x_dtype == RMLX_DTYPE_BF16;
 
   // Tile choice {MF, NF, NW} (tile rows 16*MF, tile columns 16*NF*NW): least estimated time =
   // rounds of workgroups over the CUs x work per tile / measured relative efficiency of the tile.
@@ -420,7 +434,7 @@ int32_t launch_qmm_rw(const QmmArgs& a, uint32_t group_size, hipStream_t s) {
 #endif
 #define RW_CASE(MFV, NFV, NWV)                                                                 \
   if (mf == MFV && nf == NFV && nw == NWV) {                                                   \
-    if (a.bits == 4) launch_rw<MFV, NFV, 4, NWV>(p, s); else launch_rw<MFV, NFV, 8, NWV>(p, s); \
+    if (a.bits == 4) launch_rw<MFV, NFV, 4, NWV>(p, x_bf16, s); else launch_rw<MFV, NFV, 8, NWV>(p, x_bf16, s); \
   }
   RW_CASE(4, 2, 8) RW_CASE(4, 1, 8) RW_CASE(2, 1, 8) RW_CASE(2, 1, 4) RW_CASE(4, 2, 4) RW_CASE(2, 2, 4)
   RW_CASE(8, 1, 8)
