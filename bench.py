@@ -84,7 +84,7 @@ def bench_matmul(ops, rt, timer, rng, m, n, k, bits, x_dtype, steps, warmup, min
         x64 = xh.astype(np.float64)
     outs = [rt.DeviceBuffer((m, n), rt.F16) for _ in range(min(n_sets, 8))]
     ms = timer.run(lambda c: ops.qmm_encode_many(qws, xd, outs, c, stream=timer.stream, kernel=kernel), steps, warmup)
-    res = {"us": ms * 1e3, "n_weight_sets": n_sets,
+    res = {"us": ms * 1e3, "steps": steps, "n_weight_sets": n_sets,
            "bytes": matmul_bytes(m, n, k, bits, act_bytes=2), "flops": 2 * m * n * k}
     res["gbs"] = res["bytes"] / (ms * 1e-3) / 1e9
     res["tflops"] = res["flops"] / (ms * 1e-3) / 1e12
@@ -180,7 +180,6 @@ def main():
                                  "write_bytes": rows * 4096 * 2}
     del src, ident
     if not args.quick:
-        small = max(20, args.steps // 20)
         extra["q4_qmv_m1_4096_cache_resident"] = bench_matmul(ops, rt, timer, rng, 1, 4096, 4096, 4, "f16",
                                                               args.steps, args.warmup, 0, check=False)
         for m in (1, 4, 8):
@@ -188,12 +187,14 @@ def main():
                                                        args.warmup, GiB + GiB // 8, check=(m == 8))
         extra["q8_qmv_m1_4096"] = bench_matmul(ops, rt, timer, rng, 1, 4096, 4096, 8, "f16", args.steps, args.warmup,
                                                GiB + GiB // 8)
+        # the GEMM sections run as many steps as the headline: the GPU needs tens of milliseconds of
+        # sustained matrix work before its clock settles (a 100-launch window reads 15 % slower)
         for m in (128, 512):
-            r = bench_matmul(ops, rt, timer, rng, m, 4096, 4096, 4, "f16", small, 10, 4 * 9437184)
+            r = bench_matmul(ops, rt, timer, rng, m, 4096, 4096, 4, "f16", args.steps, args.warmup, 4 * 9437184)
             r["mfma_frac"] = r["tflops"] / MFMA_F16_PEAK_TF
             extra[f"q4_qmm_m{m}_4096"] = r
         for name, kern in (("q8_qmm_bf16_m128_n12288", rt.KERNEL_AUTO), ("q8_qmm_bf16_m128_n12288_bf16_mfma", rt.KERNEL_QMM_BF16)):
-            r = bench_matmul(ops, rt, timer, rng, 128, 12288, 4096, 8, "bf16", small, 10, 4 * 53477376, kernel=kern)
+            r = bench_matmul(ops, rt, timer, rng, 128, 12288, 4096, 8, "bf16", args.steps, args.warmup, 4 * 53477376, kernel=kern)
             r["mfma_frac"] = r["tflops"] / MFMA_F16_PEAK_TF
             r["hbm_frac"] = r["gbs"] / HBM_PEAK_GBS
             extra[name] = r
@@ -202,7 +203,7 @@ def main():
         experts = (gate_up, down, ops.QuantizedWeight.from_numpy(*gate_up, 64, 4),
                    ops.QuantizedWeight.from_numpy(*down, 64, 4))
         for T in (4, 32, 128):
-            r = bench_moe(ops, rt, timer, rng, T, max(10, small // 2), 5, experts)
+            r = bench_moe(ops, rt, timer, rng, T, max(50, args.steps // 10), 10, experts)
             r["hbm_frac"] = r["gbs"] / HBM_PEAK_GBS
             extra[f"moe_q4_T{T}"] = r
 

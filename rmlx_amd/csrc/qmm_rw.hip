@@ -411,7 +411,7 @@ int32_t launch_qmm_rw(const QmmArgs& a, uint32_t group_size, hipStream_t s) {
   // rounds of workgroups over the CUs x work per tile / measured relative efficiency of the tile.
   const uint32_t cus = (uint32_t)ctx().num_cus;
   static const struct { int mf, nf, nw; float eff; } cand[] = {
-      {8, 1, 8, 1.03f}, {4, 2, 8, 1.0f}, {4, 2, 4, 0.9f}, {4, 1, 8, 0.8f}, {2, 2, 4, 0.65f}, {2, 1, 8, 0.6f}, {2, 1, 4, 0.5f}};
+      {8, 1, 8, 1.01f}, {4, 2, 8, 1.0f}, {4, 1, 8, 0.93f}, {4, 2, 4, 0.9f}, {2, 2, 4, 0.7f}, {2, 1, 4, 0.55f}, {2, 1, 8, 0.45f}};
   int mf = 2, nf = 1, nw = 4;
   float best = 0.f;
   for (const auto& c : cand) {
