@@ -268,75 +268,96 @@ __global__ __launch_bounds__(kThreads) void qmv_q4_kernel(KParams p) {
     }
     QMV_MARK(p, 2);
 
-    // ---- 2b. per (row, group) sums of the activations, on the matrix unit while the weights are
-    //          still in flight: columns 0-7 of a constant B operand hold the unpack offsets
-    //          (1024 for even k, 64 for odd k, in slot order), columns 8-15 hold ones, so
-    //          accumulator column n < 8 receives sum(off*x) and column n >= 8 sum(x) of its rows.
-    f4 xsums[kSpwMax];
+    // ---- 2b/3 for 8 rows: slab by slab (few live registers).  The per (row, group) sums of the
+    //          activations come from the matrix unit: columns 0-7 of a constant B operand hold the
+    //          unpack offsets (1024 for even k, 64 for odd k, in slot order), columns 8-15 hold
+    //          ones, so accumulator column n < 8 receives sum(off*x) and column n >= 8 sum(x) of
+    //          its rows; lane n^8 holds the other one.
+    if constexpr (kMfmaSums) {
+      u4 sv[TILES], bv[TILES];
 #pragma unroll
-    for (int it = 0; it < kSpwMax; ++it) {
-      xsums[it] = (f4){0.f, 0.f, 0.f, 0.f};
-      if (kMfmaSums && it < my) {
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          h8 av = (h8){0, 0, 0, 0, 0, 0, 0, 0};
-          if (a_active) av = *reinterpret_cast<const h8*>(xs + ((it * 4 + j) * kSlots) * 16 + a_slot_off);
-          xsums[it] = __builtin_amdgcn_mfma_f32_16x16x32_f16(av, bconst, xsums[it], 0, 0, 0);
-        }
+      for (int t = 0; t < TILES; ++t) {
+        const u4 other = (u4){swap16(sbv[t].x), swap16(sbv[t].y), swap16(sbv[t].z), swap16(sbv[t].w)};
+        sv[t] = (g & 1) ? other : sbv[t];
+        bv[t] = (g & 1) ? sbv[t] : other;
       }
-    }
-
-    // ---- 3. weights: integer dot per group via MFMA (independent slabs interleaved), then
-    //         acc += scale * (dot - sum(off*x)) + bias * sum(x) in f32 ------------------------
-#pragma unroll
-    for (int t = 0; t < TILES; ++t) {
-      f4 c[kSpwMax];
-#pragma unroll
-      for (int it = 0; it < kSpwMax; ++it) c[it] = (f4){0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        h8 av[kSpwMax];
-#pragma unroll
-        for (int it = 0; it < kSpwMax; ++it) {
-          av[it] = (h8){0, 0, 0, 0, 0, 0, 0, 0};
-          if (it < my && a_active)
-            av[it] = *reinterpret_cast<const h8*>(xs + ((it * 4 + j) * kSlots) * 16 + a_slot_off);
-        }
-#pragma unroll
-        for (int it = 0; it < kSpwMax; ++it) {
-          if (it < my) {
-            const uint32_t wd = j == 0 ? wreg[t][it].x : (j == 1 ? wreg[t][it].y : (j == 2 ? wreg[t][it].z : wreg[t][it].w));
-            c[it] = __builtin_amdgcn_mfma_f32_16x16x32_f16(av[it], unpack_q4_word(wd), c[it], 0, 0, 0);
-          }
-        }
-      }
-      const u4 other = (u4){swap16(sbv[t].x), swap16(sbv[t].y), swap16(sbv[t].z), swap16(sbv[t].w)};
-      const u4 sv = (g & 1) ? other : sbv[t];
-      const u4 bv = (g & 1) ? sbv[t] : other;
 #pragma unroll
       for (int it = 0; it < kSpwMax; ++it) {
         if (it < my) {
-          const uint32_t swd = it == 0 ? sv.x : (it == 1 ? sv.y : (it == 2 ? sv.z : sv.w));
-          const uint32_t bwd = it == 0 ? bv.x : (it == 1 ? bv.y : (it == 2 ? bv.z : bv.w));
-          const float sc = __half2float(__ushort_as_half((unsigned short)(par ? swd >> 16 : swd & 0xFFFFu)));
-          const float bi = __half2float(__ushort_as_half((unsigned short)(par ? bwd >> 16 : bwd & 0xFFFFu)));
-          if constexpr (kMfmaSums) {
-            // own column holds sum(off*x) (n < 8) or sum(x) (n >= 8) of rows 4g..4g+3, lane n^8 the other
+          f4 own = (f4){0.f, 0.f, 0.f, 0.f};
+          f4 c[TILES];
+#pragma unroll
+          for (int t = 0; t < TILES; ++t) c[t] = (f4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            h8 av = (h8){0, 0, 0, 0, 0, 0, 0, 0};
+            if (a_active) av = *reinterpret_cast<const h8*>(xs + ((it * 4 + j) * kSlots) * 16 + a_slot_off);
+            own = __builtin_amdgcn_mfma_f32_16x16x32_f16(av, bconst, own, 0, 0, 0);
+#pragma unroll
+            for (int t = 0; t < TILES; ++t) {
+              const uint32_t wd = j == 0 ? wreg[t][it].x : (j == 1 ? wreg[t][it].y : (j == 2 ? wreg[t][it].z : wreg[t][it].w));
+              c[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(av, unpack_q4_word(wd), c[t], 0, 0, 0);
+            }
+          }
+          const float o0 = swap8(own.x), o1 = swap8(own.y), o2 = swap8(own.z), o3 = swap8(own.w);
+#pragma unroll
+          for (int t = 0; t < TILES; ++t) {
+            const uint32_t swd = it == 0 ? sv[t].x : (it == 1 ? sv[t].y : (it == 2 ? sv[t].z : sv[t].w));
+            const uint32_t bwd = it == 0 ? bv[t].x : (it == 1 ? bv[t].y : (it == 2 ? bv[t].z : bv[t].w));
+            const float sc = __half2float(__ushort_as_half((unsigned short)(par ? swd >> 16 : swd & 0xFFFFu)));
+            const float bi = __half2float(__ushort_as_half((unsigned short)(par ? bwd >> 16 : bwd & 0xFFFFu)));
             const float ce = n < 8 ? -sc : bi, co = n < 8 ? bi : -sc;
-            const f4 own = xsums[it];
-            const float o0 = swap8(own.x), o1 = swap8(own.y), o2 = swap8(own.z), o3 = swap8(own.w);
-            F[t][0] += sc * c[it][0] + ce * own.x + co * o0;
-            F[t][1] += sc * c[it][1] + ce * own.y + co * o1;
-            F[t][2] += sc * c[it][2] + ce * own.z + co * o2;
-            F[t][3] += sc * c[it][3] + ce * own.w + co * o3;
-          } else {
-            const float* sp = sums + ((it * 2 + par) * 8 + (g & 1) * 4) * 2;
-            const f4 c01 = *reinterpret_cast<const f4*>(sp);      // (-xoff, xsum) of accumulator rows 4g, 4g+1
-            const f4 c23 = *reinterpret_cast<const f4*>(sp + 4);  // rows 4g+2, 4g+3
-            F[t][0] += sc * (c[it][0] + c01[0]) + bi * c01[1];
-            F[t][1] += sc * (c[it][1] + c01[2]) + bi * c01[3];
-            F[t][2] += sc * (c[it][2] + c23[0]) + bi * c23[1];
-            F[t][3] += sc * (c[it][3] + c23[2]) + bi * c23[3];
+            F[t][0] += sc * c[t][0] + ce * own.x + co * o0;
+            F[t][1] += sc * c[t][1] + ce * own.y + co * o1;
+            F[t][2] += sc * c[t][2] + ce * own.z + co * o2;
+            F[t][3] += sc * c[t][3] + ce * own.w + co * o3;
+          }
+        }
+      }
+    } else {
+      // ---- 3. weights: integer dot per group via MFMA (independent slabs interleaved), then
+      //         acc += scale * (dot - sum(off*x)) + bias * sum(x) in f32 ------------------------
+#pragma unroll
+      for (int t = 0; t < TILES; ++t) {
+        f4 c[kSpwMax];
+#pragma unroll
+        for (int it = 0; it < kSpwMax; ++it) c[it] = (f4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          h8 av[kSpwMax];
+#pragma unroll
+          for (int it = 0; it < kSpwMax; ++it) {
+            av[it] = (h8){0, 0, 0, 0, 0, 0, 0, 0};
+            if (it < my && a_active)
+              av[it] = *reinterpret_cast<const h8*>(xs + ((it * 4 + j) * kSlots) * 16 + a_slot_off);
+          }
+#pragma unroll
+          for (int it = 0; it < kSpwMax; ++it) {
+            if (it < my) {
+              const uint32_t wd = j == 0 ? wreg[t][it].x : (j == 1 ? wreg[t][it].y : (j == 2 ? wreg[t][it].z : wreg[t][it].w));
+              c[it] = __builtin_amdgcn_mfma_f32_16x16x32_f16(av[it], unpack_q4_word(wd), c[it], 0, 0, 0);
+            }
+          }
+        }
+        const u4 other = (u4){swap16(sbv[t].x), swap16(sbv[t].y), swap16(sbv[t].z), swap16(sbv[t].w)};
+        const u4 sv = (g & 1) ? other : sbv[t];
+        const u4 bv = (g & 1) ? sbv[t] : other;
+#pragma unroll
+        for (int it = 0; it < kSpwMax; ++it) {
+          if (it < my) {
+            const uint32_t swd = it == 0 ? sv.x : (it == 1 ? sv.y : (it == 2 ? sv.z : sv.w));
+            const uint32_t bwd = it == 0 ? bv.x : (it == 1 ? bv.y : (it == 2 ? bv.z : bv.w));
+            const float sc = __half2float(__ushort_as_half((unsigned short)(par ? swd >> 16 : swd & 0xFFFFu)));
+            const float bi = __half2float(__ushort_as_half((unsigned short)(par ? bwd >> 16 : bwd & 0xFFFFu)));
+            {
+              const float* sp = sums + ((it * 2 + par) * 8 + (g & 1) * 4) * 2;
+              const f4 c01 = *reinterpret_cast<const f4*>(sp);      // (-xoff, xsum) of accumulator rows 4g, 4g+1
+              const f4 c23 = *reinterpret_cast<const f4*>(sp + 4);  // rows 4g+2, 4g+3
+              F[t][0] += sc * (c[it][0] + c01[0]) + bi * c01[1];
+              F[t][1] += sc * (c[it][1] + c01[2]) + bi * c01[3];
+              F[t][2] += sc * (c[it][2] + c23[0]) + bi * c23[1];
+              F[t][3] += sc * (c[it][3] + c23[2]) + bi * c23[3];
+            }
           }
         }
       }
