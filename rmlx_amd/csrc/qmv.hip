@@ -482,11 +482,11 @@ int32_t launch_qmv_q4(const QmvArgs& a, hipStream_t s) {
   int mr = a.mr;
   if (mr == 0) mr = tab ? 8 : (a.M >= 5 ? 8 : (a.M >= 3 ? 4 : (a.M == 2 ? 2 : 1)));
   // With 8 rows every wave takes two tiles (rows r and r+16) for the same staged activations when
-  // that still leaves at least four workgroups per CU: the activation traffic and staging work per
+  // that still gives every CU a workgroup: the activation traffic and staging work per
   // weight byte halve.
   const uint32_t nt = 8 / ks;
   const bool pair = !a.dual && mr == 8 && a.N % (32 * nt) == 0 &&
-                    (uint64_t)(a.N / (32 * nt)) * chunks >= 4ull * (uint32_t)ctx().num_cus;
+                    (uint64_t)(a.N / (32 * nt)) * chunks >= 1ull * (uint32_t)ctx().num_cus;
   dim3 grid(a.N / (16 * nt * (pair ? 2 : 1)), chunks);
   if (pair) {
     launch_t<8, 2, true>(p, tab, grid, s);
