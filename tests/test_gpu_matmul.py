@@ -373,3 +373,13 @@ def test_fused_epilogue_validation(hip):
         ops.qmm_swiglu(xd, qw, DeviceBuffer.from_numpy(np.zeros((4, 64), np.float32)))
     with pytest.raises(ops.KernelError, match="gate_result must be Float16 or Float32"):
         ops.qmm_swiglu(xd, qw, DeviceBuffer.from_numpy(np.zeros((8, 64), np.uint32)))
+
+
+@pytest.mark.parametrize("m,n,k", [(13, 9216, 4096), (16, 9216, 4096), (16, 8192, 1536), (8, 16384, 512), (9, 8192, 2048)])
+def test_qmv_paired_tiles(hip, m, n, k):
+    """Shapes whose 8-row chunks take two 16-row tiles per wave (grid still covers the CUs)."""
+    rng = np.random.default_rng(m + n + k)
+    words, s, b = make_weight(rng, n, k, 4)
+    x = make_x(rng, m, k)
+    ref = model.qmm(x_as_f64(x, "f16"), words, s, b, 64, 4)
+    assert_close(_run(hip, words, s, b, x, 4, kernel=1), ref, f"qmv paired M={m} N={n} K={k}")
