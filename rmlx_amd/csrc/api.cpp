@@ -141,7 +141,12 @@ int32_t run_matmul_plain(const rmlx_qweight* qw, const void* x, int32_t x_dtype,
   const bool can_qmm = can_qmm_lds || can_qmm_rw;
 
   if (kernel == KERNEL_AUTO) {
-    if (can_qmv && M <= kQmvMaxM) kernel = KERNEL_QMV;
+    // The GEMV streams the weights once per chunk of 8 rows (from L2 after the first chunk); the GEMM
+    // has a floor of about 15 us on this chip while its grid is small.  Measured crossover:
+    // chunks * N * K <= 6 * 4096 * 4096 (M <= 48 at 4096 x 4096, M <= 16 at 9216 x 4096).
+    const bool small_m = M <= kQmvMaxM ||
+                         (qw->bits == 4 && (uint64_t)((M + 7) / 8) * N * K <= 6ull * 4096 * 4096);
+    if (can_qmv && small_m) kernel = KERNEL_QMV;
     else if (can_qmm) kernel = KERNEL_QMM;
     else if (can_qmv) kernel = KERNEL_QMV;
     else kernel = KERNEL_GENERIC;
