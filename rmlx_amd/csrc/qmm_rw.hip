@@ -223,8 +223,13 @@ __global__ __launch_bounds__(64 * NW) void qmm_rw_kernel(RwParams p) {
   auto load_sb = [&](uint32_t blk, u4 (&ds)[NF], u4 (&db)[NF]) {
 #pragma unroll
     for (int f = 0; f < NF; ++f) {
+#if defined(QMM_RW_EXP) && (QMM_RW_EXP & 16)
+      ds[f] = (u4){0x20002000u + blk, 0x20002000u, 0x20012001u, 0x20002000u};
+      db[f] = (u4){0xa000a000u + blk, 0xa000a000u, 0xa001a001u, 0xa000a000u};
+#else
       ds[f] = reinterpret_cast<const u4*>(sptr[f])[blk];
       db[f] = reinterpret_cast<const u4*>(bptr[f])[blk];
+#endif
     }
   };
   auto load_w = [&](uint32_t it, u4 (&dst)[NF][WL]) {
@@ -232,7 +237,11 @@ __global__ __launch_bounds__(64 * NW) void qmm_rw_kernel(RwParams p) {
     for (int f = 0; f < NF; ++f)
 #pragma unroll
       for (int h = 0; h < WL; ++h) {
+#if defined(QMM_RW_EXP) && (QMM_RW_EXP & 8)
+        dst[f][h] = (u4){it * 3u + f, (uint32_t)lane, it, (uint32_t)h};
+#else
         dst[f][h] = wptr[f][(uint64_t)it * (4 * WL) + h * 4];
+#endif
       }
   };
   const uint32_t last = S - 1, last_blk = S / kUnroll - 1;
@@ -263,6 +272,9 @@ __global__ __launch_bounds__(64 * NW) void qmm_rw_kernel(RwParams p) {
       const u4 q = wq[u % kUnroll][f][0];
       const uint32_t word = j == 0 ? q.x : (j == 1 ? q.y : (j == 2 ? q.z : q.w));
       scale_pair(u, f, 0, s2, b2);
+#if defined(QMM_RW_EXP) && (QMM_RW_EXP & 1)
+      return __builtin_bit_cast(h8, (u4){word, word ^ h2bits(s2), word, word ^ h2bits(b2)});
+#endif
       return dequant_q4_word(word, s2, b2, dq);
     } else {
       constexpr int hmax = WL - 1;
@@ -310,16 +322,24 @@ __global__ __launch_bounds__(64 * NW) void qmm_rw_kernel(RwParams p) {
         if (f == 0) {
 #pragma unroll
           for (int i = 0; i < MF; ++i)
+#if defined(QMM_RW_EXP) && (QMM_RW_EXP & 2)
+            a_nxt[i] = __builtin_bit_cast(h8, (u4){(uint32_t)lane, it, (uint32_t)(i + j), 0x3c003c00u});
+#else
             a_nxt[i] = __builtin_bit_cast(h8, j < 3 ? a_stage[i * 256 + lds_r[j < 3 ? j + 1 : 0]] : a_stage_next[i * 256 + lds_r[0]]);
+#endif
         }
         // this step's share of the ring traffic: LDS writes of chunk it+2 in the first half, the
         // global loads of chunk it+4 into the same registers in the second half, weights last
 #pragma unroll
         for (int q = 0; q < AL; ++q) {
+#if defined(QMM_RW_EXP) && (QMM_RW_EXP & 4)
+          if (s == q * NS / (2 * AL) && it == 0xFFFFFFFFu) a_stage_write[lds_w[q]] = ra[u % 2][q];
+#else
           if (s == q * NS / (2 * AL)) a_stage_write[lds_w[q]] = to_slot_order(ra[u % 2][q]);
           if (s == NS / 2 + q * NS / (2 * AL)) {
             ra[u % 2][q] = *reinterpret_cast<const u4*>(xsrc[q] + (uint64_t)clampi(it + 4) * kBlockK);
           }
+#endif
         }
         // next weight operand (the one of the first step of the next iteration after the last step)
         if (s + 1 < NS) wv_nxt = weight_operand(u, (s + 1) / NF, (s + 1) % NF);
@@ -336,7 +356,9 @@ __global__ __launch_bounds__(64 * NW) void qmm_rw_kernel(RwParams p) {
         __builtin_amdgcn_sched_barrier(0);
       }
       RW_MARK(p, it, 4);
+#if !(defined(QMM_RW_EXP) && (QMM_RW_EXP & 32))
       __syncthreads();
+#endif
       RW_MARK(p, it, 5);
     }
 #pragma unroll
