@@ -106,8 +106,9 @@ bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) ==
 // ---- the dispatch ladder --------------------------------------------------------------------
 // The reference picks by M: QMV for M=1, batched QMV up to a per-chip limit, split-K Steel for
 // 32 <= M < 128 and NAX above (crates/rmlx-core/src/ops/quantized.rs:7200-7256).  Here: the
-// streaming MFMA GEMV (weights read once for up to 8 rows) up to 16 rows, the LDS-staged MFMA
-// GEMM above, the portable kernel for every shape the fast kernels do not take.
+// streaming MFMA GEMV (weights read once per chunk of 8 rows; 16 rows for 8-bit weights) for small
+// M, the register-weights MFMA GEMM above (the LDS-staged GEMM when K is not a multiple of 512),
+// the portable kernel for every shape the fast kernels do not take.
 enum { KERNEL_AUTO = 0, KERNEL_QMV = 1, KERNEL_QMM = 2, KERNEL_GENERIC = 3, KERNEL_QMM_BF16 = 4, KERNEL_QMM_LDS = 5 };
 constexpr uint32_t kQmvMaxM = 16;
 
