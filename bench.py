@@ -28,7 +28,7 @@ MFMA_F16_PEAK_TF = 2500.0  # dense f16 / bf16 MFMA
 # (FETCH_SIZE and WRITE_SIZE, each scaled by what it reads for the plain copy below); the runs and
 # the scaling are recorded in profiles/bench_all_configs_hbm_traffic_pmc.txt.  Counters cannot be
 # read from inside this process, so the figures are carried here and re-measured with the kernels.
-MEASURED_TRAFFIC_BYTES = {"qmv_q4_m1_4096": 9523736, "qmm_q4_m512_4096": 39826428}
+MEASURED_TRAFFIC_BYTES = {"qmv_q4_m1_4096": 9517591, "qmm_q4_m512_4096": 39721264}
 
 
 def matmul_bytes(m, n, k, bits, gs=64, act_bytes=2):
@@ -234,7 +234,7 @@ def main():
                    "parity_max_err": head.get("max_err"), "parity_tol": head.get("tol")},
         "roofline": {"bound": "hbm", "achieved": head["gbs"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": head["gbs"] / HBM_PEAK_GBS, "traffic": MEASURED_TRAFFIC_BYTES["qmv_q4_m1_4096"],
-                     "kernel": "qmv_q4_kernel<1,1,false,4>", "bytes_per_launch": head["bytes"],
+                     "kernel": "qmv_q4_kernel<1,1,false,4,false>", "bytes_per_launch": head["bytes"],
                      "avg_launch_us": head["us"]},
     }
     if not args.quick and "q4_qmm_m512_4096" in extra:
@@ -243,7 +243,7 @@ def main():
                              "roofline": {"bound": "mfma", "achieved": q["tflops"], "peak": MFMA_F16_PEAK_TF,
                                           "unit": "TFLOP/s", "frac": q["mfma_frac"],
                                           "traffic": MEASURED_TRAFFIC_BYTES["qmm_q4_m512_4096"],
-                                          "kernel": "qmm_rw_kernel<4,2,4,4>", "avg_launch_us": q["us"]}}
+                                          "kernel": "qmm_rw_kernel<4,1,4,8,false>", "avg_launch_us": q["us"]}}
     if not args.no_cpu:
         line["cpu_baseline"] = cpu_baseline(np.random.default_rng(1001), 3.0 if args.quick else 10.0)
     line["extra"] = extra
