@@ -106,11 +106,15 @@ bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) ==
 // ---- the dispatch ladder --------------------------------------------------------------------
 // The reference picks by M: QMV for M=1, batched QMV up to a per-chip limit, split-K Steel for
 // 32 <= M < 128 and NAX above (crates/rmlx-core/src/ops/quantized.rs:7200-7256).  Here: the
-// streaming MFMA GEMV (weights read once per chunk of 8 rows; 16 rows for 8-bit weights) for small
-// M, the register-weights MFMA GEMM above (the LDS-staged GEMM when K is not a multiple of 512),
-// the portable kernel for every shape the fast kernels do not take.
-enum { KERNEL_AUTO = 0, KERNEL_QMV = 1, KERNEL_QMM = 2, KERNEL_GENERIC = 3, KERNEL_QMM_BF16 = 4, KERNEL_QMM_LDS = 5 };
+// single-row GEMV for M = 1 (and for a few rows when the group size is not 64), the streaming MFMA
+// GEMV (weights read once per chunk of 8 rows; 16 rows for 8-bit weights) for small M, the
+// register-weights MFMA GEMM above (the LDS-staged GEMM when K is not a multiple of 512), the
+// portable kernel for every shape the fast kernels do not take.
+enum { KERNEL_AUTO = 0, KERNEL_QMV = 1, KERNEL_QMM = 2, KERNEL_GENERIC = 3, KERNEL_QMM_BF16 = 4, KERNEL_QMM_LDS = 5,
+       KERNEL_QMV_ROWS = 6 };
 constexpr uint32_t kQmvMaxM = 16;
+constexpr uint32_t kM1MaxRows = 1;        // group size 64: rows taken by the single-row kernel
+constexpr uint32_t kM1MaxRowsOther = 16;  // group sizes 32 / 128: the alternative is the portable kernel
 
 struct Epilogue { int kind = EPI_NONE; const void* ptr = nullptr; int32_t dtype = RMLX_DTYPE_F16; };
 
@@ -137,6 +141,8 @@ int32_t run_matmul_plain(const rmlx_qweight* qw, const void* x, int32_t x_dtype,
   const bool ptr_ok = aligned16(qw->w) && aligned16(qw->s) && aligned16(qw->b) && aligned16(x);
   const bool can_qmv = ptr_ok && ((qw->bits == 4 && qmv_q4_supported(N, K, qw->group_size)) ||
                                   (qw->bits == 8 && qmv_q8_supported(N, K, qw->group_size)));
+  const bool can_m1 = ptr_ok && qmv_m1_supported(N, K, qw->group_size, qw->bits) &&
+                      M <= (qw->group_size == 64 ? kM1MaxRows : kM1MaxRowsOther);
   const bool can_qmm_lds = ptr_ok && qmm_supported(N, K, qw->group_size, qw->bits);
   const bool can_qmm_rw = ptr_ok && qmm_rw_supported(N, K, qw->group_size, qw->bits);
   const bool can_qmm = can_qmm_lds || can_qmm_rw;
@@ -147,11 +153,11 @@ int32_t run_matmul_plain(const rmlx_qweight* qw, const void* x, int32_t x_dtype,
     // chunks * N * K <= 6 * 4096 * 4096 (M <= 48 at 4096 x 4096, M <= 16 at 9216 x 4096).
     const bool small_m = M <= kQmvMaxM ||
                          (qw->bits == 4 && (uint64_t)((M + 7) / 8) * N * K <= 6ull * 4096 * 4096);
-    if (can_qmv && small_m) kernel = KERNEL_QMV;
+    if ((can_qmv && small_m) || can_m1) kernel = KERNEL_QMV;
     else if (can_qmm) kernel = KERNEL_QMM;
     else if (can_qmv) kernel = KERNEL_QMV;
     else kernel = KERNEL_GENERIC;
-  } else if (kernel == KERNEL_QMV && !can_qmv) {
+  } else if ((kernel == KERNEL_QMV && !can_qmv && !can_m1) || (kernel == KERNEL_QMV_ROWS && !can_qmv)) {
     return fail(RMLX_INVALID_SHAPE,
                 "qmv kernel requires bits in {4,8}, group_size=64, N %% 16 == 0, K %% 512 == 0 (4-bit) or "
                 "K %% 2048 == 0 (8-bit) and 16-byte aligned buffers (N=%u K=%u bits=%u group_size=%u)",
@@ -167,7 +173,7 @@ int32_t run_matmul_plain(const rmlx_qweight* qw, const void* x, int32_t x_dtype,
   } else if (kernel == KERNEL_QMM_BF16 && !(can_qmm_lds && qw->bits == 8 && x_dtype == RMLX_DTYPE_BF16)) {
     return fail(RMLX_INVALID_SHAPE, "the bf16 MFMA GEMM takes Bfloat16 activations and 8-bit weights (got %s, bits=%u)",
                 dtype_name(x_dtype), qw->bits);
-  } else if (kernel < 0 || kernel > KERNEL_QMM_LDS) {
+  } else if (kernel < 0 || kernel > KERNEL_QMV_ROWS) {
     return fail(RMLX_NOT_FOUND, "unknown kernel selector %d", kernel);
   }
 
@@ -208,6 +214,10 @@ int32_t run_matmul_plain(const rmlx_qweight* qw, const void* x, int32_t x_dtype,
     xk = cast.ptr;
   }
 
+  if (kernel == KERNEL_QMV && can_m1)
+    return launch_qmv_m1(qw->w, qw->s, qw->b, static_cast<const __half*>(xk), out, M, N, K, qw->group_size, qw->bits,
+                         stream);
+  if (kernel == KERNEL_QMV_ROWS) kernel = KERNEL_QMV;
   if (kernel == KERNEL_QMV && qw->bits == 8)
     return launch_qmv_q8(qw->w, qw->s, qw->b, static_cast<const __half*>(xk), out, M, N, K, stream);
   if (kernel == KERNEL_QMV) {

@@ -130,6 +130,11 @@ bool qmv_q4_supported(uint32_t N, uint32_t K, uint32_t group_size);
 bool qmv_q8_supported(uint32_t N, uint32_t K, uint32_t group_size);
 int32_t launch_qmv_q8(const uint32_t* w, const __half* s, const __half* b, const __half* x, __half* out, uint32_t M,
                       uint32_t N, uint32_t K, hipStream_t stream);
+// Single-row GEMV (qmv_m1.hip): 4- or 8-bit weights, group size 32 / 64 / 128, f16 activations; M rows are
+// M independent passes over the weights (grid.y).
+bool qmv_m1_supported(uint32_t N, uint32_t K, uint32_t group_size, uint32_t bits);
+int32_t launch_qmv_m1(const uint32_t* w, const __half* s, const __half* b, const __half* x, __half* out, uint32_t M,
+                      uint32_t N, uint32_t K, uint32_t group_size, uint32_t bits, hipStream_t stream);
 // chunk table for gather_qmm: batch b owns rows [b*mpb, (b+1)*mpb) and expert indices[b]
 int32_t launch_build_gather_chunks(const uint32_t* indices, uint32_t batch, uint32_t mpb, uint32_t n_experts,
                                    uint32_t* chunk_tab, hipStream_t s);

@@ -1,0 +1,248 @@
+// Single-row quantized GEMV for gfx950 (decode: one activation row per pass over the weights).
+//
+// Replaces the reference's affine_qmv_fast_q4 / affine_qmv_fast_q8 at M = 1
+// (crates/rmlx-core/src/ops/quantized.rs:394-600, 620-695, dispatched from :1309-1411).
+//
+// With one activation row the matrix unit has nothing to share between rows, so this kernel is
+// organised around the memory system instead:
+//   * A wave-wide 16-byte load covers 1 KB of ONE weight row (2048 4-bit or 1024 8-bit values):
+//     fully contiguous, where the MFMA operand layout of the multi-row kernel makes every lane
+//     quad touch four different rows.  A wave owns two adjacent weight rows over the whole K, so a
+//     workgroup (8 waves, 16 rows) streams one contiguous block, and every load of a pass is in
+//     flight before the first one is consumed.
+//   * Lane l of a wave always works on the same k positions of a chunk, so its activations live
+//     in registers for all rows: the workgroup stages x once into LDS (already permuted to the
+//     order the nibble unpacking produces, together with the per-lane sums the offset removal
+//     needs) and a wave reads its 16 registers per chunk from there.
+//   * Dot products run on v_dot2_f32_f16 with exact magic-number int -> f16 conversion
+//     ((w & 0x000F000F) | 0x64006400 = (1024 + q0, 1024 + q4), ...); per lane and row
+//     acc = sum(x * (off + q)), and  scale * (acc - sum(off * x)) + bias * sum(x)  is added in f32.
+//     A quantisation group is 1, 2, 4 or 8 whole lanes (group sizes 32 / 64 / 128), so no
+//     cross-lane work is needed before the final wave-wide sum, and a wave writes its two
+//     outputs itself: no cross-wave reduction, one barrier (after staging x).
+#include "common.hpp"
+
+namespace rmlx {
+namespace {
+
+typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+typedef _Float16 h8 __attribute__((ext_vector_type(8)));
+typedef uint32_t u4 __attribute__((ext_vector_type(4)));
+
+constexpr int kThreads = 512;
+constexpr int kRowsPerWg = 16;   // two per wave
+constexpr uint32_t kMaxK = 16384;  // x image + sums must fit the default dynamic LDS limit; 4 x loads per thread
+
+struct M1Params {
+  const uint32_t* w; const __half* s; const __half* b;
+  const __half* x;
+  __half* out;
+  uint32_t N, K;
+};
+
+__device__ __forceinline__ h2 as_h2(uint32_t v) { return __builtin_bit_cast(h2, v); }
+
+template <int CTRL>
+__device__ __forceinline__ float dpp_add(float v) {
+  return v + __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, true));
+}
+
+// sum over the 64 lanes, same value returned in every lane
+__device__ __forceinline__ float wave_sum(float v) {
+  v = dpp_add<0xB1>(v);   // quad_perm [1,0,3,2]: lane ^ 1
+  v = dpp_add<0x4E>(v);   // quad_perm [2,3,0,1]: lane ^ 2
+  v = dpp_add<0x141>(v);  // row_half_mirror: the other quad of each 8
+  v = dpp_add<0x140>(v);  // row_mirror: the other 8 of each 16
+  v += __builtin_bit_cast(float, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, v), 0x401F));  // lane ^ 16
+  const int bits = __builtin_bit_cast(int, v);
+  return __builtin_bit_cast(float, __builtin_amdgcn_readlane(bits, 0)) +
+         __builtin_bit_cast(float, __builtin_amdgcn_readlane(bits, 32));
+}
+
+// x halves (k0..k7) -> pair order (k0,k4),(k1,k5),(k2,k6),(k3,k7) of the nibble unpacking
+__device__ __forceinline__ u4 to_pair_order(u4 d) {
+  u4 o;
+  o.x = __builtin_amdgcn_perm(d.z, d.x, 0x05040100u);
+  o.y = __builtin_amdgcn_perm(d.z, d.x, 0x07060302u);
+  o.z = __builtin_amdgcn_perm(d.w, d.y, 0x05040100u);
+  o.w = __builtin_amdgcn_perm(d.w, d.y, 0x07060302u);
+  return o;
+}
+
+template <int BITS, int GS>
+__global__ __launch_bounds__(kThreads) void qmv_m1_kernel(M1Params p) {
+  constexpr int kChunkK = 8192 / BITS;         // k values of one wave-wide 16-byte load: 2048 / 1024
+  constexpr int kLaneK = kChunkK / 64;         // values per lane and chunk: 32 / 16
+  constexpr int kXU = kLaneK / 8;              // 16-byte activation units per lane and chunk: 4 / 2
+  constexpr int kLanesPerGroup = GS / kLaneK;  // whole lanes per quantisation group
+  constexpr int kGroupsPerChunk = kChunkK / GS;
+  static_assert(kLanesPerGroup >= 1, "a lane must not straddle quantisation groups");
+
+  extern __shared__ __attribute__((aligned(16))) char lds[];
+  const uint32_t K = p.K, KH = K / kChunkK, G = K / GS, nunits = K / 8;
+  u4* xl = reinterpret_cast<u4*>(lds);                  // [chunk][unit j][lane]
+  float2* cs = reinterpret_cast<float2*>(lds + 2 * K);  // [chunk][lane]: (sum(off * x), sum(x)) of the lane's values
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const uint32_t row0 = blockIdx.x * kRowsPerWg + wave * 2;
+  const u4* xg = reinterpret_cast<const u4*>(p.x + (uint64_t)blockIdx.y * K);
+
+  // ---- 1. loads, small ones first (the memory counter retires in order): activations ... ------
+  u4 xv[4];
+  {
+    const uint32_t u0 = (uint32_t)tid < nunits ? (uint32_t)tid : nunits - 1;
+    xv[0] = xg[u0];
+#pragma unroll
+    for (int i = 1; i < 4; ++i) {
+      xv[i] = (u4){0u, 0u, 0u, 0u};
+      if (nunits > (uint32_t)i * kThreads) {  // uniform; the last round may be partial (clamped, stored under a guard)
+        const uint32_t u = tid + i * kThreads;
+        xv[i] = xg[u < nunits ? u : nunits - 1];
+      }
+    }
+  }
+  // ---- ... then the first two chunks of both rows with their scales and biases ----------------
+  struct Batch { u4 w[2][2]; uint32_t s[2][2], b[2][2]; };  // [chunk of the batch][row]
+  const u4* wrow[2];
+  const unsigned short* srow[2];
+  const unsigned short* brow[2];
+#pragma unroll
+  for (int r = 0; r < 2; ++r) {
+    wrow[r] = reinterpret_cast<const u4*>(p.w + (uint64_t)(row0 + r) * (K * BITS / 32)) + lane;
+    srow[r] = reinterpret_cast<const unsigned short*>(p.s) + (uint64_t)(row0 + r) * G + lane / kLanesPerGroup;
+    brow[r] = reinterpret_cast<const unsigned short*>(p.b) + (uint64_t)(row0 + r) * G + lane / kLanesPerGroup;
+  }
+  auto load_batch = [&](uint32_t c0, Batch& t) {
+#pragma unroll
+    for (int cc = 0; cc < 2; ++cc) {
+      const uint32_t c = c0 + cc < KH ? c0 + cc : KH - 1;  // an odd chunk count re-reads the last chunk (unused)
+#pragma unroll
+      for (int r = 0; r < 2; ++r) {
+        t.s[cc][r] = srow[r][c * kGroupsPerChunk];
+        t.b[cc][r] = brow[r][c * kGroupsPerChunk];
+      }
+#pragma unroll
+      for (int r = 0; r < 2; ++r) t.w[cc][r] = wrow[r][(uint64_t)c * 64];
+    }
+  };
+  Batch ba, bb;
+  load_batch(0, ba);
+
+  // ---- 2. stage x: unit u = 8 consecutive k = (chunk, lane, j); image in the order a wave reads it ----
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const uint32_t u = tid + i * kThreads;
+    if (u < nunits) {
+      const uint32_t c = u / (64 * kXU), rem = u % (64 * kXU), l = rem / kXU, j = rem % kXU;
+      xl[(c * kXU + j) * 64 + l] = BITS == 4 ? to_pair_order(xv[i]) : xv[i];
+      const h8 hv = __builtin_bit_cast(h8, xv[i]);
+      float xs8 = 0.f, xo8 = 0.f;
+#pragma unroll
+      for (int e = 0; e < 8; e += 2) {
+        xs8 += (float)hv[e] + (float)hv[e + 1];
+        xo8 += 1024.0f * (float)hv[e] + (BITS == 4 ? 64.0f : 1024.0f) * (float)hv[e + 1];
+      }
+      // the kXU units of a lane sit in adjacent threads of one quad (unit counts are multiples of 4)
+      xs8 = dpp_add<0xB1>(xs8);
+      xo8 = dpp_add<0xB1>(xo8);
+      if (kXU == 4) {
+        xs8 = dpp_add<0x4E>(xs8);
+        xo8 = dpp_add<0x4E>(xo8);
+      }
+      if (j == 0) cs[c * 64 + l] = make_float2(xo8, xs8);
+    }
+  }
+  __syncthreads();
+
+  // ---- 3. chunk by chunk: registers of x from LDS, then both rows --------------------------------
+  float racc[2] = {0.f, 0.f};
+  uint32_t m0 = 0x000F000Fu, m1 = 0x00F000F0u, k0 = 0x64006400u, k1 = 0x54005400u;
+  asm volatile("" : "+s"(m0), "+s"(m1), "+v"(k0), "+v"(k1));  // constants in registers: and+or is one instruction
+  auto process = [&](uint32_t c0, const Batch& t) {
+#pragma unroll
+    for (int cc = 0; cc < 2; ++cc) {
+      const uint32_t c = c0 + cc;
+      if (c < KH) {
+        uint32_t xr[kXU][4];
+#pragma unroll
+        for (int j = 0; j < kXU; ++j) {
+          const u4 v = xl[(c * kXU + j) * 64 + lane];
+          xr[j][0] = v.x; xr[j][1] = v.y; xr[j][2] = v.z; xr[j][3] = v.w;
+        }
+        const float2 k = cs[c * 64 + lane];
+#pragma unroll
+        for (int r = 0; r < 2; ++r) {
+          const u4 wv = t.w[cc][r];
+          const uint32_t wd[4] = {wv.x, wv.y, wv.z, wv.w};
+          float acc0 = 0.f, acc1 = 0.f;
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            if (BITS == 4) {
+              const uint32_t hi = wd[j] >> 8;
+              acc0 = __builtin_amdgcn_fdot2(as_h2((wd[j] & m0) | k0), as_h2(xr[j][0]), acc0, false);
+              acc1 = __builtin_amdgcn_fdot2(as_h2((wd[j] & m1) | k1), as_h2(xr[j][1]), acc1, false);
+              acc0 = __builtin_amdgcn_fdot2(as_h2((hi & m0) | k0), as_h2(xr[j][2]), acc0, false);
+              acc1 = __builtin_amdgcn_fdot2(as_h2((hi & m1) | k1), as_h2(xr[j][3]), acc1, false);
+            } else {  // bytes (q0,q1,q2,q3) -> (1024 + q0, 1024 + q1), (1024 + q2, 1024 + q3): natural order
+              const int u = j >> 1, e = (j & 1) * 2;
+              acc0 = __builtin_amdgcn_fdot2(as_h2(__builtin_amdgcn_perm(0x64646464u, wd[j], 0x04010400u)),
+                                            as_h2(xr[u % kXU][e]), acc0, false);
+              acc1 = __builtin_amdgcn_fdot2(as_h2(__builtin_amdgcn_perm(0x64646464u, wd[j], 0x04030402u)),
+                                            as_h2(xr[u % kXU][e + 1]), acc1, false);
+            }
+          }
+          const float sc = __half2float(__ushort_as_half((unsigned short)t.s[cc][r]));
+          const float bi = __half2float(__ushort_as_half((unsigned short)t.b[cc][r]));
+          racc[r] += sc * ((acc0 + acc1) - k.x) + bi * k.y;
+        }
+      }
+    }
+  };
+  for (uint32_t c0 = 0; c0 < KH; c0 += 4) {
+    const bool more1 = c0 + 2 < KH, more2 = c0 + 4 < KH;
+    if (more1) load_batch(c0 + 2, bb);
+    process(c0, ba);
+    if (more1) {
+      if (more2) load_batch(c0 + 4, ba);
+      process(c0 + 2, bb);
+    }
+  }
+
+  // ---- 4. wave-wide sums, two outputs per wave ------------------------------------------------------
+  const float t0 = wave_sum(racc[0]), t1 = wave_sum(racc[1]);
+  if (lane < 2) p.out[(uint64_t)blockIdx.y * p.N + row0 + lane] = __float2half(lane ? t1 : t0);
+}
+
+template <int BITS>
+void launch_bits(const M1Params& p, uint32_t M, uint32_t group_size, hipStream_t s) {
+  const dim3 grid(p.N / kRowsPerWg, M), block(kThreads);
+  const size_t lds = 2 * (size_t)p.K + (size_t)p.K / (128 / BITS) * sizeof(float2);
+  switch (group_size) {
+    case 32: hipLaunchKernelGGL((qmv_m1_kernel<BITS, 32>), grid, block, lds, s, p); break;
+    case 64: hipLaunchKernelGGL((qmv_m1_kernel<BITS, 64>), grid, block, lds, s, p); break;
+    default: hipLaunchKernelGGL((qmv_m1_kernel<BITS, 128>), grid, block, lds, s, p); break;
+  }
+}
+
+}  // namespace
+
+bool qmv_m1_supported(uint32_t N, uint32_t K, uint32_t group_size, uint32_t bits) {
+  if (bits != 4 && bits != 8) return false;
+  if (group_size != 32 && group_size != 64 && group_size != 128) return false;
+  return N > 0 && K > 0 && N % kRowsPerWg == 0 && K % (8192 / bits) == 0 && K <= kMaxK;
+}
+
+int32_t launch_qmv_m1(const uint32_t* w, const __half* s, const __half* b, const __half* x, __half* out, uint32_t M,
+                      uint32_t N, uint32_t K, uint32_t group_size, uint32_t bits, hipStream_t stream) {
+  if (!qmv_m1_supported(N, K, group_size, bits))
+    return fail(RMLX_INVALID_SHAPE, "qmv_m1: unsupported shape N=%u K=%u bits=%u group_size=%u", N, K, bits, group_size);
+  if (M == 0) return RMLX_OK;
+  if (M > 65535) return fail(RMLX_INVALID_SHAPE, "qmv_m1: at most 65535 rows per launch (M=%u)", M);
+  M1Params p{w, s, b, x, out, N, K};
+  if (bits == 4) launch_bits<4>(p, M, group_size, stream);
+  else launch_bits<8>(p, M, group_size, stream);
+  RMLX_HIP_CHECK(hipGetLastError());
+  return RMLX_OK;
+}
+
+}  // namespace rmlx

@@ -383,3 +383,44 @@ def test_qmv_paired_tiles(hip, m, n, k):
     x = make_x(rng, m, k)
     ref = model.qmm(x_as_f64(x, "f16"), words, s, b, 64, 4)
     assert_close(_run(hip, words, s, b, x, 4, kernel=1), ref, f"qmv paired M={m} N={n} K={k}")
+
+
+# ---- single-row GEMV (decode; affine_qmv_fast_q4 / _q8, quantized.rs:394-695) ---------------------------
+
+@pytest.mark.parametrize("bits", [4, 8])
+@pytest.mark.parametrize("gs", [32, 64, 128])
+@pytest.mark.parametrize("n,k", [(16, 2048), (64, 4096), (48, 6144), (32, 8192), (16, 16384)])
+def test_single_row_gemv(hip, bits, gs, n, k):
+    """M = 1 at every group size the weight type admits; at group sizes 32 / 128 the kernel also takes a
+    few rows (one pass over the weights per row)."""
+    from rmlx_amd import runtime as rt
+    rng = np.random.default_rng(bits * 1000 + gs + n + k)
+    words, s, b = make_weight(rng, n, k, bits, gs)
+    for m in ((1,) if gs == 64 else (1, 3, 16)):
+        x = make_x(rng, m, k)
+        ref = model.qmm(x_as_f64(x, "f16"), words, s, b, gs, bits)
+        assert_close(_run(hip, words, s, b, x, bits, gs=gs), ref, f"auto bits={bits} gs={gs} N={n} K={k} M={m}")
+        assert_close(_run(hip, words, s, b, x, bits, gs=gs, kernel=rt.KERNEL_QMV), ref,
+                     f"qmv bits={bits} gs={gs} N={n} K={k} M={m}")
+
+
+@pytest.mark.parametrize("bits", [4, 8])
+def test_single_row_gemv_positions_and_multi_row_kernel_agree(hip, bits):
+    """One-hot activations pick out single weights exactly (every k position of a lane, chunk borders), and
+    the multi-row kernel forced onto one row gives the same numbers within the tolerance."""
+    from rmlx_amd import runtime as rt
+    n, k = 32, 4096
+    rng = np.random.default_rng(40 + bits)
+    words, s, b = make_weight(rng, n, k, bits)
+    s1, b0 = np.ones_like(s), np.zeros_like(b)
+    q = model.unpack_u32(words, bits).astype(np.float64)
+    ks = np.array(list(range(40)) + [63, 64, 127, 128, 1023, 1024, 2047, 2048, 2049, 2079, 2080, 4064, 4095])
+    for kk in ks:  # one row per call: the single-row kernel
+        x = np.zeros((1, k), np.float16)
+        x[0, kk] = 1.0
+        out = _run(hip, words, s1, b0, x, bits)
+        assert np.array_equal(out[0].astype(np.float64), q[:, kk]), f"k={kk}"
+    x = make_x(rng, 1, k)
+    ref = model.qmm(x_as_f64(x, "f16"), words, s, b, 64, bits)
+    assert_close(_run(hip, words, s, b, x, bits, kernel=rt.KERNEL_QMV_ROWS), ref, "multi-row kernel at M=1")
+    assert_close(_run(hip, words, s, b, x, bits, kernel=rt.KERNEL_QMV), ref, "single-row kernel")
