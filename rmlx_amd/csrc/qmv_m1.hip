@@ -7,9 +7,11 @@
 // organised around the memory system instead:
 //   * A wave-wide 16-byte load covers 1 KB of ONE weight row (2048 4-bit or 1024 8-bit values):
 //     fully contiguous, where the MFMA operand layout of the multi-row kernel makes every lane
-//     quad touch four different rows.  A wave owns two adjacent weight rows over the whole K, so a
-//     workgroup (8 waves, 16 rows) streams one contiguous block, and every load of a pass is in
-//     flight before the first one is consumed.
+//     quad touch four different rows.  A wave owns one or two adjacent weight rows over the whole K, so a
+//     workgroup (8 waves) streams one contiguous block, and every load of a pass is in
+//     flight before the first one is consumed.  (One row per wave when K < 12288: finer-grained
+//     waves overlap arrival and arithmetic better; measured.)  With a single activation row the
+//     weights are loaded non-temporally: nothing reads them a second time.
 //   * Lane l of a wave always works on the same k positions of a chunk, so its activations live
 //     in registers for all rows: the workgroup stages x once into LDS (already permuted to the
 //     order the nibble unpacking produces, together with the per-lane sums the offset removal
@@ -30,7 +32,7 @@ typedef _Float16 h8 __attribute__((ext_vector_type(8)));
 typedef uint32_t u4 __attribute__((ext_vector_type(4)));
 
 constexpr int kThreads = 512;
-constexpr int kRowsPerWg = 16;   // two per wave
+constexpr int kWaves = 8;
 constexpr uint32_t kMaxK = 16384;  // x image + sums must fit the default dynamic LDS limit; 4 x loads per thread
 
 struct M1Params {
@@ -69,7 +71,8 @@ __device__ __forceinline__ u4 to_pair_order(u4 d) {
   return o;
 }
 
-template <int BITS, int GS>
+// R = weight rows per wave (1 or 2); NT = non-temporal weight loads (single activation row).
+template <int BITS, int GS, int R, bool NT>
 __global__ __launch_bounds__(kThreads) void qmv_m1_kernel(M1Params p) {
   constexpr int kChunkK = 8192 / BITS;         // k values of one wave-wide 16-byte load: 2048 / 1024
   constexpr int kLaneK = kChunkK / 64;         // values per lane and chunk: 32 / 16
@@ -84,7 +87,7 @@ __global__ __launch_bounds__(kThreads) void qmv_m1_kernel(M1Params p) {
   float2* cs = reinterpret_cast<float2*>(lds + 2 * K);  // [chunk][lane]: (sum(off * x), sum(x)) of the lane's values
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const uint32_t row0 = blockIdx.x * kRowsPerWg + wave * 2;
+  const uint32_t row0 = blockIdx.x * (kWaves * R) + wave * R;
   const u4* xg = reinterpret_cast<const u4*>(p.x + (uint64_t)blockIdx.y * K);
 
   // ---- 1. loads, small ones first (the memory counter retires in order): activations ... ------
@@ -101,13 +104,13 @@ __global__ __launch_bounds__(kThreads) void qmv_m1_kernel(M1Params p) {
       }
     }
   }
-  // ---- ... then the first two chunks of both rows with their scales and biases ----------------
-  struct Batch { u4 w[2][2]; uint32_t s[2][2], b[2][2]; };  // [chunk of the batch][row]
-  const u4* wrow[2];
-  const unsigned short* srow[2];
-  const unsigned short* brow[2];
+  // ---- ... then the first two chunks of the wave's rows with their scales and biases ----------------
+  struct Batch { u4 w[2][R]; uint32_t s[2][R], b[2][R]; };  // [chunk of the batch][row]
+  const u4* wrow[R];
+  const unsigned short* srow[R];
+  const unsigned short* brow[R];
 #pragma unroll
-  for (int r = 0; r < 2; ++r) {
+  for (int r = 0; r < R; ++r) {
     wrow[r] = reinterpret_cast<const u4*>(p.w + (uint64_t)(row0 + r) * (K * BITS / 32)) + lane;
     srow[r] = reinterpret_cast<const unsigned short*>(p.s) + (uint64_t)(row0 + r) * G + lane / kLanesPerGroup;
     brow[r] = reinterpret_cast<const unsigned short*>(p.b) + (uint64_t)(row0 + r) * G + lane / kLanesPerGroup;
@@ -117,12 +120,13 @@ __global__ __launch_bounds__(kThreads) void qmv_m1_kernel(M1Params p) {
     for (int cc = 0; cc < 2; ++cc) {
       const uint32_t c = c0 + cc < KH ? c0 + cc : KH - 1;  // an odd chunk count re-reads the last chunk (unused)
 #pragma unroll
-      for (int r = 0; r < 2; ++r) {
+      for (int r = 0; r < R; ++r) {
         t.s[cc][r] = srow[r][c * kGroupsPerChunk];
         t.b[cc][r] = brow[r][c * kGroupsPerChunk];
       }
 #pragma unroll
-      for (int r = 0; r < 2; ++r) t.w[cc][r] = wrow[r][(uint64_t)c * 64];
+      for (int r = 0; r < R; ++r)
+        t.w[cc][r] = NT ? __builtin_nontemporal_load(wrow[r] + (uint64_t)c * 64) : wrow[r][(uint64_t)c * 64];
     }
   };
   Batch ba, bb;
@@ -154,8 +158,10 @@ __global__ __launch_bounds__(kThreads) void qmv_m1_kernel(M1Params p) {
   }
   __syncthreads();
 
-  // ---- 3. chunk by chunk: registers of x from LDS, then both rows --------------------------------
-  float racc[2] = {0.f, 0.f};
+  // ---- 3. chunk by chunk: registers of x from LDS, then the wave's rows --------------------------------
+  float racc[R];
+#pragma unroll
+  for (int r = 0; r < R; ++r) racc[r] = 0.f;
   uint32_t m0 = 0x000F000Fu, m1 = 0x00F000F0u, k0 = 0x64006400u, k1 = 0x54005400u;
   asm volatile("" : "+s"(m0), "+s"(m1), "+v"(k0), "+v"(k1));  // constants in registers: and+or is one instruction
   auto process = [&](uint32_t c0, const Batch& t) {
@@ -171,7 +177,7 @@ __global__ __launch_bounds__(kThreads) void qmv_m1_kernel(M1Params p) {
         }
         const float2 k = cs[c * 64 + lane];
 #pragma unroll
-        for (int r = 0; r < 2; ++r) {
+        for (int r = 0; r < R; ++r) {
           const u4 wv = t.w[cc][r];
           const uint32_t wd[4] = {wv.x, wv.y, wv.z, wv.w};
           float acc0 = 0.f, acc1 = 0.f;
@@ -208,19 +214,36 @@ __global__ __launch_bounds__(kThreads) void qmv_m1_kernel(M1Params p) {
     }
   }
 
-  // ---- 4. wave-wide sums, two outputs per wave ------------------------------------------------------
-  const float t0 = wave_sum(racc[0]), t1 = wave_sum(racc[1]);
-  if (lane < 2) p.out[(uint64_t)blockIdx.y * p.N + row0 + lane] = __float2half(lane ? t1 : t0);
+  // ---- 4. wave-wide sums; lane r writes the output of row r ----------------------------------------
+  float mine = 0.f;
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    const float t = wave_sum(racc[r]);
+    mine = lane == r ? t : mine;
+  }
+  if (lane < R) p.out[(uint64_t)blockIdx.y * p.N + row0 + lane] = __float2half(mine);
+}
+
+template <int BITS, int R, bool NT>
+void launch_r(const M1Params& p, uint32_t M, uint32_t group_size, hipStream_t s) {
+  const dim3 grid(p.N / (kWaves * R), M), block(kThreads);
+  const size_t lds = 2 * (size_t)p.K + (size_t)p.K / (128 / BITS) * sizeof(float2);
+  switch (group_size) {
+    case 32: hipLaunchKernelGGL((qmv_m1_kernel<BITS, 32, R, NT>), grid, block, lds, s, p); break;
+    case 64: hipLaunchKernelGGL((qmv_m1_kernel<BITS, 64, R, NT>), grid, block, lds, s, p); break;
+    default: hipLaunchKernelGGL((qmv_m1_kernel<BITS, 128, R, NT>), grid, block, lds, s, p); break;
+  }
 }
 
 template <int BITS>
 void launch_bits(const M1Params& p, uint32_t M, uint32_t group_size, hipStream_t s) {
-  const dim3 grid(p.N / kRowsPerWg, M), block(kThreads);
-  const size_t lds = 2 * (size_t)p.K + (size_t)p.K / (128 / BITS) * sizeof(float2);
-  switch (group_size) {
-    case 32: hipLaunchKernelGGL((qmv_m1_kernel<BITS, 32>), grid, block, lds, s, p); break;
-    case 64: hipLaunchKernelGGL((qmv_m1_kernel<BITS, 64>), grid, block, lds, s, p); break;
-    default: hipLaunchKernelGGL((qmv_m1_kernel<BITS, 128>), grid, block, lds, s, p); break;
+  // two rows per wave for long rows (more bytes in flight per wave), else one; several activation
+  // rows re-read the weights from L2, so only a single row streams them non-temporally
+  const bool two = p.K >= 12288 && p.N % (kWaves * 2) == 0;
+  if (M == 1) {
+    if (two) launch_r<BITS, 2, true>(p, M, group_size, s); else launch_r<BITS, 1, true>(p, M, group_size, s);
+  } else {
+    if (two) launch_r<BITS, 2, false>(p, M, group_size, s); else launch_r<BITS, 1, false>(p, M, group_size, s);
   }
 }
 
@@ -229,7 +252,7 @@ void launch_bits(const M1Params& p, uint32_t M, uint32_t group_size, hipStream_t
 bool qmv_m1_supported(uint32_t N, uint32_t K, uint32_t group_size, uint32_t bits) {
   if (bits != 4 && bits != 8) return false;
   if (group_size != 32 && group_size != 64 && group_size != 128) return false;
-  return N > 0 && K > 0 && N % kRowsPerWg == 0 && K % (8192 / bits) == 0 && K <= kMaxK;
+  return N > 0 && K > 0 && N % kWaves == 0 && K % (8192 / bits) == 0 && K <= kMaxK;
 }
 
 int32_t launch_qmv_m1(const uint32_t* w, const __half* s, const __half* b, const __half* x, __half* out, uint32_t M,

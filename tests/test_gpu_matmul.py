@@ -389,7 +389,7 @@ def test_qmv_paired_tiles(hip, m, n, k):
 
 @pytest.mark.parametrize("bits", [4, 8])
 @pytest.mark.parametrize("gs", [32, 64, 128])
-@pytest.mark.parametrize("n,k", [(16, 2048), (64, 4096), (48, 6144), (32, 8192), (16, 16384)])
+@pytest.mark.parametrize("n,k", [(16, 2048), (24, 4096), (64, 4096), (48, 6144), (32, 8192), (40, 12288), (16, 16384)])
 def test_single_row_gemv(hip, bits, gs, n, k):
     """M = 1 at every group size the weight type admits; at group sizes 32 / 128 the kernel also takes a
     few rows (one pass over the weights per row)."""
