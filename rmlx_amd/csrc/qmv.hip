@@ -52,7 +52,7 @@ struct KParams {
   void* out;
   uint32_t K, ld_out, M, out_f32;
   uint32_t ks;  // k-parts per pass (1, 2, 4 or 8); tiles per workgroup = 8 / ks
-  uint32_t pad_;
+  uint32_t tpw;  // consecutive tiles per workgroup (> 1 only when one pass covers K: the staged activations are reused)
   const uint32_t* w1;
   const __half* s1;
   const __half* b1;
@@ -112,15 +112,16 @@ struct __attribute__((packed, aligned(4))) U4Unaligned { uint32_t v[4]; };
 // TAB = rows come from a device chunk table (gather_qmm, MoE); SPW = slabs per wave and pass when
 // every wave of every pass owns the same number (3 or 4: no guards, fewer registers, two
 // workgroups per CU), 0 = decided at run time.
-template <int MR, int TILES, bool TAB, int SPW, bool PAIR>
-__global__ __launch_bounds__(kThreads) void qmv_q4_kernel(KParams p) {
+// REUSE = one pass covers K and the workgroup takes several tiles: the activations are staged once,
+// before the tile loop (their registers are free again when the weight loads start).
+template <int MR, int TILES, bool TAB, int SPW, bool PAIR, bool REUSE>
+__global__ __launch_bounds__(kThreads, (REUSE && MR == 8 && TILES == 2) ? 4 : 1) void qmv_q4_kernel(KParams p) {
+  static_assert(!REUSE || SPW != 0, "reuse needs a uniform slab count");
   static_assert(!PAIR || TILES == 2, "paired tiles need two tile slots");
   constexpr int kSlots = 4 * MR;                       // 16-byte slots per (slab, j)
   constexpr int kXsWave = kSpwMax * 4 * kSlots * 16;   // bytes of activation image per wave
-  constexpr int kRedBytes = kWaves * TILES * 256 * 4;
-  constexpr int kXsBytes = kWaves * kXsWave;
-  constexpr int kXsAlloc = kXsBytes > kRedBytes ? kXsBytes : kRedBytes;
-  __shared__ __attribute__((aligned(16))) char xs_all[kXsAlloc];
+  __shared__ __attribute__((aligned(16))) char xs_all[kWaves * kXsWave];
+  __shared__ float red[kWaves * TILES * 8 * 16];  // cross-wave reduction: [wave][tile][activation row][column]
   // Activation sums per (row, group): on the matrix unit for 8 rows (see 2b), with lane shuffles
   // while staging for fewer rows (cheaper there: the extra MFMAs would outweigh ~45 VALU per row).
   constexpr bool kMfmaSums = MR == 8;
@@ -154,20 +155,7 @@ __global__ __launch_bounds__(kThreads) void qmv_q4_kernel(KParams p) {
   const uint32_t words_per_row = K >> 3, groups_per_row = K >> 6, slabs_total = K >> 7;
   constexpr bool pair = PAIR;
   const uint32_t rows_per_slot = pair ? 32u : 16u;  // weight rows (of one matrix) per wave tile slot
-  const uint32_t tile_row = (blockIdx.x * NT + tw) * rows_per_slot;
 
-  const u4* wrow[TILES];
-  const __half* sbrow[TILES];
-#pragma unroll
-  for (int t = 0; t < TILES; ++t) {
-    const uint64_t e_w = TAB ? expert * p.estride_w : 0, e_s = TAB ? expert * p.estride_s : 0;
-    const bool first = t == 0 || pair;                       // which matrix
-    const uint32_t wr = tile_row + n + (pair ? 16 * t : 0);  // which row of it
-    wrow[t] = reinterpret_cast<const u4*>((first ? p.w0 : p.w1) + e_w + (uint64_t)wr * words_per_row) + g;
-    // scales live in the lanes with even g, biases in the lanes with odd g (exchanged later)
-    const __half* sb = (g & 1) ? (first ? p.b0 : p.b1) : (first ? p.s0 : p.s1);
-    sbrow[t] = sb + e_s + (uint64_t)wr * groups_per_row;
-  }
   uint32_t srcs[MR];  // source rows of the activations (wave-uniform)
 #pragma unroll
   for (int m = 0; m < MR; ++m) {
@@ -184,52 +172,18 @@ __global__ __launch_bounds__(kThreads) void qmv_q4_kernel(KParams p) {
   const u4 bconst_bits = n < 8 ? (u4){0x64006400u, 0x54005400u, 0x64006400u, 0x54005400u}
                                : (u4){0x3C003C00u, 0x3C003C00u, 0x3C003C00u, 0x3C003C00u};
   const h8 bconst = __builtin_bit_cast(h8, bconst_bits);
-
-  f4 F[TILES];
-#pragma unroll
-  for (int t = 0; t < TILES; ++t) F[t] = (f4){0.f, 0.f, 0.f, 0.f};
   QMV_MARK(p, 0);
 
-  for (uint32_t slab0 = 0; slab0 < slabs_total; slab0 += KS * kSpwMax) {
-    const uint32_t ns = slabs_total - slab0 < KS * kSpwMax ? slabs_total - slab0 : KS * kSpwMax;  // slabs of this pass
-    const int spw = SPW ? SPW : (int)((ns + KS - 1) / KS);
-    const int sl = (int)(slab0 + kp * spw);       // first slab of this wave
-    int my_rt = (int)ns - (int)(kp * spw);
-    my_rt = my_rt < 0 ? 0 : (my_rt > spw ? spw : my_rt);
-    const int my = SPW ? SPW : my_rt;
-
-    // ---- 1. every global load of the pass, small ones first --------------------------------
-    u4 xv[MR];
+  // activations of a pass: lane l of the wave loads 8 consecutive k of every row (slabs sl .. sl+my-1)
+  auto load_x = [&](int sl, int my, u4 (&xv)[MR]) {
 #pragma unroll
     for (int m = 0; m < MR; ++m) {
       xv[m] = (u4){0u, 0u, 0u, 0u};
       if ((uint32_t)m < rows && lane < my * 16)
         xv[m] = *reinterpret_cast<const u4*>(p.x + (uint64_t)srcs[m] * K + (uint32_t)(sl * 16 + lane) * 8);
     }
-    u4 sbv[TILES];  // word `it` = (group 2*it, group 2*it+1) of slab sl+it: scales or biases, by lane
-#pragma unroll
-    for (int t = 0; t < TILES; ++t) {
-      sbv[t] = (u4){0u, 0u, 0u, 0u};
-      const uint32_t* sp = reinterpret_cast<const uint32_t*>(sbrow[t]) + sl;
-      if (my == kSpwMax) {  // 4 slabs: one 16-byte load (4-byte aligned is enough for the hardware)
-        const U4Unaligned v = *reinterpret_cast<const U4Unaligned*>(sp);
-        sbv[t] = (u4){v.v[0], v.v[1], v.v[2], v.v[3]};
-      } else {
-        if (my > 0) sbv[t].x = sp[0];
-        if (my > 1) sbv[t].y = sp[1];
-        if (my > 2) sbv[t].z = sp[2];
-      }
-    }
-    u4 wreg[TILES][kSpwMax];
-#pragma unroll
-    for (int it = 0; it < kSpwMax; ++it) {
-      if (it < my) {
-#pragma unroll
-        for (int t = 0; t < TILES; ++t) wreg[t][it] = *(wrow[t] + (sl + it) * 4);
-      }
-    }
-    QMV_MARK(p, 1);
-
+  };
+  auto stage_x = [&](const u4 (&xv)[MR]) {
     if constexpr (kMfmaSums) {
       // ---- 2. this wave's activations -> its LDS image in operand order ------------------------
       {
@@ -266,6 +220,73 @@ __global__ __launch_bounds__(kThreads) void qmv_q4_kernel(KParams p) {
         }
       }
     }
+  };
+  if constexpr (REUSE) {  // single pass: slab0 = 0, SPW slabs per wave
+    u4 xv[MR];
+    load_x((int)(kp * SPW), SPW, xv);
+    stage_x(xv);
+  }
+
+  // ---- tiles of this workgroup: consecutive, so it streams one contiguous block of weight rows.
+  //      With one pass over K the activation image (and the sums) staged for the first tile serve
+  //      all of them.
+  const uint32_t ntiles = REUSE ? p.tpw : 1u;  // (without reuse the launcher gives every workgroup one tile)
+  for (uint32_t ti = 0; ti < ntiles; ++ti) {
+  const uint32_t wg_tile = blockIdx.x * ntiles + ti;
+  const uint32_t tile_row = (wg_tile * NT + tw) * rows_per_slot;
+
+  const u4* wrow[TILES];
+  const __half* sbrow[TILES];
+#pragma unroll
+  for (int t = 0; t < TILES; ++t) {
+    const uint64_t e_w = TAB ? expert * p.estride_w : 0, e_s = TAB ? expert * p.estride_s : 0;
+    const bool first = t == 0 || pair;                       // which matrix
+    const uint32_t wr = tile_row + n + (pair ? 16 * t : 0);  // which row of it
+    wrow[t] = reinterpret_cast<const u4*>((first ? p.w0 : p.w1) + e_w + (uint64_t)wr * words_per_row) + g;
+    // scales live in the lanes with even g, biases in the lanes with odd g (exchanged later)
+    const __half* sb = (g & 1) ? (first ? p.b0 : p.b1) : (first ? p.s0 : p.s1);
+    sbrow[t] = sb + e_s + (uint64_t)wr * groups_per_row;
+  }
+  f4 F[TILES];
+#pragma unroll
+  for (int t = 0; t < TILES; ++t) F[t] = (f4){0.f, 0.f, 0.f, 0.f};
+
+  for (uint32_t slab0 = 0; slab0 < slabs_total; slab0 += KS * kSpwMax) {
+    const uint32_t ns = slabs_total - slab0 < KS * kSpwMax ? slabs_total - slab0 : KS * kSpwMax;  // slabs of this pass
+    const int spw = SPW ? SPW : (int)((ns + KS - 1) / KS);
+    const int sl = (int)(slab0 + kp * spw);       // first slab of this wave
+    int my_rt = (int)ns - (int)(kp * spw);
+    my_rt = my_rt < 0 ? 0 : (my_rt > spw ? spw : my_rt);
+    const int my = SPW ? SPW : my_rt;
+
+    // ---- 1. every global load of the pass, small ones first --------------------------------
+    u4 xv[MR];
+    if constexpr (!REUSE) load_x(sl, my, xv);
+    u4 sbv[TILES];  // word `it` = (group 2*it, group 2*it+1) of slab sl+it: scales or biases, by lane
+#pragma unroll
+    for (int t = 0; t < TILES; ++t) {
+      sbv[t] = (u4){0u, 0u, 0u, 0u};
+      const uint32_t* sp = reinterpret_cast<const uint32_t*>(sbrow[t]) + sl;
+      if (my == kSpwMax) {  // 4 slabs: one 16-byte load (4-byte aligned is enough for the hardware)
+        const U4Unaligned v = *reinterpret_cast<const U4Unaligned*>(sp);
+        sbv[t] = (u4){v.v[0], v.v[1], v.v[2], v.v[3]};
+      } else {
+        if (my > 0) sbv[t].x = sp[0];
+        if (my > 1) sbv[t].y = sp[1];
+        if (my > 2) sbv[t].z = sp[2];
+      }
+    }
+    u4 wreg[TILES][kSpwMax];
+#pragma unroll
+    for (int it = 0; it < kSpwMax; ++it) {
+      if (it < my) {
+#pragma unroll
+        for (int t = 0; t < TILES; ++t) wreg[t][it] = *(wrow[t] + (sl + it) * 4);
+      }
+    }
+    QMV_MARK(p, 1);
+
+    if constexpr (!REUSE) stage_x(xv);
     QMV_MARK(p, 2);
 
     // ---- 2b/3 for 8 rows: slab by slab (few live registers).  The per (row, group) sums of the
@@ -365,31 +386,38 @@ __global__ __launch_bounds__(kThreads) void qmv_q4_kernel(KParams p) {
     QMV_MARK(p, 4);
   }
 
-  // ---- 4. reduce over the k-parts and over the two group halves, write out -------------------
+  // ---- 4. reduce over the two group halves (lane + 32 holds the other one) and over the
+  //         k-parts, write out -------------------------------------------------------------------
   QMV_MARK(p, 5);
-  __syncthreads();  // every wave is done with its activation image (the buffer is reused)
+  __syncthreads();  // the previous tile's sums have been read
   QMV_MARK(p, 6);
-  float* red = reinterpret_cast<float*>(xs_all);
+  // (index arithmetic of this part is kept inside the tile loop on purpose: hoisted out, it
+  // costs registers for the whole kernel)
+  uint32_t tid_t = tid;
+  asm volatile("" : "+v"(tid_t));
+  {
+    const uint32_t lane_t = tid_t & 63, wave_t = tid_t >> 6, n_t = lane_t & 15, g_t = lane_t >> 4;
 #pragma unroll
-  for (int t = 0; t < TILES; ++t)
+    for (int t = 0; t < TILES; ++t)
 #pragma unroll
-    for (int i = 0; i < 4; ++i) red[((wave * TILES + t) * 16 + g * 4 + i) * 16 + n] = F[t][i];
+      for (int i = 0; i < 4; ++i) {
+        const float v = F[t][i] + __shfl_xor(F[t][i], 32, 64);
+        if (g_t < 2) red[((wave_t * TILES + t) * 8 + g_t * 4 + i) * 16 + n_t] = v;
+      }
+  }
   __syncthreads();
   QMV_MARK(p, 7);
-  for (uint32_t o = tid; o < NT * 128; o += kThreads) {
+  for (uint32_t o = tid_t; o < NT * 128; o += kThreads) {
     const uint32_t otw = o >> 7, m = (o >> 4) & 7, nn = o & 15;
     if (m < rows) {
       float v[TILES];
 #pragma unroll
       for (int t = 0; t < TILES; ++t) {
         float acc = 0.f;
-        for (uint32_t q = 0; q < KS; ++q) {
-          const uint32_t w = otw * KS + q;
-          acc += red[((w * TILES + t) * 16 + m) * 16 + nn] + red[((w * TILES + t) * 16 + m + 8) * 16 + nn];
-        }
+        for (uint32_t q = 0; q < KS; ++q) acc += red[(((otw * KS + q) * TILES + t) * 8 + m) * 16 + nn];
         v[t] = acc;
       }
-      const uint64_t obase = (uint64_t)(row0 + m) * p.ld_out + (blockIdx.x * NT + otw) * rows_per_slot + nn;
+      const uint64_t obase = (uint64_t)(row0 + m) * p.ld_out + (wg_tile * NT + otw) * rows_per_slot + nn;
       if (TILES == 2 && !pair) v[0] = silu_f(v[0]) * v[TILES - 1];
 #pragma unroll
       for (int t = 0; t < TILES; ++t) {
@@ -401,13 +429,21 @@ __global__ __launch_bounds__(kThreads) void qmv_q4_kernel(KParams p) {
       }
     }
   }
+  }  // tiles of this workgroup
   QMV_MARK(p, 8);
 }
 
 template <int MR, int TILES, int SPW, bool PAIR>
 void launch_s(const KParams& p, bool tab, dim3 grid, hipStream_t s) {
-  if (tab) hipLaunchKernelGGL((qmv_q4_kernel<MR, TILES, true, SPW, PAIR>), grid, dim3(kThreads), 0, s, p);
-  else hipLaunchKernelGGL((qmv_q4_kernel<MR, TILES, false, SPW, PAIR>), grid, dim3(kThreads), 0, s, p);
+  if constexpr (SPW != 0) {
+    if (p.tpw > 1) {
+      if (tab) hipLaunchKernelGGL((qmv_q4_kernel<MR, TILES, true, SPW, PAIR, true>), grid, dim3(kThreads), 0, s, p);
+      else hipLaunchKernelGGL((qmv_q4_kernel<MR, TILES, false, SPW, PAIR, true>), grid, dim3(kThreads), 0, s, p);
+      return;
+    }
+  }
+  if (tab) hipLaunchKernelGGL((qmv_q4_kernel<MR, TILES, true, SPW, PAIR, false>), grid, dim3(kThreads), 0, s, p);
+  else hipLaunchKernelGGL((qmv_q4_kernel<MR, TILES, false, SPW, PAIR, false>), grid, dim3(kThreads), 0, s, p);
 }
 
 template <int MR, int TILES, bool PAIR = false>
@@ -487,7 +523,19 @@ int32_t launch_qmv_q4(const QmvArgs& a, hipStream_t s) {
   const uint32_t nt = 8 / ks;
   const bool pair = !a.dual && mr == 8 && a.N % (32 * nt) == 0 &&
                     (uint64_t)(a.N / (32 * nt)) * chunks >= 1ull * (uint32_t)ctx().num_cus;
-  dim3 grid(a.N / (16 * nt * (pair ? 2 : 1)), chunks);
+  // Tiles per workgroup: with one pass over K a workgroup keeps its staged activations for several
+  // consecutive tiles (staging 8 rows costs as many bytes as the two tiles it serves), as long as
+  // every CU still gets two workgroups.
+  const uint32_t tiles_x = a.N / (16 * nt * (pair ? 2 : 1));
+  uint32_t tpw = 1;
+  const bool uniform_single_pass = slabs == ks * kSpwMax || slabs == ks * 3;  // the kernels with a fixed slab count
+  if (uniform_single_pass) {
+    static const uint32_t cand[] = {8, 6, 4, 3, 2};
+    for (uint32_t c : cand)
+      if (tiles_x % c == 0 && (uint64_t)(tiles_x / c) * chunks >= 2ull * (uint32_t)ctx().num_cus) { tpw = c; break; }
+  }
+  p.tpw = tpw;
+  dim3 grid(tiles_x / tpw, chunks);
   if (pair) {
     launch_t<8, 2, true>(p, tab, grid, s);
   } else if (a.dual) {
