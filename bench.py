@@ -234,7 +234,7 @@ def main():
                    "parity_max_err": head.get("max_err"), "parity_tol": head.get("tol")},
         "roofline": {"bound": "hbm", "achieved": head["gbs"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": head["gbs"] / HBM_PEAK_GBS, "traffic": MEASURED_TRAFFIC_BYTES["qmv_q4_m1_4096"],
-                     "kernel": "qmv_q4_kernel<1,1,false,4,false>", "bytes_per_launch": head["bytes"],
+                     "kernel": "qmv_m1_kernel<4,64,1,true>", "bytes_per_launch": head["bytes"],
                      "avg_launch_us": head["us"]},
     }
     if not args.quick and "q4_qmm_m512_4096" in extra:

@@ -530,9 +530,14 @@ int32_t launch_qmv_q4(const QmvArgs& a, hipStream_t s) {
   uint32_t tpw = 1;
   const bool uniform_single_pass = slabs == ks * kSpwMax || slabs == ks * 3;  // the kernels with a fixed slab count
   if (uniform_single_pass) {
+    // With a chunk table, consecutive chunks often belong to one expert (more than 8 rows): a grid
+    // width that is a multiple of the 8 XCDs puts their workgroups for the same tiles on one XCD,
+    // next to each other in time, so the second chunk finds the weights in that L2.
     static const uint32_t cand[] = {8, 6, 4, 3, 2};
-    for (uint32_t c : cand)
-      if (tiles_x % c == 0 && (uint64_t)(tiles_x / c) * chunks >= 2ull * (uint32_t)ctx().num_cus) { tpw = c; break; }
+    for (int pass = tab ? 0 : 1; pass < 2 && tpw == 1; ++pass)
+      for (uint32_t c : cand)
+        if (tiles_x % c == 0 && (pass == 1 || (tiles_x / c) % 8 == 0) &&
+            (uint64_t)(tiles_x / c) * chunks >= 2ull * (uint32_t)ctx().num_cus) { tpw = c; break; }
   }
   p.tpw = tpw;
   dim3 grid(tiles_x / tpw, chunks);
