@@ -164,8 +164,8 @@ int32_t run_matmul_plain(const rmlx_qweight* qw, const void* x, int32_t x_dtype,
                 N, K, qw->bits, qw->group_size);
   } else if (kernel == KERNEL_QMM && !can_qmm) {
     return fail(RMLX_INVALID_SHAPE,
-                "qmm kernel requires bits in {4,8}, group_size=64, N %% 64 == 0, K %% 256 == 0 and 16-byte aligned "
-                "buffers (N=%u K=%u bits=%u group_size=%u)", N, K, qw->bits, qw->group_size);
+                "qmm kernel requires bits in {4,8}, N %% 64 == 0, 16-byte aligned buffers and K %% 512 == 0 (group sizes "
+                "32/64/128) or K %% 256 == 0 (group size 64) (N=%u K=%u bits=%u group_size=%u)", N, K, qw->bits, qw->group_size);
   } else if (kernel == KERNEL_QMM_LDS && !can_qmm_lds) {
     return fail(RMLX_INVALID_SHAPE,
                 "the LDS-staged qmm kernel requires bits in {4,8}, group_size=64, N %% 64 == 0, K %% 256 == 0 and "

@@ -111,8 +111,11 @@ __device__ __forceinline__ h8 dequant_q8_pair(uint32_t w0, uint32_t w1, h2 s2, h
 
 // MF = 16-row activation fragments per workgroup (tile rows = 16*MF), NF = 16-row weight fragments
 // per wave (tile columns = 64*NF), BITS = 4 or 8.
-template <int MF, int NF, int BITS, int NW, bool XBF16>
+// GS = quantisation group size (32, 64 or 128): it only decides which (scale, bias) pair a lane uses.
+template <int MF, int NF, int BITS, int NW, bool XBF16, int GS>
 __global__ __launch_bounds__(64 * NW) void qmm_rw_kernel(RwParams p) {
+  constexpr int kSbWords = 4 * (kBlockK / GS) / 2;  // 32-bit words of scales of one row and four iterations: 8 / 4 / 2
+  constexpr int kSbVecs = (kSbWords + 3) / 4;       // 16-byte registers holding them
   constexpr int kThreads = 64 * NW;
   constexpr int AL = MF * 256 / kThreads;      // 16-byte activation loads per thread and chunk
   static_assert(AL * kThreads == MF * 256, "chunk must divide over the workgroup");
@@ -141,7 +144,7 @@ __global__ __launch_bounds__(64 * NW) void qmm_rw_kernel(RwParams p) {
     nt = wg / p.tiles_m;
   }
 
-  const uint32_t K = p.K, S = K / kBlockK, G = K / 64;
+  const uint32_t K = p.K, S = K / kBlockK, G = K / GS;
   const uint32_t row_base = nt * (NW * 16 * NF) + wave * (16 * NF) + n;
 
   const u4* wptr[NF];
@@ -189,7 +192,7 @@ __global__ __launch_bounds__(64 * NW) void qmm_rw_kernel(RwParams p) {
   // The loop is unrolled by four so that every ring index is a compile-time constant.
   u4 ra[2][AL];
   u4 wq[kUnroll][NF][WL];
-  u4 s_cur[NF], b_cur[NF], s_nxt[NF], b_nxt[NF];
+  u4 s_cur[NF][kSbVecs], b_cur[NF][kSbVecs], s_nxt[NF][kSbVecs], b_nxt[NF][kSbVecs];
 
   // Q4: halves (k0..k7) -> slots (k0,k4,k1,k5,k2,k6,k3,k7), the order the nibble unpacking produces
   auto to_slot_order = [&](u4 v) {
@@ -220,15 +223,24 @@ __global__ __launch_bounds__(64 * NW) void qmm_rw_kernel(RwParams p) {
 #pragma unroll
     for (int q = 0; q < AL; ++q) a_lds[stage * kChunk + lds_w[q]] = to_slot_order(src[q]);
   };
-  auto load_sb = [&](uint32_t blk, u4 (&ds)[NF], u4 (&db)[NF]) {
+  auto load_sb = [&](uint32_t blk, u4 (&ds)[NF][kSbVecs], u4 (&db)[NF][kSbVecs]) {
 #pragma unroll
     for (int f = 0; f < NF; ++f) {
 #if defined(QMM_RW_EXP) && (QMM_RW_EXP & 16)
-      ds[f] = (u4){0x20002000u + blk, 0x20002000u, 0x20012001u, 0x20002000u};
-      db[f] = (u4){0xa000a000u + blk, 0xa000a000u, 0xa001a001u, 0xa000a000u};
+      ds[f][0] = (u4){0x20002000u + blk, 0x20002000u, 0x20012001u, 0x20002000u};
+      db[f][0] = (u4){0xa000a000u + blk, 0xa000a000u, 0xa001a001u, 0xa000a000u};
 #else
-      ds[f] = reinterpret_cast<const u4*>(sptr[f])[blk];
-      db[f] = reinterpret_cast<const u4*>(bptr[f])[blk];
+      if (GS == 128) {  // 4 groups = 8 bytes per row and four iterations
+        const u2 sv = reinterpret_cast<const u2*>(sptr[f])[blk], bv = reinterpret_cast<const u2*>(bptr[f])[blk];
+        ds[f][0] = (u4){sv.x, sv.y, 0u, 0u};
+        db[f][0] = (u4){bv.x, bv.y, 0u, 0u};
+      } else {
+#pragma unroll
+        for (int v = 0; v < kSbVecs; ++v) {
+          ds[f][v] = reinterpret_cast<const u4*>(sptr[f])[blk * kSbVecs + v];
+          db[f][v] = reinterpret_cast<const u4*>(bptr[f])[blk * kSbVecs + v];
+        }
+      }
 #endif
     }
   };
@@ -251,17 +263,35 @@ __global__ __launch_bounds__(64 * NW) void qmm_rw_kernel(RwParams p) {
   DqConst dq;
   dq.m0 = 0x000F000Fu; dq.m1 = 0x00F000F0u; dq.k0 = 0x64006400u; dq.k1 = 0x54005400u;
   asm volatile("" : "+s"(dq.m0), "+s"(dq.m1), "+v"(dq.k0), "+v"(dq.k1));
-  // Q4: the lane's group within a 128-wide block is g/2 -> which half of the f16 pair it scales with
-  const uint32_t sel_lane = (g >> 1) ? 0x03020302u : 0x01000100u;
+  // Which f16 of a scale word a lane uses.  Half h of a row's scale block belongs to iteration h / GPB
+  // and group h % GPB of its 128-wide k block (GPB = 128 / GS groups per block); a lane's k values lie
+  // in group (32g) / GS (Q4) or (64h + 16g) / GS (Q8, load h).
+  constexpr uint32_t kSelLo = 0x01000100u, kSelHi = 0x03020302u;
+  const uint32_t sel_g1 = (g >> 1) ? kSelHi : kSelLo, sel_g0 = (g & 1) ? kSelHi : kSelLo;
 
   // scale / bias operand pairs of iteration slot u of the current block (u == kUnroll: first
   // iteration of the next block)
+  auto word_of = [](const u4& v, int c) { return c == 0 ? v.x : (c == 1 ? v.y : (c == 2 ? v.z : v.w)); };
   auto scale_pair = [&](int u, int f, int h, h2& s2, h2& b2) {
-    const u4 sv = u < kUnroll ? s_cur[f] : s_nxt[f], bv = u < kUnroll ? b_cur[f] : b_nxt[f];
+    const u4 (&sv)[kSbVecs] = u < kUnroll ? s_cur[f] : s_nxt[f];
+    const u4 (&bv)[kSbVecs] = u < kUnroll ? b_cur[f] : b_nxt[f];
     const int w = u % kUnroll;
-    const uint32_t sw = w == 0 ? sv.x : (w == 1 ? sv.y : (w == 2 ? sv.z : sv.w));
-    const uint32_t bw = w == 0 ? bv.x : (w == 1 ? bv.y : (w == 2 ? bv.z : bv.w));
-    const uint32_t sel = BITS == 4 ? sel_lane : (h ? 0x03020302u : 0x01000100u);
+    uint32_t sw, bw, sel;
+    if (GS == 64) {         // word w = (group 0, group 1) of iteration w
+      sw = word_of(sv[0], w); bw = word_of(bv[0], w);
+      sel = BITS == 4 ? sel_g1 : (h ? kSelHi : kSelLo);
+    } else if (GS == 128) {  // half w = the one group of iteration w
+      sw = word_of(sv[0], w >> 1); bw = word_of(bv[0], w >> 1);
+      sel = (w & 1) ? kSelHi : kSelLo;
+    } else if (BITS == 4) {  // GS 32: half 4w + g
+      const int c = 2 * (w & 1);
+      sw = (g >> 1) ? word_of(sv[w >> 1], c + 1) : word_of(sv[w >> 1], c);
+      bw = (g >> 1) ? word_of(bv[w >> 1], c + 1) : word_of(bv[w >> 1], c);
+      sel = sel_g0;
+    } else {                 // GS 32, Q8: half 4w + 2h + g/2
+      sw = word_of(sv[w >> 1], 2 * (w & 1) + h); bw = word_of(bv[w >> 1], 2 * (w & 1) + h);
+      sel = sel_g1;
+    }
     s2 = __builtin_bit_cast(h2, __builtin_amdgcn_perm(sw, sw, sel));
     b2 = __builtin_bit_cast(h2, __builtin_amdgcn_perm(bw, bw, sel));
   };
@@ -362,7 +392,9 @@ __global__ __launch_bounds__(64 * NW) void qmm_rw_kernel(RwParams p) {
       RW_MARK(p, it, 5);
     }
 #pragma unroll
-    for (int f = 0; f < NF; ++f) { s_cur[f] = s_nxt[f]; b_cur[f] = b_nxt[f]; }
+    for (int f = 0; f < NF; ++f)
+#pragma unroll
+      for (int v = 0; v < kSbVecs; ++v) { s_cur[f][v] = s_nxt[f][v]; b_cur[f][v] = b_nxt[f][v]; }
   }
 
   // ---- epilogue: lane holds row m = lane%16 of fragment i, columns 4g..4g+3 of fragment f ------
@@ -399,13 +431,13 @@ __global__ __launch_bounds__(64 * NW) void qmm_rw_kernel(RwParams p) {
   RW_MARK_ALL(p, 1);
 }
 
-template <int MF, int NF, int BITS, int NW>
+template <int MF, int NF, int BITS, int NW, int GS = 64>
 void launch_rw(RwParams p, bool x_bf16, hipStream_t s) {
   p.tiles_m = (p.M + 16 * MF - 1) / (16 * MF);
   p.tiles_n = p.N / (NW * 16 * NF);
   const dim3 grid(p.tiles_m * p.tiles_n), block(64 * NW);
-  if (x_bf16) hipLaunchKernelGGL((qmm_rw_kernel<MF, NF, BITS, NW, true>), grid, block, 0, s, p);
-  else hipLaunchKernelGGL((qmm_rw_kernel<MF, NF, BITS, NW, false>), grid, block, 0, s, p);
+  if (x_bf16) hipLaunchKernelGGL((qmm_rw_kernel<MF, NF, BITS, NW, true, GS>), grid, block, 0, s, p);
+  else hipLaunchKernelGGL((qmm_rw_kernel<MF, NF, BITS, NW, false, GS>), grid, block, 0, s, p);
 }
 
 }  // namespace
@@ -416,7 +448,7 @@ int g_qmm_rw_force_mf = 0, g_qmm_rw_force_nf = 0, g_qmm_rw_force_nw = 4;
 #endif
 
 bool qmm_rw_supported(uint32_t N, uint32_t K, uint32_t group_size, uint32_t bits) {
-  return group_size == 64 && (bits == 4 || bits == 8) && N > 0 && K > 0 && N % 64 == 0 &&
+  return (group_size == 32 || group_size == 64 || group_size == 128) && (bits == 4 || bits == 8) && N > 0 && K > 0 && N % 64 == 0 &&
          K % (kBlockK * kUnroll) == 0;
 }
 
@@ -439,6 +471,8 @@ int32_t launch_qmm_rw(const QmmArgs& a, uint32_t group_size, hipStream_t s) {
   for (const auto& c : cand) {
     const uint32_t bn = 16 * c.nf * c.nw;
     if (a.N % bn != 0) continue;
+    // group sizes 32 / 128 are built for two tiles only (64 x 128 and 32 x 64)
+    if (group_size != 64 && !((c.mf == 4 && c.nf == 1 && c.nw == 8) || (c.mf == 2 && c.nf == 1 && c.nw == 4))) continue;
     const uint32_t wgs = ((a.M + 16 * c.mf - 1) / (16 * c.mf)) * (a.N / bn);
     const float cost = (float)((wgs + cus - 1) / cus) * (float)(c.mf * c.nf * c.nw) / c.eff;
     if (best == 0.f || cost < best) { best = cost; mf = c.mf; nf = c.nf; nw = c.nw; }
@@ -458,8 +492,17 @@ int32_t launch_qmm_rw(const QmmArgs& a, uint32_t group_size, hipStream_t s) {
   if (mf == MFV && nf == NFV && nw == NWV) {                                                   \
     if (a.bits == 4) launch_rw<MFV, NFV, 4, NWV>(p, x_bf16, s); else launch_rw<MFV, NFV, 8, NWV>(p, x_bf16, s); \
   }
-  RW_CASE(4, 2, 8) RW_CASE(4, 1, 8) RW_CASE(2, 1, 8) RW_CASE(2, 1, 4) RW_CASE(4, 2, 4) RW_CASE(2, 2, 4)
-  RW_CASE(8, 1, 8)
+#define RW_CASE_GS(MFV, NFV, NWV, GSV)                                                         \
+  if (mf == MFV && nf == NFV && nw == NWV && group_size == GSV) {                              \
+    if (a.bits == 4) launch_rw<MFV, NFV, 4, NWV, GSV>(p, x_bf16, s); else launch_rw<MFV, NFV, 8, NWV, GSV>(p, x_bf16, s); \
+  }
+  if (group_size == 64) {
+    RW_CASE(4, 2, 8) RW_CASE(4, 1, 8) RW_CASE(2, 1, 8) RW_CASE(2, 1, 4) RW_CASE(4, 2, 4) RW_CASE(2, 2, 4)
+    RW_CASE(8, 1, 8)
+  } else {
+    RW_CASE_GS(4, 1, 8, 32) RW_CASE_GS(2, 1, 4, 32) RW_CASE_GS(4, 1, 8, 128) RW_CASE_GS(2, 1, 4, 128)
+  }
+#undef RW_CASE_GS
 #undef RW_CASE
   RMLX_HIP_CHECK(hipGetLastError());
   return RMLX_OK;

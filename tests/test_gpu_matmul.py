@@ -424,3 +424,41 @@ def test_single_row_gemv_positions_and_multi_row_kernel_agree(hip, bits):
     ref = model.qmm(x_as_f64(x, "f16"), words, s, b, 64, bits)
     assert_close(_run(hip, words, s, b, x, bits, kernel=rt.KERNEL_QMV_ROWS), ref, "multi-row kernel at M=1")
     assert_close(_run(hip, words, s, b, x, bits, kernel=rt.KERNEL_QMV), ref, "single-row kernel")
+
+
+@pytest.mark.parametrize("bits", [4, 8])
+@pytest.mark.parametrize("gs", [32, 128])
+@pytest.mark.parametrize("m,n,k,dtype", [(33, 64, 512, "f16"), (100, 128, 1024, "f16"), (200, 256, 1536, "bf16"),
+                                          (64, 192, 2048, "f16"), (17, 64, 512, "f32")])
+def test_qmm_group_sizes_32_and_128(hip, bits, gs, m, n, k, dtype):
+    """The register-weights GEMM at the other group sizes the weight type admits: same result as the oracle and
+    as the portable kernel."""
+    from rmlx_amd import runtime as rt
+    rng = np.random.default_rng(bits + gs + m + n + k)
+    words, s, b = make_weight(rng, n, k, bits, gs)
+    x = make_x(rng, m, k, dtype)
+    ref = model.qmm(x_as_f64(x, dtype), words, s, b, gs, bits)
+    assert_close(_run(hip, words, s, b, x, bits, gs=gs, dtype=dtype), ref, f"auto bits={bits} gs={gs} M={m}")
+    assert_close(_run(hip, words, s, b, x, bits, gs=gs, dtype=dtype, kernel=rt.KERNEL_QMM), ref,
+                 f"qmm bits={bits} gs={gs} M={m}")
+    assert_close(_run(hip, words, s, b, x, bits, gs=gs, dtype=dtype, kernel=rt.KERNEL_GENERIC), ref,
+                 f"portable bits={bits} gs={gs} M={m}")
+
+
+def test_qmm_group_size_positions(hip):
+    """Scales that differ per group and a one-hot row pick out s[n, k / gs] exactly: every lane group, both
+    halves of a scale word, block borders."""
+    from rmlx_amd import runtime as rt
+    for bits in (4, 8):
+        for gs in (32, 64, 128):
+            n, k, m = 64, 1024, 32
+            rng = np.random.default_rng(gs * 10 + bits)
+            words = np.full((n, k * bits // 32), 0x11111111 if bits == 4 else 0x01010101, np.uint32)  # q = 1 everywhere
+            s = (rng.integers(1, 64, size=(n, k // gs)) / 8.0).astype(np.float16)
+            b = np.zeros((n, k // gs), np.float16)
+            ks = rng.choice(k, size=m, replace=False)
+            x = np.zeros((m, k), np.float16)
+            x[np.arange(m), ks] = 1.0
+            out = _run(hip, words, s, b, x, bits, gs=gs, kernel=rt.KERNEL_QMM)
+            want = s[:, ks // gs].T.astype(np.float64)
+            assert np.array_equal(out.astype(np.float64), want), f"bits={bits} gs={gs}"
