@@ -124,7 +124,7 @@ int32_t rmlx_hip_affine_quantized_matmul_batched(const rmlx_qweight* qw, const r
 /* Same contract as the batched entry point but forces one kernel family (the reference
  * exposes its kernels individually too, e.g. `affine_qmv_batched_f16_q4` quantized.rs:1675,
  * `affine_quantized_matmul_nax` :8517).  kernel: 0 = auto, 1 = streaming GEMV (qmv: the
- * single-row kernel where it applies -- M = 1, or M <= 16 at group sizes 32 / 128 -- else the multi-row one),
+ * single-row kernel where it applies -- M <= 2, or M <= 16 at group sizes 32 / 128 -- else the multi-row one),
  * 2 = MFMA GEMM (qmm, f16 MFMA; bf16 activations are converted, which is exact for
  * normal-range values; the register-weights kernel when K % 512 == 0, else the LDS-staged one),
  * 3 = portable scalar kernel (any bits/group size the type admits),

@@ -106,14 +106,14 @@ bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) ==
 // ---- the dispatch ladder --------------------------------------------------------------------
 // The reference picks by M: QMV for M=1, batched QMV up to a per-chip limit, split-K Steel for
 // 32 <= M < 128 and NAX above (crates/rmlx-core/src/ops/quantized.rs:7200-7256).  Here: the
-// single-row GEMV for M = 1 (and for a few rows when the group size is not 64), the streaming MFMA
+// single-row GEMV for M <= 2 (and up to 16 rows when the group size is not 64), the streaming MFMA
 // GEMV (weights read once per chunk of 8 rows; 16 rows for 8-bit weights) for small M, the
 // register-weights MFMA GEMM above (the LDS-staged GEMM when K is not a multiple of 512), the
 // portable kernel for every shape the fast kernels do not take.
 enum { KERNEL_AUTO = 0, KERNEL_QMV = 1, KERNEL_QMM = 2, KERNEL_GENERIC = 3, KERNEL_QMM_BF16 = 4, KERNEL_QMM_LDS = 5,
        KERNEL_QMV_ROWS = 6 };
 constexpr uint32_t kQmvMaxM = 16;
-constexpr uint32_t kM1MaxRows = 1;        // group size 64: rows taken by the single-row kernel
+constexpr uint32_t kM1MaxRows = 2;        // group size 64: rows taken by the single-row kernel (measured: 3 and 4 rows are faster on the matrix unit)
 constexpr uint32_t kM1MaxRowsOther = 16;  // group sizes 32 / 128: the alternative is the portable kernel
 
 struct Epilogue { int kind = EPI_NONE; const void* ptr = nullptr; int32_t dtype = RMLX_DTYPE_F16; };

@@ -20,8 +20,10 @@
 //     ((w & 0x000F000F) | 0x64006400 = (1024 + q0, 1024 + q4), ...); per lane and row
 //     acc = sum(x * (off + q)), and  scale * (acc - sum(off * x)) + bias * sum(x)  is added in f32.
 //     A quantisation group is 1, 2, 4 or 8 whole lanes (group sizes 32 / 64 / 128), so no
-//     cross-lane work is needed before the final wave-wide sum, and a wave writes its two
+//     cross-lane work is needed before the final wave-wide sum, and a wave writes its
 //     outputs itself: no cross-wave reduction, one barrier (after staging x).
+//   * Up to four activation rows share a pass: the unpacked weight pairs are reused, each row adds
+//     its own registers of x and 16 dot instructions per chunk and lane.
 #include "common.hpp"
 
 namespace rmlx {
@@ -39,7 +41,7 @@ struct M1Params {
   const uint32_t* w; const __half* s; const __half* b;
   const __half* x;
   __half* out;
-  uint32_t N, K;
+  uint32_t N, K, M;
 };
 
 __device__ __forceinline__ h2 as_h2(uint32_t v) { return __builtin_bit_cast(h2, v); }
@@ -71,8 +73,10 @@ __device__ __forceinline__ u4 to_pair_order(u4 d) {
   return o;
 }
 
-// R = weight rows per wave (1 or 2); NT = non-temporal weight loads (single activation row).
-template <int BITS, int GS, int R, bool NT>
+// R = weight rows per wave (1 or 2); NT = non-temporal weight loads (one pass over the weights);
+// MR = activation rows per pass (1, 2 or 4): their registers share the unpacked weights, so a few
+// rows cost one pass over the weights plus 16 dot instructions per row, chunk and lane.
+template <int BITS, int GS, int R, bool NT, int MR>
 __global__ __launch_bounds__(kThreads) void qmv_m1_kernel(M1Params p) {
   constexpr int kChunkK = 8192 / BITS;         // k values of one wave-wide 16-byte load: 2048 / 1024
   constexpr int kLaneK = kChunkK / 64;         // values per lane and chunk: 32 / 16
@@ -83,24 +87,29 @@ __global__ __launch_bounds__(kThreads) void qmv_m1_kernel(M1Params p) {
 
   extern __shared__ __attribute__((aligned(16))) char lds[];
   const uint32_t K = p.K, KH = K / kChunkK, G = K / GS, nunits = K / 8;
-  u4* xl = reinterpret_cast<u4*>(lds);                  // [chunk][unit j][lane]
-  float2* cs = reinterpret_cast<float2*>(lds + 2 * K);  // [chunk][lane]: (sum(off * x), sum(x)) of the lane's values
+  // per activation row: image [chunk][unit j][lane], then sums [chunk][lane] = (sum(off * x), sum(x)) of the lane's values
+  const uint32_t cs_bytes = K / kLaneK * sizeof(float2);
+  auto xl = [&](int m) { return reinterpret_cast<u4*>(lds + (size_t)m * 2 * K); };
+  auto cs = [&](int m) { return reinterpret_cast<float2*>(lds + (size_t)MR * 2 * K + (size_t)m * cs_bytes); };
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const uint32_t row0 = blockIdx.x * (kWaves * R) + wave * R;
-  const u4* xg = reinterpret_cast<const u4*>(p.x + (uint64_t)blockIdx.y * K);
+  const uint32_t mrow0 = blockIdx.y * MR;  // first activation row of this pass (rows past M repeat the last one, unstored)
 
   // ---- 1. loads, small ones first (the memory counter retires in order): activations ... ------
-  u4 xv[4];
-  {
+  u4 xv[MR][4];
+#pragma unroll
+  for (int m = 0; m < MR; ++m) {
+    const uint32_t rm = mrow0 + m < p.M ? mrow0 + m : p.M - 1;
+    const u4* xg = reinterpret_cast<const u4*>(p.x + (uint64_t)rm * K);
     const uint32_t u0 = (uint32_t)tid < nunits ? (uint32_t)tid : nunits - 1;
-    xv[0] = xg[u0];
+    xv[m][0] = xg[u0];
 #pragma unroll
     for (int i = 1; i < 4; ++i) {
-      xv[i] = (u4){0u, 0u, 0u, 0u};
+      xv[m][i] = (u4){0u, 0u, 0u, 0u};
       if (nunits > (uint32_t)i * kThreads) {  // uniform; the last round may be partial (clamped, stored under a guard)
         const uint32_t u = tid + i * kThreads;
-        xv[i] = xg[u < nunits ? u : nunits - 1];
+        xv[m][i] = xg[u < nunits ? u : nunits - 1];
       }
     }
   }
@@ -134,12 +143,14 @@ __global__ __launch_bounds__(kThreads) void qmv_m1_kernel(M1Params p) {
 
   // ---- 2. stage x: unit u = 8 consecutive k = (chunk, lane, j); image in the order a wave reads it ----
 #pragma unroll
+  for (int m = 0; m < MR; ++m)
+#pragma unroll
   for (int i = 0; i < 4; ++i) {
     const uint32_t u = tid + i * kThreads;
     if (u < nunits) {
       const uint32_t c = u / (64 * kXU), rem = u % (64 * kXU), l = rem / kXU, j = rem % kXU;
-      xl[(c * kXU + j) * 64 + l] = BITS == 4 ? to_pair_order(xv[i]) : xv[i];
-      const h8 hv = __builtin_bit_cast(h8, xv[i]);
+      xl(m)[(c * kXU + j) * 64 + l] = BITS == 4 ? to_pair_order(xv[m][i]) : xv[m][i];
+      const h8 hv = __builtin_bit_cast(h8, xv[m][i]);
       float xs8 = 0.f, xo8 = 0.f;
 #pragma unroll
       for (int e = 0; e < 8; e += 2) {
@@ -153,15 +164,17 @@ __global__ __launch_bounds__(kThreads) void qmv_m1_kernel(M1Params p) {
         xs8 = dpp_add<0x4E>(xs8);
         xo8 = dpp_add<0x4E>(xo8);
       }
-      if (j == 0) cs[c * 64 + l] = make_float2(xo8, xs8);
+      if (j == 0) cs(m)[c * 64 + l] = make_float2(xo8, xs8);
     }
   }
   __syncthreads();
 
   // ---- 3. chunk by chunk: registers of x from LDS, then the wave's rows --------------------------------
-  float racc[R];
+  float racc[R][MR];
 #pragma unroll
-  for (int r = 0; r < R; ++r) racc[r] = 0.f;
+  for (int r = 0; r < R; ++r)
+#pragma unroll
+    for (int m = 0; m < MR; ++m) racc[r][m] = 0.f;
   uint32_t m0 = 0x000F000Fu, m1 = 0x00F000F0u, k0 = 0x64006400u, k1 = 0x54005400u;
   asm volatile("" : "+s"(m0), "+s"(m1), "+v"(k0), "+v"(k1));  // constants in registers: and+or is one instruction
   auto process = [&](uint32_t c0, const Batch& t) {
@@ -169,37 +182,52 @@ __global__ __launch_bounds__(kThreads) void qmv_m1_kernel(M1Params p) {
     for (int cc = 0; cc < 2; ++cc) {
       const uint32_t c = c0 + cc;
       if (c < KH) {
-        uint32_t xr[kXU][4];
+        uint32_t xr[MR][kXU][4];
+        float2 k[MR];
 #pragma unroll
-        for (int j = 0; j < kXU; ++j) {
-          const u4 v = xl[(c * kXU + j) * 64 + lane];
-          xr[j][0] = v.x; xr[j][1] = v.y; xr[j][2] = v.z; xr[j][3] = v.w;
+        for (int m = 0; m < MR; ++m) {
+#pragma unroll
+          for (int j = 0; j < kXU; ++j) {
+            const u4 v = xl(m)[(c * kXU + j) * 64 + lane];
+            xr[m][j][0] = v.x; xr[m][j][1] = v.y; xr[m][j][2] = v.z; xr[m][j][3] = v.w;
+          }
+          k[m] = cs(m)[c * 64 + lane];
         }
-        const float2 k = cs[c * 64 + lane];
 #pragma unroll
         for (int r = 0; r < R; ++r) {
           const u4 wv = t.w[cc][r];
           const uint32_t wd[4] = {wv.x, wv.y, wv.z, wv.w};
-          float acc0 = 0.f, acc1 = 0.f;
+          float acc0[MR], acc1[MR];
+#pragma unroll
+          for (int m = 0; m < MR; ++m) acc0[m] = acc1[m] = 0.f;
 #pragma unroll
           for (int j = 0; j < 4; ++j) {
             if (BITS == 4) {
               const uint32_t hi = wd[j] >> 8;
-              acc0 = __builtin_amdgcn_fdot2(as_h2((wd[j] & m0) | k0), as_h2(xr[j][0]), acc0, false);
-              acc1 = __builtin_amdgcn_fdot2(as_h2((wd[j] & m1) | k1), as_h2(xr[j][1]), acc1, false);
-              acc0 = __builtin_amdgcn_fdot2(as_h2((hi & m0) | k0), as_h2(xr[j][2]), acc0, false);
-              acc1 = __builtin_amdgcn_fdot2(as_h2((hi & m1) | k1), as_h2(xr[j][3]), acc1, false);
+              const h2 p0 = as_h2((wd[j] & m0) | k0), p1 = as_h2((wd[j] & m1) | k1);
+              const h2 p2 = as_h2((hi & m0) | k0), p3 = as_h2((hi & m1) | k1);
+#pragma unroll
+              for (int m = 0; m < MR; ++m) {
+                acc0[m] = __builtin_amdgcn_fdot2(p0, as_h2(xr[m][j][0]), acc0[m], false);
+                acc1[m] = __builtin_amdgcn_fdot2(p1, as_h2(xr[m][j][1]), acc1[m], false);
+                acc0[m] = __builtin_amdgcn_fdot2(p2, as_h2(xr[m][j][2]), acc0[m], false);
+                acc1[m] = __builtin_amdgcn_fdot2(p3, as_h2(xr[m][j][3]), acc1[m], false);
+              }
             } else {  // bytes (q0,q1,q2,q3) -> (1024 + q0, 1024 + q1), (1024 + q2, 1024 + q3): natural order
               const int u = j >> 1, e = (j & 1) * 2;
-              acc0 = __builtin_amdgcn_fdot2(as_h2(__builtin_amdgcn_perm(0x64646464u, wd[j], 0x04010400u)),
-                                            as_h2(xr[u % kXU][e]), acc0, false);
-              acc1 = __builtin_amdgcn_fdot2(as_h2(__builtin_amdgcn_perm(0x64646464u, wd[j], 0x04030402u)),
-                                            as_h2(xr[u % kXU][e + 1]), acc1, false);
+              const h2 p0 = as_h2(__builtin_amdgcn_perm(0x64646464u, wd[j], 0x04010400u));
+              const h2 p1 = as_h2(__builtin_amdgcn_perm(0x64646464u, wd[j], 0x04030402u));
+#pragma unroll
+              for (int m = 0; m < MR; ++m) {
+                acc0[m] = __builtin_amdgcn_fdot2(p0, as_h2(xr[m][u % kXU][e]), acc0[m], false);
+                acc1[m] = __builtin_amdgcn_fdot2(p1, as_h2(xr[m][u % kXU][e + 1]), acc1[m], false);
+              }
             }
           }
           const float sc = __half2float(__ushort_as_half((unsigned short)t.s[cc][r]));
           const float bi = __half2float(__ushort_as_half((unsigned short)t.b[cc][r]));
-          racc[r] += sc * ((acc0 + acc1) - k.x) + bi * k.y;
+#pragma unroll
+          for (int m = 0; m < MR; ++m) racc[r][m] += sc * ((acc0[m] + acc1[m]) - k[m].x) + bi * k[m].y;
         }
       }
     }
@@ -214,36 +242,49 @@ __global__ __launch_bounds__(kThreads) void qmv_m1_kernel(M1Params p) {
     }
   }
 
-  // ---- 4. wave-wide sums; lane r writes the output of row r ----------------------------------------
+  // ---- 4. wave-wide sums; lane r * MR + m writes the output of (weight row r, activation row m) ------
   float mine = 0.f;
 #pragma unroll
-  for (int r = 0; r < R; ++r) {
-    const float t = wave_sum(racc[r]);
-    mine = lane == r ? t : mine;
-  }
-  if (lane < R) p.out[(uint64_t)blockIdx.y * p.N + row0 + lane] = __float2half(mine);
+  for (int r = 0; r < R; ++r)
+#pragma unroll
+    for (int m = 0; m < MR; ++m) {
+      const float t = wave_sum(racc[r][m]);
+      mine = lane == r * MR + m ? t : mine;
+    }
+  if (lane < R * MR && mrow0 + lane % MR < p.M)
+    p.out[(uint64_t)(mrow0 + lane % MR) * p.N + row0 + lane / MR] = __float2half(mine);
 }
 
-template <int BITS, int R, bool NT>
-void launch_r(const M1Params& p, uint32_t M, uint32_t group_size, hipStream_t s) {
-  const dim3 grid(p.N / (kWaves * R), M), block(kThreads);
-  const size_t lds = 2 * (size_t)p.K + (size_t)p.K / (128 / BITS) * sizeof(float2);
+template <int BITS, int R, bool NT, int MR>
+void launch_r(const M1Params& p, uint32_t group_size, hipStream_t s) {
+  const dim3 grid(p.N / (kWaves * R), (p.M + MR - 1) / MR), block(kThreads);
+  const size_t lds = (size_t)MR * (2 * (size_t)p.K + (size_t)p.K / (128 / BITS) * sizeof(float2));
   switch (group_size) {
-    case 32: hipLaunchKernelGGL((qmv_m1_kernel<BITS, 32, R, NT>), grid, block, lds, s, p); break;
-    case 64: hipLaunchKernelGGL((qmv_m1_kernel<BITS, 64, R, NT>), grid, block, lds, s, p); break;
-    default: hipLaunchKernelGGL((qmv_m1_kernel<BITS, 128, R, NT>), grid, block, lds, s, p); break;
+    case 32: hipLaunchKernelGGL((qmv_m1_kernel<BITS, 32, R, NT, MR>), grid, block, lds, s, p); break;
+    case 64: hipLaunchKernelGGL((qmv_m1_kernel<BITS, 64, R, NT, MR>), grid, block, lds, s, p); break;
+    default: hipLaunchKernelGGL((qmv_m1_kernel<BITS, 128, R, NT, MR>), grid, block, lds, s, p); break;
   }
 }
 
 template <int BITS>
-void launch_bits(const M1Params& p, uint32_t M, uint32_t group_size, hipStream_t s) {
-  // two rows per wave for long rows (more bytes in flight per wave), else one; several activation
-  // rows re-read the weights from L2, so only a single row streams them non-temporally
-  const bool two = p.K >= 12288 && p.N % (kWaves * 2) == 0;
-  if (M == 1) {
-    if (two) launch_r<BITS, 2, true>(p, M, group_size, s); else launch_r<BITS, 1, true>(p, M, group_size, s);
+void launch_bits(const M1Params& p, uint32_t group_size, hipStream_t s) {
+  // activation rows per pass: as many of 4 / 2 as fit the default dynamic LDS limit
+  const size_t per_row = 2 * (size_t)p.K + (size_t)p.K / (128 / BITS) * sizeof(float2);
+  int mr = p.M >= 3 ? 4 : (int)p.M;
+  while (mr > 1 && (size_t)mr * per_row > 65536) mr /= 2;
+  const bool one_pass = (p.M + mr - 1) / mr == 1;  // several passes re-read the weights from L2: no non-temporal loads
+  if (mr == 4) {
+    if (one_pass) launch_r<BITS, 1, true, 4>(p, group_size, s); else launch_r<BITS, 1, false, 4>(p, group_size, s);
+  } else if (mr == 2) {
+    if (one_pass) launch_r<BITS, 1, true, 2>(p, group_size, s); else launch_r<BITS, 1, false, 2>(p, group_size, s);
   } else {
-    if (two) launch_r<BITS, 2, false>(p, M, group_size, s); else launch_r<BITS, 1, false>(p, M, group_size, s);
+    // two weight rows per wave for long rows (more bytes in flight per wave), else one
+    const bool two = p.K >= 12288 && p.N % (kWaves * 2) == 0;
+    if (one_pass) {
+      if (two) launch_r<BITS, 2, true, 1>(p, group_size, s); else launch_r<BITS, 1, true, 1>(p, group_size, s);
+    } else {
+      if (two) launch_r<BITS, 2, false, 1>(p, group_size, s); else launch_r<BITS, 1, false, 1>(p, group_size, s);
+    }
   }
 }
 
@@ -261,9 +302,9 @@ int32_t launch_qmv_m1(const uint32_t* w, const __half* s, const __half* b, const
     return fail(RMLX_INVALID_SHAPE, "qmv_m1: unsupported shape N=%u K=%u bits=%u group_size=%u", N, K, bits, group_size);
   if (M == 0) return RMLX_OK;
   if (M > 65535) return fail(RMLX_INVALID_SHAPE, "qmv_m1: at most 65535 rows per launch (M=%u)", M);
-  M1Params p{w, s, b, x, out, N, K};
-  if (bits == 4) launch_bits<4>(p, M, group_size, stream);
-  else launch_bits<8>(p, M, group_size, stream);
+  M1Params p{w, s, b, x, out, N, K, M};
+  if (bits == 4) launch_bits<4>(p, group_size, stream);
+  else launch_bits<8>(p, group_size, stream);
   RMLX_HIP_CHECK(hipGetLastError());
   return RMLX_OK;
 }

@@ -391,12 +391,12 @@ def test_qmv_paired_tiles(hip, m, n, k):
 @pytest.mark.parametrize("gs", [32, 64, 128])
 @pytest.mark.parametrize("n,k", [(16, 2048), (24, 4096), (64, 4096), (48, 6144), (32, 8192), (40, 12288), (16, 16384)])
 def test_single_row_gemv(hip, bits, gs, n, k):
-    """M = 1 at every group size the weight type admits; at group sizes 32 / 128 the kernel also takes a
-    few rows (one pass over the weights per row)."""
+    """One to four rows (one pass over the weights) at every group size the weight type admits; at group
+    sizes 32 / 128 the kernel also takes up to 16 rows in passes of four."""
     from rmlx_amd import runtime as rt
     rng = np.random.default_rng(bits * 1000 + gs + n + k)
     words, s, b = make_weight(rng, n, k, bits, gs)
-    for m in ((1,) if gs == 64 else (1, 3, 16)):
+    for m in ((1, 2, 4) if gs == 64 else (1, 3, 16)):
         x = make_x(rng, m, k)
         ref = model.qmm(x_as_f64(x, "f16"), words, s, b, gs, bits)
         assert_close(_run(hip, words, s, b, x, bits, gs=gs), ref, f"auto bits={bits} gs={gs} N={n} K={k} M={m}")
