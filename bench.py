@@ -234,7 +234,7 @@ def main():
                    "parity_max_err": head.get("max_err"), "parity_tol": head.get("tol")},
         "roofline": {"bound": "hbm", "achieved": head["gbs"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": head["gbs"] / HBM_PEAK_GBS, "traffic": MEASURED_TRAFFIC_BYTES["qmv_q4_m1_4096"],
-                     "kernel": "qmv_m1_kernel<4,64,1,true>", "bytes_per_launch": head["bytes"],
+                     "kernel": "qmv_m1_kernel<4,64,1,true,1>", "bytes_per_launch": head["bytes"],
                      "avg_launch_us": head["us"]},
     }
     if not args.quick and "q4_qmm_m512_4096" in extra:
@@ -243,7 +243,7 @@ def main():
                              "roofline": {"bound": "mfma", "achieved": q["tflops"], "peak": MFMA_F16_PEAK_TF,
                                           "unit": "TFLOP/s", "frac": q["mfma_frac"],
                                           "traffic": MEASURED_TRAFFIC_BYTES["qmm_q4_m512_4096"],
-                                          "kernel": "qmm_rw_kernel<4,1,4,8,false>", "avg_launch_us": q["us"]}}
+                                          "kernel": "qmm_rw_kernel<4,1,4,8,false,64>", "avg_launch_us": q["us"]}}
     if not args.no_cpu:
         line["cpu_baseline"] = cpu_baseline(np.random.default_rng(1001), 3.0 if args.quick else 10.0)
     line["extra"] = extra
