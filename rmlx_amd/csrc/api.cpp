@@ -121,8 +121,8 @@ struct Epilogue { int kind = EPI_NONE; const void* ptr = nullptr; int32_t dtype 
 int32_t run_matmul_plain(const rmlx_qweight* qw, const void* x, int32_t x_dtype, uint32_t M, __half* out,
                          int32_t kernel, hipStream_t stream, const Epilogue& epi, bool* epi_done);
 
-// Matmul plus optional store epilogue: fused in the register-weights GEMM, a separate elementwise
-// pass after every other kernel.
+// Matmul plus optional store epilogue: fused in the register-weights GEMM and the single-row GEMV, a
+// separate elementwise pass after every other kernel.
 int32_t run_matmul(const rmlx_qweight* qw, const void* x, int32_t x_dtype, uint32_t M, __half* out,
                    int32_t kernel, hipStream_t stream, const Epilogue& epi = Epilogue()) {
   bool done = false;
@@ -214,9 +214,11 @@ int32_t run_matmul_plain(const rmlx_qweight* qw, const void* x, int32_t x_dtype,
     xk = cast.ptr;
   }
 
-  if (kernel == KERNEL_QMV && can_m1)
+  if (kernel == KERNEL_QMV && can_m1) {
+    *epi_done = true;
     return launch_qmv_m1(qw->w, qw->s, qw->b, static_cast<const __half*>(xk), out, M, N, K, qw->group_size, qw->bits,
-                         stream);
+                         epi.kind, epi.ptr, epi.dtype, stream);
+  }
   if (kernel == KERNEL_QMV_ROWS) kernel = KERNEL_QMV;
   if (kernel == KERNEL_QMV && qw->bits == 8)
     return launch_qmv_q8(qw->w, qw->s, qw->b, static_cast<const __half*>(xk), out, M, N, K, stream);

@@ -131,10 +131,11 @@ bool qmv_q8_supported(uint32_t N, uint32_t K, uint32_t group_size);
 int32_t launch_qmv_q8(const uint32_t* w, const __half* s, const __half* b, const __half* x, __half* out, uint32_t M,
                       uint32_t N, uint32_t K, hipStream_t stream);
 // Single-row GEMV (qmv_m1.hip): 4- or 8-bit weights, group size 32 / 64 / 128, f16 activations; M rows are
-// M independent passes over the weights (grid.y).
+// passes of up to four rows over the weights (grid.y); the store epilogue (EPI_*) is fused.
 bool qmv_m1_supported(uint32_t N, uint32_t K, uint32_t group_size, uint32_t bits);
 int32_t launch_qmv_m1(const uint32_t* w, const __half* s, const __half* b, const __half* x, __half* out, uint32_t M,
-                      uint32_t N, uint32_t K, uint32_t group_size, uint32_t bits, hipStream_t stream);
+                      uint32_t N, uint32_t K, uint32_t group_size, uint32_t bits, int epi_kind, const void* epi,
+                      int32_t epi_dtype, hipStream_t stream);
 // chunk table for gather_qmm: batch b owns rows [b*mpb, (b+1)*mpb) and expert indices[b]
 int32_t launch_build_gather_chunks(const uint32_t* indices, uint32_t batch, uint32_t mpb, uint32_t n_experts,
                                    uint32_t* chunk_tab, hipStream_t s);
@@ -147,7 +148,7 @@ struct QmmArgs {
   uint32_t M, N, K, bits;
   void* workspace;    // qmm_workspace_bytes(M, K) bytes of device scratch (fragment-major activations)
   int bf16_mfma;      // 1: bf16 activations x Q8 weights on the bf16 MFMA (weights rounded to bf16)
-  // fused store epilogue (register-weights GEMM only): 0 none, 1 out = acc + e, 2 out = silu(e) * acc
+  // fused store epilogue (register-weights GEMM; the single-row GEMV takes the same three values): 0 none, 1 out = acc + e, 2 out = silu(e) * acc
   int epi_kind;
   const void* epi;    // [M,N] f16 or f32
   int32_t epi_dtype;

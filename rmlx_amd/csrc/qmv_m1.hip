@@ -42,6 +42,8 @@ struct M1Params {
   const __half* x;
   __half* out;
   uint32_t N, K, M;
+  int32_t epi_kind, epi_dtype;  // fused store epilogue: EPI_RESIDUAL / EPI_SWIGLU with an [M,N] f16 / f32 operand
+  const void* epi;
 };
 
 __device__ __forceinline__ h2 as_h2(uint32_t v) { return __builtin_bit_cast(h2, v); }
@@ -112,6 +114,15 @@ __global__ __launch_bounds__(kThreads) void qmv_m1_kernel(M1Params p) {
         xv[m][i] = xg[u < nunits ? u : nunits - 1];
       }
     }
+  }
+  // ... the epilogue operand of the output this lane will write (lane r * MR + m) ...
+  const uint32_t out_m = mrow0 + lane % MR, out_n = row0 + lane / MR;
+  const bool writes = lane < R * MR && out_m < p.M;
+  float epi_val = 0.f;
+  if (p.epi_kind != EPI_NONE && writes) {
+    const uint64_t oi = (uint64_t)out_m * p.N + out_n;
+    epi_val = p.epi_dtype == RMLX_DTYPE_F32 ? static_cast<const float*>(p.epi)[oi]
+                                            : __half2float(static_cast<const __half*>(p.epi)[oi]);
   }
   // ---- ... then the first two chunks of the wave's rows with their scales and biases ----------------
   struct Batch { u4 w[2][R]; uint32_t s[2][R], b[2][R]; };  // [chunk of the batch][row]
@@ -251,8 +262,11 @@ __global__ __launch_bounds__(kThreads) void qmv_m1_kernel(M1Params p) {
       const float t = wave_sum(racc[r][m]);
       mine = lane == r * MR + m ? t : mine;
     }
-  if (lane < R * MR && mrow0 + lane % MR < p.M)
-    p.out[(uint64_t)(mrow0 + lane % MR) * p.N + row0 + lane / MR] = __float2half(mine);
+  if (writes) {  // residual add / SwiGLU gate in f32, one rounding (quantized.rs:3206-3246)
+    if (p.epi_kind == EPI_RESIDUAL) mine += epi_val;
+    else if (p.epi_kind == EPI_SWIGLU) mine = epi_val / (1.0f + __expf(-epi_val)) * mine;
+    p.out[(uint64_t)out_m * p.N + out_n] = __float2half(mine);
+  }
 }
 
 template <int BITS, int R, bool NT, int MR>
@@ -297,12 +311,13 @@ bool qmv_m1_supported(uint32_t N, uint32_t K, uint32_t group_size, uint32_t bits
 }
 
 int32_t launch_qmv_m1(const uint32_t* w, const __half* s, const __half* b, const __half* x, __half* out, uint32_t M,
-                      uint32_t N, uint32_t K, uint32_t group_size, uint32_t bits, hipStream_t stream) {
+                      uint32_t N, uint32_t K, uint32_t group_size, uint32_t bits, int epi_kind, const void* epi,
+                      int32_t epi_dtype, hipStream_t stream) {
   if (!qmv_m1_supported(N, K, group_size, bits))
     return fail(RMLX_INVALID_SHAPE, "qmv_m1: unsupported shape N=%u K=%u bits=%u group_size=%u", N, K, bits, group_size);
   if (M == 0) return RMLX_OK;
   if (M > 65535) return fail(RMLX_INVALID_SHAPE, "qmv_m1: at most 65535 rows per launch (M=%u)", M);
-  M1Params p{w, s, b, x, out, N, K, M};
+  M1Params p{w, s, b, x, out, N, K, M, epi_kind, epi_dtype, epi};
   if (bits == 4) launch_bits<4>(p, group_size, stream);
   else launch_bits<8>(p, group_size, stream);
   RMLX_HIP_CHECK(hipGetLastError());
