@@ -114,7 +114,7 @@ enum { KERNEL_AUTO = 0, KERNEL_QMV = 1, KERNEL_QMM = 2, KERNEL_GENERIC = 3, KERN
        KERNEL_QMV_ROWS = 6 };
 constexpr uint32_t kQmvMaxM = 16;
 constexpr uint32_t kM1MaxRows = 2;        // group size 64: rows taken by the single-row kernel (measured: 3 and 4 rows are faster on the matrix unit)
-constexpr uint32_t kM1MaxRowsOther = 16;  // group sizes 32 / 128: the alternative is the portable kernel
+constexpr uint32_t kM1MaxRowsOther = 16;  // shapes the multi-row GEMV does not take: the alternative is the portable kernel
 
 struct Epilogue { int kind = EPI_NONE; const void* ptr = nullptr; int32_t dtype = RMLX_DTYPE_F16; };
 
@@ -141,8 +141,10 @@ int32_t run_matmul_plain(const rmlx_qweight* qw, const void* x, int32_t x_dtype,
   const bool ptr_ok = aligned16(qw->w) && aligned16(qw->s) && aligned16(qw->b) && aligned16(x);
   const bool can_qmv = ptr_ok && ((qw->bits == 4 && qmv_q4_supported(N, K, qw->group_size)) ||
                                   (qw->bits == 8 && qmv_q8_supported(N, K, qw->group_size)));
+  // where the multi-row GEMV cannot take the shape (group size, K not a multiple of 512), the single-row
+  // kernel also runs small batches, in passes of four rows
   const bool can_m1 = ptr_ok && qmv_m1_supported(N, K, qw->group_size, qw->bits) &&
-                      M <= (qw->group_size == 64 ? kM1MaxRows : kM1MaxRowsOther);
+                      M <= (can_qmv ? kM1MaxRows : kM1MaxRowsOther);
   const bool can_qmm_lds = ptr_ok && qmm_supported(N, K, qw->group_size, qw->bits);
   const bool can_qmm_rw = ptr_ok && qmm_rw_supported(N, K, qw->group_size, qw->bits);
   const bool can_qmm = can_qmm_lds || can_qmm_rw;

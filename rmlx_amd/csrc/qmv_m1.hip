@@ -22,6 +22,8 @@
 //     A quantisation group is 1, 2, 4 or 8 whole lanes (group sizes 32 / 64 / 128), so no
 //     cross-lane work is needed before the final wave-wide sum, and a wave writes its
 //     outputs itself: no cross-wave reduction, one barrier (after staging x).
+//   * K is any multiple of 32 (4-bit) or 16 (8-bit) values: the lanes of the last chunk that lie
+//     past K meet zeros in the activation image.
 //   * Up to four activation rows share a pass: the unpacked weight pairs are reused, each row adds
 //     its own registers of x and 16 dot instructions per chunk and lane.
 #include "common.hpp"
@@ -88,11 +90,14 @@ __global__ __launch_bounds__(kThreads) void qmv_m1_kernel(M1Params p) {
   static_assert(kLanesPerGroup >= 1, "a lane must not straddle quantisation groups");
 
   extern __shared__ __attribute__((aligned(16))) char lds[];
-  const uint32_t K = p.K, KH = K / kChunkK, G = K / GS, nunits = K / 8;
+  // K need not be a multiple of the chunk: the lanes of the last chunk that lie past K read clamped
+  // (valid) addresses and multiply them with a zeroed activation image, i.e. contribute nothing.
+  const uint32_t K = p.K, KH = (K + kChunkK - 1) / kChunkK, G = K / GS, nunits = K / 8;
+  const uint32_t row_u4 = K / kLaneK;  // 16-byte pieces of a weight row
   // per activation row: image [chunk][unit j][lane], then sums [chunk][lane] = (sum(off * x), sum(x)) of the lane's values
-  const uint32_t cs_bytes = K / kLaneK * sizeof(float2);
-  auto xl = [&](int m) { return reinterpret_cast<u4*>(lds + (size_t)m * 2 * K); };
-  auto cs = [&](int m) { return reinterpret_cast<float2*>(lds + (size_t)MR * 2 * K + (size_t)m * cs_bytes); };
+  const uint32_t img_bytes = KH * kChunkK * 2, cs_bytes = KH * 64 * sizeof(float2);  // per activation row, whole chunks
+  auto xl = [&](int m) { return reinterpret_cast<u4*>(lds + (size_t)m * img_bytes); };
+  auto cs = [&](int m) { return reinterpret_cast<float2*>(lds + (size_t)MR * img_bytes + (size_t)m * cs_bytes); };
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const uint32_t row0 = blockIdx.x * (kWaves * R) + wave * R;
@@ -131,22 +136,25 @@ __global__ __launch_bounds__(kThreads) void qmv_m1_kernel(M1Params p) {
   const unsigned short* brow[R];
 #pragma unroll
   for (int r = 0; r < R; ++r) {
-    wrow[r] = reinterpret_cast<const u4*>(p.w + (uint64_t)(row0 + r) * (K * BITS / 32)) + lane;
-    srow[r] = reinterpret_cast<const unsigned short*>(p.s) + (uint64_t)(row0 + r) * G + lane / kLanesPerGroup;
-    brow[r] = reinterpret_cast<const unsigned short*>(p.b) + (uint64_t)(row0 + r) * G + lane / kLanesPerGroup;
+    wrow[r] = reinterpret_cast<const u4*>(p.w + (uint64_t)(row0 + r) * (K * BITS / 32));
+    srow[r] = reinterpret_cast<const unsigned short*>(p.s) + (uint64_t)(row0 + r) * G;
+    brow[r] = reinterpret_cast<const unsigned short*>(p.b) + (uint64_t)(row0 + r) * G;
   }
   auto load_batch = [&](uint32_t c0, Batch& t) {
 #pragma unroll
     for (int cc = 0; cc < 2; ++cc) {
       const uint32_t c = c0 + cc < KH ? c0 + cc : KH - 1;  // an odd chunk count re-reads the last chunk (unused)
+      uint32_t wi = c * 64 + lane, gi = c * kGroupsPerChunk + lane / kLanesPerGroup;
+      wi = wi < row_u4 ? wi : row_u4 - 1;  // lanes past K (last chunk of a K that is no chunk multiple)
+      gi = gi < G ? gi : G - 1;
 #pragma unroll
       for (int r = 0; r < R; ++r) {
-        t.s[cc][r] = srow[r][c * kGroupsPerChunk];
-        t.b[cc][r] = brow[r][c * kGroupsPerChunk];
+        t.s[cc][r] = srow[r][gi];
+        t.b[cc][r] = brow[r][gi];
       }
 #pragma unroll
       for (int r = 0; r < R; ++r)
-        t.w[cc][r] = NT ? __builtin_nontemporal_load(wrow[r] + (uint64_t)c * 64) : wrow[r][(uint64_t)c * 64];
+        t.w[cc][r] = NT ? __builtin_nontemporal_load(wrow[r] + wi) : wrow[r][wi];
     }
   };
   Batch ba, bb;
@@ -176,6 +184,10 @@ __global__ __launch_bounds__(kThreads) void qmv_m1_kernel(M1Params p) {
         xo8 = dpp_add<0x4E>(xo8);
       }
       if (j == 0) cs(m)[c * 64 + l] = make_float2(xo8, xs8);
+    } else if (u < KH * 64 * kXU) {  // image positions past K: zeros
+      const uint32_t c = u / (64 * kXU), rem = u % (64 * kXU), l = rem / kXU, j = rem % kXU;
+      xl(m)[(c * kXU + j) * 64 + l] = (u4){0u, 0u, 0u, 0u};
+      if (j == 0) cs(m)[c * 64 + l] = make_float2(0.f, 0.f);
     }
   }
   __syncthreads();
@@ -269,10 +281,17 @@ __global__ __launch_bounds__(kThreads) void qmv_m1_kernel(M1Params p) {
   }
 }
 
+// LDS bytes per activation row: image and per-lane sums over whole chunks
+template <int BITS>
+size_t lds_per_row(uint32_t K) {
+  const size_t chunk_k = 8192 / BITS, chunks = (K + chunk_k - 1) / chunk_k;
+  return chunks * (chunk_k * 2 + 64 * sizeof(float2));
+}
+
 template <int BITS, int R, bool NT, int MR>
 void launch_r(const M1Params& p, uint32_t group_size, hipStream_t s) {
   const dim3 grid(p.N / (kWaves * R), (p.M + MR - 1) / MR), block(kThreads);
-  const size_t lds = (size_t)MR * (2 * (size_t)p.K + (size_t)p.K / (128 / BITS) * sizeof(float2));
+  const size_t lds = (size_t)MR * lds_per_row<BITS>(p.K);
   switch (group_size) {
     case 32: hipLaunchKernelGGL((qmv_m1_kernel<BITS, 32, R, NT, MR>), grid, block, lds, s, p); break;
     case 64: hipLaunchKernelGGL((qmv_m1_kernel<BITS, 64, R, NT, MR>), grid, block, lds, s, p); break;
@@ -283,7 +302,7 @@ void launch_r(const M1Params& p, uint32_t group_size, hipStream_t s) {
 template <int BITS>
 void launch_bits(const M1Params& p, uint32_t group_size, hipStream_t s) {
   // activation rows per pass: as many of 4 / 2 as fit the default dynamic LDS limit
-  const size_t per_row = 2 * (size_t)p.K + (size_t)p.K / (128 / BITS) * sizeof(float2);
+  const size_t per_row = lds_per_row<BITS>(p.K);
   int mr = p.M >= 3 ? 4 : (int)p.M;
   while (mr > 1 && (size_t)mr * per_row > 65536) mr /= 2;
   const bool one_pass = (p.M + mr - 1) / mr == 1;  // several passes re-read the weights from L2: no non-temporal loads
@@ -307,7 +326,8 @@ void launch_bits(const M1Params& p, uint32_t group_size, hipStream_t s) {
 bool qmv_m1_supported(uint32_t N, uint32_t K, uint32_t group_size, uint32_t bits) {
   if (bits != 4 && bits != 8) return false;
   if (group_size != 32 && group_size != 64 && group_size != 128) return false;
-  return N > 0 && K > 0 && N % kWaves == 0 && K % (8192 / bits) == 0 && K <= kMaxK;
+  // a lane's 16 bytes of a row must be whole (32 values at 4 bits, 16 at 8) and groups must not straddle lanes
+  return N > 0 && K > 0 && N % kWaves == 0 && K % (128 / bits) == 0 && K % group_size == 0 && K <= kMaxK;
 }
 
 int32_t launch_qmv_m1(const uint32_t* w, const __half* s, const __half* b, const __half* x, __half* out, uint32_t M,

@@ -183,7 +183,7 @@ def test_input_dtypes(hip, bits, dtype):
 @pytest.mark.parametrize("gs", [32, 64, 128])
 def test_group_sizes_and_odd_shapes_portable_kernel(hip, bits, gs):
     rng = np.random.default_rng(gs + bits)
-    n, k, m = 24, 384, 5  # N not a multiple of 16, K not a multiple of 512 -> portable kernel
+    n, k, m = 24, 384, 5  # N not a multiple of 16, K not a multiple of 512: no matrix-unit kernel takes it
     words, s, b = make_weight(rng, n, k, bits, gs)
     x = make_x(rng, m, k)
     ref = model.qmm(x_as_f64(x, "f16"), words, s, b, gs, bits)
@@ -464,3 +464,25 @@ def test_qmm_group_size_positions(hip):
             out = _run(hip, words, s, b, x, bits, gs=gs, kernel=rt.KERNEL_QMM)
             want = s[:, ks // gs].T.astype(np.float64)
             assert np.array_equal(out.astype(np.float64), want), f"bits={bits} gs={gs}"
+
+
+@pytest.mark.parametrize("bits,gs", [(4, 64), (4, 32), (4, 128), (8, 64), (8, 32)])
+@pytest.mark.parametrize("n,k", [(16, 11008), (24, 3584), (8, 2560), (16, 1408), (40, 64 * 33), (8, 128)])
+def test_single_row_gemv_any_k(hip, bits, gs, n, k):
+    """K that is not a multiple of the 1 KB chunk (nor of 512): the tail lanes meet zeros.  Such shapes also
+    take a few rows on this kernel, because the multi-row GEMV needs K % 512 == 0."""
+    if k % gs != 0:
+        pytest.skip("group size does not divide K")
+    rng = np.random.default_rng(bits * 7 + gs + n + k)
+    words, s, b = make_weight(rng, n, k, bits, gs)
+    for m in (1, 2, 5, 16):
+        x = make_x(rng, m, k)
+        ref = model.qmm(x_as_f64(x, "f16"), words, s, b, gs, bits)
+        assert_close(_run(hip, words, s, b, x, bits, gs=gs), ref, f"bits={bits} gs={gs} N={n} K={k} M={m}")
+    # the last weight of a row, the first one past the last whole chunk, a group border
+    q = model.unpack_u32(words, bits).astype(np.float64)
+    for kk in sorted({k - 1, (k // 2048) * 2048 if k >= 2048 else 0, k // 2, gs - 1, min(gs, k - 1)}):
+        x = np.zeros((1, k), np.float16)
+        x[0, kk] = 1.0
+        out = _run(hip, words, np.ones_like(s), np.zeros_like(b), x, bits, gs=gs)
+        assert np.array_equal(out[0].astype(np.float64), q[:, kk]), f"bits={bits} gs={gs} K={k} k={kk}"
