@@ -37,7 +37,7 @@ typedef uint32_t u4 __attribute__((ext_vector_type(4)));
 
 constexpr int kThreads = 512;
 constexpr int kWaves = 8;
-constexpr uint32_t kMaxK = 16384;  // x image + sums must fit the default dynamic LDS limit; 4 x loads per thread
+constexpr uint32_t kMaxK = 32768;  // (the activation image and sums must also fit the default dynamic LDS limit)
 
 struct M1Params {
   const uint32_t* w; const __half* s; const __half* b;
@@ -161,15 +161,11 @@ __global__ __launch_bounds__(kThreads) void qmv_m1_kernel(M1Params p) {
   load_batch(0, ba);
 
   // ---- 2. stage x: unit u = 8 consecutive k = (chunk, lane, j); image in the order a wave reads it ----
-#pragma unroll
-  for (int m = 0; m < MR; ++m)
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const uint32_t u = tid + i * kThreads;
+  auto stage_unit = [&](int m, uint32_t u, const u4& v) {
     if (u < nunits) {
       const uint32_t c = u / (64 * kXU), rem = u % (64 * kXU), l = rem / kXU, j = rem % kXU;
-      xl(m)[(c * kXU + j) * 64 + l] = BITS == 4 ? to_pair_order(xv[m][i]) : xv[m][i];
-      const h8 hv = __builtin_bit_cast(h8, xv[m][i]);
+      xl(m)[(c * kXU + j) * 64 + l] = BITS == 4 ? to_pair_order(v) : v;
+      const h8 hv = __builtin_bit_cast(h8, v);
       float xs8 = 0.f, xo8 = 0.f;
 #pragma unroll
       for (int e = 0; e < 8; e += 2) {
@@ -188,6 +184,19 @@ __global__ __launch_bounds__(kThreads) void qmv_m1_kernel(M1Params p) {
       const uint32_t c = u / (64 * kXU), rem = u % (64 * kXU), l = rem / kXU, j = rem % kXU;
       xl(m)[(c * kXU + j) * 64 + l] = (u4){0u, 0u, 0u, 0u};
       if (j == 0) cs(m)[c * 64 + l] = make_float2(0.f, 0.f);
+    }
+  };
+#pragma unroll
+  for (int m = 0; m < MR; ++m)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) stage_unit(m, tid + i * kThreads, xv[m][i]);
+  // K > 16384: the remaining rounds, loaded here (behind the first weight loads; rare and long-running shapes)
+  for (uint32_t u = tid + 4 * kThreads; u < KH * 64 * kXU; u += kThreads) {
+#pragma unroll
+    for (int m = 0; m < MR; ++m) {
+      const uint32_t rm = mrow0 + m < p.M ? mrow0 + m : p.M - 1;
+      const u4 v = reinterpret_cast<const u4*>(p.x + (uint64_t)rm * K)[u < nunits ? u : nunits - 1];
+      stage_unit(m, u, v);
     }
   }
   __syncthreads();
@@ -327,7 +336,8 @@ bool qmv_m1_supported(uint32_t N, uint32_t K, uint32_t group_size, uint32_t bits
   if (bits != 4 && bits != 8) return false;
   if (group_size != 32 && group_size != 64 && group_size != 128) return false;
   // a lane's 16 bytes of a row must be whole (32 values at 4 bits, 16 at 8) and groups must not straddle lanes
-  return N > 0 && K > 0 && N % kWaves == 0 && K % (128 / bits) == 0 && K % group_size == 0 && K <= kMaxK;
+  if (!(N > 0 && K > 0 && N % kWaves == 0 && K % (128 / bits) == 0 && K % group_size == 0 && K <= kMaxK)) return false;
+  return (bits == 4 ? lds_per_row<4>(K) : lds_per_row<8>(K)) <= 65536;
 }
 
 int32_t launch_qmv_m1(const uint32_t* w, const __half* s, const __half* b, const __half* x, __half* out, uint32_t M,

@@ -486,3 +486,15 @@ def test_single_row_gemv_any_k(hip, bits, gs, n, k):
         x[0, kk] = 1.0
         out = _run(hip, words, np.ones_like(s), np.zeros_like(b), x, bits, gs=gs)
         assert np.array_equal(out[0].astype(np.float64), q[:, kk]), f"bits={bits} gs={gs} K={k} k={kk}"
+
+
+@pytest.mark.parametrize("bits,n,k", [(4, 16, 18944), (4, 8, 28672), (8, 16, 24576), (8, 8, 28672), (4, 8, 16384 + 64)])
+def test_single_row_gemv_long_k(hip, bits, n, k):
+    """K beyond 16384: the activation image is staged in more than four rounds (up to the LDS limit; past it
+    the multi-row kernels take over)."""
+    rng = np.random.default_rng(bits + n + k)
+    words, s, b = make_weight(rng, n, k, bits)
+    for m in (1, 2):
+        x = make_x(rng, m, k)
+        ref = model.qmm(x_as_f64(x, "f16"), words, s, b, 64, bits)
+        assert_close(_run(hip, words, s, b, x, bits), ref, f"bits={bits} N={n} K={k} M={m}")
