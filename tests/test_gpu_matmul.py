@@ -498,3 +498,22 @@ def test_single_row_gemv_long_k(hip, bits, n, k):
         x = make_x(rng, m, k)
         ref = model.qmm(x_as_f64(x, "f16"), words, s, b, 64, bits)
         assert_close(_run(hip, words, s, b, x, bits), ref, f"bits={bits} N={n} K={k} M={m}")
+
+
+def test_random_shapes_through_the_ladder(hip):
+    """Sixty seeded random (M, N, K, bits, group size) shapes through the automatic dispatch: whatever kernel
+    the ladder picks (single-row, multi-row GEMV, both GEMMs, portable) must land on the oracle."""
+    rng = np.random.default_rng(20240607)
+    for case in range(60):
+        bits = int(rng.choice([4, 8]))
+        gs = int(rng.choice([32, 64, 64, 128]))
+        n = int(rng.integers(1, 34)) * 8
+        k = int(rng.integers(1, 37)) * 128 if rng.random() < 0.6 else int(rng.integers(1, 73)) * gs
+        k = (k // gs) * gs or gs
+        m = int(rng.choice([1, 2, 3, 5, 8, 16, 17, 33, 70]))
+        dtype = str(rng.choice(["f16", "f16", "bf16", "f32"]))
+        words, s, b = make_weight(rng, n, k, bits, gs)
+        x = make_x(rng, m, k, dtype)
+        ref = model.qmm(x_as_f64(x, dtype), words, s, b, gs, bits)
+        assert_close(_run(hip, words, s, b, x, bits, gs=gs, dtype=dtype), ref,
+                     f"case {case}: M={m} N={n} K={k} bits={bits} gs={gs} {dtype}")
