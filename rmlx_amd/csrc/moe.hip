@@ -13,10 +13,69 @@ namespace {
 
 constexpr int kMaxExperts = 1024;  // LDS histogram capacity of the sort kernel
 
+// ---- wave-wide reductions on DPP (lane ^ 1, lane ^ 2, the other quad of 8, the other 8 of 16), one
+//      swizzle (lane ^ 16) and two readlanes: a fraction of the latency of six LDS shuffles ------------
+template <int CTRL>
+__device__ __forceinline__ uint32_t dpp_u32(uint32_t v) {
+  return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, CTRL, 0xF, 0xF, true);
+}
+template <int CTRL>
+__device__ __forceinline__ float dpp_f32(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, true));
+}
+__device__ __forceinline__ float swz16_f32(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, v), 0x401F));
+}
+__device__ __forceinline__ float readlane_f32(float v, int l) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), l));
+}
+__device__ __forceinline__ float wave_max(float v) {
+  v = fmaxf(v, dpp_f32<0xB1>(v));
+  v = fmaxf(v, dpp_f32<0x4E>(v));
+  v = fmaxf(v, dpp_f32<0x141>(v));
+  v = fmaxf(v, dpp_f32<0x140>(v));
+  v = fmaxf(v, swz16_f32(v));
+  return fmaxf(readlane_f32(v, 0), readlane_f32(v, 32));
+}
+__device__ __forceinline__ float wave_add(float v) {
+  v += dpp_f32<0xB1>(v);
+  v += dpp_f32<0x4E>(v);
+  v += dpp_f32<0x141>(v);
+  v += dpp_f32<0x140>(v);
+  v += swz16_f32(v);
+  return readlane_f32(v, 0) + readlane_f32(v, 32);
+}
+// lexicographic maximum of (hi, lo) over the wave; the result is uniform
+template <int CTRL>
+__device__ __forceinline__ void key_max_step(uint32_t& hi, uint32_t& lo) {
+  const uint32_t ohi = dpp_u32<CTRL>(hi), olo = dpp_u32<CTRL>(lo);
+  const bool take = ohi > hi || (ohi == hi && olo > lo);
+  hi = take ? ohi : hi;
+  lo = take ? olo : lo;
+}
+__device__ __forceinline__ void wave_key_max(uint32_t& hi, uint32_t& lo) {
+  key_max_step<0xB1>(hi, lo);
+  key_max_step<0x4E>(hi, lo);
+  key_max_step<0x141>(hi, lo);
+  key_max_step<0x140>(hi, lo);
+  {
+    const uint32_t ohi = (uint32_t)__builtin_amdgcn_ds_swizzle((int)hi, 0x401F), olo = (uint32_t)__builtin_amdgcn_ds_swizzle((int)lo, 0x401F);
+    const bool take = ohi > hi || (ohi == hi && olo > lo);
+    hi = take ? ohi : hi;
+    lo = take ? olo : lo;
+  }
+  const uint32_t h0 = (uint32_t)__builtin_amdgcn_readlane((int)hi, 0), l0 = (uint32_t)__builtin_amdgcn_readlane((int)lo, 0);
+  const uint32_t h1 = (uint32_t)__builtin_amdgcn_readlane((int)hi, 32), l1 = (uint32_t)__builtin_amdgcn_readlane((int)lo, 32);
+  const bool take = h1 > h0 || (h1 == h0 && l1 > l0);
+  hi = take ? h1 : h0;
+  lo = take ? l1 : l0;
+}
+
 // ---- routing: one wave per token -----------------------------------------------------------
 // Each lane owns experts lane, lane+64, lane+128, lane+192 (E <= 256).  Ranking uses the biased
 // logit with ties broken towards the lower expert index, which is the order of the softmax
 // values the reference ranks (exp is monotonic), made independent of the exp implementation.
+// A round's winner is the wave maximum of the key (order-preserving bits of the logit, ~index).
 __global__ __launch_bounds__(64) void topk_route_kernel(const float* __restrict__ logits,
                                                         const float* __restrict__ bias, uint32_t E,
                                                         uint32_t K, int renorm, uint32_t* __restrict__ out_idx,
@@ -38,14 +97,14 @@ __global__ __launch_bounds__(64) void topk_route_kernel(const float* __restrict_
     }
     mx = fmaxf(mx, v[j]);
   }
-  for (int off = 32; off > 0; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off, 64));
+  mx = wave_max(mx);
   float sum = 0.f;
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
     sm[j] = (lane + 64 * j < E) ? expf(v[j] - mx) : 0.f;
     sum += sm[j];
   }
-  for (int off = 32; off > 0; off >>= 1) sum += __shfl_xor(sum, off, 64);
+  sum = wave_add(sum);
   const float inv = 1.0f / sum;
 #pragma unroll
   for (int j = 0; j < 4; ++j) sm[j] *= inv;
@@ -55,17 +114,25 @@ __global__ __launch_bounds__(64) void topk_route_kernel(const float* __restrict_
   for (uint32_t k = 0; k < K; ++k) {
     float bv = NEG_INF;
     uint32_t bi = 0xFFFFFFFFu;
-    float bw = 0.f;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {  // ascending expert index inside the lane: strict > keeps the lower one
-      if (!taken[j] && (bi == 0xFFFFFFFFu || v[j] > bv)) { bv = v[j]; bi = lane + 64 * j; bw = sm[j]; }
+      if (!taken[j] && (bi == 0xFFFFFFFFu || v[j] > bv)) { bv = v[j]; bi = lane + 64 * j; }
     }
-    for (int off = 32; off > 0; off >>= 1) {
-      const float ov = __shfl_xor(bv, off, 64);
-      const uint32_t oi = __shfl_xor(bi, off, 64);
-      const float ow = __shfl_xor(bw, off, 64);
-      const bool other_better = (oi != 0xFFFFFFFFu) && (bi == 0xFFFFFFFFu || ov > bv || (ov == bv && oi < bi));
-      if (other_better) { bv = ov; bi = oi; bw = ow; }
+    // key: logits compare like their order-preserving bit patterns (-0 counted as +0), then the lower index
+    uint32_t hi = 0, lo = 0;
+    if (bi != 0xFFFFFFFFu) {
+      const uint32_t u = __float_as_uint(bv + 0.0f);
+      hi = (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+      hi = hi == 0 ? 1u : hi;  // keeps every candidate above "none" (only a NaN with all bits set maps to 0)
+      lo = 0xFFFFFFFFu - bi;
+    }
+    wave_key_max(hi, lo);
+    bi = hi == 0 ? 0xFFFFFFFFu : 0xFFFFFFFFu - lo;  // uniform
+    float bw = 0.f;
+    if (bi != 0xFFFFFFFFu) {
+      const int src = (int)(bi & 63u), jj = (int)(bi >> 6);
+      const float cand = jj == 0 ? sm[0] : (jj == 1 ? sm[1] : (jj == 2 ? sm[2] : sm[3]));
+      bw = readlane_f32(cand, __builtin_amdgcn_readfirstlane(src));
     }
 #pragma unroll
     for (int j = 0; j < 4; ++j)
@@ -188,6 +255,67 @@ __global__ __launch_bounds__(1024) void moe_sort_kernel(const uint32_t* __restri
   }
 }
 
+// At most 64 assignments (decode-sized batches): one wave, no barriers.  Lane i owns assignment i; ranks,
+// offsets and chunk positions are counted with readlane loops over the other lanes.  Same outputs as above.
+__global__ __launch_bounds__(64) void moe_sort_small_kernel(const uint32_t* __restrict__ idx, uint32_t n_assign,
+                                                            uint32_t E, uint32_t top_k, uint32_t* __restrict__ sorted,
+                                                            uint32_t* __restrict__ sorted_tok,
+                                                            uint32_t* __restrict__ inv, uint32_t* __restrict__ counts,
+                                                            uint32_t* __restrict__ offsets,
+                                                            uint32_t* __restrict__ chunk_tab,
+                                                            uint32_t* __restrict__ n_chunks) {
+  const uint32_t lane = threadIdx.x;
+  const uint32_t e = lane < n_assign ? idx[lane] : 0xFFFFFFFFu;
+  const bool valid = e < E;
+  uint32_t rank = 0, same = 0, less = 0, n_valid = 0;
+  for (int j = 0; j < 64; ++j) {
+    const uint32_t ej = (uint32_t)__builtin_amdgcn_readlane((int)e, j);
+    if (ej >= E) continue;  // uniform
+    ++n_valid;
+    same += ej == e ? 1u : 0u;
+    rank += (ej == e && j < (int)lane) ? 1u : 0u;
+    less += ej < e ? 1u : 0u;
+  }
+  const uint32_t pos = less + rank;
+  if (valid && sorted != nullptr) {
+    sorted[pos] = lane;
+    if (sorted_tok != nullptr) sorted_tok[pos] = lane / top_k;
+    if (inv != nullptr) inv[lane] = pos;
+  }
+  // the first assignment of every expert writes the expert's chunks; chunks of lower experts come first
+  const bool leader = valid && rank == 0;
+  const uint32_t my_chunks = leader ? (same + 7) / 8 : 0u;
+  uint32_t chunks_before = 0, total_chunks = 0;
+  for (int j = 0; j < 64; ++j) {
+    const uint32_t cj = (uint32_t)__builtin_amdgcn_readlane((int)my_chunks, j);
+    if (cj == 0) continue;  // uniform
+    const uint32_t ej = (uint32_t)__builtin_amdgcn_readlane((int)e, j);
+    total_chunks += cj;
+    chunks_before += ej < e ? cj : 0u;
+  }
+  if (leader && chunk_tab != nullptr) {
+    for (uint32_t c = 0; c < my_chunks; ++c) {
+      chunk_tab[3 * (chunks_before + c) + 0] = e;
+      chunk_tab[3 * (chunks_before + c) + 1] = less + 8 * c;
+      chunk_tab[3 * (chunks_before + c) + 2] = same - 8 * c < 8u ? same - 8 * c : 8u;
+    }
+  }
+  if (lane == 0 && n_chunks != nullptr) *n_chunks = total_chunks;
+  if (counts != nullptr || offsets != nullptr) {
+    for (uint32_t ee = lane; ee < E; ee += 64) {
+      uint32_t c = 0, o = 0;
+      for (int j = 0; j < 64; ++j) {
+        const uint32_t ej = (uint32_t)__builtin_amdgcn_readlane((int)e, j);
+        c += ej == ee ? 1u : 0u;
+        o += ej < ee ? 1u : 0u;
+      }
+      if (counts != nullptr) counts[ee] = c;
+      if (offsets != nullptr) offsets[ee] = o;
+    }
+    if (lane == 0 && offsets != nullptr) offsets[E] = n_valid;
+  }
+}
+
 __global__ void index_gather_kernel(const __half* __restrict__ src, uint32_t d, const uint32_t* __restrict__ idx,
                                     uint32_t src_rows, __half* __restrict__ dst) {
   const uint32_t i = blockIdx.x;
@@ -261,7 +389,12 @@ int32_t launch_topk_route(const float* logits, const float* bias, uint32_t T, ui
     hipLaunchKernelGGL(topk_route_kernel, dim3(T), dim3(64), 0, s, logits, bias, E, K, renorm, idx, w);
     RMLX_HIP_CHECK(hipGetLastError());
   }
-  if (counts != nullptr || offsets != nullptr) {
+  if ((counts != nullptr || offsets != nullptr) && T * K <= 64 && E <= (uint32_t)kMaxExperts) {
+    hipLaunchKernelGGL(moe_sort_small_kernel, dim3(1), dim3(64), 0, s, idx, T * K, E, K, (uint32_t*)nullptr,
+                       (uint32_t*)nullptr, (uint32_t*)nullptr, counts, offsets, (uint32_t*)nullptr,
+                       (uint32_t*)nullptr);
+    RMLX_HIP_CHECK(hipGetLastError());
+  } else if (counts != nullptr || offsets != nullptr) {
     hipLaunchKernelGGL(moe_sort_kernel, dim3(1), dim3(1024), 0, s, idx, T * K, E, K, (uint32_t*)nullptr,
                        (uint32_t*)nullptr, (uint32_t*)nullptr, counts, offsets, (uint32_t*)nullptr,
                        (uint32_t*)nullptr);
@@ -275,8 +408,12 @@ int32_t launch_moe_sort(const uint32_t* idx, uint32_t n_assign, uint32_t E, uint
                         uint32_t* chunk_tab, uint32_t* n_chunks, hipStream_t s) {
   if (E > (uint32_t)kMaxExperts)
     return fail(RMLX_INVALID_SHAPE, "moe_sort: n_experts (%u) exceeds maximum %d", E, kMaxExperts);
-  hipLaunchKernelGGL(moe_sort_kernel, dim3(1), dim3(1024), 0, s, idx, n_assign, E, top_k ? top_k : 1u, sorted,
-                     sorted_tok, inv, counts, offsets, chunk_tab, n_chunks);
+  if (n_assign <= 64)
+    hipLaunchKernelGGL(moe_sort_small_kernel, dim3(1), dim3(64), 0, s, idx, n_assign, E, top_k ? top_k : 1u, sorted,
+                       sorted_tok, inv, counts, offsets, chunk_tab, n_chunks);
+  else
+    hipLaunchKernelGGL(moe_sort_kernel, dim3(1), dim3(1024), 0, s, idx, n_assign, E, top_k ? top_k : 1u, sorted,
+                       sorted_tok, inv, counts, offsets, chunk_tab, n_chunks);
   RMLX_HIP_CHECK(hipGetLastError());
   return RMLX_OK;
 }
