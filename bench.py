@@ -126,6 +126,31 @@ def bench_moe(ops, rt, timer, rng, T, steps, warmup, experts):
     return res
 
 
+def bench_gather(ops, rt, timer, rng, batch, mpb, gh, gate_up, steps, warmup):
+    """gather_qmm over the stacked gate/up weights of the MoE configuration (every batch entry names an expert)."""
+    from oracle import model
+    E, n, k = gh.n_experts, gh.out_features, gh.in_features
+    idx = rng.integers(0, E, size=batch).astype(np.uint32)
+    x = rng.standard_normal((batch, mpb, k)).astype(np.float16)
+    xd, idxd = rt.DeviceBuffer.from_numpy(x), rt.DeviceBuffer.from_numpy(idx)
+    out = rt.DeviceBuffer((batch, mpb, n), rt.F16)
+
+    def run(c):
+        for _ in range(c):
+            ops.gather_qmm(xd, gh.weights_buf, gh.scales_buf, gh.biases_buf, idxd, batch, mpb, n, k, E, 64,
+                           stream=timer.stream, out=out)
+
+    ms = timer.run(run, steps, warmup)
+    distinct = len(np.unique(idx))
+    nbytes = distinct * (n * k // 2 + 4 * (n * k // 64)) + batch * mpb * (k + n) * 2
+    res = {"us": ms * 1e3, "distinct_experts": distinct, "bytes": nbytes, "gbs": nbytes / (ms * 1e-3) / 1e9}
+    e0 = int(idx[0])
+    ref = model.qmm(x[0].astype(np.float64), gate_up[0][e0], gate_up[1][e0], gate_up[2][e0], 64, 4)
+    err = float(np.abs(out.numpy()[0].astype(np.float64) - ref).max())
+    res["max_err"], res["tol"], res["pass"] = err, model.tolerance(ref), bool(err <= model.tolerance(ref))
+    return res
+
+
 def cpu_baseline(rng, budget_s=10.0):
     """The C restatement of the reference's scalar `affine_qmm` (oracle/affine_qmm_ref.c) on the
     headline configuration (M=1, K=N=4096), one host thread, repeated for about `budget_s`."""
@@ -194,6 +219,8 @@ def main():
         for m in (1, 4, 8):
             extra[f"q4_qmv_m{m}_n9216"] = bench_matmul(ops, rt, timer, rng, m, 9216, 4096, 4, "f16", args.steps,
                                                        args.warmup, GiB + GiB // 8, check=(m == 8))
+        extra["q4_qmv_m2_4096"] = bench_matmul(ops, rt, timer, rng, 2, 4096, 4096, 4, "f16", args.steps, args.warmup,
+                                               GiB + GiB // 8)
         extra["q8_qmv_m1_4096"] = bench_matmul(ops, rt, timer, rng, 1, 4096, 4096, 8, "f16", args.steps, args.warmup,
                                                GiB + GiB // 8)
         # the GEMM sections run as many steps as the headline: the GPU needs tens of milliseconds of
@@ -211,6 +238,10 @@ def main():
         down = make_weight(rng, 4096, 1536, 4, lead=(128,))
         experts = (gate_up, down, ops.QuantizedWeight.from_numpy(*gate_up, 64, 4),
                    ops.QuantizedWeight.from_numpy(*down, 64, 4))
+        for batch, mpb in ((32, 1), (32, 8)):
+            r = bench_gather(ops, rt, timer, rng, batch, mpb, experts[2], gate_up, max(50, args.steps // 10), 10)
+            r["hbm_frac"] = r["gbs"] / HBM_PEAK_GBS
+            extra[f"gather_qmm_q4_b{batch}_m{mpb}"] = r
         for T in (4, 32, 128):
             r = bench_moe(ops, rt, timer, rng, T, max(50, args.steps // 10), 10, experts)
             r["hbm_frac"] = r["gbs"] / HBM_PEAK_GBS

@@ -136,9 +136,10 @@ class QuantizedLinear:
 
 
 def gather_qmm(x, w_packed_buf, scales_buf, biases_buf, indices, batch, m_per_batch, n, k, n_experts, group_size,
-               stream=None):
+               stream=None, out=None):
     """gather_qmm (quantized.rs:9404-9599): out[b] = x[b] @ dequant(W[indices[b]])^T, f16 out."""
-    out = DeviceBuffer((batch, m_per_batch, n), F16)
+    if out is None:
+        out = DeviceBuffer((batch, m_per_batch, n), F16)
     xa, ia = x.array(), indices.array()
     rt.check(rt.lib().rmlx_hip_gather_qmm(ctypes.byref(xa), w_packed_buf.ptr, w_packed_buf.nbytes, scales_buf.ptr,
                                           scales_buf.nbytes, biases_buf.ptr, biases_buf.nbytes, ctypes.byref(ia),
