@@ -115,8 +115,10 @@ int32_t rmlx_hip_affine_quantized_matmul(const rmlx_qweight* qw, const rmlx_arra
 
 /* ---- qmm: `affine_quantized_matmul_batched` (quantized.rs:7149-7782) -----------------------
  * x: 2-D [M, in_features], f16 / f32 / bf16; out: f16 [M, out_features].  Chooses the kernel
- * by M (the reference's dispatch ladder, re-tuned for this chip): streaming MFMA GEMV for
- * small M, LDS-staged dequant + MFMA GEMM above. */
+ * by M (the reference's dispatch ladder, re-tuned for this chip): the single-row streaming
+ * GEMV for M <= 2, the multi-row streaming MFMA GEMV for small M, the MFMA GEMM (weights
+ * dequantised in registers, or staged through LDS) above, and the portable kernel for bit
+ * widths and shapes none of those takes. */
 int32_t rmlx_hip_affine_quantized_matmul_batched(const rmlx_qweight* qw, const rmlx_array* x,
                                                  void* out_f16_dev, size_t out_bytes,
                                                  rmlx_stream stream);

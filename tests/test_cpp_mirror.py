@@ -1,0 +1,93 @@
+"""include/rmlx_ops.hpp -- the C++ mirror of the reference's operator interface over the C ABI.
+
+A small C++ program (tests/cpp/ops_mirror_check.cpp) is compiled against the header with plain g++
+(the header needs no HIP headers) and linked with the C-ABI library.  Without a GPU it checks the
+validation rules and error variants; with one it runs a dense and an expert case through the mirror
+and this file compares what it wrote with the oracle.
+"""
+import os
+import subprocess
+
+import numpy as np
+import pytest
+
+from oracle import model
+from tests.helpers import assert_close, make_weight, make_x
+
+from tests.cpp.build import ROOT, build_check_program
+
+
+def test_mirror_compiles_and_validates_without_a_gpu():
+    exe = build_check_program()
+    r = subprocess.run([exe, "validate"], capture_output=True, text=True, timeout=60)
+    assert r.returncode == 0 and "validate ok" in r.stdout, r.stdout + r.stderr
+
+
+def test_mirror_names_follow_the_reference():
+    text = open(os.path.join(ROOT, "include", "rmlx_ops.hpp")).read()
+    for name in ["class KernelError", "InvalidShape", "NotFound", "class QuantizedWeight", "affine_quantized_matmul(",
+                 "affine_quantized_matmul_batched(", "qmm_add_residual(", "qmm_swiglu(", "gather_qmm(", "gpu_topk_route(",
+                 "struct TopkRouteResult", "expert_indices", "expert_weights", "expert_counts", "dispatch_offsets",
+                 "class QuantizedLinear", "class ExpertGroup", "grouped_forward(", "forward_grouped("]:
+        assert name in text, name
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("bits,gs,M", [(4, 64, 24), (8, 64, 3), (4, 128, 40)])
+def test_mirror_matches_oracle(tmp_path, bits, gs, M):
+    exe = build_check_program()
+    rng = np.random.default_rng(100 * bits + gs + M)
+    N, K, E, I, T, top_k = 384, 1024, 4, 512, 7, 2
+    d = str(tmp_path)
+
+    def put(name, a):
+        np.ascontiguousarray(a).tofile(os.path.join(d, name))
+
+    def get(name, dtype, shape):
+        return np.fromfile(os.path.join(d, name), dtype=dtype).reshape(shape)
+
+    dense = make_weight(rng, N, K, bits, gs)
+    x = make_x(rng, M, K)
+    side = rng.standard_normal((M, N)).astype(np.float32)
+    bias = rng.standard_normal(N).astype(np.float16)
+    experts = {"gate": make_weight(rng, I, K, 4, 64, lead=(E,)), "up": make_weight(rng, I, K, 4, 64, lead=(E,)),
+               "down": make_weight(rng, K, I, 4, 64, lead=(E,))}
+    xt = make_x(rng, T, K)
+    logits = rng.standard_normal((T, E)).astype(np.float32)
+    pick = rng.integers(0, E, size=T).astype(np.uint32)
+    for stem, trip in [("dense", dense)] + list(experts.items()):
+        for suffix, a in zip("wsb", trip):
+            put(f"{stem}_{suffix}.bin", a)
+    for name, a in [("x.bin", x), ("side.bin", side), ("bias.bin", bias), ("xt.bin", xt), ("logits.bin", logits),
+                    ("pick.bin", pick)]:
+        put(name, a)
+    # the expert weights are always Q4 / group 64; only the dense weight varies
+    open(os.path.join(d, "meta.txt"), "w").write(f"{N} {K} {gs} {bits} {M} {E} {I} {T} {top_k}\n")
+    print(f"mirror case bits={bits} gs={gs} M={M}", flush=True)
+    r = subprocess.run([exe, "run", d], capture_output=True, text=True, timeout=110)
+    assert r.returncode == 0 and "run ok" in r.stdout, r.stdout + r.stderr
+
+    ref = model.qmm(x, *dense, gs, bits)
+    assert_close(get("out_qmv.bin", np.float16, (N,)), ref[0], "qmv")
+    assert_close(get("out_qmm.bin", np.float16, (M, N)), ref, "qmm")
+    assert_close(get("out_residual.bin", np.float16, (M, N)), ref + side, "qmm_add_residual")
+    assert_close(get("out_swiglu.bin", np.float16, (M, N)), model.silu(side) * ref, "qmm_swiglu")
+    assert_close(get("out_linear.bin", np.float16, (M, N)), ref + bias.astype(np.float64), "QuantizedLinear")
+
+    g = experts["gate"]
+    assert_close(get("out_gather.bin", np.float16, (T, 1, I)),
+                 model.gather_qmm(xt.reshape(T, 1, K), *g, pick, 64), "gather_qmm")
+    idx, w, counts, offsets = model.topk_route(logits, top_k)
+    assert np.array_equal(get("out_route_idx.bin", np.uint32, idx.shape), idx)
+    np.testing.assert_allclose(get("out_route_w.bin", np.float32, w.shape), w, rtol=1e-5, atol=1e-6)
+    assert np.array_equal(get("out_route_counts.bin", np.uint32, counts.shape), counts)
+    assert np.array_equal(get("out_route_offsets.bin", np.uint32, offsets.shape), offsets)
+    moe_ref = model.moe_forward(xt, idx, w, experts["gate"], experts["up"], experts["down"], 64, top_k)
+    grouped = get("out_moe_grouped.bin", np.float16, (T, K))
+    assert_close(grouped, moe_ref, "MoeExperts::forward_grouped")
+    assert np.array_equal(grouped, get("out_moe.bin", np.float16, (T, K)))
+    for name, e, rows in [("out_group0.bin", 1, xt[:2]), ("out_group1.bin", 0, xt[2:])]:
+        ones = np.ones((len(rows), 1))
+        one_expert = model.moe_forward(rows, np.full((len(rows), 1), e), ones, experts["gate"], experts["up"],
+                                       experts["down"], 64, 1)
+        assert_close(get(name, np.float16, (len(rows), K)), one_expert, f"ExpertGroup item on expert {e}")
