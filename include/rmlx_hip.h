@@ -250,6 +250,28 @@ int32_t rmlx_hip_moe_forward(const rmlx_qweight* gate, const rmlx_qweight* up,
                              const rmlx_array* expert_bias, void* out_f16_dev, size_t out_bytes,
                              rmlx_stream stream);
 
+/* ---- AWQ / GPTQ INT4 dequantisation to f32 -----------------------------------------------------
+ * `awq_dequant` (quantized.rs:2269-2383, kernel :707-733): qweight u32 [rows, cols/8] packed along
+ * the columns, qzeros u32 [rows/group_size, cols/8], scales f32 [rows/group_size, cols];
+ * out f32 [rows, cols] = scales[g, col] * (nibble(qweight, col % 8) - nibble(qzeros, col % 8)), g = row / group_size.
+ * `gptq_dequant` (quantized.rs:2407-2590, kernel :749-783): qweight u32 [in_features/8, out_features]
+ * packed along the rows, qzeros u32 [num_groups, out_features/8], scales f32 [num_groups, out_features],
+ * g_idx (nullable) i32 [in_features]; out f32 [in_features, out_features] =
+ * scales[g, col] * (nibble(qweight, row % 8) - (nibble(qzeros, col % 8) + 1)), g = g_idx[row] or row / group_size.
+ * With g_idx, num_groups is what the scales buffer holds (scales_bytes / 4 / out_features), as in the
+ * reference; unlike the reference, a row whose g_idx lies outside [0, num_groups) is written as zeros
+ * instead of reading out of bounds.  Validation and messages as the reference (pack-factor multiples,
+ * group_size > 0, divisibility, the buffer lengths). */
+int32_t rmlx_hip_awq_dequant(const void* qweight_dev, size_t qweight_bytes, const void* qzeros_dev,
+                             size_t qzeros_bytes, const void* scales_f32_dev, size_t scales_bytes,
+                             size_t rows, size_t cols, size_t group_size, void* out_f32_dev,
+                             size_t out_bytes, rmlx_stream stream);
+int32_t rmlx_hip_gptq_dequant(const void* qweight_dev, size_t qweight_bytes, const void* qzeros_dev,
+                              size_t qzeros_bytes, const void* scales_f32_dev, size_t scales_bytes,
+                              const int32_t* g_idx_dev, size_t g_idx_bytes, size_t in_features,
+                              size_t out_features, size_t group_size, void* out_f32_dev,
+                              size_t out_bytes, rmlx_stream stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -9,6 +9,7 @@
 //   rmlx::ops::quantized::QuantizedWeight   crates/rmlx-core/src/ops/quantized.rs:78-177
 //   ...::affine_quantized_matmul            :1309-1411       ...::affine_quantized_matmul_batched  :7149-7782
 //   ...::qmm_add_residual / qmm_swiglu      :8227-8452       ...::gather_qmm                       :9404-9599
+//   ...::awq_dequant / gptq_dequant         :2269-2590
 //   rmlx::ops::topk_route::gpu_topk_route   crates/rmlx-core/src/ops/topk_route.rs:396-650
 //   rmlx::nn::QuantizedLinear               crates/rmlx-nn/src/quantized_linear.rs:77-201
 //   rmlx::nn::MoeExperts::forward_grouped   crates/rmlx-nn/src/moe.rs:1391-1508 (routed block of MoeLayer)
@@ -226,6 +227,27 @@ inline Array gather_qmm(const Array& x, const QuantizedWeight& stacked, const Ar
                                     stacked.biases_buf->length(), &i, batch, m_per_batch, stacked.out_features,
                                     stacked.in_features, stacked.n_experts, stacked.group_size, out.data(), out.nbytes(),
                                     raw(stream)));
+  return out;
+}
+
+// AWQ INT4 -> f32 [rows, cols] (quantized.rs:2269-2383)
+inline Array awq_dequant(const Array& qweight, const Array& qzeros, const Array& scales, size_t rows, size_t cols,
+                         size_t group_size, const Stream* stream = nullptr) {
+  Array out = Array::uninit({rows, cols}, DType::Float32);
+  detail::check(rmlx_hip_awq_dequant(qweight.data(), qweight.nbytes(), qzeros.data(), qzeros.nbytes(), scales.data(),
+                                     scales.nbytes(), rows, cols, group_size, out.data(), out.nbytes(), raw(stream)));
+  return out;
+}
+
+// GPTQ INT4 -> f32 [in_features, out_features] (quantized.rs:2407-2590); g_idx: null or i32 [in_features]
+// carried in a UInt32 array.
+inline Array gptq_dequant(const Array& qweight, const Array& qzeros, const Array& scales, const Array* g_idx,
+                          size_t in_features, size_t out_features, size_t group_size, const Stream* stream = nullptr) {
+  Array out = Array::uninit({in_features, out_features}, DType::Float32);
+  detail::check(rmlx_hip_gptq_dequant(qweight.data(), qweight.nbytes(), qzeros.data(), qzeros.nbytes(), scales.data(),
+                                      scales.nbytes(), g_idx != nullptr ? static_cast<const int32_t*>(g_idx->data()) : nullptr,
+                                      g_idx != nullptr ? g_idx->nbytes() : 0, in_features, out_features, group_size,
+                                      out.data(), out.nbytes(), raw(stream)));
   return out;
 }
 

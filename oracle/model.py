@@ -235,3 +235,54 @@ def moe_forward(x, indices, weights, gate, up, down, group_size, top_k, round_h=
         np.add.at(out, toks, wts[toks, ks][:, None] * y)
         cache.clear()
     return out
+
+
+# --------------------------------------------------------------------------------------
+# AWQ / GPTQ INT4 dequantisation (float32, bit-exact: one subtraction of small integers and
+# one multiplication per element)
+# --------------------------------------------------------------------------------------
+
+
+def awq_dequant(qweight, qzeros, scales, group_size):
+    """out[r, c] = scales[g, c] * (nibble(qweight[r, c/8], c%8) - nibble(qzeros[g, c/8], c%8)), g = r / group_size.
+
+    Follows `awq_dequant_f32` (crates/rmlx-core/src/ops/quantized.rs:707-733): packing along the
+    columns.  The reference holds no test or vector for it; pinned in tests/ by hand-computed words
+    (0x76543210 against zero word 0x11111111), by agreement with `gptq_dequant` on one logical matrix
+    packed both ways (the two index paths share nothing but `unpack_u32`, itself pinned above), and
+    by an element-at-a-time walk of the kernel's index arithmetic on small shapes.
+    """
+    qweight = np.asarray(qweight, dtype=np.uint32)
+    rows = qweight.shape[0]
+    nib = unpack_u32(qweight, 4).astype(np.float32)
+    zero = unpack_u32(np.asarray(qzeros, dtype=np.uint32), 4).astype(np.float32)
+    g = np.arange(rows) // group_size
+    return (np.asarray(scales, dtype=np.float32)[g] * (nib - zero[g])).astype(np.float32)
+
+
+def gptq_dequant(qweight, qzeros, scales, g_idx, group_size):
+    """out[r, c] = scales[g, c] * (nibble(qweight[r/8, c], r%8) - (nibble(qzeros[g, c/8], c%8) + 1)),
+    g = g_idx[r] if given else r / group_size.
+
+    Follows `gptq_dequant_f32` (crates/rmlx-core/src/ops/quantized.rs:749-783): packing along the rows
+    and the zero point stored minus one.  Rows whose g_idx is outside [0, groups) give zeros (the
+    reference reads out of bounds there; the library defines the result instead).  Pinned as
+    `awq_dequant`, plus: identity g_idx == no g_idx, and a permuted g_idx against the logical matrices.
+    """
+    qweight = np.asarray(qweight, dtype=np.uint32)
+    packed_rows, n = qweight.shape
+    k = packed_rows * 8
+    shifts = (np.arange(8, dtype=np.uint32) * np.uint32(4))[None, :, None]
+    nib = ((qweight[:, None, :] >> shifts) & np.uint32(15)).reshape(k, n).astype(np.float32)
+    zero = (unpack_u32(np.asarray(qzeros, dtype=np.uint32), 4).astype(np.float32) + np.float32(1))
+    scales = np.asarray(scales, dtype=np.float32)
+    groups = scales.shape[0]
+    if g_idx is None:
+        g = np.arange(k, dtype=np.int64) // group_size
+    else:
+        g = np.asarray(g_idx).astype(np.int32).view(np.uint32).astype(np.int64)  # the kernel's uint(g_idx[row])
+    valid = g < groups
+    gc = np.where(valid, g, 0)
+    out = scales[gc] * (nib - zero[gc])
+    out[~valid] = 0
+    return out.astype(np.float32)

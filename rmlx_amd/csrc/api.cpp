@@ -923,4 +923,88 @@ int32_t rmlx_hip_moe_forward(const rmlx_qweight* gate, const rmlx_qweight* up, c
   return finish(s);
 }
 
+// ---- AWQ / GPTQ dequantisation ---------------------------------------------------------------------
+
+int32_t rmlx_hip_awq_dequant(const void* qweight_dev, size_t qweight_bytes, const void* qzeros_dev,
+                             size_t qzeros_bytes, const void* scales_f32_dev, size_t scales_bytes, size_t rows,
+                             size_t cols, size_t group_size, void* out_f32_dev, size_t out_bytes,
+                             rmlx_stream stream) {
+  RMLX_TRY(require_init());
+  if (cols % 8 != 0) return fail(RMLX_INVALID_SHAPE, "awq_dequant: cols (%zu) must be a multiple of 8 (pack factor)", cols);
+  if (group_size == 0) return fail(RMLX_INVALID_SHAPE, "awq_dequant: group_size must be > 0");
+  if (rows % group_size != 0)
+    return fail(RMLX_INVALID_SHAPE, "awq_dequant: rows (%zu) must be a multiple of group_size (%zu)", rows, group_size);
+  const size_t num_groups = rows / group_size, cols_packed = cols / 8;
+  if (qweight_bytes < rows * cols_packed * 4)
+    return fail(RMLX_INVALID_SHAPE, "awq_dequant: qweight buffer too small: %zu bytes < expected %zu bytes for [%zu, %zu]",
+                qweight_bytes, rows * cols_packed * 4, rows, cols_packed);
+  if (qzeros_bytes < num_groups * cols_packed * 4)
+    return fail(RMLX_INVALID_SHAPE, "awq_dequant: qzeros buffer too small: %zu bytes < expected %zu bytes for [%zu, %zu]",
+                qzeros_bytes, num_groups * cols_packed * 4, num_groups, cols_packed);
+  if (scales_bytes < num_groups * cols * 4)
+    return fail(RMLX_INVALID_SHAPE, "awq_dequant: scales buffer too small: %zu bytes < expected %zu bytes for [%zu, %zu]",
+                scales_bytes, num_groups * cols * 4, num_groups, cols);
+  RMLX_TRY(check_out("awq_dequant", out_bytes, rows * cols * 4));
+  uint32_t r32, c32, g32;
+  RMLX_TRY(checked_u32(rows, "rows", &r32));
+  RMLX_TRY(checked_u32(cols, "cols", &c32));
+  RMLX_TRY(checked_u32(group_size, "group_size", &g32));
+  if (rows * cols != 0 && (qweight_dev == nullptr || qzeros_dev == nullptr || scales_f32_dev == nullptr || out_f32_dev == nullptr))
+    return fail(RMLX_INVALID_SHAPE, "awq_dequant: null device buffer");
+  hipStream_t s = (hipStream_t)stream;
+  RMLX_TRY(launch_awq_dequant(static_cast<const uint32_t*>(qweight_dev), static_cast<const uint32_t*>(qzeros_dev),
+                              static_cast<const float*>(scales_f32_dev), static_cast<float*>(out_f32_dev), r32, c32,
+                              g32, s));
+  return finish(s);
+}
+
+int32_t rmlx_hip_gptq_dequant(const void* qweight_dev, size_t qweight_bytes, const void* qzeros_dev,
+                              size_t qzeros_bytes, const void* scales_f32_dev, size_t scales_bytes,
+                              const int32_t* g_idx_dev, size_t g_idx_bytes, size_t in_features, size_t out_features,
+                              size_t group_size, void* out_f32_dev, size_t out_bytes, rmlx_stream stream) {
+  RMLX_TRY(require_init());
+  if (in_features % 8 != 0)
+    return fail(RMLX_INVALID_SHAPE, "gptq_dequant: in_features (%zu) must be a multiple of 8 (pack factor)", in_features);
+  if (out_features % 8 != 0)
+    return fail(RMLX_INVALID_SHAPE, "gptq_dequant: out_features (%zu) must be a multiple of 8 (pack factor for qzeros)",
+                out_features);
+  if (group_size == 0) return fail(RMLX_INVALID_SHAPE, "gptq_dequant: group_size must be > 0");
+  const bool has_g_idx = g_idx_dev != nullptr;
+  if (!has_g_idx && in_features % group_size != 0)
+    return fail(RMLX_INVALID_SHAPE,
+                "gptq_dequant: in_features (%zu) must be a multiple of group_size (%zu) when g_idx is not provided",
+                in_features, group_size);
+  const size_t rows_packed = in_features / 8, cols_packed = out_features / 8;
+  // with g_idx the group count is whatever the scales buffer holds (quantized.rs:2443-2450)
+  const size_t num_groups = has_g_idx ? (out_features == 0 ? 0 : scales_bytes / 4 / out_features) : in_features / group_size;
+  if (qweight_bytes < rows_packed * out_features * 4)
+    return fail(RMLX_INVALID_SHAPE, "gptq_dequant: qweight buffer too small: %zu bytes < expected %zu bytes for [%zu, %zu]",
+                qweight_bytes, rows_packed * out_features * 4, rows_packed, out_features);
+  if (qzeros_bytes < num_groups * cols_packed * 4)
+    return fail(RMLX_INVALID_SHAPE, "gptq_dequant: qzeros buffer too small: %zu bytes < expected %zu bytes for [%zu, %zu]",
+                qzeros_bytes, num_groups * cols_packed * 4, num_groups, cols_packed);
+  if (scales_bytes < num_groups * out_features * 4)
+    return fail(RMLX_INVALID_SHAPE, "gptq_dequant: scales buffer too small: %zu bytes < expected %zu bytes for [%zu, %zu]",
+                scales_bytes, num_groups * out_features * 4, num_groups, out_features);
+  if (has_g_idx && g_idx_bytes < in_features * 4)
+    return fail(RMLX_INVALID_SHAPE, "gptq_dequant: g_idx buffer too small: %zu bytes < expected %zu bytes for [%zu]",
+                g_idx_bytes, in_features * 4, in_features);
+  RMLX_TRY(check_out("gptq_dequant", out_bytes, in_features * out_features * 4));
+  uint32_t k32, n32, g32, ng32;
+  RMLX_TRY(checked_u32(in_features, "in_features", &k32));
+  RMLX_TRY(checked_u32(out_features, "out_features", &n32));
+  RMLX_TRY(checked_u32(group_size, "group_size", &g32));
+  RMLX_TRY(checked_u32(num_groups, "num_groups", &ng32));
+  if (in_features * out_features != 0) {
+    if (qweight_dev == nullptr || qzeros_dev == nullptr || scales_f32_dev == nullptr || out_f32_dev == nullptr)
+      return fail(RMLX_INVALID_SHAPE, "gptq_dequant: null device buffer");
+    if (num_groups == 0) return fail(RMLX_INVALID_SHAPE, "gptq_dequant: the scales buffer holds no complete group");
+  }
+  hipStream_t s = (hipStream_t)stream;
+  RMLX_TRY(launch_gptq_dequant(static_cast<const uint32_t*>(qweight_dev), static_cast<const uint32_t*>(qzeros_dev),
+                               static_cast<const float*>(scales_f32_dev), g_idx_dev, static_cast<float*>(out_f32_dev),
+                               k32, n32, g32, ng32, s));
+  return finish(s);
+}
+
 }  // extern "C"

@@ -182,6 +182,11 @@ int32_t launch_silu_gate(const __half* g, const __half* u, __half* out, size_t n
 int32_t launch_moe_combine(const float* y, const uint32_t* inv, const float* weights, uint32_t T,
                            uint32_t top_k, uint32_t D, __half* out, hipStream_t s);
 int32_t launch_add_bias_rows(__half* out, const __half* bias, uint32_t M, uint32_t N, hipStream_t s);
+int32_t launch_awq_dequant(const uint32_t* qweight, const uint32_t* qzeros, const float* scales, float* out,
+                           uint32_t rows, uint32_t cols, uint32_t group_size, hipStream_t s);
+int32_t launch_gptq_dequant(const uint32_t* qweight, const uint32_t* qzeros, const float* scales,
+                            const int32_t* g_idx, float* out, uint32_t in_features, uint32_t out_features,
+                            uint32_t group_size, uint32_t num_groups, hipStream_t s);
 int32_t launch_check_indices(const uint32_t* idx, uint32_t n, uint32_t limit, uint32_t* flag, hipStream_t s);
 
 }  // namespace rmlx

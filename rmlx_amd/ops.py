@@ -196,6 +196,29 @@ def silu_gate(gate_in, up_in, stream=None):
     return out
 
 
+def awq_dequant(qweight, qzeros, scales, rows, cols, group_size, stream=None, out=None):
+    """`awq_dequant` (crates/rmlx-core/src/ops/quantized.rs:2269-2383): qweight u32 [rows, cols/8], qzeros u32
+    [rows/group_size, cols/8], scales f32 [rows/group_size, cols] -> f32 [rows, cols]."""
+    if out is None:
+        out = DeviceBuffer((rows, cols), F32)
+    rt.check(rt.lib().rmlx_hip_awq_dequant(qweight.ptr, qweight.nbytes, qzeros.ptr, qzeros.nbytes, scales.ptr,
+                                           scales.nbytes, rows, cols, group_size, out.ptr, out.nbytes, _h(stream)))
+    return out
+
+
+def gptq_dequant(qweight, qzeros, scales, g_idx, in_features, out_features, group_size, stream=None, out=None):
+    """`gptq_dequant` (crates/rmlx-core/src/ops/quantized.rs:2407-2590): qweight u32 [in/8, out], qzeros u32
+    [groups, out/8], scales f32 [groups, out], g_idx (None or i32 [in], carried as its u32 bit pattern)
+    -> f32 [in, out]."""
+    if out is None:
+        out = DeviceBuffer((in_features, out_features), F32)
+    rt.check(rt.lib().rmlx_hip_gptq_dequant(qweight.ptr, qweight.nbytes, qzeros.ptr, qzeros.nbytes, scales.ptr,
+                                            scales.nbytes, g_idx.ptr if g_idx is not None else None,
+                                            g_idx.nbytes if g_idx is not None else 0, in_features, out_features,
+                                            group_size, out.ptr, out.nbytes, _h(stream)))
+    return out
+
+
 class ExpertGroup:
     """`ExpertGroup` (crates/rmlx-nn/src/expert_group.rs) over Q4 stacked expert weights."""
 
