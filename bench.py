@@ -151,6 +151,41 @@ def bench_gather(ops, rt, timer, rng, batch, mpb, gh, gate_up, steps, warmup):
     return res
 
 
+def bench_dequant(ops, rt, timer, rng, fmt, k, n, gs, steps, warmup):
+    """AWQ / GPTQ INT4 -> f32 dequantisation of one [k, n] matrix (store-bound: 4 bytes out per element).
+    Four input sets alternate; the packed inputs are an eighth of the traffic, the f32 output the rest."""
+    from oracle import model
+    groups = k // gs
+    sets = []
+    for _ in range(4):
+        shape = (k, n // 8) if fmt == "awq" else (k // 8, n)
+        qw = rng.integers(0, 2**32, size=shape, dtype=np.uint64).astype(np.uint32)
+        qz = rng.integers(0, 2**32, size=(groups, n // 8), dtype=np.uint64).astype(np.uint32)
+        sc = rng.uniform(0.001, 0.05, size=(groups, n)).astype(np.float32)
+        sets.append((qw, qz, sc, [rt.DeviceBuffer.from_numpy(a) for a in (qw, qz, sc)]))
+    out = rt.DeviceBuffer((k, n), rt.F32)
+
+    def launch(i):
+        d = sets[i % 4][3]
+        if fmt == "awq":
+            ops.awq_dequant(d[0], d[1], d[2], k, n, gs, stream=timer.stream, out=out)
+        else:
+            ops.gptq_dequant(d[0], d[1], d[2], None, k, n, gs, stream=timer.stream, out=out)
+
+    def run(c):
+        for i in range(c):
+            launch(i)
+
+    ms = timer.run(run, steps, warmup)
+    nbytes = k * n * 4 + k * n // 2 + groups * n // 2 + groups * n * 4
+    launch(0)
+    timer.stream.sync()
+    qw, qz, sc, _ = sets[0]
+    ref = model.awq_dequant(qw, qz, sc, gs) if fmt == "awq" else model.gptq_dequant(qw, qz, sc, None, gs)
+    return {"us": ms * 1e3, "bytes": nbytes, "gbs": nbytes / (ms * 1e-3) / 1e9,
+            "hbm_frac": nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, "pass": bool(np.array_equal(out.numpy(), ref))}
+
+
 def cpu_baseline(rng, budget_s=10.0):
     """The C restatement of the reference's scalar `affine_qmm` (oracle/affine_qmm_ref.c) on the
     headline configuration (M=1, K=N=4096), one host thread, repeated for about `budget_s`."""
@@ -234,6 +269,9 @@ def main():
             r["mfma_frac"] = r["tflops"] / MFMA_F16_PEAK_TF
             r["hbm_frac"] = r["gbs"] / HBM_PEAK_GBS
             extra[name] = r
+        for fmt in ("awq", "gptq"):
+            extra[f"{fmt}_dequant_4096x4096_gs128"] = bench_dequant(ops, rt, timer, rng, fmt, 4096, 4096, 128,
+                                                                    max(50, args.steps // 10), 10)
         gate_up = make_weight(rng, 3072, 4096, 4, lead=(128,))
         down = make_weight(rng, 4096, 1536, 4, lead=(128,))
         experts = (gate_up, down, ops.QuantizedWeight.from_numpy(*gate_up, 64, 4),

@@ -2,7 +2,7 @@
 // and :2407-2590).  Pure streaming: every output element is written once (4 bytes) and costs half a byte of
 // packed weight plus a share of one zero-point word and one scale, so the kernels are bound by the f32
 // store stream.  Both move 16 bytes per lane per access:
-//   awq_dequant_kernel   lane = 4 adjacent columns of 4 consecutive rows   (packing runs along columns)
+//   awq_dequant_kernel   lane = 4 adjacent columns of 8 consecutive rows   (packing runs along columns)
 //   gptq_dequant_kernel  lane = 4 adjacent columns of the 8 rows one packed word row holds (packing runs
 //                        along rows), so one 16-byte load feeds eight 16-byte stores
 // and a one-element-per-thread kernel takes the cases whose pointers are not 16-byte aligned.
@@ -29,33 +29,43 @@ __device__ __forceinline__ float4 dequant4(uint32_t q, uint32_t z, int zero_plus
   return o;
 }
 
-// grid = (row blocks of 4, column blocks of 4*kThreads)
+constexpr int kAwqRows = 8;  // rows per lane: 128 bytes of output per lane, as in the GPTQ kernel
+
+// grid = row blocks of kAwqRows x column blocks of 4*kThreads, the column block varying fastest so that
+// the workgroups in flight together cover contiguous memory
 __global__ __launch_bounds__(kThreads) void awq_dequant_kernel(const uint32_t* __restrict__ qweight,
                                                                const uint32_t* __restrict__ qzeros,
                                                                const float* __restrict__ scales,
                                                                float* __restrict__ out, uint32_t rows, uint32_t cols,
-                                                               uint32_t group_size) {
-  const uint32_t quad = blockIdx.y * kThreads + threadIdx.x;  // columns 4*quad .. 4*quad+3
+                                                               uint32_t group_size, uint32_t col_blocks) {
+  const uint32_t quad = (blockIdx.x % col_blocks) * kThreads + threadIdx.x;  // columns 4*quad .. 4*quad+3
   if (quad * 4 >= cols) return;
-  const uint32_t r0 = blockIdx.x * 4;
+  const uint32_t r0 = (blockIdx.x / col_blocks) * kAwqRows;
   const uint32_t words = cols / 8;
   const uint32_t shift = (quad & 1) * 16;
-  uint32_t q[4], g[4];
+  // Lanes 2j and 2j+1 share the packed words of columns 8j..8j+7: the even lane fetches those of the even
+  // rows, the odd lane those of the odd rows, and one lane swap hands each the other's word.
+  uint32_t q[kAwqRows], g[kAwqRows];
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const uint32_t r = r0 + i < rows ? r0 + i : rows - 1;
-    q[i] = __builtin_nontemporal_load(qweight + (size_t)r * words + quad / 2);
-    g[i] = r / group_size;
+  for (int i = 0; i < kAwqRows; i += 2) {
+    const uint32_t mine = r0 + i + (quad & 1);
+    const uint32_t r = mine < rows ? mine : rows - 1;
+    const uint32_t w = qweight[(size_t)r * words + quad / 2];
+    const uint32_t other = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)w, 0xB1, 0xF, 0xF, true);  // lane ^ 1
+    q[i] = (quad & 1) ? other : w;
+    q[i + 1] = (quad & 1) ? w : other;
   }
-  uint32_t z[4];
-  float4 s[4];
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
+  for (int i = 0; i < kAwqRows; ++i) g[i] = (r0 + i < rows ? r0 + i : rows - 1) / group_size;
+  uint32_t z[kAwqRows];
+  float4 s[kAwqRows];
+#pragma unroll
+  for (int i = 0; i < kAwqRows; ++i) {
     z[i] = qzeros[(size_t)g[i] * words + quad / 2];
     s[i] = *reinterpret_cast<const float4*>(scales + (size_t)g[i] * cols + quad * 4);
   }
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
+  for (int i = 0; i < kAwqRows; ++i) {
     if (r0 + i < rows) {
       const float4 o = dequant4(q[i] >> shift, z[i] >> shift, 0, s[i]);
       store4(out + (size_t)(r0 + i) * cols + quad * 4, o);
@@ -63,17 +73,18 @@ __global__ __launch_bounds__(kThreads) void awq_dequant_kernel(const uint32_t* _
   }
 }
 
-// grid = (packed rows, column blocks of 4*kThreads).  Rows whose group index is outside
+// grid = packed rows x column blocks of 4*kThreads, the column block varying fastest.  Rows whose group index is outside
 // [0, num_groups) -- only possible through g_idx -- are written as zeros.
 __global__ __launch_bounds__(kThreads) void gptq_dequant_kernel(const uint32_t* __restrict__ qweight,
                                                                 const uint32_t* __restrict__ qzeros,
                                                                 const float* __restrict__ scales,
                                                                 const int32_t* __restrict__ g_idx,
                                                                 float* __restrict__ out, uint32_t out_features,
-                                                                uint32_t group_size, uint32_t num_groups) {
-  const uint32_t quad = blockIdx.y * kThreads + threadIdx.x;
+                                                                uint32_t group_size, uint32_t num_groups,
+                                                                uint32_t col_blocks) {
+  const uint32_t quad = (blockIdx.x % col_blocks) * kThreads + threadIdx.x;
   if (quad * 4 >= out_features) return;
-  const uint32_t pr = blockIdx.x;
+  const uint32_t pr = blockIdx.x / col_blocks;
   const uint32_t zwords = out_features / 8;
   const uint32_t shift = (quad & 1) * 16;
   const uint4 w = *reinterpret_cast<const uint4*>(qweight + (size_t)pr * out_features + quad * 4);
@@ -130,10 +141,11 @@ int32_t launch_awq_dequant(const uint32_t* qweight, const uint32_t* qzeros, cons
   if (rows == 0 || cols == 0) return RMLX_OK;
   const uint32_t num_groups = rows / group_size;
   if (aligned16(scales) && aligned16(out)) {
-    const dim3 grid((rows + 3) / 4, (cols / 4 + kThreads - 1) / kThreads);
-    if (grid.y > 65535) return fail(RMLX_INVALID_SHAPE, "awq_dequant: cols (%u) too large", cols);
-    hipLaunchKernelGGL(awq_dequant_kernel, grid, dim3(kThreads), 0, s, qweight, qzeros, scales, out, rows, cols,
-                       group_size);
+    const uint32_t col_blocks = (cols / 4 + kThreads - 1) / kThreads;
+    const size_t blocks = (size_t)((rows + kAwqRows - 1) / kAwqRows) * col_blocks;
+    if (blocks > 0x7fffffffull) return fail(RMLX_INVALID_SHAPE, "awq_dequant: matrix too large");
+    hipLaunchKernelGGL(awq_dequant_kernel, dim3((unsigned)blocks), dim3(kThreads), 0, s, qweight, qzeros, scales, out,
+                       rows, cols, group_size, col_blocks);
   } else {
     const size_t blocks = ((size_t)rows * cols + kThreads - 1) / kThreads;
     if (blocks > 0x7fffffffull) return fail(RMLX_INVALID_SHAPE, "awq_dequant: matrix too large");
@@ -149,10 +161,11 @@ int32_t launch_gptq_dequant(const uint32_t* qweight, const uint32_t* qzeros, con
                             uint32_t group_size, uint32_t num_groups, hipStream_t s) {
   if (in_features == 0 || out_features == 0) return RMLX_OK;
   if (aligned16(qweight) && aligned16(scales) && aligned16(out)) {
-    const dim3 grid(in_features / 8, (out_features / 4 + kThreads - 1) / kThreads);
-    if (grid.y > 65535) return fail(RMLX_INVALID_SHAPE, "gptq_dequant: out_features (%u) too large", out_features);
-    hipLaunchKernelGGL(gptq_dequant_kernel, grid, dim3(kThreads), 0, s, qweight, qzeros, scales, g_idx, out,
-                       out_features, group_size, num_groups);
+    const uint32_t col_blocks = (out_features / 4 + kThreads - 1) / kThreads;
+    const size_t blocks = (size_t)(in_features / 8) * col_blocks;
+    if (blocks > 0x7fffffffull) return fail(RMLX_INVALID_SHAPE, "gptq_dequant: matrix too large");
+    hipLaunchKernelGGL(gptq_dequant_kernel, dim3((unsigned)blocks), dim3(kThreads), 0, s, qweight, qzeros, scales,
+                       g_idx, out, out_features, group_size, num_groups, col_blocks);
   } else {
     const size_t blocks = ((size_t)in_features * out_features + kThreads - 1) / kThreads;
     if (blocks > 0x7fffffffull) return fail(RMLX_INVALID_SHAPE, "gptq_dequant: matrix too large");
