@@ -150,11 +150,18 @@ int32_t run_matmul_plain(const rmlx_qweight* qw, const void* x, int32_t x_dtype,
   const bool can_qmm = can_qmm_lds || can_qmm_rw;
 
   if (kernel == KERNEL_AUTO) {
-    // The GEMV streams the weights once per chunk of 8 rows (from L2 after the first chunk); the GEMM
-    // has a floor of about 15 us on this chip while its grid is small.  Measured crossover:
-    // chunks * N * K <= 6 * 4096 * 4096 (M <= 48 at 4096 x 4096, M <= 16 at 9216 x 4096).
-    const bool small_m = M <= kQmvMaxM ||
-                         (qw->bits == 4 && (uint64_t)((M + 7) / 8) * N * K <= 6ull * 4096 * 4096);
+    // The multi-row GEMV streams the weights once per pass of 8 rows (4-bit; two passes share a workgroup
+    // up to 16 rows) or 16 rows (8-bit); the GEMM splits K over several workgroups per tile while its grid
+    // is small, which puts its floor near 9 us at 4096 x 4096.  Measured crossovers, W = weight bytes:
+    //   4-bit: GEMV up to 8 rows (unless K > 8192, where its k loop is the longer one), up to 16 rows while
+    //          W <= 12 MiB (4096 x 4096 is 8 MiB; at 9216 x 4096 the GEMM wins from 9 rows on);
+    //   8-bit: GEMV up to 16 rows while W <= 48 MiB (4096 x 4096 is 16 MiB; at 12288 x 4096 the GEMM wins).
+    const uint64_t wbytes = (uint64_t)N * K * qw->bits / 8;
+    // Without the register-weights GEMM (K not a multiple of 512) the alternative is the LDS-staged GEMM with
+    // a floor of about 15 us: there the 4-bit GEMV keeps up to passes * W <= 48 MiB.
+    const bool small_m = !can_qmm_rw ? M <= kQmvMaxM || (qw->bits == 4 && (uint64_t)((M + 7) / 8) * wbytes <= (48ull << 20))
+                         : qw->bits == 4 ? (M <= 8 && K <= 8192) || (M <= kQmvMaxM && wbytes <= (12ull << 20))
+                                         : (M <= kQmvMaxM && wbytes <= (48ull << 20));
     if ((can_qmv && small_m) || can_m1) kernel = KERNEL_QMV;
     else if (can_qmm) kernel = KERNEL_QMM;
     else if (can_qmv) kernel = KERNEL_QMV;
@@ -192,7 +199,10 @@ int32_t run_matmul_plain(const rmlx_qweight* qw, const void* x, int32_t x_dtype,
       RMLX_TRY(launch_cast_to_f16(x, x_dtype, static_cast<__half*>(cast.ptr), (size_t)M * K, stream));
       xk = cast.ptr;
     }
-    QmmArgs a{qw->w, qw->s, qw->b, xk, xk_dtype, out, M, N, K, qw->bits, nullptr, 0, epi.kind, epi.ptr, epi.dtype};
+    Scratch partial;  // f32 partial sums when the launch is split over K
+    const size_t partial_bytes = qmm_rw_workspace_bytes(M, N, K, qw->group_size, qw->bits);
+    if (partial_bytes != 0) RMLX_TRY(partial.alloc(partial_bytes, stream));
+    QmmArgs a{qw->w, qw->s, qw->b, xk, xk_dtype, out, M, N, K, qw->bits, partial.ptr, 0, epi.kind, epi.ptr, epi.dtype};
     *epi_done = true;
     return launch_qmm_rw(a, qw->group_size, stream);
   }

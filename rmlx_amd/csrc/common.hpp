@@ -157,6 +157,8 @@ enum { EPI_NONE = 0, EPI_RESIDUAL = 1, EPI_SWIGLU = 2 };
 // out[i] = out[i] + e[i]  /  silu(e[i]) * out[i], in place on f16 out (kernels without a fused epilogue)
 int32_t launch_epilogue(__half* out, int kind, const void* e, int32_t e_dtype, size_t n, hipStream_t s);
 size_t qmm_workspace_bytes(uint32_t M, uint32_t K);
+// split-K partial sums of the register-weights GEMM (0 when the launch is not split); pass the buffer in QmmArgs::workspace
+size_t qmm_rw_workspace_bytes(uint32_t M, uint32_t N, uint32_t K, uint32_t group_size, uint32_t bits);
 bool qmm_supported(uint32_t N, uint32_t K, uint32_t group_size, uint32_t bits);
 int32_t launch_qmm(const QmmArgs& a, hipStream_t s);
 // Register-weights GEMM (qmm_rw.hip): f16 activations only, no workspace.

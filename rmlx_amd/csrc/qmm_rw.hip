@@ -49,6 +49,10 @@ struct RwParams {
   uint32_t tiles_m, tiles_n;
   int32_t epi_kind, epi_dtype;  // fused store epilogue: EPI_RESIDUAL / EPI_SWIGLU with an [M,N] f16 / f32 operand
   const void* epi;
+  // split-K: grid.y = ksplit workgroups per tile, each over K / ksplit; f32 partial sums [ksplit, M, N]
+  // are added up (and the epilogue applied) by splitk_reduce_kernel
+  uint32_t ksplit;
+  float* partial;
 #ifdef QMM_RW_TRACE
   unsigned long long* trace;
 #endif
@@ -144,7 +148,9 @@ __global__ __launch_bounds__(64 * NW) void qmm_rw_kernel(RwParams p) {
     nt = wg / p.tiles_m;
   }
 
-  const uint32_t K = p.K, S = K / kBlockK, G = K / GS;
+  const uint32_t K = p.K, G = K / GS;
+  const uint32_t S = K / kBlockK / p.ksplit;   // iterations of this workgroup
+  const uint32_t it_first = blockIdx.y * S;    // its first 128-wide k block
   const uint32_t row_base = nt * (NW * 16 * NF) + wave * (16 * NF) + n;
 
   const u4* wptr[NF];
@@ -153,9 +159,9 @@ __global__ __launch_bounds__(64 * NW) void qmm_rw_kernel(RwParams p) {
 #pragma unroll
   for (int f = 0; f < NF; ++f) {
     const uint64_t row = row_base + f * 16;
-    wptr[f] = reinterpret_cast<const u4*>(p.w + row * (K * BITS / 32)) + g;
-    sptr[f] = p.s + row * G;
-    bptr[f] = p.b + row * G;
+    wptr[f] = reinterpret_cast<const u4*>(p.w + row * (K * BITS / 32)) + g + (uint64_t)it_first * (4 * WL);
+    sptr[f] = p.s + row * G + it_first * (kBlockK / GS);
+    bptr[f] = p.b + row * G + it_first * (kBlockK / GS);
   }
   // Activation chunk of an iteration: 16*MF rows x 128 k = 16 sixteen-byte segments per row.  Unit
   // q*kThreads + tid -> (row, segment): 16 consecutive lanes read one row's 256 contiguous bytes.
@@ -170,7 +176,7 @@ __global__ __launch_bounds__(64 * NW) void qmm_rw_kernel(RwParams p) {
     const uint32_t unit = q * kThreads + tid, r = unit >> 4, seg = unit & 15;
     uint32_t row = mt * (16 * MF) + r;
     if (row >= p.M) row = p.M - 1;  // rows past M are computed on stale data and never stored
-    xsrc[q] = p.x + (uint64_t)row * K + seg * 8;
+    xsrc[q] = p.x + (uint64_t)row * K + seg * 8 + (uint64_t)it_first * kBlockK;
     const uint32_t j = BITS == 4 ? (seg & 3) : (2 * (seg >> 3) + (seg & 1));
     const uint32_t gq = BITS == 4 ? (seg >> 2) : ((seg >> 1) & 3);
     lds_w[q] = ((r >> 4) * 4 + j) * 64 + gq * 16 + ((r & 15) ^ (4 * j + gq));
@@ -406,6 +412,10 @@ __global__ __launch_bounds__(64 * NW) void qmm_rw_kernel(RwParams p) {
       for (int f = 0; f < NF; ++f) {
         const uint32_t col = nt * (NW * 16 * NF) + wave * (16 * NF) + f * 16 + 4 * g;
         f4 v = acc[i][f];
+        if (p.ksplit > 1) {
+          *reinterpret_cast<f4*>(p.partial + ((uint64_t)blockIdx.y * p.M + m) * p.N + col) = v;
+          continue;
+        }
         if (p.epi_kind != EPI_NONE) {  // residual add / SwiGLU gate in f32, one rounding (quantized.rs:3206-3246)
           f4 e;
           if (p.epi_dtype == RMLX_DTYPE_F32) {
@@ -431,11 +441,35 @@ __global__ __launch_bounds__(64 * NW) void qmm_rw_kernel(RwParams p) {
   RW_MARK_ALL(p, 1);
 }
 
+// out[m, c..c+3] = epilogue(sum over the ksplit partial sums, in split order); one thread per four columns
+__global__ __launch_bounds__(256) void splitk_reduce_kernel(RwParams p) {
+  const size_t i = ((size_t)blockIdx.x * 256 + threadIdx.x) * 4, total = (size_t)p.M * p.N;
+  if (i >= total) return;
+  f4 v = *reinterpret_cast<const f4*>(p.partial + i);
+  for (uint32_t z = 1; z < p.ksplit; ++z) v += *reinterpret_cast<const f4*>(p.partial + z * total + i);
+  if (p.epi_kind != EPI_NONE) {
+    f4 e;
+    if (p.epi_dtype == RMLX_DTYPE_F32) {
+      e = *reinterpret_cast<const f4*>(static_cast<const float*>(p.epi) + i);
+    } else {
+      const u2 eb = *reinterpret_cast<const u2*>(static_cast<const __half*>(p.epi) + i);
+      const uint32_t ex = eb.x, ey = eb.y;
+      const h2 e0 = __builtin_bit_cast(h2, ex), e1 = __builtin_bit_cast(h2, ey);
+      e = (f4){(float)e0[0], (float)e0[1], (float)e1[0], (float)e1[1]};
+    }
+#pragma unroll
+    for (int q = 0; q < 4; ++q) v[q] = p.epi_kind == EPI_RESIDUAL ? v[q] + e[q] : e[q] / (1.0f + __expf(-e[q])) * v[q];
+  }
+  const h2 lo = {(_Float16)v[0], (_Float16)v[1]};
+  const h2 hi = {(_Float16)v[2], (_Float16)v[3]};
+  *reinterpret_cast<u2*>(p.out + i) = (u2){h2bits(lo), h2bits(hi)};
+}
+
 template <int MF, int NF, int BITS, int NW, int GS = 64>
 void launch_rw(RwParams p, bool x_bf16, hipStream_t s) {
   p.tiles_m = (p.M + 16 * MF - 1) / (16 * MF);
   p.tiles_n = p.N / (NW * 16 * NF);
-  const dim3 grid(p.tiles_m * p.tiles_n), block(64 * NW);
+  const dim3 grid(p.tiles_m * p.tiles_n, p.ksplit), block(64 * NW);
   if (x_bf16) hipLaunchKernelGGL((qmm_rw_kernel<MF, NF, BITS, NW, true, GS>), grid, block, 0, s, p);
   else hipLaunchKernelGGL((qmm_rw_kernel<MF, NF, BITS, NW, false, GS>), grid, block, 0, s, p);
 }
@@ -444,7 +478,7 @@ void launch_rw(RwParams p, bool x_bf16, hipStream_t s) {
 
 #ifdef QMM_RW_TRACE
 unsigned long long* g_qmm_rw_trace = nullptr;
-int g_qmm_rw_force_mf = 0, g_qmm_rw_force_nf = 0, g_qmm_rw_force_nw = 4;
+int g_qmm_rw_force_mf = 0, g_qmm_rw_force_nf = 0, g_qmm_rw_force_nw = 4, g_qmm_rw_force_ks = 0;
 #endif
 
 bool qmm_rw_supported(uint32_t N, uint32_t K, uint32_t group_size, uint32_t bits) {
@@ -453,6 +487,51 @@ bool qmm_rw_supported(uint32_t N, uint32_t K, uint32_t group_size, uint32_t bits
 }
 
 
+namespace {
+struct RwPlan { int mf, nf, nw; uint32_t ksplit; };
+
+// Tile choice {MF, NF, NW} (tile rows 16*MF, tile columns 16*NF*NW): least estimated time =
+// rounds of workgroups over the CUs x work per tile / measured relative efficiency of the tile.
+// Split-K: a launch that leaves SIMDs empty is bound by the length of its k loop (every 128-wide k block
+// is a dependent chain of loads, LDS traffic and a barrier); splitting K over 2 or 4 workgroups per tile
+// shortens the loop and fills the SIMDs, at the price of a small reduction kernel.  It stops paying as
+// soon as every SIMD has a wave: the unpacking keeps the SIMDs busy, so more waves only take turns.
+RwPlan plan_rw(uint32_t M, uint32_t N, uint32_t K, uint32_t group_size) {
+  const uint32_t cus = (uint32_t)ctx().num_cus;
+  static const struct { int mf, nf, nw; float eff; } cand[] = {
+      {8, 1, 8, 1.01f}, {4, 2, 8, 1.0f}, {4, 1, 8, 0.93f}, {4, 2, 4, 0.9f}, {2, 2, 4, 0.7f}, {2, 1, 4, 0.55f}, {2, 1, 8, 0.45f}};
+  RwPlan r{2, 1, 4, 1};
+  float best = 0.f;
+  uint32_t best_wgs = 0;
+  for (const auto& c : cand) {
+    const uint32_t bn = 16 * c.nf * c.nw;
+    if (N % bn != 0) continue;
+    // group sizes 32 / 128 are built for two tiles only (64 x 128 and 32 x 64)
+    if (group_size != 64 && !((c.mf == 4 && c.nf == 1 && c.nw == 8) || (c.mf == 2 && c.nf == 1 && c.nw == 4))) continue;
+    const uint32_t wgs = ((M + 16 * c.mf - 1) / (16 * c.mf)) * (N / bn);
+    const float cost = (float)((wgs + cus - 1) / cus) * (float)(c.mf * c.nf * c.nw) / c.eff;
+    if (best == 0.f || cost < best) { best = cost; r.mf = c.mf; r.nf = c.nf; r.nw = c.nw; best_wgs = wgs; }
+  }
+  // time ~ fixed + (k blocks per workgroup) x (block time, which grows once a SIMD holds more than one
+  // wave: the unpacking keeps a SIMD busy) + the reduction pass; measured: 0.33 us per block, 3 us
+  const float waves = (float)(best_wgs * (uint32_t)r.nw), simds = (float)(cus * 4), blocks = (float)(K / kBlockK);
+  float best_t = 0.f;
+  for (uint32_t ks = 1; ks <= 4; ks *= 2) {
+    if (K % (ks * kBlockK * kUnroll) != 0) continue;
+    const float load = waves * (float)ks / simds;
+    const float t = blocks / (float)ks * 0.33f * (load > 1.f ? load : 1.f) + (ks > 1 ? 3.f : 0.f);
+    if (best_t == 0.f || t < best_t - 0.5f) { best_t = t; r.ksplit = ks; }
+  }
+  return r;
+}
+}  // namespace
+
+size_t qmm_rw_workspace_bytes(uint32_t M, uint32_t N, uint32_t K, uint32_t group_size, uint32_t bits) {
+  if (M == 0 || !qmm_rw_supported(N, K, group_size, bits)) return 0;
+  const RwPlan r = plan_rw(M, N, K, group_size);
+  return r.ksplit > 1 ? (size_t)r.ksplit * M * N * sizeof(float) : 0;
+}
+
 int32_t launch_qmm_rw(const QmmArgs& a, uint32_t group_size, hipStream_t s) {
   if (!qmm_rw_supported(a.N, a.K, group_size, a.bits))
     return fail(RMLX_INVALID_SHAPE, "qmm: unsupported shape N=%u K=%u bits=%u group_size=%u", a.N, a.K, a.bits, group_size);
@@ -460,31 +539,19 @@ int32_t launch_qmm_rw(const QmmArgs& a, uint32_t group_size, hipStream_t s) {
   if (a.x_dtype != RMLX_DTYPE_F16 && a.x_dtype != RMLX_DTYPE_BF16)
     return fail(RMLX_RUNTIME_ERROR, "qmm: f32 activations must be cast to f16 first");
   const bool x_bf16 = a.x_dtype == RMLX_DTYPE_BF16;
-
-  // Tile choice {MF, NF, NW} (tile rows 16*MF, tile columns 16*NF*NW): least estimated time =
-  // rounds of workgroups over the CUs x work per tile / measured relative efficiency of the tile.
-  const uint32_t cus = (uint32_t)ctx().num_cus;
-  static const struct { int mf, nf, nw; float eff; } cand[] = {
-      {8, 1, 8, 1.01f}, {4, 2, 8, 1.0f}, {4, 1, 8, 0.93f}, {4, 2, 4, 0.9f}, {2, 2, 4, 0.7f}, {2, 1, 4, 0.55f}, {2, 1, 8, 0.45f}};
-  int mf = 2, nf = 1, nw = 4;
-  float best = 0.f;
-  for (const auto& c : cand) {
-    const uint32_t bn = 16 * c.nf * c.nw;
-    if (a.N % bn != 0) continue;
-    // group sizes 32 / 128 are built for two tiles only (64 x 128 and 32 x 64)
-    if (group_size != 64 && !((c.mf == 4 && c.nf == 1 && c.nw == 8) || (c.mf == 2 && c.nf == 1 && c.nw == 4))) continue;
-    const uint32_t wgs = ((a.M + 16 * c.mf - 1) / (16 * c.mf)) * (a.N / bn);
-    const float cost = (float)((wgs + cus - 1) / cus) * (float)(c.mf * c.nf * c.nw) / c.eff;
-    if (best == 0.f || cost < best) { best = cost; mf = c.mf; nf = c.nf; nw = c.nw; }
-  }
+  RwPlan plan = plan_rw(a.M, a.N, a.K, group_size);
+  if (a.workspace == nullptr) plan.ksplit = 1;  // no room for partial sums: one workgroup per tile
 #ifdef QMM_RW_TRACE
-  if (g_qmm_rw_force_mf) { mf = g_qmm_rw_force_mf; nf = g_qmm_rw_force_nf; nw = g_qmm_rw_force_nw; }
+  if (g_qmm_rw_force_mf) { plan.mf = g_qmm_rw_force_mf; plan.nf = g_qmm_rw_force_nf; plan.nw = g_qmm_rw_force_nw; }
+  if (g_qmm_rw_force_ks) plan.ksplit = (uint32_t)g_qmm_rw_force_ks;
 #endif
+  const int mf = plan.mf, nf = plan.nf, nw = plan.nw;
   RwParams p{};
   p.w = a.w; p.s = a.s; p.b = a.b;
   p.x = static_cast<const __half*>(a.x);
   p.out = a.out; p.M = a.M; p.N = a.N; p.K = a.K;
   p.epi_kind = a.epi_kind; p.epi = a.epi; p.epi_dtype = a.epi_dtype;
+  p.ksplit = plan.ksplit; p.partial = static_cast<float*>(a.workspace);
 #ifdef QMM_RW_TRACE
   p.trace = g_qmm_rw_trace;
 #endif
@@ -505,6 +572,11 @@ int32_t launch_qmm_rw(const QmmArgs& a, uint32_t group_size, hipStream_t s) {
 #undef RW_CASE_GS
 #undef RW_CASE
   RMLX_HIP_CHECK(hipGetLastError());
+  if (p.ksplit > 1) {
+    const size_t quads = (size_t)p.M * p.N / 4;
+    hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned)((quads + 255) / 256)), dim3(256), 0, s, p);
+    RMLX_HIP_CHECK(hipGetLastError());
+  }
   return RMLX_OK;
 }
 

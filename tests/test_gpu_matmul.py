@@ -377,6 +377,33 @@ def test_fused_epilogue_validation(hip):
         ops.qmm_swiglu(xd, qw, DeviceBuffer.from_numpy(np.zeros((8, 64), np.uint32)))
 
 
+@pytest.mark.parametrize("m,n,k,bits,gs,dtype", [(17, 4096, 4096, 4, 64, "f16"), (33, 1024, 4096, 4, 64, "bf16"),
+                                                 (64, 4096, 14336, 4, 64, "f16"), (5, 256, 8192, 8, 64, "f16"),
+                                                 (40, 512, 2048, 8, 128, "f16"), (24, 1536, 1024, 4, 32, "f16"),
+                                                 (100, 192, 1024, 4, 64, "f32"), (16, 64, 512, 4, 64, "f16")])
+def test_qmm_split_k(hip, m, n, k, bits, gs, dtype):
+    """Small grids of the register-weights GEMM split K over 2 or 4 workgroups per tile and add the f32
+    partial sums in a second kernel (the counterpart of the reference's split-K kernel for 32 <= M < 128,
+    quantized.rs:4572-4786, 6927-7103): the split must land on the oracle like the single pass, also
+    with the store epilogues, which then run in the reduction kernel."""
+    from rmlx_amd import ops
+    from rmlx_amd.runtime import DeviceBuffer
+    rng = np.random.default_rng(m + n + k + bits + gs)
+    words, s, b = make_weight(rng, n, k, bits, gs)
+    x = make_x(rng, m, k, dtype)
+    ref = model.qmm(x_as_f64(x, dtype), words, s, b, gs, bits)
+    print(f"split-k M={m} N={n} K={k} bits={bits} gs={gs} {dtype}", flush=True)
+    assert_close(_run(hip, words, s, b, x, bits, gs=gs, dtype=dtype, kernel=2), ref, "qmm")
+    if m > 16:  # the automatic ladder takes the GEMM here, so the epilogue entry points reach the reduction kernel
+        qw = ops.QuantizedWeight.from_numpy(words, s, b, gs, bits)
+        xd = _dev(hip, x, dtype)
+        for edt in (np.float16, np.float32):
+            e = rng.standard_normal((m, n)).astype(edt)
+            ed = DeviceBuffer.from_numpy(e)
+            assert_close(ops.qmm_add_residual(xd, qw, ed).numpy(), ref + e.astype(np.float64), "qmm_add_residual")
+            assert_close(ops.qmm_swiglu(xd, qw, ed).numpy(), model.silu(e.astype(np.float64)) * ref, "qmm_swiglu")
+
+
 @pytest.mark.parametrize("m,n,k", [(13, 9216, 4096), (16, 9216, 4096), (16, 8192, 1536), (8, 16384, 512), (9, 8192, 2048)])
 def test_qmv_paired_tiles(hip, m, n, k):
     """Shapes whose 8-row chunks take two 16-row tiles per wave (grid still covers the CUs)."""
