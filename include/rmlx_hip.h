@@ -149,6 +149,14 @@ int32_t rmlx_hip_qmm_add_residual(const rmlx_qweight* qw, const rmlx_array* x, c
 int32_t rmlx_hip_qmm_swiglu(const rmlx_qweight* qw, const rmlx_array* x, const rmlx_array* gate_result,
                             void* out_f16_dev, size_t out_bytes, rmlx_stream stream);
 
+/* RMSNorm prologue of the reference's Q4 MMA kernel (`has_norm`, function constant 203: quantized.rs:2955-2992, A loader
+ * :3070-3095; no host entry point of the reference sets it): the activations are normalised on the way in,
+ * x'[m,k] = (half(x[m,k]) * half(inv_rms[m])) * norm_weight[k], each product rounded to f16, and out = x' @ dequant(W)^T.
+ * x: [M, in_features] f16 / f32 / bf16; norm_weight: f16 [in_features]; inv_rms: f32 [M] (the caller's 1/rms of each row).
+ * Fused into the single-row GEMV (M <= 2); a separate elementwise pass in front of the other kernels. */
+int32_t rmlx_hip_qmm_norm(const rmlx_qweight* qw, const rmlx_array* x, const rmlx_array* norm_weight,
+                          const rmlx_array* inv_rms, void* out_f16_dev, size_t out_bytes, rmlx_stream stream);
+
 /* Encode `count` batched matmuls back to back on `stream` with no synchronisation in between:
  * the `_into_cb` usage of the reference, which encodes every QMM of a decoder stack into one
  * command buffer (`affine_quantized_matmul_batched_into_cb`, quantized.rs:7797-7802;

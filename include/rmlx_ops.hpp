@@ -217,6 +217,17 @@ inline Array qmm_swiglu(const Array& x, const QuantizedWeight& qw, const Array& 
   return out;
 }
 
+// out = ((x * half(inv_rms[m])) * norm_weight[k]) @ dequant(W)^T: the RMSNorm prologue (`has_norm`) of the
+// reference's MMA kernel (quantized.rs:2955-2992, 3070-3095); norm_weight f16 [K], inv_rms f32 [M]
+inline Array qmm_norm(const Array& x, const QuantizedWeight& qw, const Array& norm_weight, const Array& inv_rms,
+                      const Stream* stream = nullptr) {
+  const size_t m = x.ndim() == 2 ? x.shape()[0] : 0;
+  Array out = Array::uninit({m, qw.out_features}, DType::Float16);
+  const rmlx_array v = x.view(), w = norm_weight.view(), r = inv_rms.view();
+  detail::check(rmlx_hip_qmm_norm(qw.handle(), &v, &w, &r, out.data(), out.nbytes(), raw(stream)));
+  return out;
+}
+
 // out[b] = x[b] @ dequant(W[indices[b]])^T over stacked expert weights
 inline Array gather_qmm(const Array& x, const QuantizedWeight& stacked, const Array& indices, size_t batch,
                         size_t m_per_batch, const Stream* stream = nullptr) {

@@ -94,6 +94,17 @@ def qmm(x, words, scales, biases, group_size, bits):
     return np.asarray(x, dtype=np.float64) @ w.T
 
 
+def norm_rows(x, inv_rms, norm_weight):
+    """x'[m,k] = (half(x[m,k]) * half(inv_rms[m])) * norm_weight[k], each product rounded to f16: the A loader of
+    the reference's Q4 MMA kernel under `has_norm` (crates/rmlx-core/src/ops/quantized.rs:3070-3095).  No host
+    entry point or test of the reference exercises it; pinned in tests/ by what the formula fixes (unit
+    inv_rms and norm_weight leave x unchanged bit for bit, powers of two scale exactly, the result equals
+    qmm of the separately normalised rows) -- numpy's float16 product is the IEEE round-to-nearest-even one."""
+    xh = np.asarray(x).astype(np.float16)
+    rs = np.asarray(inv_rms, dtype=np.float32).astype(np.float16)[:, None]
+    return ((xh * rs).astype(np.float16) * np.asarray(norm_weight, dtype=np.float16)[None, :]).astype(np.float16)
+
+
 def gather_qmm(x, words, scales, biases, indices, group_size, bits=4):
     """out[b] = x[b] @ dequant(W[indices[b]])^T for stacked expert weights [E,N,K*bits/32]
     (crates/rmlx-core/src/ops/quantized.rs:9279-9290, 9300-9368).  x is [batch, M_b, K] or

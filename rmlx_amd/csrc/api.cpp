@@ -116,7 +116,12 @@ constexpr uint32_t kQmvMaxM = 16;
 constexpr uint32_t kM1MaxRows = 2;        // group size 64: rows taken by the single-row kernel (measured: 3 and 4 rows are faster on the matrix unit)
 constexpr uint32_t kM1MaxRowsOther = 16;  // shapes the multi-row GEMV does not take: the alternative is the portable kernel
 
-struct Epilogue { int kind = EPI_NONE; const void* ptr = nullptr; int32_t dtype = RMLX_DTYPE_F16; };
+// What is fused around a matmul: the store epilogue (kind / ptr / dtype) and the RMSNorm prologue
+// (norm_w [K] f16 and inv_rms [M] f32; both null = none).
+struct Epilogue {
+  int kind = EPI_NONE; const void* ptr = nullptr; int32_t dtype = RMLX_DTYPE_F16;
+  const __half* norm_w = nullptr; const float* inv_rms = nullptr;
+};
 
 int32_t run_matmul_plain(const rmlx_qweight* qw, const void* x, int32_t x_dtype, uint32_t M, __half* out,
                          int32_t kernel, hipStream_t stream, const Epilogue& epi, bool* epi_done);
@@ -186,6 +191,19 @@ int32_t run_matmul_plain(const rmlx_qweight* qw, const void* x, int32_t x_dtype,
     return fail(RMLX_NOT_FOUND, "unknown kernel selector %d", kernel);
   }
 
+  // RMSNorm prologue: fused into the single-row GEMV for one or two rows (while it stages the activations);
+  // every other case gets the normalised activations from a pass of its own.
+  const __half* norm_w = epi.norm_w;
+  const float* inv_rms = epi.inv_rms;
+  Scratch normed;
+  if (norm_w != nullptr && !(kernel == KERNEL_QMV && can_m1 && qmv_m1_fuses_norm(M, K, qw->bits))) {
+    RMLX_TRY(normed.alloc((size_t)M * K * sizeof(__half), stream));
+    RMLX_TRY(launch_norm_rows(x, x_dtype, norm_w, inv_rms, M, K, static_cast<__half*>(normed.ptr), stream));
+    x = normed.ptr;
+    x_dtype = RMLX_DTYPE_F16;
+    norm_w = nullptr;
+  }
+
   if (kernel == KERNEL_QMM && can_qmm_rw) {
     // Register-weights GEMM: f16 / bf16 activations straight from the row-major matrix, no workspace
     // (bf16 -> f16 inside the kernel: exact for normal-range values, and f16 weights keep 11
@@ -229,7 +247,7 @@ int32_t run_matmul_plain(const rmlx_qweight* qw, const void* x, int32_t x_dtype,
   if (kernel == KERNEL_QMV && can_m1) {
     *epi_done = true;
     return launch_qmv_m1(qw->w, qw->s, qw->b, static_cast<const __half*>(xk), out, M, N, K, qw->group_size, qw->bits,
-                         epi.kind, epi.ptr, epi.dtype, stream);
+                         epi.kind, epi.ptr, epi.dtype, norm_w, norm_w != nullptr ? inv_rms : nullptr, stream);
   }
   if (kernel == KERNEL_QMV_ROWS) kernel = KERNEL_QMV;
   if (kernel == KERNEL_QMV && qw->bits == 8)
@@ -552,6 +570,34 @@ int32_t qmm_with_epilogue(const char* what, const char* operand, int kind, const
   return finish((hipStream_t)stream);
 }
 }  // namespace
+
+int32_t rmlx_hip_qmm_norm(const rmlx_qweight* qw, const rmlx_array* x, const rmlx_array* norm_weight,
+                          const rmlx_array* inv_rms, void* out_f16_dev, size_t out_bytes, rmlx_stream stream) {
+  RMLX_TRY(require_init());
+  if (qw == nullptr || x == nullptr || norm_weight == nullptr || inv_rms == nullptr)
+    return fail(RMLX_INVALID_SHAPE, "qmm_norm: null argument");
+  RMLX_TRY(check_x_dtype("qmm_norm", x->dtype));
+  if (x->ndim != 2) return fail(RMLX_INVALID_SHAPE, "qmm_norm requires 2D input x, got %dD", x->ndim);
+  if (x->shape[1] != qw->in_features)
+    return fail(RMLX_INVALID_SHAPE, "x.shape[1] (%zu) != in_features (%zu)", x->shape[1], qw->in_features);
+  if (qw->bits != 4 && qw->bits != 8) return fail(RMLX_INVALID_SHAPE, "qmm_norm requires bits==4 or bits==8, got %u", qw->bits);
+  if (qw->n_experts != 1) return fail(RMLX_INVALID_SHAPE, "qmm_norm: weight is a stacked expert weight");
+  if (norm_weight->dtype != RMLX_DTYPE_F16 || numel(norm_weight) != qw->in_features)
+    return fail(RMLX_INVALID_SHAPE, "qmm_norm: norm_weight must be Float16 [%zu], got %s with %zu elements", qw->in_features,
+                dtype_name(norm_weight->dtype), numel(norm_weight));
+  if (inv_rms->dtype != RMLX_DTYPE_F32 || numel(inv_rms) != x->shape[0])
+    return fail(RMLX_INVALID_SHAPE, "qmm_norm: inv_rms must be Float32 [%zu], got %s with %zu elements", x->shape[0],
+                dtype_name(inv_rms->dtype), numel(inv_rms));
+  if (!aligned16(norm_weight->data)) return fail(RMLX_INVALID_SHAPE, "qmm_norm: norm_weight must be 16-byte aligned");
+  uint32_t M;
+  RMLX_TRY(checked_u32(x->shape[0], "M", &M));
+  RMLX_TRY(check_out("qmm_norm", out_bytes, (size_t)M * qw->out_features * 2));
+  Epilogue fuse;
+  fuse.norm_w = static_cast<const __half*>(norm_weight->data);
+  fuse.inv_rms = static_cast<const float*>(inv_rms->data);
+  RMLX_TRY(run_matmul(qw, x->data, x->dtype, M, static_cast<__half*>(out_f16_dev), KERNEL_AUTO, (hipStream_t)stream, fuse));
+  return finish((hipStream_t)stream);
+}
 
 int32_t rmlx_hip_qmm_add_residual(const rmlx_qweight* qw, const rmlx_array* x, const rmlx_array* residual,
                                   void* out_f16_dev, size_t out_bytes, rmlx_stream stream) {

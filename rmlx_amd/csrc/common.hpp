@@ -135,7 +135,11 @@ int32_t launch_qmv_q8(const uint32_t* w, const __half* s, const __half* b, const
 bool qmv_m1_supported(uint32_t N, uint32_t K, uint32_t group_size, uint32_t bits);
 int32_t launch_qmv_m1(const uint32_t* w, const __half* s, const __half* b, const __half* x, __half* out, uint32_t M,
                       uint32_t N, uint32_t K, uint32_t group_size, uint32_t bits, int epi_kind, const void* epi,
-                      int32_t epi_dtype, hipStream_t stream);
+                      int32_t epi_dtype, const __half* norm_w, const float* inv_rms, hipStream_t stream);
+bool qmv_m1_fuses_norm(uint32_t M, uint32_t K, uint32_t bits);
+// dst[m,k] = (half(x[m,k]) * half(inv_rms[m])) * norm_w[k], each product rounded to f16 (the RMSNorm prologue as a separate pass)
+int32_t launch_norm_rows(const void* x, int32_t x_dtype, const __half* norm_w, const float* inv_rms, uint32_t M,
+                         uint32_t K, __half* dst, hipStream_t s);
 // chunk table for gather_qmm: batch b owns rows [b*mpb, (b+1)*mpb) and expert indices[b]
 int32_t launch_build_gather_chunks(const uint32_t* indices, uint32_t batch, uint32_t mpb, uint32_t n_experts,
                                    uint32_t* chunk_tab, hipStream_t s);

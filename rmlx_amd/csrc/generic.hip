@@ -19,6 +19,22 @@ __global__ void cast_to_f16_kernel(const void* src, int src_dtype, __half* dst, 
   }
 }
 
+// RMSNorm prologue as a pass of its own (the kernels without a fused prologue): the reference's A loader
+// computes half(x) * half(inv_rms[row]) * norm_weight[k] in half precision (quantized.rs:3070-3095)
+__global__ void norm_rows_kernel(const void* src, int src_dtype, const __half* __restrict__ norm_w,
+                                 const float* __restrict__ inv_rms, uint32_t K, __half* dst, size_t n) {
+  size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const size_t stride = (size_t)gridDim.x * blockDim.x;
+  for (; i < n; i += stride) {
+    const _Float16 xh = src_dtype == RMLX_DTYPE_F16 ? reinterpret_cast<const _Float16*>(src)[i]
+                        : src_dtype == RMLX_DTYPE_F32 ? (_Float16)reinterpret_cast<const float*>(src)[i]
+                                                      : (_Float16)bf16_to_f32(reinterpret_cast<const uint16_t*>(src)[i]);
+    const _Float16 rs = (_Float16)inv_rms[i / K];
+    const _Float16 scaled = xh * rs;
+    reinterpret_cast<_Float16*>(dst)[i] = scaled * reinterpret_cast<const _Float16*>(norm_w)[i % K];
+  }
+}
+
 __global__ void cast_f16_to_f32_kernel(const __half* src, float* dst, size_t n) {
   size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
   const size_t stride = (size_t)gridDim.x * blockDim.x;
@@ -96,6 +112,17 @@ int32_t launch_cast_to_f16(const void* src, int32_t src_dtype, __half* dst, size
   size_t blocks = (n + 255) / 256;
   if (blocks > 4096) blocks = 4096;
   hipLaunchKernelGGL(cast_to_f16_kernel, dim3((unsigned)blocks), dim3(256), 0, s, src, src_dtype, dst, n);
+  RMLX_HIP_CHECK(hipGetLastError());
+  return RMLX_OK;
+}
+
+int32_t launch_norm_rows(const void* x, int32_t x_dtype, const __half* norm_w, const float* inv_rms, uint32_t M,
+                         uint32_t K, __half* dst, hipStream_t s) {
+  const size_t n = (size_t)M * K;
+  if (n == 0) return RMLX_OK;
+  size_t blocks = (n + 255) / 256;
+  if (blocks > 4096) blocks = 4096;
+  hipLaunchKernelGGL(norm_rows_kernel, dim3((unsigned)blocks), dim3(256), 0, s, x, x_dtype, norm_w, inv_rms, K, dst, n);
   RMLX_HIP_CHECK(hipGetLastError());
   return RMLX_OK;
 }

@@ -46,6 +46,9 @@ struct M1Params {
   uint32_t N, K, M;
   int32_t epi_kind, epi_dtype;  // fused store epilogue: EPI_RESIDUAL / EPI_SWIGLU with an [M,N] f16 / f32 operand
   const void* epi;
+  // fused RMSNorm prologue (null = none): x[m,k] <- (x[m,k] * half(inv_rms[m])) * norm_w[k], each product rounded to f16
+  const __half* norm_w;
+  const float* inv_rms;
 };
 
 __device__ __forceinline__ h2 as_h2(uint32_t v) { return __builtin_bit_cast(h2, v); }
@@ -80,8 +83,12 @@ __device__ __forceinline__ u4 to_pair_order(u4 d) {
 // R = weight rows per wave (1 or 2); NT = non-temporal weight loads (one pass over the weights);
 // MR = activation rows per pass (1, 2 or 4): their registers share the unpacked weights, so a few
 // rows cost one pass over the weights plus 16 dot instructions per row, chunk and lane.
-template <int BITS, int GS, int R, bool NT, int MR>
-__global__ __launch_bounds__(kThreads) void qmv_m1_kernel(M1Params p) {
+// NORM = RMSNorm prologue applied while the activations are staged (kernels of their own: the extra
+// registers would cost the plain kernels occupancy).
+template <int BITS, int GS, int R, bool NT, int MR, bool NORM = false>
+// (8-bit, one row: asking the compiler for eight waves per SIMD changes no register count but the schedule;
+// measured 4-13 % faster.  The 4-bit kernel would spill under that bound and is slower with it.)
+__global__ __launch_bounds__(kThreads, (BITS == 8 && MR == 1 && R == 1) ? 8 : 1) void qmv_m1_kernel(M1Params p) {
   constexpr int kChunkK = 8192 / BITS;         // k values of one wave-wide 16-byte load: 2048 / 1024
   constexpr int kLaneK = kChunkK / 64;         // values per lane and chunk: 32 / 16
   constexpr int kXU = kLaneK / 8;              // 16-byte activation units per lane and chunk: 4 / 2
@@ -119,6 +126,21 @@ __global__ __launch_bounds__(kThreads) void qmv_m1_kernel(M1Params p) {
         xv[m][i] = xg[u < nunits ? u : nunits - 1];
       }
     }
+  }
+  // RMSNorm prologue of the reference's MMA kernel (`has_norm`, quantized.rs:3070-3095) applied while staging
+  auto normalise = [&](int m, uint32_t u, u4 v) {
+    const uint32_t rm = mrow0 + m < p.M ? mrow0 + m : p.M - 1;
+    const _Float16 rs = (_Float16)p.inv_rms[rm];
+    const h8 nw = __builtin_bit_cast(h8, reinterpret_cast<const u4*>(p.norm_w)[u < nunits ? u : nunits - 1]);
+    const h8 scaled = __builtin_bit_cast(h8, v) * (h8){rs, rs, rs, rs, rs, rs, rs, rs};
+    return __builtin_bit_cast(u4, scaled * nw);
+  };
+  if constexpr (NORM) {
+#pragma unroll
+    for (int m = 0; m < MR; ++m)
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        if (i == 0 || nunits > (uint32_t)i * kThreads) xv[m][i] = normalise(m, tid + i * kThreads, xv[m][i]);
   }
   // ... the epilogue operand of the output this lane will write (lane r * MR + m) ...
   const uint32_t out_m = mrow0 + lane % MR, out_n = row0 + lane / MR;
@@ -195,7 +217,8 @@ __global__ __launch_bounds__(kThreads) void qmv_m1_kernel(M1Params p) {
 #pragma unroll
     for (int m = 0; m < MR; ++m) {
       const uint32_t rm = mrow0 + m < p.M ? mrow0 + m : p.M - 1;
-      const u4 v = reinterpret_cast<const u4*>(p.x + (uint64_t)rm * K)[u < nunits ? u : nunits - 1];
+      u4 v = reinterpret_cast<const u4*>(p.x + (uint64_t)rm * K)[u < nunits ? u : nunits - 1];
+      if constexpr (NORM) v = normalise(m, u, v);
       stage_unit(m, u, v);
     }
   }
@@ -301,6 +324,16 @@ template <int BITS, int R, bool NT, int MR>
 void launch_r(const M1Params& p, uint32_t group_size, hipStream_t s) {
   const dim3 grid(p.N / (kWaves * R), (p.M + MR - 1) / MR), block(kThreads);
   const size_t lds = (size_t)MR * lds_per_row<BITS>(p.K);
+  if constexpr (NT && MR <= 2) {  // the prologue is fused for one or two rows in one pass
+    if (p.norm_w != nullptr) {
+      switch (group_size) {
+        case 32: hipLaunchKernelGGL((qmv_m1_kernel<BITS, 32, R, NT, MR, true>), grid, block, lds, s, p); break;
+        case 64: hipLaunchKernelGGL((qmv_m1_kernel<BITS, 64, R, NT, MR, true>), grid, block, lds, s, p); break;
+        default: hipLaunchKernelGGL((qmv_m1_kernel<BITS, 128, R, NT, MR, true>), grid, block, lds, s, p); break;
+      }
+      return;
+    }
+  }
   switch (group_size) {
     case 32: hipLaunchKernelGGL((qmv_m1_kernel<BITS, 32, R, NT, MR>), grid, block, lds, s, p); break;
     case 64: hipLaunchKernelGGL((qmv_m1_kernel<BITS, 64, R, NT, MR>), grid, block, lds, s, p); break;
@@ -320,8 +353,10 @@ void launch_bits(const M1Params& p, uint32_t group_size, hipStream_t s) {
   } else if (mr == 2) {
     if (one_pass) launch_r<BITS, 1, true, 2>(p, group_size, s); else launch_r<BITS, 1, false, 2>(p, group_size, s);
   } else {
-    // two weight rows per wave for long rows (more bytes in flight per wave), else one
-    const bool two = p.K >= 12288 && p.N % (kWaves * 2) == 0;
+    // two weight rows per wave for long rows (more bytes in flight per wave) and, with 4-bit weights, for
+    // tall matrices (the activation registers read from LDS serve both rows; measured 3-9 % from N = 12288
+    // on; the 8-bit kernel reads half as many activations per weight byte and is faster with one), else one
+    const bool two = (p.K >= 12288 || (BITS == 4 && p.N >= 12288)) && p.N % (kWaves * 2) == 0;
     if (one_pass) {
       if (two) launch_r<BITS, 2, true, 1>(p, group_size, s); else launch_r<BITS, 1, true, 1>(p, group_size, s);
     } else {
@@ -340,14 +375,21 @@ bool qmv_m1_supported(uint32_t N, uint32_t K, uint32_t group_size, uint32_t bits
   return (bits == 4 ? lds_per_row<4>(K) : lds_per_row<8>(K)) <= 65536;
 }
 
+// The RMSNorm prologue is fused when all rows (at most two) share one pass over the weights.
+bool qmv_m1_fuses_norm(uint32_t M, uint32_t K, uint32_t bits) {
+  return M >= 1 && M <= 2 && (size_t)M * (bits == 4 ? lds_per_row<4>(K) : lds_per_row<8>(K)) <= 65536;
+}
+
 int32_t launch_qmv_m1(const uint32_t* w, const __half* s, const __half* b, const __half* x, __half* out, uint32_t M,
                       uint32_t N, uint32_t K, uint32_t group_size, uint32_t bits, int epi_kind, const void* epi,
-                      int32_t epi_dtype, hipStream_t stream) {
+                      int32_t epi_dtype, const __half* norm_w, const float* inv_rms, hipStream_t stream) {
   if (!qmv_m1_supported(N, K, group_size, bits))
     return fail(RMLX_INVALID_SHAPE, "qmv_m1: unsupported shape N=%u K=%u bits=%u group_size=%u", N, K, bits, group_size);
   if (M == 0) return RMLX_OK;
   if (M > 65535) return fail(RMLX_INVALID_SHAPE, "qmv_m1: at most 65535 rows per launch (M=%u)", M);
-  M1Params p{w, s, b, x, out, N, K, M, epi_kind, epi_dtype, epi};
+  if (norm_w != nullptr && !qmv_m1_fuses_norm(M, K, bits))
+    return fail(RMLX_RUNTIME_ERROR, "qmv_m1: the RMSNorm prologue is fused for at most two rows in one pass (M=%u K=%u)", M, K);
+  M1Params p{w, s, b, x, out, N, K, M, epi_kind, epi_dtype, epi, norm_w, inv_rms};
   if (bits == 4) launch_bits<4>(p, group_size, stream);
   else launch_bits<8>(p, group_size, stream);
   RMLX_HIP_CHECK(hipGetLastError());

@@ -85,6 +85,17 @@ def qmm_swiglu(x, qw, gate_result, stream=None):
     return out
 
 
+def qmm_norm(x, qw, norm_weight, inv_rms, stream=None, out=None):
+    """QMM with the RMSNorm prologue of the reference's MMA kernel (`has_norm`, quantized.rs:2955-2992, 3070-3095):
+    x'[m,k] = (half(x[m,k]) * half(inv_rms[m])) * norm_weight[k]; norm_weight f16 [K], inv_rms f32 [M]; f16 out."""
+    if out is None:
+        out = DeviceBuffer((x.shape[0] if len(x.shape) == 2 else 0, qw.out_features), F16)
+    a, w, r = x.array(), norm_weight.array(), inv_rms.array()
+    rt.check(rt.lib().rmlx_hip_qmm_norm(qw.handle, ctypes.byref(a), ctypes.byref(w), ctypes.byref(r), out.ptr, out.nbytes,
+                                        _h(stream)))
+    return out
+
+
 def qmm_encode_many(qws, x, outs, count, stream=None, kernel=rt.KERNEL_AUTO):
     """Encode `count` matmuls back to back (weights and outputs are cycled) -- see rmlx_hip_qmm_encode_many."""
     qarr = (ctypes.c_void_p * len(qws))(*[q.handle for q in qws])

@@ -404,6 +404,59 @@ def test_qmm_split_k(hip, m, n, k, bits, gs, dtype):
             assert_close(ops.qmm_swiglu(xd, qw, ed).numpy(), model.silu(e.astype(np.float64)) * ref, "qmm_swiglu")
 
 
+@pytest.mark.parametrize("m,n,k,bits,gs,dtype", [(1, 4096, 4096, 4, 64, "f16"), (2, 1024, 11008, 4, 64, "f16"),
+                                                 (1, 512, 18944, 4, 64, "f16"), (1, 256, 2048, 8, 32, "f32"),
+                                                 (2, 768, 1024, 8, 128, "bf16"), (5, 1024, 4096, 4, 64, "f16"),
+                                                 (40, 512, 2048, 4, 64, "bf16"), (3, 24, 96, 4, 32, "f16")])
+def test_qmm_norm_prologue(hip, m, n, k, bits, gs, dtype):
+    """RMSNorm prologue (`has_norm` of the reference's MMA kernel, quantized.rs:3070-3095): fused into the
+    single-row GEMV, a pass of its own in front of the other kernels.  Checked against the oracle, and bit
+    for bit against the plain matmul of rows normalised on the host with the same f16 roundings."""
+    from rmlx_amd import ops
+    from rmlx_amd.runtime import DeviceBuffer
+    rng = np.random.default_rng(m + n + k + bits)
+    words, s, b = make_weight(rng, n, k, bits, gs)
+    x = make_x(rng, m, k, dtype)
+    nw = rng.uniform(0.5, 1.5, size=k).astype(np.float16)
+    inv_rms = rng.uniform(0.3, 3.0, size=m).astype(np.float32)
+    xn = model.norm_rows(x_as_f64(x, dtype), inv_rms, nw)
+    ref = model.qmm(xn.astype(np.float64), words, s, b, gs, bits)
+    qw = ops.QuantizedWeight.from_numpy(words, s, b, gs, bits)
+    print(f"qmm_norm M={m} N={n} K={k} bits={bits} gs={gs} {dtype}", flush=True)
+    got = ops.qmm_norm(_dev(hip, x, dtype), qw, DeviceBuffer.from_numpy(nw), DeviceBuffer.from_numpy(inv_rms)).numpy()
+    assert_close(got, ref, "qmm_norm")
+    plain = ops.affine_quantized_matmul_batched(DeviceBuffer.from_numpy(xn), qw).numpy()
+    assert np.array_equal(got, plain)
+
+
+def test_qmm_norm_identity_scaling_and_validation(hip):
+    from rmlx_amd import ops
+    from rmlx_amd.runtime import DeviceBuffer
+    rng = np.random.default_rng(8)
+    n, k = 256, 1024
+    words, s, b = make_weight(rng, n, k, 4)
+    qw = ops.QuantizedWeight.from_numpy(words, s, b, 64, 4)
+    for m in (1, 6):
+        x = make_x(rng, m, k)
+        xd = DeviceBuffer.from_numpy(x)
+        plain = ops.affine_quantized_matmul_batched(xd, qw).numpy()
+        ones_w, ones_r = DeviceBuffer.from_numpy(np.ones(k, np.float16)), DeviceBuffer.from_numpy(np.ones(m, np.float32))
+        assert np.array_equal(ops.qmm_norm(xd, qw, ones_w, ones_r).numpy(), plain)
+        # a power of two per row scales the activations, hence the f32 sums and the f16 results, exactly
+        twos = DeviceBuffer.from_numpy(np.full(m, 2.0, np.float32))
+        assert np.array_equal(ops.qmm_norm(xd, qw, ones_w, twos).numpy(), (plain.astype(np.float32) * 2).astype(np.float16))
+    xd = DeviceBuffer.from_numpy(make_x(rng, 2, k))
+    w16, r32 = DeviceBuffer.from_numpy(np.ones(k, np.float16)), DeviceBuffer.from_numpy(np.ones(2, np.float32))
+    with pytest.raises(ops.KernelError, match=r"norm_weight must be Float16 \[1024\]"):
+        ops.qmm_norm(xd, qw, DeviceBuffer.from_numpy(np.ones(k, np.float32)), r32)
+    with pytest.raises(ops.KernelError, match=r"norm_weight must be Float16 \[1024\]"):
+        ops.qmm_norm(xd, qw, DeviceBuffer.from_numpy(np.ones(k - 8, np.float16)), r32)
+    with pytest.raises(ops.KernelError, match=r"inv_rms must be Float32 \[2\]"):
+        ops.qmm_norm(xd, qw, w16, DeviceBuffer.from_numpy(np.ones(3, np.float32)))
+    with pytest.raises(ops.KernelError, match=r"inv_rms must be Float32 \[2\]"):
+        ops.qmm_norm(xd, qw, w16, DeviceBuffer.from_numpy(np.ones(2, np.float16)))
+
+
 @pytest.mark.parametrize("m,n,k", [(13, 9216, 4096), (16, 9216, 4096), (16, 8192, 1536), (8, 16384, 512), (9, 8192, 2048)])
 def test_qmv_paired_tiles(hip, m, n, k):
     """Shapes whose 8-row chunks take two 16-row tiles per wave (grid still covers the CUs)."""
