@@ -130,6 +130,11 @@ static int run(const std::string& dir) {
   store(dir + "/out_residual.bin", q::qmm_add_residual(x, *qw, side));
   store(dir + "/out_swiglu.bin", q::qmm_swiglu(x, *qw, side));
   {
+    Array norm_weight = load(dir + "/norm_weight.bin", {k}, DType::Float16);
+    Array inv_rms = load(dir + "/inv_rms.bin", {m}, DType::Float32);
+    store(dir + "/out_norm.bin", q::qmm_norm(x, *qw, norm_weight, inv_rms));
+  }
+  {
     rmlx::Stream stream;  // the enqueue-only twin, then one synchronisation
     Array bias = load(dir + "/bias.bin", {n}, DType::Float16);
     rmlx::nn::QuantizedLinear lin(qw, bias.buffer());

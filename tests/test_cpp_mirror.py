@@ -26,7 +26,7 @@ def test_mirror_compiles_and_validates_without_a_gpu():
 def test_mirror_names_follow_the_reference():
     text = open(os.path.join(ROOT, "include", "rmlx_ops.hpp")).read()
     for name in ["class KernelError", "InvalidShape", "NotFound", "class QuantizedWeight", "affine_quantized_matmul(",
-                 "affine_quantized_matmul_batched(", "qmm_add_residual(", "qmm_swiglu(", "gather_qmm(", "gpu_topk_route(",
+                 "affine_quantized_matmul_batched(", "qmm_add_residual(", "qmm_swiglu(", "qmm_norm(", "awq_dequant(", "gptq_dequant(", "gather_qmm(", "gpu_topk_route(",
                  "struct TopkRouteResult", "expert_indices", "expert_weights", "expert_counts", "dispatch_offsets",
                  "class QuantizedLinear", "class ExpertGroup", "grouped_forward(", "forward_grouped("]:
         assert name in text, name
@@ -50,6 +50,8 @@ def test_mirror_matches_oracle(tmp_path, bits, gs, M):
     x = make_x(rng, M, K)
     side = rng.standard_normal((M, N)).astype(np.float32)
     bias = rng.standard_normal(N).astype(np.float16)
+    norm_weight = rng.uniform(0.5, 1.5, size=K).astype(np.float16)
+    inv_rms = rng.uniform(0.3, 3.0, size=M).astype(np.float32)
     experts = {"gate": make_weight(rng, I, K, 4, 64, lead=(E,)), "up": make_weight(rng, I, K, 4, 64, lead=(E,)),
                "down": make_weight(rng, K, I, 4, 64, lead=(E,))}
     xt = make_x(rng, T, K)
@@ -58,7 +60,7 @@ def test_mirror_matches_oracle(tmp_path, bits, gs, M):
     for stem, trip in [("dense", dense)] + list(experts.items()):
         for suffix, a in zip("wsb", trip):
             put(f"{stem}_{suffix}.bin", a)
-    for name, a in [("x.bin", x), ("side.bin", side), ("bias.bin", bias), ("xt.bin", xt), ("logits.bin", logits),
+    for name, a in [("x.bin", x), ("side.bin", side), ("bias.bin", bias), ("norm_weight.bin", norm_weight), ("inv_rms.bin", inv_rms), ("xt.bin", xt), ("logits.bin", logits),
                     ("pick.bin", pick)]:
         put(name, a)
     # the expert weights are always Q4 / group 64; only the dense weight varies
@@ -73,6 +75,8 @@ def test_mirror_matches_oracle(tmp_path, bits, gs, M):
     assert_close(get("out_residual.bin", np.float16, (M, N)), ref + side, "qmm_add_residual")
     assert_close(get("out_swiglu.bin", np.float16, (M, N)), model.silu(side) * ref, "qmm_swiglu")
     assert_close(get("out_linear.bin", np.float16, (M, N)), ref + bias.astype(np.float64), "QuantizedLinear")
+    normed = model.norm_rows(x, inv_rms, norm_weight).astype(np.float64)
+    assert_close(get("out_norm.bin", np.float16, (M, N)), model.qmm(normed, *dense, gs, bits), "qmm_norm")
 
     g = experts["gate"]
     assert_close(get("out_gather.bin", np.float16, (T, 1, I)),
