@@ -50,6 +50,10 @@ DeviceCtx& ctx() {
 
 int32_t require_init() {
   if (!ctx().ready) return fail(RMLX_RUNTIME_ERROR, "rmlx_hip_init() has not been called (no GPU context)");
+  // The current device is a per-thread setting of the runtime: a thread other than the one that called
+  // rmlx_hip_init starts on device 0.
+  int cur = -1;
+  if (hipGetDevice(&cur) == hipSuccess && cur != ctx().device) RMLX_HIP_CHECK(hipSetDevice(ctx().device));
   return RMLX_OK;
 }
 
