@@ -912,10 +912,16 @@ int32_t rmlx_hip_expert_group_grouped_forward(const rmlx_qweight* gate, const rm
   return finish(s);
 }
 
-int32_t rmlx_hip_moe_forward_grouped(const rmlx_qweight* gate, const rmlx_qweight* up, const rmlx_qweight* down,
-                                     const rmlx_array* x, const uint32_t* expert_indices_dev,
-                                     const float* expert_weights_dev, size_t top_k, void* out_f16_dev, size_t out_bytes,
-                                     rmlx_stream stream) {
+}  // extern "C"
+
+namespace {
+// Routing fused in front of the grouping (decode-sized batches): f32 logits [T, E], optional f32 bias [E];
+// the picks and their weights are written to idx_out / w_out.
+struct FusedRoute { const float* logits; const float* bias; uint32_t* idx_out; float* w_out; };
+
+int32_t moe_grouped_impl(const rmlx_qweight* gate, const rmlx_qweight* up, const rmlx_qweight* down,
+                         const rmlx_array* x, const uint32_t* expert_indices_dev, const float* expert_weights_dev,
+                         size_t top_k, void* out_f16_dev, size_t out_bytes, rmlx_stream stream, const FusedRoute* route) {
   RMLX_TRY(require_init());
   ExpertShapes sh;
   RMLX_TRY(check_expert_weights("MoeLayer", gate, up, down, &sh));
@@ -950,7 +956,11 @@ int32_t rmlx_hip_moe_forward_grouped(const rmlx_qweight* gate, const rmlx_qweigh
   uint32_t* inv = sorted_tok + A;
   uint32_t* chunk_tab = inv + A;
   uint32_t* n_chunks = chunk_tab + 3 * (size_t)max_chunks;
-  RMLX_TRY(launch_moe_sort(expert_indices_dev, A, sh.E, (uint32_t)top_k, sorted, sorted_tok, inv, nullptr, nullptr, chunk_tab, n_chunks, s));
+  if (route != nullptr)
+    RMLX_TRY(launch_route_sort_small(route->logits, route->bias, T32, sh.E, (uint32_t)top_k, 1, route->idx_out, route->w_out,
+                                     sorted, sorted_tok, inv, chunk_tab, n_chunks, s));
+  else
+    RMLX_TRY(launch_moe_sort(expert_indices_dev, A, sh.E, (uint32_t)top_k, sorted, sorted_tok, inv, nullptr, nullptr, chunk_tab, n_chunks, s));
   RMLX_TRY(h.alloc((size_t)A * sh.I * 2, s));
   RMLX_TRY(y.alloc((size_t)A * sh.D * 4, s));
   RMLX_TRY(run_expert_ffn(gate, up, down, sh, xk, sorted_tok, chunk_tab, n_chunks, max_chunks,
@@ -958,6 +968,17 @@ int32_t rmlx_hip_moe_forward_grouped(const rmlx_qweight* gate, const rmlx_qweigh
   RMLX_TRY(launch_moe_combine(static_cast<const float*>(y.ptr), inv, expert_weights_dev, T32, (uint32_t)top_k, sh.D,
                               static_cast<__half*>(out_f16_dev), s));
   return finish(s);
+}
+}  // namespace
+
+extern "C" {
+
+int32_t rmlx_hip_moe_forward_grouped(const rmlx_qweight* gate, const rmlx_qweight* up, const rmlx_qweight* down,
+                                     const rmlx_array* x, const uint32_t* expert_indices_dev,
+                                     const float* expert_weights_dev, size_t top_k, void* out_f16_dev, size_t out_bytes,
+                                     rmlx_stream stream) {
+  return moe_grouped_impl(gate, up, down, x, expert_indices_dev, expert_weights_dev, top_k, out_f16_dev, out_bytes, stream,
+                          nullptr);
 }
 
 int32_t rmlx_hip_moe_forward(const rmlx_qweight* gate, const rmlx_qweight* up, const rmlx_qweight* down,
@@ -977,6 +998,15 @@ int32_t rmlx_hip_moe_forward(const rmlx_qweight* gate, const rmlx_qweight* up, c
   RMLX_TRY(route.alloc(T * top_k * 8 + 16, s));
   uint32_t* idx = static_cast<uint32_t*>(route.ptr);
   float* wts = reinterpret_cast<float*>(idx + T * top_k);
+  // Decode-sized batches with f32 logits: routing and grouping share one launch.
+  if (gate != nullptr && gate_logits->dtype == RMLX_DTYPE_F32 && gate_logits->data != nullptr && top_k <= gate->n_experts &&
+      (expert_bias == nullptr || (expert_bias->dtype == RMLX_DTYPE_F32 && expert_bias->ndim == 1 &&
+                                  expert_bias->shape[0] == gate->n_experts && expert_bias->data != nullptr)) &&
+      T <= 8 && route_sort_fusable((uint32_t)T, (uint32_t)gate->n_experts, (uint32_t)top_k)) {
+    const FusedRoute fr{static_cast<const float*>(gate_logits->data),
+                        expert_bias != nullptr ? static_cast<const float*>(expert_bias->data) : nullptr, idx, wts};
+    return moe_grouped_impl(gate, up, down, x, idx, wts, top_k, out_f16_dev, out_bytes, stream, &fr);
+  }
   // Asynchronous inner calls need a real stream handle: the null stream means "synchronous".
   RMLX_TRY(rmlx_hip_topk_route(gate_logits, top_k, expert_bias, 1, idx, wts, nullptr, nullptr, stream));
   RMLX_TRY(rmlx_hip_moe_forward_grouped(gate, up, down, x, idx, wts, top_k, out_f16_dev, out_bytes, stream));

@@ -179,6 +179,11 @@ int32_t launch_topk_route(const float* logits, const float* bias, uint32_t T, ui
 int32_t launch_moe_sort(const uint32_t* idx, uint32_t n_assign, uint32_t E, uint32_t top_k, uint32_t* sorted,
                         uint32_t* sorted_tok, uint32_t* inv, uint32_t* counts, uint32_t* offsets,
                         uint32_t* chunk_tab, uint32_t* n_chunks, hipStream_t s);
+// Decode-sized batches (at most 8 tokens, 64 assignments): routing and grouping in one launch.
+bool route_sort_fusable(uint32_t T, uint32_t E, uint32_t K);
+int32_t launch_route_sort_small(const float* logits, const float* bias, uint32_t T, uint32_t E, uint32_t K,
+                                int renorm, uint32_t* idx, float* w, uint32_t* sorted, uint32_t* sorted_tok,
+                                uint32_t* inv, uint32_t* chunk_tab, uint32_t* n_chunks, hipStream_t s);
 int32_t launch_index_gather(const __half* src, uint32_t d, const uint32_t* idx, uint32_t n, uint32_t src_rows,
                             __half* dst, hipStream_t s);
 int32_t launch_scatter_weighted_add(const __half* src, uint32_t n, uint32_t d, const uint32_t* tok,

@@ -76,12 +76,11 @@ __device__ __forceinline__ void wave_key_max(uint32_t& hi, uint32_t& lo) {
 // logit with ties broken towards the lower expert index, which is the order of the softmax
 // values the reference ranks (exp is monotonic), made independent of the exp implementation.
 // A round's winner is the wave maximum of the key (order-preserving bits of the logit, ~index).
-__global__ __launch_bounds__(64) void topk_route_kernel(const float* __restrict__ logits,
-                                                        const float* __restrict__ bias, uint32_t E,
-                                                        uint32_t K, int renorm, uint32_t* __restrict__ out_idx,
-                                                        float* __restrict__ out_w) {
-  const uint32_t row = blockIdx.x;
-  const uint32_t lane = threadIdx.x;
+// (`lds_idx`: optional copy of the picks in workgroup memory, for a sort fused behind the routing)
+__device__ __forceinline__ void route_token(const float* __restrict__ logits, const float* __restrict__ bias,
+                                            uint32_t E, uint32_t K, int renorm, uint32_t* __restrict__ out_idx,
+                                            float* __restrict__ out_w, uint32_t row, uint32_t lane,
+                                            uint32_t* lds_idx) {
   const float NEG_INF = -__builtin_inff();
   float v[4], sm[4];
   bool taken[4];
@@ -150,8 +149,16 @@ __global__ __launch_bounds__(64) void topk_route_kernel(const float* __restrict_
     for (uint32_t k = 0; k < K; ++k) {
       out_idx[(size_t)row * K + k] = isel[k];
       out_w[(size_t)row * K + k] = wsel[k] * scale;
+      if (lds_idx != nullptr) lds_idx[row * K + k] = isel[k];
     }
   }
+}
+
+__global__ __launch_bounds__(64) void topk_route_kernel(const float* __restrict__ logits,
+                                                        const float* __restrict__ bias, uint32_t E,
+                                                        uint32_t K, int renorm, uint32_t* __restrict__ out_idx,
+                                                        float* __restrict__ out_w) {
+  route_token(logits, bias, E, K, renorm, out_idx, out_w, blockIdx.x, threadIdx.x, nullptr);
 }
 
 // ---- histogram + scan + stable counting sort, one workgroup --------------------------------
@@ -257,15 +264,11 @@ __global__ __launch_bounds__(1024) void moe_sort_kernel(const uint32_t* __restri
 
 // At most 64 assignments (decode-sized batches): one wave, no barriers.  Lane i owns assignment i; ranks,
 // offsets and chunk positions are counted with readlane loops over the other lanes.  Same outputs as above.
-__global__ __launch_bounds__(64) void moe_sort_small_kernel(const uint32_t* __restrict__ idx, uint32_t n_assign,
-                                                            uint32_t E, uint32_t top_k, uint32_t* __restrict__ sorted,
-                                                            uint32_t* __restrict__ sorted_tok,
-                                                            uint32_t* __restrict__ inv, uint32_t* __restrict__ counts,
-                                                            uint32_t* __restrict__ offsets,
-                                                            uint32_t* __restrict__ chunk_tab,
-                                                            uint32_t* __restrict__ n_chunks) {
-  const uint32_t lane = threadIdx.x;
-  const uint32_t e = lane < n_assign ? idx[lane] : 0xFFFFFFFFu;
+__device__ __forceinline__ void sort_small(uint32_t lane, uint32_t e, uint32_t E, uint32_t top_k,
+                                           uint32_t* __restrict__ sorted, uint32_t* __restrict__ sorted_tok,
+                                           uint32_t* __restrict__ inv, uint32_t* __restrict__ counts,
+                                           uint32_t* __restrict__ offsets, uint32_t* __restrict__ chunk_tab,
+                                           uint32_t* __restrict__ n_chunks) {
   const bool valid = e < E;
   uint32_t rank = 0, same = 0, less = 0, n_valid = 0;
   for (int j = 0; j < 64; ++j) {
@@ -314,6 +317,37 @@ __global__ __launch_bounds__(64) void moe_sort_small_kernel(const uint32_t* __re
     }
     if (lane == 0 && offsets != nullptr) offsets[E] = n_valid;
   }
+}
+
+__global__ __launch_bounds__(64) void moe_sort_small_kernel(const uint32_t* __restrict__ idx, uint32_t n_assign,
+                                                            uint32_t E, uint32_t top_k, uint32_t* __restrict__ sorted,
+                                                            uint32_t* __restrict__ sorted_tok,
+                                                            uint32_t* __restrict__ inv, uint32_t* __restrict__ counts,
+                                                            uint32_t* __restrict__ offsets,
+                                                            uint32_t* __restrict__ chunk_tab,
+                                                            uint32_t* __restrict__ n_chunks) {
+  const uint32_t lane = threadIdx.x;
+  sort_small(lane, lane < n_assign ? idx[lane] : 0xFFFFFFFFu, E, top_k, sorted, sorted_tok, inv, counts, offsets,
+             chunk_tab, n_chunks);
+}
+
+// Routing and grouping of a decode-sized batch in one launch: at most 8 tokens and 64 assignments.  Wave t
+// routes token t and leaves its picks in workgroup memory; after the barrier wave 0 sorts them.
+__global__ __launch_bounds__(512) void route_sort_small_kernel(const float* __restrict__ logits,
+                                                               const float* __restrict__ bias, uint32_t T, uint32_t E,
+                                                               uint32_t K, int renorm, uint32_t* __restrict__ out_idx,
+                                                               float* __restrict__ out_w, uint32_t* __restrict__ sorted,
+                                                               uint32_t* __restrict__ sorted_tok,
+                                                               uint32_t* __restrict__ inv,
+                                                               uint32_t* __restrict__ chunk_tab,
+                                                               uint32_t* __restrict__ n_chunks) {
+  __shared__ uint32_t picks[64];
+  const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  if (wave < T) route_token(logits, bias, E, K, renorm, out_idx, out_w, wave, lane, picks);
+  __syncthreads();
+  if (wave == 0)
+    sort_small(lane, lane < T * K ? picks[lane] : 0xFFFFFFFFu, E, K, sorted, sorted_tok, inv, nullptr, nullptr,
+               chunk_tab, n_chunks);
 }
 
 __global__ void index_gather_kernel(const __half* __restrict__ src, uint32_t d, const uint32_t* __restrict__ idx,
@@ -400,6 +434,20 @@ int32_t launch_topk_route(const float* logits, const float* bias, uint32_t T, ui
                        (uint32_t*)nullptr);
     RMLX_HIP_CHECK(hipGetLastError());
   }
+  return RMLX_OK;
+}
+
+bool route_sort_fusable(uint32_t T, uint32_t E, uint32_t K) {
+  return T >= 1 && T <= 8 && T * K <= 64 && E <= 256 && K >= 1 && K <= 8;
+}
+
+int32_t launch_route_sort_small(const float* logits, const float* bias, uint32_t T, uint32_t E, uint32_t K,
+                                int renorm, uint32_t* idx, float* w, uint32_t* sorted, uint32_t* sorted_tok,
+                                uint32_t* inv, uint32_t* chunk_tab, uint32_t* n_chunks, hipStream_t s) {
+  if (!route_sort_fusable(T, E, K)) return fail(RMLX_RUNTIME_ERROR, "route_sort_small: T=%u E=%u K=%u not supported", T, E, K);
+  hipLaunchKernelGGL(route_sort_small_kernel, dim3(1), dim3(64 * T), 0, s, logits, bias, T, E, K, renorm, idx, w, sorted,
+                     sorted_tok, inv, chunk_tab, n_chunks);
+  RMLX_HIP_CHECK(hipGetLastError());
   return RMLX_OK;
 }
 

@@ -253,6 +253,32 @@ def _experts(rng, E, D, I, fused):
     return gate, up, down, gate_h, up_h, down_h
 
 
+@pytest.mark.parametrize("T,E,K", [(1, 128, 8), (8, 128, 8), (7, 200, 3), (8, 256, 8), (3, 5, 5), (9, 128, 7)])
+def test_moe_forward_routes_like_the_two_step_path(hip, T, E, K):
+    """Up to 8 tokens / 64 assignments with f32 logits, routing and grouping share one launch: the result must
+    equal, bit for bit, routing first and calling the grouped block with its outputs -- with and without an
+    expert bias, and also for an f16 bias (which takes the two-step path inside)."""
+    from rmlx_amd import ops
+    from rmlx_amd.runtime import DeviceBuffer
+    rng = np.random.default_rng(T * 31 + E + K)
+    D, I = 512, 512
+    gate, up, down, gh, uh, dh = _experts(rng, E, D, I, False)
+    xd = DeviceBuffer.from_numpy(make_x(rng, T, D))
+    logits = rng.standard_normal((T, E)).astype(np.float32)
+    logits[0, : min(E, 3)] = 1.5  # ties go to the lower index on both paths
+    ld = DeviceBuffer.from_numpy(logits)
+    for bias in (None, rng.standard_normal(E).astype(np.float32), rng.standard_normal(E).astype(np.float16)):
+        bd = DeviceBuffer.from_numpy(bias) if bias is not None else None
+        print(f"moe route T={T} E={E} K={K} bias={None if bias is None else bias.dtype}", flush=True)
+        one = ops.moe_forward(gh, uh, dh, xd, ld, K, expert_bias=bd).numpy()
+        r = ops.gpu_topk_route(ld, K, expert_bias=bd)
+        two = ops.moe_forward_grouped(gh, uh, dh, xd, r.expert_indices, r.expert_weights, K).numpy()
+        assert np.array_equal(one, two)
+        idx, w, _, _ = model.topk_route(logits, K, bias=None if bias is None else bias.astype(np.float32))
+        assert np.array_equal(r.expert_indices.numpy(), idx)
+        assert_close(one, model.moe_forward(xd.numpy(), idx, w, gate, up, down, 64, K), "moe_forward")
+
+
 @pytest.mark.parametrize("fused", [False, True])
 @pytest.mark.parametrize("T,E,K,D,I", [(1, 4, 2, 512, 512), (9, 8, 2, 1024, 512), (40, 6, 3, 512, 1536), (64, 4, 4, 512, 512)])
 def test_moe_forward_small(hip, fused, T, E, K, D, I):
