@@ -108,8 +108,9 @@ __device__ __forceinline__ void route_token(const float* __restrict__ logits, co
 #pragma unroll
   for (int j = 0; j < 4; ++j) sm[j] *= inv;
 
-  float wsel[8];
-  uint32_t isel[8];
+  // lane k keeps the k-th pick (no register arrays indexed by the round counter)
+  float my_w = 0.f;
+  uint32_t my_idx = 0xFFFFFFFFu;
   for (uint32_t k = 0; k < K; ++k) {
     float bv = NEG_INF;
     uint32_t bi = 0xFFFFFFFFu;
@@ -136,21 +137,22 @@ __device__ __forceinline__ void route_token(const float* __restrict__ logits, co
 #pragma unroll
     for (int j = 0; j < 4; ++j)
       if (bi == lane + 64 * j) taken[j] = true;
-    isel[k] = bi;
-    wsel[k] = bw;
+    if (lane == k) {
+      my_idx = bi;
+      my_w = bw;
+    }
   }
-  if (lane == 0) {
-    float scale = 1.0f;
-    if (renorm) {
-      float ws = 0.f;
-      for (uint32_t k = 0; k < K; ++k) ws += wsel[k];
-      scale = ws > 0.f ? 1.0f / ws : 0.f;
-    }
-    for (uint32_t k = 0; k < K; ++k) {
-      out_idx[(size_t)row * K + k] = isel[k];
-      out_w[(size_t)row * K + k] = wsel[k] * scale;
-      if (lds_idx != nullptr) lds_idx[row * K + k] = isel[k];
-    }
+  float scale = 1.0f;
+  if (renorm) {
+    // sum of the K picks in pick order (lanes 0 .. K-1), the order a serial loop would add them in
+    float ws = 0.f;
+    for (uint32_t k = 0; k < K; ++k) ws += readlane_f32(my_w, (int)k);
+    scale = ws > 0.f ? 1.0f / ws : 0.f;
+  }
+  if (lane < K) {
+    out_idx[(size_t)row * K + lane] = my_idx;
+    out_w[(size_t)row * K + lane] = my_w * scale;
+    if (lds_idx != nullptr) lds_idx[row * K + lane] = my_idx;
   }
 }
 
@@ -264,14 +266,14 @@ __global__ __launch_bounds__(1024) void moe_sort_kernel(const uint32_t* __restri
 
 // At most 64 assignments (decode-sized batches): one wave, no barriers.  Lane i owns assignment i; ranks,
 // offsets and chunk positions are counted with readlane loops over the other lanes.  Same outputs as above.
-__device__ __forceinline__ void sort_small(uint32_t lane, uint32_t e, uint32_t E, uint32_t top_k,
+__device__ __forceinline__ void sort_small(uint32_t lane, uint32_t n, uint32_t e, uint32_t E, uint32_t top_k,
                                            uint32_t* __restrict__ sorted, uint32_t* __restrict__ sorted_tok,
                                            uint32_t* __restrict__ inv, uint32_t* __restrict__ counts,
                                            uint32_t* __restrict__ offsets, uint32_t* __restrict__ chunk_tab,
                                            uint32_t* __restrict__ n_chunks) {
-  const bool valid = e < E;
+  const bool valid = e < E;  // (lanes past the n assignments hold an invalid expert)
   uint32_t rank = 0, same = 0, less = 0, n_valid = 0;
-  for (int j = 0; j < 64; ++j) {
+  for (int j = 0; j < (int)n; ++j) {
     const uint32_t ej = (uint32_t)__builtin_amdgcn_readlane((int)e, j);
     if (ej >= E) continue;  // uniform
     ++n_valid;
@@ -289,7 +291,7 @@ __device__ __forceinline__ void sort_small(uint32_t lane, uint32_t e, uint32_t E
   const bool leader = valid && rank == 0;
   const uint32_t my_chunks = leader ? (same + 7) / 8 : 0u;
   uint32_t chunks_before = 0, total_chunks = 0;
-  for (int j = 0; j < 64; ++j) {
+  for (int j = 0; j < (int)n; ++j) {
     const uint32_t cj = (uint32_t)__builtin_amdgcn_readlane((int)my_chunks, j);
     if (cj == 0) continue;  // uniform
     const uint32_t ej = (uint32_t)__builtin_amdgcn_readlane((int)e, j);
@@ -327,7 +329,7 @@ __global__ __launch_bounds__(64) void moe_sort_small_kernel(const uint32_t* __re
                                                             uint32_t* __restrict__ chunk_tab,
                                                             uint32_t* __restrict__ n_chunks) {
   const uint32_t lane = threadIdx.x;
-  sort_small(lane, lane < n_assign ? idx[lane] : 0xFFFFFFFFu, E, top_k, sorted, sorted_tok, inv, counts, offsets,
+  sort_small(lane, n_assign, lane < n_assign ? idx[lane] : 0xFFFFFFFFu, E, top_k, sorted, sorted_tok, inv, counts, offsets,
              chunk_tab, n_chunks);
 }
 
@@ -346,7 +348,7 @@ __global__ __launch_bounds__(512) void route_sort_small_kernel(const float* __re
   if (wave < T) route_token(logits, bias, E, K, renorm, out_idx, out_w, wave, lane, picks);
   __syncthreads();
   if (wave == 0)
-    sort_small(lane, lane < T * K ? picks[lane] : 0xFFFFFFFFu, E, K, sorted, sorted_tok, inv, nullptr, nullptr,
+    sort_small(lane, T * K, lane < T * K ? picks[lane] : 0xFFFFFFFFu, E, K, sorted, sorted_tok, inv, nullptr, nullptr,
                chunk_tab, n_chunks);
 }
 
