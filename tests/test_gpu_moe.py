@@ -255,9 +255,9 @@ def _experts(rng, E, D, I, fused):
 
 @pytest.mark.parametrize("T,E,K", [(1, 128, 8), (8, 128, 8), (7, 200, 3), (8, 256, 8), (3, 5, 5), (9, 128, 7)])
 def test_moe_forward_routes_like_the_two_step_path(hip, T, E, K):
-    """Up to 8 tokens / 64 assignments with f32 logits, routing and grouping share one launch: the result must
-    equal, bit for bit, routing first and calling the grouped block with its outputs -- with and without an
-    expert bias, and also for an f16 bias (which takes the two-step path inside)."""
+    """Up to 8 tokens / 64 assignments with f32 logits, routing and grouping share one launch: the picks must
+    be those of routing alone, and the result that of calling the grouped block with them -- with and without
+    an expert bias, and also for an f16 bias (which takes the two-step path inside)."""
     from rmlx_amd import ops
     from rmlx_amd.runtime import DeviceBuffer
     rng = np.random.default_rng(T * 31 + E + K)
@@ -273,10 +273,33 @@ def test_moe_forward_routes_like_the_two_step_path(hip, T, E, K):
         one = ops.moe_forward(gh, uh, dh, xd, ld, K, expert_bias=bd).numpy()
         r = ops.gpu_topk_route(ld, K, expert_bias=bd)
         two = ops.moe_forward_grouped(gh, uh, dh, xd, r.expert_indices, r.expert_weights, K).numpy()
-        assert np.array_equal(one, two)
         idx, w, _, _ = model.topk_route(logits, K, bias=None if bias is None else bias.astype(np.float32))
         assert np.array_equal(r.expert_indices.numpy(), idx)
-        assert_close(one, model.moe_forward(xd.numpy(), idx, w, gate, up, down, 64, K), "moe_forward")
+        ref = model.moe_forward(xd.numpy(), idx, w, gate, up, down, 64, K)
+        assert_close(one, ref, "moe_forward")
+        assert_close(two, ref, "moe_forward_grouped")
+        # (the one-call path knows its picks are distinct per token and may run kernels built for fewer rows
+        # per expert than the grouped entry point, which must allow for repeated experts: same picks, same
+        # weights, results within the tolerance of each other rather than bit-equal)
+        assert np.abs(one.astype(np.float64) - two.astype(np.float64)).max() <= model.tolerance(ref)
+
+
+@pytest.mark.parametrize("T,K", [(1, 2), (1, 8), (2, 3), (3, 4)])
+def test_moe_forward_grouped_with_repeated_experts(hip, T, K):
+    """Caller-supplied picks may name one expert several times for a token; decode-sized batches run kernels
+    built for few rows per expert, whose bound must then count assignments, not tokens."""
+    from rmlx_amd import ops
+    from rmlx_amd.runtime import DeviceBuffer
+    rng = np.random.default_rng(T * 10 + K)
+    E, D, I = 6, 512, 1024
+    gate, up, down, gh, uh, dh = _experts(rng, E, D, I, False)
+    x = make_x(rng, T, D)
+    idx = np.full(T * K, 4, np.uint32)   # every assignment goes to expert 4
+    idx[-1] = 1
+    w = rng.uniform(0.1, 1.0, size=T * K).astype(np.float32)
+    out = ops.moe_forward_grouped(gh, uh, dh, DeviceBuffer.from_numpy(x), DeviceBuffer.from_numpy(idx),
+                                  DeviceBuffer.from_numpy(w), K).numpy()
+    assert_close(out, model.moe_forward(x, idx, w, gate, up, down, 64, K), "repeated experts")
 
 
 @pytest.mark.parametrize("fused", [False, True])
@@ -292,11 +315,13 @@ def test_moe_forward_small(hip, fused, T, E, K, D, I):
     ref = model.moe_forward(x, idx, w, gate, up, down, 64, K)
     out = ops.moe_forward(gh, uh, dh, DeviceBuffer.from_numpy(x), DeviceBuffer.from_numpy(logits), K).numpy()
     assert_close(out, ref, "moe_forward")
-    # routing on the device followed by the grouped block == the one-call entry point, bit for bit
+    # routing on the device followed by the grouped block == the one-call entry point
     r = ops.gpu_topk_route(DeviceBuffer.from_numpy(logits), K)
     assert np.array_equal(r.expert_indices.numpy(), idx)
     out2 = ops.moe_forward_grouped(gh, uh, dh, DeviceBuffer.from_numpy(x), r.expert_indices, r.expert_weights, K).numpy()
-    assert np.array_equal(out, out2)
+    if T > 8:  # (smaller batches: the one-call path may run kernels built for fewer rows per expert)
+        assert np.array_equal(out, out2)
+    assert_close(out2, ref, "moe_forward_grouped with device routing")
     out3 = ops.moe_forward_grouped(gh, uh, dh, DeviceBuffer.from_numpy(x), DeviceBuffer.from_numpy(idx),
                                    DeviceBuffer.from_numpy(w), K).numpy()
     assert_close(out3, ref, "moe_forward_grouped with host routing")
