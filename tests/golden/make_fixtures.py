@@ -17,6 +17,10 @@ so that every later change of the oracle or of the HIP kernels is checked agains
       logits f32 [T,E]; expert_indices u32 [T*K]; expert_weights f32 [T*K]; expert_counts u32 [E];
       dispatch_offsets u32 [E+1]; sorted_assignments u32 [T*K]   (topk_route.rs:212-388, moe.rs:1439-1447)
 
+  dequant_<awq|gptq>_<R>x<C>_gs<G>_seed<S>[_gidx].npz
+      qweight / qzeros u32, scales f32, g_idx i32 (GPTQ with act-order only), out f32 [R,C]
+      (`awq_dequant_f32` / `gptq_dequant_f32`, quantized.rs:707-783)
+
 Run from the repository root:  python tests/golden/make_fixtures.py
 Nothing here reads the reference tree; the fixtures are data only.
 """
@@ -39,6 +43,9 @@ LCG_CASES = [
     (16, 64, 512, 64, 42),                                            # kernel-sized twin (qmv / qmm shapes)
 ]
 ROUTE_CASES = [(4, 8, 2, 11), (32, 128, 8, 12), (7, 200, 3, 13)]
+# (format, rows, cols, group_size, seed, with g_idx)
+DEQUANT_CASES = [("awq", 16, 24, 4, 21, False), ("awq", 64, 128, 32, 24, False), ("gptq", 32, 16, 8, 22, False),
+                 ("gptq", 32, 16, 8, 23, True), ("gptq", 128, 64, 32, 25, True)]
 
 
 def lcg_case(m, n, k, gs, seed, bits):
@@ -64,8 +71,29 @@ def route_case(t, e, k, seed):
                 dispatch_offsets=offsets, sorted_assignments=sorted_assign)
 
 
+def dequant_case(fmt, rows, cols, gs, seed, with_gidx):
+    rng = np.random.default_rng(seed)
+    groups = rows // gs
+    shape = (rows, cols // 8) if fmt == "awq" else (rows // 8, cols)
+    qweight = rng.integers(0, 2**32, size=shape, dtype=np.uint64).astype(np.uint32)
+    qzeros = rng.integers(0, 2**32, size=(groups, cols // 8), dtype=np.uint64).astype(np.uint32)
+    scales = rng.uniform(0.001, 0.05, size=(groups, cols)).astype(np.float32)
+    d = dict(qweight=qweight, qzeros=qzeros, scales=scales)
+    if fmt == "awq":
+        d["out"] = model.awq_dequant(qweight, qzeros, scales, gs)
+    else:
+        g_idx = rng.integers(0, groups, size=rows).astype(np.int32) if with_gidx else None
+        if with_gidx:
+            d["g_idx"] = g_idx
+        d["out"] = model.gptq_dequant(qweight, qzeros, scales, g_idx, gs)
+    return d
+
+
 def main():
     refpath.build()
+    for (fmt, rows, cols, gs, seed, with_gidx) in DEQUANT_CASES:
+        name = f"dequant_{fmt}_{rows}x{cols}_gs{gs}_seed{seed}{'_gidx' if with_gidx else ''}.npz"
+        np.savez_compressed(os.path.join(HERE, name), **dequant_case(fmt, rows, cols, gs, seed, with_gidx))
     for (m, n, k, gs, seed) in LCG_CASES:
         for bits in (4, 8):
             np.savez_compressed(os.path.join(HERE, f"lcg_{m}x{n}x{k}_gs{gs}_q{bits}_seed{seed}.npz"),

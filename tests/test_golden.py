@@ -18,6 +18,7 @@ from tests.helpers import assert_close
 GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
 LCG_FILES = sorted(glob.glob(os.path.join(GOLDEN, "lcg_*.npz")))
 ROUTE_FILES = sorted(glob.glob(os.path.join(GOLDEN, "route_*.npz")))
+DEQUANT_FILES = sorted(glob.glob(os.path.join(GOLDEN, "dequant_*.npz")))
 
 
 def _lcg_meta(path):
@@ -27,7 +28,42 @@ def _lcg_meta(path):
 
 
 def test_fixture_inventory():
-    assert len(LCG_FILES) == 12 and len(ROUTE_FILES) == 3
+    assert len(LCG_FILES) == 12 and len(ROUTE_FILES) == 3 and len(DEQUANT_FILES) == 5
+
+
+def _dequant_meta(path):
+    fmt, rows, cols, gs = re.match(r"dequant_(awq|gptq)_(\d+)x(\d+)_gs(\d+)_", os.path.basename(path)).groups()
+    return fmt, int(rows), int(cols), int(gs)
+
+
+def _dequant_oracle(path):
+    fmt, rows, cols, gs = _dequant_meta(path)
+    f = np.load(path)
+    if fmt == "awq":
+        return f, model.awq_dequant(f["qweight"], f["qzeros"], f["scales"], gs)
+    return f, model.gptq_dequant(f["qweight"], f["qzeros"], f["scales"], f["g_idx"] if "g_idx" in f else None, gs)
+
+
+@pytest.mark.parametrize("path", DEQUANT_FILES, ids=os.path.basename)
+def test_oracle_reproduces_dequant_fixture(path):
+    f, out = _dequant_oracle(path)
+    assert out.dtype == np.float32 and np.array_equal(out, f["out"])
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("path", DEQUANT_FILES, ids=os.path.basename)
+def test_gpu_matches_dequant_fixture(hip, path):
+    from rmlx_amd import ops
+    from rmlx_amd.runtime import DeviceBuffer
+    fmt, rows, cols, gs = _dequant_meta(path)
+    f = np.load(path)
+    dev = [DeviceBuffer.from_numpy(f[k]) for k in ("qweight", "qzeros", "scales")]
+    if fmt == "awq":
+        got = ops.awq_dequant(*dev, rows, cols, gs).numpy()
+    else:
+        g_idx = DeviceBuffer.from_numpy(f["g_idx"].view(np.uint32)) if "g_idx" in f else None
+        got = ops.gptq_dequant(*dev, g_idx, rows, cols, gs).numpy()
+    assert np.array_equal(got, f["out"])
 
 
 @pytest.mark.parametrize("path", LCG_FILES, ids=os.path.basename)
