@@ -327,6 +327,28 @@ def test_moe_forward_small(hip, fused, T, E, K, D, I):
     assert_close(out3, ref, "moe_forward_grouped with host routing")
 
 
+def test_random_moe_shapes(hip):
+    """Twenty seeded random (T, E, K, D, I, fused, bias) blocks through the one-call entry point."""
+    from rmlx_amd import ops
+    from rmlx_amd.runtime import DeviceBuffer
+    rng = np.random.default_rng(20250101)
+    for case in range(20):
+        E = int(rng.integers(1, 40))
+        K = int(rng.integers(1, min(8, E) + 1))
+        T = int(rng.choice([1, 2, 3, 5, 8, 9, 17, 40]))
+        D, I = int(rng.integers(1, 4)) * 512, int(rng.integers(1, 4)) * 512
+        fused = bool(rng.integers(0, 2))
+        gate, up, down, gh, uh, dh = _experts(rng, E, D, I, fused)
+        x = make_x(rng, T, D)
+        logits = (2.0 * rng.standard_normal((T, E))).astype(np.float32)
+        bias = rng.standard_normal(E).astype(np.float32) if rng.integers(0, 2) else None
+        print(f"moe case {case}: T={T} E={E} K={K} D={D} I={I} fused={fused} bias={bias is not None}", flush=True)
+        out = ops.moe_forward(gh, uh, dh, DeviceBuffer.from_numpy(x), DeviceBuffer.from_numpy(logits), K,
+                              expert_bias=DeviceBuffer.from_numpy(bias) if bias is not None else None).numpy()
+        idx, w, _, _ = model.topk_route(logits, K, bias=bias)
+        assert_close(out, model.moe_forward(x, idx, w, gate, up, down, 64, K), f"case {case}")
+
+
 def test_grouped_forward_equals_per_expert_loop(hip):
     """grouped == individual (expert_group.rs:972-1019), against the float64 expert FFN."""
     from rmlx_amd import ops
