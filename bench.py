@@ -258,14 +258,17 @@ def main():
                                                GiB + GiB // 8)
         extra["q8_qmv_m1_4096"] = bench_matmul(ops, rt, timer, rng, 1, 4096, 4096, 8, "f16", args.steps, args.warmup,
                                                GiB + GiB // 8)
-        # the GEMM sections run as many steps as the headline: the GPU needs tens of milliseconds of
-        # sustained matrix work before its clock settles (a 100-launch window reads 15 % slower)
+        # the GEMM sections run at least 10 000 steps: the GPU needs a few hundred milliseconds of sustained
+        # matrix work before its clock settles (a 100-launch window reads 15 % slower, a 2 000-launch one 3 %)
+        gemm_steps = max(args.steps, 10000)
         for m in (128, 512):
-            r = bench_matmul(ops, rt, timer, rng, m, 4096, 4096, 4, "f16", args.steps, args.warmup, 4 * 9437184)
+            r = bench_matmul(ops, rt, timer, rng, m, 4096, 4096, 4, "f16", gemm_steps, args.warmup, 4 * 9437184)
+            r["steps"] = gemm_steps
             r["mfma_frac"] = r["tflops"] / MFMA_F16_PEAK_TF
             extra[f"q4_qmm_m{m}_4096"] = r
         for name, kern in (("q8_qmm_bf16_m128_n12288", rt.KERNEL_AUTO), ("q8_qmm_bf16_m128_n12288_bf16_mfma", rt.KERNEL_QMM_BF16)):
-            r = bench_matmul(ops, rt, timer, rng, 128, 12288, 4096, 8, "bf16", args.steps, args.warmup, 4 * 53477376, kernel=kern)
+            r = bench_matmul(ops, rt, timer, rng, 128, 12288, 4096, 8, "bf16", gemm_steps, args.warmup, 4 * 53477376, kernel=kern)
+            r["steps"] = gemm_steps
             r["mfma_frac"] = r["tflops"] / MFMA_F16_PEAK_TF
             r["hbm_frac"] = r["gbs"] / HBM_PEAK_GBS
             extra[name] = r
@@ -312,7 +315,8 @@ def main():
                              "roofline": {"bound": "mfma", "achieved": q["tflops"], "peak": MFMA_F16_PEAK_TF,
                                           "unit": "TFLOP/s", "frac": q["mfma_frac"],
                                           "traffic": MEASURED_TRAFFIC_BYTES["qmm_q4_m512_4096"],
-                                          "kernel": "qmm_rw_kernel<4,1,4,8,false,64>", "avg_launch_us": q["us"]}}
+                                          "kernel": "qmm_rw_kernel<4,1,4,8,false,64>", "avg_launch_us": q["us"]},
+                             "steps": q["steps"]}
     if not args.no_cpu:
         line["cpu_baseline"] = cpu_baseline(np.random.default_rng(1001), 3.0 if args.quick else 10.0)
     line["extra"] = extra
