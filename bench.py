@@ -28,7 +28,7 @@ MFMA_F16_PEAK_TF = 2500.0  # dense f16 / bf16 MFMA
 # (FETCH_SIZE and WRITE_SIZE, each scaled by what it reads for the plain copy below); the runs and
 # the scaling are recorded in profiles/bench_all_configs_hbm_traffic_pmc.txt.  Counters cannot be
 # read from inside this process, so the figures are carried here and re-measured with the kernels.
-MEASURED_TRAFFIC_BYTES = {"qmv_q4_m1_4096": 9553529, "qmm_q4_m512_4096": 39716906}
+MEASURED_TRAFFIC_BYTES = {"qmv_q4_m1_4096": 9541193, "qmm_q4_m512_4096": 39728849}
 
 
 def matmul_bytes(m, n, k, bits, gs=64, act_bytes=2):
@@ -220,8 +220,8 @@ def cpu_baseline(rng, budget_s=10.0):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=2000)
-    ap.add_argument("--warmup", type=int, default=200)
+    ap.add_argument("--steps", type=int, default=20000)
+    ap.add_argument("--warmup", type=int, default=2000)
     ap.add_argument("--quick", action="store_true", help="headline configuration only, short CPU baseline")
     ap.add_argument("--no-cpu", action="store_true")
     args = ap.parse_args()
@@ -260,7 +260,8 @@ def main():
                                                GiB + GiB // 8)
         # the GEMM sections run at least 10 000 steps: the GPU needs a few hundred milliseconds of sustained
         # matrix work before its clock settles (a 100-launch window reads 15 % slower, a 2 000-launch one 3 %)
-        gemm_steps = max(args.steps, 10000)
+        # (short runs, as under a counter pass, keep their own count)
+        gemm_steps = max(args.steps, 10000) if args.steps >= 1000 else args.steps
         for m in (128, 512):
             r = bench_matmul(ops, rt, timer, rng, m, 4096, 4096, 4, "f16", gemm_steps, args.warmup, 4 * 9437184)
             r["steps"] = gemm_steps
@@ -306,7 +307,7 @@ def main():
                    "parity_max_err": head.get("max_err"), "parity_tol": head.get("tol")},
         "roofline": {"bound": "hbm", "achieved": head["gbs"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": head["gbs"] / HBM_PEAK_GBS, "traffic": MEASURED_TRAFFIC_BYTES["qmv_q4_m1_4096"],
-                     "kernel": "qmv_m1_kernel<4,64,1,true,1>", "bytes_per_launch": head["bytes"],
+                     "kernel": "qmv_m1_kernel<4,64,1,true,1,false>", "bytes_per_launch": head["bytes"],
                      "avg_launch_us": head["us"]},
     }
     if not args.quick and "q4_qmm_m512_4096" in extra:
