@@ -208,7 +208,7 @@ def silu(x):
     return x / (1.0 + np.exp(-x))
 
 
-def moe_forward(x, indices, weights, gate, up, down, group_size, top_k, round_h=np.float16):
+def moe_forward(x, indices, weights, gate, up, down, group_size, top_k, round_h=np.float16, bits=4):
     """out[t] = sum_k w[t,k] * down_e( silu(gate_e x_t) * up_e x_t ), e = indices[t,k].
 
     Composition of `ExpertGroup::grouped_forward` (crates/rmlx-nn/src/expert_group.rs:445-524:
@@ -231,7 +231,7 @@ def moe_forward(x, indices, weights, gate, up, down, group_size, top_k, round_h=
     def deq(trip, e):
         key = (id(trip[0]), int(e))
         if key not in cache:
-            cache[key] = dequantize(trip[0][e], trip[1][e], trip[2][e], group_size, 4)
+            cache[key] = dequantize(trip[0][e], trip[1][e], trip[2][e], group_size, bits)
         return cache[key]
 
     for e in np.unique(idx):

@@ -283,6 +283,7 @@ int32_t check_out(const char* who, size_t have, size_t need) {
 struct ExpertShapes {
   uint32_t E, D, I;
   bool fused;
+  bool portable;  // not Q4 / group 64 / dims in multiples of 512: the portable kernels run the block
 };
 
 int32_t check_expert_weights(const char* who, const rmlx_qweight* gate, const rmlx_qweight* up,
@@ -297,22 +298,48 @@ int32_t check_expert_weights(const char* who, const rmlx_qweight* gate, const rm
     return fail(RMLX_INVALID_SHAPE, "%s: down weight must be [%zu, %zu, %zu], got [%zu, %zu, %zu]", who, E, D, I,
                 down->n_experts, down->out_features, down->in_features);
   const rmlx_qweight* all[3] = {gate, up, down};
+  bool fast = true;
   for (const rmlx_qweight* q : all) {
     if (q == nullptr) continue;
-    if (q->bits != 4 || q->group_size != 64)
-      return fail(RMLX_NOT_FOUND, "%s: expert weights must be Q4 with group_size 64 (got bits=%u group_size=%u)",
-                  who, q->bits, q->group_size);
-    if (!aligned16(q->w) || !aligned16(q->s) || !aligned16(q->b))
-      return fail(RMLX_INVALID_SHAPE, "%s: expert weight buffers must be 16-byte aligned", who);
+    if (q->bits != 2 && q->bits != 4 && q->bits != 8)
+      return fail(RMLX_NOT_FOUND, "%s: no kernel for %u-bit expert weights (2, 4 and 8 are implemented)", who, q->bits);
+    if (q->bits != 4 || q->group_size != 64 || !aligned16(q->w) || !aligned16(q->s) || !aligned16(q->b)) fast = false;
   }
   RMLX_TRY(checked_u32(E, "num_experts", &sh->E));
   RMLX_TRY(checked_u32(D, "hidden_dim", &sh->D));
   RMLX_TRY(checked_u32(I, "intermediate_dim", &sh->I));
-  if (!qmv_q4_supported(sh->I, sh->D, 64) || !qmv_q4_supported(sh->D, sh->I, 64))
-    return fail(RMLX_NOT_FOUND, "%s: no kernel for hidden_dim=%u intermediate_dim=%u (both must be multiples of 512)",
-                who, sh->D, sh->I);
+  if (!qmv_q4_supported(sh->I, sh->D, 64) || !qmv_q4_supported(sh->D, sh->I, 64)) fast = false;
   sh->fused = fused;
+  sh->portable = !fast;
   return RMLX_OK;
+}
+
+// The same block on the portable kernels, for expert weights the streaming GEMV does not take (2- or 8-bit,
+// group sizes 32 / 128, dimensions that are no multiples of 512): every position multiplies with its own
+// expert's rows.  x: f16 [positions, D] (already gathered); expert_of: device u32 [positions]; y: f16 [positions, D].
+int32_t run_expert_ffn_portable(const rmlx_qweight* gate, const rmlx_qweight* up, const rmlx_qweight* down,
+                                const ExpertShapes& sh, const __half* x, const uint32_t* expert_of, uint32_t positions,
+                                __half* y, hipStream_t stream) {
+  Scratch gu, h;
+  const uint32_t gu_cols = 2 * sh.I;
+  RMLX_TRY(gu.alloc((size_t)positions * gu_cols * sizeof(__half), stream));
+  RMLX_TRY(h.alloc((size_t)positions * sh.I * sizeof(__half), stream));
+  __half* g_out = static_cast<__half*>(gu.ptr);
+  if (sh.fused) {  // one weight of 2I rows per expert, gate rows first: [positions, 2I]
+    GenericArgs a{gate->w, gate->s, gate->b, x, g_out, expert_of, 1, positions, gu_cols, sh.D, gate->group_size, gate->bits, sh.E};
+    RMLX_TRY(launch_generic(a, stream));
+    RMLX_TRY(launch_silu_gate_strided(g_out, g_out + sh.I, gu_cols, static_cast<__half*>(h.ptr), positions, sh.I, stream));
+  } else {         // [positions, I] twice
+    __half* u_out = g_out + (size_t)positions * sh.I;
+    GenericArgs a{gate->w, gate->s, gate->b, x, g_out, expert_of, 1, positions, sh.I, sh.D, gate->group_size, gate->bits, sh.E};
+    GenericArgs b{up->w, up->s, up->b, x, u_out, expert_of, 1, positions, sh.I, sh.D, up->group_size, up->bits, sh.E};
+    RMLX_TRY(launch_generic(a, stream));
+    RMLX_TRY(launch_generic(b, stream));
+    RMLX_TRY(launch_silu_gate(g_out, u_out, static_cast<__half*>(h.ptr), (size_t)positions * sh.I, stream));
+  }
+  GenericArgs d{down->w, down->s, down->b, static_cast<const __half*>(h.ptr), y, expert_of, 1, positions, sh.D, sh.I,
+                down->group_size, down->bits, sh.E};
+  return launch_generic(d, stream);
 }
 
 // gate/up + SwiGLU then down, over a device chunk table.  h: f16 [positions, I] scratch.
@@ -902,6 +929,17 @@ int32_t rmlx_hip_expert_group_grouped_forward(const rmlx_qweight* gate, const rm
     RMLX_TRY(launch_cast_to_f16(x->data, x->dtype, static_cast<__half*>(cast.ptr), total * sh.D, s));
     xk = static_cast<const __half*>(cast.ptr);
   }
+  if (sh.portable) {  // expert of every packed row, then the portable kernels
+    std::vector<uint32_t> expert_of;
+    expert_of.reserve(total);
+    for (size_t i = 0; i < n_items; ++i) expert_of.insert(expert_of.end(), batch_sizes_host[i], expert_idx_host[i]);
+    RMLX_TRY(dtab.alloc(total * 4, s));
+    RMLX_HIP_CHECK(hipMemcpyAsync(dtab.ptr, expert_of.data(), total * 4, hipMemcpyHostToDevice, s));
+    RMLX_HIP_CHECK(hipStreamSynchronize(s));  // `expert_of` is pageable host memory owned by this call
+    RMLX_TRY(run_expert_ffn_portable(gate, up, down, sh, xk, static_cast<const uint32_t*>(dtab.ptr), rows,
+                                     static_cast<__half*>(out_f16_dev), s));
+    return finish(s);
+  }
   if (!aligned16(xk)) return fail(RMLX_INVALID_SHAPE, "ExpertGroup: input must be 16-byte aligned");
   RMLX_TRY(dtab.alloc(tab.size() * 4, s));
   RMLX_HIP_CHECK(hipMemcpyAsync(dtab.ptr, tab.data(), tab.size() * 4, hipMemcpyHostToDevice, s));
@@ -947,6 +985,27 @@ int32_t moe_grouped_impl(const rmlx_qweight* gate, const rmlx_qweight* up, const
     RMLX_TRY(cast.alloc(T * sh.D * 2, s));
     RMLX_TRY(launch_cast_to_f16(x->data, x->dtype, static_cast<__half*>(cast.ptr), T * sh.D, s));
     xk = static_cast<const __half*>(cast.ptr);
+  }
+  if (sh.portable) {
+    // Assignments stay in their own order: position a holds token a / top_k and expert idx[a].
+    if (route != nullptr)
+      RMLX_TRY(launch_topk_route(route->logits, route->bias, T32, sh.E, (uint32_t)top_k, 1, route->idx_out, route->w_out,
+                                 nullptr, nullptr, s));
+    Scratch xr, y16;
+    RMLX_TRY(meta.alloc((size_t)2 * A * 4, s));
+    uint32_t* tok = static_cast<uint32_t*>(meta.ptr);
+    uint32_t* ident = tok + A;
+    RMLX_TRY(launch_identity_positions(tok, ident, A, (uint32_t)top_k, s));
+    RMLX_TRY(xr.alloc((size_t)A * sh.D * 2, s));
+    RMLX_TRY(launch_index_gather(xk, sh.D, tok, A, T32, static_cast<__half*>(xr.ptr), s));
+    RMLX_TRY(y16.alloc((size_t)A * sh.D * 2, s));
+    RMLX_TRY(run_expert_ffn_portable(gate, up, down, sh, static_cast<const __half*>(xr.ptr), expert_indices_dev, A,
+                                     static_cast<__half*>(y16.ptr), s));
+    RMLX_TRY(y.alloc((size_t)A * sh.D * 4, s));
+    RMLX_TRY(launch_cast_f16_to_f32(static_cast<const __half*>(y16.ptr), static_cast<float*>(y.ptr), (size_t)A * sh.D, s));
+    RMLX_TRY(launch_moe_combine(static_cast<const float*>(y.ptr), ident, expert_weights_dev, T32, (uint32_t)top_k, sh.D,
+                                static_cast<__half*>(out_f16_dev), s));
+    return finish(s);
   }
   if (!aligned16(xk)) return fail(RMLX_INVALID_SHAPE, "MoeLayer: input must be 16-byte aligned");
   // meta: sorted[A] | sorted_tok[A] | inv[A] | chunk_tab[3*max_chunks] | n_chunks[1]

@@ -189,6 +189,11 @@ int32_t launch_index_gather(const __half* src, uint32_t d, const uint32_t* idx, 
 int32_t launch_scatter_weighted_add(const __half* src, uint32_t n, uint32_t d, const uint32_t* tok,
                                     const float* w, __half* dst, uint32_t dst_rows, hipStream_t s);
 int32_t launch_silu_gate(const __half* g, const __half* u, __half* out, size_t n, hipStream_t s);
+// out[r, c] = silu(g[r*ld + c]) * u[r*ld + c]
+int32_t launch_silu_gate_strided(const __half* g, const __half* u, uint32_t ld, __half* out, uint32_t rows,
+                                 uint32_t cols, hipStream_t s);
+// tok[a] = a / top_k, inv[a] = a  (assignments kept in their own order)
+int32_t launch_identity_positions(uint32_t* tok, uint32_t* inv, uint32_t n, uint32_t top_k, hipStream_t s);
 // out[t,:] = sum_k w[t*K+k] * y[inv[t*K+k],:]  (y f32 rows at sorted positions)
 int32_t launch_moe_combine(const float* y, const uint32_t* inv, const float* weights, uint32_t T,
                            uint32_t top_k, uint32_t D, __half* out, hipStream_t s);

@@ -384,6 +384,27 @@ __global__ void silu_gate_kernel(const __half* __restrict__ g, const __half* __r
   }
 }
 
+// out[r, c] = silu(g[r*ld + c]) * u[r*ld + c]: gate and up halves of one [rows, ld] matrix
+__global__ void silu_gate_strided_kernel(const __half* __restrict__ g, const __half* __restrict__ u, uint32_t ld,
+                                         __half* __restrict__ out, uint32_t rows, uint32_t cols) {
+  size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const size_t stride = (size_t)gridDim.x * blockDim.x, n = (size_t)rows * cols;
+  for (; i < n; i += stride) {
+    const size_t r = i / cols, c = i % cols;
+    const float x = __half2float(g[r * ld + c]);
+    out[i] = __float2half(x / (1.0f + __expf(-x)) * __half2float(u[r * ld + c]));
+  }
+}
+
+// assignments in their own order: token of assignment a is a / top_k, its position is a
+__global__ void identity_positions_kernel(uint32_t* __restrict__ tok, uint32_t* __restrict__ inv, uint32_t n, uint32_t top_k) {
+  const uint32_t a = blockIdx.x * blockDim.x + threadIdx.x;
+  if (a < n) {
+    tok[a] = a / top_k;
+    inv[a] = a;
+  }
+}
+
 // out[t,:] = sum_k w[t*K+k] * y[inv[t*K+k],:], k ascending, f32.  grid = (T, column blocks of 1024):
 // every thread owns four columns, loads its rows of all top_k experts first and sums in order.
 __global__ __launch_bounds__(256) void moe_combine_kernel(const float* __restrict__ y,
@@ -489,6 +510,24 @@ int32_t launch_silu_gate(const __half* g, const __half* u, __half* out, size_t n
   size_t blocks = (n + 255) / 256;
   if (blocks > 8192) blocks = 8192;
   hipLaunchKernelGGL(silu_gate_kernel, dim3((unsigned)blocks), dim3(256), 0, s, g, u, out, n);
+  RMLX_HIP_CHECK(hipGetLastError());
+  return RMLX_OK;
+}
+
+int32_t launch_silu_gate_strided(const __half* g, const __half* u, uint32_t ld, __half* out, uint32_t rows,
+                                 uint32_t cols, hipStream_t s) {
+  const size_t n = (size_t)rows * cols;
+  if (n == 0) return RMLX_OK;
+  size_t blocks = (n + 255) / 256;
+  if (blocks > 8192) blocks = 8192;
+  hipLaunchKernelGGL(silu_gate_strided_kernel, dim3((unsigned)blocks), dim3(256), 0, s, g, u, ld, out, rows, cols);
+  RMLX_HIP_CHECK(hipGetLastError());
+  return RMLX_OK;
+}
+
+int32_t launch_identity_positions(uint32_t* tok, uint32_t* inv, uint32_t n, uint32_t top_k, hipStream_t s) {
+  if (n == 0) return RMLX_OK;
+  hipLaunchKernelGGL(identity_positions_kernel, dim3((n + 255) / 256), dim3(256), 0, s, tok, inv, n, top_k);
   RMLX_HIP_CHECK(hipGetLastError());
   return RMLX_OK;
 }

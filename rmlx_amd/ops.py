@@ -231,7 +231,7 @@ def gptq_dequant(qweight, qzeros, scales, g_idx, in_features, out_features, grou
 
 
 class ExpertGroup:
-    """`ExpertGroup` (crates/rmlx-nn/src/expert_group.rs) over Q4 stacked expert weights."""
+    """`ExpertGroup` (crates/rmlx-nn/src/expert_group.rs) over stacked quantized expert weights."""
 
     def __init__(self, gate, up, down):
         self.gate, self.up, self.down = gate, up, down

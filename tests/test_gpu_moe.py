@@ -349,6 +349,52 @@ def test_random_moe_shapes(hip):
         assert_close(out, model.moe_forward(x, idx, w, gate, up, down, 64, K), f"case {case}")
 
 
+@pytest.mark.parametrize("bits,gs,D,I,fused", [(8, 64, 512, 512, False), (4, 32, 512, 1024, True), (4, 128, 384, 640, False),
+                                               (8, 32, 96, 160, True), (2, 64, 256, 128, False)])
+def test_moe_on_the_portable_kernels(hip, bits, gs, D, I, fused):
+    """Expert weights the streaming GEMV does not take (8- or 2-bit, group sizes 32 / 128, dimensions that are
+    no multiples of 512) run the same block on the portable kernels: routed block (one call and grouped) and
+    `ExpertGroup::grouped_forward`, against the oracle."""
+    from rmlx_amd import ops
+    from rmlx_amd.runtime import DeviceBuffer
+    rng = np.random.default_rng(bits * 100 + gs + D)
+    E, T, K = 5, 6, 2
+
+    def weight(n, k):
+        return make_weight(rng, n, k, bits if bits != 2 else 4, gs, lead=(E,)) if bits != 2 else _two_bit(rng, E, n, k, gs)
+
+    if fused:
+        gu = weight(2 * I, D)
+        gate, up = tuple(a[:, :I] for a in gu), tuple(a[:, I:] for a in gu)
+        gh, uh = ops.QuantizedWeight.from_numpy(*gu, gs, bits), None
+    else:
+        gate, up = weight(I, D), weight(I, D)
+        gh, uh = ops.QuantizedWeight.from_numpy(*gate, gs, bits), ops.QuantizedWeight.from_numpy(*up, gs, bits)
+    down = weight(D, I)
+    dh = ops.QuantizedWeight.from_numpy(*down, gs, bits)
+    x = make_x(rng, T, D)
+    logits = rng.standard_normal((T, E)).astype(np.float32)
+    idx, w, _, _ = model.topk_route(logits, K)
+    ref = model.moe_forward(x, idx, w, gate, up, down, gs, K, bits=bits)
+    xd = DeviceBuffer.from_numpy(x)
+    print(f"portable moe bits={bits} gs={gs} D={D} I={I} fused={fused}", flush=True)
+    assert_close(ops.moe_forward(gh, uh, dh, xd, DeviceBuffer.from_numpy(logits), K).numpy(), ref, "moe_forward")
+    assert_close(ops.moe_forward_grouped(gh, uh, dh, xd, DeviceBuffer.from_numpy(idx), DeviceBuffer.from_numpy(w), K).numpy(),
+                 ref, "moe_forward_grouped")
+    group = ops.ExpertGroup(gh, uh, dh)
+    items = [(3, make_x(rng, 2, D)), (0, make_x(rng, 5, D))]
+    outs = group.grouped_forward([(e, DeviceBuffer.from_numpy(v)) for e, v in items])
+    for (e, v), (_, yv) in zip(items, outs):
+        ones = np.ones((len(v), 1))
+        assert_close(yv, model.moe_forward(v, np.full((len(v), 1), e), ones, gate, up, down, gs, 1, bits=bits), f"expert {e}")
+
+
+def _two_bit(rng, E, n, k, gs):
+    words = rng.integers(0, 2**32, size=(E, n, k // 16), dtype=np.uint64).astype(np.uint32)
+    scales = rng.uniform(0.02, 0.08, size=(E, n, k // gs)).astype(np.float16)
+    return words, scales, (-1.5 * scales.astype(np.float32)).astype(np.float16)
+
+
 def test_grouped_forward_equals_per_expert_loop(hip):
     """grouped == individual (expert_group.rs:972-1019), against the float64 expert FFN."""
     from rmlx_amd import ops
