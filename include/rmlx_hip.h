@@ -133,7 +133,7 @@ int32_t rmlx_hip_affine_quantized_matmul_batched(const rmlx_qweight* qw, const r
  * 4 = LDS-staged MFMA GEMM on the bf16 matrix instruction (Q8 weights and bf16 activations
  * only; weights are rounded to bf16, so its error is about four times that of kernel 2),
  * 5 = LDS-staged MFMA GEMM (f16 MFMA, K % 256 == 0),
- * 6 = multi-row streaming GEMV also for a single row (group size 64 only). */
+ * 6 = multi-row streaming GEMV also for a single row (group sizes 64 and 128). */
 int32_t rmlx_hip_qmm_select(const rmlx_qweight* qw, const rmlx_array* x, int32_t kernel,
                             void* out_f16_dev, size_t out_bytes, rmlx_stream stream);
 
@@ -230,7 +230,7 @@ int32_t rmlx_hip_silu_gate(const void* gate_in_f16_dev, const void* up_in_f16_de
  * Literal contract: `n_items` (expert_idx, input [batch_i, D]) pairs, inputs packed one
  * after another in x ([sum batch_i, D] f16); out receives the per-item outputs in the same
  * packing.  Per item: y = (silu(x Wg^T) * (x Wu^T)) Wd^T with stacked expert weights (the streaming kernels
- * take 4-bit weights with group size 64 and dimensions in multiples of 512; every other 2- / 4- / 8-bit weight the
+ * take 4-bit weights with group size 64 or 128 and dimensions in multiples of 512; every other 2- / 4- / 8-bit weight the
  * type admits runs the same block on the portable kernels)
  * gate/up [E, I, D] and down [E, D, I].  `up` may be NULL when `gate` holds the fused
  * [E, 2I, D] layout (gate rows first).  expert_idx and batch_sizes are HOST arrays.

@@ -261,7 +261,7 @@ int32_t run_matmul_plain(const rmlx_qweight* qw, const void* x, int32_t x_dtype,
     a.w0 = qw->w; a.s0 = qw->s; a.b0 = qw->b;
     a.N = N; a.K = K;
     a.x = static_cast<const __half*>(xk);
-    a.out = out; a.ld_out = N; a.M = M;
+    a.out = out; a.ld_out = N; a.M = M; a.group_size = qw->group_size;
     return launch_qmv_q4(a, stream);
   }
   GenericArgs g{qw->w, qw->s, qw->b, static_cast<const __half*>(xk), out, nullptr, 0, M, N, K,
@@ -303,12 +303,15 @@ int32_t check_expert_weights(const char* who, const rmlx_qweight* gate, const rm
     if (q == nullptr) continue;
     if (q->bits != 2 && q->bits != 4 && q->bits != 8)
       return fail(RMLX_NOT_FOUND, "%s: no kernel for %u-bit expert weights (2, 4 and 8 are implemented)", who, q->bits);
-    if (q->bits != 4 || q->group_size != 64 || !aligned16(q->w) || !aligned16(q->s) || !aligned16(q->b)) fast = false;
+    // the streaming kernels take 4-bit weights with group size 64 or 128 (gate and up share one launch)
+    if (q->bits != 4 || (q->group_size != 64 && q->group_size != 128) || !aligned16(q->w) || !aligned16(q->s) || !aligned16(q->b))
+      fast = false;
   }
   RMLX_TRY(checked_u32(E, "num_experts", &sh->E));
   RMLX_TRY(checked_u32(D, "hidden_dim", &sh->D));
   RMLX_TRY(checked_u32(I, "intermediate_dim", &sh->I));
   if (!qmv_q4_supported(sh->I, sh->D, 64) || !qmv_q4_supported(sh->D, sh->I, 64)) fast = false;
+  if (up != nullptr && up->group_size != gate->group_size) fast = false;
   sh->fused = fused;
   sh->portable = !fast;
   return RMLX_OK;
@@ -351,15 +354,16 @@ int32_t run_expert_ffn(const rmlx_qweight* gate, const rmlx_qweight* up, const r
   a.w0 = gate->w; a.s0 = gate->s; a.b0 = gate->b;
   if (sh.fused) {
     a.w1 = gate->w + (size_t)sh.I * (sh.D / 8);
-    a.s1 = gate->s + (size_t)sh.I * (sh.D / 64);
-    a.b1 = gate->b + (size_t)sh.I * (sh.D / 64);
+    a.s1 = gate->s + (size_t)sh.I * (sh.D / gate->group_size);
+    a.b1 = gate->b + (size_t)sh.I * (sh.D / gate->group_size);
   } else {
     a.w1 = up->w; a.s1 = up->s; a.b1 = up->b;
   }
   const size_t rows_per_expert = sh.fused ? 2 * (size_t)sh.I : sh.I;
   a.N = sh.I; a.K = sh.D;
   a.expert_stride_w = rows_per_expert * (sh.D / 8);
-  a.expert_stride_s = rows_per_expert * (sh.D / 64);
+  a.expert_stride_s = rows_per_expert * (sh.D / gate->group_size);
+  a.group_size = gate->group_size;
   a.x = x; a.row_map = row_map;
   a.out = h; a.ld_out = sh.I; a.out_f32 = 0; a.dual = 1;
   a.chunk_tab = chunk_tab; a.n_chunks_dev = n_chunks; a.max_chunks = max_chunks; a.mr = 8;
@@ -369,7 +373,8 @@ int32_t run_expert_ffn(const rmlx_qweight* gate, const rmlx_qweight* up, const r
   d.w0 = down->w; d.s0 = down->s; d.b0 = down->b;
   d.N = sh.D; d.K = sh.I;
   d.expert_stride_w = (size_t)sh.D * (sh.I / 8);
-  d.expert_stride_s = (size_t)sh.D * (sh.I / 64);
+  d.expert_stride_s = (size_t)sh.D * (sh.I / down->group_size);
+  d.group_size = down->group_size;
   d.x = h; d.row_map = nullptr;
   d.out = y; d.ld_out = sh.D; d.out_f32 = y_f32; d.dual = 0;
   d.chunk_tab = chunk_tab; d.n_chunks_dev = n_chunks; d.max_chunks = max_chunks; d.mr = 8;
@@ -761,7 +766,7 @@ int32_t rmlx_hip_gather_qmm(const rmlx_array* x, const void* w_packed_dev, size_
   const uint32_t* w = static_cast<const uint32_t*>(w_packed_dev);
   const __half* sc = static_cast<const __half*>(scales_dev);
   const __half* bi = static_cast<const __half*>(biases_dev);
-  const bool fast = group_size == 64 && qmv_q4_supported(N32, K32, 64) && aligned16(w) && aligned16(sc) &&
+  const bool fast = qmv_q4_supported(N32, K32, group_size) && aligned16(w) && aligned16(sc) &&
                     aligned16(bi) && aligned16(xk);
   if (fast) {
     const uint32_t per = ((uint32_t)m_per_batch + 7) / 8, n_chunks = B32 * per;
@@ -777,6 +782,7 @@ int32_t rmlx_hip_gather_qmm(const rmlx_array* x, const void* w_packed_dev, size_
     a.x = xk; a.out = out_f16_dev; a.ld_out = N32;
     a.chunk_tab = static_cast<const uint32_t*>(tab.ptr); a.max_chunks = n_chunks;
     a.mr = m_per_batch >= 5 ? 8 : (m_per_batch >= 3 ? 4 : (m_per_batch == 2 ? 2 : 1));
+    a.group_size = group_size;
     RMLX_TRY(launch_qmv_q4(a, s));
   } else {
     GenericArgs g{w, sc, bi, xk, static_cast<__half*>(out_f16_dev), idx, (uint32_t)m_per_batch, rows, N32, K32,

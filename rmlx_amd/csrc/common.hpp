@@ -123,6 +123,7 @@ struct QmvArgs {
   uint32_t max_chunks;       // grid.y when chunk_tab != null
   uint32_t M;                // used when chunk_tab == null
   uint32_t mr;               // rows staged per chunk (1,2,4,8); 0 -> derive from M
+  uint32_t group_size;       // 64 (also when 0) or 128
 };
 int32_t launch_qmv_q4(const QmvArgs& a, hipStream_t s);
 bool qmv_q4_supported(uint32_t N, uint32_t K, uint32_t group_size);

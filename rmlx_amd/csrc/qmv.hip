@@ -52,6 +52,7 @@ struct KParams {
   void* out;
   uint32_t K, ld_out, M, out_f32;
   uint32_t ks;  // k-parts per pass (1, 2, 4 or 8); tiles per workgroup = 8 / ks
+  uint32_t gs128;  // quantisation group size 128 instead of 64
   uint32_t tpw;  // consecutive tiles per workgroup (> 1 only when one pass covers K: the staged activations are reused)
   const uint32_t* w1;
   const __half* s1;
@@ -152,7 +153,8 @@ __global__ __launch_bounds__(kThreads, (REUSE && MR == 8 && TILES == 2) ? 4 : 1)
   // ---- which weights: tile tw of this workgroup, k-part kp of every pass --------------------
   const uint32_t K = p.K, KS = p.ks, NT = kWaves / KS;
   const uint32_t kp = wave % KS, tw = wave / KS;
-  const uint32_t words_per_row = K >> 3, groups_per_row = K >> 6, slabs_total = K >> 7;
+  // group size 128 (p.gs128): one scale per slab, applied to both halves of it
+  const uint32_t words_per_row = K >> 3, groups_per_row = p.gs128 ? K >> 7 : K >> 6, slabs_total = K >> 7;
   constexpr bool pair = PAIR;
   const uint32_t rows_per_slot = pair ? 32u : 16u;  // weight rows (of one matrix) per wave tile slot
 
@@ -266,6 +268,12 @@ __global__ __launch_bounds__(kThreads, (REUSE && MR == 8 && TILES == 2) ? 4 : 1)
 #pragma unroll
     for (int t = 0; t < TILES; ++t) {
       sbv[t] = (u4){0u, 0u, 0u, 0u};
+      if (p.gs128) {  // four slabs = four halves; word `it` holds slab it's value twice
+        const unsigned short* hp = reinterpret_cast<const unsigned short*>(sbrow[t]) + sl;
+        const uint32_t h0 = my > 0 ? hp[0] : 0u, h1 = my > 1 ? hp[1] : 0u, h2 = my > 2 ? hp[2] : 0u, h3 = my > 3 ? hp[3] : 0u;
+        sbv[t] = (u4){h0 | (h0 << 16), h1 | (h1 << 16), h2 | (h2 << 16), h3 | (h3 << 16)};
+        continue;
+      }
       const uint32_t* sp = reinterpret_cast<const uint32_t*>(sbrow[t]) + sl;
       if (my == kSpwMax) {  // 4 slabs: one 16-byte load (4-byte aligned is enough for the hardware)
         const U4Unaligned v = *reinterpret_cast<const U4Unaligned*>(sp);
@@ -488,7 +496,7 @@ unsigned long long* g_qmv_trace = nullptr;
 #endif
 
 bool qmv_q4_supported(uint32_t N, uint32_t K, uint32_t group_size) {
-  return group_size == 64 && N % 16 == 0 && K % 512 == 0 && N > 0 && K > 0;
+  return (group_size == 64 || group_size == 128) && N % 16 == 0 && K % 512 == 0 && N > 0 && K > 0;
 }
 
 int32_t launch_qmv_q4(const QmvArgs& a, hipStream_t s) {
@@ -499,6 +507,7 @@ int32_t launch_qmv_q4(const QmvArgs& a, hipStream_t s) {
   p.x = a.x; p.row_map = a.row_map; p.chunk_tab = a.chunk_tab; p.n_chunks = a.n_chunks_dev;
   p.out = a.out; p.estride_w = a.expert_stride_w; p.estride_s = a.expert_stride_s;
   p.K = a.K; p.ld_out = a.ld_out; p.M = a.M; p.out_f32 = a.out_f32;
+  p.gs128 = a.group_size == 128 ? 1u : 0u;
 #ifdef QMV_TRACE
   p.trace = g_qmv_trace;
 #endif

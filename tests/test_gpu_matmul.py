@@ -457,6 +457,21 @@ def test_qmm_norm_identity_scaling_and_validation(hip):
         ops.qmm_norm(xd, qw, w16, DeviceBuffer.from_numpy(np.ones(2, np.float16)))
 
 
+@pytest.mark.parametrize("m,n,k", [(3, 1024, 4096), (8, 512, 1536), (13, 9216, 4096), (16, 2048, 512), (5, 64, 2048)])
+def test_multi_row_gemv_group_size_128(hip, m, n, k):
+    """Group size 128 on the streaming GEMV: one scale per 128-wide slab, applied to both of its halves."""
+    rng = np.random.default_rng(m + n + k)
+    words, s, b = make_weight(rng, n, k, 4, 128)
+    x = make_x(rng, m, k)
+    ref = model.qmm(x_as_f64(x, "f16"), words, s, b, 128, 4)
+    assert_close(_run(hip, words, s, b, x, 4, gs=128, kernel=1), ref, f"qmv gs128 M={m} N={n} K={k}")
+    # group positions: a weight that is non-zero in one group only
+    s2, b2 = np.zeros_like(s), np.zeros_like(b)
+    s2[:, -1] = s[:, -1]
+    ref2 = model.qmm(x_as_f64(x, "f16"), words, s2, b2, 128, 4)
+    assert_close(_run(hip, words, s2, b2, x, 4, gs=128, kernel=1), ref2, "last group only")
+
+
 @pytest.mark.parametrize("m,n,k", [(13, 9216, 4096), (16, 9216, 4096), (16, 8192, 1536), (8, 16384, 512), (9, 8192, 2048)])
 def test_qmv_paired_tiles(hip, m, n, k):
     """Shapes whose 8-row chunks take two 16-row tiles per wave (grid still covers the CUs)."""

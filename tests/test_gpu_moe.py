@@ -159,11 +159,11 @@ def _gather_setup(rng, E, n, k, batch, mpb, dtype=np.float16):
 
 
 @pytest.mark.parametrize("E,n,k,batch,mpb", [(2, 4, 32, 2, 1), (4, 64, 512, 9, 1), (8, 128, 1024, 5, 3),
-                                              (3, 48, 1536, 4, 11), (128, 1536, 4096, 32, 1)])
+                                              (3, 48, 1536, 4, 11), (128, 1536, 4096, 32, 1), (6, 256, 2048, 7, 2)])
 def test_gather_qmm_matches_oracle(hip, E, n, k, batch, mpb):
     from rmlx_amd import ops
     rng = np.random.default_rng(E * 7 + n)
-    gs = 32 if k == 32 else 64
+    gs = 32 if k == 32 else (128 if k == 2048 else 64)
     from rmlx_amd.runtime import DeviceBuffer
     words, s, b = make_weight(rng, n, k, 4, gs, lead=(E,))
     x = rng.standard_normal((batch, mpb, k)).astype(np.float16)
@@ -350,7 +350,8 @@ def test_random_moe_shapes(hip):
 
 
 @pytest.mark.parametrize("bits,gs,D,I,fused", [(8, 64, 512, 512, False), (4, 32, 512, 1024, True), (4, 128, 384, 640, False),
-                                               (8, 32, 96, 160, True), (2, 64, 256, 128, False)])
+                                               (8, 32, 96, 160, True), (2, 64, 256, 128, False),
+                                               (4, 128, 512, 1024, True), (4, 128, 1024, 1536, False)])  # the last two: streaming kernels, group 128
 def test_moe_on_the_portable_kernels(hip, bits, gs, D, I, fused):
     """Expert weights the streaming GEMV does not take (8- or 2-bit, group sizes 32 / 128, dimensions that are
     no multiples of 512) run the same block on the portable kernels: routed block (one call and grouped) and
@@ -358,7 +359,7 @@ def test_moe_on_the_portable_kernels(hip, bits, gs, D, I, fused):
     from rmlx_amd import ops
     from rmlx_amd.runtime import DeviceBuffer
     rng = np.random.default_rng(bits * 100 + gs + D)
-    E, T, K = 5, 6, 2
+    E, T, K = 5, 6 if gs != 128 or D % 512 else 21, 2
 
     def weight(n, k):
         return make_weight(rng, n, k, bits if bits != 2 else 4, gs, lead=(E,)) if bits != 2 else _two_bit(rng, E, n, k, gs)
