@@ -177,7 +177,7 @@ int32_t run_matmul_plain(const rmlx_qweight* qw, const void* x, int32_t x_dtype,
     else kernel = KERNEL_GENERIC;
   } else if ((kernel == KERNEL_QMV && !can_qmv && !can_m1) || (kernel == KERNEL_QMV_ROWS && !can_qmv)) {
     return fail(RMLX_INVALID_SHAPE,
-                "qmv kernel requires bits in {4,8}, group_size=64, N %% 16 == 0, K %% 512 == 0 (4-bit) or "
+                "qmv kernel requires bits in {4,8}, group_size 64 (4-bit: or 128), N %% 16 == 0, K %% 512 == 0 (4-bit) or "
                 "K %% 2048 == 0 (8-bit) and 16-byte aligned buffers (N=%u K=%u bits=%u group_size=%u)",
                 N, K, qw->bits, qw->group_size);
   } else if (kernel == KERNEL_QMM && !can_qmm) {
