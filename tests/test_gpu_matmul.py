@@ -457,6 +457,27 @@ def test_qmm_norm_identity_scaling_and_validation(hip):
         ops.qmm_norm(xd, qw, w16, DeviceBuffer.from_numpy(np.ones(2, np.float16)))
 
 
+@pytest.mark.parametrize("m", [1, 2, 4, 40])
+def test_vocabulary_sized_projection(hip, m):
+    """N = 151 936 output rows (a vocabulary projection, 311 MB of 4-bit weights): rows at both ends and a
+    random sample are checked against the oracle, every output must be finite."""
+    from rmlx_amd import ops
+    from rmlx_amd.runtime import DeviceBuffer
+    rng = np.random.default_rng(151936 + m)
+    n, k = 151936, 4096
+    words = rng.integers(0, 2**32, size=(n, k // 8), dtype=np.uint64).astype(np.uint32)
+    s = rng.uniform(0.005, 0.02, size=(n, k // 64)).astype(np.float16)
+    b = (-8 * s.astype(np.float32)).astype(np.float16)
+    x = make_x(rng, m, k)
+    print(f"vocabulary projection M={m}", flush=True)
+    qw = ops.QuantizedWeight.from_numpy(words, s, b, 64, 4)
+    out = ops.affine_quantized_matmul_batched(DeviceBuffer.from_numpy(x), qw).numpy()
+    assert out.shape == (m, n) and np.all(np.isfinite(out))
+    rows = np.unique(np.concatenate([np.arange(256), np.arange(n - 256, n), rng.integers(0, n, size=512)]))
+    ref = model.qmm(x_as_f64(x, "f16"), words[rows], s[rows], b[rows], 64, 4)
+    assert_close(out[:, rows], ref, f"M={m}")
+
+
 @pytest.mark.parametrize("m,n,k", [(3, 1024, 4096), (8, 512, 1536), (13, 9216, 4096), (16, 2048, 512), (5, 64, 2048)])
 def test_multi_row_gemv_group_size_128(hip, m, n, k):
     """Group size 128 on the streaming GEMV: one scale per 128-wide slab, applied to both of its halves."""
