@@ -98,7 +98,7 @@ def bench_matmul(ops, rt, timer, rng, m, n, k, bits, x_dtype, steps, warmup, min
     return res
 
 
-def bench_moe(ops, rt, timer, rng, T, steps, warmup, experts):
+def bench_moe(ops, rt, timer, rng, T, steps, warmup, experts, bits=4):
     from oracle import model
     gate_up, down, gh, dh = experts
     x = rng.standard_normal((T, 4096)).astype(np.float16)
@@ -113,14 +113,14 @@ def bench_moe(ops, rt, timer, rng, T, steps, warmup, experts):
     ms = timer.run(run, steps, warmup)
     idx, w, _, _ = model.topk_route(logits, 8)
     distinct = len(np.unique(idx))
-    nbytes = distinct * 10616832 + T * 4096 * 2 * 2 + T * 128 * 4
+    nbytes = distinct * (18874368 * bits // 8 + 1179648) + T * 4096 * 2 * 2 + T * 128 * 4
     res = {"us": ms * 1e3, "distinct_experts": distinct, "bytes": nbytes, "gbs": nbytes / (ms * 1e-3) / 1e9,
            "flops": 2 * 8 * T * (4096 * 3072 + 1536 * 4096)}
     toks = np.arange(min(T, 2))
     sel = (toks[:, None] * 8 + np.arange(8)[None, :]).reshape(-1)
     gate = tuple(a[:, :1536] for a in gate_up)
     up = tuple(a[:, 1536:] for a in gate_up)
-    ref = model.moe_forward(x[toks], idx[sel], w[sel], gate, up, down, 64, 8)
+    ref = model.moe_forward(x[toks], idx[sel], w[sel], gate, up, down, 64, 8, bits=bits)
     err = float(np.abs(out.numpy()[toks].astype(np.float64) - ref).max())
     res["max_err"], res["tol"], res["pass"] = err, model.tolerance(ref), bool(err <= model.tolerance(ref))
     return res
@@ -288,6 +288,15 @@ def main():
             r = bench_moe(ops, rt, timer, rng, T, max(50, args.steps // 10), 10, experts)
             r["hbm_frac"] = r["gbs"] / HBM_PEAK_GBS
             extra[f"moe_q4_T{T}"] = r
+        del experts, gate_up, down
+        gate_up = make_weight(rng, 3072, 4096, 8, lead=(128,))
+        down = make_weight(rng, 4096, 1536, 8, lead=(128,))
+        experts = (gate_up, down, ops.QuantizedWeight.from_numpy(*gate_up, 64, 8),
+                   ops.QuantizedWeight.from_numpy(*down, 64, 8))
+        for T in (4, 32):
+            r = bench_moe(ops, rt, timer, rng, T, max(50, args.steps // 10), 10, experts, bits=8)
+            r["hbm_frac"] = r["gbs"] / HBM_PEAK_GBS
+            extra[f"moe_q8_T{T}"] = r
 
     line = {
         "metric": "Q4 qmv HBM GB/s (M=1, K=N=4096)",

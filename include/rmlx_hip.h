@@ -230,8 +230,9 @@ int32_t rmlx_hip_silu_gate(const void* gate_in_f16_dev, const void* up_in_f16_de
  * Literal contract: `n_items` (expert_idx, input [batch_i, D]) pairs, inputs packed one
  * after another in x ([sum batch_i, D] f16); out receives the per-item outputs in the same
  * packing.  Per item: y = (silu(x Wg^T) * (x Wu^T)) Wd^T with stacked expert weights (the streaming kernels
- * take 4-bit weights with group size 64 or 128 and dimensions in multiples of 512; every other 2- / 4- / 8-bit weight the
- * type admits runs the same block on the portable kernels)
+ * take 4-bit weights with group size 64 or 128 and dimensions in multiples of 512, and 8-bit weights with group size 64
+ * and dimensions in multiples of 256; every other 2- / 4- / 8-bit weight the type admits runs the same block on the
+ * portable kernels)
  * gate/up [E, I, D] and down [E, D, I].  `up` may be NULL when `gate` holds the fused
  * [E, 2I, D] layout (gate rows first).  expert_idx and batch_sizes are HOST arrays.
  * Validation as the reference: idx < E, n_items == 0 -> nothing to do. */

@@ -178,7 +178,7 @@ int32_t run_matmul_plain(const rmlx_qweight* qw, const void* x, int32_t x_dtype,
   } else if ((kernel == KERNEL_QMV && !can_qmv && !can_m1) || (kernel == KERNEL_QMV_ROWS && !can_qmv)) {
     return fail(RMLX_INVALID_SHAPE,
                 "qmv kernel requires bits in {4,8}, group_size 64 (4-bit: or 128), N %% 16 == 0, K %% 512 == 0 (4-bit) or "
-                "K %% 2048 == 0 (8-bit) and 16-byte aligned buffers (N=%u K=%u bits=%u group_size=%u)",
+                "K %% 256 == 0 (8-bit) and 16-byte aligned buffers (N=%u K=%u bits=%u group_size=%u)",
                 N, K, qw->bits, qw->group_size);
   } else if (kernel == KERNEL_QMM && !can_qmm) {
     return fail(RMLX_INVALID_SHAPE,
@@ -283,7 +283,7 @@ int32_t check_out(const char* who, size_t have, size_t need) {
 struct ExpertShapes {
   uint32_t E, D, I;
   bool fused;
-  bool portable;  // not Q4 / group 64 / dims in multiples of 512: the portable kernels run the block
+  bool portable;  // weights the streaming kernels do not take: the portable kernels run the block
 };
 
 int32_t check_expert_weights(const char* who, const rmlx_qweight* gate, const rmlx_qweight* up,
@@ -303,22 +303,27 @@ int32_t check_expert_weights(const char* who, const rmlx_qweight* gate, const rm
     if (q == nullptr) continue;
     if (q->bits != 2 && q->bits != 4 && q->bits != 8)
       return fail(RMLX_NOT_FOUND, "%s: no kernel for %u-bit expert weights (2, 4 and 8 are implemented)", who, q->bits);
-    // the streaming kernels take 4-bit weights with group size 64 or 128 (gate and up share one launch)
-    if (q->bits != 4 || (q->group_size != 64 && q->group_size != 128) || !aligned16(q->w) || !aligned16(q->s) || !aligned16(q->b))
-      fast = false;
+    // the streaming kernels take 4-bit weights with group size 64 or 128 and 8-bit weights with group size 64,
+    // the same width for all three projections (gate and up share one launch)
+    const bool gs_ok = q->bits == 4 ? (q->group_size == 64 || q->group_size == 128) : (q->bits == 8 && q->group_size == 64);
+    if (!gs_ok || q->bits != gate->bits || !aligned16(q->w) || !aligned16(q->s) || !aligned16(q->b)) fast = false;
   }
   RMLX_TRY(checked_u32(E, "num_experts", &sh->E));
   RMLX_TRY(checked_u32(D, "hidden_dim", &sh->D));
   RMLX_TRY(checked_u32(I, "intermediate_dim", &sh->I));
-  if (!qmv_q4_supported(sh->I, sh->D, 64) || !qmv_q4_supported(sh->D, sh->I, 64)) fast = false;
+  if (gate->bits == 8) {
+    if (!qmv_q8_supported(sh->I, sh->D, 64) || !qmv_q8_supported(sh->D, sh->I, 64)) fast = false;
+  } else if (!qmv_q4_supported(sh->I, sh->D, 64) || !qmv_q4_supported(sh->D, sh->I, 64)) {
+    fast = false;
+  }
   if (up != nullptr && up->group_size != gate->group_size) fast = false;
   sh->fused = fused;
   sh->portable = !fast;
   return RMLX_OK;
 }
 
-// The same block on the portable kernels, for expert weights the streaming GEMV does not take (2- or 8-bit,
-// group sizes 32 / 128, dimensions that are no multiples of 512): every position multiplies with its own
+// The same block on the portable kernels, for expert weights the streaming GEMV does not take (2-bit,
+// group size 32, 8-bit at group size 128, dimensions that are no multiples of 512 (4-bit) or 256 / 16 (8-bit)): every position multiplies with its own
 // expert's rows.  x: f16 [positions, D] (already gathered); expert_of: device u32 [positions]; y: f16 [positions, D].
 int32_t run_expert_ffn_portable(const rmlx_qweight* gate, const rmlx_qweight* up, const rmlx_qweight* down,
                                 const ExpertShapes& sh, const __half* x, const uint32_t* expert_of, uint32_t positions,
@@ -350,10 +355,11 @@ int32_t run_expert_ffn(const rmlx_qweight* gate, const rmlx_qweight* up, const r
                        const ExpertShapes& sh, const __half* x, const uint32_t* row_map,
                        const uint32_t* chunk_tab, const uint32_t* n_chunks, uint32_t max_chunks, __half* h,
                        void* y, int y_f32, hipStream_t stream) {
+  const uint32_t per = 32 / gate->bits;  // values per u32 word: 8 (4-bit) or 4 (8-bit)
   QmvArgs a{};
   a.w0 = gate->w; a.s0 = gate->s; a.b0 = gate->b;
   if (sh.fused) {
-    a.w1 = gate->w + (size_t)sh.I * (sh.D / 8);
+    a.w1 = gate->w + (size_t)sh.I * (sh.D / per);
     a.s1 = gate->s + (size_t)sh.I * (sh.D / gate->group_size);
     a.b1 = gate->b + (size_t)sh.I * (sh.D / gate->group_size);
   } else {
@@ -361,24 +367,24 @@ int32_t run_expert_ffn(const rmlx_qweight* gate, const rmlx_qweight* up, const r
   }
   const size_t rows_per_expert = sh.fused ? 2 * (size_t)sh.I : sh.I;
   a.N = sh.I; a.K = sh.D;
-  a.expert_stride_w = rows_per_expert * (sh.D / 8);
+  a.expert_stride_w = rows_per_expert * (sh.D / per);
   a.expert_stride_s = rows_per_expert * (sh.D / gate->group_size);
   a.group_size = gate->group_size;
   a.x = x; a.row_map = row_map;
   a.out = h; a.ld_out = sh.I; a.out_f32 = 0; a.dual = 1;
   a.chunk_tab = chunk_tab; a.n_chunks_dev = n_chunks; a.max_chunks = max_chunks; a.mr = 8;
-  RMLX_TRY(launch_qmv_q4(a, stream));
+  RMLX_TRY(gate->bits == 8 ? launch_qmv_q8_tab(a, stream) : launch_qmv_q4(a, stream));
 
   QmvArgs d{};
   d.w0 = down->w; d.s0 = down->s; d.b0 = down->b;
   d.N = sh.D; d.K = sh.I;
-  d.expert_stride_w = (size_t)sh.D * (sh.I / 8);
+  d.expert_stride_w = (size_t)sh.D * (sh.I / per);
   d.expert_stride_s = (size_t)sh.D * (sh.I / down->group_size);
   d.group_size = down->group_size;
   d.x = h; d.row_map = nullptr;
   d.out = y; d.ld_out = sh.D; d.out_f32 = y_f32; d.dual = 0;
   d.chunk_tab = chunk_tab; d.n_chunks_dev = n_chunks; d.max_chunks = max_chunks; d.mr = 8;
-  return launch_qmv_q4(d, stream);
+  return gate->bits == 8 ? launch_qmv_q8_tab(d, stream) : launch_qmv_q4(d, stream);
 }
 
 }  // namespace

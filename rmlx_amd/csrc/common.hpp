@@ -131,6 +131,8 @@ bool qmv_q4_supported(uint32_t N, uint32_t K, uint32_t group_size);
 bool qmv_q8_supported(uint32_t N, uint32_t K, uint32_t group_size);
 int32_t launch_qmv_q8(const uint32_t* w, const __half* s, const __half* b, const __half* x, __half* out, uint32_t M,
                       uint32_t N, uint32_t K, hipStream_t stream);
+// chunk-table mode for the expert projections (expert strides in u32 words / halves as for the 4-bit kernel)
+int32_t launch_qmv_q8_tab(const QmvArgs& a, hipStream_t stream);
 // Single-row GEMV (qmv_m1.hip): 4- or 8-bit weights, group size 32 / 64 / 128, f16 activations; M rows are
 // passes of up to four rows over the weights (grid.y); the store epilogue (EPI_*) is fused.
 bool qmv_m1_supported(uint32_t N, uint32_t K, uint32_t group_size, uint32_t bits);

@@ -457,6 +457,16 @@ def test_qmm_norm_identity_scaling_and_validation(hip):
         ops.qmm_norm(xd, qw, w16, DeviceBuffer.from_numpy(np.ones(2, np.float16)))
 
 
+@pytest.mark.parametrize("m,n,k", [(3, 512, 256), (16, 1024, 768), (9, 4096, 11008), (5, 64, 2304), (16, 256, 4096)])
+def test_q8_multi_row_gemv_any_k_multiple_of_256(hip, m, n, k):
+    """The 8-bit streaming GEMV takes K in multiples of 256: waves whose slabs lie past K sit the pass out."""
+    rng = np.random.default_rng(m + n + k)
+    words, s, b = make_weight(rng, n, k, 8)
+    x = make_x(rng, m, k)
+    ref = model.qmm(x_as_f64(x, "f16"), words, s, b, 64, 8)
+    assert_close(_run(hip, words, s, b, x, 8, kernel=6), ref, f"q8 qmv M={m} N={n} K={k}")
+
+
 @pytest.mark.parametrize("m", [1, 2, 4, 40])
 def test_vocabulary_sized_projection(hip, m):
     """N = 151 936 output rows (a vocabulary projection, 311 MB of 4-bit weights): rows at both ends and a

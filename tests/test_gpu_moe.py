@@ -351,15 +351,17 @@ def test_random_moe_shapes(hip):
 
 @pytest.mark.parametrize("bits,gs,D,I,fused", [(8, 64, 512, 512, False), (4, 32, 512, 1024, True), (4, 128, 384, 640, False),
                                                (8, 32, 96, 160, True), (2, 64, 256, 128, False),
-                                               (4, 128, 512, 1024, True), (4, 128, 1024, 1536, False)])  # the last two: streaming kernels, group 128
-def test_moe_on_the_portable_kernels(hip, bits, gs, D, I, fused):
-    """Expert weights the streaming GEMV does not take (8- or 2-bit, group sizes 32 / 128, dimensions that are
-    no multiples of 512) run the same block on the portable kernels: routed block (one call and grouped) and
-    `ExpertGroup::grouped_forward`, against the oracle."""
+                                               (4, 128, 512, 1024, True), (4, 128, 1024, 1536, False),   # streaming kernels, group 128
+                                               (8, 64, 1024, 1536, True), (8, 64, 4096, 768, False)])   # streaming 8-bit kernel
+def test_moe_other_bit_widths_and_group_sizes(hip, bits, gs, D, I, fused):
+    """Expert weights beyond 4 bits / group 64: 8-bit (group 64) and 4-bit group 128 weights stream through the
+    fast kernels when the dimensions allow; 2-bit weights, group size 32 and other dimensions run the same
+    block on the portable kernels.  Routed block (one call and grouped) and `ExpertGroup::grouped_forward`,
+    against the oracle."""
     from rmlx_amd import ops
     from rmlx_amd.runtime import DeviceBuffer
     rng = np.random.default_rng(bits * 100 + gs + D)
-    E, T, K = 5, 6 if gs != 128 or D % 512 else 21, 2
+    E, T, K = 5, 21 if D >= 1024 or (gs == 128 and D % 512 == 0) else 6, 2
 
     def weight(n, k):
         return make_weight(rng, n, k, bits if bits != 2 else 4, gs, lead=(E,)) if bits != 2 else _two_bit(rng, E, n, k, gs)
