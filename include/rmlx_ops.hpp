@@ -386,6 +386,9 @@ class MoeExperts {
                                                out.nbytes(), raw(stream)));
     return out;
   }
+  // Average rows per expert from which the expert projections (here and in ExpertGroup) run on the grouped
+  // MFMA GEMM instead of the streaming GEMV; 0 = never; process-wide.  Returns the previous value.
+  static uint32_t set_expert_gemm_min_rows(uint32_t min_rows) { return rmlx_hip_set_expert_gemm_min_rows(min_rows); }
   // routing included: gate_logits [T, E]
   Array forward(const Array& x, const Array& gate_logits, size_t top_k, const Array* expert_bias = nullptr,
                 const Stream* stream = nullptr) const {

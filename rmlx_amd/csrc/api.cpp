@@ -1,6 +1,7 @@
 // Host side of the C ABI: validation (same rules and messages as the reference's Rust entry
 // points), the dispatch ladder, and the composition of the MoE block.  No arithmetic happens
 // here and there is no CPU fallback: every path ends in a HIP kernel launch or an error.
+#include <atomic>
 #include <cinttypes>
 #include <cstring>
 #include <map>
@@ -284,7 +285,12 @@ struct ExpertShapes {
   uint32_t E, D, I;
   bool fused;
   bool portable;  // weights the streaming kernels do not take: the portable kernels run the block
+  bool gemm;      // the grouped GEMM takes them too (batches with many rows per expert)
 };
+
+// Average rows per expert from which the expert projections run on the grouped GEMM instead of the streaming
+// GEMV (which re-reads an expert's weights once per 8 rows); 0 = never.  Measured crossover.
+std::atomic<uint32_t> g_expert_gemm_min_rows{12};
 
 int32_t check_expert_weights(const char* who, const rmlx_qweight* gate, const rmlx_qweight* up,
                              const rmlx_qweight* down, ExpertShapes* sh) {
@@ -319,7 +325,15 @@ int32_t check_expert_weights(const char* who, const rmlx_qweight* gate, const rm
   if (up != nullptr && up->group_size != gate->group_size) fast = false;
   sh->fused = fused;
   sh->portable = !fast;
+  sh->gemm = fast && gate->group_size == 64 && down->group_size == 64 &&
+             qmm_rw_grouped_supported(sh->I, sh->D, 64, gate->bits) && qmm_rw_grouped_supported(sh->D, sh->I, 64, gate->bits);
   return RMLX_OK;
+}
+
+// true when `rows` positions over at most `groups` experts are multiplied by the grouped GEMM
+bool expert_gemm_pays(const ExpertShapes& sh, uint64_t rows, uint64_t groups) {
+  const uint32_t min_rows = g_expert_gemm_min_rows.load(std::memory_order_relaxed);
+  return sh.gemm && min_rows != 0 && groups != 0 && rows >= (uint64_t)min_rows * groups;
 }
 
 // The same block on the portable kernels, for expert weights the streaming GEMV does not take (2-bit,
@@ -354,8 +368,34 @@ int32_t run_expert_ffn_portable(const rmlx_qweight* gate, const rmlx_qweight* up
 int32_t run_expert_ffn(const rmlx_qweight* gate, const rmlx_qweight* up, const rmlx_qweight* down,
                        const ExpertShapes& sh, const __half* x, const uint32_t* row_map,
                        const uint32_t* chunk_tab, const uint32_t* n_chunks, uint32_t max_chunks, __half* h,
-                       void* y, int y_f32, hipStream_t stream) {
+                       void* y, int y_f32, bool gemm, hipStream_t stream) {
   const uint32_t per = 32 / gate->bits;  // values per u32 word: 8 (4-bit) or 4 (8-bit)
+  if (gemm) {  // the table holds row tiles of kGroupedTileRows rows and n_chunks its length
+    GroupedQmmArgs a{};
+    a.w = gate->w; a.s = gate->s; a.b = gate->b;
+    if (sh.fused) {
+      a.w1 = gate->w + (size_t)sh.I * (sh.D / per);
+      a.s1 = gate->s + (size_t)sh.I * (sh.D / 64);
+      a.b1 = gate->b + (size_t)sh.I * (sh.D / 64);
+    } else {
+      a.w1 = up->w; a.s1 = up->s; a.b1 = up->b;
+    }
+    const size_t rows = sh.fused ? 2 * (size_t)sh.I : sh.I;
+    a.N = sh.I; a.K = sh.D; a.bits = gate->bits;
+    a.expert_stride_w = rows * (sh.D / per);
+    a.expert_stride_s = rows * (sh.D / 64);
+    a.x = x; a.row_map = row_map; a.out = h; a.out_f32 = 0;
+    a.tile_tab = chunk_tab; a.n_tiles_dev = n_chunks; a.max_tiles = max_chunks;
+    RMLX_TRY(launch_qmm_rw_grouped(a, stream));
+    GroupedQmmArgs d{};
+    d.w = down->w; d.s = down->s; d.b = down->b;
+    d.N = sh.D; d.K = sh.I; d.bits = down->bits;
+    d.expert_stride_w = (size_t)sh.D * (sh.I / per);
+    d.expert_stride_s = (size_t)sh.D * (sh.I / 64);
+    d.x = h; d.row_map = nullptr; d.out = y; d.out_f32 = y_f32;
+    d.tile_tab = chunk_tab; d.n_tiles_dev = n_chunks; d.max_tiles = max_chunks;
+    return launch_qmm_rw_grouped(d, stream);
+  }
   QmvArgs a{};
   a.w0 = gate->w; a.s0 = gate->s; a.b0 = gate->b;
   if (sh.fused) {
@@ -774,12 +814,30 @@ int32_t rmlx_hip_gather_qmm(const rmlx_array* x, const void* w_packed_dev, size_
   const __half* bi = static_cast<const __half*>(biases_dev);
   const bool fast = qmv_q4_supported(N32, K32, group_size) && aligned16(w) && aligned16(sc) &&
                     aligned16(bi) && aligned16(xk);
-  if (fast) {
+  const uint32_t gemm_min_rows = g_expert_gemm_min_rows.load(std::memory_order_relaxed);
+  if (fast && gemm_min_rows != 0 && m_per_batch >= gemm_min_rows && qmm_rw_grouped_supported(N32, K32, group_size, 4)) {
+    // many rows per entry: row tiles of one expert each on the grouped MFMA GEMM
+    const uint32_t per = ((uint32_t)m_per_batch + kGroupedTileRows - 1) / kGroupedTileRows;
+    const uint64_t n_tiles = (uint64_t)B32 * per;
+    if (n_tiles > 0x7FFFFFu) return fail(RMLX_INVALID_SHAPE, "gather_qmm: too many row tiles (%" PRIu64 ")", n_tiles);
+    Scratch tab;
+    RMLX_TRY(tab.alloc((size_t)n_tiles * 12 + 4, s));
+    uint32_t* t = static_cast<uint32_t*>(tab.ptr);
+    RMLX_TRY(launch_build_gather_chunks(idx, B32, (uint32_t)m_per_batch, E32, kGroupedTileRows, t, t + 3 * n_tiles, s));
+    GroupedQmmArgs a{};
+    a.w = w; a.s = sc; a.b = bi;
+    a.N = N32; a.K = K32; a.bits = 4;
+    a.expert_stride_w = (uint64_t)n * (k / 8);
+    a.expert_stride_s = (uint64_t)n * gpr;
+    a.x = xk; a.out = out_f16_dev;
+    a.tile_tab = t; a.n_tiles_dev = t + 3 * n_tiles; a.max_tiles = (uint32_t)n_tiles;
+    RMLX_TRY(launch_qmm_rw_grouped(a, s));
+  } else if (fast) {
     const uint32_t per = ((uint32_t)m_per_batch + 7) / 8, n_chunks = B32 * per;
     if (n_chunks > 65535) return fail(RMLX_INVALID_SHAPE, "gather_qmm: too many row chunks (%u)", n_chunks);
     Scratch tab;
     RMLX_TRY(tab.alloc((size_t)n_chunks * 12, s));
-    RMLX_TRY(launch_build_gather_chunks(idx, B32, (uint32_t)m_per_batch, E32, static_cast<uint32_t*>(tab.ptr), s));
+    RMLX_TRY(launch_build_gather_chunks(idx, B32, (uint32_t)m_per_batch, E32, 8, static_cast<uint32_t*>(tab.ptr), nullptr, s));
     QmvArgs a{};
     a.w0 = w; a.s0 = sc; a.b0 = bi;
     a.N = N32; a.K = K32;
@@ -857,7 +915,7 @@ int32_t rmlx_hip_moe_sort(const uint32_t* expert_indices_dev, size_t n_assign, s
   RMLX_TRY(checked_u32(n_experts, "n_experts", &E));
   if (E == 0) return fail(RMLX_INVALID_SHAPE, "moe_sort: n_experts must be non-zero");
   hipStream_t s = (hipStream_t)stream;
-  RMLX_TRY(launch_moe_sort(expert_indices_dev, A, E, 1, sorted_assign_dev, nullptr, nullptr, nullptr, offsets_dev, nullptr, nullptr, s));
+  RMLX_TRY(launch_moe_sort(expert_indices_dev, A, E, 1, sorted_assign_dev, nullptr, nullptr, nullptr, offsets_dev, nullptr, nullptr, 8, s));
   return finish(s);
 }
 
@@ -909,14 +967,19 @@ int32_t rmlx_hip_expert_group_grouped_forward(const rmlx_qweight* gate, const rm
   if (x == nullptr || expert_idx_host == nullptr || batch_sizes_host == nullptr)
     return fail(RMLX_INVALID_SHAPE, "ExpertGroup: null argument");
   size_t total = 0;
+  for (size_t i = 0; i < n_items; ++i) total += batch_sizes_host[i];
+  // row chunks of one expert each: 8 rows for the streaming GEMV, whole row tiles for the grouped GEMM
+  const bool gemm = expert_gemm_pays(sh, total, n_items);
+  const uint32_t chunk_rows = gemm ? kGroupedTileRows : 8u;
   std::vector<uint32_t> tab;
+  total = 0;
   for (size_t i = 0; i < n_items; ++i) {
     if (expert_idx_host[i] >= sh.E)
       return fail(RMLX_INVALID_SHAPE, "ExpertGroup: expert_idx %u >= num_experts %u", expert_idx_host[i], sh.E);
-    for (uint32_t r = 0; r < batch_sizes_host[i]; r += 8) {
+    for (uint32_t r = 0; r < batch_sizes_host[i]; r += chunk_rows) {
       tab.push_back(expert_idx_host[i]);
       tab.push_back((uint32_t)(total + r));
-      tab.push_back(batch_sizes_host[i] - r < 8u ? batch_sizes_host[i] - r : 8u);
+      tab.push_back(batch_sizes_host[i] - r < chunk_rows ? batch_sizes_host[i] - r : chunk_rows);
     }
     total += batch_sizes_host[i];
   }
@@ -932,6 +995,7 @@ int32_t rmlx_hip_expert_group_grouped_forward(const rmlx_qweight* gate, const rm
   if (total == 0) return RMLX_OK;
   const uint32_t n_chunks = (uint32_t)(tab.size() / 3);
   if (n_chunks > 65535) return fail(RMLX_INVALID_SHAPE, "ExpertGroup: too many row chunks (%u)", n_chunks);
+  tab.push_back(n_chunks);  // the table's length travels behind it
 
   hipStream_t s = (hipStream_t)stream;
   Scratch cast, dtab, h;
@@ -957,8 +1021,9 @@ int32_t rmlx_hip_expert_group_grouped_forward(const rmlx_qweight* gate, const rm
   RMLX_HIP_CHECK(hipMemcpyAsync(dtab.ptr, tab.data(), tab.size() * 4, hipMemcpyHostToDevice, s));
   RMLX_HIP_CHECK(hipStreamSynchronize(s));  // `tab` is pageable host memory owned by this call
   RMLX_TRY(h.alloc(total * sh.I * 2, s));
-  RMLX_TRY(run_expert_ffn(gate, up, down, sh, xk, nullptr, static_cast<const uint32_t*>(dtab.ptr), nullptr, n_chunks,
-                          static_cast<__half*>(h.ptr), out_f16_dev, 0, s));
+  const uint32_t* dev_tab = static_cast<const uint32_t*>(dtab.ptr);
+  RMLX_TRY(run_expert_ffn(gate, up, down, sh, xk, nullptr, dev_tab, dev_tab + 3 * (size_t)n_chunks, n_chunks,
+                          static_cast<__half*>(h.ptr), out_f16_dev, 0, gemm, s));
   return finish(s);
 }
 
@@ -987,7 +1052,10 @@ int32_t moe_grouped_impl(const rmlx_qweight* gate, const rmlx_qweight* up, const
   RMLX_TRY(checked_u32(T * top_k, "seq_len * top_k", &A));
   RMLX_TRY(check_out("MoeLayer", out_bytes, T * sh.D * 2));
   if (T == 0) return RMLX_OK;
-  const uint32_t max_chunks = A / 8 + (A < sh.E ? A : sh.E);
+  // many rows per expert: the grouped GEMM over row tiles instead of the streaming GEMV over chunks of 8 rows
+  const bool gemm = route == nullptr && expert_gemm_pays(sh, A, sh.E);
+  const uint32_t chunk_rows = gemm ? kGroupedTileRows : 8u;
+  const uint32_t max_chunks = A / chunk_rows + (A < sh.E ? A : sh.E);
   if (max_chunks > 65535) return fail(RMLX_INVALID_SHAPE, "MoeLayer: too many row chunks (%u); split the batch", max_chunks);
 
   hipStream_t s = (hipStream_t)stream;
@@ -1031,11 +1099,12 @@ int32_t moe_grouped_impl(const rmlx_qweight* gate, const rmlx_qweight* up, const
     RMLX_TRY(launch_route_sort_small(route->logits, route->bias, T32, sh.E, (uint32_t)top_k, 1, route->idx_out, route->w_out,
                                      sorted, sorted_tok, inv, chunk_tab, n_chunks, s));
   else
-    RMLX_TRY(launch_moe_sort(expert_indices_dev, A, sh.E, (uint32_t)top_k, sorted, sorted_tok, inv, nullptr, nullptr, chunk_tab, n_chunks, s));
+    RMLX_TRY(launch_moe_sort(expert_indices_dev, A, sh.E, (uint32_t)top_k, sorted, sorted_tok, inv, nullptr, nullptr, chunk_tab, n_chunks,
+                             chunk_rows, s));
   RMLX_TRY(h.alloc((size_t)A * sh.I * 2, s));
   RMLX_TRY(y.alloc((size_t)A * sh.D * 4, s));
   RMLX_TRY(run_expert_ffn(gate, up, down, sh, xk, sorted_tok, chunk_tab, n_chunks, max_chunks,
-                          static_cast<__half*>(h.ptr), y.ptr, 1, s));
+                          static_cast<__half*>(h.ptr), y.ptr, 1, gemm, s));
   RMLX_TRY(launch_moe_combine(static_cast<const float*>(y.ptr), inv, expert_weights_dev, T32, (uint32_t)top_k, sh.D,
                               static_cast<__half*>(out_f16_dev), s));
   return finish(s);
@@ -1043,6 +1112,10 @@ int32_t moe_grouped_impl(const rmlx_qweight* gate, const rmlx_qweight* up, const
 }  // namespace
 
 extern "C" {
+
+uint32_t rmlx_hip_set_expert_gemm_min_rows(uint32_t min_rows) {
+  return g_expert_gemm_min_rows.exchange(min_rows, std::memory_order_relaxed);
+}
 
 int32_t rmlx_hip_moe_forward_grouped(const rmlx_qweight* gate, const rmlx_qweight* up, const rmlx_qweight* down,
                                      const rmlx_array* x, const uint32_t* expert_indices_dev,

@@ -143,9 +143,11 @@ bool qmv_m1_fuses_norm(uint32_t M, uint32_t K, uint32_t bits);
 // dst[m,k] = (half(x[m,k]) * half(inv_rms[m])) * norm_w[k], each product rounded to f16 (the RMSNorm prologue as a separate pass)
 int32_t launch_norm_rows(const void* x, int32_t x_dtype, const __half* norm_w, const float* inv_rms, uint32_t M,
                          uint32_t K, __half* dst, hipStream_t s);
-// chunk table for gather_qmm: batch b owns rows [b*mpb, (b+1)*mpb) and expert indices[b]
+// chunk table for gather_qmm: batch b owns rows [b*mpb, (b+1)*mpb) and expert indices[b]; chunks of at most
+// chunk_rows rows (an index out of range sets bit 31 of the count: zeros are written); n_chunks (nullable)
+// receives the table's length
 int32_t launch_build_gather_chunks(const uint32_t* indices, uint32_t batch, uint32_t mpb, uint32_t n_experts,
-                                   uint32_t* chunk_tab, hipStream_t s);
+                                   uint32_t chunk_rows, uint32_t* chunk_tab, uint32_t* n_chunks, hipStream_t s);
 
 struct QmmArgs {
   const uint32_t* w; const __half* s; const __half* b;
@@ -171,6 +173,27 @@ int32_t launch_qmm(const QmmArgs& a, hipStream_t s);
 // Register-weights GEMM (qmm_rw.hip): f16 activations only, no workspace.
 bool qmm_rw_supported(uint32_t N, uint32_t K, uint32_t group_size, uint32_t bits);
 int32_t launch_qmm_rw(const QmmArgs& a, uint32_t group_size, hipStream_t s);
+// Grouped form of the same GEMM for the expert projections of batches with many rows per expert: every
+// row tile (kGroupedTileRows rows of one expert) takes its expert and rows from a device table of
+// (expert, first row position, row count) triples (bit 31 of the count: write zeros instead of computing;
+// not for a pair); `n_tiles_dev` holds the table's length.  With a second
+// weight (w1 / s1 / b1: the up projection) the store writes silu(x Wg^T) * (x Wu^T).  Group size 64.
+constexpr uint32_t kGroupedTileRows = 64;
+struct GroupedQmmArgs {
+  const uint32_t* w; const __half* s; const __half* b;     // expert 0 of the (gate) weight
+  const uint32_t* w1; const __half* s1; const __half* b1;  // expert 0 of the up weight, or null
+  uint32_t N, K, bits;       // output columns (of a pair: columns of the product), input features
+  uint64_t expert_stride_w;  // u32 words per expert
+  uint64_t expert_stride_s;  // halves per expert
+  const __half* x;           // [x_rows, K] f16
+  const uint32_t* row_map;   // nullable: source row of position p is row_map[p]
+  void* out;                 // f16 [positions, N] (f32 when out_f32; not for a pair)
+  int out_f32;
+  const uint32_t* tile_tab; const uint32_t* n_tiles_dev;
+  uint32_t max_tiles;        // row tiles the grid covers (>= *n_tiles_dev)
+};
+bool qmm_rw_grouped_supported(uint32_t N, uint32_t K, uint32_t group_size, uint32_t bits);
+int32_t launch_qmm_rw_grouped(const GroupedQmmArgs& a, hipStream_t s);
 
 // MoE helpers
 int32_t launch_topk_route(const float* logits, const float* bias, uint32_t T, uint32_t E, uint32_t K,
@@ -181,7 +204,7 @@ int32_t launch_topk_route(const float* logits, const float* bias, uint32_t T, ui
 // sorted_tok (nullable): token of each sorted position, sorted[p] / top_k.
 int32_t launch_moe_sort(const uint32_t* idx, uint32_t n_assign, uint32_t E, uint32_t top_k, uint32_t* sorted,
                         uint32_t* sorted_tok, uint32_t* inv, uint32_t* counts, uint32_t* offsets,
-                        uint32_t* chunk_tab, uint32_t* n_chunks, hipStream_t s);
+                        uint32_t* chunk_tab, uint32_t* n_chunks, uint32_t chunk_rows, hipStream_t s);
 // Decode-sized batches (at most 8 tokens, 64 assignments): routing and grouping in one launch.
 bool route_sort_fusable(uint32_t T, uint32_t E, uint32_t K);
 int32_t launch_route_sort_small(const float* logits, const float* bias, uint32_t T, uint32_t E, uint32_t K,

@@ -196,7 +196,7 @@ __global__ __launch_bounds__(1024) void moe_sort_kernel(const uint32_t* __restri
                                                         uint32_t* __restrict__ inv, uint32_t* __restrict__ counts,
                                                         uint32_t* __restrict__ offsets,
                                                         uint32_t* __restrict__ chunk_tab,
-                                                        uint32_t* __restrict__ n_chunks) {
+                                                        uint32_t* __restrict__ n_chunks, uint32_t chunk_rows) {
   __shared__ uint32_t cnt[kMaxExperts];
   __shared__ uint32_t cur[kMaxExperts];  // running cursor of every expert
   __shared__ uint32_t wave_tot[16];
@@ -208,11 +208,11 @@ __global__ __launch_bounds__(1024) void moe_sort_kernel(const uint32_t* __restri
     if (e < E) atomicAdd(&cnt[e], 1u);
   }
   __syncthreads();
-  // thread e owns expert e: offsets, counts, its chunks of at most 8 rows
+  // thread e owns expert e: offsets, counts, its chunks of at most chunk_rows rows
   const uint32_t my_cnt = tid < E ? cnt[tid] : 0u;
   uint32_t total_rows, total_chunks;
   const uint32_t my_off = block_exclusive_scan_1024(my_cnt, wave_tot, &total_rows);
-  const uint32_t my_chunks = (my_cnt + 7) / 8;
+  const uint32_t my_chunks = (my_cnt + chunk_rows - 1) / chunk_rows;
   const uint32_t my_chunk0 = block_exclusive_scan_1024(my_chunks, wave_tot, &total_chunks);
   cur[tid] = my_off;
   if (tid < E) {
@@ -221,8 +221,8 @@ __global__ __launch_bounds__(1024) void moe_sort_kernel(const uint32_t* __restri
     if (chunk_tab != nullptr) {
       for (uint32_t c = 0; c < my_chunks; ++c) {
         chunk_tab[3 * (my_chunk0 + c) + 0] = tid;
-        chunk_tab[3 * (my_chunk0 + c) + 1] = my_off + 8 * c;
-        chunk_tab[3 * (my_chunk0 + c) + 2] = my_cnt - 8 * c < 8u ? my_cnt - 8 * c : 8u;
+        chunk_tab[3 * (my_chunk0 + c) + 1] = my_off + chunk_rows * c;
+        chunk_tab[3 * (my_chunk0 + c) + 2] = my_cnt - chunk_rows * c < chunk_rows ? my_cnt - chunk_rows * c : chunk_rows;
       }
     }
   }
@@ -454,7 +454,7 @@ int32_t launch_topk_route(const float* logits, const float* bias, uint32_t T, ui
   } else if (counts != nullptr || offsets != nullptr) {
     hipLaunchKernelGGL(moe_sort_kernel, dim3(1), dim3(1024), 0, s, idx, T * K, E, K, (uint32_t*)nullptr,
                        (uint32_t*)nullptr, (uint32_t*)nullptr, counts, offsets, (uint32_t*)nullptr,
-                       (uint32_t*)nullptr);
+                       (uint32_t*)nullptr, 8u);
     RMLX_HIP_CHECK(hipGetLastError());
   }
   return RMLX_OK;
@@ -476,15 +476,16 @@ int32_t launch_route_sort_small(const float* logits, const float* bias, uint32_t
 
 int32_t launch_moe_sort(const uint32_t* idx, uint32_t n_assign, uint32_t E, uint32_t top_k, uint32_t* sorted,
                         uint32_t* sorted_tok, uint32_t* inv, uint32_t* counts, uint32_t* offsets,
-                        uint32_t* chunk_tab, uint32_t* n_chunks, hipStream_t s) {
+                        uint32_t* chunk_tab, uint32_t* n_chunks, uint32_t chunk_rows, hipStream_t s) {
   if (E > (uint32_t)kMaxExperts)
     return fail(RMLX_INVALID_SHAPE, "moe_sort: n_experts (%u) exceeds maximum %d", E, kMaxExperts);
-  if (n_assign <= 64)
+  if (chunk_rows == 0) return fail(RMLX_RUNTIME_ERROR, "moe_sort: chunk_rows must be non-zero");
+  if (n_assign <= 64 && chunk_rows == 8)  // the one-wave kernel writes chunks of 8 rows
     hipLaunchKernelGGL(moe_sort_small_kernel, dim3(1), dim3(64), 0, s, idx, n_assign, E, top_k ? top_k : 1u, sorted,
                        sorted_tok, inv, counts, offsets, chunk_tab, n_chunks);
   else
     hipLaunchKernelGGL(moe_sort_kernel, dim3(1), dim3(1024), 0, s, idx, n_assign, E, top_k ? top_k : 1u, sorted,
-                       sorted_tok, inv, counts, offsets, chunk_tab, n_chunks);
+                       sorted_tok, inv, counts, offsets, chunk_tab, n_chunks, chunk_rows);
   RMLX_HIP_CHECK(hipGetLastError());
   return RMLX_OK;
 }

@@ -53,6 +53,13 @@ struct RwParams {
   // are added up (and the epilogue applied) by splitk_reduce_kernel
   uint32_t ksplit;
   float* partial;
+  // grouped launches (one expert per row tile): table of (expert, first row, rows) per row tile and its
+  // length on the device, optional gather of the activation rows, expert strides in u32 words / f16
+  // elements, the second weight of a gate/up pair (fragment 1 of every wave), f32 output
+  const uint32_t* tile_tab; const uint32_t* n_tiles; const uint32_t* row_map;
+  uint64_t estride_w, estride_s;
+  const uint32_t* w1; const __half* s1; const __half* b1;
+  int32_t out_f32;
 #ifdef QMM_RW_TRACE
   unsigned long long* trace;
 #endif
@@ -116,8 +123,13 @@ __device__ __forceinline__ h8 dequant_q8_pair(uint32_t w0, uint32_t w1, h2 s2, h
 // MF = 16-row activation fragments per workgroup (tile rows = 16*MF), NF = 16-row weight fragments
 // per wave (tile columns = 64*NF), BITS = 4 or 8.
 // GS = quantisation group size (32, 64 or 128): it only decides which (scale, bias) pair a lane uses.
-template <int MF, int NF, int BITS, int NW, bool XBF16, int GS>
-__global__ __launch_bounds__(64 * NW) void qmm_rw_kernel(RwParams p) {
+// MODE 0: one weight, row tiles of one [M,K] matrix.  MODE 1: grouped -- row tile t of the grid takes its
+// expert and its rows from the tile table (rows of different experts never share a tile); workgroups past
+// the table's length leave at once.  MODE 2: grouped gate/up pair -- fragment 0 of a wave multiplies gate
+// rows, fragment 1 the same rows of the up weight (NF == 2), and the store writes silu(gate) * up.
+template <int MF, int NF, int BITS, int NW, bool XBF16, int GS, int MODE>
+__device__ __forceinline__ void qmm_rw_body(const RwParams& p) {
+  static_assert(MODE != 2 || NF == 2, "a gate/up pair takes two weight fragments per wave");
   constexpr int kSbWords = 4 * (kBlockK / GS) / 2;  // 32-bit words of scales of one row and four iterations: 8 / 4 / 2
   constexpr int kSbVecs = (kSbWords + 3) / 4;       // 16-byte registers holding them
   constexpr int kThreads = 64 * NW;
@@ -136,9 +148,38 @@ __global__ __launch_bounds__(64 * NW) void qmm_rw_kernel(RwParams p) {
   // XCD x = id % 8 runs the ids congruent to x.  Give every XCD a compact block of tiles, half of
   // the row tiles x a quarter of the column tiles when those divide, so that what its L2 has to
   // fetch (its activation rows + its weight panels) is smallest; else whole weight panels per XCD.
-  uint32_t wg = blockIdx.x, mt, nt;
+  uint32_t wg = blockIdx.x, mt = 0, nt;
+  uint32_t row_lo = 0, row_hi = 0;  // rows of the activation / output matrix this tile covers: [row_lo, row_hi)
+  const uint32_t* wbase[2] = {p.w, p.w1};
+  const __half* sbase[2] = {p.s, p.s1};
+  const __half* bbase[2] = {p.b, p.b1};
   const uint32_t total = p.tiles_m * p.tiles_n;
-  if (total % 8 == 0 && p.tiles_m % 2 == 0 && p.tiles_n % 4 == 0) {
+  if (MODE != 0) {
+    // consecutive ids share a row tile (its activations); with tiles_n a multiple of 8 the row tiles of one
+    // expert land on the same XCD for every column tile, so its L2 serves the second read of a weight panel
+    nt = wg % p.tiles_n;
+    const uint32_t te = wg / p.tiles_n;
+    if (te >= *p.n_tiles) return;
+    const uint32_t expert = p.tile_tab[3 * te];
+    row_lo = p.tile_tab[3 * te + 1];
+    const uint32_t cnt = p.tile_tab[3 * te + 2];
+    row_hi = row_lo + (cnt & 0x7FFFFFFFu);
+    if (MODE == 1 && (cnt >> 31)) {  // rows whose expert index is out of range: zeros
+      constexpr uint32_t cols = NW * 16 * NF;
+      for (uint32_t i = threadIdx.x; i < (row_hi - row_lo) * cols; i += 64 * NW) {
+        const uint64_t o = (uint64_t)(row_lo + i / cols) * p.N + nt * cols + i % cols;
+        if (p.out_f32) reinterpret_cast<float*>(p.out)[o] = 0.f;
+        else p.out[o] = __float2half(0.f);
+      }
+      return;
+    }
+#pragma unroll
+    for (int d = 0; d < 2; ++d) {
+      wbase[d] += (uint64_t)expert * p.estride_w;
+      sbase[d] += (uint64_t)expert * p.estride_s;
+      bbase[d] += (uint64_t)expert * p.estride_s;
+    }
+  } else if (total % 8 == 0 && p.tiles_m % 2 == 0 && p.tiles_n % 4 == 0) {
     const uint32_t xcd = wg % 8, local = wg / 8, bm = p.tiles_m / 2, bn = p.tiles_n / 4;
     mt = (xcd % 2) * bm + local % bm;
     nt = (xcd / 2) * bn + local / bm;
@@ -147,21 +188,23 @@ __global__ __launch_bounds__(64 * NW) void qmm_rw_kernel(RwParams p) {
     mt = wg % p.tiles_m;
     nt = wg / p.tiles_m;
   }
+  if (MODE == 0) { row_lo = mt * (16 * MF); row_hi = p.M; }
 
   const uint32_t K = p.K, G = K / GS;
   const uint32_t S = K / kBlockK / p.ksplit;   // iterations of this workgroup
   const uint32_t it_first = blockIdx.y * S;    // its first 128-wide k block
-  const uint32_t row_base = nt * (NW * 16 * NF) + wave * (16 * NF) + n;
+  const uint32_t row_base = MODE == 2 ? nt * (NW * 16) + wave * 16 + n : nt * (NW * 16 * NF) + wave * (16 * NF) + n;
 
   const u4* wptr[NF];
   const __half* sptr[NF];
   const __half* bptr[NF];
 #pragma unroll
   for (int f = 0; f < NF; ++f) {
-    const uint64_t row = row_base + f * 16;
-    wptr[f] = reinterpret_cast<const u4*>(p.w + row * (K * BITS / 32)) + g + (uint64_t)it_first * (4 * WL);
-    sptr[f] = p.s + row * G + it_first * (kBlockK / GS);
-    bptr[f] = p.b + row * G + it_first * (kBlockK / GS);
+    const uint64_t row = MODE == 2 ? row_base : row_base + f * 16;
+    const int d = MODE == 2 ? f : 0;
+    wptr[f] = reinterpret_cast<const u4*>(wbase[d] + row * (K * BITS / 32)) + g + (uint64_t)it_first * (4 * WL);
+    sptr[f] = sbase[d] + row * G + it_first * (kBlockK / GS);
+    bptr[f] = bbase[d] + row * G + it_first * (kBlockK / GS);
   }
   // Activation chunk of an iteration: 16*MF rows x 128 k = 16 sixteen-byte segments per row.  Unit
   // q*kThreads + tid -> (row, segment): 16 consecutive lanes read one row's 256 contiguous bytes.
@@ -174,8 +217,9 @@ __global__ __launch_bounds__(64 * NW) void qmm_rw_kernel(RwParams p) {
 #pragma unroll
   for (int q = 0; q < AL; ++q) {
     const uint32_t unit = q * kThreads + tid, r = unit >> 4, seg = unit & 15;
-    uint32_t row = mt * (16 * MF) + r;
-    if (row >= p.M) row = p.M - 1;  // rows past M are computed on stale data and never stored
+    uint32_t row = row_lo + r;
+    if (row >= row_hi) row = row_hi - 1;  // rows past the end are computed on stale data and never stored
+    if (MODE != 0 && p.row_map != nullptr) row = p.row_map[row];
     xsrc[q] = p.x + (uint64_t)row * K + seg * 8 + (uint64_t)it_first * kBlockK;
     const uint32_t j = BITS == 4 ? (seg & 3) : (2 * (seg >> 3) + (seg & 1));
     const uint32_t gq = BITS == 4 ? (seg >> 2) : ((seg >> 1) & 3);
@@ -406,14 +450,28 @@ __global__ __launch_bounds__(64 * NW) void qmm_rw_kernel(RwParams p) {
   // ---- epilogue: lane holds row m = lane%16 of fragment i, columns 4g..4g+3 of fragment f ------
 #pragma unroll
   for (int i = 0; i < MF; ++i) {
-    const uint32_t m = mt * (16 * MF) + i * 16 + n;
-    if (m < p.M) {
+    const uint32_t m = row_lo + i * 16 + n;
+    if (m < row_hi) {
+      if (MODE == 2) {  // h = silu(gate) * up in f32, one rounding; p.N = columns of h
+        const uint32_t col = nt * (NW * 16) + wave * 16 + 4 * g;
+        f4 v;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) v[q] = acc[i][0][q] / (1.0f + __expf(-acc[i][0][q])) * acc[i][NF - 1][q];
+        const h2 lo = {(_Float16)v[0], (_Float16)v[1]};
+        const h2 hi = {(_Float16)v[2], (_Float16)v[3]};
+        *reinterpret_cast<u2*>(p.out + (uint64_t)m * p.N + col) = (u2){h2bits(lo), h2bits(hi)};
+        continue;
+      }
 #pragma unroll
       for (int f = 0; f < NF; ++f) {
         const uint32_t col = nt * (NW * 16 * NF) + wave * (16 * NF) + f * 16 + 4 * g;
         f4 v = acc[i][f];
-        if (p.ksplit > 1) {
+        if (MODE == 0 && p.ksplit > 1) {
           *reinterpret_cast<f4*>(p.partial + ((uint64_t)blockIdx.y * p.M + m) * p.N + col) = v;
+          continue;
+        }
+        if (MODE == 1 && p.out_f32) {
+          *reinterpret_cast<f4*>(reinterpret_cast<float*>(p.out) + (uint64_t)m * p.N + col) = v;
           continue;
         }
         if (p.epi_kind != EPI_NONE) {  // residual add / SwiGLU gate in f32, one rounding (quantized.rs:3206-3246)
@@ -439,6 +497,17 @@ __global__ __launch_bounds__(64 * NW) void qmm_rw_kernel(RwParams p) {
   }
   RW_MARK(p, 8, 7);
   RW_MARK_ALL(p, 1);
+}
+
+template <int MF, int NF, int BITS, int NW, bool XBF16, int GS>
+__global__ __launch_bounds__(64 * NW) void qmm_rw_kernel(RwParams p) {
+  qmm_rw_body<MF, NF, BITS, NW, XBF16, GS, 0>(p);
+}
+
+// DUAL: gate/up pair with the SwiGLU store (see MODE 2 above)
+template <int MF, int NF, int BITS, int NW, bool DUAL>
+__global__ __launch_bounds__(64 * NW) void qmm_rw_grouped_kernel(RwParams p) {
+  qmm_rw_body<MF, NF, BITS, NW, false, 64, DUAL ? 2 : 1>(p);
 }
 
 // out[m, c..c+3] = epilogue(sum over the ksplit partial sums, in split order); one thread per four columns
@@ -577,6 +646,42 @@ int32_t launch_qmm_rw(const QmmArgs& a, uint32_t group_size, hipStream_t s) {
     hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned)((quads + 255) / 256)), dim3(256), 0, s, p);
     RMLX_HIP_CHECK(hipGetLastError());
   }
+  return RMLX_OK;
+}
+
+bool qmm_rw_grouped_supported(uint32_t N, uint32_t K, uint32_t group_size, uint32_t bits) {
+  return group_size == 64 && (bits == 4 || bits == 8) && N > 0 && K > 0 && N % 128 == 0 && K % (kBlockK * kUnroll) == 0;
+}
+
+int32_t launch_qmm_rw_grouped(const GroupedQmmArgs& a, hipStream_t s) {
+  if (!qmm_rw_grouped_supported(a.N, a.K, 64, a.bits))
+    return fail(RMLX_INVALID_SHAPE, "grouped qmm: unsupported shape N=%u K=%u bits=%u", a.N, a.K, a.bits);
+  if (a.max_tiles == 0) return RMLX_OK;
+  const bool dual = a.w1 != nullptr;
+  if (dual && a.out_f32) return fail(RMLX_RUNTIME_ERROR, "grouped qmm: the gate/up pair writes f16");
+  if (a.tile_tab == nullptr || a.n_tiles_dev == nullptr) return fail(RMLX_RUNTIME_ERROR, "grouped qmm: no tile table");
+  RwParams p{};
+  p.w = a.w; p.s = a.s; p.b = a.b; p.w1 = a.w1; p.s1 = a.s1; p.b1 = a.b1;
+  p.x = a.x; p.row_map = a.row_map;
+  p.out = static_cast<__half*>(a.out); p.out_f32 = a.out_f32;
+  p.M = 0; p.N = a.N; p.K = a.K;
+  p.epi_kind = EPI_NONE; p.ksplit = 1;
+  p.tile_tab = a.tile_tab; p.n_tiles = a.n_tiles_dev;
+  p.estride_w = a.expert_stride_w; p.estride_s = a.expert_stride_s;
+  p.tiles_m = a.max_tiles;
+  // row tiles of 16 * 4 = kGroupedTileRows rows, 8 waves; a pair: 128 columns of each weight per workgroup,
+  // one weight: 256 columns when they divide, else 128
+  const bool wide = !dual && a.N % 256 == 0;
+  p.tiles_n = a.N / (wide ? 256 : 128);
+  if ((uint64_t)p.tiles_m * p.tiles_n > 0x7FFFFFFFull) return fail(RMLX_INVALID_SHAPE, "grouped qmm: grid too large");
+  const dim3 grid(p.tiles_m * p.tiles_n), block(512);
+#define RWG_LAUNCH(BITSV)                                                                                   \
+  if (dual) hipLaunchKernelGGL((qmm_rw_grouped_kernel<4, 2, BITSV, 8, true>), grid, block, 0, s, p);          \
+  else if (wide) hipLaunchKernelGGL((qmm_rw_grouped_kernel<4, 2, BITSV, 8, false>), grid, block, 0, s, p);    \
+  else hipLaunchKernelGGL((qmm_rw_grouped_kernel<4, 1, BITSV, 8, false>), grid, block, 0, s, p);
+  if (a.bits == 4) { RWG_LAUNCH(4) } else { RWG_LAUNCH(8) }
+#undef RWG_LAUNCH
+  RMLX_HIP_CHECK(hipGetLastError());
   return RMLX_OK;
 }
 

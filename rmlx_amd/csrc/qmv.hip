@@ -467,12 +467,14 @@ void launch_t(const KParams& p, bool tab, dim3 grid, hipStream_t s) {
 }
 
 __global__ void build_gather_chunks_kernel(const uint32_t* indices, uint32_t batch, uint32_t mpb,
-                                           uint32_t n_experts, uint32_t* chunk_tab) {
-  const uint32_t per = (mpb + 7) / 8;
+                                           uint32_t n_experts, uint32_t chunk_rows, uint32_t* chunk_tab,
+                                           uint32_t* n_chunks) {
+  const uint32_t per = (mpb + chunk_rows - 1) / chunk_rows;
   const uint32_t c = blockIdx.x * blockDim.x + threadIdx.x;
   if (c >= batch * per) return;
-  const uint32_t b = c / per, r = (c % per) * 8;
-  uint32_t e = indices[b], rows = mpb - r < 8u ? mpb - r : 8u;
+  if (c == 0 && n_chunks != nullptr) *n_chunks = batch * per;
+  const uint32_t b = c / per, r = (c % per) * chunk_rows;
+  uint32_t e = indices[b], rows = mpb - r < chunk_rows ? mpb - r : chunk_rows;
   if (e >= n_experts) { e = 0; rows |= 0x80000000u; }
   chunk_tab[3 * c + 0] = e;
   chunk_tab[3 * c + 1] = b * mpb + r;
@@ -482,11 +484,12 @@ __global__ void build_gather_chunks_kernel(const uint32_t* indices, uint32_t bat
 }  // namespace
 
 int32_t launch_build_gather_chunks(const uint32_t* indices, uint32_t batch, uint32_t mpb, uint32_t n_experts,
-                                   uint32_t* chunk_tab, hipStream_t s) {
-  const uint32_t n = batch * ((mpb + 7) / 8);
+                                   uint32_t chunk_rows, uint32_t* chunk_tab, uint32_t* n_chunks, hipStream_t s) {
+  if (chunk_rows == 0) return fail(RMLX_RUNTIME_ERROR, "gather chunks: chunk_rows must be non-zero");
+  const uint32_t n = batch * ((mpb + chunk_rows - 1) / chunk_rows);
   if (n == 0) return RMLX_OK;
   hipLaunchKernelGGL(build_gather_chunks_kernel, dim3((n + 255) / 256), dim3(256), 0, s, indices, batch, mpb,
-                     n_experts, chunk_tab);
+                     n_experts, chunk_rows, chunk_tab, n_chunks);
   RMLX_HIP_CHECK(hipGetLastError());
   return RMLX_OK;
 }

@@ -270,6 +270,12 @@ class ExpertGroup:
         return res
 
 
+def set_expert_gemm_min_rows(min_rows):
+    """Average rows per expert from which the expert projections run on the grouped MFMA GEMM instead of the
+    streaming GEMV (0 = never; process-wide).  Returns the previous value."""
+    return int(rt.lib().rmlx_hip_set_expert_gemm_min_rows(int(min_rows)))
+
+
 def moe_forward_grouped(gate, up, down, x, expert_indices, expert_weights, top_k, stream=None, out=None):
     if out is None:
         out = DeviceBuffer((x.shape[0], x.shape[1]), F16)

@@ -41,7 +41,7 @@ EXPORTS = [
     "rmlx_hip_gather_qmm", "rmlx_hip_topk_route", "rmlx_hip_moe_sort", "rmlx_hip_index_gather",
     "rmlx_hip_scatter_weighted_add", "rmlx_hip_silu_gate", "rmlx_hip_expert_group_grouped_forward",
     "rmlx_hip_moe_forward_grouped", "rmlx_hip_moe_forward", "rmlx_hip_awq_dequant", "rmlx_hip_gptq_dequant",
-    "rmlx_hip_qmm_norm",
+    "rmlx_hip_qmm_norm", "rmlx_hip_set_expert_gemm_min_rows",
 ]
 
 _lib = None
@@ -103,6 +103,8 @@ def lib():
         fn = getattr(L, name)
         fn.argtypes = argtypes
         fn.restype = i32
+    L.rmlx_hip_set_expert_gemm_min_rows.argtypes = [u32]
+    L.rmlx_hip_set_expert_gemm_min_rows.restype = u32
     _lib = L
     return L
 

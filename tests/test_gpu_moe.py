@@ -235,6 +235,38 @@ def test_gather_qmm_async_out_of_range_rows_are_zero(hip):
     assert np.all(out[~good] == 0)
 
 
+@pytest.mark.parametrize("n,k,mpb", [(128, 512, 12), (384, 1024, 70), (256, 512, 64), (128, 1536, 129)])
+def test_gather_qmm_many_rows_per_entry_on_the_grouped_gemm(hip, n, k, mpb):
+    """From 12 rows per batch entry on, gather_qmm multiplies with the grouped MFMA GEMM (row tiles of 64 rows of one
+    expert; the last tile of an entry ragged).  Against the oracle; on a stream, rows of an out-of-range index are zero."""
+    from rmlx_amd import ops
+    from rmlx_amd.runtime import DeviceBuffer, Stream
+    rng = np.random.default_rng(n + k + mpb)
+    E, batch = 5, 6
+    words, s, b = make_weight(rng, n, k, 4, lead=(E,))
+    x = rng.standard_normal((batch, mpb, k)).astype(np.float16)
+    idx = np.array([4, 0, 3, 3, 1, 0], np.uint32)
+    print(f"gather_qmm gemm n={n} k={k} mpb={mpb}", flush=True)
+    xd, wd, sd, bd = [DeviceBuffer.from_numpy(a) for a in (x, words, s, b)]
+    out = ops.gather_qmm(xd, wd, sd, bd, DeviceBuffer.from_numpy(idx), batch, mpb, n, k, E, 64).numpy()
+    ref = model.gather_qmm(x, words, s, b, idx, 64)
+    assert_close(out, ref, "gather_qmm (GEMM)")
+    prev = ops.set_expert_gemm_min_rows(0)
+    try:
+        out_stream = ops.gather_qmm(xd, wd, sd, bd, DeviceBuffer.from_numpy(idx), batch, mpb, n, k, E, 64).numpy()
+    finally:
+        ops.set_expert_gemm_min_rows(prev)
+    assert_close(out_stream, ref, "gather_qmm (streaming GEMV)")
+    bad = np.array([4, 9, 3, 7, 1, 0], np.uint32)
+    st = Stream()
+    out = ops.gather_qmm(xd, wd, sd, bd, DeviceBuffer.from_numpy(bad), batch, mpb, n, k, E, 64, stream=st)
+    st.sync()
+    out = out.numpy()
+    good = bad < E
+    assert_close(out[good], model.gather_qmm(x[good], words, s, b, bad[good], 64), "valid entries")
+    assert np.all(out[~good] == 0)
+
+
 # ---- expert FFN and the fused block ----------------------------------------------------------------------------
 
 def _experts(rng, E, D, I, fused):
@@ -390,6 +422,57 @@ def test_moe_other_bit_widths_and_group_sizes(hip, bits, gs, D, I, fused):
     for (e, v), (_, yv) in zip(items, outs):
         ones = np.ones((len(v), 1))
         assert_close(yv, model.moe_forward(v, np.full((len(v), 1), e), ones, gate, up, down, gs, 1, bits=bits), f"expert {e}")
+
+
+@pytest.mark.parametrize("bits,D,I,fused", [(4, 512, 512, True), (4, 1024, 1536, False), (8, 512, 1024, True), (8, 1024, 512, False)])
+def test_moe_many_rows_per_expert_on_the_grouped_gemm(hip, bits, D, I, fused):
+    """Batches with many rows per expert (here 75 on average; from 12 on) multiply with the grouped MFMA GEMM: row tiles
+    of 64 rows of one expert.  Skewed routing gives one expert three tiles, another a ragged one and one almost
+    nothing.  Checked against the oracle, and the streaming GEMV path (threshold 0) on the same inputs beside it."""
+    from rmlx_amd import ops
+    from rmlx_amd.runtime import DeviceBuffer
+    rng = np.random.default_rng(bits * 1000 + D + I)
+    E, T, K = 4, 150, 2
+
+    def weight(n, k):
+        return make_weight(rng, n, k, bits, 64, lead=(E,))
+
+    if fused:
+        gu = weight(2 * I, D)
+        gate, up = tuple(a[:, :I] for a in gu), tuple(a[:, I:] for a in gu)
+        gh, uh = ops.QuantizedWeight.from_numpy(*gu, 64, bits), None
+    else:
+        gate, up = weight(I, D), weight(I, D)
+        gh, uh = ops.QuantizedWeight.from_numpy(*gate, 64, bits), ops.QuantizedWeight.from_numpy(*up, 64, bits)
+    down = weight(D, I)
+    dh = ops.QuantizedWeight.from_numpy(*down, 64, bits)
+    x = make_x(rng, T, D)
+    logits = rng.standard_normal((T, E)).astype(np.float32)
+    logits[:, 0] += 3.0
+    logits[:, 3] -= 4.0
+    idx, w, counts, _ = model.topk_route(logits, K)
+    assert counts.max() > 128 and counts.min() < 16, counts
+    ref = model.moe_forward(x, idx, w, gate, up, down, 64, K, bits=bits)
+    xd, idxd, wd = DeviceBuffer.from_numpy(x), DeviceBuffer.from_numpy(idx), DeviceBuffer.from_numpy(w)
+    print(f"grouped gemm moe bits={bits} D={D} I={I} fused={fused} counts={counts.tolist()}", flush=True)
+    prev = ops.set_expert_gemm_min_rows(12)
+    try:
+        out_gemm = ops.moe_forward_grouped(gh, uh, dh, xd, idxd, wd, K).numpy()
+        assert_close(out_gemm, ref, "moe_forward_grouped (GEMM)")
+        assert_close(ops.moe_forward(gh, uh, dh, xd, DeviceBuffer.from_numpy(logits), K).numpy(), ref, "moe_forward (GEMM)")
+        group = ops.ExpertGroup(gh, uh, dh)
+        items = [(3, make_x(rng, 70, D)), (0, make_x(rng, 1, D)), (2, make_x(rng, 64, D)), (3, make_x(rng, 33, D)),
+                 (1, make_x(rng, 129, D))]
+        outs = group.grouped_forward([(e, DeviceBuffer.from_numpy(v)) for e, v in items])
+        for (e, v), (_, yv) in zip(items, outs):
+            ones = np.ones((len(v), 1))
+            assert_close(yv, model.moe_forward(v, np.full((len(v), 1), e), ones, gate, up, down, 64, 1, bits=bits),
+                         f"ExpertGroup (GEMM) expert {e} rows {len(v)}")
+        ops.set_expert_gemm_min_rows(0)
+        out_stream = ops.moe_forward_grouped(gh, uh, dh, xd, idxd, wd, K).numpy()
+        assert_close(out_stream, ref, "moe_forward_grouped (streaming GEMV)")
+    finally:
+        ops.set_expert_gemm_min_rows(prev)
 
 
 def _two_bit(rng, E, n, k, gs):
