@@ -280,12 +280,14 @@ def main():
         down = make_weight(rng, 4096, 1536, 4, lead=(128,))
         experts = (gate_up, down, ops.QuantizedWeight.from_numpy(*gate_up, 64, 4),
                    ops.QuantizedWeight.from_numpy(*down, 64, 4))
-        for batch, mpb in ((32, 1), (32, 8)):
+        for batch, mpb in ((32, 1), (32, 8), (32, 64)):
             r = bench_gather(ops, rt, timer, rng, batch, mpb, experts[2], gate_up, max(50, args.steps // 10), 10)
             r["hbm_frac"] = r["gbs"] / HBM_PEAK_GBS
             extra[f"gather_qmm_q4_b{batch}_m{mpb}"] = r
-        for T in (4, 32, 128):
-            r = bench_moe(ops, rt, timer, rng, T, max(50, args.steps // 10), 10, experts)
+        for T in (4, 32, 128, 512, 2048):  # from 8 rows per expert on average (T = 128) on the grouped MFMA GEMM
+            r = bench_moe(ops, rt, timer, rng, T, max(50, args.steps // (10 if T <= 128 else 40)), 10, experts)
+            r["tflops"] = r["flops"] / (r["us"] * 1e-6) / 1e12
+            r["mfma_frac"] = r["tflops"] / MFMA_F16_PEAK_TF
             r["hbm_frac"] = r["gbs"] / HBM_PEAK_GBS
             extra[f"moe_q4_T{T}"] = r
         del experts, gate_up, down
@@ -293,8 +295,9 @@ def main():
         down = make_weight(rng, 4096, 1536, 8, lead=(128,))
         experts = (gate_up, down, ops.QuantizedWeight.from_numpy(*gate_up, 64, 8),
                    ops.QuantizedWeight.from_numpy(*down, 64, 8))
-        for T in (4, 32):
-            r = bench_moe(ops, rt, timer, rng, T, max(50, args.steps // 10), 10, experts, bits=8)
+        for T in (4, 32, 512):
+            r = bench_moe(ops, rt, timer, rng, T, max(50, args.steps // (10 if T <= 128 else 40)), 10, experts, bits=8)
+            r["tflops"] = r["flops"] / (r["us"] * 1e-6) / 1e12
             r["hbm_frac"] = r["gbs"] / HBM_PEAK_GBS
             extra[f"moe_q8_T{T}"] = r
 

@@ -290,7 +290,7 @@ struct ExpertShapes {
 
 // Average rows per expert from which the expert projections run on the grouped GEMM instead of the streaming
 // GEMV (which re-reads an expert's weights once per 8 rows); 0 = never.  Measured crossover.
-std::atomic<uint32_t> g_expert_gemm_min_rows{12};
+std::atomic<uint32_t> g_expert_gemm_min_rows{8};
 
 int32_t check_expert_weights(const char* who, const rmlx_qweight* gate, const rmlx_qweight* up,
                              const rmlx_qweight* down, ExpertShapes* sh) {
@@ -330,10 +330,12 @@ int32_t check_expert_weights(const char* who, const rmlx_qweight* gate, const rm
   return RMLX_OK;
 }
 
-// true when `rows` positions over at most `groups` experts are multiplied by the grouped GEMM
-bool expert_gemm_pays(const ExpertShapes& sh, uint64_t rows, uint64_t groups) {
+// Rows per tile when `rows` positions over at most `groups` experts are multiplied by the grouped GEMM (half
+// tiles while an expert has 24 rows or fewer on average: less padding, more workgroups per CU), else 0
+uint32_t expert_gemm_tile_rows(const ExpertShapes& sh, uint64_t rows, uint64_t groups) {
   const uint32_t min_rows = g_expert_gemm_min_rows.load(std::memory_order_relaxed);
-  return sh.gemm && min_rows != 0 && groups != 0 && rows >= (uint64_t)min_rows * groups;
+  if (!sh.gemm || min_rows == 0 || groups == 0 || rows < (uint64_t)min_rows * groups) return 0;
+  return rows <= 24 * groups ? 32u : kGroupedTileRows;
 }
 
 // The same block on the portable kernels, for expert weights the streaming GEMV does not take (2-bit,
@@ -368,9 +370,9 @@ int32_t run_expert_ffn_portable(const rmlx_qweight* gate, const rmlx_qweight* up
 int32_t run_expert_ffn(const rmlx_qweight* gate, const rmlx_qweight* up, const rmlx_qweight* down,
                        const ExpertShapes& sh, const __half* x, const uint32_t* row_map,
                        const uint32_t* chunk_tab, const uint32_t* n_chunks, uint32_t max_chunks, __half* h,
-                       void* y, int y_f32, bool gemm, hipStream_t stream) {
+                       void* y, int y_f32, uint32_t gemm_tile_rows, hipStream_t stream) {
   const uint32_t per = 32 / gate->bits;  // values per u32 word: 8 (4-bit) or 4 (8-bit)
-  if (gemm) {  // the table holds row tiles of kGroupedTileRows rows and n_chunks its length
+  if (gemm_tile_rows != 0) {  // the table holds row tiles of that many rows and n_chunks its length
     GroupedQmmArgs a{};
     a.w = gate->w; a.s = gate->s; a.b = gate->b;
     if (sh.fused) {
@@ -385,7 +387,7 @@ int32_t run_expert_ffn(const rmlx_qweight* gate, const rmlx_qweight* up, const r
     a.expert_stride_w = rows * (sh.D / per);
     a.expert_stride_s = rows * (sh.D / 64);
     a.x = x; a.row_map = row_map; a.out = h; a.out_f32 = 0;
-    a.tile_tab = chunk_tab; a.n_tiles_dev = n_chunks; a.max_tiles = max_chunks;
+    a.tile_tab = chunk_tab; a.n_tiles_dev = n_chunks; a.max_tiles = max_chunks; a.tile_rows = gemm_tile_rows;
     RMLX_TRY(launch_qmm_rw_grouped(a, stream));
     GroupedQmmArgs d{};
     d.w = down->w; d.s = down->s; d.b = down->b;
@@ -393,7 +395,7 @@ int32_t run_expert_ffn(const rmlx_qweight* gate, const rmlx_qweight* up, const r
     d.expert_stride_w = (size_t)sh.D * (sh.I / per);
     d.expert_stride_s = (size_t)sh.D * (sh.I / 64);
     d.x = h; d.row_map = nullptr; d.out = y; d.out_f32 = y_f32;
-    d.tile_tab = chunk_tab; d.n_tiles_dev = n_chunks; d.max_tiles = max_chunks;
+    d.tile_tab = chunk_tab; d.n_tiles_dev = n_chunks; d.max_tiles = max_chunks; d.tile_rows = gemm_tile_rows;
     return launch_qmm_rw_grouped(d, stream);
   }
   QmvArgs a{};
@@ -815,22 +817,27 @@ int32_t rmlx_hip_gather_qmm(const rmlx_array* x, const void* w_packed_dev, size_
   const bool fast = qmv_q4_supported(N32, K32, group_size) && aligned16(w) && aligned16(sc) &&
                     aligned16(bi) && aligned16(xk);
   const uint32_t gemm_min_rows = g_expert_gemm_min_rows.load(std::memory_order_relaxed);
-  if (fast && gemm_min_rows != 0 && m_per_batch >= gemm_min_rows && qmm_rw_grouped_supported(N32, K32, group_size, 4)) {
+  // Every entry has exactly m_per_batch rows, so the streaming GEMV wastes nothing up to a full chunk of 8 rows
+  // and the crossover lies higher than for routed batches: one and a half times the threshold (measured: 8 rows
+  // per entry 50 us streamed, 64 us on the GEMM; 64 rows 91 us on the GEMM).
+  if (fast && gemm_min_rows != 0 && m_per_batch >= gemm_min_rows + gemm_min_rows / 2 &&
+      qmm_rw_grouped_supported(N32, K32, group_size, 4)) {
     // many rows per entry: row tiles of one expert each on the grouped MFMA GEMM
-    const uint32_t per = ((uint32_t)m_per_batch + kGroupedTileRows - 1) / kGroupedTileRows;
+    const uint32_t tile_rows = m_per_batch <= 32 ? 32u : kGroupedTileRows;
+    const uint32_t per = ((uint32_t)m_per_batch + tile_rows - 1) / tile_rows;
     const uint64_t n_tiles = (uint64_t)B32 * per;
     if (n_tiles > 0x7FFFFFu) return fail(RMLX_INVALID_SHAPE, "gather_qmm: too many row tiles (%" PRIu64 ")", n_tiles);
     Scratch tab;
     RMLX_TRY(tab.alloc((size_t)n_tiles * 12 + 4, s));
     uint32_t* t = static_cast<uint32_t*>(tab.ptr);
-    RMLX_TRY(launch_build_gather_chunks(idx, B32, (uint32_t)m_per_batch, E32, kGroupedTileRows, t, t + 3 * n_tiles, s));
+    RMLX_TRY(launch_build_gather_chunks(idx, B32, (uint32_t)m_per_batch, E32, tile_rows, t, t + 3 * n_tiles, s));
     GroupedQmmArgs a{};
     a.w = w; a.s = sc; a.b = bi;
     a.N = N32; a.K = K32; a.bits = 4;
     a.expert_stride_w = (uint64_t)n * (k / 8);
     a.expert_stride_s = (uint64_t)n * gpr;
     a.x = xk; a.out = out_f16_dev;
-    a.tile_tab = t; a.n_tiles_dev = t + 3 * n_tiles; a.max_tiles = (uint32_t)n_tiles;
+    a.tile_tab = t; a.n_tiles_dev = t + 3 * n_tiles; a.max_tiles = (uint32_t)n_tiles; a.tile_rows = tile_rows;
     RMLX_TRY(launch_qmm_rw_grouped(a, s));
   } else if (fast) {
     const uint32_t per = ((uint32_t)m_per_batch + 7) / 8, n_chunks = B32 * per;
@@ -969,8 +976,8 @@ int32_t rmlx_hip_expert_group_grouped_forward(const rmlx_qweight* gate, const rm
   size_t total = 0;
   for (size_t i = 0; i < n_items; ++i) total += batch_sizes_host[i];
   // row chunks of one expert each: 8 rows for the streaming GEMV, whole row tiles for the grouped GEMM
-  const bool gemm = expert_gemm_pays(sh, total, n_items);
-  const uint32_t chunk_rows = gemm ? kGroupedTileRows : 8u;
+  const uint32_t gemm = expert_gemm_tile_rows(sh, total, n_items);
+  const uint32_t chunk_rows = gemm ? gemm : 8u;
   std::vector<uint32_t> tab;
   total = 0;
   for (size_t i = 0; i < n_items; ++i) {
@@ -1053,8 +1060,8 @@ int32_t moe_grouped_impl(const rmlx_qweight* gate, const rmlx_qweight* up, const
   RMLX_TRY(check_out("MoeLayer", out_bytes, T * sh.D * 2));
   if (T == 0) return RMLX_OK;
   // many rows per expert: the grouped GEMM over row tiles instead of the streaming GEMV over chunks of 8 rows
-  const bool gemm = route == nullptr && expert_gemm_pays(sh, A, sh.E);
-  const uint32_t chunk_rows = gemm ? kGroupedTileRows : 8u;
+  const uint32_t gemm = route == nullptr ? expert_gemm_tile_rows(sh, A, sh.E) : 0u;
+  const uint32_t chunk_rows = gemm ? gemm : 8u;
   const uint32_t max_chunks = A / chunk_rows + (A < sh.E ? A : sh.E);
   if (max_chunks > 65535) return fail(RMLX_INVALID_SHAPE, "MoeLayer: too many row chunks (%u); split the batch", max_chunks);
 

@@ -191,6 +191,7 @@ struct GroupedQmmArgs {
   int out_f32;
   const uint32_t* tile_tab; const uint32_t* n_tiles_dev;
   uint32_t max_tiles;        // row tiles the grid covers (>= *n_tiles_dev)
+  uint32_t tile_rows;        // rows per tile the table was built for: 32 or kGroupedTileRows
 };
 bool qmm_rw_grouped_supported(uint32_t N, uint32_t K, uint32_t group_size, uint32_t bits);
 int32_t launch_qmm_rw_grouped(const GroupedQmmArgs& a, hipStream_t s);

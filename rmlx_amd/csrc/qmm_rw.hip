@@ -674,12 +674,18 @@ int32_t launch_qmm_rw_grouped(const GroupedQmmArgs& a, hipStream_t s) {
   const bool wide = !dual && a.N % 256 == 0;
   p.tiles_n = a.N / (wide ? 256 : 128);
   if ((uint64_t)p.tiles_m * p.tiles_n > 0x7FFFFFFFull) return fail(RMLX_INVALID_SHAPE, "grouped qmm: grid too large");
+  if (a.tile_rows != 32 && a.tile_rows != kGroupedTileRows)
+    return fail(RMLX_RUNTIME_ERROR, "grouped qmm: row tiles of %u rows", a.tile_rows);
   const dim3 grid(p.tiles_m * p.tiles_n), block(512);
-#define RWG_LAUNCH(BITSV)                                                                                   \
-  if (dual) hipLaunchKernelGGL((qmm_rw_grouped_kernel<4, 2, BITSV, 8, true>), grid, block, 0, s, p);          \
-  else if (wide) hipLaunchKernelGGL((qmm_rw_grouped_kernel<4, 2, BITSV, 8, false>), grid, block, 0, s, p);    \
-  else hipLaunchKernelGGL((qmm_rw_grouped_kernel<4, 1, BITSV, 8, false>), grid, block, 0, s, p);
-  if (a.bits == 4) { RWG_LAUNCH(4) } else { RWG_LAUNCH(8) }
+#define RWG_LAUNCH(MFV, BITSV)                                                                                \
+  if (dual) hipLaunchKernelGGL((qmm_rw_grouped_kernel<MFV, 2, BITSV, 8, true>), grid, block, 0, s, p);          \
+  else if (wide) hipLaunchKernelGGL((qmm_rw_grouped_kernel<MFV, 2, BITSV, 8, false>), grid, block, 0, s, p);    \
+  else hipLaunchKernelGGL((qmm_rw_grouped_kernel<MFV, 1, BITSV, 8, false>), grid, block, 0, s, p);
+  if (a.tile_rows == 32) {
+    if (a.bits == 4) { RWG_LAUNCH(2, 4) } else { RWG_LAUNCH(2, 8) }
+  } else {
+    if (a.bits == 4) { RWG_LAUNCH(4, 4) } else { RWG_LAUNCH(4, 8) }
+  }
 #undef RWG_LAUNCH
   RMLX_HIP_CHECK(hipGetLastError());
   return RMLX_OK;
