@@ -167,8 +167,10 @@ __global__ __launch_bounds__(64) void topk_route_kernel(const float* __restrict_
 // Deterministic by construction.  Offsets and the chunk table come from block-wide exclusive scans
 // of the per-expert counts.  Placement walks the assignments in blocks of 1024: every wave ranks
 // its 64 consecutive assignments among themselves (lane l counts the lanes below it with the same
-// expert), then the waves take turns, in order, to add the running cursor of their experts, so
-// ids of one expert keep their original order (numpy.argsort(kind="stable")).
+// expert) and leaves its count per expert in LDS; thread e turns the 16 counts of expert e into an
+// exclusive prefix over the waves; position = running cursor of the expert + prefix of the wave +
+// rank in the wave, so ids of one expert keep their original order (numpy.argsort(kind="stable")).
+// Four barriers per block of 1024 ids.
 __device__ __forceinline__ uint32_t block_exclusive_scan_1024(uint32_t v, uint32_t* wave_tot, uint32_t* total) {
   const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   uint32_t inc = v;
@@ -200,8 +202,11 @@ __global__ __launch_bounds__(1024) void moe_sort_kernel(const uint32_t* __restri
   __shared__ uint32_t cnt[kMaxExperts];
   __shared__ uint32_t cur[kMaxExperts];  // running cursor of every expert
   __shared__ uint32_t wave_tot[16];
+  __shared__ uint16_t wcnt[16][kMaxExperts];  // placement: per (wave, expert) counts of a block of 1024 ids
   const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   cnt[tid] = 0;  // kMaxExperts == blockDim.x
+#pragma unroll
+  for (int w = 0; w < 16; ++w) wcnt[w][tid] = 0;
   __syncthreads();
   for (uint32_t i = tid; i < n_assign; i += 1024) {
     const uint32_t e = idx[i];
@@ -232,34 +237,45 @@ __global__ __launch_bounds__(1024) void moe_sort_kernel(const uint32_t* __restri
   }
   if (sorted == nullptr) return;
 
+  const int e_bits = 32 - __builtin_clz(E | 1u);  // bits that tell valid expert ids apart
+  const uint64_t lanes_below = (1ull << lane) - 1ull;
+  uint32_t e_next = tid < n_assign ? idx[tid] : 0xFFFFFFFFu;
   for (uint32_t base = 0; base < n_assign; base += 1024) {
-    const uint32_t nb = n_assign - base < 1024u ? n_assign - base : 1024u;
-    const uint32_t e = tid < nb ? idx[base + tid] : 0xFFFFFFFFu;
+    const uint32_t e = e_next;
+    e_next = base + 1024 + tid < n_assign ? idx[base + 1024 + tid] : 0xFFFFFFFFu;  // in flight during this block
     const bool valid = e < E;
-    // rank among the wave's 64 assignments, and how many of them share the expert
-    uint32_t rank = 0, same_total = 0;
-    for (int j = 0; j < 64; ++j) {
-      const uint32_t ej = (uint32_t)__builtin_amdgcn_readlane((int)e, j);
-      const uint32_t same = ej == e ? 1u : 0u;
-      same_total += same;
-      rank += (j < (int)lane) ? same : 0u;
+    // rank among the wave's 64 assignments, and how many of them share the expert: the lanes holding the same
+    // expert are the intersection, over the bits of the id, of the lanes that agree with this one on that bit
+    uint64_t peers = __ballot(valid);
+    for (int bit = 0; bit < e_bits; ++bit) {
+      const uint64_t set = __ballot((e >> bit) & 1u);
+      peers &= ((e >> bit) & 1u) ? set : ~set;
     }
-    const uint32_t n_waves = (nb + 63) / 64;
-    uint32_t pos = 0;
-    for (uint32_t w = 0; w < n_waves; ++w) {
-      __syncthreads();  // cursor updates of wave w-1 (and of the previous block) are visible
-      uint32_t c0 = 0;
-      if (wave == w && valid) c0 = cur[e];
-      if (wave == w && valid) {
-        pos = c0 + rank;
-        if (rank + 1 == same_total) cur[e] = c0 + same_total;  // the last one of its expert moves the cursor
+    const uint32_t rank = (uint32_t)__popcll(peers & lanes_below), same_total = (uint32_t)__popcll(peers);
+    // assignments of (wave, expert) in this block -> exclusive prefix over the waves, per expert
+    if (valid && rank + 1 == same_total) wcnt[wave][e] = (uint16_t)same_total;
+    __syncthreads();
+    uint32_t run = 0;
+    if (tid < E) {
+#pragma unroll
+      for (int w = 0; w < 16; ++w) {
+        const uint32_t c = wcnt[w][tid];
+        wcnt[w][tid] = (uint16_t)run;
+        run += c;
       }
     }
+    __syncthreads();
     if (valid) {
+      const uint32_t pos = cur[e] + wcnt[wave][e] + rank;
       sorted[pos] = base + tid;
       if (sorted_tok != nullptr) sorted_tok[pos] = (base + tid) / top_k;
       if (inv != nullptr) inv[base + tid] = pos;
     }
+    __syncthreads();
+    // thread t owns column t of wcnt and cur[t]: cursor forward, column cleared for the next block
+    cur[tid] += run;
+#pragma unroll
+    for (int w = 0; w < 16; ++w) wcnt[w][tid] = 0;
     __syncthreads();
   }
 }

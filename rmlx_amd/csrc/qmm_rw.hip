@@ -128,7 +128,7 @@ __device__ __forceinline__ h8 dequant_q8_pair(uint32_t w0, uint32_t w1, h2 s2, h
 // the table's length leave at once.  MODE 2: grouped gate/up pair -- fragment 0 of a wave multiplies gate
 // rows, fragment 1 the same rows of the up weight (NF == 2), and the store writes silu(gate) * up.
 template <int MF, int NF, int BITS, int NW, bool XBF16, int GS, int MODE>
-__device__ __forceinline__ void qmm_rw_body(const RwParams& p) {
+__device__ __forceinline__ void qmm_rw_body(const RwParams p) {  // by value: a reference makes every store a possible change of p
   static_assert(MODE != 2 || NF == 2, "a gate/up pair takes two weight fragments per wave");
   constexpr int kSbWords = 4 * (kBlockK / GS) / 2;  // 32-bit words of scales of one row and four iterations: 8 / 4 / 2
   constexpr int kSbVecs = (kSbWords + 3) / 4;       // 16-byte registers holding them

@@ -95,7 +95,7 @@ def test_topk_route_ties_go_to_lower_index(hip):
     assert np.allclose(w[:4], 0.25)
 
 
-@pytest.mark.parametrize("A,E", [(32, 128), (256, 128), (1024, 128), (2500, 7), (1, 4), (4096, 256)])
+@pytest.mark.parametrize("A,E", [(32, 128), (256, 128), (1024, 128), (2500, 7), (1, 4), (4096, 256), (16384, 128), (20011, 1000), (3000, 1)])
 def test_moe_sort_is_stable_argsort(hip, A, E):
     from rmlx_amd import ops
     from rmlx_amd.runtime import DeviceBuffer
