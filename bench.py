@@ -262,9 +262,10 @@ def main():
         # matrix work before its clock settles (a 100-launch window reads 15 % slower, a 2 000-launch one 3 %)
         # (short runs, as under a counter pass, keep their own count)
         gemm_steps = max(args.steps, 10000) if args.steps >= 1000 else args.steps
-        for m in (128, 512):
-            r = bench_matmul(ops, rt, timer, rng, m, 4096, 4096, 4, "f16", gemm_steps, args.warmup, 4 * 9437184)
-            r["steps"] = gemm_steps
+        for m in (128, 512, 4096):
+            m_steps = gemm_steps if m <= 512 else max(50, gemm_steps // 10)
+            r = bench_matmul(ops, rt, timer, rng, m, 4096, 4096, 4, "f16", m_steps, min(args.warmup, m_steps), 4 * 9437184)
+            r["steps"] = m_steps
             r["mfma_frac"] = r["tflops"] / MFMA_F16_PEAK_TF
             extra[f"q4_qmm_m{m}_4096"] = r
         for name, kern in (("q8_qmm_bf16_m128_n12288", rt.KERNEL_AUTO), ("q8_qmm_bf16_m128_n12288_bf16_mfma", rt.KERNEL_QMM_BF16)):
