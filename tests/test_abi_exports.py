@@ -65,3 +65,15 @@ def test_qweight_validation_needs_no_gpu():
         per = 32 // bits
         assert create(((8 * 64 + per - 1) // per) * 4, 16, 16, 64, bits, 8, 64) == rt.OK
         L.rmlx_hip_qweight_destroy(h)
+
+
+def test_expert_gemm_threshold_is_plain_host_state():
+    """The GEMV / grouped-GEMM threshold of the expert projections: default 8 rows per expert, set returns the old value."""
+    from rmlx_amd import ops
+    prev = ops.set_expert_gemm_min_rows(5)
+    try:
+        assert prev == 8
+        assert ops.set_expert_gemm_min_rows(0) == 5
+        assert ops.set_expert_gemm_min_rows(prev) == 0
+    finally:
+        ops.set_expert_gemm_min_rows(prev)
