@@ -257,9 +257,9 @@ int32_t rmlx_hip_moe_forward_grouped(const rmlx_qweight* gate, const rmlx_qweigh
 /* Kernel choice of the expert projections (ExpertGroup and both MoeLayer entry points): batches with at least
  * `min_rows` rows per expert on average (rows / num_experts, for ExpertGroup rows / n_items) multiply with the
  * grouped MFMA GEMM (row tiles of 32 or 64 rows of one expert, weights dequantised in registers; 4- / 8-bit, group
- * size 64, dimensions in multiples of 512), smaller ones with the streaming GEMV, which reads an expert's
+ * sizes 32 / 64 / 128 (one for the three projections), dimensions in multiples of 512), smaller ones with the streaming GEMV, which reads an expert's
  * weights once per 8 rows; gather_qmm does the same from one and a half times as many rows per batch entry on
- * (4-bit, group size 64, N % 128 == 0, K % 512 == 0).  0 = never the GEMM.  The default (8) is the measured crossover; the setting is
+ * (4-bit, group sizes 32 / 64 / 128, N % 128 == 0, K % 512 == 0).  0 = never the GEMM.  The default (8) is the measured crossover; the setting is
  * process-wide.  No counterpart in the reference, whose MoE layer picks its kernels by a configured
  * `MoeStrategy` (crates/rmlx-nn/src/moe.rs:515-541).  Returns the previous value. */
 uint32_t rmlx_hip_set_expert_gemm_min_rows(uint32_t min_rows);

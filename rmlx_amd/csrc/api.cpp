@@ -304,7 +304,7 @@ int32_t check_expert_weights(const char* who, const rmlx_qweight* gate, const rm
     return fail(RMLX_INVALID_SHAPE, "%s: down weight must be [%zu, %zu, %zu], got [%zu, %zu, %zu]", who, E, D, I,
                 down->n_experts, down->out_features, down->in_features);
   const rmlx_qweight* all[3] = {gate, up, down};
-  bool fast = true;
+  bool fast = true, uniform = true;  // uniform: one bit width and one group size, 16-byte aligned buffers
   for (const rmlx_qweight* q : all) {
     if (q == nullptr) continue;
     if (q->bits != 2 && q->bits != 4 && q->bits != 8)
@@ -313,6 +313,8 @@ int32_t check_expert_weights(const char* who, const rmlx_qweight* gate, const rm
     // the same width for all three projections (gate and up share one launch)
     const bool gs_ok = q->bits == 4 ? (q->group_size == 64 || q->group_size == 128) : (q->bits == 8 && q->group_size == 64);
     if (!gs_ok || q->bits != gate->bits || !aligned16(q->w) || !aligned16(q->s) || !aligned16(q->b)) fast = false;
+    if (q->bits != gate->bits || q->group_size != gate->group_size || !aligned16(q->w) || !aligned16(q->s) || !aligned16(q->b))
+      uniform = false;
   }
   RMLX_TRY(checked_u32(E, "num_experts", &sh->E));
   RMLX_TRY(checked_u32(D, "hidden_dim", &sh->D));
@@ -325,8 +327,9 @@ int32_t check_expert_weights(const char* who, const rmlx_qweight* gate, const rm
   if (up != nullptr && up->group_size != gate->group_size) fast = false;
   sh->fused = fused;
   sh->portable = !fast;
-  sh->gemm = fast && gate->group_size == 64 && down->group_size == 64 &&
-             qmm_rw_grouped_supported(sh->I, sh->D, 64, gate->bits) && qmm_rw_grouped_supported(sh->D, sh->I, 64, gate->bits);
+  // the grouped GEMM also takes group sizes the streaming kernels do not (32; 128 at 8 bits)
+  sh->gemm = uniform && qmm_rw_grouped_supported(sh->I, sh->D, gate->group_size, gate->bits) &&
+             qmm_rw_grouped_supported(sh->D, sh->I, gate->group_size, gate->bits);
   return RMLX_OK;
 }
 
@@ -373,27 +376,28 @@ int32_t run_expert_ffn(const rmlx_qweight* gate, const rmlx_qweight* up, const r
                        void* y, int y_f32, uint32_t gemm_tile_rows, hipStream_t stream) {
   const uint32_t per = 32 / gate->bits;  // values per u32 word: 8 (4-bit) or 4 (8-bit)
   if (gemm_tile_rows != 0) {  // the table holds row tiles of that many rows and n_chunks its length
+    const uint32_t gs = gate->group_size;  // one group size for the three projections (ExpertShapes::gemm)
     GroupedQmmArgs a{};
     a.w = gate->w; a.s = gate->s; a.b = gate->b;
     if (sh.fused) {
       a.w1 = gate->w + (size_t)sh.I * (sh.D / per);
-      a.s1 = gate->s + (size_t)sh.I * (sh.D / 64);
-      a.b1 = gate->b + (size_t)sh.I * (sh.D / 64);
+      a.s1 = gate->s + (size_t)sh.I * (sh.D / gs);
+      a.b1 = gate->b + (size_t)sh.I * (sh.D / gs);
     } else {
       a.w1 = up->w; a.s1 = up->s; a.b1 = up->b;
     }
     const size_t rows = sh.fused ? 2 * (size_t)sh.I : sh.I;
-    a.N = sh.I; a.K = sh.D; a.bits = gate->bits;
+    a.N = sh.I; a.K = sh.D; a.bits = gate->bits; a.group_size = gs;
     a.expert_stride_w = rows * (sh.D / per);
-    a.expert_stride_s = rows * (sh.D / 64);
+    a.expert_stride_s = rows * (sh.D / gs);
     a.x = x; a.row_map = row_map; a.out = h; a.out_f32 = 0;
     a.tile_tab = chunk_tab; a.n_tiles_dev = n_chunks; a.max_tiles = max_chunks; a.tile_rows = gemm_tile_rows;
     RMLX_TRY(launch_qmm_rw_grouped(a, stream));
     GroupedQmmArgs d{};
     d.w = down->w; d.s = down->s; d.b = down->b;
-    d.N = sh.D; d.K = sh.I; d.bits = down->bits;
+    d.N = sh.D; d.K = sh.I; d.bits = down->bits; d.group_size = gs;
     d.expert_stride_w = (size_t)sh.D * (sh.I / per);
-    d.expert_stride_s = (size_t)sh.D * (sh.I / 64);
+    d.expert_stride_s = (size_t)sh.D * (sh.I / gs);
     d.x = h; d.row_map = nullptr; d.out = y; d.out_f32 = y_f32;
     d.tile_tab = chunk_tab; d.n_tiles_dev = n_chunks; d.max_tiles = max_chunks; d.tile_rows = gemm_tile_rows;
     return launch_qmm_rw_grouped(d, stream);
@@ -820,8 +824,8 @@ int32_t rmlx_hip_gather_qmm(const rmlx_array* x, const void* w_packed_dev, size_
   // Every entry has exactly m_per_batch rows, so the streaming GEMV wastes nothing up to a full chunk of 8 rows
   // and the crossover lies higher than for routed batches: one and a half times the threshold (measured: 8 rows
   // per entry 50 us streamed, 64 us on the GEMM; 64 rows 91 us on the GEMM).
-  if (fast && gemm_min_rows != 0 && m_per_batch >= gemm_min_rows + gemm_min_rows / 2 &&
-      qmm_rw_grouped_supported(N32, K32, group_size, 4)) {
+  if (gemm_min_rows != 0 && m_per_batch >= gemm_min_rows + gemm_min_rows / 2 && aligned16(w) && aligned16(sc) &&
+      aligned16(bi) && aligned16(xk) && qmm_rw_grouped_supported(N32, K32, group_size, 4)) {
     // many rows per entry: row tiles of one expert each on the grouped MFMA GEMM
     const uint32_t tile_rows = m_per_batch <= 32 ? 32u : kGroupedTileRows;
     const uint32_t per = ((uint32_t)m_per_batch + tile_rows - 1) / tile_rows;
@@ -833,7 +837,7 @@ int32_t rmlx_hip_gather_qmm(const rmlx_array* x, const void* w_packed_dev, size_
     RMLX_TRY(launch_build_gather_chunks(idx, B32, (uint32_t)m_per_batch, E32, tile_rows, t, t + 3 * n_tiles, s));
     GroupedQmmArgs a{};
     a.w = w; a.s = sc; a.b = bi;
-    a.N = N32; a.K = K32; a.bits = 4;
+    a.N = N32; a.K = K32; a.bits = 4; a.group_size = group_size;
     a.expert_stride_w = (uint64_t)n * (k / 8);
     a.expert_stride_s = (uint64_t)n * gpr;
     a.x = xk; a.out = out_f16_dev;
@@ -1012,7 +1016,7 @@ int32_t rmlx_hip_expert_group_grouped_forward(const rmlx_qweight* gate, const rm
     RMLX_TRY(launch_cast_to_f16(x->data, x->dtype, static_cast<__half*>(cast.ptr), total * sh.D, s));
     xk = static_cast<const __half*>(cast.ptr);
   }
-  if (sh.portable) {  // expert of every packed row, then the portable kernels
+  if (sh.portable && !gemm) {  // expert of every packed row, then the portable kernels
     std::vector<uint32_t> expert_of;
     expert_of.reserve(total);
     for (size_t i = 0; i < n_items; ++i) expert_of.insert(expert_of.end(), batch_sizes_host[i], expert_idx_host[i]);
@@ -1073,7 +1077,7 @@ int32_t moe_grouped_impl(const rmlx_qweight* gate, const rmlx_qweight* up, const
     RMLX_TRY(launch_cast_to_f16(x->data, x->dtype, static_cast<__half*>(cast.ptr), T * sh.D, s));
     xk = static_cast<const __half*>(cast.ptr);
   }
-  if (sh.portable) {
+  if (sh.portable && !gemm) {
     // Assignments stay in their own order: position a holds token a / top_k and expert idx[a].
     if (route != nullptr)
       RMLX_TRY(launch_topk_route(route->logits, route->bias, T32, sh.E, (uint32_t)top_k, 1, route->idx_out, route->w_out,

@@ -177,12 +177,13 @@ int32_t launch_qmm_rw(const QmmArgs& a, uint32_t group_size, hipStream_t s);
 // row tile (kGroupedTileRows rows of one expert) takes its expert and rows from a device table of
 // (expert, first row position, row count) triples (bit 31 of the count: write zeros instead of computing;
 // not for a pair); `n_tiles_dev` holds the table's length.  With a second
-// weight (w1 / s1 / b1: the up projection) the store writes silu(x Wg^T) * (x Wu^T).  Group size 64.
+// weight (w1 / s1 / b1: the up projection) the store writes silu(x Wg^T) * (x Wu^T).
 constexpr uint32_t kGroupedTileRows = 64;
 struct GroupedQmmArgs {
   const uint32_t* w; const __half* s; const __half* b;     // expert 0 of the (gate) weight
   const uint32_t* w1; const __half* s1; const __half* b1;  // expert 0 of the up weight, or null
   uint32_t N, K, bits;       // output columns (of a pair: columns of the product), input features
+  uint32_t group_size;       // 32, 64 or 128
   uint64_t expert_stride_w;  // u32 words per expert
   uint64_t expert_stride_s;  // halves per expert
   const __half* x;           // [x_rows, K] f16

@@ -505,9 +505,9 @@ __global__ __launch_bounds__(64 * NW) void qmm_rw_kernel(RwParams p) {
 }
 
 // DUAL: gate/up pair with the SwiGLU store (see MODE 2 above)
-template <int MF, int NF, int BITS, int NW, bool DUAL>
+template <int MF, int NF, int BITS, int NW, bool DUAL, int GS = 64>
 __global__ __launch_bounds__(64 * NW) void qmm_rw_grouped_kernel(RwParams p) {
-  qmm_rw_body<MF, NF, BITS, NW, false, 64, DUAL ? 2 : 1>(p);
+  qmm_rw_body<MF, NF, BITS, NW, false, GS, DUAL ? 2 : 1>(p);
 }
 
 // out[m, c..c+3] = epilogue(sum over the ksplit partial sums, in split order); one thread per four columns
@@ -650,12 +650,14 @@ int32_t launch_qmm_rw(const QmmArgs& a, uint32_t group_size, hipStream_t s) {
 }
 
 bool qmm_rw_grouped_supported(uint32_t N, uint32_t K, uint32_t group_size, uint32_t bits) {
-  return group_size == 64 && (bits == 4 || bits == 8) && N > 0 && K > 0 && N % 128 == 0 && K % (kBlockK * kUnroll) == 0;
+  return (group_size == 32 || group_size == 64 || group_size == 128) && (bits == 4 || bits == 8) && N > 0 && K > 0 &&
+         N % 128 == 0 && K % (kBlockK * kUnroll) == 0;
 }
 
 int32_t launch_qmm_rw_grouped(const GroupedQmmArgs& a, hipStream_t s) {
-  if (!qmm_rw_grouped_supported(a.N, a.K, 64, a.bits))
-    return fail(RMLX_INVALID_SHAPE, "grouped qmm: unsupported shape N=%u K=%u bits=%u", a.N, a.K, a.bits);
+  if (!qmm_rw_grouped_supported(a.N, a.K, a.group_size, a.bits))
+    return fail(RMLX_INVALID_SHAPE, "grouped qmm: unsupported shape N=%u K=%u bits=%u group_size=%u", a.N, a.K, a.bits,
+                a.group_size);
   if (a.max_tiles == 0) return RMLX_OK;
   const bool dual = a.w1 != nullptr;
   if (dual && a.out_f32) return fail(RMLX_RUNTIME_ERROR, "grouped qmm: the gate/up pair writes f16");
@@ -677,15 +679,17 @@ int32_t launch_qmm_rw_grouped(const GroupedQmmArgs& a, hipStream_t s) {
   if (a.tile_rows != 32 && a.tile_rows != kGroupedTileRows)
     return fail(RMLX_RUNTIME_ERROR, "grouped qmm: row tiles of %u rows", a.tile_rows);
   const dim3 grid(p.tiles_m * p.tiles_n), block(512);
-#define RWG_LAUNCH(MFV, BITSV)                                                                                \
-  if (dual) hipLaunchKernelGGL((qmm_rw_grouped_kernel<MFV, 2, BITSV, 8, true>), grid, block, 0, s, p);          \
-  else if (wide) hipLaunchKernelGGL((qmm_rw_grouped_kernel<MFV, 2, BITSV, 8, false>), grid, block, 0, s, p);    \
-  else hipLaunchKernelGGL((qmm_rw_grouped_kernel<MFV, 1, BITSV, 8, false>), grid, block, 0, s, p);
-  if (a.tile_rows == 32) {
-    if (a.bits == 4) { RWG_LAUNCH(2, 4) } else { RWG_LAUNCH(2, 8) }
-  } else {
-    if (a.bits == 4) { RWG_LAUNCH(4, 4) } else { RWG_LAUNCH(4, 8) }
-  }
+#define RWG_LAUNCH(MFV, BITSV, GSV)                                                                                \
+  if (dual) hipLaunchKernelGGL((qmm_rw_grouped_kernel<MFV, 2, BITSV, 8, true, GSV>), grid, block, 0, s, p);          \
+  else if (wide) hipLaunchKernelGGL((qmm_rw_grouped_kernel<MFV, 2, BITSV, 8, false, GSV>), grid, block, 0, s, p);    \
+  else hipLaunchKernelGGL((qmm_rw_grouped_kernel<MFV, 1, BITSV, 8, false, GSV>), grid, block, 0, s, p);
+#define RWG_TILE(BITSV, GSV)                                     \
+  if (a.tile_rows == 32) { RWG_LAUNCH(2, BITSV, GSV) } else { RWG_LAUNCH(4, BITSV, GSV) }
+#define RWG_BITS(GSV) \
+  if (a.bits == 4) { RWG_TILE(4, GSV) } else { RWG_TILE(8, GSV) }
+  if (a.group_size == 64) { RWG_BITS(64) } else if (a.group_size == 32) { RWG_BITS(32) } else { RWG_BITS(128) }
+#undef RWG_BITS
+#undef RWG_TILE
 #undef RWG_LAUNCH
   RMLX_HIP_CHECK(hipGetLastError());
   return RMLX_OK;

@@ -235,35 +235,36 @@ def test_gather_qmm_async_out_of_range_rows_are_zero(hip):
     assert np.all(out[~good] == 0)
 
 
-@pytest.mark.parametrize("n,k,mpb", [(128, 512, 12), (384, 1024, 70), (256, 512, 64), (128, 1536, 129)])
-def test_gather_qmm_many_rows_per_entry_on_the_grouped_gemm(hip, n, k, mpb):
+@pytest.mark.parametrize("n,k,mpb,gs", [(128, 512, 12, 64), (384, 1024, 70, 64), (256, 512, 64, 64), (128, 1536, 129, 64),
+                                        (128, 512, 40, 32), (256, 1024, 70, 128)])
+def test_gather_qmm_many_rows_per_entry_on_the_grouped_gemm(hip, n, k, mpb, gs):
     """From 12 rows per batch entry on, gather_qmm multiplies with the grouped MFMA GEMM (row tiles of 64 rows of one
     expert; the last tile of an entry ragged).  Against the oracle; on a stream, rows of an out-of-range index are zero."""
     from rmlx_amd import ops
     from rmlx_amd.runtime import DeviceBuffer, Stream
     rng = np.random.default_rng(n + k + mpb)
     E, batch = 5, 6
-    words, s, b = make_weight(rng, n, k, 4, lead=(E,))
+    words, s, b = make_weight(rng, n, k, 4, gs, lead=(E,))
     x = rng.standard_normal((batch, mpb, k)).astype(np.float16)
     idx = np.array([4, 0, 3, 3, 1, 0], np.uint32)
-    print(f"gather_qmm gemm n={n} k={k} mpb={mpb}", flush=True)
+    print(f"gather_qmm gemm n={n} k={k} mpb={mpb} gs={gs}", flush=True)
     xd, wd, sd, bd = [DeviceBuffer.from_numpy(a) for a in (x, words, s, b)]
-    out = ops.gather_qmm(xd, wd, sd, bd, DeviceBuffer.from_numpy(idx), batch, mpb, n, k, E, 64).numpy()
-    ref = model.gather_qmm(x, words, s, b, idx, 64)
+    out = ops.gather_qmm(xd, wd, sd, bd, DeviceBuffer.from_numpy(idx), batch, mpb, n, k, E, gs).numpy()
+    ref = model.gather_qmm(x, words, s, b, idx, gs)
     assert_close(out, ref, "gather_qmm (GEMM)")
     prev = ops.set_expert_gemm_min_rows(0)
     try:
-        out_stream = ops.gather_qmm(xd, wd, sd, bd, DeviceBuffer.from_numpy(idx), batch, mpb, n, k, E, 64).numpy()
+        out_stream = ops.gather_qmm(xd, wd, sd, bd, DeviceBuffer.from_numpy(idx), batch, mpb, n, k, E, gs).numpy()
     finally:
         ops.set_expert_gemm_min_rows(prev)
     assert_close(out_stream, ref, "gather_qmm (streaming GEMV)")
     bad = np.array([4, 9, 3, 7, 1, 0], np.uint32)
     st = Stream()
-    out = ops.gather_qmm(xd, wd, sd, bd, DeviceBuffer.from_numpy(bad), batch, mpb, n, k, E, 64, stream=st)
+    out = ops.gather_qmm(xd, wd, sd, bd, DeviceBuffer.from_numpy(bad), batch, mpb, n, k, E, gs, stream=st)
     st.sync()
     out = out.numpy()
     good = bad < E
-    assert_close(out[good], model.gather_qmm(x[good], words, s, b, bad[good], 64), "valid entries")
+    assert_close(out[good], model.gather_qmm(x[good], words, s, b, bad[good], gs), "valid entries")
     assert np.all(out[~good] == 0)
 
 
@@ -425,38 +426,41 @@ def test_moe_other_bit_widths_and_group_sizes(hip, bits, gs, D, I, fused):
 
 
 @pytest.mark.parametrize("T", [150, 50])
-@pytest.mark.parametrize("bits,D,I,fused", [(4, 512, 512, True), (4, 1024, 1536, False), (8, 512, 1024, True), (8, 1024, 512, False)])
-def test_moe_many_rows_per_expert_on_the_grouped_gemm(hip, bits, D, I, fused, T):
+@pytest.mark.parametrize("bits,gs,D,I,fused", [(4, 64, 512, 512, True), (4, 64, 1024, 1536, False), (8, 64, 512, 1024, True),
+                                               (8, 64, 1024, 512, False), (4, 32, 512, 1024, True), (4, 128, 1024, 512, False),
+                                               (8, 32, 512, 512, False), (8, 128, 512, 512, True)])
+def test_moe_many_rows_per_expert_on_the_grouped_gemm(hip, bits, gs, D, I, fused, T):
     """Batches with many rows per expert (here 75 or 25 on average; from 8 on) multiply with the grouped MFMA GEMM: row
     tiles of 64 rows of one expert (32 rows while the average is at most 32).  Skewed routing gives one expert
-    three tiles, another a ragged one and one almost nothing.  Checked against the oracle, and the streaming GEMV
-    path (threshold 0) on the same inputs beside it."""
+    three tiles, another a ragged one and one almost nothing.  Group sizes 32, 64 and 128.  Checked against the
+    oracle, and the path below the threshold (streaming GEMV, or the portable kernels where it does not take the
+    group size) on the same inputs beside it."""
     from rmlx_amd import ops
     from rmlx_amd.runtime import DeviceBuffer
-    rng = np.random.default_rng(bits * 1000 + D + I + T)
+    rng = np.random.default_rng(bits * 1000 + D + I + T + gs)
     E, K = 4, 2
 
     def weight(n, k):
-        return make_weight(rng, n, k, bits, 64, lead=(E,))
+        return make_weight(rng, n, k, bits, gs, lead=(E,))
 
     if fused:
         gu = weight(2 * I, D)
         gate, up = tuple(a[:, :I] for a in gu), tuple(a[:, I:] for a in gu)
-        gh, uh = ops.QuantizedWeight.from_numpy(*gu, 64, bits), None
+        gh, uh = ops.QuantizedWeight.from_numpy(*gu, gs, bits), None
     else:
         gate, up = weight(I, D), weight(I, D)
-        gh, uh = ops.QuantizedWeight.from_numpy(*gate, 64, bits), ops.QuantizedWeight.from_numpy(*up, 64, bits)
+        gh, uh = ops.QuantizedWeight.from_numpy(*gate, gs, bits), ops.QuantizedWeight.from_numpy(*up, gs, bits)
     down = weight(D, I)
-    dh = ops.QuantizedWeight.from_numpy(*down, 64, bits)
+    dh = ops.QuantizedWeight.from_numpy(*down, gs, bits)
     x = make_x(rng, T, D)
     logits = rng.standard_normal((T, E)).astype(np.float32)
     logits[:, 0] += 3.0
     logits[:, 3] -= 4.0
     idx, w, counts, _ = model.topk_route(logits, K)
     assert counts.max() > (128 if T == 150 else 32) and counts.min() < 8, counts
-    ref = model.moe_forward(x, idx, w, gate, up, down, 64, K, bits=bits)
+    ref = model.moe_forward(x, idx, w, gate, up, down, gs, K, bits=bits)
     xd, idxd, wd = DeviceBuffer.from_numpy(x), DeviceBuffer.from_numpy(idx), DeviceBuffer.from_numpy(w)
-    print(f"grouped gemm moe T={T} bits={bits} D={D} I={I} fused={fused} counts={counts.tolist()}", flush=True)
+    print(f"grouped gemm moe T={T} bits={bits} gs={gs} D={D} I={I} fused={fused} counts={counts.tolist()}", flush=True)
     prev = ops.set_expert_gemm_min_rows(8)
     try:
         out_gemm = ops.moe_forward_grouped(gh, uh, dh, xd, idxd, wd, K).numpy()
@@ -468,11 +472,11 @@ def test_moe_many_rows_per_expert_on_the_grouped_gemm(hip, bits, D, I, fused, T)
         outs = group.grouped_forward([(e, DeviceBuffer.from_numpy(v)) for e, v in items])
         for (e, v), (_, yv) in zip(items, outs):
             ones = np.ones((len(v), 1))
-            assert_close(yv, model.moe_forward(v, np.full((len(v), 1), e), ones, gate, up, down, 64, 1, bits=bits),
+            assert_close(yv, model.moe_forward(v, np.full((len(v), 1), e), ones, gate, up, down, gs, 1, bits=bits),
                          f"ExpertGroup (GEMM) expert {e} rows {len(v)}")
         ops.set_expert_gemm_min_rows(0)
         out_stream = ops.moe_forward_grouped(gh, uh, dh, xd, idxd, wd, K).numpy()
-        assert_close(out_stream, ref, "moe_forward_grouped (streaming GEMV)")
+        assert_close(out_stream, ref, "moe_forward_grouped (below the threshold)")
     finally:
         ops.set_expert_gemm_min_rows(prev)
 
