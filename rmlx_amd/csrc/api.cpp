@@ -118,7 +118,8 @@ bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) ==
 enum { KERNEL_AUTO = 0, KERNEL_QMV = 1, KERNEL_QMM = 2, KERNEL_GENERIC = 3, KERNEL_QMM_BF16 = 4, KERNEL_QMM_LDS = 5,
        KERNEL_QMV_ROWS = 6 };
 constexpr uint32_t kQmvMaxM = 16;
-constexpr uint32_t kM1MaxRows = 2;        // group size 64: rows taken by the single-row kernel (measured: 3 and 4 rows are faster on the matrix unit)
+// group size 64: rows taken by the single-row kernel (measured: 3 and 4 rows are faster on the matrix unit)
+constexpr uint32_t kM1MaxRows = 2;
 constexpr uint32_t kM1MaxRowsOther = 16;  // shapes the multi-row GEMV does not take: the alternative is the portable kernel
 
 // What is fused around a matmul: the store epilogue (kind / ptr / dtype) and the RMSNorm prologue
@@ -342,8 +343,8 @@ uint32_t expert_gemm_tile_rows(const ExpertShapes& sh, uint64_t rows, uint64_t g
 }
 
 // The same block on the portable kernels, for expert weights the streaming GEMV does not take (2-bit,
-// group size 32, 8-bit at group size 128, dimensions that are no multiples of 512 (4-bit) or 256 / 16 (8-bit)): every position multiplies with its own
-// expert's rows.  x: f16 [positions, D] (already gathered); expert_of: device u32 [positions]; y: f16 [positions, D].
+// group size 32, 8-bit at group size 128, dimensions that are no multiples of 512 (4-bit) or 256 / 16
+// (8-bit)) in batches below the grouped GEMM's threshold: every position multiplies with its own expert's rows.  x: f16 [positions, D] (already gathered); expert_of: device u32 [positions]; y: f16 [positions, D].
 int32_t run_expert_ffn_portable(const rmlx_qweight* gate, const rmlx_qweight* up, const rmlx_qweight* down,
                                 const ExpertShapes& sh, const __half* x, const uint32_t* expert_of, uint32_t positions,
                                 __half* y, hipStream_t stream) {
