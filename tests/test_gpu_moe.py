@@ -481,6 +481,29 @@ def test_moe_many_rows_per_expert_on_the_grouped_gemm(hip, bits, gs, D, I, fused
         ops.set_expert_gemm_min_rows(prev)
 
 
+@pytest.mark.parametrize("E,K,T,x_dtype", [(1, 1, 100, "f16"), (3, 3, 40, "f32"), (2, 1, 129, "f16"), (6, 2, 33, "f32")])
+def test_grouped_gemm_edge_routings(hip, E, K, T, x_dtype):
+    """Corner cases of the routed block above the GEMM threshold: a single expert, every expert for every token,
+    one row more than two full tiles, f32 activations (cast on the way in)."""
+    from rmlx_amd import ops
+    from rmlx_amd.runtime import DeviceBuffer
+    rng = np.random.default_rng(E * 100 + K * 10 + T)
+    D, I = 512, 512
+    gate, up, down, gh, uh, dh = _experts(rng, E, D, I, E % 2 == 0)
+    x = make_x(rng, T, D)
+    logits = rng.standard_normal((T, E)).astype(np.float32)
+    idx, w, counts, _ = model.topk_route(logits, K)
+    assert T * K >= 8 * E
+    ref = model.moe_forward(x, idx, w, gate, up, down, 64, K)
+    xin = x if x_dtype == "f16" else x.astype(np.float32)
+    print(f"grouped gemm edge E={E} K={K} T={T} x={x_dtype} counts={counts.tolist()}", flush=True)
+    out = ops.moe_forward_grouped(gh, uh, dh, DeviceBuffer.from_numpy(xin), DeviceBuffer.from_numpy(idx),
+                                  DeviceBuffer.from_numpy(w), K).numpy()
+    assert_close(out, ref, "moe_forward_grouped")
+    out2 = ops.moe_forward(gh, uh, dh, DeviceBuffer.from_numpy(xin), DeviceBuffer.from_numpy(logits), K).numpy()
+    assert_close(out2, ref, "moe_forward")  # (routing weights from the device: equal to the oracle's up to f32 rounding)
+
+
 def _two_bit(rng, E, n, k, gs):
     words = rng.integers(0, 2**32, size=(E, n, k // 16), dtype=np.uint64).astype(np.uint32)
     scales = rng.uniform(0.02, 0.08, size=(E, n, k // gs)).astype(np.float16)
