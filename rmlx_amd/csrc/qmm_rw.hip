@@ -155,11 +155,15 @@ __device__ __forceinline__ void qmm_rw_body(const RwParams p) {  // by value: a 
   const __half* bbase[2] = {p.b, p.b1};
   const uint32_t total = p.tiles_m * p.tiles_n;
   if (MODE != 0) {
-    // consecutive ids share a row tile (its activations); with tiles_n a multiple of 8 the row tiles of one
-    // expert land on the same XCD for every column tile, so its L2 serves the second read of a weight panel
-    nt = wg % p.tiles_n;
-    const uint32_t te = wg / p.tiles_n;
-    if (te >= *p.n_tiles) return;
+    // Consecutive workgroup ids go round-robin over the 8 XCDs.  XCD x takes a contiguous run of the table
+    // (an eighth of its row tiles) and walks it row tile by row tile, column tiles inside: the workgroups that
+    // share a row tile's activations, and the consecutive row tiles of one expert that share its weight panels,
+    // run on one XCD at about the same time, so each is fetched into one L2 once.
+    const uint32_t n_t = *p.n_tiles, run = (n_t + 7) / 8;
+    const uint32_t xcd = wg % 8, local = wg / 8, tl = local / p.tiles_n;
+    nt = local % p.tiles_n;
+    const uint32_t te = xcd * run + tl;
+    if (tl >= run || te >= n_t) return;
     const uint32_t expert = p.tile_tab[3 * te];
     row_lo = p.tile_tab[3 * te + 1];
     const uint32_t cnt = p.tile_tab[3 * te + 2];
@@ -670,7 +674,7 @@ int32_t launch_qmm_rw_grouped(const GroupedQmmArgs& a, hipStream_t s) {
   p.epi_kind = EPI_NONE; p.ksplit = 1;
   p.tile_tab = a.tile_tab; p.n_tiles = a.n_tiles_dev;
   p.estride_w = a.expert_stride_w; p.estride_s = a.expert_stride_s;
-  p.tiles_m = a.max_tiles;
+  p.tiles_m = (a.max_tiles + 7) / 8 * 8;  // (the grid covers eight equal runs of row tiles, one per XCD)
   // row tiles of 16 * 4 = kGroupedTileRows rows, 8 waves; a pair: 128 columns of each weight per workgroup,
   // one weight: 256 columns when they divide, else 128
   const bool wide = !dual && a.N % 256 == 0;
