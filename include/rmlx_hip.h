@@ -231,8 +231,9 @@ int32_t rmlx_hip_silu_gate(const void* gate_in_f16_dev, const void* up_in_f16_de
  * after another in x ([sum batch_i, D] f16); out receives the per-item outputs in the same
  * packing.  Per item: y = (silu(x Wg^T) * (x Wu^T)) Wd^T with stacked expert weights (the streaming kernels
  * take 4-bit weights with group size 64 or 128 and dimensions in multiples of 512, and 8-bit weights with group size 64
- * and dimensions in multiples of 256; every other 2- / 4- / 8-bit weight the type admits runs the same block on the
- * portable kernels)
+ * and dimensions in multiples of 256; batches with many rows per expert take the grouped MFMA GEMM, see
+ * rmlx_hip_set_expert_gemm_min_rows; every other 2- / 4- / 8-bit weight the type admits runs the same block
+ * on the portable kernels)
  * gate/up [E, I, D] and down [E, D, I].  `up` may be NULL when `gate` holds the fused
  * [E, 2I, D] layout (gate rows first).  expert_idx and batch_sizes are HOST arrays.
  * Validation as the reference: idx < E, n_items == 0 -> nothing to do. */
@@ -254,14 +255,15 @@ int32_t rmlx_hip_moe_forward_grouped(const rmlx_qweight* gate, const rmlx_qweigh
                                      const float* expert_weights_dev, size_t top_k,
                                      void* out_f16_dev, size_t out_bytes, rmlx_stream stream);
 
-/* Kernel choice of the expert projections (ExpertGroup and both MoeLayer entry points): batches with at least
- * `min_rows` rows per expert on average (rows / num_experts, for ExpertGroup rows / n_items) multiply with the
- * grouped MFMA GEMM (row tiles of 32 or 64 rows of one expert, weights dequantised in registers; 4- / 8-bit, group
- * sizes 32 / 64 / 128 (one for the three projections), dimensions in multiples of 512), smaller ones with the streaming GEMV, which reads an expert's
- * weights once per 8 rows; gather_qmm does the same from one and a half times as many rows per batch entry on
- * (4-bit, group sizes 32 / 64 / 128, N % 128 == 0, K % 512 == 0).  0 = never the GEMM.  The default (8) is the measured crossover; the setting is
- * process-wide.  No counterpart in the reference, whose MoE layer picks its kernels by a configured
- * `MoeStrategy` (crates/rmlx-nn/src/moe.rs:515-541).  Returns the previous value. */
+/* Kernel choice of the expert projections (ExpertGroup and both MoeLayer entry points): batches with at
+ * least `min_rows` rows per expert on average (rows / num_experts; for ExpertGroup rows / n_items) multiply
+ * with the grouped MFMA GEMM -- row tiles of 32 or 64 rows of one expert, weights dequantised in registers;
+ * 4- / 8-bit, group sizes 32 / 64 / 128 (one for the three projections), hidden and intermediate dimensions
+ * in multiples of 512 -- smaller ones with the streaming GEMV, which reads an expert's weights once per 8
+ * rows.  gather_qmm does the same from one and a half times as many rows per batch entry on (4-bit, group
+ * sizes 32 / 64 / 128, N % 128 == 0, K % 512 == 0).  0 = never the GEMM.  The default (8) is the measured
+ * crossover; the setting is process-wide.  No counterpart in the reference, whose MoE layer picks its
+ * kernels by a configured `MoeStrategy` (crates/rmlx-nn/src/moe.rs:515-541).  Returns the previous value. */
 uint32_t rmlx_hip_set_expert_gemm_min_rows(uint32_t min_rows);
 
 /* Routing + the block above in one call: gate_logits [T,E] (the router's output). */
