@@ -558,3 +558,32 @@ def test_config5_moe(hip, config5, T):
     ref = model.moe_forward(x[toks], idx[sel], w[sel], gate, up, down, 64, 8)
     assert_close(out[toks], ref, f"config5 T={T}")
     assert np.all(np.isfinite(out.astype(np.float32)))
+
+
+@pytest.mark.parametrize("T", [300, 700])
+def test_config5_moe_prefill_sizes(hip, config5, T):
+    """Config 5 at prefill-sized batches (19 / 44 rows per expert on average: the grouped GEMM with 32- / 64-row tiles).
+    The oracle checks a sample of tokens; every token is checked against the streaming GEMV path (threshold 0) on the
+    same inputs, which shares no matrix kernel with the GEMM path."""
+    from rmlx_amd import ops
+    from rmlx_amd.runtime import DeviceBuffer
+    gate, up, down, gh, uh, dh = config5
+    rng = np.random.default_rng(7000 + T)
+    x = make_x(rng, T, 4096)
+    logits = rng.standard_normal((T, 128)).astype(np.float32)
+    idx, w, _, _ = model.topk_route(logits, 8)
+    xd, idxd, wd = DeviceBuffer.from_numpy(x), DeviceBuffer.from_numpy(idx), DeviceBuffer.from_numpy(w)
+    print(f"config5 prefill T={T}", flush=True)
+    out = ops.moe_forward_grouped(gh, uh, dh, xd, idxd, wd, 8).numpy()
+    prev = ops.set_expert_gemm_min_rows(0)
+    try:
+        out_stream = ops.moe_forward_grouped(gh, uh, dh, xd, idxd, wd, 8).numpy()
+    finally:
+        ops.set_expert_gemm_min_rows(prev)
+    toks = np.sort(rng.choice(T, size=6, replace=False))
+    sel = (toks[:, None] * 8 + np.arange(8)[None, :]).reshape(-1)
+    ref = model.moe_forward(x[toks], idx[sel], w[sel], gate, up, down, 64, 8)
+    assert_close(out[toks], ref, f"config5 T={T} (GEMM)")
+    assert_close(out_stream[toks], ref, f"config5 T={T} (streaming)")
+    tol = model.tolerance(out_stream.astype(np.float64))
+    assert np.abs(out.astype(np.float64) - out_stream.astype(np.float64)).max() <= tol
