@@ -287,6 +287,7 @@ struct ExpertShapes {
   bool fused;
   bool portable;  // weights the streaming kernels do not take: the portable kernels run the block
   bool gemm;      // the grouped GEMM takes them too (batches with many rows per expert)
+  uint32_t bits;  // of the gate weight
 };
 
 // Average rows per expert from which the expert projections run on the grouped GEMM instead of the streaming
@@ -327,6 +328,7 @@ int32_t check_expert_weights(const char* who, const rmlx_qweight* gate, const rm
   }
   if (up != nullptr && up->group_size != gate->group_size) fast = false;
   sh->fused = fused;
+  sh->bits = gate->bits;
   sh->portable = !fast;
   // the grouped GEMM also takes group sizes the streaming kernels do not (32; 128 at 8 bits)
   sh->gemm = uniform && qmm_rw_grouped_supported(sh->I, sh->D, gate->group_size, gate->bits) &&
@@ -337,7 +339,10 @@ int32_t check_expert_weights(const char* who, const rmlx_qweight* gate, const rm
 // Rows per tile when `rows` positions over at most `groups` experts are multiplied by the grouped GEMM (half
 // tiles while an expert has 24 rows or fewer on average: less padding, more workgroups per CU), else 0
 uint32_t expert_gemm_tile_rows(const ExpertShapes& sh, uint64_t rows, uint64_t groups) {
-  const uint32_t min_rows = g_expert_gemm_min_rows.load(std::memory_order_relaxed);
+  uint32_t min_rows = g_expert_gemm_min_rows.load(std::memory_order_relaxed);
+  // 8-bit experts cross over at three eighths of the threshold (measured: 3 rows per expert against 8 for 4-bit
+  // ones; twice the bytes per row make the GEMV's second pass over an expert dearer)
+  if (sh.bits == 8 && min_rows != 0) min_rows = (3 * min_rows + 7) / 8;
   if (!sh.gemm || min_rows == 0 || groups == 0 || rows < (uint64_t)min_rows * groups) return 0;
   return rows <= 24 * groups ? 32u : kGroupedTileRows;
 }
