@@ -288,11 +288,12 @@ struct ExpertShapes {
   bool portable;  // weights the streaming kernels do not take: the portable kernels run the block
   bool gemm;      // the grouped GEMM takes them too (batches with many rows per expert)
   uint32_t bits;  // of the gate weight
+  bool gemm64;    // group size 64 (the 16-row tile is built for it only)
 };
 
 // Average rows per expert from which the expert projections run on the grouped GEMM instead of the streaming
 // GEMV (which re-reads an expert's weights once per 8 rows); 0 = never.  Measured crossover.
-std::atomic<uint32_t> g_expert_gemm_min_rows{8};
+std::atomic<uint32_t> g_expert_gemm_min_rows{6};
 
 int32_t check_expert_weights(const char* who, const rmlx_qweight* gate, const rmlx_qweight* up,
                              const rmlx_qweight* down, ExpertShapes* sh) {
@@ -329,6 +330,7 @@ int32_t check_expert_weights(const char* who, const rmlx_qweight* gate, const rm
   if (up != nullptr && up->group_size != gate->group_size) fast = false;
   sh->fused = fused;
   sh->bits = gate->bits;
+  sh->gemm64 = gate->group_size == 64;
   sh->portable = !fast;
   // the grouped GEMM also takes group sizes the streaming kernels do not (32; 128 at 8 bits)
   sh->gemm = uniform && qmm_rw_grouped_supported(sh->I, sh->D, gate->group_size, gate->bits) &&
@@ -340,10 +342,11 @@ int32_t check_expert_weights(const char* who, const rmlx_qweight* gate, const rm
 // tiles while an expert has 24 rows or fewer on average: less padding, more workgroups per CU), else 0
 uint32_t expert_gemm_tile_rows(const ExpertShapes& sh, uint64_t rows, uint64_t groups) {
   uint32_t min_rows = g_expert_gemm_min_rows.load(std::memory_order_relaxed);
-  // 8-bit experts cross over at three eighths of the threshold (measured: 3 rows per expert against 8 for 4-bit
-  // ones; twice the bytes per row make the GEMV's second pass over an expert dearer)
-  if (sh.bits == 8 && min_rows != 0) min_rows = (3 * min_rows + 7) / 8;
+  // 8-bit experts cross over at an eighth of the threshold (measured: from one row per expert on, against 6 for
+  // 4-bit ones: with 16-row tiles the GEMM streams 8-bit weights faster than the 8-bit GEMV does)
+  if (sh.bits == 8 && min_rows != 0) min_rows = (min_rows + 7) / 8;
   if (!sh.gemm || min_rows == 0 || groups == 0 || rows < (uint64_t)min_rows * groups) return 0;
+  if (rows <= 7 * groups && sh.gemm64) return 16u;  // (four-wave workgroups, 16 rows: built for group size 64)
   return rows <= 24 * groups ? 32u : kGroupedTileRows;
 }
 
@@ -828,9 +831,9 @@ int32_t rmlx_hip_gather_qmm(const rmlx_array* x, const void* w_packed_dev, size_
                     aligned16(bi) && aligned16(xk);
   const uint32_t gemm_min_rows = g_expert_gemm_min_rows.load(std::memory_order_relaxed);
   // Every entry has exactly m_per_batch rows, so the streaming GEMV wastes nothing up to a full chunk of 8 rows
-  // and the crossover lies higher than for routed batches: one and a half times the threshold (measured: 8 rows
+  // and the crossover lies higher than for routed batches: twice the threshold (measured: 8 rows
   // per entry 50 us streamed, 64 us on the GEMM; 64 rows 91 us on the GEMM).
-  if (gemm_min_rows != 0 && m_per_batch >= gemm_min_rows + gemm_min_rows / 2 && aligned16(w) && aligned16(sc) &&
+  if (gemm_min_rows != 0 && m_per_batch >= 2 * gemm_min_rows && aligned16(w) && aligned16(sc) &&
       aligned16(bi) && aligned16(xk) && qmm_rw_grouped_supported(N32, K32, group_size, 4)) {
     // many rows per entry: row tiles of one expert each on the grouped MFMA GEMM
     const uint32_t tile_rows = m_per_batch <= 32 ? 32u : kGroupedTileRows;

@@ -677,18 +677,20 @@ int32_t launch_qmm_rw_grouped(const GroupedQmmArgs& a, hipStream_t s) {
   p.tiles_m = (a.max_tiles + 7) / 8 * 8;  // (the grid covers eight equal runs of row tiles, one per XCD)
   // row tiles of 16 * 4 = kGroupedTileRows rows, 8 waves; a pair: 128 columns of each weight per workgroup,
   // one weight: 256 columns when they divide, else 128
-  const bool wide = !dual && a.N % 256 == 0;
-  p.tiles_n = a.N / (wide ? 256 : 128);
+  const uint32_t nw = a.tile_rows == 16 ? 4 : 8;
+  const bool wide = !dual && a.N % (nw * 32) == 0;
+  p.tiles_n = a.N / (wide ? nw * 32 : nw * 16);
   if ((uint64_t)p.tiles_m * p.tiles_n > 0x7FFFFFFFull) return fail(RMLX_INVALID_SHAPE, "grouped qmm: grid too large");
-  if (a.tile_rows != 32 && a.tile_rows != kGroupedTileRows)
+  if (a.tile_rows != 16 && a.tile_rows != 32 && a.tile_rows != kGroupedTileRows)
     return fail(RMLX_RUNTIME_ERROR, "grouped qmm: row tiles of %u rows", a.tile_rows);
-  const dim3 grid(p.tiles_m * p.tiles_n), block(512);
-#define RWG_LAUNCH(MFV, BITSV, GSV)                                                                                \
-  if (dual) hipLaunchKernelGGL((qmm_rw_grouped_kernel<MFV, 2, BITSV, 8, true, GSV>), grid, block, 0, s, p);          \
-  else if (wide) hipLaunchKernelGGL((qmm_rw_grouped_kernel<MFV, 2, BITSV, 8, false, GSV>), grid, block, 0, s, p);    \
-  else hipLaunchKernelGGL((qmm_rw_grouped_kernel<MFV, 1, BITSV, 8, false, GSV>), grid, block, 0, s, p);
+  const dim3 grid(p.tiles_m * p.tiles_n), block(64 * nw);
+#define RWG_LAUNCH(MFV, NWV, BITSV, GSV)                                                                              \
+  if (dual) hipLaunchKernelGGL((qmm_rw_grouped_kernel<MFV, 2, BITSV, NWV, true, GSV>), grid, block, 0, s, p);          \
+  else if (wide) hipLaunchKernelGGL((qmm_rw_grouped_kernel<MFV, 2, BITSV, NWV, false, GSV>), grid, block, 0, s, p);    \
+  else hipLaunchKernelGGL((qmm_rw_grouped_kernel<MFV, 1, BITSV, NWV, false, GSV>), grid, block, 0, s, p);
 #define RWG_TILE(BITSV, GSV)                                     \
-  if (a.tile_rows == 32) { RWG_LAUNCH(2, BITSV, GSV) } else { RWG_LAUNCH(4, BITSV, GSV) }
+  if (a.tile_rows == 16) { if (GSV == 64) { RWG_LAUNCH(1, 4, BITSV, 64) } }  \
+  else if (a.tile_rows == 32) { RWG_LAUNCH(2, 8, BITSV, GSV) } else { RWG_LAUNCH(4, 8, BITSV, GSV) }
 #define RWG_BITS(GSV) \
   if (a.bits == 4) { RWG_TILE(4, GSV) } else { RWG_TILE(8, GSV) }
   if (a.group_size == 64) { RWG_BITS(64) } else if (a.group_size == 32) { RWG_BITS(32) } else { RWG_BITS(128) }

@@ -68,11 +68,11 @@ def test_qweight_validation_needs_no_gpu():
 
 
 def test_expert_gemm_threshold_is_plain_host_state():
-    """The GEMV / grouped-GEMM threshold of the expert projections: default 8 rows per expert, set returns the old value."""
+    """The GEMV / grouped-GEMM threshold of the expert projections: default 6 rows per expert, set returns the old value."""
     from rmlx_amd import ops
     prev = ops.set_expert_gemm_min_rows(5)
     try:
-        assert prev == 8
+        assert prev == 6
         assert ops.set_expert_gemm_min_rows(0) == 5
         assert ops.set_expert_gemm_min_rows(prev) == 0
     finally:

@@ -430,7 +430,7 @@ def test_moe_other_bit_widths_and_group_sizes(hip, bits, gs, D, I, fused):
                                                (8, 64, 1024, 512, False), (4, 32, 512, 1024, True), (4, 128, 1024, 512, False),
                                                (8, 32, 512, 512, False), (8, 128, 512, 512, True)])
 def test_moe_many_rows_per_expert_on_the_grouped_gemm(hip, bits, gs, D, I, fused, T):
-    """Batches with many rows per expert (here 75 or 25 on average; from 8 on) multiply with the grouped MFMA GEMM: row
+    """Batches with many rows per expert (here 75 or 25 on average; from 6 on) multiply with the grouped MFMA GEMM: row
     tiles of 64 rows of one expert (32 rows while the average is at most 32).  Skewed routing gives one expert
     three tiles, another a ragged one and one almost nothing.  Group sizes 32, 64 and 128.  Checked against the
     oracle, and the path below the threshold (streaming GEMV, or the portable kernels where it does not take the
@@ -461,7 +461,7 @@ def test_moe_many_rows_per_expert_on_the_grouped_gemm(hip, bits, gs, D, I, fused
     ref = model.moe_forward(x, idx, w, gate, up, down, gs, K, bits=bits)
     xd, idxd, wd = DeviceBuffer.from_numpy(x), DeviceBuffer.from_numpy(idx), DeviceBuffer.from_numpy(w)
     print(f"grouped gemm moe T={T} bits={bits} gs={gs} D={D} I={I} fused={fused} counts={counts.tolist()}", flush=True)
-    prev = ops.set_expert_gemm_min_rows(8)
+    prev = ops.set_expert_gemm_min_rows(6)
     try:
         out_gemm = ops.moe_forward_grouped(gh, uh, dh, xd, idxd, wd, K).numpy()
         assert_close(out_gemm, ref, "moe_forward_grouped (GEMM)")
@@ -587,3 +587,43 @@ def test_config5_moe_prefill_sizes(hip, config5, T):
     assert_close(out_stream[toks], ref, f"config5 T={T} (streaming)")
     tol = model.tolerance(out_stream.astype(np.float64))
     assert np.abs(out.astype(np.float64) - out_stream.astype(np.float64)).max() <= tol
+
+
+@pytest.mark.parametrize("bits,E,T,D,I,fused", [(4, 4, 13, 512, 512, True), (4, 4, 13, 1024, 1536, False), (8, 8, 12, 512, 512, True),
+                                                (8, 16, 9, 1024, 512, False), (8, 128, 64, 512, 1024, True)])
+def test_moe_few_rows_per_expert_on_16_row_tiles(hip, bits, E, T, D, I, fused):
+    """Between the GEMM threshold (6 rows per expert on average; 8-bit experts: 1) and 7 rows the grouped GEMM runs
+    16-row tiles in four-wave workgroups.  Against the oracle, with the streaming GEMV path beside it."""
+    from rmlx_amd import ops
+    from rmlx_amd.runtime import DeviceBuffer
+    rng = np.random.default_rng(bits * 7 + E + T + D)
+    K = 2
+    assert (6 if bits == 4 else 1) * E <= T * K <= 7 * E
+
+    def weight(n, k):
+        return make_weight(rng, n, k, bits, 64, lead=(E,))
+
+    if fused:
+        gu = weight(2 * I, D)
+        gate, up = tuple(a[:, :I] for a in gu), tuple(a[:, I:] for a in gu)
+        gh, uh = ops.QuantizedWeight.from_numpy(*gu, 64, bits), None
+    else:
+        gate, up = weight(I, D), weight(I, D)
+        gh, uh = ops.QuantizedWeight.from_numpy(*gate, 64, bits), ops.QuantizedWeight.from_numpy(*up, 64, bits)
+    down = weight(D, I)
+    dh = ops.QuantizedWeight.from_numpy(*down, 64, bits)
+    x = make_x(rng, T, D)
+    logits = rng.standard_normal((T, E)).astype(np.float32)
+    if E <= 16:
+        logits[:, 1] += 2.0  # one expert with more than 16 rows: two tiles
+    idx, w, counts, _ = model.topk_route(logits, K)
+    ref = model.moe_forward(x, idx, w, gate, up, down, 64, K, bits=bits)
+    xd, idxd, wd = DeviceBuffer.from_numpy(x), DeviceBuffer.from_numpy(idx), DeviceBuffer.from_numpy(w)
+    print(f"16-row tiles bits={bits} E={E} T={T} D={D} I={I} fused={fused} counts={counts.tolist()}", flush=True)
+    assert_close(ops.moe_forward_grouped(gh, uh, dh, xd, idxd, wd, K).numpy(), ref, "moe_forward_grouped (16-row tiles)")
+    assert_close(ops.moe_forward(gh, uh, dh, xd, DeviceBuffer.from_numpy(logits), K).numpy(), ref, "moe_forward (16-row tiles)")
+    prev = ops.set_expert_gemm_min_rows(0)
+    try:
+        assert_close(ops.moe_forward_grouped(gh, uh, dh, xd, idxd, wd, K).numpy(), ref, "moe_forward_grouped (streaming)")
+    finally:
+        ops.set_expert_gemm_min_rows(prev)
