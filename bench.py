@@ -28,7 +28,7 @@ MFMA_F16_PEAK_TF = 2500.0  # dense f16 / bf16 MFMA
 # (FETCH_SIZE and WRITE_SIZE, each scaled by what it reads for the plain copy below); the runs and
 # the scaling are recorded in profiles/bench_all_configs_hbm_traffic_pmc.txt.  Counters cannot be
 # read from inside this process, so the figures are carried here and re-measured with the kernels.
-MEASURED_TRAFFIC_BYTES = {"qmv_q4_m1_4096": 9541116, "qmm_q4_m512_4096": 39722529}
+MEASURED_TRAFFIC_BYTES = {"qmv_q4_m1_4096": 9541139, "qmm_q4_m512_4096": 39722504}
 
 
 def matmul_bytes(m, n, k, bits, gs=64, act_bytes=2):
