@@ -260,7 +260,7 @@ int32_t rmlx_hip_moe_forward_grouped(const rmlx_qweight* gate, const rmlx_qweigh
  * with the grouped MFMA GEMM -- row tiles of 16, 32 or 64 rows of one expert, weights dequantised in registers;
  * 4- / 8-bit, group sizes 32 / 64 / 128 (one for the three projections), hidden and intermediate dimensions
  * in multiples of 512 -- smaller ones with the streaming GEMV, which reads an expert's weights once per 8
- * rows (8-bit experts switch at an eighth of `min_rows`, rounded up).  gather_qmm does the same from twice as many rows per batch entry on (4-bit, group
+ * rows (8-bit experts switch at an eighth of `min_rows`, rounded up).  gather_qmm does the same from one and a half times as many rows per batch entry on (4-bit, group
  * sizes 32 / 64 / 128, N % 128 == 0, K % 512 == 0).  0 = never the GEMM.  The default (6) is the measured
  * crossover; the setting is process-wide.  No counterpart in the reference, whose MoE layer picks its
  * kernels by a configured `MoeStrategy` (crates/rmlx-nn/src/moe.rs:515-541).  Returns the previous value. */

@@ -831,12 +831,13 @@ int32_t rmlx_hip_gather_qmm(const rmlx_array* x, const void* w_packed_dev, size_
                     aligned16(bi) && aligned16(xk);
   const uint32_t gemm_min_rows = g_expert_gemm_min_rows.load(std::memory_order_relaxed);
   // Every entry has exactly m_per_batch rows, so the streaming GEMV wastes nothing up to a full chunk of 8 rows
-  // and the crossover lies higher than for routed batches: twice the threshold (measured: 8 rows
-  // per entry 50 us streamed, 64 us on the GEMM; 64 rows 91 us on the GEMM).
-  if (gemm_min_rows != 0 && m_per_batch >= 2 * gemm_min_rows && aligned16(w) && aligned16(sc) &&
+  // and the crossover lies higher than for routed batches: one and a half times the threshold, i.e. from 9 rows
+  // on, where the GEMV needs a second pass (measured, 32 entries over 3072 x 4096 weights: 8 rows 50 us streamed;
+  // 12 / 16 / 32 rows 61 / 64 / 76 us on the GEMM with 16- / 32-row tiles against 95 / 99 / 172 us streamed).
+  if (gemm_min_rows != 0 && m_per_batch >= gemm_min_rows + gemm_min_rows / 2 && aligned16(w) && aligned16(sc) &&
       aligned16(bi) && aligned16(xk) && qmm_rw_grouped_supported(N32, K32, group_size, 4)) {
     // many rows per entry: row tiles of one expert each on the grouped MFMA GEMM
-    const uint32_t tile_rows = m_per_batch <= 32 ? 32u : kGroupedTileRows;
+    const uint32_t tile_rows = m_per_batch <= 16 && group_size == 64 ? 16u : (m_per_batch <= 32 ? 32u : kGroupedTileRows);
     const uint32_t per = ((uint32_t)m_per_batch + tile_rows - 1) / tile_rows;
     const uint64_t n_tiles = (uint64_t)B32 * per;
     if (n_tiles > 0x7FFFFFu) return fail(RMLX_INVALID_SHAPE, "gather_qmm: too many row tiles (%" PRIu64 ")", n_tiles);

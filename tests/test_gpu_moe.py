@@ -235,11 +235,11 @@ def test_gather_qmm_async_out_of_range_rows_are_zero(hip):
     assert np.all(out[~good] == 0)
 
 
-@pytest.mark.parametrize("n,k,mpb,gs", [(128, 512, 12, 64), (384, 1024, 70, 64), (256, 512, 64, 64), (128, 1536, 129, 64),
+@pytest.mark.parametrize("n,k,mpb,gs", [(128, 512, 9, 64), (128, 512, 12, 64), (256, 1024, 17, 64), (384, 1024, 70, 64), (256, 512, 64, 64), (128, 1536, 129, 64),
                                         (128, 512, 40, 32), (256, 1024, 70, 128)])
 def test_gather_qmm_many_rows_per_entry_on_the_grouped_gemm(hip, n, k, mpb, gs):
-    """From 12 rows per batch entry on, gather_qmm multiplies with the grouped MFMA GEMM (row tiles of 64 rows of one
-    expert; the last tile of an entry ragged).  Against the oracle; on a stream, rows of an out-of-range index are zero."""
+    """From 9 rows per batch entry on, gather_qmm multiplies with the grouped MFMA GEMM (row tiles of 16, 32 or 64 rows
+    of one expert; the last tile of an entry ragged).  Against the oracle; on a stream, rows of an out-of-range index are zero."""
     from rmlx_amd import ops
     from rmlx_amd.runtime import DeviceBuffer, Stream
     rng = np.random.default_rng(n + k + mpb)
