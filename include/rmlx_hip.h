@@ -83,7 +83,13 @@ int32_t rmlx_hip_memcpy_d2h(void* dst_host, const void* src_dev, size_t bytes, r
 int32_t rmlx_hip_memcpy_d2d(void* dst_dev, const void* src_dev, size_t bytes, rmlx_stream stream);
 int32_t rmlx_hip_stream_create(rmlx_stream* out);
 int32_t rmlx_hip_stream_sync(rmlx_stream stream);
+/* Synchronises the stream, hands its idle scratch blocks back to the driver and destroys it. */
 int32_t rmlx_hip_stream_destroy(rmlx_stream stream);
+/* The library keeps the scratch blocks of a stream (dtype casts, split-K partial sums, MoE intermediates) for
+ * the next call on that stream, so steady-state calls do not allocate.  This synchronises the stream (NULL = the
+ * default stream of synchronous calls) and frees its idle blocks, e.g. after one unusually large batch.  The
+ * counterpart of the reference's thread-local array pool going out of scope (crates/rmlx-core/src/array.rs:33-47). */
+int32_t rmlx_hip_trim_pool(rmlx_stream stream);
 int32_t rmlx_hip_event_create(rmlx_event* out);
 int32_t rmlx_hip_event_record(rmlx_event ev, rmlx_stream stream);
 int32_t rmlx_hip_event_sync(rmlx_event ev);

@@ -128,17 +128,55 @@ def tolerance(ref):
 # --------------------------------------------------------------------------------------
 
 
-def topk_route(logits, top_k, bias=None, renormalize=True, rank_by="logit"):
+def exp_neg_exact(x):
+    """exp(x) for x <= 0 as a fixed sequence of f32 multiplies and adds, each rounded once: Cody-Waite reduction
+    x = n ln2 + r, the degree-5 polynomial of Cephes' expf for (e^r - 1 - r) / r^2, scaling by 2^n; arguments
+    below -80 give 0.  The reference evaluates Metal's `fast::exp` here (topk_route.rs:256-257, 294), whose bits
+    no other machine reproduces; this routine is a definition both the library's routing kernel and this model
+    follow operation by operation, so they see the same ties.  Pinned in tests/ against float64 `exp` (a few
+    ulp) and by exact powers of two at multiples of ln 2 being monotone."""
+    x = np.asarray(x, dtype=np.float32)
+    f = np.float32
+    with np.errstate(invalid="ignore", over="ignore"):
+        n = np.rint(x * f(1.44269504))
+        r = x - n * f(0.693359375)
+        r = r - n * f(-2.12194440e-4)
+        p = np.full(x.shape, f(1.9875691500e-4), np.float32)
+        for c in (1.3981999507e-3, 8.3334519073e-3, 4.1665795894e-2, 1.6666665459e-1, 5.0000001201e-1):
+            p = p * r + f(c)
+        p = p * (r * r)
+        p = p + r
+        p = p + f(1.0)
+        ni = np.where(np.isfinite(n) & (n >= -126), n, 0).astype(np.int64)
+        two_n = ((ni + 127).astype(np.uint32) << np.uint32(23)).view(np.float32)
+        out = (p * two_n).astype(np.float32)
+    return np.where(x < f(-80.0), f(0.0), out).astype(np.float32)
+
+
+def _pairwise_sum_f32(v):
+    """Balanced pairwise tree over a power-of-two number of f32 values: ((v0+v1)+(v2+v3))+..."""
+    v = np.asarray(v, dtype=np.float32)
+    while v.size > 1:
+        v = (v[0::2] + v[1::2]).astype(np.float32)
+    return np.float32(v[0])
+
+
+def topk_route(logits, top_k, bias=None, renormalize=True, rank_by="softmax"):
     """softmax over E -> top-k by repeated argmax (strict >, ties -> lowest index) ->
     weights / sum(top-k) -> histogram -> exclusive scan.
 
     Restates `moe_topk_route_f32` + `moe_prefix_scan_u32`
     (crates/rmlx-core/src/ops/topk_route.rs:212-388).  Softmax is evaluated in f32 like the
-    kernel (max-subtracted, multiplied by 1/sum).  `rank_by="softmax"` ranks the f32 softmax
-    values as the kernel does; `rank_by="logit"` ranks the (biased) logits, which is the same
-    order unless two distinct logits collapse to one float after exp.
-    Pinned by the reference's behavioural tests (:674-751, :764-783, :815-840) and by a
-    brute-force stable argsort in tests/.
+    kernel: `exp(l - max) * (1 / sum)` (:294), the experts ranked by that f32 value with strict `>`
+    over ascending index and selected ones skipped (:283-300), so equal values -- an underflowing
+    tail, two logits that collapse after exp -- go to the lower index.  `exp` is `exp_neg_exact`;
+    the sum adds experts j, j+64, j+128, j+192 in that order for j = 0..63 and then the 64 partial
+    sums as a balanced pairwise tree (the reference's order is its threadgroup reduction, which
+    its tests do not pin).  `rank_by="logit"` ranks the (biased) logits instead: the same order
+    wherever the softmax values are distinct.
+    Pinned in tests/ by the reference's behavioural tests (:674-751, :764-783, :815-840), a
+    brute-force stable argsort, hand-written picks on underflowing rows, and the weights against
+    float64 softmax closed forms (renormalised top-k weights = softmax over the selected logits).
     Returns (indices u32 [T*K], weights f32 [T*K], counts u32 [E], offsets u32 [E+1]).
     """
     lg = np.asarray(logits, dtype=np.float32)
@@ -150,8 +188,13 @@ def topk_route(logits, top_k, bias=None, renormalize=True, rank_by="logit"):
     for t in range(T):
         row = lg[t]
         mx = np.float32(row.max()) if E else np.float32(0)
-        ex = np.exp((row - mx).astype(np.float32)).astype(np.float32)
-        inv = np.float32(1.0) / np.float32(ex.sum(dtype=np.float32))
+        ex = exp_neg_exact((row - mx).astype(np.float32))
+        lanes = np.zeros((4, 64), np.float32)
+        lanes.reshape(-1)[:E] = ex
+        part = np.zeros(64, np.float32)
+        for j in range(4):
+            part = (part + lanes[j]).astype(np.float32)
+        inv = np.float32(1.0) / _pairwise_sum_f32(part)
         sm = (ex * inv).astype(np.float32)
         key = sm if rank_by == "softmax" else row
         taken = np.zeros(E, bool)
@@ -208,6 +251,45 @@ def silu(x):
     return x / (1.0 + np.exp(-x))
 
 
+def scatter_weighted_add(src, tok_indices, weights, num_tokens):
+    """out[tok_indices[a], :] += weights[a] * src[a, :] over the assignments a in ascending order, out zero-initialised
+    (`scatter_weighted_add`, crates/rmlx-core/src/ops/moe_kernels.rs:306-363; the reference accumulates in the
+    array dtype, this model in float64).  Pinned by the reference's known answer (:420-450)."""
+    src = np.asarray(src, dtype=np.float64)
+    out = np.zeros((num_tokens, src.shape[1]), np.float64)
+    for a in range(src.shape[0]):
+        out[int(tok_indices[a])] += float(weights[a]) * src[a]
+    return out
+
+
+def combine_cpu(expert_outputs, weights, indices, batch_size, top_k, hidden_dim):
+    """out[t, :] = sum_k weights[t*K+k] * expert_outputs[indices[t*K+k]][t, :] with out-of-range experts skipped
+    (`MoeCombineExchange::combine_cpu`, crates/rmlx-distributed/src/moe_exchange.rs:2288-2320).  Pinned by the
+    reference's known answers (crates/rmlx-distributed/tests/moe_tests.rs:115-135, 660-687)."""
+    out = np.zeros((batch_size, hidden_dim), np.float64)
+    for t in range(batch_size):
+        for k in range(top_k):
+            flat = t * top_k + k
+            e = int(indices[flat])
+            if e < len(expert_outputs):
+                eo = np.asarray(expert_outputs[e], dtype=np.float64).reshape(-1)
+                if (t + 1) * hidden_dim <= eo.size:
+                    out[t] += float(weights[flat]) * eo[t * hidden_dim:(t + 1) * hidden_dim]
+    return out
+
+
+def expert_ffn(x, gate_w, up_w, down_w, round_h=np.float16):
+    """y = (silu(x Wg^T) * (x Wu^T)) Wd^T for dequantised [out, in] weight matrices: `Expert::forward`
+    (crates/rmlx-nn/src/moe.rs:188-200) / the per-expert body of `ExpertGroup::grouped_forward`
+    (crates/rmlx-nn/src/expert_group.rs:445-524).  The hidden activation is rounded to `round_h` (the reference
+    stores it in the input dtype, expert_group.rs:380-383); everything else is float64."""
+    x = np.asarray(x, dtype=np.float64)
+    h = silu(x @ gate_w.T) * (x @ up_w.T)
+    if round_h is not None:
+        h = h.astype(round_h).astype(np.float64)
+    return h @ down_w.T
+
+
 def moe_forward(x, indices, weights, gate, up, down, group_size, top_k, round_h=np.float16, bits=4):
     """out[t] = sum_k w[t,k] * down_e( silu(gate_e x_t) * up_e x_t ), e = indices[t,k].
 
@@ -215,37 +297,30 @@ def moe_forward(x, indices, weights, gate, up, down, group_size, top_k, round_h=
     gate GEMM, up GEMM, silu_gate, down GEMM) and the weighted scatter-add
     (crates/rmlx-nn/src/moe.rs:1851-1932; `scatter_weighted_add`,
     crates/rmlx-core/src/ops/moe_kernels.rs:306-363), with expert weights in the stacked Q4
-    layout of `gather_qmv_fast_f16_q4` (quantized.rs:9605-9620).  The hidden activation is
-    rounded to `round_h` (the reference stores it in the input dtype, expert_group.rs:380-383);
-    everything else is float64.  `gate`, `up`, `down` are (words, scales, biases) triples with a
-    leading expert axis.  Pinned by the scatter known answer (moe_kernels.rs:420-450) and by
-    equality with a per-expert loop on small shapes in tests/.
+    layout of `gather_qmv_fast_f16_q4` (quantized.rs:9605-9620).  `gate`, `up`, `down` are
+    (words, scales, biases) triples with a leading expert axis.  Assignments are grouped by expert
+    in (token, k) order (`moe_sort`), every group runs `expert_ffn`, and the rows go back through
+    `scatter_weighted_add` with the token of each sorted position.
+    Pinned in tests/: the combine step by the reference's known answers for `scatter_weighted_add`
+    and `combine_cpu`; the whole function by a brute per-(token, k) loop that dequantises with the C
+    restatement of `dequantize_q4_row` and shares no code with this one, on small shapes with
+    top_k > 1 and repeated experts, and by one-hot / identity closed forms.
     """
     x = np.asarray(x, dtype=np.float64)
     T, D = x.shape
-    out = np.zeros((T, D), np.float64)
-    idx = np.asarray(indices).reshape(T, top_k)
-    wts = np.asarray(weights, dtype=np.float64).reshape(T, top_k)
-    cache = {}
-
-    def deq(trip, e):
-        key = (id(trip[0]), int(e))
-        if key not in cache:
-            cache[key] = dequantize(trip[0][e], trip[1][e], trip[2][e], group_size, bits)
-        return cache[key]
-
-    for e in np.unique(idx):
-        toks, ks = np.nonzero(idx == e)
-        xe = x[toks]
-        g = xe @ deq(gate, e).T
-        u = xe @ deq(up, e).T
-        h = silu(g) * u
-        if round_h is not None:
-            h = h.astype(round_h).astype(np.float64)
-        y = h @ deq(down, e).T
-        np.add.at(out, toks, wts[toks, ks][:, None] * y)
-        cache.clear()
-    return out
+    idx = np.asarray(indices).reshape(-1)
+    wts = np.asarray(weights, dtype=np.float64).reshape(-1)
+    E = gate[0].shape[0]
+    order, offsets = moe_sort(idx, E)
+    tok = order // top_k
+    y = np.zeros((order.size, D), np.float64)
+    for e in range(E):
+        lo, hi = int(offsets[e]), int(offsets[e + 1])
+        if lo == hi:
+            continue
+        wg, wu, wd = (dequantize(t[0][e], t[1][e], t[2][e], group_size, bits) for t in (gate, up, down))
+        y[lo:hi] = expert_ffn(x[tok[lo:hi]], wg, wu, wd, round_h)
+    return scatter_weighted_add(y, tok, wts[order], T)
 
 
 # --------------------------------------------------------------------------------------

@@ -104,6 +104,20 @@ void Scratch::release() {
   }
 }
 
+// Frees the idle scratch blocks of a stream (the caller has synchronised it); `forget` also drops its entry.
+int32_t trim_pool(hipStream_t s, bool forget) {
+  std::vector<Block> blocks;
+  {
+    std::lock_guard<std::mutex> lock(g_pool_mutex);
+    auto it = g_pool.find(s);
+    if (it == g_pool.end()) return RMLX_OK;
+    blocks.swap(it->second);
+    if (forget) g_pool.erase(it);
+  }
+  for (const Block& b : blocks) RMLX_HIP_CHECK(hipFree(b.ptr));
+  return RMLX_OK;
+}
+
 namespace {
 
 bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
@@ -526,8 +540,17 @@ int32_t rmlx_hip_stream_sync(rmlx_stream stream) {
   return RMLX_OK;
 }
 int32_t rmlx_hip_stream_destroy(rmlx_stream stream) {
+  // The stream's scratch blocks go back to the driver first: a later stream may get the same handle value and
+  // must not inherit blocks whose last kernels were ordered on this one.
+  RMLX_HIP_CHECK(hipStreamSynchronize((hipStream_t)stream));
+  RMLX_TRY(trim_pool((hipStream_t)stream, true));
   RMLX_HIP_CHECK(hipStreamDestroy((hipStream_t)stream));
   return RMLX_OK;
+}
+int32_t rmlx_hip_trim_pool(rmlx_stream stream) {
+  RMLX_TRY(require_init());
+  RMLX_HIP_CHECK(hipStreamSynchronize((hipStream_t)stream));
+  return trim_pool((hipStream_t)stream, false);
 }
 int32_t rmlx_hip_event_create(rmlx_event* out) {
   RMLX_TRY(require_init());

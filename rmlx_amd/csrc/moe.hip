@@ -72,10 +72,34 @@ __device__ __forceinline__ void wave_key_max(uint32_t& hi, uint32_t& lo) {
 }
 
 // ---- routing: one wave per token -----------------------------------------------------------
-// Each lane owns experts lane, lane+64, lane+128, lane+192 (E <= 256).  Ranking uses the biased
-// logit with ties broken towards the lower expert index, which is the order of the softmax
-// values the reference ranks (exp is monotonic), made independent of the exp implementation.
-// A round's winner is the wave maximum of the key (order-preserving bits of the logit, ~index).
+// exp(x) for x <= 0 from plain f32 multiplies and adds, each rounded once (no fused multiply-add, no
+// hardware transcendental): the same sequence of IEEE operations gives the same bits on any machine, so a
+// CPU restatement reproduces the softmax values -- and with them the ties the ranking sees -- exactly.
+// Cody-Waite reduction x = n ln2 + r, degree-5 polynomial for (e^r - 1 - r) / r^2, scale by 2^n.  Arguments
+// below -80 give 0, which keeps every softmax value (at least e^-80 / 256) a normal number.
+__device__ __forceinline__ float exp_neg_exact(float x) {
+#pragma clang fp contract(off)
+  if (x < -80.0f) return 0.0f;
+  const float n = __builtin_rintf(x * 1.44269504f);
+  float r = x - n * 0.693359375f;
+  r = r - n * -2.12194440e-4f;
+  float p = 1.9875691500e-4f;
+  p = p * r + 1.3981999507e-3f;
+  p = p * r + 8.3334519073e-3f;
+  p = p * r + 4.1665795894e-2f;
+  p = p * r + 1.6666665459e-1f;
+  p = p * r + 5.0000001201e-1f;
+  p = p * (r * r);
+  p = p + r;
+  p = p + 1.0f;
+  return p * __uint_as_float((uint32_t)((int)n + 127) << 23);
+}
+
+// Each lane owns experts lane, lane+64, lane+128, lane+192 (E <= 256).  Ranking follows the reference:
+// the f32 softmax value exp(l - max) * (1 / sum) with strict >, so equal values (two logits that collapse
+// after exp, an underflowing tail) go to the lower expert index (topk_route.rs:283-300).  A round's winner
+// is the wave maximum of the key (bits of the non-negative softmax value, ~index).  The sum runs over the
+// four values of a lane in ascending order and then over the lanes as a balanced pairwise tree.
 // (`lds_idx`: optional copy of the picks in workgroup memory, for a sort fused behind the routing)
 __device__ __forceinline__ void route_token(const float* __restrict__ logits, const float* __restrict__ bias,
                                             uint32_t E, uint32_t K, int renorm, uint32_t* __restrict__ out_idx,
@@ -100,7 +124,7 @@ __device__ __forceinline__ void route_token(const float* __restrict__ logits, co
   float sum = 0.f;
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
-    sm[j] = (lane + 64 * j < E) ? expf(v[j] - mx) : 0.f;
+    sm[j] = (lane + 64 * j < E) ? exp_neg_exact(v[j] - mx) : 0.f;
     sum += sm[j];
   }
   sum = wave_add(sum);
@@ -116,9 +140,9 @@ __device__ __forceinline__ void route_token(const float* __restrict__ logits, co
     uint32_t bi = 0xFFFFFFFFu;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {  // ascending expert index inside the lane: strict > keeps the lower one
-      if (!taken[j] && (bi == 0xFFFFFFFFu || v[j] > bv)) { bv = v[j]; bi = lane + 64 * j; }
+      if (!taken[j] && (bi == 0xFFFFFFFFu || sm[j] > bv)) { bv = sm[j]; bi = lane + 64 * j; }
     }
-    // key: logits compare like their order-preserving bit patterns (-0 counted as +0), then the lower index
+    // key: softmax values compare like their order-preserving bit patterns (-0 counted as +0), then the lower index
     uint32_t hi = 0, lo = 0;
     if (bi != 0xFFFFFFFFu) {
       const uint32_t u = __float_as_uint(bv + 0.0f);
@@ -270,6 +294,8 @@ __global__ __launch_bounds__(1024) void moe_sort_kernel(const uint32_t* __restri
       sorted[pos] = base + tid;
       if (sorted_tok != nullptr) sorted_tok[pos] = (base + tid) / top_k;
       if (inv != nullptr) inv[base + tid] = pos;
+    } else if (inv != nullptr && base + tid < n_assign) {
+      inv[base + tid] = 0xFFFFFFFFu;  // an expert id outside [0, E): the combine step skips the assignment
     }
     __syncthreads();
     // thread t owns column t of wcnt and cur[t]: cursor forward, column cleared for the next block
@@ -303,6 +329,7 @@ __device__ __forceinline__ void sort_small(uint32_t lane, uint32_t n, uint32_t e
     if (sorted_tok != nullptr) sorted_tok[pos] = lane / top_k;
     if (inv != nullptr) inv[lane] = pos;
   }
+  if (!valid && lane < n && inv != nullptr) inv[lane] = 0xFFFFFFFFu;  // skipped by the combine step
   // the first assignment of every expert writes the expert's chunks; chunks of lower experts come first
   const bool leader = valid && rank == 0;
   const uint32_t my_chunks = leader ? (same + 7) / 8 : 0u;
@@ -423,10 +450,12 @@ __global__ void identity_positions_kernel(uint32_t* __restrict__ tok, uint32_t* 
 
 // out[t,:] = sum_k w[t*K+k] * y[inv[t*K+k],:], k ascending, f32.  grid = (T, column blocks of 1024):
 // every thread owns four columns, loads its rows of all top_k experts first and sums in order.
+// Assignments whose position is not below n_rows (the grouping kernels mark an expert id outside
+// [0, E) that way) contribute nothing.
 __global__ __launch_bounds__(256) void moe_combine_kernel(const float* __restrict__ y,
                                                           const uint32_t* __restrict__ inv,
                                                           const float* __restrict__ weights, uint32_t top_k,
-                                                          uint32_t D, __half* __restrict__ out) {
+                                                          uint32_t D, uint32_t n_rows, __half* __restrict__ out) {
   const uint32_t t = blockIdx.x;
   const uint32_t c = (blockIdx.y * 256 + threadIdx.x) * 4;
   if (c >= D) return;
@@ -437,8 +466,11 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(const float* __restric
     w[k] = 0.f;
     v[k] = make_float4(0.f, 0.f, 0.f, 0.f);
     if (k < top_k) {
-      w[k] = weights[(size_t)t * top_k + k];
-      v[k] = *reinterpret_cast<const float4*>(y + (size_t)inv[(size_t)t * top_k + k] * D + c);
+      const uint32_t pos = inv[(size_t)t * top_k + k];
+      if (pos < n_rows) {
+        w[k] = weights[(size_t)t * top_k + k];
+        v[k] = *reinterpret_cast<const float4*>(y + (size_t)pos * D + c);
+      }
     }
   }
   float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
@@ -553,7 +585,7 @@ int32_t launch_moe_combine(const float* y, const uint32_t* inv, const float* wei
                            uint32_t D, __half* out, hipStream_t s) {
   if (T == 0) return RMLX_OK;
   if (top_k > 8 || D % 4 != 0) return fail(RMLX_INVALID_SHAPE, "moe_combine: top_k <= 8 and D %% 4 == 0 required (top_k=%u D=%u)", top_k, D);
-  hipLaunchKernelGGL(moe_combine_kernel, dim3(T, (D + 1023) / 1024), dim3(256), 0, s, y, inv, weights, top_k, D, out);
+  hipLaunchKernelGGL(moe_combine_kernel, dim3(T, (D + 1023) / 1024), dim3(256), 0, s, y, inv, weights, top_k, D, T * top_k, out);
   RMLX_HIP_CHECK(hipGetLastError());
   return RMLX_OK;
 }

@@ -34,7 +34,7 @@ class RmlxArray(ctypes.Structure):
 EXPORTS = [
     "rmlx_hip_last_error", "rmlx_hip_init", "rmlx_hip_device_info", "rmlx_hip_malloc", "rmlx_hip_free",
     "rmlx_hip_memset", "rmlx_hip_memcpy_h2d", "rmlx_hip_memcpy_d2h", "rmlx_hip_memcpy_d2d",
-    "rmlx_hip_stream_create", "rmlx_hip_stream_sync", "rmlx_hip_stream_destroy", "rmlx_hip_event_create",
+    "rmlx_hip_stream_create", "rmlx_hip_stream_sync", "rmlx_hip_stream_destroy", "rmlx_hip_trim_pool", "rmlx_hip_event_create",
     "rmlx_hip_event_record", "rmlx_hip_event_sync", "rmlx_hip_event_elapsed_ms", "rmlx_hip_event_destroy",
     "rmlx_hip_qweight_create", "rmlx_hip_qweight_destroy", "rmlx_hip_affine_quantized_matmul",
     "rmlx_hip_affine_quantized_matmul_batched", "rmlx_hip_qmm_select", "rmlx_hip_qmm_add_residual", "rmlx_hip_qmm_swiglu", "rmlx_hip_qmm_encode_many", "rmlx_hip_quantized_linear_forward",
@@ -72,6 +72,7 @@ def lib():
         "rmlx_hip_stream_create": [ctypes.POINTER(vp)],
         "rmlx_hip_stream_sync": [vp],
         "rmlx_hip_stream_destroy": [vp],
+        "rmlx_hip_trim_pool": [vp],
         "rmlx_hip_event_create": [ctypes.POINTER(vp)],
         "rmlx_hip_event_record": [vp, vp],
         "rmlx_hip_event_sync": [vp],

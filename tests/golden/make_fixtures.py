@@ -13,7 +13,7 @@ so that every later change of the oracle or of the HIP kernels is checked agains
       out_tiled f32 [M,N]   (`affine_qmm` / `affine_qmm_q8` loop nest, quantized.rs:2649-2836)
       out_naive f32 [M,N]   (`naive_matmul_with_dequant`, :10678-10719)
       out_f64  f64 [M,N]    (float64 matmul of the f32-dequantized weights)
-  route_T<T>_E<E>_K<K>_seed<S>.npz
+  route_T<T>_E<E>_K<K>_seed<S>[_wide].npz
       logits f32 [T,E]; expert_indices u32 [T*K]; expert_weights f32 [T*K]; expert_counts u32 [E];
       dispatch_offsets u32 [E+1]; sorted_assignments u32 [T*K]   (topk_route.rs:212-388, moe.rs:1439-1447)
 
@@ -42,7 +42,9 @@ LCG_CASES = [
     (32, 8, 64, 32, 7),                                               # :10933-10998, 11802-11866
     (16, 64, 512, 64, 42),                                            # kernel-sized twin (qmv / qmm shapes)
 ]
-ROUTE_CASES = [(4, 8, 2, 11), (32, 128, 8, 12), (7, 200, 3, 13)]
+# (T, E, K, seed, logit scale); the last case is so wide that most of a row underflows after exp: its picks past the
+# first few are ties at 0.0 that go to the lowest free index
+ROUTE_CASES = [(4, 8, 2, 11, 4.0), (32, 128, 8, 12, 4.0), (7, 200, 3, 13, 4.0), (8, 16, 8, 14, 400.0)]
 # (format, rows, cols, group_size, seed, with g_idx)
 DEQUANT_CASES = [("awq", 16, 24, 4, 21, False), ("awq", 64, 128, 32, 24, False), ("gptq", 32, 16, 8, 22, False),
                  ("gptq", 32, 16, 8, 23, True), ("gptq", 128, 64, 32, 25, True)]
@@ -62,9 +64,9 @@ def lcg_case(m, n, k, gs, seed, bits):
     )
 
 
-def route_case(t, e, k, seed):
+def route_case(t, e, k, seed, scale):
     g = refpath.Lcg(seed)
-    logits = (4.0 * g.fill(t * e)).reshape(t, e).astype(np.float32)
+    logits = (scale * g.fill(t * e)).reshape(t, e).astype(np.float32)
     idx, w, counts, offsets = model.topk_route(logits, k)
     sorted_assign, _ = model.moe_sort(idx, e)
     return dict(logits=logits, expert_indices=idx, expert_weights=w.astype(np.float32), expert_counts=counts,
@@ -98,8 +100,9 @@ def main():
         for bits in (4, 8):
             np.savez_compressed(os.path.join(HERE, f"lcg_{m}x{n}x{k}_gs{gs}_q{bits}_seed{seed}.npz"),
                                 **lcg_case(m, n, k, gs, seed, bits))
-    for (t, e, k, seed) in ROUTE_CASES:
-        np.savez_compressed(os.path.join(HERE, f"route_T{t}_E{e}_K{k}_seed{seed}.npz"), **route_case(t, e, k, seed))
+    for (t, e, k, seed, scale) in ROUTE_CASES:
+        name = f"route_T{t}_E{e}_K{k}_seed{seed}{'_wide' if scale > 100 else ''}.npz"
+        np.savez_compressed(os.path.join(HERE, name), **route_case(t, e, k, seed, scale))
     print("wrote", len([f for f in os.listdir(HERE) if f.endswith(".npz")]), "fixtures")
 
 

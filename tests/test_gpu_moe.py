@@ -74,14 +74,13 @@ def test_topk_route_matches_oracle(hip, T, E, K):
     ridx, rw, rcounts, roff = model.topk_route(logits, K)
     assert np.array_equal(idx, ridx)
     assert np.array_equal(counts, rcounts) and np.array_equal(off, roff)
-    assert np.allclose(w, rw, rtol=1e-5, atol=1e-6)
-    # ranking by the f32 softmax value (what the reference kernel compares) gives the same picks here
-    sidx, _, _, _ = model.topk_route(logits, K, rank_by="softmax")
-    assert np.array_equal(idx, sidx)
-    # brute force: stable argsort of -logit
-    brute = np.argsort(-logits, axis=1, kind="stable")[:, :K].reshape(-1)
-    assert np.array_equal(idx, brute.astype(np.uint32))
-    assert np.allclose(w.reshape(T, K).sum(1), 1.0, atol=1e-5)
+    assert np.array_equal(w, rw)  # kernel and oracle evaluate the softmax with the same sequence of f32 operations
+    # brute force: stable argsort of the float64 softmax; weights: float64 softmax over the picked logits
+    e64 = np.exp(logits.astype(np.float64) - logits.max(axis=1, keepdims=True))
+    brute = np.argsort(-e64, axis=1, kind="stable")[:, :K]
+    assert np.array_equal(idx, brute.reshape(-1).astype(np.uint32))
+    sel = np.take_along_axis(e64, brute, axis=1)
+    assert np.allclose(w.reshape(T, K), sel / sel.sum(axis=1, keepdims=True), rtol=0, atol=1e-6)
 
 
 def test_topk_route_ties_go_to_lower_index(hip):
@@ -93,6 +92,35 @@ def test_topk_route_ties_go_to_lower_index(hip):
     assert list(idx[4:8]) == [5, 70, 129, 0]
     assert list(idx[8:]) == [0, 1, 2, 3]
     assert np.allclose(w[:4], 0.25)
+
+
+def test_topk_route_ranks_softmax_values(hip):
+    """The reference ranks the f32 softmax value with strict > (topk_route.rs:283-300): logits whose softmax value
+    underflows tie at 0.0 and go to the lowest free index, whatever their own order.  Expected picks written by hand."""
+    logits = np.array([
+        [0, -200, -150, -160, -170, -300, -120, -110],   # after expert 0 everything is 0.0 -> 1, 2
+        [-500, -400, -300, -200, -100, 0, -450, -350],   # 5, then 0, 1
+        [1, 1, 1, 1, 1, 1, 1, 1],                        # all equal -> 0, 1, 2
+        [-100, -100, -100, 7, -100, -100, 7, -100],      # exact tie at the top, then an underflowing tail -> 3, 6, 0
+    ], np.float32)
+    want = np.array([[0, 1, 2], [5, 0, 1], [0, 1, 2], [3, 6, 0]], np.uint32)
+    idx, w, counts, _ = _route(hip, logits, 3)
+    assert np.array_equal(idx.reshape(4, 3), want)
+    assert np.allclose(w.reshape(4, 3), [[1, 0, 0], [1, 0, 0], [1 / 3] * 3, [0.5, 0.5, 0]], atol=1e-6)
+    assert np.array_equal(counts, np.bincount(want.reshape(-1), minlength=8))
+    ridx, rw, _, _ = model.topk_route(logits, 3)
+    assert np.array_equal(idx, ridx) and np.array_equal(w, rw)
+    for r in range(4):  # the same rows reached through a wide expert_bias on all-zero logits
+        idx_b, w_b, _, _ = _route(hip, np.zeros((1, 8), np.float32), 3, bias=logits[r])
+        assert np.array_equal(idx_b, want[r]) and np.array_equal(w_b, w.reshape(4, 3)[r])
+    # a wide row over all four expert slots of a lane (E = 256), ties far apart in index
+    wide = np.full((2, 256), -300.0, np.float32)
+    wide[0, [200, 13]] = [5.0, 4.0]
+    wide[0, 100] = -250.0  # larger logit than the rest of the tail, same softmax value: must not be preferred
+    wide[1, 255] = 0.0
+    idx, _, _, _ = _route(hip, wide, 5)
+    assert list(idx[:5]) == [200, 13, 0, 1, 2] and list(idx[5:]) == [255, 0, 1, 2, 3]
+    assert np.array_equal(idx, model.topk_route(wide, 5)[0])
 
 
 @pytest.mark.parametrize("A,E", [(32, 128), (256, 128), (1024, 128), (2500, 7), (1, 4), (4096, 256), (16384, 128), (20011, 1000), (3000, 1)])
@@ -284,6 +312,30 @@ def _experts(rng, E, D, I, fused):
     down = make_weight(rng, D, I, 4, lead=(E,))
     down_h = ops.QuantizedWeight.from_numpy(*down, 64, 4)
     return gate, up, down, gate_h, up_h, down_h
+
+
+@pytest.mark.parametrize("T,E,K,D,I", [(6, 8, 4, 512, 512), (20, 32, 4, 512, 512), (100, 4, 2, 512, 512), (12, 6, 2, 256, 384)])
+def test_moe_forward_grouped_skips_out_of_range_experts(hip, T, E, K, D, I):
+    """Caller-supplied expert ids outside [0, E) contribute nothing (the reference's combine skips them,
+    crates/rmlx-distributed/src/moe_exchange.rs:2305): one-wave grouping (<= 64 assignments), the workgroup-wide
+    grouping below and above the grouped-GEMM threshold, and the portable kernels (D, I no multiples of 512)."""
+    from rmlx_amd import ops
+    from rmlx_amd.runtime import DeviceBuffer
+    rng = np.random.default_rng(T + E + K + D)
+    gate, up, down, gh, uh, dh = _experts(rng, E, D, I, False)
+    x = make_x(rng, T, D)
+    idx = np.stack([rng.permutation(E)[:K] for _ in range(T)]).astype(np.uint32).reshape(-1)
+    w = rng.uniform(0.1, 1.0, T * K).astype(np.float32)
+    bad = rng.choice(T * K, size=max(2, T * K // 7), replace=False)
+    idx_bad = idx.copy()
+    idx_bad[bad] = np.where(np.arange(bad.size) % 2 == 0, E, 0xFFFFFFFF).astype(np.uint32)
+    w_ref = w.copy()
+    w_ref[bad] = 0.0
+    ref = model.moe_forward(x, idx, w_ref, gate, up, down, 64, K)
+    print(f"out-of-range experts T={T} E={E} K={K} D={D} I={I} bad={sorted(bad.tolist())}", flush=True)
+    out = ops.moe_forward_grouped(gh, uh, dh, DeviceBuffer.from_numpy(x), DeviceBuffer.from_numpy(idx_bad),
+                                  DeviceBuffer.from_numpy(w), K).numpy()
+    assert_close(out, ref, "out-of-range experts skipped")
 
 
 @pytest.mark.parametrize("T,E,K", [(1, 128, 8), (8, 128, 8), (7, 200, 3), (8, 256, 8), (3, 5, 5), (9, 128, 7)])
@@ -552,19 +604,20 @@ def test_config5_moe(hip, config5, T):
     logits = rng.standard_normal((T, 128)).astype(np.float32)
     out = ops.moe_forward(gh, uh, dh, DeviceBuffer.from_numpy(x), DeviceBuffer.from_numpy(logits), 8).numpy()
     idx, w, _, _ = model.topk_route(logits, 8)
-    # the oracle is evaluated on a sample of tokens (all of them for T <= 4): each token needs 8 experts dequantized
-    toks = np.arange(T) if T <= 4 else np.sort(rng.choice(T, size=6, replace=False))
-    sel = (toks[:, None] * 8 + np.arange(8)[None, :]).reshape(-1)
-    ref = model.moe_forward(x[toks], idx[sel], w[sel], gate, up, down, 64, 8)
-    assert_close(out[toks], ref, f"config5 T={T}")
-    assert np.all(np.isfinite(out.astype(np.float32)))
+    ref = model.moe_forward(x, idx, w, gate, up, down, 64, 8)  # every token (the model dequantises one expert at a time)
+    assert_close(out, ref, f"config5 T={T}")
+    # the two-step path on the same inputs: routing on the device, then the block on its outputs
+    r = ops.gpu_topk_route(DeviceBuffer.from_numpy(logits), 8)
+    assert np.array_equal(r.expert_indices.numpy(), idx) and np.array_equal(r.expert_weights.numpy(), w)
+    out2 = ops.moe_forward_grouped(gh, uh, dh, DeviceBuffer.from_numpy(x), r.expert_indices, r.expert_weights, 8).numpy()
+    assert_close(out2, ref, f"config5 T={T} (two-step)")
 
 
 @pytest.mark.parametrize("T", [300, 700])
 def test_config5_moe_prefill_sizes(hip, config5, T):
     """Config 5 at prefill-sized batches (19 / 44 rows per expert on average: the grouped GEMM with 32- / 64-row tiles).
-    The oracle checks a sample of tokens; every token is checked against the streaming GEMV path (threshold 0) on the
-    same inputs, which shares no matrix kernel with the GEMM path."""
+    The oracle checks every token, of the GEMM path and of the streaming GEMV path (threshold 0) on the same inputs,
+    which shares no matrix kernel with the GEMM path."""
     from rmlx_amd import ops
     from rmlx_amd.runtime import DeviceBuffer
     gate, up, down, gh, uh, dh = config5
@@ -580,13 +633,9 @@ def test_config5_moe_prefill_sizes(hip, config5, T):
         out_stream = ops.moe_forward_grouped(gh, uh, dh, xd, idxd, wd, 8).numpy()
     finally:
         ops.set_expert_gemm_min_rows(prev)
-    toks = np.sort(rng.choice(T, size=6, replace=False))
-    sel = (toks[:, None] * 8 + np.arange(8)[None, :]).reshape(-1)
-    ref = model.moe_forward(x[toks], idx[sel], w[sel], gate, up, down, 64, 8)
-    assert_close(out[toks], ref, f"config5 T={T} (GEMM)")
-    assert_close(out_stream[toks], ref, f"config5 T={T} (streaming)")
-    tol = model.tolerance(out_stream.astype(np.float64))
-    assert np.abs(out.astype(np.float64) - out_stream.astype(np.float64)).max() <= tol
+    ref = model.moe_forward(x, idx, w, gate, up, down, 64, 8)
+    assert_close(out, ref, f"config5 T={T} (GEMM)")
+    assert_close(out_stream, ref, f"config5 T={T} (streaming)")
 
 
 @pytest.mark.parametrize("bits,E,T,D,I,fused", [(4, 4, 13, 512, 512, True), (4, 4, 13, 1024, 1536, False), (8, 8, 12, 512, 512, True),
