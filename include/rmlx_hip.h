@@ -279,6 +279,22 @@ int32_t rmlx_hip_moe_forward(const rmlx_qweight* gate, const rmlx_qweight* up,
                              const rmlx_array* expert_bias, void* out_f16_dev, size_t out_bytes,
                              rmlx_stream stream);
 
+/* rmlx_hip_moe_forward for callers that cannot allocate: code under HIP graph capture, tight serving loops and
+ * harnesses that forbid hipMalloc.  No counterpart in the reference.  Same arguments, same kernels and the same
+ * result as rmlx_hip_moe_forward, but every intermediate (routing output, grouping tables, hidden activations,
+ * per-assignment expert outputs, dtype casts) is carved from a workspace of 8 MiB that is part of the library's
+ * device code (one copy per GPU, held until the process ends; rmlx_hip_init resolves its address), so the call
+ * makes no hipMalloc / hipFree and touches no pool.  Limits: batches whose intermediates exceed the workspace
+ * (about seq_len * top_k * (4 * hidden + 2 * intermediate + 36) bytes: 53 tokens at top-8, hidden 4096,
+ * intermediate 1536) are rejected with InvalidShape before anything is launched; expert weights that only the
+ * portable kernels take are rejected with NotFound.  Every call on a GPU uses the same workspace: calls that
+ * overlap on one GPU (two streams, two threads) race; consecutive calls on one stream are ordered. */
+int32_t rmlx_hip_moe_forward_noalloc(const rmlx_qweight* gate, const rmlx_qweight* up,
+                                     const rmlx_qweight* down, const rmlx_array* x,
+                                     const rmlx_array* gate_logits, size_t top_k,
+                                     const rmlx_array* expert_bias, void* out_f16_dev, size_t out_bytes,
+                                     rmlx_stream stream);
+
 /* ---- AWQ / GPTQ INT4 dequantisation to f32 -----------------------------------------------------
  * `awq_dequant` (quantized.rs:2269-2383, kernel :707-733): qweight u32 [rows, cols/8] packed along
  * the columns, qzeros u32 [rows/group_size, cols/8], scales f32 [rows/group_size, cols];

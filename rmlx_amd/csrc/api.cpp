@@ -10,7 +10,18 @@
 
 #include "common.hpp"
 
+// Workspace of the entry point that allocates nothing (rmlx_hip_moe_forward_noalloc): device memory that exists
+// from the moment the code object is loaded until the process ends, one copy per GPU.  Host code never uses this
+// name as an address: rmlx_hip_init resolves the device address once per device and every use goes through that.
+constexpr size_t kStaticScratchBytes = 8u << 20;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
 namespace rmlx {
+
+namespace {
+constexpr int kMaxDevices = 64;
+void* g_static_scratch[kMaxDevices] = {};  // device address of `scratch` on every device rmlx_hip_init has seen
+}  // namespace
 
 std::string& last_error() {
   thread_local std::string e;
@@ -73,10 +84,21 @@ std::mutex g_pool_mutex;
 std::map<hipStream_t, std::vector<Block>> g_pool;
 }  // namespace
 
-int32_t Scratch::alloc(size_t bytes, hipStream_t s) {
+int32_t Scratch::alloc(size_t bytes, hipStream_t s, Arena* arena) {
   release();
   stream = s;
   if (bytes == 0) bytes = 16;
+  if (arena != nullptr) {  // carved from the caller's block, 256-byte aligned, never handed to the pool
+    const size_t start = (arena->used + 255) & ~(size_t)255;
+    if (start + bytes > arena->capacity)
+      return fail(RMLX_INVALID_SHAPE, "the call needs more than the %zu bytes of the static workspace", arena->capacity);
+    ptr = arena->base + start;
+    size = bytes;
+    arena->used = start + bytes;
+    pooled = false;
+    return RMLX_OK;
+  }
+  pooled = true;
   {
     std::lock_guard<std::mutex> lock(g_pool_mutex);
     std::vector<Block>& free_list = g_pool[s];
@@ -97,11 +119,11 @@ int32_t Scratch::alloc(size_t bytes, hipStream_t s) {
 }
 
 void Scratch::release() {
-  if (ptr != nullptr) {
+  if (ptr != nullptr && pooled) {
     std::lock_guard<std::mutex> lock(g_pool_mutex);
     g_pool[stream].push_back(Block{ptr, size});
-    ptr = nullptr;
   }
+  ptr = nullptr;
 }
 
 // Frees the idle scratch blocks of a stream (the caller has synchronised it); `forget` also drops its entry.
@@ -477,6 +499,11 @@ int32_t rmlx_hip_init(int32_t device) {
   RMLX_HIP_CHECK(hipGetDeviceProperties(&prop, device));
   if (std::strncmp(prop.gcnArchName, "gfx950", 6) != 0)
     return fail(RMLX_RUNTIME_ERROR, "device %d is %s; this library only contains gfx950 code", device, prop.gcnArchName);
+  if (device < kMaxDevices && g_static_scratch[device] == nullptr) {
+    void* p = nullptr;
+    RMLX_HIP_CHECK(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+    g_static_scratch[device] = p;
+  }
   ctx().device = device;
   ctx().num_cus = prop.multiProcessorCount;
   ctx().ready = true;
@@ -902,9 +929,12 @@ int32_t rmlx_hip_gather_qmm(const rmlx_array* x, const void* w_packed_dev, size_
 
 // ---- routing / grouping / data movement ----------------------------------------------------------------
 
-int32_t rmlx_hip_topk_route(const rmlx_array* gate_logits, size_t top_k, const rmlx_array* expert_bias,
-                            int32_t renormalize, uint32_t* expert_indices_dev, float* expert_weights_dev,
-                            uint32_t* expert_counts_dev, uint32_t* dispatch_offsets_dev, rmlx_stream stream) {
+}  // extern "C"
+
+namespace {
+int32_t topk_route_impl(const rmlx_array* gate_logits, size_t top_k, const rmlx_array* expert_bias,
+                        int32_t renormalize, uint32_t* expert_indices_dev, float* expert_weights_dev,
+                        uint32_t* expert_counts_dev, uint32_t* dispatch_offsets_dev, rmlx_stream stream, Arena* arena) {
   RMLX_TRY(require_init());
   if (gate_logits == nullptr) return fail(RMLX_INVALID_SHAPE, "gpu_topk_route: null gate_logits");
   if (gate_logits->ndim != 2)
@@ -933,7 +963,7 @@ int32_t rmlx_hip_topk_route(const rmlx_array* gate_logits, size_t top_k, const r
   Scratch lg32, bias32;
   const float* lg = static_cast<const float*>(gate_logits->data);
   if (gate_logits->dtype == RMLX_DTYPE_F16) {
-    RMLX_TRY(lg32.alloc(T * E * 4, s));
+    RMLX_TRY(lg32.alloc(T * E * 4, s, arena));
     RMLX_TRY(launch_cast_f16_to_f32(static_cast<const __half*>(gate_logits->data), static_cast<float*>(lg32.ptr), T * E, s));
     lg = static_cast<const float*>(lg32.ptr);
   }
@@ -941,7 +971,7 @@ int32_t rmlx_hip_topk_route(const rmlx_array* gate_logits, size_t top_k, const r
   if (expert_bias != nullptr) {
     bias = static_cast<const float*>(expert_bias->data);
     if (expert_bias->dtype == RMLX_DTYPE_F16) {
-      RMLX_TRY(bias32.alloc(E * 4, s));
+      RMLX_TRY(bias32.alloc(E * 4, s, arena));
       RMLX_TRY(launch_cast_f16_to_f32(static_cast<const __half*>(expert_bias->data), static_cast<float*>(bias32.ptr), E, s));
       bias = static_cast<const float*>(bias32.ptr);
     }
@@ -949,6 +979,16 @@ int32_t rmlx_hip_topk_route(const rmlx_array* gate_logits, size_t top_k, const r
   RMLX_TRY(launch_topk_route(lg, bias, T32, (uint32_t)E, (uint32_t)top_k, renormalize, expert_indices_dev,
                              expert_weights_dev, expert_counts_dev, dispatch_offsets_dev, s));
   return finish(s);
+}
+}  // namespace
+
+extern "C" {
+
+int32_t rmlx_hip_topk_route(const rmlx_array* gate_logits, size_t top_k, const rmlx_array* expert_bias,
+                            int32_t renormalize, uint32_t* expert_indices_dev, float* expert_weights_dev,
+                            uint32_t* expert_counts_dev, uint32_t* dispatch_offsets_dev, rmlx_stream stream) {
+  return topk_route_impl(gate_logits, top_k, expert_bias, renormalize, expert_indices_dev, expert_weights_dev,
+                         expert_counts_dev, dispatch_offsets_dev, stream, nullptr);
 }
 
 int32_t rmlx_hip_moe_sort(const uint32_t* expert_indices_dev, size_t n_assign, size_t n_experts,
@@ -1080,7 +1120,8 @@ struct FusedRoute { const float* logits; const float* bias; uint32_t* idx_out; f
 
 int32_t moe_grouped_impl(const rmlx_qweight* gate, const rmlx_qweight* up, const rmlx_qweight* down,
                          const rmlx_array* x, const uint32_t* expert_indices_dev, const float* expert_weights_dev,
-                         size_t top_k, void* out_f16_dev, size_t out_bytes, rmlx_stream stream, const FusedRoute* route) {
+                         size_t top_k, void* out_f16_dev, size_t out_bytes, rmlx_stream stream, const FusedRoute* route,
+                         Arena* arena) {
   RMLX_TRY(require_init());
   ExpertShapes sh;
   RMLX_TRY(check_expert_weights("MoeLayer", gate, up, down, &sh));
@@ -1106,10 +1147,14 @@ int32_t moe_grouped_impl(const rmlx_qweight* gate, const rmlx_qweight* up, const
   Scratch cast, meta, h, y;
   const __half* xk = static_cast<const __half*>(x->data);
   if (x->dtype != RMLX_DTYPE_F16) {
-    RMLX_TRY(cast.alloc(T * sh.D * 2, s));
+    RMLX_TRY(cast.alloc(T * sh.D * 2, s, arena));
     RMLX_TRY(launch_cast_to_f16(x->data, x->dtype, static_cast<__half*>(cast.ptr), T * sh.D, s));
     xk = static_cast<const __half*>(cast.ptr);
   }
+  if (sh.portable && !gemm && arena != nullptr)
+    return fail(RMLX_NOT_FOUND, "MoeLayer: these expert weights run on the portable kernels, which the entry point "
+                                "without allocations does not cover (4-bit group 64 / 128 or 8-bit group 64, aligned "
+                                "buffers, dimensions in multiples of 512 / 256)");
   if (sh.portable && !gemm) {
     // Assignments stay in their own order: position a holds token a / top_k and expert idx[a].
     if (route != nullptr)
@@ -1133,7 +1178,7 @@ int32_t moe_grouped_impl(const rmlx_qweight* gate, const rmlx_qweight* up, const
   }
   if (!aligned16(xk)) return fail(RMLX_INVALID_SHAPE, "MoeLayer: input must be 16-byte aligned");
   // meta: sorted[A] | sorted_tok[A] | inv[A] | chunk_tab[3*max_chunks] | n_chunks[1]
-  RMLX_TRY(meta.alloc(((size_t)3 * A + 3 * (size_t)max_chunks + 4) * 4, s));
+  RMLX_TRY(meta.alloc(((size_t)3 * A + 3 * (size_t)max_chunks + 4) * 4, s, arena));
   uint32_t* sorted = static_cast<uint32_t*>(meta.ptr);
   uint32_t* sorted_tok = sorted + A;
   uint32_t* inv = sorted_tok + A;
@@ -1145,8 +1190,8 @@ int32_t moe_grouped_impl(const rmlx_qweight* gate, const rmlx_qweight* up, const
   else
     RMLX_TRY(launch_moe_sort(expert_indices_dev, A, sh.E, (uint32_t)top_k, sorted, sorted_tok, inv, nullptr, nullptr, chunk_tab, n_chunks,
                              chunk_rows, s));
-  RMLX_TRY(h.alloc((size_t)A * sh.I * 2, s));
-  RMLX_TRY(y.alloc((size_t)A * sh.D * 4, s));
+  RMLX_TRY(h.alloc((size_t)A * sh.I * 2, s, arena));
+  RMLX_TRY(y.alloc((size_t)A * sh.D * 4, s, arena));
   RMLX_TRY(run_expert_ffn(gate, up, down, sh, xk, sorted_tok, chunk_tab, n_chunks, max_chunks,
                           static_cast<__half*>(h.ptr), y.ptr, 1, gemm, s));
   RMLX_TRY(launch_moe_combine(static_cast<const float*>(y.ptr), inv, expert_weights_dev, T32, (uint32_t)top_k, sh.D,
@@ -1166,12 +1211,16 @@ int32_t rmlx_hip_moe_forward_grouped(const rmlx_qweight* gate, const rmlx_qweigh
                                      const float* expert_weights_dev, size_t top_k, void* out_f16_dev, size_t out_bytes,
                                      rmlx_stream stream) {
   return moe_grouped_impl(gate, up, down, x, expert_indices_dev, expert_weights_dev, top_k, out_f16_dev, out_bytes, stream,
-                          nullptr);
+                          nullptr, nullptr);
 }
 
-int32_t rmlx_hip_moe_forward(const rmlx_qweight* gate, const rmlx_qweight* up, const rmlx_qweight* down,
-                             const rmlx_array* x, const rmlx_array* gate_logits, size_t top_k,
-                             const rmlx_array* expert_bias, void* out_f16_dev, size_t out_bytes, rmlx_stream stream) {
+}  // extern "C"
+
+namespace {
+int32_t moe_forward_impl(const rmlx_qweight* gate, const rmlx_qweight* up, const rmlx_qweight* down,
+                         const rmlx_array* x, const rmlx_array* gate_logits, size_t top_k,
+                         const rmlx_array* expert_bias, void* out_f16_dev, size_t out_bytes, rmlx_stream stream,
+                         Arena* arena) {
   RMLX_TRY(require_init());
   if (x == nullptr || gate_logits == nullptr) return fail(RMLX_INVALID_SHAPE, "MoeLayer: null argument");
   if (gate_logits->ndim != 2 || x->ndim != 2 || gate_logits->shape[0] != x->shape[0])
@@ -1183,7 +1232,7 @@ int32_t rmlx_hip_moe_forward(const rmlx_qweight* gate, const rmlx_qweight* up, c
   if (top_k == 0 || top_k > 8) return fail(RMLX_INVALID_SHAPE, "gpu_topk_route: top_k must be in [1, 8], got %zu", top_k);
   hipStream_t s = (hipStream_t)stream;
   Scratch route;
-  RMLX_TRY(route.alloc(T * top_k * 8 + 16, s));
+  RMLX_TRY(route.alloc(T * top_k * 8 + 16, s, arena));
   uint32_t* idx = static_cast<uint32_t*>(route.ptr);
   float* wts = reinterpret_cast<float*>(idx + T * top_k);
   // Decode-sized batches with f32 logits: routing and grouping share one launch.
@@ -1193,12 +1242,55 @@ int32_t rmlx_hip_moe_forward(const rmlx_qweight* gate, const rmlx_qweight* up, c
       T <= 8 && route_sort_fusable((uint32_t)T, (uint32_t)gate->n_experts, (uint32_t)top_k)) {
     const FusedRoute fr{static_cast<const float*>(gate_logits->data),
                         expert_bias != nullptr ? static_cast<const float*>(expert_bias->data) : nullptr, idx, wts};
-    return moe_grouped_impl(gate, up, down, x, idx, wts, top_k, out_f16_dev, out_bytes, stream, &fr);
+    return moe_grouped_impl(gate, up, down, x, idx, wts, top_k, out_f16_dev, out_bytes, stream, &fr, arena);
   }
   // Asynchronous inner calls need a real stream handle: the null stream means "synchronous".
-  RMLX_TRY(rmlx_hip_topk_route(gate_logits, top_k, expert_bias, 1, idx, wts, nullptr, nullptr, stream));
-  RMLX_TRY(rmlx_hip_moe_forward_grouped(gate, up, down, x, idx, wts, top_k, out_f16_dev, out_bytes, stream));
+  RMLX_TRY(topk_route_impl(gate_logits, top_k, expert_bias, 1, idx, wts, nullptr, nullptr, stream, arena));
+  RMLX_TRY(moe_grouped_impl(gate, up, down, x, idx, wts, top_k, out_f16_dev, out_bytes, stream, nullptr, arena));
   return finish(s);
+}
+}  // namespace
+
+extern "C" {
+
+int32_t rmlx_hip_moe_forward(const rmlx_qweight* gate, const rmlx_qweight* up, const rmlx_qweight* down,
+                             const rmlx_array* x, const rmlx_array* gate_logits, size_t top_k,
+                             const rmlx_array* expert_bias, void* out_f16_dev, size_t out_bytes, rmlx_stream stream) {
+  return moe_forward_impl(gate, up, down, x, gate_logits, top_k, expert_bias, out_f16_dev, out_bytes, stream, nullptr);
+}
+
+// The routed block for callers that cannot allocate (HIP graph capture, serving loops that forbid it): every
+// intermediate is carved from the static workspace, so the call makes no hipMalloc / hipFree.  Calls on one GPU
+// share that workspace: two of them in flight at the same time race.
+int32_t rmlx_hip_moe_forward_noalloc(const rmlx_qweight* gate, const rmlx_qweight* up, const rmlx_qweight* down,
+                                     const rmlx_array* x, const rmlx_array* gate_logits, size_t top_k,
+                                     const rmlx_array* expert_bias, void* out_f16_dev, size_t out_bytes,
+                                     rmlx_stream stream) {
+  RMLX_TRY(require_init());
+  void* base = ctx().device < kMaxDevices ? g_static_scratch[ctx().device] : nullptr;
+  if (base == nullptr) return fail(RMLX_RUNTIME_ERROR, "the static workspace was not resolved on device %d", ctx().device);
+  if (gate == nullptr || down == nullptr || x == nullptr || gate_logits == nullptr)
+    return fail(RMLX_INVALID_SHAPE, "MoeLayer: null argument");
+  if (x->ndim == 2 && top_k >= 1 && top_k <= 8) {
+    // upper bound of what the block carves, every piece rounded up to 256 bytes
+    const size_t T = x->shape[0], A = T * top_k, E = gate->n_experts, D = gate->in_features;
+    const size_t I = up == nullptr ? gate->out_features / 2 : gate->out_features;
+    auto r256 = [](size_t b) { return (b + 255) & ~(size_t)255; };
+    const size_t max_chunks = A / 8 + (A < E ? A : E);
+    size_t need = r256(A * 8 + 16) + r256((3 * A + 3 * max_chunks + 4) * 4) + r256(A * I * 2) + r256(A * D * 4);
+    if (x->dtype != RMLX_DTYPE_F16) need += r256(T * D * 2);
+    if (gate_logits->dtype == RMLX_DTYPE_F16) need += r256(T * E * 4);
+    if (expert_bias != nullptr && expert_bias->dtype == RMLX_DTYPE_F16) need += r256(E * 4);
+    if (need > kStaticScratchBytes)
+      return fail(RMLX_INVALID_SHAPE,
+                  "MoeLayer (entry point without allocations): %zu tokens x top-%zu at hidden %zu / intermediate %zu need "
+                  "%zu bytes of workspace, the static workspace holds %zu; split the batch or call rmlx_hip_moe_forward",
+                  T, top_k, D, I, need, kStaticScratchBytes);
+  }
+  Arena arena;
+  arena.base = static_cast<char*>(base);
+  arena.capacity = kStaticScratchBytes;
+  return moe_forward_impl(gate, up, down, x, gate_logits, top_k, expert_bias, out_f16_dev, out_bytes, stream, &arena);
 }
 
 // ---- AWQ / GPTQ dequantisation ---------------------------------------------------------------------

@@ -60,11 +60,18 @@ int32_t finish(hipStream_t stream);
 
 // Stream-ordered scratch from a per-stream pool (see api.cpp).  Used for dtype casts, the
 // re-laid-out activations of the GEMM and the MoE intermediates; the f16 qmv path needs none.
+// A caller-provided block that scratch is carved from instead of the pool (entry points that must not allocate).
+struct Arena {
+  char* base = nullptr;
+  size_t capacity = 0, used = 0;
+};
+
 struct Scratch {
   void* ptr = nullptr;
   size_t size = 0;
   hipStream_t stream = nullptr;
-  int32_t alloc(size_t bytes, hipStream_t s);
+  bool pooled = false;
+  int32_t alloc(size_t bytes, hipStream_t s, Arena* arena = nullptr);
   void release();
   ~Scratch() { release(); }
 };

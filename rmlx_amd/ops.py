@@ -286,12 +286,15 @@ def moe_forward_grouped(gate, up, down, x, expert_indices, expert_weights, top_k
     return out
 
 
-def moe_forward(gate, up, down, x, gate_logits, top_k, expert_bias=None, stream=None, out=None):
+def moe_forward(gate, up, down, x, gate_logits, top_k, expert_bias=None, stream=None, out=None, noalloc=False):
+    """Routing + routed expert block.  `noalloc=True` takes the entry point that carves every intermediate from the
+    library's static workspace (the caller must pass `out`: this wrapper would otherwise allocate it)."""
     if out is None:
         out = DeviceBuffer((x.shape[0], x.shape[1]), F16)
     xa, la = x.array(), gate_logits.array()
     ba = expert_bias.array() if expert_bias is not None else None
-    rt.check(rt.lib().rmlx_hip_moe_forward(gate.handle, up.handle if up is not None else None, down.handle,
+    fn = rt.lib().rmlx_hip_moe_forward_noalloc if noalloc else rt.lib().rmlx_hip_moe_forward
+    rt.check(fn(gate.handle, up.handle if up is not None else None, down.handle,
                                            ctypes.byref(xa), ctypes.byref(la), top_k,
                                            ctypes.byref(ba) if ba is not None else None, out.ptr, out.nbytes,
                                            _h(stream)))

@@ -40,7 +40,7 @@ EXPORTS = [
     "rmlx_hip_affine_quantized_matmul_batched", "rmlx_hip_qmm_select", "rmlx_hip_qmm_add_residual", "rmlx_hip_qmm_swiglu", "rmlx_hip_qmm_encode_many", "rmlx_hip_quantized_linear_forward",
     "rmlx_hip_gather_qmm", "rmlx_hip_topk_route", "rmlx_hip_moe_sort", "rmlx_hip_index_gather",
     "rmlx_hip_scatter_weighted_add", "rmlx_hip_silu_gate", "rmlx_hip_expert_group_grouped_forward",
-    "rmlx_hip_moe_forward_grouped", "rmlx_hip_moe_forward", "rmlx_hip_awq_dequant", "rmlx_hip_gptq_dequant",
+    "rmlx_hip_moe_forward_grouped", "rmlx_hip_moe_forward", "rmlx_hip_moe_forward_noalloc", "rmlx_hip_awq_dequant", "rmlx_hip_gptq_dequant",
     "rmlx_hip_qmm_norm", "rmlx_hip_set_expert_gemm_min_rows",
 ]
 
@@ -96,6 +96,7 @@ def lib():
         "rmlx_hip_expert_group_grouped_forward": [vp, vp, vp, sz, vp, vp, arr, vp, sz, vp],
         "rmlx_hip_moe_forward_grouped": [vp, vp, vp, arr, vp, vp, sz, vp, sz, vp],
         "rmlx_hip_moe_forward": [vp, vp, vp, arr, arr, sz, arr, vp, sz, vp],
+        "rmlx_hip_moe_forward_noalloc": [vp, vp, vp, arr, arr, sz, arr, vp, sz, vp],
         "rmlx_hip_qmm_norm": [vp, arr, arr, arr, vp, sz, vp],
         "rmlx_hip_awq_dequant": [vp, sz, vp, sz, vp, sz, sz, sz, sz, vp, sz, vp],
         "rmlx_hip_gptq_dequant": [vp, sz, vp, sz, vp, sz, vp, sz, sz, sz, sz, vp, sz, vp],

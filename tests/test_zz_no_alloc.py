@@ -1,0 +1,89 @@
+"""The entry point that allocates nothing (rmlx_hip_moe_forward_noalloc) against rmlx_hip_moe_forward, through the
+C ABI: same kernels over a static workspace instead of pooled scratch, so the outputs must be bit-identical.
+Two calls in a row on the same workspace, the second with a smaller input, then the limits."""
+
+import numpy as np
+import pytest
+
+from oracle import model
+from tests.helpers import assert_close, make_weight, make_x
+
+pytestmark = pytest.mark.gpu
+
+
+def _experts(rng, E, D, I, bits=4):
+    from rmlx_amd import ops
+    gu = make_weight(rng, 2 * I, D, bits, lead=(E,))
+    down = make_weight(rng, D, I, bits, lead=(E,))
+    gate, up = tuple(a[:, :I] for a in gu), tuple(a[:, I:] for a in gu)
+    return gate, up, down, ops.QuantizedWeight.from_numpy(*gu, 64, bits), ops.QuantizedWeight.from_numpy(*down, 64, bits)
+
+
+def _both(gh, dh, x, logits, K, bias=None):
+    """(pooled entry point, no-allocation entry point) on the same device inputs."""
+    from rmlx_amd import ops
+    from rmlx_amd.runtime import DeviceBuffer
+    xd, ld = DeviceBuffer.from_numpy(x), DeviceBuffer.from_numpy(logits)
+    bd = DeviceBuffer.from_numpy(bias) if bias is not None else None
+    want = ops.moe_forward(gh, None, dh, xd, ld, K, expert_bias=bd).numpy()
+    out = DeviceBuffer.from_numpy(np.full((x.shape[0], x.shape[1]), np.nan, np.float16))  # must be overwritten
+    got = ops.moe_forward(gh, None, dh, xd, ld, K, expert_bias=bd, out=out, noalloc=True).numpy()
+    return want, got
+
+
+def test_noalloc_matches_the_pooled_entry_point_on_two_calls_in_a_row(hip):
+    rng = np.random.default_rng(77)
+    E, D, I, K = 16, 1024, 512, 4
+    gate, up, down, gh, dh = _experts(rng, E, D, I)
+    # first call: 40 tokens (two-step routing, workgroup-wide grouping); second: 5 tokens (one fused launch) on the
+    # workspace the first call left behind; third: enough rows per expert for the grouped GEMM
+    for T in (40, 5, 48):
+        x = make_x(rng, T, D)
+        logits = rng.standard_normal((T, E)).astype(np.float32)
+        print(f"noalloc T={T} E={E} D={D} I={I} K={K}", flush=True)
+        want, got = _both(gh, dh, x, logits, K)
+        assert np.array_equal(want.view(np.uint16), got.view(np.uint16)), f"T={T}"
+        idx, w, _, _ = model.topk_route(logits, K)
+        assert_close(got, model.moe_forward(x, idx, w, gate, up, down, 64, K), f"oracle T={T}")
+
+
+def test_noalloc_casts_and_bias_come_from_the_workspace_too(hip):
+    rng = np.random.default_rng(78)
+    E, D, I, K = 8, 512, 512, 2
+    gate, up, down, gh, dh = _experts(rng, E, D, I, bits=8)
+    x = rng.standard_normal((9, D)).astype(np.float32)          # f32 activations: cast inside
+    logits = rng.standard_normal((9, E)).astype(np.float16)     # f16 logits and bias: widened inside
+    bias = rng.standard_normal(E).astype(np.float16)
+    print("noalloc f32 x, f16 logits, f16 bias, 8-bit experts", flush=True)
+    want, got = _both(gh, dh, x, logits, K, bias)
+    assert np.array_equal(want.view(np.uint16), got.view(np.uint16))
+    x2 = x[:3]
+    want, got = _both(gh, dh, x2, logits[:3], K, bias)
+    assert np.array_equal(want.view(np.uint16), got.view(np.uint16))
+
+
+def test_noalloc_limits(hip):
+    from rmlx_amd import ops
+    from rmlx_amd.runtime import F16, DeviceBuffer
+    rng = np.random.default_rng(79)
+    E, D, I, K = 8, 4096, 1536, 8
+    _, _, _, gh, dh = _experts(rng, E, D, I)
+    for T, ok in ((53, True), (54, False), (400, False)):
+        xd = DeviceBuffer.from_numpy(make_x(rng, T, D))
+        ld = DeviceBuffer.from_numpy(rng.standard_normal((T, E)).astype(np.float32))
+        out = DeviceBuffer((T, D), F16)
+        print(f"noalloc limit T={T}", flush=True)
+        if ok:
+            got = ops.moe_forward(gh, None, dh, xd, ld, K, out=out, noalloc=True).numpy()
+            assert np.array_equal(got.view(np.uint16), ops.moe_forward(gh, None, dh, xd, ld, K).numpy().view(np.uint16))
+        else:
+            with pytest.raises(ops.KernelError, match="static workspace holds 8388608"):
+                ops.moe_forward(gh, None, dh, xd, ld, K, out=out, noalloc=True)
+    # weights that only the portable kernels take (group size 32 below the grouped-GEMM threshold)
+    gu = make_weight(rng, 2 * 64, 64, 4, 32, lead=(4,))
+    dn = make_weight(rng, 64, 64, 4, 32, lead=(4,))
+    g32, d32 = ops.QuantizedWeight.from_numpy(*gu, 32, 4), ops.QuantizedWeight.from_numpy(*dn, 32, 4)
+    xd = DeviceBuffer.from_numpy(make_x(rng, 2, 64))
+    ld = DeviceBuffer.from_numpy(rng.standard_normal((2, 4)).astype(np.float32))
+    with pytest.raises(ops.KernelError, match="portable kernels"):
+        ops.moe_forward(g32, None, d32, xd, ld, 2, out=DeviceBuffer((2, 64), F16), noalloc=True)
