@@ -1,18 +1,20 @@
 #!/usr/bin/env python3
 """Benchmark of the quantized-matmul hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--quick]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--only a,b,...] [--no-cpu]
 
-Headline (`value`): Q4 qmv at M=1, K=N=4096 (group 64, f16) in GB/s of algorithmic bytes.  A step
-is one launch of the qmv kernel; weights are cycled over enough distinct sets (> 1 GiB) that
-every launch streams from HBM instead of the L2 / Infinity Cache.  All inputs are resident in
-HBM before the timed region.  The other benchmark configurations (qmv at N=9216, Q4 qmm at
-M=128/512, Q8 bf16 qmm, the MoE block) are timed the same way and reported under "extra".
-One JSON line is printed on stdout.
+Headline (`value`): Q4 qmv at M=1, K=N=4096 (group 64, f16) in GB/s of algorithmic bytes.  A step is a
+train of TRAIN (200) back-to-back launches of the kernel on one stream; the weights are cycled over enough
+distinct sets (> 1 GiB) that every launch streams from HBM instead of the L2 / Infinity Cache.  W warm-up
+steps and an untimed settle phase come first, then exactly K steps are timed with HIP events on that stream.
+All inputs are resident in HBM before the timed region.  The other benchmark configurations (qmv at N=9216,
+Q4 qmm at M=128/512, Q8 bf16 qmm, gather_qmm, the MoE block), the machine floors (empty launch, plain read,
+MFMA-only loop) and the CPU baselines are reported under "extra" / "cpu_baseline".  One JSON line on stdout.
 """
 import argparse
 import json
 import os
+import re
 import sys
 import time
 
@@ -23,12 +25,22 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0      # MI355X HBM3E
 MFMA_F16_PEAK_TF = 2500.0  # dense f16 / bf16 MFMA
+TRAIN = 200                # launches per step of the matmul sections
+GEMM_MIN_LAUNCHES = 10000  # the clock needs tens of milliseconds of sustained matrix work to settle
+SETTLE_S = 0.25            # untimed run of the workload in front of every timed region
 
-# HBM-side bytes per launch of the two roofline kernels, from rocprofv3 counter runs of this script
-# (FETCH_SIZE and WRITE_SIZE, each scaled by what it reads for the plain copy below); the runs and
-# the scaling are recorded in profiles/bench_all_configs_hbm_traffic_pmc.txt.  Counters cannot be
-# read from inside this process, so the figures are carried here and re-measured with the kernels.
-MEASURED_TRAFFIC_BYTES = {"qmv_q4_m1_4096": 9541139, "qmm_q4_m512_4096": 39722504}
+
+def measured_traffic():
+    """HBM-side bytes per launch of the two roofline kernels, from the committed rocprofv3 counter summary
+    (lines `traffic_bytes_per_launch <key> <bytes>`; FETCH_SIZE and WRITE_SIZE of two counter runs of this
+    script, each scaled by what it reads for the plain copy this script also launches).  Counters cannot be
+    read from inside the process, so the figures travel in that file; None when it is absent."""
+    out = {}
+    path = os.path.join(ROOT, "profiles", "bench_hbm_traffic_pmc.txt")
+    if os.path.exists(path):
+        for m in re.finditer(r"traffic_bytes_per_launch\s+(\S+)\s+(\d+)", open(path).read()):
+            out[m.group(1)] = int(m.group(2))
+    return out
 
 
 def matmul_bytes(m, n, k, bits, gs=64, act_bytes=2):
@@ -53,18 +65,29 @@ class Timer:
         self.stream = rt.Stream()
         self.e0, self.e1 = rt.Event(), rt.Event()
 
-    def run(self, fn, steps, warmup):
-        fn(warmup)
+    def run(self, fn, launches, warmup, chunk=TRAIN):
+        """fn(c) enqueues c launches.  Warm-up, an untimed settle phase of about SETTLE_S, then `launches`
+        launches between two events; returns milliseconds per launch."""
+        fn(max(1, warmup))
         self.stream.sync()
+        t0 = time.perf_counter()
+        while time.perf_counter() - t0 < SETTLE_S:
+            fn(chunk)
+            self.stream.sync()
         self.e0.record(self.stream)
-        fn(steps)
+        done = 0
+        while done < launches:  # enqueued train by train: the queue never runs dry, the host stays ahead
+            c = min(chunk, launches - done)
+            fn(c)
+            done += c
         self.e1.record(self.stream)
         self.e1.sync()
         self.stream.sync()
-        return self.e0.elapsed_ms(self.e1) / steps  # ms per step
+        return self.e0.elapsed_ms(self.e1) / launches
 
 
-def bench_matmul(ops, rt, timer, rng, m, n, k, bits, x_dtype, steps, warmup, min_total_bytes, check=True, kernel=0):
+def bench_matmul(ops, rt, timer, rng, m, n, k, bits, x_dtype, launches, warmup, min_total_bytes, check=True, kernel=0,
+                 check_rows=None):
     from oracle import model
     wbytes = n * k * bits // 8 + 4 * (n * k // 64)
     n_sets = max(1, -(-min_total_bytes // wbytes))
@@ -83,22 +106,24 @@ def bench_matmul(ops, rt, timer, rng, m, n, k, bits, x_dtype, steps, warmup, min
         xd = rt.DeviceBuffer.from_numpy(xh)
         x64 = xh.astype(np.float64)
     outs = [rt.DeviceBuffer((m, n), rt.F16) for _ in range(min(n_sets, 8))]
-    ms = timer.run(lambda c: ops.qmm_encode_many(qws, xd, outs, c, stream=timer.stream, kernel=kernel), steps, warmup)
-    res = {"us": ms * 1e3, "steps": steps, "n_weight_sets": n_sets,
+    ms = timer.run(lambda c: ops.qmm_encode_many(qws, xd, outs, c, stream=timer.stream, kernel=kernel), launches, warmup)
+    res = {"us": ms * 1e3, "launches": launches, "n_weight_sets": n_sets,
            "bytes": matmul_bytes(m, n, k, bits, act_bytes=2), "flops": 2 * m * n * k}
     res["gbs"] = res["bytes"] / (ms * 1e-3) / 1e9
+    res["hbm_frac"] = res["gbs"] / HBM_PEAK_GBS
     res["tflops"] = res["flops"] / (ms * 1e-3) / 1e12
     if check:  # parity of the timed configuration against the oracle, on weight set 0
         ops.qmm_encode_many(qws[:1], xd, outs[:1], 1, stream=timer.stream, kernel=kernel)
         timer.stream.sync()
-        ref = model.qmm(x64, *base, 64, bits)
-        err = float(np.abs(outs[0].numpy().astype(np.float64) - ref).max())
+        rows = slice(None) if check_rows is None else slice(0, check_rows)  # (of very tall weights: the first rows)
+        ref = model.qmm(x64, base[0][rows], base[1][rows], base[2][rows], 64, bits)
+        err = float(np.abs(outs[0].numpy().astype(np.float64)[:, rows] - ref).max())
         res["max_err"], res["tol"] = err, model.tolerance(ref)
         res["pass"] = bool(err <= res["tol"])
     return res
 
 
-def bench_moe(ops, rt, timer, rng, T, steps, warmup, experts, bits=4):
+def bench_moe(ops, rt, timer, rng, T, calls, experts, bits=4):
     from oracle import model
     gate_up, down, gh, dh = experts
     x = rng.standard_normal((T, 4096)).astype(np.float16)
@@ -110,11 +135,11 @@ def bench_moe(ops, rt, timer, rng, T, steps, warmup, experts, bits=4):
         for _ in range(c):
             ops.moe_forward(gh, None, dh, xd, ld, 8, stream=timer.stream, out=out)
 
-    ms = timer.run(run, steps, warmup)
+    ms = timer.run(run, calls, 10, chunk=20)
     idx, w, _, _ = model.topk_route(logits, 8)
     distinct = len(np.unique(idx))
     nbytes = distinct * (18874368 * bits // 8 + 1179648) + T * 4096 * 2 * 2 + T * 128 * 4
-    res = {"us": ms * 1e3, "distinct_experts": distinct, "bytes": nbytes, "gbs": nbytes / (ms * 1e-3) / 1e9,
+    res = {"us": ms * 1e3, "calls": calls, "distinct_experts": distinct, "bytes": nbytes, "gbs": nbytes / (ms * 1e-3) / 1e9,
            "flops": 2 * 8 * T * (4096 * 3072 + 1536 * 4096)}
     toks = np.arange(min(T, 2))
     sel = (toks[:, None] * 8 + np.arange(8)[None, :]).reshape(-1)
@@ -126,7 +151,7 @@ def bench_moe(ops, rt, timer, rng, T, steps, warmup, experts, bits=4):
     return res
 
 
-def bench_gather(ops, rt, timer, rng, batch, mpb, gh, gate_up, steps, warmup):
+def bench_gather(ops, rt, timer, rng, batch, mpb, gh, gate_up, calls):
     """gather_qmm over the stacked gate/up weights of the MoE configuration (every batch entry names an expert)."""
     from oracle import model
     E, n, k = gh.n_experts, gh.out_features, gh.in_features
@@ -140,10 +165,10 @@ def bench_gather(ops, rt, timer, rng, batch, mpb, gh, gate_up, steps, warmup):
             ops.gather_qmm(xd, gh.weights_buf, gh.scales_buf, gh.biases_buf, idxd, batch, mpb, n, k, E, 64,
                            stream=timer.stream, out=out)
 
-    ms = timer.run(run, steps, warmup)
+    ms = timer.run(run, calls, 10, chunk=20)
     distinct = len(np.unique(idx))
     nbytes = distinct * (n * k // 2 + 4 * (n * k // 64)) + batch * mpb * (k + n) * 2
-    res = {"us": ms * 1e3, "distinct_experts": distinct, "bytes": nbytes, "gbs": nbytes / (ms * 1e-3) / 1e9}
+    res = {"us": ms * 1e3, "calls": calls, "distinct_experts": distinct, "bytes": nbytes, "gbs": nbytes / (ms * 1e-3) / 1e9}
     e0 = int(idx[0])
     ref = model.qmm(x[0].astype(np.float64), gate_up[0][e0], gate_up[1][e0], gate_up[2][e0], 64, 4)
     err = float(np.abs(out.numpy()[0].astype(np.float64) - ref).max())
@@ -151,7 +176,7 @@ def bench_gather(ops, rt, timer, rng, batch, mpb, gh, gate_up, steps, warmup):
     return res
 
 
-def bench_dequant(ops, rt, timer, rng, fmt, k, n, gs, steps, warmup):
+def bench_dequant(ops, rt, timer, rng, fmt, k, n, gs, launches):
     """AWQ / GPTQ INT4 -> f32 dequantisation of one [k, n] matrix (store-bound: 4 bytes out per element).
     Four input sets alternate; the packed inputs are an eighth of the traffic, the f32 output the rest."""
     from oracle import model
@@ -176,57 +201,154 @@ def bench_dequant(ops, rt, timer, rng, fmt, k, n, gs, steps, warmup):
         for i in range(c):
             launch(i)
 
-    ms = timer.run(run, steps, warmup)
+    ms = timer.run(run, launches, 10, chunk=50)
     nbytes = k * n * 4 + k * n // 2 + groups * n // 2 + groups * n * 4
     launch(0)
     timer.stream.sync()
     qw, qz, sc, _ = sets[0]
     ref = model.awq_dequant(qw, qz, sc, gs) if fmt == "awq" else model.gptq_dequant(qw, qz, sc, None, gs)
-    return {"us": ms * 1e3, "bytes": nbytes, "gbs": nbytes / (ms * 1e-3) / 1e9,
+    return {"us": ms * 1e3, "launches": launches, "bytes": nbytes, "gbs": nbytes / (ms * 1e-3) / 1e9,
             "hbm_frac": nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, "pass": bool(np.array_equal(out.numpy(), ref))}
 
 
-def cpu_baseline(rng, budget_s=10.0):
-    """The C restatement of the reference's scalar `affine_qmm` (oracle/affine_qmm_ref.c) on the
-    headline configuration (M=1, K=N=4096), one host thread, repeated for about `budget_s`."""
-    from oracle import model, refpath
-    n = k = 4096
-    words, s, b = make_weight(rng, n, k, 4)
-    x = rng.standard_normal((1, k)).astype(np.float16).astype(np.float32)
-    wb, s32, b32 = model.words_to_bytes(words), s.astype(np.float32), b.astype(np.float32)
-    refpath.affine_qmm(x, wb, s32, b32, 1, n, k, 64)  # warm
+def bench_floors(rt, timer, launches):
+    """What the machine does with nothing but the launch / the loads / the matrix instructions, timed with the same
+    events on the same stream as everything else: the figures the achieved fractions are to be read against."""
+    L = rt.lib()
+    sink = rt.DeviceBuffer((64,), rt.U32)
+    st = timer.stream.handle
+    floors = {}
+
+    def go(kind, src, nbytes, n_src, iters, count):
+        rt.check(L.rmlx_hip_measure_floor(kind, src, nbytes, n_src, iters, sink.ptr, count, st))
+
+    ms = timer.run(lambda c: go(rt.FLOOR_EMPTY, None, 0, 0, 0, c), launches, TRAIN)
+    floors["empty_kernel_us"] = ms * 1e3
+    for label, nbytes, total in (("9.45MB", 9453568, 1200 << 20), ("21.3MB", 21260288, 1300 << 20),
+                                 ("75.5MB", 75505664, 1300 << 20), ("1GiB", 1 << 30, 1 << 30)):
+        nbytes = -(-nbytes // 16) * 16
+        n_src = max(1, total // nbytes)
+        src = rt.DeviceBuffer((n_src * nbytes // 4,), rt.U32)
+        rt.check(L.rmlx_hip_memset(src.ptr, 1, n_src * nbytes, None))
+        n_launch = launches if nbytes < (64 << 20) else max(20, launches // 20)
+        best = None
+        for name, kind in (("u2", rt.FLOOR_READ2), ("u4", rt.FLOOR_READ4), ("u8", rt.FLOOR_READ8)):
+            ms = timer.run(lambda c: go(kind, src.ptr, nbytes, n_src, 0, c), n_launch, min(TRAIN, n_launch),
+                           chunk=min(TRAIN, n_launch))
+            r = {"us": ms * 1e3, "gbs": nbytes / (ms * 1e-3) / 1e9, "loads_in_flight_per_lane": int(name[1:])}
+            if best is None or r["us"] < best["us"]:
+                best = r
+            floors[f"read_{label}_{name}_us"] = r["us"]
+        best["bytes"], best["copies_cycled"] = nbytes, n_src
+        floors[f"read_{label}"] = best
+        src.free()
+    iters, blocks = 2048, 0
+    info_blocks = 2 * rt.device_info()["compute_units"]
+    n_mfma = max(20, launches // 20)
+    ms = timer.run(lambda c: go(rt.FLOOR_MFMA, None, blocks, 0, iters, c), n_mfma, 5, chunk=20)
+    flops = info_blocks * 8 * iters * 16 * 16384
+    floors["mfma_loop"] = {"us": ms * 1e3, "tflops": flops / (ms * 1e-3) / 1e12, "workgroups": info_blocks,
+                           "frac_of_peak": flops / (ms * 1e-3) / 1e12 / MFMA_F16_PEAK_TF}
+    return floors
+
+
+def _time_reps(fn, budget_s, max_reps=1000):
+    fn()  # warm
     reps, t0 = 0, time.perf_counter()
     while True:
-        refpath.affine_qmm(x, wb, s32, b32, 1, n, k, 64)
+        fn()
         reps += 1
         el = time.perf_counter() - t0
-        if el >= budget_s:
-            break
-    per = el / reps
-    # the same loop nest with the output columns split over the host cores this job may use
+        if el >= budget_s or reps >= max_reps:
+            return el / reps, reps, el
+
+
+def cpu_baseline(rng, budget_s, all_configs):
+    """The C restatement of the reference's scalar `affine_qmm` / `affine_qmm_q8` (oracle/affine_qmm_ref.c) timed
+    on this host: the headline configuration on one thread (the reference's CPU path is single-threaded) and with
+    the output columns split over the host threads; beside it, one bounded run of every other configuration."""
+    from oracle import model, refpath
     threads = min(16, os.cpu_count() or 1)
-    treps, t0 = 0, time.perf_counter()
-    while time.perf_counter() - t0 < budget_s / 4:
-        refpath.affine_qmm_threads(x, wb, s32, b32, 1, n, k, 64, threads=threads)
-        treps += 1
-    tper = (time.perf_counter() - t0) / treps
-    return {"value": matmul_bytes(1, n, k, 4) / per / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
-            "sample": f"{reps} repetitions of the full M=1 K=N=4096 Q4 matmul ({el:.1f} s, {per * 1e3:.2f} ms each)",
-            "us_per_matmul": per * 1e6, "host_cores_available": os.cpu_count(),
-            "all_cores": {"value": matmul_bytes(1, n, k, 4) / tper / 1e9, "unit": "GB/s", "cores": threads,
-                          "us_per_matmul": tper * 1e6, "sample": f"{treps} repetitions, columns split over {threads} threads"}}
+
+    def matmul_case(m, n, k, bits, nthreads, budget):
+        words, s, b = make_weight(rng, n, k, bits)
+        x = rng.standard_normal((m, k)).astype(np.float16).astype(np.float32)
+        wb, s32, b32 = model.words_to_bytes(words), s.astype(np.float32), b.astype(np.float32)
+        if nthreads == 1:
+            per, reps, el = _time_reps(lambda: refpath.affine_qmm(x, wb, s32, b32, m, n, k, 64, bits), budget)
+        else:
+            per, reps, el = _time_reps(lambda: refpath.affine_qmm_threads(x, wb, s32, b32, m, n, k, 64, bits, threads=nthreads), budget)
+        nb, fl = matmul_bytes(m, n, k, bits), 2 * m * n * k
+        return {"ms": per * 1e3, "gbs": nb / per / 1e9, "gflops": fl / per / 1e9, "cores": nthreads,
+                "sample": f"{reps} run(s) of the full M={m} N={n} K={k} Q{bits} matmul ({el:.1f} s)"}
+
+    head = matmul_case(1, 4096, 4096, 4, 1, budget_s)
+    out = {"value": head["gbs"], "unit": "GB/s", "cores": 1, "kind": "port", "sample": head["sample"],
+           "us_per_matmul": head["ms"] * 1e3, "host_cores_available": os.cpu_count()}
+    allc = matmul_case(1, 4096, 4096, 4, threads, budget_s / 4)
+    out["all_cores"] = {"value": allc["gbs"], "unit": "GB/s", "cores": threads, "us_per_matmul": allc["ms"] * 1e3,
+                        "sample": allc["sample"] + f", columns split over {threads} threads"}
+    if not all_configs:
+        return out
+    cfg = {}
+    cfg["config2_q4_qmv_m1_n9216"] = matmul_case(1, 9216, 4096, 4, 1, 2.0)
+    cfg["config2_q4_qmv_m8_n9216"] = matmul_case(8, 9216, 4096, 4, 1, 2.0)
+    cfg["config3_q4_qmm_m128_4096"] = matmul_case(128, 4096, 4096, 4, threads, 1.0)
+    cfg["config3_q4_qmm_m512_4096"] = matmul_case(512, 4096, 4096, 4, threads, 1.0)
+    cfg["config4_q8_qmm_m128_n12288"] = matmul_case(128, 12288, 4096, 8, threads, 1.0)
+    # config 5: per-expert `affine_qmm` on the gathered rows + SwiGLU + weighted sum.  Only the experts the routing
+    # touches are generated (same shapes and distributions as the GPU run); T = 4 on one thread, T = 32 on all.
+    for T, nthreads in ((4, 1), (32, threads)):
+        logits = rng.standard_normal((T, 128)).astype(np.float32)
+        idx, w, _, _ = model.topk_route(logits, 8)
+        x = rng.standard_normal((T, 4096)).astype(np.float16).astype(np.float32)
+        order, offsets = model.moe_sort(idx, 128)
+        used = [e for e in range(128) if offsets[e + 1] > offsets[e]]
+        weights = {}
+        for e in used:
+            gu, dn = make_weight(rng, 3072, 4096, 4), make_weight(rng, 4096, 1536, 4)
+            weights[e] = [(model.words_to_bytes(t[0]), t[1].astype(np.float32), t[2].astype(np.float32)) for t in (gu, dn)]
+
+        def mm(xe, trip, n, k):
+            if nthreads == 1:
+                return refpath.affine_qmm(xe, *trip, xe.shape[0], n, k, 64, 4)
+            return refpath.affine_qmm_threads(xe, *trip, xe.shape[0], n, k, 64, 4, threads=nthreads)
+
+        def block():
+            out_t = np.zeros((T, 4096), np.float32)
+            for e in used:
+                pos = order[offsets[e]:offsets[e + 1]]
+                xe = np.ascontiguousarray(x[pos // 8])
+                gu = mm(xe, weights[e][0], 3072, 4096)
+                g, u = gu[:, :1536], gu[:, 1536:]
+                h = np.ascontiguousarray((g / (1.0 + np.exp(-g)) * u).astype(np.float32))
+                y = mm(h, weights[e][1], 4096, 1536)
+                np.add.at(out_t, pos // 8, w[pos][:, None] * y)
+            return out_t
+
+        t0 = time.perf_counter()
+        block()
+        el = time.perf_counter() - t0
+        nbytes = len(used) * (18874368 // 2 + 1179648)
+        cfg[f"config5_moe_q4_T{T}"] = {"ms": el * 1e3, "gbs": nbytes / el / 1e9, "cores": nthreads,
+                                       "sample": f"1 run of the routed block, {len(used)} distinct experts ({el:.1f} s)"}
+    out["configs"] = cfg
+    return out
 
 
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20000)
-    ap.add_argument("--warmup", type=int, default=2000)
-    ap.add_argument("--quick", action="store_true", help="headline configuration only, short CPU baseline")
+    ap.add_argument("--steps", type=int, default=50, help=f"timed steps; a step is a train of {TRAIN} launches")
+    ap.add_argument("--warmup", type=int, default=10, help="untimed warm-up steps")
+    ap.add_argument("--only", default="", help="comma-separated sections: headline, floors, qmv, qmm, dequant, gather, moe, moe8, large")
+    ap.add_argument("--quick", action="store_true", help="headline and floors only, short CPU baseline")
     ap.add_argument("--no-cpu", action="store_true")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)")
+    sections = set(filter(None, args.only.split(","))) or ({"headline", "floors"} if args.quick else
+                                                           {"headline", "floors", "qmv", "qmm", "dequant", "gather", "moe", "moe8", "large"})
 
     from rmlx_amd import ops, runtime as rt
     rt.init(0)
@@ -234,10 +356,13 @@ def main():
     timer = Timer(rt)
     rng = np.random.default_rng(1001)
     GiB = 1 << 30
+    launches, warm = args.steps * TRAIN, args.warmup * TRAIN
+    gemm_launches = max(launches, GEMM_MIN_LAUNCHES)
+    traffic = measured_traffic()
 
     # ---- headline: Q4 qmv M=1 K=N=4096, weights cycled through > 1 GiB ---------------------------------
-    head = bench_matmul(ops, rt, timer, rng, 1, 4096, 4096, 4, "f16", args.steps, args.warmup, GiB + GiB // 8)
-    extra = {"device": info, "q4_qmv_m1_4096": head}
+    head = bench_matmul(ops, rt, timer, rng, 1, 4096, 4096, 4, "f16", launches, warm, GiB + GiB // 8)
+    extra = {"device": info, "launches_per_step": TRAIN, "q4_qmv_m1_4096": head}
     # A plain copy of known size (identity `index_gather`, 128 MiB in, 128 MiB out) so that a counter
     # run of this same command can scale FETCH_SIZE / WRITE_SIZE by what they read for it.
     rows = 16384
@@ -248,60 +373,69 @@ def main():
     extra["copy_calibration"] = {"kernel": "index_gather_kernel", "read_bytes": rows * 4096 * 2 + rows * 4,
                                  "write_bytes": rows * 4096 * 2}
     del src, ident
-    if not args.quick:
+    if "floors" in sections:
+        extra["floors"] = bench_floors(rt, timer, launches)
+    if "qmv" in sections:
         extra["q4_qmv_m1_4096_cache_resident"] = bench_matmul(ops, rt, timer, rng, 1, 4096, 4096, 4, "f16",
-                                                              args.steps, args.warmup, 0, check=False)
+                                                              launches, warm, 0, check=False)
         for m in (1, 4, 8):
-            extra[f"q4_qmv_m{m}_n9216"] = bench_matmul(ops, rt, timer, rng, m, 9216, 4096, 4, "f16", args.steps,
-                                                       args.warmup, GiB + GiB // 8, check=(m == 8))
-        extra["q4_qmv_m2_4096"] = bench_matmul(ops, rt, timer, rng, 2, 4096, 4096, 4, "f16", args.steps, args.warmup,
-                                               GiB + GiB // 8)
-        extra["q8_qmv_m1_4096"] = bench_matmul(ops, rt, timer, rng, 1, 4096, 4096, 8, "f16", args.steps, args.warmup,
-                                               GiB + GiB // 8)
-        # the GEMM sections run at least 10 000 steps: the GPU needs a few hundred milliseconds of sustained
-        # matrix work before its clock settles (a 100-launch window reads 15 % slower, a 2 000-launch one 3 %)
-        # (short runs, as under a counter pass, keep their own count)
-        gemm_steps = max(args.steps, 10000) if args.steps >= 1000 else args.steps
+            extra[f"q4_qmv_m{m}_n9216"] = bench_matmul(ops, rt, timer, rng, m, 9216, 4096, 4, "f16", launches,
+                                                       warm, GiB + GiB // 8, check=(m == 8))
+        extra["q4_qmv_m2_4096"] = bench_matmul(ops, rt, timer, rng, 2, 4096, 4096, 4, "f16", launches, warm, GiB + GiB // 8)
+        extra["q8_qmv_m1_4096"] = bench_matmul(ops, rt, timer, rng, 1, 4096, 4096, 8, "f16", launches, warm, GiB + GiB // 8)
+        # long K, short N: the shapes the reference sends to its split-K GEMV (K > 8192 and N <= 2048)
+        extra["q4_qmv_m1_n2048_k16384"] = bench_matmul(ops, rt, timer, rng, 1, 2048, 16384, 4, "f16", launches, warm, GiB + GiB // 8)
+    if "large" in sections:  # launches long enough that start-up cost no longer matters
+        big = max(400, launches // 10)
+        extra["q4_qmv_m1_n32768"] = bench_matmul(ops, rt, timer, rng, 1, 32768, 4096, 4, "f16", big, TRAIN, GiB + GiB // 8)
+        extra["q4_qmv_m1_n151936"] = bench_matmul(ops, rt, timer, rng, 1, 151936, 4096, 4, "f16", max(100, big // 4), 20,
+                                                  GiB + GiB // 8, check_rows=4096)
+    if "qmm" in sections:
         for m in (128, 512, 4096):
-            m_steps = gemm_steps if m <= 512 else max(50, gemm_steps // 10)
-            r = bench_matmul(ops, rt, timer, rng, m, 4096, 4096, 4, "f16", m_steps, min(args.warmup, m_steps), 4 * 9437184)
-            r["steps"] = m_steps
+            m_launches = gemm_launches if m <= 512 else max(50, gemm_launches // 10)
+            r = bench_matmul(ops, rt, timer, rng, m, 4096, 4096, 4, "f16", m_launches, TRAIN, 4 * 9437184)
             r["mfma_frac"] = r["tflops"] / MFMA_F16_PEAK_TF
             extra[f"q4_qmm_m{m}_4096"] = r
         for name, kern in (("q8_qmm_bf16_m128_n12288", rt.KERNEL_AUTO), ("q8_qmm_bf16_m128_n12288_bf16_mfma", rt.KERNEL_QMM_BF16)):
-            r = bench_matmul(ops, rt, timer, rng, 128, 12288, 4096, 8, "bf16", gemm_steps, args.warmup, 4 * 53477376, kernel=kern)
-            r["steps"] = gemm_steps
+            r = bench_matmul(ops, rt, timer, rng, 128, 12288, 4096, 8, "bf16", gemm_launches, TRAIN, 4 * 53477376, kernel=kern)
             r["mfma_frac"] = r["tflops"] / MFMA_F16_PEAK_TF
-            r["hbm_frac"] = r["gbs"] / HBM_PEAK_GBS
             extra[name] = r
+    if "dequant" in sections:
         for fmt in ("awq", "gptq"):
-            extra[f"{fmt}_dequant_4096x4096_gs128"] = bench_dequant(ops, rt, timer, rng, fmt, 4096, 4096, 128,
-                                                                    max(50, args.steps // 10), 10)
+            extra[f"{fmt}_dequant_4096x4096_gs128"] = bench_dequant(ops, rt, timer, rng, fmt, 4096, 4096, 128, max(200, launches // 10))
+    if sections & {"gather", "moe"}:
         gate_up = make_weight(rng, 3072, 4096, 4, lead=(128,))
         down = make_weight(rng, 4096, 1536, 4, lead=(128,))
         experts = (gate_up, down, ops.QuantizedWeight.from_numpy(*gate_up, 64, 4),
                    ops.QuantizedWeight.from_numpy(*down, 64, 4))
-        for batch, mpb in ((32, 1), (32, 8), (32, 64)):
-            r = bench_gather(ops, rt, timer, rng, batch, mpb, experts[2], gate_up, max(50, args.steps // 10), 10)
-            r["hbm_frac"] = r["gbs"] / HBM_PEAK_GBS
-            extra[f"gather_qmm_q4_b{batch}_m{mpb}"] = r
-        for T in (4, 32, 128, 512, 2048):  # from 8 rows per expert on average (T = 128) on the grouped MFMA GEMM
-            r = bench_moe(ops, rt, timer, rng, T, max(50, args.steps // (10 if T <= 128 else 40)), 10, experts)
-            r["tflops"] = r["flops"] / (r["us"] * 1e-6) / 1e12
-            r["mfma_frac"] = r["tflops"] / MFMA_F16_PEAK_TF
-            r["hbm_frac"] = r["gbs"] / HBM_PEAK_GBS
-            extra[f"moe_q4_T{T}"] = r
+        calls = max(200, launches // 10)
+        if "gather" in sections:
+            for batch, mpb in ((32, 1), (32, 8), (32, 64)):
+                r = bench_gather(ops, rt, timer, rng, batch, mpb, experts[2], gate_up, calls)
+                r["hbm_frac"] = r["gbs"] / HBM_PEAK_GBS
+                extra[f"gather_qmm_q4_b{batch}_m{mpb}"] = r
+        if "moe" in sections:
+            for T in (4, 32, 128, 512, 2048):  # from 6 rows per expert on average on the grouped MFMA GEMM
+                r = bench_moe(ops, rt, timer, rng, T, calls if T <= 128 else max(50, calls // 4), experts)
+                r["tflops"] = r["flops"] / (r["us"] * 1e-6) / 1e12
+                r["mfma_frac"] = r["tflops"] / MFMA_F16_PEAK_TF
+                r["hbm_frac"] = r["gbs"] / HBM_PEAK_GBS
+                extra[f"moe_q4_T{T}"] = r
         del experts, gate_up, down
+    if "moe8" in sections:
         gate_up = make_weight(rng, 3072, 4096, 8, lead=(128,))
         down = make_weight(rng, 4096, 1536, 8, lead=(128,))
         experts = (gate_up, down, ops.QuantizedWeight.from_numpy(*gate_up, 64, 8),
                    ops.QuantizedWeight.from_numpy(*down, 64, 8))
+        calls = max(200, launches // 10)
         for T in (4, 32, 512):
-            r = bench_moe(ops, rt, timer, rng, T, max(50, args.steps // (10 if T <= 128 else 40)), 10, experts, bits=8)
+            r = bench_moe(ops, rt, timer, rng, T, calls if T <= 128 else max(50, calls // 4), experts, bits=8)
             r["tflops"] = r["flops"] / (r["us"] * 1e-6) / 1e12
             r["hbm_frac"] = r["gbs"] / HBM_PEAK_GBS
             extra[f"moe_q8_T{T}"] = r
+        del experts, gate_up, down
 
+    step_ms = head["us"] * TRAIN / 1e3
     line = {
         "metric": "Q4 qmv HBM GB/s (M=1, K=N=4096)",
         "value": head["gbs"],
@@ -309,30 +443,30 @@ def main():
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,
-        "ms_per_step": head["us"] / 1e3,
+        "ms_per_step": step_ms,
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
         "dtype": "f16",
         "data": "synthetic",
-        "config": {"workload": "Q4 qmv M=1 K=4096 N=4096 group_size=64 f16 activations, "
+        "config": {"workload": f"Q4 qmv M=1 K=4096 N=4096 group_size=64 f16 activations; one step = {TRAIN} back-to-back launches, "
                                f"{head['n_weight_sets']} distinct weight sets cycled (HBM-resident, > 1 GiB)",
-                   "parity_max_err": head.get("max_err"), "parity_tol": head.get("tol")},
+                   "launches_per_step": TRAIN, "parity_max_err": head.get("max_err"), "parity_tol": head.get("tol")},
         "roofline": {"bound": "hbm", "achieved": head["gbs"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": head["gbs"] / HBM_PEAK_GBS, "traffic": MEASURED_TRAFFIC_BYTES["qmv_q4_m1_4096"],
-                     "kernel": "qmv_m1_kernel<4,64,1,true,1,false>", "bytes_per_launch": head["bytes"],
-                     "avg_launch_us": head["us"]},
+                     "frac": head["gbs"] / HBM_PEAK_GBS, "traffic": traffic.get("qmv_q4_m1_4096"),
+                     "kernel": "qmv_m1_kernel", "bytes_per_launch": head["bytes"], "avg_launch_us": head["us"]},
     }
-    if not args.quick and "q4_qmm_m512_4096" in extra:
+    if "q4_qmm_m512_4096" in extra:
         q = extra["q4_qmm_m512_4096"]
         line["secondary"] = {"metric": "Q4 qmm TFLOPS (M=512, K=N=4096)", "value": q["tflops"], "unit": "TFLOP/s",
                              "roofline": {"bound": "mfma", "achieved": q["tflops"], "peak": MFMA_F16_PEAK_TF,
                                           "unit": "TFLOP/s", "frac": q["mfma_frac"],
-                                          "traffic": MEASURED_TRAFFIC_BYTES["qmm_q4_m512_4096"],
-                                          "kernel": "qmm_rw_kernel<4,1,4,8,false,64>", "avg_launch_us": q["us"]},
-                             "steps": q["steps"]}
+                                          "traffic": traffic.get("qmm_q4_m512_4096"),
+                                          "kernel": "qmm_rw_kernel", "avg_launch_us": q["us"]},
+                             "launches": q["launches"]}
     if not args.no_cpu:
-        line["cpu_baseline"] = cpu_baseline(np.random.default_rng(1001), 3.0 if args.quick else 10.0)
+        line["cpu_baseline"] = cpu_baseline(np.random.default_rng(1001), 3.0 if args.quick else 10.0,
+                                            all_configs=not args.quick and not args.only)
     line["extra"] = extra
     print(json.dumps(line))
 

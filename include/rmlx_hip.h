@@ -317,6 +317,20 @@ int32_t rmlx_hip_gptq_dequant(const void* qweight_dev, size_t qweight_bytes, con
                               size_t out_features, size_t group_size, void* out_f32_dev,
                               size_t out_bytes, rmlx_stream stream);
 
+/* ---- machine floors (measurement aid; no counterpart in the reference) ---------------------------------
+ * `count` back-to-back launches, on `stream`, of a kernel that does nothing but one thing, so that a benchmark
+ * can time them with the same events as the matmul kernels:
+ *   RMLX_FLOOR_EMPTY          an empty kernel (launch cost);
+ *   RMLX_FLOOR_READ2/4/8      a plain streaming read of `bytes` bytes with 16-byte non-temporal loads, 2 / 4 / 8
+ *                             loads in flight per lane, 512-thread workgroups; launch i reads copy i % n_src of
+ *                             the n_src consecutive copies at src_dev (cycle more than the caches hold);
+ *   RMLX_FLOOR_MFMA           `iters` rounds of 16 independent v_mfma_f32_16x16x32_f16 per wave, 8 waves per
+ *                             workgroup, `bytes` workgroups (0 = two per CU): 8 * 16 * 16384 * iters flop each.
+ * sink_dev: at least 16 bytes of device memory (never written in practice; keeps the work alive). */
+enum { RMLX_FLOOR_EMPTY = 0, RMLX_FLOOR_READ4 = 1, RMLX_FLOOR_READ8 = 2, RMLX_FLOOR_MFMA = 3, RMLX_FLOOR_READ2 = 4 };
+int32_t rmlx_hip_measure_floor(int32_t kind, const void* src_dev, size_t bytes, size_t n_src, uint32_t iters,
+                               void* sink_dev, size_t count, rmlx_stream stream);
+
 #ifdef __cplusplus
 }
 #endif

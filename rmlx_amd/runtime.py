@@ -15,6 +15,7 @@ LIB_PATH = os.path.join(_HERE, "lib", "librmlx_hip.so")
 OK, INVALID_SHAPE, NOT_FOUND, RUNTIME_ERROR = 0, 1, 2, 3
 F32, F16, BF16, U32, U8 = 0, 1, 2, 3, 4
 KERNEL_AUTO, KERNEL_QMV, KERNEL_QMM, KERNEL_GENERIC, KERNEL_QMM_BF16, KERNEL_QMM_LDS, KERNEL_QMV_ROWS = 0, 1, 2, 3, 4, 5, 6
+FLOOR_EMPTY, FLOOR_READ4, FLOOR_READ8, FLOOR_MFMA, FLOOR_READ2 = 0, 1, 2, 3, 4  # rmlx_hip_measure_floor kinds
 
 
 class KernelError(RuntimeError):
@@ -41,7 +42,7 @@ EXPORTS = [
     "rmlx_hip_gather_qmm", "rmlx_hip_topk_route", "rmlx_hip_moe_sort", "rmlx_hip_index_gather",
     "rmlx_hip_scatter_weighted_add", "rmlx_hip_silu_gate", "rmlx_hip_expert_group_grouped_forward",
     "rmlx_hip_moe_forward_grouped", "rmlx_hip_moe_forward", "rmlx_hip_moe_forward_noalloc", "rmlx_hip_awq_dequant", "rmlx_hip_gptq_dequant",
-    "rmlx_hip_qmm_norm", "rmlx_hip_set_expert_gemm_min_rows",
+    "rmlx_hip_qmm_norm", "rmlx_hip_set_expert_gemm_min_rows", "rmlx_hip_measure_floor",
 ]
 
 _lib = None
@@ -73,6 +74,7 @@ def lib():
         "rmlx_hip_stream_sync": [vp],
         "rmlx_hip_stream_destroy": [vp],
         "rmlx_hip_trim_pool": [vp],
+        "rmlx_hip_measure_floor": [i32, vp, sz, sz, u32, vp, sz, vp],
         "rmlx_hip_event_create": [ctypes.POINTER(vp)],
         "rmlx_hip_event_record": [vp, vp],
         "rmlx_hip_event_sync": [vp],
