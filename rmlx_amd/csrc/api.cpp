@@ -152,7 +152,7 @@ bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) ==
 // register-weights MFMA GEMM above (the LDS-staged GEMM when K is not a multiple of 512), the
 // portable kernel for every shape the fast kernels do not take.
 enum { KERNEL_AUTO = 0, KERNEL_QMV = 1, KERNEL_QMM = 2, KERNEL_GENERIC = 3, KERNEL_QMM_BF16 = 4, KERNEL_QMM_LDS = 5,
-       KERNEL_QMV_ROWS = 6 };
+       KERNEL_QMV_ROWS = 6, KERNEL_QMM_K2 = 7, KERNEL_QMM_RW = 8 };
 constexpr uint32_t kQmvMaxM = 16;
 // group size 64: rows taken by the single-row kernel (measured: 3 and 4 rows are faster on the matrix unit)
 constexpr uint32_t kM1MaxRows = 2;
@@ -195,6 +195,7 @@ int32_t run_matmul_plain(const rmlx_qweight* qw, const void* x, int32_t x_dtype,
   const bool can_qmm_lds = ptr_ok && qmm_supported(N, K, qw->group_size, qw->bits);
   const bool can_qmm_rw = ptr_ok && qmm_rw_supported(N, K, qw->group_size, qw->bits);
   const bool can_qmm = can_qmm_lds || can_qmm_rw;
+  const bool can_qmm_k2 = ptr_ok && qmm_k2_supported(N, K, qw->group_size, qw->bits);
 
   if (kernel == KERNEL_AUTO) {
     // The multi-row GEMV streams the weights once per pass of 8 rows (4-bit; two passes share a workgroup
@@ -229,9 +230,22 @@ int32_t run_matmul_plain(const rmlx_qweight* qw, const void* x, int32_t x_dtype,
   } else if (kernel == KERNEL_QMM_BF16 && !(can_qmm_lds && qw->bits == 8 && x_dtype == RMLX_DTYPE_BF16)) {
     return fail(RMLX_INVALID_SHAPE, "the bf16 MFMA GEMM takes Bfloat16 activations and 8-bit weights (got %s, bits=%u)",
                 dtype_name(x_dtype), qw->bits);
-  } else if (kernel < 0 || kernel > KERNEL_QMV_ROWS) {
+  } else if ((kernel == KERNEL_QMM_K2 && !can_qmm_k2) || (kernel == KERNEL_QMM_RW && !can_qmm_rw)) {
+    return fail(RMLX_INVALID_SHAPE,
+                "the register-weights qmm kernels require bits in {4,8}, N %% 64 == 0, K %% 512 == 0 and 16-byte aligned "
+                "buffers (N=%u K=%u bits=%u group_size=%u)", N, K, qw->bits, qw->group_size);
+  } else if (kernel < 0 || kernel > KERNEL_QMM_RW) {
     return fail(RMLX_NOT_FOUND, "unknown kernel selector %d", kernel);
   }
+  // The K-split GEMM (64 x 128 tiles, 32x32x16 MFMAs) where its grid is one round over most of the chip: measured
+  // 23.8 against 25.4 us at M = 512, 4096 x 4096 and 27.8 against 28.8 us at M = 128, N = 12288 (8-bit); with fewer
+  // tiles the smaller tiles of the register-weights GEMM keep more CUs busy, with several rounds its 128-row tiles
+  // unpack every weight for twice as many rows.
+  if (kernel == KERNEL_QMM && can_qmm_k2) {
+    const uint64_t tiles = (uint64_t)((M + 63) / 64) * (N / 128), cus = (uint64_t)ctx().num_cus;
+    if (tiles * 10 >= cus * 7 && tiles <= cus) kernel = KERNEL_QMM_K2;
+  }
+  if (kernel == KERNEL_QMM_RW) kernel = KERNEL_QMM;
 
   // RMSNorm prologue: fused into the single-row GEMV for one or two rows (while it stages the activations);
   // every other case gets the normalised activations from a pass of its own.
@@ -246,6 +260,20 @@ int32_t run_matmul_plain(const rmlx_qweight* qw, const void* x, int32_t x_dtype,
     norm_w = nullptr;
   }
 
+  if (kernel == KERNEL_QMM_K2) {
+    Scratch cast;
+    const void* xk = x;
+    int32_t xk_dtype = x_dtype;
+    if (x_dtype == RMLX_DTYPE_F32) {
+      xk_dtype = RMLX_DTYPE_F16;
+      RMLX_TRY(cast.alloc((size_t)M * K * sizeof(__half), stream));
+      RMLX_TRY(launch_cast_to_f16(x, x_dtype, static_cast<__half*>(cast.ptr), (size_t)M * K, stream));
+      xk = cast.ptr;
+    }
+    QmmArgs a{qw->w, qw->s, qw->b, xk, xk_dtype, out, M, N, K, qw->bits, nullptr, 0, epi.kind, epi.ptr, epi.dtype};
+    *epi_done = true;
+    return launch_qmm_k2(a, qw->group_size, stream);
+  }
   if (kernel == KERNEL_QMM && can_qmm_rw) {
     // Register-weights GEMM: f16 / bf16 activations straight from the row-major matrix, no workspace
     // (bf16 -> f16 inside the kernel: exact for normal-range values, and f16 weights keep 11

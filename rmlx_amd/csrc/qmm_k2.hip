@@ -1,0 +1,393 @@
+// Quantized GEMM for gfx950, prefill-sized batches (M from about 100 rows on): weights in registers, 32x32x16
+// MFMAs, the K extent of every 128-wide block split over two halves of the workgroup.
+//
+// Replaces the reference's affine_qmm_nax_q4 / affine_qmm_mma_q8 for large M
+// (crates/rmlx-core/src/ops/quantized.rs:3331-3565, 5838-5971).
+//
+// What bounds a quantized GEMM tile on this part, per 128-wide k block of a 64 x 128 tile (measured):
+//   matrix unit   512 clk per SIMD;   L2 -> CU fill  about 45 B/clk per CU (25 KB of activations + weights: 570 clk);
+//   LDS           about 150 B/clk per CU;   vector unit  13 instructions per 8 weights unpacked.
+// The layout keeps all four near the matrix time:
+//   * v_mfma_f32_32x32x16_f16: a 1 KB operand feeds 32 768 flop, twice the 16x16x32 form, so the activation
+//     operands read from LDS per block halve (64 KB instead of 128 KB per workgroup).
+//   * Tile 64 activation rows x 128 weight rows, eight waves = 4 column groups (32 weight rows each) x 2 k halves.
+//     Wave (wn, kh) multiplies its 32 weight rows by all 64 activation rows over k half kh of every block: 4 k steps
+//     x 2 activation fragments = 8 MFMAs per block.  Every weight is loaded and unpacked by exactly one wave: lane
+//     (row, half) loads 16 contiguous bytes (Q4: 32 values; Q8: 2 x 16 bytes) and dequantises word ks straight
+//     into the operand of k step ks.  Weights never touch LDS.
+//   * Activations go global -> registers -> LDS (permuted to the slot order of the nibble unpacking, xor-swizzled:
+//     writes and reads are bank-conflict free), two stages; operands are read one block ahead into the registers
+//     the previous block has just released.
+//   * Addresses are buffer resources (uniform base in scalar registers) plus one 32-bit offset per thread, and the
+//     loads past the last block are simply not issued, so every s_waitcnt count is exact.
+//   * At the end the two k halves are added through LDS (fixed order: deterministic), which also transposes the
+//     accumulator layout into row-contiguous stores, with the fused epilogue.
+#include <type_traits>
+
+#include "common.hpp"
+
+namespace rmlx {
+namespace {
+
+typedef _Float16 h8 __attribute__((ext_vector_type(8)));
+typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+typedef float f4 __attribute__((ext_vector_type(4)));
+typedef float f16v __attribute__((ext_vector_type(16)));
+typedef uint32_t u4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u2 __attribute__((ext_vector_type(2)));
+
+constexpr int kTileM = 64, kTileN = 128, kBlockK = 128, kThreads = 512;
+constexpr int kUnroll = 4;                       // depth of the weight register ring; scales come per four blocks
+constexpr int kChunkUnits = kTileM * 16;         // 16-byte units of one activation chunk (64 rows x 128 k): 1024
+constexpr int kAL = kChunkUnits / kThreads;      // units per thread and chunk: 2
+
+struct K2Params {
+  const uint32_t* w; const __half* s; const __half* b;
+  const __half* x;  // [M,K] row-major f16 (bf16 bits when XBF16)
+  __half* out;
+  uint32_t M, N, K, tiles_m, tiles_n;
+  int32_t epi_kind, epi_dtype;
+  const void* epi;
+};
+
+__device__ __forceinline__ uint32_t h2bits(h2 v) { return __builtin_bit_cast(uint32_t, v); }
+
+struct DqConst { uint32_t m0, m1, k0, k1; };
+// 8 Q4 values of one word -> f16 weights in slot order (k0,k4,k1,k5,k2,k6,k3,k7); exact int -> f16 through the
+// magic numbers 1024 + q and 64 + q, then w = s*q + b in packed f16
+__device__ __forceinline__ h8 dequant_q4_word(uint32_t w, h2 s2, h2 b2, const DqConst& c) {
+  const uint32_t t = w >> 8;
+  const h2 k1024 = {(_Float16)1024.0f, (_Float16)1024.0f}, k64 = {(_Float16)64.0f, (_Float16)64.0f};
+  const h2 p0 = __builtin_bit_cast(h2, (w & c.m0) | c.k0) - k1024;
+  const h2 p1 = __builtin_bit_cast(h2, (w & c.m1) | c.k1) - k64;
+  const h2 p2 = __builtin_bit_cast(h2, (t & c.m0) | c.k0) - k1024;
+  const h2 p3 = __builtin_bit_cast(h2, (t & c.m1) | c.k1) - k64;
+  u4 o;
+  o.x = h2bits(p0 * s2 + b2);
+  o.y = h2bits(p1 * s2 + b2);
+  o.z = h2bits(p2 * s2 + b2);
+  o.w = h2bits(p3 * s2 + b2);
+  return __builtin_bit_cast(h8, o);
+}
+// 8 Q8 values of two words -> f16 weights in natural order
+__device__ __forceinline__ h8 dequant_q8_pair(uint32_t w0, uint32_t w1, h2 s2, h2 b2) {
+  const h2 k1024 = {(_Float16)1024.0f, (_Float16)1024.0f};
+  const h2 p0 = __builtin_bit_cast(h2, __builtin_amdgcn_perm(0x64646464u, w0, 0x04010400u)) - k1024;
+  const h2 p1 = __builtin_bit_cast(h2, __builtin_amdgcn_perm(0x64646464u, w0, 0x04030402u)) - k1024;
+  const h2 p2 = __builtin_bit_cast(h2, __builtin_amdgcn_perm(0x64646464u, w1, 0x04010400u)) - k1024;
+  const h2 p3 = __builtin_bit_cast(h2, __builtin_amdgcn_perm(0x64646464u, w1, 0x04030402u)) - k1024;
+  u4 o;
+  o.x = h2bits(p0 * s2 + b2);
+  o.y = h2bits(p1 * s2 + b2);
+  o.z = h2bits(p2 * s2 + b2);
+  o.w = h2bits(p3 * s2 + b2);
+  return __builtin_bit_cast(h8, o);
+}
+
+// LDS slot (16 bytes) of activation unit (row R of the tile, segment seg = 8 consecutive k of the block).  Segment
+// seg = 8 kh + 4 hh + ks is read by the waves of k half kh in k step ks, lane half hh; fragment R/32, lane row R%32:
+// a contiguous 1 KB run per (fragment, kh, ks).  The xor keeps that run a permutation and spreads the 16 segments
+// of a row, which one load instruction delivers to 16 neighbouring lanes, over all banks.
+__device__ __forceinline__ uint32_t act_slot(uint32_t R, uint32_t seg) {
+  return (((R >> 5) * 2 + (seg >> 3)) * 4 + (seg & 3)) * 64 + (((((seg >> 2) & 1) << 5) | (R & 31)) ^ seg);
+}
+
+template <int BITS, bool XBF16, int GS>
+__global__ __launch_bounds__(kThreads) void qmm_k2_kernel(const K2Params p) {
+  constexpr int WV = BITS == 4 ? 1 : 2;                  // 16-byte weight loads per lane and block
+  constexpr int kSbBytes = 4 * (kBlockK / GS) * 2;       // scales of one row and four blocks: 16 / 32 / 8 bytes
+  constexpr int kSbVecs = kSbBytes > 16 ? 2 : 1;
+  __shared__ u4 lds[4096];  // 64 KB: two activation stages of 16 KB; all of it for the final transposition
+
+  const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, wn = wave & 3, kh = wave >> 2;
+  const uint32_t r = lane & 31, hh = lane >> 5;
+
+  // workgroup -> tile: ids go round-robin over the 8 XCDs (one L2 each); every XCD gets a compact block of tiles
+  // (half of the row tiles x a quarter of the column tiles when those divide), so that what its L2 fetches is small
+  uint32_t wg = blockIdx.x, mt, nt;
+  const uint32_t total = p.tiles_m * p.tiles_n;
+  if (total % 8 == 0 && p.tiles_m % 2 == 0 && p.tiles_n % 4 == 0) {
+    const uint32_t xcd = wg % 8, local = wg / 8, bm = p.tiles_m / 2, bn = p.tiles_n / 4;
+    mt = (xcd % 2) * bm + local % bm;
+    nt = (xcd / 2) * bn + local / bm;
+  } else {
+    if (total % 8 == 0) wg = (wg % 8) * (total / 8) + wg / 8;
+    mt = wg % p.tiles_m;
+    nt = wg / p.tiles_m;
+  }
+  const uint32_t K = p.K, S = K / kBlockK, G = K / GS;
+  const uint32_t row_lo = mt * kTileM;
+
+  // ---- addresses: buffer resources (uniform base + byte range, in scalar registers) + one 32-bit byte offset per
+  // thread; the per-block parts of an address are uniform and ride in the scalar offset operand.  Reads past a
+  // resource's range return zero, which is what rows past M must contribute.
+  auto make_rsrc = [](const void* base, uint64_t bytes) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int)(bytes > 0xFFFFFFFFull ? 0xFFFFFFFFull : bytes), 0x00020000);
+  };
+  const uint32_t row_words = K * BITS / 32;
+  const __amdgpu_buffer_rsrc_t xr = make_rsrc(p.x + (uint64_t)row_lo * K, (uint64_t)(p.M - row_lo) * K * 2);
+  const __amdgpu_buffer_rsrc_t wr = make_rsrc(p.w + (uint64_t)nt * kTileN * row_words, (uint64_t)kTileN * row_words * 4);
+  const __amdgpu_buffer_rsrc_t sr = make_rsrc(p.s + (uint64_t)nt * kTileN * G, (uint64_t)kTileN * G * 2);
+  const __amdgpu_buffer_rsrc_t br = make_rsrc(p.b + (uint64_t)nt * kTileN * G, (uint64_t)kTileN * G * 2);
+  // activations: unit q*512 + tid -> (tile row 32 q + tid/16, segment tid%16); 16 neighbouring lanes read one row's
+  // 256 contiguous bytes
+  const uint32_t seg = tid & 15, R0 = tid >> 4;
+  const uint32_t xoff = (R0 * K + seg * 8) * 2;  // unit q: + 32 q rows
+  const uint32_t lds_w0 = act_slot(R0, seg);     // unit q: + q * 512 slots
+  // operand reads of k step ks (fragment i: + 512 slots, stage: + 1024 slots)
+  uint32_t lds_r[4];
+#pragma unroll
+  for (int ks = 0; ks < 4; ++ks) lds_r[ks] = (kh * 4 + ks) * 64 + (((hh << 5) | r) ^ (8 * kh + 4 * hh + ks));
+  // weights: row nt*128 + 32 wn + r; this lane's values of block it are k = 128 it + 64 kh + 32 hh .. + 31
+  const uint32_t woff = ((32 * wn + r) * row_words) * 4 + (8 * kh + 4 * hh) * 4 * WV;
+  const uint32_t soff = (32 * wn + r) * G * 2;
+
+  f16v acc[2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int e = 0; e < 16; ++e) acc[i][e] = 0.f;
+
+  u4 ra[2][kAL];              // activation chunks in flight (global -> registers -> LDS)
+  u4 wq[kUnroll][WV];         // weights, four blocks ahead
+  u4 s_cur[kSbVecs], b_cur[kSbVecs], s_nxt[kSbVecs], b_nxt[kSbVecs];  // scales / biases of four blocks
+
+  auto to_slot_order = [&](u4 v) {
+    if (XBF16) {  // bf16 activations: to f16 through f32 (exact for normal-range values)
+      uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const float lo = __uint_as_float(w[e] << 16), hi = __uint_as_float(w[e] & 0xFFFF0000u);
+        w[e] = h2bits((h2){(_Float16)lo, (_Float16)hi});
+      }
+      v = (u4){w[0], w[1], w[2], w[3]};
+    }
+    if (BITS != 4) return v;
+    u4 o;  // halves (k0..k7) -> slots (k0,k4,k1,k5,k2,k6,k3,k7)
+    o.x = __builtin_amdgcn_perm(v.z, v.x, 0x05040100u);
+    o.y = __builtin_amdgcn_perm(v.z, v.x, 0x07060302u);
+    o.z = __builtin_amdgcn_perm(v.w, v.y, 0x05040100u);
+    o.w = __builtin_amdgcn_perm(v.w, v.y, 0x07060302u);
+    return o;
+  };
+  auto load_a = [&](uint32_t it, u4 (&dst)[kAL]) {
+#pragma unroll
+    for (int q = 0; q < kAL; ++q)
+      dst[q] = __builtin_amdgcn_raw_buffer_load_b128(xr, xoff, it * (kBlockK * 2) + q * 32 * K * 2, 0);
+  };
+  auto store_a = [&](uint32_t stage, const u4 (&src)[kAL]) {
+#pragma unroll
+    for (int q = 0; q < kAL; ++q) lds[stage * kChunkUnits + q * 512 + lds_w0] = to_slot_order(src[q]);
+  };
+  auto load_w = [&](uint32_t it, int u) {
+#pragma unroll
+    for (int v = 0; v < WV; ++v) wq[u][v] = __builtin_amdgcn_raw_buffer_load_b128(wr, woff, it * (16 * 4 * WV) + v * 16, 0);
+  };
+  // the scales / biases of blocks 4 blk .. 4 blk + 3 of this lane's row
+  auto load_sb = [&](uint32_t blk, u4 (&ds)[kSbVecs], u4 (&db)[kSbVecs]) {
+    if (GS == 128) {
+      const u2 sv = __builtin_amdgcn_raw_buffer_load_b64(sr, soff, blk * 8, 0), bv = __builtin_amdgcn_raw_buffer_load_b64(br, soff, blk * 8, 0);
+      ds[0] = (u4){sv.x, sv.y, 0u, 0u};
+      db[0] = (u4){bv.x, bv.y, 0u, 0u};
+    } else {
+#pragma unroll
+      for (int v = 0; v < kSbVecs; ++v) {
+        ds[v] = __builtin_amdgcn_raw_buffer_load_b128(sr, soff, blk * kSbBytes + v * 16, 0);
+        db[v] = __builtin_amdgcn_raw_buffer_load_b128(br, soff, blk * kSbBytes + v * 16, 0);
+      }
+    }
+  };
+  DqConst dq;
+  dq.m0 = 0x000F000Fu; dq.m1 = 0x00F000F0u; dq.k0 = 0x64006400u; dq.k1 = 0x54005400u;
+  asm volatile("" : "+s"(dq.m0), "+s"(dq.m1), "+v"(dq.k0), "+v"(dq.k1));
+  // (scale, bias) pair of block slot u (u == kUnroll: block 0 of the next four).  This lane's 32 values of a block
+  // lie in group (128 it + 64 kh + 32 hh) / GS: GS 64 -> half kh of word u; GS 32 -> half hh of word 2u + kh;
+  // GS 128 -> half u%2 of word u/2.
+  constexpr uint32_t kSelLo = 0x01000100u, kSelHi = 0x03020302u;
+  const uint32_t sel_kh = kh ? kSelHi : kSelLo, sel_hh = hh ? kSelHi : kSelLo;
+  auto word_of = [](const u4& v, int c) { return c == 0 ? v.x : (c == 1 ? v.y : (c == 2 ? v.z : v.w)); };
+  auto scale_pair = [&](int u, h2& s2, h2& b2) {
+    const u4 (&sv)[kSbVecs] = u < kUnroll ? s_cur : s_nxt;
+    const u4 (&bv)[kSbVecs] = u < kUnroll ? b_cur : b_nxt;
+    const int c = u % kUnroll;
+    uint32_t sw, bw, sel;
+    if (GS == 64) {
+      sw = word_of(sv[0], c); bw = word_of(bv[0], c); sel = sel_kh;
+    } else if (GS == 128) {
+      sw = word_of(sv[0], c >> 1); bw = word_of(bv[0], c >> 1); sel = (c & 1) ? kSelHi : kSelLo;
+    } else {  // word 2c + kh of the eight
+      const u4& s4 = sv[(c >> 1) % kSbVecs];
+      const u4& b4 = bv[(c >> 1) % kSbVecs];
+      sw = kh ? word_of(s4, 2 * (c & 1) + 1) : word_of(s4, 2 * (c & 1));
+      bw = kh ? word_of(b4, 2 * (c & 1) + 1) : word_of(b4, 2 * (c & 1));
+      sel = sel_hh;
+    }
+    s2 = __builtin_bit_cast(h2, __builtin_amdgcn_perm(sw, sw, sel));
+    b2 = __builtin_bit_cast(h2, __builtin_amdgcn_perm(bw, bw, sel));
+  };
+  // weight operand of k step ks of block slot u, given the block's (scale, bias)
+  auto weight_operand = [&](int u, int ks, h2 s2, h2 b2) -> h8 {
+    const int c = u % kUnroll;
+    if (BITS == 4) return dequant_q4_word(word_of(wq[c][0], ks), s2, b2, dq);
+    const u4& q = wq[c][(ks >> 1) % WV];
+    return (ks & 1) ? dequant_q8_pair(q.z, q.w, s2, b2) : dequant_q8_pair(q.x, q.y, s2, b2);
+  };
+  auto read_b = [&](uint32_t stage, int i, int ks) -> h8 {
+    return __builtin_bit_cast(h8, lds[stage * kChunkUnits + i * 512 + lds_r[ks]]);
+  };
+
+  // ---- prologue: chunks 0 and 1 in LDS, chunks 2 and 3 in the register sets, weights of blocks 0..3 ----------
+  const uint32_t last = S - 1;
+  auto clampi = [&](uint32_t it) { return it < last ? it : last; };
+  load_a(0, ra[0]);
+  load_a(clampi(1), ra[1]);
+  load_sb(0, s_cur, b_cur);
+#pragma unroll
+  for (int u = 0; u < kUnroll; ++u) load_w(u, u);  // (S >= 4)
+  store_a(0, ra[0]);
+  store_a(1, ra[1]);
+  load_a(clampi(2), ra[0]);
+  load_a(clampi(3), ra[1]);
+  __syncthreads();
+  h8 bf[2][4];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) bf[i][ks] = read_b(0, i, ks);
+  __syncthreads();  // block 0 overwrites stage 0 with chunk 2: every wave must have taken its operands of chunk 0 first
+  h2 s2, b2;
+  scale_pair(0, s2, b2);
+  h8 aw = weight_operand(0, 0, s2, b2), aw_nxt;
+
+  // Block `it` (u = it % 4): its activation operands are already in bf[] (read during block it-1 from stage it%2,
+  // which nothing reads any more); stage (it+1)%2 holds chunk it+1 and is read into bf[] as the slots come free;
+  // chunk it+2 is written into stage it%2 from the register set that chunk it+4 is then loaded into.  Four k steps
+  // of two MFMAs, each carrying its share of the other work and unpacking the next weight operand; one barrier per
+  // block.  MAIN: blocks that still prefetch (all but the last four).  LOADSB: the block that fetches the scales of
+  // the four blocks after the next four.
+  auto block = [&](auto uc, auto mainc, uint32_t it) {
+    constexpr int u = decltype(uc)::value;
+    constexpr bool MAIN = decltype(mainc)::value;
+    const uint32_t st_nxt = (u + 1) & 1, st_wr = u & 1;
+    const bool writes = MAIN || it + 2 < S;  // (uniform)
+    if (MAIN && u == 0) load_sb(it / kUnroll + 1, s_nxt, b_nxt);
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) {
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(aw, bf[i][ks], acc[i], 0, 0, 0);
+        bf[i][ks] = read_b(st_nxt, i, ks);  // the slot is free: next block's operand (past the last block: unused)
+      }
+      if (ks < 3) {
+        aw_nxt = weight_operand(u, ks + 1, s2, b2);
+      } else {
+        scale_pair(u + 1, s2, b2);
+        aw_nxt = weight_operand(u + 1, 0, s2, b2);
+      }
+      if (ks < kAL && writes) lds[st_wr * kChunkUnits + ks * 512 + lds_w0] = to_slot_order(ra[u % 2][ks]);
+      if (MAIN && ks == 2) load_a(it + 4, ra[u % 2]);
+      aw = aw_nxt;
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    if (MAIN) load_w(it + kUnroll, u);  // (every word of wq[u] has been unpacked)
+    if (u == 3) {
+#pragma unroll
+      for (int v = 0; v < kSbVecs; ++v) { s_cur[v] = s_nxt[v]; b_cur[v] = b_nxt[v]; }
+    }
+    __syncthreads();
+  };
+  using std::integral_constant;
+  uint32_t it0 = 0;
+  for (; it0 + kUnroll < S; it0 += kUnroll) {
+    block(integral_constant<int, 0>{}, integral_constant<bool, true>{}, it0);
+    block(integral_constant<int, 1>{}, integral_constant<bool, true>{}, it0 + 1);
+    block(integral_constant<int, 2>{}, integral_constant<bool, true>{}, it0 + 2);
+    block(integral_constant<int, 3>{}, integral_constant<bool, true>{}, it0 + 3);
+  }
+  block(integral_constant<int, 0>{}, integral_constant<bool, false>{}, it0);
+  block(integral_constant<int, 1>{}, integral_constant<bool, false>{}, it0 + 1);
+  block(integral_constant<int, 2>{}, integral_constant<bool, false>{}, it0 + 2);
+  block(integral_constant<int, 3>{}, integral_constant<bool, false>{}, it0 + 3);
+
+  // ---- the two k halves -> one, and accumulator layout -> rows: through LDS ------------------------------------
+  // A lane holds, of fragment i: activation row m = 32 i + r, weight rows 32 wn + 8 (e/4) + 4 hh + e%4.  Partial
+  // [kh][m][32 groups of four weight rows], the group index xor-ed with m % 32 so that a wave's stores (32 rows at
+  // a stride of 512 bytes) spread over the banks.
+  float* red = reinterpret_cast<float*>(lds);
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const uint32_t m = 32 * i + r;
+#pragma unroll
+    for (int eg = 0; eg < 4; ++eg) {
+      const uint32_t cg = 8 * wn + 2 * eg + hh;  // weight rows 4 cg .. 4 cg + 3 of the tile
+      f4 v;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) v[e] = acc[i][eg * 4 + e];
+      *reinterpret_cast<f4*>(red + ((size_t)(kh * kTileM + m) * 32 + (cg ^ (m & 31))) * 4) = v;
+    }
+  }
+  __syncthreads();
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {  // 64 rows x 32 groups = 2048 units of four outputs: four per thread
+    const uint32_t g = q * kThreads + tid, m = g >> 5, cgp = g & 31, cg = cgp ^ (m & 31);
+    f4 v = *reinterpret_cast<const f4*>(red + ((size_t)m * 32 + cgp) * 4);
+    v += *reinterpret_cast<const f4*>(red + ((size_t)(kTileM + m) * 32 + cgp) * 4);
+    const uint32_t row = row_lo + m, col = nt * kTileN + 4 * cg;
+    if (row < p.M) {
+      const uint64_t o = (uint64_t)row * p.N + col;
+      if (p.epi_kind != EPI_NONE) {  // residual add / SwiGLU gate in f32, one rounding (quantized.rs:3206-3246)
+        f4 e;
+        if (p.epi_dtype == RMLX_DTYPE_F32) {
+          e = *reinterpret_cast<const f4*>(static_cast<const float*>(p.epi) + o);
+        } else {
+          const u2 eb = *reinterpret_cast<const u2*>(static_cast<const __half*>(p.epi) + o);
+          const uint32_t ex = eb.x, ey = eb.y;
+          const h2 e0 = __builtin_bit_cast(h2, ex), e1 = __builtin_bit_cast(h2, ey);
+          e = (f4){(float)e0[0], (float)e0[1], (float)e1[0], (float)e1[1]};
+        }
+#pragma unroll
+        for (int c = 0; c < 4; ++c) v[c] = p.epi_kind == EPI_RESIDUAL ? v[c] + e[c] : e[c] / (1.0f + __expf(-e[c])) * v[c];
+      }
+      const h2 lo = {(_Float16)v[0], (_Float16)v[1]};
+      const h2 hi = {(_Float16)v[2], (_Float16)v[3]};
+      *reinterpret_cast<u2*>(p.out + o) = (u2){h2bits(lo), h2bits(hi)};
+    }
+  }
+}
+
+}  // namespace
+
+bool qmm_k2_supported(uint32_t N, uint32_t K, uint32_t group_size, uint32_t bits) {
+  return (group_size == 32 || group_size == 64 || group_size == 128) && (bits == 4 || bits == 8) && N > 0 && K > 0 &&
+         N % kTileN == 0 && K % (kBlockK * kUnroll) == 0;
+}
+
+int32_t launch_qmm_k2(const QmmArgs& a, uint32_t group_size, hipStream_t s) {
+  if (!qmm_k2_supported(a.N, a.K, group_size, a.bits))
+    return fail(RMLX_INVALID_SHAPE, "qmm: unsupported shape N=%u K=%u bits=%u group_size=%u", a.N, a.K, a.bits, group_size);
+  if (a.M == 0) return RMLX_OK;
+  if (a.x_dtype != RMLX_DTYPE_F16 && a.x_dtype != RMLX_DTYPE_BF16)
+    return fail(RMLX_RUNTIME_ERROR, "qmm: f32 activations must be cast to f16 first");
+  K2Params p{};
+  p.w = a.w; p.s = a.s; p.b = a.b;
+  p.x = static_cast<const __half*>(a.x);
+  p.out = a.out; p.M = a.M; p.N = a.N; p.K = a.K;
+  p.tiles_m = (a.M + kTileM - 1) / kTileM;
+  p.tiles_n = a.N / kTileN;
+  p.epi_kind = a.epi_kind; p.epi = a.epi; p.epi_dtype = a.epi_dtype;
+  if ((uint64_t)p.tiles_m * p.tiles_n > 0x7FFFFFFFull) return fail(RMLX_INVALID_SHAPE, "qmm: grid too large");
+  const dim3 grid(p.tiles_m * p.tiles_n), block(kThreads);
+  const bool xb = a.x_dtype == RMLX_DTYPE_BF16;
+#define K2_LAUNCH(BITSV, GSV)                                                                        \
+  if (xb) hipLaunchKernelGGL((qmm_k2_kernel<BITSV, true, GSV>), grid, block, 0, s, p);              \
+  else hipLaunchKernelGGL((qmm_k2_kernel<BITSV, false, GSV>), grid, block, 0, s, p);
+#define K2_BITS(GSV) \
+  if (a.bits == 4) { K2_LAUNCH(4, GSV) } else { K2_LAUNCH(8, GSV) }
+  if (group_size == 64) { K2_BITS(64) } else if (group_size == 32) { K2_BITS(32) } else { K2_BITS(128) }
+#undef K2_BITS
+#undef K2_LAUNCH
+  RMLX_HIP_CHECK(hipGetLastError());
+  return RMLX_OK;
+}
+
+}  // namespace rmlx
