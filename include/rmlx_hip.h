@@ -198,6 +198,18 @@ int32_t rmlx_hip_gather_qmm(const rmlx_array* x, const void* w_packed_dev, size_
                             const rmlx_array* indices, size_t batch, size_t m_per_batch,
                             size_t n, size_t k, size_t n_experts, uint32_t group_size,
                             void* out_f16_dev, size_t out_bytes, rmlx_stream stream);
+/* The same with the kernel family forced (the reference exposes `gather_qmm` and `gather_qmv_fast_f16_q4`
+ * separately, quantized.rs:9404, 10061).  kernel: 0 = auto (streaming GEMV up to 8 rows per entry, grouped MFMA
+ * GEMM from 9 rows on where it takes the shape: N % 128 == 0, K % 512 == 0; the portable kernel for every other
+ * shape), 1 = streaming GEMV (group size 64 / 128, N % 16 == 0, K % 512 == 0), 2 = grouped MFMA GEMM,
+ * 3 = portable kernel. */
+int32_t rmlx_hip_gather_qmm_select(const rmlx_array* x, const void* w_packed_dev, size_t w_bytes,
+                                   const void* scales_dev, size_t scales_bytes,
+                                   const void* biases_dev, size_t biases_bytes,
+                                   const rmlx_array* indices, size_t batch, size_t m_per_batch,
+                                   size_t n, size_t k, size_t n_experts, uint32_t group_size,
+                                   int32_t kernel, void* out_f16_dev, size_t out_bytes,
+                                   rmlx_stream stream);
 
 /* ---- gpu_topk_route (crates/rmlx-core/src/ops/topk_route.rs:433-650) -----------------------
  * gate_logits [T,E] f32 or f16 -> expert_indices u32 [T*K] (descending, ties to the lower
@@ -240,7 +252,7 @@ int32_t rmlx_hip_silu_gate(const void* gate_in_f16_dev, const void* up_in_f16_de
  * packing.  Per item: y = (silu(x Wg^T) * (x Wu^T)) Wd^T with stacked expert weights (the streaming kernels
  * take 4-bit weights with group size 64 or 128 and dimensions in multiples of 512, and 8-bit weights with group size 64
  * and dimensions in multiples of 256; batches with many rows per expert take the grouped MFMA GEMM, see
- * rmlx_hip_set_expert_gemm_min_rows; every other 2- / 4- / 8-bit weight the type admits runs the same block
+ * rmlx_hip_qweight_set_expert_gemm_min_rows; every other 2- / 4- / 8-bit weight the type admits runs the same block
  * on the portable kernels)
  * gate/up [E, I, D] and down [E, D, I].  `up` may be NULL when `gate` holds the fused
  * [E, 2I, D] layout (gate rows first).  expert_idx and batch_sizes are HOST arrays.
@@ -263,16 +275,16 @@ int32_t rmlx_hip_moe_forward_grouped(const rmlx_qweight* gate, const rmlx_qweigh
                                      const float* expert_weights_dev, size_t top_k,
                                      void* out_f16_dev, size_t out_bytes, rmlx_stream stream);
 
-/* Kernel choice of the expert projections (ExpertGroup and both MoeLayer entry points): batches with at
- * least `min_rows` rows per expert on average (rows / num_experts; for ExpertGroup rows / n_items) multiply
- * with the grouped MFMA GEMM -- row tiles of 16, 32 or 64 rows of one expert, weights dequantised in registers;
- * 4- / 8-bit, group sizes 32 / 64 / 128 (one for the three projections), hidden and intermediate dimensions
- * in multiples of 512 -- smaller ones with the streaming GEMV, which reads an expert's weights once per 8
- * rows (8-bit experts switch at an eighth of `min_rows`, rounded up).  gather_qmm does the same from one and a half times as many rows per batch entry on (4-bit, group
- * sizes 32 / 64 / 128, N % 128 == 0, K % 512 == 0).  0 = never the GEMM.  The default (6) is the measured
- * crossover; the setting is process-wide.  No counterpart in the reference, whose MoE layer picks its
- * kernels by a configured `MoeStrategy` (crates/rmlx-nn/src/moe.rs:515-541).  Returns the previous value. */
-uint32_t rmlx_hip_set_expert_gemm_min_rows(uint32_t min_rows);
+/* Kernel choice of the expert projections (ExpertGroup and the MoeLayer entry points): batches with at least
+ * `min_rows` rows per expert on average (rows / num_experts; for ExpertGroup rows / n_items) multiply with the
+ * grouped MFMA GEMM -- row tiles of 16, 32 or 64 rows of one expert, weights dequantised in registers; 4- / 8-bit,
+ * group sizes 32 / 64 / 128 (one for the three projections), hidden and intermediate dimensions in multiples of
+ * 512 -- smaller ones with the streaming GEMV, which reads an expert's weights once per 8 rows (8-bit experts
+ * switch at an eighth of `min_rows`, rounded up).  0 = never the GEMM; the default (6) is the measured crossover.
+ * The value lives in the handle of the stacked GATE weight and applies to the calls that pass that handle: there
+ * is no process-wide state.  Set it before other threads use the handle.  The counterpart of choosing a
+ * `MoeStrategy` for a layer in the reference (crates/rmlx-nn/src/moe.rs:515-541).  Returns the previous value. */
+uint32_t rmlx_hip_qweight_set_expert_gemm_min_rows(rmlx_qweight* gate_qw, uint32_t min_rows);
 
 /* Routing + the block above in one call: gate_logits [T,E] (the router's output). */
 int32_t rmlx_hip_moe_forward(const rmlx_qweight* gate, const rmlx_qweight* up,

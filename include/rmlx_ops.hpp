@@ -173,6 +173,7 @@ class QuantizedWeight {
   QuantizedWeight(const QuantizedWeight&) = delete;
   QuantizedWeight& operator=(const QuantizedWeight&) = delete;
   const rmlx_qweight* handle() const { return handle_; }
+  uint32_t set_expert_gemm_min_rows(uint32_t min_rows) const { return rmlx_hip_qweight_set_expert_gemm_min_rows(handle_, min_rows); }
 
   std::shared_ptr<Buffer> weights_buf, scales_buf, biases_buf;
   uint32_t group_size, bits;
@@ -386,9 +387,10 @@ class MoeExperts {
                                                out.nbytes(), raw(stream)));
     return out;
   }
-  // Average rows per expert from which the expert projections (here and in ExpertGroup) run on the grouped
-  // MFMA GEMM instead of the streaming GEMV; 0 = never; process-wide.  Returns the previous value.
-  static uint32_t set_expert_gemm_min_rows(uint32_t min_rows) { return rmlx_hip_set_expert_gemm_min_rows(min_rows); }
+  // Average rows per expert from which the expert projections of this layer run on the grouped MFMA GEMM instead
+  // of the streaming GEMV; 0 = never.  Kept in the gate weight's handle (so an ExpertGroup over the same weights
+  // follows it); returns the previous value.
+  uint32_t set_expert_gemm_min_rows(uint32_t min_rows) { return gate_->set_expert_gemm_min_rows(min_rows); }
   // routing included: gate_logits [T, E]
   Array forward(const Array& x, const Array& gate_logits, size_t top_k, const Array* expert_bias = nullptr,
                 const Stream* stream = nullptr) const {

@@ -1,7 +1,6 @@
 // Host side of the C ABI: validation (same rules and messages as the reference's Rust entry
 // points), the dispatch ladder, and the composition of the MoE block.  No arithmetic happens
 // here and there is no CPU fallback: every path ends in a HIP kernel launch or an error.
-#include <atomic>
 #include <cinttypes>
 #include <cstring>
 #include <map>
@@ -353,11 +352,13 @@ struct ExpertShapes {
   bool gemm;      // the grouped GEMM takes them too (batches with many rows per expert)
   uint32_t bits;  // of the gate weight
   bool gemm64;    // group size 64 (the 16-row tile is built for it only)
+  uint32_t gemm_min_rows;  // of the gate weight's handle (rmlx_hip_qweight_set_expert_gemm_min_rows)
 };
 
-// Average rows per expert from which the expert projections run on the grouped GEMM instead of the streaming
-// GEMV (which re-reads an expert's weights once per 8 rows); 0 = never.  Measured crossover.
-std::atomic<uint32_t> g_expert_gemm_min_rows{6};
+// gather_qmm takes raw buffers, so its GEMV / grouped-GEMM crossover is a constant: every entry has exactly
+// m_per_batch rows, the streaming GEMV wastes nothing up to a full chunk of 8 rows, and the GEMM wins from 9 rows on.
+constexpr uint32_t kGatherGemmMinRows = 9;
+enum { GATHER_AUTO = 0, GATHER_STREAM = 1, GATHER_GEMM = 2, GATHER_PORTABLE = 3 };
 
 int32_t check_expert_weights(const char* who, const rmlx_qweight* gate, const rmlx_qweight* up,
                              const rmlx_qweight* down, ExpertShapes* sh) {
@@ -395,6 +396,7 @@ int32_t check_expert_weights(const char* who, const rmlx_qweight* gate, const rm
   sh->fused = fused;
   sh->bits = gate->bits;
   sh->gemm64 = gate->group_size == 64;
+  sh->gemm_min_rows = gate->expert_gemm_min_rows;
   sh->portable = !fast;
   // the grouped GEMM also takes group sizes the streaming kernels do not (32; 128 at 8 bits)
   sh->gemm = uniform && qmm_rw_grouped_supported(sh->I, sh->D, gate->group_size, gate->bits) &&
@@ -405,7 +407,7 @@ int32_t check_expert_weights(const char* who, const rmlx_qweight* gate, const rm
 // Rows per tile when `rows` positions over at most `groups` experts are multiplied by the grouped GEMM (half
 // tiles while an expert has 24 rows or fewer on average: less padding, more workgroups per CU), else 0
 uint32_t expert_gemm_tile_rows(const ExpertShapes& sh, uint64_t rows, uint64_t groups) {
-  uint32_t min_rows = g_expert_gemm_min_rows.load(std::memory_order_relaxed);
+  uint32_t min_rows = sh.gemm_min_rows;
   // 8-bit experts cross over at an eighth of the threshold (measured: from one row per expert on, against 6 for
   // 4-bit ones: with 16-row tiles the GEMM streams 8-bit weights faster than the 8-bit GEMV does)
   if (sh.bits == 8 && min_rows != 0) min_rows = (min_rows + 7) / 8;
@@ -837,12 +839,13 @@ int32_t rmlx_hip_quantized_linear_forward(const rmlx_qweight* qw, const rmlx_arr
 
 // ---- gather_qmm -----------------------------------------------------------------------------------
 
-int32_t rmlx_hip_gather_qmm(const rmlx_array* x, const void* w_packed_dev, size_t w_bytes, const void* scales_dev,
-                            size_t scales_bytes, const void* biases_dev, size_t biases_bytes,
-                            const rmlx_array* indices, size_t batch, size_t m_per_batch, size_t n, size_t k,
-                            size_t n_experts, uint32_t group_size, void* out_f16_dev, size_t out_bytes,
-                            rmlx_stream stream) {
+int32_t rmlx_hip_gather_qmm_select(const rmlx_array* x, const void* w_packed_dev, size_t w_bytes, const void* scales_dev,
+                                   size_t scales_bytes, const void* biases_dev, size_t biases_bytes,
+                                   const rmlx_array* indices, size_t batch, size_t m_per_batch, size_t n, size_t k,
+                                   size_t n_experts, uint32_t group_size, int32_t kernel, void* out_f16_dev,
+                                   size_t out_bytes, rmlx_stream stream) {
   RMLX_TRY(require_init());
+  if (kernel < GATHER_AUTO || kernel > GATHER_PORTABLE) return fail(RMLX_NOT_FOUND, "gather_qmm: unknown kernel selector %d", kernel);
   if (x == nullptr || indices == nullptr) return fail(RMLX_INVALID_SHAPE, "gather_qmm: null argument");
   if (x->dtype != RMLX_DTYPE_F32 && x->dtype != RMLX_DTYPE_F16)
     return fail(RMLX_INVALID_SHAPE, "gather_qmm requires Float32 or Float16 input x, got %s", dtype_name(x->dtype));
@@ -907,13 +910,14 @@ int32_t rmlx_hip_gather_qmm(const rmlx_array* x, const void* w_packed_dev, size_
   const __half* bi = static_cast<const __half*>(biases_dev);
   const bool fast = qmv_q4_supported(N32, K32, group_size) && aligned16(w) && aligned16(sc) &&
                     aligned16(bi) && aligned16(xk);
-  const uint32_t gemm_min_rows = g_expert_gemm_min_rows.load(std::memory_order_relaxed);
-  // Every entry has exactly m_per_batch rows, so the streaming GEMV wastes nothing up to a full chunk of 8 rows
-  // and the crossover lies higher than for routed batches: one and a half times the threshold, i.e. from 9 rows
-  // on, where the GEMV needs a second pass (measured, 32 entries over 3072 x 4096 weights: 8 rows 50 us streamed;
-  // 12 / 16 / 32 rows 61 / 64 / 76 us on the GEMM with 16- / 32-row tiles against 95 / 99 / 172 us streamed).
-  if (gemm_min_rows != 0 && m_per_batch >= gemm_min_rows + gemm_min_rows / 2 && aligned16(w) && aligned16(sc) &&
-      aligned16(bi) && aligned16(xk) && qmm_rw_grouped_supported(N32, K32, group_size, 4)) {
+  // (measured, 32 entries over 3072 x 4096 weights: 8 rows 50 us streamed; 12 / 16 / 32 rows 61 / 64 / 76 us on the GEMM
+  // with 16- / 32-row tiles against 95 / 99 / 172 us streamed)
+  const bool can_gemm = aligned16(w) && aligned16(sc) && aligned16(bi) && aligned16(xk) &&
+                        qmm_rw_grouped_supported(N32, K32, group_size, 4);
+  if ((kernel == GATHER_GEMM && !can_gemm) || (kernel == GATHER_STREAM && !fast))
+    return fail(RMLX_INVALID_SHAPE, "gather_qmm: the selected kernel does not take N=%u K=%u group_size=%u (or a buffer is not 16-byte aligned)",
+                N32, K32, group_size);
+  if (kernel == GATHER_GEMM || (kernel == GATHER_AUTO && can_gemm && m_per_batch >= kGatherGemmMinRows)) {
     // many rows per entry: row tiles of one expert each on the grouped MFMA GEMM
     const uint32_t tile_rows = m_per_batch <= 16 && group_size == 64 ? 16u : (m_per_batch <= 32 ? 32u : kGroupedTileRows);
     const uint32_t per = ((uint32_t)m_per_batch + tile_rows - 1) / tile_rows;
@@ -931,9 +935,9 @@ int32_t rmlx_hip_gather_qmm(const rmlx_array* x, const void* w_packed_dev, size_
     a.x = xk; a.out = out_f16_dev;
     a.tile_tab = t; a.n_tiles_dev = t + 3 * n_tiles; a.max_tiles = (uint32_t)n_tiles; a.tile_rows = tile_rows;
     RMLX_TRY(launch_qmm_rw_grouped(a, s));
-  } else if (fast) {
-    const uint32_t per = ((uint32_t)m_per_batch + 7) / 8, n_chunks = B32 * per;
-    if (n_chunks > 65535) return fail(RMLX_INVALID_SHAPE, "gather_qmm: too many row chunks (%u)", n_chunks);
+  } else if (fast && kernel != GATHER_PORTABLE) {
+    const uint64_t per = ((uint64_t)m_per_batch + 7) / 8, n_chunks = (uint64_t)B32 * per;
+    if (n_chunks > 0x7FFFFFFFull) return fail(RMLX_INVALID_SHAPE, "gather_qmm: too many row chunks (%" PRIu64 ")", n_chunks);
     Scratch tab;
     RMLX_TRY(tab.alloc((size_t)n_chunks * 12, s));
     RMLX_TRY(launch_build_gather_chunks(idx, B32, (uint32_t)m_per_batch, E32, 8, static_cast<uint32_t*>(tab.ptr), nullptr, s));
@@ -943,16 +947,30 @@ int32_t rmlx_hip_gather_qmm(const rmlx_array* x, const void* w_packed_dev, size_
     a.expert_stride_w = (uint64_t)n * (k / 8);
     a.expert_stride_s = (uint64_t)n * gpr;
     a.x = xk; a.out = out_f16_dev; a.ld_out = N32;
-    a.chunk_tab = static_cast<const uint32_t*>(tab.ptr); a.max_chunks = n_chunks;
     a.mr = m_per_batch >= 5 ? 8 : (m_per_batch >= 3 ? 4 : (m_per_batch == 2 ? 2 : 1));
     a.group_size = group_size;
-    RMLX_TRY(launch_qmv_q4(a, s));
+    // a launch takes at most 65535 chunks (the chunk index is the second grid dimension); the table's entries
+    // name absolute rows, so a longer table is simply walked in pieces
+    for (uint64_t first = 0; first < n_chunks; first += 65535) {
+      a.chunk_tab = static_cast<const uint32_t*>(tab.ptr) + 3 * first;
+      a.max_chunks = (uint32_t)(n_chunks - first < 65535 ? n_chunks - first : 65535);
+      RMLX_TRY(launch_qmv_q4(a, s));
+    }
   } else {
     GenericArgs g{w, sc, bi, xk, static_cast<__half*>(out_f16_dev), idx, (uint32_t)m_per_batch, rows, N32, K32,
                   group_size, 4, E32};
     RMLX_TRY(launch_generic(g, s));
   }
   return finish(s);
+}
+
+int32_t rmlx_hip_gather_qmm(const rmlx_array* x, const void* w_packed_dev, size_t w_bytes, const void* scales_dev,
+                            size_t scales_bytes, const void* biases_dev, size_t biases_bytes,
+                            const rmlx_array* indices, size_t batch, size_t m_per_batch, size_t n, size_t k,
+                            size_t n_experts, uint32_t group_size, void* out_f16_dev, size_t out_bytes,
+                            rmlx_stream stream) {
+  return rmlx_hip_gather_qmm_select(x, w_packed_dev, w_bytes, scales_dev, scales_bytes, biases_dev, biases_bytes, indices,
+                                    batch, m_per_batch, n, k, n_experts, group_size, GATHER_AUTO, out_f16_dev, out_bytes, stream);
 }
 
 // ---- routing / grouping / data movement ----------------------------------------------------------------
@@ -1230,8 +1248,11 @@ int32_t moe_grouped_impl(const rmlx_qweight* gate, const rmlx_qweight* up, const
 
 extern "C" {
 
-uint32_t rmlx_hip_set_expert_gemm_min_rows(uint32_t min_rows) {
-  return g_expert_gemm_min_rows.exchange(min_rows, std::memory_order_relaxed);
+uint32_t rmlx_hip_qweight_set_expert_gemm_min_rows(rmlx_qweight* qw, uint32_t min_rows) {
+  if (qw == nullptr) return 0;
+  const uint32_t prev = qw->expert_gemm_min_rows;
+  qw->expert_gemm_min_rows = min_rows;
+  return prev;
 }
 
 int32_t rmlx_hip_moe_forward_grouped(const rmlx_qweight* gate, const rmlx_qweight* up, const rmlx_qweight* down,

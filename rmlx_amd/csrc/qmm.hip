@@ -35,20 +35,8 @@ struct QmmParams {
   const uint16_t* x;  // f16 or bf16 bits in fragment-major layout (see relayout_a_kernel)
   __half* out;
   uint32_t M, N, K;
-#ifdef QMM_TRACE
-  unsigned long long* trace;  // development only: shader clock at a few points of the first steps
-#endif
 };
 
-#ifdef QMM_TRACE
-#define QMM_MARK(p, step, i)                                                                     \
-  do {                                                                                           \
-    if ((p).trace != nullptr && blockIdx.x == 0 && (threadIdx.x & 63) == 0 && (step) >= 8 && (step) < 12) \
-      (p).trace[((threadIdx.x >> 6) * 4 + ((step) - 8)) * 8 + (i)] = __builtin_readcyclecounter(); \
-  } while (0)
-#else
-#define QMM_MARK(p, step, i) do {} while (0)
-#endif
 
 __device__ __forceinline__ uint32_t h2bits(h2 v) { return __builtin_bit_cast(uint32_t, v); }
 
@@ -235,7 +223,6 @@ __global__ __launch_bounds__(kThreads) void qmm_kernel(QmmParams p) {
 #pragma unroll
     for (int d = 0; d < kDepth; ++d) {
       const int step = step0 + d;
-      QMM_MARK(p, step, 0);
       // fragments of the next step (its tile was written during the previous step)
       read_frags((d + 1) & 3, bf[(d + 1) & 1]);
       // tile of step+2: weights sit in ring slot (d+2)&3, their group is step+2
@@ -272,9 +259,7 @@ __global__ __launch_bounds__(kThreads) void qmm_kernel(QmmParams p) {
         if (q >= KK * TI * TJ / 2) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
         if (q == KK * TI * TJ / 2 || q == KK * TI * TJ / 2 + 1) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
       }
-      QMM_MARK(p, step, 3);
       __syncthreads();
-      QMM_MARK(p, step, 4);
     }
     sb_cur[0] = sb_next[0]; sb_cur[1] = sb_next[1];
     sb_next[0] = sb_nn[0]; sb_next[1] = sb_nn[1];
@@ -360,9 +345,6 @@ void launch_t(const QmmParams& p, hipStream_t s) {
 
 }  // namespace
 
-#ifdef QMM_TRACE
-unsigned long long* g_qmm_trace = nullptr;
-#endif
 
 bool qmm_supported(uint32_t N, uint32_t K, uint32_t group_size, uint32_t bits) {
   return group_size == 64 && (bits == 4 || bits == 8) && N % 64 == 0 && K % (BK * kDepth) == 0 && N > 0 && K > 0;
@@ -384,9 +366,6 @@ int32_t launch_qmm(const QmmArgs& a, hipStream_t s) {
                        reinterpret_cast<u4*>(a.workspace), a.M, a.K, want_bf16 ? 1 : 0);
   }
   QmmParams p{a.w, a.s, a.b, reinterpret_cast<const uint16_t*>(a.workspace), a.out, a.M, a.N, a.K};
-#ifdef QMM_TRACE
-  p.trace = g_qmm_trace;
-#endif
   // 128-row tiles only when they still give (most of) the CUs a workgroup
   const uint32_t tiles128 = ((a.M + 127) / 128) * (a.N / 64);
   const bool big = a.M > 64 && tiles128 * 4 >= (uint32_t)ctx().num_cus * 3;

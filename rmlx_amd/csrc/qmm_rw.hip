@@ -60,29 +60,7 @@ struct RwParams {
   uint64_t estride_w, estride_s;
   const uint32_t* w1; const __half* s1; const __half* b1;
   int32_t out_f32;
-#ifdef QMM_RW_TRACE
-  unsigned long long* trace;
-#endif
 };
-
-#ifdef QMM_RW_TRACE
-#ifndef RW_TRACE_WG
-#define RW_TRACE_WG 0
-#endif
-#define RW_MARK(p, it, i)                                                                          \
-  do {                                                                                             \
-    if ((p).trace != nullptr && blockIdx.x == RW_TRACE_WG && (threadIdx.x & 63) == 0 && (it) >= 8 && (it) < 12) \
-      (p).trace[((threadIdx.x >> 6) * 4 + ((it) - 8)) * 8 + (i)] = __builtin_readcyclecounter();    \
-  } while (0)
-#define RW_MARK_ALL(p, i)                                                              \
-  do {                                                                                 \
-    if ((p).trace != nullptr && threadIdx.x == 0)                                      \
-      (p).trace[1024 + blockIdx.x * 2 + (i)] = __builtin_readcyclecounter();            \
-  } while (0)
-#else
-#define RW_MARK(p, it, i) do {} while (0)
-#define RW_MARK_ALL(p, i) do {} while (0)
-#endif
 
 __device__ __forceinline__ uint32_t h2bits(h2 v) { return __builtin_bit_cast(uint32_t, v); }
 
@@ -141,8 +119,6 @@ __device__ __forceinline__ void qmm_rw_body(const RwParams p) {  // by value: a 
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int n = lane & 15, g = lane >> 4;
-  RW_MARK(p, 8, 6);
-  RW_MARK_ALL(p, 0);
 
   // Workgroup -> tile.  Consecutive workgroup ids go round-robin over the 8 XCDs (one L2 each), so
   // XCD x = id % 8 runs the ids congruent to x.  Give every XCD a compact block of tiles, half of
@@ -280,10 +256,6 @@ __device__ __forceinline__ void qmm_rw_body(const RwParams p) {  // by value: a 
   auto load_sb = [&](uint32_t blk, u4 (&ds)[NF][kSbVecs], u4 (&db)[NF][kSbVecs]) {
 #pragma unroll
     for (int f = 0; f < NF; ++f) {
-#if defined(QMM_RW_EXP) && (QMM_RW_EXP & 16)
-      ds[f][0] = (u4){0x20002000u + blk, 0x20002000u, 0x20012001u, 0x20002000u};
-      db[f][0] = (u4){0xa000a000u + blk, 0xa000a000u, 0xa001a001u, 0xa000a000u};
-#else
       if (GS == 128) {  // 4 groups = 8 bytes per row and four iterations
         const u2 sv = reinterpret_cast<const u2*>(sptr[f])[blk], bv = reinterpret_cast<const u2*>(bptr[f])[blk];
         ds[f][0] = (u4){sv.x, sv.y, 0u, 0u};
@@ -295,7 +267,6 @@ __device__ __forceinline__ void qmm_rw_body(const RwParams p) {  // by value: a 
           db[f][v] = reinterpret_cast<const u4*>(bptr[f])[blk * kSbVecs + v];
         }
       }
-#endif
     }
   };
   auto load_w = [&](uint32_t it, u4 (&dst)[NF][WL]) {
@@ -303,11 +274,7 @@ __device__ __forceinline__ void qmm_rw_body(const RwParams p) {  // by value: a 
     for (int f = 0; f < NF; ++f)
 #pragma unroll
       for (int h = 0; h < WL; ++h) {
-#if defined(QMM_RW_EXP) && (QMM_RW_EXP & 8)
-        dst[f][h] = (u4){it * 3u + f, (uint32_t)lane, it, (uint32_t)h};
-#else
         dst[f][h] = wptr[f][(uint64_t)it * (4 * WL) + h * 4];
-#endif
       }
   };
   const uint32_t last = S - 1, last_blk = S / kUnroll - 1;
@@ -356,9 +323,6 @@ __device__ __forceinline__ void qmm_rw_body(const RwParams p) {  // by value: a 
       const u4 q = wq[u % kUnroll][f][0];
       const uint32_t word = j == 0 ? q.x : (j == 1 ? q.y : (j == 2 ? q.z : q.w));
       scale_pair(u, f, 0, s2, b2);
-#if defined(QMM_RW_EXP) && (QMM_RW_EXP & 1)
-      return __builtin_bit_cast(h8, (u4){word, word ^ h2bits(s2), word, word ^ h2bits(b2)});
-#endif
       return dequant_q4_word(word, s2, b2, dq);
     } else {
       constexpr int hmax = WL - 1;
@@ -394,7 +358,6 @@ __device__ __forceinline__ void qmm_rw_body(const RwParams p) {  // by value: a 
 #pragma unroll
     for (int u = 0; u < kUnroll; ++u) {
       const uint32_t it = it0 + u;
-      RW_MARK(p, it, 0);
       const u4* a_stage = a_lds + (it % kStages) * kChunk;
       const u4* a_stage_next = a_lds + ((it + 1) % kStages) * kChunk;
       u4* a_stage_write = a_lds + ((it + 2) % kStages) * kChunk;
@@ -406,24 +369,16 @@ __device__ __forceinline__ void qmm_rw_body(const RwParams p) {  // by value: a 
         if (f == 0) {
 #pragma unroll
           for (int i = 0; i < MF; ++i)
-#if defined(QMM_RW_EXP) && (QMM_RW_EXP & 2)
-            a_nxt[i] = __builtin_bit_cast(h8, (u4){(uint32_t)lane, it, (uint32_t)(i + j), 0x3c003c00u});
-#else
             a_nxt[i] = __builtin_bit_cast(h8, j < 3 ? a_stage[i * 256 + lds_r[j < 3 ? j + 1 : 0]] : a_stage_next[i * 256 + lds_r[0]]);
-#endif
         }
         // this step's share of the ring traffic: LDS writes of chunk it+2 in the first half, the
         // global loads of chunk it+4 into the same registers in the second half, weights last
 #pragma unroll
         for (int q = 0; q < AL; ++q) {
-#if defined(QMM_RW_EXP) && (QMM_RW_EXP & 4)
-          if (s == q * NS / (2 * AL) && it == 0xFFFFFFFFu) a_stage_write[lds_w[q]] = ra[u % 2][q];
-#else
           if (s == q * NS / (2 * AL)) a_stage_write[lds_w[q]] = to_slot_order(ra[u % 2][q]);
           if (s == NS / 2 + q * NS / (2 * AL)) {
             ra[u % 2][q] = *reinterpret_cast<const u4*>(xsrc[q] + (uint64_t)clampi(it + 4) * kBlockK);
           }
-#endif
         }
         // next weight operand (the one of the first step of the next iteration after the last step)
         if (s + 1 < NS) wv_nxt = weight_operand(u, (s + 1) / NF, (s + 1) % NF);
@@ -439,11 +394,7 @@ __device__ __forceinline__ void qmm_rw_body(const RwParams p) {  // by value: a 
         wv_cur = wv_nxt;
         __builtin_amdgcn_sched_barrier(0);
       }
-      RW_MARK(p, it, 4);
-#if !(defined(QMM_RW_EXP) && (QMM_RW_EXP & 32))
       __syncthreads();
-#endif
-      RW_MARK(p, it, 5);
     }
 #pragma unroll
     for (int f = 0; f < NF; ++f)
@@ -499,8 +450,6 @@ __device__ __forceinline__ void qmm_rw_body(const RwParams p) {  // by value: a 
       }
     }
   }
-  RW_MARK(p, 8, 7);
-  RW_MARK_ALL(p, 1);
 }
 
 template <int MF, int NF, int BITS, int NW, bool XBF16, int GS>
@@ -548,11 +497,6 @@ void launch_rw(RwParams p, bool x_bf16, hipStream_t s) {
 }
 
 }  // namespace
-
-#ifdef QMM_RW_TRACE
-unsigned long long* g_qmm_rw_trace = nullptr;
-int g_qmm_rw_force_mf = 0, g_qmm_rw_force_nf = 0, g_qmm_rw_force_nw = 4, g_qmm_rw_force_ks = 0;
-#endif
 
 bool qmm_rw_supported(uint32_t N, uint32_t K, uint32_t group_size, uint32_t bits) {
   return (group_size == 32 || group_size == 64 || group_size == 128) && (bits == 4 || bits == 8) && N > 0 && K > 0 && N % 64 == 0 &&
@@ -614,10 +558,6 @@ int32_t launch_qmm_rw(const QmmArgs& a, uint32_t group_size, hipStream_t s) {
   const bool x_bf16 = a.x_dtype == RMLX_DTYPE_BF16;
   RwPlan plan = plan_rw(a.M, a.N, a.K, group_size);
   if (a.workspace == nullptr) plan.ksplit = 1;  // no room for partial sums: one workgroup per tile
-#ifdef QMM_RW_TRACE
-  if (g_qmm_rw_force_mf) { plan.mf = g_qmm_rw_force_mf; plan.nf = g_qmm_rw_force_nf; plan.nw = g_qmm_rw_force_nw; }
-  if (g_qmm_rw_force_ks) plan.ksplit = (uint32_t)g_qmm_rw_force_ks;
-#endif
   const int mf = plan.mf, nf = plan.nf, nw = plan.nw;
   RwParams p{};
   p.w = a.w; p.s = a.s; p.b = a.b;
@@ -625,9 +565,6 @@ int32_t launch_qmm_rw(const QmmArgs& a, uint32_t group_size, hipStream_t s) {
   p.out = a.out; p.M = a.M; p.N = a.N; p.K = a.K;
   p.epi_kind = a.epi_kind; p.epi = a.epi; p.epi_dtype = a.epi_dtype;
   p.ksplit = plan.ksplit; p.partial = static_cast<float*>(a.workspace);
-#ifdef QMM_RW_TRACE
-  p.trace = g_qmm_rw_trace;
-#endif
 #define RW_CASE(MFV, NFV, NWV)                                                                 \
   if (mf == MFV && nf == NFV && nw == NWV) {                                                   \
     if (a.bits == 4) launch_rw<MFV, NFV, 4, NWV>(p, x_bf16, s); else launch_rw<MFV, NFV, 8, NWV>(p, x_bf16, s); \

@@ -61,20 +61,8 @@ struct KParams {
   const uint32_t* chunk_tab;
   const uint32_t* n_chunks;
   uint64_t estride_w, estride_s;
-#ifdef QMV_TRACE
-  unsigned long long* trace;  // development only: per-phase shader clock of workgroup 0 / each wave
-#endif
 };
 
-#ifdef QMV_TRACE
-#define QMV_MARK(p, i)                                                                   \
-  do {                                                                                   \
-    if ((p).trace != nullptr && blockIdx.x == 0 && blockIdx.y == 0 && (threadIdx.x & 63) == 0) \
-      (p).trace[(threadIdx.x >> 6) * 16 + (i)] = __builtin_readcyclecounter();           \
-  } while (0)
-#else
-#define QMV_MARK(p, i) do {} while (0)
-#endif
 
 __device__ __forceinline__ h8 unpack_q4_word(uint32_t w) {
   uint32_t t = w >> 8;
@@ -174,7 +162,6 @@ __global__ __launch_bounds__(kThreads, (REUSE && MR == 8 && TILES == 2) ? 4 : 1)
   const u4 bconst_bits = n < 8 ? (u4){0x64006400u, 0x54005400u, 0x64006400u, 0x54005400u}
                                : (u4){0x3C003C00u, 0x3C003C00u, 0x3C003C00u, 0x3C003C00u};
   const h8 bconst = __builtin_bit_cast(h8, bconst_bits);
-  QMV_MARK(p, 0);
 
   // activations of a pass: lane l of the wave loads 8 consecutive k of every row (slabs sl .. sl+my-1)
   auto load_x = [&](int sl, int my, u4 (&xv)[MR]) {
@@ -292,10 +279,8 @@ __global__ __launch_bounds__(kThreads, (REUSE && MR == 8 && TILES == 2) ? 4 : 1)
         for (int t = 0; t < TILES; ++t) wreg[t][it] = *(wrow[t] + (sl + it) * 4);
       }
     }
-    QMV_MARK(p, 1);
 
     if constexpr (!REUSE) stage_x(xv);
-    QMV_MARK(p, 2);
 
     // ---- 2b/3 for 8 rows: slab by slab (few live registers).  The per (row, group) sums of the
     //          activations come from the matrix unit: columns 0-7 of a constant B operand hold the
@@ -391,14 +376,11 @@ __global__ __launch_bounds__(kThreads, (REUSE && MR == 8 && TILES == 2) ? 4 : 1)
         }
       }
     }
-    QMV_MARK(p, 4);
   }
 
   // ---- 4. reduce over the two group halves (lane + 32 holds the other one) and over the
   //         k-parts, write out -------------------------------------------------------------------
-  QMV_MARK(p, 5);
   __syncthreads();  // the previous tile's sums have been read
-  QMV_MARK(p, 6);
   // (index arithmetic of this part is kept inside the tile loop on purpose: hoisted out, it
   // costs registers for the whole kernel)
   uint32_t tid_t = tid;
@@ -414,7 +396,6 @@ __global__ __launch_bounds__(kThreads, (REUSE && MR == 8 && TILES == 2) ? 4 : 1)
       }
   }
   __syncthreads();
-  QMV_MARK(p, 7);
   for (uint32_t o = tid_t; o < NT * 128; o += kThreads) {
     const uint32_t otw = o >> 7, m = (o >> 4) & 7, nn = o & 15;
     if (m < rows) {
@@ -438,7 +419,6 @@ __global__ __launch_bounds__(kThreads, (REUSE && MR == 8 && TILES == 2) ? 4 : 1)
     }
   }
   }  // tiles of this workgroup
-  QMV_MARK(p, 8);
 }
 
 template <int MR, int TILES, int SPW, bool PAIR>
@@ -494,9 +474,6 @@ int32_t launch_build_gather_chunks(const uint32_t* indices, uint32_t batch, uint
   return RMLX_OK;
 }
 
-#ifdef QMV_TRACE
-unsigned long long* g_qmv_trace = nullptr;
-#endif
 
 bool qmv_q4_supported(uint32_t N, uint32_t K, uint32_t group_size) {
   return (group_size == 64 || group_size == 128) && N % 16 == 0 && K % 512 == 0 && N > 0 && K > 0;
@@ -511,9 +488,6 @@ int32_t launch_qmv_q4(const QmvArgs& a, hipStream_t s) {
   p.out = a.out; p.estride_w = a.expert_stride_w; p.estride_s = a.expert_stride_s;
   p.K = a.K; p.ld_out = a.ld_out; p.M = a.M; p.out_f32 = a.out_f32;
   p.gs128 = a.group_size == 128 ? 1u : 0u;
-#ifdef QMV_TRACE
-  p.trace = g_qmv_trace;
-#endif
   const bool tab = a.chunk_tab != nullptr;
   uint32_t chunks = tab ? a.max_chunks : (a.M + 7) / 8;
   if (chunks == 0) return RMLX_OK;

@@ -40,6 +40,11 @@ class QuantizedWeight:
         return cls(DeviceBuffer.from_numpy(words), DeviceBuffer.from_numpy(np.ascontiguousarray(scales, np.float16)),
                    DeviceBuffer.from_numpy(np.ascontiguousarray(biases, np.float16)), group_size, bits, n, k, e)
 
+    def set_expert_gemm_min_rows(self, min_rows):
+        """(stacked gate weight) average rows per expert from which the expert projections of the blocks that use
+        this handle run on the grouped MFMA GEMM instead of the streaming GEMV (0 = never).  Returns the previous value."""
+        return int(rt.lib().rmlx_hip_qweight_set_expert_gemm_min_rows(self.handle, int(min_rows)))
+
     def groups_per_row(self):
         return self.in_features // self.group_size
 
@@ -147,15 +152,16 @@ class QuantizedLinear:
 
 
 def gather_qmm(x, w_packed_buf, scales_buf, biases_buf, indices, batch, m_per_batch, n, k, n_experts, group_size,
-               stream=None, out=None):
-    """gather_qmm (quantized.rs:9404-9599): out[b] = x[b] @ dequant(W[indices[b]])^T, f16 out."""
+               stream=None, out=None, kernel=0):
+    """gather_qmm (quantized.rs:9404-9599): out[b] = x[b] @ dequant(W[indices[b]])^T, f16 out.  `kernel` forces a
+    family (runtime.GATHER_*)."""
     if out is None:
         out = DeviceBuffer((batch, m_per_batch, n), F16)
     xa, ia = x.array(), indices.array()
-    rt.check(rt.lib().rmlx_hip_gather_qmm(ctypes.byref(xa), w_packed_buf.ptr, w_packed_buf.nbytes, scales_buf.ptr,
-                                          scales_buf.nbytes, biases_buf.ptr, biases_buf.nbytes, ctypes.byref(ia),
-                                          batch, m_per_batch, n, k, n_experts, group_size, out.ptr, out.nbytes,
-                                          _h(stream)))
+    rt.check(rt.lib().rmlx_hip_gather_qmm_select(ctypes.byref(xa), w_packed_buf.ptr, w_packed_buf.nbytes, scales_buf.ptr,
+                                                 scales_buf.nbytes, biases_buf.ptr, biases_buf.nbytes, ctypes.byref(ia),
+                                                 batch, m_per_batch, n, k, n_experts, group_size, kernel, out.ptr,
+                                                 out.nbytes, _h(stream)))
     return out
 
 
@@ -268,12 +274,6 @@ class ExpertGroup:
             res.append((int(e), host[row:row + int(sz)]))
             row += int(sz)
         return res
-
-
-def set_expert_gemm_min_rows(min_rows):
-    """Average rows per expert from which the expert projections run on the grouped MFMA GEMM instead of the
-    streaming GEMV (0 = never; process-wide).  Returns the previous value."""
-    return int(rt.lib().rmlx_hip_set_expert_gemm_min_rows(int(min_rows)))
 
 
 def moe_forward_grouped(gate, up, down, x, expert_indices, expert_weights, top_k, stream=None, out=None):

@@ -16,6 +16,7 @@ OK, INVALID_SHAPE, NOT_FOUND, RUNTIME_ERROR = 0, 1, 2, 3
 F32, F16, BF16, U32, U8 = 0, 1, 2, 3, 4
 KERNEL_AUTO, KERNEL_QMV, KERNEL_QMM, KERNEL_GENERIC, KERNEL_QMM_BF16, KERNEL_QMM_LDS, KERNEL_QMV_ROWS = 0, 1, 2, 3, 4, 5, 6
 KERNEL_QMM_K2, KERNEL_QMM_RW = 7, 8
+GATHER_AUTO, GATHER_STREAM, GATHER_GEMM, GATHER_PORTABLE = 0, 1, 2, 3  # rmlx_hip_gather_qmm_select kernels
 FLOOR_EMPTY, FLOOR_READ4, FLOOR_READ8, FLOOR_MFMA, FLOOR_READ2 = 0, 1, 2, 3, 4  # rmlx_hip_measure_floor kinds
 
 
@@ -43,7 +44,7 @@ EXPORTS = [
     "rmlx_hip_gather_qmm", "rmlx_hip_topk_route", "rmlx_hip_moe_sort", "rmlx_hip_index_gather",
     "rmlx_hip_scatter_weighted_add", "rmlx_hip_silu_gate", "rmlx_hip_expert_group_grouped_forward",
     "rmlx_hip_moe_forward_grouped", "rmlx_hip_moe_forward", "rmlx_hip_moe_forward_noalloc", "rmlx_hip_awq_dequant", "rmlx_hip_gptq_dequant",
-    "rmlx_hip_qmm_norm", "rmlx_hip_set_expert_gemm_min_rows", "rmlx_hip_measure_floor",
+    "rmlx_hip_qmm_norm", "rmlx_hip_qweight_set_expert_gemm_min_rows", "rmlx_hip_gather_qmm_select", "rmlx_hip_measure_floor",
 ]
 
 _lib = None
@@ -91,6 +92,7 @@ def lib():
         "rmlx_hip_qmm_encode_many": [ctypes.POINTER(vp), sz, arr, ctypes.POINTER(vp), sz, sz, sz, i32, vp],
         "rmlx_hip_quantized_linear_forward": [vp, arr, vp, vp, sz, vp],
         "rmlx_hip_gather_qmm": [arr, vp, sz, vp, sz, vp, sz, arr, sz, sz, sz, sz, sz, u32, vp, sz, vp],
+        "rmlx_hip_gather_qmm_select": [arr, vp, sz, vp, sz, vp, sz, arr, sz, sz, sz, sz, sz, u32, i32, vp, sz, vp],
         "rmlx_hip_topk_route": [arr, sz, arr, i32, vp, vp, vp, vp, vp],
         "rmlx_hip_moe_sort": [vp, sz, sz, vp, vp, vp],
         "rmlx_hip_index_gather": [vp, sz, sz, vp, sz, vp, vp],
@@ -108,8 +110,8 @@ def lib():
         fn = getattr(L, name)
         fn.argtypes = argtypes
         fn.restype = i32
-    L.rmlx_hip_set_expert_gemm_min_rows.argtypes = [u32]
-    L.rmlx_hip_set_expert_gemm_min_rows.restype = u32
+    L.rmlx_hip_qweight_set_expert_gemm_min_rows.argtypes = [vp, u32]
+    L.rmlx_hip_qweight_set_expert_gemm_min_rows.restype = u32
     _lib = L
     return L
 

@@ -67,13 +67,20 @@ def test_qweight_validation_needs_no_gpu():
         L.rmlx_hip_qweight_destroy(h)
 
 
-def test_expert_gemm_threshold_is_plain_host_state():
-    """The GEMV / grouped-GEMM threshold of the expert projections: default 6 rows per expert, set returns the old value."""
-    from rmlx_amd import ops
-    prev = ops.set_expert_gemm_min_rows(5)
+def test_expert_gemm_threshold_lives_in_the_handle():
+    """The GEMV / grouped-GEMM threshold of the expert projections: default 6 rows per expert, per weight handle (no
+    process-wide state), set returns the old value."""
+    from rmlx_amd import runtime as rt
+    L = rt.lib()
+    hs = [ctypes.c_void_p(), ctypes.c_void_p()]
+    for h in hs:
+        assert L.rmlx_hip_qweight_create(ctypes.c_void_p(16), 1 << 20, ctypes.c_void_p(16), 1 << 20, ctypes.c_void_p(16), 1 << 20,
+                                         64, 4, 64, 64, 2, ctypes.byref(h)) == rt.OK
     try:
-        assert prev == 6
-        assert ops.set_expert_gemm_min_rows(0) == 5
-        assert ops.set_expert_gemm_min_rows(prev) == 0
+        assert L.rmlx_hip_qweight_set_expert_gemm_min_rows(hs[0], 5) == 6
+        assert L.rmlx_hip_qweight_set_expert_gemm_min_rows(hs[0], 0) == 5
+        assert L.rmlx_hip_qweight_set_expert_gemm_min_rows(hs[1], 9) == 6  # the other handle kept its default
+        assert L.rmlx_hip_qweight_set_expert_gemm_min_rows(hs[0], 6) == 0
     finally:
-        ops.set_expert_gemm_min_rows(prev)
+        for h in hs:
+            L.rmlx_hip_qweight_destroy(h)

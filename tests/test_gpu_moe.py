@@ -268,7 +268,7 @@ def test_gather_qmm_async_out_of_range_rows_are_zero(hip):
 def test_gather_qmm_many_rows_per_entry_on_the_grouped_gemm(hip, n, k, mpb, gs):
     """From 9 rows per batch entry on, gather_qmm multiplies with the grouped MFMA GEMM (row tiles of 16, 32 or 64 rows
     of one expert; the last tile of an entry ragged).  Against the oracle; on a stream, rows of an out-of-range index are zero."""
-    from rmlx_amd import ops
+    from rmlx_amd import ops, runtime as rt
     from rmlx_amd.runtime import DeviceBuffer, Stream
     rng = np.random.default_rng(n + k + mpb)
     E, batch = 5, 6
@@ -280,12 +280,11 @@ def test_gather_qmm_many_rows_per_entry_on_the_grouped_gemm(hip, n, k, mpb, gs):
     out = ops.gather_qmm(xd, wd, sd, bd, DeviceBuffer.from_numpy(idx), batch, mpb, n, k, E, gs).numpy()
     ref = model.gather_qmm(x, words, s, b, idx, gs)
     assert_close(out, ref, "gather_qmm (GEMM)")
-    prev = ops.set_expert_gemm_min_rows(0)
-    try:
-        out_stream = ops.gather_qmm(xd, wd, sd, bd, DeviceBuffer.from_numpy(idx), batch, mpb, n, k, E, gs).numpy()
-    finally:
-        ops.set_expert_gemm_min_rows(prev)
-    assert_close(out_stream, ref, "gather_qmm (streaming GEMV)")
+    if gs != 32:  # (the streaming GEMV takes group sizes 64 and 128)
+        out_stream = ops.gather_qmm(xd, wd, sd, bd, DeviceBuffer.from_numpy(idx), batch, mpb, n, k, E, gs, kernel=rt.GATHER_STREAM).numpy()
+        assert_close(out_stream, ref, "gather_qmm (streaming GEMV)")
+    out_port = ops.gather_qmm(xd, wd, sd, bd, DeviceBuffer.from_numpy(idx), batch, mpb, n, k, E, gs, kernel=rt.GATHER_PORTABLE).numpy()
+    assert_close(out_port, ref, "gather_qmm (portable)")
     bad = np.array([4, 9, 3, 7, 1, 0], np.uint32)
     st = Stream()
     out = ops.gather_qmm(xd, wd, sd, bd, DeviceBuffer.from_numpy(bad), batch, mpb, n, k, E, gs, stream=st)
@@ -513,7 +512,7 @@ def test_moe_many_rows_per_expert_on_the_grouped_gemm(hip, bits, gs, D, I, fused
     ref = model.moe_forward(x, idx, w, gate, up, down, gs, K, bits=bits)
     xd, idxd, wd = DeviceBuffer.from_numpy(x), DeviceBuffer.from_numpy(idx), DeviceBuffer.from_numpy(w)
     print(f"grouped gemm moe T={T} bits={bits} gs={gs} D={D} I={I} fused={fused} counts={counts.tolist()}", flush=True)
-    prev = ops.set_expert_gemm_min_rows(6)
+    prev = gh.set_expert_gemm_min_rows(6)
     try:
         out_gemm = ops.moe_forward_grouped(gh, uh, dh, xd, idxd, wd, K).numpy()
         assert_close(out_gemm, ref, "moe_forward_grouped (GEMM)")
@@ -526,11 +525,11 @@ def test_moe_many_rows_per_expert_on_the_grouped_gemm(hip, bits, gs, D, I, fused
             ones = np.ones((len(v), 1))
             assert_close(yv, model.moe_forward(v, np.full((len(v), 1), e), ones, gate, up, down, gs, 1, bits=bits),
                          f"ExpertGroup (GEMM) expert {e} rows {len(v)}")
-        ops.set_expert_gemm_min_rows(0)
+        gh.set_expert_gemm_min_rows(0)
         out_stream = ops.moe_forward_grouped(gh, uh, dh, xd, idxd, wd, K).numpy()
         assert_close(out_stream, ref, "moe_forward_grouped (below the threshold)")
     finally:
-        ops.set_expert_gemm_min_rows(prev)
+        gh.set_expert_gemm_min_rows(prev)
 
 
 @pytest.mark.parametrize("E,K,T,x_dtype", [(1, 1, 100, "f16"), (3, 3, 40, "f32"), (2, 1, 129, "f16"), (6, 2, 33, "f32")])
@@ -628,11 +627,11 @@ def test_config5_moe_prefill_sizes(hip, config5, T):
     xd, idxd, wd = DeviceBuffer.from_numpy(x), DeviceBuffer.from_numpy(idx), DeviceBuffer.from_numpy(w)
     print(f"config5 prefill T={T}", flush=True)
     out = ops.moe_forward_grouped(gh, uh, dh, xd, idxd, wd, 8).numpy()
-    prev = ops.set_expert_gemm_min_rows(0)
+    prev = gh.set_expert_gemm_min_rows(0)
     try:
         out_stream = ops.moe_forward_grouped(gh, uh, dh, xd, idxd, wd, 8).numpy()
     finally:
-        ops.set_expert_gemm_min_rows(prev)
+        gh.set_expert_gemm_min_rows(prev)
     ref = model.moe_forward(x, idx, w, gate, up, down, 64, 8)
     assert_close(out, ref, f"config5 T={T} (GEMM)")
     assert_close(out_stream, ref, f"config5 T={T} (streaming)")
@@ -671,8 +670,8 @@ def test_moe_few_rows_per_expert_on_16_row_tiles(hip, bits, E, T, D, I, fused):
     print(f"16-row tiles bits={bits} E={E} T={T} D={D} I={I} fused={fused} counts={counts.tolist()}", flush=True)
     assert_close(ops.moe_forward_grouped(gh, uh, dh, xd, idxd, wd, K).numpy(), ref, "moe_forward_grouped (16-row tiles)")
     assert_close(ops.moe_forward(gh, uh, dh, xd, DeviceBuffer.from_numpy(logits), K).numpy(), ref, "moe_forward (16-row tiles)")
-    prev = ops.set_expert_gemm_min_rows(0)
+    prev = gh.set_expert_gemm_min_rows(0)
     try:
         assert_close(ops.moe_forward_grouped(gh, uh, dh, xd, idxd, wd, K).numpy(), ref, "moe_forward_grouped (streaming)")
     finally:
-        ops.set_expert_gemm_min_rows(prev)
+        gh.set_expert_gemm_min_rows(prev)
