@@ -64,14 +64,26 @@ struct KParams {
 };
 
 
-__device__ __forceinline__ h8 unpack_q4_word(uint32_t w) {
+// The masks and offsets arrive in registers (Q4Consts): with one of each pair in a scalar and one in a vector
+// register, and + or is a single instruction.
+struct Q4Consts { uint32_t m0, m1, k0, k1; };
+__device__ __forceinline__ h8 unpack_q4_word(uint32_t w, const Q4Consts& q) {
   uint32_t t = w >> 8;
   u4 p;
-  p.x = (w & 0x000F000Fu) | 0x64006400u;  // k+0, k+4   (+1024)
-  p.y = (w & 0x00F000F0u) | 0x54005400u;  // k+1, k+5   (+64)
-  p.z = (t & 0x000F000Fu) | 0x64006400u;  // k+2, k+6   (+1024)
-  p.w = (t & 0x00F000F0u) | 0x54005400u;  // k+3, k+7   (+64)
+  p.x = (w & q.m0) | q.k0;  // k+0, k+4   (+1024)
+  p.y = (w & q.m1) | q.k1;  // k+1, k+5   (+64)
+  p.z = (t & q.m0) | q.k0;  // k+2, k+6   (+1024)
+  p.w = (t & q.m1) | q.k1;  // k+3, k+7   (+64)
   return __builtin_bit_cast(h8, p);
+}
+
+// v + (value of lane ^ 32): v_permlane32_swap exchanges the upper half of its first operand with the lower half
+// of its second, so both registers end up holding one half of v in all lanes.  (Written as assembly: through the
+// builtin this compiler reads the first result twice.  The wait states cover a vector write just before.)
+__device__ __forceinline__ float add_other_half(float v) {
+  uint32_t a = __builtin_bit_cast(uint32_t, v), b = a;
+  asm volatile("s_nop 1\n\tv_permlane32_swap_b32_e32 %0, %1" : "+v"(a), "+v"(b));
+  return __builtin_bit_cast(float, a) + __builtin_bit_cast(float, b);
 }
 
 // x halves (k0..k7) -> slot order (0,4,1,5,2,6,3,7), matching unpack_q4_word.
@@ -107,21 +119,22 @@ template <int MR, int TILES, bool TAB, int SPW, bool PAIR, bool REUSE>
 __global__ __launch_bounds__(kThreads, (REUSE && MR == 8 && TILES == 2) ? 4 : 1) void qmv_q4_kernel(KParams p) {
   static_assert(!REUSE || SPW != 0, "reuse needs a uniform slab count");
   static_assert(!PAIR || TILES == 2, "paired tiles need two tile slots");
-  constexpr int kSlots = 4 * MR;                       // 16-byte slots per (slab, j)
-  constexpr int kXsWave = kSpwMax * 4 * kSlots * 16;   // bytes of activation image per wave
+  constexpr int kSlots = 4 * MR;                       // 16-byte activation slots per (slab, j) block ...
+  constexpr int kBlk = kSlots + 1;                     // ... followed by one slot of zeros (read by the lanes whose operand rows are empty)
+  constexpr int kXsWave = kSpwMax * 4 * kBlk * 16;     // bytes of activation image per wave
   __shared__ __attribute__((aligned(16))) char xs_all[kWaves * kXsWave];
   __shared__ float red[kWaves * TILES * 8 * 16];  // cross-wave reduction: [wave][tile][activation row][column]
-  // Activation sums per (row, group): on the matrix unit for 8 rows (see 2b), with lane shuffles
-  // while staging for fewer rows (cheaper there: the extra MFMAs would outweigh ~45 VALU per row).
-  constexpr bool kMfmaSums = MR == 8;
-  __shared__ __attribute__((aligned(16))) float sums_all[kMfmaSums ? 4 : kWaves * kSpwMax * 2 * 8 * 2];  // [wave][group][row][-xoff, xsum]
+  // Activation sums per (row, group) come from the matrix unit (see 2b).  With one pass over K they are computed
+  // once, before the tile loop, and wait in LDS; otherwise every pass computes them beside its products.
+  constexpr bool kPreSums = REUSE;
+  __shared__ __attribute__((aligned(16))) float sums_all[!kPreSums ? 4 : kWaves * kSpwMax * 2 * 8 * 2];  // [wave][group][row][-xoff, xsum]
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int n = lane & 15;   // weight row within the tile / accumulator column
   const int g = lane >> 4;   // k sub-block of the slab / accumulator row group
   const int par = g >> 1;    // which of the slab's two quantisation groups this lane scales
   char* xs = xs_all + wave * kXsWave;
-  float* sums = sums_all + (kMfmaSums ? 0 : wave * (kSpwMax * 2 * 8 * 2));
+  float* sums = sums_all + (!kPreSums ? 0 : wave * (kSpwMax * 2 * 8 * 2));
 
   // ---- which rows -----------------------------------------------------------------------
   uint32_t expert = 0, row0 = blockIdx.y * 8, rows;
@@ -156,7 +169,10 @@ __global__ __launch_bounds__(kThreads, (REUSE && MR == 8 && TILES == 2) ? 4 : 1)
   // A-operand activity: accumulator rows 0-7 take group 0 (g<2), rows 8-15 group 1 (g>=2).
   const int am = n & 7;
   const bool a_active = ((n < 8) == (g < 2)) && (am < MR);
-  const int a_slot_off = (g * MR + am) * 16;
+  const int a_slot_off = (a_active ? g * MR + am : kSlots) * 16;  // the others read the block's zero slot
+  if (lane < kSpwMax * 4) *reinterpret_cast<u4*>(xs + (lane * kBlk + kSlots) * 16) = (u4){0u, 0u, 0u, 0u};
+  Q4Consts qc{0x000F000Fu, 0x00F000F0u, 0x64006400u, 0x54005400u};
+  asm volatile("" : "+s"(qc.m0), "+s"(qc.m1), "+v"(qc.k0), "+v"(qc.k1));
 
   // constant B operand of the activation sums (see 2b)
   const u4 bconst_bits = n < 8 ? (u4){0x64006400u, 0x54005400u, 0x64006400u, 0x54005400u}
@@ -172,86 +188,52 @@ __global__ __launch_bounds__(kThreads, (REUSE && MR == 8 && TILES == 2) ? 4 : 1)
         xv[m] = *reinterpret_cast<const u4*>(p.x + (uint64_t)srcs[m] * K + (uint32_t)(sl * 16 + lane) * 8);
     }
   };
+  // this wave's activations -> its LDS image in operand order
   auto stage_x = [&](const u4 (&xv)[MR]) {
-    if constexpr (kMfmaSums) {
-      // ---- 2. this wave's activations -> its LDS image in operand order ------------------------
-      {
-        const int ls = lane >> 4, gg = (lane >> 2) & 3, j = lane & 3;
+    const int ls = lane >> 4, gg = (lane >> 2) & 3, j = lane & 3;
 #pragma unroll
-        for (int m = 0; m < MR; ++m)
-          *reinterpret_cast<u4*>(xs + ((ls * 4 + j) * kSlots + gg * MR + m) * 16) = permute_x8(xv[m]);
-      }
-    } else {
-      // ---- 2. this wave's activations -> its LDS image in operand order; sums per (row, group) --
-      {
-        const int ls = lane >> 4, gg = (lane >> 2) & 3, j = lane & 3;
+    for (int m = 0; m < MR; ++m)
+      *reinterpret_cast<u4*>(xs + ((ls * 4 + j) * kBlk + gg * MR + m) * 16) = permute_x8(xv[m]);
+  };
+  auto stage_sums = [&]() {
+    if constexpr (kPreSums) {
+      // sums of the staged activations, once for all tiles: accumulator row 4g+j of column 0 holds sum(off*x), of
+      // column 8 sum(x) (see 2b); rows 0-7 are the activation rows of the slab's first group, rows 8-15 of its second
 #pragma unroll
-        for (int m = 0; m < MR; ++m) {
-          *reinterpret_cast<u4*>(xs + ((ls * 4 + j) * kSlots + gg * MR + m) * 16) = permute_x8(xv[m]);
-          // this lane's 8 activations: plain sum and sum weighted by the unpack offsets
-          // (even k -> 1024, odd k -> 64); 8 consecutive lanes make up one group of 64
-          const h8 hv = __builtin_bit_cast(h8, xv[m]);
-          float xs8 = 0.f, xo8 = 0.f;
+      for (int it = 0; it < SPW; ++it) {
+        f4 own = (f4){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-          for (int e = 0; e < 8; e += 2) {
-            xs8 += (float)hv[e] + (float)hv[e + 1];
-            xo8 += 1024.0f * (float)hv[e] + 64.0f * (float)hv[e + 1];
-          }
-#pragma unroll
-          for (int off = 1; off < 8; off <<= 1) {
-            xs8 += __shfl_xor(xs8, off, 64);
-            xo8 += __shfl_xor(xo8, off, 64);
-          }
-          if ((lane & 7) == 0) {  // sums[group][m] = (-sum(off*x), sum(x)); rows >= MR stay unused
-            sums[((lane >> 3) * 8 + m) * 2 + 0] = -xo8;
-            sums[((lane >> 3) * 8 + m) * 2 + 1] = xs8;
-          }
+        for (int j = 0; j < 4; ++j) {
+          const h8 av = *reinterpret_cast<const h8*>(xs + ((it * 4 + j) * kBlk) * 16 + a_slot_off);
+          own = __builtin_amdgcn_mfma_f32_16x16x32_f16(av, bconst, own, 0, 0, 0);
         }
+        float* sp = sums + ((it * 2 + par) * 8 + (g & 1) * 4) * 2;
+        if (n == 0) { sp[0] = -own.x; sp[2] = -own.y; sp[4] = -own.z; sp[6] = -own.w; }
+        if (n == 8) { sp[1] = own.x; sp[3] = own.y; sp[5] = own.z; sp[7] = own.w; }
       }
     }
   };
-  if constexpr (REUSE) {  // single pass: slab0 = 0, SPW slabs per wave
-    u4 xv[MR];
-    load_x((int)(kp * SPW), SPW, xv);
-    stage_x(xv);
-  }
 
   // ---- tiles of this workgroup: consecutive, so it streams one contiguous block of weight rows.
   //      With one pass over K the activation image (and the sums) staged for the first tile serve
   //      all of them.
   const uint32_t ntiles = REUSE ? p.tpw : 1u;  // (without reuse the launcher gives every workgroup one tile)
-  for (uint32_t ti = 0; ti < ntiles; ++ti) {
-  const uint32_t wg_tile = blockIdx.x * ntiles + ti;
-  const uint32_t tile_row = (wg_tile * NT + tw) * rows_per_slot;
-
-  const u4* wrow[TILES];
-  const __half* sbrow[TILES];
-#pragma unroll
-  for (int t = 0; t < TILES; ++t) {
-    const uint64_t e_w = TAB ? expert * p.estride_w : 0, e_s = TAB ? expert * p.estride_s : 0;
-    const bool first = t == 0 || pair;                       // which matrix
-    const uint32_t wr = tile_row + n + (pair ? 16 * t : 0);  // which row of it
-    wrow[t] = reinterpret_cast<const u4*>((first ? p.w0 : p.w1) + e_w + (uint64_t)wr * words_per_row) + g;
-    // scales live in the lanes with even g, biases in the lanes with odd g (exchanged later)
-    const __half* sb = (g & 1) ? (first ? p.b0 : p.b1) : (first ? p.s0 : p.s1);
-    sbrow[t] = sb + e_s + (uint64_t)wr * groups_per_row;
-  }
-  f4 F[TILES];
-#pragma unroll
-  for (int t = 0; t < TILES; ++t) F[t] = (f4){0.f, 0.f, 0.f, 0.f};
-
-  for (uint32_t slab0 = 0; slab0 < slabs_total; slab0 += KS * kSpwMax) {
-    const uint32_t ns = slabs_total - slab0 < KS * kSpwMax ? slabs_total - slab0 : KS * kSpwMax;  // slabs of this pass
-    const int spw = SPW ? SPW : (int)((ns + KS - 1) / KS);
-    const int sl = (int)(slab0 + kp * spw);       // first slab of this wave
-    int my_rt = (int)ns - (int)(kp * spw);
-    my_rt = my_rt < 0 ? 0 : (my_rt > spw ? spw : my_rt);
-    const int my = SPW ? SPW : my_rt;
-
-    // ---- 1. every global load of the pass, small ones first --------------------------------
-    u4 xv[MR];
-    if constexpr (!REUSE) load_x(sl, my, xv);
-    u4 sbv[TILES];  // word `it` = (group 2*it, group 2*it+1) of slab sl+it: scales or biases, by lane
+  // every global load of one tile's slabs sl .. sl+my-1: scales / biases first (the memory counter retires in order)
+  auto load_tile = [&](uint32_t wg_tile, int sl, int my, u4 (&sbv)[TILES], u4 (&wreg)[TILES][kSpwMax]) {
+    const uint32_t tile_row = (wg_tile * NT + tw) * rows_per_slot;
+    const u4* wrow[TILES];
+    const __half* sbrow[TILES];
+  #pragma unroll
+    for (int t = 0; t < TILES; ++t) {
+      const uint64_t e_w = TAB ? expert * p.estride_w : 0, e_s = TAB ? expert * p.estride_s : 0;
+      const bool first = t == 0 || pair;                       // which matrix
+      const uint32_t wr = tile_row + n + (pair ? 16 * t : 0);  // which row of it
+      wrow[t] = reinterpret_cast<const u4*>((first ? p.w0 : p.w1) + e_w + (uint64_t)wr * words_per_row) + g;
+      // scales live in the lanes with even g, biases in the lanes with odd g (exchanged later)
+      const __half* sb = (g & 1) ? (first ? p.b0 : p.b1) : (first ? p.s0 : p.s1);
+      sbrow[t] = sb + e_s + (uint64_t)wr * groups_per_row;
+    }
+    // sbv word `it` = (group 2*it, group 2*it+1) of slab sl+it: scales or biases, by lane
 #pragma unroll
     for (int t = 0; t < TILES; ++t) {
       sbv[t] = (u4){0u, 0u, 0u, 0u};
@@ -271,7 +253,6 @@ __global__ __launch_bounds__(kThreads, (REUSE && MR == 8 && TILES == 2) ? 4 : 1)
         if (my > 2) sbv[t].z = sp[2];
       }
     }
-    u4 wreg[TILES][kSpwMax];
 #pragma unroll
     for (int it = 0; it < kSpwMax; ++it) {
       if (it < my) {
@@ -279,15 +260,55 @@ __global__ __launch_bounds__(kThreads, (REUSE && MR == 8 && TILES == 2) ? 4 : 1)
         for (int t = 0; t < TILES; ++t) wreg[t][it] = *(wrow[t] + (sl + it) * 4);
       }
     }
-
-    if constexpr (!REUSE) stage_x(xv);
-
+  };
+  // the tile's slabs against the staged activations: F += scale * (dot - sum(off*x)) + bias * sum(x)
+  auto compute_tile = [&](int my, const u4 (&sbv)[TILES], const u4 (&wreg)[TILES][kSpwMax], f4 (&F)[TILES]) {
     // ---- 2b/3 for 8 rows: slab by slab (few live registers).  The per (row, group) sums of the
     //          activations come from the matrix unit: columns 0-7 of a constant B operand hold the
     //          unpack offsets (1024 for even k, 64 for odd k, in slot order), columns 8-15 hold
     //          ones, so accumulator column n < 8 receives sum(off*x) and column n >= 8 sum(x) of
     //          its rows; lane n^8 holds the other one.
-    if constexpr (kMfmaSums) {
+    if constexpr (kPreSums) {
+      // ---- 8 rows, several tiles per workgroup: the sums wait in LDS; slab by slab (few live registers) ----
+      u4 sv[TILES], bv[TILES];
+#pragma unroll
+      for (int t = 0; t < TILES; ++t) {
+        const u4 other = (u4){swap16(sbv[t].x), swap16(sbv[t].y), swap16(sbv[t].z), swap16(sbv[t].w)};
+        sv[t] = (g & 1) ? other : sbv[t];
+        bv[t] = (g & 1) ? sbv[t] : other;
+      }
+#pragma unroll
+      for (int it = 0; it < kSpwMax; ++it) {
+        if (it < my) {
+          f4 c[TILES];
+#pragma unroll
+          for (int t = 0; t < TILES; ++t) c[t] = (f4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            const h8 av = *reinterpret_cast<const h8*>(xs + ((it * 4 + j) * kBlk) * 16 + a_slot_off);
+#pragma unroll
+            for (int t = 0; t < TILES; ++t) {
+              const uint32_t wd = j == 0 ? wreg[t][it].x : (j == 1 ? wreg[t][it].y : (j == 2 ? wreg[t][it].z : wreg[t][it].w));
+              c[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(av, unpack_q4_word(wd, qc), c[t], 0, 0, 0);
+            }
+          }
+          const float* sp = sums + ((it * 2 + par) * 8 + (g & 1) * 4) * 2;
+          const f4 c01 = *reinterpret_cast<const f4*>(sp);      // (-xoff, xsum) of accumulator rows 4g, 4g+1
+          const f4 c23 = *reinterpret_cast<const f4*>(sp + 4);  // rows 4g+2, 4g+3
+#pragma unroll
+          for (int t = 0; t < TILES; ++t) {
+            const uint32_t swd = it == 0 ? sv[t].x : (it == 1 ? sv[t].y : (it == 2 ? sv[t].z : sv[t].w));
+            const uint32_t bwd = it == 0 ? bv[t].x : (it == 1 ? bv[t].y : (it == 2 ? bv[t].z : bv[t].w));
+            const float sc = __half2float(__ushort_as_half((unsigned short)(par ? swd >> 16 : swd & 0xFFFFu)));
+            const float bi = __half2float(__ushort_as_half((unsigned short)(par ? bwd >> 16 : bwd & 0xFFFFu)));
+            F[t][0] += sc * (c[t][0] + c01[0]) + bi * c01[1];
+            F[t][1] += sc * (c[t][1] + c01[2]) + bi * c01[3];
+            F[t][2] += sc * (c[t][2] + c23[0]) + bi * c23[1];
+            F[t][3] += sc * (c[t][3] + c23[2]) + bi * c23[3];
+          }
+        }
+      }
+    } else {
       u4 sv[TILES], bv[TILES];
 #pragma unroll
       for (int t = 0; t < TILES; ++t) {
@@ -304,13 +325,12 @@ __global__ __launch_bounds__(kThreads, (REUSE && MR == 8 && TILES == 2) ? 4 : 1)
           for (int t = 0; t < TILES; ++t) c[t] = (f4){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
           for (int j = 0; j < 4; ++j) {
-            h8 av = (h8){0, 0, 0, 0, 0, 0, 0, 0};
-            if (a_active) av = *reinterpret_cast<const h8*>(xs + ((it * 4 + j) * kSlots) * 16 + a_slot_off);
+            const h8 av = *reinterpret_cast<const h8*>(xs + ((it * 4 + j) * kBlk) * 16 + a_slot_off);
             own = __builtin_amdgcn_mfma_f32_16x16x32_f16(av, bconst, own, 0, 0, 0);
 #pragma unroll
             for (int t = 0; t < TILES; ++t) {
               const uint32_t wd = j == 0 ? wreg[t][it].x : (j == 1 ? wreg[t][it].y : (j == 2 ? wreg[t][it].z : wreg[t][it].w));
-              c[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(av, unpack_q4_word(wd), c[t], 0, 0, 0);
+              c[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(av, unpack_q4_word(wd, qc), c[t], 0, 0, 0);
             }
           }
           const float o0 = swap8(own.x), o1 = swap8(own.y), o2 = swap8(own.z), o3 = swap8(own.w);
@@ -328,56 +348,9 @@ __global__ __launch_bounds__(kThreads, (REUSE && MR == 8 && TILES == 2) ? 4 : 1)
           }
         }
       }
-    } else {
-      // ---- 3. weights: integer dot per group via MFMA (independent slabs interleaved), then
-      //         acc += scale * (dot - sum(off*x)) + bias * sum(x) in f32 ------------------------
-#pragma unroll
-      for (int t = 0; t < TILES; ++t) {
-        f4 c[kSpwMax];
-#pragma unroll
-        for (int it = 0; it < kSpwMax; ++it) c[it] = (f4){0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          h8 av[kSpwMax];
-#pragma unroll
-          for (int it = 0; it < kSpwMax; ++it) {
-            av[it] = (h8){0, 0, 0, 0, 0, 0, 0, 0};
-            if (it < my && a_active)
-              av[it] = *reinterpret_cast<const h8*>(xs + ((it * 4 + j) * kSlots) * 16 + a_slot_off);
-          }
-#pragma unroll
-          for (int it = 0; it < kSpwMax; ++it) {
-            if (it < my) {
-              const uint32_t wd = j == 0 ? wreg[t][it].x : (j == 1 ? wreg[t][it].y : (j == 2 ? wreg[t][it].z : wreg[t][it].w));
-              c[it] = __builtin_amdgcn_mfma_f32_16x16x32_f16(av[it], unpack_q4_word(wd), c[it], 0, 0, 0);
-            }
-          }
-        }
-        const u4 other = (u4){swap16(sbv[t].x), swap16(sbv[t].y), swap16(sbv[t].z), swap16(sbv[t].w)};
-        const u4 sv = (g & 1) ? other : sbv[t];
-        const u4 bv = (g & 1) ? sbv[t] : other;
-#pragma unroll
-        for (int it = 0; it < kSpwMax; ++it) {
-          if (it < my) {
-            const uint32_t swd = it == 0 ? sv.x : (it == 1 ? sv.y : (it == 2 ? sv.z : sv.w));
-            const uint32_t bwd = it == 0 ? bv.x : (it == 1 ? bv.y : (it == 2 ? bv.z : bv.w));
-            const float sc = __half2float(__ushort_as_half((unsigned short)(par ? swd >> 16 : swd & 0xFFFFu)));
-            const float bi = __half2float(__ushort_as_half((unsigned short)(par ? bwd >> 16 : bwd & 0xFFFFu)));
-            {
-              const float* sp = sums + ((it * 2 + par) * 8 + (g & 1) * 4) * 2;
-              const f4 c01 = *reinterpret_cast<const f4*>(sp);      // (-xoff, xsum) of accumulator rows 4g, 4g+1
-              const f4 c23 = *reinterpret_cast<const f4*>(sp + 4);  // rows 4g+2, 4g+3
-              F[t][0] += sc * (c[it][0] + c01[0]) + bi * c01[1];
-              F[t][1] += sc * (c[it][1] + c01[2]) + bi * c01[3];
-              F[t][2] += sc * (c[it][2] + c23[0]) + bi * c23[1];
-              F[t][3] += sc * (c[it][3] + c23[2]) + bi * c23[3];
-            }
-          }
-        }
-      }
     }
-  }
-
+  };
+  auto finish_tile = [&](uint32_t wg_tile, f4 (&F)[TILES]) {
   // ---- 4. reduce over the two group halves (lane + 32 holds the other one) and over the
   //         k-parts, write out -------------------------------------------------------------------
   __syncthreads();  // the previous tile's sums have been read
@@ -391,7 +364,7 @@ __global__ __launch_bounds__(kThreads, (REUSE && MR == 8 && TILES == 2) ? 4 : 1)
     for (int t = 0; t < TILES; ++t)
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        const float v = F[t][i] + __shfl_xor(F[t][i], 32, 64);
+        const float v = add_other_half(F[t][i]);
         if (g_t < 2) red[((wave_t * TILES + t) * 8 + g_t * 4 + i) * 16 + n_t] = v;
       }
   }
@@ -418,13 +391,87 @@ __global__ __launch_bounds__(kThreads, (REUSE && MR == 8 && TILES == 2) ? 4 : 1)
       }
     }
   }
-  }  // tiles of this workgroup
+  };
+
+  if constexpr (REUSE && MR == 8) {
+    // one pass: slabs kp*SPW .. of every tile; the activations and the first tile's weights are requested together.
+    // (Eight rows: a second register set for the next tile's weights would cost the second workgroup per CU,
+    // which hides more latency than the prefetch; measured.)
+    const int sl = (int)(kp * SPW);
+    const uint32_t first = blockIdx.x * ntiles;
+    u4 sbv[TILES];
+    u4 wreg[TILES][kSpwMax];
+    {
+      u4 xv[MR];
+      load_x(sl, SPW, xv);
+      // (two tiles: their first weights do not fit beside the activations in the registers of four waves per SIMD)
+      if constexpr (TILES == 1) load_tile(first, sl, SPW, sbv, wreg);
+      stage_x(xv);
+      stage_sums();
+    }
+    for (uint32_t ti = 0; ti < ntiles; ++ti) {
+      f4 F[TILES];
+      if (TILES == 2 || ti > 0) load_tile(first + ti, sl, SPW, sbv, wreg);
+#pragma unroll
+      for (int t = 0; t < TILES; ++t) F[t] = (f4){0.f, 0.f, 0.f, 0.f};
+      compute_tile(SPW, sbv, wreg, F);
+      finish_tile(first + ti, F);
+    }
+  } else if constexpr (REUSE) {  // fewer rows: the weights of the next tile are in flight while this one is multiplied
+    const int sl = (int)(kp * SPW);
+    u4 sbv_a[TILES], sbv_b[TILES];
+    u4 wreg_a[TILES][kSpwMax], wreg_b[TILES][kSpwMax];
+    const uint32_t first = blockIdx.x * ntiles;
+    {
+      u4 xv[MR];
+      load_x(sl, SPW, xv);
+      load_tile(first, sl, SPW, sbv_a, wreg_a);
+      stage_x(xv);
+      stage_sums();
+    }
+    for (uint32_t ti = 0; ti < ntiles; ti += 2) {
+      f4 F[TILES];
+      if (ti + 1 < ntiles) load_tile(first + ti + 1, sl, SPW, sbv_b, wreg_b);
+#pragma unroll
+      for (int t = 0; t < TILES; ++t) F[t] = (f4){0.f, 0.f, 0.f, 0.f};
+      compute_tile(SPW, sbv_a, wreg_a, F);
+      finish_tile(first + ti, F);
+      if (ti + 1 < ntiles) {
+        if (ti + 2 < ntiles) load_tile(first + ti + 2, sl, SPW, sbv_a, wreg_a);
+#pragma unroll
+        for (int t = 0; t < TILES; ++t) F[t] = (f4){0.f, 0.f, 0.f, 0.f};
+        compute_tile(SPW, sbv_b, wreg_b, F);
+        finish_tile(first + ti + 1, F);
+      }
+    }
+  } else {
+    const uint32_t wg_tile = blockIdx.x;
+    f4 F[TILES];
+#pragma unroll
+    for (int t = 0; t < TILES; ++t) F[t] = (f4){0.f, 0.f, 0.f, 0.f};
+    for (uint32_t slab0 = 0; slab0 < slabs_total; slab0 += KS * kSpwMax) {
+      const uint32_t ns = slabs_total - slab0 < KS * kSpwMax ? slabs_total - slab0 : KS * kSpwMax;  // slabs of this pass
+      const int spw = SPW ? SPW : (int)((ns + KS - 1) / KS);
+      const int sl = (int)(slab0 + kp * spw);       // first slab of this wave
+      int my_rt = (int)ns - (int)(kp * spw);
+      my_rt = my_rt < 0 ? 0 : (my_rt > spw ? spw : my_rt);
+      const int my = SPW ? SPW : my_rt;
+      u4 xv[MR];
+      load_x(sl, my, xv);
+      u4 sbv[TILES];
+      u4 wreg[TILES][kSpwMax];
+      load_tile(wg_tile, sl, my, sbv, wreg);
+      stage_x(xv);
+      compute_tile(my, sbv, wreg, F);
+    }
+    finish_tile(wg_tile, F);
+  }
 }
 
 template <int MR, int TILES, int SPW, bool PAIR>
 void launch_s(const KParams& p, bool tab, dim3 grid, hipStream_t s) {
   if constexpr (SPW != 0) {
-    if (p.tpw > 1) {
+    if (p.K / 128 == p.ks * SPW) {  // one pass over K: the kernel that requests activations and first weights together
       if (tab) hipLaunchKernelGGL((qmv_q4_kernel<MR, TILES, true, SPW, PAIR, true>), grid, dim3(kThreads), 0, s, p);
       else hipLaunchKernelGGL((qmv_q4_kernel<MR, TILES, false, SPW, PAIR, true>), grid, dim3(kThreads), 0, s, p);
       return;
