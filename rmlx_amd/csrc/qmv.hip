@@ -113,10 +113,13 @@ struct __attribute__((packed, aligned(4))) U4Unaligned { uint32_t v[4]; };
 // TAB = rows come from a device chunk table (gather_qmm, MoE); SPW = slabs per wave and pass when
 // every wave of every pass owns the same number (3 or 4: no guards, fewer registers, two
 // workgroups per CU), 0 = decided at run time.
-// REUSE = one pass covers K and the workgroup takes several tiles: the activations are staged once,
+// REUSE != 0: one pass covers K, so the activations are staged once, before the tile loop; 2 = with fewer than
+// 8 rows, the next tile's weights are loaded into a second register set while the current tile is multiplied
+// (for workgroups that take several tiles; a workgroup with one tile keeps the registers for a third resident
+// workgroup per CU);
 // before the tile loop (their registers are free again when the weight loads start).
-template <int MR, int TILES, bool TAB, int SPW, bool PAIR, bool REUSE>
-__global__ __launch_bounds__(kThreads, (REUSE && MR == 8 && TILES == 2) ? 4 : 1) void qmv_q4_kernel(KParams p) {
+template <int MR, int TILES, bool TAB, int SPW, bool PAIR, int REUSE>
+__global__ __launch_bounds__(kThreads, (REUSE != 0 && MR == 8 && TILES == 2) ? 4 : 1) void qmv_q4_kernel(KParams p) {
   static_assert(!REUSE || SPW != 0, "reuse needs a uniform slab count");
   static_assert(!PAIR || TILES == 2, "paired tiles need two tile slots");
   constexpr int kSlots = 4 * MR;                       // 16-byte activation slots per (slab, j) block ...
@@ -126,7 +129,7 @@ __global__ __launch_bounds__(kThreads, (REUSE && MR == 8 && TILES == 2) ? 4 : 1)
   __shared__ float red[kWaves * TILES * 8 * 16];  // cross-wave reduction: [wave][tile][activation row][column]
   // Activation sums per (row, group) come from the matrix unit (see 2b).  With one pass over K they are computed
   // once, before the tile loop, and wait in LDS; otherwise every pass computes them beside its products.
-  constexpr bool kPreSums = REUSE;
+  constexpr bool kPreSums = REUSE != 0;
   __shared__ __attribute__((aligned(16))) float sums_all[!kPreSums ? 4 : kWaves * kSpwMax * 2 * 8 * 2];  // [wave][group][row][-xoff, xsum]
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -350,7 +353,7 @@ __global__ __launch_bounds__(kThreads, (REUSE && MR == 8 && TILES == 2) ? 4 : 1)
       }
     }
   };
-  auto finish_tile = [&](uint32_t wg_tile, f4 (&F)[TILES]) {
+  auto finish_tile = [&](uint32_t wg_tile, f4 (&F)[TILES], bool first_tile) {
   // ---- 4. reduce over the two group halves (lane + 32 holds the other one) and over the
   //         k-parts, write out -------------------------------------------------------------------
   __syncthreads();  // the previous tile's sums have been read
@@ -376,7 +379,16 @@ __global__ __launch_bounds__(kThreads, (REUSE && MR == 8 && TILES == 2) ? 4 : 1)
 #pragma unroll
       for (int t = 0; t < TILES; ++t) {
         float acc = 0.f;
-        for (uint32_t q = 0; q < KS; ++q) acc += red[(((otw * KS + q) * TILES + t) * 8 + m) * 16 + nn];
+        if (KS == 8) {  // (four reads in flight at a time instead of a chain of eight)
+#pragma unroll
+          for (uint32_t q = 0; q < 8; q += 4) {
+            const float* rp = red + ((q * TILES + t) * 8 + m) * 16 + nn;
+            const float r0 = rp[0], r1 = rp[TILES * 128], r2 = rp[2 * TILES * 128], r3 = rp[3 * TILES * 128];
+            acc += (r0 + r1) + (r2 + r3);
+          }
+        } else {
+          for (uint32_t q = 0; q < KS; ++q) acc += red[(((otw * KS + q) * TILES + t) * 8 + m) * 16 + nn];
+        }
         v[t] = acc;
       }
       const uint64_t obase = (uint64_t)(row0 + m) * p.ld_out + (wg_tile * NT + otw) * rows_per_slot + nn;
@@ -393,7 +405,7 @@ __global__ __launch_bounds__(kThreads, (REUSE && MR == 8 && TILES == 2) ? 4 : 1)
   }
   };
 
-  if constexpr (REUSE && MR == 8) {
+  if constexpr (REUSE == 1) {
     // one pass: slabs kp*SPW .. of every tile; the activations and the first tile's weights are requested together.
     // (Eight rows: a second register set for the next tile's weights would cost the second workgroup per CU,
     // which hides more latency than the prefetch; measured.)
@@ -415,9 +427,9 @@ __global__ __launch_bounds__(kThreads, (REUSE && MR == 8 && TILES == 2) ? 4 : 1)
 #pragma unroll
       for (int t = 0; t < TILES; ++t) F[t] = (f4){0.f, 0.f, 0.f, 0.f};
       compute_tile(SPW, sbv, wreg, F);
-      finish_tile(first + ti, F);
+      finish_tile(first + ti, F, ti == 0);
     }
-  } else if constexpr (REUSE) {  // fewer rows: the weights of the next tile are in flight while this one is multiplied
+  } else if constexpr (REUSE == 2) {  // fewer rows, several tiles: the weights of the next tile are in flight while this one is multiplied
     const int sl = (int)(kp * SPW);
     u4 sbv_a[TILES], sbv_b[TILES];
     u4 wreg_a[TILES][kSpwMax], wreg_b[TILES][kSpwMax];
@@ -435,13 +447,13 @@ __global__ __launch_bounds__(kThreads, (REUSE && MR == 8 && TILES == 2) ? 4 : 1)
 #pragma unroll
       for (int t = 0; t < TILES; ++t) F[t] = (f4){0.f, 0.f, 0.f, 0.f};
       compute_tile(SPW, sbv_a, wreg_a, F);
-      finish_tile(first + ti, F);
+      finish_tile(first + ti, F, ti == 0);
       if (ti + 1 < ntiles) {
         if (ti + 2 < ntiles) load_tile(first + ti + 2, sl, SPW, sbv_a, wreg_a);
 #pragma unroll
         for (int t = 0; t < TILES; ++t) F[t] = (f4){0.f, 0.f, 0.f, 0.f};
         compute_tile(SPW, sbv_b, wreg_b, F);
-        finish_tile(first + ti + 1, F);
+        finish_tile(first + ti + 1, F, false);
       }
     }
   } else {
@@ -464,21 +476,27 @@ __global__ __launch_bounds__(kThreads, (REUSE && MR == 8 && TILES == 2) ? 4 : 1)
       stage_x(xv);
       compute_tile(my, sbv, wreg, F);
     }
-    finish_tile(wg_tile, F);
+    finish_tile(wg_tile, F, true);
   }
 }
 
 template <int MR, int TILES, int SPW, bool PAIR>
 void launch_s(const KParams& p, bool tab, dim3 grid, hipStream_t s) {
   if constexpr (SPW != 0) {
-    if (p.K / 128 == p.ks * SPW) {  // one pass over K: the kernel that requests activations and first weights together
-      if (tab) hipLaunchKernelGGL((qmv_q4_kernel<MR, TILES, true, SPW, PAIR, true>), grid, dim3(kThreads), 0, s, p);
-      else hipLaunchKernelGGL((qmv_q4_kernel<MR, TILES, false, SPW, PAIR, true>), grid, dim3(kThreads), 0, s, p);
+    if (p.K / 128 == p.ks * SPW) {  // one pass over K: the kernels that stage the activations once
+      constexpr int kPipe = MR < 8 ? 2 : 1;
+      if (p.tpw > 1) {
+        if (tab) hipLaunchKernelGGL((qmv_q4_kernel<MR, TILES, true, SPW, PAIR, kPipe>), grid, dim3(kThreads), 0, s, p);
+        else hipLaunchKernelGGL((qmv_q4_kernel<MR, TILES, false, SPW, PAIR, kPipe>), grid, dim3(kThreads), 0, s, p);
+      } else {
+        if (tab) hipLaunchKernelGGL((qmv_q4_kernel<MR, TILES, true, SPW, PAIR, 1>), grid, dim3(kThreads), 0, s, p);
+        else hipLaunchKernelGGL((qmv_q4_kernel<MR, TILES, false, SPW, PAIR, 1>), grid, dim3(kThreads), 0, s, p);
+      }
       return;
     }
   }
-  if (tab) hipLaunchKernelGGL((qmv_q4_kernel<MR, TILES, true, SPW, PAIR, false>), grid, dim3(kThreads), 0, s, p);
-  else hipLaunchKernelGGL((qmv_q4_kernel<MR, TILES, false, SPW, PAIR, false>), grid, dim3(kThreads), 0, s, p);
+  if (tab) hipLaunchKernelGGL((qmv_q4_kernel<MR, TILES, true, SPW, PAIR, 0>), grid, dim3(kThreads), 0, s, p);
+  else hipLaunchKernelGGL((qmv_q4_kernel<MR, TILES, false, SPW, PAIR, 0>), grid, dim3(kThreads), 0, s, p);
 }
 
 template <int MR, int TILES, bool PAIR = false>
@@ -570,7 +588,7 @@ int32_t launch_qmv_q4(const QmvArgs& a, hipStream_t s) {
     for (int pass = tab ? 0 : 1; pass < 2 && tpw == 1; ++pass)
       for (uint32_t c : cand)
         if (tiles_x % c == 0 && (pass == 1 || (tiles_x / c) % 8 == 0) &&
-            (uint64_t)(tiles_x / c) * chunks >= 2ull * (uint32_t)ctx().num_cus) { tpw = c; break; }
+            (uint64_t)(tiles_x / c) * chunks >= (tab ? 2ull : 1ull) * (uint32_t)ctx().num_cus) { tpw = c; break; }
   }
   p.tpw = tpw;
   dim3 grid(tiles_x / tpw, chunks);

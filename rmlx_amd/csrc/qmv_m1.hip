@@ -85,7 +85,10 @@ __device__ __forceinline__ u4 to_pair_order(u4 d) {
 // rows cost one pass over the weights plus 16 dot instructions per row, chunk and lane.
 // NORM = RMSNorm prologue applied while the activations are staged (kernels of their own: the extra
 // registers would cost the plain kernels occupancy).
-template <int BITS, int GS, int R, bool NT, int MR, bool NORM = false>
+// KP = waves per weight row (1, 2 or 4; split K, the counterpart of affine_qmv_splitk_f16_q4 + qmm_splitk_accum_f16,
+// quantized.rs:992-1233): wave w takes the chunks kp, kp + KP, ... of row w / KP (kp = w % KP) and the partial sums
+// meet in workgroup memory.  For long rows of a short matrix, where one wave per row leaves most of the chip idle.
+template <int BITS, int GS, int R, bool NT, int MR, bool NORM = false, int KP = 1>
 // (8-bit, one row: asking the compiler for eight waves per SIMD changes no register count but the schedule;
 // measured 4-13 % faster.  The 4-bit kernel would spill under that bound and is slower with it.)
 __global__ __launch_bounds__(kThreads, (BITS == 8 && MR == 1 && R == 1) ? 8 : 1) void qmv_m1_kernel(M1Params p) {
@@ -107,7 +110,11 @@ __global__ __launch_bounds__(kThreads, (BITS == 8 && MR == 1 && R == 1) ? 8 : 1)
   auto cs = [&](int m) { return reinterpret_cast<float2*>(lds + (size_t)MR * img_bytes + (size_t)m * cs_bytes); };
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const uint32_t row0 = blockIdx.x * (kWaves * R) + wave * R;
+  static_assert(KP == 1 || R == 1, "split rows: one row per wave group");
+  const uint32_t row0 = blockIdx.x * (kWaves * R / KP) + (wave / KP) * R;
+  const uint32_t kp = wave % KP;
+  // this wave's chunks: kp, kp + KP, ... (KHw of them)
+  const uint32_t KHw = KP == 1 ? KH : (KH > kp ? (KH - kp + KP - 1) / KP : 0u);
   const uint32_t mrow0 = blockIdx.y * MR;  // first activation row of this pass (rows past M repeat the last one, unstored)
 
   // ---- 1. loads, small ones first (the memory counter retires in order): activations ... ------
@@ -165,7 +172,7 @@ __global__ __launch_bounds__(kThreads, (BITS == 8 && MR == 1 && R == 1) ? 8 : 1)
   auto load_batch = [&](uint32_t c0, Batch& t) {
 #pragma unroll
     for (int cc = 0; cc < 2; ++cc) {
-      const uint32_t c = c0 + cc < KH ? c0 + cc : KH - 1;  // an odd chunk count re-reads the last chunk (unused)
+      const uint32_t c = c0 + cc < KHw ? kp + KP * (c0 + cc) : KH - 1;  // an odd chunk count re-reads the last chunk (unused)
       uint32_t wi = c * 64 + lane, gi = c * kGroupsPerChunk + lane / kLanesPerGroup;
       wi = wi < row_u4 ? wi : row_u4 - 1;  // lanes past K (last chunk of a K that is no chunk multiple)
       gi = gi < G ? gi : G - 1;
@@ -235,8 +242,8 @@ __global__ __launch_bounds__(kThreads, (BITS == 8 && MR == 1 && R == 1) ? 8 : 1)
   auto process = [&](uint32_t c0, const Batch& t) {
 #pragma unroll
     for (int cc = 0; cc < 2; ++cc) {
-      const uint32_t c = c0 + cc;
-      if (c < KH) {
+      const uint32_t c = kp + KP * (c0 + cc);
+      if (c0 + cc < KHw) {
         uint32_t xr[MR][kXU][4];
         float2 k[MR];
 #pragma unroll
@@ -287,8 +294,8 @@ __global__ __launch_bounds__(kThreads, (BITS == 8 && MR == 1 && R == 1) ? 8 : 1)
       }
     }
   };
-  for (uint32_t c0 = 0; c0 < KH; c0 += 4) {
-    const bool more1 = c0 + 2 < KH, more2 = c0 + 4 < KH;
+  for (uint32_t c0 = 0; c0 < KHw; c0 += 4) {
+    const bool more1 = c0 + 2 < KHw, more2 = c0 + 4 < KHw;
     if (more1) load_batch(c0 + 2, bb);
     process(c0, ba);
     if (more1) {
@@ -306,10 +313,273 @@ __global__ __launch_bounds__(kThreads, (BITS == 8 && MR == 1 && R == 1) ? 8 : 1)
       const float t = wave_sum(racc[r][m]);
       mine = lane == r * MR + m ? t : mine;
     }
-  if (writes) {  // residual add / SwiGLU gate in f32, one rounding (quantized.rs:3206-3246)
+  if constexpr (KP > 1) {  // partial sums of a row's KP waves, added in wave order by the first of them
+    float* part = reinterpret_cast<float*>(lds);
+    __syncthreads();  // every wave has read its activations
+    if (lane < MR) part[wave * MR + lane] = mine;
+    __syncthreads();
+    if (lane < MR) {
+      mine = part[wave * MR + lane];
+#pragma unroll
+      for (int q = 1; q < KP; ++q) mine += kp == 0 ? part[(wave + q) * MR + lane] : 0.f;
+    }
+  }
+  if (writes && kp == 0) {  // residual add / SwiGLU gate in f32, one rounding (quantized.rs:3206-3246)
     if (p.epi_kind == EPI_RESIDUAL) mine += epi_val;
     else if (p.epi_kind == EPI_SWIGLU) mine = epi_val / (1.0f + __expf(-epi_val)) * mine;
     p.out[(uint64_t)out_m * p.N + out_n] = __float2half(mine);
+  }
+}
+
+// The same kernel for matrices with more row blocks than the chip keeps resident: the grid is sized to the resident
+// workgroups and each of them walks several row blocks (see `my_blocks`).
+template <int BITS, int GS, int R, bool NT, int MR, bool NORM = false>
+// (8-bit, one row: asking the compiler for eight waves per SIMD changes no register count but the schedule;
+// measured 4-13 % faster.  The 4-bit kernel would spill under that bound and is slower with it.)
+__global__ __launch_bounds__(kThreads, 1) void qmv_m1_loop_kernel(M1Params p) {
+  constexpr int kChunkK = 8192 / BITS;         // k values of one wave-wide 16-byte load: 2048 / 1024
+  constexpr int kLaneK = kChunkK / 64;         // values per lane and chunk: 32 / 16
+  constexpr int kXU = kLaneK / 8;              // 16-byte activation units per lane and chunk: 4 / 2
+  constexpr int kLanesPerGroup = GS / kLaneK;  // whole lanes per quantisation group
+  constexpr int kGroupsPerChunk = kChunkK / GS;
+  static_assert(kLanesPerGroup >= 1, "a lane must not straddle quantisation groups");
+
+  extern __shared__ __attribute__((aligned(16))) char lds[];
+  // K need not be a multiple of the chunk: the lanes of the last chunk that lie past K read clamped
+  // (valid) addresses and multiply them with a zeroed activation image, i.e. contribute nothing.
+  const uint32_t K = p.K, KH = (K + kChunkK - 1) / kChunkK, G = K / GS, nunits = K / 8;
+  const uint32_t row_u4 = K / kLaneK;  // 16-byte pieces of a weight row
+  // per activation row: image [chunk][unit j][lane], then sums [chunk][lane] = (sum(off * x), sum(x)) of the lane's values
+  const uint32_t img_bytes = KH * kChunkK * 2, cs_bytes = KH * 64 * sizeof(float2);  // per activation row, whole chunks
+  auto xl = [&](int m) { return reinterpret_cast<u4*>(lds + (size_t)m * img_bytes); };
+  auto cs = [&](int m) { return reinterpret_cast<float2*>(lds + (size_t)MR * img_bytes + (size_t)m * cs_bytes); };
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const uint32_t mrow0 = blockIdx.y * MR;  // first activation row of this pass (rows past M repeat the last one, unstored)
+  // Row blocks (kWaves * R weight rows) of this workgroup: blockIdx.x, blockIdx.x + gridDim.x, ...  The launcher
+  // sizes the grid to what the chip keeps resident, so the activations are staged once per workgroup and the
+  // next block's weights are already in flight while the current block is multiplied.
+  const uint32_t nblk = p.N / (kWaves * R);
+  const uint32_t my_blocks = blockIdx.x < nblk ? (nblk - 1 - blockIdx.x) / gridDim.x + 1 : 0u;
+  auto block_row0 = [&](uint32_t i) { return (blockIdx.x + i * gridDim.x) * (kWaves * R) + wave * R; };
+
+  // ---- 1. loads, small ones first (the memory counter retires in order): activations ... ------
+  u4 xv[MR][4];
+#pragma unroll
+  for (int m = 0; m < MR; ++m) {
+    const uint32_t rm = mrow0 + m < p.M ? mrow0 + m : p.M - 1;
+    const u4* xg = reinterpret_cast<const u4*>(p.x + (uint64_t)rm * K);
+    const uint32_t u0 = (uint32_t)tid < nunits ? (uint32_t)tid : nunits - 1;
+    xv[m][0] = xg[u0];
+#pragma unroll
+    for (int i = 1; i < 4; ++i) {
+      xv[m][i] = (u4){0u, 0u, 0u, 0u};
+      if (nunits > (uint32_t)i * kThreads) {  // uniform; the last round may be partial (clamped, stored under a guard)
+        const uint32_t u = tid + i * kThreads;
+        xv[m][i] = xg[u < nunits ? u : nunits - 1];
+      }
+    }
+  }
+  // RMSNorm prologue of the reference's MMA kernel (`has_norm`, quantized.rs:3070-3095) applied while staging
+  auto normalise = [&](int m, uint32_t u, u4 v) {
+    const uint32_t rm = mrow0 + m < p.M ? mrow0 + m : p.M - 1;
+    const _Float16 rs = (_Float16)p.inv_rms[rm];
+    const h8 nw = __builtin_bit_cast(h8, reinterpret_cast<const u4*>(p.norm_w)[u < nunits ? u : nunits - 1]);
+    const h8 scaled = __builtin_bit_cast(h8, v) * (h8){rs, rs, rs, rs, rs, rs, rs, rs};
+    return __builtin_bit_cast(u4, scaled * nw);
+  };
+  if constexpr (NORM) {
+#pragma unroll
+    for (int m = 0; m < MR; ++m)
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        if (i == 0 || nunits > (uint32_t)i * kThreads) xv[m][i] = normalise(m, tid + i * kThreads, xv[m][i]);
+  }
+  // ---- ... then the first two chunks of the wave's rows with their scales and biases ----------------
+  // A batch is two chunks of the wave's rows in one block; the batches of all blocks of the workgroup form one
+  // sequence (block 0: chunks 0-1, 2-3, ..., block 1: chunks 0-1, ...) that is loaded one batch ahead.
+  struct Batch { u4 w[2][R]; uint32_t s[2][R], b[2][R]; float epi; };  // [chunk of the batch][row]; epi: see below
+  const uint32_t batches_per_block = (KH + 1) / 2, n_batches = my_blocks * batches_per_block;
+  // the output this lane writes at the end of a block: (weight row lane / MR, activation row lane % MR)
+  const uint32_t out_m = mrow0 + lane % MR;
+  const bool writes = lane < R * MR && out_m < p.M;
+  uint32_t ld_blk = 0, ld_c0 = 0;  // block and first chunk of the next batch to load
+  auto load_batch = [&](Batch& t) {
+    const uint32_t row0 = block_row0(ld_blk);
+    const u4* wrow[R];
+    const unsigned short* srow[R];
+    const unsigned short* brow[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      wrow[r] = reinterpret_cast<const u4*>(p.w + (uint64_t)(row0 + r) * (K * BITS / 32));
+      srow[r] = reinterpret_cast<const unsigned short*>(p.s) + (uint64_t)(row0 + r) * G;
+      brow[r] = reinterpret_cast<const unsigned short*>(p.b) + (uint64_t)(row0 + r) * G;
+    }
+    // the epilogue operand of the block's outputs travels with its first batch
+    t.epi = 0.f;
+    if (ld_c0 == 0 && p.epi_kind != EPI_NONE && writes) {
+      const uint64_t oi = (uint64_t)out_m * p.N + row0 + lane / MR;
+      t.epi = p.epi_dtype == RMLX_DTYPE_F32 ? static_cast<const float*>(p.epi)[oi]
+                                            : __half2float(static_cast<const __half*>(p.epi)[oi]);
+    }
+#pragma unroll
+    for (int cc = 0; cc < 2; ++cc) {
+      const uint32_t c = ld_c0 + cc < KH ? ld_c0 + cc : KH - 1;  // an odd chunk count re-reads the last chunk (unused)
+      uint32_t wi = c * 64 + lane, gi = c * kGroupsPerChunk + lane / kLanesPerGroup;
+      wi = wi < row_u4 ? wi : row_u4 - 1;  // lanes past K (last chunk of a K that is no chunk multiple)
+      gi = gi < G ? gi : G - 1;
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        t.s[cc][r] = srow[r][gi];
+        t.b[cc][r] = brow[r][gi];
+      }
+#pragma unroll
+      for (int r = 0; r < R; ++r)
+        t.w[cc][r] = NT ? __builtin_nontemporal_load(wrow[r] + wi) : wrow[r][wi];
+    }
+    ld_c0 += 2;
+    if (ld_c0 >= KH) { ld_c0 = 0; ++ld_blk; }
+  };
+  Batch ba, bb;
+  if (n_batches > 0) load_batch(ba);
+
+  // ---- 2. stage x: unit u = 8 consecutive k = (chunk, lane, j); image in the order a wave reads it ----
+  auto stage_unit = [&](int m, uint32_t u, const u4& v) {
+    if (u < nunits) {
+      const uint32_t c = u / (64 * kXU), rem = u % (64 * kXU), l = rem / kXU, j = rem % kXU;
+      xl(m)[(c * kXU + j) * 64 + l] = BITS == 4 ? to_pair_order(v) : v;
+      const h8 hv = __builtin_bit_cast(h8, v);
+      float xs8 = 0.f, xo8 = 0.f;
+#pragma unroll
+      for (int e = 0; e < 8; e += 2) {
+        xs8 += (float)hv[e] + (float)hv[e + 1];
+        xo8 += 1024.0f * (float)hv[e] + (BITS == 4 ? 64.0f : 1024.0f) * (float)hv[e + 1];
+      }
+      // the kXU units of a lane sit in adjacent threads of one quad (unit counts are multiples of 4)
+      xs8 = dpp_add<0xB1>(xs8);
+      xo8 = dpp_add<0xB1>(xo8);
+      if (kXU == 4) {
+        xs8 = dpp_add<0x4E>(xs8);
+        xo8 = dpp_add<0x4E>(xo8);
+      }
+      if (j == 0) cs(m)[c * 64 + l] = make_float2(xo8, xs8);
+    } else if (u < KH * 64 * kXU) {  // image positions past K: zeros
+      const uint32_t c = u / (64 * kXU), rem = u % (64 * kXU), l = rem / kXU, j = rem % kXU;
+      xl(m)[(c * kXU + j) * 64 + l] = (u4){0u, 0u, 0u, 0u};
+      if (j == 0) cs(m)[c * 64 + l] = make_float2(0.f, 0.f);
+    }
+  };
+#pragma unroll
+  for (int m = 0; m < MR; ++m)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) stage_unit(m, tid + i * kThreads, xv[m][i]);
+  // K > 16384: the remaining rounds, loaded here (behind the first weight loads; rare and long-running shapes)
+  for (uint32_t u = tid + 4 * kThreads; u < KH * 64 * kXU; u += kThreads) {
+#pragma unroll
+    for (int m = 0; m < MR; ++m) {
+      const uint32_t rm = mrow0 + m < p.M ? mrow0 + m : p.M - 1;
+      u4 v = reinterpret_cast<const u4*>(p.x + (uint64_t)rm * K)[u < nunits ? u : nunits - 1];
+      if constexpr (NORM) v = normalise(m, u, v);
+      stage_unit(m, u, v);
+    }
+  }
+  __syncthreads();
+
+  // ---- 3. batch by batch: registers of x from LDS, then the wave's rows; 4. at the end of a block the wave-wide
+  //         sums: lane r * MR + m writes the output of (weight row r, activation row m) ---------------------------
+  float racc[R][MR];
+  uint32_t m0 = 0x000F000Fu, m1 = 0x00F000F0u, k0 = 0x64006400u, k1 = 0x54005400u;
+  asm volatile("" : "+s"(m0), "+s"(m1), "+v"(k0), "+v"(k1));  // constants in registers: and+or is one instruction
+  uint32_t pr_blk = 0, pr_c0 = 0;  // block and first chunk of the batch being processed
+  float epi_val = 0.f;
+  auto process = [&](const Batch& t) {
+    if (pr_c0 == 0) {
+      epi_val = t.epi;
+#pragma unroll
+      for (int r = 0; r < R; ++r)
+#pragma unroll
+        for (int m = 0; m < MR; ++m) racc[r][m] = 0.f;
+    }
+#pragma unroll
+    for (int cc = 0; cc < 2; ++cc) {
+      const uint32_t c = pr_c0 + cc;
+      if (c < KH) {
+        uint32_t xr[MR][kXU][4];
+        float2 k[MR];
+#pragma unroll
+        for (int m = 0; m < MR; ++m) {
+#pragma unroll
+          for (int j = 0; j < kXU; ++j) {
+            const u4 v = xl(m)[(c * kXU + j) * 64 + lane];
+            xr[m][j][0] = v.x; xr[m][j][1] = v.y; xr[m][j][2] = v.z; xr[m][j][3] = v.w;
+          }
+          k[m] = cs(m)[c * 64 + lane];
+        }
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+          const u4 wv = t.w[cc][r];
+          const uint32_t wd[4] = {wv.x, wv.y, wv.z, wv.w};
+          float acc0[MR], acc1[MR];
+#pragma unroll
+          for (int m = 0; m < MR; ++m) acc0[m] = acc1[m] = 0.f;
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            if (BITS == 4) {
+              const uint32_t hi = wd[j] >> 8;
+              const h2 p0 = as_h2((wd[j] & m0) | k0), p1 = as_h2((wd[j] & m1) | k1);
+              const h2 p2 = as_h2((hi & m0) | k0), p3 = as_h2((hi & m1) | k1);
+#pragma unroll
+              for (int m = 0; m < MR; ++m) {
+                acc0[m] = __builtin_amdgcn_fdot2(p0, as_h2(xr[m][j][0]), acc0[m], false);
+                acc1[m] = __builtin_amdgcn_fdot2(p1, as_h2(xr[m][j][1]), acc1[m], false);
+                acc0[m] = __builtin_amdgcn_fdot2(p2, as_h2(xr[m][j][2]), acc0[m], false);
+                acc1[m] = __builtin_amdgcn_fdot2(p3, as_h2(xr[m][j][3]), acc1[m], false);
+              }
+            } else {  // bytes (q0,q1,q2,q3) -> (1024 + q0, 1024 + q1), (1024 + q2, 1024 + q3): natural order
+              const int u = j >> 1, e = (j & 1) * 2;
+              const h2 p0 = as_h2(__builtin_amdgcn_perm(0x64646464u, wd[j], 0x04010400u));
+              const h2 p1 = as_h2(__builtin_amdgcn_perm(0x64646464u, wd[j], 0x04030402u));
+#pragma unroll
+              for (int m = 0; m < MR; ++m) {
+                acc0[m] = __builtin_amdgcn_fdot2(p0, as_h2(xr[m][u % kXU][e]), acc0[m], false);
+                acc1[m] = __builtin_amdgcn_fdot2(p1, as_h2(xr[m][u % kXU][e + 1]), acc1[m], false);
+              }
+            }
+          }
+          const float sc = __half2float(__ushort_as_half((unsigned short)t.s[cc][r]));
+          const float bi = __half2float(__ushort_as_half((unsigned short)t.b[cc][r]));
+#pragma unroll
+          for (int m = 0; m < MR; ++m) racc[r][m] += sc * ((acc0[m] + acc1[m]) - k[m].x) + bi * k[m].y;
+        }
+      }
+    }
+    pr_c0 += 2;
+    if (pr_c0 >= KH) {  // the block is complete
+      float mine = 0.f;
+#pragma unroll
+      for (int r = 0; r < R; ++r)
+#pragma unroll
+        for (int m = 0; m < MR; ++m) {
+          const float t2 = wave_sum(racc[r][m]);
+          mine = lane == r * MR + m ? t2 : mine;
+        }
+      if (writes) {  // residual add / SwiGLU gate in f32, one rounding (quantized.rs:3206-3246)
+        if (p.epi_kind == EPI_RESIDUAL) mine += epi_val;
+        else if (p.epi_kind == EPI_SWIGLU) mine = epi_val / (1.0f + __expf(-epi_val)) * mine;
+        p.out[(uint64_t)out_m * p.N + block_row0(pr_blk) + lane / MR] = __float2half(mine);
+      }
+      pr_c0 = 0;
+      ++pr_blk;
+    }
+  };
+  for (uint32_t u = 0; u < n_batches; u += 2) {
+    const bool more1 = u + 1 < n_batches, more2 = u + 2 < n_batches;
+    if (more1) load_batch(bb);
+    process(ba);
+    if (more1) {
+      if (more2) load_batch(ba);
+      process(bb);
+    }
   }
 }
 
@@ -320,24 +590,63 @@ size_t lds_per_row(uint32_t K) {
   return chunks * (chunk_k * 2 + 64 * sizeof(float2));
 }
 
-template <int BITS, int R, bool NT, int MR>
+// Workgroups of `kernel` that the chip keeps resident at once (per-instantiation cache, keyed by the LDS size).
+template <typename Kernel>
+uint32_t resident_workgroups(Kernel kernel, size_t lds) {
+  static size_t cached_lds = ~(size_t)0;
+  static uint32_t cached = 0;
+  if (cached_lds != lds) {
+    int per_cu = 0;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, kThreads, lds) != hipSuccess || per_cu < 1) per_cu = 1;
+    cached = (uint32_t)per_cu * (uint32_t)ctx().num_cus;
+    cached_lds = lds;
+  }
+  return cached;
+}
+
+template <int BITS, int GS, int R, bool NT, int MR, bool NORM, int KP = 1>
+void launch_k(const M1Params& p, size_t lds, hipStream_t s) {
+  if constexpr (KP > 1) {  // split rows: short matrices only, every row group has its workgroup
+    hipLaunchKernelGGL((qmv_m1_kernel<BITS, GS, R, NT, MR, NORM, KP>), dim3(p.N / (kWaves / KP), (p.M + MR - 1) / MR),
+                       dim3(kThreads), lds, s, p);
+    return;
+  }
+  // one workgroup per row block while all of them are resident together, else as many as are (they loop)
+  auto looping = qmv_m1_loop_kernel<BITS, GS, R, NT, MR, NORM>;
+  const uint32_t nblk = p.N / (kWaves * R), passes = (p.M + MR - 1) / MR;
+  uint32_t gx = resident_workgroups(looping, lds) / passes;
+  gx = gx < 1 ? 1 : gx;
+  // (as many workgroups as are resident, even where that leaves some of them one block more than others: fewer
+  // workgroups with equal shares are slower, 8.1 against 6.7 us at N = 9216)
+  if (gx < nblk) hipLaunchKernelGGL(looping, dim3(gx, passes), dim3(kThreads), lds, s, p);
+  else hipLaunchKernelGGL((qmv_m1_kernel<BITS, GS, R, NT, MR, NORM>), dim3(nblk, passes), dim3(kThreads), lds, s, p);
+}
+
+template <int BITS, int R, bool NT, int MR, int KP = 1>
 void launch_r(const M1Params& p, uint32_t group_size, hipStream_t s) {
-  const dim3 grid(p.N / (kWaves * R), (p.M + MR - 1) / MR), block(kThreads);
   const size_t lds = (size_t)MR * lds_per_row<BITS>(p.K);
+  if constexpr (KP > 1) {
+    switch (group_size) {
+      case 32: launch_k<BITS, 32, R, NT, MR, false, KP>(p, lds, s); break;
+      case 64: launch_k<BITS, 64, R, NT, MR, false, KP>(p, lds, s); break;
+      default: launch_k<BITS, 128, R, NT, MR, false, KP>(p, lds, s); break;
+    }
+    return;
+  }
   if constexpr (NT && MR <= 2) {  // the prologue is fused for one or two rows in one pass
     if (p.norm_w != nullptr) {
       switch (group_size) {
-        case 32: hipLaunchKernelGGL((qmv_m1_kernel<BITS, 32, R, NT, MR, true>), grid, block, lds, s, p); break;
-        case 64: hipLaunchKernelGGL((qmv_m1_kernel<BITS, 64, R, NT, MR, true>), grid, block, lds, s, p); break;
-        default: hipLaunchKernelGGL((qmv_m1_kernel<BITS, 128, R, NT, MR, true>), grid, block, lds, s, p); break;
+        case 32: launch_k<BITS, 32, R, NT, MR, true>(p, lds, s); break;
+        case 64: launch_k<BITS, 64, R, NT, MR, true>(p, lds, s); break;
+        default: launch_k<BITS, 128, R, NT, MR, true>(p, lds, s); break;
       }
       return;
     }
   }
   switch (group_size) {
-    case 32: hipLaunchKernelGGL((qmv_m1_kernel<BITS, 32, R, NT, MR>), grid, block, lds, s, p); break;
-    case 64: hipLaunchKernelGGL((qmv_m1_kernel<BITS, 64, R, NT, MR>), grid, block, lds, s, p); break;
-    default: hipLaunchKernelGGL((qmv_m1_kernel<BITS, 128, R, NT, MR>), grid, block, lds, s, p); break;
+    case 32: launch_k<BITS, 32, R, NT, MR, false>(p, lds, s); break;
+    case 64: launch_k<BITS, 64, R, NT, MR, false>(p, lds, s); break;
+    default: launch_k<BITS, 128, R, NT, MR, false>(p, lds, s); break;
   }
 }
 
@@ -357,6 +666,16 @@ void launch_bits(const M1Params& p, uint32_t group_size, hipStream_t s) {
     // tall matrices (the activation registers read from LDS serve both rows; measured 3-9 % from N = 12288
     // on; the 8-bit kernel reads half as many activations per weight byte and is faster with one), else one
     const bool two = (p.K >= 12288 || (BITS == 4 && p.N >= 12288)) && p.N % (kWaves * 2) == 0;
+    // Long rows of a short matrix (the reference's split-K case, K > 8192 and N <= 2048, quantized.rs:7246-7250):
+    // with one wave per row the grid would not fill the chip, so 2 or 4 waves share a row until there are two
+    // workgroups per CU (every wave keeps at least two chunks).
+    const uint32_t chunks = (p.K * BITS + 8191) / 8192, cus = (uint32_t)ctx().num_cus;
+    int kp = 1;
+    while (kp < 4 && p.N / kWaves * kp < 2 * cus && chunks >= 4u * kp && p.N % (kWaves / (2 * kp)) == 0) kp *= 2;
+    if (kp > 1 && p.norm_w == nullptr && one_pass) {
+      if (kp == 2) launch_r<BITS, 1, true, 1, 2>(p, group_size, s); else launch_r<BITS, 1, true, 1, 4>(p, group_size, s);
+      return;
+    }
     if (one_pass) {
       if (two) launch_r<BITS, 2, true, 1>(p, group_size, s); else launch_r<BITS, 1, true, 1>(p, group_size, s);
     } else {

@@ -532,6 +532,54 @@ def test_single_row_gemv(hip, bits, gs, n, k):
                      f"qmv bits={bits} gs={gs} N={n} K={k} M={m}")
 
 
+@pytest.mark.parametrize("n,k,bits,gs", [(2048, 16384, 4, 64), (1024, 12288, 8, 64), (64, 8192, 4, 32),
+                                         (136, 16384, 4, 128), (520, 10240, 8, 128), (8, 16384, 4, 64)])
+def test_single_row_split_k(hip, n, k, bits, gs):
+    """Long rows of a short matrix (the reference's split-K case `K > 8192 && N <= 2048`, quantized.rs:992-1233,
+    7246-7250): two or four waves share a weight row and add their partial sums in workgroup memory.  Against the
+    oracle, with one-hot activations in every 1 KB chunk of a row (each lands in another wave), and through the
+    fused store epilogues."""
+    from rmlx_amd import ops
+    from rmlx_amd.runtime import DeviceBuffer
+    rng = np.random.default_rng(n + k + bits + gs)
+    words, s, b = make_weight(rng, n, k, bits, gs)
+    x = make_x(rng, 1, k)
+    ref = model.qmm(x_as_f64(x, "f16"), words, s, b, gs, bits)
+    assert_close(_run(hip, words, s, b, x, bits, gs=gs), ref, f"split-K N={n} K={k} bits={bits} gs={gs}")
+    assert_close(_run(hip, words, s, b, x, bits, gs=gs, qmv_entry=True), ref, "through the qmv entry point")
+    q = model.unpack_u32(words, bits).astype(np.float64)
+    chunk = 8192 // bits
+    for kk in sorted({c * chunk + off for c in range(k // chunk) for off in (0, chunk - 1)} | {k - 1}):
+        x1 = np.zeros((1, k), np.float16)
+        x1[0, kk] = 1.0
+        out = _run(hip, words, np.ones_like(s), np.zeros_like(b), x1, bits, gs=gs)
+        assert np.array_equal(out[0].astype(np.float64), q[:, kk]), f"k={kk}"
+    e = rng.standard_normal((1, n)).astype(np.float32)
+    qw = ops.QuantizedWeight.from_numpy(words, s, b, gs, bits)
+    xd, ed = DeviceBuffer.from_numpy(x), DeviceBuffer.from_numpy(e)
+    assert_close(ops.qmm_add_residual(xd, qw, ed).numpy(), ref + e, "split-K + residual")
+    assert_close(ops.qmm_swiglu(xd, qw, ed).numpy(), model.silu(e.astype(np.float64)) * ref, "split-K + SwiGLU")
+
+
+@pytest.mark.parametrize("n,k,bits,m", [(16400, 2048, 4, 1), (9216, 4096, 4, 1), (24584, 1024, 8, 2), (33000, 2048, 4, 3)])
+def test_single_row_gemv_more_row_blocks_than_resident_workgroups(hip, n, k, bits, m):
+    """Tall matrices: the grid is sized to the workgroups the chip keeps resident and each of them walks several
+    row blocks (an uneven share included); every output row against the oracle, plain and with the residual
+    epilogue (whose operand is fetched per block)."""
+    from rmlx_amd import ops
+    from rmlx_amd.runtime import DeviceBuffer
+    rng = np.random.default_rng(n + k + bits)
+    gs = 128 if m == 3 else 64  # (three rows stay on this kernel because N = 33000 is no multiple of 16, which the multi-row GEMV needs)
+    words, s, b = make_weight(rng, n, k, bits, gs)
+    x = make_x(rng, m, k)
+    ref = model.qmm(x_as_f64(x, "f16"), words, s, b, gs, bits)
+    assert_close(_run(hip, words, s, b, x, bits, gs=gs), ref, f"looping grid N={n} K={k} bits={bits} M={m}")
+    e = rng.standard_normal((m, n)).astype(np.float16)
+    qw = ops.QuantizedWeight.from_numpy(words, s, b, gs, bits)
+    out = ops.qmm_add_residual(DeviceBuffer.from_numpy(x), qw, DeviceBuffer.from_numpy(e)).numpy()
+    assert_close(out, ref + e.astype(np.float64), "looping grid + residual")
+
+
 @pytest.mark.parametrize("bits", [4, 8])
 def test_single_row_gemv_positions_and_multi_row_kernel_agree(hip, bits):
     """One-hot activations pick out single weights exactly (every k position of a lane, chunk borders), and
