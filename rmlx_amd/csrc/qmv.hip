@@ -309,6 +309,9 @@ __global__ __launch_bounds__(kThreads, (REUSE != 0 && MR == 8 && TILES == 2) ? 4
             F[t][2] += sc * (c[t][2] + c23[0]) + bi * c23[1];
             F[t][3] += sc * (c[t][3] + c23[2]) + bi * c23[3];
           }
+          // (keeps the operand reads of later slabs from being hoisted above this one: they would cost the registers
+          // that let a third workgroup share the CU)
+          if constexpr (MR < 8 && TILES == 1) __builtin_amdgcn_sched_barrier(0);
         }
       }
     } else {
@@ -405,7 +408,25 @@ __global__ __launch_bounds__(kThreads, (REUSE != 0 && MR == 8 && TILES == 2) ? 4
   }
   };
 
-  if constexpr (REUSE == 1) {
+  if constexpr (REUSE == 1 && MR < 8) {
+    // one pass, one tile per workgroup (the launcher gives these kernels no more): straight-line code, which keeps
+    // the registers low enough for a third resident workgroup per CU
+    const int sl = (int)(kp * SPW);
+    u4 sbv[TILES];
+    u4 wreg[TILES][kSpwMax];
+    {
+      u4 xv[MR];
+      load_x(sl, SPW, xv);
+      load_tile(blockIdx.x, sl, SPW, sbv, wreg);
+      stage_x(xv);
+      stage_sums();
+    }
+    f4 F[TILES];
+#pragma unroll
+    for (int t = 0; t < TILES; ++t) F[t] = (f4){0.f, 0.f, 0.f, 0.f};
+    compute_tile(SPW, sbv, wreg, F);
+    finish_tile(blockIdx.x, F, true);
+  } else if constexpr (REUSE == 1) {
     // one pass: slabs kp*SPW .. of every tile; the activations and the first tile's weights are requested together.
     // (Eight rows: a second register set for the next tile's weights would cost the second workgroup per CU,
     // which hides more latency than the prefetch; measured.)
@@ -588,7 +609,7 @@ int32_t launch_qmv_q4(const QmvArgs& a, hipStream_t s) {
     for (int pass = tab ? 0 : 1; pass < 2 && tpw == 1; ++pass)
       for (uint32_t c : cand)
         if (tiles_x % c == 0 && (pass == 1 || (tiles_x / c) % 8 == 0) &&
-            (uint64_t)(tiles_x / c) * chunks >= (tab ? 2ull : 1ull) * (uint32_t)ctx().num_cus) { tpw = c; break; }
+            (uint64_t)(tiles_x / c) * chunks >= 2ull * (uint32_t)ctx().num_cus) { tpw = c; break; }
   }
   p.tpw = tpw;
   dim3 grid(tiles_x / tpw, chunks);
