@@ -280,7 +280,7 @@ int32_t rmlx_hip_moe_forward_grouped(const rmlx_qweight* gate, const rmlx_qweigh
  * grouped MFMA GEMM -- row tiles of 16, 32 or 64 rows of one expert, weights dequantised in registers; 4- / 8-bit,
  * group sizes 32 / 64 / 128 (one for the three projections), hidden and intermediate dimensions in multiples of
  * 512 -- smaller ones with the streaming GEMV, which reads an expert's weights once per 8 rows (8-bit experts
- * switch at an eighth of `min_rows`, rounded up).  0 = never the GEMM; the default (6) is the measured crossover.
+ * switch at an eighth of `min_rows`, rounded up).  0 = never the GEMM; the default (8) is the measured crossover.
  * The value lives in the handle of the stacked GATE weight and applies to the calls that pass that handle: there
  * is no process-wide state.  Set it before other threads use the handle.  The counterpart of choosing a
  * `MoeStrategy` for a layer in the reference (crates/rmlx-nn/src/moe.rs:515-541).  Returns the previous value. */

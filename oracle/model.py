@@ -36,6 +36,39 @@ def unpack_u32(words, bits):
     return vals.reshape(words.shape[:-1] + (words.shape[-1] * per,)).astype(np.uint8)
 
 
+def words_per_group(group_size, bits):
+    """`u32s_per_group = group_size / (32 / bits)` of the reference's portable kernel `affine_qmv`
+    (crates/rmlx-core/src/ops/quantized.rs:232-236), both divisions rounding down: 3 / 6 / 12 words of 10 values at
+    3 bits, 6 / 12 / 25 words of 5 values at 6 bits (group sizes 32 / 64 / 128)."""
+    return group_size // (32 // bits)
+
+
+def pack_grouped(q, group_size, bits):
+    """Row layout `affine_qmv` reads (quantized.rs:232-270): the words of group 0, then of group 1, ...; value k of word w
+    of group g is element g * group_size + w * (32 / bits) + k.  Elements of a group past its last whole word get no
+    word.  Equal to `pack_u32` at 2, 4 and 8 bits.  q [..., K] -> u32 [..., K / group_size * words_per_group]."""
+    q = np.asarray(q, dtype=np.uint32)
+    per, wpg = 32 // bits, words_per_group(group_size, bits)
+    g = q.reshape(q.shape[:-1] + (q.shape[-1] // group_size, group_size))[..., : wpg * per]
+    g = g.reshape(g.shape[:-1] + (wpg, per))
+    shifts = np.arange(per, dtype=np.uint32) * np.uint32(bits)
+    w = np.bitwise_or.reduce(g << shifts, axis=-1).astype(np.uint32)
+    return w.reshape(w.shape[:-2] + (w.shape[-2] * wpg,))
+
+
+def unpack_grouped(words, group_size, bits):
+    """Inverse of `pack_grouped`: (values [..., K] with zeros where a group has no word, covered [K] bool)."""
+    words = np.asarray(words, dtype=np.uint32)
+    per, wpg = 32 // bits, words_per_group(group_size, bits)
+    groups = words.shape[-1] // wpg
+    vals = unpack_u32(words, bits).reshape(words.shape[:-1] + (groups, wpg * per))
+    q = np.zeros(words.shape[:-1] + (groups, group_size), np.uint8)
+    q[..., : wpg * per] = vals
+    covered = np.zeros((groups, group_size), bool)
+    covered[:, : wpg * per] = True
+    return q.reshape(words.shape[:-1] + (groups * group_size,)), covered.reshape(-1)
+
+
 def words_to_bytes(words):
     """Byte image the reference's CPU path consumes: for Q4 low nibble = even k, for Q8 one
     byte per value; equal to the little-endian bytes of the u32 words
@@ -78,9 +111,16 @@ def dequantize(words, scales, biases, group_size, bits):
     [3,5,10,1] -> [6.5,10.5,20.5,2.5] known answer (:10601-10624) and by agreement with the C
     restatement of `dequantize_q4_row`.
     """
-    q = unpack_u32(words, bits).astype(np.float64)
     s = np.repeat(np.asarray(scales, dtype=np.float64), group_size, axis=-1)
     b = np.repeat(np.asarray(biases, dtype=np.float64), group_size, axis=-1)
+    if 32 % bits != 0:
+        # 3 and 6 bits, layout and coverage of `affine_qmv` (quantized.rs:232-270, the only kernel of the reference
+        # that takes them): an element without a word adds nothing to `scale * sum(q x) + bias * sum(x)`, i.e. its
+        # weight is 0.  No test or fixture of the reference holds such a weight; pinned in tests/ by a loop-for-loop
+        # restatement of the kernel on small shapes and by the closed forms its coverage fixes.
+        q, covered = unpack_grouped(words, group_size, bits)
+        return np.where(covered, s * q.astype(np.float64) + b, 0.0)
+    q = unpack_u32(words, bits).astype(np.float64)
     return s * q + b
 
 

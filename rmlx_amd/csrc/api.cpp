@@ -376,7 +376,7 @@ int32_t check_expert_weights(const char* who, const rmlx_qweight* gate, const rm
   for (const rmlx_qweight* q : all) {
     if (q == nullptr) continue;
     if (q->bits != 2 && q->bits != 4 && q->bits != 8)
-      return fail(RMLX_NOT_FOUND, "%s: no kernel for %u-bit expert weights (2, 4 and 8 are implemented)", who, q->bits);
+      return fail(RMLX_NOT_FOUND, "%s: no kernel for %u-bit expert weights (2, 4 and 8 are implemented; 3- and 6-bit weights run on the matmul entry points)", who, q->bits);
     // the streaming kernels take 4-bit weights with group size 64 or 128 and 8-bit weights with group size 64,
     // the same width for all three projections (gate and up share one launch)
     const bool gs_ok = q->bits == 4 ? (q->group_size == 64 || q->group_size == 128) : (q->bits == 8 && q->group_size == 64);

@@ -90,7 +90,7 @@ struct rmlx_qweight {
   size_t n_experts;     // 1 for a plain linear weight
   // stacked expert weights: average rows per expert from which the expert projections run on the grouped MFMA GEMM
   // instead of the streaming GEMV (read from the gate weight of a block; 0 = never)
-  uint32_t expert_gemm_min_rows = 6;
+  uint32_t expert_gemm_min_rows = 8;
 };
 
 namespace rmlx {

@@ -54,9 +54,14 @@ __global__ __launch_bounds__(64) void generic_qmm_kernel(GenericArgs a) {
   const uint32_t m0 = batch * rpi + (blockIdx.y % passes) * kGenRows;
   const uint32_t mend = (batch + 1) * rpi < a.M ? (batch + 1) * rpi : a.M;
   const uint32_t lane = threadIdx.x;
-  const uint32_t per = 32 / a.bits;            // values per word (bits in {2,4,8})
-  const uint32_t words = a.K / per;
+  // Layout of the reference's affine_qmv (quantized.rs:210-291): 32 / bits values per word, group_size / (32 / bits)
+  // words per group, a row is its groups' words one after another.  At 2, 4 and 8 bits that is the flat packing; at
+  // 3 and 6 bits a word holds 10 / 5 values (2 bits unused) and the values of a group past its last whole word
+  // (2 of 32, 4 of 64, 8 of 128) have no word: they count for nothing, in the product and in the bias term alike.
+  const uint32_t per = 32 / a.bits;
+  const uint32_t wpg = a.group_size / per;
   const uint32_t gpr = a.K / a.group_size;
+  const uint32_t words = gpr * wpg;
   const uint32_t mask = (1u << a.bits) - 1u;
 
   float acc[kGenRows] = {0.f, 0.f, 0.f, 0.f};
@@ -72,11 +77,10 @@ __global__ __launch_bounds__(64) void generic_qmm_kernel(GenericArgs a) {
     const __half* brow = a.b + ((uint64_t)expert * a.N + nrow) * gpr;
     for (uint32_t wi = lane; wi < words; wi += 64) {
       const uint32_t word = wrow[wi];
+      const uint32_t grp = wi / wpg, kbase = grp * a.group_size + (wi % wpg) * per;
       for (uint32_t i = 0; i < per; ++i) {
-        const uint32_t k = wi * per + i;
-        if (k >= a.K) break;
+        const uint32_t k = kbase + i;
         const float q = (float)((word >> (i * a.bits)) & mask);
-        const uint32_t grp = k / a.group_size;
         const float wv = __half2float(srow[grp]) * q + __half2float(brow[grp]);
 #pragma unroll
         for (int r = 0; r < kGenRows; ++r)
@@ -138,8 +142,8 @@ int32_t launch_cast_f16_to_f32(const __half* src, float* dst, size_t n, hipStrea
 
 int32_t launch_generic(const GenericArgs& a, hipStream_t s) {
   if (a.M == 0 || a.N == 0) return RMLX_OK;
-  if (a.bits != 2 && a.bits != 4 && a.bits != 8)
-    return fail(RMLX_NOT_FOUND, "no kernel for %u-bit weights (2, 4 and 8 are implemented)", a.bits);
+  if (a.bits != 2 && a.bits != 3 && a.bits != 4 && a.bits != 6 && a.bits != 8)
+    return fail(RMLX_NOT_FOUND, "no kernel for %u-bit weights", a.bits);
   GenericArgs k = a;
   if (k.indices == nullptr) k.rows_per_index = a.M;
   const uint32_t batches = (a.M + k.rows_per_index - 1) / k.rows_per_index;

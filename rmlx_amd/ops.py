@@ -32,12 +32,21 @@ class QuantizedWeight:
 
     @classmethod
     def from_numpy(cls, words, scales, biases, group_size, bits):
-        """words u32 [N, K*bits/32] or [E, N, ...]; scales/biases f16."""
+        """words u32 [N, K*bits/32] or [E, N, ...]; scales/biases f16 [.., N, K/group_size].  (3 and 6 bits: the
+        rows hold whole words per group, K / group_size * (group_size // (32 // bits)) of them.)"""
         words = np.ascontiguousarray(words, np.uint32)
+        scales = np.ascontiguousarray(scales, np.float16)
         e = words.shape[0] if words.ndim == 3 else 1
         n = words.shape[-2]
-        k = words.shape[-1] * 32 // bits
-        return cls(DeviceBuffer.from_numpy(words), DeviceBuffer.from_numpy(np.ascontiguousarray(scales, np.float16)),
+        k = scales.shape[-1] * group_size
+        if 32 % bits != 0:
+            # the constructor follows the reference's size check, ceil(N * K / (32 // bits)) words, which is more
+            # than the rows of this layout occupy: pad the buffer
+            need = -(-(e * n * k) // (32 // bits))
+            flat = np.zeros(max(need, words.size), np.uint32)
+            flat[:words.size] = words.reshape(-1)
+            words = flat
+        return cls(DeviceBuffer.from_numpy(words), DeviceBuffer.from_numpy(scales),
                    DeviceBuffer.from_numpy(np.ascontiguousarray(biases, np.float16)), group_size, bits, n, k, e)
 
     def set_expert_gemm_min_rows(self, min_rows):

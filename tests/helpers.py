@@ -6,8 +6,8 @@ from oracle import model
 
 def make_weight(rng, n, k, bits=4, group_size=64, lead=()):
     """Uniform q, f16 scale ~ U[lo,hi], bias = -(2^(bits-1)) * scale (exact in f16)."""
-    lo, hi = (0.005, 0.02) if bits == 4 else (0.0005, 0.002)
-    shape = tuple(lead) + (n, k * bits // 32)
+    lo, hi = (0.005, 0.02) if bits <= 4 else (0.0005, 0.002)
+    shape = tuple(lead) + (n, k // group_size * model.words_per_group(group_size, bits))  # k * bits / 32 at 2, 4, 8 bits
     words = rng.integers(0, 2**32, size=shape, dtype=np.uint64).astype(np.uint32)
     scales = rng.uniform(lo, hi, size=tuple(lead) + (n, k // group_size)).astype(np.float16)
     biases = (-(2.0 ** (bits - 1)) * scales.astype(np.float32)).astype(np.float16)

@@ -77,10 +77,10 @@ def test_expert_gemm_threshold_lives_in_the_handle():
         assert L.rmlx_hip_qweight_create(ctypes.c_void_p(16), 1 << 20, ctypes.c_void_p(16), 1 << 20, ctypes.c_void_p(16), 1 << 20,
                                          64, 4, 64, 64, 2, ctypes.byref(h)) == rt.OK
     try:
-        assert L.rmlx_hip_qweight_set_expert_gemm_min_rows(hs[0], 5) == 6
+        assert L.rmlx_hip_qweight_set_expert_gemm_min_rows(hs[0], 5) == 8
         assert L.rmlx_hip_qweight_set_expert_gemm_min_rows(hs[0], 0) == 5
-        assert L.rmlx_hip_qweight_set_expert_gemm_min_rows(hs[1], 9) == 6  # the other handle kept its default
-        assert L.rmlx_hip_qweight_set_expert_gemm_min_rows(hs[0], 6) == 0
+        assert L.rmlx_hip_qweight_set_expert_gemm_min_rows(hs[1], 9) == 8  # the other handle kept its default
+        assert L.rmlx_hip_qweight_set_expert_gemm_min_rows(hs[0], 8) == 0
     finally:
         for h in hs:
             L.rmlx_hip_qweight_destroy(h)

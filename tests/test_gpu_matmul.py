@@ -513,6 +513,35 @@ def test_qmv_paired_tiles(hip, m, n, k):
     assert_close(_run(hip, words, s, b, x, 4, kernel=1), ref, f"qmv paired M={m} N={n} K={k}")
 
 
+# ---- 3- and 6-bit weights (the reference's portable affine_qmv, quantized.rs:210-291) ---------------------
+
+@pytest.mark.parametrize("bits", [3, 6])
+@pytest.mark.parametrize("gs", [32, 64, 128])
+@pytest.mark.parametrize("n,k", [(24, 256), (7, 1024), (130, 384)])
+def test_three_and_six_bit_weights(hip, bits, gs, n, k):
+    """The bit widths the weight type admits beside 2 / 4 / 8: `affine_quantized_matmul` runs them on the portable
+    kernel with the reference's layout (10 / 5 values per word, whole words per group), the batched entry point
+    rejects them like the reference's and takes them when the portable kernel is selected."""
+    from rmlx_amd import ops, runtime as rt
+    if k % gs != 0:
+        pytest.skip("group size does not divide K")
+    rng = np.random.default_rng(bits * 1000 + gs + n + k)
+    words, s, b = make_weight(rng, n, k, bits, gs)
+    x = make_x(rng, 5, k)
+    ref = model.qmm(x_as_f64(x, "f16"), words, s, b, gs, bits)
+    assert_close(_run(hip, words, s, b, x[:1], bits, gs=gs, qmv_entry=True), ref[:1], f"qmv bits={bits} gs={gs}")
+    assert_close(_run(hip, words, s, b, x, bits, gs=gs, kernel=rt.KERNEL_GENERIC), ref, f"portable bits={bits} gs={gs} M=5")
+    with pytest.raises(ops.KernelError, match="affine_quantized_matmul_batched requires bits==4 or bits==8"):
+        _run(hip, words, s, b, x, bits, gs=gs)
+    # every covered position picks out its value exactly; the positions of a group past its last whole word give 0
+    q, covered = model.unpack_grouped(words, gs, bits)
+    for kk in sorted({0, 1, 32 // bits - 1, 32 // bits, gs - 1, gs, gs + 9, k - gs, k - 1}):
+        x1 = np.zeros((1, k), np.float16)
+        x1[0, kk] = 1.0
+        out = _run(hip, words, np.ones_like(s), np.zeros_like(b), x1, bits, gs=gs, qmv_entry=True)
+        assert np.array_equal(out[0].astype(np.float64), q[:, kk].astype(np.float64) * covered[kk]), f"k={kk}"
+
+
 # ---- single-row GEMV (decode; affine_qmv_fast_q4 / _q8, quantized.rs:394-695) ---------------------------
 
 @pytest.mark.parametrize("bits", [4, 8])
