@@ -108,6 +108,14 @@ __device__ __forceinline__ float swap8(float v) {  // value of lane ^ 8
 
 struct __attribute__((packed, aligned(4))) U4Unaligned { uint32_t v[4]; };
 
+// Workgroup barrier for data exchanged through LDS: waits for this wave's LDS traffic only.  (__syncthreads() also
+// waits for every global load in flight, i.e. for the next tile's weights that were requested on purpose.)
+__device__ __forceinline__ void lds_barrier() {
+  asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+  __builtin_amdgcn_s_barrier();
+  asm volatile("" ::: "memory");
+}
+
 // MR = activation rows staged per pass (1, 2, 4 or 8); TILES = 1, or 2 (fused gate/up, or two
 // 16-row tiles of one matrix sharing the staged activations: PAIR);
 // TAB = rows come from a device chunk table (gather_qmm, MoE); SPW = slabs per wave and pass when
@@ -359,7 +367,7 @@ __global__ __launch_bounds__(kThreads, (REUSE != 0 && MR == 8 && TILES == 2) ? 4
   auto finish_tile = [&](uint32_t wg_tile, f4 (&F)[TILES], bool first_tile) {
   // ---- 4. reduce over the two group halves (lane + 32 holds the other one) and over the
   //         k-parts, write out -------------------------------------------------------------------
-  __syncthreads();  // the previous tile's sums have been read
+  lds_barrier();  // the previous tile's sums have been read
   // (index arithmetic of this part is kept inside the tile loop on purpose: hoisted out, it
   // costs registers for the whole kernel)
   uint32_t tid_t = tid;
@@ -374,7 +382,7 @@ __global__ __launch_bounds__(kThreads, (REUSE != 0 && MR == 8 && TILES == 2) ? 4
         if (g_t < 2) red[((wave_t * TILES + t) * 8 + g_t * 4 + i) * 16 + n_t] = v;
       }
   }
-  __syncthreads();
+  lds_barrier();
   for (uint32_t o = tid_t; o < NT * 128; o += kThreads) {
     const uint32_t otw = o >> 7, m = (o >> 4) & 7, nn = o & 15;
     if (m < rows) {
