@@ -140,7 +140,8 @@ __global__ __launch_bounds__(kThreads, (REUSE != 0 && MR == 8 && TILES == 2) ? 4
   constexpr bool kPreSums = REUSE != 0;
   __shared__ __attribute__((aligned(16))) float sums_all[!kPreSums ? 4 : kWaves * kSpwMax * 2 * 8 * 2];  // [wave][group][row][-xoff, xsum]
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // (in a scalar register, with everything derived from it)
   const int n = lane & 15;   // weight row within the tile / accumulator column
   const int g = lane >> 4;   // k sub-block of the slab / accumulator row group
   const int par = g >> 1;    // which of the slab's two quantisation groups this lane scales
@@ -234,6 +235,11 @@ __global__ __launch_bounds__(kThreads, (REUSE != 0 && MR == 8 && TILES == 2) ? 4
     const uint32_t tile_row = (wg_tile * NT + tw) * rows_per_slot;
     const u4* wrow[TILES];
     const __half* sbrow[TILES];
+    // (the lane's part of the addresses is recomputed per tile on purpose: kept across the tile loop it costs
+    // registers the 8-row kernels do not have)
+    uint32_t lane_l = lane;
+    asm volatile("" : "+v"(lane_l));
+    const uint32_t n = lane_l & 15, g = lane_l >> 4;
   #pragma unroll
     for (int t = 0; t < TILES; ++t) {
       const uint64_t e_w = TAB ? expert * p.estride_w : 0, e_s = TAB ? expert * p.estride_s : 0;
@@ -319,7 +325,7 @@ __global__ __launch_bounds__(kThreads, (REUSE != 0 && MR == 8 && TILES == 2) ? 4
           }
           // (keeps the operand reads of later slabs from being hoisted above this one: they would cost the registers
           // that let a third workgroup share the CU)
-          if constexpr (MR < 8 && TILES == 1) __builtin_amdgcn_sched_barrier(0);
+          __builtin_amdgcn_sched_barrier(0);
         }
       }
     } else {
@@ -364,9 +370,10 @@ __global__ __launch_bounds__(kThreads, (REUSE != 0 && MR == 8 && TILES == 2) ? 4
       }
     }
   };
-  auto finish_tile = [&](uint32_t wg_tile, f4 (&F)[TILES], bool first_tile) {
   // ---- 4. reduce over the two group halves (lane + 32 holds the other one) and over the
-  //         k-parts, write out -------------------------------------------------------------------
+  //         k-parts, write out.  In two steps, so that a tile loop can request the next tile's weights
+  //         between them, when the accumulators are free again. ----------------------------------------
+  auto reduce_halves = [&](f4 (&F)[TILES]) {
   lds_barrier();  // the previous tile's sums have been read
   // (index arithmetic of this part is kept inside the tile loop on purpose: hoisted out, it
   // costs registers for the whole kernel)
@@ -382,7 +389,11 @@ __global__ __launch_bounds__(kThreads, (REUSE != 0 && MR == 8 && TILES == 2) ? 4
         if (g_t < 2) red[((wave_t * TILES + t) * 8 + g_t * 4 + i) * 16 + n_t] = v;
       }
   }
+  };
+  auto reduce_parts_and_store = [&](uint32_t wg_tile) {
   lds_barrier();
+  uint32_t tid_t = tid;
+  asm volatile("" : "+v"(tid_t));
   for (uint32_t o = tid_t; o < NT * 128; o += kThreads) {
     const uint32_t otw = o >> 7, m = (o >> 4) & 7, nn = o & 15;
     if (m < rows) {
@@ -415,6 +426,10 @@ __global__ __launch_bounds__(kThreads, (REUSE != 0 && MR == 8 && TILES == 2) ? 4
     }
   }
   };
+  auto finish_tile = [&](uint32_t wg_tile, f4 (&F)[TILES], bool) {
+    reduce_halves(F);
+    reduce_parts_and_store(wg_tile);
+  };
 
   if constexpr (REUSE == 1 && MR < 8) {
     // one pass, one tile per workgroup (the launcher gives these kernels no more): straight-line code, which keeps
@@ -436,8 +451,10 @@ __global__ __launch_bounds__(kThreads, (REUSE != 0 && MR == 8 && TILES == 2) ? 4
     finish_tile(blockIdx.x, F, true);
   } else if constexpr (REUSE == 1) {
     // one pass: slabs kp*SPW .. of every tile; the activations and the first tile's weights are requested together.
-    // (Eight rows: a second register set for the next tile's weights would cost the second workgroup per CU,
-    // which hides more latency than the prefetch; measured.)
+    // One register set for the weights (eight rows: a second one would cost the second workgroup per CU, which
+    // hides more latency than it; measured): the next tile's weights are requested as soon as the products of the
+    // current tile have consumed the registers and the accumulators are on their way through LDS, and arrive while
+    // the partial sums are added up and written.
     const int sl = (int)(kp * SPW);
     const uint32_t first = blockIdx.x * ntiles;
     u4 sbv[TILES];
@@ -448,15 +465,17 @@ __global__ __launch_bounds__(kThreads, (REUSE != 0 && MR == 8 && TILES == 2) ? 4
       // (two tiles: their first weights do not fit beside the activations in the registers of four waves per SIMD)
       if constexpr (TILES == 1) load_tile(first, sl, SPW, sbv, wreg);
       stage_x(xv);
+      if constexpr (TILES == 2) load_tile(first, sl, SPW, sbv, wreg);
       stage_sums();
     }
     for (uint32_t ti = 0; ti < ntiles; ++ti) {
       f4 F[TILES];
-      if (TILES == 2 || ti > 0) load_tile(first + ti, sl, SPW, sbv, wreg);
 #pragma unroll
       for (int t = 0; t < TILES; ++t) F[t] = (f4){0.f, 0.f, 0.f, 0.f};
       compute_tile(SPW, sbv, wreg, F);
-      finish_tile(first + ti, F, ti == 0);
+      reduce_halves(F);
+      if (ti + 1 < ntiles) load_tile(first + ti + 1, sl, SPW, sbv, wreg);
+      reduce_parts_and_store(first + ti);
     }
   } else if constexpr (REUSE == 2) {  // fewer rows, several tiles: the weights of the next tile are in flight while this one is multiplied
     const int sl = (int)(kp * SPW);
