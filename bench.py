@@ -249,6 +249,26 @@ def bench_floors(rt, timer, launches):
     flops = info_blocks * 8 * iters * 16 * 16384
     floors["mfma_loop"] = {"us": ms * 1e3, "tflops": flops / (ms * 1e-3) / 1e12, "workgroups": info_blocks,
                            "frac_of_peak": flops / (ms * 1e-3) / 1e12 / MFMA_F16_PEAK_TF}
+    # the matrix rate with and-or instructions of a 4-bit unpacking on the vector ALU of the same SIMD
+    for v in (2, 4, 6, 8):
+        ms = timer.run(lambda c: go(rt.FLOOR_MFMA_VALU, None, blocks, v, iters, c), n_mfma, 5, chunk=20)
+        floors[f"mfma_loop_with_{v}_valu_per_mfma"] = {"us": ms * 1e3, "tflops": flops / (ms * 1e-3) / 1e12}
+    # LDS operand reads: bytes per clock and CU at 8 and 16 waves per CU
+    cus, clk = rt.device_info()["compute_units"], rt.device_info()["clock_khz"] * 1e3
+    for waves in (8, 16):
+        ms = timer.run(lambda c: go(rt.FLOOR_LDS, None, 0, waves, iters, c), n_mfma, 5, chunk=20)
+        per_cu = waves * 64 * 128 * iters
+        floors[f"lds_read_{waves}_waves"] = {"us": ms * 1e3, "bytes_per_clk_per_cu": per_cu / (ms * 1e-3 * clk),
+                                             "tbs_all_cus": per_cu * cus / (ms * 1e-3) / 1e12}
+    # reads that hit the L2 of every XCD (all workgroups walk one 2 MB source): the rate at which hits fill the CUs
+    nbytes = 2 << 20
+    src = rt.DeviceBuffer((nbytes // 4,), rt.U32)
+    rt.check(L.rmlx_hip_memset(src.ptr, 1, nbytes, None))
+    ms = timer.run(lambda c: go(rt.FLOOR_L2_READ, src.ptr, nbytes, 0, 256, c), n_mfma, 5, chunk=20)
+    per_cu = 2 * 256 * 32768
+    floors["l2_hit_read"] = {"us": ms * 1e3, "bytes_per_clk_per_cu": per_cu / (ms * 1e-3 * clk),
+                             "tbs_all_cus": per_cu * cus / (ms * 1e-3) / 1e12}
+    src.free()
     return floors
 
 

@@ -339,9 +339,18 @@ int32_t rmlx_hip_gptq_dequant(const void* qweight_dev, size_t qweight_bytes, con
  *                             loads in flight per lane, 512-thread workgroups; launch i reads copy i % n_src of
  *                             the n_src consecutive copies at src_dev (cycle more than the caches hold);
  *   RMLX_FLOOR_MFMA           `iters` rounds of 16 independent v_mfma_f32_16x16x32_f16 per wave, 8 waves per
- *                             workgroup, `bytes` workgroups (0 = two per CU): 8 * 16 * 16384 * iters flop each.
+ *                             workgroup, `bytes` workgroups (0 = two per CU): 8 * 16 * 16384 * iters flop each;
+ *   RMLX_FLOOR_MFMA_VALU      the same loop with n_src (2, 4, 6 or 8) and-or vector instructions behind every MFMA:
+ *                             the matrix rate left while the vector ALU unpacks beside it;
+ *   RMLX_FLOOR_LDS            `iters` rounds of eight conflict-free 16-byte LDS reads per lane, n_src (8 or 16)
+ *                             waves per workgroup, `bytes` workgroups (0 = one per CU): waves * 64 * 128 * iters
+ *                             bytes each;
+ *   RMLX_FLOOR_L2_READ        n_src workgroups (0 = two per CU) of 512 threads each read iters * 32 KB from a source
+ *                             of `bytes` bytes (a power of two, small enough to stay in one L2) that all of them
+ *                             walk: the rate at which L2 hits reach the CUs.
  * sink_dev: at least 16 bytes of device memory (never written in practice; keeps the work alive). */
-enum { RMLX_FLOOR_EMPTY = 0, RMLX_FLOOR_READ4 = 1, RMLX_FLOOR_READ8 = 2, RMLX_FLOOR_MFMA = 3, RMLX_FLOOR_READ2 = 4 };
+enum { RMLX_FLOOR_EMPTY = 0, RMLX_FLOOR_READ4 = 1, RMLX_FLOOR_READ8 = 2, RMLX_FLOOR_MFMA = 3, RMLX_FLOOR_READ2 = 4,
+       RMLX_FLOOR_MFMA_VALU = 5, RMLX_FLOOR_LDS = 6, RMLX_FLOOR_L2_READ = 7 };
 int32_t rmlx_hip_measure_floor(int32_t kind, const void* src_dev, size_t bytes, size_t n_src, uint32_t iters,
                                void* sink_dev, size_t count, rmlx_stream stream);
 
