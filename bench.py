@@ -64,10 +64,13 @@ class Timer:
         self.rt = rt
         self.stream = rt.Stream()
         self.e0, self.e1 = rt.Event(), rt.Event()
+        self.cap = 0  # --max-launches: also bounds the trains of the settle phase
 
     def run(self, fn, launches, warmup, chunk=TRAIN):
         """fn(c) enqueues c launches.  Warm-up, an untimed settle phase of about SETTLE_S, then `launches`
         launches between two events; returns milliseconds per launch."""
+        if self.cap > 0:
+            launches, warmup, chunk = min(launches, self.cap), min(warmup, self.cap), min(chunk, self.cap)
         fn(max(1, warmup))
         self.stream.sync()
         t0 = time.perf_counter()
@@ -364,6 +367,8 @@ def main():
     ap.add_argument("--only", default="", help="comma-separated sections: headline, floors, qmv, qmm, dequant, gather, moe, moe8, large")
     ap.add_argument("--quick", action="store_true", help="headline and floors only, short CPU baseline")
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--max-launches", type=int, default=0,
+                    help="cap on the launches of every timed run (for hardware-counter runs, where each dispatch is slow)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)")
@@ -378,9 +383,18 @@ def main():
     GiB = 1 << 30
     launches, warm = args.steps * TRAIN, args.warmup * TRAIN
     gemm_launches = max(launches, GEMM_MIN_LAUNCHES)
+    train_warm = TRAIN
+    if args.max_launches > 0:
+        launches, warm, gemm_launches = min(launches, args.max_launches), min(warm, args.max_launches), args.max_launches
+        train_warm = min(TRAIN, args.max_launches)
+        timer.cap = args.max_launches
+
+    def progress(what):  # (a line per section on stderr: long profiler runs are not silent)
+        print(f"[bench] {what}", file=sys.stderr, flush=True)
     traffic = measured_traffic()
 
     # ---- headline: Q4 qmv M=1 K=N=4096, weights cycled through > 1 GiB ---------------------------------
+    progress("headline")
     head = bench_matmul(ops, rt, timer, rng, 1, 4096, 4096, 4, "f16", launches, warm, GiB + GiB // 8)
     extra = {"device": info, "launches_per_step": TRAIN, "q4_qmv_m1_4096": head}
     # A plain copy of known size (identity `index_gather`, 128 MiB in, 128 MiB out) so that a counter
@@ -394,8 +408,10 @@ def main():
                                  "write_bytes": rows * 4096 * 2}
     del src, ident
     if "floors" in sections:
+        progress("floors")
         extra["floors"] = bench_floors(rt, timer, launches)
     if "qmv" in sections:
+        progress("qmv")
         extra["q4_qmv_m1_4096_cache_resident"] = bench_matmul(ops, rt, timer, rng, 1, 4096, 4096, 4, "f16",
                                                               launches, warm, 0, check=False)
         for m in (1, 4, 8):
@@ -405,25 +421,29 @@ def main():
         extra["q8_qmv_m1_4096"] = bench_matmul(ops, rt, timer, rng, 1, 4096, 4096, 8, "f16", launches, warm, GiB + GiB // 8)
         # long K, short N: the shapes the reference sends to its split-K GEMV (K > 8192 and N <= 2048)
         extra["q4_qmv_m1_n2048_k16384"] = bench_matmul(ops, rt, timer, rng, 1, 2048, 16384, 4, "f16", launches, warm, GiB + GiB // 8)
-    if "large" in sections:  # launches long enough that start-up cost no longer matters
+    if "large" in sections:
+        progress("large")  # launches long enough that start-up cost no longer matters
         big = max(400, launches // 10)
-        extra["q4_qmv_m1_n32768"] = bench_matmul(ops, rt, timer, rng, 1, 32768, 4096, 4, "f16", big, TRAIN, GiB + GiB // 8)
+        extra["q4_qmv_m1_n32768"] = bench_matmul(ops, rt, timer, rng, 1, 32768, 4096, 4, "f16", big, train_warm, GiB + GiB // 8)
         extra["q4_qmv_m1_n151936"] = bench_matmul(ops, rt, timer, rng, 1, 151936, 4096, 4, "f16", max(100, big // 4), 20,
                                                   GiB + GiB // 8, check_rows=4096)
     if "qmm" in sections:
+        progress("qmm")
         for m in (128, 512, 4096):
             m_launches = gemm_launches if m <= 512 else max(50, gemm_launches // 10)
-            r = bench_matmul(ops, rt, timer, rng, m, 4096, 4096, 4, "f16", m_launches, TRAIN, 4 * 9437184)
+            r = bench_matmul(ops, rt, timer, rng, m, 4096, 4096, 4, "f16", m_launches, train_warm, 4 * 9437184)
             r["mfma_frac"] = r["tflops"] / MFMA_F16_PEAK_TF
             extra[f"q4_qmm_m{m}_4096"] = r
         for name, kern in (("q8_qmm_bf16_m128_n12288", rt.KERNEL_AUTO), ("q8_qmm_bf16_m128_n12288_bf16_mfma", rt.KERNEL_QMM_BF16)):
-            r = bench_matmul(ops, rt, timer, rng, 128, 12288, 4096, 8, "bf16", gemm_launches, TRAIN, 4 * 53477376, kernel=kern)
+            r = bench_matmul(ops, rt, timer, rng, 128, 12288, 4096, 8, "bf16", gemm_launches, train_warm, 4 * 53477376, kernel=kern)
             r["mfma_frac"] = r["tflops"] / MFMA_F16_PEAK_TF
             extra[name] = r
     if "dequant" in sections:
+        progress("dequant")
         for fmt in ("awq", "gptq"):
             extra[f"{fmt}_dequant_4096x4096_gs128"] = bench_dequant(ops, rt, timer, rng, fmt, 4096, 4096, 128, max(200, launches // 10))
     if sections & {"gather", "moe"}:
+        progress("gather / moe")
         gate_up = make_weight(rng, 3072, 4096, 4, lead=(128,))
         down = make_weight(rng, 4096, 1536, 4, lead=(128,))
         experts = (gate_up, down, ops.QuantizedWeight.from_numpy(*gate_up, 64, 4),
@@ -443,6 +463,7 @@ def main():
                 extra[f"moe_q4_T{T}"] = r
         del experts, gate_up, down
     if "moe8" in sections:
+        progress("moe8")
         gate_up = make_weight(rng, 3072, 4096, 8, lead=(128,))
         down = make_weight(rng, 4096, 1536, 8, lead=(128,))
         experts = (gate_up, down, ops.QuantizedWeight.from_numpy(*gate_up, 64, 8),
@@ -482,7 +503,7 @@ def main():
                              "roofline": {"bound": "mfma", "achieved": q["tflops"], "peak": MFMA_F16_PEAK_TF,
                                           "unit": "TFLOP/s", "frac": q["mfma_frac"],
                                           "traffic": traffic.get("qmm_q4_m512_4096"),
-                                          "kernel": "qmm_rw_kernel", "avg_launch_us": q["us"]},
+                                          "kernel": "qmm_k2_kernel", "avg_launch_us": q["us"]},
                              "launches": q["launches"]}
     if not args.no_cpu:
         line["cpu_baseline"] = cpu_baseline(np.random.default_rng(1001), 3.0 if args.quick else 10.0,
