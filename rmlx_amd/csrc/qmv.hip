@@ -28,7 +28,14 @@
 //     folded into the f32 result with  acc += scale * (dot - sum(off*x)) + bias * sum(x).
 //   * Each wave stages exactly the activations it consumes (wave-private LDS, no barrier).  The
 //     per-(row, group) sums sum(x) and sum(off*x) come from the matrix unit too: one extra MFMA per
-//     product against a constant operand, issued while the weights are still in flight.
+//     product against a constant operand (computed once per workgroup where one pass covers K).
+//   * The kernel is bound by instruction issue before it is bound by memory (a wave moves 4 KB of
+//     weights per tile): operand lanes whose rows are empty read a zero slot instead of being masked,
+//     the unpacking constants sit in registers (and + or = one instruction), the two group halves
+//     meet through v_permlane32_swap, and the operand reads of a tile are scheduled slab by slab
+//     (low register count: up to three workgroups per CU).
+//   * Barriers of the tile reduction wait for LDS traffic only, and a workgroup that walks several
+//     tiles requests the next tile's weights as soon as the current accumulators have left for LDS.
 #include "common.hpp"
 
 namespace rmlx {

@@ -26,6 +26,10 @@
 //     past K meet zeros in the activation image.
 //   * Up to four activation rows share a pass: the unpacked weight pairs are reused, each row adds
 //     its own registers of x and 16 dot instructions per chunk and lane.
+//   * Matrices with more row blocks than the chip keeps resident run a looping form of the kernel:
+//     the grid is the resident workgroups, each stages the activations once and walks several row
+//     blocks with the next block's weights in flight.  Long rows of a short matrix split K over 2 or
+//     4 waves of the workgroup.
 #include "common.hpp"
 
 namespace rmlx {
