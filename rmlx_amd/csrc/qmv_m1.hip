@@ -84,49 +84,42 @@ __device__ __forceinline__ u4 to_pair_order(u4 d) {
   return o;
 }
 
-// R = weight rows per wave (1 or 2); NT = non-temporal weight loads (one pass over the weights);
-// MR = activation rows per pass (1, 2 or 4): their registers share the unpacked weights, so a few
-// rows cost one pass over the weights plus 16 dot instructions per row, chunk and lane.
-// NORM = RMSNorm prologue applied while the activations are staged (kernels of their own: the extra
-// registers would cost the plain kernels occupancy).
-// KP = waves per weight row (1, 2 or 4; split K, the counterpart of affine_qmv_splitk_f16_q4 + qmm_splitk_accum_f16,
-// quantized.rs:992-1233): wave w takes the chunks kp, kp + KP, ... of row w / KP (kp = w % KP) and the partial sums
-// meet in workgroup memory.  For long rows of a short matrix, where one wave per row leaves most of the chip idle.
-template <int BITS, int GS, int R, bool NT, int MR, bool NORM = false, int KP = 1>
-// (8-bit, one row: asking the compiler for eight waves per SIMD changes no register count but the schedule;
-// measured 4-13 % faster.  The 4-bit kernel would spill under that bound and is slower with it.)
-__global__ __launch_bounds__(kThreads, (BITS == 8 && MR == 1 && R == 1) ? 8 : 1) void qmv_m1_kernel(M1Params p) {
-  constexpr int kChunkK = 8192 / BITS;         // k values of one wave-wide 16-byte load: 2048 / 1024
-  constexpr int kLaneK = kChunkK / 64;         // values per lane and chunk: 32 / 16
-  constexpr int kXU = kLaneK / 8;              // 16-byte activation units per lane and chunk: 4 / 2
-  constexpr int kLanesPerGroup = GS / kLaneK;  // whole lanes per quantisation group
-  constexpr int kGroupsPerChunk = kChunkK / GS;
-  static_assert(kLanesPerGroup >= 1, "a lane must not straddle quantisation groups");
+// ---- pieces shared by the two kernels below ---------------------------------------------------------------------
+// Geometry of the activation image a workgroup keeps in LDS: per activation row the image [chunk][unit j][lane]
+// (a unit = 8 consecutive k = 16 bytes), then the sums [chunk][lane] = (sum(off * x), sum(x)) of the lane's values.
+template <int BITS, int MR>
+struct XImage {
+  static constexpr int kChunkK = 8192 / BITS;  // k values of one wave-wide 16-byte load: 2048 / 1024
+  static constexpr int kLaneK = kChunkK / 64;  // values per lane and chunk: 32 / 16
+  static constexpr int kXU = kLaneK / 8;       // 16-byte activation units per lane and chunk: 4 / 2
+  char* lds;
+  uint32_t K, KH, nunits, img_bytes, cs_bytes;  // KH whole chunks; image and sums bytes per activation row
+  __device__ XImage(char* lds_, uint32_t K_)
+      : lds(lds_), K(K_), KH((K_ + kChunkK - 1) / kChunkK), nunits(K_ / 8), img_bytes(KH * kChunkK * 2),
+        cs_bytes(KH * 64 * (uint32_t)sizeof(float2)) {}
+  __device__ u4* xl(int m) const { return reinterpret_cast<u4*>(lds + (size_t)m * img_bytes); }
+  __device__ float2* cs(int m) const { return reinterpret_cast<float2*>(lds + (size_t)MR * img_bytes + (size_t)m * cs_bytes); }
+};
 
-  extern __shared__ __attribute__((aligned(16))) char lds[];
-  // K need not be a multiple of the chunk: the lanes of the last chunk that lie past K read clamped
-  // (valid) addresses and multiply them with a zeroed activation image, i.e. contribute nothing.
-  const uint32_t K = p.K, KH = (K + kChunkK - 1) / kChunkK, G = K / GS, nunits = K / 8;
-  const uint32_t row_u4 = K / kLaneK;  // 16-byte pieces of a weight row
-  // per activation row: image [chunk][unit j][lane], then sums [chunk][lane] = (sum(off * x), sum(x)) of the lane's values
-  const uint32_t img_bytes = KH * kChunkK * 2, cs_bytes = KH * 64 * sizeof(float2);  // per activation row, whole chunks
-  auto xl = [&](int m) { return reinterpret_cast<u4*>(lds + (size_t)m * img_bytes); };
-  auto cs = [&](int m) { return reinterpret_cast<float2*>(lds + (size_t)MR * img_bytes + (size_t)m * cs_bytes); };
+// RMSNorm prologue of the reference's MMA kernel (`has_norm`, quantized.rs:3070-3095) applied to one 16-byte unit
+__device__ __forceinline__ u4 normalise_unit(const __half* norm_w, const float* inv_rms, uint32_t row, uint32_t u,
+                                             uint32_t nunits, u4 v) {
+  const _Float16 rs = (_Float16)inv_rms[row];
+  const h8 nw = __builtin_bit_cast(h8, reinterpret_cast<const u4*>(norm_w)[u < nunits ? u : nunits - 1]);
+  const h8 scaled = __builtin_bit_cast(h8, v) * (h8){rs, rs, rs, rs, rs, rs, rs, rs};
+  return __builtin_bit_cast(u4, scaled * nw);
+}
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  static_assert(KP == 1 || R == 1, "split rows: one row per wave group");
-  const uint32_t row0 = blockIdx.x * (kWaves * R / KP) + (wave / KP) * R;
-  const uint32_t kp = wave % KP;
-  // this wave's chunks: kp, kp + KP, ... (KHw of them)
-  const uint32_t KHw = KP == 1 ? KH : (KH > kp ? (KH - kp + KP - 1) / KP : 0u);
-  const uint32_t mrow0 = blockIdx.y * MR;  // first activation row of this pass (rows past M repeat the last one, unstored)
-
-  // ---- 1. loads, small ones first (the memory counter retires in order): activations ... ------
-  u4 xv[MR][4];
+// 1. The activation loads of a workgroup (the first four rounds of 512 units; issued before the weight loads
+//    because the memory counter retires in order), normalised on the way when NORM.  Rows past M repeat the last one.
+template <int BITS, int MR, bool NORM>
+__device__ __forceinline__ void load_activations(const XImage<BITS, MR> g, const __half* x, uint32_t M, uint32_t mrow0,
+                                                 const __half* norm_w, const float* inv_rms, int tid, u4 (&xv)[MR][4]) {
+  const uint32_t nunits = g.nunits;
 #pragma unroll
   for (int m = 0; m < MR; ++m) {
-    const uint32_t rm = mrow0 + m < p.M ? mrow0 + m : p.M - 1;
-    const u4* xg = reinterpret_cast<const u4*>(p.x + (uint64_t)rm * K);
+    const uint32_t rm = mrow0 + m < M ? mrow0 + m : M - 1;
+    const u4* xg = reinterpret_cast<const u4*>(x + (uint64_t)rm * g.K);
     const uint32_t u0 = (uint32_t)tid < nunits ? (uint32_t)tid : nunits - 1;
     xv[m][0] = xg[u0];
 #pragma unroll
@@ -138,21 +131,167 @@ __global__ __launch_bounds__(kThreads, (BITS == 8 && MR == 1 && R == 1) ? 8 : 1)
       }
     }
   }
-  // RMSNorm prologue of the reference's MMA kernel (`has_norm`, quantized.rs:3070-3095) applied while staging
-  auto normalise = [&](int m, uint32_t u, u4 v) {
-    const uint32_t rm = mrow0 + m < p.M ? mrow0 + m : p.M - 1;
-    const _Float16 rs = (_Float16)p.inv_rms[rm];
-    const h8 nw = __builtin_bit_cast(h8, reinterpret_cast<const u4*>(p.norm_w)[u < nunits ? u : nunits - 1]);
-    const h8 scaled = __builtin_bit_cast(h8, v) * (h8){rs, rs, rs, rs, rs, rs, rs, rs};
-    return __builtin_bit_cast(u4, scaled * nw);
-  };
   if constexpr (NORM) {
 #pragma unroll
-    for (int m = 0; m < MR; ++m)
+    for (int m = 0; m < MR; ++m) {
+      const uint32_t rm = mrow0 + m < M ? mrow0 + m : M - 1;
 #pragma unroll
       for (int i = 0; i < 4; ++i)
-        if (i == 0 || nunits > (uint32_t)i * kThreads) xv[m][i] = normalise(m, tid + i * kThreads, xv[m][i]);
+        if (i == 0 || nunits > (uint32_t)i * kThreads)
+          xv[m][i] = normalise_unit(norm_w, inv_rms, rm, tid + i * kThreads, nunits, xv[m][i]);
+    }
   }
+}
+
+// 2. Stage x: unit u = 8 consecutive k = (chunk, lane, j); image in the order a wave reads it, per-lane sums
+//    beside it.  The caller puts the workgroup barrier behind it.
+template <int BITS, int MR, bool NORM>
+__device__ __forceinline__ void stage_activations(const XImage<BITS, MR> g, const __half* x, uint32_t M, uint32_t mrow0,
+                                                  const __half* norm_w, const float* inv_rms, int tid,
+                                                  const u4 (&xv)[MR][4]) {
+  constexpr int kXU = XImage<BITS, MR>::kXU;
+  const uint32_t nunits = g.nunits, KH = g.KH;
+  auto stage_unit = [&](int m, uint32_t u, const u4& v) {
+    if (u < nunits) {
+      const uint32_t c = u / (64 * kXU), rem = u % (64 * kXU), l = rem / kXU, j = rem % kXU;
+      g.xl(m)[(c * kXU + j) * 64 + l] = BITS == 4 ? to_pair_order(v) : v;
+      const h8 hv = __builtin_bit_cast(h8, v);
+      float xs8 = 0.f, xo8 = 0.f;
+#pragma unroll
+      for (int e = 0; e < 8; e += 2) {
+        xs8 += (float)hv[e] + (float)hv[e + 1];
+        xo8 += 1024.0f * (float)hv[e] + (BITS == 4 ? 64.0f : 1024.0f) * (float)hv[e + 1];
+      }
+      // the kXU units of a lane sit in adjacent threads of one quad (unit counts are multiples of 4)
+      xs8 = dpp_add<0xB1>(xs8);
+      xo8 = dpp_add<0xB1>(xo8);
+      if (kXU == 4) {
+        xs8 = dpp_add<0x4E>(xs8);
+        xo8 = dpp_add<0x4E>(xo8);
+      }
+      if (j == 0) g.cs(m)[c * 64 + l] = make_float2(xo8, xs8);
+    } else if (u < KH * 64 * kXU) {  // image positions past K: zeros
+      const uint32_t c = u / (64 * kXU), rem = u % (64 * kXU), l = rem / kXU, j = rem % kXU;
+      g.xl(m)[(c * kXU + j) * 64 + l] = (u4){0u, 0u, 0u, 0u};
+      if (j == 0) g.cs(m)[c * 64 + l] = make_float2(0.f, 0.f);
+    }
+  };
+#pragma unroll
+  for (int m = 0; m < MR; ++m)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) stage_unit(m, tid + i * kThreads, xv[m][i]);
+  // K > 16384: the remaining rounds, loaded here (behind the first weight loads; rare and long-running shapes)
+  for (uint32_t u = tid + 4 * kThreads; u < KH * 64 * kXU; u += kThreads) {
+#pragma unroll
+    for (int m = 0; m < MR; ++m) {
+      const uint32_t rm = mrow0 + m < M ? mrow0 + m : M - 1;
+      u4 v = reinterpret_cast<const u4*>(x + (uint64_t)rm * g.K)[u < nunits ? u : nunits - 1];
+      if constexpr (NORM) v = normalise_unit(norm_w, inv_rms, rm, u, nunits, v);
+      stage_unit(m, u, v);
+    }
+  }
+}
+
+// masks and offsets of the nibble unpacking, held in registers: and + or is one instruction
+struct UnpackConsts { uint32_t m0, m1, k0, k1; };
+
+// 3. One chunk of the wave's R rows against the registers of x read from LDS:
+//    racc[r][m] += scale * (sum(x * (off + q)) - sum(off * x)) + bias * sum(x)
+template <int BITS, int R, int MR>
+__device__ __forceinline__ void dot_chunk(const XImage<BITS, MR> g, uint32_t c, int lane, const u4 (&w)[R],
+                                          const uint32_t (&s)[R], const uint32_t (&b)[R], const UnpackConsts& uc,
+                                          float (&racc)[R][MR]) {
+  constexpr int kXU = XImage<BITS, MR>::kXU;
+  uint32_t xr[MR][kXU][4];
+  float2 k[MR];
+#pragma unroll
+  for (int m = 0; m < MR; ++m) {
+#pragma unroll
+    for (int j = 0; j < kXU; ++j) {
+      const u4 v = g.xl(m)[(c * kXU + j) * 64 + lane];
+      xr[m][j][0] = v.x; xr[m][j][1] = v.y; xr[m][j][2] = v.z; xr[m][j][3] = v.w;
+    }
+    k[m] = g.cs(m)[c * 64 + lane];
+  }
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    const u4 wv = w[r];
+    const uint32_t wd[4] = {wv.x, wv.y, wv.z, wv.w};
+    float acc0[MR], acc1[MR];
+#pragma unroll
+    for (int m = 0; m < MR; ++m) acc0[m] = acc1[m] = 0.f;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      if (BITS == 4) {
+        const uint32_t hi = wd[j] >> 8;
+        const h2 p0 = as_h2((wd[j] & uc.m0) | uc.k0), p1 = as_h2((wd[j] & uc.m1) | uc.k1);
+        const h2 p2 = as_h2((hi & uc.m0) | uc.k0), p3 = as_h2((hi & uc.m1) | uc.k1);
+#pragma unroll
+        for (int m = 0; m < MR; ++m) {
+          acc0[m] = __builtin_amdgcn_fdot2(p0, as_h2(xr[m][j][0]), acc0[m], false);
+          acc1[m] = __builtin_amdgcn_fdot2(p1, as_h2(xr[m][j][1]), acc1[m], false);
+          acc0[m] = __builtin_amdgcn_fdot2(p2, as_h2(xr[m][j][2]), acc0[m], false);
+          acc1[m] = __builtin_amdgcn_fdot2(p3, as_h2(xr[m][j][3]), acc1[m], false);
+        }
+      } else {  // bytes (q0,q1,q2,q3) -> (1024 + q0, 1024 + q1), (1024 + q2, 1024 + q3): natural order
+        const int u = j >> 1, e = (j & 1) * 2;
+        const h2 p0 = as_h2(__builtin_amdgcn_perm(0x64646464u, wd[j], 0x04010400u));
+        const h2 p1 = as_h2(__builtin_amdgcn_perm(0x64646464u, wd[j], 0x04030402u));
+#pragma unroll
+        for (int m = 0; m < MR; ++m) {
+          acc0[m] = __builtin_amdgcn_fdot2(p0, as_h2(xr[m][u % kXU][e]), acc0[m], false);
+          acc1[m] = __builtin_amdgcn_fdot2(p1, as_h2(xr[m][u % kXU][e + 1]), acc1[m], false);
+        }
+      }
+    }
+    const float sc = __half2float(__ushort_as_half((unsigned short)s[r]));
+    const float bi = __half2float(__ushort_as_half((unsigned short)b[r]));
+#pragma unroll
+    for (int m = 0; m < MR; ++m) racc[r][m] += sc * ((acc0[m] + acc1[m]) - k[m].x) + bi * k[m].y;
+  }
+  // (several activation rows: keeps the LDS reads of the next chunk from being hoisted above this one, which would
+  // double the registers of x that are live)
+  if constexpr (MR > 1) __builtin_amdgcn_sched_barrier(0);
+}
+
+// R = weight rows per wave (1 or 2); NT = non-temporal weight loads (one pass over the weights);
+// MR = activation rows per pass (1, 2 or 4): their registers share the unpacked weights, so a few
+// rows cost one pass over the weights plus 16 dot instructions per row, chunk and lane.
+// NORM = RMSNorm prologue applied while the activations are staged (kernels of their own: the extra
+// registers would cost the plain kernels occupancy).
+// KP = waves per weight row (1, 2 or 4; split K, the counterpart of affine_qmv_splitk_f16_q4 + qmm_splitk_accum_f16,
+// quantized.rs:992-1233): wave w takes the chunks kp, kp + KP, ... of row w / KP (kp = w % KP) and the partial sums
+// meet in workgroup memory.  For long rows of a short matrix, where one wave per row leaves most of the chip idle.
+template <int BITS, int GS, int R, bool NT, int MR, bool NORM = false, int KP = 1>
+// (8-bit, one row: asking the compiler for eight waves per SIMD changes no register count but the schedule;
+// measured 4-13 % faster.  The 4-bit kernel would spill under that bound and is slower with it.  Two activation
+// rows: without a bound the scheduler spends 124 registers on a schedule that is 12 % slower than the one it finds
+// within the 96 of five waves per SIMD.)
+__global__ __launch_bounds__(kThreads, (BITS == 8 && MR == 1 && R == 1) ? 8 : (MR == 2 ? 5 : 1)) void qmv_m1_kernel(M1Params p) {
+  using Image = XImage<BITS, MR>;
+  constexpr int kChunkK = Image::kChunkK, kLaneK = Image::kLaneK;
+  constexpr int kLanesPerGroup = GS / kLaneK;  // whole lanes per quantisation group
+  constexpr int kGroupsPerChunk = kChunkK / GS;
+  static_assert(kLanesPerGroup >= 1, "a lane must not straddle quantisation groups");
+
+  extern __shared__ __attribute__((aligned(16))) char lds[];
+  // K need not be a multiple of the chunk: the lanes of the last chunk that lie past K read clamped
+  // (valid) addresses and multiply them with a zeroed activation image, i.e. contribute nothing.
+  const Image img(lds, p.K);
+  const uint32_t K = p.K, KH = img.KH, G = K / GS;
+  const uint32_t row_u4 = K / kLaneK;  // 16-byte pieces of a weight row
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  static_assert(KP == 1 || R == 1, "split rows: one row per wave group");
+  const uint32_t row0 = blockIdx.x * (kWaves * R / KP) + (wave / KP) * R;
+  const uint32_t kp = wave % KP;
+  // this wave's chunks: kp, kp + KP, ... (KHw of them)
+  const uint32_t KHw = KP == 1 ? KH : (KH > kp ? (KH - kp + KP - 1) / KP : 0u);
+  const uint32_t mrow0 = blockIdx.y * MR;  // first activation row of this pass (rows past M repeat the last one, unstored)
+
+  // ---- 1. loads, small ones first (the memory counter retires in order): activations ... ------
+  u4 xv[MR][4];
+  load_activations<BITS, MR, NORM>(img, p.x, p.M, mrow0, p.norm_w, p.inv_rms, tid, xv);
   // ... the epilogue operand of the output this lane will write (lane r * MR + m) ...
   const uint32_t out_m = mrow0 + lane % MR, out_n = row0 + lane / MR;
   const bool writes = lane < R * MR && out_m < p.M;
@@ -193,46 +332,8 @@ __global__ __launch_bounds__(kThreads, (BITS == 8 && MR == 1 && R == 1) ? 8 : 1)
   Batch ba, bb;
   load_batch(0, ba);
 
-  // ---- 2. stage x: unit u = 8 consecutive k = (chunk, lane, j); image in the order a wave reads it ----
-  auto stage_unit = [&](int m, uint32_t u, const u4& v) {
-    if (u < nunits) {
-      const uint32_t c = u / (64 * kXU), rem = u % (64 * kXU), l = rem / kXU, j = rem % kXU;
-      xl(m)[(c * kXU + j) * 64 + l] = BITS == 4 ? to_pair_order(v) : v;
-      const h8 hv = __builtin_bit_cast(h8, v);
-      float xs8 = 0.f, xo8 = 0.f;
-#pragma unroll
-      for (int e = 0; e < 8; e += 2) {
-        xs8 += (float)hv[e] + (float)hv[e + 1];
-        xo8 += 1024.0f * (float)hv[e] + (BITS == 4 ? 64.0f : 1024.0f) * (float)hv[e + 1];
-      }
-      // the kXU units of a lane sit in adjacent threads of one quad (unit counts are multiples of 4)
-      xs8 = dpp_add<0xB1>(xs8);
-      xo8 = dpp_add<0xB1>(xo8);
-      if (kXU == 4) {
-        xs8 = dpp_add<0x4E>(xs8);
-        xo8 = dpp_add<0x4E>(xo8);
-      }
-      if (j == 0) cs(m)[c * 64 + l] = make_float2(xo8, xs8);
-    } else if (u < KH * 64 * kXU) {  // image positions past K: zeros
-      const uint32_t c = u / (64 * kXU), rem = u % (64 * kXU), l = rem / kXU, j = rem % kXU;
-      xl(m)[(c * kXU + j) * 64 + l] = (u4){0u, 0u, 0u, 0u};
-      if (j == 0) cs(m)[c * 64 + l] = make_float2(0.f, 0.f);
-    }
-  };
-#pragma unroll
-  for (int m = 0; m < MR; ++m)
-#pragma unroll
-    for (int i = 0; i < 4; ++i) stage_unit(m, tid + i * kThreads, xv[m][i]);
-  // K > 16384: the remaining rounds, loaded here (behind the first weight loads; rare and long-running shapes)
-  for (uint32_t u = tid + 4 * kThreads; u < KH * 64 * kXU; u += kThreads) {
-#pragma unroll
-    for (int m = 0; m < MR; ++m) {
-      const uint32_t rm = mrow0 + m < p.M ? mrow0 + m : p.M - 1;
-      u4 v = reinterpret_cast<const u4*>(p.x + (uint64_t)rm * K)[u < nunits ? u : nunits - 1];
-      if constexpr (NORM) v = normalise(m, u, v);
-      stage_unit(m, u, v);
-    }
-  }
+  // ---- 2. stage x into the LDS image ---------------------------------------------------------------------
+  stage_activations<BITS, MR, NORM>(img, p.x, p.M, mrow0, p.norm_w, p.inv_rms, tid, xv);
   __syncthreads();
 
   // ---- 3. chunk by chunk: registers of x from LDS, then the wave's rows --------------------------------
@@ -241,61 +342,13 @@ __global__ __launch_bounds__(kThreads, (BITS == 8 && MR == 1 && R == 1) ? 8 : 1)
   for (int r = 0; r < R; ++r)
 #pragma unroll
     for (int m = 0; m < MR; ++m) racc[r][m] = 0.f;
-  uint32_t m0 = 0x000F000Fu, m1 = 0x00F000F0u, k0 = 0x64006400u, k1 = 0x54005400u;
-  asm volatile("" : "+s"(m0), "+s"(m1), "+v"(k0), "+v"(k1));  // constants in registers: and+or is one instruction
+  UnpackConsts uc{0x000F000Fu, 0x00F000F0u, 0x64006400u, 0x54005400u};
+  asm volatile("" : "+s"(uc.m0), "+s"(uc.m1), "+v"(uc.k0), "+v"(uc.k1));
   auto process = [&](uint32_t c0, const Batch& t) {
 #pragma unroll
     for (int cc = 0; cc < 2; ++cc) {
       const uint32_t c = kp + KP * (c0 + cc);
-      if (c0 + cc < KHw) {
-        uint32_t xr[MR][kXU][4];
-        float2 k[MR];
-#pragma unroll
-        for (int m = 0; m < MR; ++m) {
-#pragma unroll
-          for (int j = 0; j < kXU; ++j) {
-            const u4 v = xl(m)[(c * kXU + j) * 64 + lane];
-            xr[m][j][0] = v.x; xr[m][j][1] = v.y; xr[m][j][2] = v.z; xr[m][j][3] = v.w;
-          }
-          k[m] = cs(m)[c * 64 + lane];
-        }
-#pragma unroll
-        for (int r = 0; r < R; ++r) {
-          const u4 wv = t.w[cc][r];
-          const uint32_t wd[4] = {wv.x, wv.y, wv.z, wv.w};
-          float acc0[MR], acc1[MR];
-#pragma unroll
-          for (int m = 0; m < MR; ++m) acc0[m] = acc1[m] = 0.f;
-#pragma unroll
-          for (int j = 0; j < 4; ++j) {
-            if (BITS == 4) {
-              const uint32_t hi = wd[j] >> 8;
-              const h2 p0 = as_h2((wd[j] & m0) | k0), p1 = as_h2((wd[j] & m1) | k1);
-              const h2 p2 = as_h2((hi & m0) | k0), p3 = as_h2((hi & m1) | k1);
-#pragma unroll
-              for (int m = 0; m < MR; ++m) {
-                acc0[m] = __builtin_amdgcn_fdot2(p0, as_h2(xr[m][j][0]), acc0[m], false);
-                acc1[m] = __builtin_amdgcn_fdot2(p1, as_h2(xr[m][j][1]), acc1[m], false);
-                acc0[m] = __builtin_amdgcn_fdot2(p2, as_h2(xr[m][j][2]), acc0[m], false);
-                acc1[m] = __builtin_amdgcn_fdot2(p3, as_h2(xr[m][j][3]), acc1[m], false);
-              }
-            } else {  // bytes (q0,q1,q2,q3) -> (1024 + q0, 1024 + q1), (1024 + q2, 1024 + q3): natural order
-              const int u = j >> 1, e = (j & 1) * 2;
-              const h2 p0 = as_h2(__builtin_amdgcn_perm(0x64646464u, wd[j], 0x04010400u));
-              const h2 p1 = as_h2(__builtin_amdgcn_perm(0x64646464u, wd[j], 0x04030402u));
-#pragma unroll
-              for (int m = 0; m < MR; ++m) {
-                acc0[m] = __builtin_amdgcn_fdot2(p0, as_h2(xr[m][u % kXU][e]), acc0[m], false);
-                acc1[m] = __builtin_amdgcn_fdot2(p1, as_h2(xr[m][u % kXU][e + 1]), acc1[m], false);
-              }
-            }
-          }
-          const float sc = __half2float(__ushort_as_half((unsigned short)t.s[cc][r]));
-          const float bi = __half2float(__ushort_as_half((unsigned short)t.b[cc][r]));
-#pragma unroll
-          for (int m = 0; m < MR; ++m) racc[r][m] += sc * ((acc0[m] + acc1[m]) - k[m].x) + bi * k[m].y;
-        }
-      }
+      if (c0 + cc < KHw) dot_chunk<BITS, R, MR>(img, c, lane, t.w[cc], t.s[cc], t.b[cc], uc, racc);
     }
   };
   for (uint32_t c0 = 0; c0 < KHw; c0 += 4) {
@@ -341,9 +394,8 @@ template <int BITS, int GS, int R, bool NT, int MR, bool NORM = false>
 // (8-bit, one row: asking the compiler for eight waves per SIMD changes no register count but the schedule;
 // measured 4-13 % faster.  The 4-bit kernel would spill under that bound and is slower with it.)
 __global__ __launch_bounds__(kThreads, 1) void qmv_m1_loop_kernel(M1Params p) {
-  constexpr int kChunkK = 8192 / BITS;         // k values of one wave-wide 16-byte load: 2048 / 1024
-  constexpr int kLaneK = kChunkK / 64;         // values per lane and chunk: 32 / 16
-  constexpr int kXU = kLaneK / 8;              // 16-byte activation units per lane and chunk: 4 / 2
+  using Image = XImage<BITS, MR>;
+  constexpr int kChunkK = Image::kChunkK, kLaneK = Image::kLaneK;
   constexpr int kLanesPerGroup = GS / kLaneK;  // whole lanes per quantisation group
   constexpr int kGroupsPerChunk = kChunkK / GS;
   static_assert(kLanesPerGroup >= 1, "a lane must not straddle quantisation groups");
@@ -351,12 +403,9 @@ __global__ __launch_bounds__(kThreads, 1) void qmv_m1_loop_kernel(M1Params p) {
   extern __shared__ __attribute__((aligned(16))) char lds[];
   // K need not be a multiple of the chunk: the lanes of the last chunk that lie past K read clamped
   // (valid) addresses and multiply them with a zeroed activation image, i.e. contribute nothing.
-  const uint32_t K = p.K, KH = (K + kChunkK - 1) / kChunkK, G = K / GS, nunits = K / 8;
+  const Image img(lds, p.K);
+  const uint32_t K = p.K, KH = img.KH, G = K / GS;
   const uint32_t row_u4 = K / kLaneK;  // 16-byte pieces of a weight row
-  // per activation row: image [chunk][unit j][lane], then sums [chunk][lane] = (sum(off * x), sum(x)) of the lane's values
-  const uint32_t img_bytes = KH * kChunkK * 2, cs_bytes = KH * 64 * sizeof(float2);  // per activation row, whole chunks
-  auto xl = [&](int m) { return reinterpret_cast<u4*>(lds + (size_t)m * img_bytes); };
-  auto cs = [&](int m) { return reinterpret_cast<float2*>(lds + (size_t)MR * img_bytes + (size_t)m * cs_bytes); };
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const uint32_t mrow0 = blockIdx.y * MR;  // first activation row of this pass (rows past M repeat the last one, unstored)
@@ -369,36 +418,7 @@ __global__ __launch_bounds__(kThreads, 1) void qmv_m1_loop_kernel(M1Params p) {
 
   // ---- 1. loads, small ones first (the memory counter retires in order): activations ... ------
   u4 xv[MR][4];
-#pragma unroll
-  for (int m = 0; m < MR; ++m) {
-    const uint32_t rm = mrow0 + m < p.M ? mrow0 + m : p.M - 1;
-    const u4* xg = reinterpret_cast<const u4*>(p.x + (uint64_t)rm * K);
-    const uint32_t u0 = (uint32_t)tid < nunits ? (uint32_t)tid : nunits - 1;
-    xv[m][0] = xg[u0];
-#pragma unroll
-    for (int i = 1; i < 4; ++i) {
-      xv[m][i] = (u4){0u, 0u, 0u, 0u};
-      if (nunits > (uint32_t)i * kThreads) {  // uniform; the last round may be partial (clamped, stored under a guard)
-        const uint32_t u = tid + i * kThreads;
-        xv[m][i] = xg[u < nunits ? u : nunits - 1];
-      }
-    }
-  }
-  // RMSNorm prologue of the reference's MMA kernel (`has_norm`, quantized.rs:3070-3095) applied while staging
-  auto normalise = [&](int m, uint32_t u, u4 v) {
-    const uint32_t rm = mrow0 + m < p.M ? mrow0 + m : p.M - 1;
-    const _Float16 rs = (_Float16)p.inv_rms[rm];
-    const h8 nw = __builtin_bit_cast(h8, reinterpret_cast<const u4*>(p.norm_w)[u < nunits ? u : nunits - 1]);
-    const h8 scaled = __builtin_bit_cast(h8, v) * (h8){rs, rs, rs, rs, rs, rs, rs, rs};
-    return __builtin_bit_cast(u4, scaled * nw);
-  };
-  if constexpr (NORM) {
-#pragma unroll
-    for (int m = 0; m < MR; ++m)
-#pragma unroll
-      for (int i = 0; i < 4; ++i)
-        if (i == 0 || nunits > (uint32_t)i * kThreads) xv[m][i] = normalise(m, tid + i * kThreads, xv[m][i]);
-  }
+  load_activations<BITS, MR, NORM>(img, p.x, p.M, mrow0, p.norm_w, p.inv_rms, tid, xv);
   // ---- ... then the first two chunks of the wave's rows with their scales and biases ----------------
   // A batch is two chunks of the wave's rows in one block; the batches of all blocks of the workgroup form one
   // sequence (block 0: chunks 0-1, 2-3, ..., block 1: chunks 0-1, ...) that is loaded one batch ahead.
@@ -447,53 +467,15 @@ __global__ __launch_bounds__(kThreads, 1) void qmv_m1_loop_kernel(M1Params p) {
   Batch ba, bb;
   if (n_batches > 0) load_batch(ba);
 
-  // ---- 2. stage x: unit u = 8 consecutive k = (chunk, lane, j); image in the order a wave reads it ----
-  auto stage_unit = [&](int m, uint32_t u, const u4& v) {
-    if (u < nunits) {
-      const uint32_t c = u / (64 * kXU), rem = u % (64 * kXU), l = rem / kXU, j = rem % kXU;
-      xl(m)[(c * kXU + j) * 64 + l] = BITS == 4 ? to_pair_order(v) : v;
-      const h8 hv = __builtin_bit_cast(h8, v);
-      float xs8 = 0.f, xo8 = 0.f;
-#pragma unroll
-      for (int e = 0; e < 8; e += 2) {
-        xs8 += (float)hv[e] + (float)hv[e + 1];
-        xo8 += 1024.0f * (float)hv[e] + (BITS == 4 ? 64.0f : 1024.0f) * (float)hv[e + 1];
-      }
-      // the kXU units of a lane sit in adjacent threads of one quad (unit counts are multiples of 4)
-      xs8 = dpp_add<0xB1>(xs8);
-      xo8 = dpp_add<0xB1>(xo8);
-      if (kXU == 4) {
-        xs8 = dpp_add<0x4E>(xs8);
-        xo8 = dpp_add<0x4E>(xo8);
-      }
-      if (j == 0) cs(m)[c * 64 + l] = make_float2(xo8, xs8);
-    } else if (u < KH * 64 * kXU) {  // image positions past K: zeros
-      const uint32_t c = u / (64 * kXU), rem = u % (64 * kXU), l = rem / kXU, j = rem % kXU;
-      xl(m)[(c * kXU + j) * 64 + l] = (u4){0u, 0u, 0u, 0u};
-      if (j == 0) cs(m)[c * 64 + l] = make_float2(0.f, 0.f);
-    }
-  };
-#pragma unroll
-  for (int m = 0; m < MR; ++m)
-#pragma unroll
-    for (int i = 0; i < 4; ++i) stage_unit(m, tid + i * kThreads, xv[m][i]);
-  // K > 16384: the remaining rounds, loaded here (behind the first weight loads; rare and long-running shapes)
-  for (uint32_t u = tid + 4 * kThreads; u < KH * 64 * kXU; u += kThreads) {
-#pragma unroll
-    for (int m = 0; m < MR; ++m) {
-      const uint32_t rm = mrow0 + m < p.M ? mrow0 + m : p.M - 1;
-      u4 v = reinterpret_cast<const u4*>(p.x + (uint64_t)rm * K)[u < nunits ? u : nunits - 1];
-      if constexpr (NORM) v = normalise(m, u, v);
-      stage_unit(m, u, v);
-    }
-  }
+  // ---- 2. stage x into the LDS image ---------------------------------------------------------------------
+  stage_activations<BITS, MR, NORM>(img, p.x, p.M, mrow0, p.norm_w, p.inv_rms, tid, xv);
   __syncthreads();
 
   // ---- 3. batch by batch: registers of x from LDS, then the wave's rows; 4. at the end of a block the wave-wide
   //         sums: lane r * MR + m writes the output of (weight row r, activation row m) ---------------------------
   float racc[R][MR];
-  uint32_t m0 = 0x000F000Fu, m1 = 0x00F000F0u, k0 = 0x64006400u, k1 = 0x54005400u;
-  asm volatile("" : "+s"(m0), "+s"(m1), "+v"(k0), "+v"(k1));  // constants in registers: and+or is one instruction
+  UnpackConsts uc{0x000F000Fu, 0x00F000F0u, 0x64006400u, 0x54005400u};
+  asm volatile("" : "+s"(uc.m0), "+s"(uc.m1), "+v"(uc.k0), "+v"(uc.k1));
   uint32_t pr_blk = 0, pr_c0 = 0;  // block and first chunk of the batch being processed
   float epi_val = 0.f;
   auto process = [&](const Batch& t) {
@@ -507,55 +489,7 @@ __global__ __launch_bounds__(kThreads, 1) void qmv_m1_loop_kernel(M1Params p) {
 #pragma unroll
     for (int cc = 0; cc < 2; ++cc) {
       const uint32_t c = pr_c0 + cc;
-      if (c < KH) {
-        uint32_t xr[MR][kXU][4];
-        float2 k[MR];
-#pragma unroll
-        for (int m = 0; m < MR; ++m) {
-#pragma unroll
-          for (int j = 0; j < kXU; ++j) {
-            const u4 v = xl(m)[(c * kXU + j) * 64 + lane];
-            xr[m][j][0] = v.x; xr[m][j][1] = v.y; xr[m][j][2] = v.z; xr[m][j][3] = v.w;
-          }
-          k[m] = cs(m)[c * 64 + lane];
-        }
-#pragma unroll
-        for (int r = 0; r < R; ++r) {
-          const u4 wv = t.w[cc][r];
-          const uint32_t wd[4] = {wv.x, wv.y, wv.z, wv.w};
-          float acc0[MR], acc1[MR];
-#pragma unroll
-          for (int m = 0; m < MR; ++m) acc0[m] = acc1[m] = 0.f;
-#pragma unroll
-          for (int j = 0; j < 4; ++j) {
-            if (BITS == 4) {
-              const uint32_t hi = wd[j] >> 8;
-              const h2 p0 = as_h2((wd[j] & m0) | k0), p1 = as_h2((wd[j] & m1) | k1);
-              const h2 p2 = as_h2((hi & m0) | k0), p3 = as_h2((hi & m1) | k1);
-#pragma unroll
-              for (int m = 0; m < MR; ++m) {
-                acc0[m] = __builtin_amdgcn_fdot2(p0, as_h2(xr[m][j][0]), acc0[m], false);
-                acc1[m] = __builtin_amdgcn_fdot2(p1, as_h2(xr[m][j][1]), acc1[m], false);
-                acc0[m] = __builtin_amdgcn_fdot2(p2, as_h2(xr[m][j][2]), acc0[m], false);
-                acc1[m] = __builtin_amdgcn_fdot2(p3, as_h2(xr[m][j][3]), acc1[m], false);
-              }
-            } else {  // bytes (q0,q1,q2,q3) -> (1024 + q0, 1024 + q1), (1024 + q2, 1024 + q3): natural order
-              const int u = j >> 1, e = (j & 1) * 2;
-              const h2 p0 = as_h2(__builtin_amdgcn_perm(0x64646464u, wd[j], 0x04010400u));
-              const h2 p1 = as_h2(__builtin_amdgcn_perm(0x64646464u, wd[j], 0x04030402u));
-#pragma unroll
-              for (int m = 0; m < MR; ++m) {
-                acc0[m] = __builtin_amdgcn_fdot2(p0, as_h2(xr[m][u % kXU][e]), acc0[m], false);
-                acc1[m] = __builtin_amdgcn_fdot2(p1, as_h2(xr[m][u % kXU][e + 1]), acc1[m], false);
-              }
-            }
-          }
-          const float sc = __half2float(__ushort_as_half((unsigned short)t.s[cc][r]));
-          const float bi = __half2float(__ushort_as_half((unsigned short)t.b[cc][r]));
-#pragma unroll
-          for (int m = 0; m < MR; ++m) racc[r][m] += sc * ((acc0[m] + acc1[m]) - k[m].x) + bi * k[m].y;
-        }
-      }
+      if (c < KH) dot_chunk<BITS, R, MR>(img, c, lane, t.w[cc], t.s[cc], t.b[cc], uc, racc);
     }
     pr_c0 += 2;
     if (pr_c0 >= KH) {  // the block is complete
