@@ -528,11 +528,12 @@ size_t lds_per_row(uint32_t K) {
   return chunks * (chunk_k * 2 + 64 * sizeof(float2));
 }
 
-// Workgroups of `kernel` that the chip keeps resident at once (per-instantiation cache, keyed by the LDS size).
+// Workgroups of `kernel` that the chip keeps resident at once (cache per instantiation and host thread, keyed by
+// the LDS size).
 template <typename Kernel>
 uint32_t resident_workgroups(Kernel kernel, size_t lds) {
-  static size_t cached_lds = ~(size_t)0;
-  static uint32_t cached = 0;
+  static thread_local size_t cached_lds = ~(size_t)0;
+  static thread_local uint32_t cached = 0;
   if (cached_lds != lds) {
     int per_cu = 0;
     if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, kThreads, lds) != hipSuccess || per_cu < 1) per_cu = 1;
