@@ -151,7 +151,7 @@ bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) ==
 // register-weights MFMA GEMM above (the LDS-staged GEMM when K is not a multiple of 512), the
 // portable kernel for every shape the fast kernels do not take.
 enum { KERNEL_AUTO = 0, KERNEL_QMV = 1, KERNEL_QMM = 2, KERNEL_GENERIC = 3, KERNEL_QMM_BF16 = 4, KERNEL_QMM_LDS = 5,
-       KERNEL_QMV_ROWS = 6, KERNEL_QMM_K2 = 7, KERNEL_QMM_RW = 8 };
+       KERNEL_QMV_ROWS = 6, KERNEL_QMM_K2 = 7, KERNEL_QMM_RW = 8, KERNEL_QMM_K2_TALL = 9 };
 constexpr uint32_t kQmvMaxM = 16;
 // group size 64: rows taken by the single-row kernel (measured: 3 and 4 rows are faster on the matrix unit)
 constexpr uint32_t kM1MaxRows = 2;
@@ -195,6 +195,7 @@ int32_t run_matmul_plain(const rmlx_qweight* qw, const void* x, int32_t x_dtype,
   const bool can_qmm_rw = ptr_ok && qmm_rw_supported(N, K, qw->group_size, qw->bits);
   const bool can_qmm = can_qmm_lds || can_qmm_rw;
   const bool can_qmm_k2 = ptr_ok && qmm_k2_supported(N, K, qw->group_size, qw->bits);
+  const bool can_qmm_k2_tall = can_qmm_k2 && qmm_k2_tall_supported(qw->group_size, qw->bits);
 
   if (kernel == KERNEL_AUTO) {
     // The multi-row GEMV streams the weights once per pass of 8 rows (4-bit; two passes share a workgroup
@@ -233,17 +234,28 @@ int32_t run_matmul_plain(const rmlx_qweight* qw, const void* x, int32_t x_dtype,
     return fail(RMLX_INVALID_SHAPE,
                 "the register-weights qmm kernels require bits in {4,8}, N %% 64 == 0, K %% 512 == 0 and 16-byte aligned "
                 "buffers (N=%u K=%u bits=%u group_size=%u)", N, K, qw->bits, qw->group_size);
-  } else if (kernel < 0 || kernel > KERNEL_QMM_RW) {
+  } else if (kernel == KERNEL_QMM_K2_TALL && !can_qmm_k2_tall) {
+    return fail(RMLX_INVALID_SHAPE,
+                "the 128 x 128 K-split qmm kernel requires 4-bit weights with group size 64 or 128 or 8-bit weights with group "
+                "size 128, N %% 128 == 0, K %% 512 == 0 and 16-byte aligned buffers (N=%u K=%u bits=%u group_size=%u)",
+                N, K, qw->bits, qw->group_size);
+  } else if (kernel < 0 || kernel > KERNEL_QMM_K2_TALL) {
     return fail(RMLX_NOT_FOUND, "unknown kernel selector %d", kernel);
   }
-  // The K-split GEMM (64 x 128 tiles, 32x32x16 MFMAs) where its grid is one round over most of the chip: measured
-  // 23.8 against 25.4 us at M = 512, 4096 x 4096 and 27.8 against 28.8 us at M = 128, N = 12288 (8-bit); with fewer
-  // tiles the smaller tiles of the register-weights GEMM keep more CUs busy, with several rounds its 128-row tiles
-  // unpack every weight for twice as many rows.
+  // The K-split GEMM (32x32x16 MFMAs, K split inside the workgroup).  64 x 128 tiles where that grid is one round over
+  // most of the chip: measured 23.8 against 25.4 us at M = 512, 4096 x 4096 and 27.8 against 28.8 us at M = 128,
+  // N = 12288 (8-bit).  128 x 128 tiles (every unpacked weight operand feeds four MFMAs) from 0.6 rounds of those on:
+  // 29.6 against 35.5 us at M = 640, 37.0 against 41.4 us at M = 1024, 153 against 175 us at M = 4096 (4096 x 4096), 30.9
+  // against 37.8 us at M = 192, N = 12288.  With fewer tiles the smaller tiles of the register-weights GEMM keep more
+  // CUs busy.
+  uint32_t k2_tile_rows = kernel == KERNEL_QMM_K2_TALL ? 128 : 64;
   if (kernel == KERNEL_QMM && can_qmm_k2) {
-    const uint64_t tiles = (uint64_t)((M + 63) / 64) * (N / 128), cus = (uint64_t)ctx().num_cus;
+    const uint64_t tiles = (uint64_t)((M + 63) / 64) * (N / 128), tall = (uint64_t)((M + 127) / 128) * (N / 128);
+    const uint64_t cus = (uint64_t)ctx().num_cus;
     if (tiles * 10 >= cus * 7 && tiles <= cus) kernel = KERNEL_QMM_K2;
+    else if (can_qmm_k2_tall && tall * 10 >= cus * 6) { kernel = KERNEL_QMM_K2; k2_tile_rows = 128; }
   }
+  if (kernel == KERNEL_QMM_K2_TALL) kernel = KERNEL_QMM_K2;
   if (kernel == KERNEL_QMM_RW) kernel = KERNEL_QMM;
 
   // RMSNorm prologue: fused into the single-row GEMV for one or two rows (while it stages the activations);
@@ -271,7 +283,7 @@ int32_t run_matmul_plain(const rmlx_qweight* qw, const void* x, int32_t x_dtype,
     }
     QmmArgs a{qw->w, qw->s, qw->b, xk, xk_dtype, out, M, N, K, qw->bits, nullptr, 0, epi.kind, epi.ptr, epi.dtype};
     *epi_done = true;
-    return launch_qmm_k2(a, qw->group_size, stream);
+    return launch_qmm_k2(a, qw->group_size, k2_tile_rows, stream);
   }
   if (kernel == KERNEL_QMM && can_qmm_rw) {
     // Register-weights GEMM: f16 / bf16 activations straight from the row-major matrix, no workspace

@@ -183,10 +183,12 @@ int32_t launch_qmm(const QmmArgs& a, hipStream_t s);
 // Register-weights GEMM (qmm_rw.hip): f16 activations only, no workspace.
 bool qmm_rw_supported(uint32_t N, uint32_t K, uint32_t group_size, uint32_t bits);
 int32_t launch_qmm_rw(const QmmArgs& a, uint32_t group_size, hipStream_t s);
-// K-split GEMM (qmm_k2.hip) for prefill-sized batches: 64 x 128 tiles, 32x32x16 MFMAs, the two halves of a workgroup split K; f16 / bf16
-// activations, no workspace, fused store epilogue.
+// K-split GEMM (qmm_k2.hip) for prefill-sized batches: 64 x 128 or 128 x 128 tiles (tile_rows), 32x32x16 MFMAs, the two
+// halves of a workgroup split K; f16 / bf16 activations, no workspace, fused store epilogue.  The 128-row tile is built
+// for the weight formats whose kernel fits the register file (4-bit with group size 64 / 128, 8-bit with group size 128).
 bool qmm_k2_supported(uint32_t N, uint32_t K, uint32_t group_size, uint32_t bits);
-int32_t launch_qmm_k2(const QmmArgs& a, uint32_t group_size, hipStream_t s);
+bool qmm_k2_tall_supported(uint32_t group_size, uint32_t bits);
+int32_t launch_qmm_k2(const QmmArgs& a, uint32_t group_size, uint32_t tile_rows, hipStream_t s);
 // Grouped form of the same GEMM for the expert projections of batches with many rows per expert: every
 // row tile (kGroupedTileRows rows of one expert) takes its expert and rows from a device table of
 // (expert, first row position, row count) triples (bit 31 of the count: write zeros instead of computing;

@@ -36,10 +36,8 @@ typedef float f16v __attribute__((ext_vector_type(16)));
 typedef uint32_t u4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u2 __attribute__((ext_vector_type(2)));
 
-constexpr int kTileM = 64, kTileN = 128, kBlockK = 128, kThreads = 512;
+constexpr int kTileN = 128, kBlockK = 128, kThreads = 512;
 constexpr int kUnroll = 4;                       // depth of the weight register ring; scales come per four blocks
-constexpr int kChunkUnits = kTileM * 16;         // 16-byte units of one activation chunk (64 rows x 128 k): 1024
-constexpr int kAL = kChunkUnits / kThreads;      // units per thread and chunk: 2
 
 struct K2Params {
   const uint32_t* w; const __half* s; const __half* b;
@@ -92,12 +90,17 @@ __device__ __forceinline__ uint32_t act_slot(uint32_t R, uint32_t seg) {
   return (((R >> 5) * 2 + (seg >> 3)) * 4 + (seg & 3)) * 64 + (((((seg >> 2) & 1) << 5) | (R & 31)) ^ seg);
 }
 
-template <int BITS, bool XBF16, int GS>
+// MFR: activation fragments of 32 rows per tile (2: 64 x 128 tiles; 4: 128 x 128 tiles, every unpacked weight operand
+// then feeds four MFMAs)
+template <int BITS, bool XBF16, int GS, int MFR>
 __global__ __launch_bounds__(kThreads) void qmm_k2_kernel(const K2Params p) {
+  constexpr int kTileM = 32 * MFR;
+  constexpr int kChunkUnits = kTileM * 16;               // 16-byte units of one activation chunk (rows x 128 k): 1024 / 2048
+  constexpr int kAL = kChunkUnits / kThreads;            // units per thread and chunk: 2 / 4
   constexpr int WV = BITS == 4 ? 1 : 2;                  // 16-byte weight loads per lane and block
   constexpr int kSbBytes = 4 * (kBlockK / GS) * 2;       // scales of one row and four blocks: 16 / 32 / 8 bytes
   constexpr int kSbVecs = kSbBytes > 16 ? 2 : 1;
-  __shared__ u4 lds[4096];  // 64 KB: two activation stages of 16 KB; all of it for the final transposition
+  __shared__ u4 lds[4096];  // 64 KB: two activation stages of 16 / 32 KB; all of it for the final transposition
 
   const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, wn = wave & 3, kh = wave >> 2;
   const uint32_t r = lane & 31, hh = lane >> 5;
@@ -132,7 +135,9 @@ __global__ __launch_bounds__(kThreads) void qmm_k2_kernel(const K2Params p) {
   // activations: unit q*512 + tid -> (tile row 32 q + tid/16, segment tid%16); 16 neighbouring lanes read one row's
   // 256 contiguous bytes
   const uint32_t seg = tid & 15, R0 = tid >> 4;
-  const uint32_t xoff = (R0 * K + seg * 8) * 2;  // unit q: + 32 q rows
+  uint32_t xoff[kAL];  // unit q: row R0 + 32 q (in the range-checked part of the address: rows past M read zero)
+#pragma unroll
+  for (int q = 0; q < kAL; ++q) xoff[q] = ((R0 + 32 * q) * K + seg * 8) * 2;
   const uint32_t lds_w0 = act_slot(R0, seg);     // unit q: + q * 512 slots
   // operand reads of k step ks (fragment i: + 512 slots, stage: + 1024 slots)
   uint32_t lds_r[4];
@@ -142,9 +147,9 @@ __global__ __launch_bounds__(kThreads) void qmm_k2_kernel(const K2Params p) {
   const uint32_t woff = ((32 * wn + r) * row_words) * 4 + (8 * kh + 4 * hh) * 4 * WV;
   const uint32_t soff = (32 * wn + r) * G * 2;
 
-  f16v acc[2];
+  f16v acc[MFR];
 #pragma unroll
-  for (int i = 0; i < 2; ++i)
+  for (int i = 0; i < MFR; ++i)
 #pragma unroll
     for (int e = 0; e < 16; ++e) acc[i][e] = 0.f;
 
@@ -173,7 +178,7 @@ __global__ __launch_bounds__(kThreads) void qmm_k2_kernel(const K2Params p) {
   auto load_a = [&](uint32_t it, u4 (&dst)[kAL]) {
 #pragma unroll
     for (int q = 0; q < kAL; ++q)
-      dst[q] = __builtin_amdgcn_raw_buffer_load_b128(xr, xoff, it * (kBlockK * 2) + q * 32 * K * 2, 0);
+      dst[q] = __builtin_amdgcn_raw_buffer_load_b128(xr, xoff[q], it * (kBlockK * 2), 0);
   };
   auto store_a = [&](uint32_t stage, const u4 (&src)[kAL]) {
 #pragma unroll
@@ -249,9 +254,9 @@ __global__ __launch_bounds__(kThreads) void qmm_k2_kernel(const K2Params p) {
   load_a(clampi(2), ra[0]);
   load_a(clampi(3), ra[1]);
   __syncthreads();
-  h8 bf[2][4];
+  h8 bf[MFR][4];
 #pragma unroll
-  for (int i = 0; i < 2; ++i)
+  for (int i = 0; i < MFR; ++i)
 #pragma unroll
     for (int ks = 0; ks < 4; ++ks) bf[i][ks] = read_b(0, i, ks);
   __syncthreads();  // block 0 overwrites stage 0 with chunk 2: every wave must have taken its operands of chunk 0 first
@@ -274,7 +279,7 @@ __global__ __launch_bounds__(kThreads) void qmm_k2_kernel(const K2Params p) {
 #pragma unroll
     for (int ks = 0; ks < 4; ++ks) {
 #pragma unroll
-      for (int i = 0; i < 2; ++i) {
+      for (int i = 0; i < MFR; ++i) {
         acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(aw, bf[i][ks], acc[i], 0, 0, 0);
         bf[i][ks] = read_b(st_nxt, i, ks);  // the slot is free: next block's operand (past the last block: unused)
       }
@@ -285,7 +290,7 @@ __global__ __launch_bounds__(kThreads) void qmm_k2_kernel(const K2Params p) {
         aw_nxt = weight_operand(u + 1, 0, s2, b2);
       }
       if (ks < kAL && writes) lds[st_wr * kChunkUnits + ks * 512 + lds_w0] = to_slot_order(ra[u % 2][ks]);
-      if (MAIN && ks == 2) load_a(it + 4, ra[u % 2]);
+      if (MAIN && ks == (kAL > 3 ? kAL - 1 : 2)) load_a(it + 4, ra[u % 2]);  // (its last unit has just been written)
       aw = aw_nxt;
       __builtin_amdgcn_sched_barrier(0);
     }
@@ -313,7 +318,11 @@ __global__ __launch_bounds__(kThreads) void qmm_k2_kernel(const K2Params p) {
   // A lane holds, of fragment i: activation row m = 32 i + r, weight rows 32 wn + 8 (e/4) + 4 hh + e%4.  Partial
   // [kh][m][32 groups of four weight rows], the group index xor-ed with m % 32 so that a wave's stores (32 rows at
   // a stride of 512 bytes) spread over the banks.
+  // 64 rows (two fragments) per pass: 2 x 64 x 128 floats fill the 64 KB.
   float* red = reinterpret_cast<float*>(lds);
+#pragma unroll
+  for (int pass = 0; pass < MFR / 2; ++pass) {
+  if (pass > 0) __syncthreads();  // the previous pass has been read
 #pragma unroll
   for (int i = 0; i < 2; ++i) {
     const uint32_t m = 32 * i + r;
@@ -322,8 +331,8 @@ __global__ __launch_bounds__(kThreads) void qmm_k2_kernel(const K2Params p) {
       const uint32_t cg = 8 * wn + 2 * eg + hh;  // weight rows 4 cg .. 4 cg + 3 of the tile
       f4 v;
 #pragma unroll
-      for (int e = 0; e < 4; ++e) v[e] = acc[i][eg * 4 + e];
-      *reinterpret_cast<f4*>(red + ((size_t)(kh * kTileM + m) * 32 + (cg ^ (m & 31))) * 4) = v;
+      for (int e = 0; e < 4; ++e) v[e] = acc[2 * pass + i][eg * 4 + e];
+      *reinterpret_cast<f4*>(red + ((size_t)(kh * 64 + m) * 32 + (cg ^ (m & 31))) * 4) = v;
     }
   }
   __syncthreads();
@@ -331,8 +340,8 @@ __global__ __launch_bounds__(kThreads) void qmm_k2_kernel(const K2Params p) {
   for (int q = 0; q < 4; ++q) {  // 64 rows x 32 groups = 2048 units of four outputs: four per thread
     const uint32_t g = q * kThreads + tid, m = g >> 5, cgp = g & 31, cg = cgp ^ (m & 31);
     f4 v = *reinterpret_cast<const f4*>(red + ((size_t)m * 32 + cgp) * 4);
-    v += *reinterpret_cast<const f4*>(red + ((size_t)(kTileM + m) * 32 + cgp) * 4);
-    const uint32_t row = row_lo + m, col = nt * kTileN + 4 * cg;
+    v += *reinterpret_cast<const f4*>(red + ((size_t)(64 + m) * 32 + cgp) * 4);
+    const uint32_t row = row_lo + 64 * pass + m, col = nt * kTileN + 4 * cg;
     if (row < p.M) {
       const uint64_t o = (uint64_t)row * p.N + col;
       if (p.epi_kind != EPI_NONE) {  // residual add / SwiGLU gate in f32, one rounding (quantized.rs:3206-3246)
@@ -353,6 +362,7 @@ __global__ __launch_bounds__(kThreads) void qmm_k2_kernel(const K2Params p) {
       *reinterpret_cast<u2*>(p.out + o) = (u2){h2bits(lo), h2bits(hi)};
     }
   }
+  }
 }
 
 }  // namespace
@@ -362,7 +372,13 @@ bool qmm_k2_supported(uint32_t N, uint32_t K, uint32_t group_size, uint32_t bits
          N % kTileN == 0 && K % (kBlockK * kUnroll) == 0;
 }
 
-int32_t launch_qmm_k2(const QmmArgs& a, uint32_t group_size, hipStream_t s) {
+bool qmm_k2_tall_supported(uint32_t group_size, uint32_t bits) {
+  return (bits == 4 && (group_size == 64 || group_size == 128)) || (bits == 8 && group_size == 128);
+}
+
+int32_t launch_qmm_k2(const QmmArgs& a, uint32_t group_size, uint32_t tile_rows, hipStream_t s) {
+  if (tile_rows != 64 && !(tile_rows == 128 && qmm_k2_tall_supported(group_size, a.bits)))
+    return fail(RMLX_INVALID_SHAPE, "qmm: no K-split kernel with %u-row tiles for bits=%u group_size=%u", tile_rows, a.bits, group_size);
   if (!qmm_k2_supported(a.N, a.K, group_size, a.bits))
     return fail(RMLX_INVALID_SHAPE, "qmm: unsupported shape N=%u K=%u bits=%u group_size=%u", a.N, a.K, a.bits, group_size);
   if (a.M == 0) return RMLX_OK;
@@ -372,20 +388,31 @@ int32_t launch_qmm_k2(const QmmArgs& a, uint32_t group_size, hipStream_t s) {
   p.w = a.w; p.s = a.s; p.b = a.b;
   p.x = static_cast<const __half*>(a.x);
   p.out = a.out; p.M = a.M; p.N = a.N; p.K = a.K;
-  p.tiles_m = (a.M + kTileM - 1) / kTileM;
+  p.tiles_m = (a.M + tile_rows - 1) / tile_rows;
   p.tiles_n = a.N / kTileN;
   p.epi_kind = a.epi_kind; p.epi = a.epi; p.epi_dtype = a.epi_dtype;
   if ((uint64_t)p.tiles_m * p.tiles_n > 0x7FFFFFFFull) return fail(RMLX_INVALID_SHAPE, "qmm: grid too large");
   const dim3 grid(p.tiles_m * p.tiles_n), block(kThreads);
-  const bool xb = a.x_dtype == RMLX_DTYPE_BF16;
-#define K2_LAUNCH(BITSV, GSV)                                                                        \
-  if (xb) hipLaunchKernelGGL((qmm_k2_kernel<BITSV, true, GSV>), grid, block, 0, s, p);              \
-  else hipLaunchKernelGGL((qmm_k2_kernel<BITSV, false, GSV>), grid, block, 0, s, p);
-#define K2_BITS(GSV) \
-  if (a.bits == 4) { K2_LAUNCH(4, GSV) } else { K2_LAUNCH(8, GSV) }
-  if (group_size == 64) { K2_BITS(64) } else if (group_size == 32) { K2_BITS(32) } else { K2_BITS(128) }
-#undef K2_BITS
-#undef K2_LAUNCH
+  const bool xb = a.x_dtype == RMLX_DTYPE_BF16, tall = tile_rows == 128;
+  auto launch = [&](auto bits_c, auto gs_c, auto mfr_c) {
+    constexpr int B = decltype(bits_c)::value, GSV = decltype(gs_c)::value, MFRV = decltype(mfr_c)::value;
+    if (xb) hipLaunchKernelGGL((qmm_k2_kernel<B, true, GSV, MFRV>), grid, block, 0, s, p);
+    else hipLaunchKernelGGL((qmm_k2_kernel<B, false, GSV, MFRV>), grid, block, 0, s, p);
+  };
+  using std::integral_constant;
+  typedef integral_constant<int, 2> Low;
+  typedef integral_constant<int, 4> Tall;
+  typedef integral_constant<int, 4> B4;
+  typedef integral_constant<int, 8> B8;
+  if (a.bits == 4) {
+    if (group_size == 64) { if (tall) launch(B4{}, integral_constant<int, 64>{}, Tall{}); else launch(B4{}, integral_constant<int, 64>{}, Low{}); }
+    else if (group_size == 128) { if (tall) launch(B4{}, integral_constant<int, 128>{}, Tall{}); else launch(B4{}, integral_constant<int, 128>{}, Low{}); }
+    else launch(B4{}, integral_constant<int, 32>{}, Low{});
+  } else {
+    if (group_size == 64) launch(B8{}, integral_constant<int, 64>{}, Low{});
+    else if (group_size == 128) { if (tall) launch(B8{}, integral_constant<int, 128>{}, Tall{}); else launch(B8{}, integral_constant<int, 128>{}, Low{}); }
+    else launch(B8{}, integral_constant<int, 32>{}, Low{});
+  }
   RMLX_HIP_CHECK(hipGetLastError());
   return RMLX_OK;
 }

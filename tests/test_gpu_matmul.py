@@ -721,6 +721,61 @@ def test_k_split_gemm_positions_epilogues_and_dispatch(hip):
         _run(hip, *make_weight(rng, 64, 256, 4), make_x(rng, 8, 256), 4, kernel=rt.KERNEL_QMM_K2)
 
 
+@pytest.mark.parametrize("bits,gs", [(4, 64), (4, 128), (8, 128)])
+@pytest.mark.parametrize("m,n,k,dtype", [(128, 128, 512, "f16"), (130, 256, 1024, "f16"), (512, 1024, 1536, "bf16"), (1, 128, 512, "f16"),
+                                         (333, 384, 2048, "f32"), (193, 128, 4096, "f16")])
+def test_k_split_gemm_tall_tiles(hip, bits, gs, m, n, k, dtype):
+    """The same kernel with 128 x 128 tiles (kernel selector 9): the weight formats it is built for, ragged M with one to
+    four empty 32-row fragments in the last tile, all activation dtypes; bit-identical to the 64-row tiles (every output
+    sums the same products in the same order)."""
+    from rmlx_amd import runtime as rt
+    rng = np.random.default_rng(bits * 1000 + gs + m + n + k + 1)
+    words, s, b = make_weight(rng, n, k, bits, gs)
+    x = make_x(rng, m, k, dtype)
+    ref = model.qmm(x_as_f64(x, dtype), words, s, b, gs, bits)
+    out = _run(hip, words, s, b, x, bits, dtype=dtype, gs=gs, kernel=rt.KERNEL_QMM_K2_TALL)
+    assert_close(out, ref, f"k-split gemm, 128-row tiles M={m} N={n} K={k} bits={bits} gs={gs} {dtype}")
+    assert np.array_equal(out, _run(hip, words, s, b, x, bits, dtype=dtype, gs=gs, kernel=rt.KERNEL_QMM_K2))
+
+
+def test_k_split_gemm_tall_tiles_positions_epilogues_and_dispatch(hip):
+    """One-hot rows against per-group scales (every fragment, lane half, k step, k half and scale word of the 128-row
+    tile); the fused epilogues; the shapes the ladder sends to the 128-row tiles; formats it is not built for."""
+    from rmlx_amd import ops, runtime as rt
+    from rmlx_amd.runtime import DeviceBuffer
+    for bits, gs in ((4, 64), (4, 128), (8, 128)):
+        n, k, m = 128, 1024, 128
+        rng = np.random.default_rng(gs * 10 + bits + 1)
+        words = np.full((n, k * bits // 32), 0x11111111 if bits == 4 else 0x01010101, np.uint32)  # q = 1 everywhere
+        s = (rng.integers(1, 64, size=(n, k // gs)) / 8.0).astype(np.float16)
+        b = np.zeros((n, k // gs), np.float16)
+        ks = rng.choice(k, size=m, replace=False)
+        x = np.zeros((m, k), np.float16)
+        x[np.arange(m), ks] = 1.0
+        out = _run(hip, words, s, b, x, bits, gs=gs, kernel=rt.KERNEL_QMM_K2_TALL)
+        assert np.array_equal(out.astype(np.float64), s[:, ks // gs].T.astype(np.float64)), f"bits={bits} gs={gs}"
+    rng = np.random.default_rng(98)
+    cus = rt.device_info()["compute_units"]
+    n, k = 2048, 1024
+    m = 128 * ((6 * cus + 9) // 10 // (n // 128) + 1) - 28  # 128-row tiles: 0.6 rounds over the chip or more; ragged
+    words, s, b = make_weight(rng, n, k, 4)
+    x = make_x(rng, m, k)
+    base = model.qmm(x_as_f64(x, "f16"), words, s, b, 64, 4)
+    auto = _run(hip, words, s, b, x, 4)
+    assert_close(auto, base, "auto")
+    assert np.array_equal(auto, _run(hip, words, s, b, x, 4, kernel=rt.KERNEL_QMM_K2_TALL))
+    qw = ops.QuantizedWeight.from_numpy(words, s, b, 64, 4)
+    xd = DeviceBuffer.from_numpy(x)
+    for edtype in (np.float16, np.float32):
+        e = rng.standard_normal((m, n)).astype(edtype)
+        ed = DeviceBuffer.from_numpy(e)
+        assert_close(ops.qmm_add_residual(xd, qw, ed).numpy(), base + e.astype(np.float64), "qmm_add_residual")
+        assert_close(ops.qmm_swiglu(xd, qw, ed).numpy(), model.silu(e.astype(np.float64)) * base, "qmm_swiglu")
+    for bits, gs in ((4, 32), (8, 64), (8, 32)):
+        with pytest.raises(ops.KernelError, match="128 x 128 K-split qmm kernel requires"):
+            _run(hip, *make_weight(rng, 128, 512, bits, gs), make_x(rng, 8, 512), bits, gs=gs, kernel=rt.KERNEL_QMM_K2_TALL)
+
+
 @pytest.mark.parametrize("bits,gs", [(4, 64), (4, 32), (4, 128), (8, 64), (8, 32)])
 @pytest.mark.parametrize("n,k", [(16, 11008), (24, 3584), (8, 2560), (16, 1408), (40, 64 * 33), (8, 128)])
 def test_single_row_gemv_any_k(hip, bits, gs, n, k):
