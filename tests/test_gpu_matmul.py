@@ -771,6 +771,17 @@ def test_k_split_gemm_tall_tiles_positions_epilogues_and_dispatch(hip):
         ed = DeviceBuffer.from_numpy(e)
         assert_close(ops.qmm_add_residual(xd, qw, ed).numpy(), base + e.astype(np.float64), "qmm_add_residual")
         assert_close(ops.qmm_swiglu(xd, qw, ed).numpy(), model.silu(e.astype(np.float64)) * base, "qmm_swiglu")
+    # the large prefill shape (4096 x 4096 weights, 4096 rows; the ladder sends it to the 128-row tiles): rows sampled
+    # from every row tile against the oracle, every row against the register-weights GEMM
+    m = n = k = 4096
+    words, s, b = make_weight(rng, n, k, 4)
+    x = make_x(rng, m, k)
+    auto = _run(hip, words, s, b, x, 4)
+    assert np.array_equal(auto, _run(hip, words, s, b, x, 4, kernel=rt.KERNEL_QMM_K2_TALL))
+    rows = (np.arange(32)[:, None] * 128 + rng.integers(0, 128, size=(32, 2))).reshape(-1)
+    assert_close(auto[rows], model.qmm(x_as_f64(x[rows], "f16"), words, s, b, 64, 4), "4096 x 4096 x 4096, sampled rows")
+    other = _run(hip, words, s, b, x, 4, kernel=rt.KERNEL_QMM_RW).astype(np.float64)
+    assert np.abs(auto.astype(np.float64) - other).max() <= 2.0 ** -9 * np.abs(other).max()  # two f16 roundings of one value
     for bits, gs in ((4, 32), (8, 64), (8, 32)):
         with pytest.raises(ops.KernelError, match="128 x 128 K-split qmm kernel requires"):
             _run(hip, *make_weight(rng, 128, 512, bits, gs), make_x(rng, 8, 512), bits, gs=gs, kernel=rt.KERNEL_QMM_K2_TALL)
