@@ -142,7 +142,7 @@ int32_t rmlx_hip_affine_quantized_matmul_batched(const rmlx_qweight* qw, const r
  * 6 = multi-row streaming GEMV also for a single row (group sizes 64 and 128),
  * 7 = K-split MFMA GEMM (64 x 128 tiles, 32x32x16 MFMAs; N % 128 == 0, K % 512 == 0; what kernel 2 resolves to
  * when that grid is one round over most of the chip), 8 = the register-weights GEMM whatever the shape,
- * 9 = the K-split MFMA GEMM with 128 x 128 tiles (4-bit weights with group size 64 / 128, 8-bit with group size 128; what
+ * 9 = the K-split MFMA GEMM with 128 x 128 tiles (not for 8-bit weights at group size 32 / 64 with bf16 activations; what
  * kernel 2 resolves to when those tiles make 0.6 rounds over the chip or more). */
 int32_t rmlx_hip_qmm_select(const rmlx_qweight* qw, const rmlx_array* x, int32_t kernel,
                             void* out_f16_dev, size_t out_bytes, rmlx_stream stream);

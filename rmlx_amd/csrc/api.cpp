@@ -195,7 +195,7 @@ int32_t run_matmul_plain(const rmlx_qweight* qw, const void* x, int32_t x_dtype,
   const bool can_qmm_rw = ptr_ok && qmm_rw_supported(N, K, qw->group_size, qw->bits);
   const bool can_qmm = can_qmm_lds || can_qmm_rw;
   const bool can_qmm_k2 = ptr_ok && qmm_k2_supported(N, K, qw->group_size, qw->bits);
-  const bool can_qmm_k2_tall = can_qmm_k2 && qmm_k2_tall_supported(qw->group_size, qw->bits);
+  const bool can_qmm_k2_tall = can_qmm_k2 && qmm_k2_tall_supported(qw->group_size, qw->bits, x_dtype == RMLX_DTYPE_BF16);
 
   if (kernel == KERNEL_AUTO) {
     // The multi-row GEMV streams the weights once per pass of 8 rows (4-bit; two passes share a workgroup
@@ -236,8 +236,8 @@ int32_t run_matmul_plain(const rmlx_qweight* qw, const void* x, int32_t x_dtype,
                 "buffers (N=%u K=%u bits=%u group_size=%u)", N, K, qw->bits, qw->group_size);
   } else if (kernel == KERNEL_QMM_K2_TALL && !can_qmm_k2_tall) {
     return fail(RMLX_INVALID_SHAPE,
-                "the 128 x 128 K-split qmm kernel requires 4-bit weights with group size 64 or 128 or 8-bit weights with group "
-                "size 128, N %% 128 == 0, K %% 512 == 0 and 16-byte aligned buffers (N=%u K=%u bits=%u group_size=%u)",
+                "the 128 x 128 K-split qmm kernel requires bits in {4,8} (8-bit weights at group size 32 / 64: f16 or f32 "
+                "activations), N %% 128 == 0, K %% 512 == 0 and 16-byte aligned buffers (N=%u K=%u bits=%u group_size=%u)",
                 N, K, qw->bits, qw->group_size);
   } else if (kernel < 0 || kernel > KERNEL_QMM_K2_TALL) {
     return fail(RMLX_NOT_FOUND, "unknown kernel selector %d", kernel);

@@ -185,9 +185,9 @@ bool qmm_rw_supported(uint32_t N, uint32_t K, uint32_t group_size, uint32_t bits
 int32_t launch_qmm_rw(const QmmArgs& a, uint32_t group_size, hipStream_t s);
 // K-split GEMM (qmm_k2.hip) for prefill-sized batches: 64 x 128 or 128 x 128 tiles (tile_rows), 32x32x16 MFMAs, the two
 // halves of a workgroup split K; f16 / bf16 activations, no workspace, fused store epilogue.  The 128-row tile is built
-// for the weight formats whose kernel fits the register file (4-bit with group size 64 / 128, 8-bit with group size 128).
+// for every format whose kernel fits the register file (all but 8-bit weights at group size 32 / 64 with bf16 activations).
 bool qmm_k2_supported(uint32_t N, uint32_t K, uint32_t group_size, uint32_t bits);
-bool qmm_k2_tall_supported(uint32_t group_size, uint32_t bits);
+bool qmm_k2_tall_supported(uint32_t group_size, uint32_t bits, bool x_bf16);
 int32_t launch_qmm_k2(const QmmArgs& a, uint32_t group_size, uint32_t tile_rows, hipStream_t s);
 // Grouped form of the same GEMM for the expert projections of batches with many rows per expert: every
 // row tile (kGroupedTileRows rows of one expert) takes its expert and rows from a device table of

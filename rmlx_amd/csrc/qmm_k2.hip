@@ -153,7 +153,10 @@ __global__ __launch_bounds__(kThreads) void qmm_k2_kernel(const K2Params p) {
 #pragma unroll
     for (int e = 0; e < 16; ++e) acc[i][e] = 0.f;
 
-  u4 ra[2][kAL];              // activation chunks in flight (global -> registers -> LDS)
+  // activation chunks in flight (global -> registers -> LDS): two register sets (a chunk is requested two blocks before
+  // it is written to LDS), or one where the second would not fit the register file (requested one block before)
+  constexpr int kSets = (MFR == 4 && (BITS == 8 || GS == 32)) ? 1 : 2;
+  u4 ra[kSets][kAL];
   u4 wq[kUnroll][WV];         // weights, four blocks ahead
   u4 s_cur[kSbVecs], b_cur[kSbVecs], s_nxt[kSbVecs], b_nxt[kSbVecs];  // scales / biases of four blocks
 
@@ -245,14 +248,20 @@ __global__ __launch_bounds__(kThreads) void qmm_k2_kernel(const K2Params p) {
   const uint32_t last = S - 1;
   auto clampi = [&](uint32_t it) { return it < last ? it : last; };
   load_a(0, ra[0]);
-  load_a(clampi(1), ra[1]);
+  if constexpr (kSets == 2) load_a(clampi(1), ra[kSets - 1]);
   load_sb(0, s_cur, b_cur);
 #pragma unroll
   for (int u = 0; u < kUnroll; ++u) load_w(u, u);  // (S >= 4)
   store_a(0, ra[0]);
-  store_a(1, ra[1]);
-  load_a(clampi(2), ra[0]);
-  load_a(clampi(3), ra[1]);
+  if constexpr (kSets == 2) {
+    store_a(1, ra[1]);
+    load_a(clampi(2), ra[0]);
+    load_a(clampi(3), ra[1]);
+  } else {
+    load_a(clampi(1), ra[0]);
+    store_a(1, ra[0]);
+    load_a(clampi(2), ra[0]);
+  }
   __syncthreads();
   h8 bf[MFR][4];
 #pragma unroll
@@ -289,8 +298,11 @@ __global__ __launch_bounds__(kThreads) void qmm_k2_kernel(const K2Params p) {
         scale_pair(u + 1, s2, b2);
         aw_nxt = weight_operand(u + 1, 0, s2, b2);
       }
-      if (ks < kAL && writes) lds[st_wr * kChunkUnits + ks * 512 + lds_w0] = to_slot_order(ra[u % 2][ks]);
-      if (MAIN && ks == (kAL > 3 ? kAL - 1 : 2)) load_a(it + 4, ra[u % 2]);  // (its last unit has just been written)
+      if (ks < kAL && writes) lds[st_wr * kChunkUnits + ks * 512 + lds_w0] = to_slot_order(ra[u % kSets][ks]);
+      if (ks == (kAL > 3 ? kAL - 1 : 2)) {  // (the set's last unit has just been written)
+        if constexpr (kSets == 2) { if (MAIN) load_a(it + 4, ra[u % 2]); }
+        else if (it + 3 < S) load_a(it + 3, ra[0]);  // (uniform)
+      }
       aw = aw_nxt;
       __builtin_amdgcn_sched_barrier(0);
     }
@@ -372,13 +384,16 @@ bool qmm_k2_supported(uint32_t N, uint32_t K, uint32_t group_size, uint32_t bits
          N % kTileN == 0 && K % (kBlockK * kUnroll) == 0;
 }
 
-bool qmm_k2_tall_supported(uint32_t group_size, uint32_t bits) {
-  return (bits == 4 && (group_size == 64 || group_size == 128)) || (bits == 8 && group_size == 128);
+bool qmm_k2_tall_supported(uint32_t group_size, uint32_t bits, bool x_bf16) {
+  // (8-bit weights at group size 32 / 64 with bf16 activations: that build would spill registers)
+  return (bits == 4 || bits == 8) && (group_size == 32 || group_size == 64 || group_size == 128) &&
+         !(bits == 8 && x_bf16 && group_size != 128);
 }
 
 int32_t launch_qmm_k2(const QmmArgs& a, uint32_t group_size, uint32_t tile_rows, hipStream_t s) {
-  if (tile_rows != 64 && !(tile_rows == 128 && qmm_k2_tall_supported(group_size, a.bits)))
-    return fail(RMLX_INVALID_SHAPE, "qmm: no K-split kernel with %u-row tiles for bits=%u group_size=%u", tile_rows, a.bits, group_size);
+  if (tile_rows != 64 && !(tile_rows == 128 && qmm_k2_tall_supported(group_size, a.bits, a.x_dtype == RMLX_DTYPE_BF16)))
+    return fail(RMLX_INVALID_SHAPE, "qmm: no K-split kernel with %u-row tiles for bits=%u group_size=%u (%s activations)", tile_rows,
+                a.bits, group_size, a.x_dtype == RMLX_DTYPE_BF16 ? "bf16" : "f16");
   if (!qmm_k2_supported(a.N, a.K, group_size, a.bits))
     return fail(RMLX_INVALID_SHAPE, "qmm: unsupported shape N=%u K=%u bits=%u group_size=%u", a.N, a.K, a.bits, group_size);
   if (a.M == 0) return RMLX_OK;
@@ -396,23 +411,24 @@ int32_t launch_qmm_k2(const QmmArgs& a, uint32_t group_size, uint32_t tile_rows,
   const bool xb = a.x_dtype == RMLX_DTYPE_BF16, tall = tile_rows == 128;
   auto launch = [&](auto bits_c, auto gs_c, auto mfr_c) {
     constexpr int B = decltype(bits_c)::value, GSV = decltype(gs_c)::value, MFRV = decltype(mfr_c)::value;
-    if (xb) hipLaunchKernelGGL((qmm_k2_kernel<B, true, GSV, MFRV>), grid, block, 0, s, p);
-    else hipLaunchKernelGGL((qmm_k2_kernel<B, false, GSV, MFRV>), grid, block, 0, s, p);
+    if (xb) {
+      if constexpr (!(MFRV == 4 && B == 8 && GSV != 128)) hipLaunchKernelGGL((qmm_k2_kernel<B, true, GSV, MFRV>), grid, block, 0, s, p);
+    } else {
+      hipLaunchKernelGGL((qmm_k2_kernel<B, false, GSV, MFRV>), grid, block, 0, s, p);
+    }
   };
   using std::integral_constant;
   typedef integral_constant<int, 2> Low;
   typedef integral_constant<int, 4> Tall;
   typedef integral_constant<int, 4> B4;
   typedef integral_constant<int, 8> B8;
-  if (a.bits == 4) {
-    if (group_size == 64) { if (tall) launch(B4{}, integral_constant<int, 64>{}, Tall{}); else launch(B4{}, integral_constant<int, 64>{}, Low{}); }
-    else if (group_size == 128) { if (tall) launch(B4{}, integral_constant<int, 128>{}, Tall{}); else launch(B4{}, integral_constant<int, 128>{}, Low{}); }
-    else launch(B4{}, integral_constant<int, 32>{}, Low{});
-  } else {
-    if (group_size == 64) launch(B8{}, integral_constant<int, 64>{}, Low{});
-    else if (group_size == 128) { if (tall) launch(B8{}, integral_constant<int, 128>{}, Tall{}); else launch(B8{}, integral_constant<int, 128>{}, Low{}); }
-    else launch(B8{}, integral_constant<int, 32>{}, Low{});
-  }
+  auto by_height = [&](auto bits_c, auto gs_c) { if (tall) launch(bits_c, gs_c, Tall{}); else launch(bits_c, gs_c, Low{}); };
+  auto by_group = [&](auto bits_c) {
+    if (group_size == 64) by_height(bits_c, integral_constant<int, 64>{});
+    else if (group_size == 128) by_height(bits_c, integral_constant<int, 128>{});
+    else by_height(bits_c, integral_constant<int, 32>{});
+  };
+  if (a.bits == 4) by_group(B4{}); else by_group(B8{});
   RMLX_HIP_CHECK(hipGetLastError());
   return RMLX_OK;
 }

@@ -721,17 +721,22 @@ def test_k_split_gemm_positions_epilogues_and_dispatch(hip):
         _run(hip, *make_weight(rng, 64, 256, 4), make_x(rng, 8, 256), 4, kernel=rt.KERNEL_QMM_K2)
 
 
-@pytest.mark.parametrize("bits,gs", [(4, 64), (4, 128), (8, 128)])
+@pytest.mark.parametrize("bits,gs", [(4, 64), (4, 32), (4, 128), (8, 64), (8, 32), (8, 128)])
 @pytest.mark.parametrize("m,n,k,dtype", [(128, 128, 512, "f16"), (130, 256, 1024, "f16"), (512, 1024, 1536, "bf16"), (1, 128, 512, "f16"),
                                          (333, 384, 2048, "f32"), (193, 128, 4096, "f16")])
 def test_k_split_gemm_tall_tiles(hip, bits, gs, m, n, k, dtype):
-    """The same kernel with 128 x 128 tiles (kernel selector 9): the weight formats it is built for, ragged M with one to
-    four empty 32-row fragments in the last tile, all activation dtypes; bit-identical to the 64-row tiles (every output
-    sums the same products in the same order)."""
-    from rmlx_amd import runtime as rt
+    """The same kernel with 128 x 128 tiles (kernel selector 9): every bit width and group size (with one or two
+    activation register sets), ragged M with one to four empty 32-row fragments in the last tile, all activation dtypes;
+    bit-identical to the 64-row tiles (every output sums the same products in the same order).  8-bit weights at group
+    size 32 / 64 with bf16 activations have no such build."""
+    from rmlx_amd import ops, runtime as rt
     rng = np.random.default_rng(bits * 1000 + gs + m + n + k + 1)
     words, s, b = make_weight(rng, n, k, bits, gs)
     x = make_x(rng, m, k, dtype)
+    if bits == 8 and gs != 128 and dtype == "bf16":
+        with pytest.raises(ops.KernelError, match="128 x 128 K-split qmm kernel requires"):
+            _run(hip, words, s, b, x, bits, dtype=dtype, gs=gs, kernel=rt.KERNEL_QMM_K2_TALL)
+        return
     ref = model.qmm(x_as_f64(x, dtype), words, s, b, gs, bits)
     out = _run(hip, words, s, b, x, bits, dtype=dtype, gs=gs, kernel=rt.KERNEL_QMM_K2_TALL)
     assert_close(out, ref, f"k-split gemm, 128-row tiles M={m} N={n} K={k} bits={bits} gs={gs} {dtype}")
@@ -740,10 +745,10 @@ def test_k_split_gemm_tall_tiles(hip, bits, gs, m, n, k, dtype):
 
 def test_k_split_gemm_tall_tiles_positions_epilogues_and_dispatch(hip):
     """One-hot rows against per-group scales (every fragment, lane half, k step, k half and scale word of the 128-row
-    tile); the fused epilogues; the shapes the ladder sends to the 128-row tiles; formats it is not built for."""
+    tile); the fused epilogues; the shapes the ladder sends to the 128-row tiles; shapes it does not take."""
     from rmlx_amd import ops, runtime as rt
     from rmlx_amd.runtime import DeviceBuffer
-    for bits, gs in ((4, 64), (4, 128), (8, 128)):
+    for bits, gs in ((4, 64), (4, 32), (4, 128), (8, 64), (8, 32), (8, 128)):
         n, k, m = 128, 1024, 128
         rng = np.random.default_rng(gs * 10 + bits + 1)
         words = np.full((n, k * bits // 32), 0x11111111 if bits == 4 else 0x01010101, np.uint32)  # q = 1 everywhere
@@ -782,9 +787,8 @@ def test_k_split_gemm_tall_tiles_positions_epilogues_and_dispatch(hip):
     assert_close(auto[rows], model.qmm(x_as_f64(x[rows], "f16"), words, s, b, 64, 4), "4096 x 4096 x 4096, sampled rows")
     other = _run(hip, words, s, b, x, 4, kernel=rt.KERNEL_QMM_RW).astype(np.float64)
     assert np.abs(auto.astype(np.float64) - other).max() <= 2.0 ** -9 * np.abs(other).max()  # two f16 roundings of one value
-    for bits, gs in ((4, 32), (8, 64), (8, 32)):
-        with pytest.raises(ops.KernelError, match="128 x 128 K-split qmm kernel requires"):
-            _run(hip, *make_weight(rng, 128, 512, bits, gs), make_x(rng, 8, 512), bits, gs=gs, kernel=rt.KERNEL_QMM_K2_TALL)
+    with pytest.raises(ops.KernelError, match="128 x 128 K-split qmm kernel requires"):
+        _run(hip, *make_weight(rng, 64, 512, 4, 64), make_x(rng, 8, 512), 4, kernel=rt.KERNEL_QMM_K2_TALL)  # N % 128 != 0
 
 
 @pytest.mark.parametrize("bits,gs", [(4, 64), (4, 32), (4, 128), (8, 64), (8, 32)])
