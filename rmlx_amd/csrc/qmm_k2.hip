@@ -96,8 +96,12 @@ __device__ __forceinline__ uint32_t act_slot(uint32_t R, uint32_t seg) {
 
 // MFR: activation fragments of 32 rows per tile (2: 64 x 128 tiles; 4: 128 x 128 tiles, every unpacked weight operand
 // then feeds four MFMAs)
-template <int BITS, bool XBF16, int GS, int MFR>
+// SBLDS: the tile's scales and biases wait in LDS (64-row tiles, group size 64, K <= 4096: a row's 128 bytes of either are
+// one cache line, fetched once; read from global memory 16 bytes per four blocks, every read pulls the whole line
+// through the CU's L1 again: measured 1.56 x the useful bytes between L2 and the CU).
+template <int BITS, bool XBF16, int GS, int MFR, bool SBLDS = false>
 __global__ __launch_bounds__(kThreads) void qmm_k2_kernel(const K2Params p) {
+  static_assert(!SBLDS || (GS == 64 && MFR == 2), "scales in LDS: 64-row tiles, group size 64");
   constexpr int kTileM = 32 * MFR;
   constexpr int kChunkUnits = kTileM * 16;               // 16-byte units of one activation chunk (rows x 128 k): 1024 / 2048
   constexpr int kAL = kChunkUnits / kThreads;            // units per thread and chunk: 2 / 4
@@ -196,8 +200,14 @@ __global__ __launch_bounds__(kThreads) void qmm_k2_kernel(const K2Params p) {
     for (int v = 0; v < WV; ++v) wq[u][v] = __builtin_amdgcn_raw_buffer_load_b128(wr, woff, it * (16 * 4 * WV) + v * 16, 0);
   };
   // the scales / biases of blocks 4 blk .. 4 blk + 3 of this lane's row
+  // (SBLDS: slot of (row, unit of four blocks) behind the two activation stages; the xor spreads the 32 rows of a wave
+  // over the banks)
+  auto sb_slot = [&](uint32_t which, uint32_t row, uint32_t unit) { return 2048 + which * 1024 + row * 8 + (unit ^ (row & 7)); };
   auto load_sb = [&](uint32_t blk, u4 (&ds)[kSbVecs], u4 (&db)[kSbVecs]) {
-    if (GS == 128) {
+    if constexpr (SBLDS) {
+      ds[0] = lds[sb_slot(0, 32 * wn + r, blk & 7)];
+      db[0] = lds[sb_slot(1, 32 * wn + r, blk & 7)];
+    } else if (GS == 128) {
       const u2 sv = __builtin_amdgcn_raw_buffer_load_b64(sr, soff, blk * 8, 0), bv = __builtin_amdgcn_raw_buffer_load_b64(br, soff, blk * 8, 0);
       ds[0] = (u4){sv.x, sv.y, 0u, 0u};
       db[0] = (u4){bv.x, bv.y, 0u, 0u};
@@ -253,7 +263,17 @@ __global__ __launch_bounds__(kThreads) void qmm_k2_kernel(const K2Params p) {
   auto clampi = [&](uint32_t it) { return it < last ? it : last; };
   load_a(0, ra[0]);
   if constexpr (kSets == 2) load_a(clampi(1), ra[kSets - 1]);
-  load_sb(0, s_cur, b_cur);
+  if constexpr (SBLDS) {  // 128 rows x (scales, biases) x up to 8 units of 16 bytes: four pieces per thread, whole lines per row
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const uint32_t piece = q * kThreads + tid, which = piece >> 10, row = (piece >> 3) & 127, unit = piece & 7;
+      u4 v = (u4){0u, 0u, 0u, 0u};
+      if (unit * 16 < G * 2) v = __builtin_amdgcn_raw_buffer_load_b128(which ? br : sr, row * G * 2 + unit * 16, 0, 0);
+      lds[sb_slot(which, row, unit)] = v;
+    }
+  } else {
+    load_sb(0, s_cur, b_cur);
+  }
 #pragma unroll
   for (int u = 0; u < kUnroll; ++u) load_w(u, u);  // (S >= 4)
   store_a(0, ra[0]);
@@ -267,6 +287,7 @@ __global__ __launch_bounds__(kThreads) void qmm_k2_kernel(const K2Params p) {
     load_a(clampi(2), ra[0]);
   }
   __syncthreads();
+  if constexpr (SBLDS) load_sb(0, s_cur, b_cur);
   h8 bf[MFR][4];
 #pragma unroll
   for (int i = 0; i < MFR; ++i)
@@ -413,8 +434,16 @@ int32_t launch_qmm_k2(const QmmArgs& a, uint32_t group_size, uint32_t tile_rows,
   if ((uint64_t)p.tiles_m * p.tiles_n > 0x7FFFFFFFull) return fail(RMLX_INVALID_SHAPE, "qmm: grid too large");
   const dim3 grid(p.tiles_m * p.tiles_n), block(kThreads);
   const bool xb = a.x_dtype == RMLX_DTYPE_BF16, tall = tile_rows == 128;
+  const bool sb_lds = group_size == 64 && !tall && a.K <= 4096;
   auto launch = [&](auto bits_c, auto gs_c, auto mfr_c) {
     constexpr int B = decltype(bits_c)::value, GSV = decltype(gs_c)::value, MFRV = decltype(mfr_c)::value;
+    if constexpr (GSV == 64 && MFRV == 2) {
+      if (sb_lds) {
+        if (xb) hipLaunchKernelGGL((qmm_k2_kernel<B, true, GSV, MFRV, true>), grid, block, 0, s, p);
+        else hipLaunchKernelGGL((qmm_k2_kernel<B, false, GSV, MFRV, true>), grid, block, 0, s, p);
+        return;
+      }
+    }
     if (xb) {
       if constexpr (!(MFRV == 4 && B == 8 && GSV != 128)) hipLaunchKernelGGL((qmm_k2_kernel<B, true, GSV, MFRV>), grid, block, 0, s, p);
     } else {

@@ -671,10 +671,12 @@ def test_qmm_group_size_positions(hip):
 
 @pytest.mark.parametrize("bits,gs", [(4, 64), (4, 32), (4, 128), (8, 64), (8, 32), (8, 128)])
 @pytest.mark.parametrize("m,n,k,dtype", [(64, 128, 512, "f16"), (130, 256, 1024, "f16"), (512, 1024, 1536, "bf16"), (1, 128, 512, "f16"),
-                                         (333, 384, 2048, "f32"), (65, 128, 4096, "f16")])
+                                         (333, 384, 2048, "f32"), (65, 128, 4096, "f16"), (96, 256, 4608, "f16")])
 def test_k_split_gemm(hip, bits, gs, m, n, k, dtype):
     """The K-split GEMM (64 x 128 tiles, 32x32x16 MFMAs; kernel selector 7) on its own: every bit width and group
-    size, ragged M (rows past M read as zero), one and several k-block groups, all activation dtypes."""
+    size, ragged M (rows past M read as zero), one and several k-block groups, all activation dtypes; at group size 64
+    K up to 4096 (scales and biases staged in LDS, rows shorter than a cache line included) and beyond (read from
+    global memory as at the other group sizes)."""
     from rmlx_amd import runtime as rt
     rng = np.random.default_rng(bits * 1000 + gs + m + n + k)
     words, s, b = make_weight(rng, n, k, bits, gs)
