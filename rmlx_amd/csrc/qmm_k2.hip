@@ -22,8 +22,8 @@
 //     loads past the last block are simply not issued, so every s_waitcnt count is exact.
 //   * At the end the two k halves are added through LDS (fixed order: deterministic), which also transposes the
 //     accumulator layout into row-contiguous stores, with the fused epilogue.
-//   * A SIMD issues a matrix or a vector instruction, not both at once (their times add: 16 MFMAs x 32 clk + 126 vector
-//     instructions x 4 clk per block of the 64-row tile, which is what the k loop takes).  For batches that fill the chip
+//   * The vector instructions of the unpacking hide behind the matrix instructions only in part (measured: the k loop of
+//     the 64-row tile takes the sum, 16 MFMAs x 32 clk + 126 vector instructions x 4 clk per block and SIMD).  For batches that fill the chip
 //     with 128 x 128 tiles the same code runs with four activation fragments per wave (MFR = 4): every unpacked weight
 //     operand feeds four MFMAs, 64 MFMAs against 71 vector instructions per wave and block.
 #include <type_traits>
