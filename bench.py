@@ -30,16 +30,25 @@ GEMM_MIN_LAUNCHES = 10000  # the clock needs tens of milliseconds of sustained m
 SETTLE_S = 0.25            # untimed run of the workload in front of every timed region
 
 
-def measured_traffic():
-    """HBM-side bytes per launch of the two roofline kernels, from the committed rocprofv3 counter summary
-    (lines `traffic_bytes_per_launch <key> <bytes>`; FETCH_SIZE and WRITE_SIZE of two counter runs of this
-    script, each scaled by what it reads for the plain copy this script also launches).  Counters cannot be
-    read from inside the process, so the figures travel in that file; None when it is absent."""
-    out = {}
-    path = os.path.join(ROOT, "profiles", "bench_hbm_traffic_pmc.txt")
-    if os.path.exists(path):
-        for m in re.finditer(r"traffic_bytes_per_launch\s+(\S+)\s+(\d+)", open(path).read()):
-            out[m.group(1)] = int(m.group(2))
+def measured_profiles():
+    """Figures that only a profiler run can give, read from the committed rocprofv3 summaries under profiles/
+    (counters and traces cannot be read from inside the process): `traffic_bytes_per_launch <key> <bytes>` (FETCH_SIZE
+    + WRITE_SIZE of two counter runs of this script, each scaled by what it reads for the plain copy this script also
+    launches) and `kernel_trace_avg_us <key> <us>` (average kernel duration in a kernel trace of this script).  Every
+    figure is returned with the file it came from and that file's `measured_at` line, so a stale figure can be told."""
+    out = {"traffic": {}, "trace_us": {}}
+    pdir = os.path.join(ROOT, "profiles")
+    if os.path.isdir(pdir):
+        for name in sorted(os.listdir(pdir)):
+            if not name.endswith(".txt"):
+                continue
+            text = open(os.path.join(pdir, name)).read()
+            at = re.search(r"^measured_at\s+(.+)$", text, re.M)
+            src = {"file": f"profiles/{name}", "measured_at": at.group(1).strip() if at else None}
+            for m in re.finditer(r"^traffic_bytes_per_launch\s+(\S+)\s+(\d+)", text, re.M):
+                out["traffic"][m.group(1)] = dict(src, bytes=int(m.group(2)))
+            for m in re.finditer(r"^kernel_trace_avg_us\s+(\S+)\s+([0-9.]+)", text, re.M):
+                out["trace_us"][m.group(1)] = dict(src, us=float(m.group(2)))
     return out
 
 
@@ -66,15 +75,15 @@ class Timer:
         self.e0, self.e1 = rt.Event(), rt.Event()
         self.cap = 0  # --max-launches: also bounds the trains of the settle phase
 
-    def run(self, fn, launches, warmup, chunk=TRAIN):
+    def run(self, fn, launches, warmup, chunk=TRAIN, uncapped=False):
         """fn(c) enqueues c launches.  Warm-up, an untimed settle phase of about SETTLE_S, then `launches`
         launches between two events; returns milliseconds per launch."""
-        if self.cap > 0:
+        if self.cap > 0 and not uncapped:
             launches, warmup, chunk = min(launches, self.cap), min(warmup, self.cap), min(chunk, self.cap)
         fn(max(1, warmup))
         self.stream.sync()
         t0 = time.perf_counter()
-        while time.perf_counter() - t0 < SETTLE_S:
+        while time.perf_counter() - t0 < (SETTLE_S if self.cap == 0 else 0.0):
             fn(chunk)
             self.stream.sync()
         self.e0.record(self.stream)
@@ -90,7 +99,7 @@ class Timer:
 
 
 def bench_matmul(ops, rt, timer, rng, m, n, k, bits, x_dtype, launches, warmup, min_total_bytes, check=True, kernel=0,
-                 check_rows=None):
+                 check_rows=None, graph=False):
     from oracle import model
     wbytes = n * k * bits // 8 + 4 * (n * k // 64)
     n_sets = max(1, -(-min_total_bytes // wbytes))
@@ -109,7 +118,19 @@ def bench_matmul(ops, rt, timer, rng, m, n, k, bits, x_dtype, launches, warmup, 
         xd = rt.DeviceBuffer.from_numpy(xh)
         x64 = xh.astype(np.float64)
     outs = [rt.DeviceBuffer((m, n), rt.F16) for _ in range(min(n_sets, 8))]
-    ms = timer.run(lambda c: ops.qmm_encode_many(qws, xd, outs, c, stream=timer.stream, kernel=kernel), launches, warmup)
+    if graph:  # the train is recorded once and replayed: no host work per launch (kernel nodes only)
+        with rt.Graph.record(timer.stream) as g:
+            ops.qmm_encode_many(qws, xd, outs, TRAIN, stream=timer.stream, kernel=kernel)
+
+        def replay(c):
+            for _ in range(max(1, c // TRAIN)):
+                g.launch()
+        launches = max(TRAIN, launches // TRAIN * TRAIN)
+        if timer.cap > 0:
+            launches = TRAIN
+        ms = timer.run(replay, launches, warmup, chunk=TRAIN, uncapped=True)
+    else:
+        ms = timer.run(lambda c: ops.qmm_encode_many(qws, xd, outs, c, stream=timer.stream, kernel=kernel), launches, warmup)
     res = {"us": ms * 1e3, "launches": launches, "n_weight_sets": n_sets,
            "bytes": matmul_bytes(m, n, k, bits, act_bytes=2), "flops": 2 * m * n * k}
     res["gbs"] = res["bytes"] / (ms * 1e-3) / 1e9
@@ -367,6 +388,8 @@ def main():
     ap.add_argument("--only", default="", help="comma-separated sections: headline, floors, qmv, qmm, dequant, gather, moe, moe8, large")
     ap.add_argument("--quick", action="store_true", help="headline and floors only, short CPU baseline")
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--no-graph", action="store_true",
+                    help="skip the second headline measurement that replays the train from a recorded graph")
     ap.add_argument("--max-launches", type=int, default=0,
                     help="cap on the launches of every timed run (for hardware-counter runs, where each dispatch is slow)")
     args = ap.parse_args()
@@ -391,12 +414,18 @@ def main():
 
     def progress(what):  # (a line per section on stderr: long profiler runs are not silent)
         print(f"[bench] {what}", file=sys.stderr, flush=True)
-    traffic = measured_traffic()
+    prof = measured_profiles()
 
     # ---- headline: Q4 qmv M=1 K=N=4096, weights cycled through > 1 GiB ---------------------------------
     progress("headline")
     head = bench_matmul(ops, rt, timer, rng, 1, 4096, 4096, 4, "f16", launches, warm, GiB + GiB // 8)
     extra = {"device": info, "launches_per_step": TRAIN, "q4_qmv_m1_4096": head}
+    if not args.no_graph:
+        # The same train recorded once and replayed (kernel nodes only): no host work per launch, so a kernel trace
+        # of this section shows the kernels as close together as they run without the tracer.
+        progress("headline, graph replay")
+        extra["q4_qmv_m1_4096_graph_replay"] = bench_matmul(ops, rt, timer, rng, 1, 4096, 4096, 4, "f16", launches, TRAIN,
+                                                            GiB + GiB // 8, graph=True)
     # A plain copy of known size (identity `index_gather`, 128 MiB in, 128 MiB out) so that a counter
     # run of this same command can scale FETCH_SIZE / WRITE_SIZE by what they read for it.
     rows = 16384
@@ -431,11 +460,11 @@ def main():
         progress("qmm")
         for m in (128, 512, 4096):
             m_launches = gemm_launches if m <= 512 else max(50, gemm_launches // 10)
-            r = bench_matmul(ops, rt, timer, rng, m, 4096, 4096, 4, "f16", m_launches, train_warm, 4 * 9437184)
+            r = bench_matmul(ops, rt, timer, rng, m, 4096, 4096, 4, "f16", m_launches, train_warm, GiB + GiB // 8)
             r["mfma_frac"] = r["tflops"] / MFMA_F16_PEAK_TF
             extra[f"q4_qmm_m{m}_4096"] = r
         for name, kern in (("q8_qmm_bf16_m128_n12288", rt.KERNEL_AUTO), ("q8_qmm_bf16_m128_n12288_bf16_mfma", rt.KERNEL_QMM_BF16)):
-            r = bench_matmul(ops, rt, timer, rng, 128, 12288, 4096, 8, "bf16", gemm_launches, train_warm, 4 * 53477376, kernel=kern)
+            r = bench_matmul(ops, rt, timer, rng, 128, 12288, 4096, 8, "bf16", gemm_launches, train_warm, GiB + GiB // 8, kernel=kern)
             r["mfma_frac"] = r["tflops"] / MFMA_F16_PEAK_TF
             extra[name] = r
     if "dequant" in sections:
@@ -455,7 +484,7 @@ def main():
                 r["hbm_frac"] = r["gbs"] / HBM_PEAK_GBS
                 extra[f"gather_qmm_q4_b{batch}_m{mpb}"] = r
         if "moe" in sections:
-            for T in (4, 32, 128, 512, 2048):  # from 6 rows per expert on average on the grouped MFMA GEMM
+            for T in (4, 32, 128, 512, 2048):  # from 10 rows per expert on average on the grouped MFMA GEMM
                 r = bench_moe(ops, rt, timer, rng, T, calls if T <= 128 else max(50, calls // 4), experts)
                 r["tflops"] = r["flops"] / (r["us"] * 1e-6) / 1e12
                 r["mfma_frac"] = r["tflops"] / MFMA_F16_PEAK_TF
@@ -494,17 +523,42 @@ def main():
                                f"{head['n_weight_sets']} distinct weight sets cycled (HBM-resident, > 1 GiB)",
                    "launches_per_step": TRAIN, "parity_max_err": head.get("max_err"), "parity_tol": head.get("tol")},
         "roofline": {"bound": "hbm", "achieved": head["gbs"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": head["gbs"] / HBM_PEAK_GBS, "traffic": traffic.get("qmv_q4_m1_4096"),
+                     "frac": head["gbs"] / HBM_PEAK_GBS, "traffic": None,
                      "kernel": "qmv_m1_kernel", "bytes_per_launch": head["bytes"], "avg_launch_us": head["us"]},
     }
+
+    def annotate(roof, key, algorithmic, peak_per_us):
+        """Adds what the committed profiler summaries hold for this kernel: HBM traffic per launch and the average
+        kernel duration of a kernel trace (with the fraction it gives), each with its source file."""
+        t = prof["traffic"].get(key)
+        if t is not None:
+            roof["traffic"], roof["traffic_source"] = t["bytes"], {k: t[k] for k in ("file", "measured_at")}
+        k = prof["trace_us"].get(key)
+        if k is not None:
+            roof["kernel_trace_avg_us"] = k["us"]
+            roof["frac_kernel_trace"] = algorithmic / k["us"] / peak_per_us
+            roof["kernel_trace_source"] = {x: k[x] for x in ("file", "measured_at")}
+
+    annotate(line["roofline"], "qmv_q4_m1_4096", head["bytes"], HBM_PEAK_GBS * 1e3)
+    g = extra.get("q4_qmv_m1_4096_graph_replay")
+    if g is not None:
+        line["roofline"]["graph_replay_launch_us"] = g["us"]
+        line["roofline"]["frac_graph_replay"] = g["gbs"] / HBM_PEAK_GBS
+    fl = extra.get("floors", {}).get("read_9.45MB")
+    if fl is not None:
+        # what a kernel that only reads the same bytes reaches in the same train: the ceiling of `frac` at this size
+        line["roofline"]["floor_frac"] = fl["gbs"] / HBM_PEAK_GBS
+        line["roofline"]["floor_us"] = fl["us"]
     if "q4_qmm_m512_4096" in extra:
         q = extra["q4_qmm_m512_4096"]
+        roof = {"bound": "mfma", "achieved": q["tflops"], "peak": MFMA_F16_PEAK_TF, "unit": "TFLOP/s", "frac": q["mfma_frac"],
+                "traffic": None, "kernel": "qmm_k2_kernel", "avg_launch_us": q["us"], "flops_per_launch": q["flops"]}
+        annotate(roof, "qmm_q4_m512_4096", q["flops"], MFMA_F16_PEAK_TF * 1e6)
+        ml = extra.get("floors", {}).get("mfma_loop")
+        if ml is not None:  # the matrix instructions alone, no loads and no unpacking
+            roof["floor_frac"] = ml["frac_of_peak"]
         line["secondary"] = {"metric": "Q4 qmm TFLOPS (M=512, K=N=4096)", "value": q["tflops"], "unit": "TFLOP/s",
-                             "roofline": {"bound": "mfma", "achieved": q["tflops"], "peak": MFMA_F16_PEAK_TF,
-                                          "unit": "TFLOP/s", "frac": q["mfma_frac"],
-                                          "traffic": traffic.get("qmm_q4_m512_4096"),
-                                          "kernel": "qmm_k2_kernel", "avg_launch_us": q["us"]},
-                             "launches": q["launches"]}
+                             "roofline": roof, "launches": q["launches"]}
     if not args.no_cpu:
         line["cpu_baseline"] = cpu_baseline(np.random.default_rng(1001), 3.0 if args.quick else 10.0,
                                             all_configs=not args.quick and not args.only)

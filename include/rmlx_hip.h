@@ -32,6 +32,11 @@
 extern "C" {
 #endif
 
+/* The library is built with hidden visibility: the functions declared here are its whole dynamic symbol table. */
+#if defined(__GNUC__) || defined(__clang__)
+#pragma GCC visibility push(default)
+#endif
+
 /* ---- status / dtype ------------------------------------------------------------------ */
 
 enum {
@@ -90,6 +95,20 @@ int32_t rmlx_hip_stream_destroy(rmlx_stream stream);
  * default stream of synchronous calls) and frees its idle blocks, e.g. after one unusually large batch.  The
  * counterpart of the reference's thread-local array pool going out of scope (crates/rmlx-core/src/array.rs:33-47). */
 int32_t rmlx_hip_trim_pool(rmlx_stream stream);
+/* Number of device allocations (hipMalloc) the library's scratch pool has made in this process so far.  It does not
+ * move across a call that took everything from blocks the pool already held, or across rmlx_hip_moe_forward_noalloc;
+ * a caller that is about to capture a graph can check just that.  (No counterpart in the reference.) */
+uint64_t rmlx_hip_scratch_allocations(void);
+/* Recording and replaying a train of calls (the counterpart of encoding several `_into_cb` calls into one command
+ * buffer and committing it, crates/rmlx-core/src/ops/quantized.rs:7797-7802): between graph_begin and graph_end
+ * every call on `stream` is recorded instead of run; graph_launch replays the recording on a stream.  Only calls
+ * that neither allocate nor synchronise may be recorded (the f16 qmv / qmm paths, rmlx_hip_moe_forward_noalloc; a
+ * pooled call whose scratch the stream's pool already holds), and the buffers they name must stay alive. */
+typedef void* rmlx_graph;             /* a hipGraphExec_t */
+int32_t rmlx_hip_graph_begin(rmlx_stream stream);
+int32_t rmlx_hip_graph_end(rmlx_stream stream, rmlx_graph* out);
+int32_t rmlx_hip_graph_launch(rmlx_graph graph, rmlx_stream stream);
+int32_t rmlx_hip_graph_destroy(rmlx_graph graph);
 int32_t rmlx_hip_event_create(rmlx_event* out);
 int32_t rmlx_hip_event_record(rmlx_event ev, rmlx_stream stream);
 int32_t rmlx_hip_event_sync(rmlx_event ev);
@@ -282,11 +301,18 @@ int32_t rmlx_hip_moe_forward_grouped(const rmlx_qweight* gate, const rmlx_qweigh
  * grouped MFMA GEMM -- row tiles of 16, 32 or 64 rows of one expert, weights dequantised in registers; 4- / 8-bit,
  * group sizes 32 / 64 / 128 (one for the three projections), hidden and intermediate dimensions in multiples of
  * 512 -- smaller ones with the streaming GEMV, which reads an expert's weights once per 8 rows (8-bit experts
- * switch at an eighth of `min_rows`, rounded up).  0 = never the GEMM; the default (8) is the measured crossover.
+ * switch at an eighth of `min_rows`, at least 1).  0 = never the GEMM; the default (10) is the measured crossover.
  * The value lives in the handle of the stacked GATE weight and applies to the calls that pass that handle: there
  * is no process-wide state.  Set it before other threads use the handle.  The counterpart of choosing a
  * `MoeStrategy` for a layer in the reference (crates/rmlx-nn/src/moe.rs:515-541).  Returns the previous value. */
 uint32_t rmlx_hip_qweight_set_expert_gemm_min_rows(rmlx_qweight* gate_qw, uint32_t min_rows);
+/* Which streaming kernel runs the expert projections of decode-sized batches (below the grouped GEMM's threshold) of a
+ * block whose gate weight is `qw`: 0 = the library's choice, 1 = K split over the waves of a workgroup, chunks of 8
+ * rows, 2 = a wave per 16-row weight tile, chunks of 8 rows, 3 = a wave per tile, chunks of 16 rows (4-bit weights,
+ * group size 64; other weights keep kernel 1).  Returns the previous value; the tests use it to check that the kernels
+ * agree.  (No counterpart in the reference, which has one kernel for this: gather_qmv_fast_f16_q4,
+ * crates/rmlx-core/src/ops/quantized.rs:9752-9842.) */
+uint32_t rmlx_hip_qweight_set_expert_stream_kernel(rmlx_qweight* qw, uint32_t kind);
 
 /* Routing + the block above in one call: gate_logits [T,E] (the router's output). */
 int32_t rmlx_hip_moe_forward(const rmlx_qweight* gate, const rmlx_qweight* up,
@@ -355,6 +381,10 @@ enum { RMLX_FLOOR_EMPTY = 0, RMLX_FLOOR_READ4 = 1, RMLX_FLOOR_READ8 = 2, RMLX_FL
        RMLX_FLOOR_MFMA_VALU = 5, RMLX_FLOOR_LDS = 6, RMLX_FLOOR_L2_READ = 7 };
 int32_t rmlx_hip_measure_floor(int32_t kind, const void* src_dev, size_t bytes, size_t n_src, uint32_t iters,
                                void* sink_dev, size_t count, rmlx_stream stream);
+
+#if defined(__GNUC__) || defined(__clang__)
+#pragma GCC visibility pop
+#endif
 
 #ifdef __cplusplus
 }

@@ -81,6 +81,7 @@ namespace {
 struct Block { void* ptr; size_t bytes; };
 std::mutex g_pool_mutex;
 std::map<hipStream_t, std::vector<Block>> g_pool;
+uint64_t g_pool_allocations = 0;  // hipMalloc calls made for the pool (guarded by g_pool_mutex)
 }  // namespace
 
 int32_t Scratch::alloc(size_t bytes, hipStream_t s, Arena* arena) {
@@ -114,6 +115,10 @@ int32_t Scratch::alloc(size_t bytes, hipStream_t s, Arena* arena) {
   const size_t rounded = (bytes + 0xFFFFF) & ~(size_t)0xFFFFF;  // 1 MiB granularity
   RMLX_HIP_CHECK(hipMalloc(&ptr, rounded));
   size = rounded;
+  {
+    std::lock_guard<std::mutex> lock(g_pool_mutex);
+    ++g_pool_allocations;
+  }
   return RMLX_OK;
 }
 
@@ -135,7 +140,13 @@ int32_t trim_pool(hipStream_t s, bool forget) {
     blocks.swap(it->second);
     if (forget) g_pool.erase(it);
   }
-  for (const Block& b : blocks) RMLX_HIP_CHECK(hipFree(b.ptr));
+  // every block is handed back; the first failure is what the caller hears about
+  hipError_t first = hipSuccess;
+  for (const Block& b : blocks) {
+    const hipError_t e = hipFree(b.ptr);
+    if (e != hipSuccess && first == hipSuccess) first = e;
+  }
+  if (first != hipSuccess) return fail(RMLX_RUNTIME_ERROR, "hipFree of a pooled scratch block failed: %s", hipGetErrorString(first));
   return RMLX_OK;
 }
 
@@ -194,7 +205,9 @@ int32_t run_matmul_plain(const rmlx_qweight* qw, const void* x, int32_t x_dtype,
   const bool can_qmm_lds = ptr_ok && qmm_supported(N, K, qw->group_size, qw->bits);
   const bool can_qmm_rw = ptr_ok && qmm_rw_supported(N, K, qw->group_size, qw->bits);
   const bool can_qmm = can_qmm_lds || can_qmm_rw;
-  const bool can_qmm_k2 = ptr_ok && qmm_k2_supported(N, K, qw->group_size, qw->bits);
+  // (its stores and the reads of the fused epilogue operand are 8- / 16-byte vectors)
+  const bool can_qmm_k2 = ptr_ok && aligned16(out) && (epi.ptr == nullptr || aligned16(epi.ptr)) &&
+                          qmm_k2_supported(N, K, qw->group_size, qw->bits);
   const bool can_qmm_k2_tall = can_qmm_k2 && qmm_k2_tall_supported(qw->group_size, qw->bits, x_dtype == RMLX_DTYPE_BF16);
 
   if (kernel == KERNEL_AUTO) {
@@ -365,6 +378,9 @@ struct ExpertShapes {
   uint32_t bits;  // of the gate weight
   bool gemm64;    // group size 64 (the 16-row tile is built for it only)
   uint32_t gemm_min_rows;  // of the gate weight's handle (rmlx_hip_qweight_set_expert_gemm_min_rows)
+  uint32_t stream_kernel;  // of the gate weight's handle (rmlx_hip_qweight_set_expert_stream_kernel)
+  bool wave_tiles;         // the wave-per-tile streaming kernel takes the three projections (4-bit, group size 64)
+  bool wave_down;          // ... takes the down projection over chunks of 8 rows
 };
 
 // gather_qmm takes raw buffers, so its GEMV / grouped-GEMM crossover is a constant: every entry has exactly
@@ -409,6 +425,10 @@ int32_t check_expert_weights(const char* who, const rmlx_qweight* gate, const rm
   sh->bits = gate->bits;
   sh->gemm64 = gate->group_size == 64;
   sh->gemm_min_rows = gate->expert_gemm_min_rows;
+  sh->stream_kernel = gate->expert_stream_kernel;
+  const bool q4_gs64 = fast && gate->bits == 4 && gate->group_size == 64 && down->group_size == 64;
+  sh->wave_tiles = q4_gs64 && qmv_wt_supported(sh->I, sh->D, 64, 16) && qmv_wt_supported(sh->D, sh->I, 64, 16);
+  sh->wave_down = q4_gs64 && qmv_wt_supported(sh->D, sh->I, 64, 8);
   sh->portable = !fast;
   // the grouped GEMM also takes group sizes the streaming kernels do not (32; 128 at 8 bits)
   sh->gemm = uniform && qmm_rw_grouped_supported(sh->I, sh->D, gate->group_size, gate->bits) &&
@@ -420,12 +440,29 @@ int32_t check_expert_weights(const char* who, const rmlx_qweight* gate, const rm
 // tiles while an expert has 24 rows or fewer on average: less padding, more workgroups per CU), else 0
 uint32_t expert_gemm_tile_rows(const ExpertShapes& sh, uint64_t rows, uint64_t groups) {
   uint32_t min_rows = sh.gemm_min_rows;
-  // 8-bit experts cross over at an eighth of the threshold (measured: from one row per expert on, against 6 for
-  // 4-bit ones: with 16-row tiles the GEMM streams 8-bit weights faster than the 8-bit GEMV does)
-  if (sh.bits == 8 && min_rows != 0) min_rows = (min_rows + 7) / 8;
+  // 8-bit experts cross over at an eighth of the threshold, rounded down (measured: from one row per expert on, against
+  // 10 for 4-bit ones: with 16-row tiles the GEMM streams 8-bit weights faster than the 8-bit GEMV does)
+  if (sh.bits == 8 && min_rows != 0) min_rows = min_rows >= 16 ? min_rows / 8 : 1;
   if (!sh.gemm || min_rows == 0 || groups == 0 || rows < (uint64_t)min_rows * groups) return 0;
   if (rows <= 7 * groups && sh.gemm64) return 16u;  // (four-wave workgroups, 16 rows: built for group size 64)
   return rows <= 24 * groups ? 32u : kGroupedTileRows;
+}
+
+// Which streaming kernel runs the two projections of a decode-sized batch, and over chunks of how many rows.
+// gate_up / down: 0 = the K-split kernel (qmv.hip), else the wave-per-tile kernel (qmv_wt.hip) with chunks of that many
+// rows (8 or 16).  Selector of the gate handle: 1 = K-split for both, 2 / 3 = wave per tile for both with chunks of 8 / 16
+// rows, 0 (the library's choice) and 4 = K-split for gate / up, wave per tile for a down projection whose rows are
+// shorter than 4096 (measured at D = 4096, I = 1536: the block takes 254 against 269 us at T = 32 and 348 against 368 us at
+// T = 128; a wave-per-tile gate / up projection is 30 % slower than the K-split one, which reads a tile's 32 KB as one
+// contiguous block).
+struct StreamPlan { uint32_t gate_up, down, chunk_rows; };
+StreamPlan expert_stream_plan(const ExpertShapes& sh) {
+  StreamPlan pl{0, 0, 8};
+  if (sh.stream_kernel == 1) return pl;
+  if (sh.stream_kernel == 2 && sh.wave_tiles) pl = StreamPlan{8, 8, 8};
+  else if (sh.stream_kernel == 3 && sh.wave_tiles) pl = StreamPlan{16, 16, 16};
+  else if (sh.wave_down && sh.I < 4096) pl.down = 8;
+  return pl;
 }
 
 // The same block on the portable kernels, for expert weights the streaming GEMV does not take (2-bit,
@@ -460,7 +497,7 @@ int32_t run_expert_ffn_portable(const rmlx_qweight* gate, const rmlx_qweight* up
 int32_t run_expert_ffn(const rmlx_qweight* gate, const rmlx_qweight* up, const rmlx_qweight* down,
                        const ExpertShapes& sh, const __half* x, const uint32_t* row_map,
                        const uint32_t* chunk_tab, const uint32_t* n_chunks, uint32_t max_chunks, __half* h,
-                       void* y, int y_f32, uint32_t gemm_tile_rows, hipStream_t stream) {
+                       void* y, int y_f32, uint32_t gemm_tile_rows, const StreamPlan& plan, hipStream_t stream) {
   const uint32_t per = 32 / gate->bits;  // values per u32 word: 8 (4-bit) or 4 (8-bit)
   if (gemm_tile_rows != 0) {  // the table holds row tiles of that many rows and n_chunks its length
     const uint32_t gs = gate->group_size;  // one group size for the three projections (ExpertShapes::gemm)
@@ -506,7 +543,9 @@ int32_t run_expert_ffn(const rmlx_qweight* gate, const rmlx_qweight* up, const r
   a.x = x; a.row_map = row_map;
   a.out = h; a.ld_out = sh.I; a.out_f32 = 0; a.dual = 1;
   a.chunk_tab = chunk_tab; a.n_chunks_dev = n_chunks; a.max_chunks = max_chunks; a.mr = 8;
-  RMLX_TRY(gate->bits == 8 ? launch_qmv_q8_tab(a, stream) : launch_qmv_q4(a, stream));
+  // (the table holds chunks of at most plan.chunk_rows rows)
+  if (plan.gate_up != 0) RMLX_TRY(launch_qmv_wt(a, plan.gate_up, stream));
+  else RMLX_TRY(gate->bits == 8 ? launch_qmv_q8_tab(a, stream) : launch_qmv_q4(a, stream));
 
   QmvArgs d{};
   d.w0 = down->w; d.s0 = down->s; d.b0 = down->b;
@@ -517,6 +556,7 @@ int32_t run_expert_ffn(const rmlx_qweight* gate, const rmlx_qweight* up, const r
   d.x = h; d.row_map = nullptr;
   d.out = y; d.ld_out = sh.D; d.out_f32 = y_f32; d.dual = 0;
   d.chunk_tab = chunk_tab; d.n_chunks_dev = n_chunks; d.max_chunks = max_chunks; d.mr = 8;
+  if (plan.down != 0) return launch_qmv_wt(d, plan.down, stream);
   return gate->bits == 8 ? launch_qmv_q8_tab(d, stream) : launch_qmv_q4(d, stream);
 }
 
@@ -611,15 +651,51 @@ int32_t rmlx_hip_stream_sync(rmlx_stream stream) {
 int32_t rmlx_hip_stream_destroy(rmlx_stream stream) {
   // The stream's scratch blocks go back to the driver first: a later stream may get the same handle value and
   // must not inherit blocks whose last kernels were ordered on this one.
-  RMLX_HIP_CHECK(hipStreamSynchronize((hipStream_t)stream));
-  RMLX_TRY(trim_pool((hipStream_t)stream, true));
-  RMLX_HIP_CHECK(hipStreamDestroy((hipStream_t)stream));
+  // Every step runs whatever the one before it returned (nothing may leak); the first error is reported.
+  const hipError_t sync_err = hipStreamSynchronize((hipStream_t)stream);
+  const int32_t trim_status = trim_pool((hipStream_t)stream, true);
+  const std::string trim_msg = last_error();
+  const hipError_t destroy_err = hipStreamDestroy((hipStream_t)stream);
+  if (sync_err != hipSuccess) return fail(RMLX_RUNTIME_ERROR, "hipStreamSynchronize failed: %s", hipGetErrorString(sync_err));
+  if (trim_status != RMLX_OK) { last_error() = trim_msg; return trim_status; }
+  if (destroy_err != hipSuccess) return fail(RMLX_RUNTIME_ERROR, "hipStreamDestroy failed: %s", hipGetErrorString(destroy_err));
   return RMLX_OK;
 }
 int32_t rmlx_hip_trim_pool(rmlx_stream stream) {
   RMLX_TRY(require_init());
   RMLX_HIP_CHECK(hipStreamSynchronize((hipStream_t)stream));
   return trim_pool((hipStream_t)stream, false);
+}
+int32_t rmlx_hip_graph_begin(rmlx_stream stream) {
+  RMLX_TRY(require_init());
+  if (stream == nullptr) return fail(RMLX_INVALID_SHAPE, "graph_begin: recording needs a stream (the null stream is synchronous)");
+  RMLX_HIP_CHECK(hipStreamBeginCapture((hipStream_t)stream, hipStreamCaptureModeThreadLocal));
+  return RMLX_OK;
+}
+int32_t rmlx_hip_graph_end(rmlx_stream stream, rmlx_graph* out) {
+  if (out == nullptr) return fail(RMLX_INVALID_SHAPE, "graph_end: out handle pointer is null");
+  *out = nullptr;
+  hipGraph_t g = nullptr;
+  RMLX_HIP_CHECK(hipStreamEndCapture((hipStream_t)stream, &g));
+  hipGraphExec_t exec = nullptr;
+  const hipError_t e = hipGraphInstantiate(&exec, g, nullptr, nullptr, 0);
+  (void)hipGraphDestroy(g);
+  if (e != hipSuccess) return fail(RMLX_RUNTIME_ERROR, "hipGraphInstantiate failed: %s", hipGetErrorString(e));
+  *out = exec;
+  return RMLX_OK;
+}
+int32_t rmlx_hip_graph_launch(rmlx_graph graph, rmlx_stream stream) {
+  if (graph == nullptr) return fail(RMLX_INVALID_SHAPE, "graph_launch: null graph");
+  RMLX_HIP_CHECK(hipGraphLaunch((hipGraphExec_t)graph, (hipStream_t)stream));
+  return RMLX_OK;
+}
+int32_t rmlx_hip_graph_destroy(rmlx_graph graph) {
+  if (graph != nullptr) RMLX_HIP_CHECK(hipGraphExecDestroy((hipGraphExec_t)graph));
+  return RMLX_OK;
+}
+uint64_t rmlx_hip_scratch_allocations(void) {
+  std::lock_guard<std::mutex> lock(g_pool_mutex);
+  return g_pool_allocations;
 }
 int32_t rmlx_hip_event_create(rmlx_event* out) {
   RMLX_TRY(require_init());
@@ -1112,7 +1188,8 @@ int32_t rmlx_hip_expert_group_grouped_forward(const rmlx_qweight* gate, const rm
   for (size_t i = 0; i < n_items; ++i) total += batch_sizes_host[i];
   // row chunks of one expert each: 8 rows for the streaming GEMV, whole row tiles for the grouped GEMM
   const uint32_t gemm = expert_gemm_tile_rows(sh, total, n_items);
-  const uint32_t chunk_rows = gemm ? gemm : 8u;
+  const StreamPlan plan = expert_stream_plan(sh);
+  const uint32_t chunk_rows = gemm ? gemm : plan.chunk_rows;
   std::vector<uint32_t> tab;
   total = 0;
   for (size_t i = 0; i < n_items; ++i) {
@@ -1165,7 +1242,7 @@ int32_t rmlx_hip_expert_group_grouped_forward(const rmlx_qweight* gate, const rm
   RMLX_TRY(h.alloc(total * sh.I * 2, s));
   const uint32_t* dev_tab = static_cast<const uint32_t*>(dtab.ptr);
   RMLX_TRY(run_expert_ffn(gate, up, down, sh, xk, nullptr, dev_tab, dev_tab + 3 * (size_t)n_chunks, n_chunks,
-                          static_cast<__half*>(h.ptr), out_f16_dev, 0, gemm, s));
+                          static_cast<__half*>(h.ptr), out_f16_dev, 0, gemm, plan, s));
   return finish(s);
 }
 
@@ -1197,7 +1274,13 @@ int32_t moe_grouped_impl(const rmlx_qweight* gate, const rmlx_qweight* up, const
   if (T == 0) return RMLX_OK;
   // many rows per expert: the grouped GEMM over row tiles instead of the streaming GEMV over chunks of 8 rows
   const uint32_t gemm = route == nullptr ? expert_gemm_tile_rows(sh, A, sh.E) : 0u;
-  const uint32_t chunk_rows = gemm ? gemm : 8u;
+  StreamPlan plan = expert_stream_plan(sh);
+  if (route != nullptr && plan.chunk_rows != 8) {  // (the fused routing + grouping launch writes chunks of 8 rows)
+    plan.chunk_rows = 8;
+    if (plan.gate_up) plan.gate_up = 8;
+    if (plan.down) plan.down = 8;
+  }
+  const uint32_t chunk_rows = gemm ? gemm : plan.chunk_rows;
   const uint32_t max_chunks = A / chunk_rows + (A < sh.E ? A : sh.E);
   if (max_chunks > 65535) return fail(RMLX_INVALID_SHAPE, "MoeLayer: too many row chunks (%u); split the batch", max_chunks);
 
@@ -1251,7 +1334,7 @@ int32_t moe_grouped_impl(const rmlx_qweight* gate, const rmlx_qweight* up, const
   RMLX_TRY(h.alloc((size_t)A * sh.I * 2, s, arena));
   RMLX_TRY(y.alloc((size_t)A * sh.D * 4, s, arena));
   RMLX_TRY(run_expert_ffn(gate, up, down, sh, xk, sorted_tok, chunk_tab, n_chunks, max_chunks,
-                          static_cast<__half*>(h.ptr), y.ptr, 1, gemm, s));
+                          static_cast<__half*>(h.ptr), y.ptr, 1, gemm, plan, s));
   RMLX_TRY(launch_moe_combine(static_cast<const float*>(y.ptr), inv, expert_weights_dev, T32, (uint32_t)top_k, sh.D,
                               static_cast<__half*>(out_f16_dev), s));
   return finish(s);
@@ -1264,6 +1347,13 @@ uint32_t rmlx_hip_qweight_set_expert_gemm_min_rows(rmlx_qweight* qw, uint32_t mi
   if (qw == nullptr) return 0;
   const uint32_t prev = qw->expert_gemm_min_rows;
   qw->expert_gemm_min_rows = min_rows;
+  return prev;
+}
+
+uint32_t rmlx_hip_qweight_set_expert_stream_kernel(rmlx_qweight* qw, uint32_t kind) {
+  if (qw == nullptr) return 0;
+  const uint32_t prev = qw->expert_stream_kernel;
+  if (kind <= 4) qw->expert_stream_kernel = kind;
   return prev;
 }
 

@@ -90,7 +90,10 @@ struct rmlx_qweight {
   size_t n_experts;     // 1 for a plain linear weight
   // stacked expert weights: average rows per expert from which the expert projections run on the grouped MFMA GEMM
   // instead of the streaming GEMV (read from the gate weight of a block; 0 = never)
-  uint32_t expert_gemm_min_rows = 8;
+  uint32_t expert_gemm_min_rows = 10;
+  // stacked expert weights: which streaming kernel runs decode-sized batches (read from the gate weight of a block):
+  // 0 = the library's choice, 1 = K split over the waves of a workgroup (qmv.hip), 2 = a wave per tile (qmv_wt.hip)
+  uint32_t expert_stream_kernel = 0;
 };
 
 namespace rmlx {
@@ -137,6 +140,10 @@ struct QmvArgs {
 };
 int32_t launch_qmv_q4(const QmvArgs& a, hipStream_t s);
 bool qmv_q4_supported(uint32_t N, uint32_t K, uint32_t group_size);
+// Wave-per-tile streaming GEMV (qmv_wt.hip): the same arguments; chunks of at most chunk_rows (8 or 16) rows, a wave owns
+// a 16-row weight tile over all of K (no cross-wave reduction), group size 64, K <= 4096 (16-row chunks: 8192)
+bool qmv_wt_supported(uint32_t N, uint32_t K, uint32_t group_size, uint32_t chunk_rows);
+int32_t launch_qmv_wt(const QmvArgs& a, uint32_t chunk_rows, hipStream_t s);
 // 8-bit streaming GEMV (qmv_q8.hip): f16 activations [M,K], chunks of 16 rows.
 bool qmv_q8_supported(uint32_t N, uint32_t K, uint32_t group_size);
 int32_t launch_qmv_q8(const uint32_t* w, const __half* s, const __half* b, const __half* x, __half* out, uint32_t M,

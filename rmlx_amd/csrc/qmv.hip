@@ -37,13 +37,12 @@
 //   * Barriers of the tile reduction wait for LDS traffic only, and a workgroup that walks several
 //     tiles requests the next tile's weights as soon as the current accumulators have left for LDS.
 #include "common.hpp"
+#include "q4_stream.hpp"
 
 namespace rmlx {
 namespace {
 
-typedef _Float16 h8 __attribute__((ext_vector_type(8)));
-typedef float f4 __attribute__((ext_vector_type(4)));
-typedef uint32_t u4 __attribute__((ext_vector_type(4)));
+using namespace q4;
 
 constexpr int kThreads = 512;
 constexpr int kWaves = 8;
@@ -71,57 +70,6 @@ struct KParams {
 };
 
 
-// The masks and offsets arrive in registers (Q4Consts): with one of each pair in a scalar and one in a vector
-// register, and + or is a single instruction.
-struct Q4Consts { uint32_t m0, m1, k0, k1; };
-__device__ __forceinline__ h8 unpack_q4_word(uint32_t w, const Q4Consts& q) {
-  uint32_t t = w >> 8;
-  u4 p;
-  p.x = (w & q.m0) | q.k0;  // k+0, k+4   (+1024)
-  p.y = (w & q.m1) | q.k1;  // k+1, k+5   (+64)
-  p.z = (t & q.m0) | q.k0;  // k+2, k+6   (+1024)
-  p.w = (t & q.m1) | q.k1;  // k+3, k+7   (+64)
-  return __builtin_bit_cast(h8, p);
-}
-
-// v + (value of lane ^ 32): v_permlane32_swap exchanges the upper half of its first operand with the lower half
-// of its second, so both registers end up holding one half of v in all lanes.  (Written as assembly: through the
-// builtin this compiler reads the first result twice.  The wait states cover a vector write just before.)
-__device__ __forceinline__ float add_other_half(float v) {
-  uint32_t a = __builtin_bit_cast(uint32_t, v), b = a;
-  asm volatile("s_nop 1\n\tv_permlane32_swap_b32_e32 %0, %1" : "+v"(a), "+v"(b));
-  return __builtin_bit_cast(float, a) + __builtin_bit_cast(float, b);
-}
-
-// x halves (k0..k7) -> slot order (0,4,1,5,2,6,3,7), matching unpack_q4_word.
-__device__ __forceinline__ u4 permute_x8(u4 d) {
-  u4 o;
-  o.x = __builtin_amdgcn_perm(d.z, d.x, 0x05040100u);
-  o.y = __builtin_amdgcn_perm(d.z, d.x, 0x07060302u);
-  o.z = __builtin_amdgcn_perm(d.w, d.y, 0x05040100u);
-  o.w = __builtin_amdgcn_perm(d.w, d.y, 0x07060302u);
-  return o;
-}
-
-__device__ __forceinline__ float silu_f(float v) { return v / (1.0f + __expf(-v)); }
-
-__device__ __forceinline__ uint32_t swap16(uint32_t v) {  // value of lane ^ 16
-  return (uint32_t)__builtin_amdgcn_ds_swizzle((int)v, 0x401F);
-}
-
-__device__ __forceinline__ float swap8(float v) {  // value of lane ^ 8
-  return __builtin_bit_cast(float, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, v), 0x201F));
-}
-
-struct __attribute__((packed, aligned(4))) U4Unaligned { uint32_t v[4]; };
-
-// Workgroup barrier for data exchanged through LDS: waits for this wave's LDS traffic only.  (__syncthreads() also
-// waits for every global load in flight, i.e. for the next tile's weights that were requested on purpose.)
-__device__ __forceinline__ void lds_barrier() {
-  asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-  __builtin_amdgcn_s_barrier();
-  asm volatile("" ::: "memory");
-}
 
 // MR = activation rows staged per pass (1, 2, 4 or 8); TILES = 1, or 2 (fused gate/up, or two
 // 16-row tiles of one matrix sharing the staged activations: PAIR);
@@ -226,9 +174,10 @@ __global__ __launch_bounds__(kThreads, (REUSE != 0 && MR == 8 && TILES == 2) ? 4
           const h8 av = *reinterpret_cast<const h8*>(xs + ((it * 4 + j) * kBlk) * 16 + a_slot_off);
           own = __builtin_amdgcn_mfma_f32_16x16x32_f16(av, bconst, own, 0, 0, 0);
         }
+        // per (slab, group, half of the rows): -sum(off*x) of the four rows, then their sum(x)
         float* sp = sums + ((it * 2 + par) * 8 + (g & 1) * 4) * 2;
-        if (n == 0) { sp[0] = -own.x; sp[2] = -own.y; sp[4] = -own.z; sp[6] = -own.w; }
-        if (n == 8) { sp[1] = own.x; sp[3] = own.y; sp[5] = own.z; sp[7] = own.w; }
+        if (n == 0) *reinterpret_cast<f4*>(sp) = -own;
+        if (n == 8) *reinterpret_cast<f4*>(sp + 4) = own;
       }
     }
   };
@@ -285,50 +234,55 @@ __global__ __launch_bounds__(kThreads, (REUSE != 0 && MR == 8 && TILES == 2) ? 4
       }
     }
   };
+  // The lane's half of every scale / bias word (the group `par` of each slab it multiplies), two slabs per register:
+  // one byte permute per two slabs replaces a shift, a mask and a select per slab, the exchange between the lanes
+  // that loaded scales and those that loaded biases moves two registers instead of four, and the halves are
+  // consumed as f16 operands of mixed-precision fmas.
+  const uint32_t half_sel = par ? 0x07060302u : 0x05040100u;
+  auto pick_halves = [&](const u4& v, uint32_t (&sv)[2], uint32_t (&bv)[2]) {
+    const uint32_t own0 = __builtin_amdgcn_perm(v.y, v.x, half_sel), own1 = __builtin_amdgcn_perm(v.w, v.z, half_sel);
+    const uint32_t oth0 = swap16(own0), oth1 = swap16(own1);
+    sv[0] = (g & 1) ? oth0 : own0; sv[1] = (g & 1) ? oth1 : own1;
+    bv[0] = (g & 1) ? own0 : oth0; bv[1] = (g & 1) ? own1 : oth1;
+  };
+  auto half_at = [](const uint32_t (&o)[2], int it) -> float {
+    const uint32_t wd = o[it >> 1];
+    const unsigned short h = (it & 1) ? (unsigned short)(wd >> 16) : (unsigned short)(wd & 0xFFFFu);
+    return (float)__builtin_bit_cast(_Float16, h);
+  };
   // the tile's slabs against the staged activations: F += scale * (dot - sum(off*x)) + bias * sum(x)
   auto compute_tile = [&](int my, const u4 (&sbv)[TILES], const u4 (&wreg)[TILES][kSpwMax], f4 (&F)[TILES]) {
-    // ---- 2b/3 for 8 rows: slab by slab (few live registers).  The per (row, group) sums of the
-    //          activations come from the matrix unit: columns 0-7 of a constant B operand hold the
-    //          unpack offsets (1024 for even k, 64 for odd k, in slot order), columns 8-15 hold
-    //          ones, so accumulator column n < 8 receives sum(off*x) and column n >= 8 sum(x) of
-    //          its rows; lane n^8 holds the other one.
-    if constexpr (kPreSums) {
-      // ---- 8 rows, several tiles per workgroup: the sums wait in LDS; slab by slab (few live registers) ----
-      u4 sv[TILES], bv[TILES];
+    // Slab by slab (few live registers).  The per (row, group) sums of the activations come from the matrix
+    // unit: columns 0-7 of a constant B operand hold the unpack offsets (1024 for even k, 64 for odd k, in slot
+    // order), columns 8-15 hold ones, so accumulator column n < 8 receives sum(off*x) and column n >= 8 sum(x)
+    // of its rows; lane n^8 holds the other one.
+    uint32_t sv[TILES][2], bv[TILES][2];
 #pragma unroll
-      for (int t = 0; t < TILES; ++t) {
-        const u4 other = (u4){swap16(sbv[t].x), swap16(sbv[t].y), swap16(sbv[t].z), swap16(sbv[t].w)};
-        sv[t] = (g & 1) ? other : sbv[t];
-        bv[t] = (g & 1) ? sbv[t] : other;
-      }
+    for (int t = 0; t < TILES; ++t) pick_halves(sbv[t], sv[t], bv[t]);
+    if constexpr (kPreSums) {
+      // ---- one pass over K: the sums wait in LDS ----
 #pragma unroll
       for (int it = 0; it < kSpwMax; ++it) {
         if (it < my) {
+          // the accumulators start from -sum(off*x) of their rows, so the chain ends in dot - sum(off*x)
+          const float* sp = sums + ((it * 2 + par) * 8 + (g & 1) * 4) * 2;
+          const f4 negoff = *reinterpret_cast<const f4*>(sp);    // accumulator rows 4g .. 4g+3
+          const f4 xsum = *reinterpret_cast<const f4*>(sp + 4);
           f4 c[TILES];
-#pragma unroll
-          for (int t = 0; t < TILES; ++t) c[t] = (f4){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
           for (int j = 0; j < 4; ++j) {
             const h8 av = *reinterpret_cast<const h8*>(xs + ((it * 4 + j) * kBlk) * 16 + a_slot_off);
 #pragma unroll
             for (int t = 0; t < TILES; ++t) {
               const uint32_t wd = j == 0 ? wreg[t][it].x : (j == 1 ? wreg[t][it].y : (j == 2 ? wreg[t][it].z : wreg[t][it].w));
-              c[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(av, unpack_q4_word(wd, qc), c[t], 0, 0, 0);
+              c[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(av, unpack_q4_word(wd, qc), j == 0 ? negoff : c[t], 0, 0, 0);
             }
           }
-          const float* sp = sums + ((it * 2 + par) * 8 + (g & 1) * 4) * 2;
-          const f4 c01 = *reinterpret_cast<const f4*>(sp);      // (-xoff, xsum) of accumulator rows 4g, 4g+1
-          const f4 c23 = *reinterpret_cast<const f4*>(sp + 4);  // rows 4g+2, 4g+3
 #pragma unroll
           for (int t = 0; t < TILES; ++t) {
-            const uint32_t swd = it == 0 ? sv[t].x : (it == 1 ? sv[t].y : (it == 2 ? sv[t].z : sv[t].w));
-            const uint32_t bwd = it == 0 ? bv[t].x : (it == 1 ? bv[t].y : (it == 2 ? bv[t].z : bv[t].w));
-            const float sc = __half2float(__ushort_as_half((unsigned short)(par ? swd >> 16 : swd & 0xFFFFu)));
-            const float bi = __half2float(__ushort_as_half((unsigned short)(par ? bwd >> 16 : bwd & 0xFFFFu)));
-            F[t][0] += sc * (c[t][0] + c01[0]) + bi * c01[1];
-            F[t][1] += sc * (c[t][1] + c01[2]) + bi * c01[3];
-            F[t][2] += sc * (c[t][2] + c23[0]) + bi * c23[1];
-            F[t][3] += sc * (c[t][3] + c23[2]) + bi * c23[3];
+            const float sc = half_at(sv[t], it), bi = half_at(bv[t], it);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) F[t][i] = fmaf(sc, c[t][i], fmaf(bi, xsum[i], F[t][i]));
           }
           // (keeps the operand reads of later slabs from being hoisted above this one: they would cost the registers
           // that let a third workgroup share the CU)
@@ -336,13 +290,7 @@ __global__ __launch_bounds__(kThreads, (REUSE != 0 && MR == 8 && TILES == 2) ? 4
         }
       }
     } else {
-      u4 sv[TILES], bv[TILES];
-#pragma unroll
-      for (int t = 0; t < TILES; ++t) {
-        const u4 other = (u4){swap16(sbv[t].x), swap16(sbv[t].y), swap16(sbv[t].z), swap16(sbv[t].w)};
-        sv[t] = (g & 1) ? other : sbv[t];
-        bv[t] = (g & 1) ? sbv[t] : other;
-      }
+      // ---- several passes over K: every pass computes the sums beside its products ----
 #pragma unroll
       for (int it = 0; it < kSpwMax; ++it) {
         if (it < my) {
@@ -363,15 +311,12 @@ __global__ __launch_bounds__(kThreads, (REUSE != 0 && MR == 8 && TILES == 2) ? 4
           const float o0 = swap8(own.x), o1 = swap8(own.y), o2 = swap8(own.z), o3 = swap8(own.w);
 #pragma unroll
           for (int t = 0; t < TILES; ++t) {
-            const uint32_t swd = it == 0 ? sv[t].x : (it == 1 ? sv[t].y : (it == 2 ? sv[t].z : sv[t].w));
-            const uint32_t bwd = it == 0 ? bv[t].x : (it == 1 ? bv[t].y : (it == 2 ? bv[t].z : bv[t].w));
-            const float sc = __half2float(__ushort_as_half((unsigned short)(par ? swd >> 16 : swd & 0xFFFFu)));
-            const float bi = __half2float(__ushort_as_half((unsigned short)(par ? bwd >> 16 : bwd & 0xFFFFu)));
+            const float sc = half_at(sv[t], it), bi = half_at(bv[t], it);
             const float ce = n < 8 ? -sc : bi, co = n < 8 ? bi : -sc;
-            F[t][0] += sc * c[t][0] + ce * own.x + co * o0;
-            F[t][1] += sc * c[t][1] + ce * own.y + co * o1;
-            F[t][2] += sc * c[t][2] + ce * own.z + co * o2;
-            F[t][3] += sc * c[t][3] + ce * own.w + co * o3;
+            F[t][0] = fmaf(sc, c[t][0], fmaf(ce, own.x, fmaf(co, o0, F[t][0])));
+            F[t][1] = fmaf(sc, c[t][1], fmaf(ce, own.y, fmaf(co, o1, F[t][1])));
+            F[t][2] = fmaf(sc, c[t][2], fmaf(ce, own.z, fmaf(co, o2, F[t][2])));
+            F[t][3] = fmaf(sc, c[t][3], fmaf(ce, own.w, fmaf(co, o3, F[t][3])));
           }
         }
       }

@@ -54,6 +54,11 @@ class QuantizedWeight:
         this handle run on the grouped MFMA GEMM instead of the streaming GEMV (0 = never).  Returns the previous value."""
         return int(rt.lib().rmlx_hip_qweight_set_expert_gemm_min_rows(self.handle, int(min_rows)))
 
+    def set_expert_stream_kernel(self, kind):
+        """(stacked gate weight) streaming kernel of decode-sized batches: 0 the library's choice, 1 K split over the
+        waves of a workgroup, 2 / 3 a wave per weight tile with chunks of 8 / 16 rows.  Returns the previous value."""
+        return int(rt.lib().rmlx_hip_qweight_set_expert_stream_kernel(self.handle, int(kind)))
+
     def groups_per_row(self):
         return self.in_features // self.group_size
 

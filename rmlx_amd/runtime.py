@@ -37,14 +37,15 @@ class RmlxArray(ctypes.Structure):
 EXPORTS = [
     "rmlx_hip_last_error", "rmlx_hip_init", "rmlx_hip_device_info", "rmlx_hip_malloc", "rmlx_hip_free",
     "rmlx_hip_memset", "rmlx_hip_memcpy_h2d", "rmlx_hip_memcpy_d2h", "rmlx_hip_memcpy_d2d",
-    "rmlx_hip_stream_create", "rmlx_hip_stream_sync", "rmlx_hip_stream_destroy", "rmlx_hip_trim_pool", "rmlx_hip_event_create",
+    "rmlx_hip_stream_create", "rmlx_hip_stream_sync", "rmlx_hip_stream_destroy", "rmlx_hip_trim_pool", "rmlx_hip_scratch_allocations", "rmlx_hip_graph_begin",
+    "rmlx_hip_graph_end", "rmlx_hip_graph_launch", "rmlx_hip_graph_destroy", "rmlx_hip_event_create",
     "rmlx_hip_event_record", "rmlx_hip_event_sync", "rmlx_hip_event_elapsed_ms", "rmlx_hip_event_destroy",
     "rmlx_hip_qweight_create", "rmlx_hip_qweight_destroy", "rmlx_hip_affine_quantized_matmul",
     "rmlx_hip_affine_quantized_matmul_batched", "rmlx_hip_qmm_select", "rmlx_hip_qmm_add_residual", "rmlx_hip_qmm_swiglu", "rmlx_hip_qmm_encode_many", "rmlx_hip_quantized_linear_forward",
     "rmlx_hip_gather_qmm", "rmlx_hip_topk_route", "rmlx_hip_moe_sort", "rmlx_hip_index_gather",
     "rmlx_hip_scatter_weighted_add", "rmlx_hip_silu_gate", "rmlx_hip_expert_group_grouped_forward",
     "rmlx_hip_moe_forward_grouped", "rmlx_hip_moe_forward", "rmlx_hip_moe_forward_noalloc", "rmlx_hip_awq_dequant", "rmlx_hip_gptq_dequant",
-    "rmlx_hip_qmm_norm", "rmlx_hip_qweight_set_expert_gemm_min_rows", "rmlx_hip_gather_qmm_select", "rmlx_hip_measure_floor",
+    "rmlx_hip_qmm_norm", "rmlx_hip_qweight_set_expert_gemm_min_rows", "rmlx_hip_qweight_set_expert_stream_kernel", "rmlx_hip_gather_qmm_select", "rmlx_hip_measure_floor",
 ]
 
 _lib = None
@@ -77,6 +78,10 @@ def lib():
         "rmlx_hip_stream_destroy": [vp],
         "rmlx_hip_trim_pool": [vp],
         "rmlx_hip_measure_floor": [i32, vp, sz, sz, u32, vp, sz, vp],
+        "rmlx_hip_graph_begin": [vp],
+        "rmlx_hip_graph_end": [vp, ctypes.POINTER(vp)],
+        "rmlx_hip_graph_launch": [vp, vp],
+        "rmlx_hip_graph_destroy": [vp],
         "rmlx_hip_event_create": [ctypes.POINTER(vp)],
         "rmlx_hip_event_record": [vp, vp],
         "rmlx_hip_event_sync": [vp],
@@ -112,6 +117,10 @@ def lib():
         fn.restype = i32
     L.rmlx_hip_qweight_set_expert_gemm_min_rows.argtypes = [vp, u32]
     L.rmlx_hip_qweight_set_expert_gemm_min_rows.restype = u32
+    L.rmlx_hip_qweight_set_expert_stream_kernel.argtypes = [vp, u32]
+    L.rmlx_hip_qweight_set_expert_stream_kernel.restype = u32
+    L.rmlx_hip_scratch_allocations.argtypes = []
+    L.rmlx_hip_scratch_allocations.restype = ctypes.c_uint64
     _lib = L
     return L
 
@@ -128,6 +137,11 @@ def init(device=0):
     global _initialised
     check(lib().rmlx_hip_init(device))
     _initialised = True
+
+
+def scratch_allocations():
+    """Device allocations the library's scratch pool has made so far in this process."""
+    return int(lib().rmlx_hip_scratch_allocations())
 
 
 def device_info():
@@ -204,6 +218,39 @@ class Stream:
         try:
             if self.handle:
                 lib().rmlx_hip_stream_destroy(self.handle)
+        except Exception:
+            pass
+
+
+class Graph:
+    """A recorded train of calls on a stream: `with Graph.record(stream) as g: ...calls...`, then `g.launch(stream)`."""
+
+    def __init__(self, stream):
+        self.stream, self.handle = stream, None
+
+    @classmethod
+    def record(cls, stream):
+        return cls(stream)
+
+    def __enter__(self):
+        check(lib().rmlx_hip_graph_begin(self.stream.handle))
+        return self
+
+    def __exit__(self, exc_type, exc, tb):
+        p = ctypes.c_void_p()
+        status = lib().rmlx_hip_graph_end(self.stream.handle, ctypes.byref(p))
+        if exc_type is None:
+            check(status)
+            self.handle = p.value
+        return False
+
+    def launch(self, stream=None):
+        check(lib().rmlx_hip_graph_launch(self.handle, (stream or self.stream).handle))
+
+    def __del__(self):
+        try:
+            if self.handle:
+                lib().rmlx_hip_graph_destroy(self.handle)
         except Exception:
             pass
 

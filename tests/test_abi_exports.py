@@ -28,6 +28,17 @@ def test_library_exports_every_declared_symbol():
         assert hasattr(lib, name), name
 
 
+def test_library_exports_nothing_else():
+    """Hidden visibility plus a version script: the dynamic symbol table is exactly the header's functions."""
+    import shutil
+    import subprocess
+    from rmlx_amd import runtime
+    nm = shutil.which("nm") or "/opt/rocm/llvm/bin/llvm-nm"
+    out = subprocess.run([nm, "-D", "--defined-only", runtime.LIB_PATH], capture_output=True, text=True, check=True).stdout
+    exported = sorted(line.split()[-1] for line in out.splitlines() if line.strip())
+    assert exported == _declared()
+
+
 def test_calls_fail_loudly_without_a_gpu_context():
     """No CPU fallback: compute entry points refuse to run before rmlx_hip_init succeeded."""
     from rmlx_amd import runtime as rt
@@ -68,7 +79,7 @@ def test_qweight_validation_needs_no_gpu():
 
 
 def test_expert_gemm_threshold_lives_in_the_handle():
-    """The GEMV / grouped-GEMM threshold of the expert projections: default 6 rows per expert, per weight handle (no
+    """The GEMV / grouped-GEMM threshold of the expert projections: default 10 rows per expert, per weight handle (no
     process-wide state), set returns the old value."""
     from rmlx_amd import runtime as rt
     L = rt.lib()
@@ -77,10 +88,10 @@ def test_expert_gemm_threshold_lives_in_the_handle():
         assert L.rmlx_hip_qweight_create(ctypes.c_void_p(16), 1 << 20, ctypes.c_void_p(16), 1 << 20, ctypes.c_void_p(16), 1 << 20,
                                          64, 4, 64, 64, 2, ctypes.byref(h)) == rt.OK
     try:
-        assert L.rmlx_hip_qweight_set_expert_gemm_min_rows(hs[0], 5) == 8
+        assert L.rmlx_hip_qweight_set_expert_gemm_min_rows(hs[0], 5) == 10
         assert L.rmlx_hip_qweight_set_expert_gemm_min_rows(hs[0], 0) == 5
-        assert L.rmlx_hip_qweight_set_expert_gemm_min_rows(hs[1], 9) == 8  # the other handle kept its default
-        assert L.rmlx_hip_qweight_set_expert_gemm_min_rows(hs[0], 8) == 0
+        assert L.rmlx_hip_qweight_set_expert_gemm_min_rows(hs[1], 9) == 10  # the other handle kept its default
+        assert L.rmlx_hip_qweight_set_expert_gemm_min_rows(hs[0], 10) == 0
     finally:
         for h in hs:
             L.rmlx_hip_qweight_destroy(h)

@@ -612,6 +612,75 @@ def test_config5_moe(hip, config5, T):
     assert_close(out2, ref, f"config5 T={T} (two-step)")
 
 
+@pytest.mark.parametrize("T", [5, 37, 128])
+def test_config5_expert_stream_kernels_agree(hip, config5, T):
+    """The streaming kernels of decode-sized batches on config 5, every token against the oracle: K split over the waves
+    of a workgroup (1), a wave per weight tile over chunks of 8 rows (2) and of 16 rows (3: at T = 128 most experts have
+    9 to 16 rows, a few more than 16), the hybrid the library picks (0 / 4).  The grouped GEMM is switched off."""
+    from rmlx_amd import ops
+    from rmlx_amd.runtime import DeviceBuffer
+    gate, up, down, gh, uh, dh = config5
+    rng = np.random.default_rng(5100 + T)
+    x = make_x(rng, T, 4096)
+    logits = rng.standard_normal((T, 128)).astype(np.float32)
+    idx, w, counts, _ = model.topk_route(logits, 8)
+    ref = model.moe_forward(x, idx, w, gate, up, down, 64, 8)
+    xd, ld = DeviceBuffer.from_numpy(x), DeviceBuffer.from_numpy(logits)
+    idxd, wd = DeviceBuffer.from_numpy(idx), DeviceBuffer.from_numpy(w)
+    prev_rows, prev_kind = gh.set_expert_gemm_min_rows(0), gh.set_expert_stream_kernel(0)
+    try:
+        for kind in (0, 1, 2, 3, 4):
+            gh.set_expert_stream_kernel(kind)
+            print(f"config5 stream kernel {kind} T={T} max rows per expert {int(counts.max())}", flush=True)
+            assert_close(ops.moe_forward(gh, uh, dh, xd, ld, 8).numpy(), ref, f"config5 T={T} stream kernel {kind}")
+            assert_close(ops.moe_forward_grouped(gh, uh, dh, xd, idxd, wd, 8).numpy(), ref, f"config5 T={T} stream kernel {kind} (two-step)")
+    finally:
+        gh.set_expert_gemm_min_rows(prev_rows)
+        gh.set_expert_stream_kernel(prev_kind)
+
+
+@pytest.mark.parametrize("E,T,K,D,I,fused", [(4, 9, 2, 1024, 1536, False), (3, 20, 3, 512, 2560, True), (8, 3, 2, 2048, 512, True)])
+def test_wave_per_tile_kernel_shapes(hip, E, T, K, D, I, fused):
+    """The wave-per-tile kernel on other shapes: separate gate and up weights, tile counts that are no multiple of a
+    workgroup's share (I = 2560: 160 tiles over 8-wave workgroups), one pass per tile (K = 512), experts with more than 8
+    and more than 16 rows, ExpertGroup on the same kernels."""
+    from rmlx_amd import ops
+    from rmlx_amd.runtime import DeviceBuffer
+    rng = np.random.default_rng(E * 100 + T + D)
+
+    def weight(n, k):
+        return make_weight(rng, n, k, 4, 64, lead=(E,))
+
+    if fused:
+        gu = weight(2 * I, D)
+        gate, up = tuple(a[:, :I] for a in gu), tuple(a[:, I:] for a in gu)
+        gh, uh = ops.QuantizedWeight.from_numpy(*gu, 64, 4), None
+    else:
+        gate, up = weight(I, D), weight(I, D)
+        gh, uh = ops.QuantizedWeight.from_numpy(*gate, 64, 4), ops.QuantizedWeight.from_numpy(*up, 64, 4)
+    down = weight(D, I)
+    dh = ops.QuantizedWeight.from_numpy(*down, 64, 4)
+    x = make_x(rng, T, D)
+    logits = rng.standard_normal((T, E)).astype(np.float32)
+    logits[:, 0] += 3.0  # expert 0 takes (nearly) every token
+    idx, w, counts, _ = model.topk_route(logits, K)
+    ref = model.moe_forward(x, idx, w, gate, up, down, 64, K)
+    xd, ld = DeviceBuffer.from_numpy(x), DeviceBuffer.from_numpy(logits)
+    gh.set_expert_gemm_min_rows(0)
+    for kind in (1, 2, 3, 4):
+        gh.set_expert_stream_kernel(kind)
+        print(f"wave-per-tile shapes E={E} T={T} D={D} I={I} fused={fused} kind={kind} counts={counts.tolist()}", flush=True)
+        assert_close(ops.moe_forward(gh, uh, dh, xd, ld, K).numpy(), ref, f"stream kernel {kind}")
+        group = ops.ExpertGroup(gh, uh, dh)
+        sizes = (11, 1, 8, 17)
+        items = [(e % E, make_x(rng, m, D)) for e, m in zip((1, 0, 2, 1), sizes)]
+        outs = group.grouped_forward([(e, DeviceBuffer.from_numpy(v)) for e, v in items])
+        for (e, v), (_, yv) in zip(items, outs):
+            ones = np.ones((len(v), 1))
+            assert_close(yv, model.moe_forward(v, np.full((len(v), 1), e), ones, gate, up, down, 64, 1),
+                         f"ExpertGroup stream kernel {kind} expert {e} rows {len(v)}")
+
+
 @pytest.mark.parametrize("T", [300, 700])
 def test_config5_moe_prefill_sizes(hip, config5, T):
     """Config 5 at prefill-sized batches (19 / 44 rows per expert on average: the grouped GEMM with 32- / 64-row tiles).
@@ -640,8 +709,10 @@ def test_config5_moe_prefill_sizes(hip, config5, T):
 @pytest.mark.parametrize("bits,E,T,D,I,fused", [(4, 4, 13, 512, 512, True), (4, 4, 13, 1024, 1536, False), (8, 8, 12, 512, 512, True),
                                                 (8, 16, 9, 1024, 512, False), (8, 128, 64, 512, 1024, True)])
 def test_moe_few_rows_per_expert_on_16_row_tiles(hip, bits, E, T, D, I, fused):
-    """Between the GEMM threshold (6 rows per expert on average; 8-bit experts: 1) and 7 rows the grouped GEMM runs
-    16-row tiles in four-wave workgroups.  Against the oracle, with the streaming GEMV path beside it."""
+    """With the GEMM threshold lowered to 6 rows per expert on average (the default is 10; 8-bit experts: an eighth of
+    it, at least 1), batches of up to 7 rows per expert run the grouped GEMM on 16-row tiles in four-wave workgroups - for
+    4-bit weights the fused gate / up instantiation that no default setting reaches.  Against the oracle, with the
+    streaming GEMV path beside it."""
     from rmlx_amd import ops
     from rmlx_amd.runtime import DeviceBuffer
     rng = np.random.default_rng(bits * 7 + E + T + D)
@@ -668,10 +739,11 @@ def test_moe_few_rows_per_expert_on_16_row_tiles(hip, bits, E, T, D, I, fused):
     ref = model.moe_forward(x, idx, w, gate, up, down, 64, K, bits=bits)
     xd, idxd, wd = DeviceBuffer.from_numpy(x), DeviceBuffer.from_numpy(idx), DeviceBuffer.from_numpy(w)
     print(f"16-row tiles bits={bits} E={E} T={T} D={D} I={I} fused={fused} counts={counts.tolist()}", flush=True)
-    assert_close(ops.moe_forward_grouped(gh, uh, dh, xd, idxd, wd, K).numpy(), ref, "moe_forward_grouped (16-row tiles)")
-    assert_close(ops.moe_forward(gh, uh, dh, xd, DeviceBuffer.from_numpy(logits), K).numpy(), ref, "moe_forward (16-row tiles)")
-    prev = gh.set_expert_gemm_min_rows(0)
+    prev = gh.set_expert_gemm_min_rows(6)
     try:
+        assert_close(ops.moe_forward_grouped(gh, uh, dh, xd, idxd, wd, K).numpy(), ref, "moe_forward_grouped (16-row tiles)")
+        assert_close(ops.moe_forward(gh, uh, dh, xd, DeviceBuffer.from_numpy(logits), K).numpy(), ref, "moe_forward (16-row tiles)")
+        gh.set_expert_gemm_min_rows(0)
         assert_close(ops.moe_forward_grouped(gh, uh, dh, xd, idxd, wd, K).numpy(), ref, "moe_forward_grouped (streaming)")
     finally:
         gh.set_expert_gemm_min_rows(prev)

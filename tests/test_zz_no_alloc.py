@@ -47,6 +47,30 @@ def test_noalloc_matches_the_pooled_entry_point_on_two_calls_in_a_row(hip):
         assert_close(got, model.moe_forward(x, idx, w, gate, up, down, 64, K), f"oracle T={T}")
 
 
+def test_noalloc_allocates_nothing(hip):
+    """What the entry point is for: with the default stream's pool emptied first, a pooled call has to allocate and
+    the call over the static workspace does not - for every dtype combination that carves casts from the workspace."""
+    from rmlx_amd import ops, runtime as rt
+    from rmlx_amd.runtime import F16, DeviceBuffer
+    rng = np.random.default_rng(80)
+    E, D, I, K = 16, 1024, 512, 4
+    _, _, _, gh, dh = _experts(rng, E, D, I)
+    cases = [(rng.standard_normal((40, D)).astype(np.float16), rng.standard_normal((40, E)).astype(np.float32), None),
+             (rng.standard_normal((5, D)).astype(np.float32), rng.standard_normal((5, E)).astype(np.float16),
+              rng.standard_normal(E).astype(np.float16)),
+             (rng.standard_normal((48, D)).astype(np.float16), rng.standard_normal((48, E)).astype(np.float32), None)]
+    bufs = [(DeviceBuffer.from_numpy(x), DeviceBuffer.from_numpy(l), None if b is None else DeviceBuffer.from_numpy(b),
+             DeviceBuffer((len(x), D), F16)) for x, l, b in cases]
+    rt.check(rt.lib().rmlx_hip_trim_pool(None))
+    before = rt.scratch_allocations()
+    for xd, ld, bd, out in bufs:
+        print(f"noalloc counter T={xd.shape[0]}", flush=True)
+        ops.moe_forward(gh, None, dh, xd, ld, K, expert_bias=bd, out=out, noalloc=True)
+    assert rt.scratch_allocations() == before
+    ops.moe_forward(gh, None, dh, bufs[0][0], bufs[0][1], K)  # the pooled entry point on an empty pool
+    assert rt.scratch_allocations() > before
+
+
 def test_noalloc_casts_and_bias_come_from_the_workspace_too(hip):
     rng = np.random.default_rng(78)
     E, D, I, K = 8, 512, 512, 2
