@@ -213,16 +213,18 @@ int32_t run_matmul_plain(const rmlx_qweight* qw, const void* x, int32_t x_dtype,
   if (kernel == KERNEL_AUTO) {
     // The multi-row GEMV streams the weights once per pass of 8 rows (4-bit; two passes share a workgroup
     // up to 16 rows) or 16 rows (8-bit); the GEMM splits K over several workgroups per tile while its grid
-    // is small, which puts its floor near 9 us at 4096 x 4096.  Measured crossovers, W = weight bytes:
-    //   4-bit: GEMV up to 8 rows (unless K > 8192, where its k loop is the longer one), up to 16 rows while
-    //          W <= 12 MiB (4096 x 4096 is 8 MiB; at 9216 x 4096 the GEMM wins from 9 rows on);
-    //   8-bit: GEMV up to 16 rows while W <= 48 MiB (4096 x 4096 is 16 MiB; at 12288 x 4096 the GEMM wins).
+    // is small, which puts its floor near 9 us at 4096 x 4096.  Measured crossovers (W = weight bytes):
+    //   4-bit: GEMV up to 8 rows at every shape (N x K = 28672 x 4096: 18 against 22 us, 4096 x 14336: 13 against 18,
+    //          2048 x 16384: 10 against 16, 1024 x 28672: 16 against 23); 9 to 16 rows while W <= 12 MiB or N <= 8192
+    //          (4096 x 8192: 9 against 12 us, 4096 x 16384: 17 against 19, 8192 x 8192: 17 against 18; at 9216 x 4096 and
+    //          beyond the GEMM's grid is large enough to win: 28672 x 4096 22 against 29 us);
+    //   8-bit: GEMV up to 16 rows while W < 48 MiB (4096 x 4096 is 16 MiB; at 12288 x 4096 the GEMM wins, 19 against 23 us).
     const uint64_t wbytes = (uint64_t)N * K * qw->bits / 8;
     // Without the register-weights GEMM (K not a multiple of 512) the alternative is the LDS-staged GEMM with
     // a floor of about 15 us: there the 4-bit GEMV keeps up to passes * W <= 48 MiB.
     const bool small_m = !can_qmm_rw ? M <= kQmvMaxM || (qw->bits == 4 && (uint64_t)((M + 7) / 8) * wbytes <= (48ull << 20))
-                         : qw->bits == 4 ? (M <= 8 && K <= 8192) || (M <= kQmvMaxM && wbytes <= (12ull << 20))
-                                         : (M <= kQmvMaxM && wbytes <= (48ull << 20));
+                         : qw->bits == 4 ? M <= 8 || (M <= kQmvMaxM && (wbytes <= (12ull << 20) || N <= 8192))
+                                         : (M <= kQmvMaxM && wbytes < (48ull << 20));
     if ((can_qmv && small_m) || can_m1) kernel = KERNEL_QMV;
     else if (can_qmm) kernel = KERNEL_QMM;
     else if (can_qmv) kernel = KERNEL_QMV;
@@ -265,8 +267,11 @@ int32_t run_matmul_plain(const rmlx_qweight* qw, const void* x, int32_t x_dtype,
   if (kernel == KERNEL_QMM && can_qmm_k2) {
     const uint64_t tiles = (uint64_t)((M + 63) / 64) * (N / 128), tall = (uint64_t)((M + 127) / 128) * (N / 128);
     const uint64_t cus = (uint64_t)ctx().num_cus;
-    if (tiles * 10 >= cus * 7 && tiles <= cus) kernel = KERNEL_QMM_K2;
-    else if (can_qmm_k2_tall && tall * 10 >= cus * 6) { kernel = KERNEL_QMM_K2; k2_tile_rows = 128; }
+    // (a tile height only while at most a quarter of its rows is padding: 16 rows on 128-row tiles over a very wide
+    // matrix measured 150 against 103 us on the register-weights GEMM, N = 151936)
+    const bool fits64 = (uint64_t)((M + 63) / 64) * 64 * 3 <= (uint64_t)M * 4, fits128 = (uint64_t)((M + 127) / 128) * 128 * 3 <= (uint64_t)M * 4;
+    if (fits64 && tiles * 10 >= cus * 7 && tiles <= cus) kernel = KERNEL_QMM_K2;
+    else if (fits128 && can_qmm_k2_tall && tall * 10 >= cus * 6) { kernel = KERNEL_QMM_K2; k2_tile_rows = 128; }
   }
   if (kernel == KERNEL_QMM_K2_TALL) kernel = KERNEL_QMM_K2;
   if (kernel == KERNEL_QMM_RW) kernel = KERNEL_QMM;
