@@ -202,6 +202,8 @@ int32_t run_matmul_plain(const rmlx_qweight* qw, const void* x, int32_t x_dtype,
   // kernel also runs small batches, in passes of four rows
   const bool can_m1 = ptr_ok && qmv_m1_supported(N, K, qw->group_size, qw->bits) &&
                       M <= (can_qmv ? kM1MaxRows : kM1MaxRowsOther);
+  // 2-bit weights: the single-row kernel of their own, up to 16 rows in passes of one (the alternative is the portable kernel)
+  const bool can_q2 = ptr_ok && qw->bits == 2 && M <= kM1MaxRowsOther && qmv_q2_supported(N, K, qw->group_size);
   const bool can_qmm_lds = ptr_ok && qmm_supported(N, K, qw->group_size, qw->bits);
   const bool can_qmm_rw = ptr_ok && qmm_rw_supported(N, K, qw->group_size, qw->bits);
   const bool can_qmm = can_qmm_lds || can_qmm_rw;
@@ -225,11 +227,11 @@ int32_t run_matmul_plain(const rmlx_qweight* qw, const void* x, int32_t x_dtype,
     const bool small_m = !can_qmm_rw ? M <= kQmvMaxM || (qw->bits == 4 && (uint64_t)((M + 7) / 8) * wbytes <= (48ull << 20))
                          : qw->bits == 4 ? M <= 8 || (M <= kQmvMaxM && (wbytes <= (12ull << 20) || N <= 8192))
                                          : (M <= kQmvMaxM && wbytes < (48ull << 20));
-    if ((can_qmv && small_m) || can_m1) kernel = KERNEL_QMV;
+    if ((can_qmv && small_m) || can_m1 || can_q2) kernel = KERNEL_QMV;
     else if (can_qmm) kernel = KERNEL_QMM;
     else if (can_qmv) kernel = KERNEL_QMV;
     else kernel = KERNEL_GENERIC;
-  } else if ((kernel == KERNEL_QMV && !can_qmv && !can_m1) || (kernel == KERNEL_QMV_ROWS && !can_qmv)) {
+  } else if ((kernel == KERNEL_QMV && !can_qmv && !can_m1 && !can_q2) || (kernel == KERNEL_QMV_ROWS && !can_qmv)) {
     return fail(RMLX_INVALID_SHAPE,
                 "qmv kernel requires bits in {4,8}, group_size 64 (4-bit: or 128), N %% 16 == 0, K %% 512 == 0 (4-bit) or "
                 "K %% 256 == 0 (8-bit) and 16-byte aligned buffers (N=%u K=%u bits=%u group_size=%u)",
@@ -343,6 +345,8 @@ int32_t run_matmul_plain(const rmlx_qweight* qw, const void* x, int32_t x_dtype,
     xk = cast.ptr;
   }
 
+  if (kernel == KERNEL_QMV && can_q2)
+    return launch_qmv_q2(qw->w, qw->s, qw->b, static_cast<const __half*>(xk), out, M, N, K, qw->group_size, stream);
   if (kernel == KERNEL_QMV && can_m1) {
     *epi_done = true;
     return launch_qmv_m1(qw->w, qw->s, qw->b, static_cast<const __half*>(xk), out, M, N, K, qw->group_size, qw->bits,
@@ -350,7 +354,7 @@ int32_t run_matmul_plain(const rmlx_qweight* qw, const void* x, int32_t x_dtype,
   }
   if (kernel == KERNEL_QMV_ROWS) kernel = KERNEL_QMV;
   if (kernel == KERNEL_QMV && qw->bits == 8)
-    return launch_qmv_q8(qw->w, qw->s, qw->b, static_cast<const __half*>(xk), out, M, N, K, stream);
+    return launch_qmv_q8(qw->w, qw->s, qw->b, static_cast<const __half*>(xk), out, M, N, K, qw->group_size, stream);
   if (kernel == KERNEL_QMV) {
     QmvArgs a{};
     a.w0 = qw->w; a.s0 = qw->s; a.b0 = qw->b;
@@ -386,6 +390,7 @@ struct ExpertShapes {
   uint32_t stream_kernel;  // of the gate weight's handle (rmlx_hip_qweight_set_expert_stream_kernel)
   bool wave_tiles;         // the wave-per-tile streaming kernel takes the three projections (4-bit, group size 64)
   bool wave_down;          // ... takes the down projection over chunks of 8 rows
+  bool wave_gs32;          // 4-bit weights with group size 32: the wave-per-tile kernel is the only streaming kernel for them
 };
 
 // gather_qmm takes raw buffers, so its GEMV / grouped-GEMM crossover is a constant: every entry has exactly
@@ -410,9 +415,9 @@ int32_t check_expert_weights(const char* who, const rmlx_qweight* gate, const rm
     if (q == nullptr) continue;
     if (q->bits != 2 && q->bits != 4 && q->bits != 8)
       return fail(RMLX_NOT_FOUND, "%s: no kernel for %u-bit expert weights (2, 4 and 8 are implemented; 3- and 6-bit weights run on the matmul entry points)", who, q->bits);
-    // the streaming kernels take 4-bit weights with group size 64 or 128 and 8-bit weights with group size 64,
-    // the same width for all three projections (gate and up share one launch)
-    const bool gs_ok = q->bits == 4 ? (q->group_size == 64 || q->group_size == 128) : (q->bits == 8 && q->group_size == 64);
+    // the K-split streaming kernels take 4- and 8-bit weights with group size 64 or 128, the same width for all three
+    // projections (gate and up share one launch); 4-bit weights with group size 32 run on the wave-per-tile kernel
+    const bool gs_ok = (q->bits == 4 || q->bits == 8) && (q->group_size == 64 || q->group_size == 128);
     if (!gs_ok || q->bits != gate->bits || !aligned16(q->w) || !aligned16(q->s) || !aligned16(q->b)) fast = false;
     if (q->bits != gate->bits || q->group_size != gate->group_size || !aligned16(q->w) || !aligned16(q->s) || !aligned16(q->b))
       uniform = false;
@@ -421,7 +426,7 @@ int32_t check_expert_weights(const char* who, const rmlx_qweight* gate, const rm
   RMLX_TRY(checked_u32(D, "hidden_dim", &sh->D));
   RMLX_TRY(checked_u32(I, "intermediate_dim", &sh->I));
   if (gate->bits == 8) {
-    if (!qmv_q8_supported(sh->I, sh->D, 64) || !qmv_q8_supported(sh->D, sh->I, 64)) fast = false;
+    if (!qmv_q8_supported(sh->I, sh->D, gate->group_size) || !qmv_q8_supported(sh->D, sh->I, down->group_size)) fast = false;
   } else if (!qmv_q4_supported(sh->I, sh->D, 64) || !qmv_q4_supported(sh->D, sh->I, 64)) {
     fast = false;
   }
@@ -434,6 +439,10 @@ int32_t check_expert_weights(const char* who, const rmlx_qweight* gate, const rm
   const bool q4_gs64 = fast && gate->bits == 4 && gate->group_size == 64 && down->group_size == 64;
   sh->wave_tiles = q4_gs64 && qmv_wt_supported(sh->I, sh->D, 64, 16) && qmv_wt_supported(sh->D, sh->I, 64, 16);
   sh->wave_down = q4_gs64 && qmv_wt_supported(sh->D, sh->I, 64, 8);
+  // 4-bit experts with group size 32: both projections on the wave-per-tile kernel, chunks of 8 rows
+  sh->wave_gs32 = uniform && gate->bits == 4 && gate->group_size == 32 && qmv_wt_supported(sh->I, sh->D, 32, 8) &&
+                  qmv_wt_supported(sh->D, sh->I, 32, 8);
+  if (sh->wave_gs32) fast = true;
   sh->portable = !fast;
   // the grouped GEMM also takes group sizes the streaming kernels do not (32; 128 at 8 bits)
   sh->gemm = uniform && qmm_rw_grouped_supported(sh->I, sh->D, gate->group_size, gate->bits) &&
@@ -463,6 +472,7 @@ uint32_t expert_gemm_tile_rows(const ExpertShapes& sh, uint64_t rows, uint64_t g
 struct StreamPlan { uint32_t gate_up, down, chunk_rows; };
 StreamPlan expert_stream_plan(const ExpertShapes& sh) {
   StreamPlan pl{0, 0, 8};
+  if (sh.wave_gs32) return StreamPlan{8, 8, 8};
   if (sh.stream_kernel == 1) return pl;
   if (sh.stream_kernel == 2 && sh.wave_tiles) pl = StreamPlan{8, 8, 8};
   else if (sh.stream_kernel == 3 && sh.wave_tiles) pl = StreamPlan{16, 16, 16};

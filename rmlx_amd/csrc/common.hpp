@@ -144,10 +144,10 @@ bool qmv_q4_supported(uint32_t N, uint32_t K, uint32_t group_size);
 // a 16-row weight tile over all of K (no cross-wave reduction), group size 64, K <= 4096 (16-row chunks: 8192)
 bool qmv_wt_supported(uint32_t N, uint32_t K, uint32_t group_size, uint32_t chunk_rows);
 int32_t launch_qmv_wt(const QmvArgs& a, uint32_t chunk_rows, hipStream_t s);
-// 8-bit streaming GEMV (qmv_q8.hip): f16 activations [M,K], chunks of 16 rows.
+// 8-bit streaming GEMV (qmv_q8.hip): f16 activations [M,K], chunks of 16 rows, group size 64 or 128.
 bool qmv_q8_supported(uint32_t N, uint32_t K, uint32_t group_size);
 int32_t launch_qmv_q8(const uint32_t* w, const __half* s, const __half* b, const __half* x, __half* out, uint32_t M,
-                      uint32_t N, uint32_t K, hipStream_t stream);
+                      uint32_t N, uint32_t K, uint32_t group_size, hipStream_t stream);
 // chunk-table mode for the expert projections (expert strides in u32 words / halves as for the 4-bit kernel)
 int32_t launch_qmv_q8_tab(const QmvArgs& a, hipStream_t stream);
 // Single-row GEMV (qmv_m1.hip): 4- or 8-bit weights, group size 32 / 64 / 128, f16 activations; M rows are
@@ -157,6 +157,11 @@ int32_t launch_qmv_m1(const uint32_t* w, const __half* s, const __half* b, const
                       uint32_t N, uint32_t K, uint32_t group_size, uint32_t bits, int epi_kind, const void* epi,
                       int32_t epi_dtype, const __half* norm_w, const float* inv_rms, hipStream_t stream);
 bool qmv_m1_fuses_norm(uint32_t M, uint32_t K, uint32_t bits);
+// Single-row GEMV for 2-bit weights (qmv_q2.hip): group size 32 / 64 / 128, f16 activations, one activation row per
+// pass over the weights (grid.y = M), f16 out
+bool qmv_q2_supported(uint32_t N, uint32_t K, uint32_t group_size);
+int32_t launch_qmv_q2(const uint32_t* w, const __half* s, const __half* b, const __half* x, __half* out, uint32_t M,
+                      uint32_t N, uint32_t K, uint32_t group_size, hipStream_t stream);
 // dst[m,k] = (half(x[m,k]) * half(inv_rms[m])) * norm_w[k], each product rounded to f16 (the RMSNorm prologue as a separate pass)
 int32_t launch_norm_rows(const void* x, int32_t x_dtype, const __half* norm_w, const float* inv_rms, uint32_t M,
                          uint32_t K, __half* dst, hipStream_t s);

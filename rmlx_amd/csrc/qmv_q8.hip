@@ -7,8 +7,9 @@
 // Same skeleton as the 4-bit kernel (qmv.hip): a workgroup is 8 independent waves that split K,
 // every lane issues all 128-bit weight loads of a pass up front, the waves meet only in the final
 // reduction.  What differs:
-//   * A slab is 16 rows x 64 k = exactly one quantisation group (group size 64), so no row-splitting
-//     trick is needed and all 16 accumulator rows carry activation rows: up to 16 rows per pass.
+//   * A slab is 16 rows x 64 k = exactly one quantisation group (group size 64; at group size 128 two
+//     neighbouring slabs share one), so no row-splitting trick is needed and all 16 accumulator rows
+//     carry activation rows: up to 16 rows per pass.
 //   * Lane (n = lane%16, g = lane/16) holds the 16 bytes k = 16g..16g+15 of weight row n: two MFMA
 //     operands of 8 values in natural order.  Bytes become f16 with one v_perm each pair
 //     (0x6400 | q = 1024 + q); the offset is removed per (row, slab) as -1024 * sum(x).
@@ -34,6 +35,7 @@ struct Q8Params {
   const __half* x;
   void* out;               // f16 (f32 when out_f32)
   uint32_t K, ld_out, M, out_f32;
+  uint32_t gs128;          // quantisation group size 128 instead of 64
   // chunk-table mode (expert projections): (expert, first row position, rows <= 16) per blockIdx.y
   const uint32_t* row_map;    // nullable: source row of position p
   const uint32_t* chunk_tab;
@@ -59,7 +61,7 @@ __global__ __launch_bounds__(kThreads) void qmv_q8_kernel(Q8Params p) {
   __shared__ float red[kWaves * TILES * 256];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int n = lane & 15, g = lane >> 4;  // weight row of the tile / k sub-block; also activation row n
-  const uint32_t K = p.K, slabs_total = K >> 6, groups_per_row = K >> 6;
+  const uint32_t K = p.K, slabs_total = K >> 6, groups_per_row = p.gs128 ? K >> 7 : K >> 6;
   uint32_t expert = 0, row0 = blockIdx.y * 16, rows;
   bool write_zeros = false;
   if (TAB) {
@@ -110,8 +112,14 @@ __global__ __launch_bounds__(kThreads) void qmv_q8_kernel(Q8Params p) {
     uint2 sv[TILES], bv[TILES];
 #pragma unroll
     for (int t = 0; t < TILES; ++t) {
-      sv[t] = *reinterpret_cast<const uint2*>(srow[t] + sl);  // scales of the 4 slabs (8-byte aligned: sl % 4 == 0)
-      bv[t] = *reinterpret_cast<const uint2*>(brow[t] + sl);
+      if (p.gs128) {  // two groups for the four slabs: every value twice
+        const uint32_t s2 = *reinterpret_cast<const uint32_t*>(srow[t] + (sl >> 1)), b2 = *reinterpret_cast<const uint32_t*>(brow[t] + (sl >> 1));
+        sv[t] = make_uint2(__builtin_amdgcn_perm(s2, s2, 0x01000100u), __builtin_amdgcn_perm(s2, s2, 0x03020302u));
+        bv[t] = make_uint2(__builtin_amdgcn_perm(b2, b2, 0x01000100u), __builtin_amdgcn_perm(b2, b2, 0x03020302u));
+      } else {
+        sv[t] = *reinterpret_cast<const uint2*>(srow[t] + sl);  // scales of the 4 slabs (8-byte aligned: sl % 4 == 0)
+        bv[t] = *reinterpret_cast<const uint2*>(brow[t] + sl);
+      }
     }
     u4 wreg[TILES][kSpw];
 #pragma unroll
@@ -180,16 +188,17 @@ __global__ __launch_bounds__(kThreads) void qmv_q8_kernel(Q8Params p) {
 }  // namespace
 
 bool qmv_q8_supported(uint32_t N, uint32_t K, uint32_t group_size) {
-  return group_size == 64 && N > 0 && K > 0 && N % 16 == 0 && K % (64 * kSpw) == 0;
+  return (group_size == 64 || group_size == 128) && N > 0 && K > 0 && N % 16 == 0 && K % (64 * kSpw) == 0;
 }
 
 int32_t launch_qmv_q8(const uint32_t* w, const __half* s, const __half* b, const __half* x, __half* out, uint32_t M,
-                      uint32_t N, uint32_t K, hipStream_t stream) {
-  if (!qmv_q8_supported(N, K, 64))
+                      uint32_t N, uint32_t K, uint32_t group_size, hipStream_t stream) {
+  if (!qmv_q8_supported(N, K, group_size))
     return fail(RMLX_INVALID_SHAPE, "qmv_q8: N %% 16 and K %% 256 required (N=%u K=%u)", N, K);
   if (M == 0) return RMLX_OK;
   Q8Params p{};
   p.w = w; p.s = s; p.b = b; p.x = x; p.out = out; p.K = K; p.ld_out = N; p.M = M;
+  p.gs128 = group_size == 128 ? 1u : 0u;
   hipLaunchKernelGGL((qmv_q8_kernel<false, 1>), dim3(N / 16, (M + 15) / 16), dim3(kThreads), 0, stream, p);
   RMLX_HIP_CHECK(hipGetLastError());
   return RMLX_OK;
@@ -197,8 +206,8 @@ int32_t launch_qmv_q8(const uint32_t* w, const __half* s, const __half* b, const
 
 // Chunk-table launch (expert projections): a.N weight rows per expert, chunks of at most 16 rows.
 int32_t launch_qmv_q8_tab(const QmvArgs& a, hipStream_t stream) {
-  if (!qmv_q8_supported(a.N, a.K, 64))
-    return fail(RMLX_INVALID_SHAPE, "qmv_q8: N %% 16 and K %% 256 required (N=%u K=%u)", a.N, a.K);
+  if (!qmv_q8_supported(a.N, a.K, a.group_size == 0 ? 64 : a.group_size))
+    return fail(RMLX_INVALID_SHAPE, "qmv_q8: N %% 16, K %% 256 and group size 64 or 128 required (N=%u K=%u)", a.N, a.K);
   if (a.chunk_tab == nullptr || a.max_chunks == 0) return a.chunk_tab == nullptr ? fail(RMLX_RUNTIME_ERROR, "qmv_q8: no chunk table") : RMLX_OK;
   if (a.max_chunks > 65535) return fail(RMLX_INVALID_SHAPE, "qmv_q8: too many row chunks (%u)", a.max_chunks);
   Q8Params p{};
@@ -207,6 +216,7 @@ int32_t launch_qmv_q8_tab(const QmvArgs& a, hipStream_t stream) {
   p.x = a.x; p.out = a.out; p.K = a.K; p.ld_out = a.ld_out; p.M = 0; p.out_f32 = a.out_f32;
   p.row_map = a.row_map; p.chunk_tab = a.chunk_tab; p.n_chunks = a.n_chunks_dev;
   p.estride_w = a.expert_stride_w; p.estride_s = a.expert_stride_s;
+  p.gs128 = a.group_size == 128 ? 1u : 0u;
   const dim3 grid(a.N / 16, a.max_chunks);
   if (a.dual) hipLaunchKernelGGL((qmv_q8_kernel<true, 2>), grid, dim3(kThreads), 0, stream, p);
   else hipLaunchKernelGGL((qmv_q8_kernel<true, 1>), grid, dim3(kThreads), 0, stream, p);

@@ -48,14 +48,17 @@ struct WtParams {
 // RH = 8-row halves of a chunk (1: up to 8 rows, 2: up to 16); NW = waves per workgroup; DUAL = gate and up tiles with
 // silu(g) * u written; TAB = rows come from a device chunk table; kPass = slabs per pass (one 16-byte load per lane,
 // tile and slab; two register sets of a pass each are in flight or in use).
-template <int RH, int NW, bool DUAL, bool TAB, int kPass, int NS>
+// GC = MFMA chains per slab: 1 for group size 64 (the 16 accumulator rows carry 8 activation rows x the slab's two
+// groups), 2 for group size 32 (four groups per slab: chain c carries groups 2c and 2c + 1, so the matrix instructions
+// and the operand reads double while the weights are still unpacked once).
+template <int RH, int NW, bool DUAL, bool TAB, int kPass, int NS, int GC>
 __global__ __launch_bounds__(NW * 64, NW == 8 && RH == 1 ? 4 : 1) void qmv_wt_kernel(WtParams p) {
   extern __shared__ __attribute__((aligned(16))) char smem[];
   constexpr int TILES = DUAL ? 2 : 1;
   constexpr int NT = NW * 64;
   const uint32_t K = p.K, S = K >> 7, NP = S / kPass, upr = K >> 3;  // slabs, passes, 16-byte activation units per row
   const uint32_t img_half = S * 4 * kBlk * 16;                        // bytes of one 8-row image
-  float* const sums_all = reinterpret_cast<float*>(smem + RH * img_half);  // [half][slab][group][rows 0-3 / 4-7][-xoff x 4, xsum x 4]
+  float* const sums_all = reinterpret_cast<float*>(smem + RH * img_half);  // [half][slab][chain][group of the chain][rows 0-3 / 4-7][-xoff x 4, xsum x 4]
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -83,7 +86,8 @@ __global__ __launch_bounds__(NW * 64, NW == 8 && RH == 1 ? 4 : 1) void qmv_wt_ke
   const uint32_t n_steps = my_tiles * NP;
 
   // ---- addresses --------------------------------------------------------------------------
-  const uint32_t row_bytes = K >> 1, gpr = K >> 6;  // packed bytes and quantisation groups per weight row
+  const uint32_t row_bytes = K >> 1, gpr = (K >> 6) * GC;  // packed bytes and quantisation groups per weight row
+  constexpr int kSbWords = kPass * GC;  // scale (or bias) words of a pass: two groups per word
   auto make_rsrc = [](const void* base, uint64_t bytes) {
     return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int)(bytes > 0xFFFFFFFFull ? 0xFFFFFFFFull : bytes), 0x00020000);
   };
@@ -99,7 +103,7 @@ __global__ __launch_bounds__(NW * 64, NW == 8 && RH == 1 ? 4 : 1) void qmv_wt_ke
 
   struct Set {  // what one pass of one tile needs: 4 slabs of weights and their scales / biases, per tile slot
     u4 w[TILES][kPass];
-    uint32_t sb[TILES][kPass];  // word `it`: the two groups of slab `it` (scales or biases, by lane)
+    uint32_t sb[TILES][kSbWords];  // word it * GC + c: the two groups of chain c of slab `it` (scales or biases, by lane)
   };
   // the loads of pass `pass` of tile `tile` (wave-uniform): scales / biases first, the memory counter retires in order
   // Waves start at different passes of their tiles (and wrap around): at any moment the waves of the chip then read
@@ -110,13 +114,16 @@ __global__ __launch_bounds__(NW * 64, NW == 8 && RH == 1 ? 4 : 1) void qmv_wt_ke
     const uint32_t tile_row = tile * 16;
 #pragma unroll
     for (int t = 0; t < TILES; ++t) {
-      const uint32_t* sp = reinterpret_cast<const uint32_t*>(sb_base[t] + (uint64_t)tile_row * gpr) + pass * kPass;
-      if constexpr (kPass == 4) {  // (4-byte aligned is enough for the hardware)
-        const U4Unaligned v = *reinterpret_cast<const U4Unaligned*>(sp);
-        st.sb[t][0] = v.v[0]; st.sb[t][1] = v.v[1]; st.sb[t][2] = v.v[2]; st.sb[t][3] = v.v[3];
-      } else {
+      const uint32_t* sp = reinterpret_cast<const uint32_t*>(sb_base[t] + (uint64_t)tile_row * gpr) + pass * kSbWords;
+      if constexpr (kSbWords == 2) {  // (4-byte aligned is enough for the hardware)
         const U2Unaligned v = *reinterpret_cast<const U2Unaligned*>(sp);
         st.sb[t][0] = v.v[0]; st.sb[t][1] = v.v[1];
+      } else {
+#pragma unroll
+        for (int q = 0; q < kSbWords / 4; ++q) {
+          const U4Unaligned v = *reinterpret_cast<const U4Unaligned*>(sp + 4 * q);
+          st.sb[t][4 * q] = v.v[0]; st.sb[t][4 * q + 1] = v.v[1]; st.sb[t][4 * q + 2] = v.v[2]; st.sb[t][4 * q + 3] = v.v[3];
+        }
       }
     }
     const uint32_t soff = tile_row * row_bytes + pass * (kPass * 64);
@@ -159,10 +166,15 @@ __global__ __launch_bounds__(NW * 64, NW == 8 && RH == 1 ? 4 : 1) void qmv_wt_ke
     *reinterpret_cast<u4*>(smem + (z / (S * 4)) * img_half + ((z % (S * 4)) * kBlk + 32) * 16) = (u4){0u, 0u, 0u, 0u};
   lds_barrier();
 
-  // A-operand activity: accumulator rows 0-7 take a slab's first group (g < 2), rows 8-15 its second (g >= 2); the
-  // other lanes read the block's zero slot.
-  const bool a_active = (n < 8) == (g < 2);
-  const uint32_t a_slot_off = (a_active ? (uint32_t)g * 8 + (n & 7) : 32u) * 16;
+  // A-operand activity.  Group size 64: accumulator rows 0-7 take a slab's first group (k sub-blocks g < 2), rows 8-15
+  // its second (g >= 2).  Group size 32: a k sub-block is a group; chain c gives rows 0-7 sub-block 2c and rows 8-15
+  // sub-block 2c + 1.  The other lanes read the block's zero slot.
+  uint32_t a_slot_off[GC];
+#pragma unroll
+  for (int c = 0; c < GC; ++c) {
+    const bool a_active = GC == 1 ? (n < 8) == (g < 2) : g == 2 * c + (n >= 8 ? 1 : 0);
+    a_slot_off[c] = (a_active ? (uint32_t)g * 8 + (n & 7) : 32u) * 16;
+  }
   Q4Consts qc{0x000F000Fu, 0x00F000F0u, 0x64006400u, 0x54005400u};
   asm volatile("" : "+s"(qc.m0), "+s"(qc.m1), "+v"(qc.k0), "+v"(qc.k1));
 
@@ -175,15 +187,18 @@ __global__ __launch_bounds__(NW * 64, NW == 8 && RH == 1 ? 4 : 1) void qmv_wt_ke
     const h8 bconst = __builtin_bit_cast(h8, bconst_bits);
     for (uint32_t q = wave; q < RH * S; q += NW) {
       const uint32_t h = q / S, slab = q % S;
-      f4 own = (f4){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const h8 av = *reinterpret_cast<const h8*>(smem + h * img_half + ((slab * 4 + j) * kBlk) * 16 + a_slot_off);
-        own = __builtin_amdgcn_mfma_f32_16x16x32_f16(av, bconst, own, 0, 0, 0);
+      for (int c = 0; c < GC; ++c) {
+        f4 own = (f4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const h8 av = *reinterpret_cast<const h8*>(smem + h * img_half + ((slab * 4 + j) * kBlk) * 16 + a_slot_off[c]);
+          own = __builtin_amdgcn_mfma_f32_16x16x32_f16(av, bconst, own, 0, 0, 0);
+        }
+        float* sp = sums_all + (((q * GC + c) * 2 + par) * 2 + (g & 1)) * 8;
+        if (n == 0) *reinterpret_cast<f4*>(sp) = -own;
+        if (n == 8) *reinterpret_cast<f4*>(sp + 4) = own;
       }
-      float* sp = sums_all + ((q * 2 + par) * 2 + (g & 1)) * 8;
-      if (n == 0) *reinterpret_cast<f4*>(sp) = -own;
-      if (n == 8) *reinterpret_cast<f4*>(sp + 4) = own;
     }
   }
   lds_barrier();
@@ -191,9 +206,9 @@ __global__ __launch_bounds__(NW * 64, NW == 8 && RH == 1 ? 4 : 1) void qmv_wt_ke
 
   // ---- 3. the wave's tiles, pass by pass -------------------------------------------------------------------------
   const uint32_t half_sel = par ? 0x07060302u : 0x05040100u;  // the lane's group of every (scale, scale) word
-  auto half_at = [](const uint32_t (&o)[kPass / 2], int it) -> float {
-    const uint32_t wd = o[it >> 1];
-    const unsigned short hb = (it & 1) ? (unsigned short)(wd >> 16) : (unsigned short)(wd & 0xFFFFu);
+  auto half_at = [](const uint32_t (&o)[kSbWords / 2], int widx) -> float {
+    const uint32_t wd = o[widx >> 1];
+    const unsigned short hb = (widx & 1) ? (unsigned short)(wd >> 16) : (unsigned short)(wd & 0xFFFFu);
     return (float)__builtin_bit_cast(_Float16, hb);
   };
   f4 F[RH][TILES];
@@ -205,11 +220,11 @@ __global__ __launch_bounds__(NW * 64, NW == 8 && RH == 1 ? 4 : 1) void qmv_wt_ke
 #pragma unroll
         for (int t = 0; t < TILES; ++t) F[h][t] = (f4){0.f, 0.f, 0.f, 0.f};
     }
-    uint32_t sv[TILES][kPass / 2], bv[TILES][kPass / 2];  // the lane's group of every slab, two slabs per register
+    uint32_t sv[TILES][kSbWords / 2], bv[TILES][kSbWords / 2];  // the lane's group of every word, two words per register
 #pragma unroll
     for (int t = 0; t < TILES; ++t)
 #pragma unroll
-      for (int q = 0; q < kPass / 2; ++q) {
+      for (int q = 0; q < kSbWords / 2; ++q) {
         const uint32_t own = __builtin_amdgcn_perm(st.sb[t][2 * q + 1], st.sb[t][2 * q], half_sel), oth = swap16(own);
         sv[t][q] = (g & 1) ? oth : own;
         bv[t][q] = (g & 1) ? own : oth;
@@ -218,16 +233,18 @@ __global__ __launch_bounds__(NW * 64, NW == 8 && RH == 1 ? 4 : 1) void qmv_wt_ke
 #pragma unroll
     for (int it = 0; it < kPass; ++it) {
       const uint32_t slab = slab0 + it;
-      f4 c[RH][TILES];
-      f4 xsum[RH];
+      f4 c[RH][GC][TILES];
+      f4 xsum[RH][GC];
 #pragma unroll
-      for (int h = 0; h < RH; ++h) {
-        const float* sp = sums_all + (((h * S + slab) * 2 + par) * 2 + (g & 1)) * 8;
-        const f4 negoff = *reinterpret_cast<const f4*>(sp);
-        xsum[h] = *reinterpret_cast<const f4*>(sp + 4);
+      for (int h = 0; h < RH; ++h)
 #pragma unroll
-        for (int t = 0; t < TILES; ++t) c[h][t] = negoff;  // the chain ends in dot - sum(off*x)
-      }
+        for (int ch = 0; ch < GC; ++ch) {
+          const float* sp = sums_all + ((((h * S + slab) * GC + ch) * 2 + par) * 2 + (g & 1)) * 8;
+          const f4 negoff = *reinterpret_cast<const f4*>(sp);
+          xsum[h][ch] = *reinterpret_cast<const f4*>(sp + 4);
+#pragma unroll
+          for (int t = 0; t < TILES; ++t) c[h][ch][t] = negoff;  // the chain ends in dot - sum(off*x)
+        }
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         h8 bw[TILES];
@@ -237,20 +254,24 @@ __global__ __launch_bounds__(NW * 64, NW == 8 && RH == 1 ? 4 : 1) void qmv_wt_ke
           bw[t] = unpack_q4_word(wd, qc);
         }
 #pragma unroll
-        for (int h = 0; h < RH; ++h) {
-          const h8 av = *reinterpret_cast<const h8*>(smem + h * img_half + ((slab * 4 + j) * kBlk) * 16 + a_slot_off);
-#pragma unroll
-          for (int t = 0; t < TILES; ++t) c[h][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(av, bw[t], c[h][t], 0, 0, 0);
-        }
-      }
-#pragma unroll
-      for (int t = 0; t < TILES; ++t) {
-        const float sc = half_at(sv[t], it), bi = half_at(bv[t], it);
-#pragma unroll
         for (int h = 0; h < RH; ++h)
 #pragma unroll
-          for (int i = 0; i < 4; ++i) F[h][t][i] = fmaf(sc, c[h][t][i], fmaf(bi, xsum[h][i], F[h][t][i]));
+          for (int ch = 0; ch < GC; ++ch) {
+            const h8 av = *reinterpret_cast<const h8*>(smem + h * img_half + ((slab * 4 + j) * kBlk) * 16 + a_slot_off[ch]);
+#pragma unroll
+            for (int t = 0; t < TILES; ++t) c[h][ch][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(av, bw[t], c[h][ch][t], 0, 0, 0);
+          }
       }
+#pragma unroll
+      for (int t = 0; t < TILES; ++t)
+#pragma unroll
+        for (int ch = 0; ch < GC; ++ch) {
+          const float sc = half_at(sv[t], it * GC + ch), bi = half_at(bv[t], it * GC + ch);
+#pragma unroll
+          for (int h = 0; h < RH; ++h)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) F[h][t][i] = fmaf(sc, c[h][ch][t][i], fmaf(bi, xsum[h][ch][i], F[h][t][i]));
+        }
     }
     if (c_pass == NP - 1) {
       // the tile is complete: add the two group halves (lane ^ 32), lanes with g < 2 write rows 4g .. 4g+3, column n
@@ -289,7 +310,7 @@ __global__ __launch_bounds__(NW * 64, NW == 8 && RH == 1 ? 4 : 1) void qmv_wt_ke
   }
 }
 
-template <int RH, int NW, bool DUAL, int kPass, int NS>
+template <int RH, int NW, bool DUAL, int kPass, int NS, int GC = 1>
 int32_t launch_one(const WtParams& p, bool tab, dim3 grid, size_t lds_bytes, hipStream_t s) {
   auto go = [&](auto kernel) -> int32_t {
     static bool configured = false;  // (per instantiation; the attribute is idempotent, so a race only repeats the call)
@@ -300,23 +321,32 @@ int32_t launch_one(const WtParams& p, bool tab, dim3 grid, size_t lds_bytes, hip
     hipLaunchKernelGGL(kernel, grid, dim3(NW * 64), lds_bytes, s, p);
     return RMLX_OK;
   };
-  if (tab) return go(qmv_wt_kernel<RH, NW, DUAL, true, kPass, NS>);
-  return go(qmv_wt_kernel<RH, NW, DUAL, false, kPass, NS>);
+  if (tab) return go(qmv_wt_kernel<RH, NW, DUAL, true, kPass, NS, GC>);
+  return go(qmv_wt_kernel<RH, NW, DUAL, false, kPass, NS, GC>);
 }
 
 }  // namespace
 
+// bytes of LDS a workgroup needs: per 8-row half the image (33 slots of 16 bytes per (slab, product)) and the sums
+static size_t wt_lds_bytes(uint32_t K, uint32_t group_size, uint32_t chunk_rows) {
+  const size_t slabs = K >> 7, chains = group_size == 32 ? 2 : 1;
+  return (size_t)(chunk_rows > 8 ? 2 : 1) * (slabs * 4 * kBlk * 16 + slabs * chains * 128);
+}
+
 bool qmv_wt_supported(uint32_t N, uint32_t K, uint32_t group_size, uint32_t chunk_rows) {
-  // one activation unit per thread while staging: K / 8 <= threads (8 waves: K <= 4096, 16 waves: K <= 8192)
+  // one activation unit per thread while staging: K / 8 <= threads (8 waves: K <= 4096, 16 waves: K <= 8192);
+  // group size 32 runs chunks of 8 rows only
+  if (!(chunk_rows == 8 || (chunk_rows == 16 && group_size == 64))) return false;
   const uint32_t max_k = chunk_rows > 8 ? 8192u : 4096u;
-  const size_t lds = (size_t)(chunk_rows > 8 ? 2 : 1) * ((K >> 7) * 4 * kBlk * 16 + (K >> 7) * 128);
-  return group_size == 64 && N % 16 == 0 && K % 512 == 0 && N > 0 && K > 0 && K <= max_k && lds <= 160 * 1024 &&
-         (chunk_rows == 8 || chunk_rows == 16);
+  return (group_size == 64 || group_size == 32) && N % 16 == 0 && K % 512 == 0 && N > 0 && K > 0 && K <= max_k &&
+         wt_lds_bytes(K, group_size, chunk_rows) <= 160 * 1024;
 }
 
 int32_t launch_qmv_wt(const QmvArgs& a, uint32_t chunk_rows, hipStream_t s) {
-  if (!qmv_wt_supported(a.N, a.K, a.group_size == 0 ? 64 : a.group_size, chunk_rows))
-    return fail(RMLX_INVALID_SHAPE, "qmv_wt: N %% 16, K %% 512, K <= %u and group size 64 required (N=%u K=%u)", chunk_rows > 8 ? 8192u : 4096u, a.N, a.K);
+  const uint32_t gs = a.group_size == 0 ? 64 : a.group_size;
+  if (!qmv_wt_supported(a.N, a.K, gs, chunk_rows))
+    return fail(RMLX_INVALID_SHAPE, "qmv_wt: N %% 16, K %% 512, K <= %u and group size 64 (8-row chunks: or 32) required (N=%u K=%u group_size=%u)",
+                chunk_rows > 8 ? 8192u : 4096u, a.N, a.K, gs);
   WtParams p{};
   p.w0 = a.w0; p.s0 = a.s0; p.b0 = a.b0;
   p.w1 = a.dual ? a.w1 : a.w0; p.s1 = a.dual ? a.s1 : a.s0; p.b1 = a.dual ? a.b1 : a.b0;
@@ -331,7 +361,7 @@ int32_t launch_qmv_wt(const QmvArgs& a, uint32_t chunk_rows, hipStream_t s) {
   // 16-row chunks: the fused gate / up kernel needs more than the 128 registers of a 16-wave workgroup, so it runs 8
   // waves (its LDS images leave room for one workgroup per CU either way)
   const uint32_t rh = chunk_rows > 8 ? 2 : 1, nw = rh == 2 && !a.dual ? 16 : 8;
-  const size_t lds = (size_t)rh * ((a.K >> 7) * 4 * kBlk * 16 + (a.K >> 7) * 128);
+  const size_t lds = wt_lds_bytes(a.K, gs, chunk_rows);
   // tiles per wave: as many as leave about four workgroups per slot of the chip (a workgroup stages the chunk's
   // activations once for all of them)
   const uint64_t slots = (uint64_t)ctx().num_cus * (rh == 2 ? 1 : 2);  // resident workgroups
@@ -344,7 +374,8 @@ int32_t launch_qmv_wt(const QmvArgs& a, uint32_t chunk_rows, hipStream_t s) {
   // (ring depths measured on the routed block at T = 32 / 128: a third set for the fused kernel 317 / 438 us against
   // 306 / 424 us with two; passes of two slabs in a ring of four or three for the plain kernel 263 / 261 us against 255 us
   // with passes of four in a ring of two - more requests in flight per wave make this access pattern slower, not faster)
-  if (rh == 2) st = a.dual ? launch_one<2, 8, true, 2, 2>(p, tab, grid, lds, s) : launch_one<2, 16, false, 4, 2>(p, tab, grid, lds, s);
+  if (gs == 32) st = a.dual ? launch_one<1, 8, true, 2, 2, 2>(p, tab, grid, lds, s) : launch_one<1, 8, false, 2, 2, 2>(p, tab, grid, lds, s);
+  else if (rh == 2) st = a.dual ? launch_one<2, 8, true, 2, 2>(p, tab, grid, lds, s) : launch_one<2, 16, false, 4, 2>(p, tab, grid, lds, s);
   else st = a.dual ? launch_one<1, 8, true, 2, 2>(p, tab, grid, lds, s) : launch_one<1, 8, false, 4, 2>(p, tab, grid, lds, s);
   RMLX_TRY(st);
   RMLX_HIP_CHECK(hipGetLastError());

@@ -892,3 +892,17 @@ def test_ladder_picks_within_15_percent_of_the_fastest_family(hip, n, k, bits, m
         best = min(v for f, v in times.items() if f != "auto")
         print("  " + " ".join(f"{f}={v:.1f}us" for f, v in times.items()), flush=True)
         assert times["auto"] <= 1.15 * best, (m, times)
+
+
+@pytest.mark.parametrize("m", [3, 8, 16])
+@pytest.mark.parametrize("n,k", [(512, 1024), (1024, 4096)])
+def test_q8_group_128_on_the_streaming_gemv(hip, n, k, m):
+    """8-bit weights at group size 128 on the multi-row streaming GEMV (two neighbouring 64-wide slabs share a scale),
+    forced and through the ladder, against the oracle."""
+    from rmlx_amd import runtime as rt
+    rng = np.random.default_rng(n + k + m)
+    words, s, b = make_weight(rng, n, k, 8, 128)
+    x = make_x(rng, m, k)
+    ref = model.qmm(x.astype(np.float64), words, s, b, 128, 8)
+    assert_close(_run(hip, words, s, b, x, 8, gs=128, kernel=rt.KERNEL_QMV_ROWS), ref, f"Q8 gs128 M={m} N={n} K={k} (streaming GEMV)")
+    assert_close(_run(hip, words, s, b, x, 8, gs=128), ref, f"Q8 gs128 M={m} N={n} K={k} (auto)")

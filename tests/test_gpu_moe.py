@@ -436,11 +436,13 @@ def test_random_moe_shapes(hip):
 @pytest.mark.parametrize("bits,gs,D,I,fused", [(8, 64, 512, 512, False), (4, 32, 512, 1024, True), (4, 128, 384, 640, False),
                                                (8, 32, 96, 160, True), (2, 64, 256, 128, False),
                                                (4, 128, 512, 1024, True), (4, 128, 1024, 1536, False),   # streaming kernels, group 128
-                                               (8, 64, 1024, 1536, True), (8, 64, 4096, 768, False)])   # streaming 8-bit kernel
+                                               (8, 64, 1024, 1536, True), (8, 64, 4096, 768, False),    # streaming 8-bit kernel
+                                               (8, 128, 512, 1024, True), (8, 128, 1024, 768, False),   # ... at group size 128
+                                               (4, 32, 1024, 1536, False), (4, 32, 2048, 512, True)])   # wave-per-tile kernel, group 32
 def test_moe_other_bit_widths_and_group_sizes(hip, bits, gs, D, I, fused):
-    """Expert weights beyond 4 bits / group 64: 8-bit (group 64) and 4-bit group 128 weights stream through the
-    fast kernels when the dimensions allow; 2-bit weights, group size 32 and other dimensions run the same
-    block on the portable kernels.  Routed block (one call and grouped) and `ExpertGroup::grouped_forward`,
+    """Expert weights beyond 4 bits / group 64: 8-bit (group 64 / 128) and 4-bit group 128 weights stream through the
+    K-split kernels and 4-bit group 32 weights through the wave-per-tile kernel when the dimensions allow; 2-bit
+    weights, 8-bit weights at group size 32 and other dimensions run the same block on the portable kernels.  Routed block (one call and grouped) and `ExpertGroup::grouped_forward`,
     against the oracle."""
     from rmlx_amd import ops
     from rmlx_amd.runtime import DeviceBuffer
