@@ -396,6 +396,9 @@ struct ExpertShapes {
 // gather_qmm takes raw buffers, so its GEMV / grouped-GEMM crossover is a constant: every entry has exactly
 // m_per_batch rows, the streaming GEMV wastes nothing up to a full chunk of 8 rows, and the GEMM wins from 9 rows on.
 constexpr uint32_t kGatherGemmMinRows = 9;
+// routed block: up to this many assignments run without grouping (every assignment its own chunk, combine fused into
+// the down projection)
+constexpr uint32_t kDirectMaxAssignments = 32;
 enum { GATHER_AUTO = 0, GATHER_STREAM = 1, GATHER_GEMM = 2, GATHER_PORTABLE = 3 };
 
 int32_t check_expert_weights(const char* who, const rmlx_qweight* gate, const rmlx_qweight* up,
@@ -562,6 +565,7 @@ int32_t run_expert_ffn(const rmlx_qweight* gate, const rmlx_qweight* up, const r
   if (plan.gate_up != 0) RMLX_TRY(launch_qmv_wt(a, plan.gate_up, stream));
   else RMLX_TRY(gate->bits == 8 ? launch_qmv_q8_tab(a, stream) : launch_qmv_q4(a, stream));
 
+  if (y == nullptr) return RMLX_OK;  // (the caller runs the down projection itself)
   QmvArgs d{};
   d.w0 = down->w; d.s0 = down->s; d.b0 = down->b;
   d.N = sh.D; d.K = sh.I;
@@ -1333,6 +1337,26 @@ int32_t moe_grouped_impl(const rmlx_qweight* gate, const rmlx_qweight* up, const
     return finish(s);
   }
   if (!aligned16(xk)) return fail(RMLX_INVALID_SHAPE, "MoeLayer: input must be 16-byte aligned");
+  // A few tokens (at most 32 assignments), routed here: no grouping at all.  Every assignment is a chunk of one row in
+  // assignment order, and the down projection adds the token's weighted expert outputs itself - three launches (routing,
+  // gate / up, down + combine) instead of four, no [assignments, D] intermediate.  An expert picked by two tokens is
+  // streamed once per token (at 4 tokens of 8 picks over 128 experts: 32 chunks for 31 experts).
+  if (route != nullptr && A <= kDirectMaxAssignments && sh.stream_kernel != 1 && sh.wave_down &&
+      qmv_wt_combine_supported(sh.D, sh.I, down->group_size, (uint32_t)top_k)) {
+    RMLX_TRY(meta.alloc(((size_t)4 * A + 4) * 4, s, arena));  // tok[A] | chunk_tab[3 A] | n_chunks[1]
+    uint32_t* tok = static_cast<uint32_t*>(meta.ptr);
+    uint32_t* chunk_tab = tok + A;
+    uint32_t* n_chunks = chunk_tab + 3 * (size_t)A;
+    RMLX_TRY(launch_route_direct_small(route->logits, route->bias, T32, sh.E, (uint32_t)top_k, 1, route->idx_out, route->w_out,
+                                       tok, chunk_tab, n_chunks, s));
+    RMLX_TRY(h.alloc((size_t)A * sh.I * 2, s, arena));
+    RMLX_TRY(run_expert_ffn(gate, up, down, sh, xk, tok, chunk_tab, n_chunks, A, static_cast<__half*>(h.ptr), nullptr, 0, 0,
+                            StreamPlan{0, 0, 8}, s));
+    RMLX_TRY(launch_qmv_wt_combine(down->w, down->s, down->b, (uint64_t)sh.D * (sh.I / 8), (uint64_t)sh.D * (sh.I / down->group_size),
+                                   sh.E, static_cast<const __half*>(h.ptr), route->idx_out, route->w_out, T32, (uint32_t)top_k,
+                                   sh.D, sh.I, static_cast<__half*>(out_f16_dev), s));
+    return finish(s);
+  }
   // meta: sorted[A] | sorted_tok[A] | inv[A] | chunk_tab[3*max_chunks] | n_chunks[1]
   RMLX_TRY(meta.alloc(((size_t)3 * A + 3 * (size_t)max_chunks + 4) * 4, s, arena));
   uint32_t* sorted = static_cast<uint32_t*>(meta.ptr);

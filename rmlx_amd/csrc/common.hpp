@@ -144,6 +144,14 @@ bool qmv_q4_supported(uint32_t N, uint32_t K, uint32_t group_size);
 // a 16-row weight tile over all of K (no cross-wave reduction), group size 64, K <= 4096 (16-row chunks: 8192)
 bool qmv_wt_supported(uint32_t N, uint32_t K, uint32_t group_size, uint32_t chunk_rows);
 int32_t launch_qmv_wt(const QmvArgs& a, uint32_t chunk_rows, hipStream_t s);
+// Down projection of a few tokens with the weighted combine fused behind it (qmv_wt.hip): h [T * top_k, K] f16 in
+// assignment order, out[t] = sum_k wts[t, k] * (h[t * top_k + k] . W[idx[t * top_k + k]]^T) in ascending k, f16 [T, N];
+// 4-bit weights, group size 64, K <= 4096
+bool qmv_wt_combine_supported(uint32_t N, uint32_t K, uint32_t group_size, uint32_t top_k);
+int32_t launch_qmv_wt_combine(const uint32_t* w, const __half* s, const __half* b, uint64_t expert_stride_w,
+                              uint64_t expert_stride_s, uint32_t n_experts, const __half* h, const uint32_t* idx,
+                              const float* wts, uint32_t T, uint32_t top_k, uint32_t N, uint32_t K, __half* out,
+                              hipStream_t stream);
 // 8-bit streaming GEMV (qmv_q8.hip): f16 activations [M,K], chunks of 16 rows, group size 64 or 128.
 bool qmv_q8_supported(uint32_t N, uint32_t K, uint32_t group_size);
 int32_t launch_qmv_q8(const uint32_t* w, const __half* s, const __half* b, const __half* x, __half* out, uint32_t M,
@@ -240,6 +248,10 @@ bool route_sort_fusable(uint32_t T, uint32_t E, uint32_t K);
 int32_t launch_route_sort_small(const float* logits, const float* bias, uint32_t T, uint32_t E, uint32_t K,
                                 int renorm, uint32_t* idx, float* w, uint32_t* sorted, uint32_t* sorted_tok,
                                 uint32_t* inv, uint32_t* chunk_tab, uint32_t* n_chunks, hipStream_t s);
+// Decode-sized batches without grouping: routing only, every assignment a chunk of one row (tok[a] = its token)
+int32_t launch_route_direct_small(const float* logits, const float* bias, uint32_t T, uint32_t E, uint32_t K,
+                                  int renorm, uint32_t* idx, float* w, uint32_t* tok, uint32_t* chunk_tab,
+                                  uint32_t* n_chunks, hipStream_t s);
 int32_t launch_index_gather(const __half* src, uint32_t d, const uint32_t* idx, uint32_t n, uint32_t src_rows,
                             __half* dst, hipStream_t s);
 int32_t launch_scatter_weighted_add(const __half* src, uint32_t n, uint32_t d, const uint32_t* tok,

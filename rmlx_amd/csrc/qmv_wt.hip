@@ -310,6 +310,152 @@ __global__ __launch_bounds__(NW * 64, NW == 8 && RH == 1 ? 4 : 1) void qmv_wt_ke
   }
 }
 
+// ---- down projection with the weighted combine fused behind it, for decode-sized batches ----------------------------
+// One workgroup per (token, 16-column tile): wave k multiplies the hidden row of the token's k-th assignment with that
+// assignment's expert (a wave per (expert, tile), all of K, two register sets as above) and the eight results meet in
+// LDS, where they are added as out[t] = sum_k w[t,k] * y_k in ascending k - the order and the f32 arithmetic of the
+// separate combine kernel - and written as f16.  No intermediate [assignments, N] matrix, no combine launch.  An expert
+// shared by two tokens is streamed once per token, which is why this form is for batches of a few tokens.
+struct WcParams {
+  const uint32_t* w; const __half* s; const __half* b;  // stacked weights, expert 0
+  const __half* h;        // [assignments, K] f16, row a = assignment a (token a / top_k)
+  const uint32_t* idx;    // [assignments] expert of every assignment (outside [0, n_experts): contributes nothing)
+  const float* wts;       // [assignments] combine weights
+  __half* out;            // [T, N]
+  uint32_t K, N, top_k, n_experts;
+  uint64_t estride_w, estride_s;
+};
+
+template <int kPass>
+__global__ __launch_bounds__(512) void qmv_wt_combine_kernel(WcParams p) {
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+  constexpr int kBlk1 = 5;  // slots per (slab, j) block of a one-row image: four k sub-blocks, then zeros
+  const uint32_t K = p.K, S = K >> 7, NP = S / kPass;
+  const uint32_t img_bytes = S * 4 * kBlk1 * 16, sums_bytes = S * 2 * 2 * sizeof(float);
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int n = lane & 15, g = lane >> 4, par = g >> 1;
+  char* const img = smem + wave * (img_bytes + sums_bytes);
+  float* const sums = reinterpret_cast<float*>(img + img_bytes);           // [slab][group] = (-sum(off*x), sum(x))
+  float* const red = reinterpret_cast<float*>(smem + 8 * (img_bytes + sums_bytes));  // [wave][column]
+  const uint32_t t = blockIdx.y, tile = blockIdx.x, a = t * p.top_k + wave;
+  uint32_t expert = 0xFFFFFFFFu;
+  float cw = 0.f;
+  if ((uint32_t)wave < p.top_k) {
+    expert = p.idx[a];
+    cw = p.wts[a];
+  }
+  const bool live = expert < p.n_experts;  // (wave-uniform)
+  float mine = 0.f;
+  if (live) {
+    const uint32_t row_bytes = K >> 1, gpr = K >> 6, tile_row = tile * 16;
+    const __amdgpu_buffer_rsrc_t wr = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<uint32_t*>(p.w + expert * p.estride_w), 0, (int)((uint64_t)p.N * row_bytes > 0xFFFFFFFFull ? 0xFFFFFFFFull : (uint64_t)p.N * row_bytes), 0x00020000);
+    const __half* sb_base = ((g & 1) ? p.b : p.s) + expert * p.estride_s + (uint64_t)(tile_row + n) * gpr;
+    const uint32_t lane_woff = (uint32_t)(tile_row + n) * row_bytes + (uint32_t)g * 16;
+    struct Set { u4 w[kPass]; uint32_t sb[kPass]; };
+    auto load_step = [&](uint32_t pass, Set& st) {
+      const uint32_t* sp = reinterpret_cast<const uint32_t*>(sb_base) + pass * kPass;
+      if constexpr (kPass == 4) {
+        const U4Unaligned v = *reinterpret_cast<const U4Unaligned*>(sp);
+        st.sb[0] = v.v[0]; st.sb[1] = v.v[1]; st.sb[2] = v.v[2]; st.sb[3] = v.v[3];
+      } else {
+        const U2Unaligned v = *reinterpret_cast<const U2Unaligned*>(sp);
+        st.sb[0] = v.v[0]; st.sb[1] = v.v[1];
+      }
+#pragma unroll
+      for (int it = 0; it < kPass; ++it) st.w[it] = __builtin_amdgcn_raw_buffer_load_b128(wr, lane_woff, pass * (kPass * 64) + it * 64, 0);
+    };
+    // the wave's activation row (requested first), then the first pass of weights
+    constexpr int kMaxUnits = 8;  // K <= 4096: up to 8 units of 16 bytes per lane
+    const u4* xg = reinterpret_cast<const u4*>(p.h + (uint64_t)a * K);
+    u4 xv[kMaxUnits];
+#pragma unroll
+    for (int i = 0; i < kMaxUnits; ++i) {
+      xv[i] = (u4){0u, 0u, 0u, 0u};
+      if ((uint32_t)(lane + 64 * i) < (K >> 3)) xv[i] = xg[lane + 64 * i];
+    }
+    Set sa, sbuf;
+    load_step(0, sa);
+#pragma unroll
+    for (int i = 0; i < kMaxUnits; ++i) {
+      const uint32_t u = lane + 64 * i;
+      if (u < (K >> 3)) {
+        const uint32_t slab = u >> 4, gg = (u >> 2) & 3, j = u & 3;
+        *reinterpret_cast<u4*>(img + ((slab * 4 + j) * kBlk1 + gg) * 16) = permute_x8(xv[i]);
+      }
+    }
+    for (uint32_t z = lane; z < S * 4; z += 64) *reinterpret_cast<u4*>(img + (z * kBlk1 + 4) * 16) = (u4){0u, 0u, 0u, 0u};
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // (the image is private to the wave: no barrier)
+    // accumulator row 0 takes a slab's first group (k sub-blocks g < 2), row 8 its second; the other lanes read zeros
+    const bool a_active = (n == 0 && g < 2) || (n == 8 && g >= 2);
+    const uint32_t a_slot_off = (a_active ? (uint32_t)g : 4u) * 16;
+    Q4Consts qc{0x000F000Fu, 0x00F000F0u, 0x64006400u, 0x54005400u};
+    asm volatile("" : "+s"(qc.m0), "+s"(qc.m1), "+v"(qc.k0), "+v"(qc.k1));
+    {
+      const u4 bconst_bits = n < 8 ? (u4){0x64006400u, 0x54005400u, 0x64006400u, 0x54005400u}
+                                   : (u4){0x3C003C00u, 0x3C003C00u, 0x3C003C00u, 0x3C003C00u};
+      const h8 bconst = __builtin_bit_cast(h8, bconst_bits);
+      for (uint32_t slab = 0; slab < S; ++slab) {
+        f4 own = (f4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const h8 av = *reinterpret_cast<const h8*>(img + ((slab * 4 + j) * kBlk1) * 16 + a_slot_off);
+          own = __builtin_amdgcn_mfma_f32_16x16x32_f16(av, bconst, own, 0, 0, 0);
+        }
+        // accumulator row 0 (lanes g == 0) is the first group, row 8 (lanes g == 2) the second; column 0: sum(off*x), column 8: sum(x)
+        if ((g & 1) == 0 && n == 0) sums[(slab * 2 + par) * 2] = -own.x;
+        if ((g & 1) == 0 && n == 8) sums[(slab * 2 + par) * 2 + 1] = own.x;
+      }
+    }
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    const uint32_t half_sel = par ? 0x07060302u : 0x05040100u;
+    float F = 0.f;  // row 0 / row 8 of the accumulator tile: lanes with g == 0 / g == 2, element 0
+    auto compute_step = [&](uint32_t pass, const Set& st) {
+      uint32_t sv[kPass / 2], bv[kPass / 2];
+#pragma unroll
+      for (int q = 0; q < kPass / 2; ++q) {
+        const uint32_t own = __builtin_amdgcn_perm(st.sb[2 * q + 1], st.sb[2 * q], half_sel), oth = swap16(own);
+        sv[q] = (g & 1) ? oth : own;
+        bv[q] = (g & 1) ? own : oth;
+      }
+#pragma unroll
+      for (int it = 0; it < kPass; ++it) {
+        const uint32_t slab = pass * kPass + it;
+        const float2 k2 = *reinterpret_cast<const float2*>(sums + (slab * 2 + par) * 2);
+        f4 c = (f4){k2.x, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const uint32_t wd = j == 0 ? st.w[it].x : (j == 1 ? st.w[it].y : (j == 2 ? st.w[it].z : st.w[it].w));
+          const h8 av = *reinterpret_cast<const h8*>(img + ((slab * 4 + j) * kBlk1) * 16 + a_slot_off);
+          c = __builtin_amdgcn_mfma_f32_16x16x32_f16(av, unpack_q4_word(wd, qc), c, 0, 0, 0);
+        }
+        const uint32_t swd = sv[it >> 1], bwd = bv[it >> 1];
+        const float sc = (float)__builtin_bit_cast(_Float16, (unsigned short)((it & 1) ? swd >> 16 : swd & 0xFFFFu));
+        const float bi = (float)__builtin_bit_cast(_Float16, (unsigned short)((it & 1) ? bwd >> 16 : bwd & 0xFFFFu));
+        F = fmaf(sc, c.x, fmaf(bi, k2.y, F));
+      }
+    };
+    for (uint32_t i = 0; i < NP; i += 2) {
+      if (i + 1 < NP) load_step(i + 1, sbuf);
+      compute_step(i, sa);
+      if (i + 1 < NP) {
+        if (i + 2 < NP) load_step(i + 2, sa);
+        compute_step(i + 1, sbuf);
+      }
+    }
+    // lanes with (g & 1) == 0 hold the row's two group halves (g = 0 and g = 2): lane ^ 32 is the other one
+    mine = add_other_half((g & 1) == 0 ? F : 0.f);
+  }
+  if (g == 0) red[wave * 16 + n] = mine * cw;
+  lds_barrier();
+  if (tid < 16) {
+    float acc = 0.f;
+    for (uint32_t k = 0; k < p.top_k; ++k) acc += red[k * 16 + tid];  // ascending k, as the combine kernel adds
+    p.out[(uint64_t)t * p.N + tile * 16 + tid] = __float2half(acc);
+  }
+}
+
 template <int RH, int NW, bool DUAL, int kPass, int NS, int GC = 1>
 int32_t launch_one(const WtParams& p, bool tab, dim3 grid, size_t lds_bytes, hipStream_t s) {
   auto go = [&](auto kernel) -> int32_t {
@@ -378,6 +524,31 @@ int32_t launch_qmv_wt(const QmvArgs& a, uint32_t chunk_rows, hipStream_t s) {
   else if (rh == 2) st = a.dual ? launch_one<2, 8, true, 2, 2>(p, tab, grid, lds, s) : launch_one<2, 16, false, 4, 2>(p, tab, grid, lds, s);
   else st = a.dual ? launch_one<1, 8, true, 2, 2>(p, tab, grid, lds, s) : launch_one<1, 8, false, 4, 2>(p, tab, grid, lds, s);
   RMLX_TRY(st);
+  RMLX_HIP_CHECK(hipGetLastError());
+  return RMLX_OK;
+}
+
+bool qmv_wt_combine_supported(uint32_t N, uint32_t K, uint32_t group_size, uint32_t top_k) {
+  return group_size == 64 && N % 16 == 0 && K % 512 == 0 && N > 0 && K > 0 && K <= 4096 && top_k >= 1 && top_k <= 8;
+}
+
+int32_t launch_qmv_wt_combine(const uint32_t* w, const __half* s, const __half* b, uint64_t expert_stride_w,
+                              uint64_t expert_stride_s, uint32_t n_experts, const __half* h, const uint32_t* idx,
+                              const float* wts, uint32_t T, uint32_t top_k, uint32_t N, uint32_t K, __half* out,
+                              hipStream_t stream) {
+  if (!qmv_wt_combine_supported(N, K, 64, top_k))
+    return fail(RMLX_INVALID_SHAPE, "qmv_wt_combine: N %% 16, K %% 512, K <= 4096 and top_k <= 8 required (N=%u K=%u top_k=%u)", N, K, top_k);
+  if (T == 0) return RMLX_OK;
+  if (T > 65535) return fail(RMLX_INVALID_SHAPE, "qmv_wt_combine: at most 65535 tokens per launch (T=%u)", T);
+  WcParams p{w, s, b, h, idx, wts, out, K, N, top_k, n_experts, expert_stride_w, expert_stride_s};
+  const uint32_t S = K >> 7;
+  const size_t lds = 8 * ((size_t)S * 4 * 5 * 16 + (size_t)S * 2 * 2 * sizeof(float)) + 8 * 16 * sizeof(float);
+  static bool configured = false;
+  if (!configured) {
+    RMLX_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(qmv_wt_combine_kernel<4>), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
+    configured = true;
+  }
+  hipLaunchKernelGGL(qmv_wt_combine_kernel<4>, dim3(N / 16, T), dim3(512), lds, stream, p);
   RMLX_HIP_CHECK(hipGetLastError());
   return RMLX_OK;
 }

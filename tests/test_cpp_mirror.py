@@ -89,7 +89,9 @@ def test_mirror_matches_oracle(tmp_path, bits, gs, M):
     moe_ref = model.moe_forward(xt, idx, w, experts["gate"], experts["up"], experts["down"], 64, top_k)
     grouped = get("out_moe_grouped.bin", np.float16, (T, K))
     assert_close(grouped, moe_ref, "MoeExperts::forward_grouped")
-    assert np.array_equal(grouped, get("out_moe.bin", np.float16, (T, K)))
+    # (one call: a batch of a few tokens is routed without grouping and combined inside the down projection, so the two
+    # entry points agree to rounding, not bit for bit)
+    assert_close(get("out_moe.bin", np.float16, (T, K)), moe_ref, "MoeExperts::forward")
     for name, e, rows in [("out_group0.bin", 1, xt[:2]), ("out_group1.bin", 0, xt[2:])]:
         ones = np.ones((len(rows), 1))
         one_expert = model.moe_forward(rows, np.full((len(rows), 1), e), ones, experts["gate"], experts["up"],

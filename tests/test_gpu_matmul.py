@@ -906,3 +906,32 @@ def test_q8_group_128_on_the_streaming_gemv(hip, n, k, m):
     ref = model.qmm(x.astype(np.float64), words, s, b, 128, 8)
     assert_close(_run(hip, words, s, b, x, 8, gs=128, kernel=rt.KERNEL_QMV_ROWS), ref, f"Q8 gs128 M={m} N={n} K={k} (streaming GEMV)")
     assert_close(_run(hip, words, s, b, x, 8, gs=128), ref, f"Q8 gs128 M={m} N={n} K={k} (auto)")
+
+
+@pytest.mark.parametrize("gs", [32, 64, 128])
+@pytest.mark.parametrize("n,k", [(256, 4096), (64, 1088 * 2), (4096, 4096), (128, 11008 + 256), (8, 64 * 2)])
+def test_two_bit_single_row_kernel(hip, n, k, gs):
+    """2-bit weights through affine_quantized_matmul (the reference's affine_qmv takes every bit width,
+    quantized.rs:211-290) on the 2-bit single-row kernel: whole and partial chunks of 4096 values, all three group sizes,
+    against the oracle and against the portable kernel on the same inputs; one-hot weights pick single activations."""
+    from rmlx_amd import ops, runtime as rt
+    rng = np.random.default_rng(n + k + gs)
+    k = (k // gs) * gs
+    words, s, b = make_weight(rng, n, k, 2, gs)
+    x = make_x(rng, 1, k)
+    ref = model.qmm(x.astype(np.float64), words, s, b, gs, 2)
+    got = _run(hip, words, s, b, x[0], 2, gs=gs, qmv_entry=True)
+    assert_close(got, ref, f"2-bit N={n} K={k} gs={gs}")
+    portable = _run(hip, words, s, b, x, 2, gs=gs, kernel=rt.KERNEL_GENERIC)
+    assert_close(portable, ref, f"2-bit N={n} K={k} gs={gs} (portable)")
+    # value position: q = 1 at one (row, k) with scale 1 and bias 0 everywhere returns exactly x[k] in that row
+    wz = np.zeros_like(words)
+    ones, zeros = np.ones_like(s), np.zeros_like(b)
+    picks = [(0, 0), (n - 1, k - 1), (n // 2, min(k - 1, 4097)), (3 % n, 23), (5 % n, min(k - 1, 2048 + 40))]
+    for r, kk in picks:
+        wz[r, kk // 16] |= np.uint32(1) << np.uint32(2 * (kk % 16))
+    got = _run(hip, wz, ones, zeros, x[0], 2, gs=gs, qmv_entry=True)[0].astype(np.float64)
+    want = np.zeros(n)
+    for r, kk in picks:
+        want[r] += float(x[0, kk])
+    assert np.allclose(got, want.astype(np.float16).astype(np.float64), atol=2e-3), (got[[r for r, _ in picks]], want[[r for r, _ in picks]])

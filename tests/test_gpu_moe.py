@@ -683,6 +683,39 @@ def test_wave_per_tile_kernel_shapes(hip, E, T, K, D, I, fused):
                          f"ExpertGroup stream kernel {kind} expert {e} rows {len(v)}")
 
 
+@pytest.mark.parametrize("T,E,K,D,I,bias", [(1, 128, 8, 1024, 512, False), (4, 16, 8, 512, 1536, True), (3, 8, 5, 2048, 1024, False),
+                                            (16, 64, 2, 512, 512, False), (17, 64, 2, 512, 512, True), (2, 4, 1, 512, 4096, False)])
+def test_few_tokens_run_without_grouping(hip, T, E, K, D, I, bias):
+    """`moe_forward` with at most 32 assignments routes without grouping (every assignment a chunk of one row) and adds
+    the weighted expert outputs inside the down projection; 33 and more take the grouped path.  Both against the oracle
+    and against the grouped kernels (stream kernel 1) on the same inputs: experts shared by several tokens, fewer picks
+    than waves, an expert bias, the largest batch of either side of the limit."""
+    from rmlx_amd import ops
+    from rmlx_amd.runtime import DeviceBuffer
+    rng = np.random.default_rng(T * 1000 + E + K)
+    gu = make_weight(rng, 2 * I, D, 4, 64, lead=(E,))
+    down = make_weight(rng, D, I, 4, 64, lead=(E,))
+    gate, up = tuple(a[:, :I] for a in gu), tuple(a[:, I:] for a in gu)
+    gh, dh = ops.QuantizedWeight.from_numpy(*gu, 64, 4), ops.QuantizedWeight.from_numpy(*down, 64, 4)
+    x = make_x(rng, T, D)
+    logits = rng.standard_normal((T, E)).astype(np.float32)
+    eb = rng.standard_normal(E).astype(np.float32) if bias else None
+    idx, w, _, _ = model.topk_route(logits, K, eb)
+    ref = model.moe_forward(x, idx, w, gate, up, down, 64, K)
+    xd, ld = DeviceBuffer.from_numpy(x), DeviceBuffer.from_numpy(logits)
+    bd = DeviceBuffer.from_numpy(eb) if bias else None
+    print(f"few tokens T={T} E={E} K={K} D={D} I={I} bias={bias}", flush=True)
+    direct = ops.moe_forward(gh, None, dh, xd, ld, K, expert_bias=bd).numpy()
+    assert_close(direct, ref, "moe_forward (default)")
+    prev = gh.set_expert_stream_kernel(1)
+    try:
+        grouped = ops.moe_forward(gh, None, dh, xd, ld, K, expert_bias=bd).numpy()
+    finally:
+        gh.set_expert_stream_kernel(prev)
+    assert_close(grouped, ref, "moe_forward (grouped kernels)")
+    assert np.abs(direct.astype(np.float64) - grouped.astype(np.float64)).max() <= 0.25 * model.tolerance(ref)
+
+
 @pytest.mark.parametrize("T", [300, 700])
 def test_config5_moe_prefill_sizes(hip, config5, T):
     """Config 5 at prefill-sized batches (19 / 44 rows per expert on average: the grouped GEMM with 32- / 64-row tiles).
