@@ -59,7 +59,7 @@ def matmul_bytes(m, n, k, bits, gs=64, act_bytes=2):
 
 
 def make_weight(rng, n, k, bits, lead=()):
-    lo, hi = (0.005, 0.02) if bits == 4 else (0.0005, 0.002)
+    lo, hi = (0.005, 0.02) if bits <= 4 else (0.0005, 0.002)
     words = rng.integers(0, 2**32, size=tuple(lead) + (n, k * bits // 32), dtype=np.uint32)
     s = rng.uniform(lo, hi, size=tuple(lead) + (n, k // 64)).astype(np.float16)
     b = (-(2.0 ** (bits - 1)) * s.astype(np.float32)).astype(np.float16)
@@ -99,7 +99,7 @@ class Timer:
 
 
 def bench_matmul(ops, rt, timer, rng, m, n, k, bits, x_dtype, launches, warmup, min_total_bytes, check=True, kernel=0,
-                 check_rows=None, graph=False):
+                 check_rows=None, graph=False, queued_trains=0):
     from oracle import model
     wbytes = n * k * bits // 8 + 4 * (n * k // 64)
     n_sets = max(1, -(-min_total_bytes // wbytes))
@@ -118,7 +118,24 @@ def bench_matmul(ops, rt, timer, rng, m, n, k, bits, x_dtype, launches, warmup, 
         xd = rt.DeviceBuffer.from_numpy(xh)
         x64 = xh.astype(np.float64)
     outs = [rt.DeviceBuffer((m, n), rt.F16) for _ in range(min(n_sets, 8))]
-    if graph:  # the train is recorded once and replayed: no host work per launch (kernel nodes only)
+    if queued_trains:
+        # Every train is enqueued behind a stall kernel (a few milliseconds of matrix instructions on a quarter of the
+        # CUs), so the whole train sits in the queue before its first kernel starts and runs back to back whatever a
+        # launch costs the host - under a tracer too, where the host needs longer per launch than the kernel runs.
+        L, sink = rt.lib(), rt.DeviceBuffer((64,), rt.U32)
+        total_ms = 0.0
+        for _ in range(queued_trains + 1):
+            rt.check(L.rmlx_hip_measure_floor(rt.FLOOR_MFMA, None, 64, 0, 8000, sink.ptr, 1, timer.stream.handle))
+            timer.e0.record(timer.stream)
+            ops.qmm_encode_many(qws, xd, outs, TRAIN, stream=timer.stream, kernel=kernel)
+            timer.e1.record(timer.stream)
+            timer.e1.sync()
+            total_ms += timer.e0.elapsed_ms(timer.e1)
+            if _ == 0:
+                total_ms = 0.0  # (the first train is warm-up)
+        launches = queued_trains * TRAIN
+        ms = total_ms / launches
+    elif graph:  # the train is recorded once and replayed: no host work per launch (kernel nodes only)
         with rt.Graph.record(timer.stream) as g:
             ops.qmm_encode_many(qws, xd, outs, TRAIN, stream=timer.stream, kernel=kernel)
 
@@ -385,7 +402,8 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50, help=f"timed steps; a step is a train of {TRAIN} launches")
     ap.add_argument("--warmup", type=int, default=10, help="untimed warm-up steps")
-    ap.add_argument("--only", default="", help="comma-separated sections: headline, floors, qmv, qmm, dequant, gather, moe, moe8, large")
+    ap.add_argument("--only", default="", help="comma-separated sections: headline, floors, qmv, qmm, dequant, gather, moe, moe8, large; moevariants (not in the "
+                                           "default run): the routed block at T = 96 / 128 / 160 under every choice of expert kernels")
     ap.add_argument("--quick", action="store_true", help="headline and floors only, short CPU baseline")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-graph", action="store_true",
@@ -420,9 +438,14 @@ def main():
     progress("headline")
     head = bench_matmul(ops, rt, timer, rng, 1, 4096, 4096, 4, "f16", launches, warm, GiB + GiB // 8)
     extra = {"device": info, "launches_per_step": TRAIN, "q4_qmv_m1_4096": head}
+    # The same configuration in trains that are fully enqueued before they start (behind a stall kernel): what a kernel
+    # trace of this command shows for these launches is the kernel's duration in a train, not that of a lone launch.
+    progress("headline, trains enqueued behind a stall kernel")
+    extra["q4_qmv_m1_4096_queued_trains"] = bench_matmul(ops, rt, timer, rng, 1, 4096, 4096, 4, "f16", launches, TRAIN,
+                                                         GiB + GiB // 8, queued_trains=max(5, min(args.steps, 25)))
     if not args.no_graph:
-        # The same train recorded once and replayed (kernel nodes only): no host work per launch, so a kernel trace
-        # of this section shows the kernels as close together as they run without the tracer.
+        # The same train recorded once as a graph (kernel nodes only) and replayed: no host work per launch.  (Not under
+        # rocprofv3 7.2, whose kernel tracing crashes in hipGraphLaunch: profile runs pass --no-graph.)
         progress("headline, graph replay")
         extra["q4_qmv_m1_4096_graph_replay"] = bench_matmul(ops, rt, timer, rng, 1, 4096, 4096, 4, "f16", launches, TRAIN,
                                                             GiB + GiB // 8, graph=True)
@@ -448,6 +471,7 @@ def main():
                                                        warm, GiB + GiB // 8, check=(m == 8))
         extra["q4_qmv_m2_4096"] = bench_matmul(ops, rt, timer, rng, 2, 4096, 4096, 4, "f16", launches, warm, GiB + GiB // 8)
         extra["q8_qmv_m1_4096"] = bench_matmul(ops, rt, timer, rng, 1, 4096, 4096, 8, "f16", launches, warm, GiB + GiB // 8)
+        extra["q2_qmv_m1_4096"] = bench_matmul(ops, rt, timer, rng, 1, 4096, 4096, 2, "f16", launches, warm, GiB + GiB // 8)
         # long K, short N: the shapes the reference sends to its split-K GEMV (K > 8192 and N <= 2048)
         extra["q4_qmv_m1_n2048_k16384"] = bench_matmul(ops, rt, timer, rng, 1, 2048, 16384, 4, "f16", launches, warm, GiB + GiB // 8)
     if "large" in sections:
@@ -471,7 +495,7 @@ def main():
         progress("dequant")
         for fmt in ("awq", "gptq"):
             extra[f"{fmt}_dequant_4096x4096_gs128"] = bench_dequant(ops, rt, timer, rng, fmt, 4096, 4096, 128, max(200, launches // 10))
-    if sections & {"gather", "moe"}:
+    if sections & {"gather", "moe", "moevariants"}:
         progress("gather / moe")
         gate_up = make_weight(rng, 3072, 4096, 4, lead=(128,))
         down = make_weight(rng, 4096, 1536, 4, lead=(128,))
@@ -484,12 +508,32 @@ def main():
                 r["hbm_frac"] = r["gbs"] / HBM_PEAK_GBS
                 extra[f"gather_qmm_q4_b{batch}_m{mpb}"] = r
         if "moe" in sections:
-            for T in (4, 32, 128, 512, 2048):  # from 10 rows per expert on average on the grouped MFMA GEMM
+            for T in (1, 4, 32, 128, 512, 2048):  # from 10 rows per expert on average on the grouped MFMA GEMM
                 r = bench_moe(ops, rt, timer, rng, T, calls if T <= 128 else max(50, calls // 4), experts)
                 r["tflops"] = r["flops"] / (r["us"] * 1e-6) / 1e12
                 r["mfma_frac"] = r["tflops"] / MFMA_F16_PEAK_TF
                 r["hbm_frac"] = r["gbs"] / HBM_PEAK_GBS
                 extra[f"moe_q4_T{T}"] = r
+        if "moevariants" in sections:
+            # The routed block at 6 / 8 / 10 rows per expert with every choice of expert kernels (for kernel traces:
+            # which projection costs what under which kernel).  (label, GEMM threshold, streaming kernel selector)
+            variants = (("kplit_8row_chunks", 0, 1), ("wave_per_tile_8row_chunks", 0, 2), ("wave_per_tile_16row_chunks", 0, 3),
+                        ("hybrid_kplit_gate_up_wave_down", 0, 4), ("grouped_gemm", 1, 0))
+            for T in (96, 128, 160):
+                for label, min_rows, kind in variants:
+                    # (a threshold of 1 forces the GEMM; its tile height follows the average rows per expert: 16-row tiles
+                    # at T = 96, 32-row tiles at T = 128 and 160)
+                    # (an empty marker kernel in front of every measurement: a kernel trace is split at these)
+                    rt.check(rt.lib().rmlx_hip_measure_floor(rt.FLOOR_EMPTY, None, 0, 0, 0, None, 1, timer.stream.handle))
+                    prev_rows = experts[2].set_expert_gemm_min_rows(min_rows)
+                    prev_kind = experts[2].set_expert_stream_kernel(kind)
+                    try:
+                        r = bench_moe(ops, rt, timer, rng, T, max(100, calls // 2), experts)
+                    finally:
+                        experts[2].set_expert_gemm_min_rows(prev_rows)
+                        experts[2].set_expert_stream_kernel(prev_kind)
+                    r["hbm_frac"] = r["gbs"] / HBM_PEAK_GBS
+                    extra[f"moe_q4_T{T}_{label}"] = r
         del experts, gate_up, down
     if "moe8" in sections:
         progress("moe8")
@@ -544,6 +588,9 @@ def main():
     if g is not None:
         line["roofline"]["graph_replay_launch_us"] = g["us"]
         line["roofline"]["frac_graph_replay"] = g["gbs"] / HBM_PEAK_GBS
+    qd = extra.get("q4_qmv_m1_4096_queued_trains")
+    if qd is not None:
+        line["roofline"]["queued_train_launch_us"] = qd["us"]
     fl = extra.get("floors", {}).get("read_9.45MB")
     if fl is not None:
         # what a kernel that only reads the same bytes reaches in the same train: the ceiling of `frac` at this size

@@ -905,7 +905,8 @@ int32_t rmlx_hip_qmm_encode_many(const rmlx_qweight* const* qws, size_t n_qw, co
     if (qws[i] == nullptr || qws[i]->n_experts != 1 || qws[i]->in_features != qws[0]->in_features ||
         qws[i]->out_features != qws[0]->out_features)
       return fail(RMLX_INVALID_SHAPE, "qmm_encode_many: weight %zu does not match weight 0", i);
-    if (qws[i]->bits != 4 && qws[i]->bits != 8)
+    // (a single row is the qmv entry point, which takes every bit width: quantized.rs:1309-1411)
+    if (qws[i]->bits != 4 && qws[i]->bits != 8 && !(x->shape[0] == 1))
       return fail(RMLX_INVALID_SHAPE, "affine_quantized_matmul_batched requires bits==4 or bits==8, got %u", qws[i]->bits);
   }
   if (x->shape[1] != qws[0]->in_features)
