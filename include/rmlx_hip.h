@@ -307,10 +307,11 @@ int32_t rmlx_hip_moe_forward_grouped(const rmlx_qweight* gate, const rmlx_qweigh
  * `MoeStrategy` for a layer in the reference (crates/rmlx-nn/src/moe.rs:515-541).  Returns the previous value. */
 uint32_t rmlx_hip_qweight_set_expert_gemm_min_rows(rmlx_qweight* gate_qw, uint32_t min_rows);
 /* Which streaming kernel runs the expert projections of decode-sized batches (below the grouped GEMM's threshold) of a
- * block whose gate weight is `qw`: 0 = the library's choice, 1 = K split over the waves of a workgroup, chunks of 8
- * rows, 2 = a wave per 16-row weight tile, chunks of 8 rows, 3 = a wave per tile, chunks of 16 rows (4-bit weights,
- * group size 64; other weights keep kernel 1).  Returns the previous value; the tests use it to check that the kernels
- * agree.  (No counterpart in the reference, which has one kernel for this: gather_qmv_fast_f16_q4,
+ * block whose gate weight is `qw`: 1 = K split over the waves of a workgroup, chunks of 8 rows, 2 = a wave per 16-row
+ * weight tile, chunks of 8 rows, 3 = a wave per tile, chunks of 16 rows, 4 = kernel 1 for the gate / up projection and
+ * kernel 2 for the down projection (4-bit weights, group size 64; other weights keep kernel 1), 0 = the library's
+ * choice: 3 between 7 and 8.5 rows per expert on average, else 4.  Returns the previous value; the tests use it to check
+ * that the kernels agree.  (No counterpart in the reference, which has one kernel for this: gather_qmv_fast_f16_q4,
  * crates/rmlx-core/src/ops/quantized.rs:9752-9842.) */
 uint32_t rmlx_hip_qweight_set_expert_stream_kernel(rmlx_qweight* qw, uint32_t kind);
 

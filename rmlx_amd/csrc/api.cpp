@@ -468,17 +468,24 @@ uint32_t expert_gemm_tile_rows(const ExpertShapes& sh, uint64_t rows, uint64_t g
 // Which streaming kernel runs the two projections of a decode-sized batch, and over chunks of how many rows.
 // gate_up / down: 0 = the K-split kernel (qmv.hip), else the wave-per-tile kernel (qmv_wt.hip) with chunks of that many
 // rows (8 or 16).  Selector of the gate handle: 1 = K-split for both, 2 / 3 = wave per tile for both with chunks of 8 / 16
-// rows, 0 (the library's choice) and 4 = K-split for gate / up, wave per tile for a down projection whose rows are
-// shorter than 4096 (measured at D = 4096, I = 1536: the block takes 254 against 269 us at T = 32 and 348 against 368 us at
-// T = 128; a wave-per-tile gate / up projection is 30 % slower than the K-split one, which reads a tile's 32 KB as one
-// contiguous block).
+// rows, 4 = K-split for gate / up, wave per tile for a down projection whose rows are shorter than 4096 (measured at
+// D = 4096, I = 1536: the block takes 254 against 269 us at T = 32 and 348 against 368 us at T = 128; over chunks of 8
+// rows a wave-per-tile gate / up projection is 30 % slower than the K-split one), 0 = the library's choice: 4 up to 7
+// rows per expert on average, 3 from 7 to 8.5.
 struct StreamPlan { uint32_t gate_up, down, chunk_rows; };
-StreamPlan expert_stream_plan(const ExpertShapes& sh) {
+// rows / groups: the assignments of the call and the experts (or host-side groups) they spread over
+StreamPlan expert_stream_plan(const ExpertShapes& sh, size_t rows, size_t groups) {
   StreamPlan pl{0, 0, 8};
   if (sh.wave_gs32) return StreamPlan{8, 8, 8};
   if (sh.stream_kernel == 1) return pl;
   if (sh.stream_kernel == 2 && sh.wave_tiles) pl = StreamPlan{8, 8, 8};
   else if (sh.stream_kernel == 3 && sh.wave_tiles) pl = StreamPlan{16, 16, 16};
+  // From 7 rows per expert on average most experts hold more than one chunk of 8 rows, which the K-split kernel streams
+  // once per chunk: the wave-per-tile kernels over chunks of 16 rows then win, until experts with more than 16 rows add
+  // a seventh round of workgroups to their six (measured at D = 4096, I = 1536, E = 128, K-split gate / up with the
+  // wave-per-tile down projection against chunks of 16 rows: 301 / 320 us at 6.5 rows per expert, 320 / 321 at 7,
+  // 336 / 323 at 8, 363 / 385 at 9).
+  else if (sh.stream_kernel == 0 && sh.wave_tiles && rows >= 7 * groups && 2 * rows < 17 * groups) pl = StreamPlan{16, 16, 16};
   else if (sh.wave_down && sh.I < 4096) pl.down = 8;
   return pl;
 }
@@ -1208,7 +1215,7 @@ int32_t rmlx_hip_expert_group_grouped_forward(const rmlx_qweight* gate, const rm
   for (size_t i = 0; i < n_items; ++i) total += batch_sizes_host[i];
   // row chunks of one expert each: 8 rows for the streaming GEMV, whole row tiles for the grouped GEMM
   const uint32_t gemm = expert_gemm_tile_rows(sh, total, n_items);
-  const StreamPlan plan = expert_stream_plan(sh);
+  const StreamPlan plan = expert_stream_plan(sh, total, n_items);
   const uint32_t chunk_rows = gemm ? gemm : plan.chunk_rows;
   std::vector<uint32_t> tab;
   total = 0;
@@ -1294,7 +1301,7 @@ int32_t moe_grouped_impl(const rmlx_qweight* gate, const rmlx_qweight* up, const
   if (T == 0) return RMLX_OK;
   // many rows per expert: the grouped GEMM over row tiles instead of the streaming GEMV over chunks of 8 rows
   const uint32_t gemm = route == nullptr ? expert_gemm_tile_rows(sh, A, sh.E) : 0u;
-  StreamPlan plan = expert_stream_plan(sh);
+  StreamPlan plan = expert_stream_plan(sh, A, sh.E);
   if (route != nullptr && plan.chunk_rows != 8) {  // (the fused routing + grouping launch writes chunks of 8 rows)
     plan.chunk_rows = 8;
     if (plan.gate_up) plan.gate_up = 8;

@@ -519,9 +519,11 @@ int32_t launch_qmv_wt(const QmvArgs& a, uint32_t chunk_rows, hipStream_t s) {
   int32_t st;
   // (ring depths measured on the routed block at T = 32 / 128: a third set for the fused kernel 317 / 438 us against
   // 306 / 424 us with two; passes of two slabs in a ring of four or three for the plain kernel 263 / 261 us against 255 us
-  // with passes of four in a ring of two - more requests in flight per wave make this access pattern slower, not faster)
+  // with passes of four in a ring of two.  The 16-row fused kernel runs one workgroup per CU either way and has the
+  // registers for passes of four slabs: 329 against 370 us at T = 128, while two, three or four sets of two-slab passes
+  // all take 370 to 375 us - the size of a pass matters, the depth of the ring does not)
   if (gs == 32) st = a.dual ? launch_one<1, 8, true, 2, 2, 2>(p, tab, grid, lds, s) : launch_one<1, 8, false, 2, 2, 2>(p, tab, grid, lds, s);
-  else if (rh == 2) st = a.dual ? launch_one<2, 8, true, 2, 2>(p, tab, grid, lds, s) : launch_one<2, 16, false, 4, 2>(p, tab, grid, lds, s);
+  else if (rh == 2) st = a.dual ? launch_one<2, 8, true, 4, 2>(p, tab, grid, lds, s) : launch_one<2, 16, false, 4, 2>(p, tab, grid, lds, s);
   else st = a.dual ? launch_one<1, 8, true, 2, 2>(p, tab, grid, lds, s) : launch_one<1, 8, false, 4, 2>(p, tab, grid, lds, s);
   RMLX_TRY(st);
   RMLX_HIP_CHECK(hipGetLastError());

@@ -56,7 +56,8 @@ class QuantizedWeight:
 
     def set_expert_stream_kernel(self, kind):
         """(stacked gate weight) streaming kernel of decode-sized batches: 0 the library's choice, 1 K split over the
-        waves of a workgroup, 2 / 3 a wave per weight tile with chunks of 8 / 16 rows.  Returns the previous value."""
+        waves of a workgroup, 2 / 3 a wave per weight tile with chunks of 8 / 16 rows, 4 kernel 1 for gate / up and kernel 2
+        for the down projection.  Returns the previous value."""
         return int(rt.lib().rmlx_hip_qweight_set_expert_stream_kernel(self.handle, int(kind)))
 
     def groups_per_row(self):
