@@ -162,7 +162,7 @@ bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) ==
 // register-weights MFMA GEMM above (the LDS-staged GEMM when K is not a multiple of 512), the
 // portable kernel for every shape the fast kernels do not take.
 enum { KERNEL_AUTO = 0, KERNEL_QMV = 1, KERNEL_QMM = 2, KERNEL_GENERIC = 3, KERNEL_QMM_BF16 = 4, KERNEL_QMM_LDS = 5,
-       KERNEL_QMV_ROWS = 6, KERNEL_QMM_K2 = 7, KERNEL_QMM_RW = 8, KERNEL_QMM_K2_TALL = 9 };
+       KERNEL_QMV_ROWS = 6, KERNEL_QMM_K2 = 7, KERNEL_QMM_RW = 8, KERNEL_QMM_K2_TALL = 9, KERNEL_QMM_K2_FLAT = 10 };
 constexpr uint32_t kQmvMaxM = 16;
 // group size 64: rows taken by the single-row kernel (measured: 3 and 4 rows are faster on the matrix unit)
 constexpr uint32_t kM1MaxRows = 2;
@@ -247,7 +247,7 @@ int32_t run_matmul_plain(const rmlx_qweight* qw, const void* x, int32_t x_dtype,
   } else if (kernel == KERNEL_QMM_BF16 && !(can_qmm_lds && qw->bits == 8 && x_dtype == RMLX_DTYPE_BF16)) {
     return fail(RMLX_INVALID_SHAPE, "the bf16 MFMA GEMM takes Bfloat16 activations and 8-bit weights (got %s, bits=%u)",
                 dtype_name(x_dtype), qw->bits);
-  } else if ((kernel == KERNEL_QMM_K2 && !can_qmm_k2) || (kernel == KERNEL_QMM_RW && !can_qmm_rw)) {
+  } else if (((kernel == KERNEL_QMM_K2 || kernel == KERNEL_QMM_K2_FLAT) && !can_qmm_k2) || (kernel == KERNEL_QMM_RW && !can_qmm_rw)) {
     return fail(RMLX_INVALID_SHAPE,
                 "the register-weights qmm kernels require bits in {4,8}, N %% 64 == 0, K %% 512 == 0 and 16-byte aligned "
                 "buffers (N=%u K=%u bits=%u group_size=%u)", N, K, qw->bits, qw->group_size);
@@ -256,7 +256,7 @@ int32_t run_matmul_plain(const rmlx_qweight* qw, const void* x, int32_t x_dtype,
                 "the 128 x 128 K-split qmm kernel requires bits in {4,8} (8-bit weights at group size 32 / 64: f16 or f32 "
                 "activations), N %% 128 == 0, K %% 512 == 0 and 16-byte aligned buffers (N=%u K=%u bits=%u group_size=%u)",
                 N, K, qw->bits, qw->group_size);
-  } else if (kernel < 0 || kernel > KERNEL_QMM_K2_TALL) {
+  } else if (kernel < 0 || kernel > KERNEL_QMM_K2_FLAT) {
     return fail(RMLX_NOT_FOUND, "unknown kernel selector %d", kernel);
   }
   // The K-split GEMM (32x32x16 MFMAs, K split inside the workgroup).  64 x 128 tiles where that grid is one round over
@@ -265,7 +265,7 @@ int32_t run_matmul_plain(const rmlx_qweight* qw, const void* x, int32_t x_dtype,
   // 29.6 against 35.5 us at M = 640, 37.0 against 41.4 us at M = 1024, 153 against 175 us at M = 4096 (4096 x 4096), 30.9
   // against 37.8 us at M = 192, N = 12288.  With fewer tiles the smaller tiles of the register-weights GEMM keep more
   // CUs busy.
-  uint32_t k2_tile_rows = kernel == KERNEL_QMM_K2_TALL ? 128 : 64;
+  uint32_t k2_tile_rows = kernel == KERNEL_QMM_K2_TALL ? 128 : kernel == KERNEL_QMM_K2_FLAT ? 32 : 64;
   if (kernel == KERNEL_QMM && can_qmm_k2) {
     const uint64_t tiles = (uint64_t)((M + 63) / 64) * (N / 128), tall = (uint64_t)((M + 127) / 128) * (N / 128);
     const uint64_t cus = (uint64_t)ctx().num_cus;
@@ -274,8 +274,18 @@ int32_t run_matmul_plain(const rmlx_qweight* qw, const void* x, int32_t x_dtype,
     const bool fits64 = (uint64_t)((M + 63) / 64) * 64 * 3 <= (uint64_t)M * 4, fits128 = (uint64_t)((M + 127) / 128) * 128 * 3 <= (uint64_t)M * 4;
     if (fits64 && tiles * 10 >= cus * 7 && tiles <= cus) kernel = KERNEL_QMM_K2;
     else if (fits128 && can_qmm_k2_tall && tall * 10 >= cus * 6) { kernel = KERNEL_QMM_K2; k2_tile_rows = 128; }
+    // 32 x 128 tiles: one round of them takes about 18.5 us at K = 4096 whatever their number (the length of the k loop);
+    // the register-weights GEMM is faster while its 32 x 64 tiles fit one round over the chip (15.6 us at M = 128,
+    // 4096 x 4096) and slower once it has to take larger tiles (M = 160: 24.4 us, M = 256: 21.1 against 19.3;
+    // N = 9216, M = 64: 25.0 against 19.8).  Where the 32-row tiles need more than one round, one round of 64-row tiles
+    // still wins (N = 9216, M = 128: 22.2 against 23.7 us).  Measured at K = 4096 only, so longer rows keep the other
+    // kernels; so do 8-bit weights over wide matrices (N = 12288, M = 64: 28.6 against 27.7 us).
+    else if (K <= 4096 && qmm_rw_tile_work(M, N, K, qw->group_size, qw->bits) >= 16 && !(qw->bits == 8 && N > 8192)) {
+      if (M > 32 && (uint64_t)((M + 31) / 32) * (N / 128) <= cus) { kernel = KERNEL_QMM_K2; k2_tile_rows = 32; }
+      else if (fits64 && tiles <= cus) kernel = KERNEL_QMM_K2;
+    }
   }
-  if (kernel == KERNEL_QMM_K2_TALL) kernel = KERNEL_QMM_K2;
+  if (kernel == KERNEL_QMM_K2_TALL || kernel == KERNEL_QMM_K2_FLAT) kernel = KERNEL_QMM_K2;
   if (kernel == KERNEL_QMM_RW) kernel = KERNEL_QMM;
 
   // RMSNorm prologue: fused into the single-row GEMV for one or two rows (while it stages the activations);

@@ -198,6 +198,8 @@ int32_t launch_epilogue(__half* out, int kind, const void* e, int32_t e_dtype, s
 size_t qmm_workspace_bytes(uint32_t M, uint32_t K);
 // split-K partial sums of the register-weights GEMM (0 when the launch is not split); pass the buffer in QmmArgs::workspace
 size_t qmm_rw_workspace_bytes(uint32_t M, uint32_t N, uint32_t K, uint32_t group_size, uint32_t bits);
+// 16 x 16 fragments per workgroup (tile rows / 16 x tile columns / 16) of the tile the launcher would pick; 0 = not supported
+uint32_t qmm_rw_tile_work(uint32_t M, uint32_t N, uint32_t K, uint32_t group_size, uint32_t bits);
 bool qmm_supported(uint32_t N, uint32_t K, uint32_t group_size, uint32_t bits);
 int32_t launch_qmm(const QmmArgs& a, hipStream_t s);
 // Register-weights GEMM (qmm_rw.hip): f16 activations only, no workspace.

@@ -101,10 +101,10 @@ __device__ __forceinline__ uint32_t act_slot(uint32_t R, uint32_t seg) {
 // through the CU's L1 again: measured 1.56 x the useful bytes between L2 and the CU).
 template <int BITS, bool XBF16, int GS, int MFR, bool SBLDS = false>
 __global__ __launch_bounds__(kThreads) void qmm_k2_kernel(const K2Params p) {
-  static_assert(!SBLDS || (GS == 64 && MFR == 2), "scales in LDS: 64-row tiles, group size 64");
+  static_assert(!SBLDS || (GS == 64 && MFR <= 2), "scales in LDS: tiles of at most 64 rows, group size 64");
   constexpr int kTileM = 32 * MFR;
-  constexpr int kChunkUnits = kTileM * 16;               // 16-byte units of one activation chunk (rows x 128 k): 1024 / 2048
-  constexpr int kAL = kChunkUnits / kThreads;            // units per thread and chunk: 2 / 4
+  constexpr int kChunkUnits = kTileM * 16;               // 16-byte units of one activation chunk (rows x 128 k): 512 / 1024 / 2048
+  constexpr int kAL = kChunkUnits / kThreads;            // units per thread and chunk: 1 / 2 / 4
   constexpr int WV = BITS == 4 ? 1 : 2;                  // 16-byte weight loads per lane and block
   constexpr int kSbBytes = 4 * (kBlockK / GS) * 2;       // scales of one row and four blocks: 16 / 32 / 8 bytes
   constexpr int kSbVecs = kSbBytes > 16 ? 2 : 1;
@@ -357,28 +357,30 @@ __global__ __launch_bounds__(kThreads) void qmm_k2_kernel(const K2Params p) {
   // a stride of 512 bytes) spread over the banks.
   // 64 rows (two fragments) per pass: 2 x 64 x 128 floats fill the 64 KB.
   float* red = reinterpret_cast<float*>(lds);
+  constexpr int kFr = MFR >= 2 ? 2 : 1;   // fragments per pass: 64 rows (32 with one fragment) x 128 columns x two halves
+  constexpr int kPassRows = 32 * kFr;
 #pragma unroll
-  for (int pass = 0; pass < MFR / 2; ++pass) {
+  for (int pass = 0; pass < MFR / kFr; ++pass) {
   if (pass > 0) __syncthreads();  // the previous pass has been read
 #pragma unroll
-  for (int i = 0; i < 2; ++i) {
+  for (int i = 0; i < kFr; ++i) {
     const uint32_t m = 32 * i + r;
 #pragma unroll
     for (int eg = 0; eg < 4; ++eg) {
       const uint32_t cg = 8 * wn + 2 * eg + hh;  // weight rows 4 cg .. 4 cg + 3 of the tile
       f4 v;
 #pragma unroll
-      for (int e = 0; e < 4; ++e) v[e] = acc[2 * pass + i][eg * 4 + e];
-      *reinterpret_cast<f4*>(red + ((size_t)(kh * 64 + m) * 32 + (cg ^ (m & 31))) * 4) = v;
+      for (int e = 0; e < 4; ++e) v[e] = acc[kFr * pass + i][eg * 4 + e];
+      *reinterpret_cast<f4*>(red + ((size_t)(kh * kPassRows + m) * 32 + (cg ^ (m & 31))) * 4) = v;
     }
   }
   __syncthreads();
 #pragma unroll
-  for (int q = 0; q < 4; ++q) {  // 64 rows x 32 groups = 2048 units of four outputs: four per thread
+  for (int q = 0; q < 2 * kFr; ++q) {  // rows x 32 groups = units of four outputs: four (two) per thread
     const uint32_t g = q * kThreads + tid, m = g >> 5, cgp = g & 31, cg = cgp ^ (m & 31);
     f4 v = *reinterpret_cast<const f4*>(red + ((size_t)m * 32 + cgp) * 4);
-    v += *reinterpret_cast<const f4*>(red + ((size_t)(64 + m) * 32 + cgp) * 4);
-    const uint32_t row = row_lo + 64 * pass + m, col = nt * kTileN + 4 * cg;
+    v += *reinterpret_cast<const f4*>(red + ((size_t)(kPassRows + m) * 32 + cgp) * 4);
+    const uint32_t row = row_lo + kPassRows * pass + m, col = nt * kTileN + 4 * cg;
     if (row < p.M) {
       const uint64_t o = (uint64_t)row * p.N + col;
       if (p.epi_kind != EPI_NONE) {  // residual add / SwiGLU gate in f32, one rounding (quantized.rs:3206-3246)
@@ -416,7 +418,7 @@ bool qmm_k2_tall_supported(uint32_t group_size, uint32_t bits, bool x_bf16) {
 }
 
 int32_t launch_qmm_k2(const QmmArgs& a, uint32_t group_size, uint32_t tile_rows, hipStream_t s) {
-  if (tile_rows != 64 && !(tile_rows == 128 && qmm_k2_tall_supported(group_size, a.bits, a.x_dtype == RMLX_DTYPE_BF16)))
+  if (tile_rows != 64 && tile_rows != 32 && !(tile_rows == 128 && qmm_k2_tall_supported(group_size, a.bits, a.x_dtype == RMLX_DTYPE_BF16)))
     return fail(RMLX_INVALID_SHAPE, "qmm: no K-split kernel with %u-row tiles for bits=%u group_size=%u (%s activations)", tile_rows,
                 a.bits, group_size, a.x_dtype == RMLX_DTYPE_BF16 ? "bf16" : "f16");
   if (!qmm_k2_supported(a.N, a.K, group_size, a.bits))
@@ -435,9 +437,10 @@ int32_t launch_qmm_k2(const QmmArgs& a, uint32_t group_size, uint32_t tile_rows,
   const dim3 grid(p.tiles_m * p.tiles_n), block(kThreads);
   const bool xb = a.x_dtype == RMLX_DTYPE_BF16, tall = tile_rows == 128;
   const bool sb_lds = group_size == 64 && !tall && a.K <= 4096;
+  const bool low = tile_rows == 32;
   auto launch = [&](auto bits_c, auto gs_c, auto mfr_c) {
     constexpr int B = decltype(bits_c)::value, GSV = decltype(gs_c)::value, MFRV = decltype(mfr_c)::value;
-    if constexpr (GSV == 64 && MFRV == 2) {
+    if constexpr (GSV == 64 && MFRV <= 2) {
       if (sb_lds) {
         if (xb) hipLaunchKernelGGL((qmm_k2_kernel<B, true, GSV, MFRV, true>), grid, block, 0, s, p);
         else hipLaunchKernelGGL((qmm_k2_kernel<B, false, GSV, MFRV, true>), grid, block, 0, s, p);
@@ -452,10 +455,15 @@ int32_t launch_qmm_k2(const QmmArgs& a, uint32_t group_size, uint32_t tile_rows,
   };
   using std::integral_constant;
   typedef integral_constant<int, 2> Low;
+  typedef integral_constant<int, 1> Flat;
   typedef integral_constant<int, 4> Tall;
   typedef integral_constant<int, 4> B4;
   typedef integral_constant<int, 8> B8;
-  auto by_height = [&](auto bits_c, auto gs_c) { if (tall) launch(bits_c, gs_c, Tall{}); else launch(bits_c, gs_c, Low{}); };
+  auto by_height = [&](auto bits_c, auto gs_c) {
+    if (tall) launch(bits_c, gs_c, Tall{});
+    else if (low) launch(bits_c, gs_c, Flat{});
+    else launch(bits_c, gs_c, Low{});
+  };
   auto by_group = [&](auto bits_c) {
     if (group_size == 64) by_height(bits_c, integral_constant<int, 64>{});
     else if (group_size == 128) by_height(bits_c, integral_constant<int, 128>{});

@@ -543,6 +543,12 @@ RwPlan plan_rw(uint32_t M, uint32_t N, uint32_t K, uint32_t group_size) {
 }
 }  // namespace
 
+uint32_t qmm_rw_tile_work(uint32_t M, uint32_t N, uint32_t K, uint32_t group_size, uint32_t bits) {
+  if (M == 0 || !qmm_rw_supported(N, K, group_size, bits)) return 0;
+  const RwPlan r = plan_rw(M, N, K, group_size);
+  return (uint32_t)(r.mf * r.nf * r.nw);
+}
+
 size_t qmm_rw_workspace_bytes(uint32_t M, uint32_t N, uint32_t K, uint32_t group_size, uint32_t bits) {
   if (M == 0 || !qmm_rw_supported(N, K, group_size, bits)) return 0;
   const RwPlan r = plan_rw(M, N, K, group_size);

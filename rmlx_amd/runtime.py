@@ -15,7 +15,7 @@ LIB_PATH = os.path.join(_HERE, "lib", "librmlx_hip.so")
 OK, INVALID_SHAPE, NOT_FOUND, RUNTIME_ERROR = 0, 1, 2, 3
 F32, F16, BF16, U32, U8 = 0, 1, 2, 3, 4
 KERNEL_AUTO, KERNEL_QMV, KERNEL_QMM, KERNEL_GENERIC, KERNEL_QMM_BF16, KERNEL_QMM_LDS, KERNEL_QMV_ROWS = 0, 1, 2, 3, 4, 5, 6
-KERNEL_QMM_K2, KERNEL_QMM_RW, KERNEL_QMM_K2_TALL = 7, 8, 9
+KERNEL_QMM_K2, KERNEL_QMM_RW, KERNEL_QMM_K2_TALL, KERNEL_QMM_K2_FLAT = 7, 8, 9, 10
 GATHER_AUTO, GATHER_STREAM, GATHER_GEMM, GATHER_PORTABLE = 0, 1, 2, 3  # rmlx_hip_gather_qmm_select kernels
 FLOOR_EMPTY, FLOOR_READ4, FLOOR_READ8, FLOOR_MFMA, FLOOR_READ2, FLOOR_MFMA_VALU, FLOOR_LDS, FLOOR_L2_READ = 0, 1, 2, 3, 4, 5, 6, 7  # rmlx_hip_measure_floor kinds
 

@@ -745,6 +745,48 @@ def test_k_split_gemm_tall_tiles(hip, bits, gs, m, n, k, dtype):
     assert np.array_equal(out, _run(hip, words, s, b, x, bits, dtype=dtype, gs=gs, kernel=rt.KERNEL_QMM_K2))
 
 
+@pytest.mark.parametrize("bits,gs", [(4, 64), (4, 32), (4, 128), (8, 64), (8, 32), (8, 128)])
+@pytest.mark.parametrize("m,n,k,dtype", [(32, 128, 512, "f16"), (45, 256, 1024, "f16"), (160, 512, 1536, "bf16"), (1, 128, 512, "f16"),
+                                         (97, 384, 2048, "f32"), (64, 128, 8192, "f16")])
+def test_k_split_gemm_flat_tiles(hip, bits, gs, m, n, k, dtype):
+    """The same kernel with 32 x 128 tiles (kernel selector 10: one activation fragment per wave): every bit width and
+    group size, ragged M, all activation dtypes; bit-identical to the 64-row tiles."""
+    from rmlx_amd import runtime as rt
+    rng = np.random.default_rng(bits * 1000 + gs + m + n + k + 2)
+    words, s, b = make_weight(rng, n, k, bits, gs)
+    x = make_x(rng, m, k, dtype)
+    ref = model.qmm(x_as_f64(x, dtype), words, s, b, gs, bits)
+    out = _run(hip, words, s, b, x, bits, dtype=dtype, gs=gs, kernel=rt.KERNEL_QMM_K2_FLAT)
+    assert_close(out, ref, f"k-split gemm, 32-row tiles M={m} N={n} K={k} bits={bits} gs={gs} {dtype}")
+    assert np.array_equal(out, _run(hip, words, s, b, x, bits, dtype=dtype, gs=gs, kernel=rt.KERNEL_QMM_K2))
+
+
+def test_k_split_gemm_flat_tiles_epilogues_and_dispatch(hip):
+    """The fused epilogues on the 32-row tiles and a shape the ladder sends there (one round of 32 x 128 tiles where the
+    register-weights GEMM would need tiles larger than 32 x 64)."""
+    from rmlx_amd import ops, runtime as rt
+    from rmlx_amd.runtime import DeviceBuffer
+    rng = np.random.default_rng(99)
+    cus = rt.device_info()["compute_units"]
+    n, k = 2048, 1024
+    m = 32 * (cus // (n // 128)) - 5  # as many 32 x 128 tiles as fit one round; more 32 x 64 tiles than CUs
+    words, s, b = make_weight(rng, n, k, 4)
+    x = make_x(rng, m, k)
+    base = model.qmm(x_as_f64(x, "f16"), words, s, b, 64, 4)
+    auto = _run(hip, words, s, b, x, 4)
+    assert_close(auto, base, "auto")
+    assert np.array_equal(auto, _run(hip, words, s, b, x, 4, kernel=rt.KERNEL_QMM_K2_FLAT))
+    qw = ops.QuantizedWeight.from_numpy(words, s, b, 64, 4)
+    xd = DeviceBuffer.from_numpy(x)
+    for edtype in (np.float16, np.float32):
+        e = rng.standard_normal((m, n)).astype(edtype)
+        ed = DeviceBuffer.from_numpy(e)
+        assert_close(ops.qmm_add_residual(xd, qw, ed).numpy(), base + e.astype(np.float64), "qmm_add_residual")
+        assert_close(ops.qmm_swiglu(xd, qw, ed).numpy(), model.silu(e.astype(np.float64)) * base, "qmm_swiglu")
+    with pytest.raises(ops.KernelError, match="register-weights qmm kernels require"):
+        _run(hip, *make_weight(rng, 64, 512, 4, 64), make_x(rng, 8, 512), 4, kernel=rt.KERNEL_QMM_K2_FLAT)  # N % 128 != 0
+
+
 def test_k_split_gemm_tall_tiles_positions_epilogues_and_dispatch(hip):
     """One-hot rows against per-group scales (every fragment, lane half, k step, k half and scale word of the 128-row
     tile); the fused epilogues; the shapes the ladder sends to the 128-row tiles; shapes it does not take."""
@@ -847,7 +889,8 @@ def test_random_shapes_through_the_ladder(hip):
 
 
 LADDER_SHAPES = [(4096, 14336, 4, (3, 9, 16)), (2048, 16384, 4, (5, 16)), (4096, 8192, 4, (9, 16)), (12288, 4096, 4, (9, 24)),
-                 (28672, 4096, 4, (8, 16, 100)), (12288, 4096, 8, (9, 16, 32))]
+                 (28672, 4096, 4, (8, 16, 100)), (12288, 4096, 8, (9, 16, 32)), (4096, 4096, 4, (128, 160, 256)),
+                 (9216, 4096, 4, (64, 128)), (4096, 4096, 8, (128, 192))]
 
 
 @pytest.mark.parametrize("n,k,bits,ms", LADDER_SHAPES)
@@ -864,7 +907,7 @@ def test_ladder_picks_within_15_percent_of_the_fastest_family(hip, n, k, bits, m
            for i in range(n_sets)]
     stream, e0, e1 = rt.Stream(), rt.Event(), rt.Event()
     families = {"auto": rt.KERNEL_AUTO, "qmv": rt.KERNEL_QMV_ROWS, "qmm": rt.KERNEL_QMM, "k2": rt.KERNEL_QMM_K2,
-                "rw": rt.KERNEL_QMM_RW, "k2_tall": rt.KERNEL_QMM_K2_TALL}
+                "rw": rt.KERNEL_QMM_RW, "k2_tall": rt.KERNEL_QMM_K2_TALL, "k2_flat": rt.KERNEL_QMM_K2_FLAT}
 
     def train_us(xd, outs, kernel, count=300):
         e0.record(stream)
