@@ -151,14 +151,17 @@ int32_t rmlx_hip_affine_quantized_matmul_batched(const rmlx_qweight* qw, const r
 /* Same contract as the batched entry point but forces one kernel family (the reference
  * exposes its kernels individually too, e.g. `affine_qmv_batched_f16_q4` quantized.rs:1675,
  * `affine_quantized_matmul_nax` :8517).  kernel: 0 = auto, 1 = streaming GEMV (qmv: the
- * single-row kernel where it applies -- M <= 2, or M <= 16 at group sizes 32 / 128 -- else the multi-row one),
+ * single-row kernel where it applies -- M <= 2, or M <= 16 at group size 32, of which the automatic choice keeps M <= 4
+ * where the MFMA GEMM takes the shape -- else the multi-row one),
  * 2 = MFMA GEMM (qmm, f16 MFMA; bf16 activations are converted, which is exact for
  * normal-range values; the register-weights kernel when K % 512 == 0, else the LDS-staged one),
  * 3 = portable scalar kernel (any bits/group size the type admits),
  * 4 = LDS-staged MFMA GEMM on the bf16 matrix instruction (Q8 weights and bf16 activations
  * only; weights are rounded to bf16, so its error is about four times that of kernel 2),
  * 5 = LDS-staged MFMA GEMM (f16 MFMA, K % 256 == 0),
- * 6 = multi-row streaming GEMV also for a single row (group sizes 64 and 128),
+ * 6 = multi-row streaming GEMV also for a single row (group sizes 64 and 128; 4-bit weights at group size 32 with
+ * K % 512 == 0 and K <= 4096 on the wave-per-tile form, which the automatic choice takes for 3 to 8 rows over matrices
+ * of 24576 rows or more),
  * 7 = K-split MFMA GEMM (64 x 128 tiles, 32x32x16 MFMAs; N % 128 == 0, K % 512 == 0; what kernel 2 resolves to
  * when that grid is one round over most of the chip), 8 = the register-weights GEMM whatever the shape,
  * 9 = the K-split MFMA GEMM with 128 x 128 tiles (not for 8-bit weights at group size 32 / 64 with bf16 activations; what

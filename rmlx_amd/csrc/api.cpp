@@ -164,6 +164,10 @@ bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) ==
 enum { KERNEL_AUTO = 0, KERNEL_QMV = 1, KERNEL_QMM = 2, KERNEL_GENERIC = 3, KERNEL_QMM_BF16 = 4, KERNEL_QMM_LDS = 5,
        KERNEL_QMV_ROWS = 6, KERNEL_QMM_K2 = 7, KERNEL_QMM_RW = 8, KERNEL_QMM_K2_TALL = 9, KERNEL_QMM_K2_FLAT = 10 };
 constexpr uint32_t kQmvMaxM = 16;
+// 4-bit weights at group size 32: weight rows from which the wave-per-tile kernel has the tiles to fill the chip
+constexpr uint32_t kWt32MinN = 24576;
+// rows of one pass of the single-row kernel
+constexpr uint32_t kM1PassRows = 4;
 // group size 64: rows taken by the single-row kernel (measured: 3 and 4 rows are faster on the matrix unit)
 constexpr uint32_t kM1MaxRows = 2;
 constexpr uint32_t kM1MaxRowsOther = 16;  // shapes the multi-row GEMV does not take: the alternative is the portable kernel
@@ -204,6 +208,8 @@ int32_t run_matmul_plain(const rmlx_qweight* qw, const void* x, int32_t x_dtype,
                       M <= (can_qmv ? kM1MaxRows : kM1MaxRowsOther);
   // 2-bit weights: the single-row kernel of their own, up to 16 rows in passes of one (the alternative is the portable kernel)
   const bool can_q2 = ptr_ok && qw->bits == 2 && M <= kM1MaxRowsOther && qmv_q2_supported(N, K, qw->group_size);
+  // 4-bit weights at group size 32: the wave-per-tile kernel streams the weights once per 8 rows
+  const bool can_wt32 = ptr_ok && qw->bits == 4 && qw->group_size == 32 && qmv_wt_supported(N, K, 32, 8);
   const bool can_qmm_lds = ptr_ok && qmm_supported(N, K, qw->group_size, qw->bits);
   const bool can_qmm_rw = ptr_ok && qmm_rw_supported(N, K, qw->group_size, qw->bits);
   const bool can_qmm = can_qmm_lds || can_qmm_rw;
@@ -227,11 +233,19 @@ int32_t run_matmul_plain(const rmlx_qweight* qw, const void* x, int32_t x_dtype,
     const bool small_m = !can_qmm_rw ? M <= kQmvMaxM || (qw->bits == 4 && (uint64_t)((M + 7) / 8) * wbytes <= (48ull << 20))
                          : qw->bits == 4 ? M <= 8 || (M <= kQmvMaxM && (wbytes <= (12ull << 20) || N <= 8192))
                                          : (M <= kQmvMaxM && wbytes < (48ull << 20));
-    if ((can_qmv && small_m) || can_m1 || can_q2) kernel = KERNEL_QMV;
+    // Shapes the K-split GEMV does not take (group size 32) run up to 16 rows on the single-row kernel in passes of four,
+    // which streams the weights once per pass: with the register-weights GEMM as the alternative it keeps up to 4 rows
+    // (4096 x 4096, 4-bit, group 32: 8.8 against 10.8 us at 4 rows, 11.4 against 11.1 at 8, 17.0 against 11.1 at 16;
+    // 8-bit: 7.4 / 11.4, 12.6 / 11.4, 19.8 / 11.7; N = 9216, 8-bit: 14.2 / 20.6, 23.0 / 20.6, 36.8 / 21.2).  Over very
+    // wide matrices the wave-per-tile kernel has enough tiles to fill the chip and takes 3 to 8 rows (N = 28672, 4-bit,
+    // group 32: 22.8 us against 26.9 on the single-row kernel and 25.1 on the GEMM; N = 16384: 21.4 against 17.6 on the GEMM).
+    const bool m1_first = can_m1 && (can_qmv || !can_qmm_rw || M <= kM1PassRows);
+    if (can_wt32 && N >= kWt32MinN && M >= 3 && M <= 8) kernel = KERNEL_QMV_ROWS;
+    else if ((can_qmv && small_m) || m1_first || can_q2) kernel = KERNEL_QMV;
     else if (can_qmm) kernel = KERNEL_QMM;
     else if (can_qmv) kernel = KERNEL_QMV;
     else kernel = KERNEL_GENERIC;
-  } else if ((kernel == KERNEL_QMV && !can_qmv && !can_m1 && !can_q2) || (kernel == KERNEL_QMV_ROWS && !can_qmv)) {
+  } else if ((kernel == KERNEL_QMV && !can_qmv && !can_m1 && !can_q2) || (kernel == KERNEL_QMV_ROWS && !can_qmv && !can_wt32)) {
     return fail(RMLX_INVALID_SHAPE,
                 "qmv kernel requires bits in {4,8}, group_size 64 (4-bit: or 128), N %% 16 == 0, K %% 512 == 0 (4-bit) or "
                 "K %% 256 == 0 (8-bit) and 16-byte aligned buffers (N=%u K=%u bits=%u group_size=%u)",
@@ -361,6 +375,14 @@ int32_t run_matmul_plain(const rmlx_qweight* qw, const void* x, int32_t x_dtype,
     *epi_done = true;
     return launch_qmv_m1(qw->w, qw->s, qw->b, static_cast<const __half*>(xk), out, M, N, K, qw->group_size, qw->bits,
                          epi.kind, epi.ptr, epi.dtype, norm_w, norm_w != nullptr ? inv_rms : nullptr, stream);
+  }
+  if (kernel == KERNEL_QMV_ROWS && can_wt32) {
+    QmvArgs a{};
+    a.w0 = qw->w; a.s0 = qw->s; a.b0 = qw->b;
+    a.N = N; a.K = K;
+    a.x = static_cast<const __half*>(xk);
+    a.out = out; a.ld_out = N; a.M = M; a.group_size = 32;
+    return launch_qmv_wt(a, 8, stream);
   }
   if (kernel == KERNEL_QMV_ROWS) kernel = KERNEL_QMV;
   if (kernel == KERNEL_QMV && qw->bits == 8)

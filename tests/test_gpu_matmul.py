@@ -937,6 +937,21 @@ def test_ladder_picks_within_15_percent_of_the_fastest_family(hip, n, k, bits, m
         assert times["auto"] <= 1.15 * best, (m, times)
 
 
+@pytest.mark.parametrize("m", [1, 3, 8, 11, 16])
+@pytest.mark.parametrize("n,k", [(48, 512), (512, 4096), (24576, 512)])
+def test_q4_group_32_on_the_wave_per_tile_gemv(hip, n, k, m):
+    """4-bit weights at group size 32 on the multi-row streaming GEMV (kernel selector 6: a wave per 16-row weight tile,
+    two matrix-instruction chains per slab), forced and through the ladder (which takes it for 3 to 8 rows over very wide
+    matrices, the single-row kernel up to 4 rows and the GEMM above), against the oracle."""
+    from rmlx_amd import runtime as rt
+    rng = np.random.default_rng(n + k + m + 32)
+    words, s, b = make_weight(rng, n, k, 4, 32)
+    x = make_x(rng, m, k)
+    ref = model.qmm(x.astype(np.float64), words, s, b, 32, 4)
+    assert_close(_run(hip, words, s, b, x, 4, gs=32, kernel=rt.KERNEL_QMV_ROWS), ref, f"Q4 gs32 M={m} N={n} K={k} (wave per tile)")
+    assert_close(_run(hip, words, s, b, x, 4, gs=32), ref, f"Q4 gs32 M={m} N={n} K={k} (auto)")
+
+
 @pytest.mark.parametrize("m", [3, 8, 16])
 @pytest.mark.parametrize("n,k", [(512, 1024), (1024, 4096)])
 def test_q8_group_128_on_the_streaming_gemv(hip, n, k, m):
