@@ -174,6 +174,7 @@ class QuantizedWeight {
   QuantizedWeight& operator=(const QuantizedWeight&) = delete;
   const rmlx_qweight* handle() const { return handle_; }
   uint32_t set_expert_gemm_min_rows(uint32_t min_rows) const { return rmlx_hip_qweight_set_expert_gemm_min_rows(handle_, min_rows); }
+  uint32_t set_expert_stream_kernel(uint32_t kind) const { return rmlx_hip_qweight_set_expert_stream_kernel(handle_, kind); }
 
   std::shared_ptr<Buffer> weights_buf, scales_buf, biases_buf;
   uint32_t group_size, bits;
@@ -391,6 +392,9 @@ class MoeExperts {
   // of the streaming GEMV; 0 = never.  Kept in the gate weight's handle (so an ExpertGroup over the same weights
   // follows it); returns the previous value.
   uint32_t set_expert_gemm_min_rows(uint32_t min_rows) { return gate_->set_expert_gemm_min_rows(min_rows); }
+  // Streaming kernel of decode-sized batches (0 = the library's choice; see rmlx_hip_qweight_set_expert_stream_kernel);
+  // returns the previous value.
+  uint32_t set_expert_stream_kernel(uint32_t kind) { return gate_->set_expert_stream_kernel(kind); }
   // routing included: gate_logits [T, E]
   Array forward(const Array& x, const Array& gate_logits, size_t top_k, const Array* expert_bias = nullptr,
                 const Stream* stream = nullptr) const {

@@ -1,5 +1,6 @@
-// Wave-per-tile streaming GEMV for stacked 4-bit expert weights on gfx950: the expert projections of
-// decode-sized MoE batches and gather_qmm (chunks of at most 8 or 16 rows of one expert).
+// Wave-per-tile streaming GEMV for 4-bit weights on gfx950: the expert projections of decode-sized MoE
+// batches and gather_qmm over stacked weights (chunks of at most 8 or 16 rows of one expert), and dense
+// matrices at group size 32 (chunks of 8 rows of the [M, K] activations).
 //
 // Replaces the reference's gather_qmv_fast_f16_q4 / moe_expert_matmul_q4
 // (crates/rmlx-core/src/ops/quantized.rs:9752-9842, 10257-10370).
@@ -7,7 +8,7 @@
 // The K-split kernel of qmv.hip lets eight waves share one 16-row weight tile and meet in a reduction
 // through LDS after every tile: two barriers per tile, during which a workgroup has no loads in flight.
 // Here a wave owns a whole tile (16 weight rows, all of K; fused gate / up: the same rows of both
-// matrices) and walks it in passes of four 128-k slabs with the next pass already requested into a
+// matrices) and walks it in passes of two or four 128-k slabs with the next pass already requested into a
 // second register set - across tile boundaries too - so a wave always has loads in flight and never
 // waits for another wave: after the activations are staged there is no barrier at all.
 //   * The workgroup stages the chunk's activations once, for all of K, into one LDS image in the
@@ -20,6 +21,8 @@
 //     groups of a slab, accumulators started from -sum(off*x), F += scale * c + bias * sum(x).
 //   * Weight addresses are a buffer resource per matrix (the expert's base, in scalar registers), one
 //     32-bit offset per lane and a wave-uniform offset per tile and slab.
+#include <type_traits>
+
 #include "common.hpp"
 #include "q4_stream.hpp"
 
@@ -106,8 +109,8 @@ __global__ __launch_bounds__(NW * 64, NW == 8 && RH == 1 ? 4 : 1) void qmv_wt_ke
     uint32_t sb[TILES][kSbWords];  // word it * GC + c: the two groups of chain c of slab `it` (scales or biases, by lane)
   };
   // the loads of pass `pass` of tile `tile` (wave-uniform): scales / biases first, the memory counter retires in order
-  // Waves start at different passes of their tiles (and wrap around): at any moment the waves of the chip then read
-  // different column ranges of their rows, i.e. different memory channels, instead of the same 256 bytes of every row.
+  // Waves start at different passes of their tiles (and wrap around), so that the waves of the chip do not all read the
+  // same column range of their rows at the same moment (measured: within 1 % of starting every tile at pass 0).
   const uint32_t skew = (wave * 5 + blockIdx.x * 3 + blockIdx.y) % NP;
   auto load_step = [&](uint32_t tile, uint32_t pass_i, Set& st) {
     const uint32_t pass = pass_i + skew < NP ? pass_i + skew : pass_i + skew - NP;
@@ -213,10 +216,12 @@ __global__ __launch_bounds__(NW * 64, NW == 8 && RH == 1 ? 4 : 1) void qmv_wt_ke
   };
   f4 F[RH][TILES];
   uint32_t c_tile = first + wave, c_pass = 0;  // cursor of the pass being multiplied
-  auto compute_step = [&](const Set& st) {
+  // H = 8-row halves that hold rows (wave-uniform: a chunk of at most 8 rows skips the second image)
+  auto compute_halves = [&](const Set& st, auto hc) {
+    constexpr int H = decltype(hc)::value;
     if (c_pass == 0) {
 #pragma unroll
-      for (int h = 0; h < RH; ++h)
+      for (int h = 0; h < H; ++h)
 #pragma unroll
         for (int t = 0; t < TILES; ++t) F[h][t] = (f4){0.f, 0.f, 0.f, 0.f};
     }
@@ -233,10 +238,10 @@ __global__ __launch_bounds__(NW * 64, NW == 8 && RH == 1 ? 4 : 1) void qmv_wt_ke
 #pragma unroll
     for (int it = 0; it < kPass; ++it) {
       const uint32_t slab = slab0 + it;
-      f4 c[RH][GC][TILES];
-      f4 xsum[RH][GC];
+      f4 c[H][GC][TILES];
+      f4 xsum[H][GC];
 #pragma unroll
-      for (int h = 0; h < RH; ++h)
+      for (int h = 0; h < H; ++h)
 #pragma unroll
         for (int ch = 0; ch < GC; ++ch) {
           const float* sp = sums_all + ((((h * S + slab) * GC + ch) * 2 + par) * 2 + (g & 1)) * 8;
@@ -254,7 +259,7 @@ __global__ __launch_bounds__(NW * 64, NW == 8 && RH == 1 ? 4 : 1) void qmv_wt_ke
           bw[t] = unpack_q4_word(wd, qc);
         }
 #pragma unroll
-        for (int h = 0; h < RH; ++h)
+        for (int h = 0; h < H; ++h)
 #pragma unroll
           for (int ch = 0; ch < GC; ++ch) {
             const h8 av = *reinterpret_cast<const h8*>(smem + h * img_half + ((slab * 4 + j) * kBlk) * 16 + a_slot_off[ch]);
@@ -268,7 +273,7 @@ __global__ __launch_bounds__(NW * 64, NW == 8 && RH == 1 ? 4 : 1) void qmv_wt_ke
         for (int ch = 0; ch < GC; ++ch) {
           const float sc = half_at(sv[t], it * GC + ch), bi = half_at(bv[t], it * GC + ch);
 #pragma unroll
-          for (int h = 0; h < RH; ++h)
+          for (int h = 0; h < H; ++h)
 #pragma unroll
             for (int i = 0; i < 4; ++i) F[h][t][i] = fmaf(sc, c[h][ch][t][i], fmaf(bi, xsum[h][ch][i], F[h][t][i]));
         }
@@ -277,7 +282,7 @@ __global__ __launch_bounds__(NW * 64, NW == 8 && RH == 1 ? 4 : 1) void qmv_wt_ke
       // the tile is complete: add the two group halves (lane ^ 32), lanes with g < 2 write rows 4g .. 4g+3, column n
       const uint32_t col = c_tile * 16 + n;
 #pragma unroll
-      for (int h = 0; h < RH; ++h)
+      for (int h = 0; h < H; ++h)
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
           float v[TILES];
@@ -294,6 +299,15 @@ __global__ __launch_bounds__(NW * 64, NW == 8 && RH == 1 ? 4 : 1) void qmv_wt_ke
         }
     }
     advance(c_tile, c_pass);
+  };
+  // (the fused gate / up kernel only: it runs eight waves and has the registers for both forms; in the plain 16-wave
+  // kernel the second form spills)
+  const bool one_half = RH == 2 && DUAL && rows <= 8;
+  auto compute_step = [&](const Set& st) {
+    if constexpr (RH == 2 && DUAL) {
+      if (one_half) { compute_halves(st, std::integral_constant<int, 1>{}); return; }
+    }
+    compute_halves(st, std::integral_constant<int, RH>{});
   };
 
 #pragma unroll
