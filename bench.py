@@ -518,14 +518,15 @@ def main():
             # The routed block at 6 / 8 / 10 rows per expert with every choice of expert kernels (for kernel traces:
             # which projection costs what under which kernel).  (label, GEMM threshold, streaming kernel selector)
             variants = (("kplit_8row_chunks", 0, 1), ("wave_per_tile_8row_chunks", 0, 2), ("wave_per_tile_16row_chunks", 0, 3),
-                        ("hybrid_kplit_gate_up_wave_down", 0, 4), ("grouped_gemm", 1, 0))
+                        ("hybrid_kplit_gate_up_wave_down", 0, 4), ("grouped_gemm", 1, 0), ("library_choice", None, 0))
             for T in (96, 128, 160):
                 for label, min_rows, kind in variants:
                     # (a threshold of 1 forces the GEMM; its tile height follows the average rows per expert: 16-row tiles
                     # at T = 96, 32-row tiles at T = 128 and 160)
                     # (an empty marker kernel in front of every measurement: a kernel trace is split at these)
                     rt.check(rt.lib().rmlx_hip_measure_floor(rt.FLOOR_EMPTY, None, 0, 0, 0, None, 1, timer.stream.handle))
-                    prev_rows = experts[2].set_expert_gemm_min_rows(min_rows)
+                    prev_rows = experts[2].set_expert_gemm_min_rows(0)
+                    experts[2].set_expert_gemm_min_rows(prev_rows if min_rows is None else min_rows)
                     prev_kind = experts[2].set_expert_stream_kernel(kind)
                     try:
                         r = bench_moe(ops, rt, timer, rng, T, max(100, calls // 2), experts)

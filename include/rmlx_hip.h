@@ -165,7 +165,7 @@ int32_t rmlx_hip_affine_quantized_matmul_batched(const rmlx_qweight* qw, const r
  * 7 = K-split MFMA GEMM (64 x 128 tiles, 32x32x16 MFMAs; N % 128 == 0, K % 512 == 0; what kernel 2 resolves to
  * when that grid is one round over most of the chip), 8 = the register-weights GEMM whatever the shape,
  * 9 = the K-split MFMA GEMM with 128 x 128 tiles (not for 8-bit weights at group size 32 / 64 with bf16 activations; what
- * kernel 2 resolves to when those tiles make 0.6 rounds over the chip or more), 10 = the K-split MFMA GEMM with 32 x 128
+ * kernel 2 resolves to when those tiles make 0.55 rounds over the chip or more), 10 = the K-split MFMA GEMM with 32 x 128
  * tiles (what kernel 2 resolves to when those tiles make at most one round over the chip and the register-weights GEMM
  * would need more than one round of its 32 x 64 tiles; K <= 4096). */
 int32_t rmlx_hip_qmm_select(const rmlx_qweight* qw, const rmlx_array* x, int32_t kernel,

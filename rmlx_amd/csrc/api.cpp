@@ -275,10 +275,10 @@ int32_t run_matmul_plain(const rmlx_qweight* qw, const void* x, int32_t x_dtype,
   }
   // The K-split GEMM (32x32x16 MFMAs, K split inside the workgroup).  64 x 128 tiles where that grid is one round over
   // most of the chip: measured 23.8 against 25.4 us at M = 512, 4096 x 4096 and 27.8 against 28.8 us at M = 128,
-  // N = 12288 (8-bit).  128 x 128 tiles (every unpacked weight operand feeds four MFMAs) from 0.6 rounds of those on:
+  // N = 12288 (8-bit).  128 x 128 tiles (every unpacked weight operand feeds four MFMAs) from 0.55 rounds of those on:
   // 29.6 against 35.5 us at M = 640, 37.0 against 41.4 us at M = 1024, 153 against 175 us at M = 4096 (4096 x 4096), 30.9
-  // against 37.8 us at M = 192, N = 12288.  With fewer tiles the smaller tiles of the register-weights GEMM keep more
-  // CUs busy.
+  // against 37.8 us at M = 192, N = 12288, 31.3 against 36.5 us at M = 256, N = 9216 (144 tiles).  With fewer tiles the
+  // smaller tiles of the register-weights GEMM keep more CUs busy.
   uint32_t k2_tile_rows = kernel == KERNEL_QMM_K2_TALL ? 128 : kernel == KERNEL_QMM_K2_FLAT ? 32 : 64;
   if (kernel == KERNEL_QMM && can_qmm_k2) {
     const uint64_t tiles = (uint64_t)((M + 63) / 64) * (N / 128), tall = (uint64_t)((M + 127) / 128) * (N / 128);
@@ -287,7 +287,7 @@ int32_t run_matmul_plain(const rmlx_qweight* qw, const void* x, int32_t x_dtype,
     // matrix measured 150 against 103 us on the register-weights GEMM, N = 151936)
     const bool fits64 = (uint64_t)((M + 63) / 64) * 64 * 3 <= (uint64_t)M * 4, fits128 = (uint64_t)((M + 127) / 128) * 128 * 3 <= (uint64_t)M * 4;
     if (fits64 && tiles * 10 >= cus * 7 && tiles <= cus) kernel = KERNEL_QMM_K2;
-    else if (fits128 && can_qmm_k2_tall && tall * 10 >= cus * 6) { kernel = KERNEL_QMM_K2; k2_tile_rows = 128; }
+    else if (fits128 && can_qmm_k2_tall && tall * 20 >= cus * 11) { kernel = KERNEL_QMM_K2; k2_tile_rows = 128; }
     // 32 x 128 tiles: one round of them takes about 18.5 us at K = 4096 whatever their number (the length of the k loop);
     // the register-weights GEMM is faster while its 32 x 64 tiles fit one round over the chip (15.6 us at M = 128,
     // 4096 x 4096) and slower once it has to take larger tiles (M = 160: 24.4 us, M = 256: 21.1 against 19.3;

@@ -35,7 +35,6 @@ struct Q8Params {
   const __half* x;
   void* out;               // f16 (f32 when out_f32)
   uint32_t K, ld_out, M, out_f32;
-  uint32_t gs128;          // quantisation group size 128 instead of 64
   // chunk-table mode (expert projections): (expert, first row position, rows <= 16) per blockIdx.y
   const uint32_t* row_map;    // nullable: source row of position p
   const uint32_t* chunk_tab;
@@ -56,12 +55,12 @@ __device__ __forceinline__ h8 bytes_to_f16_plus_1024(uint32_t w0, uint32_t w1) {
 // TAB: rows come from a device chunk table and the weights from the chunk's expert.  TILES == 2: the
 // workgroup multiplies the same activations with a gate tile and an up tile and writes silu(gate) * up.
 // A pass covers 32 slabs (2048 k); waves whose slabs lie past K sit it out, so K % 256 == 0 is enough.
-template <bool TAB, int TILES>
+template <bool TAB, int TILES, bool GS128>
 __global__ __launch_bounds__(kThreads) void qmv_q8_kernel(Q8Params p) {
   __shared__ float red[kWaves * TILES * 256];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int n = lane & 15, g = lane >> 4;  // weight row of the tile / k sub-block; also activation row n
-  const uint32_t K = p.K, slabs_total = K >> 6, groups_per_row = p.gs128 ? K >> 7 : K >> 6;
+  const uint32_t K = p.K, slabs_total = K >> 6, groups_per_row = GS128 ? K >> 7 : K >> 6;
   uint32_t expert = 0, row0 = blockIdx.y * 16, rows;
   bool write_zeros = false;
   if (TAB) {
@@ -112,7 +111,7 @@ __global__ __launch_bounds__(kThreads) void qmv_q8_kernel(Q8Params p) {
     uint2 sv[TILES], bv[TILES];
 #pragma unroll
     for (int t = 0; t < TILES; ++t) {
-      if (p.gs128) {  // two groups for the four slabs: every value twice
+      if (GS128) {  // two groups for the four slabs: every value twice
         const uint32_t s2 = *reinterpret_cast<const uint32_t*>(srow[t] + (sl >> 1)), b2 = *reinterpret_cast<const uint32_t*>(brow[t] + (sl >> 1));
         sv[t] = make_uint2(__builtin_amdgcn_perm(s2, s2, 0x01000100u), __builtin_amdgcn_perm(s2, s2, 0x03020302u));
         bv[t] = make_uint2(__builtin_amdgcn_perm(b2, b2, 0x01000100u), __builtin_amdgcn_perm(b2, b2, 0x03020302u));
@@ -198,8 +197,11 @@ int32_t launch_qmv_q8(const uint32_t* w, const __half* s, const __half* b, const
   if (M == 0) return RMLX_OK;
   Q8Params p{};
   p.w = w; p.s = s; p.b = b; p.x = x; p.out = out; p.K = K; p.ld_out = N; p.M = M;
-  p.gs128 = group_size == 128 ? 1u : 0u;
-  hipLaunchKernelGGL((qmv_q8_kernel<false, 1>), dim3(N / 16, (M + 15) / 16), dim3(kThreads), 0, stream, p);
+  // (the group size is a template parameter: as a run-time flag inside the pass loop it cost the 64-wide kernel
+  // 13 % on decode-sized expert batches)
+  const dim3 grid(N / 16, (M + 15) / 16);
+  if (group_size == 128) hipLaunchKernelGGL((qmv_q8_kernel<false, 1, true>), grid, dim3(kThreads), 0, stream, p);
+  else hipLaunchKernelGGL((qmv_q8_kernel<false, 1, false>), grid, dim3(kThreads), 0, stream, p);
   RMLX_HIP_CHECK(hipGetLastError());
   return RMLX_OK;
 }
@@ -216,10 +218,12 @@ int32_t launch_qmv_q8_tab(const QmvArgs& a, hipStream_t stream) {
   p.x = a.x; p.out = a.out; p.K = a.K; p.ld_out = a.ld_out; p.M = 0; p.out_f32 = a.out_f32;
   p.row_map = a.row_map; p.chunk_tab = a.chunk_tab; p.n_chunks = a.n_chunks_dev;
   p.estride_w = a.expert_stride_w; p.estride_s = a.expert_stride_s;
-  p.gs128 = a.group_size == 128 ? 1u : 0u;
   const dim3 grid(a.N / 16, a.max_chunks);
-  if (a.dual) hipLaunchKernelGGL((qmv_q8_kernel<true, 2>), grid, dim3(kThreads), 0, stream, p);
-  else hipLaunchKernelGGL((qmv_q8_kernel<true, 1>), grid, dim3(kThreads), 0, stream, p);
+  const bool gs128 = a.group_size == 128;
+  if (a.dual && gs128) hipLaunchKernelGGL((qmv_q8_kernel<true, 2, true>), grid, dim3(kThreads), 0, stream, p);
+  else if (a.dual) hipLaunchKernelGGL((qmv_q8_kernel<true, 2, false>), grid, dim3(kThreads), 0, stream, p);
+  else if (gs128) hipLaunchKernelGGL((qmv_q8_kernel<true, 1, true>), grid, dim3(kThreads), 0, stream, p);
+  else hipLaunchKernelGGL((qmv_q8_kernel<true, 1, false>), grid, dim3(kThreads), 0, stream, p);
   RMLX_HIP_CHECK(hipGetLastError());
   return RMLX_OK;
 }
