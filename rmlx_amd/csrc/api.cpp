@@ -1055,7 +1055,9 @@ int32_t rmlx_hip_gather_qmm_select(const rmlx_array* x, const void* w_packed_dev
   const uint32_t* w = static_cast<const uint32_t*>(w_packed_dev);
   const __half* sc = static_cast<const __half*>(scales_dev);
   const __half* bi = static_cast<const __half*>(biases_dev);
-  const bool fast = qmv_q4_supported(N32, K32, group_size) && aligned16(w) && aligned16(sc) &&
+  // group size 32 streams on the wave-per-tile kernel (chunks of 8 rows as well)
+  const bool wt32 = group_size == 32 && qmv_wt_supported(N32, K32, 32, 8);
+  const bool fast = (qmv_q4_supported(N32, K32, group_size) || wt32) && aligned16(w) && aligned16(sc) &&
                     aligned16(bi) && aligned16(xk);
   // (measured, 32 entries over 3072 x 4096 weights: 8 rows 50 us streamed; 12 / 16 / 32 rows 61 / 64 / 76 us on the GEMM
   // with 16- / 32-row tiles against 95 / 99 / 172 us streamed)
@@ -1101,7 +1103,7 @@ int32_t rmlx_hip_gather_qmm_select(const rmlx_array* x, const void* w_packed_dev
     for (uint64_t first = 0; first < n_chunks; first += 65535) {
       a.chunk_tab = static_cast<const uint32_t*>(tab.ptr) + 3 * first;
       a.max_chunks = (uint32_t)(n_chunks - first < 65535 ? n_chunks - first : 65535);
-      RMLX_TRY(launch_qmv_q4(a, s));
+      RMLX_TRY(wt32 ? launch_qmv_wt(a, 8, s) : launch_qmv_q4(a, s));
     }
   } else {
     GenericArgs g{w, sc, bi, xk, static_cast<__half*>(out_f16_dev), idx, (uint32_t)m_per_batch, rows, N32, K32,

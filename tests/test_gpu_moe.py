@@ -205,6 +205,24 @@ def test_gather_qmm_matches_oracle(hip, E, n, k, batch, mpb):
     assert np.array_equal(out32, out)
 
 
+@pytest.mark.parametrize("n,k,mpb", [(128, 1024, 1), (48, 512, 3), (256, 4096, 8), (64, 2048, 5)])
+def test_gather_qmm_group_size_32_streams_on_the_wave_per_tile_kernel(hip, n, k, mpb):
+    """Group size 32 with a few rows per entry: the wave-per-tile streaming kernel (automatic and forced) against the
+    oracle and the portable kernel."""
+    from rmlx_amd import ops, runtime as rt
+    from rmlx_amd.runtime import DeviceBuffer
+    rng = np.random.default_rng(n + k + mpb + 32)
+    E, batch = 5, 7
+    words, s, b = make_weight(rng, n, k, 4, 32, lead=(E,))
+    x = rng.standard_normal((batch, mpb, k)).astype(np.float16)
+    idx = rng.integers(0, E, size=batch).astype(np.uint32)
+    xd, wd, sd, bd, idd = [DeviceBuffer.from_numpy(a) for a in (x, words, s, b, idx)]
+    ref = model.gather_qmm(x, words, s, b, idx, 32)
+    assert_close(ops.gather_qmm(xd, wd, sd, bd, idd, batch, mpb, n, k, E, 32).numpy(), ref, "gather_qmm gs32 (auto)")
+    assert_close(ops.gather_qmm(xd, wd, sd, bd, idd, batch, mpb, n, k, E, 32, kernel=rt.GATHER_STREAM).numpy(), ref, "gather_qmm gs32 (streaming)")
+    assert_close(ops.gather_qmm(xd, wd, sd, bd, idd, batch, mpb, n, k, E, 32, kernel=rt.GATHER_PORTABLE).numpy(), ref, "gather_qmm gs32 (portable)")
+
+
 def test_gather_qmm_validation(hip):
     """The reference's argument-validation tests (quantized.rs:11088-11540)."""
     from rmlx_amd import ops
@@ -280,7 +298,7 @@ def test_gather_qmm_many_rows_per_entry_on_the_grouped_gemm(hip, n, k, mpb, gs):
     out = ops.gather_qmm(xd, wd, sd, bd, DeviceBuffer.from_numpy(idx), batch, mpb, n, k, E, gs).numpy()
     ref = model.gather_qmm(x, words, s, b, idx, gs)
     assert_close(out, ref, "gather_qmm (GEMM)")
-    if gs != 32:  # (the streaming GEMV takes group sizes 64 and 128)
+    if True:  # (group sizes 64 and 128 on the K-split streaming GEMV, 32 on the wave-per-tile one)
         out_stream = ops.gather_qmm(xd, wd, sd, bd, DeviceBuffer.from_numpy(idx), batch, mpb, n, k, E, gs, kernel=rt.GATHER_STREAM).numpy()
         assert_close(out_stream, ref, "gather_qmm (streaming GEMV)")
     out_port = ops.gather_qmm(xd, wd, sd, bd, DeviceBuffer.from_numpy(idx), batch, mpb, n, k, E, gs, kernel=rt.GATHER_PORTABLE).numpy()
