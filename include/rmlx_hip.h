@@ -167,7 +167,8 @@ int32_t rmlx_hip_affine_quantized_matmul_batched(const rmlx_qweight* qw, const r
  * 9 = the K-split MFMA GEMM with 128 x 128 tiles (not for 8-bit weights at group size 32 / 64 with bf16 activations; what
  * kernel 2 resolves to when those tiles make 0.55 rounds over the chip or more), 10 = the K-split MFMA GEMM with 32 x 128
  * tiles (what kernel 2 resolves to when those tiles make at most one round over the chip and the register-weights GEMM
- * would need more than one round of its 32 x 64 tiles; K <= 4096). */
+ * would need more than one round of its 32 x 64 tiles; K <= 4096), 11 = the MFMA GEMM with 32 x 64 tiles and K split four
+ * ways inside the workgroup (4-bit weights at group size 64, N % 64 == 0, K % 2048 == 0). */
 int32_t rmlx_hip_qmm_select(const rmlx_qweight* qw, const rmlx_array* x, int32_t kernel,
                             void* out_f16_dev, size_t out_bytes, rmlx_stream stream);
 
@@ -311,6 +312,16 @@ int32_t rmlx_hip_moe_forward_grouped(const rmlx_qweight* gate, const rmlx_qweigh
  * is no process-wide state.  Set it before other threads use the handle.  The counterpart of choosing a
  * `MoeStrategy` for a layer in the reference (crates/rmlx-nn/src/moe.rs:515-541).  Returns the previous value. */
 uint32_t rmlx_hip_qweight_set_expert_gemm_min_rows(rmlx_qweight* gate_qw, uint32_t min_rows);
+/* Optional second copy of a weight matrix in the order the K-split MFMA GEMMs (kernels 7, 9, 10, 11) load it: per 128
+ * weight rows and 128-wide k block the 8 KB (8-bit: 16 KB) of the tile as consecutive 1 KB wave loads, instead of 32 bytes
+ * of each of 32 rows per load.  The MLX layout stays the input and stays in use by every other kernel; the caller owns
+ * `dst_dev` (`rmlx_hip_qweight_gemm_layout_bytes(qw)` bytes = the size of the weight buffer, 16-byte aligned; 0 = the
+ * weight has no such layout: 4- or 8-bit, out_features % 128 == 0, in_features % 512 == 0, one expert) and keeps it
+ * alive while the handle uses it; `dst_dev == NULL` drops it again.  The copy is made on `stream` (NULL: before the call
+ * returns).  Results are bit-identical with and without it.  The counterpart of the reference repacking weights at load
+ * time (crates/rmlx-nn/src/safetensors_loader.rs:562-628).  Set it before other threads use the handle. */
+size_t rmlx_hip_qweight_gemm_layout_bytes(const rmlx_qweight* qw);
+int32_t rmlx_hip_qweight_set_gemm_layout(rmlx_qweight* qw, void* dst_dev, size_t dst_bytes, rmlx_stream stream);
 /* Which streaming kernel runs the expert projections of decode-sized batches (below the grouped GEMM's threshold) of a
  * block whose gate weight is `qw`: 1 = K split over the waves of a workgroup, chunks of 8 rows, 2 = a wave per 16-row
  * weight tile, chunks of 8 rows, 3 = a wave per tile, chunks of 16 rows, 4 = kernel 1 for the gate / up projection and

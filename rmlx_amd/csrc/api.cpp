@@ -162,7 +162,7 @@ bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) ==
 // register-weights MFMA GEMM above (the LDS-staged GEMM when K is not a multiple of 512), the
 // portable kernel for every shape the fast kernels do not take.
 enum { KERNEL_AUTO = 0, KERNEL_QMV = 1, KERNEL_QMM = 2, KERNEL_GENERIC = 3, KERNEL_QMM_BF16 = 4, KERNEL_QMM_LDS = 5,
-       KERNEL_QMV_ROWS = 6, KERNEL_QMM_K2 = 7, KERNEL_QMM_RW = 8, KERNEL_QMM_K2_TALL = 9, KERNEL_QMM_K2_FLAT = 10 };
+       KERNEL_QMV_ROWS = 6, KERNEL_QMM_K2 = 7, KERNEL_QMM_RW = 8, KERNEL_QMM_K2_TALL = 9, KERNEL_QMM_K2_FLAT = 10, KERNEL_QMM_K4 = 11 };
 constexpr uint32_t kQmvMaxM = 16;
 // 4-bit weights at group size 32: weight rows from which the wave-per-tile kernel has the tiles to fill the chip
 constexpr uint32_t kWt32MinN = 24576;
@@ -216,6 +216,8 @@ int32_t run_matmul_plain(const rmlx_qweight* qw, const void* x, int32_t x_dtype,
   // (its stores and the reads of the fused epilogue operand are 8- / 16-byte vectors)
   const bool can_qmm_k2 = ptr_ok && aligned16(out) && (epi.ptr == nullptr || aligned16(epi.ptr)) &&
                           qmm_k2_supported(N, K, qw->group_size, qw->bits);
+  const bool can_qmm_k4 = ptr_ok && aligned16(out) && (epi.ptr == nullptr || aligned16(epi.ptr)) &&
+                          qmm_k4_supported(N, K, qw->group_size, qw->bits);
   const bool can_qmm_k2_tall = can_qmm_k2 && qmm_k2_tall_supported(qw->group_size, qw->bits, x_dtype == RMLX_DTYPE_BF16);
 
   if (kernel == KERNEL_AUTO) {
@@ -223,15 +225,16 @@ int32_t run_matmul_plain(const rmlx_qweight* qw, const void* x, int32_t x_dtype,
     // up to 16 rows) or 16 rows (8-bit); the GEMM splits K over several workgroups per tile while its grid
     // is small, which puts its floor near 9 us at 4096 x 4096.  Measured crossovers (W = weight bytes):
     //   4-bit: GEMV up to 8 rows at every shape (N x K = 28672 x 4096: 18 against 22 us, 4096 x 14336: 13 against 18,
-    //          2048 x 16384: 10 against 16, 1024 x 28672: 16 against 23); 9 to 16 rows while W <= 12 MiB or N <= 8192
-    //          (4096 x 8192: 9 against 12 us, 4096 x 16384: 17 against 19, 8192 x 8192: 17 against 18; at 9216 x 4096 and
-    //          beyond the GEMM's grid is large enough to win: 28672 x 4096 22 against 29 us);
+    //          2048 x 16384: 10 against 16, 1024 x 28672: 16 against 23); 9 to 16 rows while W <= 12 MiB or N <= 16384
+    //          (4096 x 8192: 9 against 12 us, 4096 x 16384: 17 against 19, 8192 x 8192: 18 against 19, 12288 x 4096: 12.7 against
+    //          16.2, 16384 x 4096: 15.3 against 16.6, weights cycled through more than 1 GiB; beyond that the GEMM's grid is
+    //          large enough to win: 28672 x 4096 22 against 29 us);
     //   8-bit: GEMV up to 16 rows while W < 48 MiB (4096 x 4096 is 16 MiB; at 12288 x 4096 the GEMM wins, 19 against 23 us).
     const uint64_t wbytes = (uint64_t)N * K * qw->bits / 8;
     // Without the register-weights GEMM (K not a multiple of 512) the alternative is the LDS-staged GEMM with
     // a floor of about 15 us: there the 4-bit GEMV keeps up to passes * W <= 48 MiB.
     const bool small_m = !can_qmm_rw ? M <= kQmvMaxM || (qw->bits == 4 && (uint64_t)((M + 7) / 8) * wbytes <= (48ull << 20))
-                         : qw->bits == 4 ? M <= 8 || (M <= kQmvMaxM && (wbytes <= (12ull << 20) || N <= 8192))
+                         : qw->bits == 4 ? M <= 8 || (M <= kQmvMaxM && (wbytes <= (12ull << 20) || N <= 16384))
                                          : (M <= kQmvMaxM && wbytes < (48ull << 20));
     // Shapes the K-split GEMV does not take (group size 32) run up to 16 rows on the single-row kernel in passes of four,
     // which streams the weights once per pass: with the register-weights GEMM as the alternative it keeps up to 4 rows
@@ -270,7 +273,11 @@ int32_t run_matmul_plain(const rmlx_qweight* qw, const void* x, int32_t x_dtype,
                 "the 128 x 128 K-split qmm kernel requires bits in {4,8} (8-bit weights at group size 32 / 64: f16 or f32 "
                 "activations), N %% 128 == 0, K %% 512 == 0 and 16-byte aligned buffers (N=%u K=%u bits=%u group_size=%u)",
                 N, K, qw->bits, qw->group_size);
-  } else if (kernel < 0 || kernel > KERNEL_QMM_K2_FLAT) {
+  } else if (kernel == KERNEL_QMM_K4 && !can_qmm_k4) {
+    return fail(RMLX_INVALID_SHAPE,
+                "the 32 x 64 K-split qmm kernel requires 4-bit weights at group size 64, N %% 64 == 0, K %% 2048 == 0 and 16-byte "
+                "aligned buffers (N=%u K=%u bits=%u group_size=%u)", N, K, qw->bits, qw->group_size);
+  } else if (kernel < 0 || kernel > KERNEL_QMM_K4) {
     return fail(RMLX_NOT_FOUND, "unknown kernel selector %d", kernel);
   }
   // The K-split GEMM (32x32x16 MFMAs, K split inside the workgroup).  64 x 128 tiles where that grid is one round over
@@ -280,6 +287,15 @@ int32_t run_matmul_plain(const rmlx_qweight* qw, const void* x, int32_t x_dtype,
   // against 37.8 us at M = 192, N = 12288, 31.3 against 36.5 us at M = 256, N = 9216 (144 tiles).  With fewer tiles the
   // smaller tiles of the register-weights GEMM keep more CUs busy.
   uint32_t k2_tile_rows = kernel == KERNEL_QMM_K2_TALL ? 128 : kernel == KERNEL_QMM_K2_FLAT ? 32 : 64;
+  // 32 x 64 tiles with K split four ways in the workgroup, where they make between half a round and one round over the chip:
+  // with the tile-contiguous copy of the weights (rmlx_hip_qweight_set_gemm_layout) 13.4 against 15.7 us on the
+  // register-weights GEMM at M = 128, 4096 x 4096 (14.1 / 17.5 at M = 32, N = 9216; 36.2 / 46.0 at M = 128, K = 14336);
+  // without it only over long rows (K = 8192, M = 128: 26.1 / 28.0; K = 14336: 41.3 / 46.0; K = 4096: 15.6 / 15.7).
+  if (kernel == KERNEL_QMM && can_qmm_k4 && M > 16) {
+    const uint64_t t4 = (uint64_t)((M + 31) / 32) * (N / 64), cus = (uint64_t)ctx().num_cus;
+    const bool packed = qw->gemm_packed != nullptr && N % 128 == 0;
+    if (t4 <= cus && ((packed && t4 * 2 >= cus) || (K >= 8192 && t4 * 4 >= cus * 3))) kernel = KERNEL_QMM_K4;
+  }
   if (kernel == KERNEL_QMM && can_qmm_k2) {
     const uint64_t tiles = (uint64_t)((M + 63) / 64) * (N / 128), tall = (uint64_t)((M + 127) / 128) * (N / 128);
     const uint64_t cus = (uint64_t)ctx().num_cus;
@@ -315,6 +331,21 @@ int32_t run_matmul_plain(const rmlx_qweight* qw, const void* x, int32_t x_dtype,
     norm_w = nullptr;
   }
 
+  if (kernel == KERNEL_QMM_K4) {
+    Scratch cast;
+    const void* xk = x;
+    int32_t xk_dtype = x_dtype;
+    if (x_dtype == RMLX_DTYPE_F32) {
+      xk_dtype = RMLX_DTYPE_F16;
+      RMLX_TRY(cast.alloc((size_t)M * K * sizeof(__half), stream));
+      RMLX_TRY(launch_cast_to_f16(x, x_dtype, static_cast<__half*>(cast.ptr), (size_t)M * K, stream));
+      xk = cast.ptr;
+    }
+    QmmArgs a{qw->w, qw->s, qw->b, xk, xk_dtype, out, M, N, K, qw->bits, nullptr, 0, epi.kind, epi.ptr, epi.dtype};
+    a.w_packed = qw->gemm_packed;
+    *epi_done = true;
+    return launch_qmm_k4(a, qw->group_size, stream);
+  }
   if (kernel == KERNEL_QMM_K2) {
     Scratch cast;
     const void* xk = x;
@@ -326,6 +357,7 @@ int32_t run_matmul_plain(const rmlx_qweight* qw, const void* x, int32_t x_dtype,
       xk = cast.ptr;
     }
     QmmArgs a{qw->w, qw->s, qw->b, xk, xk_dtype, out, M, N, K, qw->bits, nullptr, 0, epi.kind, epi.ptr, epi.dtype};
+    a.w_packed = qw->gemm_packed;
     *epi_done = true;
     return launch_qmm_k2(a, qw->group_size, k2_tile_rows, stream);
   }
@@ -1423,6 +1455,35 @@ int32_t moe_grouped_impl(const rmlx_qweight* gate, const rmlx_qweight* up, const
 }  // namespace
 
 extern "C" {
+
+size_t rmlx_hip_qweight_gemm_layout_bytes(const rmlx_qweight* qw) {
+  if (qw == nullptr || qw->n_experts != 1) return 0;
+  return gemm_layout_bytes(qw->out_features, qw->in_features, qw->bits);
+}
+
+int32_t rmlx_hip_qweight_set_gemm_layout(rmlx_qweight* qw, void* dst_dev, size_t dst_bytes, rmlx_stream stream) {
+  RMLX_TRY(require_init());
+  if (qw == nullptr) return fail(RMLX_INVALID_SHAPE, "QuantizedWeight: null handle");
+  if (dst_dev == nullptr) {  // back to the one layout
+    qw->gemm_packed = nullptr;
+    return RMLX_OK;
+  }
+  const size_t need = rmlx_hip_qweight_gemm_layout_bytes(qw);
+  if (need == 0)
+    return fail(RMLX_INVALID_SHAPE, "QuantizedWeight: no GEMM layout for this weight (4- or 8-bit, out_features %% 128 == 0, in_features %% 512 == 0, "
+                                    "one expert; got bits=%u out_features=%zu in_features=%zu n_experts=%zu)", qw->bits, qw->out_features,
+                qw->in_features, qw->n_experts);
+  if (dst_bytes < need) return fail(RMLX_INVALID_SHAPE, "QuantizedWeight: GEMM layout buffer too small: %zu bytes < expected %zu bytes", dst_bytes, need);
+  if (!aligned16(dst_dev) || !aligned16(qw->w)) return fail(RMLX_INVALID_SHAPE, "QuantizedWeight: GEMM layout buffers must be 16-byte aligned");
+  uint32_t N, K;
+  RMLX_TRY(checked_u32(qw->out_features, "out_features", &N));
+  RMLX_TRY(checked_u32(qw->in_features, "in_features", &K));
+  hipStream_t s = (hipStream_t)stream;
+  RMLX_TRY(launch_gemm_repack(qw->w, N, K, qw->bits, dst_dev, s));
+  RMLX_TRY(finish(s));
+  qw->gemm_packed = dst_dev;
+  return RMLX_OK;
+}
 
 uint32_t rmlx_hip_qweight_set_expert_gemm_min_rows(rmlx_qweight* qw, uint32_t min_rows) {
   if (qw == nullptr) return 0;

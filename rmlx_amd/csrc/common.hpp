@@ -94,6 +94,9 @@ struct rmlx_qweight {
   // stacked expert weights: which streaming kernel runs decode-sized batches (read from the gate weight of a block):
   // 0 = the library's choice, 1 = K split over the waves of a workgroup (qmv.hip), 2 = a wave per tile (qmv_wt.hip)
   uint32_t expert_stream_kernel = 0;
+  // optional second copy of the weights in the tile-contiguous order of the K-split GEMMs (rmlx_hip_qweight_set_gemm_layout;
+  // the caller owns the buffer); null = none
+  const void* gemm_packed = nullptr;
 };
 
 namespace rmlx {
@@ -191,6 +194,7 @@ struct QmmArgs {
   int epi_kind;
   const void* epi;    // [M,N] f16 or f32
   int32_t epi_dtype;
+  const void* w_packed = nullptr;  // K-split GEMMs: the weights in their tile-contiguous order (gemm_layout_bytes), or null
 };
 enum { EPI_NONE = 0, EPI_RESIDUAL = 1, EPI_SWIGLU = 2 };
 // out[i] = out[i] + e[i]  /  silu(e[i]) * out[i], in place on f16 out (kernels without a fused epilogue)
@@ -211,6 +215,14 @@ int32_t launch_qmm_rw(const QmmArgs& a, uint32_t group_size, hipStream_t s);
 bool qmm_k2_supported(uint32_t N, uint32_t K, uint32_t group_size, uint32_t bits);
 bool qmm_k2_tall_supported(uint32_t group_size, uint32_t bits, bool x_bf16);
 int32_t launch_qmm_k2(const QmmArgs& a, uint32_t group_size, uint32_t tile_rows, hipStream_t s);
+// Tile-contiguous copy of a weight matrix for the K-split GEMMs: per (128 weight rows, 128-wide k block) the bytes in the
+// order the waves load them, so that every wave instruction reads 1 KB of consecutive memory instead of 32 bytes of each
+// of 32 rows.  0 bytes = the shape has no such layout (N % 128, K % 512, 4- or 8-bit).
+size_t gemm_layout_bytes(size_t N, size_t K, uint32_t bits);
+int32_t launch_gemm_repack(const uint32_t* w, uint32_t N, uint32_t K, uint32_t bits, void* dst, hipStream_t s);
+// 32 x 64 tiles with K split four ways inside the workgroup (qmm_k4.hip): 4-bit weights, group size 64, K % 2048 == 0
+bool qmm_k4_supported(uint32_t N, uint32_t K, uint32_t group_size, uint32_t bits);
+int32_t launch_qmm_k4(const QmmArgs& a, uint32_t group_size, hipStream_t s);
 // Grouped form of the same GEMM for the expert projections of batches with many rows per expert: every
 // row tile (kGroupedTileRows rows of one expert) takes its expert and rows from a device table of
 // (expert, first row position, row count) triples (bit 31 of the count: write zeros instead of computing;

@@ -45,6 +45,7 @@ constexpr int kUnroll = 4;                       // depth of the weight register
 
 struct K2Params {
   const uint32_t* w; const __half* s; const __half* b;
+  const void* w_packed;  // tile-contiguous copy of w (PACKED builds), or null
   const __half* x;  // [M,K] row-major f16 (bf16 bits when XBF16)
   __half* out;
   uint32_t M, N, K, tiles_m, tiles_n;
@@ -99,7 +100,7 @@ __device__ __forceinline__ uint32_t act_slot(uint32_t R, uint32_t seg) {
 // SBLDS: the tile's scales and biases wait in LDS (64-row tiles, group size 64, K <= 4096: a row's 128 bytes of either are
 // one cache line, fetched once; read from global memory 16 bytes per four blocks, every read pulls the whole line
 // through the CU's L1 again: measured 1.56 x the useful bytes between L2 and the CU).
-template <int BITS, bool XBF16, int GS, int MFR, bool SBLDS = false>
+template <int BITS, bool XBF16, int GS, int MFR, bool SBLDS = false, bool PACKED = false>
 __global__ __launch_bounds__(kThreads) void qmm_k2_kernel(const K2Params p) {
   static_assert(!SBLDS || (GS == 64 && MFR <= 2), "scales in LDS: tiles of at most 64 rows, group size 64");
   constexpr int kTileM = 32 * MFR;
@@ -137,7 +138,10 @@ __global__ __launch_bounds__(kThreads) void qmm_k2_kernel(const K2Params p) {
   };
   const uint32_t row_words = K * BITS / 32;
   const __amdgpu_buffer_rsrc_t xr = make_rsrc(p.x + (uint64_t)row_lo * K, (uint64_t)(p.M - row_lo) * K * 2);
-  const __amdgpu_buffer_rsrc_t wr = make_rsrc(p.w + (uint64_t)nt * kTileN * row_words, (uint64_t)kTileN * row_words * 4);
+  // (PACKED: the tile's 128 rows x K as one run of (k block, column group, k half, load, lane) x 16 bytes)
+  const __amdgpu_buffer_rsrc_t wr = PACKED
+      ? make_rsrc(static_cast<const char*>(p.w_packed) + (uint64_t)nt * kTileN * row_words * 4, (uint64_t)kTileN * row_words * 4)
+      : make_rsrc(p.w + (uint64_t)nt * kTileN * row_words, (uint64_t)kTileN * row_words * 4);
   const __amdgpu_buffer_rsrc_t sr = make_rsrc(p.s + (uint64_t)nt * kTileN * G, (uint64_t)kTileN * G * 2);
   const __amdgpu_buffer_rsrc_t br = make_rsrc(p.b + (uint64_t)nt * kTileN * G, (uint64_t)kTileN * G * 2);
   // activations: unit q*512 + tid -> (tile row 32 q + tid/16, segment tid%16); 16 neighbouring lanes read one row's
@@ -152,7 +156,8 @@ __global__ __launch_bounds__(kThreads) void qmm_k2_kernel(const K2Params p) {
 #pragma unroll
   for (int ks = 0; ks < 4; ++ks) lds_r[ks] = (kh * 4 + ks) * 64 + (((hh << 5) | r) ^ (8 * kh + 4 * hh + ks));
   // weights: row nt*128 + 32 wn + r; this lane's values of block it are k = 128 it + 64 kh + 32 hh .. + 31
-  const uint32_t woff = ((32 * wn + r) * row_words) * 4 + (8 * kh + 4 * hh) * 4 * WV;
+  const uint32_t woff = PACKED ? ((wn * 2 + kh) * WV * 64 + lane) * 16
+                               : ((32 * wn + r) * row_words) * 4 + (8 * kh + 4 * hh) * 4 * WV;
   const uint32_t soff = (32 * wn + r) * G * 2;
 
   f16v acc[MFR];
@@ -197,7 +202,9 @@ __global__ __launch_bounds__(kThreads) void qmm_k2_kernel(const K2Params p) {
   };
   auto load_w = [&](uint32_t it, int u) {
 #pragma unroll
-    for (int v = 0; v < WV; ++v) wq[u][v] = __builtin_amdgcn_raw_buffer_load_b128(wr, woff, it * (16 * 4 * WV) + v * 16, 0);
+    for (int v = 0; v < WV; ++v)
+      wq[u][v] = PACKED ? __builtin_amdgcn_raw_buffer_load_b128(wr, woff, it * (8192 * WV) + v * 1024, 0)
+                        : __builtin_amdgcn_raw_buffer_load_b128(wr, woff, it * (16 * 4 * WV) + v * 16, 0);
   };
   // the scales / biases of blocks 4 blk .. 4 blk + 3 of this lane's row
   // (SBLDS: slot of (row, unit of four blocks) behind the two activation stages; the xor spreads the 32 rows of a wave
@@ -404,7 +411,38 @@ __global__ __launch_bounds__(kThreads) void qmm_k2_kernel(const K2Params p) {
   }
 }
 
+// One thread per 16-byte unit of the destination: unit = ((((nt * S + blk) * 4 + wn) * 2 + kh) * WV + v) * 64 + lane
+// <- the 16 bytes that lane (row lane % 32, half lane / 32) of wave (wn, kh) loads as load v of k block blk of column tile nt.
+__global__ __launch_bounds__(256) void gemm_repack_kernel(const uint32_t* __restrict__ w, uint32_t K, uint32_t bits, uint64_t units,
+                                                          u4* __restrict__ dst) {
+  const uint64_t unit = (uint64_t)blockIdx.x * 256 + threadIdx.x;
+  if (unit >= units) return;
+  const uint32_t WV = bits == 4 ? 1 : 2, S = K / kBlockK, row_bytes = K * bits / 8;
+  const uint32_t lane = unit & 63;
+  uint64_t rest = unit >> 6;
+  const uint32_t v = rest % WV; rest /= WV;
+  const uint32_t kh = rest & 1, wn = (rest >> 1) & 3; rest >>= 3;
+  const uint32_t blk = rest % S, nt = rest / S;
+  const uint32_t row = nt * kTileN + 32 * wn + (lane & 31), hh = lane >> 5;
+  const uint64_t src = (uint64_t)row * row_bytes + (uint64_t)blk * (64 * WV) + (8 * kh + 4 * hh) * 4 * WV + v * 16;
+  dst[unit] = *reinterpret_cast<const u4*>(reinterpret_cast<const char*>(w) + src);
+}
+
 }  // namespace
+
+size_t gemm_layout_bytes(size_t N, size_t K, uint32_t bits) {
+  if (!(bits == 4 || bits == 8) || N == 0 || K == 0 || N % kTileN != 0 || K % (kBlockK * kUnroll) != 0) return 0;
+  return N * K * bits / 8;
+}
+
+int32_t launch_gemm_repack(const uint32_t* w, uint32_t N, uint32_t K, uint32_t bits, void* dst, hipStream_t s) {
+  const size_t bytes = gemm_layout_bytes(N, K, bits);
+  if (bytes == 0) return fail(RMLX_INVALID_SHAPE, "gemm layout: N %% 128 == 0, K %% 512 == 0 and 4- or 8-bit weights required (N=%u K=%u bits=%u)", N, K, bits);
+  const uint64_t units = bytes / 16;
+  hipLaunchKernelGGL(gemm_repack_kernel, dim3((unsigned)((units + 255) / 256)), dim3(256), 0, s, w, K, bits, units, static_cast<u4*>(dst));
+  RMLX_HIP_CHECK(hipGetLastError());
+  return RMLX_OK;
+}
 
 bool qmm_k2_supported(uint32_t N, uint32_t K, uint32_t group_size, uint32_t bits) {
   return (group_size == 32 || group_size == 64 || group_size == 128) && (bits == 4 || bits == 8) && N > 0 && K > 0 &&
@@ -428,6 +466,7 @@ int32_t launch_qmm_k2(const QmmArgs& a, uint32_t group_size, uint32_t tile_rows,
     return fail(RMLX_RUNTIME_ERROR, "qmm: f32 activations must be cast to f16 first");
   K2Params p{};
   p.w = a.w; p.s = a.s; p.b = a.b;
+  p.w_packed = a.w_packed;
   p.x = static_cast<const __half*>(a.x);
   p.out = a.out; p.M = a.M; p.N = a.N; p.K = a.K;
   p.tiles_m = (a.M + tile_rows - 1) / tile_rows;
@@ -438,20 +477,25 @@ int32_t launch_qmm_k2(const QmmArgs& a, uint32_t group_size, uint32_t tile_rows,
   const bool xb = a.x_dtype == RMLX_DTYPE_BF16, tall = tile_rows == 128;
   const bool sb_lds = group_size == 64 && !tall && a.K <= 4096;
   const bool low = tile_rows == 32;
+  const bool packed = a.w_packed != nullptr;
   auto launch = [&](auto bits_c, auto gs_c, auto mfr_c) {
     constexpr int B = decltype(bits_c)::value, GSV = decltype(gs_c)::value, MFRV = decltype(mfr_c)::value;
+    auto go = [&](auto xb_c, auto sb_c) {
+      constexpr bool XB = decltype(xb_c)::value, SB = decltype(sb_c)::value;
+      if constexpr (!(XB && MFRV == 4 && B == 8 && GSV != 128)) {
+        if (packed) hipLaunchKernelGGL((qmm_k2_kernel<B, XB, GSV, MFRV, SB, true>), grid, block, 0, s, p);
+        else hipLaunchKernelGGL((qmm_k2_kernel<B, XB, GSV, MFRV, SB, false>), grid, block, 0, s, p);
+      }
+    };
+    typedef std::true_type T;
+    typedef std::false_type F;
     if constexpr (GSV == 64 && MFRV <= 2) {
       if (sb_lds) {
-        if (xb) hipLaunchKernelGGL((qmm_k2_kernel<B, true, GSV, MFRV, true>), grid, block, 0, s, p);
-        else hipLaunchKernelGGL((qmm_k2_kernel<B, false, GSV, MFRV, true>), grid, block, 0, s, p);
+        if (xb) go(T{}, T{}); else go(F{}, T{});
         return;
       }
     }
-    if (xb) {
-      if constexpr (!(MFRV == 4 && B == 8 && GSV != 128)) hipLaunchKernelGGL((qmm_k2_kernel<B, true, GSV, MFRV>), grid, block, 0, s, p);
-    } else {
-      hipLaunchKernelGGL((qmm_k2_kernel<B, false, GSV, MFRV>), grid, block, 0, s, p);
-    }
+    if (xb) go(T{}, F{}); else go(F{}, F{});
   };
   using std::integral_constant;
   typedef integral_constant<int, 2> Low;

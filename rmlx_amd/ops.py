@@ -60,6 +60,21 @@ class QuantizedWeight:
         for the down projection.  Returns the previous value."""
         return int(rt.lib().rmlx_hip_qweight_set_expert_stream_kernel(self.handle, int(kind)))
 
+    def use_gemm_layout(self, enable=True, stream=None):
+        """Give the K-split MFMA GEMMs a tile-contiguous copy of the weights (a second device buffer of the same size,
+        owned by this object), or drop it again.  Returns False when the weight has no such layout."""
+        if not enable:
+            rt.check(rt.lib().rmlx_hip_qweight_set_gemm_layout(self.handle, None, 0, _h(stream)))
+            self._gemm_layout = None
+            return True
+        need = int(rt.lib().rmlx_hip_qweight_gemm_layout_bytes(self.handle))
+        if need == 0:
+            return False
+        buf = DeviceBuffer((need,), rt.U8)
+        rt.check(rt.lib().rmlx_hip_qweight_set_gemm_layout(self.handle, buf.ptr, buf.nbytes, _h(stream)))
+        self._gemm_layout = buf
+        return True
+
     def groups_per_row(self):
         return self.in_features // self.group_size
 

@@ -15,7 +15,7 @@ LIB_PATH = os.path.join(_HERE, "lib", "librmlx_hip.so")
 OK, INVALID_SHAPE, NOT_FOUND, RUNTIME_ERROR = 0, 1, 2, 3
 F32, F16, BF16, U32, U8 = 0, 1, 2, 3, 4
 KERNEL_AUTO, KERNEL_QMV, KERNEL_QMM, KERNEL_GENERIC, KERNEL_QMM_BF16, KERNEL_QMM_LDS, KERNEL_QMV_ROWS = 0, 1, 2, 3, 4, 5, 6
-KERNEL_QMM_K2, KERNEL_QMM_RW, KERNEL_QMM_K2_TALL, KERNEL_QMM_K2_FLAT = 7, 8, 9, 10
+KERNEL_QMM_K2, KERNEL_QMM_RW, KERNEL_QMM_K2_TALL, KERNEL_QMM_K2_FLAT, KERNEL_QMM_K4 = 7, 8, 9, 10, 11
 GATHER_AUTO, GATHER_STREAM, GATHER_GEMM, GATHER_PORTABLE = 0, 1, 2, 3  # rmlx_hip_gather_qmm_select kernels
 FLOOR_EMPTY, FLOOR_READ4, FLOOR_READ8, FLOOR_MFMA, FLOOR_READ2, FLOOR_MFMA_VALU, FLOOR_LDS, FLOOR_L2_READ = 0, 1, 2, 3, 4, 5, 6, 7  # rmlx_hip_measure_floor kinds
 
@@ -45,7 +45,7 @@ EXPORTS = [
     "rmlx_hip_gather_qmm", "rmlx_hip_topk_route", "rmlx_hip_moe_sort", "rmlx_hip_index_gather",
     "rmlx_hip_scatter_weighted_add", "rmlx_hip_silu_gate", "rmlx_hip_expert_group_grouped_forward",
     "rmlx_hip_moe_forward_grouped", "rmlx_hip_moe_forward", "rmlx_hip_moe_forward_noalloc", "rmlx_hip_awq_dequant", "rmlx_hip_gptq_dequant",
-    "rmlx_hip_qmm_norm", "rmlx_hip_qweight_set_expert_gemm_min_rows", "rmlx_hip_qweight_set_expert_stream_kernel", "rmlx_hip_gather_qmm_select", "rmlx_hip_measure_floor",
+    "rmlx_hip_qmm_norm", "rmlx_hip_qweight_set_expert_gemm_min_rows", "rmlx_hip_qweight_set_expert_stream_kernel", "rmlx_hip_qweight_gemm_layout_bytes", "rmlx_hip_qweight_set_gemm_layout", "rmlx_hip_gather_qmm_select", "rmlx_hip_measure_floor",
 ]
 
 _lib = None
@@ -119,6 +119,10 @@ def lib():
     L.rmlx_hip_qweight_set_expert_gemm_min_rows.restype = u32
     L.rmlx_hip_qweight_set_expert_stream_kernel.argtypes = [vp, u32]
     L.rmlx_hip_qweight_set_expert_stream_kernel.restype = u32
+    L.rmlx_hip_qweight_gemm_layout_bytes.argtypes = [vp]
+    L.rmlx_hip_qweight_gemm_layout_bytes.restype = ctypes.c_size_t
+    L.rmlx_hip_qweight_set_gemm_layout.argtypes = [vp, vp, ctypes.c_size_t, vp]
+    L.rmlx_hip_qweight_set_gemm_layout.restype = ctypes.c_int32
     L.rmlx_hip_scratch_allocations.argtypes = []
     L.rmlx_hip_scratch_allocations.restype = ctypes.c_uint64
     _lib = L
