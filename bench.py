@@ -99,7 +99,7 @@ class Timer:
 
 
 def bench_matmul(ops, rt, timer, rng, m, n, k, bits, x_dtype, launches, warmup, min_total_bytes, check=True, kernel=0,
-                 check_rows=None, graph=False, queued_trains=0):
+                 check_rows=None, graph=False, queued_trains=0, gemm_layout=False):
     from oracle import model
     wbytes = n * k * bits // 8 + 4 * (n * k // 64)
     n_sets = max(1, -(-min_total_bytes // wbytes))
@@ -108,6 +108,10 @@ def bench_matmul(ops, rt, timer, rng, m, n, k, bits, x_dtype, launches, warmup, 
     for i in range(1, n_sets):  # distinct buffers; contents rolled so that sets differ
         qws.append(ops.QuantizedWeight.from_numpy(np.roll(base[0], i, axis=0), np.roll(base[1], i, axis=0),
                                                   np.roll(base[2], i, axis=0), 64, bits))
+    if gemm_layout:  # every set also gets the tile-contiguous copy for the K-split GEMMs (a second buffer of the same size)
+        for q in qws:
+            if not q.use_gemm_layout(True):
+                raise RuntimeError("no GEMM layout for this weight")
     xf = rng.standard_normal((m, k)).astype(np.float32)
     if x_dtype == "bf16":
         xh = model.f32_to_bf16_bits(xf)
@@ -487,10 +491,17 @@ def main():
             r = bench_matmul(ops, rt, timer, rng, m, 4096, 4096, 4, "f16", m_launches, train_warm, GiB + GiB // 8)
             r["mfma_frac"] = r["tflops"] / MFMA_F16_PEAK_TF
             extra[f"q4_qmm_m{m}_4096"] = r
+        # the same with the optional tile-contiguous copy of the weights (rmlx_hip_qweight_set_gemm_layout)
+        r = bench_matmul(ops, rt, timer, rng, 128, 4096, 4096, 4, "f16", gemm_launches, train_warm, GiB + GiB // 8, gemm_layout=True)
+        r["mfma_frac"] = r["tflops"] / MFMA_F16_PEAK_TF
+        extra["q4_qmm_m128_4096_gemm_layout"] = r
         for name, kern in (("q8_qmm_bf16_m128_n12288", rt.KERNEL_AUTO), ("q8_qmm_bf16_m128_n12288_bf16_mfma", rt.KERNEL_QMM_BF16)):
             r = bench_matmul(ops, rt, timer, rng, 128, 12288, 4096, 8, "bf16", gemm_launches, train_warm, GiB + GiB // 8, kernel=kern)
             r["mfma_frac"] = r["tflops"] / MFMA_F16_PEAK_TF
             extra[name] = r
+        r = bench_matmul(ops, rt, timer, rng, 128, 12288, 4096, 8, "bf16", gemm_launches, train_warm, GiB + GiB // 8, gemm_layout=True)
+        r["mfma_frac"] = r["tflops"] / MFMA_F16_PEAK_TF
+        extra["q8_qmm_bf16_m128_n12288_gemm_layout"] = r
     if "dequant" in sections:
         progress("dequant")
         for fmt in ("awq", "gptq"):

@@ -326,8 +326,9 @@ int32_t rmlx_hip_qweight_set_gemm_layout(rmlx_qweight* qw, void* dst_dev, size_t
  * block whose gate weight is `qw`: 1 = K split over the waves of a workgroup, chunks of 8 rows, 2 = a wave per 16-row
  * weight tile, chunks of 8 rows, 3 = a wave per tile, chunks of 16 rows, 4 = kernel 1 for the gate / up projection and
  * kernel 2 for the down projection (4-bit weights, group size 64; other weights keep kernel 1), 0 = the library's
- * choice: 3 between 7 and 8.5 rows per expert on average, else 4.  Returns the previous value; the tests use it to check
- * that the kernels agree.  (No counterpart in the reference, which has one kernel for this: gather_qmv_fast_f16_q4,
+ * choice (4).  Kernel 3 streams an expert with 9 to 16 rows once instead of twice and is the fastest of the four from 7 rows
+ * per expert on average - as long as no expert of the batch has more than 16 rows, so it is for callers whose router bounds
+ * that.  Returns the previous value; the tests use it to check that the kernels agree.  (No counterpart in the reference, which has one kernel for this: gather_qmv_fast_f16_q4,
  * crates/rmlx-core/src/ops/quantized.rs:9752-9842.) */
 uint32_t rmlx_hip_qweight_set_expert_stream_kernel(rmlx_qweight* qw, uint32_t kind);
 

@@ -175,6 +175,14 @@ class QuantizedWeight {
   const rmlx_qweight* handle() const { return handle_; }
   uint32_t set_expert_gemm_min_rows(uint32_t min_rows) const { return rmlx_hip_qweight_set_expert_gemm_min_rows(handle_, min_rows); }
   uint32_t set_expert_stream_kernel(uint32_t kind) const { return rmlx_hip_qweight_set_expert_stream_kernel(handle_, kind); }
+  // Give the K-split GEMMs a tile-contiguous copy of the weights in `dst` (gemm_layout_bytes() bytes, kept alive by the
+  // caller via the shared pointer stored here); an empty pointer drops it.
+  size_t gemm_layout_bytes() const { return rmlx_hip_qweight_gemm_layout_bytes(handle_); }
+  void set_gemm_layout(std::shared_ptr<Buffer> dst, const Stream* stream = nullptr) {
+    detail::check(rmlx_hip_qweight_set_gemm_layout(handle_, dst ? dst->ptr() : nullptr, dst ? dst->length() : 0, raw(stream)));
+    gemm_layout_buf = std::move(dst);
+  }
+  std::shared_ptr<Buffer> gemm_layout_buf;
 
   std::shared_ptr<Buffer> weights_buf, scales_buf, biases_buf;
   uint32_t group_size, bits;

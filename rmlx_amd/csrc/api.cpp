@@ -532,10 +532,9 @@ uint32_t expert_gemm_tile_rows(const ExpertShapes& sh, uint64_t rows, uint64_t g
 // Which streaming kernel runs the two projections of a decode-sized batch, and over chunks of how many rows.
 // gate_up / down: 0 = the K-split kernel (qmv.hip), else the wave-per-tile kernel (qmv_wt.hip) with chunks of that many
 // rows (8 or 16).  Selector of the gate handle: 1 = K-split for both, 2 / 3 = wave per tile for both with chunks of 8 / 16
-// rows, 4 = K-split for gate / up, wave per tile for a down projection whose rows are shorter than 4096 (measured at
-// D = 4096, I = 1536: the block takes 254 against 269 us at T = 32 and 348 against 368 us at T = 128; over chunks of 8
-// rows a wave-per-tile gate / up projection is 30 % slower than the K-split one), 0 = the library's choice: 4 up to 7
-// rows per expert on average, 3 from 7 to 8.5.
+// rows, 0 (the library's choice) and 4 = K-split for gate / up, wave per tile for a down projection whose rows are shorter
+// than 4096 (measured at D = 4096, I = 1536: the block takes 254 against 269 us at T = 32 and 348 against 368 us at
+// T = 128; over chunks of 8 rows a wave-per-tile gate / up projection is 30 % slower than the K-split one).
 struct StreamPlan { uint32_t gate_up, down, chunk_rows; };
 // rows / groups: the assignments of the call and the experts (or host-side groups) they spread over
 StreamPlan expert_stream_plan(const ExpertShapes& sh, size_t rows, size_t groups) {
@@ -544,12 +543,11 @@ StreamPlan expert_stream_plan(const ExpertShapes& sh, size_t rows, size_t groups
   if (sh.stream_kernel == 1) return pl;
   if (sh.stream_kernel == 2 && sh.wave_tiles) pl = StreamPlan{8, 8, 8};
   else if (sh.stream_kernel == 3 && sh.wave_tiles) pl = StreamPlan{16, 16, 16};
-  // From 7 rows per expert on average most experts hold more than one chunk of 8 rows, which the K-split kernel streams
-  // once per chunk: the wave-per-tile kernels over chunks of 16 rows then win, until experts with more than 16 rows add
-  // a seventh round of workgroups to their six (measured at D = 4096, I = 1536, E = 128, K-split gate / up with the
-  // wave-per-tile down projection against chunks of 16 rows: 301 / 320 us at 6.5 rows per expert, 320 / 321 at 7,
-  // 336 / 323 at 8, 363 / 385 at 9).
-  else if (sh.stream_kernel == 0 && sh.wave_tiles && rows >= 7 * groups && 2 * rows < 17 * groups) pl = StreamPlan{16, 16, 16};
+  // (Chunks of 16 rows are not picked here: at D = 4096, I = 1536, E = 128 they take 322 us at 8 rows per expert on average
+  // against 345 us for K-split gate / up with the wave-per-tile down projection - while no expert has more than 16 rows.
+  // One that has adds a seventh round of workgroups to their six: 384 us.  Under uniform random routing that is the case
+  // for 11 / 23 / 38 % of the batches at 7 / 7.5 / 8 rows per expert, which makes the expectation a tie.  A caller whose
+  // router bounds the rows per expert selects them with selector 3.)
   else if (sh.wave_down && sh.I < 4096) pl.down = 8;
   return pl;
 }
