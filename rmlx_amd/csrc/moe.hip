@@ -45,30 +45,14 @@ __device__ __forceinline__ float wave_add(float v) {
   v += swz16_f32(v);
   return readlane_f32(v, 0) + readlane_f32(v, 32);
 }
-// lexicographic maximum of (hi, lo) over the wave; the result is uniform
-template <int CTRL>
-__device__ __forceinline__ void key_max_step(uint32_t& hi, uint32_t& lo) {
-  const uint32_t ohi = dpp_u32<CTRL>(hi), olo = dpp_u32<CTRL>(lo);
-  const bool take = ohi > hi || (ohi == hi && olo > lo);
-  hi = take ? ohi : hi;
-  lo = take ? olo : lo;
-}
-__device__ __forceinline__ void wave_key_max(uint32_t& hi, uint32_t& lo) {
-  key_max_step<0xB1>(hi, lo);
-  key_max_step<0x4E>(hi, lo);
-  key_max_step<0x141>(hi, lo);
-  key_max_step<0x140>(hi, lo);
-  {
-    const uint32_t ohi = (uint32_t)__builtin_amdgcn_ds_swizzle((int)hi, 0x401F), olo = (uint32_t)__builtin_amdgcn_ds_swizzle((int)lo, 0x401F);
-    const bool take = ohi > hi || (ohi == hi && olo > lo);
-    hi = take ? ohi : hi;
-    lo = take ? olo : lo;
-  }
-  const uint32_t h0 = (uint32_t)__builtin_amdgcn_readlane((int)hi, 0), l0 = (uint32_t)__builtin_amdgcn_readlane((int)lo, 0);
-  const uint32_t h1 = (uint32_t)__builtin_amdgcn_readlane((int)hi, 32), l1 = (uint32_t)__builtin_amdgcn_readlane((int)lo, 32);
-  const bool take = h1 > h0 || (h1 == h0 && l1 > l0);
-  hi = take ? h1 : h0;
-  lo = take ? l1 : l0;
+__device__ __forceinline__ uint32_t max_u32(uint32_t a, uint32_t b) { return a > b ? a : b; }
+__device__ __forceinline__ uint32_t wave_max_u32(uint32_t v) {
+  v = max_u32(v, dpp_u32<0xB1>(v));
+  v = max_u32(v, dpp_u32<0x4E>(v));
+  v = max_u32(v, dpp_u32<0x141>(v));
+  v = max_u32(v, dpp_u32<0x140>(v));
+  v = max_u32(v, (uint32_t)__builtin_amdgcn_ds_swizzle((int)v, 0x401F));
+  return max_u32((uint32_t)__builtin_amdgcn_readlane((int)v, 0), (uint32_t)__builtin_amdgcn_readlane((int)v, 32));
 }
 
 // ---- routing: one wave per token -----------------------------------------------------------
@@ -97,8 +81,7 @@ __device__ __forceinline__ float exp_neg_exact(float x) {
 
 // Each lane owns experts lane, lane+64, lane+128, lane+192 (E <= 256).  Ranking follows the reference:
 // the f32 softmax value exp(l - max) * (1 / sum) with strict >, so equal values (two logits that collapse
-// after exp, an underflowing tail) go to the lower expert index (topk_route.rs:283-300).  A round's winner
-// is the wave maximum of the key (bits of the non-negative softmax value, ~index).  The sum runs over the
+// after exp, an underflowing tail) go to the lower expert index (topk_route.rs:283-300).  The sum runs over the
 // four values of a lane in ascending order and then over the lanes as a balanced pairwise tree.
 // (`lds_idx`: optional copy of the picks in workgroup memory, for a sort fused behind the routing)
 __device__ __forceinline__ void route_token(const float* __restrict__ logits, const float* __restrict__ bias,
@@ -133,38 +116,31 @@ __device__ __forceinline__ void route_token(const float* __restrict__ logits, co
 #pragma unroll
   for (int j = 0; j < 4; ++j) sm[j] *= inv;
 
-  // lane k keeps the k-th pick (no register arrays indexed by the round counter)
+  // A slot's key: the bits of its non-negative softmax value (order-preserving; -0 counted as +0) plus one, zero once
+  // the slot is taken or lies past E.  A round: the wave maximum of the keys, then the lowest expert index that
+  // holds it -- slots in ascending j, inside a slot the lowest lane of the ballot.  Lane k keeps the k-th pick (no
+  // register arrays indexed by the round counter).
+  uint32_t key[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) key[j] = taken[j] ? 0u : __float_as_uint(sm[j] + 0.0f) + 1u;
   float my_w = 0.f;
   uint32_t my_idx = 0xFFFFFFFFu;
   for (uint32_t k = 0; k < K; ++k) {
-    float bv = NEG_INF;
+    const uint32_t top = wave_max_u32(max_u32(max_u32(key[0], key[1]), max_u32(key[2], key[3])));  // uniform
     uint32_t bi = 0xFFFFFFFFu;
+    if (top != 0) {
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {  // ascending expert index inside the lane: strict > keeps the lower one
-      if (!taken[j] && (bi == 0xFFFFFFFFu || sm[j] > bv)) { bv = sm[j]; bi = lane + 64 * j; }
-    }
-    // key: softmax values compare like their order-preserving bit patterns (-0 counted as +0), then the lower index
-    uint32_t hi = 0, lo = 0;
-    if (bi != 0xFFFFFFFFu) {
-      const uint32_t u = __float_as_uint(bv + 0.0f);
-      hi = (u & 0x80000000u) ? ~u : (u | 0x80000000u);
-      hi = hi == 0 ? 1u : hi;  // keeps every candidate above "none" (only a NaN with all bits set maps to 0)
-      lo = 0xFFFFFFFFu - bi;
-    }
-    wave_key_max(hi, lo);
-    bi = hi == 0 ? 0xFFFFFFFFu : 0xFFFFFFFFu - lo;  // uniform
-    float bw = 0.f;
-    if (bi != 0xFFFFFFFFu) {
-      const int src = (int)(bi & 63u), jj = (int)(bi >> 6);
-      const float cand = jj == 0 ? sm[0] : (jj == 1 ? sm[1] : (jj == 2 ? sm[2] : sm[3]));
-      bw = readlane_f32(cand, __builtin_amdgcn_readfirstlane(src));
+      for (int j = 3; j >= 0; --j) {
+        const uint64_t holders = __builtin_amdgcn_ballot_w64(key[j] == top);
+        if (holders != 0) bi = (uint32_t)__builtin_ctzll(holders) + 64u * j;
+      }
     }
 #pragma unroll
     for (int j = 0; j < 4; ++j)
-      if (bi == lane + 64 * j) taken[j] = true;
+      if (bi == lane + 64 * j) key[j] = 0u;
     if (lane == k) {
       my_idx = bi;
-      my_w = bw;
+      my_w = top != 0 ? __uint_as_float(top - 1u) : 0.f;
     }
   }
   float scale = 1.0f;
