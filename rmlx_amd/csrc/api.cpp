@@ -463,6 +463,7 @@ constexpr uint32_t kGatherGemmMinRows = 9;
 // routed block: up to this many assignments run without grouping (every assignment its own chunk, combine fused into
 // the down projection)
 constexpr uint32_t kDirectMaxAssignments = 32;
+constexpr uint32_t kOwnRouteMinAssignments = 16;  // from here on the gate / up launch of that path routes by itself
 enum { GATHER_AUTO = 0, GATHER_STREAM = 1, GATHER_GEMM = 2, GATHER_PORTABLE = 3 };
 
 int32_t check_expert_weights(const char* who, const rmlx_qweight* gate, const rmlx_qweight* up,
@@ -580,11 +581,18 @@ int32_t run_expert_ffn_portable(const rmlx_qweight* gate, const rmlx_qweight* up
   return launch_generic(d, stream);
 }
 
+// Routing fused in front of the grouping (decode-sized batches): f32 logits [T, E], optional f32 bias [E];
+// the picks and their weights are written to idx_out / w_out.
+struct FusedRoute { const float* logits; const float* bias; uint32_t* idx_out; float* w_out; };
+
 // gate/up + SwiGLU then down, over a device chunk table.  h: f16 [positions, I] scratch.
+// `own_route` (with top_k): no table -- the gate / up workgroups rank their token's experts themselves; position
+// t * top_k + k is pick k of token t (4-bit K-split kernel only: plan.gate_up == 0), max_chunks = T * top_k.
 int32_t run_expert_ffn(const rmlx_qweight* gate, const rmlx_qweight* up, const rmlx_qweight* down,
                        const ExpertShapes& sh, const __half* x, const uint32_t* row_map,
                        const uint32_t* chunk_tab, const uint32_t* n_chunks, uint32_t max_chunks, __half* h,
-                       void* y, int y_f32, uint32_t gemm_tile_rows, const StreamPlan& plan, hipStream_t stream) {
+                       void* y, int y_f32, uint32_t gemm_tile_rows, const StreamPlan& plan, hipStream_t stream,
+                       const FusedRoute* own_route = nullptr, uint32_t top_k = 0) {
   const uint32_t per = 32 / gate->bits;  // values per u32 word: 8 (4-bit) or 4 (8-bit)
   if (gemm_tile_rows != 0) {  // the table holds row tiles of that many rows and n_chunks its length
     const uint32_t gs = gate->group_size;  // one group size for the three projections (ExpertShapes::gemm)
@@ -630,6 +638,13 @@ int32_t run_expert_ffn(const rmlx_qweight* gate, const rmlx_qweight* up, const r
   a.x = x; a.row_map = row_map;
   a.out = h; a.ld_out = sh.I; a.out_f32 = 0; a.dual = 1;
   a.chunk_tab = chunk_tab; a.n_chunks_dev = n_chunks; a.max_chunks = max_chunks; a.mr = 8;
+  if (own_route != nullptr) {
+    if (plan.gate_up != 0 || gate->bits != 4 || y != nullptr)
+      return fail(RMLX_RUNTIME_ERROR, "expert FFN: routing inside the gate / up launch is for the 4-bit K-split kernel");
+    a.route_logits = own_route->logits; a.route_bias = own_route->bias;
+    a.route_idx_out = own_route->idx_out; a.route_w_out = own_route->w_out;
+    a.route_e = sh.E; a.route_k = top_k; a.route_renorm = 1;
+  }
   // (the table holds chunks of at most plan.chunk_rows rows)
   if (plan.gate_up != 0) RMLX_TRY(launch_qmv_wt(a, plan.gate_up, stream));
   else RMLX_TRY(gate->bits == 8 ? launch_qmv_q8_tab(a, stream) : launch_qmv_q4(a, stream));
@@ -1340,10 +1355,6 @@ int32_t rmlx_hip_expert_group_grouped_forward(const rmlx_qweight* gate, const rm
 }  // extern "C"
 
 namespace {
-// Routing fused in front of the grouping (decode-sized batches): f32 logits [T, E], optional f32 bias [E];
-// the picks and their weights are written to idx_out / w_out.
-struct FusedRoute { const float* logits; const float* bias; uint32_t* idx_out; float* w_out; };
-
 int32_t moe_grouped_impl(const rmlx_qweight* gate, const rmlx_qweight* up, const rmlx_qweight* down,
                          const rmlx_array* x, const uint32_t* expert_indices_dev, const float* expert_weights_dev,
                          size_t top_k, void* out_f16_dev, size_t out_bytes, rmlx_stream stream, const FusedRoute* route,
@@ -1415,15 +1426,24 @@ int32_t moe_grouped_impl(const rmlx_qweight* gate, const rmlx_qweight* up, const
   // streamed once per token (at 4 tokens of 8 picks over 128 experts: 32 chunks for 31 experts).
   if (route != nullptr && A <= kDirectMaxAssignments && sh.stream_kernel != 1 && sh.wave_down &&
       qmv_wt_combine_supported(sh.D, sh.I, down->group_size, (uint32_t)top_k)) {
-    RMLX_TRY(meta.alloc(((size_t)4 * A + 4) * 4, s, arena));  // tok[A] | chunk_tab[3 A] | n_chunks[1]
-    uint32_t* tok = static_cast<uint32_t*>(meta.ptr);
-    uint32_t* chunk_tab = tok + A;
-    uint32_t* n_chunks = chunk_tab + 3 * (size_t)A;
-    RMLX_TRY(launch_route_direct_small(route->logits, route->bias, T32, sh.E, (uint32_t)top_k, 1, route->idx_out, route->w_out,
-                                       tok, chunk_tab, n_chunks, s));
     RMLX_TRY(h.alloc((size_t)A * sh.I * 2, s, arena));
-    RMLX_TRY(run_expert_ffn(gate, up, down, sh, xk, tok, chunk_tab, n_chunks, A, static_cast<__half*>(h.ptr), nullptr, 0, 0,
-                            StreamPlan{0, 0, 8}, s));
+    if (sh.E <= 256 && A >= kOwnRouteMinAssignments) {
+      // two launches: the gate / up workgroups rank their own token's experts (one wave, while the others wait).  The
+      // ranking then sits in front of every workgroup's weight stream: it pays once the grid is several rounds of
+      // workgroups (2 tokens of 8 picks: 36.4 against 38.0 us, 4 tokens: 62.1 against 64.2 us) and costs where the grid
+      // is a single round (1 token: 26.0 against 25.3 us).
+      RMLX_TRY(run_expert_ffn(gate, up, down, sh, xk, nullptr, nullptr, nullptr, A, static_cast<__half*>(h.ptr), nullptr, 0, 0,
+                              StreamPlan{0, 0, 8}, s, route, (uint32_t)top_k));
+    } else {
+      RMLX_TRY(meta.alloc(((size_t)4 * A + 4) * 4, s, arena));  // tok[A] | chunk_tab[3 A] | n_chunks[1]
+      uint32_t* tok = static_cast<uint32_t*>(meta.ptr);
+      uint32_t* chunk_tab = tok + A;
+      uint32_t* n_chunks = chunk_tab + 3 * (size_t)A;
+      RMLX_TRY(launch_route_direct_small(route->logits, route->bias, T32, sh.E, (uint32_t)top_k, 1, route->idx_out, route->w_out,
+                                         tok, chunk_tab, n_chunks, s));
+      RMLX_TRY(run_expert_ffn(gate, up, down, sh, xk, tok, chunk_tab, n_chunks, A, static_cast<__half*>(h.ptr), nullptr, 0, 0,
+                              StreamPlan{0, 0, 8}, s));
+    }
     RMLX_TRY(launch_qmv_wt_combine(down->w, down->s, down->b, (uint64_t)sh.D * (sh.I / 8), (uint64_t)sh.D * (sh.I / down->group_size),
                                    sh.E, static_cast<const __half*>(h.ptr), route->idx_out, route->w_out, T32, (uint32_t)top_k,
                                    sh.D, sh.I, static_cast<__half*>(out_f16_dev), s));

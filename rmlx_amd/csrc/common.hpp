@@ -140,6 +140,11 @@ struct QmvArgs {
   uint32_t M;                // used when chunk_tab == null
   uint32_t mr;               // rows staged per chunk (1,2,4,8); 0 -> derive from M
   uint32_t group_size;       // 64 (also when 0) or 128
+  // launch_qmv_q4 only: the workgroups route their own token (no chunk table): chunk c of the max_chunks = T * route_k
+  // is pick c % route_k of token c / route_k, its activation row is the token, its output row is c; f32 logits
+  // [T, route_e], optional bias; the picks and normalised weights are also written to route_idx_out / route_w_out
+  const float* route_logits; const float* route_bias; uint32_t* route_idx_out; float* route_w_out;
+  uint32_t route_e, route_k; int32_t route_renorm;
 };
 int32_t launch_qmv_q4(const QmvArgs& a, hipStream_t s);
 bool qmv_q4_supported(uint32_t N, uint32_t K, uint32_t group_size);
