@@ -585,6 +585,28 @@ int32_t run_expert_ffn_portable(const rmlx_qweight* gate, const rmlx_qweight* up
 // the picks and their weights are written to idx_out / w_out.
 struct FusedRoute { const float* logits; const float* bias; uint32_t* idx_out; float* w_out; };
 
+// The fused gate / up launch of the streaming kernels: both matrices (halves of one stacked buffer, or two), x -> h.
+QmvArgs gate_up_args(const rmlx_qweight* gate, const rmlx_qweight* up, const ExpertShapes& sh, const __half* x, __half* h) {
+  const uint32_t per = 32 / gate->bits;  // values per u32 word: 8 (4-bit) or 4 (8-bit)
+  QmvArgs a{};
+  a.w0 = gate->w; a.s0 = gate->s; a.b0 = gate->b;
+  if (sh.fused) {
+    a.w1 = gate->w + (size_t)sh.I * (sh.D / per);
+    a.s1 = gate->s + (size_t)sh.I * (sh.D / gate->group_size);
+    a.b1 = gate->b + (size_t)sh.I * (sh.D / gate->group_size);
+  } else {
+    a.w1 = up->w; a.s1 = up->s; a.b1 = up->b;
+  }
+  const size_t rows_per_expert = sh.fused ? 2 * (size_t)sh.I : sh.I;
+  a.N = sh.I; a.K = sh.D;
+  a.expert_stride_w = rows_per_expert * (sh.D / per);
+  a.expert_stride_s = rows_per_expert * (sh.D / gate->group_size);
+  a.group_size = gate->group_size;
+  a.x = x;
+  a.out = h; a.ld_out = sh.I; a.out_f32 = 0; a.dual = 1;
+  return a;
+}
+
 // gate/up + SwiGLU then down, over a device chunk table.  h: f16 [positions, I] scratch.
 // `own_route` (with top_k): no table -- the gate / up workgroups rank their token's experts themselves; position
 // t * top_k + k is pick k of token t (4-bit K-split kernel only: plan.gate_up == 0), max_chunks = T * top_k.
@@ -621,22 +643,8 @@ int32_t run_expert_ffn(const rmlx_qweight* gate, const rmlx_qweight* up, const r
     d.tile_tab = chunk_tab; d.n_tiles_dev = n_chunks; d.max_tiles = max_chunks; d.tile_rows = gemm_tile_rows;
     return launch_qmm_rw_grouped(d, stream);
   }
-  QmvArgs a{};
-  a.w0 = gate->w; a.s0 = gate->s; a.b0 = gate->b;
-  if (sh.fused) {
-    a.w1 = gate->w + (size_t)sh.I * (sh.D / per);
-    a.s1 = gate->s + (size_t)sh.I * (sh.D / gate->group_size);
-    a.b1 = gate->b + (size_t)sh.I * (sh.D / gate->group_size);
-  } else {
-    a.w1 = up->w; a.s1 = up->s; a.b1 = up->b;
-  }
-  const size_t rows_per_expert = sh.fused ? 2 * (size_t)sh.I : sh.I;
-  a.N = sh.I; a.K = sh.D;
-  a.expert_stride_w = rows_per_expert * (sh.D / per);
-  a.expert_stride_s = rows_per_expert * (sh.D / gate->group_size);
-  a.group_size = gate->group_size;
-  a.x = x; a.row_map = row_map;
-  a.out = h; a.ld_out = sh.I; a.out_f32 = 0; a.dual = 1;
+  QmvArgs a = gate_up_args(gate, up, sh, x, h);
+  a.row_map = row_map;
   a.chunk_tab = chunk_tab; a.n_chunks_dev = n_chunks; a.max_chunks = max_chunks; a.mr = 8;
   if (own_route != nullptr) {
     if (plan.gate_up != 0 || gate->bits != 4 || y != nullptr)
@@ -1441,8 +1449,14 @@ int32_t moe_grouped_impl(const rmlx_qweight* gate, const rmlx_qweight* up, const
       uint32_t* n_chunks = chunk_tab + 3 * (size_t)A;
       RMLX_TRY(launch_route_direct_small(route->logits, route->bias, T32, sh.E, (uint32_t)top_k, 1, route->idx_out, route->w_out,
                                          tok, chunk_tab, n_chunks, s));
-      RMLX_TRY(run_expert_ffn(gate, up, down, sh, xk, tok, chunk_tab, n_chunks, A, static_cast<__half*>(h.ptr), nullptr, 0, 0,
-                              StreamPlan{0, 0, 8}, s));
+      // one row per expert: the single-row GEMV's layout (a wave per weight row pair, dot products instead of a matrix
+      // unit that would multiply 15 empty rows) where it takes the shape, else the K-split kernel over one-row chunks
+      if (gate->bits == 4 && qmv_m1_gate_up_supported(sh.I, sh.D, gate->group_size))
+        RMLX_TRY(launch_qmv_m1_gate_up(gate_up_args(gate, up, sh, xk, static_cast<__half*>(h.ptr)), route->idx_out, A,
+                                       (uint32_t)top_k, sh.E, s));
+      else
+        RMLX_TRY(run_expert_ffn(gate, up, down, sh, xk, tok, chunk_tab, n_chunks, A, static_cast<__half*>(h.ptr), nullptr, 0, 0,
+                                StreamPlan{0, 0, 8}, s));
     }
     RMLX_TRY(launch_qmv_wt_combine(down->w, down->s, down->b, (uint64_t)sh.D * (sh.I / 8), (uint64_t)sh.D * (sh.I / down->group_size),
                                    sh.E, static_cast<const __half*>(h.ptr), route->idx_out, route->w_out, T32, (uint32_t)top_k,

@@ -148,6 +148,12 @@ struct QmvArgs {
 };
 int32_t launch_qmv_q4(const QmvArgs& a, hipStream_t s);
 bool qmv_q4_supported(uint32_t N, uint32_t K, uint32_t group_size);
+// Gate / up projection of single rows through chosen experts (qmv_m1.hip): position a = activation row a / top_k (x, no
+// row map) through expert idx[a] of the two stacked matrices of `a` (w0 / w1, expert strides), out[a, :] = silu(gate) * up
+// in f16 [assignments, N]; 4-bit weights at group size 64, the shapes of the single-row GEMV.  chunk_tab / M / mr of `a` are not used.
+bool qmv_m1_gate_up_supported(uint32_t N, uint32_t K, uint32_t group_size);
+int32_t launch_qmv_m1_gate_up(const QmvArgs& a, const uint32_t* idx, uint32_t assignments, uint32_t top_k, uint32_t n_experts,
+                              hipStream_t stream);
 // Wave-per-tile streaming GEMV (qmv_wt.hip): the same arguments; chunks of at most chunk_rows (8 or 16) rows, a wave owns
 // a 16-row weight tile over all of K (no cross-wave reduction), group size 64, K <= 4096 (16-row chunks: 8192)
 bool qmv_wt_supported(uint32_t N, uint32_t K, uint32_t group_size, uint32_t chunk_rows);

@@ -521,6 +521,92 @@ __global__ __launch_bounds__(kThreads, 1) void qmv_m1_loop_kernel(M1Params p) {
   }
 }
 
+// ---- gate / up projection of single rows through chosen experts (routed blocks of one token or a few) ---------------
+// Assignment a (blockIdx.y) multiplies activation row a / top_k with expert idx[a] of two stacked matrices: a wave owns
+// gate row r and up row r of that expert over the whole K (the two-row form of the kernel above: the activation
+// registers read from LDS serve both) and writes silu(gate . x) * (up . x), rounded once, to out[a, r].  An expert index
+// outside [0, n_experts) writes zeros.  The counterpart of gather_qmv_fast_f16_q4 (quantized.rs:9752-9842, one activation
+// row per index) with the SwiGLU of ExpertGroup::grouped_forward (crates/rmlx-nn/src/expert_group.rs:445-524) behind it.
+struct M1GateUpParams {
+  const uint32_t* w0; const __half* s0; const __half* b0;  // gate, expert 0
+  const uint32_t* w1; const __half* s1; const __half* b1;  // up, expert 0
+  uint64_t estride_w, estride_s;                           // u32 words / halves per expert
+  const __half* x;       // [T, K] f16
+  const uint32_t* idx;   // [assignments] expert of every assignment
+  __half* out;           // [assignments, N] f16
+  uint32_t N, K, top_k, n_experts;
+};
+
+template <int GS>
+__global__ __launch_bounds__(kThreads, 1) void qmv_m1_gate_up_kernel(M1GateUpParams p) {
+  using Image = XImage<4, 1>;
+  constexpr int kChunkK = Image::kChunkK, kLaneK = Image::kLaneK;
+  constexpr int kLanesPerGroup = GS / kLaneK, kGroupsPerChunk = kChunkK / GS;
+  extern __shared__ __attribute__((aligned(16))) char lds[];
+  const Image img(lds, p.K);
+  const uint32_t K = p.K, KH = img.KH, G = K / GS, row_u4 = K / kLaneK;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const uint32_t a = blockIdx.y, row = blockIdx.x * kWaves + wave;
+  const __half* x = p.x + (uint64_t)(a / p.top_k) * K;
+
+  // loads, small ones first (the memory counter retires in order): the expert, the activations, then the rows
+  uint32_t expert = p.idx[a];
+  const bool zeros = expert >= p.n_experts;
+  expert = zeros ? 0u : expert;
+  u4 xv[1][4];
+  load_activations<4, 1, false>(img, x, 1u, 0u, nullptr, nullptr, tid, xv);
+  struct Batch { u4 w[2][2]; uint32_t s[2][2], b[2][2]; };  // [chunk of the batch][gate, up]
+  const u4* wrow[2];
+  const unsigned short* srow[2];
+  const unsigned short* brow[2];
+#pragma unroll
+  for (int r = 0; r < 2; ++r) {
+    wrow[r] = reinterpret_cast<const u4*>((r == 0 ? p.w0 : p.w1) + expert * p.estride_w + (uint64_t)row * (K / 8));
+    srow[r] = reinterpret_cast<const unsigned short*>((r == 0 ? p.s0 : p.s1) + expert * p.estride_s) + (uint64_t)row * G;
+    brow[r] = reinterpret_cast<const unsigned short*>((r == 0 ? p.b0 : p.b1) + expert * p.estride_s) + (uint64_t)row * G;
+  }
+  auto load_batch = [&](uint32_t c0, Batch& t) {
+#pragma unroll
+    for (int cc = 0; cc < 2; ++cc) {
+      const uint32_t c = c0 + cc < KH ? c0 + cc : KH - 1;  // an odd chunk count re-reads the last chunk (unused)
+      uint32_t wi = c * 64 + lane, gi = c * kGroupsPerChunk + lane / kLanesPerGroup;
+      wi = wi < row_u4 ? wi : row_u4 - 1;  // lanes past K (last chunk of a K that is no chunk multiple)
+      gi = gi < G ? gi : G - 1;
+#pragma unroll
+      for (int r = 0; r < 2; ++r) {
+        t.s[cc][r] = srow[r][gi];
+        t.b[cc][r] = brow[r][gi];
+      }
+#pragma unroll
+      for (int r = 0; r < 2; ++r) t.w[cc][r] = __builtin_nontemporal_load(wrow[r] + wi);
+    }
+  };
+  Batch ba, bb;
+  load_batch(0, ba);
+  stage_activations<4, 1, false>(img, x, 1u, 0u, nullptr, nullptr, tid, xv);
+  __syncthreads();
+
+  float racc[2][1] = {{0.f}, {0.f}};
+  UnpackConsts uc{0x000F000Fu, 0x00F000F0u, 0x64006400u, 0x54005400u};
+  asm volatile("" : "+s"(uc.m0), "+s"(uc.m1), "+v"(uc.k0), "+v"(uc.k1));
+  auto process = [&](uint32_t c0, const Batch& t) {
+#pragma unroll
+    for (int cc = 0; cc < 2; ++cc)
+      if (c0 + cc < KH) dot_chunk<4, 2, 1>(img, c0 + cc, lane, t.w[cc], t.s[cc], t.b[cc], uc, racc);
+  };
+  for (uint32_t c0 = 0; c0 < KH; c0 += 4) {
+    const bool more1 = c0 + 2 < KH, more2 = c0 + 4 < KH;
+    if (more1) load_batch(c0 + 2, bb);
+    process(c0, ba);
+    if (more1) {
+      if (more2) load_batch(c0 + 4, ba);
+      process(c0 + 2, bb);
+    }
+  }
+  const float g = wave_sum(racc[0][0]), u = wave_sum(racc[1][0]);
+  if (lane == 0) p.out[(uint64_t)a * p.N + row] = __float2half(zeros ? 0.f : g / (1.0f + __expf(-g)) * u);
+}
+
 // LDS bytes per activation row: image and per-lane sums over whole chunks
 template <int BITS>
 size_t lds_per_row(uint32_t K) {
@@ -650,6 +736,26 @@ int32_t launch_qmv_m1(const uint32_t* w, const __half* s, const __half* b, const
   M1Params p{w, s, b, x, out, N, K, M, epi_kind, epi_dtype, epi, norm_w, inv_rms};
   if (bits == 4) launch_bits<4>(p, group_size, stream);
   else launch_bits<8>(p, group_size, stream);
+  RMLX_HIP_CHECK(hipGetLastError());
+  return RMLX_OK;
+}
+
+bool qmv_m1_gate_up_supported(uint32_t N, uint32_t K, uint32_t group_size) {
+  return group_size == 64 && qmv_m1_supported(N, K, group_size, 4);  // (what the routed block of a few tokens runs)
+}
+
+int32_t launch_qmv_m1_gate_up(const QmvArgs& a, const uint32_t* idx, uint32_t assignments, uint32_t top_k, uint32_t n_experts,
+                              hipStream_t stream) {
+  if (!qmv_m1_gate_up_supported(a.N, a.K, a.group_size))
+    return fail(RMLX_INVALID_SHAPE, "qmv_m1 gate/up: unsupported shape N=%u K=%u group_size=%u", a.N, a.K, a.group_size);
+  if (assignments == 0) return RMLX_OK;
+  if (assignments > 65535 || top_k == 0 || idx == nullptr || a.w1 == nullptr || a.out_f32 || a.ld_out != a.N)
+    return fail(RMLX_RUNTIME_ERROR, "qmv_m1 gate/up: needs an expert per assignment, both matrices and a dense f16 output");
+  M1GateUpParams p{a.w0, a.s0, a.b0, a.w1, a.s1, a.b1, a.expert_stride_w, a.expert_stride_s, a.x, idx,
+                   static_cast<__half*>(a.out), a.N, a.K, top_k, n_experts};
+  const size_t lds = lds_per_row<4>(a.K);
+  const dim3 grid(a.N / kWaves, assignments);
+  hipLaunchKernelGGL(qmv_m1_gate_up_kernel<64>, grid, dim3(kThreads), lds, stream, p);
   RMLX_HIP_CHECK(hipGetLastError());
   return RMLX_OK;
 }

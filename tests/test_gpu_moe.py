@@ -386,6 +386,33 @@ def test_moe_forward_routes_like_the_two_step_path(hip, T, E, K):
         assert np.abs(one.astype(np.float64) - two.astype(np.float64)).max() <= model.tolerance(ref)
 
 
+@pytest.mark.parametrize("T,K,E,D,I,fused", [(1, 8, 16, 1024, 1536, True), (1, 1, 4, 512, 512, False), (2, 7, 16, 512, 1024, True),
+                                              (3, 5, 8, 2048, 512, False), (2, 8, 32, 1024, 512, True), (4, 8, 128, 512, 1024, True)])
+def test_moe_forward_of_a_few_tokens(hip, T, K, E, D, I, fused):
+    """At most 32 assignments are not grouped.  Fewer than 16: a routing launch, then the gate / up projection on the
+    single-row kernel (a wave per pair of gate and up rows of the assignment's expert); from 16 on the gate / up
+    workgroups rank their token's experts themselves.  Both against the oracle and against the two-step path."""
+    from rmlx_amd import ops
+    from rmlx_amd.runtime import DeviceBuffer
+    rng = np.random.default_rng(T * 100 + K * 10 + E)
+    gate, up, down, gh, uh, dh = _experts(rng, E, D, I, fused)
+    x = make_x(rng, T, D)
+    logits = rng.standard_normal((T, E)).astype(np.float32)
+    logits[0, : min(E, 2)] = logits[0].max() + 1.0  # a tie at the top: the lower index first on every path
+    xd, ld = DeviceBuffer.from_numpy(x), DeviceBuffer.from_numpy(logits)
+    for bias in (None, rng.standard_normal(E).astype(np.float32)):
+        print(f"few tokens T={T} K={K} E={E} D={D} I={I} fused={fused} bias={bias is not None}", flush=True)
+        bd = DeviceBuffer.from_numpy(bias) if bias is not None else None
+        one = ops.moe_forward(gh, uh, dh, xd, ld, K, expert_bias=bd).numpy()
+        idx, w, _, _ = model.topk_route(logits, K, bias=bias)
+        ref = model.moe_forward(x, idx, w, gate, up, down, 64, K)
+        assert_close(one, ref, "moe_forward")
+        r = ops.gpu_topk_route(ld, K, expert_bias=bd)
+        assert np.array_equal(r.expert_indices.numpy(), idx)
+        two = ops.moe_forward_grouped(gh, uh, dh, xd, r.expert_indices, r.expert_weights, K).numpy()
+        assert np.abs(one.astype(np.float64) - two.astype(np.float64)).max() <= model.tolerance(ref)
+
+
 @pytest.mark.parametrize("T,K", [(1, 2), (1, 8), (2, 3), (3, 4)])
 def test_moe_forward_grouped_with_repeated_experts(hip, T, K):
     """Caller-supplied picks may name one expert several times for a token; decode-sized batches run kernels
