@@ -226,7 +226,8 @@ int32_t rmlx_hip_gather_qmm(const rmlx_array* x, const void* w_packed_dev, size_
                             size_t n, size_t k, size_t n_experts, uint32_t group_size,
                             void* out_f16_dev, size_t out_bytes, rmlx_stream stream);
 /* The same with the kernel family forced (the reference exposes `gather_qmm` and `gather_qmv_fast_f16_q4`
- * separately, quantized.rs:9404, 10061).  kernel: 0 = auto (streaming GEMV up to 8 rows per entry, grouped MFMA
+ * separately, quantized.rs:9404, 10061).  kernel: 0 = auto (one row per entry: the single-row GEMV with a weight
+ * matrix per activation row, N % 8 == 0, K % 32 == 0, K <= 28672; streaming GEMV up to 8 rows per entry; grouped MFMA
  * GEMM from 9 rows on where it takes the shape: N % 128 == 0, K % 512 == 0; the portable kernel for every other
  * shape), 1 = streaming GEMV (group size 64 / 128, N % 16 == 0, K % 512 == 0), 2 = grouped MFMA GEMM,
  * 3 = portable kernel. */

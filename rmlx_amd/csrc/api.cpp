@@ -1137,6 +1137,11 @@ int32_t rmlx_hip_gather_qmm_select(const rmlx_array* x, const void* w_packed_dev
     a.x = xk; a.out = out_f16_dev;
     a.tile_tab = t; a.n_tiles_dev = t + 3 * n_tiles; a.max_tiles = (uint32_t)n_tiles; a.tile_rows = tile_rows;
     RMLX_TRY(launch_qmm_rw_grouped(a, s));
+  } else if (m_per_batch == 1 && kernel == GATHER_AUTO && qmv_m1_supported(N32, K32, group_size, 4) && aligned16(w) &&
+             aligned16(sc) && aligned16(bi) && aligned16(xk)) {
+    // one row per index: the single-row kernel with a weight matrix per activation row -- one launch, no chunk table
+    RMLX_TRY(launch_qmv_m1_gather(w, sc, bi, (uint64_t)n * (k / 8), (uint64_t)n * gpr, E32, xk, idx, B32,
+                                  static_cast<__half*>(out_f16_dev), N32, K32, group_size, s));
   } else if (fast && kernel != GATHER_PORTABLE) {
     const uint64_t per = ((uint64_t)m_per_batch + 7) / 8, n_chunks = (uint64_t)B32 * per;
     if (n_chunks > 0x7FFFFFFFull) return fail(RMLX_INVALID_SHAPE, "gather_qmm: too many row chunks (%" PRIu64 ")", n_chunks);

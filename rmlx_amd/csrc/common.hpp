@@ -152,6 +152,12 @@ bool qmv_q4_supported(uint32_t N, uint32_t K, uint32_t group_size);
 // row map) through expert idx[a] of the two stacked matrices of `a` (w0 / w1, expert strides), out[a, :] = silu(gate) * up
 // in f16 [assignments, N]; 4-bit weights at group size 64, the shapes of the single-row GEMV.  chunk_tab / M / mr of `a` are not used.
 bool qmv_m1_gate_up_supported(uint32_t N, uint32_t K, uint32_t group_size);
+// gather_qmm with one activation row per index on the single-row kernel (qmv_m1.hip): x [batch, K] f16, idx [batch]
+// (outside [0, n_experts): zeros), stacked 4-bit weights with strides in u32 words / halves, out [batch, N] f16; the
+// shapes qmv_m1_supported(N, K, group_size, 4) takes
+int32_t launch_qmv_m1_gather(const uint32_t* w, const __half* s, const __half* b, uint64_t estride_w, uint64_t estride_s,
+                             uint32_t n_experts, const __half* x, const uint32_t* idx, uint32_t batch, __half* out, uint32_t N,
+                             uint32_t K, uint32_t group_size, hipStream_t stream);
 int32_t launch_qmv_m1_gate_up(const QmvArgs& a, const uint32_t* idx, uint32_t assignments, uint32_t top_k, uint32_t n_experts,
                               hipStream_t stream);
 // Wave-per-tile streaming GEMV (qmv_wt.hip): the same arguments; chunks of at most chunk_rows (8 or 16) rows, a wave owns

@@ -53,6 +53,11 @@ struct M1Params {
   // fused RMSNorm prologue (null = none): x[m,k] <- (x[m,k] * half(inv_rms[m])) * norm_w[k], each product rounded to f16
   const __half* norm_w;
   const float* inv_rms;
+  // GATHER kernels: activation row m (one row per pass) multiplies expert gather_idx[m] of stacked weights (strides in u32
+  // words / halves); an index outside [0, n_experts) writes zeros
+  const uint32_t* gather_idx;
+  uint64_t estride_w, estride_s;
+  uint32_t n_experts;
 };
 
 __device__ __forceinline__ h2 as_h2(uint32_t v) { return __builtin_bit_cast(h2, v); }
@@ -262,7 +267,9 @@ __device__ __forceinline__ void dot_chunk(const XImage<BITS, MR> g, uint32_t c, 
 // KP = waves per weight row (1, 2 or 4; split K, the counterpart of affine_qmv_splitk_f16_q4 + qmm_splitk_accum_f16,
 // quantized.rs:992-1233): wave w takes the chunks kp, kp + KP, ... of row w / KP (kp = w % KP) and the partial sums
 // meet in workgroup memory.  For long rows of a short matrix, where one wave per row leaves most of the chip idle.
-template <int BITS, int GS, int R, bool NT, int MR, bool NORM = false, int KP = 1>
+// GATHER = a weight matrix per activation row (gather_qmm with one row per index: the counterpart of
+// gather_qmv_fast_f16_q4, quantized.rs:9752-9842); MR = 1.
+template <int BITS, int GS, int R, bool NT, int MR, bool NORM = false, int KP = 1, bool GATHER = false>
 // (8-bit, one row: asking the compiler for eight waves per SIMD changes no register count but the schedule;
 // measured 4-13 % faster.  The 4-bit kernel would spill under that bound and is slower with it.  Two activation
 // rows: without a bound the scheduler spends 124 registers on a schedule that is 12 % slower than the one it finds
@@ -288,6 +295,15 @@ __global__ __launch_bounds__(kThreads, (BITS == 8 && MR == 1 && R == 1) ? 8 : (M
   // this wave's chunks: kp, kp + KP, ... (KHw of them)
   const uint32_t KHw = KP == 1 ? KH : (KH > kp ? (KH - kp + KP - 1) / KP : 0u);
   const uint32_t mrow0 = blockIdx.y * MR;  // first activation row of this pass (rows past M repeat the last one, unstored)
+  static_assert(!GATHER || (MR == 1 && KP == 1 && !NORM), "a weight matrix per activation row: one row per pass");
+  uint64_t e_w = 0, e_s = 0;
+  bool gather_zeros = false;
+  if constexpr (GATHER) {
+    const uint32_t e = p.gather_idx[mrow0];
+    gather_zeros = e >= p.n_experts;
+    e_w = gather_zeros ? 0 : e * p.estride_w;
+    e_s = gather_zeros ? 0 : e * p.estride_s;
+  }
 
   // ---- 1. loads, small ones first (the memory counter retires in order): activations ... ------
   u4 xv[MR][4];
@@ -308,9 +324,9 @@ __global__ __launch_bounds__(kThreads, (BITS == 8 && MR == 1 && R == 1) ? 8 : (M
   const unsigned short* brow[R];
 #pragma unroll
   for (int r = 0; r < R; ++r) {
-    wrow[r] = reinterpret_cast<const u4*>(p.w + (uint64_t)(row0 + r) * (K * BITS / 32));
-    srow[r] = reinterpret_cast<const unsigned short*>(p.s) + (uint64_t)(row0 + r) * G;
-    brow[r] = reinterpret_cast<const unsigned short*>(p.b) + (uint64_t)(row0 + r) * G;
+    wrow[r] = reinterpret_cast<const u4*>(p.w + e_w + (uint64_t)(row0 + r) * (K * BITS / 32));
+    srow[r] = reinterpret_cast<const unsigned short*>(p.s + e_s) + (uint64_t)(row0 + r) * G;
+    brow[r] = reinterpret_cast<const unsigned short*>(p.b + e_s) + (uint64_t)(row0 + r) * G;
   }
   auto load_batch = [&](uint32_t c0, Batch& t) {
 #pragma unroll
@@ -384,13 +400,14 @@ __global__ __launch_bounds__(kThreads, (BITS == 8 && MR == 1 && R == 1) ? 8 : (M
   if (writes && kp == 0) {  // residual add / SwiGLU gate in f32, one rounding (quantized.rs:3206-3246)
     if (p.epi_kind == EPI_RESIDUAL) mine += epi_val;
     else if (p.epi_kind == EPI_SWIGLU) mine = epi_val / (1.0f + __expf(-epi_val)) * mine;
+    if (GATHER && gather_zeros) mine = 0.f;
     p.out[(uint64_t)out_m * p.N + out_n] = __float2half(mine);
   }
 }
 
 // The same kernel for matrices with more row blocks than the chip keeps resident: the grid is sized to the resident
 // workgroups and each of them walks several row blocks (see `my_blocks`).
-template <int BITS, int GS, int R, bool NT, int MR, bool NORM = false>
+template <int BITS, int GS, int R, bool NT, int MR, bool NORM = false, bool GATHER = false>
 // (8-bit, one row: asking the compiler for eight waves per SIMD changes no register count but the schedule;
 // measured 4-13 % faster.  The 4-bit kernel would spill under that bound and is slower with it.)
 __global__ __launch_bounds__(kThreads, 1) void qmv_m1_loop_kernel(M1Params p) {
@@ -409,6 +426,15 @@ __global__ __launch_bounds__(kThreads, 1) void qmv_m1_loop_kernel(M1Params p) {
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const uint32_t mrow0 = blockIdx.y * MR;  // first activation row of this pass (rows past M repeat the last one, unstored)
+  static_assert(!GATHER || (MR == 1 && !NORM), "a weight matrix per activation row: one row per pass");
+  uint64_t e_w = 0, e_s = 0;
+  bool gather_zeros = false;
+  if constexpr (GATHER) {
+    const uint32_t e = p.gather_idx[mrow0];
+    gather_zeros = e >= p.n_experts;
+    e_w = gather_zeros ? 0 : e * p.estride_w;
+    e_s = gather_zeros ? 0 : e * p.estride_s;
+  }
   // Row blocks (kWaves * R weight rows) of this workgroup: blockIdx.x, blockIdx.x + gridDim.x, ...  The launcher
   // sizes the grid to what the chip keeps resident, so the activations are staged once per workgroup and the
   // next block's weights are already in flight while the current block is multiplied.
@@ -435,9 +461,9 @@ __global__ __launch_bounds__(kThreads, 1) void qmv_m1_loop_kernel(M1Params p) {
     const unsigned short* brow[R];
 #pragma unroll
     for (int r = 0; r < R; ++r) {
-      wrow[r] = reinterpret_cast<const u4*>(p.w + (uint64_t)(row0 + r) * (K * BITS / 32));
-      srow[r] = reinterpret_cast<const unsigned short*>(p.s) + (uint64_t)(row0 + r) * G;
-      brow[r] = reinterpret_cast<const unsigned short*>(p.b) + (uint64_t)(row0 + r) * G;
+      wrow[r] = reinterpret_cast<const u4*>(p.w + e_w + (uint64_t)(row0 + r) * (K * BITS / 32));
+      srow[r] = reinterpret_cast<const unsigned short*>(p.s + e_s) + (uint64_t)(row0 + r) * G;
+      brow[r] = reinterpret_cast<const unsigned short*>(p.b + e_s) + (uint64_t)(row0 + r) * G;
     }
     // the epilogue operand of the block's outputs travels with its first batch
     t.epi = 0.f;
@@ -504,6 +530,7 @@ __global__ __launch_bounds__(kThreads, 1) void qmv_m1_loop_kernel(M1Params p) {
       if (writes) {  // residual add / SwiGLU gate in f32, one rounding (quantized.rs:3206-3246)
         if (p.epi_kind == EPI_RESIDUAL) mine += epi_val;
         else if (p.epi_kind == EPI_SWIGLU) mine = epi_val / (1.0f + __expf(-epi_val)) * mine;
+        if (GATHER && gather_zeros) mine = 0.f;
         p.out[(uint64_t)out_m * p.N + block_row0(pr_blk) + lane / MR] = __float2half(mine);
       }
       pr_c0 = 0;
@@ -629,7 +656,7 @@ uint32_t resident_workgroups(Kernel kernel, size_t lds) {
   return cached;
 }
 
-template <int BITS, int GS, int R, bool NT, int MR, bool NORM, int KP = 1>
+template <int BITS, int GS, int R, bool NT, int MR, bool NORM, int KP = 1, bool GATHER = false>
 void launch_k(const M1Params& p, size_t lds, hipStream_t s) {
   if constexpr (KP > 1) {  // split rows: short matrices only, every row group has its workgroup
     hipLaunchKernelGGL((qmv_m1_kernel<BITS, GS, R, NT, MR, NORM, KP>), dim3(p.N / (kWaves / KP), (p.M + MR - 1) / MR),
@@ -637,14 +664,14 @@ void launch_k(const M1Params& p, size_t lds, hipStream_t s) {
     return;
   }
   // one workgroup per row block while all of them are resident together, else as many as are (they loop)
-  auto looping = qmv_m1_loop_kernel<BITS, GS, R, NT, MR, NORM>;
+  auto looping = qmv_m1_loop_kernel<BITS, GS, R, NT, MR, NORM, GATHER>;
   const uint32_t nblk = p.N / (kWaves * R), passes = (p.M + MR - 1) / MR;
   uint32_t gx = resident_workgroups(looping, lds) / passes;
   gx = gx < 1 ? 1 : gx;
   // (as many workgroups as are resident, even where that leaves some of them one block more than others: fewer
   // workgroups with equal shares are slower, 8.1 against 6.7 us at N = 9216)
   if (gx < nblk) hipLaunchKernelGGL(looping, dim3(gx, passes), dim3(kThreads), lds, s, p);
-  else hipLaunchKernelGGL((qmv_m1_kernel<BITS, GS, R, NT, MR, NORM>), dim3(nblk, passes), dim3(kThreads), lds, s, p);
+  else hipLaunchKernelGGL((qmv_m1_kernel<BITS, GS, R, NT, MR, NORM, 1, GATHER>), dim3(nblk, passes), dim3(kThreads), lds, s, p);
 }
 
 template <int BITS, int R, bool NT, int MR, int KP = 1>
@@ -737,6 +764,30 @@ int32_t launch_qmv_m1(const uint32_t* w, const __half* s, const __half* b, const
   if (bits == 4) launch_bits<4>(p, group_size, stream);
   else launch_bits<8>(p, group_size, stream);
   RMLX_HIP_CHECK(hipGetLastError());
+  return RMLX_OK;
+}
+
+// gather_qmm with one activation row per index: row m of x [batch, K] through expert idx[m] of the stacked 4-bit
+// weights, out [batch, N] f16.  One launch, no chunk table: the activation row of a pass picks its matrix.
+int32_t launch_qmv_m1_gather(const uint32_t* w, const __half* s, const __half* b, uint64_t estride_w, uint64_t estride_s,
+                             uint32_t n_experts, const __half* x, const uint32_t* idx, uint32_t batch, __half* out, uint32_t N,
+                             uint32_t K, uint32_t group_size, hipStream_t stream) {
+  if (!qmv_m1_supported(N, K, group_size, 4))
+    return fail(RMLX_INVALID_SHAPE, "qmv_m1 gather: unsupported shape N=%u K=%u group_size=%u", N, K, group_size);
+  const size_t lds = lds_per_row<4>(K);
+  // (weights loaded with the ordinary cache policy: two indices may name one expert)
+  const bool two = (K >= 12288 || N >= 12288) && N % (kWaves * 2) == 0;
+  for (uint32_t first = 0; first < batch; first += 65535) {  // the activation row is the second grid dimension
+    const uint32_t rows = batch - first < 65535 ? batch - first : 65535;
+    M1Params p{w, s, b, x + (uint64_t)first * K, out + (uint64_t)first * N, N, K, rows, EPI_NONE, 0, nullptr, nullptr, nullptr,
+               idx + first, estride_w, estride_s, n_experts};
+    switch (group_size) {
+      case 32: if (two) launch_k<4, 32, 2, false, 1, false, 1, true>(p, lds, stream); else launch_k<4, 32, 1, false, 1, false, 1, true>(p, lds, stream); break;
+      case 64: if (two) launch_k<4, 64, 2, false, 1, false, 1, true>(p, lds, stream); else launch_k<4, 64, 1, false, 1, false, 1, true>(p, lds, stream); break;
+      default: if (two) launch_k<4, 128, 2, false, 1, false, 1, true>(p, lds, stream); else launch_k<4, 128, 1, false, 1, false, 1, true>(p, lds, stream); break;
+    }
+    RMLX_HIP_CHECK(hipGetLastError());
+  }
   return RMLX_OK;
 }
 

@@ -223,6 +223,40 @@ def test_gather_qmm_group_size_32_streams_on_the_wave_per_tile_kernel(hip, n, k,
     assert_close(ops.gather_qmm(xd, wd, sd, bd, idd, batch, mpb, n, k, E, 32, kernel=rt.GATHER_PORTABLE).numpy(), ref, "gather_qmm gs32 (portable)")
 
 
+@pytest.mark.parametrize("n,k,gs,batch", [(64, 512, 64, 9), (8, 32, 32, 5), (256, 4096, 64, 33), (128, 1056, 32, 4), (48, 2048, 128, 7),
+                                          (16384, 512, 64, 3), (64, 12288, 64, 2), (8, 64, 64, 70000)])
+def test_gather_qmm_of_single_rows(hip, n, k, gs, batch):
+    """One activation row per index (the reference's gather_qmv_fast_f16_q4 case): the single-row kernel with a weight
+    matrix per activation row -- one launch, whole-row contiguous loads.  Against the oracle and the other kernels;
+    repeated experts, the looping and the two-rows-per-wave forms, more entries than one grid dimension holds; on a
+    stream, rows of an out-of-range index are zero."""
+    from rmlx_amd import ops, runtime as rt
+    from rmlx_amd.runtime import DeviceBuffer, Stream
+    rng = np.random.default_rng(n + k + gs + batch)
+    E = 6
+    words, s, b = make_weight(rng, n, k, 4, gs, lead=(E,))
+    x = rng.standard_normal((batch, 1, k)).astype(np.float16)
+    idx = rng.integers(0, E, size=batch).astype(np.uint32)
+    idx[: min(batch, 2)] = 3  # one expert twice
+    print(f"gather_qmm single rows n={n} k={k} gs={gs} batch={batch}", flush=True)
+    xd, wd, sd, bd = [DeviceBuffer.from_numpy(a) for a in (x, words, s, b)]
+    ref = model.gather_qmm(x, words, s, b, idx, gs)
+    out = ops.gather_qmm(xd, wd, sd, bd, DeviceBuffer.from_numpy(idx), batch, 1, n, k, E, gs).numpy()
+    assert_close(out, ref, "gather_qmm (single-row kernel)")
+    if batch <= 64:
+        port = ops.gather_qmm(xd, wd, sd, bd, DeviceBuffer.from_numpy(idx), batch, 1, n, k, E, gs, kernel=rt.GATHER_PORTABLE).numpy()
+        assert np.abs(out.astype(np.float64) - port.astype(np.float64)).max() <= model.tolerance(ref)
+    bad = idx.copy()
+    bad[batch // 2] = E + 3
+    st = Stream()
+    o = ops.gather_qmm(xd, wd, sd, bd, DeviceBuffer.from_numpy(bad), batch, 1, n, k, E, gs, stream=st)
+    st.sync()
+    o = o.numpy()
+    assert np.all(o[batch // 2] == 0)
+    keep = np.arange(batch) != batch // 2
+    assert np.array_equal(o[keep], out[keep])
+
+
 def test_gather_qmm_validation(hip):
     """The reference's argument-validation tests (quantized.rs:11088-11540)."""
     from rmlx_amd import ops
