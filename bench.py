@@ -519,7 +519,7 @@ def main():
                 r["hbm_frac"] = r["gbs"] / HBM_PEAK_GBS
                 extra[f"gather_qmm_q4_b{batch}_m{mpb}"] = r
         if "moe" in sections:
-            for T in (1, 4, 32, 128, 512, 2048):  # from 10 rows per expert on average on the grouped MFMA GEMM
+            for T in (1, 4, 8, 32, 128, 512, 2048):  # from 10 rows per expert on average on the grouped MFMA GEMM
                 r = bench_moe(ops, rt, timer, rng, T, calls if T <= 128 else max(50, calls // 4), experts)
                 r["tflops"] = r["flops"] / (r["us"] * 1e-6) / 1e12
                 r["mfma_frac"] = r["tflops"] / MFMA_F16_PEAK_TF

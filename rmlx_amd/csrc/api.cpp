@@ -2,6 +2,7 @@
 // points), the dispatch ladder, and the composition of the MoE block.  No arithmetic happens
 // here and there is no CPU fallback: every path ends in a HIP kernel launch or an error.
 #include <cinttypes>
+#include <cmath>
 #include <cstring>
 #include <map>
 #include <mutex>
@@ -462,7 +463,16 @@ struct ExpertShapes {
 constexpr uint32_t kGatherGemmMinRows = 9;
 // routed block: up to this many assignments run without grouping (every assignment its own chunk, combine fused into
 // the down projection)
-constexpr uint32_t kDirectMaxAssignments = 32;
+constexpr uint32_t kDirectMaxAssignments = 128;
+// The form without grouping streams an expert once per assignment instead of once per distinct expert of the batch (at
+// about 6 against 5 TB/s, and without the grouping launch): worth it while the assignments are at most 1.3 x the distinct
+// experts a uniform router picks, E (1 - (1 - K/E)^T).  Measured at E = 128, top-8: 9 tokens 127 against 137 us, 10 tokens
+// 141 against 141, 12 tokens 170 against 162.
+bool ungrouped_pays(uint32_t T, uint32_t E, uint32_t K) {
+  if (E == 0 || K > E) return false;
+  const double distinct = E * (1.0 - std::pow(1.0 - (double)K / E, (double)T));
+  return (uint64_t)T * K <= kDirectMaxAssignments && (double)T * K <= 1.3 * distinct;
+}
 constexpr uint32_t kOwnRouteMinAssignments = 16;  // from here on the gate / up launch of that path routes by itself
 enum { GATHER_AUTO = 0, GATHER_STREAM = 1, GATHER_GEMM = 2, GATHER_PORTABLE = 3 };
 
@@ -608,13 +618,10 @@ QmvArgs gate_up_args(const rmlx_qweight* gate, const rmlx_qweight* up, const Exp
 }
 
 // gate/up + SwiGLU then down, over a device chunk table.  h: f16 [positions, I] scratch.
-// `own_route` (with top_k): no table -- the gate / up workgroups rank their token's experts themselves; position
-// t * top_k + k is pick k of token t (4-bit K-split kernel only: plan.gate_up == 0), max_chunks = T * top_k.
 int32_t run_expert_ffn(const rmlx_qweight* gate, const rmlx_qweight* up, const rmlx_qweight* down,
                        const ExpertShapes& sh, const __half* x, const uint32_t* row_map,
                        const uint32_t* chunk_tab, const uint32_t* n_chunks, uint32_t max_chunks, __half* h,
-                       void* y, int y_f32, uint32_t gemm_tile_rows, const StreamPlan& plan, hipStream_t stream,
-                       const FusedRoute* own_route = nullptr, uint32_t top_k = 0) {
+                       void* y, int y_f32, uint32_t gemm_tile_rows, const StreamPlan& plan, hipStream_t stream) {
   const uint32_t per = 32 / gate->bits;  // values per u32 word: 8 (4-bit) or 4 (8-bit)
   if (gemm_tile_rows != 0) {  // the table holds row tiles of that many rows and n_chunks its length
     const uint32_t gs = gate->group_size;  // one group size for the three projections (ExpertShapes::gemm)
@@ -646,13 +653,6 @@ int32_t run_expert_ffn(const rmlx_qweight* gate, const rmlx_qweight* up, const r
   QmvArgs a = gate_up_args(gate, up, sh, x, h);
   a.row_map = row_map;
   a.chunk_tab = chunk_tab; a.n_chunks_dev = n_chunks; a.max_chunks = max_chunks; a.mr = 8;
-  if (own_route != nullptr) {
-    if (plan.gate_up != 0 || gate->bits != 4 || y != nullptr)
-      return fail(RMLX_RUNTIME_ERROR, "expert FFN: routing inside the gate / up launch is for the 4-bit K-split kernel");
-    a.route_logits = own_route->logits; a.route_bias = own_route->bias;
-    a.route_idx_out = own_route->idx_out; a.route_w_out = own_route->w_out;
-    a.route_e = sh.E; a.route_k = top_k; a.route_renorm = 1;
-  }
   // (the table holds chunks of at most plan.chunk_rows rows)
   if (plan.gate_up != 0) RMLX_TRY(launch_qmv_wt(a, plan.gate_up, stream));
   else RMLX_TRY(gate->bits == 8 ? launch_qmv_q8_tab(a, stream) : launch_qmv_q4(a, stream));
@@ -1387,6 +1387,22 @@ int32_t moe_grouped_impl(const rmlx_qweight* gate, const rmlx_qweight* up, const
   RMLX_TRY(checked_u32(T * top_k, "seq_len * top_k", &A));
   RMLX_TRY(check_out("MoeLayer", out_bytes, T * sh.D * 2));
   if (T == 0) return RMLX_OK;
+  hipStream_t s = (hipStream_t)stream;
+  // Which form a call that brings logits takes.  `direct`: a few tokens, no grouping at all (below).  `own`: the gate / up
+  // workgroups of that form rank their token's experts themselves, so any number of tokens.  `small`: at most 8 tokens,
+  // which the one-workgroup routing launches (with or without grouping behind) take.  Everything else routes with the
+  // routing kernel and goes on as if the caller had brought the picks.
+  const bool single_row = gate->bits == 4 && qmv_m1_gate_up_supported(sh.I, sh.D, gate->group_size);
+  bool direct = route != nullptr && ungrouped_pays(T32, sh.E, (uint32_t)top_k) && sh.stream_kernel != 1 && sh.wave_down &&
+                qmv_wt_combine_supported(sh.D, sh.I, down->group_size, (uint32_t)top_k);
+  const bool own = direct && single_row && sh.E <= 256 && A >= kOwnRouteMinAssignments;
+  const bool small = route != nullptr && T32 <= 8 && route_sort_fusable(T32, sh.E, (uint32_t)top_k);
+  if (direct && !own && !small) direct = false;
+  if (route != nullptr && !direct && !small) {
+    RMLX_TRY(launch_topk_route(route->logits, route->bias, T32, sh.E, (uint32_t)top_k, 1, route->idx_out, route->w_out, nullptr,
+                               nullptr, s));
+    route = nullptr;
+  }
   // many rows per expert: the grouped GEMM over row tiles instead of the streaming GEMV over chunks of 8 rows
   const uint32_t gemm = route == nullptr ? expert_gemm_tile_rows(sh, A, sh.E) : 0u;
   StreamPlan plan = expert_stream_plan(sh, A, sh.E);
@@ -1399,7 +1415,6 @@ int32_t moe_grouped_impl(const rmlx_qweight* gate, const rmlx_qweight* up, const
   const uint32_t max_chunks = A / chunk_rows + (A < sh.E ? A : sh.E);
   if (max_chunks > 65535) return fail(RMLX_INVALID_SHAPE, "MoeLayer: too many row chunks (%u); split the batch", max_chunks);
 
-  hipStream_t s = (hipStream_t)stream;
   Scratch cast, meta, h, y;
   const __half* xk = static_cast<const __half*>(x->data);
   if (x->dtype != RMLX_DTYPE_F16) {
@@ -1433,20 +1448,22 @@ int32_t moe_grouped_impl(const rmlx_qweight* gate, const rmlx_qweight* up, const
     return finish(s);
   }
   if (!aligned16(xk)) return fail(RMLX_INVALID_SHAPE, "MoeLayer: input must be 16-byte aligned");
-  // A few tokens (at most 32 assignments), routed here: no grouping at all.  Every assignment is a chunk of one row in
-  // assignment order, and the down projection adds the token's weighted expert outputs itself - three launches (routing,
-  // gate / up, down + combine) instead of four, no [assignments, D] intermediate.  An expert picked by two tokens is
-  // streamed once per token (at 4 tokens of 8 picks over 128 experts: 32 chunks for 31 experts).
-  if (route != nullptr && A <= kDirectMaxAssignments && sh.stream_kernel != 1 && sh.wave_down &&
-      qmv_wt_combine_supported(sh.D, sh.I, down->group_size, (uint32_t)top_k)) {
+  // A few tokens, routed here: no grouping at all.  Every assignment is one row in assignment order, and the down
+  // projection adds the token's weighted expert outputs itself - two or three launches (routing, gate / up, down +
+  // combine) instead of four, no [assignments, D] intermediate.  An expert picked by two tokens is streamed once per
+  // token (at 4 tokens of 8 picks over 128 experts: 32 rows for 31 experts; see ungrouped_pays).
+  if (direct) {
     RMLX_TRY(h.alloc((size_t)A * sh.I * 2, s, arena));
-    if (sh.E <= 256 && A >= kOwnRouteMinAssignments) {
-      // two launches: the gate / up workgroups rank their own token's experts (one wave, while the others wait).  The
-      // ranking then sits in front of every workgroup's weight stream: it pays once the grid is several rounds of
-      // workgroups (2 tokens of 8 picks: 36.4 against 38.0 us, 4 tokens: 62.1 against 64.2 us) and costs where the grid
-      // is a single round (1 token: 26.0 against 25.3 us).
-      RMLX_TRY(run_expert_ffn(gate, up, down, sh, xk, nullptr, nullptr, nullptr, A, static_cast<__half*>(h.ptr), nullptr, 0, 0,
-                              StreamPlan{0, 0, 8}, s, route, (uint32_t)top_k));
+    // One row per expert: the gate / up projection on the single-row GEMV's layout (a wave per pair of gate and up rows,
+    // dot products instead of a matrix unit that would multiply 15 empty rows) where it takes the shape.  From 16
+    // assignments on its workgroups rank their token's experts themselves (one wave, while the activations arrive) --
+    // two launches; the ranking then stands in front of every workgroup's weight stream, which pays once a workgroup
+    // walks several row blocks (2 / 3 / 4 tokens of 8 picks) and costs where it has one or two (1 token).
+    if (own) {
+      QmvArgs a = gate_up_args(gate, up, sh, xk, static_cast<__half*>(h.ptr));
+      a.route_logits = route->logits; a.route_bias = route->bias; a.route_idx_out = route->idx_out; a.route_w_out = route->w_out;
+      a.route_renorm = 1;
+      RMLX_TRY(launch_qmv_m1_gate_up(a, nullptr, A, (uint32_t)top_k, sh.E, s));
     } else {
       RMLX_TRY(meta.alloc(((size_t)4 * A + 4) * 4, s, arena));  // tok[A] | chunk_tab[3 A] | n_chunks[1]
       uint32_t* tok = static_cast<uint32_t*>(meta.ptr);
@@ -1454,12 +1471,10 @@ int32_t moe_grouped_impl(const rmlx_qweight* gate, const rmlx_qweight* up, const
       uint32_t* n_chunks = chunk_tab + 3 * (size_t)A;
       RMLX_TRY(launch_route_direct_small(route->logits, route->bias, T32, sh.E, (uint32_t)top_k, 1, route->idx_out, route->w_out,
                                          tok, chunk_tab, n_chunks, s));
-      // one row per expert: the single-row GEMV's layout (a wave per weight row pair, dot products instead of a matrix
-      // unit that would multiply 15 empty rows) where it takes the shape, else the K-split kernel over one-row chunks
-      if (gate->bits == 4 && qmv_m1_gate_up_supported(sh.I, sh.D, gate->group_size))
+      if (single_row)
         RMLX_TRY(launch_qmv_m1_gate_up(gate_up_args(gate, up, sh, xk, static_cast<__half*>(h.ptr)), route->idx_out, A,
                                        (uint32_t)top_k, sh.E, s));
-      else
+      else  // the K-split kernel over one-row chunks
         RMLX_TRY(run_expert_ffn(gate, up, down, sh, xk, tok, chunk_tab, n_chunks, A, static_cast<__half*>(h.ptr), nullptr, 0, 0,
                                 StreamPlan{0, 0, 8}, s));
     }
@@ -1565,11 +1580,11 @@ int32_t moe_forward_impl(const rmlx_qweight* gate, const rmlx_qweight* up, const
   RMLX_TRY(route.alloc(T * top_k * 8 + 16, s, arena));
   uint32_t* idx = static_cast<uint32_t*>(route.ptr);
   float* wts = reinterpret_cast<float*>(idx + T * top_k);
-  // Decode-sized batches with f32 logits: routing and grouping share one launch.
+  // f32 logits (and bias): the block picks its routed form itself (moe_grouped_impl)
   if (gate != nullptr && gate_logits->dtype == RMLX_DTYPE_F32 && gate_logits->data != nullptr && top_k <= gate->n_experts &&
       (expert_bias == nullptr || (expert_bias->dtype == RMLX_DTYPE_F32 && expert_bias->ndim == 1 &&
                                   expert_bias->shape[0] == gate->n_experts && expert_bias->data != nullptr)) &&
-      T <= 8 && route_sort_fusable((uint32_t)T, (uint32_t)gate->n_experts, (uint32_t)top_k)) {
+      gate->n_experts <= 256) {
     const FusedRoute fr{static_cast<const float*>(gate_logits->data),
                         expert_bias != nullptr ? static_cast<const float*>(expert_bias->data) : nullptr, idx, wts};
     return moe_grouped_impl(gate, up, down, x, idx, wts, top_k, out_f16_dev, out_bytes, stream, &fr, arena);

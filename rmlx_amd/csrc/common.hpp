@@ -140,16 +140,15 @@ struct QmvArgs {
   uint32_t M;                // used when chunk_tab == null
   uint32_t mr;               // rows staged per chunk (1,2,4,8); 0 -> derive from M
   uint32_t group_size;       // 64 (also when 0) or 128
-  // launch_qmv_q4 only: the workgroups route their own token (no chunk table): chunk c of the max_chunks = T * route_k
-  // is pick c % route_k of token c / route_k, its activation row is the token, its output row is c; f32 logits
-  // [T, route_e], optional bias; the picks and normalised weights are also written to route_idx_out / route_w_out
+  // launch_qmv_m1_gate_up without an index list only: the workgroups rank their own token's experts from f32 logits
+  // [T, n_experts] (+ optional bias) and also write the picks and normalised weights to route_idx_out / route_w_out
   const float* route_logits; const float* route_bias; uint32_t* route_idx_out; float* route_w_out;
-  uint32_t route_e, route_k; int32_t route_renorm;
+  int32_t route_renorm;
 };
 int32_t launch_qmv_q4(const QmvArgs& a, hipStream_t s);
 bool qmv_q4_supported(uint32_t N, uint32_t K, uint32_t group_size);
 // Gate / up projection of single rows through chosen experts (qmv_m1.hip): position a = activation row a / top_k (x, no
-// row map) through expert idx[a] of the two stacked matrices of `a` (w0 / w1, expert strides), out[a, :] = silu(gate) * up
+// row map) through expert idx[a] (idx == null: pick a % top_k of the ranking the kernel makes itself, see route_logits) of the two stacked matrices of `a` (w0 / w1, expert strides), out[a, :] = silu(gate) * up
 // in f16 [assignments, N]; 4-bit weights at group size 64, the shapes of the single-row GEMV.  chunk_tab / M / mr of `a` are not used.
 bool qmv_m1_gate_up_supported(uint32_t N, uint32_t K, uint32_t group_size);
 // gather_qmm with one activation row per index on the single-row kernel (qmv_m1.hip): x [batch, K] f16, idx [batch]

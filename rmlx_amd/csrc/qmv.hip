@@ -38,7 +38,6 @@
 //     tiles requests the next tile's weights as soon as the current accumulators have left for LDS.
 #include "common.hpp"
 #include "q4_stream.hpp"
-#include "route.hpp"
 
 namespace rmlx {
 namespace {
@@ -68,15 +67,6 @@ struct KParams {
   const uint32_t* chunk_tab;
   const uint32_t* n_chunks;
   uint64_t estride_w, estride_s;
-  // Routing done by the workgroup itself (a few tokens, no chunk table): chunk blockIdx.y is assignment a = token
-  // a / route_k, pick a % route_k; f32 logits [T, route_e], optional bias [route_e]; the picks and weights of every
-  // token are written once, by the first workgroup of its first assignment.
-  const float* route_logits;
-  const float* route_bias;
-  uint32_t* route_idx_out;
-  float* route_w_out;
-  uint32_t route_e, route_k;
-  int32_t route_renorm;
 };
 
 
@@ -115,34 +105,8 @@ __global__ __launch_bounds__(kThreads, (REUSE != 0 && MR == 8 && TILES == 2) ? 4
 
   // ---- which rows -----------------------------------------------------------------------
   uint32_t expert = 0, row0 = blockIdx.y * 8, rows;
-  uint32_t routed_token = 0xFFFFFFFFu;  // (routing here: the one activation row of the chunk)
   bool write_zeros = false;
-  if (TAB && p.route_logits != nullptr) {
-    // One wave ranks the token's experts (the same instructions as the routing kernel: the same picks and weights);
-    // an expert index out of range cannot come out of it, but a token with fewer than route_k experts to pick from
-    // leaves picks empty: those chunks write zeros.
-    __shared__ uint32_t picks[8];
-    const uint32_t a = blockIdx.y, t = a / p.route_k, pick = a - t * p.route_k;
-    if (wave == 0) {
-      uint32_t my_idx;
-      float my_w;
-      route::token_picks(p.route_logits, p.route_bias, p.route_e, p.route_k, p.route_renorm, t, (uint32_t)lane, my_idx, my_w);
-      if ((uint32_t)lane < p.route_k) {
-        picks[lane] = my_idx;
-        if (blockIdx.x == 0 && pick == 0) {
-          p.route_idx_out[(size_t)t * p.route_k + lane] = my_idx;
-          p.route_w_out[(size_t)t * p.route_k + lane] = my_w;
-        }
-      }
-    }
-    __syncthreads();
-    expert = picks[pick];
-    write_zeros = expert >= p.route_e;
-    if (write_zeros) expert = 0;
-    row0 = a;
-    rows = 1;
-    routed_token = t;
-  } else if (TAB) {
+  if (TAB) {
     if (p.n_chunks != nullptr && blockIdx.y >= *p.n_chunks) return;
     expert = p.chunk_tab[3 * blockIdx.y + 0];
     row0 = p.chunk_tab[3 * blockIdx.y + 1];
@@ -168,7 +132,6 @@ __global__ __launch_bounds__(kThreads, (REUSE != 0 && MR == 8 && TILES == 2) ? 4
     srcs[m] = row0 + m;
     if (TAB && p.row_map != nullptr && (uint32_t)m < rows) srcs[m] = p.row_map[row0 + m];
   }
-  if (TAB && routed_token != 0xFFFFFFFFu) srcs[0] = routed_token;
 
   // A-operand activity: accumulator rows 0-7 take group 0 (g<2), rows 8-15 group 1 (g>=2).
   const int am = n & 7;
@@ -590,12 +553,7 @@ int32_t launch_qmv_q4(const QmvArgs& a, hipStream_t s) {
   p.out = a.out; p.estride_w = a.expert_stride_w; p.estride_s = a.expert_stride_s;
   p.K = a.K; p.ld_out = a.ld_out; p.M = a.M; p.out_f32 = a.out_f32;
   p.gs128 = a.group_size == 128 ? 1u : 0u;
-  p.route_logits = a.route_logits; p.route_bias = a.route_bias; p.route_idx_out = a.route_idx_out; p.route_w_out = a.route_w_out;
-  p.route_e = a.route_e; p.route_k = a.route_k; p.route_renorm = a.route_renorm;
-  if (a.route_logits != nullptr && (a.route_k == 0 || a.route_k > 8 || a.route_e == 0 || a.route_e > 256 || a.route_idx_out == nullptr ||
-                                    a.route_w_out == nullptr || a.max_chunks == 0 || a.max_chunks % a.route_k != 0))
-    return fail(RMLX_RUNTIME_ERROR, "qmv_q4: routing in the kernel takes 1..8 picks of at most 256 experts and a grid of whole tokens");
-  const bool tab = a.chunk_tab != nullptr || a.route_logits != nullptr;
+  const bool tab = a.chunk_tab != nullptr;
   uint32_t chunks = tab ? a.max_chunks : (a.M + 7) / 8;
   if (chunks == 0) return RMLX_OK;
   // k-parts per pass: 8 for K >= 4096; for smaller K the fewest parts of at most 4 slabs each,

@@ -31,6 +31,7 @@
 //     blocks with the next block's weights in flight.  Long rows of a short matrix split K over 2 or
 //     4 waves of the workgroup.
 #include "common.hpp"
+#include "route.hpp"
 
 namespace rmlx {
 namespace {
@@ -562,7 +563,36 @@ struct M1GateUpParams {
   const uint32_t* idx;   // [assignments] expert of every assignment
   __half* out;           // [assignments, N] f16
   uint32_t N, K, top_k, n_experts;
+  // Routing done by the workgroups themselves (idx == null): f32 logits [T, n_experts], optional bias [n_experts]; every
+  // workgroup ranks its token's experts (one wave, the routing kernels' own code, while the activations arrive), and the
+  // first workgroup of a token's first assignment also writes the token's picks and weights
+  const float* route_logits;
+  const float* route_bias;
+  uint32_t* route_idx_out;
+  float* route_w_out;
+  int32_t route_renorm;
 };
+
+// The expert of assignment a: from the list, or ranked here (after the caller has requested its activations).
+__device__ __forceinline__ uint32_t gate_up_expert(const M1GateUpParams& p, uint32_t a, int wave, int lane, bool first_wg) {
+  if (p.idx != nullptr) return p.idx[a];
+  __shared__ uint32_t picks[8];
+  const uint32_t t = a / p.top_k, pick = a - t * p.top_k;
+  if (wave == 0) {
+    uint32_t my_idx;
+    float my_w;
+    route::token_picks(p.route_logits, p.route_bias, p.n_experts, p.top_k, p.route_renorm, t, (uint32_t)lane, my_idx, my_w);
+    if ((uint32_t)lane < p.top_k) {
+      picks[lane] = my_idx;
+      if (first_wg && pick == 0) {
+        p.route_idx_out[(size_t)t * p.top_k + lane] = my_idx;
+        p.route_w_out[(size_t)t * p.top_k + lane] = my_w;
+      }
+    }
+  }
+  __syncthreads();
+  return picks[pick];
+}
 
 template <int GS>
 __global__ __launch_bounds__(kThreads, 1) void qmv_m1_gate_up_kernel(M1GateUpParams p) {
@@ -576,12 +606,12 @@ __global__ __launch_bounds__(kThreads, 1) void qmv_m1_gate_up_kernel(M1GateUpPar
   const uint32_t a = blockIdx.y, row = blockIdx.x * kWaves + wave;
   const __half* x = p.x + (uint64_t)(a / p.top_k) * K;
 
-  // loads, small ones first (the memory counter retires in order): the expert, the activations, then the rows
-  uint32_t expert = p.idx[a];
-  const bool zeros = expert >= p.n_experts;
-  expert = zeros ? 0u : expert;
+  // loads, small ones first (the memory counter retires in order): the activations, the expert, then the rows
   u4 xv[1][4];
   load_activations<4, 1, false>(img, x, 1u, 0u, nullptr, nullptr, tid, xv);
+  uint32_t expert = gate_up_expert(p, a, wave, lane, blockIdx.x == 0);
+  const bool zeros = expert >= p.n_experts;
+  expert = zeros ? 0u : expert;
   struct Batch { u4 w[2][2]; uint32_t s[2][2], b[2][2]; };  // [chunk of the batch][gate, up]
   const u4* wrow[2];
   const unsigned short* srow[2];
@@ -632,6 +662,93 @@ __global__ __launch_bounds__(kThreads, 1) void qmv_m1_gate_up_kernel(M1GateUpPar
   }
   const float g = wave_sum(racc[0][0]), u = wave_sum(racc[1][0]);
   if (lane == 0) p.out[(uint64_t)a * p.N + row] = __float2half(zeros ? 0.f : g / (1.0f + __expf(-g)) * u);
+}
+
+// The same for more row blocks than the chip keeps resident (a few tokens: assignments x N / 8 blocks): the grid is
+// (resident workgroups / assignments, assignments) and a workgroup walks the row blocks blockIdx.x, blockIdx.x + gridDim.x,
+// ... of its assignment, staging the activations once, the next block's weights in flight while the current one is multiplied.
+template <int GS>
+__global__ __launch_bounds__(kThreads, 1) void qmv_m1_gate_up_loop_kernel(M1GateUpParams p) {
+  using Image = XImage<4, 1>;
+  constexpr int kChunkK = Image::kChunkK, kLaneK = Image::kLaneK;
+  constexpr int kLanesPerGroup = GS / kLaneK, kGroupsPerChunk = kChunkK / GS;
+  extern __shared__ __attribute__((aligned(16))) char lds[];
+  const Image img(lds, p.K);
+  const uint32_t K = p.K, KH = img.KH, G = K / GS, row_u4 = K / kLaneK;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const uint32_t a = blockIdx.y;
+  const __half* x = p.x + (uint64_t)(a / p.top_k) * K;
+  const uint32_t nblk = p.N / kWaves;
+  const uint32_t my_blocks = blockIdx.x < nblk ? (nblk - 1 - blockIdx.x) / gridDim.x + 1 : 0u;
+  auto block_row = [&](uint32_t i) { return (blockIdx.x + i * gridDim.x) * kWaves + wave; };
+
+  u4 xv[1][4];
+  load_activations<4, 1, false>(img, x, 1u, 0u, nullptr, nullptr, tid, xv);
+  uint32_t expert = gate_up_expert(p, a, wave, lane, blockIdx.x == 0);
+  const bool zeros = expert >= p.n_experts;
+  expert = zeros ? 0u : expert;
+  struct Batch { u4 w[2][2]; uint32_t s[2][2], b[2][2]; };  // [chunk of the batch][gate, up]
+  const uint32_t batches_per_block = (KH + 1) / 2, n_batches = my_blocks * batches_per_block;
+  uint32_t ld_blk = 0, ld_c0 = 0;  // block and first chunk of the next batch to load
+  auto load_batch = [&](Batch& t) {
+    const uint32_t row = block_row(ld_blk);
+    const u4* wrow[2];
+    const unsigned short* srow[2];
+    const unsigned short* brow[2];
+#pragma unroll
+    for (int r = 0; r < 2; ++r) {
+      wrow[r] = reinterpret_cast<const u4*>((r == 0 ? p.w0 : p.w1) + expert * p.estride_w + (uint64_t)row * (K / 8));
+      srow[r] = reinterpret_cast<const unsigned short*>((r == 0 ? p.s0 : p.s1) + expert * p.estride_s) + (uint64_t)row * G;
+      brow[r] = reinterpret_cast<const unsigned short*>((r == 0 ? p.b0 : p.b1) + expert * p.estride_s) + (uint64_t)row * G;
+    }
+#pragma unroll
+    for (int cc = 0; cc < 2; ++cc) {
+      const uint32_t c = ld_c0 + cc < KH ? ld_c0 + cc : KH - 1;  // an odd chunk count re-reads the last chunk (unused)
+      uint32_t wi = c * 64 + lane, gi = c * kGroupsPerChunk + lane / kLanesPerGroup;
+      wi = wi < row_u4 ? wi : row_u4 - 1;  // lanes past K (last chunk of a K that is no chunk multiple)
+      gi = gi < G ? gi : G - 1;
+#pragma unroll
+      for (int r = 0; r < 2; ++r) {
+        t.s[cc][r] = srow[r][gi];
+        t.b[cc][r] = brow[r][gi];
+      }
+#pragma unroll
+      for (int r = 0; r < 2; ++r) t.w[cc][r] = __builtin_nontemporal_load(wrow[r] + wi);
+    }
+    ld_c0 += 2;
+    if (ld_c0 >= KH) { ld_c0 = 0; ++ld_blk; }
+  };
+  Batch ba, bb;
+  if (n_batches > 0) load_batch(ba);
+  stage_activations<4, 1, false>(img, x, 1u, 0u, nullptr, nullptr, tid, xv);
+  __syncthreads();
+
+  float racc[2][1];
+  UnpackConsts uc{0x000F000Fu, 0x00F000F0u, 0x64006400u, 0x54005400u};
+  asm volatile("" : "+s"(uc.m0), "+s"(uc.m1), "+v"(uc.k0), "+v"(uc.k1));
+  uint32_t pr_blk = 0, pr_c0 = 0;  // block and first chunk of the batch being processed
+  auto process = [&](const Batch& t) {
+    if (pr_c0 == 0) { racc[0][0] = 0.f; racc[1][0] = 0.f; }
+#pragma unroll
+    for (int cc = 0; cc < 2; ++cc)
+      if (pr_c0 + cc < KH) dot_chunk<4, 2, 1>(img, pr_c0 + cc, lane, t.w[cc], t.s[cc], t.b[cc], uc, racc);
+    pr_c0 += 2;
+    if (pr_c0 >= KH) {  // the block is complete
+      const float g = wave_sum(racc[0][0]), u = wave_sum(racc[1][0]);
+      if (lane == 0) p.out[(uint64_t)a * p.N + block_row(pr_blk)] = __float2half(zeros ? 0.f : g / (1.0f + __expf(-g)) * u);
+      pr_c0 = 0;
+      ++pr_blk;
+    }
+  };
+  for (uint32_t u = 0; u < n_batches; u += 2) {
+    const bool more1 = u + 1 < n_batches, more2 = u + 2 < n_batches;
+    if (more1) load_batch(bb);
+    process(ba);
+    if (more1) {
+      if (more2) load_batch(ba);
+      process(bb);
+    }
+  }
 }
 
 // LDS bytes per activation row: image and per-lane sums over whole chunks
@@ -800,13 +917,23 @@ int32_t launch_qmv_m1_gate_up(const QmvArgs& a, const uint32_t* idx, uint32_t as
   if (!qmv_m1_gate_up_supported(a.N, a.K, a.group_size))
     return fail(RMLX_INVALID_SHAPE, "qmv_m1 gate/up: unsupported shape N=%u K=%u group_size=%u", a.N, a.K, a.group_size);
   if (assignments == 0) return RMLX_OK;
-  if (assignments > 65535 || top_k == 0 || idx == nullptr || a.w1 == nullptr || a.out_f32 || a.ld_out != a.N)
-    return fail(RMLX_RUNTIME_ERROR, "qmv_m1 gate/up: needs an expert per assignment, both matrices and a dense f16 output");
+  const bool routes = idx == nullptr;
+  if (assignments > 65535 || top_k == 0 || a.w1 == nullptr || a.out_f32 || a.ld_out != a.N ||
+      (routes && (a.route_logits == nullptr || a.route_idx_out == nullptr || a.route_w_out == nullptr || top_k > 8 ||
+                  n_experts > 256 || assignments % top_k != 0)))
+    return fail(RMLX_RUNTIME_ERROR, "qmv_m1 gate/up: needs an expert per assignment (or logits of whole tokens, at most 8 picks "
+                                    "of 256 experts), both matrices and a dense f16 output");
   M1GateUpParams p{a.w0, a.s0, a.b0, a.w1, a.s1, a.b1, a.expert_stride_w, a.expert_stride_s, a.x, idx,
-                   static_cast<__half*>(a.out), a.N, a.K, top_k, n_experts};
+                   static_cast<__half*>(a.out), a.N, a.K, top_k, n_experts,
+                   a.route_logits, a.route_bias, a.route_idx_out, a.route_w_out, a.route_renorm};
   const size_t lds = lds_per_row<4>(a.K);
   const dim3 grid(a.N / kWaves, assignments);
-  hipLaunchKernelGGL(qmv_m1_gate_up_kernel<64>, grid, dim3(kThreads), lds, stream, p);
+  // one workgroup per row block while all of them are resident together, else as many as are (they loop)
+  auto looping = qmv_m1_gate_up_loop_kernel<64>;
+  uint32_t gx = resident_workgroups(looping, lds) / assignments;
+  gx = gx < 1 ? 1 : gx;
+  if (gx < grid.x) hipLaunchKernelGGL(looping, dim3(gx, assignments), dim3(kThreads), lds, stream, p);
+  else hipLaunchKernelGGL(qmv_m1_gate_up_kernel<64>, grid, dim3(kThreads), lds, stream, p);
   RMLX_HIP_CHECK(hipGetLastError());
   return RMLX_OK;
 }

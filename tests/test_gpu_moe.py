@@ -421,11 +421,15 @@ def test_moe_forward_routes_like_the_two_step_path(hip, T, E, K):
 
 
 @pytest.mark.parametrize("T,K,E,D,I,fused", [(1, 8, 16, 1024, 1536, True), (1, 1, 4, 512, 512, False), (2, 7, 16, 512, 1024, True),
-                                              (3, 5, 8, 2048, 512, False), (2, 8, 32, 1024, 512, True), (4, 8, 128, 512, 1024, True)])
+                                              (3, 5, 8, 2048, 512, False), (2, 8, 32, 1024, 512, True), (4, 8, 128, 512, 1024, True),
+                                              (9, 8, 128, 512, 1024, True), (16, 2, 64, 512, 512, False), (12, 8, 128, 512, 512, True),
+                                              (10, 1, 16, 512, 512, True)])
 def test_moe_forward_of_a_few_tokens(hip, T, K, E, D, I, fused):
-    """At most 32 assignments are not grouped.  Fewer than 16: a routing launch, then the gate / up projection on the
-    single-row kernel (a wave per pair of gate and up rows of the assignment's expert); from 16 on the gate / up
-    workgroups rank their token's experts themselves.  Both against the oracle and against the two-step path."""
+    """While the assignments are at most 1.3 x the distinct experts a uniform router would pick, they are not grouped.
+    Fewer than 16: a routing launch, then the gate / up projection on the single-row kernel (a wave per pair of gate and
+    up rows of the assignment's expert); from 16 on the gate / up workgroups rank their token's experts themselves (any
+    number of tokens).  The last cases lie past those bounds: more than 8 tokens that route with the routing kernel and
+    are grouped.  All against the oracle and against the two-step path."""
     from rmlx_amd import ops
     from rmlx_amd.runtime import DeviceBuffer
     rng = np.random.default_rng(T * 100 + K * 10 + E)
@@ -765,10 +769,10 @@ def test_wave_per_tile_kernel_shapes(hip, E, T, K, D, I, fused):
 @pytest.mark.parametrize("T,E,K,D,I,bias", [(1, 128, 8, 1024, 512, False), (4, 16, 8, 512, 1536, True), (3, 8, 5, 2048, 1024, False),
                                             (16, 64, 2, 512, 512, False), (17, 64, 2, 512, 512, True), (2, 4, 1, 512, 4096, False)])
 def test_few_tokens_run_without_grouping(hip, T, E, K, D, I, bias):
-    """`moe_forward` with at most 32 assignments routes without grouping (every assignment a chunk of one row) and adds
-    the weighted expert outputs inside the down projection; 33 and more take the grouped path.  Both against the oracle
-    and against the grouped kernels (stream kernel 1) on the same inputs: experts shared by several tokens, fewer picks
-    than waves, an expert bias, the largest batch of either side of the limit."""
+    """`moe_forward` of a few tokens routes without grouping (every assignment a row of its own) and adds the weighted
+    expert outputs inside the down projection.  Against the oracle and against the grouped kernels (stream kernel 1) on
+    the same inputs: experts shared by several tokens, fewer picks than waves, an expert bias, more than 8 tokens.  The
+    two sides sum in different orders and round the intermediate to f16 on their own: half the tolerance apart at most."""
     from rmlx_amd import ops
     from rmlx_amd.runtime import DeviceBuffer
     rng = np.random.default_rng(T * 1000 + E + K)
@@ -792,7 +796,7 @@ def test_few_tokens_run_without_grouping(hip, T, E, K, D, I, bias):
     finally:
         gh.set_expert_stream_kernel(prev)
     assert_close(grouped, ref, "moe_forward (grouped kernels)")
-    assert np.abs(direct.astype(np.float64) - grouped.astype(np.float64)).max() <= 0.25 * model.tolerance(ref)
+    assert np.abs(direct.astype(np.float64) - grouped.astype(np.float64)).max() <= 0.5 * model.tolerance(ref)
 
 
 @pytest.mark.parametrize("T", [300, 700])
