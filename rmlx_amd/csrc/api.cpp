@@ -230,12 +230,15 @@ int32_t run_matmul_plain(const rmlx_qweight* qw, const void* x, int32_t x_dtype,
     //          (4096 x 8192: 9 against 12 us, 4096 x 16384: 17 against 19, 8192 x 8192: 18 against 19, 12288 x 4096: 12.7 against
     //          16.2, 16384 x 4096: 15.3 against 16.6, weights cycled through more than 1 GiB; beyond that the GEMM's grid is
     //          large enough to win: 28672 x 4096 22 against 29 us);
+    //          17 to 32 rows in passes of 8 while W <= 12 MiB: 4096 x 4096 8.8 / 9.1 / 9.3 us at 17 / 24 / 32 rows against 9.6 /
+    //          9.9 / 10.3 on the GEMM; 9216 x 4096 at 32 rows: 20.9 against 17.3, so not beyond);
     //   8-bit: GEMV up to 16 rows while W < 48 MiB (4096 x 4096 is 16 MiB; at 12288 x 4096 the GEMM wins, 19 against 23 us).
     const uint64_t wbytes = (uint64_t)N * K * qw->bits / 8;
     // Without the register-weights GEMM (K not a multiple of 512) the alternative is the LDS-staged GEMM with
     // a floor of about 15 us: there the 4-bit GEMV keeps up to passes * W <= 48 MiB.
     const bool small_m = !can_qmm_rw ? M <= kQmvMaxM || (qw->bits == 4 && (uint64_t)((M + 7) / 8) * wbytes <= (48ull << 20))
-                         : qw->bits == 4 ? M <= 8 || (M <= kQmvMaxM && (wbytes <= (12ull << 20) || N <= 16384))
+                         : qw->bits == 4 ? M <= 8 || (M <= kQmvMaxM && (wbytes <= (12ull << 20) || N <= 16384)) ||
+                                               (M <= 32 && wbytes <= (12ull << 20))
                                          : (M <= kQmvMaxM && wbytes < (48ull << 20));
     // Shapes the K-split GEMV does not take (group size 32) run up to 16 rows on the single-row kernel in passes of four,
     // which streams the weights once per pass: with the register-weights GEMM as the alternative it keeps up to 4 rows
