@@ -30,6 +30,8 @@
 //     the grid is the resident workgroups, each stages the activations once and walks several row
 //     blocks with the next block's weights in flight.  Long rows of a short matrix split K over 2 or
 //     4 waves of the workgroup.
+#include <vector>
+
 #include "common.hpp"
 #include "route.hpp"
 
@@ -758,19 +760,20 @@ size_t lds_per_row(uint32_t K) {
   return chunks * (chunk_k * 2 + 64 * sizeof(float2));
 }
 
-// Workgroups of `kernel` that the chip keeps resident at once (cache per instantiation and host thread, keyed by
-// the LDS size).
+// Workgroups of `kernel` that the chip keeps resident at once (cached per host thread, kernel and LDS size: kernels of
+// one signature share this function, so the kernel's address is part of the key).
 template <typename Kernel>
 uint32_t resident_workgroups(Kernel kernel, size_t lds) {
-  static thread_local size_t cached_lds = ~(size_t)0;
-  static thread_local uint32_t cached = 0;
-  if (cached_lds != lds) {
-    int per_cu = 0;
-    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, kThreads, lds) != hipSuccess || per_cu < 1) per_cu = 1;
-    cached = (uint32_t)per_cu * (uint32_t)ctx().num_cus;
-    cached_lds = lds;
-  }
-  return cached;
+  struct Entry { const void* fn; size_t lds; uint32_t wgs; };
+  static thread_local std::vector<Entry> cache;
+  const void* fn = reinterpret_cast<const void*>(kernel);
+  for (const Entry& e : cache)
+    if (e.fn == fn && e.lds == lds) return e.wgs;
+  int per_cu = 0;
+  if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, kThreads, lds) != hipSuccess || per_cu < 1) per_cu = 1;
+  const uint32_t wgs = (uint32_t)per_cu * (uint32_t)ctx().num_cus;
+  cache.push_back({fn, lds, wgs});
+  return wgs;
 }
 
 template <int BITS, int GS, int R, bool NT, int MR, bool NORM, int KP = 1, bool GATHER = false>
