@@ -476,7 +476,6 @@ bool ungrouped_pays(uint32_t T, uint32_t E, uint32_t K) {
   const double distinct = E * (1.0 - std::pow(1.0 - (double)K / E, (double)T));
   return (uint64_t)T * K <= kDirectMaxAssignments && (double)T * K <= 1.3 * distinct;
 }
-constexpr uint32_t kOwnRouteMinAssignments = 16;  // from here on the gate / up launch of that path routes by itself
 enum { GATHER_AUTO = 0, GATHER_STREAM = 1, GATHER_GEMM = 2, GATHER_PORTABLE = 3 };
 
 int32_t check_expert_weights(const char* who, const rmlx_qweight* gate, const rmlx_qweight* up,
@@ -1391,16 +1390,14 @@ int32_t moe_grouped_impl(const rmlx_qweight* gate, const rmlx_qweight* up, const
   RMLX_TRY(check_out("MoeLayer", out_bytes, T * sh.D * 2));
   if (T == 0) return RMLX_OK;
   hipStream_t s = (hipStream_t)stream;
-  // Which form a call that brings logits takes.  `direct`: a few tokens, no grouping at all (below).  `own`: the gate / up
-  // workgroups of that form rank their token's experts themselves, so any number of tokens.  `small`: at most 8 tokens,
-  // which the one-workgroup routing launches (with or without grouping behind) take.  Everything else routes with the
-  // routing kernel and goes on as if the caller had brought the picks.
+  // `direct`: a few tokens, no grouping at all (below).  A call that brings logits instead of picks: the gate / up
+  // workgroups of the direct form rank their token's experts themselves, so any number of tokens; `small`: at most 8
+  // tokens, which the one-workgroup routing + grouping launch takes; everything else routes with the routing kernel and
+  // goes on as if the caller had brought the picks.
   const bool single_row = gate->bits == 4 && qmv_m1_gate_up_supported(sh.I, sh.D, gate->group_size);
-  bool direct = route != nullptr && ungrouped_pays(T32, sh.E, (uint32_t)top_k) && sh.stream_kernel != 1 && sh.wave_down &&
-                qmv_wt_combine_supported(sh.D, sh.I, down->group_size, (uint32_t)top_k);
-  const bool own = direct && single_row && sh.E <= 256 && A >= kOwnRouteMinAssignments;
+  const bool direct = ungrouped_pays(T32, sh.E, (uint32_t)top_k) && sh.stream_kernel != 1 && sh.wave_down && single_row &&
+                      (route == nullptr || sh.E <= 256) && qmv_wt_combine_supported(sh.D, sh.I, down->group_size, (uint32_t)top_k);
   const bool small = route != nullptr && T32 <= 8 && route_sort_fusable(T32, sh.E, (uint32_t)top_k);
-  if (direct && !own && !small) direct = false;
   if (route != nullptr && !direct && !small) {
     RMLX_TRY(launch_topk_route(route->logits, route->bias, T32, sh.E, (uint32_t)top_k, 1, route->idx_out, route->w_out, nullptr,
                                nullptr, s));
@@ -1451,38 +1448,26 @@ int32_t moe_grouped_impl(const rmlx_qweight* gate, const rmlx_qweight* up, const
     return finish(s);
   }
   if (!aligned16(xk)) return fail(RMLX_INVALID_SHAPE, "MoeLayer: input must be 16-byte aligned");
-  // A few tokens, routed here: no grouping at all.  Every assignment is one row in assignment order, and the down
-  // projection adds the token's weighted expert outputs itself - two or three launches (routing, gate / up, down +
-  // combine) instead of four, no [assignments, D] intermediate.  An expert picked by two tokens is streamed once per
+  // A few tokens: no grouping at all.  Every assignment is one row in assignment order, and the down
+  // projection adds the token's weighted expert outputs itself - two launches (gate / up that routes, down + combine)
+  // instead of four, no [assignments, D] intermediate.  An expert picked by two tokens is streamed once per
   // token (at 4 tokens of 8 picks over 128 experts: 32 rows for 31 experts; see ungrouped_pays).
   if (direct) {
     RMLX_TRY(h.alloc((size_t)A * sh.I * 2, s, arena));
     // One row per expert: the gate / up projection on the single-row GEMV's layout (a wave per pair of gate and up rows,
-    // dot products instead of a matrix unit that would multiply 15 empty rows) where it takes the shape.  From 16
-    // assignments on its workgroups rank their token's experts themselves (one wave, while the activations arrive) --
-    // two launches; the ranking then stands in front of every workgroup's weight stream, which pays once a workgroup
-    // walks several row blocks (2 / 3 / 4 tokens of 8 picks) and costs where it has one or two (1 token).
-    if (own) {
-      QmvArgs a = gate_up_args(gate, up, sh, xk, static_cast<__half*>(h.ptr));
+    // dot products instead of a matrix unit that would multiply 15 empty rows), and no routing launch: every workgroup
+    // ranks its token's experts itself, one wave, while the activations arrive (1 / 2 / 4 tokens of 8 picks: 23.4 / 37.0 /
+    // 59.5 us against 24.4 / 37.8 / 61.0 us with a routing launch in front).
+    QmvArgs a = gate_up_args(gate, up, sh, xk, static_cast<__half*>(h.ptr));
+    if (route != nullptr) {
       a.route_logits = route->logits; a.route_bias = route->bias; a.route_idx_out = route->idx_out; a.route_w_out = route->w_out;
       a.route_renorm = 1;
-      RMLX_TRY(launch_qmv_m1_gate_up(a, nullptr, A, (uint32_t)top_k, sh.E, s));
-    } else {
-      RMLX_TRY(meta.alloc(((size_t)4 * A + 4) * 4, s, arena));  // tok[A] | chunk_tab[3 A] | n_chunks[1]
-      uint32_t* tok = static_cast<uint32_t*>(meta.ptr);
-      uint32_t* chunk_tab = tok + A;
-      uint32_t* n_chunks = chunk_tab + 3 * (size_t)A;
-      RMLX_TRY(launch_route_direct_small(route->logits, route->bias, T32, sh.E, (uint32_t)top_k, 1, route->idx_out, route->w_out,
-                                         tok, chunk_tab, n_chunks, s));
-      if (single_row)
-        RMLX_TRY(launch_qmv_m1_gate_up(gate_up_args(gate, up, sh, xk, static_cast<__half*>(h.ptr)), route->idx_out, A,
-                                       (uint32_t)top_k, sh.E, s));
-      else  // the K-split kernel over one-row chunks
-        RMLX_TRY(run_expert_ffn(gate, up, down, sh, xk, tok, chunk_tab, n_chunks, A, static_cast<__half*>(h.ptr), nullptr, 0, 0,
-                                StreamPlan{0, 0, 8}, s));
     }
+    const uint32_t* picks = route != nullptr ? route->idx_out : expert_indices_dev;
+    const float* pick_weights = route != nullptr ? route->w_out : expert_weights_dev;
+    RMLX_TRY(launch_qmv_m1_gate_up(a, route != nullptr ? nullptr : picks, A, (uint32_t)top_k, sh.E, s));
     RMLX_TRY(launch_qmv_wt_combine(down->w, down->s, down->b, (uint64_t)sh.D * (sh.I / 8), (uint64_t)sh.D * (sh.I / down->group_size),
-                                   sh.E, static_cast<const __half*>(h.ptr), route->idx_out, route->w_out, T32, (uint32_t)top_k,
+                                   sh.E, static_cast<const __half*>(h.ptr), picks, pick_weights, T32, (uint32_t)top_k,
                                    sh.D, sh.I, static_cast<__half*>(out_f16_dev), s));
     return finish(s);
   }

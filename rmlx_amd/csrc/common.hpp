@@ -278,10 +278,6 @@ bool route_sort_fusable(uint32_t T, uint32_t E, uint32_t K);
 int32_t launch_route_sort_small(const float* logits, const float* bias, uint32_t T, uint32_t E, uint32_t K,
                                 int renorm, uint32_t* idx, float* w, uint32_t* sorted, uint32_t* sorted_tok,
                                 uint32_t* inv, uint32_t* chunk_tab, uint32_t* n_chunks, hipStream_t s);
-// Decode-sized batches without grouping: routing only, every assignment a chunk of one row (tok[a] = its token)
-int32_t launch_route_direct_small(const float* logits, const float* bias, uint32_t T, uint32_t E, uint32_t K,
-                                  int renorm, uint32_t* idx, float* w, uint32_t* tok, uint32_t* chunk_tab,
-                                  uint32_t* n_chunks, hipStream_t s);
 int32_t launch_index_gather(const __half* src, uint32_t d, const uint32_t* idx, uint32_t n, uint32_t src_rows,
                             __half* dst, hipStream_t s);
 int32_t launch_scatter_weighted_add(const __half* src, uint32_t n, uint32_t d, const uint32_t* tok,

@@ -19,8 +19,7 @@ constexpr int kMaxExperts = 1024;  // LDS histogram capacity of the sort kernel
 __device__ __forceinline__ void route_token(const float* __restrict__ logits, const float* __restrict__ bias,
                                             uint32_t E, uint32_t K, int renorm, uint32_t* __restrict__ out_idx,
                                             float* __restrict__ out_w, uint32_t row, uint32_t lane,
-                                            uint32_t* lds_idx, uint32_t* __restrict__ direct_tab = nullptr,
-                                            uint32_t* __restrict__ direct_tok = nullptr) {
+                                            uint32_t* lds_idx) {
   uint32_t my_idx;
   float my_w;
   route::token_picks(logits, bias, E, K, renorm, row, lane, my_idx, my_w);
@@ -28,13 +27,6 @@ __device__ __forceinline__ void route_token(const float* __restrict__ logits, co
     out_idx[(size_t)row * K + lane] = my_idx;
     out_w[(size_t)row * K + lane] = my_w;
     if (lds_idx != nullptr) lds_idx[row * K + lane] = my_idx;
-    if (direct_tab != nullptr) {  // every assignment its own chunk of one row, in assignment order (no grouping)
-      const uint32_t a = row * K + lane;
-      direct_tab[3 * a + 0] = my_idx < E ? my_idx : 0u;
-      direct_tab[3 * a + 1] = a;
-      direct_tab[3 * a + 2] = my_idx < E ? 1u : 0x80000001u;  // (bit 31: zeros are written)
-      direct_tok[a] = row;
-    }
   }
 }
 
@@ -253,20 +245,6 @@ __global__ __launch_bounds__(512) void route_sort_small_kernel(const float* __re
                chunk_tab, n_chunks);
 }
 
-// Routing of a batch of a few tokens without grouping: every assignment becomes a chunk of one row (expert, position =
-// assignment index, 1) whose activation row is its token.  An expert picked by two tokens is then streamed once per
-// token; in exchange the launch has no second phase and the expert projections see positions in assignment order.
-__global__ __launch_bounds__(512) void route_direct_small_kernel(const float* __restrict__ logits,
-                                                                 const float* __restrict__ bias, uint32_t T, uint32_t E,
-                                                                 uint32_t K, int renorm, uint32_t* __restrict__ out_idx,
-                                                                 float* __restrict__ out_w, uint32_t* __restrict__ tok,
-                                                                 uint32_t* __restrict__ chunk_tab,
-                                                                 uint32_t* __restrict__ n_chunks) {
-  const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  if (wave < T) route_token(logits, bias, E, K, renorm, out_idx, out_w, wave, lane, nullptr, chunk_tab, tok);
-  if (threadIdx.x == 0) *n_chunks = T * K;
-}
-
 __global__ void index_gather_kernel(const __half* __restrict__ src, uint32_t d, const uint32_t* __restrict__ idx,
                                     uint32_t src_rows, __half* __restrict__ dst) {
   const uint32_t i = blockIdx.x;
@@ -390,16 +368,6 @@ int32_t launch_route_sort_small(const float* logits, const float* bias, uint32_t
   if (!route_sort_fusable(T, E, K)) return fail(RMLX_RUNTIME_ERROR, "route_sort_small: T=%u E=%u K=%u not supported", T, E, K);
   hipLaunchKernelGGL(route_sort_small_kernel, dim3(1), dim3(64 * T), 0, s, logits, bias, T, E, K, renorm, idx, w, sorted,
                      sorted_tok, inv, chunk_tab, n_chunks);
-  RMLX_HIP_CHECK(hipGetLastError());
-  return RMLX_OK;
-}
-
-int32_t launch_route_direct_small(const float* logits, const float* bias, uint32_t T, uint32_t E, uint32_t K,
-                                  int renorm, uint32_t* idx, float* w, uint32_t* tok, uint32_t* chunk_tab,
-                                  uint32_t* n_chunks, hipStream_t s) {
-  if (!route_sort_fusable(T, E, K)) return fail(RMLX_RUNTIME_ERROR, "route_direct_small: T=%u E=%u K=%u not supported", T, E, K);
-  hipLaunchKernelGGL(route_direct_small_kernel, dim3(1), dim3(64 * T), 0, s, logits, bias, T, E, K, renorm, idx, w, tok,
-                     chunk_tab, n_chunks);
   RMLX_HIP_CHECK(hipGetLastError());
   return RMLX_OK;
 }

@@ -365,11 +365,13 @@ def _experts(rng, E, D, I, fused):
     return gate, up, down, gate_h, up_h, down_h
 
 
-@pytest.mark.parametrize("T,E,K,D,I", [(6, 8, 4, 512, 512), (20, 32, 4, 512, 512), (100, 4, 2, 512, 512), (12, 6, 2, 256, 384)])
+@pytest.mark.parametrize("T,E,K,D,I", [(6, 8, 4, 512, 512), (20, 32, 4, 512, 512), (100, 4, 2, 512, 512), (12, 6, 2, 256, 384),
+                                       (2, 64, 8, 1024, 512), (5, 128, 8, 512, 1024)])
 def test_moe_forward_grouped_skips_out_of_range_experts(hip, T, E, K, D, I):
     """Caller-supplied expert ids outside [0, E) contribute nothing (the reference's combine skips them,
     crates/rmlx-distributed/src/moe_exchange.rs:2305): one-wave grouping (<= 64 assignments), the workgroup-wide
-    grouping below and above the grouped-GEMM threshold, and the portable kernels (D, I no multiples of 512)."""
+    grouping below and above the grouped-GEMM threshold, the portable kernels (D, I no multiples of 512), and the form
+    without grouping that a few tokens take (the last two cases)."""
     from rmlx_amd import ops
     from rmlx_amd.runtime import DeviceBuffer
     rng = np.random.default_rng(T + E + K + D)
