@@ -837,7 +837,11 @@ void launch_bits(const M1Params& p, uint32_t group_size, hipStream_t s) {
     // two weight rows per wave for long rows (more bytes in flight per wave) and, with 4-bit weights, for
     // tall matrices (the activation registers read from LDS serve both rows; measured 3-9 % from N = 12288
     // on; the 8-bit kernel reads half as many activations per weight byte and is faster with one), else one
-    const bool two = (p.K >= 12288 || (BITS == 4 && p.N >= 12288)) && p.N % (kWaves * 2) == 0;
+    // (also where two rows per wave make the grid a whole number of workgroups per CU, at least two: N = 8192 on 256 CUs
+    // 5.8 against 6.2 us at K = 4096, 10.0 against 10.5 us at K = 8192; N = 4096, one workgroup per CU: 4.25 against 4.04)
+    const uint32_t cus_m1 = (uint32_t)ctx().num_cus;
+    const bool two = (p.K >= 12288 || (BITS == 4 && (p.N >= 12288 || (p.N % (kWaves * 2 * cus_m1) == 0 && p.N >= kWaves * 4 * cus_m1)))) &&
+                     p.N % (kWaves * 2) == 0;
     // Long rows of a short matrix (the reference's split-K case, K > 8192 and N <= 2048, quantized.rs:7246-7250):
     // with one wave per row the grid would not fill the chip, so 2 or 4 waves share a row until there are two
     // workgroups per CU (every wave keeps at least two chunks).
