@@ -575,25 +575,20 @@ struct M1GateUpParams {
   int32_t route_renorm;
 };
 
-// The expert of assignment a: from the list, or ranked here (after the caller has requested its activations).
-__device__ __forceinline__ uint32_t gate_up_expert(const M1GateUpParams& p, uint32_t a, int wave, int lane, bool first_wg) {
+// The expert of assignment a: from the list, or ranked here by the workgroup (after the caller has requested its
+// activations).
+__device__ __forceinline__ uint32_t gate_up_expert(const M1GateUpParams& p, uint32_t a, bool first_wg) {
   if (p.idx != nullptr) return p.idx[a];
-  __shared__ uint32_t picks[8];
+  __shared__ __attribute__((aligned(16))) uint32_t ws[512];
+  __shared__ uint32_t pick_idx[8];
+  __shared__ float pick_w[8];
   const uint32_t t = a / p.top_k, pick = a - t * p.top_k;
-  if (wave == 0) {
-    uint32_t my_idx;
-    float my_w;
-    route::token_picks(p.route_logits, p.route_bias, p.n_experts, p.top_k, p.route_renorm, t, (uint32_t)lane, my_idx, my_w);
-    if ((uint32_t)lane < p.top_k) {
-      picks[lane] = my_idx;
-      if (first_wg && pick == 0) {
-        p.route_idx_out[(size_t)t * p.top_k + lane] = my_idx;
-        p.route_w_out[(size_t)t * p.top_k + lane] = my_w;
-      }
-    }
+  route::token_picks_workgroup(p.route_logits, p.route_bias, p.n_experts, p.top_k, p.route_renorm, t, ws, pick_idx, pick_w);
+  if (first_wg && pick == 0 && threadIdx.x < p.top_k) {
+    p.route_idx_out[(size_t)t * p.top_k + threadIdx.x] = pick_idx[threadIdx.x];
+    p.route_w_out[(size_t)t * p.top_k + threadIdx.x] = pick_w[threadIdx.x];
   }
-  __syncthreads();
-  return picks[pick];
+  return pick_idx[pick];
 }
 
 template <int GS>
@@ -611,7 +606,7 @@ __global__ __launch_bounds__(kThreads, 1) void qmv_m1_gate_up_kernel(M1GateUpPar
   // loads, small ones first (the memory counter retires in order): the activations, the expert, then the rows
   u4 xv[1][4];
   load_activations<4, 1, false>(img, x, 1u, 0u, nullptr, nullptr, tid, xv);
-  uint32_t expert = gate_up_expert(p, a, wave, lane, blockIdx.x == 0);
+  uint32_t expert = gate_up_expert(p, a, blockIdx.x == 0);
   const bool zeros = expert >= p.n_experts;
   expert = zeros ? 0u : expert;
   struct Batch { u4 w[2][2]; uint32_t s[2][2], b[2][2]; };  // [chunk of the batch][gate, up]
@@ -686,7 +681,7 @@ __global__ __launch_bounds__(kThreads, 1) void qmv_m1_gate_up_loop_kernel(M1Gate
 
   u4 xv[1][4];
   load_activations<4, 1, false>(img, x, 1u, 0u, nullptr, nullptr, tid, xv);
-  uint32_t expert = gate_up_expert(p, a, wave, lane, blockIdx.x == 0);
+  uint32_t expert = gate_up_expert(p, a, blockIdx.x == 0);
   const bool zeros = expert >= p.n_experts;
   expert = zeros ? 0u : expert;
   struct Batch { u4 w[2][2]; uint32_t s[2][2], b[2][2]; };  // [chunk of the batch][gate, up]

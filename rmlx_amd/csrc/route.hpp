@@ -78,19 +78,18 @@ __device__ __forceinline__ float exp_neg_exact(float x) {
 // the f32 softmax value exp(l - max) * (1 / sum) with strict >, so equal values (two logits that collapse
 // after exp, an underflowing tail) go to the lower expert index (topk_route.rs:283-300).  The sum runs over the
 // four values of a lane in ascending order and then over the lanes as a balanced pairwise tree.
-// Lane k < K leaves with the k-th pick in `my_idx` (0xFFFFFFFF: none left) and its weight in `my_w`.
-__device__ __forceinline__ void token_picks(const float* __restrict__ logits, const float* __restrict__ bias, uint32_t E,
-                                            uint32_t K, int renorm, uint32_t row, uint32_t lane, uint32_t& my_idx_out,
-                                            float& my_w_out) {
+// The keys of a token's experts, one wave: lane l receives the keys of experts l, l + 64, l + 128, l + 192.  A key is
+// the bits of the expert's non-negative softmax value (order-preserving; -0 counted as +0) plus one, zero for an expert
+// index past E.
+__device__ __forceinline__ void token_keys(const float* __restrict__ logits, const float* __restrict__ bias, uint32_t E,
+                                           uint32_t row, uint32_t lane, uint32_t (&key)[4]) {
   const float NEG_INF = -__builtin_inff();
   float v[4], sm[4];
-  bool taken[4];
   float mx = NEG_INF;
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
     const uint32_t e = lane + 64 * j;
     v[j] = NEG_INF;
-    taken[j] = e >= E;
     if (e < E) {
       v[j] = logits[(size_t)row * E + e];
       if (bias != nullptr) v[j] += bias[e];
@@ -107,15 +106,18 @@ __device__ __forceinline__ void token_picks(const float* __restrict__ logits, co
   sum = wave_add(sum);
   const float inv = 1.0f / sum;
 #pragma unroll
-  for (int j = 0; j < 4; ++j) sm[j] *= inv;
+  for (int j = 0; j < 4; ++j) key[j] = lane + 64 * j < E ? __float_as_uint(sm[j] * inv + 0.0f) + 1u : 0u;
+}
 
-  // A slot's key: the bits of its non-negative softmax value (order-preserving; -0 counted as +0) plus one, zero once
-  // the slot is taken or lies past E.  A round: the wave maximum of the keys, then the lowest expert index that
-  // holds it -- slots in ascending j, inside a slot the lowest lane of the ballot.  Lane k keeps the k-th pick (no
-  // register arrays indexed by the round counter).
+// Lane k < K leaves with the k-th pick in `my_idx` (0xFFFFFFFF: none left) and its weight in `my_w`.
+__device__ __forceinline__ void token_picks(const float* __restrict__ logits, const float* __restrict__ bias, uint32_t E,
+                                            uint32_t K, int renorm, uint32_t row, uint32_t lane, uint32_t& my_idx_out,
+                                            float& my_w_out) {
   uint32_t key[4];
-#pragma unroll
-  for (int j = 0; j < 4; ++j) key[j] = taken[j] ? 0u : __float_as_uint(sm[j] + 0.0f) + 1u;
+  token_keys(logits, bias, E, row, lane, key);
+  // A round: the wave maximum of the keys, then the lowest expert index that holds it -- slots in ascending j, inside a
+  // slot the lowest lane of the ballot; a slot that is taken gets key zero.  Lane k keeps the k-th pick (no register arrays
+  // indexed by the round counter).
   float my_w = 0.f;
   uint32_t my_idx = 0xFFFFFFFFu;
   for (uint32_t k = 0; k < K; ++k) {
@@ -145,6 +147,59 @@ __device__ __forceinline__ void token_picks(const float* __restrict__ logits, co
   }
   my_idx_out = my_idx;
   my_w_out = my_w * scale;
+}
+
+// The same picks and weights by a whole workgroup (blockDim.x = 256, 512 or 1024): the first wave makes the
+// keys, then every thread counts, for one expert and a share of the others, how many rank before it (larger key, or the
+// same key and a lower index): an expert's rank is its place in the sequence of repeated arg-max rounds above, found
+// without the rounds' serial chain.  Results in workgroup memory: out_idx[k], out_w[k] for k < K (0xFFFFFFFF / 0 where
+// fewer than K experts exist); every thread may read them after the call.  `ws` is workspace of 2 * 256 words.
+__device__ __forceinline__ void token_picks_workgroup(const float* __restrict__ logits, const float* __restrict__ bias,
+                                                      uint32_t E, uint32_t K, int renorm, uint32_t row, uint32_t* ws,
+                                                      uint32_t* out_idx, float* out_w) {
+  uint32_t* keys = ws;         // [256]
+  uint32_t* rank = ws + 256;   // [256]
+  const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, nthreads = blockDim.x;
+  if (wave == 0) {
+    uint32_t key[4];
+    token_keys(logits, bias, E, row, lane, key);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) { keys[lane + 64 * j] = key[j]; rank[lane + 64 * j] = 0u; }
+    if (lane < 8) { out_idx[lane] = 0xFFFFFFFFu; out_w[lane] = 0.f; }
+  }
+  __syncthreads();
+  // thread -> (expert i, part): the slots 0 .. ep - 1 (ep = 64, 128 or 256 covers E) are split between the parts of an
+  // expert, four keys per LDS read (a wave reads one address: a broadcast)
+  uint32_t ep = 64;
+  while (ep < E) ep <<= 1;
+  const uint32_t parts = nthreads / ep, per = ep / parts;
+  if (tid < ep * parts) {
+    const uint32_t i = tid & (ep - 1), part = tid / ep, mine = keys[i];
+    uint32_t before = 0;
+    for (uint32_t j = part * per; j < (part + 1) * per; j += 4) {
+      const uint4 k4 = *reinterpret_cast<const uint4*>(keys + j);
+      before += (k4.x > mine || (k4.x == mine && j + 0 < i)) ? 1u : 0u;
+      before += (k4.y > mine || (k4.y == mine && j + 1 < i)) ? 1u : 0u;
+      before += (k4.z > mine || (k4.z == mine && j + 2 < i)) ? 1u : 0u;
+      before += (k4.w > mine || (k4.w == mine && j + 3 < i)) ? 1u : 0u;
+    }
+    if (mine != 0u && before != 0u) atomicAdd(&rank[i], before);
+  }
+  __syncthreads();
+  if (tid < 256) {
+    const uint32_t mine = keys[tid], r = rank[tid];
+    if (mine != 0u && r < K) { out_idx[r] = tid; out_w[r] = __uint_as_float(mine - 1u); }
+  }
+  __syncthreads();
+  if (renorm) {
+    // sum of the K picks in pick order, the order a serial loop would add them in (every thread computes the same)
+    float wsum = 0.f;
+    for (uint32_t k = 0; k < K; ++k) wsum += out_w[k];
+    const float scale = wsum > 0.f ? 1.0f / wsum : 0.f;
+    __syncthreads();
+    if (tid < K) out_w[tid] = out_w[tid] * scale;
+    __syncthreads();
+  }
 }
 
 }  // namespace route
