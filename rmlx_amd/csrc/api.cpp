@@ -1357,6 +1357,24 @@ int32_t rmlx_hip_expert_group_grouped_forward(const rmlx_qweight* gate, const rm
     return finish(s);
   }
   if (!aligned16(xk)) return fail(RMLX_INVALID_SHAPE, "ExpertGroup: input must be 16-byte aligned");
+  // One row per expert (a decoding token's experts): both projections on the single-row kernel's layout -- a wave per
+  // pair of gate and up rows, then a wave per down row, each expert streamed once with whole-row contiguous loads.
+  bool single_rows = !gemm && gate->bits == 4 && down->bits == 4 && sh.stream_kernel != 1 &&
+                     qmv_m1_gate_up_supported(sh.I, sh.D, gate->group_size) && qmv_m1_supported(sh.D, sh.I, down->group_size, 4) &&
+                     aligned16(down->w) && aligned16(down->s) && aligned16(down->b);
+  for (size_t i = 0; i < n_items && single_rows; ++i) single_rows = batch_sizes_host[i] == 1;
+  if (single_rows) {
+    RMLX_TRY(dtab.alloc(n_items * 4, s));
+    RMLX_HIP_CHECK(hipMemcpyAsync(dtab.ptr, expert_idx_host, n_items * 4, hipMemcpyHostToDevice, s));
+    RMLX_HIP_CHECK(hipStreamSynchronize(s));  // the caller's host array need not outlive the call
+    RMLX_TRY(h.alloc(total * sh.I * 2, s));
+    const uint32_t* experts = static_cast<const uint32_t*>(dtab.ptr);
+    RMLX_TRY(launch_qmv_m1_gate_up(gate_up_args(gate, up, sh, xk, static_cast<__half*>(h.ptr)), experts, rows, 1, sh.E, s));
+    RMLX_TRY(launch_qmv_m1_gather(down->w, down->s, down->b, (uint64_t)sh.D * (sh.I / 8), (uint64_t)sh.D * (sh.I / down->group_size),
+                                  sh.E, static_cast<const __half*>(h.ptr), experts, rows, static_cast<__half*>(out_f16_dev), sh.D,
+                                  sh.I, down->group_size, s));
+    return finish(s);
+  }
   RMLX_TRY(dtab.alloc(tab.size() * 4, s));
   RMLX_HIP_CHECK(hipMemcpyAsync(dtab.ptr, tab.data(), tab.size() * 4, hipMemcpyHostToDevice, s));
   RMLX_HIP_CHECK(hipStreamSynchronize(s));  // `tab` is pageable host memory owned by this call

@@ -673,6 +673,37 @@ def test_grouped_forward_equals_per_expert_loop(hip):
         group.grouped_forward([(0, DeviceBuffer.from_numpy(make_x(rng, 1, D + 512)))])
 
 
+@pytest.mark.parametrize("E,D,I,fused,n_items", [(16, 1024, 1536, True, 8), (6, 512, 512, False, 1), (128, 512, 1024, True, 40)])
+def test_grouped_forward_of_single_rows(hip, E, D, I, fused, n_items):
+    """Every item one row (a decoding token's experts, the same expert allowed twice): both projections on the single-row
+    kernel.  Against the float64 expert FFN and against the same items with one row more on the first (which takes the
+    streaming kernels over chunks)."""
+    from rmlx_amd import ops
+    from rmlx_amd.runtime import DeviceBuffer
+    rng = np.random.default_rng(E + D + n_items)
+    gate, up, down, gh, uh, dh = _experts(rng, E, D, I, fused)
+    group = ops.ExpertGroup(gh, uh, dh)
+    experts = rng.integers(0, E, size=n_items)
+    if n_items > 1:
+        experts[1] = experts[0]
+    items = [(int(e), make_x(rng, 1, D)) for e in experts]
+    print(f"ExpertGroup single rows E={E} D={D} I={I} fused={fused} items={n_items}", flush=True)
+    outs = group.grouped_forward([(e, DeviceBuffer.from_numpy(x)) for e, x in items])
+    assert [e for e, _ in outs] == [e for e, _ in items]
+    refs = []
+    for (e, x), (_, y) in zip(items, outs):
+        xe = x.astype(np.float64)
+        g = xe @ model.dequantize(gate[0][e], gate[1][e], gate[2][e], 64, 4).T
+        u = xe @ model.dequantize(up[0][e], up[1][e], up[2][e], 64, 4).T
+        h = (model.silu(g) * u).astype(np.float16).astype(np.float64)
+        refs.append(h @ model.dequantize(down[0][e], down[1][e], down[2][e], 64, 4).T)
+        assert_close(y, refs[-1], f"expert {e}")
+    first = np.concatenate([items[0][1], make_x(rng, 1, D)])
+    outs2 = group.grouped_forward([(items[0][0], DeviceBuffer.from_numpy(first))] + [(e, DeviceBuffer.from_numpy(x)) for e, x in items[1:]])
+    for (_, y), (_, y2), ref in zip(outs, outs2, refs):
+        assert np.abs(y.astype(np.float64) - y2[:1].astype(np.float64)).max() <= 0.5 * model.tolerance(ref)
+
+
 @pytest.fixture(scope="module")
 def config5(hip):
     """Config 5 weights: 128 experts, hidden 4096, intermediate 1536, fused gate/up, Q4 group 64."""
