@@ -619,6 +619,16 @@ QmvArgs gate_up_args(const rmlx_qweight* gate, const rmlx_qweight* up, const Exp
   return a;
 }
 
+// Both projections of these experts run on the single-row kernels (one row per expert): 4- or 8-bit, one format for the
+// three matrices, any group size, the shapes of the single-row GEMV, aligned buffers.
+bool single_row_experts(const rmlx_qweight* gate, const rmlx_qweight* up, const rmlx_qweight* down, const ExpertShapes& sh) {
+  if ((gate->bits != 4 && gate->bits != 8) || down->bits != gate->bits) return false;
+  if (up != nullptr && (up->bits != gate->bits || up->group_size != gate->group_size)) return false;
+  for (const rmlx_qweight* q : {gate, up, down})
+    if (q != nullptr && (!aligned16(q->w) || !aligned16(q->s) || !aligned16(q->b))) return false;
+  return qmv_m1_gate_up_supported(sh.I, sh.D, gate->group_size, gate->bits) && qmv_m1_supported(sh.D, sh.I, down->group_size, down->bits);
+}
+
 // gate/up + SwiGLU then down, over a device chunk table.  h: f16 [positions, I] scratch.
 int32_t run_expert_ffn(const rmlx_qweight* gate, const rmlx_qweight* up, const rmlx_qweight* down,
                        const ExpertShapes& sh, const __half* x, const uint32_t* row_map,
@@ -1143,7 +1153,7 @@ int32_t rmlx_hip_gather_qmm_select(const rmlx_array* x, const void* w_packed_dev
              aligned16(sc) && aligned16(bi) && aligned16(xk)) {
     // one row per index: the single-row kernel with a weight matrix per activation row -- one launch, no chunk table
     RMLX_TRY(launch_qmv_m1_gather(w, sc, bi, (uint64_t)n * (k / 8), (uint64_t)n * gpr, E32, xk, idx, B32,
-                                  static_cast<__half*>(out_f16_dev), N32, K32, group_size, s));
+                                  static_cast<__half*>(out_f16_dev), N32, K32, group_size, 4, s));
   } else if (fast && kernel != GATHER_PORTABLE) {
     const uint64_t per = ((uint64_t)m_per_batch + 7) / 8, n_chunks = (uint64_t)B32 * per;
     if (n_chunks > 0x7FFFFFFFull) return fail(RMLX_INVALID_SHAPE, "gather_qmm: too many row chunks (%" PRIu64 ")", n_chunks);
@@ -1359,9 +1369,7 @@ int32_t rmlx_hip_expert_group_grouped_forward(const rmlx_qweight* gate, const rm
   if (!aligned16(xk)) return fail(RMLX_INVALID_SHAPE, "ExpertGroup: input must be 16-byte aligned");
   // One row per expert (a decoding token's experts): both projections on the single-row kernel's layout -- a wave per
   // pair of gate and up rows, then a wave per down row, each expert streamed once with whole-row contiguous loads.
-  bool single_rows = !gemm && gate->bits == 4 && down->bits == 4 && sh.stream_kernel != 1 &&
-                     qmv_m1_gate_up_supported(sh.I, sh.D, gate->group_size) && qmv_m1_supported(sh.D, sh.I, down->group_size, 4) &&
-                     aligned16(down->w) && aligned16(down->s) && aligned16(down->b);
+  bool single_rows = !gemm && sh.stream_kernel != 1 && single_row_experts(gate, up, down, sh);
   for (size_t i = 0; i < n_items && single_rows; ++i) single_rows = batch_sizes_host[i] == 1;
   if (single_rows) {
     RMLX_TRY(dtab.alloc(n_items * 4, s));
@@ -1369,10 +1377,10 @@ int32_t rmlx_hip_expert_group_grouped_forward(const rmlx_qweight* gate, const rm
     RMLX_HIP_CHECK(hipStreamSynchronize(s));  // the caller's host array need not outlive the call
     RMLX_TRY(h.alloc(total * sh.I * 2, s));
     const uint32_t* experts = static_cast<const uint32_t*>(dtab.ptr);
-    RMLX_TRY(launch_qmv_m1_gate_up(gate_up_args(gate, up, sh, xk, static_cast<__half*>(h.ptr)), experts, rows, 1, sh.E, s));
-    RMLX_TRY(launch_qmv_m1_gather(down->w, down->s, down->b, (uint64_t)sh.D * (sh.I / 8), (uint64_t)sh.D * (sh.I / down->group_size),
-                                  sh.E, static_cast<const __half*>(h.ptr), experts, rows, static_cast<__half*>(out_f16_dev), sh.D,
-                                  sh.I, down->group_size, s));
+    RMLX_TRY(launch_qmv_m1_gate_up(gate_up_args(gate, up, sh, xk, static_cast<__half*>(h.ptr)), gate->bits, experts, rows, 1, sh.E, s));
+    RMLX_TRY(launch_qmv_m1_gather(down->w, down->s, down->b, (uint64_t)sh.D * (sh.I * down->bits / 32),
+                                  (uint64_t)sh.D * (sh.I / down->group_size), sh.E, static_cast<const __half*>(h.ptr), experts, rows,
+                                  static_cast<__half*>(out_f16_dev), sh.D, sh.I, down->group_size, down->bits, s));
     return finish(s);
   }
   RMLX_TRY(dtab.alloc(tab.size() * 4, s));
@@ -1412,9 +1420,10 @@ int32_t moe_grouped_impl(const rmlx_qweight* gate, const rmlx_qweight* up, const
   // workgroups of the direct form rank their token's experts themselves, so any number of tokens; `small`: at most 8
   // tokens, which the one-workgroup routing + grouping launch takes; everything else routes with the routing kernel and
   // goes on as if the caller had brought the picks.
-  const bool single_row = gate->bits == 4 && qmv_m1_gate_up_supported(sh.I, sh.D, gate->group_size);
-  const bool direct = ungrouped_pays(T32, sh.E, (uint32_t)top_k) && sh.stream_kernel != 1 && sh.wave_down && single_row &&
-                      (route == nullptr || sh.E <= 256) && qmv_wt_combine_supported(sh.D, sh.I, down->group_size, (uint32_t)top_k);
+  const bool direct = ungrouped_pays(T32, sh.E, (uint32_t)top_k) && sh.stream_kernel != 1 && single_row_experts(gate, up, down, sh) &&
+                      (route == nullptr || sh.E <= 256);
+  // (its down projection adds the weighted expert outputs itself where the wave-per-tile kernel takes the weights)
+  const bool fused_down = sh.wave_down && qmv_wt_combine_supported(sh.D, sh.I, down->group_size, (uint32_t)top_k);
   const bool small = route != nullptr && T32 <= 8 && route_sort_fusable(T32, sh.E, (uint32_t)top_k);
   if (route != nullptr && !direct && !small) {
     RMLX_TRY(launch_topk_route(route->logits, route->bias, T32, sh.E, (uint32_t)top_k, 1, route->idx_out, route->w_out, nullptr,
@@ -1444,6 +1453,40 @@ int32_t moe_grouped_impl(const rmlx_qweight* gate, const rmlx_qweight* up, const
     return fail(RMLX_NOT_FOUND, "MoeLayer: these expert weights run on the portable kernels, which the entry point "
                                 "without allocations does not cover (4-bit group 64 / 128 or 8-bit group 64, aligned "
                                 "buffers, dimensions in multiples of 512 / 256)");
+  // A few tokens: no grouping at all.  Every assignment is one row in assignment order, and the down
+  // projection adds the token's weighted expert outputs itself - two launches (gate / up that routes, down + combine)
+  // instead of four, no [assignments, D] intermediate.  An expert picked by two tokens is streamed once per
+  // token (at 4 tokens of 8 picks over 128 experts: 32 rows for 31 experts; see ungrouped_pays).
+  if (direct) {
+    if (!aligned16(xk)) return fail(RMLX_INVALID_SHAPE, "MoeLayer: input must be 16-byte aligned");
+    RMLX_TRY(h.alloc((size_t)A * sh.I * 2, s, arena));
+    // One row per expert: the gate / up projection on the single-row GEMV's layout (a wave per pair of gate and up rows,
+    // dot products instead of a matrix unit that would multiply 15 empty rows), and no routing launch: every workgroup
+    // ranks its token's experts itself, one wave, while the activations arrive (1 / 2 / 4 tokens of 8 picks: 23.4 / 37.0 /
+    // 59.5 us against 24.4 / 37.8 / 61.0 us with a routing launch in front).
+    QmvArgs a = gate_up_args(gate, up, sh, xk, static_cast<__half*>(h.ptr));
+    if (route != nullptr) {
+      a.route_logits = route->logits; a.route_bias = route->bias; a.route_idx_out = route->idx_out; a.route_w_out = route->w_out;
+      a.route_renorm = 1;
+    }
+    const uint32_t* picks = route != nullptr ? route->idx_out : expert_indices_dev;
+    const float* pick_weights = route != nullptr ? route->w_out : expert_weights_dev;
+    RMLX_TRY(launch_qmv_m1_gate_up(a, gate->bits, route != nullptr ? nullptr : picks, A, (uint32_t)top_k, sh.E, s));
+    const uint64_t down_stride_w = (uint64_t)sh.D * (sh.I * down->bits / 32), down_stride_s = (uint64_t)sh.D * (sh.I / down->group_size);
+    if (fused_down) {
+      RMLX_TRY(launch_qmv_wt_combine(down->w, down->s, down->b, down_stride_w, down_stride_s, sh.E, static_cast<const __half*>(h.ptr),
+                                     picks, pick_weights, T32, (uint32_t)top_k, sh.D, sh.I, static_cast<__half*>(out_f16_dev), s));
+    } else {
+      // other formats (8-bit, group sizes 32 / 128): the down projection as a single-row gather, then the weighted sum of
+      // a token's rows -- three launches
+      RMLX_TRY(y.alloc((size_t)A * sh.D * 2, s, arena));
+      RMLX_TRY(launch_qmv_m1_gather(down->w, down->s, down->b, down_stride_w, down_stride_s, sh.E, static_cast<const __half*>(h.ptr),
+                                    picks, A, static_cast<__half*>(y.ptr), sh.D, sh.I, down->group_size, down->bits, s));
+      RMLX_TRY(launch_moe_combine_rows_f16(static_cast<const __half*>(y.ptr), picks, pick_weights, T32, (uint32_t)top_k, sh.D, sh.E,
+                                           static_cast<__half*>(out_f16_dev), s));
+    }
+    return finish(s);
+  }
   if (sh.portable && !gemm) {
     // Assignments stay in their own order: position a holds token a / top_k and expert idx[a].
     if (route != nullptr)
@@ -1466,29 +1509,6 @@ int32_t moe_grouped_impl(const rmlx_qweight* gate, const rmlx_qweight* up, const
     return finish(s);
   }
   if (!aligned16(xk)) return fail(RMLX_INVALID_SHAPE, "MoeLayer: input must be 16-byte aligned");
-  // A few tokens: no grouping at all.  Every assignment is one row in assignment order, and the down
-  // projection adds the token's weighted expert outputs itself - two launches (gate / up that routes, down + combine)
-  // instead of four, no [assignments, D] intermediate.  An expert picked by two tokens is streamed once per
-  // token (at 4 tokens of 8 picks over 128 experts: 32 rows for 31 experts; see ungrouped_pays).
-  if (direct) {
-    RMLX_TRY(h.alloc((size_t)A * sh.I * 2, s, arena));
-    // One row per expert: the gate / up projection on the single-row GEMV's layout (a wave per pair of gate and up rows,
-    // dot products instead of a matrix unit that would multiply 15 empty rows), and no routing launch: every workgroup
-    // ranks its token's experts itself, one wave, while the activations arrive (1 / 2 / 4 tokens of 8 picks: 23.4 / 37.0 /
-    // 59.5 us against 24.4 / 37.8 / 61.0 us with a routing launch in front).
-    QmvArgs a = gate_up_args(gate, up, sh, xk, static_cast<__half*>(h.ptr));
-    if (route != nullptr) {
-      a.route_logits = route->logits; a.route_bias = route->bias; a.route_idx_out = route->idx_out; a.route_w_out = route->w_out;
-      a.route_renorm = 1;
-    }
-    const uint32_t* picks = route != nullptr ? route->idx_out : expert_indices_dev;
-    const float* pick_weights = route != nullptr ? route->w_out : expert_weights_dev;
-    RMLX_TRY(launch_qmv_m1_gate_up(a, route != nullptr ? nullptr : picks, A, (uint32_t)top_k, sh.E, s));
-    RMLX_TRY(launch_qmv_wt_combine(down->w, down->s, down->b, (uint64_t)sh.D * (sh.I / 8), (uint64_t)sh.D * (sh.I / down->group_size),
-                                   sh.E, static_cast<const __half*>(h.ptr), picks, pick_weights, T32, (uint32_t)top_k,
-                                   sh.D, sh.I, static_cast<__half*>(out_f16_dev), s));
-    return finish(s);
-  }
   // meta: sorted[A] | sorted_tok[A] | inv[A] | chunk_tab[3*max_chunks] | n_chunks[1]
   RMLX_TRY(meta.alloc(((size_t)3 * A + 3 * (size_t)max_chunks + 4) * 4, s, arena));
   uint32_t* sorted = static_cast<uint32_t*>(meta.ptr);

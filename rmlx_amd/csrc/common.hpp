@@ -149,16 +149,16 @@ int32_t launch_qmv_q4(const QmvArgs& a, hipStream_t s);
 bool qmv_q4_supported(uint32_t N, uint32_t K, uint32_t group_size);
 // Gate / up projection of single rows through chosen experts (qmv_m1.hip): position a = activation row a / top_k (x, no
 // row map) through expert idx[a] (idx == null: pick a % top_k of the ranking the kernel makes itself, see route_logits) of the two stacked matrices of `a` (w0 / w1, expert strides), out[a, :] = silu(gate) * up
-// in f16 [assignments, N]; 4-bit weights at group size 64, the shapes of the single-row GEMV.  chunk_tab / M / mr of `a` are not used.
-bool qmv_m1_gate_up_supported(uint32_t N, uint32_t K, uint32_t group_size);
+// in f16 [assignments, N]; 4- or 8-bit weights, the shapes of the single-row GEMV.  chunk_tab / M / mr of `a` are not used.
+bool qmv_m1_gate_up_supported(uint32_t N, uint32_t K, uint32_t group_size, uint32_t bits);
 // gather_qmm with one activation row per index on the single-row kernel (qmv_m1.hip): x [batch, K] f16, idx [batch]
-// (outside [0, n_experts): zeros), stacked 4-bit weights with strides in u32 words / halves, out [batch, N] f16; the
-// shapes qmv_m1_supported(N, K, group_size, 4) takes
+// (outside [0, n_experts): zeros), stacked 4- or 8-bit weights with strides in u32 words / halves, out [batch, N] f16;
+// the shapes qmv_m1_supported(N, K, group_size, bits) takes
 int32_t launch_qmv_m1_gather(const uint32_t* w, const __half* s, const __half* b, uint64_t estride_w, uint64_t estride_s,
                              uint32_t n_experts, const __half* x, const uint32_t* idx, uint32_t batch, __half* out, uint32_t N,
-                             uint32_t K, uint32_t group_size, hipStream_t stream);
-int32_t launch_qmv_m1_gate_up(const QmvArgs& a, const uint32_t* idx, uint32_t assignments, uint32_t top_k, uint32_t n_experts,
-                              hipStream_t stream);
+                             uint32_t K, uint32_t group_size, uint32_t bits, hipStream_t stream);
+int32_t launch_qmv_m1_gate_up(const QmvArgs& a, uint32_t bits, const uint32_t* idx, uint32_t assignments, uint32_t top_k,
+                              uint32_t n_experts, hipStream_t stream);
 // Wave-per-tile streaming GEMV (qmv_wt.hip): the same arguments; chunks of at most chunk_rows (8 or 16) rows, a wave owns
 // a 16-row weight tile over all of K (no cross-wave reduction), group size 64, K <= 4096 (16-row chunks: 8192)
 bool qmv_wt_supported(uint32_t N, uint32_t K, uint32_t group_size, uint32_t chunk_rows);
@@ -291,6 +291,10 @@ int32_t launch_identity_positions(uint32_t* tok, uint32_t* inv, uint32_t n, uint
 // out[t,:] = sum_k w[t*K+k] * y[inv[t*K+k],:]  (y f32 rows at sorted positions)
 int32_t launch_moe_combine(const float* y, const uint32_t* inv, const float* weights, uint32_t T,
                            uint32_t top_k, uint32_t D, __half* out, hipStream_t s);
+// The same over f16 rows in assignment order (row t * top_k + k is pick k of token t); idx: the assignments' experts
+// (outside [0, E): skipped)
+int32_t launch_moe_combine_rows_f16(const __half* y, const uint32_t* idx, const float* weights, uint32_t T, uint32_t top_k,
+                                    uint32_t D, uint32_t E, __half* out, hipStream_t s);
 int32_t launch_add_bias_rows(__half* out, const __half* bias, uint32_t M, uint32_t N, hipStream_t s);
 int32_t launch_awq_dequant(const uint32_t* qweight, const uint32_t* qzeros, const float* scales, float* out,
                            uint32_t rows, uint32_t cols, uint32_t group_size, hipStream_t s);

@@ -335,6 +335,44 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(const float* __restric
   *reinterpret_cast<uint2*>(out + (size_t)t * D + c) = o;
 }
 
+// The same sum over f16 rows in assignment order (no grouping: row t*K+k is pick k of token t): out[t,:] = sum_k
+// w[t*K+k] * y[t*K+k,:], k ascending, f32; an assignment whose expert id lies outside [0, E) contributes nothing.
+__global__ __launch_bounds__(256) void moe_combine_rows_f16_kernel(const __half* __restrict__ y,
+                                                                   const uint32_t* __restrict__ idx,
+                                                                   const float* __restrict__ weights, uint32_t top_k,
+                                                                   uint32_t D, uint32_t E, __half* __restrict__ out) {
+  const uint32_t t = blockIdx.x;
+  const uint32_t c = (blockIdx.y * 256 + threadIdx.x) * 4;
+  if (c >= D) return;
+  float w[8];
+  uint2 v[8];
+#pragma unroll
+  for (uint32_t k = 0; k < 8; ++k) {
+    w[k] = 0.f;
+    v[k] = make_uint2(0u, 0u);
+    if (k < top_k) {
+      const size_t a = (size_t)t * top_k + k;
+      if (idx[a] < E) {
+        w[k] = weights[a];
+        v[k] = *reinterpret_cast<const uint2*>(y + a * D + c);
+      }
+    }
+  }
+  float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+  for (uint32_t k = 0; k < 8; ++k) {
+    if (k < top_k) {
+      const float2 lo = __half22float2(*reinterpret_cast<const __half2*>(&v[k].x)), hi = __half22float2(*reinterpret_cast<const __half2*>(&v[k].y));
+      acc.x += w[k] * lo.x; acc.y += w[k] * lo.y; acc.z += w[k] * hi.x; acc.w += w[k] * hi.y;
+    }
+  }
+  const __half2 lo = __floats2half2_rn(acc.x, acc.y), hi = __floats2half2_rn(acc.z, acc.w);
+  uint2 o;
+  o.x = *reinterpret_cast<const uint32_t*>(&lo);
+  o.y = *reinterpret_cast<const uint32_t*>(&hi);
+  *reinterpret_cast<uint2*>(out + (size_t)t * D + c) = o;
+}
+
 }  // namespace
 
 int32_t launch_topk_route(const float* logits, const float* bias, uint32_t T, uint32_t E, uint32_t K,
@@ -436,6 +474,15 @@ int32_t launch_moe_combine(const float* y, const uint32_t* inv, const float* wei
   if (T == 0) return RMLX_OK;
   if (top_k > 8 || D % 4 != 0) return fail(RMLX_INVALID_SHAPE, "moe_combine: top_k <= 8 and D %% 4 == 0 required (top_k=%u D=%u)", top_k, D);
   hipLaunchKernelGGL(moe_combine_kernel, dim3(T, (D + 1023) / 1024), dim3(256), 0, s, y, inv, weights, top_k, D, T * top_k, out);
+  RMLX_HIP_CHECK(hipGetLastError());
+  return RMLX_OK;
+}
+
+int32_t launch_moe_combine_rows_f16(const __half* y, const uint32_t* idx, const float* weights, uint32_t T, uint32_t top_k,
+                                    uint32_t D, uint32_t E, __half* out, hipStream_t s) {
+  if (T == 0) return RMLX_OK;
+  if (top_k > 8 || D % 4 != 0) return fail(RMLX_INVALID_SHAPE, "moe_combine: top_k <= 8 and D %% 4 == 0 required (top_k=%u D=%u)", top_k, D);
+  hipLaunchKernelGGL(moe_combine_rows_f16_kernel, dim3(T, (D + 1023) / 1024), dim3(256), 0, s, y, idx, weights, top_k, D, E, out);
   RMLX_HIP_CHECK(hipGetLastError());
   return RMLX_OK;
 }

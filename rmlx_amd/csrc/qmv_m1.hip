@@ -591,9 +591,9 @@ __device__ __forceinline__ uint32_t gate_up_expert(const M1GateUpParams& p, uint
   return pick_idx[pick];
 }
 
-template <int GS>
+template <int BITS, int GS>
 __global__ __launch_bounds__(kThreads, 1) void qmv_m1_gate_up_kernel(M1GateUpParams p) {
-  using Image = XImage<4, 1>;
+  using Image = XImage<BITS, 1>;
   constexpr int kChunkK = Image::kChunkK, kLaneK = Image::kLaneK;
   constexpr int kLanesPerGroup = GS / kLaneK, kGroupsPerChunk = kChunkK / GS;
   extern __shared__ __attribute__((aligned(16))) char lds[];
@@ -605,7 +605,7 @@ __global__ __launch_bounds__(kThreads, 1) void qmv_m1_gate_up_kernel(M1GateUpPar
 
   // loads, small ones first (the memory counter retires in order): the activations, the expert, then the rows
   u4 xv[1][4];
-  load_activations<4, 1, false>(img, x, 1u, 0u, nullptr, nullptr, tid, xv);
+  load_activations<BITS, 1, false>(img, x, 1u, 0u, nullptr, nullptr, tid, xv);
   uint32_t expert = gate_up_expert(p, a, blockIdx.x == 0);
   const bool zeros = expert >= p.n_experts;
   expert = zeros ? 0u : expert;
@@ -615,7 +615,7 @@ __global__ __launch_bounds__(kThreads, 1) void qmv_m1_gate_up_kernel(M1GateUpPar
   const unsigned short* brow[2];
 #pragma unroll
   for (int r = 0; r < 2; ++r) {
-    wrow[r] = reinterpret_cast<const u4*>((r == 0 ? p.w0 : p.w1) + expert * p.estride_w + (uint64_t)row * (K / 8));
+    wrow[r] = reinterpret_cast<const u4*>((r == 0 ? p.w0 : p.w1) + expert * p.estride_w + (uint64_t)row * (K * BITS / 32));
     srow[r] = reinterpret_cast<const unsigned short*>((r == 0 ? p.s0 : p.s1) + expert * p.estride_s) + (uint64_t)row * G;
     brow[r] = reinterpret_cast<const unsigned short*>((r == 0 ? p.b0 : p.b1) + expert * p.estride_s) + (uint64_t)row * G;
   }
@@ -637,7 +637,7 @@ __global__ __launch_bounds__(kThreads, 1) void qmv_m1_gate_up_kernel(M1GateUpPar
   };
   Batch ba, bb;
   load_batch(0, ba);
-  stage_activations<4, 1, false>(img, x, 1u, 0u, nullptr, nullptr, tid, xv);
+  stage_activations<BITS, 1, false>(img, x, 1u, 0u, nullptr, nullptr, tid, xv);
   __syncthreads();
 
   float racc[2][1] = {{0.f}, {0.f}};
@@ -646,7 +646,7 @@ __global__ __launch_bounds__(kThreads, 1) void qmv_m1_gate_up_kernel(M1GateUpPar
   auto process = [&](uint32_t c0, const Batch& t) {
 #pragma unroll
     for (int cc = 0; cc < 2; ++cc)
-      if (c0 + cc < KH) dot_chunk<4, 2, 1>(img, c0 + cc, lane, t.w[cc], t.s[cc], t.b[cc], uc, racc);
+      if (c0 + cc < KH) dot_chunk<BITS, 2, 1>(img, c0 + cc, lane, t.w[cc], t.s[cc], t.b[cc], uc, racc);
   };
   for (uint32_t c0 = 0; c0 < KH; c0 += 4) {
     const bool more1 = c0 + 2 < KH, more2 = c0 + 4 < KH;
@@ -664,9 +664,9 @@ __global__ __launch_bounds__(kThreads, 1) void qmv_m1_gate_up_kernel(M1GateUpPar
 // The same for more row blocks than the chip keeps resident (a few tokens: assignments x N / 8 blocks): the grid is
 // (resident workgroups / assignments, assignments) and a workgroup walks the row blocks blockIdx.x, blockIdx.x + gridDim.x,
 // ... of its assignment, staging the activations once, the next block's weights in flight while the current one is multiplied.
-template <int GS>
+template <int BITS, int GS>
 __global__ __launch_bounds__(kThreads, 1) void qmv_m1_gate_up_loop_kernel(M1GateUpParams p) {
-  using Image = XImage<4, 1>;
+  using Image = XImage<BITS, 1>;
   constexpr int kChunkK = Image::kChunkK, kLaneK = Image::kLaneK;
   constexpr int kLanesPerGroup = GS / kLaneK, kGroupsPerChunk = kChunkK / GS;
   extern __shared__ __attribute__((aligned(16))) char lds[];
@@ -680,7 +680,7 @@ __global__ __launch_bounds__(kThreads, 1) void qmv_m1_gate_up_loop_kernel(M1Gate
   auto block_row = [&](uint32_t i) { return (blockIdx.x + i * gridDim.x) * kWaves + wave; };
 
   u4 xv[1][4];
-  load_activations<4, 1, false>(img, x, 1u, 0u, nullptr, nullptr, tid, xv);
+  load_activations<BITS, 1, false>(img, x, 1u, 0u, nullptr, nullptr, tid, xv);
   uint32_t expert = gate_up_expert(p, a, blockIdx.x == 0);
   const bool zeros = expert >= p.n_experts;
   expert = zeros ? 0u : expert;
@@ -694,7 +694,7 @@ __global__ __launch_bounds__(kThreads, 1) void qmv_m1_gate_up_loop_kernel(M1Gate
     const unsigned short* brow[2];
 #pragma unroll
     for (int r = 0; r < 2; ++r) {
-      wrow[r] = reinterpret_cast<const u4*>((r == 0 ? p.w0 : p.w1) + expert * p.estride_w + (uint64_t)row * (K / 8));
+      wrow[r] = reinterpret_cast<const u4*>((r == 0 ? p.w0 : p.w1) + expert * p.estride_w + (uint64_t)row * (K * BITS / 32));
       srow[r] = reinterpret_cast<const unsigned short*>((r == 0 ? p.s0 : p.s1) + expert * p.estride_s) + (uint64_t)row * G;
       brow[r] = reinterpret_cast<const unsigned short*>((r == 0 ? p.b0 : p.b1) + expert * p.estride_s) + (uint64_t)row * G;
     }
@@ -717,7 +717,7 @@ __global__ __launch_bounds__(kThreads, 1) void qmv_m1_gate_up_loop_kernel(M1Gate
   };
   Batch ba, bb;
   if (n_batches > 0) load_batch(ba);
-  stage_activations<4, 1, false>(img, x, 1u, 0u, nullptr, nullptr, tid, xv);
+  stage_activations<BITS, 1, false>(img, x, 1u, 0u, nullptr, nullptr, tid, xv);
   __syncthreads();
 
   float racc[2][1];
@@ -728,7 +728,7 @@ __global__ __launch_bounds__(kThreads, 1) void qmv_m1_gate_up_loop_kernel(M1Gate
     if (pr_c0 == 0) { racc[0][0] = 0.f; racc[1][0] = 0.f; }
 #pragma unroll
     for (int cc = 0; cc < 2; ++cc)
-      if (pr_c0 + cc < KH) dot_chunk<4, 2, 1>(img, pr_c0 + cc, lane, t.w[cc], t.s[cc], t.b[cc], uc, racc);
+      if (pr_c0 + cc < KH) dot_chunk<BITS, 2, 1>(img, pr_c0 + cc, lane, t.w[cc], t.s[cc], t.b[cc], uc, racc);
     pr_c0 += 2;
     if (pr_c0 >= KH) {  // the block is complete
       const float g = wave_sum(racc[0][0]), u = wave_sum(racc[1][0]);
@@ -886,38 +886,60 @@ int32_t launch_qmv_m1(const uint32_t* w, const __half* s, const __half* b, const
   return RMLX_OK;
 }
 
-// gather_qmm with one activation row per index: row m of x [batch, K] through expert idx[m] of the stacked 4-bit
+namespace {
+template <int BITS>
+void launch_gather_bits(const M1Params& p, uint32_t group_size, bool two, hipStream_t stream) {
+  const size_t lds = lds_per_row<BITS>(p.K);
+  switch (group_size) {
+    case 32: if (two) launch_k<BITS, 32, 2, false, 1, false, 1, true>(p, lds, stream); else launch_k<BITS, 32, 1, false, 1, false, 1, true>(p, lds, stream); break;
+    case 64: if (two) launch_k<BITS, 64, 2, false, 1, false, 1, true>(p, lds, stream); else launch_k<BITS, 64, 1, false, 1, false, 1, true>(p, lds, stream); break;
+    default: if (two) launch_k<BITS, 128, 2, false, 1, false, 1, true>(p, lds, stream); else launch_k<BITS, 128, 1, false, 1, false, 1, true>(p, lds, stream); break;
+  }
+}
+}  // namespace
+
+// gather_qmm with one activation row per index: row m of x [batch, K] through expert idx[m] of the stacked 4- or 8-bit
 // weights, out [batch, N] f16.  One launch, no chunk table: the activation row of a pass picks its matrix.
 int32_t launch_qmv_m1_gather(const uint32_t* w, const __half* s, const __half* b, uint64_t estride_w, uint64_t estride_s,
                              uint32_t n_experts, const __half* x, const uint32_t* idx, uint32_t batch, __half* out, uint32_t N,
-                             uint32_t K, uint32_t group_size, hipStream_t stream) {
-  if (!qmv_m1_supported(N, K, group_size, 4))
-    return fail(RMLX_INVALID_SHAPE, "qmv_m1 gather: unsupported shape N=%u K=%u group_size=%u", N, K, group_size);
-  const size_t lds = lds_per_row<4>(K);
+                             uint32_t K, uint32_t group_size, uint32_t bits, hipStream_t stream) {
+  if (!qmv_m1_supported(N, K, group_size, bits))
+    return fail(RMLX_INVALID_SHAPE, "qmv_m1 gather: unsupported shape N=%u K=%u bits=%u group_size=%u", N, K, bits, group_size);
   // (weights loaded with the ordinary cache policy: two indices may name one expert)
-  const bool two = (K >= 12288 || N >= 12288) && N % (kWaves * 2) == 0;
+  const bool two = (K >= 12288 || (bits == 4 && N >= 12288)) && N % (kWaves * 2) == 0;
   for (uint32_t first = 0; first < batch; first += 65535) {  // the activation row is the second grid dimension
     const uint32_t rows = batch - first < 65535 ? batch - first : 65535;
     M1Params p{w, s, b, x + (uint64_t)first * K, out + (uint64_t)first * N, N, K, rows, EPI_NONE, 0, nullptr, nullptr, nullptr,
                idx + first, estride_w, estride_s, n_experts};
-    switch (group_size) {
-      case 32: if (two) launch_k<4, 32, 2, false, 1, false, 1, true>(p, lds, stream); else launch_k<4, 32, 1, false, 1, false, 1, true>(p, lds, stream); break;
-      case 64: if (two) launch_k<4, 64, 2, false, 1, false, 1, true>(p, lds, stream); else launch_k<4, 64, 1, false, 1, false, 1, true>(p, lds, stream); break;
-      default: if (two) launch_k<4, 128, 2, false, 1, false, 1, true>(p, lds, stream); else launch_k<4, 128, 1, false, 1, false, 1, true>(p, lds, stream); break;
-    }
+    if (bits == 4) launch_gather_bits<4>(p, group_size, two, stream);
+    else launch_gather_bits<8>(p, group_size, two, stream);
     RMLX_HIP_CHECK(hipGetLastError());
   }
   return RMLX_OK;
 }
 
-bool qmv_m1_gate_up_supported(uint32_t N, uint32_t K, uint32_t group_size) {
-  return group_size == 64 && qmv_m1_supported(N, K, group_size, 4);  // (what the routed block of a few tokens runs)
+bool qmv_m1_gate_up_supported(uint32_t N, uint32_t K, uint32_t group_size, uint32_t bits) {
+  return qmv_m1_supported(N, K, group_size, bits);
 }
 
-int32_t launch_qmv_m1_gate_up(const QmvArgs& a, const uint32_t* idx, uint32_t assignments, uint32_t top_k, uint32_t n_experts,
-                              hipStream_t stream) {
-  if (!qmv_m1_gate_up_supported(a.N, a.K, a.group_size))
-    return fail(RMLX_INVALID_SHAPE, "qmv_m1 gate/up: unsupported shape N=%u K=%u group_size=%u", a.N, a.K, a.group_size);
+namespace {
+template <int BITS, int GS>
+void launch_gate_up(const M1GateUpParams& p, uint32_t assignments, hipStream_t stream) {
+  const size_t lds = lds_per_row<BITS>(p.K);
+  const uint32_t nblk = p.N / kWaves;
+  // one workgroup per row block while all of them are resident together, else as many as are (they loop)
+  auto looping = qmv_m1_gate_up_loop_kernel<BITS, GS>;
+  uint32_t gx = resident_workgroups(looping, lds) / assignments;
+  gx = gx < 1 ? 1 : gx;
+  if (gx < nblk) hipLaunchKernelGGL(looping, dim3(gx, assignments), dim3(kThreads), lds, stream, p);
+  else hipLaunchKernelGGL((qmv_m1_gate_up_kernel<BITS, GS>), dim3(nblk, assignments), dim3(kThreads), lds, stream, p);
+}
+}  // namespace
+
+int32_t launch_qmv_m1_gate_up(const QmvArgs& a, uint32_t bits, const uint32_t* idx, uint32_t assignments, uint32_t top_k,
+                              uint32_t n_experts, hipStream_t stream) {
+  if (!qmv_m1_gate_up_supported(a.N, a.K, a.group_size, bits))
+    return fail(RMLX_INVALID_SHAPE, "qmv_m1 gate/up: unsupported shape N=%u K=%u bits=%u group_size=%u", a.N, a.K, bits, a.group_size);
   if (assignments == 0) return RMLX_OK;
   const bool routes = idx == nullptr;
   if (assignments > 65535 || top_k == 0 || a.w1 == nullptr || a.out_f32 || a.ld_out != a.N ||
@@ -928,14 +950,19 @@ int32_t launch_qmv_m1_gate_up(const QmvArgs& a, const uint32_t* idx, uint32_t as
   M1GateUpParams p{a.w0, a.s0, a.b0, a.w1, a.s1, a.b1, a.expert_stride_w, a.expert_stride_s, a.x, idx,
                    static_cast<__half*>(a.out), a.N, a.K, top_k, n_experts,
                    a.route_logits, a.route_bias, a.route_idx_out, a.route_w_out, a.route_renorm};
-  const size_t lds = lds_per_row<4>(a.K);
-  const dim3 grid(a.N / kWaves, assignments);
-  // one workgroup per row block while all of them are resident together, else as many as are (they loop)
-  auto looping = qmv_m1_gate_up_loop_kernel<64>;
-  uint32_t gx = resident_workgroups(looping, lds) / assignments;
-  gx = gx < 1 ? 1 : gx;
-  if (gx < grid.x) hipLaunchKernelGGL(looping, dim3(gx, assignments), dim3(kThreads), lds, stream, p);
-  else hipLaunchKernelGGL(qmv_m1_gate_up_kernel<64>, grid, dim3(kThreads), lds, stream, p);
+  if (bits == 4) {
+    switch (a.group_size) {
+      case 32: launch_gate_up<4, 32>(p, assignments, stream); break;
+      case 64: launch_gate_up<4, 64>(p, assignments, stream); break;
+      default: launch_gate_up<4, 128>(p, assignments, stream); break;
+    }
+  } else {
+    switch (a.group_size) {
+      case 32: launch_gate_up<8, 32>(p, assignments, stream); break;
+      case 64: launch_gate_up<8, 64>(p, assignments, stream); break;
+      default: launch_gate_up<8, 128>(p, assignments, stream); break;
+    }
+  }
   RMLX_HIP_CHECK(hipGetLastError());
   return RMLX_OK;
 }

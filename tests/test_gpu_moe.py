@@ -453,6 +453,39 @@ def test_moe_forward_of_a_few_tokens(hip, T, K, E, D, I, fused):
         assert np.abs(one.astype(np.float64) - two.astype(np.float64)).max() <= model.tolerance(ref)
 
 
+@pytest.mark.parametrize("bits,gs", [(8, 64), (8, 32), (8, 128), (4, 32), (4, 128)])
+@pytest.mark.parametrize("T,K,E,D,I", [(1, 8, 16, 1024, 512), (3, 4, 32, 512, 1024)])
+def test_moe_forward_of_a_few_tokens_other_formats(hip, bits, gs, T, K, E, D, I):
+    """The form without grouping for 8-bit experts and for group sizes 32 / 128: gate / up on the single-row kernel, the down
+    projection as a single-row gather and the weighted sum of a token's rows in a launch of its own.  Against the oracle,
+    with logits and with the caller's picks, and through ExpertGroup with one row per item."""
+    from rmlx_amd import ops
+    from rmlx_amd.runtime import DeviceBuffer
+    rng = np.random.default_rng(bits * 1000 + gs + T)
+    gu = make_weight(rng, 2 * I, D, bits, gs, lead=(E,))
+    down = make_weight(rng, D, I, bits, gs, lead=(E,))
+    gate, up = tuple(a[:, :I] for a in gu), tuple(a[:, I:] for a in gu)
+    gh, dh = ops.QuantizedWeight.from_numpy(*gu, gs, bits), ops.QuantizedWeight.from_numpy(*down, gs, bits)
+    x = make_x(rng, T, D)
+    logits = rng.standard_normal((T, E)).astype(np.float32)
+    idx, w, _, _ = model.topk_route(logits, K)
+    ref = model.moe_forward(x, idx, w, gate, up, down, gs, K, bits=bits)
+    print(f"few tokens Q{bits} gs{gs} T={T} K={K} E={E} D={D} I={I}", flush=True)
+    xd = DeviceBuffer.from_numpy(x)
+    assert_close(ops.moe_forward(gh, None, dh, xd, DeviceBuffer.from_numpy(logits), K).numpy(), ref, "moe_forward")
+    bad = idx.copy().reshape(-1)
+    w_ref = w.copy().reshape(-1)
+    bad[1 % bad.size] = E + 7
+    w_ref[1 % bad.size] = 0.0
+    out = ops.moe_forward_grouped(gh, None, dh, xd, DeviceBuffer.from_numpy(bad.astype(np.uint32)), DeviceBuffer.from_numpy(w.reshape(-1)), K).numpy()
+    assert_close(out, model.moe_forward(x, idx, w_ref.reshape(w.shape), gate, up, down, gs, K, bits=bits), "moe_forward_grouped, one pick out of range")
+    group = ops.ExpertGroup(gh, None, dh)
+    items = [(int(e), x[:1]) for e in idx.reshape(-1)[:3]]
+    for (e, xi), (_, y) in zip(items, group.grouped_forward([(e, DeviceBuffer.from_numpy(xi)) for e, xi in items])):
+        one = model.moe_forward(xi, np.array([[e]]), np.ones((1, 1), np.float32), gate, up, down, gs, 1, bits=bits)
+        assert_close(y, one, f"ExpertGroup expert {e}")
+
+
 @pytest.mark.parametrize("T,K", [(1, 2), (1, 8), (2, 3), (3, 4)])
 def test_moe_forward_grouped_with_repeated_experts(hip, T, K):
     """Caller-supplied picks may name one expert several times for a token; decode-sized batches run kernels
