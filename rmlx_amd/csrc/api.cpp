@@ -464,17 +464,17 @@ struct ExpertShapes {
 // gather_qmm takes raw buffers, so its GEMV / grouped-GEMM crossover is a constant: every entry has exactly
 // m_per_batch rows, the streaming GEMV wastes nothing up to a full chunk of 8 rows, and the GEMM wins from 9 rows on.
 constexpr uint32_t kGatherGemmMinRows = 9;
-// routed block: up to this many assignments run without grouping (every assignment its own chunk, combine fused into
-// the down projection)
+// routed block: the form without grouping (every assignment a row of its own) is never taken beyond this many assignments
 constexpr uint32_t kDirectMaxAssignments = 128;
 // The form without grouping streams an expert once per assignment instead of once per distinct expert of the batch (at
 // about 6 against 5 TB/s, and without the grouping launch): worth it while the assignments are at most 1.3 x the distinct
 // experts a uniform router picks, E (1 - (1 - K/E)^T).  Measured at E = 128, top-8: 9 tokens 127 against 137 us, 10 tokens
-// 141 against 141, 12 tokens 170 against 162.
-bool ungrouped_pays(uint32_t T, uint32_t E, uint32_t K) {
+// 141 against 141, 12 tokens 170 against 162; 8-bit experts (three launches): 10 / 11 tokens 267 / 301 against 281 / 309 us, 12
+// tokens 321 against 314: 1.37 x.
+bool ungrouped_pays(uint32_t T, uint32_t E, uint32_t K, uint32_t bits) {
   if (E == 0 || K > E) return false;
   const double distinct = E * (1.0 - std::pow(1.0 - (double)K / E, (double)T));
-  return (uint64_t)T * K <= kDirectMaxAssignments && (double)T * K <= 1.3 * distinct;
+  return (uint64_t)T * K <= kDirectMaxAssignments && (double)T * K <= (bits == 8 ? 1.37 : 1.3) * distinct;
 }
 enum { GATHER_AUTO = 0, GATHER_STREAM = 1, GATHER_GEMM = 2, GATHER_PORTABLE = 3 };
 
@@ -1420,7 +1420,7 @@ int32_t moe_grouped_impl(const rmlx_qweight* gate, const rmlx_qweight* up, const
   // workgroups of the direct form rank their token's experts themselves, so any number of tokens; `small`: at most 8
   // tokens, which the one-workgroup routing + grouping launch takes; everything else routes with the routing kernel and
   // goes on as if the caller had brought the picks.
-  const bool direct = ungrouped_pays(T32, sh.E, (uint32_t)top_k) && sh.stream_kernel != 1 && single_row_experts(gate, up, down, sh) &&
+  const bool direct = ungrouped_pays(T32, sh.E, (uint32_t)top_k, gate->bits) && sh.stream_kernel != 1 && single_row_experts(gate, up, down, sh) &&
                       (route == nullptr || sh.E <= 256);
   // (its down projection adds the weighted expert outputs itself where the wave-per-tile kernel takes the weights)
   const bool fused_down = sh.wave_down && qmv_wt_combine_supported(sh.D, sh.I, down->group_size, (uint32_t)top_k);
