@@ -1473,12 +1473,16 @@ int32_t moe_grouped_impl(const rmlx_qweight* gate, const rmlx_qweight* up, const
     const float* pick_weights = route != nullptr ? route->w_out : expert_weights_dev;
     RMLX_TRY(launch_qmv_m1_gate_up(a, gate->bits, route != nullptr ? nullptr : picks, A, (uint32_t)top_k, sh.E, s));
     const uint64_t down_stride_w = (uint64_t)sh.D * (sh.I * down->bits / 32), down_stride_s = (uint64_t)sh.D * (sh.I / down->group_size);
-    if (fused_down) {
+    if (qmv_m1_down_combine_supported(sh.D, sh.I, down->group_size, down->bits, (uint32_t)top_k)) {
+      RMLX_TRY(launch_qmv_m1_down_combine(down->w, down->s, down->b, down_stride_w, down_stride_s, sh.E, static_cast<const __half*>(h.ptr),
+                                          picks, pick_weights, T32, (uint32_t)top_k, sh.D, sh.I, down->group_size, down->bits,
+                                          static_cast<__half*>(out_f16_dev), s));
+    } else if (fused_down) {
       RMLX_TRY(launch_qmv_wt_combine(down->w, down->s, down->b, down_stride_w, down_stride_s, sh.E, static_cast<const __half*>(h.ptr),
                                      picks, pick_weights, T32, (uint32_t)top_k, sh.D, sh.I, static_cast<__half*>(out_f16_dev), s));
     } else {
-      // other formats (8-bit, group sizes 32 / 128): the down projection as a single-row gather, then the weighted sum of
-      // a token's rows -- three launches
+      // other formats (4-bit at group sizes 32 / 128, 8-bit with a long intermediate dimension): the down projection as a
+      // single-row gather, then the weighted sum of a token's rows -- three launches
       RMLX_TRY(y.alloc((size_t)A * sh.D * 2, s, arena));
       RMLX_TRY(launch_qmv_m1_gather(down->w, down->s, down->b, down_stride_w, down_stride_s, sh.E, static_cast<const __half*>(h.ptr),
                                     picks, A, static_cast<__half*>(y.ptr), sh.D, sh.I, down->group_size, down->bits, s));

@@ -159,6 +159,14 @@ int32_t launch_qmv_m1_gather(const uint32_t* w, const __half* s, const __half* b
                              uint32_t K, uint32_t group_size, uint32_t bits, hipStream_t stream);
 int32_t launch_qmv_m1_gate_up(const QmvArgs& a, uint32_t bits, const uint32_t* idx, uint32_t assignments, uint32_t top_k,
                               uint32_t n_experts, hipStream_t stream);
+// Down projection of a few tokens with the weighted combine behind it on the single-row layout (qmv_m1.hip): h
+// [T * top_k, K] f16 in assignment order, out[t] = sum_k wts[t, k] * (h[t * top_k + k] . W[idx[t * top_k + k]]^T) in ascending
+// k, f16 [T, N]; 8-bit weights, K at most two wave-wide chunks (2048), N % 4 == 0
+bool qmv_m1_down_combine_supported(uint32_t N, uint32_t K, uint32_t group_size, uint32_t bits, uint32_t top_k);
+int32_t launch_qmv_m1_down_combine(const uint32_t* w, const __half* s, const __half* b, uint64_t estride_w, uint64_t estride_s,
+                                   uint32_t n_experts, const __half* h, const uint32_t* idx, const float* wts, uint32_t T,
+                                   uint32_t top_k, uint32_t N, uint32_t K, uint32_t group_size, uint32_t bits, __half* out,
+                                   hipStream_t stream);
 // Wave-per-tile streaming GEMV (qmv_wt.hip): the same arguments; chunks of at most chunk_rows (8 or 16) rows, a wave owns
 // a 16-row weight tile over all of K (no cross-wave reduction), group size 64, K <= 4096 (16-row chunks: 8192)
 bool qmv_wt_supported(uint32_t N, uint32_t K, uint32_t group_size, uint32_t chunk_rows);

@@ -205,22 +205,12 @@ struct UnpackConsts { uint32_t m0, m1, k0, k1; };
 
 // 3. One chunk of the wave's R rows against the registers of x read from LDS:
 //    racc[r][m] += scale * (sum(x * (off + q)) - sum(off * x)) + bias * sum(x)
+// (the products: xr = the lane's activations of the chunk in the order of the unpacking, k = their sums (sum(off * x), sum(x)))
 template <int BITS, int R, int MR>
-__device__ __forceinline__ void dot_chunk(const XImage<BITS, MR> g, uint32_t c, int lane, const u4 (&w)[R],
-                                          const uint32_t (&s)[R], const uint32_t (&b)[R], const UnpackConsts& uc,
-                                          float (&racc)[R][MR]) {
+__device__ __forceinline__ void dot_rows(const uint32_t (&xr)[MR][XImage<BITS, MR>::kXU][4], const float2 (&k)[MR],
+                                         const u4 (&w)[R], const uint32_t (&s)[R], const uint32_t (&b)[R],
+                                         const UnpackConsts& uc, float (&racc)[R][MR]) {
   constexpr int kXU = XImage<BITS, MR>::kXU;
-  uint32_t xr[MR][kXU][4];
-  float2 k[MR];
-#pragma unroll
-  for (int m = 0; m < MR; ++m) {
-#pragma unroll
-    for (int j = 0; j < kXU; ++j) {
-      const u4 v = g.xl(m)[(c * kXU + j) * 64 + lane];
-      xr[m][j][0] = v.x; xr[m][j][1] = v.y; xr[m][j][2] = v.z; xr[m][j][3] = v.w;
-    }
-    k[m] = g.cs(m)[c * 64 + lane];
-  }
 #pragma unroll
   for (int r = 0; r < R; ++r) {
     const u4 wv = w[r];
@@ -257,6 +247,25 @@ __device__ __forceinline__ void dot_chunk(const XImage<BITS, MR> g, uint32_t c, 
 #pragma unroll
     for (int m = 0; m < MR; ++m) racc[r][m] += sc * ((acc0[m] + acc1[m]) - k[m].x) + bi * k[m].y;
   }
+}
+
+template <int BITS, int R, int MR>
+__device__ __forceinline__ void dot_chunk(const XImage<BITS, MR> g, uint32_t c, int lane, const u4 (&w)[R],
+                                          const uint32_t (&s)[R], const uint32_t (&b)[R], const UnpackConsts& uc,
+                                          float (&racc)[R][MR]) {
+  constexpr int kXU = XImage<BITS, MR>::kXU;
+  uint32_t xr[MR][kXU][4];
+  float2 k[MR];
+#pragma unroll
+  for (int m = 0; m < MR; ++m) {
+#pragma unroll
+    for (int j = 0; j < kXU; ++j) {
+      const u4 v = g.xl(m)[(c * kXU + j) * 64 + lane];
+      xr[m][j][0] = v.x; xr[m][j][1] = v.y; xr[m][j][2] = v.z; xr[m][j][3] = v.w;
+    }
+    k[m] = g.cs(m)[c * 64 + lane];
+  }
+  dot_rows<BITS, R, MR>(xr, k, w, s, b, uc, racc);
   // (several activation rows: keeps the LDS reads of the next chunk from being hoisted above this one, which would
   // double the registers of x that are live)
   if constexpr (MR > 1) __builtin_amdgcn_sched_barrier(0);
@@ -748,6 +757,109 @@ __global__ __launch_bounds__(kThreads, 1) void qmv_m1_gate_up_loop_kernel(M1Gate
   }
 }
 
+// ---- down projection of a few tokens with the weighted combine behind it, single-row layout -----------------------
+// One workgroup per (token t, block of R output columns): wave k multiplies the hidden row of the token's k-th
+// assignment (row t * top_k + k of h) with R weight rows of that assignment's expert; K is at most NC chunks, so a lane
+// keeps its activations (and their sums) in registers -- no image in LDS, no barrier before the products.  The eight
+// waves' results meet in LDS and thread r adds out[t, n] = sum_k w[t,k] * y_k[n] in ascending k, the order and f32
+// arithmetic of the combine kernel, and writes f16.  An expert index outside [0, n_experts) contributes nothing.
+struct M1DownParams {
+  const uint32_t* w; const __half* s; const __half* b;  // stacked down weights, expert 0
+  uint64_t estride_w, estride_s;                        // u32 words / halves per expert
+  const __half* h;        // [T * top_k, K] f16
+  const uint32_t* idx;    // [T * top_k]
+  const float* wts;       // [T * top_k]
+  __half* out;            // [T, N] f16
+  uint32_t N, K, top_k, n_experts;
+};
+
+template <int BITS, int GS, int NC, int R>
+__global__ __launch_bounds__(kThreads, 2) void qmv_m1_down_combine_kernel(M1DownParams p) {
+  using Image = XImage<BITS, 1>;
+  constexpr int kChunkK = Image::kChunkK, kLaneK = Image::kLaneK, kXU = Image::kXU;
+  constexpr int kLanesPerGroup = GS / kLaneK, kGroupsPerChunk = kChunkK / GS;
+  __shared__ float red[kWaves][R];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const uint32_t K = p.K, G = K / GS, row_u4 = K / kLaneK, nunits = K / 8;
+  const uint32_t t = blockIdx.y, n0 = blockIdx.x * R, a = t * p.top_k + wave;
+  uint32_t expert = 0xFFFFFFFFu;
+  float cw = 0.f;
+  if ((uint32_t)wave < p.top_k) {
+    expert = p.idx[a];
+    cw = p.wts[a];
+  }
+  float res[R];
+#pragma unroll
+  for (int r = 0; r < R; ++r) res[r] = 0.f;
+  if (expert < p.n_experts) {  // (wave-uniform)
+    // loads, small ones first: the lane's activations, the scales and biases, then the weights
+    const u4* xg = reinterpret_cast<const u4*>(p.h + (uint64_t)a * K);
+    u4 xv[NC][kXU];
+#pragma unroll
+    for (int c = 0; c < NC; ++c)
+#pragma unroll
+      for (int j = 0; j < kXU; ++j) {
+        const uint32_t u = (c * 64 + lane) * kXU + j;
+        xv[c][j] = xg[u < nunits ? u : nunits - 1];
+      }
+    u4 wv[NC][R];
+    uint32_t sv[NC][R], bv[NC][R];
+#pragma unroll
+    for (int c = 0; c < NC; ++c) {
+      uint32_t wi = c * 64 + lane, gi = c * kGroupsPerChunk + lane / kLanesPerGroup;
+      wi = wi < row_u4 ? wi : row_u4 - 1;  // lanes past K meet zeros in the activations
+      gi = gi < G ? gi : G - 1;
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        sv[c][r] = reinterpret_cast<const unsigned short*>(p.s + expert * p.estride_s)[(uint64_t)(n0 + r) * G + gi];
+        bv[c][r] = reinterpret_cast<const unsigned short*>(p.b + expert * p.estride_s)[(uint64_t)(n0 + r) * G + gi];
+      }
+#pragma unroll
+      for (int r = 0; r < R; ++r)
+        wv[c][r] = reinterpret_cast<const u4*>(p.w + expert * p.estride_w + (uint64_t)(n0 + r) * (K * BITS / 32))[wi];
+    }
+    UnpackConsts uc{0x000F000Fu, 0x00F000F0u, 0x64006400u, 0x54005400u};
+    asm volatile("" : "+s"(uc.m0), "+s"(uc.m1), "+v"(uc.k0), "+v"(uc.k1));
+    float racc[R][1];
+#pragma unroll
+    for (int r = 0; r < R; ++r) racc[r][0] = 0.f;
+#pragma unroll
+    for (int c = 0; c < NC; ++c) {
+      // the lane's activations in the order of the unpacking and their sums (zeros past K)
+      uint32_t xr[1][kXU][4];
+      float xs = 0.f, xo = 0.f;
+#pragma unroll
+      for (int j = 0; j < kXU; ++j) {
+        const bool inside = (c * 64 + lane) * kXU + j < nunits;
+        const u4 raw = inside ? xv[c][j] : (u4){0u, 0u, 0u, 0u};
+        const u4 v = BITS == 4 ? to_pair_order(raw) : raw;
+        xr[0][j][0] = v.x; xr[0][j][1] = v.y; xr[0][j][2] = v.z; xr[0][j][3] = v.w;
+        const h8 hv = __builtin_bit_cast(h8, raw);
+#pragma unroll
+        for (int e = 0; e < 8; e += 2) {
+          xs += (float)hv[e] + (float)hv[e + 1];
+          xo += 1024.0f * (float)hv[e] + (BITS == 4 ? 64.0f : 1024.0f) * (float)hv[e + 1];
+        }
+      }
+      const float2 k1[1] = {make_float2(xo, xs)};
+      dot_rows<BITS, R, 1>(xr, k1, wv[c], sv[c], bv[c], uc, racc);
+    }
+#pragma unroll
+    for (int r = 0; r < R; ++r) res[r] = wave_sum(racc[r][0]) * cw;
+  }
+  if (lane == 0) {
+#pragma unroll
+    for (int r = 0; r < R; ++r) red[wave][r] = res[r];
+  }
+  __syncthreads();
+  if (tid < R) {
+    float acc = 0.f;
+    for (uint32_t k = 0; k < p.top_k; ++k) acc += red[k][tid];  // ascending k, as the combine kernel adds
+    p.out[(uint64_t)t * p.N + n0 + tid] = __float2half(acc);
+  }
+}
+
 // LDS bytes per activation row: image and per-lane sums over whole chunks
 template <int BITS>
 size_t lds_per_row(uint32_t K) {
@@ -962,6 +1074,49 @@ int32_t launch_qmv_m1_gate_up(const QmvArgs& a, uint32_t bits, const uint32_t* i
       case 64: launch_gate_up<8, 64>(p, assignments, stream); break;
       default: launch_gate_up<8, 128>(p, assignments, stream); break;
     }
+  }
+  RMLX_HIP_CHECK(hipGetLastError());
+  return RMLX_OK;
+}
+
+// Chunks of K the down + combine kernel keeps in registers (0: the shape is not for it)
+// (8-bit weights only: with 4-bit rows a wave's share is too small to pay -- hidden 4096 / intermediate 1536, 4 tokens at
+// top-8: the block 64.7 us with four rows per wave, 70.0 us with eight, against 59.7 us with the wave-per-tile kernel)
+static int down_combine_chunks(uint32_t N, uint32_t K, uint32_t group_size, uint32_t bits, uint32_t top_k) {
+  if (bits != 8 || (group_size != 32 && group_size != 64 && group_size != 128)) return 0;
+  const uint32_t chunk_k = 8192 / bits;
+  if (N == 0 || K == 0 || N % 4 != 0 || K % (128 / bits) != 0 || K % group_size != 0 || top_k < 1 || top_k > 8) return 0;
+  return K <= chunk_k ? 1 : (K <= 2 * chunk_k ? 2 : 0);
+}
+
+bool qmv_m1_down_combine_supported(uint32_t N, uint32_t K, uint32_t group_size, uint32_t bits, uint32_t top_k) {
+  return down_combine_chunks(N, K, group_size, bits, top_k) != 0;
+}
+
+namespace {
+template <int BITS, int GS>
+void launch_down_combine(const M1DownParams& p, int chunks, uint32_t T, hipStream_t stream) {
+  // (four rows per wave: the weights of a pass fit the registers of two workgroups per CU)
+  if (chunks == 1) hipLaunchKernelGGL((qmv_m1_down_combine_kernel<BITS, GS, 1, 4>), dim3(p.N / 4, T), dim3(kThreads), 0, stream, p);
+  else hipLaunchKernelGGL((qmv_m1_down_combine_kernel<BITS, GS, 2, 4>), dim3(p.N / 4, T), dim3(kThreads), 0, stream, p);
+}
+}  // namespace
+
+int32_t launch_qmv_m1_down_combine(const uint32_t* w, const __half* s, const __half* b, uint64_t estride_w, uint64_t estride_s,
+                                   uint32_t n_experts, const __half* h, const uint32_t* idx, const float* wts, uint32_t T,
+                                   uint32_t top_k, uint32_t N, uint32_t K, uint32_t group_size, uint32_t bits, __half* out,
+                                   hipStream_t stream) {
+  const int chunks = down_combine_chunks(N, K, group_size, bits, top_k);
+  if (chunks == 0)
+    return fail(RMLX_INVALID_SHAPE, "qmv_m1 down + combine: unsupported shape N=%u K=%u bits=%u group_size=%u top_k=%u", N, K, bits,
+                group_size, top_k);
+  if (T == 0) return RMLX_OK;
+  if (T > 65535) return fail(RMLX_INVALID_SHAPE, "qmv_m1 down + combine: at most 65535 tokens per launch (T=%u)", T);
+  M1DownParams p{w, s, b, estride_w, estride_s, h, idx, wts, out, N, K, top_k, n_experts};
+  switch (group_size) {
+    case 32: launch_down_combine<8, 32>(p, chunks, T, stream); break;
+    case 64: launch_down_combine<8, 64>(p, chunks, T, stream); break;
+    default: launch_down_combine<8, 128>(p, chunks, T, stream); break;
   }
   RMLX_HIP_CHECK(hipGetLastError());
   return RMLX_OK;

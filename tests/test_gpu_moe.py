@@ -454,11 +454,12 @@ def test_moe_forward_of_a_few_tokens(hip, T, K, E, D, I, fused):
 
 
 @pytest.mark.parametrize("bits,gs", [(8, 64), (8, 32), (8, 128), (4, 32), (4, 128)])
-@pytest.mark.parametrize("T,K,E,D,I", [(1, 8, 16, 1024, 512), (3, 4, 32, 512, 1024)])
+@pytest.mark.parametrize("T,K,E,D,I", [(1, 8, 16, 1024, 512), (3, 4, 32, 512, 1024), (2, 8, 16, 512, 1536), (2, 3, 8, 512, 2560)])
 def test_moe_forward_of_a_few_tokens_other_formats(hip, bits, gs, T, K, E, D, I):
-    """The form without grouping for 8-bit experts and for group sizes 32 / 128: gate / up on the single-row kernel, the down
-    projection as a single-row gather and the weighted sum of a token's rows in a launch of its own.  Against the oracle,
-    with logits and with the caller's picks, and through ExpertGroup with one row per item."""
+    """The form without grouping for 8-bit experts and for group sizes 32 / 128: gate / up on the single-row kernel; the down
+    projection of 8-bit experts with the combine behind it on the single-row layout (intermediate dimension up to one / two
+    wave-wide chunks: 512, 1024 / 1536), else as a single-row gather and the weighted sum of a token's rows in a launch of
+    its own.  Against the oracle, with logits and with the caller's picks, and through ExpertGroup with one row per item."""
     from rmlx_amd import ops
     from rmlx_amd.runtime import DeviceBuffer
     rng = np.random.default_rng(bits * 1000 + gs + T)
