@@ -466,6 +466,8 @@ struct ExpertShapes {
 constexpr uint32_t kGatherGemmMinRows = 9;
 // routed block: the form without grouping (every assignment a row of its own) is never taken beyond this many assignments
 constexpr uint32_t kDirectMaxAssignments = 128;
+// (2-bit experts have no grouped fast path: streaming an expert per assignment stays far ahead of the portable kernels)
+constexpr uint32_t kQ2UngroupedMaxAssignments = 8192;
 // The form without grouping streams an expert once per assignment instead of once per distinct expert of the batch (at
 // about 6 against 5 TB/s, and without the grouping launch): worth it while the assignments are at most 1.3 x the distinct
 // experts a uniform router picks, E (1 - (1 - K/E)^T).  Measured at E = 128, top-8: 9 tokens 127 against 137 us, 10 tokens
@@ -1489,6 +1491,43 @@ int32_t moe_grouped_impl(const rmlx_qweight* gate, const rmlx_qweight* up, const
       RMLX_TRY(launch_moe_combine_rows_f16(static_cast<const __half*>(y.ptr), picks, pick_weights, T32, (uint32_t)top_k, sh.D, sh.E,
                                            static_cast<__half*>(out_f16_dev), s));
     }
+    return finish(s);
+  }
+  // 2-bit experts: the form without grouping on the 2-bit single-row kernel with a weight matrix per row -- routing,
+  // gate / up, SwiGLU, down, weighted sum, every expert streamed once per assignment in whole rows (the portable kernels
+  // below are the alternative).
+  if (sh.portable && !gemm && gate->bits == 2 && down->bits == 2 && (up == nullptr || (up->bits == 2 && up->group_size == gate->group_size)) &&
+      A <= kQ2UngroupedMaxAssignments && qmv_q2_supported(sh.I, sh.D, gate->group_size) &&
+      qmv_q2_supported(sh.D, sh.I, down->group_size) && aligned16(xk) && aligned16(gate->w) && aligned16(down->w) &&
+      (up == nullptr || aligned16(up->w)) && (!sh.fused || ((size_t)sh.I * (sh.D / 16) * 4) % 16 == 0)) {
+    if (route != nullptr)
+      RMLX_TRY(launch_topk_route(route->logits, route->bias, T32, sh.E, (uint32_t)top_k, 1, route->idx_out, route->w_out,
+                                 nullptr, nullptr, s));
+    Scratch gu, y16;
+    const uint32_t gs = gate->group_size;
+    const size_t rows_per_expert = sh.fused ? 2 * (size_t)sh.I : sh.I;
+    const uint64_t gw = rows_per_expert * (sh.D / 16), gsb = rows_per_expert * (sh.D / gs);
+    RMLX_TRY(gu.alloc((size_t)A * 2 * sh.I * 2, s));
+    RMLX_TRY(h.alloc((size_t)A * sh.I * 2, s));
+    __half* g_out = static_cast<__half*>(gu.ptr);
+    if (sh.fused) {  // one stacked matrix: [A, 2I] = (gate | up)
+      RMLX_TRY(launch_qmv_q2_gather(gate->w, gate->s, gate->b, gw, gsb, sh.E, xk, (uint32_t)top_k, expert_indices_dev, A, g_out,
+                                    2 * sh.I, sh.D, gs, s));
+      RMLX_TRY(launch_silu_gate_strided(g_out, g_out + sh.I, 2 * sh.I, static_cast<__half*>(h.ptr), A, sh.I, s));
+    } else {
+      __half* u_out = g_out + (size_t)A * sh.I;
+      RMLX_TRY(launch_qmv_q2_gather(gate->w, gate->s, gate->b, gw, gsb, sh.E, xk, (uint32_t)top_k, expert_indices_dev, A, g_out, sh.I,
+                                    sh.D, gs, s));
+      RMLX_TRY(launch_qmv_q2_gather(up->w, up->s, up->b, gw, gsb, sh.E, xk, (uint32_t)top_k, expert_indices_dev, A, u_out, sh.I, sh.D,
+                                    gs, s));
+      RMLX_TRY(launch_silu_gate(g_out, u_out, static_cast<__half*>(h.ptr), (size_t)A * sh.I, s));
+    }
+    RMLX_TRY(y16.alloc((size_t)A * sh.D * 2, s));
+    RMLX_TRY(launch_qmv_q2_gather(down->w, down->s, down->b, (uint64_t)sh.D * (sh.I / 16), (uint64_t)sh.D * (sh.I / down->group_size),
+                                  sh.E, static_cast<const __half*>(h.ptr), 1, expert_indices_dev, A, static_cast<__half*>(y16.ptr), sh.D,
+                                  sh.I, down->group_size, s));
+    RMLX_TRY(launch_moe_combine_rows_f16(static_cast<const __half*>(y16.ptr), expert_indices_dev, expert_weights_dev, T32,
+                                         (uint32_t)top_k, sh.D, sh.E, static_cast<__half*>(out_f16_dev), s));
     return finish(s);
   }
   if (sh.portable && !gemm) {

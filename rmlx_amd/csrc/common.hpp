@@ -197,6 +197,11 @@ bool qmv_m1_fuses_norm(uint32_t M, uint32_t K, uint32_t bits);
 bool qmv_q2_supported(uint32_t N, uint32_t K, uint32_t group_size);
 int32_t launch_qmv_q2(const uint32_t* w, const __half* s, const __half* b, const __half* x, __half* out, uint32_t M,
                       uint32_t N, uint32_t K, uint32_t group_size, hipStream_t stream);
+// The same with a weight matrix per output row (qmv_q2.hip): row m = activation row m / x_div of x through expert idx[m]
+// of stacked 2-bit weights (outside [0, n_experts): zeros), out [batch, N] f16
+int32_t launch_qmv_q2_gather(const uint32_t* w, const __half* s, const __half* b, uint64_t estride_w, uint64_t estride_s,
+                             uint32_t n_experts, const __half* x, uint32_t x_div, const uint32_t* idx, uint32_t batch, __half* out,
+                             uint32_t N, uint32_t K, uint32_t group_size, hipStream_t stream);
 // dst[m,k] = (half(x[m,k]) * half(inv_rms[m])) * norm_w[k], each product rounded to f16 (the RMSNorm prologue as a separate pass)
 int32_t launch_norm_rows(const void* x, int32_t x_dtype, const __half* norm_w, const float* inv_rms, uint32_t M,
                          uint32_t K, __half* dst, hipStream_t s);

@@ -34,6 +34,11 @@ struct Q2Params {
   const __half* x;
   __half* out;
   uint32_t N, K, M;
+  // a weight matrix per output row m (null: one matrix): expert gather_idx[m] of stacked weights (strides in u32 words /
+  // halves; an index outside [0, n_experts) writes zeros), multiplied with activation row m / x_div
+  const uint32_t* gather_idx;
+  uint64_t estride_w, estride_s;
+  uint32_t n_experts, x_div;
 };
 
 __device__ __forceinline__ h2 as_h2(uint32_t v) { return __builtin_bit_cast(h2, v); }
@@ -64,7 +69,8 @@ __host__ __device__ inline size_t q2_lds_bytes(uint32_t K) {
   return chunks * (kChunkK * 2 + 64 * 2 * sizeof(float2));
 }
 
-template <int GS>
+// GATHER: a weight matrix per output row and workgroups that walk several row blocks (see Q2Params and below)
+template <int GS, bool GATHER>
 __global__ __launch_bounds__(kThreads) void qmv_q2_kernel(Q2Params p) {
   extern __shared__ __attribute__((aligned(16))) char lds[];
   const uint32_t K = p.K, KH = (K + kChunkK - 1) / kChunkK, G = K / GS, nunits = K / 8;
@@ -72,10 +78,26 @@ __global__ __launch_bounds__(kThreads) void qmv_q2_kernel(Q2Params p) {
   u4* const img = reinterpret_cast<u4*>(lds);
   float2* const cs = reinterpret_cast<float2*>(lds + (size_t)KH * kChunkK * 2);
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const uint32_t row = blockIdx.x * kWaves + wave, m = blockIdx.y;
+  const uint32_t m = blockIdx.y;
+  // Row blocks (kWaves weight rows) of this workgroup: blockIdx.x, blockIdx.x + gridDim.x, ... -- one per workgroup in the
+  // plain launch; a gather over many rows sizes the grid to what the chip keeps resident, so the activations are staged
+  // once per workgroup and the next block's weights are in flight while the current block is multiplied.
+  const uint32_t nblk = p.N / kWaves;
+  const uint32_t my_blocks = !GATHER ? 1u : (blockIdx.x < nblk ? (nblk - 1 - blockIdx.x) / gridDim.x + 1 : 0u);
+  auto block_row = [&](uint32_t i) { return (blockIdx.x + i * gridDim.x) * kWaves + wave; };
+  uint64_t e_w = 0, e_s = 0;
+  bool zeros = false;
+  uint32_t xrow = m;
+  if constexpr (GATHER) {
+    const uint32_t e = p.gather_idx[m];
+    zeros = e >= p.n_experts;
+    e_w = zeros ? 0 : e * p.estride_w;
+    e_s = zeros ? 0 : e * p.estride_s;
+    xrow = m / p.x_div;
+  }
 
   // ---- 1. loads, the activations first (the memory counter retires in order), then the row's first two chunks --------
-  const u4* xg = reinterpret_cast<const u4*>(p.x + (uint64_t)m * K);
+  const u4* xg = reinterpret_cast<const u4*>(p.x + (uint64_t)xrow * K);
   u4 xv[4];
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
@@ -83,11 +105,17 @@ __global__ __launch_bounds__(kThreads) void qmv_q2_kernel(Q2Params p) {
     xv[i] = (u4){0u, 0u, 0u, 0u};
     if (u < nunits) xv[i] = xg[u];
   }
-  const u4* wrow = reinterpret_cast<const u4*>(p.w + (uint64_t)row * (K / 16));
-  const unsigned short* srow = reinterpret_cast<const unsigned short*>(p.s) + (uint64_t)row * G;
-  const unsigned short* brow = reinterpret_cast<const unsigned short*>(p.b) + (uint64_t)row * G;
   struct Chunk { u4 w; uint32_t s[2], b[2]; };
-  auto load_chunk = [&](uint32_t c, Chunk& t) {
+  // the chunks of all blocks of the workgroup form one sequence (block 0: chunks 0 .. KH - 1, block 1: ...), loaded two
+  // ahead of their use
+  const uint32_t n_items = my_blocks * KH;
+  uint32_t ld_item = 0;
+  auto load_chunk = [&](Chunk& t) {
+    const uint32_t row = block_row(ld_item / KH), c = ld_item % KH;
+    ++ld_item;
+    const u4* wrow = reinterpret_cast<const u4*>(p.w + e_w + (uint64_t)row * (K / 16));
+    const unsigned short* srow = reinterpret_cast<const unsigned short*>(p.s + e_s) + (uint64_t)row * G;
+    const unsigned short* brow = reinterpret_cast<const unsigned short*>(p.b + e_s) + (uint64_t)row * G;
     uint32_t wi = c * 64 + lane;
     wi = wi < row_u4 ? wi : row_u4 - 1;  // lanes past K meet zeros in the image
 #pragma unroll
@@ -100,8 +128,8 @@ __global__ __launch_bounds__(kThreads) void qmv_q2_kernel(Q2Params p) {
     t.w = __builtin_nontemporal_load(wrow + wi);
   };
   Chunk ca, cb;
-  load_chunk(0, ca);
-  if (KH > 1) load_chunk(1, cb);
+  if (n_items > 0) load_chunk(ca);
+  if (n_items > 1) load_chunk(cb);
 
   // ---- 2. stage x: unit u = 8 consecutive k = (chunk, lane, word j, byte half h); the two units of a word sit in
   //         neighbouring threads and exchange their values to build the pair blocks ------------------------------------
@@ -143,7 +171,10 @@ __global__ __launch_bounds__(kThreads) void qmv_q2_kernel(Q2Params p) {
   uint32_t mk[4] = {0x00030003u, 0x000C000Cu, 0x00300030u, 0x00C000C0u};
   uint32_t mg[4] = {0x64006400u, 0x5C005C00u, 0x54005400u, 0x4C004C00u};
   float racc = 0.f;
-  auto dot_chunk = [&](uint32_t c, const Chunk& t) {
+  uint32_t pr_item = 0;
+  auto dot_chunk = [&](const Chunk& t) {
+    const uint32_t c = pr_item % KH;
+    if (c == 0) racc = 0.f;
     const uint32_t wd[4] = {t.w.x, t.w.y, t.w.z, t.w.w};
     const float2 k0 = cs[(c * 64 + lane) * 2], k1 = cs[(c * 64 + lane) * 2 + 1];
     float acc[2] = {0.f, 0.f};
@@ -167,17 +198,20 @@ __global__ __launch_bounds__(kThreads) void qmv_q2_kernel(Q2Params p) {
       const float2 k = hl ? k1 : k0;
       racc += sc * (acc[hl] - k.x) + bi * k.y;
     }
+    if (c == KH - 1) {  // the block's row is complete
+      const float total = wave_sum(racc);
+      if (lane == 0) p.out[(uint64_t)m * p.N + block_row(pr_item / KH)] = __float2half(zeros ? 0.f : total);
+    }
+    ++pr_item;
   };
-  for (uint32_t c = 0; c < KH; c += 2) {
-    dot_chunk(c, ca);
-    if (c + 2 < KH) load_chunk(c + 2, ca);
-    if (c + 1 < KH) {
-      dot_chunk(c + 1, cb);
-      if (c + 3 < KH) load_chunk(c + 3, cb);
+  for (uint32_t i = 0; i < n_items; i += 2) {
+    dot_chunk(ca);
+    if (i + 2 < n_items) load_chunk(ca);
+    if (i + 1 < n_items) {
+      dot_chunk(cb);
+      if (i + 3 < n_items) load_chunk(cb);
     }
   }
-  const float total = wave_sum(racc);
-  if (lane == 0) p.out[(uint64_t)m * p.N + row] = __float2half(total);
 }
 
 }  // namespace
@@ -194,15 +228,42 @@ int32_t launch_qmv_q2(const uint32_t* w, const __half* s, const __half* b, const
     return fail(RMLX_INVALID_SHAPE, "qmv_q2: unsupported shape N=%u K=%u group_size=%u", N, K, group_size);
   if (M == 0) return RMLX_OK;
   if (M > 65535) return fail(RMLX_INVALID_SHAPE, "qmv_q2: at most 65535 rows per launch (M=%u)", M);
-  Q2Params p{w, s, b, x, out, N, K, M};
+  Q2Params p{w, s, b, x, out, N, K, M, nullptr, 0, 0, 0, 1};
   const dim3 grid(N / kWaves, M);
   const size_t lds = q2_lds_bytes(K);
   switch (group_size) {
-    case 32: hipLaunchKernelGGL(qmv_q2_kernel<32>, grid, dim3(kThreads), lds, stream, p); break;
-    case 64: hipLaunchKernelGGL(qmv_q2_kernel<64>, grid, dim3(kThreads), lds, stream, p); break;
-    default: hipLaunchKernelGGL(qmv_q2_kernel<128>, grid, dim3(kThreads), lds, stream, p); break;
+    case 32: hipLaunchKernelGGL((qmv_q2_kernel<32, false>), grid, dim3(kThreads), lds, stream, p); break;
+    case 64: hipLaunchKernelGGL((qmv_q2_kernel<64, false>), grid, dim3(kThreads), lds, stream, p); break;
+    default: hipLaunchKernelGGL((qmv_q2_kernel<128, false>), grid, dim3(kThreads), lds, stream, p); break;
   }
   RMLX_HIP_CHECK(hipGetLastError());
+  return RMLX_OK;
+}
+
+// One activation row per index through stacked 2-bit weights: output row m = activation row m / x_div of x through
+// expert idx[m] (outside [0, n_experts): zeros), out [batch, N] f16; strides in u32 words / halves.
+int32_t launch_qmv_q2_gather(const uint32_t* w, const __half* s, const __half* b, uint64_t estride_w, uint64_t estride_s,
+                             uint32_t n_experts, const __half* x, uint32_t x_div, const uint32_t* idx, uint32_t batch, __half* out,
+                             uint32_t N, uint32_t K, uint32_t group_size, hipStream_t stream) {
+  if (!qmv_q2_supported(N, K, group_size))
+    return fail(RMLX_INVALID_SHAPE, "qmv_q2 gather: unsupported shape N=%u K=%u group_size=%u", N, K, group_size);
+  if (idx == nullptr || x_div == 0) return fail(RMLX_RUNTIME_ERROR, "qmv_q2 gather: needs an expert per row");
+  const size_t lds = q2_lds_bytes(K);
+  for (uint32_t first = 0; first < batch; first += 65535 / x_div * x_div) {  // the row is the second grid dimension
+    const uint32_t step = 65535 / x_div * x_div, rows = batch - first < step ? batch - first : step;
+    Q2Params p{w, s, b, x + (uint64_t)(first / x_div) * K, out + (uint64_t)first * N, N, K, rows, idx + first, estride_w, estride_s,
+               n_experts, x_div};
+    // as many workgroups per row as stay resident together (four per CU by their threads), at most one per row block
+    uint32_t gx = 4u * (uint32_t)ctx().num_cus / rows;
+    gx = gx < 1 ? 1 : (gx > N / kWaves ? N / kWaves : gx);
+    const dim3 grid(gx, rows);
+    switch (group_size) {
+      case 32: hipLaunchKernelGGL((qmv_q2_kernel<32, true>), grid, dim3(kThreads), lds, stream, p); break;
+      case 64: hipLaunchKernelGGL((qmv_q2_kernel<64, true>), grid, dim3(kThreads), lds, stream, p); break;
+      default: hipLaunchKernelGGL((qmv_q2_kernel<128, true>), grid, dim3(kThreads), lds, stream, p); break;
+    }
+    RMLX_HIP_CHECK(hipGetLastError());
+  }
   return RMLX_OK;
 }
 

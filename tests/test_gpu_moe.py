@@ -487,6 +487,39 @@ def test_moe_forward_of_a_few_tokens_other_formats(hip, bits, gs, T, K, E, D, I)
         assert_close(y, one, f"ExpertGroup expert {e}")
 
 
+@pytest.mark.parametrize("gs", [32, 64, 128])
+@pytest.mark.parametrize("T,K,E,D,I,fused", [(1, 8, 16, 1024, 512, True), (3, 4, 32, 512, 1024, False), (2, 2, 8, 4096, 1536, True)])
+def test_moe_forward_of_a_few_tokens_two_bit_experts(hip, gs, T, K, E, D, I, fused):
+    """2-bit experts, a few tokens: the form without grouping on the 2-bit single-row kernel with a weight matrix per row
+    (gate / up, SwiGLU, down, weighted sum).  Against the oracle, with logits and with the caller's picks (one of them out
+    of range), stacked and separate gate / up weights."""
+    from rmlx_amd import ops
+    from rmlx_amd.runtime import DeviceBuffer
+    rng = np.random.default_rng(gs * 10 + T + E)
+    if fused:
+        gu = _two_bit(rng, E, 2 * I, D, gs)
+        gate, up = tuple(a[:, :I] for a in gu), tuple(a[:, I:] for a in gu)
+        gh, uh = ops.QuantizedWeight.from_numpy(*gu, gs, 2), None
+    else:
+        gate, up = _two_bit(rng, E, I, D, gs), _two_bit(rng, E, I, D, gs)
+        gh, uh = ops.QuantizedWeight.from_numpy(*gate, gs, 2), ops.QuantizedWeight.from_numpy(*up, gs, 2)
+    down = _two_bit(rng, E, D, I, gs)
+    dh = ops.QuantizedWeight.from_numpy(*down, gs, 2)
+    x = make_x(rng, T, D)
+    logits = rng.standard_normal((T, E)).astype(np.float32)
+    idx, w, _, _ = model.topk_route(logits, K)
+    ref = model.moe_forward(x, idx, w, gate, up, down, gs, K, bits=2)
+    print(f"few tokens Q2 gs{gs} T={T} K={K} E={E} D={D} I={I} fused={fused}", flush=True)
+    xd = DeviceBuffer.from_numpy(x)
+    assert_close(ops.moe_forward(gh, uh, dh, xd, DeviceBuffer.from_numpy(logits), K).numpy(), ref, "moe_forward")
+    bad = idx.copy().reshape(-1)
+    w_ref = w.copy().reshape(-1)
+    bad[-1] = E + 1
+    w_ref[-1] = 0.0
+    out = ops.moe_forward_grouped(gh, uh, dh, xd, DeviceBuffer.from_numpy(bad.astype(np.uint32)), DeviceBuffer.from_numpy(w.reshape(-1)), K).numpy()
+    assert_close(out, model.moe_forward(x, idx, w_ref.reshape(w.shape), gate, up, down, gs, K, bits=2), "moe_forward_grouped, one pick out of range")
+
+
 @pytest.mark.parametrize("T,K", [(1, 2), (1, 8), (2, 3), (3, 4)])
 def test_moe_forward_grouped_with_repeated_experts(hip, T, K):
     """Caller-supplied picks may name one expert several times for a token; decode-sized batches run kernels
