@@ -466,8 +466,9 @@ struct ExpertShapes {
 constexpr uint32_t kGatherGemmMinRows = 9;
 // routed block: the form without grouping (every assignment a row of its own) is never taken beyond this many assignments
 constexpr uint32_t kDirectMaxAssignments = 128;
-// (2-bit experts have no grouped fast path: streaming an expert per assignment stays far ahead of the portable kernels)
-constexpr uint32_t kQ2UngroupedMaxAssignments = 8192;
+// (experts without a grouped fast path, 2-bit ones among them: streaming an expert per assignment stays far ahead of the
+// portable kernels up to this many assignments)
+constexpr uint32_t kUngroupedOnlyMaxAssignments = 8192;
 // The form without grouping streams an expert once per assignment instead of once per distinct expert of the batch (at
 // about 6 against 5 TB/s, and without the grouping launch): worth it while the assignments are at most 1.3 x the distinct
 // experts a uniform router picks, E (1 - (1 - K/E)^T).  Measured at E = 128, top-8: 9 tokens 127 against 137 us, 10 tokens
@@ -1422,8 +1423,11 @@ int32_t moe_grouped_impl(const rmlx_qweight* gate, const rmlx_qweight* up, const
   // workgroups of the direct form rank their token's experts themselves, so any number of tokens; `small`: at most 8
   // tokens, which the one-workgroup routing + grouping launch takes; everything else routes with the routing kernel and
   // goes on as if the caller had brought the picks.
-  const bool direct = ungrouped_pays(T32, sh.E, (uint32_t)top_k, gate->bits) && sh.stream_kernel != 1 && single_row_experts(gate, up, down, sh) &&
-                      (route == nullptr || sh.E <= 256);
+  // (weights that no grouped fast kernel takes -- dimensions off the multiples of 512 / 256, 8-bit at group size 32 -- stay
+  // on it at every batch size: an expert per assignment on the single-row kernels is far ahead of the portable kernels)
+  const bool only_single_row = sh.portable && !sh.gemm && A <= kUngroupedOnlyMaxAssignments;
+  const bool direct = (ungrouped_pays(T32, sh.E, (uint32_t)top_k, gate->bits) || only_single_row) && sh.stream_kernel != 1 &&
+                      single_row_experts(gate, up, down, sh) && (route == nullptr || sh.E <= 256);
   // (its down projection adds the weighted expert outputs itself where the wave-per-tile kernel takes the weights)
   const bool fused_down = sh.wave_down && qmv_wt_combine_supported(sh.D, sh.I, down->group_size, (uint32_t)top_k);
   const bool small = route != nullptr && T32 <= 8 && route_sort_fusable(T32, sh.E, (uint32_t)top_k);
@@ -1497,7 +1501,7 @@ int32_t moe_grouped_impl(const rmlx_qweight* gate, const rmlx_qweight* up, const
   // gate / up, SwiGLU, down, weighted sum, every expert streamed once per assignment in whole rows (the portable kernels
   // below are the alternative).
   if (sh.portable && !gemm && gate->bits == 2 && down->bits == 2 && (up == nullptr || (up->bits == 2 && up->group_size == gate->group_size)) &&
-      A <= kQ2UngroupedMaxAssignments && qmv_q2_supported(sh.I, sh.D, gate->group_size) &&
+      A <= kUngroupedOnlyMaxAssignments && qmv_q2_supported(sh.I, sh.D, gate->group_size) &&
       qmv_q2_supported(sh.D, sh.I, down->group_size) && aligned16(xk) && aligned16(gate->w) && aligned16(down->w) &&
       (up == nullptr || aligned16(up->w)) && (!sh.fused || ((size_t)sh.I * (sh.D / 16) * 4) % 16 == 0)) {
     if (route != nullptr)

@@ -520,6 +520,31 @@ def test_moe_forward_of_a_few_tokens_two_bit_experts(hip, gs, T, K, E, D, I, fus
     assert_close(out, model.moe_forward(x, idx, w_ref.reshape(w.shape), gate, up, down, gs, K, bits=2), "moe_forward_grouped, one pick out of range")
 
 
+@pytest.mark.parametrize("bits,gs,D,I", [(4, 32, 1056, 800), (4, 64, 2880, 2880), (8, 32, 512, 1024), (8, 64, 1088, 576)])
+@pytest.mark.parametrize("T", [3, 40])
+def test_moe_forward_of_shapes_without_a_grouped_kernel(hip, bits, gs, D, I, T):
+    """Expert dimensions off the multiples of 512 / 256 (e.g. a hidden size of 2880) and 8-bit weights at group size 32:
+    no chunked or grouped fast kernel takes them, the single-row kernels do (K % 32 == 0, N % 8 == 0), so the form without
+    grouping runs them at every batch size.  Against the oracle, with logits and with the caller's picks."""
+    from rmlx_amd import ops
+    from rmlx_amd.runtime import DeviceBuffer
+    rng = np.random.default_rng(bits + gs + D + T)
+    E, K = 6, 2
+    gu = make_weight(rng, 2 * I, D, bits, gs, lead=(E,))
+    down = make_weight(rng, D, I, bits, gs, lead=(E,))
+    gate, up = tuple(a[:, :I] for a in gu), tuple(a[:, I:] for a in gu)
+    gh, dh = ops.QuantizedWeight.from_numpy(*gu, gs, bits), ops.QuantizedWeight.from_numpy(*down, gs, bits)
+    x = make_x(rng, T, D)
+    logits = rng.standard_normal((T, E)).astype(np.float32)
+    idx, w, _, _ = model.topk_route(logits, K)
+    ref = model.moe_forward(x, idx, w, gate, up, down, gs, K, bits=bits)
+    print(f"no grouped kernel Q{bits} gs{gs} D={D} I={I} T={T}", flush=True)
+    xd = DeviceBuffer.from_numpy(x)
+    assert_close(ops.moe_forward(gh, None, dh, xd, DeviceBuffer.from_numpy(logits), K).numpy(), ref, "moe_forward")
+    out = ops.moe_forward_grouped(gh, None, dh, xd, DeviceBuffer.from_numpy(idx), DeviceBuffer.from_numpy(w), K).numpy()
+    assert_close(out, ref, "moe_forward_grouped")
+
+
 @pytest.mark.parametrize("T,K", [(1, 2), (1, 8), (2, 3), (3, 4)])
 def test_moe_forward_grouped_with_repeated_experts(hip, T, K):
     """Caller-supplied picks may name one expert several times for a token; decode-sized batches run kernels
