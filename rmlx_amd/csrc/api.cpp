@@ -203,17 +203,19 @@ int32_t run_matmul_plain(const rmlx_qweight* qw, const void* x, int32_t x_dtype,
   const bool ptr_ok = aligned16(qw->w) && aligned16(qw->s) && aligned16(qw->b) && aligned16(x);
   const bool can_qmv = ptr_ok && ((qw->bits == 4 && qmv_q4_supported(N, K, qw->group_size)) ||
                                   (qw->bits == 8 && qmv_q8_supported(N, K, qw->group_size)));
-  // where the multi-row GEMV cannot take the shape (group size, K not a multiple of 512), the single-row
-  // kernel also runs small batches, in passes of four rows
-  const bool can_m1 = ptr_ok && qmv_m1_supported(N, K, qw->group_size, qw->bits) &&
-                      M <= (can_qmv ? kM1MaxRows : kM1MaxRowsOther);
-  // 2-bit weights: the single-row kernel of their own, up to 16 rows in passes of one (the alternative is the portable kernel)
-  const bool can_q2 = ptr_ok && qw->bits == 2 && M <= kM1MaxRowsOther && qmv_q2_supported(N, K, qw->group_size);
-  // 4-bit weights at group size 32: the wave-per-tile kernel streams the weights once per 8 rows
-  const bool can_wt32 = ptr_ok && qw->bits == 4 && qw->group_size == 32 && qmv_wt_supported(N, K, 32, 8);
   const bool can_qmm_lds = ptr_ok && qmm_supported(N, K, qw->group_size, qw->bits);
   const bool can_qmm_rw = ptr_ok && qmm_rw_supported(N, K, qw->group_size, qw->bits);
   const bool can_qmm = can_qmm_lds || can_qmm_rw;
+  // where the multi-row GEMV cannot take the shape (group size, K not a multiple of 512), the single-row
+  // kernel also runs small batches, in passes of four rows -- and every batch where no GEMM takes the shape either (K not
+  // a multiple of 256, e.g. a hidden size of 2880 or 896): after the first pass the weights come from L2 / Infinity Cache,
+  // about 4 us per four rows at 4096 x 2880 against 40 us on the portable kernel
+  const uint32_t m1_rows_other = can_qmm ? kM1MaxRowsOther : 65535u;
+  const bool can_m1 = ptr_ok && qmv_m1_supported(N, K, qw->group_size, qw->bits) && M <= (can_qmv ? kM1MaxRows : m1_rows_other);
+  // 2-bit weights: the single-row kernel of their own in passes of one row (the alternative is the portable kernel)
+  const bool can_q2 = ptr_ok && qw->bits == 2 && M <= 65535u && qmv_q2_supported(N, K, qw->group_size);
+  // 4-bit weights at group size 32: the wave-per-tile kernel streams the weights once per 8 rows
+  const bool can_wt32 = ptr_ok && qw->bits == 4 && qw->group_size == 32 && qmv_wt_supported(N, K, 32, 8);
   // (its stores and the reads of the fused epilogue operand are 8- / 16-byte vectors)
   const bool can_qmm_k2 = ptr_ok && aligned16(out) && (epi.ptr == nullptr || aligned16(epi.ptr)) &&
                           qmm_k2_supported(N, K, qw->group_size, qw->bits);

@@ -920,6 +920,19 @@ def test_single_row_gemv_long_k(hip, bits, n, k):
         assert_close(_run(hip, words, s, b, x, bits), ref, f"bits={bits} N={n} K={k} M={m}")
 
 
+@pytest.mark.parametrize("bits,n,k", [(4, 512, 2880), (8, 256, 896), (4, 384, 1152)])
+@pytest.mark.parametrize("m", [17, 70, 300])
+def test_batches_on_shapes_without_a_gemm(hip, bits, n, k, m):
+    """K off the multiples of 256 (hidden sizes such as 2880, 896, 1152), where no MFMA GEMM takes the shape: batches
+    beyond 16 rows run on the single-row kernels in passes (the weights come from cache after the first) instead of the
+    portable kernel.  Against the oracle."""
+    rng = np.random.default_rng(bits + n + k + m)
+    words, s, b = make_weight(rng, n, k, bits, 64)
+    x = make_x(rng, m, k)
+    ref = model.qmm(x.astype(np.float64), words, s, b, 64, bits)
+    assert_close(_run(hip, words, s, b, x, bits), ref, f"Q{bits} M={m} N={n} K={k}")
+
+
 def test_random_shapes_through_the_ladder(hip):
     """Sixty seeded random (M, N, K, bits, group size) shapes through the automatic dispatch: whatever kernel
     the ladder picks (single-row, multi-row GEMV, both GEMMs, portable) must land on the oracle."""
