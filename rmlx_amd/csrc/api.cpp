@@ -208,8 +208,8 @@ int32_t run_matmul_plain(const rmlx_qweight* qw, const void* x, int32_t x_dtype,
   const bool can_qmm = can_qmm_lds || can_qmm_rw;
   // where the multi-row GEMV cannot take the shape (group size, K not a multiple of 512), the single-row
   // kernel also runs small batches, in passes of four rows -- and every batch where no GEMM takes the shape either (K not
-  // a multiple of 256, e.g. a hidden size of 2880 or 896): after the first pass the weights come from L2 / Infinity Cache,
-  // about 4 us per four rows at 4096 x 2880 against 40 us on the portable kernel
+  // a multiple of 256 at group sizes 32 and 128, K not a multiple of 64): after the first pass the weights come from
+  // L2 / Infinity Cache, about 4 us per four rows at 4096 x 2880 against 40 us on the portable kernel
   const uint32_t m1_rows_other = can_qmm ? kM1MaxRowsOther : 65535u;
   const bool can_m1 = ptr_ok && qmv_m1_supported(N, K, qw->group_size, qw->bits) && M <= (can_qmv ? kM1MaxRows : m1_rows_other);
   // 2-bit weights: the single-row kernel of their own in passes of one row (the alternative is the portable kernel)
@@ -248,7 +248,11 @@ int32_t run_matmul_plain(const rmlx_qweight* qw, const void* x, int32_t x_dtype,
     // 8-bit: 7.4 / 11.4, 12.6 / 11.4, 19.8 / 11.7; N = 9216, 8-bit: 14.2 / 20.6, 23.0 / 20.6, 36.8 / 21.2).  Over very
     // wide matrices the wave-per-tile kernel has enough tiles to fill the chip and takes 3 to 8 rows (N = 28672, 4-bit,
     // group 32: 22.8 us against 26.9 on the single-row kernel and 25.1 on the GEMM; N = 16384: 21.4 against 17.6 on the GEMM).
-    const bool m1_first = can_m1 && (can_qmv || !can_qmm_rw || M <= kM1PassRows);
+    // With only the LDS-staged GEMM as the alternative (K a multiple of 64 but not of 256, floor 10 to 23 us) the passes keep
+    // up to 16 rows, except over small matrices, where the third pass already costs more than the GEMM (4-bit, 16 rows:
+    // 4864 x 896 13.2 against 10.6 us, 6912 x 1152 16.9 against 12.3; 4096 x 2880 16.2 against 22.8, 5120 x 2880 19.0 against 22.8).
+    const bool passes_lose = !can_qmv && !can_qmm_rw && can_qmm_lds && M > 8 && wbytes < (5ull << 20);
+    const bool m1_first = can_m1 && !passes_lose && (can_qmv || !can_qmm_rw || M <= kM1PassRows);
     if (can_wt32 && N >= kWt32MinN && M >= 3 && M <= 8) kernel = KERNEL_QMV_ROWS;
     else if ((can_qmv && small_m) || m1_first || can_q2) kernel = KERNEL_QMV;
     else if (can_qmm) kernel = KERNEL_QMM;

@@ -35,6 +35,7 @@ struct QmmParams {
   const uint16_t* x;  // f16 or bf16 bits in fragment-major layout (see relayout_a_kernel)
   __half* out;
   uint32_t M, N, K;
+  uint32_t Kx;  // columns of the fragment-major activations: K rounded up to whole unrolled iterations, zeros past K
 };
 
 
@@ -85,7 +86,10 @@ __device__ __forceinline__ u2 dequant_q8_word_bf16(uint32_t w, float s, float b)
   return o;
 }
 
-template <int BM, int BN, int BITS, bool XBF16>
+// TAIL: K is a multiple of 64 but not of 256.  The loop runs over the activations' padded width; the steps past K multiply
+// zero activations by the weights of the last real step (weight, scale and bias loads are clamped to the row), and scales
+// and biases are fetched as single halves (a row of them starts on a 2-byte boundary only when K / 64 is odd).
+template <int BM, int BN, int BITS, bool XBF16, bool TAIL>
 __global__ __launch_bounds__(kThreads) void qmm_kernel(QmmParams p) {
   constexpr int WM = BM / 4;                   // rows per wave: the 4 waves are stacked along M
   constexpr int TI = WM / 16, TJ = BN / 16;    // 16x16 MFMA tiles per wave
@@ -113,7 +117,9 @@ __global__ __launch_bounds__(kThreads) void qmm_kernel(QmmParams p) {
   const uint32_t m0 = (id % tiles_m) * BM, n0 = (id / tiles_m) * BN;
 
   const uint32_t K = p.K, gpr = K >> 6;
-  const int steps = K / BK;  // a multiple of kDepth (checked on the host)
+  const uint32_t Kx = TAIL ? p.Kx : K;
+  const int steps = Kx / BK;          // a multiple of kDepth (checked on the host)
+  const int wlast = (int)gpr - 1;     // the last step that has weights
 
   // weight staging coordinates
   const int brow = tid >> 2, bq = tid & 3;  // weight row in tile, 16-value quarter of the 64-k step
@@ -130,7 +136,7 @@ __global__ __launch_bounds__(kThreads) void qmm_kernel(QmmParams p) {
 #pragma unroll
   for (int i = 0; i < TI; ++i) {
     const uint32_t mt = (m0 + wave * WM) / 16 + i;
-    aptr[i] = reinterpret_cast<const u4*>(p.x) + (uint64_t)(mt < mt_last ? mt : mt_last) * (K / 32) * 64 + lane;
+    aptr[i] = reinterpret_cast<const u4*>(p.x) + (uint64_t)(mt < mt_last ? mt : mt_last) * (Kx / 32) * 64 + lane;
   }
 
   // Register ring of kDepth k-steps: global loads run kDepth steps ahead of the MFMAs.  Scales
@@ -147,6 +153,7 @@ __global__ __launch_bounds__(kThreads) void qmm_kernel(QmmParams p) {
         areg[slot][kk][i] = aptr[i][(step * KK + kk) * 64];
   };
   auto load_w = [&](int step, int slot) {
+    if (TAIL) step = step < wlast ? step : wlast;
     if (BITS == 4) {
       const u2 v = *reinterpret_cast<const u2*>(wptr + step * (BK * BITS / 32));
       wreg[slot][0] = v.x; wreg[slot][1] = v.y;
@@ -156,8 +163,20 @@ __global__ __launch_bounds__(kThreads) void qmm_kernel(QmmParams p) {
     }
   };
   auto load_sb = [&](int group0, u2 (&dst)[2]) {
-    dst[0] = *reinterpret_cast<const u2*>(sptr + group0);
-    dst[1] = *reinterpret_cast<const u2*>(bptr + group0);
+    if (TAIL) {
+      uint32_t sv[4], bv[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const int gq = group0 + e < wlast ? group0 + e : wlast;
+        sv[e] = reinterpret_cast<const uint16_t*>(sptr)[gq];
+        bv[e] = reinterpret_cast<const uint16_t*>(bptr)[gq];
+      }
+      dst[0] = (u2){sv[0] | (sv[1] << 16), sv[2] | (sv[3] << 16)};
+      dst[1] = (u2){bv[0] | (bv[1] << 16), bv[2] | (bv[3] << 16)};
+    } else {
+      dst[0] = *reinterpret_cast<const u2*>(sptr + group0);
+      dst[1] = *reinterpret_cast<const u2*>(bptr + group0);
+    }
   };
   auto pick16 = [](const u2& v, int e) -> uint16_t {  // element e (0..3) of four packed halves
     const uint32_t wd = e < 2 ? v.x : v.y;
@@ -285,8 +304,8 @@ __global__ __launch_bounds__(kThreads) void qmm_kernel(QmmParams p) {
 // The dtype cast is fused in.
 __global__ __launch_bounds__(256) void relayout_a_kernel(const void* __restrict__ src, int src_dtype,
                                                          u4* __restrict__ dst, uint32_t M, uint32_t K,
-                                                         int to_bf16) {
-  const uint32_t kchunks = K / 32;
+                                                         uint32_t Kx, int to_bf16) {
+  const uint32_t kchunks = Kx / 32;  // chunks past K hold zeros
   const uint64_t units = (uint64_t)((M + 15) / 16) * kchunks * 64;
   for (uint64_t u = (uint64_t)blockIdx.x * 256 + threadIdx.x; u < units; u += (uint64_t)gridDim.x * 256) {
     const uint32_t lane = (uint32_t)(u & 63);
@@ -296,7 +315,9 @@ __global__ __launch_bounds__(256) void relayout_a_kernel(const void* __restrict_
     if (row >= M) row = M - 1;
     const uint64_t off = (uint64_t)row * K + kc * 32 + (lane >> 4) * 8;
     u4 o;
-    if (src_dtype == RMLX_DTYPE_F32) {
+    if (kc * 32 >= K) {
+      o = (u4){0u, 0u, 0u, 0u};
+    } else if (src_dtype == RMLX_DTYPE_F32) {
       const float* f = reinterpret_cast<const float*>(src) + off;
       uint32_t w[4];
 #pragma unroll
@@ -340,32 +361,36 @@ __global__ __launch_bounds__(256) void relayout_a_kernel(const void* __restrict_
 template <int BM, int BITS, bool XBF16>
 void launch_t(const QmmParams& p, hipStream_t s) {
   const uint32_t tiles = ((p.M + BM - 1) / BM) * (p.N / 64);
-  hipLaunchKernelGGL((qmm_kernel<BM, 64, BITS, XBF16>), dim3(tiles), dim3(kThreads), 0, s, p);
+  if (p.Kx != p.K) hipLaunchKernelGGL((qmm_kernel<BM, 64, BITS, XBF16, true>), dim3(tiles), dim3(kThreads), 0, s, p);
+  else hipLaunchKernelGGL((qmm_kernel<BM, 64, BITS, XBF16, false>), dim3(tiles), dim3(kThreads), 0, s, p);
 }
+
+uint32_t padded_k(uint32_t K) { return (K + BK * kDepth - 1) / (BK * kDepth) * (BK * kDepth); }
 
 }  // namespace
 
 
 bool qmm_supported(uint32_t N, uint32_t K, uint32_t group_size, uint32_t bits) {
-  return group_size == 64 && (bits == 4 || bits == 8) && N % 64 == 0 && K % (BK * kDepth) == 0 && N > 0 && K > 0;
+  return group_size == 64 && (bits == 4 || bits == 8) && N % 64 == 0 && K % BK == 0 && N > 0 && K >= BK * kDepth;
 }
 
-size_t qmm_workspace_bytes(uint32_t M, uint32_t K) { return (size_t)((M + 15) / 16) * 16 * K * 2; }
+size_t qmm_workspace_bytes(uint32_t M, uint32_t K) { return (size_t)((M + 15) / 16) * 16 * padded_k(K) * 2; }
 
 int32_t launch_qmm(const QmmArgs& a, hipStream_t s) {
   if (!qmm_supported(a.N, a.K, 64, a.bits))
     return fail(RMLX_INVALID_SHAPE, "qmm: unsupported shape N=%u K=%u bits=%u", a.N, a.K, a.bits);
   if (a.M == 0) return RMLX_OK;
   if (a.workspace == nullptr) return fail(RMLX_RUNTIME_ERROR, "qmm: missing activation workspace");
+  const uint32_t Kx = padded_k(a.K);
   const bool want_bf16 = a.bf16_mfma && a.bits == 8 && a.x_dtype == RMLX_DTYPE_BF16;
   {
-    const uint64_t units = (uint64_t)((a.M + 15) / 16) * (a.K / 32) * 64;
+    const uint64_t units = (uint64_t)((a.M + 15) / 16) * (Kx / 32) * 64;
     uint64_t blocks = (units + 255) / 256;
     if (blocks > 4096) blocks = 4096;
     hipLaunchKernelGGL(relayout_a_kernel, dim3((unsigned)blocks), dim3(256), 0, s, a.x, a.x_dtype,
-                       reinterpret_cast<u4*>(a.workspace), a.M, a.K, want_bf16 ? 1 : 0);
+                       reinterpret_cast<u4*>(a.workspace), a.M, a.K, Kx, want_bf16 ? 1 : 0);
   }
-  QmmParams p{a.w, a.s, a.b, reinterpret_cast<const uint16_t*>(a.workspace), a.out, a.M, a.N, a.K};
+  QmmParams p{a.w, a.s, a.b, reinterpret_cast<const uint16_t*>(a.workspace), a.out, a.M, a.N, a.K, Kx};
   // 128-row tiles only when they still give (most of) the CUs a workgroup
   const uint32_t tiles128 = ((a.M + 127) / 128) * (a.N / 64);
   const bool big = a.M > 64 && tiles128 * 4 >= (uint32_t)ctx().num_cus * 3;

@@ -923,14 +923,39 @@ def test_single_row_gemv_long_k(hip, bits, n, k):
 @pytest.mark.parametrize("bits,n,k", [(4, 512, 2880), (8, 256, 896), (4, 384, 1152)])
 @pytest.mark.parametrize("m", [17, 70, 300])
 def test_batches_on_shapes_without_a_gemm(hip, bits, n, k, m):
-    """K off the multiples of 256 (hidden sizes such as 2880, 896, 1152), where no MFMA GEMM takes the shape: batches
-    beyond 16 rows run on the single-row kernels in passes (the weights come from cache after the first) instead of the
-    portable kernel.  Against the oracle."""
+    """K off the multiples of 256 (hidden sizes such as 2880, 896, 1152): batches beyond 16 rows run on the LDS-staged GEMM
+    with padded activations at group size 64, on the single-row kernels in passes at the other group sizes, instead of
+    the portable kernel.  Against the oracle."""
     rng = np.random.default_rng(bits + n + k + m)
     words, s, b = make_weight(rng, n, k, bits, 64)
     x = make_x(rng, m, k)
     ref = model.qmm(x.astype(np.float64), words, s, b, 64, bits)
     assert_close(_run(hip, words, s, b, x, bits), ref, f"Q{bits} M={m} N={n} K={k}")
+
+
+@pytest.mark.parametrize("bits,dtype", [(4, "f16"), (8, "f16"), (8, "bf16"), (4, "f32")])
+@pytest.mark.parametrize("n,k", [(64, 320), (128, 448), (192, 2880), (64, 1152)])
+def test_staged_gemm_with_k_off_its_unrolled_iteration(hip, bits, dtype, n, k):
+    """The LDS-staged GEMM where K is a multiple of 64 but not of 256 (an odd number of groups per row puts a row's scales
+    on a 2-byte boundary): the activations are padded with zeros to whole iterations, weight and scale loads stop at the
+    row's end.  Scales and biases of the neighbouring rows are large, so a load past the row's end would show.  Against
+    the oracle, at one partial tile, whole tiles and 128-row tiles."""
+    from rmlx_amd import runtime as rt
+    rng = np.random.default_rng(bits * 7 + n + k)
+    words, s, b = make_weight(rng, n, k, bits, 64)
+    for m in (17, 64, 300):
+        x = make_x(rng, m, k, dtype)
+        ref = model.qmm(x_as_f64(x, dtype), words, s, b, 64, bits)
+        for kernel in (rt.KERNEL_QMM_LDS, rt.KERNEL_AUTO) + ((rt.KERNEL_QMM_BF16,) if (bits, dtype) == (8, "bf16") else ()):
+            assert_close(_run(hip, words, s, b, x, bits, dtype=dtype, kernel=kernel), ref,
+                         f"Q{bits} {dtype} M={m} N={n} K={k} kernel={kernel}")
+    # the last row's scales end the buffer: nothing may be read past it (the device allocation ends there too)
+    x = make_x(rng, 33, k, dtype)
+    s2, b2 = s.copy(), b.copy()
+    s2[:, -1] = 0
+    b2[:, -1] = 0
+    ref = model.qmm(x_as_f64(x, dtype), words, s2, b2, 64, bits)
+    assert_close(_run(hip, words, s2, b2, x, bits, dtype=dtype, kernel=rt.KERNEL_QMM_LDS), ref, "last group zeroed")
 
 
 def test_random_shapes_through_the_ladder(hip):
