@@ -347,8 +347,8 @@ int32_t rmlx_hip_moe_forward(const rmlx_qweight* gate, const rmlx_qweight* up,
  * device code (one copy per GPU, held until the process ends; rmlx_hip_init resolves its address), so the call
  * makes no hipMalloc / hipFree and touches no pool.  Limits: batches whose intermediates exceed the workspace
  * (about seq_len * top_k * (4 * hidden + 2 * intermediate + 36) bytes: 53 tokens at top-8, hidden 4096,
- * intermediate 1536) are rejected with InvalidShape before anything is launched; expert weights that only the
- * portable kernels take are rejected with NotFound.  Every call on a GPU uses the same workspace: calls that
+ * intermediate 1536; 2-bit experts: seq_len * top_k * (2 * hidden + 6 * intermediate)) are rejected with InvalidShape;
+ * expert weights that only the portable kernels take are rejected with NotFound.  Every call on a GPU uses the same workspace: calls that
  * overlap on one GPU (two streams, two threads) race; consecutive calls on one stream are ordered. */
 int32_t rmlx_hip_moe_forward_noalloc(const rmlx_qweight* gate, const rmlx_qweight* up,
                                      const rmlx_qweight* down, const rmlx_array* x,

@@ -1461,10 +1461,6 @@ int32_t moe_grouped_impl(const rmlx_qweight* gate, const rmlx_qweight* up, const
     RMLX_TRY(launch_cast_to_f16(x->data, x->dtype, static_cast<__half*>(cast.ptr), T * sh.D, s));
     xk = static_cast<const __half*>(cast.ptr);
   }
-  if (sh.portable && !gemm && arena != nullptr)
-    return fail(RMLX_NOT_FOUND, "MoeLayer: these expert weights run on the portable kernels, which the entry point "
-                                "without allocations does not cover (4-bit group 64 / 128 or 8-bit group 64, aligned "
-                                "buffers, dimensions in multiples of 512 / 256)");
   // A few tokens: no grouping at all.  Every assignment is one row in assignment order, and the down
   // projection adds the token's weighted expert outputs itself - two launches (gate / up that routes, down + combine)
   // instead of four, no [assignments, D] intermediate.  An expert picked by two tokens is streamed once per
@@ -1517,8 +1513,8 @@ int32_t moe_grouped_impl(const rmlx_qweight* gate, const rmlx_qweight* up, const
     const uint32_t gs = gate->group_size;
     const size_t rows_per_expert = sh.fused ? 2 * (size_t)sh.I : sh.I;
     const uint64_t gw = rows_per_expert * (sh.D / 16), gsb = rows_per_expert * (sh.D / gs);
-    RMLX_TRY(gu.alloc((size_t)A * 2 * sh.I * 2, s));
-    RMLX_TRY(h.alloc((size_t)A * sh.I * 2, s));
+    RMLX_TRY(gu.alloc((size_t)A * 2 * sh.I * 2, s, arena));
+    RMLX_TRY(h.alloc((size_t)A * sh.I * 2, s, arena));
     __half* g_out = static_cast<__half*>(gu.ptr);
     if (sh.fused) {  // one stacked matrix: [A, 2I] = (gate | up)
       RMLX_TRY(launch_qmv_q2_gather(gate->w, gate->s, gate->b, gw, gsb, sh.E, xk, (uint32_t)top_k, expert_indices_dev, A, g_out,
@@ -1532,7 +1528,7 @@ int32_t moe_grouped_impl(const rmlx_qweight* gate, const rmlx_qweight* up, const
                                     gs, s));
       RMLX_TRY(launch_silu_gate(g_out, u_out, static_cast<__half*>(h.ptr), (size_t)A * sh.I, s));
     }
-    RMLX_TRY(y16.alloc((size_t)A * sh.D * 2, s));
+    RMLX_TRY(y16.alloc((size_t)A * sh.D * 2, s, arena));
     RMLX_TRY(launch_qmv_q2_gather(down->w, down->s, down->b, (uint64_t)sh.D * (sh.I / 16), (uint64_t)sh.D * (sh.I / down->group_size),
                                   sh.E, static_cast<const __half*>(h.ptr), 1, expert_indices_dev, A, static_cast<__half*>(y16.ptr), sh.D,
                                   sh.I, down->group_size, s));
@@ -1540,6 +1536,10 @@ int32_t moe_grouped_impl(const rmlx_qweight* gate, const rmlx_qweight* up, const
                                          (uint32_t)top_k, sh.D, sh.E, static_cast<__half*>(out_f16_dev), s));
     return finish(s);
   }
+  if (sh.portable && !gemm && arena != nullptr)
+    return fail(RMLX_NOT_FOUND, "MoeLayer: these expert weights run on the portable kernels, which the entry point "
+                                "without allocations does not cover (2-, 4- or 8-bit weights, group size 32, 64 or 128, "
+                                "16-byte aligned buffers, whole 16-byte pieces of a row per lane)");
   if (sh.portable && !gemm) {
     // Assignments stay in their own order: position a holds token a / top_k and expert idx[a].
     if (route != nullptr)

@@ -103,11 +103,22 @@ def test_noalloc_limits(hip):
         else:
             with pytest.raises(ops.KernelError, match="static workspace holds 8388608"):
                 ops.moe_forward(gh, None, dh, xd, ld, K, out=out, noalloc=True)
-    # weights that only the portable kernels take (group size 32 below the grouped-GEMM threshold)
-    gu = make_weight(rng, 2 * 64, 64, 4, 32, lead=(4,))
-    dn = make_weight(rng, 64, 64, 4, 32, lead=(4,))
-    g32, d32 = ops.QuantizedWeight.from_numpy(*gu, 32, 4), ops.QuantizedWeight.from_numpy(*dn, 32, 4)
-    xd = DeviceBuffer.from_numpy(make_x(rng, 2, 64))
+    # expert formats with no grouped kernel run an expert per assignment on the single-row kernels, workspace included:
+    # 4-bit at group size 32 below the grouped GEMM's dimensions, and 2-bit experts
+    for bits, gs, d, i in ((4, 32, 64, 64), (2, 64, 128, 64)):
+        gu = make_weight(rng, 2 * i, d, bits, gs, lead=(4,))
+        dn = make_weight(rng, d, i, bits, gs, lead=(4,))
+        gq, dq = ops.QuantizedWeight.from_numpy(*gu, gs, bits), ops.QuantizedWeight.from_numpy(*dn, gs, bits)
+        xd = DeviceBuffer.from_numpy(make_x(rng, 3, d))
+        ld = DeviceBuffer.from_numpy(rng.standard_normal((3, 4)).astype(np.float32))
+        print(f"noalloc ungrouped-only experts bits={bits} gs={gs}", flush=True)
+        got = ops.moe_forward(gq, None, dq, xd, ld, 2, out=DeviceBuffer((3, d), F16), noalloc=True).numpy()
+        assert np.array_equal(got.view(np.uint16), ops.moe_forward(gq, None, dq, xd, ld, 2).numpy().view(np.uint16))
+    # weights that only the portable kernels take (2-bit rows that are no whole 16-byte pieces)
+    gu = make_weight(rng, 2 * 96, 96, 2, 32, lead=(4,))
+    dn = make_weight(rng, 96, 96, 2, 32, lead=(4,))
+    gp, dp = ops.QuantizedWeight.from_numpy(*gu, 32, 2), ops.QuantizedWeight.from_numpy(*dn, 32, 2)
+    xd = DeviceBuffer.from_numpy(make_x(rng, 2, 96))
     ld = DeviceBuffer.from_numpy(rng.standard_normal((2, 4)).astype(np.float32))
     with pytest.raises(ops.KernelError, match="portable kernels"):
-        ops.moe_forward(g32, None, d32, xd, ld, 2, out=DeviceBuffer((2, 64), F16), noalloc=True)
+        ops.moe_forward(gp, None, dp, xd, ld, 2, out=DeviceBuffer((2, 96), F16), noalloc=True)
