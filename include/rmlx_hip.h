@@ -154,11 +154,11 @@ int32_t rmlx_hip_affine_quantized_matmul_batched(const rmlx_qweight* qw, const r
  * single-row kernel where it applies -- M <= 2, or M <= 16 at group size 32, of which the automatic choice keeps M <= 4
  * where the MFMA GEMM takes the shape -- else the multi-row one),
  * 2 = MFMA GEMM (qmm, f16 MFMA; bf16 activations are converted, which is exact for
- * normal-range values; the register-weights kernel when K % 512 == 0, else the LDS-staged one),
+ * normal-range values; the register-weights kernel when K % 512 == 0, else the LDS-staged one: K % 64 == 0),
  * 3 = portable scalar kernel (any bits/group size the type admits),
  * 4 = LDS-staged MFMA GEMM on the bf16 matrix instruction (Q8 weights and bf16 activations
  * only; weights are rounded to bf16, so its error is about four times that of kernel 2),
- * 5 = LDS-staged MFMA GEMM (f16 MFMA, K % 64 == 0, K >= 256),
+ * 5 = LDS-staged MFMA GEMM (f16 MFMA, every group size, K % 64 == 0, K >= 256),
  * 6 = multi-row streaming GEMV also for a single row (group sizes 64 and 128; 4-bit weights at group size 32 with
  * K % 512 == 0 and K <= 4096 on the wave-per-tile form, which the automatic choice takes for 3 to 8 rows over matrices
  * of 24576 rows or more),

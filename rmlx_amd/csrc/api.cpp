@@ -265,15 +265,15 @@ int32_t run_matmul_plain(const rmlx_qweight* qw, const void* x, int32_t x_dtype,
                 N, K, qw->bits, qw->group_size);
   } else if (kernel == KERNEL_QMM && !can_qmm) {
     return fail(RMLX_INVALID_SHAPE,
-                "qmm kernel requires bits in {4,8}, N %% 64 == 0, 16-byte aligned buffers and K %% 512 == 0 (group sizes "
-                "32/64/128) or K %% 256 == 0 (group size 64) (N=%u K=%u bits=%u group_size=%u)", N, K, qw->bits, qw->group_size);
+                "qmm kernel requires bits in {4,8}, N %% 64 == 0, 16-byte aligned buffers, K %% 64 == 0 and K >= 256 "
+                "(N=%u K=%u bits=%u group_size=%u)", N, K, qw->bits, qw->group_size);
   } else if (kernel == KERNEL_QMM_LDS && !can_qmm_lds) {
     return fail(RMLX_INVALID_SHAPE,
-                "the LDS-staged qmm kernel requires bits in {4,8}, group_size=64, N %% 64 == 0, K %% 256 == 0 and "
+                "the LDS-staged qmm kernel requires bits in {4,8}, N %% 64 == 0, K %% 64 == 0, K >= 256 and "
                 "16-byte aligned buffers (N=%u K=%u bits=%u group_size=%u)", N, K, qw->bits, qw->group_size);
-  } else if (kernel == KERNEL_QMM_BF16 && !(can_qmm_lds && qw->bits == 8 && x_dtype == RMLX_DTYPE_BF16)) {
-    return fail(RMLX_INVALID_SHAPE, "the bf16 MFMA GEMM takes Bfloat16 activations and 8-bit weights (got %s, bits=%u)",
-                dtype_name(x_dtype), qw->bits);
+  } else if (kernel == KERNEL_QMM_BF16 && !(can_qmm_lds && qw->bits == 8 && qw->group_size == 64 && x_dtype == RMLX_DTYPE_BF16)) {
+    return fail(RMLX_INVALID_SHAPE, "the bf16 MFMA GEMM takes Bfloat16 activations and 8-bit weights at group size 64 (got %s, bits=%u, "
+                "group_size=%u)", dtype_name(x_dtype), qw->bits, qw->group_size);
   } else if (((kernel == KERNEL_QMM_K2 || kernel == KERNEL_QMM_K2_FLAT) && !can_qmm_k2) || (kernel == KERNEL_QMM_RW && !can_qmm_rw)) {
     return fail(RMLX_INVALID_SHAPE,
                 "the register-weights qmm kernels require bits in {4,8}, N %% 64 == 0, K %% 512 == 0 and 16-byte aligned "
@@ -399,6 +399,7 @@ int32_t run_matmul_plain(const rmlx_qweight* qw, const void* x, int32_t x_dtype,
     Scratch ws;
     RMLX_TRY(ws.alloc(qmm_workspace_bytes(M, K), stream));
     QmmArgs a{qw->w, qw->s, qw->b, x, x_dtype, out, M, N, K, qw->bits, ws.ptr, kernel == KERNEL_QMM_BF16 ? 1 : 0};
+    a.group_size = qw->group_size;
     return launch_qmm(a, stream);
   }
 

@@ -224,6 +224,7 @@ struct QmmArgs {
   const void* epi;    // [M,N] f16 or f32
   int32_t epi_dtype;
   const void* w_packed = nullptr;  // K-split GEMMs: the weights in their tile-contiguous order (gemm_layout_bytes), or null
+  uint32_t group_size = 64;        // LDS-staged GEMM (the other GEMMs take it as a launch argument)
 };
 enum { EPI_NONE = 0, EPI_RESIDUAL = 1, EPI_SWIGLU = 2 };
 // out[i] = out[i] + e[i]  /  silu(e[i]) * out[i], in place on f16 out (kernels without a fused epilogue)

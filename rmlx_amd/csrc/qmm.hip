@@ -36,6 +36,7 @@ struct QmmParams {
   __half* out;
   uint32_t M, N, K;
   uint32_t Kx;  // columns of the fragment-major activations: K rounded up to whole unrolled iterations, zeros past K
+  uint32_t group_size;
 };
 
 
@@ -89,8 +90,12 @@ __device__ __forceinline__ u2 dequant_q8_word_bf16(uint32_t w, float s, float b)
 // TAIL: K is a multiple of 64 but not of 256.  The loop runs over the activations' padded width; the steps past K multiply
 // zero activations by the weights of the last real step (weight, scale and bias loads are clamped to the row), and scales
 // and biases are fetched as single halves (a row of them starts on a 2-byte boundary only when K / 64 is odd).
-template <int BM, int BN, int BITS, bool XBF16, bool TAIL>
+// GS: the quantisation group size.  A thread's 16 values of a step lie in one group at every size; at 32 and 128 the
+// (scale, bias) of a step is fetched as single halves like in the TAIL form (group 2 * step + quarter / 2, step / 2).
+template <int BM, int BN, int BITS, bool XBF16, bool TAIL, int GS>
 __global__ __launch_bounds__(kThreads) void qmm_kernel(QmmParams p) {
+  static_assert(GS == 32 || GS == 64 || GS == 128, "group sizes of the format");
+  constexpr bool kHalfLoads = TAIL || GS != 64;
   constexpr int WM = BM / 4;                   // rows per wave: the 4 waves are stacked along M
   constexpr int TI = WM / 16, TJ = BN / 16;    // 16x16 MFMA tiles per wave
   constexpr int KK = BK / 32;                  // MFMA k-substeps per step
@@ -116,10 +121,10 @@ __global__ __launch_bounds__(kThreads) void qmm_kernel(QmmParams p) {
   if (total % 8 == 0) id = (id % 8) * (total / 8) + id / 8;
   const uint32_t m0 = (id % tiles_m) * BM, n0 = (id / tiles_m) * BN;
 
-  const uint32_t K = p.K, gpr = K >> 6;
+  const uint32_t K = p.K, gpr = K / GS;
   const uint32_t Kx = TAIL ? p.Kx : K;
   const int steps = Kx / BK;          // a multiple of kDepth (checked on the host)
-  const int wlast = (int)gpr - 1;     // the last step that has weights
+  const int wlast = (int)(K / BK) - 1;  // the last step that has weights
 
   // weight staging coordinates
   const int brow = tid >> 2, bq = tid & 3;  // weight row in tile, 16-value quarter of the 64-k step
@@ -163,11 +168,12 @@ __global__ __launch_bounds__(kThreads) void qmm_kernel(QmmParams p) {
     }
   };
   auto load_sb = [&](int group0, u2 (&dst)[2]) {
-    if (TAIL) {
+    if (kHalfLoads) {  // group0 is a step index: the groups of this thread's quarter of steps group0 .. group0 + 3
       uint32_t sv[4], bv[4];
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
-        const int gq = group0 + e < wlast ? group0 + e : wlast;
+        const int st = group0 + e < wlast ? group0 + e : wlast;
+        const int gq = GS == 32 ? 2 * st + (bq >> 1) : GS == 128 ? st >> 1 : st;
         sv[e] = reinterpret_cast<const uint16_t*>(sptr)[gq];
         bv[e] = reinterpret_cast<const uint16_t*>(bptr)[gq];
       }
@@ -361,8 +367,17 @@ __global__ __launch_bounds__(256) void relayout_a_kernel(const void* __restrict_
 template <int BM, int BITS, bool XBF16>
 void launch_t(const QmmParams& p, hipStream_t s) {
   const uint32_t tiles = ((p.M + BM - 1) / BM) * (p.N / 64);
-  if (p.Kx != p.K) hipLaunchKernelGGL((qmm_kernel<BM, 64, BITS, XBF16, true>), dim3(tiles), dim3(kThreads), 0, s, p);
-  else hipLaunchKernelGGL((qmm_kernel<BM, 64, BITS, XBF16, false>), dim3(tiles), dim3(kThreads), 0, s, p);
+  const bool tail = p.Kx != p.K;
+  if (!XBF16 && p.group_size == 32) {
+    if (tail) hipLaunchKernelGGL((qmm_kernel<BM, 64, BITS, false, true, 32>), dim3(tiles), dim3(kThreads), 0, s, p);
+    else hipLaunchKernelGGL((qmm_kernel<BM, 64, BITS, false, false, 32>), dim3(tiles), dim3(kThreads), 0, s, p);
+  } else if (!XBF16 && p.group_size == 128) {
+    if (tail) hipLaunchKernelGGL((qmm_kernel<BM, 64, BITS, false, true, 128>), dim3(tiles), dim3(kThreads), 0, s, p);
+    else hipLaunchKernelGGL((qmm_kernel<BM, 64, BITS, false, false, 128>), dim3(tiles), dim3(kThreads), 0, s, p);
+  } else {
+    if (tail) hipLaunchKernelGGL((qmm_kernel<BM, 64, BITS, XBF16, true, 64>), dim3(tiles), dim3(kThreads), 0, s, p);
+    else hipLaunchKernelGGL((qmm_kernel<BM, 64, BITS, XBF16, false, 64>), dim3(tiles), dim3(kThreads), 0, s, p);
+  }
 }
 
 uint32_t padded_k(uint32_t K) { return (K + BK * kDepth - 1) / (BK * kDepth) * (BK * kDepth); }
@@ -371,14 +386,16 @@ uint32_t padded_k(uint32_t K) { return (K + BK * kDepth - 1) / (BK * kDepth) * (
 
 
 bool qmm_supported(uint32_t N, uint32_t K, uint32_t group_size, uint32_t bits) {
-  return group_size == 64 && (bits == 4 || bits == 8) && N % 64 == 0 && K % BK == 0 && N > 0 && K >= BK * kDepth;
+  return (group_size == 32 || group_size == 64 || group_size == 128) && (bits == 4 || bits == 8) && N % 64 == 0 && K % BK == 0 &&
+         K % group_size == 0 && N > 0 && K >= BK * kDepth;
 }
 
 size_t qmm_workspace_bytes(uint32_t M, uint32_t K) { return (size_t)((M + 15) / 16) * 16 * padded_k(K) * 2; }
 
 int32_t launch_qmm(const QmmArgs& a, hipStream_t s) {
-  if (!qmm_supported(a.N, a.K, 64, a.bits))
-    return fail(RMLX_INVALID_SHAPE, "qmm: unsupported shape N=%u K=%u bits=%u", a.N, a.K, a.bits);
+  if (!qmm_supported(a.N, a.K, a.group_size, a.bits))
+    return fail(RMLX_INVALID_SHAPE, "qmm: unsupported shape N=%u K=%u bits=%u group_size=%u", a.N, a.K, a.bits, a.group_size);
+  if (a.bf16_mfma && a.group_size != 64) return fail(RMLX_INVALID_SHAPE, "qmm: the bf16 MFMA form takes group size 64");
   if (a.M == 0) return RMLX_OK;
   if (a.workspace == nullptr) return fail(RMLX_RUNTIME_ERROR, "qmm: missing activation workspace");
   const uint32_t Kx = padded_k(a.K);
@@ -390,7 +407,7 @@ int32_t launch_qmm(const QmmArgs& a, hipStream_t s) {
     hipLaunchKernelGGL(relayout_a_kernel, dim3((unsigned)blocks), dim3(256), 0, s, a.x, a.x_dtype,
                        reinterpret_cast<u4*>(a.workspace), a.M, a.K, Kx, want_bf16 ? 1 : 0);
   }
-  QmmParams p{a.w, a.s, a.b, reinterpret_cast<const uint16_t*>(a.workspace), a.out, a.M, a.N, a.K, Kx};
+  QmmParams p{a.w, a.s, a.b, reinterpret_cast<const uint16_t*>(a.workspace), a.out, a.M, a.N, a.K, Kx, a.group_size};
   // 128-row tiles only when they still give (most of) the CUs a workgroup
   const uint32_t tiles128 = ((a.M + 127) / 128) * (a.N / 64);
   const bool big = a.M > 64 && tiles128 * 4 >= (uint32_t)ctx().num_cus * 3;

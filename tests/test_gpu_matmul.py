@@ -958,6 +958,31 @@ def test_staged_gemm_with_k_off_its_unrolled_iteration(hip, bits, dtype, n, k):
     assert_close(_run(hip, words, s2, b2, x, bits, dtype=dtype, kernel=rt.KERNEL_QMM_LDS), ref, "last group zeroed")
 
 
+@pytest.mark.parametrize("bits", [4, 8])
+@pytest.mark.parametrize("gs", [32, 128])
+@pytest.mark.parametrize("n,k", [(64, 256), (128, 384), (64, 768), (192, 2944), (64, 1280)])
+def test_staged_gemm_at_group_sizes_32_and_128(hip, bits, gs, n, k):
+    """The LDS-staged GEMM at the other group sizes (two groups per 64-wide step, or one group per two steps), with K on
+    and off whole unrolled iterations: what K not a multiple of 512 runs on at these group sizes.  Every group gets its
+    own scale and bias magnitude, so a wrong group index shows.  Against the oracle."""
+    from rmlx_amd import runtime as rt
+    if k % gs:
+        pytest.skip("K is not a multiple of the group size")
+    rng = np.random.default_rng(bits * 11 + gs + n + k)
+    words, s, b = make_weight(rng, n, k, bits, gs)
+    ramp = (1.0 + np.arange(k // gs) % 7).astype(np.float16)
+    s = (s * ramp).astype(np.float16)
+    b = (b * ramp[::-1]).astype(np.float16)
+    for m, dtype in ((17, "f16"), (70, "bf16"), (300, "f32")):
+        x = make_x(rng, m, k, dtype)
+        ref = model.qmm(x_as_f64(x, dtype), words, s, b, gs, bits)
+        for kernel in (rt.KERNEL_QMM_LDS, rt.KERNEL_AUTO):
+            assert_close(_run(hip, words, s, b, x, bits, gs=gs, dtype=dtype, kernel=kernel), ref,
+                         f"Q{bits} gs={gs} {dtype} M={m} N={n} K={k} kernel={kernel}")
+    with pytest.raises(Exception, match="group size 64"):
+        _run(hip, words, s, b, make_x(rng, 32, k, "bf16"), bits, gs=gs, dtype="bf16", kernel=rt.KERNEL_QMM_BF16)
+
+
 def test_random_shapes_through_the_ladder(hip):
     """Sixty seeded random (M, N, K, bits, group size) shapes through the automatic dispatch: whatever kernel
     the ladder picks (single-row, multi-row GEMV, both GEMMs, portable) must land on the oracle."""
