@@ -201,7 +201,9 @@ int32_t run_matmul_plain(const rmlx_qweight* qw, const void* x, int32_t x_dtype,
   RMLX_TRY(checked_u32(qw->in_features, "in_features", &K));
   if (M == 0) return RMLX_OK;
   const bool ptr_ok = aligned16(qw->w) && aligned16(qw->s) && aligned16(qw->b) && aligned16(x);
-  const bool can_qmv = ptr_ok && ((qw->bits == 4 && qmv_q4_supported(N, K, qw->group_size)) ||
+  // (the dense ladder keeps the reference's K % 512 rule for the 4-bit multi-row GEMV, quantized.rs:1603-1608; the kernel
+  // itself takes whole slabs of 128, which the expert projections use)
+  const bool can_qmv = ptr_ok && ((qw->bits == 4 && K % 512 == 0 && qmv_q4_supported(N, K, qw->group_size)) ||
                                   (qw->bits == 8 && qmv_q8_supported(N, K, qw->group_size)));
   const bool can_qmm_lds = ptr_ok && qmm_supported(N, K, qw->group_size, qw->bits);
   const bool can_qmm_rw = ptr_ok && qmm_rw_supported(N, K, qw->group_size, qw->bits);
@@ -547,6 +549,8 @@ uint32_t expert_gemm_tile_rows(const ExpertShapes& sh, uint64_t rows, uint64_t g
   // 8-bit experts cross over at an eighth of the threshold, rounded down (measured: from one row per expert on, against
   // 10 for 4-bit ones: with 16-row tiles the GEMM streams 8-bit weights faster than the 8-bit GEMV does)
   if (sh.bits == 8 && min_rows != 0) min_rows = min_rows >= 16 ? min_rows / 8 : 1;
+  // experts that no streaming kernel takes: the alternative streams an expert once per assignment, the GEMM once
+  if (sh.portable && min_rows != 0) min_rows = 1;
   if (!sh.gemm || min_rows == 0 || groups == 0 || rows < (uint64_t)min_rows * groups) return 0;
   if (rows <= 7 * groups && sh.gemm64) return 16u;  // (four-wave workgroups, 16 rows: built for group size 64)
   return rows <= 24 * groups ? 32u : kGroupedTileRows;
@@ -1430,21 +1434,23 @@ int32_t moe_grouped_impl(const rmlx_qweight* gate, const rmlx_qweight* up, const
   // workgroups of the direct form rank their token's experts themselves, so any number of tokens; `small`: at most 8
   // tokens, which the one-workgroup routing + grouping launch takes; everything else routes with the routing kernel and
   // goes on as if the caller had brought the picks.
-  // (weights that no grouped fast kernel takes -- dimensions off the multiples of 512 / 256, 8-bit at group size 32 -- stay
-  // on it at every batch size: an expert per assignment on the single-row kernels is far ahead of the portable kernels)
-  const bool only_single_row = sh.portable && !sh.gemm && A <= kUngroupedOnlyMaxAssignments;
+  // (weights that no streaming kernel takes -- dimensions off the multiples of 128, group size 32 with long or odd rows --
+  // stay on it until the grouped GEMM takes the batch, at every batch size where that does not take the shape either: an
+  // expert per assignment on the single-row kernels is far ahead of the portable kernels)
+  const uint32_t gemm_rows = expert_gemm_tile_rows(sh, A, sh.E);  // (0: the batch is below the grouped GEMM's threshold)
+  const bool only_single_row = sh.portable && gemm_rows == 0 && A <= kUngroupedOnlyMaxAssignments;
   const bool direct = (ungrouped_pays(T32, sh.E, (uint32_t)top_k, gate->bits) || only_single_row) && sh.stream_kernel != 1 &&
                       single_row_experts(gate, up, down, sh) && (route == nullptr || sh.E <= 256);
   // (its down projection adds the weighted expert outputs itself where the wave-per-tile kernel takes the weights)
   const bool fused_down = sh.wave_down && qmv_wt_combine_supported(sh.D, sh.I, down->group_size, (uint32_t)top_k);
-  const bool small = route != nullptr && T32 <= 8 && route_sort_fusable(T32, sh.E, (uint32_t)top_k);
+  const bool small = route != nullptr && !sh.portable && T32 <= 8 && route_sort_fusable(T32, sh.E, (uint32_t)top_k);
   if (route != nullptr && !direct && !small) {
     RMLX_TRY(launch_topk_route(route->logits, route->bias, T32, sh.E, (uint32_t)top_k, 1, route->idx_out, route->w_out, nullptr,
                                nullptr, s));
     route = nullptr;
   }
   // many rows per expert: the grouped GEMM over row tiles instead of the streaming GEMV over chunks of 8 rows
-  const uint32_t gemm = route == nullptr ? expert_gemm_tile_rows(sh, A, sh.E) : 0u;
+  const uint32_t gemm = route == nullptr ? gemm_rows : 0u;
   StreamPlan plan = expert_stream_plan(sh, A, sh.E);
   if (route != nullptr && plan.chunk_rows != 8) {  // (the fused routing + grouping launch writes chunks of 8 rows)
     plan.chunk_rows = 8;
@@ -1482,7 +1488,8 @@ int32_t moe_grouped_impl(const rmlx_qweight* gate, const rmlx_qweight* up, const
     const float* pick_weights = route != nullptr ? route->w_out : expert_weights_dev;
     RMLX_TRY(launch_qmv_m1_gate_up(a, gate->bits, route != nullptr ? nullptr : picks, A, (uint32_t)top_k, sh.E, s));
     const uint64_t down_stride_w = (uint64_t)sh.D * (sh.I * down->bits / 32), down_stride_s = (uint64_t)sh.D * (sh.I / down->group_size);
-    if (qmv_m1_down_combine_supported(sh.D, sh.I, down->group_size, down->bits, (uint32_t)top_k)) {
+    // (4-bit: where the wave-per-tile kernel takes the weights its down + combine is ahead, 59.7 against 64.7 us at 4 tokens)
+    if (qmv_m1_down_combine_supported(sh.D, sh.I, down->group_size, down->bits, (uint32_t)top_k) && (down->bits == 8 || !fused_down)) {
       RMLX_TRY(launch_qmv_m1_down_combine(down->w, down->s, down->b, down_stride_w, down_stride_s, sh.E, static_cast<const __half*>(h.ptr),
                                           picks, pick_weights, T32, (uint32_t)top_k, sh.D, sh.I, down->group_size, down->bits,
                                           static_cast<__half*>(out_f16_dev), s));
@@ -1490,8 +1497,8 @@ int32_t moe_grouped_impl(const rmlx_qweight* gate, const rmlx_qweight* up, const
       RMLX_TRY(launch_qmv_wt_combine(down->w, down->s, down->b, down_stride_w, down_stride_s, sh.E, static_cast<const __half*>(h.ptr),
                                      picks, pick_weights, T32, (uint32_t)top_k, sh.D, sh.I, static_cast<__half*>(out_f16_dev), s));
     } else {
-      // other formats (4-bit at group sizes 32 / 128, 8-bit with a long intermediate dimension): the down projection as a
-      // single-row gather, then the weighted sum of a token's rows -- three launches
+      // a long intermediate dimension (beyond 4096 at 4 bits, 2048 at 8): the down projection as a single-row gather, then
+      // the weighted sum of a token's rows -- three launches
       RMLX_TRY(y.alloc((size_t)A * sh.D * 2, s, arena));
       RMLX_TRY(launch_qmv_m1_gather(down->w, down->s, down->b, down_stride_w, down_stride_s, sh.E, static_cast<const __half*>(h.ptr),
                                     picks, A, static_cast<__half*>(y.ptr), sh.D, sh.I, down->group_size, down->bits, s));

@@ -105,9 +105,13 @@ __device__ __forceinline__ h8 dequant_q8_pair(uint32_t w0, uint32_t w1, h2 s2, h
 // expert and its rows from the tile table (rows of different experts never share a tile); workgroups past
 // the table's length leave at once.  MODE 2: grouped gate/up pair -- fragment 0 of a wave multiplies gate
 // rows, fragment 1 the same rows of the up weight (NF == 2), and the store writes silu(gate) * up.
-template <int MF, int NF, int BITS, int NW, bool XBF16, int GS, int MODE>
+// TAIL (group sizes 32 and 64): K is a multiple of 128 but not of 512.  The last unrolled round of the loop then holds iterations past
+// K: their activation chunks are written to LDS as zeros, weight loads repeat the last block, and the scales and biases
+// of a round are fetched word by word with the index clamped to the row (a 16-byte load would run past the row's end).
+template <int MF, int NF, int BITS, int NW, bool XBF16, int GS, int MODE, bool TAIL = false>
 __device__ __forceinline__ void qmm_rw_body(const RwParams p) {  // by value: a reference makes every store a possible change of p
   static_assert(MODE != 2 || NF == 2, "a gate/up pair takes two weight fragments per wave");
+  static_assert(!TAIL || (GS != 128 && MODE != 0), "the tail form is built for grouped launches at group sizes 32 and 64");
   constexpr int kSbWords = 4 * (kBlockK / GS) / 2;  // 32-bit words of scales of one row and four iterations: 8 / 4 / 2
   constexpr int kSbVecs = (kSbWords + 3) / 4;       // 16-byte registers holding them
   constexpr int kThreads = 64 * NW;
@@ -256,7 +260,22 @@ __device__ __forceinline__ void qmm_rw_body(const RwParams p) {  // by value: a 
   auto load_sb = [&](uint32_t blk, u4 (&ds)[NF][kSbVecs], u4 (&db)[NF][kSbVecs]) {
 #pragma unroll
     for (int f = 0; f < NF; ++f) {
-      if (GS == 128) {  // 4 groups = 8 bytes per row and four iterations
+      if (TAIL) {  // words of a round in row order (2 or 4 groups per iteration: 1 or 2 words); the row ends after iteration S - 1
+        constexpr uint32_t kWordsPerIt = kBlockK / GS / 2;
+        const uint32_t last_word = S * kWordsPerIt - 1;
+#pragma unroll
+        for (int v = 0; v < kSbVecs; ++v) {
+          uint32_t sw[4], bw[4];
+#pragma unroll
+          for (int c = 0; c < 4; ++c) {
+            const uint32_t want = (blk * kSbVecs + v) * 4 + c, wi = want < last_word ? want : last_word;
+            sw[c] = reinterpret_cast<const uint32_t*>(sptr[f])[wi];
+            bw[c] = reinterpret_cast<const uint32_t*>(bptr[f])[wi];
+          }
+          ds[f][v] = (u4){sw[0], sw[1], sw[2], sw[3]};
+          db[f][v] = (u4){bw[0], bw[1], bw[2], bw[3]};
+        }
+      } else if (GS == 128) {  // 4 groups = 8 bytes per row and four iterations
         const u2 sv = reinterpret_cast<const u2*>(sptr[f])[blk], bv = reinterpret_cast<const u2*>(bptr[f])[blk];
         ds[f][0] = (u4){sv.x, sv.y, 0u, 0u};
         db[f][0] = (u4){bv.x, bv.y, 0u, 0u};
@@ -277,7 +296,7 @@ __device__ __forceinline__ void qmm_rw_body(const RwParams p) {  // by value: a 
         dst[f][h] = wptr[f][(uint64_t)it * (4 * WL) + h * 4];
       }
   };
-  const uint32_t last = S - 1, last_blk = S / kUnroll - 1;
+  const uint32_t last = S - 1, last_blk = (S + kUnroll - 1) / kUnroll - 1;
   auto clampi = [&](uint32_t it) { return it < last ? it : last; };
 
   // Constants of the unpacking kept in registers so that and+or is one instruction.
@@ -375,7 +394,11 @@ __device__ __forceinline__ void qmm_rw_body(const RwParams p) {  // by value: a 
         // global loads of chunk it+4 into the same registers in the second half, weights last
 #pragma unroll
         for (int q = 0; q < AL; ++q) {
-          if (s == q * NS / (2 * AL)) a_stage_write[lds_w[q]] = to_slot_order(ra[u % 2][q]);
+          if (s == q * NS / (2 * AL)) {
+            u4 av = to_slot_order(ra[u % 2][q]);
+            if (TAIL && it + 2 >= S) av = (u4){0u, 0u, 0u, 0u};  // (a chunk past K: these iterations add nothing)
+            a_stage_write[lds_w[q]] = av;
+          }
           if (s == NS / 2 + q * NS / (2 * AL)) {
             ra[u % 2][q] = *reinterpret_cast<const u4*>(xsrc[q] + (uint64_t)clampi(it + 4) * kBlockK);
           }
@@ -458,9 +481,9 @@ __global__ __launch_bounds__(64 * NW) void qmm_rw_kernel(RwParams p) {
 }
 
 // DUAL: gate/up pair with the SwiGLU store (see MODE 2 above)
-template <int MF, int NF, int BITS, int NW, bool DUAL, int GS = 64>
+template <int MF, int NF, int BITS, int NW, bool DUAL, int GS = 64, bool TAIL = false>
 __global__ __launch_bounds__(64 * NW) void qmm_rw_grouped_kernel(RwParams p) {
-  qmm_rw_body<MF, NF, BITS, NW, false, GS, DUAL ? 2 : 1>(p);
+  qmm_rw_body<MF, NF, BITS, NW, false, GS, DUAL ? 2 : 1, TAIL>(p);
 }
 
 // out[m, c..c+3] = epilogue(sum over the ksplit partial sums, in split order); one thread per four columns
@@ -597,8 +620,9 @@ int32_t launch_qmm_rw(const QmmArgs& a, uint32_t group_size, hipStream_t s) {
 }
 
 bool qmm_rw_grouped_supported(uint32_t N, uint32_t K, uint32_t group_size, uint32_t bits) {
+  // (group sizes 32 and 64 also take K in whole 128-wide blocks, at least two: the tail form)
   return (group_size == 32 || group_size == 64 || group_size == 128) && (bits == 4 || bits == 8) && N > 0 && K > 0 &&
-         N % 128 == 0 && K % (kBlockK * kUnroll) == 0;
+         N % 128 == 0 && (K % (kBlockK * kUnroll) == 0 || (group_size != 128 && K % kBlockK == 0 && K >= 2 * kBlockK));
 }
 
 int32_t launch_qmm_rw_grouped(const GroupedQmmArgs& a, hipStream_t s) {
@@ -627,10 +651,13 @@ int32_t launch_qmm_rw_grouped(const GroupedQmmArgs& a, hipStream_t s) {
   if (a.tile_rows != 16 && a.tile_rows != 32 && a.tile_rows != kGroupedTileRows)
     return fail(RMLX_RUNTIME_ERROR, "grouped qmm: row tiles of %u rows", a.tile_rows);
   const dim3 grid(p.tiles_m * p.tiles_n), block(64 * nw);
-#define RWG_LAUNCH(MFV, NWV, BITSV, GSV)                                                                              \
-  if (dual) hipLaunchKernelGGL((qmm_rw_grouped_kernel<MFV, 2, BITSV, NWV, true, GSV>), grid, block, 0, s, p);          \
-  else if (wide) hipLaunchKernelGGL((qmm_rw_grouped_kernel<MFV, 2, BITSV, NWV, false, GSV>), grid, block, 0, s, p);    \
-  else hipLaunchKernelGGL((qmm_rw_grouped_kernel<MFV, 1, BITSV, NWV, false, GSV>), grid, block, 0, s, p);
+  const bool tail = a.K % (kBlockK * kUnroll) != 0;
+#define RWG_FORMS(MFV, NWV, BITSV, GSV, TAILV)                                                                              \
+  if (dual) hipLaunchKernelGGL((qmm_rw_grouped_kernel<MFV, 2, BITSV, NWV, true, GSV, TAILV>), grid, block, 0, s, p);          \
+  else if (wide) hipLaunchKernelGGL((qmm_rw_grouped_kernel<MFV, 2, BITSV, NWV, false, GSV, TAILV>), grid, block, 0, s, p);    \
+  else hipLaunchKernelGGL((qmm_rw_grouped_kernel<MFV, 1, BITSV, NWV, false, GSV, TAILV>), grid, block, 0, s, p);
+#define RWG_LAUNCH(MFV, NWV, BITSV, GSV)                                         \
+  if (GSV != 128 && tail) { RWG_FORMS(MFV, NWV, BITSV, (GSV == 128 ? 64 : GSV), true) } else { RWG_FORMS(MFV, NWV, BITSV, GSV, false) }
 #define RWG_TILE(BITSV, GSV)                                     \
   if (a.tile_rows == 16) { if (GSV == 64) { RWG_LAUNCH(1, 4, BITSV, 64) } }  \
   else if (a.tile_rows == 32) { RWG_LAUNCH(2, 8, BITSV, GSV) } else { RWG_LAUNCH(4, 8, BITSV, GSV) }
@@ -640,6 +667,7 @@ int32_t launch_qmm_rw_grouped(const GroupedQmmArgs& a, hipStream_t s) {
 #undef RWG_BITS
 #undef RWG_TILE
 #undef RWG_LAUNCH
+#undef RWG_FORMS
   RMLX_HIP_CHECK(hipGetLastError());
   return RMLX_OK;
 }

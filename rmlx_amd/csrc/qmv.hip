@@ -540,12 +540,13 @@ int32_t launch_build_gather_chunks(const uint32_t* indices, uint32_t batch, uint
 }
 
 
+// K in whole slabs of 128: a wave takes up to four slabs per pass, the last part of a pass may be shorter or empty.
 bool qmv_q4_supported(uint32_t N, uint32_t K, uint32_t group_size) {
-  return (group_size == 64 || group_size == 128) && N % 16 == 0 && K % 512 == 0 && N > 0 && K > 0;
+  return (group_size == 64 || group_size == 128) && N % 16 == 0 && K % 128 == 0 && N > 0 && K > 0;
 }
 
 int32_t launch_qmv_q4(const QmvArgs& a, hipStream_t s) {
-  if (!qmv_q4_supported(a.N, a.K, 64)) return fail(RMLX_INVALID_SHAPE, "qmv_q4: N %% 16 and K %% 512 required (N=%u K=%u)", a.N, a.K);
+  if (!qmv_q4_supported(a.N, a.K, 64)) return fail(RMLX_INVALID_SHAPE, "qmv_q4: N %% 16 and K %% 128 required (N=%u K=%u)", a.N, a.K);
   KParams p{};
   p.w0 = a.w0; p.s0 = a.s0; p.b0 = a.b0;
   p.w1 = a.dual ? a.w1 : a.w0; p.s1 = a.dual ? a.s1 : a.s0; p.b1 = a.dual ? a.b1 : a.b0;

@@ -1083,7 +1083,7 @@ int32_t launch_qmv_m1_gate_up(const QmvArgs& a, uint32_t bits, const uint32_t* i
 // (8-bit weights only: with 4-bit rows a wave's share is too small to pay -- hidden 4096 / intermediate 1536, 4 tokens at
 // top-8: the block 64.7 us with four rows per wave, 70.0 us with eight, against 59.7 us with the wave-per-tile kernel)
 static int down_combine_chunks(uint32_t N, uint32_t K, uint32_t group_size, uint32_t bits, uint32_t top_k) {
-  if (bits != 8 || (group_size != 32 && group_size != 64 && group_size != 128)) return 0;
+  if ((bits != 4 && bits != 8) || (group_size != 32 && group_size != 64 && group_size != 128)) return 0;
   const uint32_t chunk_k = 8192 / bits;
   if (N == 0 || K == 0 || N % 4 != 0 || K % (128 / bits) != 0 || K % group_size != 0 || top_k < 1 || top_k > 8) return 0;
   return K <= chunk_k ? 1 : (K <= 2 * chunk_k ? 2 : 0);
@@ -1113,10 +1113,18 @@ int32_t launch_qmv_m1_down_combine(const uint32_t* w, const __half* s, const __h
   if (T == 0) return RMLX_OK;
   if (T > 65535) return fail(RMLX_INVALID_SHAPE, "qmv_m1 down + combine: at most 65535 tokens per launch (T=%u)", T);
   M1DownParams p{w, s, b, estride_w, estride_s, h, idx, wts, out, N, K, top_k, n_experts};
-  switch (group_size) {
-    case 32: launch_down_combine<8, 32>(p, chunks, T, stream); break;
-    case 64: launch_down_combine<8, 64>(p, chunks, T, stream); break;
-    default: launch_down_combine<8, 128>(p, chunks, T, stream); break;
+  if (bits == 8) {
+    switch (group_size) {
+      case 32: launch_down_combine<8, 32>(p, chunks, T, stream); break;
+      case 64: launch_down_combine<8, 64>(p, chunks, T, stream); break;
+      default: launch_down_combine<8, 128>(p, chunks, T, stream); break;
+    }
+  } else {
+    switch (group_size) {
+      case 32: launch_down_combine<4, 32>(p, chunks, T, stream); break;
+      case 64: launch_down_combine<4, 64>(p, chunks, T, stream); break;
+      default: launch_down_combine<4, 128>(p, chunks, T, stream); break;
+    }
   }
   RMLX_HIP_CHECK(hipGetLastError());
   return RMLX_OK;

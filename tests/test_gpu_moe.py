@@ -545,6 +545,40 @@ def test_moe_forward_of_shapes_without_a_grouped_kernel(hip, bits, gs, D, I, T):
     assert_close(out, ref, "moe_forward_grouped")
 
 
+@pytest.mark.parametrize("bits,gs,D,I", [(4, 64, 512, 384), (4, 64, 1024, 640), (4, 64, 2048, 768), (4, 64, 768, 1408),
+                                         (8, 64, 1024, 640), (4, 32, 1024, 640), (8, 32, 640, 384), (4, 128, 1024, 640)])
+@pytest.mark.parametrize("T", [3, 24, 70, 300])
+def test_moe_forward_of_dimensions_in_whole_blocks_of_128(hip, bits, gs, D, I, T):
+    """Expert dimensions that are multiples of 128 but not of 512 (an intermediate size of 768 or 1408): the K-split
+    streaming GEMV walks whole slabs of 128 with a shorter last part, the grouped GEMM pads its last unrolled round with
+    zero activations (group sizes 32 and 64).  3 tokens run the form without grouping, 24 the streaming chunks (group size
+    32, which has none for these rows: the GEMM), 70 and 300 the grouped GEMM on 32- and 64-row tiles; group size 128 has no
+    tail form and stays on the streaming chunks.  Against the oracle, with logits and with the caller's picks."""
+    from rmlx_amd import ops
+    from rmlx_amd.runtime import DeviceBuffer
+    rng = np.random.default_rng(bits + gs + D + I + T)
+    E, K = 8, 2
+    gu = make_weight(rng, 2 * I, D, bits, gs, lead=(E,))
+    down = make_weight(rng, D, I, bits, gs, lead=(E,))
+    gate, up = tuple(a[:, :I] for a in gu), tuple(a[:, I:] for a in gu)
+    gh, dh = ops.QuantizedWeight.from_numpy(*gu, gs, bits), ops.QuantizedWeight.from_numpy(*down, gs, bits)
+    x = make_x(rng, T, D)
+    logits = rng.standard_normal((T, E)).astype(np.float32)
+    idx, w, _, _ = model.topk_route(logits, K)
+    ref = model.moe_forward(x, idx, w, gate, up, down, gs, K, bits=bits)
+    print(f"blocks of 128 Q{bits} gs={gs} D={D} I={I} T={T}", flush=True)
+    xd = DeviceBuffer.from_numpy(x)
+    assert_close(ops.moe_forward(gh, None, dh, xd, DeviceBuffer.from_numpy(logits), K).numpy(), ref, "moe_forward")
+    out = ops.moe_forward_grouped(gh, None, dh, xd, DeviceBuffer.from_numpy(idx), DeviceBuffer.from_numpy(w), K).numpy()
+    assert_close(out, ref, "moe_forward_grouped")
+    if bits == 4:  # every streaming / tile choice the handle offers
+        for min_rows, kind in ((0, 1), (1, 0)):
+            gh.set_expert_gemm_min_rows(min_rows)
+            gh.set_expert_stream_kernel(kind)
+            out = ops.moe_forward_grouped(gh, None, dh, xd, DeviceBuffer.from_numpy(idx), DeviceBuffer.from_numpy(w), K).numpy()
+            assert_close(out, ref, f"moe_forward_grouped min_rows={min_rows} stream kernel {kind}")
+
+
 @pytest.mark.parametrize("T,K", [(1, 2), (1, 8), (2, 3), (3, 4)])
 def test_moe_forward_grouped_with_repeated_experts(hip, T, K):
     """Caller-supplied picks may name one expert several times for a token; decode-sized batches run kernels
