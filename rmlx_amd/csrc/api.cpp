@@ -201,9 +201,8 @@ int32_t run_matmul_plain(const rmlx_qweight* qw, const void* x, int32_t x_dtype,
   RMLX_TRY(checked_u32(qw->in_features, "in_features", &K));
   if (M == 0) return RMLX_OK;
   const bool ptr_ok = aligned16(qw->w) && aligned16(qw->s) && aligned16(qw->b) && aligned16(x);
-  // (the dense ladder keeps the reference's K % 512 rule for the 4-bit multi-row GEMV, quantized.rs:1603-1608; the kernel
-  // itself takes whole slabs of 128, which the expert projections use)
-  const bool can_qmv = ptr_ok && ((qw->bits == 4 && K % 512 == 0 && qmv_q4_supported(N, K, qw->group_size)) ||
+  // (the 4-bit multi-row GEMV takes K in whole slabs of 128; the reference's kernel needs K % 512 == 0, quantized.rs:1603-1608)
+  const bool can_qmv = ptr_ok && ((qw->bits == 4 && qmv_q4_supported(N, K, qw->group_size)) ||
                                   (qw->bits == 8 && qmv_q8_supported(N, K, qw->group_size)));
   const bool can_qmm_lds = ptr_ok && qmm_supported(N, K, qw->group_size, qw->bits);
   const bool can_qmm_rw = ptr_ok && qmm_rw_supported(N, K, qw->group_size, qw->bits);
@@ -262,7 +261,7 @@ int32_t run_matmul_plain(const rmlx_qweight* qw, const void* x, int32_t x_dtype,
     else kernel = KERNEL_GENERIC;
   } else if ((kernel == KERNEL_QMV && !can_qmv && !can_m1 && !can_q2) || (kernel == KERNEL_QMV_ROWS && !can_qmv && !can_wt32)) {
     return fail(RMLX_INVALID_SHAPE,
-                "qmv kernel requires bits in {4,8}, group_size 64 (4-bit: or 128), N %% 16 == 0, K %% 512 == 0 (4-bit) or "
+                "qmv kernel requires bits in {4,8}, group_size 64 (4-bit: or 128), N %% 16 == 0, K %% 128 == 0 (4-bit) or "
                 "K %% 256 == 0 (8-bit) and 16-byte aligned buffers (N=%u K=%u bits=%u group_size=%u)",
                 N, K, qw->bits, qw->group_size);
   } else if (kernel == KERNEL_QMM && !can_qmm) {
@@ -278,8 +277,8 @@ int32_t run_matmul_plain(const rmlx_qweight* qw, const void* x, int32_t x_dtype,
                 "group_size=%u)", dtype_name(x_dtype), qw->bits, qw->group_size);
   } else if (((kernel == KERNEL_QMM_K2 || kernel == KERNEL_QMM_K2_FLAT) && !can_qmm_k2) || (kernel == KERNEL_QMM_RW && !can_qmm_rw)) {
     return fail(RMLX_INVALID_SHAPE,
-                "the register-weights qmm kernels require bits in {4,8}, N %% 64 == 0, K %% 512 == 0 and 16-byte aligned "
-                "buffers (N=%u K=%u bits=%u group_size=%u)", N, K, qw->bits, qw->group_size);
+                "the register-weights qmm kernels require bits in {4,8}, N %% 64 == 0, K %% 512 == 0 (selector 8 at group size 64: "
+                "K %% 128 == 0, K >= 512) and 16-byte aligned buffers (N=%u K=%u bits=%u group_size=%u)", N, K, qw->bits, qw->group_size);
   } else if (kernel == KERNEL_QMM_K2_TALL && !can_qmm_k2_tall) {
     return fail(RMLX_INVALID_SHAPE,
                 "the 128 x 128 K-split qmm kernel requires bits in {4,8} (8-bit weights at group size 32 / 64: f16 or f32 "

@@ -37,6 +37,8 @@ typedef float f4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u2 __attribute__((ext_vector_type(2)));
 
+struct __attribute__((packed, aligned(4))) U4Tail { uint32_t v[4]; };  // a 16-byte load from a 4-byte aligned address
+
 constexpr int kBlockK = 128;  // k extent of one main-loop iteration
 constexpr int kStages = 4;
 constexpr int kUnroll = 4;   // main-loop unrolling = depth of the weight register ring
@@ -107,11 +109,11 @@ __device__ __forceinline__ h8 dequant_q8_pair(uint32_t w0, uint32_t w1, h2 s2, h
 // rows, fragment 1 the same rows of the up weight (NF == 2), and the store writes silu(gate) * up.
 // TAIL (group sizes 32 and 64): K is a multiple of 128 but not of 512.  The last unrolled round of the loop then holds iterations past
 // K: their activation chunks are written to LDS as zeros, weight loads repeat the last block, and the scales and biases
-// of a round are fetched word by word with the index clamped to the row (a 16-byte load would run past the row's end).
+// of the last round come from a load that ends with the row (group size 32: word by word with the index clamped).
 template <int MF, int NF, int BITS, int NW, bool XBF16, int GS, int MODE, bool TAIL = false>
 __device__ __forceinline__ void qmm_rw_body(const RwParams p) {  // by value: a reference makes every store a possible change of p
   static_assert(MODE != 2 || NF == 2, "a gate/up pair takes two weight fragments per wave");
-  static_assert(!TAIL || (GS != 128 && MODE != 0), "the tail form is built for grouped launches at group sizes 32 and 64");
+  static_assert(!TAIL || GS != 128, "the tail form is built for group sizes 32 and 64");
   constexpr int kSbWords = 4 * (kBlockK / GS) / 2;  // 32-bit words of scales of one row and four iterations: 8 / 4 / 2
   constexpr int kSbVecs = (kSbWords + 3) / 4;       // 16-byte registers holding them
   constexpr int kThreads = 64 * NW;
@@ -260,7 +262,17 @@ __device__ __forceinline__ void qmm_rw_body(const RwParams p) {  // by value: a 
   auto load_sb = [&](uint32_t blk, u4 (&ds)[NF][kSbVecs], u4 (&db)[NF][kSbVecs]) {
 #pragma unroll
     for (int f = 0; f < NF; ++f) {
-      if (TAIL) {  // words of a round in row order (2 or 4 groups per iteration: 1 or 2 words); the row ends after iteration S - 1
+      if (TAIL && GS == 64) {
+        // One word per iteration, S >= 4 words per row.  The 16 bytes of a round that would run past the row's end start
+        // early enough to end with the row (4-byte aligned: enough for the hardware), and the words move down to
+        // their places; what then sits behind the row's last word belongs to iterations past K.
+        // (the move happens late in the round before, see settle_sb: done here it would wait for the load at once)
+        const uint32_t want = blk * 4, wo = want < S - 4 ? want : S - 4;  // (wave-uniform)
+        const U4Tail sv = *reinterpret_cast<const U4Tail*>(reinterpret_cast<const uint32_t*>(sptr[f]) + wo);
+        const U4Tail bv = *reinterpret_cast<const U4Tail*>(reinterpret_cast<const uint32_t*>(bptr[f]) + wo);
+        ds[f][0] = (u4){sv.v[0], sv.v[1], sv.v[2], sv.v[3]};
+        db[f][0] = (u4){bv.v[0], bv.v[1], bv.v[2], bv.v[3]};
+      } else if (TAIL) {  // words of a round in row order (4 groups per iteration: 2 words); the row ends after iteration S - 1
         constexpr uint32_t kWordsPerIt = kBlockK / GS / 2;
         const uint32_t last_word = S * kWordsPerIt - 1;
 #pragma unroll
@@ -286,6 +298,16 @@ __device__ __forceinline__ void qmm_rw_body(const RwParams p) {  // by value: a 
           db[f][v] = reinterpret_cast<const u4*>(bptr[f])[blk * kSbVecs + v];
         }
       }
+    }
+  };
+  // tail form at group size 64: the words of round blk, as loaded by load_sb, move down to their places
+  auto settle_sb = [&](uint32_t blk, u4 (&ds)[NF][kSbVecs], u4 (&db)[NF][kSbVecs]) {
+    const uint32_t want = blk * 4, wo = want < S - 4 ? want : S - 4, d = want - wo;  // (wave-uniform)
+#pragma unroll
+    for (int f = 0; f < NF; ++f) {
+      const u4 sv = ds[f][0], bv = db[f][0];
+      ds[f][0] = (u4){d == 0 ? sv.x : d == 1 ? sv.y : d == 2 ? sv.z : sv.w, d == 0 ? sv.y : d == 1 ? sv.z : sv.w, d == 0 ? sv.z : sv.w, sv.w};
+      db[f][0] = (u4){d == 0 ? bv.x : d == 1 ? bv.y : d == 2 ? bv.z : bv.w, d == 0 ? bv.y : d == 1 ? bv.z : bv.w, d == 0 ? bv.z : bv.w, bv.w};
     }
   };
   auto load_w = [&](uint32_t it, u4 (&dst)[NF][WL]) {
@@ -377,6 +399,9 @@ __device__ __forceinline__ void qmm_rw_body(const RwParams p) {  // by value: a 
 #pragma unroll
     for (int u = 0; u < kUnroll; ++u) {
       const uint32_t it = it0 + u;
+      // (the next round's scales and biases were requested three iterations ago; its first weight operand is unpacked in
+      // this iteration's last step)
+      if (TAIL && GS == 64 && u == kUnroll - 1) settle_sb(blk < last_blk ? blk + 1 : last_blk, s_nxt, b_nxt);
       const u4* a_stage = a_lds + (it % kStages) * kChunk;
       const u4* a_stage_next = a_lds + ((it + 1) % kStages) * kChunk;
       u4* a_stage_write = a_lds + ((it + 2) % kStages) * kChunk;
@@ -475,9 +500,9 @@ __device__ __forceinline__ void qmm_rw_body(const RwParams p) {  // by value: a 
   }
 }
 
-template <int MF, int NF, int BITS, int NW, bool XBF16, int GS>
+template <int MF, int NF, int BITS, int NW, bool XBF16, int GS, bool TAIL>
 __global__ __launch_bounds__(64 * NW) void qmm_rw_kernel(RwParams p) {
-  qmm_rw_body<MF, NF, BITS, NW, XBF16, GS, 0>(p);
+  qmm_rw_body<MF, NF, BITS, NW, XBF16, GS, 0, TAIL>(p);
 }
 
 // DUAL: gate/up pair with the SwiGLU store (see MODE 2 above)
@@ -515,15 +540,22 @@ void launch_rw(RwParams p, bool x_bf16, hipStream_t s) {
   p.tiles_m = (p.M + 16 * MF - 1) / (16 * MF);
   p.tiles_n = p.N / (NW * 16 * NF);
   const dim3 grid(p.tiles_m * p.tiles_n, p.ksplit), block(64 * NW);
-  if (x_bf16) hipLaunchKernelGGL((qmm_rw_kernel<MF, NF, BITS, NW, true, GS>), grid, block, 0, s, p);
-  else hipLaunchKernelGGL((qmm_rw_kernel<MF, NF, BITS, NW, false, GS>), grid, block, 0, s, p);
+  const bool tail = (p.K / kBlockK / p.ksplit) % kUnroll != 0;  // (group size 64 only: checked by qmm_rw_supported)
+  if (GS == 64 && tail) {
+    if (x_bf16) hipLaunchKernelGGL((qmm_rw_kernel<MF, NF, BITS, NW, true, 64, true>), grid, block, 0, s, p);
+    else hipLaunchKernelGGL((qmm_rw_kernel<MF, NF, BITS, NW, false, 64, true>), grid, block, 0, s, p);
+  } else {
+    if (x_bf16) hipLaunchKernelGGL((qmm_rw_kernel<MF, NF, BITS, NW, true, GS, false>), grid, block, 0, s, p);
+    else hipLaunchKernelGGL((qmm_rw_kernel<MF, NF, BITS, NW, false, GS, false>), grid, block, 0, s, p);
+  }
 }
 
 }  // namespace
 
 bool qmm_rw_supported(uint32_t N, uint32_t K, uint32_t group_size, uint32_t bits) {
+  // (group size 64 also takes K in whole 128-wide blocks, at least four: the tail form)
   return (group_size == 32 || group_size == 64 || group_size == 128) && (bits == 4 || bits == 8) && N > 0 && K > 0 && N % 64 == 0 &&
-         K % (kBlockK * kUnroll) == 0;
+         (K % (kBlockK * kUnroll) == 0 || (group_size == 64 && K % kBlockK == 0 && K >= 4 * kBlockK));
 }
 
 
@@ -557,7 +589,9 @@ RwPlan plan_rw(uint32_t M, uint32_t N, uint32_t K, uint32_t group_size) {
   const float waves = (float)(best_wgs * (uint32_t)r.nw), simds = (float)(cus * 4), blocks = (float)(K / kBlockK);
   float best_t = 0.f;
   for (uint32_t ks = 1; ks <= 4; ks *= 2) {
-    if (K % (ks * kBlockK * kUnroll) != 0) continue;
+    // (a split leaves whole unrolled rounds; where K itself has a tail, whole blocks, at least four)
+    const uint32_t nb = K / kBlockK;
+    if (K % (kBlockK * kUnroll) == 0 ? K % (ks * kBlockK * kUnroll) != 0 : (nb % ks != 0 || nb / ks < 4)) continue;
     const float load = waves * (float)ks / simds;
     const float t = blocks / (float)ks * 0.33f * (load > 1.f ? load : 1.f) + (ks > 1 ? 3.f : 0.f);
     if (best_t == 0.f || t < best_t - 0.5f) { best_t = t; r.ksplit = ks; }
@@ -620,9 +654,9 @@ int32_t launch_qmm_rw(const QmmArgs& a, uint32_t group_size, hipStream_t s) {
 }
 
 bool qmm_rw_grouped_supported(uint32_t N, uint32_t K, uint32_t group_size, uint32_t bits) {
-  // (group sizes 32 and 64 also take K in whole 128-wide blocks, at least two: the tail form)
+  // (group sizes 32 and 64 also take K in whole 128-wide blocks, at least four: the tail form)
   return (group_size == 32 || group_size == 64 || group_size == 128) && (bits == 4 || bits == 8) && N > 0 && K > 0 &&
-         N % 128 == 0 && (K % (kBlockK * kUnroll) == 0 || (group_size != 128 && K % kBlockK == 0 && K >= 2 * kBlockK));
+         N % 128 == 0 && (K % (kBlockK * kUnroll) == 0 || (group_size != 128 && K % kBlockK == 0 && K >= 4 * kBlockK));
 }
 
 int32_t launch_qmm_rw_grouped(const GroupedQmmArgs& a, hipStream_t s) {
