@@ -1008,6 +1008,25 @@ def test_gemms_and_multi_row_gemv_with_k_in_whole_blocks_of_128(hip, bits, n, k)
                          f"Q{bits} {dtype} M={m} N={n} K={k} kernel={kernel}")
 
 
+@pytest.mark.parametrize("bits,n,k", [(4, 9728, 896), (4, 16384, 1024), (4, 6144, 2048), (8, 8192, 512), (4, 4864, 896)])
+def test_one_and_two_rows_over_short_rows_of_tall_matrices(hip, bits, n, k):
+    """One or two activation rows over a tall matrix of short rows (an up projection from a hidden size of 896, a
+    vocabulary head): the automatic choice runs the multi-row GEMV there, the single-row kernel elsewhere.  Both against
+    the oracle, and the automatic choice agrees with one of them bit for bit."""
+    from rmlx_amd import runtime as rt
+    rng = np.random.default_rng(bits + n + k)
+    words, s, b = make_weight(rng, n, k, bits, 64)
+    for m in (1, 2):
+        x = make_x(rng, m, k)
+        ref = model.qmm(x.astype(np.float64), words, s, b, 64, bits)
+        auto = _run(hip, words, s, b, x, bits)
+        single = _run(hip, words, s, b, x, bits, kernel=rt.KERNEL_QMV)
+        rows = _run(hip, words, s, b, x, bits, kernel=rt.KERNEL_QMV_ROWS)
+        for got, what in ((auto, "auto"), (single, "single-row"), (rows, "multi-row")):
+            assert_close(got, ref, f"Q{bits} M={m} N={n} K={k} {what}")
+        assert np.array_equal(auto.view(np.uint16), single.view(np.uint16)) or np.array_equal(auto.view(np.uint16), rows.view(np.uint16))
+
+
 def test_random_shapes_through_the_ladder(hip):
     """Sixty seeded random (M, N, K, bits, group size) shapes through the automatic dispatch: whatever kernel
     the ladder picks (single-row, multi-row GEMV, both GEMMs, portable) must land on the oracle."""
