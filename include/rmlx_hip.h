@@ -154,7 +154,8 @@ int32_t rmlx_hip_affine_quantized_matmul_batched(const rmlx_qweight* qw, const r
  * single-row kernel where it applies -- M <= 2, or M <= 16 at group size 32, of which the automatic choice keeps M <= 4
  * where the MFMA GEMM takes the shape -- else the multi-row one),
  * 2 = MFMA GEMM (qmm, f16 MFMA; bf16 activations are converted, which is exact for
- * normal-range values; the register-weights kernel when K % 512 == 0, else the LDS-staged one: K % 64 == 0),
+ * normal-range values; the register-weights kernel when K % 512 == 0 (group size 64: K % 128 == 0, K >= 512), else the
+ * LDS-staged one: K % 64 == 0),
  * 3 = portable scalar kernel (any bits/group size the type admits),
  * 4 = LDS-staged MFMA GEMM on the bf16 matrix instruction (Q8 weights and bf16 activations
  * only; weights are rounded to bf16, so its error is about four times that of kernel 2),
@@ -228,8 +229,9 @@ int32_t rmlx_hip_gather_qmm(const rmlx_array* x, const void* w_packed_dev, size_
 /* The same with the kernel family forced (the reference exposes `gather_qmm` and `gather_qmv_fast_f16_q4`
  * separately, quantized.rs:9404, 10061).  kernel: 0 = auto (one row per entry: the single-row GEMV with a weight
  * matrix per activation row, N % 8 == 0, K % 32 == 0, K <= 28672; streaming GEMV up to 8 rows per entry; grouped MFMA
- * GEMM from 9 rows on where it takes the shape: N % 128 == 0, K % 512 == 0; the portable kernel for every other
- * shape), 1 = streaming GEMV (group size 64 / 128, N % 16 == 0, K % 512 == 0), 2 = grouped MFMA GEMM,
+ * GEMM from 9 rows on where it takes the shape: N % 128 == 0, K % 512 == 0, at group sizes 32 / 64 also K % 128 == 0
+ * from 512 on; the portable kernel for every other shape), 1 = streaming GEMV (group size 64 / 128, N % 16 == 0,
+ * K % 128 == 0), 2 = grouped MFMA GEMM,
  * 3 = portable kernel. */
 int32_t rmlx_hip_gather_qmm_select(const rmlx_array* x, const void* w_packed_dev, size_t w_bytes,
                                    const void* scales_dev, size_t scales_bytes,
