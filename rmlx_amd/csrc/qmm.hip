@@ -167,18 +167,26 @@ __global__ __launch_bounds__(kThreads) void qmm_kernel(QmmParams p) {
       wreg[slot][0] = v.x; wreg[slot][1] = v.y; wreg[slot][WPT - 2] = v.z; wreg[slot][WPT - 1] = v.w;
     }
   };
+  // single halves (kHalfLoads): loaded as they are and packed into the two words only when the round that requested them
+  // ends -- packed at once, every round would wait for its own loads
+  auto load_halves = [&](int step0, uint32_t (&sv)[4], uint32_t (&bv)[4]) {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const int st = step0 + e < wlast ? step0 + e : wlast;
+      const int gq = GS == 32 ? 2 * st + (bq >> 1) : GS == 128 ? st >> 1 : st;
+      sv[e] = reinterpret_cast<const uint16_t*>(sptr)[gq];
+      bv[e] = reinterpret_cast<const uint16_t*>(bptr)[gq];
+    }
+  };
+  auto pack_halves = [&](const uint32_t (&sv)[4], const uint32_t (&bv)[4], u2 (&dst)[2]) {
+    dst[0] = (u2){sv[0] | (sv[1] << 16), sv[2] | (sv[3] << 16)};
+    dst[1] = (u2){bv[0] | (bv[1] << 16), bv[2] | (bv[3] << 16)};
+  };
   auto load_sb = [&](int group0, u2 (&dst)[2]) {
     if (kHalfLoads) {  // group0 is a step index: the groups of this thread's quarter of steps group0 .. group0 + 3
       uint32_t sv[4], bv[4];
-#pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        const int st = group0 + e < wlast ? group0 + e : wlast;
-        const int gq = GS == 32 ? 2 * st + (bq >> 1) : GS == 128 ? st >> 1 : st;
-        sv[e] = reinterpret_cast<const uint16_t*>(sptr)[gq];
-        bv[e] = reinterpret_cast<const uint16_t*>(bptr)[gq];
-      }
-      dst[0] = (u2){sv[0] | (sv[1] << 16), sv[2] | (sv[3] << 16)};
-      dst[1] = (u2){bv[0] | (bv[1] << 16), bv[2] | (bv[3] << 16)};
+      load_halves(group0, sv, bv);
+      pack_halves(sv, bv, dst);
     } else {
       dst[0] = *reinterpret_cast<const u2*>(sptr + group0);
       dst[1] = *reinterpret_cast<const u2*>(bptr + group0);
@@ -244,7 +252,9 @@ __global__ __launch_bounds__(kThreads) void qmm_kernel(QmmParams p) {
   for (int step0 = 0; step0 < steps; step0 += kDepth) {
     // scales / biases of groups step0+8 .. step0+11 (needed two iterations from now)
     u2 sb_nn[2];
-    load_sb(step0 + 8 < steps ? step0 + 8 : 0, sb_nn);
+    uint32_t sv_nn[4], bv_nn[4];
+    if (kHalfLoads) load_halves(step0 + 8 < steps ? step0 + 8 : 0, sv_nn, bv_nn);
+    else load_sb(step0 + 8 < steps ? step0 + 8 : 0, sb_nn);
 #pragma unroll
     for (int d = 0; d < kDepth; ++d) {
       const int step = step0 + d;
@@ -287,6 +297,7 @@ __global__ __launch_bounds__(kThreads) void qmm_kernel(QmmParams p) {
       __syncthreads();
     }
     sb_cur[0] = sb_next[0]; sb_cur[1] = sb_next[1];
+    if (kHalfLoads) pack_halves(sv_nn, bv_nn, sb_nn);
     sb_next[0] = sb_nn[0]; sb_next[1] = sb_nn[1];
   }
 
