@@ -259,16 +259,20 @@ int32_t run_matmul_plain(const rmlx_qweight* qw, const void* x, int32_t x_dtype,
     // over K.  Measured, single-row against multi-row, us: one row, 4-bit: 9728 x 896 5.4 / 4.4, 6912 x 1152 4.6 / 4.2,
     // 13824 x 1152 6.3 / 5.1, 8960 x 1536 5.4 / 5.2, 17920 x 1536 7.1 / 6.5, 16384 x 1024 6.3 / 4.8, 151936 x 896 37.7 / 16.1,
     // 151936 x 1536 39.0 / 25.7 (but 4864 x 896 3.6 / 4.3, 8192 x 1024 4.0 / 4.5, 8192 x 512 4.0 / 4.5, 6144 x 2048 3.9 / 4.7);
-    // two rows: 9728 x 896 6.7 / 4.6, 4864 x 896 5.2 / 4.5, 8192 x 512 6.1 / 4.6, 6144 x 2048 5.3 / 4.8, 16384 x 2048 9.6 / 6.8,
-    // 151936 x 896 58.3 / 15.8 (but 4096 x 1024 3.9 / 4.5, 4096 x 1536 4.0 / 4.1); 8-bit, two rows: 8192 x 512 5.7 / 3.5,
+    // 65536 x 2048 19.8 / 17.7, 151936 x 2048 42.9 / 37.7 (32768 x 2048 a tie);
+    // two rows, where the single-row kernel's second row costs a second set of dot products per weight: 9728 x 896 6.7 / 4.6,
+    // 4864 x 896 5.2 / 4.5, 8192 x 512 6.1 / 4.6, 6144 x 2048 5.3 / 4.8, 16384 x 2048 9.6 / 6.8, 151936 x 896 58.3 / 15.8,
+    // 8192 x 3072 7.6 / 5.5, 8192 x 4096 7.6 / 6.7, 12288 x 4096 10.2 / 8.7, 28672 x 4096 19.6 / 18.1, 8192 x 8192 12.3 / 11.5,
+    // 151936 x 3072 79.1 / 54.2 (but 4096 x 1024 3.9 / 4.5, 4096 x 1536 4.0 / 4.1, 4096 x 8192 6.6 / 8.1, 4096 x 14336 10.7 /
+    // 12.9: up to 4096 weight rows the single-row kernel keeps two); 8-bit, two rows: 8192 x 512 5.7 / 3.5,
     // 8192 x 1024 5.8 / 4.3, 16384 x 1024 7.6 / 6.4 (one row: the single-row kernel keeps up).  A fused epilogue or norm
     // stays with the single-row kernel, which applies it in the same launch.
     const bool plain = epi.kind == EPI_NONE && epi.ptr == nullptr && epi.norm_w == nullptr;
     bool short_rows = false;
     if (plain && can_qmv && can_m1 && M <= 2) {
       const uint64_t mib = 1ull << 20;
-      if (qw->bits == 4 && M == 1) short_rows = K < 2048 && wbytes * 2 >= (K % 512 != 0 ? 7 : 13) * mib;
-      else if (qw->bits == 4) short_rows = K <= 2048 && N > 4096 && wbytes >= 2 * mib;
+      if (qw->bits == 4 && M == 1) short_rows = (K < 2048 && wbytes * 2 >= (K % 512 != 0 ? 7 : 13) * mib) || (K == 2048 && wbytes >= 48 * mib);
+      else if (qw->bits == 4) short_rows = K <= 8192 && N > 4096 && wbytes >= 2 * mib;
       else if (M == 2) short_rows = K <= 1024 && wbytes >= 4 * mib;
     }
     if (short_rows) kernel = KERNEL_QMV_ROWS;
