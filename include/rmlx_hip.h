@@ -328,8 +328,10 @@ int32_t rmlx_hip_qweight_set_gemm_layout(rmlx_qweight* qw, void* dst_dev, size_t
 /* Which streaming kernel runs the expert projections of decode-sized batches (below the grouped GEMM's threshold) of a
  * block whose gate weight is `qw`: 1 = K split over the waves of a workgroup, chunks of 8 rows, 2 = a wave per 16-row
  * weight tile, chunks of 8 rows, 3 = a wave per tile, chunks of 16 rows, 4 = kernel 1 for the gate / up projection and
- * kernel 2 for the down projection (4-bit weights, group size 64; other weights keep kernel 1), 0 = the library's
- * choice (4).  Kernel 3 streams an expert with 9 to 16 rows once instead of twice and is the fastest of the four from 7 rows
+ * kernel 2 for the down projection (4-bit weights, group size 64; other weights keep kernel 1), 5 = as 4 with the gate / up
+ * projection in two launches, the experts split by their row count: up to 8 rows on kernel 1, more on kernel 3, so every
+ * expert is streamed once whatever the largest row count, 0 = the library's choice (4; 5 from 6 rows per expert on
+ * average).  Kernel 3 streams an expert with 9 to 16 rows once instead of twice and is the fastest of the four from 7 rows
  * per expert on average - as long as no expert of the batch has more than 16 rows, so it is for callers whose router bounds
  * that.  Returns the previous value; the tests use it to check that the kernels agree.  (No counterpart in the reference, which has one kernel for this: gather_qmv_fast_f16_q4,
  * crates/rmlx-core/src/ops/quantized.rs:9752-9842.) */

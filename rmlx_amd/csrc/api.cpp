@@ -496,6 +496,11 @@ struct ExpertShapes {
 constexpr uint32_t kGatherGemmMinRows = 9;
 // routed block: the form without grouping (every assignment a row of its own) is never taken beyond this many assignments
 constexpr uint32_t kDirectMaxAssignments = 128;
+// twice the average rows per expert from which the gate / up projection of a decode-sized batch runs in two launches, the
+// experts split by their row count (moe_grouped_impl)
+// (E = 128, top-8, D = 4096, I = 1536, against K-split gate / up over chunks of 8: 88 tokens 322 / 308 us, 96 tokens 319 / 324,
+// 128 tokens 353 / 363, 160 tokens 387 / 402 and 400 on the grouped GEMM, 192 tokens 400 / 397 on the GEMM)
+constexpr uint32_t kSplitMinRows2 = 12;
 // (experts without a grouped fast path, 2-bit ones among them: streaming an expert per assignment stays far ahead of the
 // portable kernels up to this many assignments)
 constexpr uint32_t kUngroupedOnlyMaxAssignments = 8192;
@@ -582,7 +587,8 @@ uint32_t expert_gemm_tile_rows(const ExpertShapes& sh, uint64_t rows, uint64_t g
 // rows (8 or 16).  Selector of the gate handle: 1 = K-split for both, 2 / 3 = wave per tile for both with chunks of 8 / 16
 // rows, 0 (the library's choice) and 4 = K-split for gate / up, wave per tile for a down projection whose rows are shorter
 // than 4096 (measured at D = 4096, I = 1536: the block takes 254 against 269 us at T = 32 and 348 against 368 us at
-// T = 128; over chunks of 8 rows a wave-per-tile gate / up projection is 30 % slower than the K-split one).
+// T = 128; over chunks of 8 rows a wave-per-tile gate / up projection is 30 % slower than the K-split one); 5 = as 4, the gate /
+// up projection in two launches with the experts split by their row count (moe_grouped_impl; the routed block only).
 struct StreamPlan { uint32_t gate_up, down, chunk_rows; };
 // rows / groups: the assignments of the call and the experts (or host-side groups) they spread over
 StreamPlan expert_stream_plan(const ExpertShapes& sh, size_t rows, size_t groups) {
@@ -599,6 +605,10 @@ StreamPlan expert_stream_plan(const ExpertShapes& sh, size_t rows, size_t groups
   else if (sh.wave_down && sh.I < 4096) pl.down = 8;
   return pl;
 }
+
+// Gate / up projection in two launches over two chunk tables (see launch_moe_sort): tab = first table, cap_small entries, then
+// the second, cap_big entries; n[2] = their lengths on the device.
+struct SplitTables { const uint32_t* tab; const uint32_t* n; uint32_t cap_small, cap_big; };
 
 // The same block on the portable kernels, for expert weights the streaming GEMV does not take (2-bit,
 // group size 32, 8-bit at group size 128, dimensions that are no multiples of 512 (4-bit) or 256 / 16
@@ -668,7 +678,8 @@ bool single_row_experts(const rmlx_qweight* gate, const rmlx_qweight* up, const 
 int32_t run_expert_ffn(const rmlx_qweight* gate, const rmlx_qweight* up, const rmlx_qweight* down,
                        const ExpertShapes& sh, const __half* x, const uint32_t* row_map,
                        const uint32_t* chunk_tab, const uint32_t* n_chunks, uint32_t max_chunks, __half* h,
-                       void* y, int y_f32, uint32_t gemm_tile_rows, const StreamPlan& plan, hipStream_t stream) {
+                       void* y, int y_f32, uint32_t gemm_tile_rows, const StreamPlan& plan, hipStream_t stream,
+                       const SplitTables* split = nullptr) {
   const uint32_t per = 32 / gate->bits;  // values per u32 word: 8 (4-bit) or 4 (8-bit)
   if (gemm_tile_rows != 0) {  // the table holds row tiles of that many rows and n_chunks its length
     const uint32_t gs = gate->group_size;  // one group size for the three projections (ExpertShapes::gemm)
@@ -701,7 +712,14 @@ int32_t run_expert_ffn(const rmlx_qweight* gate, const rmlx_qweight* up, const r
   a.row_map = row_map;
   a.chunk_tab = chunk_tab; a.n_chunks_dev = n_chunks; a.max_chunks = max_chunks; a.mr = 8;
   // (the table holds chunks of at most plan.chunk_rows rows)
-  if (plan.gate_up != 0) RMLX_TRY(launch_qmv_wt(a, plan.gate_up, stream));
+  if (split != nullptr) {
+    // experts with up to 8 rows: one chunk each on the K-split kernel; the others in chunks of up to 16 rows on the
+    // wave-per-tile kernel with two activation images, which streams their weights once
+    a.chunk_tab = split->tab; a.n_chunks_dev = split->n; a.max_chunks = split->cap_small;
+    RMLX_TRY(launch_qmv_q4(a, stream));
+    a.chunk_tab = split->tab + 3 * (size_t)split->cap_small; a.n_chunks_dev = split->n + 1; a.max_chunks = split->cap_big;
+    RMLX_TRY(launch_qmv_wt(a, 16, stream));
+  } else if (plan.gate_up != 0) RMLX_TRY(launch_qmv_wt(a, plan.gate_up, stream));
   else RMLX_TRY(gate->bits == 8 ? launch_qmv_q8_tab(a, stream) : launch_qmv_q4(a, stream));
 
   if (y == nullptr) return RMLX_OK;  // (the caller runs the down projection itself)
@@ -1591,23 +1609,33 @@ int32_t moe_grouped_impl(const rmlx_qweight* gate, const rmlx_qweight* up, const
     return finish(s);
   }
   if (!aligned16(xk)) return fail(RMLX_INVALID_SHAPE, "MoeLayer: input must be 16-byte aligned");
-  // meta: sorted[A] | sorted_tok[A] | inv[A] | chunk_tab[3*max_chunks] | n_chunks[1]
-  RMLX_TRY(meta.alloc(((size_t)3 * A + 3 * (size_t)max_chunks + 4) * 4, s, arena));
+  // Gate / up in two launches, the experts split by their row count (see run_expert_ffn): between the batch sizes where
+  // nearly every expert is one chunk of 8 rows and the grouped GEMM's threshold, chunks of 8 stream an expert with 9 to 16
+  // rows twice and chunks of 16 on the wave-per-tile kernel are slower for the others.
+  const bool split = route == nullptr && gemm == 0 && sh.bits == 4 && sh.wave_tiles && plan.gate_up == 0 && plan.chunk_rows == 8 &&
+                     (sh.stream_kernel == 5 || (sh.stream_kernel == 0 && (uint64_t)A * 2 >= (uint64_t)kSplitMinRows2 * sh.E));
+  const uint32_t cap_small = A < sh.E ? A : sh.E, cap_big = A / 8 + 1;
+  const size_t split_words = split ? 3 * ((size_t)cap_small + cap_big) + 4 : 0;
+  // meta: sorted[A] | sorted_tok[A] | inv[A] | chunk_tab[3*max_chunks] | n_chunks[1] (| split tables | their lengths[2])
+  RMLX_TRY(meta.alloc(((size_t)3 * A + 3 * (size_t)max_chunks + 4 + split_words) * 4, s, arena));
   uint32_t* sorted = static_cast<uint32_t*>(meta.ptr);
   uint32_t* sorted_tok = sorted + A;
   uint32_t* inv = sorted_tok + A;
   uint32_t* chunk_tab = inv + A;
   uint32_t* n_chunks = chunk_tab + 3 * (size_t)max_chunks;
+  uint32_t* split_tab = split ? n_chunks + 4 : nullptr;
+  uint32_t* split_n = split ? split_tab + 3 * ((size_t)cap_small + cap_big) : nullptr;
+  const SplitTables split_tabs{split_tab, split_n, cap_small, cap_big};
   if (route != nullptr)
     RMLX_TRY(launch_route_sort_small(route->logits, route->bias, T32, sh.E, (uint32_t)top_k, 1, route->idx_out, route->w_out,
                                      sorted, sorted_tok, inv, chunk_tab, n_chunks, s));
   else
     RMLX_TRY(launch_moe_sort(expert_indices_dev, A, sh.E, (uint32_t)top_k, sorted, sorted_tok, inv, nullptr, nullptr, chunk_tab, n_chunks,
-                             chunk_rows, s));
+                             chunk_rows, s, split_tab, split_n, cap_small));
   RMLX_TRY(h.alloc((size_t)A * sh.I * 2, s, arena));
   RMLX_TRY(y.alloc((size_t)A * sh.D * 4, s, arena));
   RMLX_TRY(run_expert_ffn(gate, up, down, sh, xk, sorted_tok, chunk_tab, n_chunks, max_chunks,
-                          static_cast<__half*>(h.ptr), y.ptr, 1, gemm, plan, s));
+                          static_cast<__half*>(h.ptr), y.ptr, 1, gemm, plan, s, split ? &split_tabs : nullptr));
   RMLX_TRY(launch_moe_combine(static_cast<const float*>(y.ptr), inv, expert_weights_dev, T32, (uint32_t)top_k, sh.D,
                               static_cast<__half*>(out_f16_dev), s));
   return finish(s);
@@ -1655,7 +1683,7 @@ uint32_t rmlx_hip_qweight_set_expert_gemm_min_rows(rmlx_qweight* qw, uint32_t mi
 uint32_t rmlx_hip_qweight_set_expert_stream_kernel(rmlx_qweight* qw, uint32_t kind) {
   if (qw == nullptr) return 0;
   const uint32_t prev = qw->expert_stream_kernel;
-  if (kind <= 4) qw->expert_stream_kernel = kind;
+  if (kind <= 5) qw->expert_stream_kernel = kind;
   return prev;
 }
 
@@ -1730,7 +1758,8 @@ int32_t rmlx_hip_moe_forward_noalloc(const rmlx_qweight* gate, const rmlx_qweigh
     const size_t I = up == nullptr ? gate->out_features / 2 : gate->out_features;
     auto r256 = [](size_t b) { return (b + 255) & ~(size_t)255; };
     const size_t max_chunks = A / 8 + (A < E ? A : E);
-    size_t need = r256(A * 8 + 16) + r256((3 * A + 3 * max_chunks + 4) * 4) + r256(A * I * 2) + r256(A * D * 4);
+    const size_t split_words = 3 * ((A < E ? A : E) + A / 8 + 1) + 4;  // (the two tables of the split gate / up launch)
+    size_t need = r256(A * 8 + 16) + r256((3 * A + 3 * max_chunks + 4 + split_words) * 4) + r256(A * I * 2) + r256(A * D * 4);
     if (x->dtype != RMLX_DTYPE_F16) need += r256(T * D * 2);
     if (gate_logits->dtype == RMLX_DTYPE_F16) need += r256(T * E * 4);
     if (expert_bias != nullptr && expert_bias->dtype == RMLX_DTYPE_F16) need += r256(E * 4);

@@ -286,7 +286,10 @@ int32_t launch_topk_route(const float* logits, const float* bias, uint32_t T, ui
 // sorted_tok (nullable): token of each sorted position, sorted[p] / top_k.
 int32_t launch_moe_sort(const uint32_t* idx, uint32_t n_assign, uint32_t E, uint32_t top_k, uint32_t* sorted,
                         uint32_t* sorted_tok, uint32_t* inv, uint32_t* counts, uint32_t* offsets,
-                        uint32_t* chunk_tab, uint32_t* n_chunks, uint32_t chunk_rows, hipStream_t s);
+                        uint32_t* chunk_tab, uint32_t* n_chunks, uint32_t chunk_rows, hipStream_t s,
+                        // (nullable) a second pair of tables that splits the experts by their row count: up to 8 rows -> one
+                        // chunk in split_tab[0 .. 3 * split_cap), more -> chunks of at most 16 rows behind it; split_n[2]: lengths
+                        uint32_t* split_tab = nullptr, uint32_t* split_n = nullptr, uint32_t split_cap = 0);
 // Decode-sized batches (at most 8 tokens, 64 assignments): routing and grouping in one launch.
 bool route_sort_fusable(uint32_t T, uint32_t E, uint32_t K);
 int32_t launch_route_sort_small(const float* logits, const float* bias, uint32_t T, uint32_t E, uint32_t K,

@@ -72,7 +72,9 @@ __global__ __launch_bounds__(1024) void moe_sort_kernel(const uint32_t* __restri
                                                         uint32_t* __restrict__ inv, uint32_t* __restrict__ counts,
                                                         uint32_t* __restrict__ offsets,
                                                         uint32_t* __restrict__ chunk_tab,
-                                                        uint32_t* __restrict__ n_chunks, uint32_t chunk_rows) {
+                                                        uint32_t* __restrict__ n_chunks, uint32_t chunk_rows,
+                                                        uint32_t* __restrict__ split_tab, uint32_t* __restrict__ split_n,
+                                                        uint32_t split_cap) {
   __shared__ uint32_t cnt[kMaxExperts];
   __shared__ uint32_t cur[kMaxExperts];  // running cursor of every expert
   __shared__ uint32_t wave_tot[16];
@@ -108,6 +110,26 @@ __global__ __launch_bounds__(1024) void moe_sort_kernel(const uint32_t* __restri
   if (tid == 0) {
     if (offsets != nullptr) offsets[E] = total_rows;
     if (n_chunks != nullptr) *n_chunks = total_chunks;
+  }
+  // A second pair of tables that splits the experts by their row count: up to 8 rows -> one chunk in the first table
+  // (split_cap entries), more -> chunks of at most 16 rows in the second (behind the first); split_n = the two lengths.
+  if (split_tab != nullptr) {
+    uint32_t n_small, n_big;
+    const uint32_t small = my_cnt >= 1 && my_cnt <= 8 ? 1u : 0u, big = my_cnt > 8 ? (my_cnt + 15) / 16 : 0u;
+    const uint32_t small0 = block_exclusive_scan_1024(small, wave_tot, &n_small);
+    const uint32_t big0 = block_exclusive_scan_1024(big, wave_tot, &n_big);
+    if (small) {
+      split_tab[3 * small0 + 0] = tid;
+      split_tab[3 * small0 + 1] = my_off;
+      split_tab[3 * small0 + 2] = my_cnt;
+    }
+    uint32_t* bt = split_tab + 3 * (size_t)split_cap;
+    for (uint32_t c = 0; c < big; ++c) {
+      bt[3 * (big0 + c) + 0] = tid;
+      bt[3 * (big0 + c) + 1] = my_off + 16 * c;
+      bt[3 * (big0 + c) + 2] = my_cnt - 16 * c < 16 ? my_cnt - 16 * c : 16;
+    }
+    if (tid == 0) { split_n[0] = n_small; split_n[1] = n_big; }
   }
   if (sorted == nullptr) return;
 
@@ -390,7 +412,7 @@ int32_t launch_topk_route(const float* logits, const float* bias, uint32_t T, ui
   } else if (counts != nullptr || offsets != nullptr) {
     hipLaunchKernelGGL(moe_sort_kernel, dim3(1), dim3(1024), 0, s, idx, T * K, E, K, (uint32_t*)nullptr,
                        (uint32_t*)nullptr, (uint32_t*)nullptr, counts, offsets, (uint32_t*)nullptr,
-                       (uint32_t*)nullptr, 8u);
+                       (uint32_t*)nullptr, 8u, (uint32_t*)nullptr, (uint32_t*)nullptr, 0u);
     RMLX_HIP_CHECK(hipGetLastError());
   }
   return RMLX_OK;
@@ -412,16 +434,17 @@ int32_t launch_route_sort_small(const float* logits, const float* bias, uint32_t
 
 int32_t launch_moe_sort(const uint32_t* idx, uint32_t n_assign, uint32_t E, uint32_t top_k, uint32_t* sorted,
                         uint32_t* sorted_tok, uint32_t* inv, uint32_t* counts, uint32_t* offsets,
-                        uint32_t* chunk_tab, uint32_t* n_chunks, uint32_t chunk_rows, hipStream_t s) {
+                        uint32_t* chunk_tab, uint32_t* n_chunks, uint32_t chunk_rows, hipStream_t s, uint32_t* split_tab,
+                        uint32_t* split_n, uint32_t split_cap) {
   if (E > (uint32_t)kMaxExperts)
     return fail(RMLX_INVALID_SHAPE, "moe_sort: n_experts (%u) exceeds maximum %d", E, kMaxExperts);
   if (chunk_rows == 0) return fail(RMLX_RUNTIME_ERROR, "moe_sort: chunk_rows must be non-zero");
-  if (n_assign <= 64 && chunk_rows == 8)  // the one-wave kernel writes chunks of 8 rows
+  if (n_assign <= 64 && chunk_rows == 8 && split_tab == nullptr)  // the one-wave kernel writes chunks of 8 rows
     hipLaunchKernelGGL(moe_sort_small_kernel, dim3(1), dim3(64), 0, s, idx, n_assign, E, top_k ? top_k : 1u, sorted,
                        sorted_tok, inv, counts, offsets, chunk_tab, n_chunks);
   else
     hipLaunchKernelGGL(moe_sort_kernel, dim3(1), dim3(1024), 0, s, idx, n_assign, E, top_k ? top_k : 1u, sorted,
-                       sorted_tok, inv, counts, offsets, chunk_tab, n_chunks, chunk_rows);
+                       sorted_tok, inv, counts, offsets, chunk_tab, n_chunks, chunk_rows, split_tab, split_n, split_cap);
   RMLX_HIP_CHECK(hipGetLastError());
   return RMLX_OK;
 }

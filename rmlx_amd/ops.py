@@ -57,7 +57,8 @@ class QuantizedWeight:
     def set_expert_stream_kernel(self, kind):
         """(stacked gate weight) streaming kernel of decode-sized batches: 0 the library's choice, 1 K split over the
         waves of a workgroup, 2 / 3 a wave per weight tile with chunks of 8 / 16 rows, 4 kernel 1 for gate / up and kernel 2
-        for the down projection.  Returns the previous value."""
+        for the down projection, 5 as 4 with the gate / up projection in two launches (experts with up to 8 rows on kernel 1,
+        the others on kernel 3).  Returns the previous value."""
         return int(rt.lib().rmlx_hip_qweight_set_expert_stream_kernel(self.handle, int(kind)))
 
     def use_gemm_layout(self, enable=True, stream=None):

@@ -860,7 +860,9 @@ def test_config5_moe(hip, config5, T):
 def test_config5_expert_stream_kernels_agree(hip, config5, T):
     """The streaming kernels of decode-sized batches on config 5, every token against the oracle: K split over the waves
     of a workgroup (1), a wave per weight tile over chunks of 8 rows (2) and of 16 rows (3: at T = 128 most experts have
-    9 to 16 rows, a few more than 16), the hybrid the library picks (0 / 4).  The grouped GEMM is switched off."""
+    9 to 16 rows, a few more than 16), the hybrid (4), the gate / up projection in two launches with the experts split by
+    their row count (5: up to 8 rows on kernel 1, more on kernel 3) and the library's choice among them (0).  The grouped
+    GEMM is switched off."""
     from rmlx_amd import ops
     from rmlx_amd.runtime import DeviceBuffer
     gate, up, down, gh, uh, dh = config5
@@ -873,7 +875,7 @@ def test_config5_expert_stream_kernels_agree(hip, config5, T):
     idxd, wd = DeviceBuffer.from_numpy(idx), DeviceBuffer.from_numpy(w)
     prev_rows, prev_kind = gh.set_expert_gemm_min_rows(0), gh.set_expert_stream_kernel(0)
     try:
-        for kind in (0, 1, 2, 3, 4):
+        for kind in (0, 1, 2, 3, 4, 5):
             gh.set_expert_stream_kernel(kind)
             print(f"config5 stream kernel {kind} T={T} max rows per expert {int(counts.max())}", flush=True)
             assert_close(ops.moe_forward(gh, uh, dh, xd, ld, 8).numpy(), ref, f"config5 T={T} stream kernel {kind}")
@@ -911,7 +913,7 @@ def test_wave_per_tile_kernel_shapes(hip, E, T, K, D, I, fused):
     ref = model.moe_forward(x, idx, w, gate, up, down, 64, K)
     xd, ld = DeviceBuffer.from_numpy(x), DeviceBuffer.from_numpy(logits)
     gh.set_expert_gemm_min_rows(0)
-    for kind in (1, 2, 3, 4):
+    for kind in (1, 2, 3, 4, 5):
         gh.set_expert_stream_kernel(kind)
         print(f"wave-per-tile shapes E={E} T={T} D={D} I={I} fused={fused} kind={kind} counts={counts.tolist()}", flush=True)
         assert_close(ops.moe_forward(gh, uh, dh, xd, ld, K).numpy(), ref, f"stream kernel {kind}")
