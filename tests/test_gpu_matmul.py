@@ -343,7 +343,8 @@ def test_q8_qmv_closed_form_and_positions(hip):
 # ---- fused store epilogues (qmm_add_residual_into_cb / qmm_swiglu_into_cb, quantized.rs:8227-8452) -------
 
 @pytest.mark.parametrize("m,n,k,bits", [(64, 256, 512, 4), (130, 128, 1024, 4), (40, 128, 512, 8), (4, 64, 512, 4), (9, 24, 128, 4),
-                                      (1, 64, 2048, 4), (2, 72, 4096, 4), (1, 32, 1024, 8), (2, 16, 2048, 8)])
+                                      (1, 64, 2048, 4), (2, 72, 4096, 4), (1, 32, 1024, 8), (2, 16, 2048, 8),
+                                      (64, 256, 640, 4), (130, 128, 1408, 8), (6, 64, 1152, 4), (300, 64, 320, 4), (2, 4104, 512, 4)])
 @pytest.mark.parametrize("edtype", ["f16", "f32"])
 def test_fused_epilogues(hip, m, n, k, bits, edtype):
     """GEMM and single-row GEMV (fused), multi-row GEMV and portable (separate pass) kernels against the f64
@@ -407,7 +408,8 @@ def test_qmm_split_k(hip, m, n, k, bits, gs, dtype):
 @pytest.mark.parametrize("m,n,k,bits,gs,dtype", [(1, 4096, 4096, 4, 64, "f16"), (2, 1024, 11008, 4, 64, "f16"),
                                                  (1, 512, 18944, 4, 64, "f16"), (1, 256, 2048, 8, 32, "f32"),
                                                  (2, 768, 1024, 8, 128, "bf16"), (5, 1024, 4096, 4, 64, "f16"),
-                                                 (40, 512, 2048, 4, 64, "bf16"), (3, 24, 96, 4, 32, "f16")])
+                                                 (40, 512, 2048, 4, 64, "bf16"), (3, 24, 96, 4, 32, "f16"),
+                                                 (40, 256, 640, 4, 64, "f16"), (300, 128, 2880, 4, 64, "bf16"), (6, 64, 1408, 4, 64, "f16")])
 def test_qmm_norm_prologue(hip, m, n, k, bits, gs, dtype):
     """RMSNorm prologue (`has_norm` of the reference's MMA kernel, quantized.rs:3070-3095): fused into the
     single-row GEMV, a pass of its own in front of the other kernels.  Checked against the oracle, and bit
