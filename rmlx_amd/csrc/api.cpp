@@ -1415,8 +1415,18 @@ int32_t rmlx_hip_expert_group_grouped_forward(const rmlx_qweight* gate, const rm
     RMLX_TRY(dtab.alloc(total * 4, s));
     RMLX_HIP_CHECK(hipMemcpyAsync(dtab.ptr, expert_of.data(), total * 4, hipMemcpyHostToDevice, s));
     RMLX_HIP_CHECK(hipStreamSynchronize(s));  // `expert_of` is pageable host memory owned by this call
-    RMLX_TRY(run_expert_ffn_portable(gate, up, down, sh, xk, static_cast<const uint32_t*>(dtab.ptr), rows,
-                                     static_cast<__half*>(out_f16_dev), s));
+    const uint32_t* experts = static_cast<const uint32_t*>(dtab.ptr);
+    // where the single-row kernels take the weights (4- / 8-bit, rows in whole 16-byte pieces: a hidden size of 2880), every
+    // row multiplies with its own expert on them -- an expert streamed once per row, far ahead of the portable kernels
+    if (rows <= kUngroupedOnlyMaxAssignments && sh.stream_kernel != 1 && aligned16(xk) && single_row_experts(gate, up, down, sh)) {
+      RMLX_TRY(h.alloc(total * sh.I * 2, s));
+      RMLX_TRY(launch_qmv_m1_gate_up(gate_up_args(gate, up, sh, xk, static_cast<__half*>(h.ptr)), gate->bits, experts, rows, 1, sh.E, s));
+      RMLX_TRY(launch_qmv_m1_gather(down->w, down->s, down->b, (uint64_t)sh.D * (sh.I * down->bits / 32),
+                                    (uint64_t)sh.D * (sh.I / down->group_size), sh.E, static_cast<const __half*>(h.ptr), experts, rows,
+                                    static_cast<__half*>(out_f16_dev), sh.D, sh.I, down->group_size, down->bits, s));
+      return finish(s);
+    }
+    RMLX_TRY(run_expert_ffn_portable(gate, up, down, sh, xk, experts, rows, static_cast<__half*>(out_f16_dev), s));
     return finish(s);
   }
   if (!aligned16(xk)) return fail(RMLX_INVALID_SHAPE, "ExpertGroup: input must be 16-byte aligned");

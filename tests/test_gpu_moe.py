@@ -831,6 +831,29 @@ def test_grouped_forward_of_single_rows(hip, E, D, I, fused, n_items):
         assert np.abs(y.astype(np.float64) - y2[:1].astype(np.float64)).max() <= 0.5 * model.tolerance(ref)
 
 
+@pytest.mark.parametrize("bits,gs,D,I", [(4, 64, 960, 2880), (8, 32, 544, 96), (4, 32, 1056, 800)])
+def test_grouped_forward_of_shapes_without_a_grouped_kernel(hip, bits, gs, D, I):
+    """ExpertGroup over expert dimensions that no chunked or grouped kernel takes (off the multiples of 128, 8-bit at group
+    size 32 with short rows): every row multiplies with its own expert on the single-row kernels instead of the portable ones.
+    Items of 1, 5, 17 and 40 rows, an expert named twice.  Against the float64 expert FFN."""
+    from rmlx_amd import ops
+    from rmlx_amd.runtime import DeviceBuffer
+    rng = np.random.default_rng(bits + gs + D + I)
+    E = 5
+    gu = make_weight(rng, 2 * I, D, bits, gs, lead=(E,))
+    down = make_weight(rng, D, I, bits, gs, lead=(E,))
+    gate, up = tuple(a[:, :I] for a in gu), tuple(a[:, I:] for a in gu)
+    gh, dh = ops.QuantizedWeight.from_numpy(*gu, gs, bits), ops.QuantizedWeight.from_numpy(*down, gs, bits)
+    group = ops.ExpertGroup(gh, None, dh)
+    items = [(e, make_x(rng, m, D)) for e, m in ((3, 1), (0, 5), (3, 17), (4, 40))]
+    print(f"ExpertGroup without a grouped kernel Q{bits} gs{gs} D={D} I={I}", flush=True)
+    outs = group.grouped_forward([(e, DeviceBuffer.from_numpy(x)) for e, x in items])
+    for (e, x), (e2, y) in zip(items, outs):
+        assert e == e2
+        ones = np.ones((len(x), 1))
+        assert_close(y, model.moe_forward(x, np.full((len(x), 1), e), ones, gate, up, down, gs, 1, bits=bits), f"expert {e} rows {len(x)}")
+
+
 @pytest.fixture(scope="module")
 def config5(hip):
     """Config 5 weights: 128 experts, hidden 4096, intermediate 1536, fused gate/up, Q4 group 64."""
