@@ -1207,6 +1207,12 @@ int32_t rmlx_hip_gather_qmm_select(const rmlx_array* x, const void* w_packed_dev
     // one row per index: the single-row kernel with a weight matrix per activation row -- one launch, no chunk table
     RMLX_TRY(launch_qmv_m1_gather(w, sc, bi, (uint64_t)n * (k / 8), (uint64_t)n * gpr, E32, xk, idx, B32,
                                   static_cast<__half*>(out_f16_dev), N32, K32, group_size, 4, s));
+  } else if (!fast && kernel == GATHER_AUTO && rows <= kUngroupedOnlyMaxAssignments && qmv_m1_supported(N32, K32, group_size, 4) &&
+             aligned16(w) && aligned16(sc) && aligned16(bi) && aligned16(xk)) {
+    // several rows per index over a shape no streaming or grouped kernel takes (rows off the multiples of 128): every row on
+    // the single-row kernel with its entry's weight matrix, instead of the portable kernel
+    RMLX_TRY(launch_qmv_m1_gather(w, sc, bi, (uint64_t)n * (k / 8), (uint64_t)n * gpr, E32, xk, idx, rows,
+                                  static_cast<__half*>(out_f16_dev), N32, K32, group_size, 4, s, (uint32_t)m_per_batch));
   } else if (fast && kernel != GATHER_PORTABLE) {
     const uint64_t per = ((uint64_t)m_per_batch + 7) / 8, n_chunks = (uint64_t)B32 * per;
     if (n_chunks > 0x7FFFFFFFull) return fail(RMLX_INVALID_SHAPE, "gather_qmm: too many row chunks (%" PRIu64 ")", n_chunks);

@@ -156,7 +156,8 @@ bool qmv_m1_gate_up_supported(uint32_t N, uint32_t K, uint32_t group_size, uint3
 // the shapes qmv_m1_supported(N, K, group_size, bits) takes
 int32_t launch_qmv_m1_gather(const uint32_t* w, const __half* s, const __half* b, uint64_t estride_w, uint64_t estride_s,
                              uint32_t n_experts, const __half* x, const uint32_t* idx, uint32_t batch, __half* out, uint32_t N,
-                             uint32_t K, uint32_t group_size, uint32_t bits, hipStream_t stream);
+                             uint32_t K, uint32_t group_size, uint32_t bits, hipStream_t stream,
+                             uint32_t rows_per_index = 1);  // batch rows; rows_per_index consecutive rows share idx[row / rows_per_index]
 int32_t launch_qmv_m1_gate_up(const QmvArgs& a, uint32_t bits, const uint32_t* idx, uint32_t assignments, uint32_t top_k,
                               uint32_t n_experts, hipStream_t stream);
 // Down projection of a few tokens with the weighted combine behind it on the single-row layout (qmv_m1.hip): h

@@ -61,6 +61,9 @@ struct M1Params {
   const uint32_t* gather_idx;
   uint64_t estride_w, estride_s;
   uint32_t n_experts;
+  // (gather_div consecutive rows share an index: row m of this launch, which starts at row gather_row0 of the call, takes
+  // gather_idx[(gather_row0 + m) / gather_div]; 0 or 1 = an index per row)
+  uint32_t gather_div = 1, gather_row0 = 0;
 };
 
 __device__ __forceinline__ h2 as_h2(uint32_t v) { return __builtin_bit_cast(h2, v); }
@@ -311,7 +314,7 @@ __global__ __launch_bounds__(kThreads, (BITS == 8 && MR == 1 && R == 1) ? 8 : (M
   uint64_t e_w = 0, e_s = 0;
   bool gather_zeros = false;
   if constexpr (GATHER) {
-    const uint32_t e = p.gather_idx[mrow0];
+    const uint32_t e = p.gather_idx[p.gather_div > 1 ? (p.gather_row0 + mrow0) / p.gather_div : mrow0];
     gather_zeros = e >= p.n_experts;
     e_w = gather_zeros ? 0 : e * p.estride_w;
     e_s = gather_zeros ? 0 : e * p.estride_s;
@@ -442,7 +445,7 @@ __global__ __launch_bounds__(kThreads, 1) void qmv_m1_loop_kernel(M1Params p) {
   uint64_t e_w = 0, e_s = 0;
   bool gather_zeros = false;
   if constexpr (GATHER) {
-    const uint32_t e = p.gather_idx[mrow0];
+    const uint32_t e = p.gather_idx[p.gather_div > 1 ? (p.gather_row0 + mrow0) / p.gather_div : mrow0];
     gather_zeros = e >= p.n_experts;
     e_w = gather_zeros ? 0 : e * p.estride_w;
     e_s = gather_zeros ? 0 : e * p.estride_s;
@@ -1014,7 +1017,7 @@ void launch_gather_bits(const M1Params& p, uint32_t group_size, bool two, hipStr
 // weights, out [batch, N] f16.  One launch, no chunk table: the activation row of a pass picks its matrix.
 int32_t launch_qmv_m1_gather(const uint32_t* w, const __half* s, const __half* b, uint64_t estride_w, uint64_t estride_s,
                              uint32_t n_experts, const __half* x, const uint32_t* idx, uint32_t batch, __half* out, uint32_t N,
-                             uint32_t K, uint32_t group_size, uint32_t bits, hipStream_t stream) {
+                             uint32_t K, uint32_t group_size, uint32_t bits, hipStream_t stream, uint32_t rows_per_index) {
   if (!qmv_m1_supported(N, K, group_size, bits))
     return fail(RMLX_INVALID_SHAPE, "qmv_m1 gather: unsupported shape N=%u K=%u bits=%u group_size=%u", N, K, bits, group_size);
   // (weights loaded with the ordinary cache policy: two indices may name one expert)
@@ -1022,7 +1025,8 @@ int32_t launch_qmv_m1_gather(const uint32_t* w, const __half* s, const __half* b
   for (uint32_t first = 0; first < batch; first += 65535) {  // the activation row is the second grid dimension
     const uint32_t rows = batch - first < 65535 ? batch - first : 65535;
     M1Params p{w, s, b, x + (uint64_t)first * K, out + (uint64_t)first * N, N, K, rows, EPI_NONE, 0, nullptr, nullptr, nullptr,
-               idx + first, estride_w, estride_s, n_experts};
+               rows_per_index > 1 ? idx : idx + first, estride_w, estride_s, n_experts};
+    if (rows_per_index > 1) { p.gather_div = rows_per_index; p.gather_row0 = first; }
     if (bits == 4) launch_gather_bits<4>(p, group_size, two, stream);
     else launch_gather_bits<8>(p, group_size, two, stream);
     RMLX_HIP_CHECK(hipGetLastError());

@@ -188,7 +188,8 @@ def _gather_setup(rng, E, n, k, batch, mpb, dtype=np.float16):
 
 @pytest.mark.parametrize("E,n,k,batch,mpb", [(2, 4, 32, 2, 1), (4, 64, 512, 9, 1), (8, 128, 1024, 5, 3),
                                               (3, 48, 1536, 4, 11), (128, 1536, 4096, 32, 1), (6, 256, 2048, 7, 2),
-                                              (5, 64, 640, 6, 3), (4, 48, 1408, 3, 8), (7, 32, 768, 9, 1)])
+                                              (5, 64, 640, 6, 3), (4, 48, 1408, 3, 8), (7, 32, 768, 9, 1),
+                                              (5, 64, 960, 6, 3), (3, 48, 2880, 4, 11)])
 def test_gather_qmm_matches_oracle(hip, E, n, k, batch, mpb):
     from rmlx_amd import ops
     rng = np.random.default_rng(E * 7 + n)
