@@ -252,7 +252,11 @@ int32_t run_matmul_plain(const rmlx_qweight* qw, const void* x, int32_t x_dtype,
     // With only the LDS-staged GEMM as the alternative (K a multiple of 64 but not of 256, floor 10 to 23 us) the passes keep
     // up to 16 rows, except over small matrices, where the third pass already costs more than the GEMM (4-bit, 16 rows:
     // 4864 x 896 13.2 against 10.6 us, 6912 x 1152 16.9 against 12.3; 4096 x 2880 16.2 against 22.8, 5120 x 2880 19.0 against 22.8).
-    const bool passes_lose = !can_qmv && !can_qmm_rw && can_qmm_lds && M > 8 && wbytes < (5ull << 20);
+    // Short rows make a pass dearer still (a whole-row wave leaves lanes idle below 2048 values): group size 32, 13824 x 1152,
+    // 8 / 16 rows 17.5 / 29.9 against 13.0 us, 9728 x 896 at 8 rows 13.7 against 10.8; tiny matrices keep the passes (128 x 896,
+    // 16 rows: about 7 against 9.9 us).
+    const bool passes_lose = !can_qmv && !can_qmm_rw && can_qmm_lds &&
+                             ((M > 8 && wbytes >= (1ull << 20) && wbytes < (5ull << 20)) || (M > 4 && K < 2048 && wbytes >= (3ull << 20)));
     const bool m1_first = can_m1 && !passes_lose && (can_qmv || !can_qmm_rw || M <= kM1PassRows);
     // One or two rows over short rows of a tall matrix: a wave of the single-row kernel owns a whole row, and a row of fewer
     // than 2048 values leaves part of its lanes without a load (896: 28 of 64), while the multi-row GEMV splits its tiles
