@@ -234,14 +234,17 @@ int32_t run_matmul_plain(const rmlx_qweight* qw, const void* x, int32_t x_dtype,
     //          16.2, 16384 x 4096: 15.3 against 16.6, weights cycled through more than 1 GiB; beyond that the GEMM's grid is
     //          large enough to win: 28672 x 4096 22 against 29 us);
     //          17 to 32 rows in passes of 8 while W <= 12 MiB: 4096 x 4096 8.8 / 9.1 / 9.3 us at 17 / 24 / 32 rows against 9.6 /
-    //          9.9 / 10.3 on the GEMM; 9216 x 4096 at 32 rows: 20.9 against 17.3, so not beyond);
+    //          9.9 / 10.3 on the GEMM; 9216 x 4096 at 32 rows: 20.9 against 17.3, so not beyond; over more than 4096 weight rows
+    //          of fewer than 4096 values the GEMM's short k loop wins: 16384 x 1024 at 17 / 32 rows 8.6 / 9.3 against 6.2 us,
+    //          8192 x 1536 7.4 / 8.2 against 7.0, 8192 x 2048 at 32 rows 9.2 against 8.3, while 4096 x 3072 keeps the passes, 7.9
+    //          against 9.4, as do 4096 x 2048 and 2048 x 2048);
     //   8-bit: GEMV up to 16 rows while W < 48 MiB (4096 x 4096 is 16 MiB; at 12288 x 4096 the GEMM wins, 19 against 23 us).
     const uint64_t wbytes = (uint64_t)N * K * qw->bits / 8;
     // Without the register-weights GEMM (K not a multiple of 512) the alternative is the LDS-staged GEMM with
     // a floor of about 15 us: there the 4-bit GEMV keeps up to passes * W <= 48 MiB.
     const bool small_m = !can_qmm_rw ? M <= kQmvMaxM || (qw->bits == 4 && (uint64_t)((M + 7) / 8) * wbytes <= (48ull << 20))
                          : qw->bits == 4 ? M <= 8 || (M <= kQmvMaxM && (wbytes <= (12ull << 20) || N <= 16384)) ||
-                                               (M <= 32 && wbytes <= (12ull << 20))
+                                               (M <= 32 && wbytes <= (12ull << 20) && (N <= 4096 || K >= 4096))
                                          : (M <= kQmvMaxM && wbytes < (48ull << 20));
     // Shapes the K-split GEMV does not take (group size 32) run up to 16 rows on the single-row kernel in passes of four,
     // which streams the weights once per pass: with the register-weights GEMM as the alternative it keeps up to 4 rows
@@ -398,7 +401,12 @@ int32_t run_matmul_plain(const rmlx_qweight* qw, const void* x, int32_t x_dtype,
     *epi_done = true;
     return launch_qmm_k2(a, qw->group_size, k2_tile_rows, stream);
   }
-  if (kernel == KERNEL_QMM && can_qmm_rw) {
+  // Group size 32 with a K tail (K in whole blocks of 128, not of 512): the register-weights GEMM has two small tile shapes
+  // for this group size and pads its last round; from 256 rows on the LDS-staged GEMM with its 128-row tiles is ahead
+  // (13824 x 1152: 256 / 512 / 2048 rows 21.6 / 38.9 / 132 against 25.9 / 51.5 / 170 us; 9728 x 896: 17.8 / 26.3 / 77 against
+  // 20.0 / 29.9 / 96; 4096 x 11008 at 2048 rows: a tie), below that the register-weights GEMM (32 rows: 8.7 against 12.6 us).
+  const bool lds_first = kernel == KERNEL_QMM && can_qmm_lds && qw->group_size == 32 && K % 512 != 0 && M >= 256;
+  if (kernel == KERNEL_QMM && can_qmm_rw && !lds_first) {
     // Register-weights GEMM: f16 / bf16 activations straight from the row-major matrix, no workspace
     // (bf16 -> f16 inside the kernel: exact for normal-range values, and f16 weights keep 11
     // significant bits); f32 activations are cast first.

@@ -109,7 +109,7 @@ __device__ __forceinline__ h8 dequant_q8_pair(uint32_t w0, uint32_t w1, h2 s2, h
 // rows, fragment 1 the same rows of the up weight (NF == 2), and the store writes silu(gate) * up.
 // TAIL (group sizes 32 and 64): K is a multiple of 128 but not of 512.  The last unrolled round of the loop then holds iterations past
 // K: their activation chunks are written to LDS as zeros, weight loads repeat the last block, and the scales and biases
-// of the last round come from a load that ends with the row (group size 32: word by word with the index clamped).
+// of the last round come from loads that end with the row.
 template <int MF, int NF, int BITS, int NW, bool XBF16, int GS, int MODE, bool TAIL = false>
 __device__ __forceinline__ void qmm_rw_body(const RwParams p) {  // by value: a reference makes every store a possible change of p
   static_assert(MODE != 2 || NF == 2, "a gate/up pair takes two weight fragments per wave");
@@ -262,30 +262,20 @@ __device__ __forceinline__ void qmm_rw_body(const RwParams p) {  // by value: a 
   auto load_sb = [&](uint32_t blk, u4 (&ds)[NF][kSbVecs], u4 (&db)[NF][kSbVecs]) {
 #pragma unroll
     for (int f = 0; f < NF; ++f) {
-      if (TAIL && GS == 64) {
-        // One word per iteration, S >= 4 words per row.  The 16 bytes of a round that would run past the row's end start
-        // early enough to end with the row (4-byte aligned: enough for the hardware), and the words move down to
-        // their places; what then sits behind the row's last word belongs to iterations past K.
+      if (TAIL) {
+        // kWordsPerIt words per iteration (one at group size 64, two at 32), S * kWordsPerIt >= 4 * kWordsPerIt words per
+        // row.  The 16-byte loads of a round that would run past the row's end start early enough to end with the row
+        // (4-byte aligned: enough for the hardware), and the words move down to their places; what then sits behind
+        // the row's last word belongs to iterations past K.
         // (the move happens late in the round before, see settle_sb: done here it would wait for the load at once)
-        const uint32_t want = blk * 4, wo = want < S - 4 ? want : S - 4;  // (wave-uniform)
-        const U4Tail sv = *reinterpret_cast<const U4Tail*>(reinterpret_cast<const uint32_t*>(sptr[f]) + wo);
-        const U4Tail bv = *reinterpret_cast<const U4Tail*>(reinterpret_cast<const uint32_t*>(bptr[f]) + wo);
-        ds[f][0] = (u4){sv.v[0], sv.v[1], sv.v[2], sv.v[3]};
-        db[f][0] = (u4){bv.v[0], bv.v[1], bv.v[2], bv.v[3]};
-      } else if (TAIL) {  // words of a round in row order (4 groups per iteration: 2 words); the row ends after iteration S - 1
-        constexpr uint32_t kWordsPerIt = kBlockK / GS / 2;
-        const uint32_t last_word = S * kWordsPerIt - 1;
+        constexpr uint32_t kWordsPerIt = GS == 128 ? 1 : kBlockK / GS / 2, kRound = 4 * kWordsPerIt;  // (no tail form at group size 128)
+        const uint32_t want = blk * kRound, wo = want < S * kWordsPerIt - kRound ? want : S * kWordsPerIt - kRound;  // (wave-uniform)
 #pragma unroll
         for (int v = 0; v < kSbVecs; ++v) {
-          uint32_t sw[4], bw[4];
-#pragma unroll
-          for (int c = 0; c < 4; ++c) {
-            const uint32_t want = (blk * kSbVecs + v) * 4 + c, wi = want < last_word ? want : last_word;
-            sw[c] = reinterpret_cast<const uint32_t*>(sptr[f])[wi];
-            bw[c] = reinterpret_cast<const uint32_t*>(bptr[f])[wi];
-          }
-          ds[f][v] = (u4){sw[0], sw[1], sw[2], sw[3]};
-          db[f][v] = (u4){bw[0], bw[1], bw[2], bw[3]};
+          const U4Tail sv = *reinterpret_cast<const U4Tail*>(reinterpret_cast<const uint32_t*>(sptr[f]) + wo + 4 * v);
+          const U4Tail bv = *reinterpret_cast<const U4Tail*>(reinterpret_cast<const uint32_t*>(bptr[f]) + wo + 4 * v);
+          ds[f][v] = (u4){sv.v[0], sv.v[1], sv.v[2], sv.v[3]};
+          db[f][v] = (u4){bv.v[0], bv.v[1], bv.v[2], bv.v[3]};
         }
       } else if (GS == 128) {  // 4 groups = 8 bytes per row and four iterations
         const u2 sv = reinterpret_cast<const u2*>(sptr[f])[blk], bv = reinterpret_cast<const u2*>(bptr[f])[blk];
@@ -300,15 +290,26 @@ __device__ __forceinline__ void qmm_rw_body(const RwParams p) {  // by value: a 
       }
     }
   };
-  // tail form at group size 64: the words of round blk, as loaded by load_sb, move down to their places
+  // tail form: the words of round blk, as loaded by load_sb, move down to their places (by whole iterations)
   auto settle_sb = [&](uint32_t blk, u4 (&ds)[NF][kSbVecs], u4 (&db)[NF][kSbVecs]) {
-    const uint32_t want = blk * 4, wo = want < S - 4 ? want : S - 4, d = want - wo;  // (wave-uniform)
+    constexpr uint32_t kWordsPerIt = GS == 128 ? 1 : kBlockK / GS / 2, kRound = 4 * kWordsPerIt;  // (no tail form at group size 128)
+    const uint32_t want = blk * kRound, wo = want < S * kWordsPerIt - kRound ? want : S * kWordsPerIt - kRound;
+    const uint32_t its = (want - wo) / kWordsPerIt;  // (wave-uniform: 0 .. 3 iterations)
+    auto moved = [&](u4 (&v)[kSbVecs]) {
+      uint32_t in[kRound], out[kRound];
 #pragma unroll
-    for (int f = 0; f < NF; ++f) {
-      const u4 sv = ds[f][0], bv = db[f][0];
-      ds[f][0] = (u4){d == 0 ? sv.x : d == 1 ? sv.y : d == 2 ? sv.z : sv.w, d == 0 ? sv.y : d == 1 ? sv.z : sv.w, d == 0 ? sv.z : sv.w, sv.w};
-      db[f][0] = (u4){d == 0 ? bv.x : d == 1 ? bv.y : d == 2 ? bv.z : bv.w, d == 0 ? bv.y : d == 1 ? bv.z : bv.w, d == 0 ? bv.z : bv.w, bv.w};
-    }
+      for (int c = 0; c < (int)kRound; ++c) in[c] = c % 4 == 0 ? v[c / 4].x : (c % 4 == 1 ? v[c / 4].y : (c % 4 == 2 ? v[c / 4].z : v[c / 4].w));
+#pragma unroll
+      for (int c = 0; c < (int)kRound; ++c) {
+        constexpr int last = (int)kRound - 1, k = (int)kWordsPerIt;
+        const uint32_t a1 = in[c + k < last ? c + k : last], a2 = in[c + 2 * k < last ? c + 2 * k : last], a3 = in[c + 3 * k < last ? c + 3 * k : last];
+        out[c] = its == 0 ? in[c] : (its == 1 ? a1 : (its == 2 ? a2 : a3));
+      }
+#pragma unroll
+      for (int q = 0; q < kSbVecs; ++q) v[q] = (u4){out[4 * q], out[4 * q + 1], out[4 * q + 2], out[4 * q + 3]};
+    };
+#pragma unroll
+    for (int f = 0; f < NF; ++f) { moved(ds[f]); moved(db[f]); }
   };
   auto load_w = [&](uint32_t it, u4 (&dst)[NF][WL]) {
 #pragma unroll
@@ -401,7 +402,7 @@ __device__ __forceinline__ void qmm_rw_body(const RwParams p) {  // by value: a 
       const uint32_t it = it0 + u;
       // (the next round's scales and biases were requested three iterations ago; its first weight operand is unpacked in
       // this iteration's last step)
-      if (TAIL && GS == 64 && u == kUnroll - 1) settle_sb(blk < last_blk ? blk + 1 : last_blk, s_nxt, b_nxt);
+      if (TAIL && u == kUnroll - 1) settle_sb(blk < last_blk ? blk + 1 : last_blk, s_nxt, b_nxt);
       const u4* a_stage = a_lds + (it % kStages) * kChunk;
       const u4* a_stage_next = a_lds + ((it + 1) % kStages) * kChunk;
       u4* a_stage_write = a_lds + ((it + 2) % kStages) * kChunk;
@@ -540,10 +541,11 @@ void launch_rw(RwParams p, bool x_bf16, hipStream_t s) {
   p.tiles_m = (p.M + 16 * MF - 1) / (16 * MF);
   p.tiles_n = p.N / (NW * 16 * NF);
   const dim3 grid(p.tiles_m * p.tiles_n, p.ksplit), block(64 * NW);
-  const bool tail = (p.K / kBlockK / p.ksplit) % kUnroll != 0;  // (group size 64 only: checked by qmm_rw_supported)
-  if (GS == 64 && tail) {
-    if (x_bf16) hipLaunchKernelGGL((qmm_rw_kernel<MF, NF, BITS, NW, true, 64, true>), grid, block, 0, s, p);
-    else hipLaunchKernelGGL((qmm_rw_kernel<MF, NF, BITS, NW, false, 64, true>), grid, block, 0, s, p);
+  const bool tail = (p.K / kBlockK / p.ksplit) % kUnroll != 0;  // (group sizes 32 and 64 only: checked by qmm_rw_supported)
+  constexpr int kTailGs = GS == 128 ? 64 : GS;
+  if (GS != 128 && tail) {
+    if (x_bf16) hipLaunchKernelGGL((qmm_rw_kernel<MF, NF, BITS, NW, true, kTailGs, true>), grid, block, 0, s, p);
+    else hipLaunchKernelGGL((qmm_rw_kernel<MF, NF, BITS, NW, false, kTailGs, true>), grid, block, 0, s, p);
   } else {
     if (x_bf16) hipLaunchKernelGGL((qmm_rw_kernel<MF, NF, BITS, NW, true, GS, false>), grid, block, 0, s, p);
     else hipLaunchKernelGGL((qmm_rw_kernel<MF, NF, BITS, NW, false, GS, false>), grid, block, 0, s, p);
@@ -553,9 +555,9 @@ void launch_rw(RwParams p, bool x_bf16, hipStream_t s) {
 }  // namespace
 
 bool qmm_rw_supported(uint32_t N, uint32_t K, uint32_t group_size, uint32_t bits) {
-  // (group size 64 also takes K in whole 128-wide blocks, at least four: the tail form)
+  // (group sizes 32 and 64 also take K in whole 128-wide blocks, at least four: the tail form)
   return (group_size == 32 || group_size == 64 || group_size == 128) && (bits == 4 || bits == 8) && N > 0 && K > 0 && N % 64 == 0 &&
-         (K % (kBlockK * kUnroll) == 0 || (group_size == 64 && K % kBlockK == 0 && K >= 4 * kBlockK));
+         (K % (kBlockK * kUnroll) == 0 || (group_size != 128 && K % kBlockK == 0 && K >= 4 * kBlockK));
 }
 
 

@@ -985,29 +985,29 @@ def test_staged_gemm_at_group_sizes_32_and_128(hip, bits, gs, n, k):
         _run(hip, words, s, b, make_x(rng, 32, k, "bf16"), bits, gs=gs, dtype="bf16", kernel=rt.KERNEL_QMM_BF16)
 
 
-@pytest.mark.parametrize("bits", [4, 8])
+@pytest.mark.parametrize("bits,gs", [(4, 64), (8, 64), (4, 32), (8, 32)])
 @pytest.mark.parametrize("n,k", [(64, 256), (128, 384), (256, 640), (64, 1408), (128, 2816)])
-def test_gemms_and_multi_row_gemv_with_k_in_whole_blocks_of_128(hip, bits, n, k):
+def test_gemms_and_multi_row_gemv_with_k_in_whole_blocks_of_128(hip, bits, gs, n, k):
     """K a multiple of 128 but not of 512 (11008, 8960, 4864, 6912 in real models): the register-weights GEMM pads its last
     unrolled round with zero activations and clamps weight, scale and bias loads to the row; the 4-bit multi-row GEMV walks
     whole slabs with a shorter last part.  Scales and biases grow along the row so a wrong or repeated group shows.
     Against the oracle through the automatic choice and every kernel that takes the shape, f16 / bf16 / f32 rows."""
     from rmlx_amd import runtime as rt
-    rng = np.random.default_rng(bits * 13 + n + k)
-    words, s, b = make_weight(rng, n, k, bits, 64)
-    ramp = (1.0 + np.arange(k // 64) % 5).astype(np.float16)
+    rng = np.random.default_rng(bits * 13 + gs + n + k)
+    words, s, b = make_weight(rng, n, k, bits, gs)
+    ramp = (1.0 + np.arange(k // gs) % 5).astype(np.float16)
     s, b = (s * ramp).astype(np.float16), (b * ramp[::-1]).astype(np.float16)
     for m, dtype in ((3, "f16"), (8, "bf16"), (16, "f16"), (17, "f16"), (70, "bf16"), (130, "f32"), (600, "f16")):
         x = make_x(rng, m, k, dtype)
-        ref = model.qmm(x_as_f64(x, dtype), words, s, b, 64, bits)
+        ref = model.qmm(x_as_f64(x, dtype), words, s, b, gs, bits)
         kernels = [rt.KERNEL_AUTO, rt.KERNEL_QMM, rt.KERNEL_QMM_LDS]
         if k >= 512:  # (the tail form wants four blocks; shorter rows run on the LDS-staged GEMM)
             kernels.append(rt.KERNEL_QMM_RW)
-        if bits == 4:
+        if bits == 4 and gs == 64:
             kernels.append(rt.KERNEL_QMV)
         for kernel in kernels:
-            assert_close(_run(hip, words, s, b, x, bits, dtype=dtype, kernel=kernel), ref,
-                         f"Q{bits} {dtype} M={m} N={n} K={k} kernel={kernel}")
+            assert_close(_run(hip, words, s, b, x, bits, gs=gs, dtype=dtype, kernel=kernel), ref,
+                         f"Q{bits} gs={gs} {dtype} M={m} N={n} K={k} kernel={kernel}")
 
 
 @pytest.mark.parametrize("bits,n,k", [(4, 9728, 896), (4, 16384, 1024), (4, 6144, 2048), (8, 8192, 512), (4, 4864, 896)])
