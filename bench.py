@@ -529,7 +529,8 @@ def main():
             # The routed block at 6 / 8 / 10 rows per expert with every choice of expert kernels (for kernel traces:
             # which projection costs what under which kernel).  (label, GEMM threshold, streaming kernel selector)
             variants = (("kplit_8row_chunks", 0, 1), ("wave_per_tile_8row_chunks", 0, 2), ("wave_per_tile_16row_chunks", 0, 3),
-                        ("hybrid_kplit_gate_up_wave_down", 0, 4), ("grouped_gemm", 1, 0), ("library_choice", None, 0))
+                        ("hybrid_kplit_gate_up_wave_down", 0, 4), ("split_by_rows_kplit_and_16row", 0, 5), ("grouped_gemm", 1, 0),
+                        ("library_choice", None, 0))
             for T in (96, 128, 160):
                 for label, min_rows, kind in variants:
                     # (a threshold of 1 forces the GEMM; its tile height follows the average rows per expert: 16-row tiles
