@@ -11,7 +11,10 @@ pytestmark = pytest.mark.gpu
 
 LADDER_SHAPES = [(4096, 14336, 4, (3, 9, 16)), (2048, 16384, 4, (5, 16)), (4096, 8192, 4, (9, 16)), (12288, 4096, 4, (9, 24)),
                  (28672, 4096, 4, (8, 16, 100)), (12288, 4096, 8, (9, 16, 32)), (4096, 4096, 4, (128, 160, 256)),
-                 (9216, 4096, 4, (64, 128)), (4096, 4096, 8, (128, 192)), (4096, 8192, 4, (128,))]
+                 (9216, 4096, 4, (64, 128)), (4096, 4096, 8, (128, 192)), (4096, 8192, 4, (128,)),
+                 # short rows of tall matrices, K in whole blocks of 128, one or two rows over many weight rows
+                 (9728, 896, 4, (1, 2, 24)), (16384, 1024, 4, (1, 2, 17, 32)), (4096, 11008, 4, (8, 64, 512)), (8192, 3072, 4, (2,)),
+                 (13824, 1152, 4, (32, 512)), (65536, 1024, 4, (1,)), (8192, 512, 8, (2,))]
 
 
 @pytest.mark.parametrize("n,k,bits,ms", LADDER_SHAPES)
@@ -27,7 +30,8 @@ def test_ladder_picks_within_15_percent_of_the_fastest_family(hip, n, k, bits, m
     qws = [ops.QuantizedWeight.from_numpy(np.roll(base[0], i, 0), np.roll(base[1], i, 0), np.roll(base[2], i, 0), 64, bits)
            for i in range(n_sets)]
     stream, e0, e1 = rt.Stream(), rt.Event(), rt.Event()
-    families = {"auto": rt.KERNEL_AUTO, "qmv": rt.KERNEL_QMV_ROWS, "qmm": rt.KERNEL_QMM, "k2": rt.KERNEL_QMM_K2,
+    families = {"auto": rt.KERNEL_AUTO, "qmv": rt.KERNEL_QMV_ROWS, "single": rt.KERNEL_QMV, "qmm": rt.KERNEL_QMM, "k2": rt.KERNEL_QMM_K2,
+                "lds": rt.KERNEL_QMM_LDS,
                 "rw": rt.KERNEL_QMM_RW, "k2_tall": rt.KERNEL_QMM_K2_TALL, "k2_flat": rt.KERNEL_QMM_K2_FLAT, "k4": rt.KERNEL_QMM_K4}
 
     def train_us(xd, outs, kernel, count=300):
