@@ -1641,7 +1641,10 @@ int32_t moe_grouped_impl(const rmlx_qweight* gate, const rmlx_qweight* up, const
   // nearly every expert is one chunk of 8 rows and the grouped GEMM's threshold, chunks of 8 stream an expert with 9 to 16
   // rows twice and chunks of 16 on the wave-per-tile kernel are slower for the others.
   const bool split = route == nullptr && gemm == 0 && sh.bits == 4 && sh.wave_tiles && plan.gate_up == 0 && plan.chunk_rows == 8 &&
-                     (sh.stream_kernel == 5 || (sh.stream_kernel == 0 && (uint64_t)A * 2 >= (uint64_t)kSplitMinRows2 * sh.E));
+                     (sh.stream_kernel == 5 || (sh.stream_kernel == 0 && (uint64_t)A * 2 >= (uint64_t)kSplitMinRows2 * sh.E &&
+                                                (uint64_t)sh.I * sh.D >= (4ull << 20)));  // (small experts: the second launch costs
+                                                                                          // more than it saves, E = 40, D = 1536,
+                                                                                          // I = 512 at 32 tokens: 48 against 35 us)
   const uint32_t cap_small = A < sh.E ? A : sh.E, cap_big = A / 8 + 1;
   const size_t split_words = split ? 3 * ((size_t)cap_small + cap_big) + 4 : 0;
   // meta: sorted[A] | sorted_tok[A] | inv[A] | chunk_tab[3*max_chunks] | n_chunks[1] (| split tables | their lengths[2])

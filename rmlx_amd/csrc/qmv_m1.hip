@@ -85,6 +85,17 @@ __device__ __forceinline__ float wave_sum(float v) {
          __builtin_bit_cast(float, __builtin_amdgcn_readlane(bits, 32));
 }
 
+// sum over the 32 lanes of a half of the wave, returned in every lane of that half (the same additions as wave_sum up to its
+// last one)
+__device__ __forceinline__ float half_wave_sum(float v) {
+  v = dpp_add<0xB1>(v);
+  v = dpp_add<0x4E>(v);
+  v = dpp_add<0x141>(v);
+  v = dpp_add<0x140>(v);
+  v += __builtin_bit_cast(float, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, v), 0x401F));  // lane ^ 16
+  return v;
+}
+
 // x halves (k0..k7) -> pair order (k0,k4),(k1,k5),(k2,k6),(k3,k7) of the nibble unpacking
 __device__ __forceinline__ u4 to_pair_order(u4 d) {
   u4 o;
@@ -776,16 +787,21 @@ struct M1DownParams {
   uint32_t N, K, top_k, n_experts;
 };
 
-template <int BITS, int GS, int NC, int R>
+// HALF (rows of at most 32 sixteen-byte pieces: K <= 1024 at 4 bits, 512 at 8): the two halves of a wave take R weight rows each
+// -- lanes 0-31 rows n0 .. n0+R-1, lanes 32-63 the next R -- so a short row does not leave more than half of the lanes
+// without a load (K = 768 at 4 bits: 24 of 32 lanes busy instead of 24 of 64).  Same products, same summation order per row.
+template <int BITS, int GS, int NC, int R, bool HALF = false>
 __global__ __launch_bounds__(kThreads, 2) void qmv_m1_down_combine_kernel(M1DownParams p) {
+  static_assert(!HALF || NC == 1, "half-wave rows: one chunk");
   using Image = XImage<BITS, 1>;
   constexpr int kChunkK = Image::kChunkK, kLaneK = Image::kLaneK, kXU = Image::kXU;
   constexpr int kLanesPerGroup = GS / kLaneK, kGroupsPerChunk = kChunkK / GS;
-  __shared__ float red[kWaves][R];
-  const int tid = threadIdx.x, lane = tid & 63;
+  constexpr int RW = HALF ? 2 * R : R;  // weight rows per wave
+  __shared__ float red[kWaves][RW];
+  const int tid = threadIdx.x, wlane = tid & 63, lane = HALF ? (wlane & 31) : wlane, half = HALF ? (wlane >> 5) : 0;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const uint32_t K = p.K, G = K / GS, row_u4 = K / kLaneK, nunits = K / 8;
-  const uint32_t t = blockIdx.y, n0 = blockIdx.x * R, a = t * p.top_k + wave;
+  const uint32_t t = blockIdx.y, n0 = blockIdx.x * RW + half * R, a = t * p.top_k + wave;
   uint32_t expert = 0xFFFFFFFFu;
   float cw = 0.f;
   if ((uint32_t)wave < p.top_k) {
@@ -849,17 +865,17 @@ __global__ __launch_bounds__(kThreads, 2) void qmv_m1_down_combine_kernel(M1Down
       dot_rows<BITS, R, 1>(xr, k1, wv[c], sv[c], bv[c], uc, racc);
     }
 #pragma unroll
-    for (int r = 0; r < R; ++r) res[r] = wave_sum(racc[r][0]) * cw;
+    for (int r = 0; r < R; ++r) res[r] = (HALF ? half_wave_sum(racc[r][0]) : wave_sum(racc[r][0])) * cw;
   }
   if (lane == 0) {
 #pragma unroll
-    for (int r = 0; r < R; ++r) red[wave][r] = res[r];
+    for (int r = 0; r < R; ++r) red[wave][half * R + r] = res[r];
   }
   __syncthreads();
-  if (tid < R) {
+  if (tid < RW) {
     float acc = 0.f;
     for (uint32_t k = 0; k < p.top_k; ++k) acc += red[k][tid];  // ascending k, as the combine kernel adds
-    p.out[(uint64_t)t * p.N + n0 + tid] = __float2half(acc);
+    p.out[(uint64_t)t * p.N + blockIdx.x * RW + tid] = __float2half(acc);
   }
 }
 
@@ -1101,7 +1117,10 @@ namespace {
 template <int BITS, int GS>
 void launch_down_combine(const M1DownParams& p, int chunks, uint32_t T, hipStream_t stream) {
   // (four rows per wave: the weights of a pass fit the registers of two workgroups per CU)
-  if (chunks == 1) hipLaunchKernelGGL((qmv_m1_down_combine_kernel<BITS, GS, 1, 4>), dim3(p.N / 4, T), dim3(kThreads), 0, stream, p);
+  // (short rows, N in whole blocks of 8: two groups of four rows per wave)
+  if (chunks == 1 && p.K * BITS / 8 <= 512 && p.N % 8 == 0)
+    hipLaunchKernelGGL((qmv_m1_down_combine_kernel<BITS, GS, 1, 4, true>), dim3(p.N / 8, T), dim3(kThreads), 0, stream, p);
+  else if (chunks == 1) hipLaunchKernelGGL((qmv_m1_down_combine_kernel<BITS, GS, 1, 4>), dim3(p.N / 4, T), dim3(kThreads), 0, stream, p);
   else hipLaunchKernelGGL((qmv_m1_down_combine_kernel<BITS, GS, 2, 4>), dim3(p.N / 4, T), dim3(kThreads), 0, stream, p);
 }
 }  // namespace
