@@ -47,6 +47,36 @@ def test_noalloc_matches_the_pooled_entry_point_on_two_calls_in_a_row(hip):
         assert_close(got, model.moe_forward(x, idx, w, gate, up, down, 64, K), f"oracle T={T}")
 
 
+def test_noalloc_with_the_gate_up_projection_in_two_launches(hip):
+    """Between 6 rows per expert on average and the grouped GEMM's threshold, experts of config-5 size run the gate / up
+    projection in two launches over two more chunk tables: those come from the workspace too.  Bit-identical to the pooled
+    entry point, against the oracle on the first tokens, and again with a smaller batch behind it."""
+    from rmlx_amd import ops
+    rng = np.random.default_rng(81)
+    E, D, I, K = 48, 4096, 1536, 8
+    one = _experts(rng, 1, D, I)
+
+    def tiled(a):  # (one random expert repeated: the routing still spreads the rows over all of them)
+        return np.ascontiguousarray(np.broadcast_to(a, (E,) + a.shape[1:]))
+
+    gate, up, down = (tuple(tiled(a) for a in t) for t in one[:3])
+    gu = tuple(np.concatenate([g, u], axis=1) for g, u in zip(gate, up))
+    gh, dh = ops.QuantizedWeight.from_numpy(*gu, 64, 4), ops.QuantizedWeight.from_numpy(*down, 64, 4)
+    for T in (40, 37):  # 6.7 and 6.2 rows per expert
+        x = make_x(rng, T, D)
+        logits = rng.standard_normal((T, E)).astype(np.float32)
+        print(f"noalloc split gate / up T={T}", flush=True)
+        want, got = _both(gh, dh, x, logits, K)
+        assert np.array_equal(want.view(np.uint16), got.view(np.uint16)), f"T={T}"
+        idx, w, _, _ = model.topk_route(logits, K)
+        assert_close(got[:2], model.moe_forward(x[:2], idx[:2 * K], w[:2 * K], gate, up, down, 64, K), f"oracle T={T}")
+        prev = gh.set_expert_stream_kernel(4)  # the same batch with one gate / up launch: both sides pass the oracle
+        try:
+            assert_close(_both(gh, dh, x, logits, K)[1][:2], model.moe_forward(x[:2], idx[:2 * K], w[:2 * K], gate, up, down, 64, K), "one launch")
+        finally:
+            gh.set_expert_stream_kernel(prev)
+
+
 def test_noalloc_allocates_nothing(hip):
     """What the entry point is for: with the default stream's pool emptied first, a pooled call has to allocate and
     the call over the static workspace does not - for every dtype combination that carves casts from the workspace."""
