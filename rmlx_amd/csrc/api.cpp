@@ -438,10 +438,14 @@ int32_t run_matmul_plain(const rmlx_qweight* qw, const void* x, int32_t x_dtype,
     return launch_qmm(a, stream);
   }
 
-  // Activations of the other kernels: f16 (f32 / bf16 are cast first).
+  // Activations of the other kernels: f16 (f32 / bf16 are cast first) -- except that the single-row kernel converts bf16
+  // activations itself while it stages them, for one or two rows in one pass: a decoding step of a bf16 model pays no
+  // cast launch in front of every matmul (same conversion, same bits).
+  const bool m1_bf16 = kernel == KERNEL_QMV && !can_q2 && can_m1 && x_dtype == RMLX_DTYPE_BF16 && norm_w == nullptr &&
+                       qmv_m1_fuses_norm(M, K, qw->bits);
   Scratch cast;
   const void* xk = x;
-  if (x_dtype != RMLX_DTYPE_F16) {
+  if (x_dtype != RMLX_DTYPE_F16 && !m1_bf16) {
     RMLX_TRY(cast.alloc((size_t)M * K * sizeof(__half), stream));
     RMLX_TRY(launch_cast_to_f16(x, x_dtype, static_cast<__half*>(cast.ptr), (size_t)M * K, stream));
     xk = cast.ptr;
@@ -452,7 +456,7 @@ int32_t run_matmul_plain(const rmlx_qweight* qw, const void* x, int32_t x_dtype,
   if (kernel == KERNEL_QMV && can_m1) {
     *epi_done = true;
     return launch_qmv_m1(qw->w, qw->s, qw->b, static_cast<const __half*>(xk), out, M, N, K, qw->group_size, qw->bits,
-                         epi.kind, epi.ptr, epi.dtype, norm_w, norm_w != nullptr ? inv_rms : nullptr, stream);
+                         epi.kind, epi.ptr, epi.dtype, norm_w, norm_w != nullptr ? inv_rms : nullptr, stream, m1_bf16 ? 1 : 0);
   }
   if (kernel == KERNEL_QMV_ROWS && can_wt32) {
     QmvArgs a{};
@@ -1530,7 +1534,9 @@ int32_t moe_grouped_impl(const rmlx_qweight* gate, const rmlx_qweight* up, const
 
   Scratch cast, meta, h, y;
   const __half* xk = static_cast<const __half*>(x->data);
-  if (x->dtype != RMLX_DTYPE_F16) {
+  // (the form without grouping converts bf16 activations itself while it stages them: no cast launch in a decoding step)
+  const bool direct_bf16 = direct && x->dtype == RMLX_DTYPE_BF16;
+  if (x->dtype != RMLX_DTYPE_F16 && !direct_bf16) {
     RMLX_TRY(cast.alloc(T * sh.D * 2, s, arena));
     RMLX_TRY(launch_cast_to_f16(x->data, x->dtype, static_cast<__half*>(cast.ptr), T * sh.D, s));
     xk = static_cast<const __half*>(cast.ptr);
@@ -1547,6 +1553,7 @@ int32_t moe_grouped_impl(const rmlx_qweight* gate, const rmlx_qweight* up, const
     // ranks its token's experts itself, one wave, while the activations arrive (1 / 2 / 4 tokens of 8 picks: 23.4 / 37.0 /
     // 59.5 us against 24.4 / 37.8 / 61.0 us with a routing launch in front).
     QmvArgs a = gate_up_args(gate, up, sh, xk, static_cast<__half*>(h.ptr));
+    a.x_bf16 = direct_bf16 ? 1 : 0;
     if (route != nullptr) {
       a.route_logits = route->logits; a.route_bias = route->bias; a.route_idx_out = route->idx_out; a.route_w_out = route->w_out;
       a.route_renorm = 1;

@@ -144,6 +144,7 @@ struct QmvArgs {
   // [T, n_experts] (+ optional bias) and also write the picks and normalised weights to route_idx_out / route_w_out
   const float* route_logits; const float* route_bias; uint32_t* route_idx_out; float* route_w_out;
   int32_t route_renorm;
+  int32_t x_bf16;  // launch_qmv_m1_gate_up only: x holds bf16 bits, converted to f16 while they are staged
 };
 int32_t launch_qmv_q4(const QmvArgs& a, hipStream_t s);
 bool qmv_q4_supported(uint32_t N, uint32_t K, uint32_t group_size);
@@ -191,7 +192,8 @@ int32_t launch_qmv_q8_tab(const QmvArgs& a, hipStream_t stream);
 bool qmv_m1_supported(uint32_t N, uint32_t K, uint32_t group_size, uint32_t bits);
 int32_t launch_qmv_m1(const uint32_t* w, const __half* s, const __half* b, const __half* x, __half* out, uint32_t M,
                       uint32_t N, uint32_t K, uint32_t group_size, uint32_t bits, int epi_kind, const void* epi,
-                      int32_t epi_dtype, const __half* norm_w, const float* inv_rms, hipStream_t stream);
+                      int32_t epi_dtype, const __half* norm_w, const float* inv_rms, hipStream_t stream,
+                      int32_t x_bf16 = 0);  // 1: x holds bf16 bits, converted while staged (M <= 2 in one pass, no norm prologue)
 bool qmv_m1_fuses_norm(uint32_t M, uint32_t K, uint32_t bits);
 // Single-row GEMV for 2-bit weights (qmv_q2.hip): group size 32 / 64 / 128, f16 activations, one activation row per
 // pass over the weights (grid.y = M), f16 out

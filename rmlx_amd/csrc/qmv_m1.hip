@@ -64,6 +64,7 @@ struct M1Params {
   // (gather_div consecutive rows share an index: row m of this launch, which starts at row gather_row0 of the call, takes
   // gather_idx[(gather_row0 + m) / gather_div]; 0 or 1 = an index per row)
   uint32_t gather_div = 1, gather_row0 = 0;
+  int32_t x_bf16 = 0;  // the activations are bf16 bits (kernels built with the conversion prologue only, see launch_r)
 };
 
 __device__ __forceinline__ h2 as_h2(uint32_t v) { return __builtin_bit_cast(h2, v); }
@@ -132,9 +133,24 @@ __device__ __forceinline__ u4 normalise_unit(const __half* norm_w, const float* 
   return __builtin_bit_cast(u4, scaled * nw);
 }
 
+// Prologue kinds of the activation staging (the NORM template parameter): none, the RMSNorm prologue, bf16 activations
+// converted to f16 on the way (through f32, rounded to nearest even: what the separate cast kernel does).
+constexpr int kPrologueNone = 0, kPrologueNorm = 1, kPrologueBf16 = 2;
+
+__device__ __forceinline__ u4 bf16_unit_to_f16(u4 v) {
+  uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    const float lo = __uint_as_float(w[e] << 16), hi = __uint_as_float(w[e] & 0xFFFF0000u);
+    const h2 pair = {(_Float16)lo, (_Float16)hi};
+    w[e] = __builtin_bit_cast(uint32_t, pair);
+  }
+  return (u4){w[0], w[1], w[2], w[3]};
+}
+
 // 1. The activation loads of a workgroup (the first four rounds of 512 units; issued before the weight loads
 //    because the memory counter retires in order), normalised on the way when NORM.  Rows past M repeat the last one.
-template <int BITS, int MR, bool NORM>
+template <int BITS, int MR, int NORM>
 __device__ __forceinline__ void load_activations(const XImage<BITS, MR> g, const __half* x, uint32_t M, uint32_t mrow0,
                                                  const __half* norm_w, const float* inv_rms, int tid, u4 (&xv)[MR][4]) {
   const uint32_t nunits = g.nunits;
@@ -153,7 +169,13 @@ __device__ __forceinline__ void load_activations(const XImage<BITS, MR> g, const
       }
     }
   }
-  if constexpr (NORM) {
+  if constexpr (NORM == kPrologueBf16) {
+#pragma unroll
+    for (int m = 0; m < MR; ++m)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) xv[m][i] = bf16_unit_to_f16(xv[m][i]);
+  }
+  if constexpr (NORM == kPrologueNorm) {
 #pragma unroll
     for (int m = 0; m < MR; ++m) {
       const uint32_t rm = mrow0 + m < M ? mrow0 + m : M - 1;
@@ -167,7 +189,7 @@ __device__ __forceinline__ void load_activations(const XImage<BITS, MR> g, const
 
 // 2. Stage x: unit u = 8 consecutive k = (chunk, lane, j); image in the order a wave reads it, per-lane sums
 //    beside it.  The caller puts the workgroup barrier behind it.
-template <int BITS, int MR, bool NORM>
+template <int BITS, int MR, int NORM>
 __device__ __forceinline__ void stage_activations(const XImage<BITS, MR> g, const __half* x, uint32_t M, uint32_t mrow0,
                                                   const __half* norm_w, const float* inv_rms, int tid,
                                                   const u4 (&xv)[MR][4]) {
@@ -208,7 +230,8 @@ __device__ __forceinline__ void stage_activations(const XImage<BITS, MR> g, cons
     for (int m = 0; m < MR; ++m) {
       const uint32_t rm = mrow0 + m < M ? mrow0 + m : M - 1;
       u4 v = reinterpret_cast<const u4*>(x + (uint64_t)rm * g.K)[u < nunits ? u : nunits - 1];
-      if constexpr (NORM) v = normalise_unit(norm_w, inv_rms, rm, u, nunits, v);
+      if constexpr (NORM == kPrologueBf16) v = bf16_unit_to_f16(v);
+      if constexpr (NORM == kPrologueNorm) v = normalise_unit(norm_w, inv_rms, rm, u, nunits, v);
       stage_unit(m, u, v);
     }
   }
@@ -295,7 +318,7 @@ __device__ __forceinline__ void dot_chunk(const XImage<BITS, MR> g, uint32_t c, 
 // meet in workgroup memory.  For long rows of a short matrix, where one wave per row leaves most of the chip idle.
 // GATHER = a weight matrix per activation row (gather_qmm with one row per index: the counterpart of
 // gather_qmv_fast_f16_q4, quantized.rs:9752-9842); MR = 1.
-template <int BITS, int GS, int R, bool NT, int MR, bool NORM = false, int KP = 1, bool GATHER = false>
+template <int BITS, int GS, int R, bool NT, int MR, int NORM = 0, int KP = 1, bool GATHER = false>
 // (8-bit, one row: asking the compiler for eight waves per SIMD changes no register count but the schedule;
 // measured 4-13 % faster.  The 4-bit kernel would spill under that bound and is slower with it.  Two activation
 // rows: without a bound the scheduler spends 124 registers on a schedule that is 12 % slower than the one it finds
@@ -433,7 +456,7 @@ __global__ __launch_bounds__(kThreads, (BITS == 8 && MR == 1 && R == 1) ? 8 : (M
 
 // The same kernel for matrices with more row blocks than the chip keeps resident: the grid is sized to the resident
 // workgroups and each of them walks several row blocks (see `my_blocks`).
-template <int BITS, int GS, int R, bool NT, int MR, bool NORM = false, bool GATHER = false>
+template <int BITS, int GS, int R, bool NT, int MR, int NORM = 0, bool GATHER = false>
 // (8-bit, one row: asking the compiler for eight waves per SIMD changes no register count but the schedule;
 // measured 4-13 % faster.  The 4-bit kernel would spill under that bound and is slower with it.)
 __global__ __launch_bounds__(kThreads, 1) void qmv_m1_loop_kernel(M1Params p) {
@@ -614,7 +637,7 @@ __device__ __forceinline__ uint32_t gate_up_expert(const M1GateUpParams& p, uint
   return pick_idx[pick];
 }
 
-template <int BITS, int GS>
+template <int BITS, int GS, bool XBF = false>  // XBF: the activations are bf16 bits, converted while they are staged
 __global__ __launch_bounds__(kThreads, 1) void qmv_m1_gate_up_kernel(M1GateUpParams p) {
   using Image = XImage<BITS, 1>;
   constexpr int kChunkK = Image::kChunkK, kLaneK = Image::kLaneK;
@@ -628,7 +651,7 @@ __global__ __launch_bounds__(kThreads, 1) void qmv_m1_gate_up_kernel(M1GateUpPar
 
   // loads, small ones first (the memory counter retires in order): the activations, the expert, then the rows
   u4 xv[1][4];
-  load_activations<BITS, 1, false>(img, x, 1u, 0u, nullptr, nullptr, tid, xv);
+  load_activations<BITS, 1, XBF ? kPrologueBf16 : kPrologueNone>(img, x, 1u, 0u, nullptr, nullptr, tid, xv);
   uint32_t expert = gate_up_expert(p, a, blockIdx.x == 0);
   const bool zeros = expert >= p.n_experts;
   expert = zeros ? 0u : expert;
@@ -660,7 +683,7 @@ __global__ __launch_bounds__(kThreads, 1) void qmv_m1_gate_up_kernel(M1GateUpPar
   };
   Batch ba, bb;
   load_batch(0, ba);
-  stage_activations<BITS, 1, false>(img, x, 1u, 0u, nullptr, nullptr, tid, xv);
+  stage_activations<BITS, 1, XBF ? kPrologueBf16 : kPrologueNone>(img, x, 1u, 0u, nullptr, nullptr, tid, xv);
   __syncthreads();
 
   float racc[2][1] = {{0.f}, {0.f}};
@@ -687,7 +710,7 @@ __global__ __launch_bounds__(kThreads, 1) void qmv_m1_gate_up_kernel(M1GateUpPar
 // The same for more row blocks than the chip keeps resident (a few tokens: assignments x N / 8 blocks): the grid is
 // (resident workgroups / assignments, assignments) and a workgroup walks the row blocks blockIdx.x, blockIdx.x + gridDim.x,
 // ... of its assignment, staging the activations once, the next block's weights in flight while the current one is multiplied.
-template <int BITS, int GS>
+template <int BITS, int GS, bool XBF = false>
 __global__ __launch_bounds__(kThreads, 1) void qmv_m1_gate_up_loop_kernel(M1GateUpParams p) {
   using Image = XImage<BITS, 1>;
   constexpr int kChunkK = Image::kChunkK, kLaneK = Image::kLaneK;
@@ -703,7 +726,7 @@ __global__ __launch_bounds__(kThreads, 1) void qmv_m1_gate_up_loop_kernel(M1Gate
   auto block_row = [&](uint32_t i) { return (blockIdx.x + i * gridDim.x) * kWaves + wave; };
 
   u4 xv[1][4];
-  load_activations<BITS, 1, false>(img, x, 1u, 0u, nullptr, nullptr, tid, xv);
+  load_activations<BITS, 1, XBF ? kPrologueBf16 : kPrologueNone>(img, x, 1u, 0u, nullptr, nullptr, tid, xv);
   uint32_t expert = gate_up_expert(p, a, blockIdx.x == 0);
   const bool zeros = expert >= p.n_experts;
   expert = zeros ? 0u : expert;
@@ -740,7 +763,7 @@ __global__ __launch_bounds__(kThreads, 1) void qmv_m1_gate_up_loop_kernel(M1Gate
   };
   Batch ba, bb;
   if (n_batches > 0) load_batch(ba);
-  stage_activations<BITS, 1, false>(img, x, 1u, 0u, nullptr, nullptr, tid, xv);
+  stage_activations<BITS, 1, XBF ? kPrologueBf16 : kPrologueNone>(img, x, 1u, 0u, nullptr, nullptr, tid, xv);
   __syncthreads();
 
   float racc[2][1];
@@ -902,7 +925,7 @@ uint32_t resident_workgroups(Kernel kernel, size_t lds) {
   return wgs;
 }
 
-template <int BITS, int GS, int R, bool NT, int MR, bool NORM, int KP = 1, bool GATHER = false>
+template <int BITS, int GS, int R, bool NT, int MR, int NORM, int KP = 1, bool GATHER = false>
 void launch_k(const M1Params& p, size_t lds, hipStream_t s) {
   if constexpr (KP > 1) {  // split rows: short matrices only, every row group has its workgroup
     hipLaunchKernelGGL((qmv_m1_kernel<BITS, GS, R, NT, MR, NORM, KP>), dim3(p.N / (kWaves / KP), (p.M + MR - 1) / MR),
@@ -931,20 +954,28 @@ void launch_r(const M1Params& p, uint32_t group_size, hipStream_t s) {
     }
     return;
   }
-  if constexpr (NT && MR <= 2) {  // the prologue is fused for one or two rows in one pass
+  if constexpr (NT && MR <= 2) {  // the prologues are fused for one or two rows in one pass
     if (p.norm_w != nullptr) {
       switch (group_size) {
-        case 32: launch_k<BITS, 32, R, NT, MR, true>(p, lds, s); break;
-        case 64: launch_k<BITS, 64, R, NT, MR, true>(p, lds, s); break;
-        default: launch_k<BITS, 128, R, NT, MR, true>(p, lds, s); break;
+        case 32: launch_k<BITS, 32, R, NT, MR, kPrologueNorm>(p, lds, s); break;
+        case 64: launch_k<BITS, 64, R, NT, MR, kPrologueNorm>(p, lds, s); break;
+        default: launch_k<BITS, 128, R, NT, MR, kPrologueNorm>(p, lds, s); break;
+      }
+      return;
+    }
+    if (p.x_bf16) {
+      switch (group_size) {
+        case 32: launch_k<BITS, 32, R, NT, MR, kPrologueBf16>(p, lds, s); break;
+        case 64: launch_k<BITS, 64, R, NT, MR, kPrologueBf16>(p, lds, s); break;
+        default: launch_k<BITS, 128, R, NT, MR, kPrologueBf16>(p, lds, s); break;
       }
       return;
     }
   }
   switch (group_size) {
-    case 32: launch_k<BITS, 32, R, NT, MR, false>(p, lds, s); break;
-    case 64: launch_k<BITS, 64, R, NT, MR, false>(p, lds, s); break;
-    default: launch_k<BITS, 128, R, NT, MR, false>(p, lds, s); break;
+    case 32: launch_k<BITS, 32, R, NT, MR, kPrologueNone>(p, lds, s); break;
+    case 64: launch_k<BITS, 64, R, NT, MR, kPrologueNone>(p, lds, s); break;
+    default: launch_k<BITS, 128, R, NT, MR, kPrologueNone>(p, lds, s); break;
   }
 }
 
@@ -974,7 +1005,7 @@ void launch_bits(const M1Params& p, uint32_t group_size, hipStream_t s) {
     const uint32_t chunks = (p.K * BITS + 8191) / 8192, cus = (uint32_t)ctx().num_cus;
     int kp = 1;
     while (kp < 4 && p.N / kWaves * kp < 2 * cus && chunks >= 4u * kp && p.N % (kWaves / (2 * kp)) == 0) kp *= 2;
-    if (kp > 1 && p.norm_w == nullptr && one_pass) {
+    if (kp > 1 && p.norm_w == nullptr && !p.x_bf16 && one_pass) {
       if (kp == 2) launch_r<BITS, 1, true, 1, 2>(p, group_size, s); else launch_r<BITS, 1, true, 1, 4>(p, group_size, s);
       return;
     }
@@ -1003,14 +1034,17 @@ bool qmv_m1_fuses_norm(uint32_t M, uint32_t K, uint32_t bits) {
 
 int32_t launch_qmv_m1(const uint32_t* w, const __half* s, const __half* b, const __half* x, __half* out, uint32_t M,
                       uint32_t N, uint32_t K, uint32_t group_size, uint32_t bits, int epi_kind, const void* epi,
-                      int32_t epi_dtype, const __half* norm_w, const float* inv_rms, hipStream_t stream) {
+                      int32_t epi_dtype, const __half* norm_w, const float* inv_rms, hipStream_t stream, int32_t x_bf16) {
   if (!qmv_m1_supported(N, K, group_size, bits))
     return fail(RMLX_INVALID_SHAPE, "qmv_m1: unsupported shape N=%u K=%u bits=%u group_size=%u", N, K, bits, group_size);
+  if (x_bf16 && (norm_w != nullptr || !qmv_m1_fuses_norm(M, K, bits)))
+    return fail(RMLX_RUNTIME_ERROR, "qmv_m1: bf16 activations are converted inside for at most two rows in one pass and without the RMSNorm prologue (M=%u K=%u)", M, K);
   if (M == 0) return RMLX_OK;
   if (M > 65535) return fail(RMLX_INVALID_SHAPE, "qmv_m1: at most 65535 rows per launch (M=%u)", M);
   if (norm_w != nullptr && !qmv_m1_fuses_norm(M, K, bits))
     return fail(RMLX_RUNTIME_ERROR, "qmv_m1: the RMSNorm prologue is fused for at most two rows in one pass (M=%u K=%u)", M, K);
   M1Params p{w, s, b, x, out, N, K, M, epi_kind, epi_dtype, epi, norm_w, inv_rms};
+  p.x_bf16 = x_bf16;
   if (bits == 4) launch_bits<4>(p, group_size, stream);
   else launch_bits<8>(p, group_size, stream);
   RMLX_HIP_CHECK(hipGetLastError());
@@ -1055,16 +1089,21 @@ bool qmv_m1_gate_up_supported(uint32_t N, uint32_t K, uint32_t group_size, uint3
 }
 
 namespace {
-template <int BITS, int GS>
-void launch_gate_up(const M1GateUpParams& p, uint32_t assignments, hipStream_t stream) {
+template <int BITS, int GS, bool XBF>
+void launch_gate_up_x(const M1GateUpParams& p, uint32_t assignments, hipStream_t stream) {
   const size_t lds = lds_per_row<BITS>(p.K);
   const uint32_t nblk = p.N / kWaves;
   // one workgroup per row block while all of them are resident together, else as many as are (they loop)
-  auto looping = qmv_m1_gate_up_loop_kernel<BITS, GS>;
+  auto looping = qmv_m1_gate_up_loop_kernel<BITS, GS, XBF>;
   uint32_t gx = resident_workgroups(looping, lds) / assignments;
   gx = gx < 1 ? 1 : gx;
   if (gx < nblk) hipLaunchKernelGGL(looping, dim3(gx, assignments), dim3(kThreads), lds, stream, p);
-  else hipLaunchKernelGGL((qmv_m1_gate_up_kernel<BITS, GS>), dim3(nblk, assignments), dim3(kThreads), lds, stream, p);
+  else hipLaunchKernelGGL((qmv_m1_gate_up_kernel<BITS, GS, XBF>), dim3(nblk, assignments), dim3(kThreads), lds, stream, p);
+}
+template <int BITS, int GS>
+void launch_gate_up(const M1GateUpParams& p, uint32_t assignments, bool x_bf16, hipStream_t stream) {
+  if (x_bf16) launch_gate_up_x<BITS, GS, true>(p, assignments, stream);
+  else launch_gate_up_x<BITS, GS, false>(p, assignments, stream);
 }
 }  // namespace
 
@@ -1084,15 +1123,15 @@ int32_t launch_qmv_m1_gate_up(const QmvArgs& a, uint32_t bits, const uint32_t* i
                    a.route_logits, a.route_bias, a.route_idx_out, a.route_w_out, a.route_renorm};
   if (bits == 4) {
     switch (a.group_size) {
-      case 32: launch_gate_up<4, 32>(p, assignments, stream); break;
-      case 64: launch_gate_up<4, 64>(p, assignments, stream); break;
-      default: launch_gate_up<4, 128>(p, assignments, stream); break;
+      case 32: launch_gate_up<4, 32>(p, assignments, a.x_bf16 != 0, stream); break;
+      case 64: launch_gate_up<4, 64>(p, assignments, a.x_bf16 != 0, stream); break;
+      default: launch_gate_up<4, 128>(p, assignments, a.x_bf16 != 0, stream); break;
     }
   } else {
     switch (a.group_size) {
-      case 32: launch_gate_up<8, 32>(p, assignments, stream); break;
-      case 64: launch_gate_up<8, 64>(p, assignments, stream); break;
-      default: launch_gate_up<8, 128>(p, assignments, stream); break;
+      case 32: launch_gate_up<8, 32>(p, assignments, a.x_bf16 != 0, stream); break;
+      case 64: launch_gate_up<8, 64>(p, assignments, a.x_bf16 != 0, stream); break;
+      default: launch_gate_up<8, 128>(p, assignments, a.x_bf16 != 0, stream); break;
     }
   }
   RMLX_HIP_CHECK(hipGetLastError());

@@ -1029,6 +1029,29 @@ def test_one_and_two_rows_over_short_rows_of_tall_matrices(hip, bits, n, k):
         assert np.array_equal(auto.view(np.uint16), single.view(np.uint16)) or np.array_equal(auto.view(np.uint16), rows.view(np.uint16))
 
 
+@pytest.mark.parametrize("bits,gs,n,k", [(4, 64, 4096, 4096), (8, 64, 512, 2048), (4, 32, 256, 1152), (4, 128, 4096, 18944), (8, 128, 4096, 2560)])
+def test_bf16_rows_are_converted_inside_the_single_row_kernel(hip, bits, gs, n, k):
+    """One or two bf16 activation rows: the single-row kernel converts them to f16 while it stages them (no cast launch in
+    front of a decoding step's matmuls).  Bit-identical to the same matmul over the rows converted on the host the way
+    the cast kernel does (through f32, round to nearest even), and on the oracle; with a fused epilogue as well."""
+    from rmlx_amd import ops
+    from rmlx_amd.runtime import DeviceBuffer
+    rng = np.random.default_rng(bits + gs + n + k)
+    words, s, b = make_weight(rng, n, k, bits, gs)
+    qw = ops.QuantizedWeight.from_numpy(words, s, b, gs, bits)
+    for m in (1, 2):
+        x = make_x(rng, m, k, "bf16")
+        x16 = model.bf16_bits_to_f32(x).astype(np.float16)
+        got = _run(hip, words, s, b, x, bits, gs=gs, dtype="bf16")
+        want = _run(hip, words, s, b, x16, bits, gs=gs)
+        assert np.array_equal(got.view(np.uint16), want.view(np.uint16)), (m, n, k)
+        assert_close(got, model.qmm(x_as_f64(x, "bf16"), words, s, b, gs, bits), f"bf16 M={m} N={n} K={k} Q{bits} gs={gs}")
+        e = rng.standard_normal((m, n)).astype(np.float16)
+        res = ops.qmm_add_residual(_dev(hip, x, "bf16"), qw, DeviceBuffer.from_numpy(e)).numpy()
+        res16 = ops.qmm_add_residual(DeviceBuffer.from_numpy(x16), qw, DeviceBuffer.from_numpy(e)).numpy()
+        assert np.array_equal(res.view(np.uint16), res16.view(np.uint16))
+
+
 def test_random_shapes_through_the_ladder(hip):
     """Sixty seeded random (M, N, K, bits, group size) shapes through the automatic dispatch: whatever kernel
     the ladder picks (single-row, multi-row GEMV, both GEMMs, portable) must land on the oracle."""

@@ -581,6 +581,34 @@ def test_moe_forward_of_dimensions_in_whole_blocks_of_128(hip, bits, gs, D, I, T
             assert_close(out, ref, f"moe_forward_grouped min_rows={min_rows} stream kernel {kind}")
 
 
+@pytest.mark.parametrize("bits,gs,D,I", [(4, 64, 1024, 512), (8, 64, 512, 768), (4, 32, 512, 640)])
+@pytest.mark.parametrize("T", [1, 3, 40])
+def test_moe_forward_of_bf16_activations(hip, bits, gs, D, I, T):
+    """bf16 activations: a few tokens are converted inside the gate / up kernel of the form without grouping while it stages
+    them (no cast launch), larger batches by a cast in front.  Bit-identical to the same call over the rows converted on the
+    host (through f32, round to nearest even), and on the oracle."""
+    from rmlx_amd import ops
+    from rmlx_amd.runtime import BF16, DeviceBuffer
+    rng = np.random.default_rng(bits + gs + D + I + T)
+    E, K = 8, 2
+    gu = make_weight(rng, 2 * I, D, bits, gs, lead=(E,))
+    down = make_weight(rng, D, I, bits, gs, lead=(E,))
+    gate, up = tuple(a[:, :I] for a in gu), tuple(a[:, I:] for a in gu)
+    gh, dh = ops.QuantizedWeight.from_numpy(*gu, gs, bits), ops.QuantizedWeight.from_numpy(*down, gs, bits)
+    xb = make_x(rng, T, D, "bf16")
+    x16 = model.bf16_bits_to_f32(xb).astype(np.float16)
+    logits = rng.standard_normal((T, E)).astype(np.float32)
+    idx, w, _, _ = model.topk_route(logits, K)
+    ld = DeviceBuffer.from_numpy(logits)
+    print(f"moe bf16 Q{bits} gs{gs} D={D} I={I} T={T}", flush=True)
+    got = ops.moe_forward(gh, None, dh, DeviceBuffer.from_numpy(xb, BF16), ld, K).numpy()
+    want = ops.moe_forward(gh, None, dh, DeviceBuffer.from_numpy(x16), ld, K).numpy()
+    assert np.array_equal(got.view(np.uint16), want.view(np.uint16))
+    assert_close(got, model.moe_forward(x16, idx, w, gate, up, down, gs, K, bits=bits), "bf16 activations")
+    got2 = ops.moe_forward_grouped(gh, None, dh, DeviceBuffer.from_numpy(xb, BF16), DeviceBuffer.from_numpy(idx), DeviceBuffer.from_numpy(w), K).numpy()
+    assert np.array_equal(got2.view(np.uint16), want.view(np.uint16))
+
+
 @pytest.mark.parametrize("T,K", [(1, 2), (1, 8), (2, 3), (3, 4)])
 def test_moe_forward_grouped_with_repeated_experts(hip, T, K):
     """Caller-supplied picks may name one expert several times for a token; decode-sized batches run kernels
