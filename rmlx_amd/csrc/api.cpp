@@ -443,9 +443,12 @@ int32_t run_matmul_plain(const rmlx_qweight* qw, const void* x, int32_t x_dtype,
   // cast launch in front of every matmul (same conversion, same bits).
   const bool m1_bf16 = kernel == KERNEL_QMV && !can_q2 && can_m1 && x_dtype == RMLX_DTYPE_BF16 && norm_w == nullptr &&
                        qmv_m1_fuses_norm(M, K, qw->bits);
+  // (so does the 4-bit multi-row GEMV, for every row count it takes)
+  const bool rows_bf16 = x_dtype == RMLX_DTYPE_BF16 && qw->bits == 4 && can_qmv && !can_q2 &&
+                         ((kernel == KERNEL_QMV && !can_m1) || (kernel == KERNEL_QMV_ROWS && !can_wt32));
   Scratch cast;
   const void* xk = x;
-  if (x_dtype != RMLX_DTYPE_F16 && !m1_bf16) {
+  if (x_dtype != RMLX_DTYPE_F16 && !m1_bf16 && !rows_bf16) {
     RMLX_TRY(cast.alloc((size_t)M * K * sizeof(__half), stream));
     RMLX_TRY(launch_cast_to_f16(x, x_dtype, static_cast<__half*>(cast.ptr), (size_t)M * K, stream));
     xk = cast.ptr;
@@ -475,6 +478,7 @@ int32_t run_matmul_plain(const rmlx_qweight* qw, const void* x, int32_t x_dtype,
     a.N = N; a.K = K;
     a.x = static_cast<const __half*>(xk);
     a.out = out; a.ld_out = N; a.M = M; a.group_size = qw->group_size;
+    a.x_bf16 = rows_bf16 ? 1 : 0;
     return launch_qmv_q4(a, stream);
   }
   GenericArgs g{qw->w, qw->s, qw->b, static_cast<const __half*>(xk), out, nullptr, 0, M, N, K,

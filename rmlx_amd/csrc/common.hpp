@@ -144,7 +144,7 @@ struct QmvArgs {
   // [T, n_experts] (+ optional bias) and also write the picks and normalised weights to route_idx_out / route_w_out
   const float* route_logits; const float* route_bias; uint32_t* route_idx_out; float* route_w_out;
   int32_t route_renorm;
-  int32_t x_bf16;  // launch_qmv_m1_gate_up only: x holds bf16 bits, converted to f16 while they are staged
+  int32_t x_bf16;  // launch_qmv_m1_gate_up and launch_qmv_q4: x holds bf16 bits, converted to f16 while they are staged
 };
 int32_t launch_qmv_q4(const QmvArgs& a, hipStream_t s);
 bool qmv_q4_supported(uint32_t N, uint32_t K, uint32_t group_size);

@@ -43,6 +43,19 @@ __device__ __forceinline__ u4 permute_x8(u4 d) {
   return o;
 }
 
+// 8 bf16 values -> 8 f16 values through f32, rounded to nearest even (what the cast kernel does)
+__device__ __forceinline__ u4 bf16x8_to_f16(u4 v) {
+  typedef _Float16 h2c __attribute__((ext_vector_type(2)));
+  uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    const float lo = __uint_as_float(w[e] << 16), hi = __uint_as_float(w[e] & 0xFFFF0000u);
+    const h2c pair = {(_Float16)lo, (_Float16)hi};
+    w[e] = __builtin_bit_cast(uint32_t, pair);
+  }
+  return (u4){w[0], w[1], w[2], w[3]};
+}
+
 __device__ __forceinline__ float silu_f(float v) { return v / (1.0f + __expf(-v)); }
 
 __device__ __forceinline__ uint32_t swap16(uint32_t v) {  // value of lane ^ 16

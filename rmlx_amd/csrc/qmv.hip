@@ -67,6 +67,7 @@ struct KParams {
   const uint32_t* chunk_tab;
   const uint32_t* n_chunks;
   uint64_t estride_w, estride_s;
+  uint32_t x_bf16;  // x holds bf16 bits: converted to f16 while the activations are staged
 };
 
 
@@ -158,6 +159,12 @@ __global__ __launch_bounds__(kThreads, (REUSE != 0 && MR == 8 && TILES == 2) ? 4
   // this wave's activations -> its LDS image in operand order
   auto stage_x = [&](const u4 (&xv)[MR]) {
     const int ls = lane >> 4, gg = (lane >> 2) & 3, j = lane & 3;
+    if (p.x_bf16) {  // (wave-uniform; the f16 path pays a scalar compare)
+#pragma unroll
+      for (int m = 0; m < MR; ++m)
+        *reinterpret_cast<u4*>(xs + ((ls * 4 + j) * kBlk + gg * MR + m) * 16) = permute_x8(bf16x8_to_f16(xv[m]));
+      return;
+    }
 #pragma unroll
     for (int m = 0; m < MR; ++m)
       *reinterpret_cast<u4*>(xs + ((ls * 4 + j) * kBlk + gg * MR + m) * 16) = permute_x8(xv[m]);
@@ -554,6 +561,7 @@ int32_t launch_qmv_q4(const QmvArgs& a, hipStream_t s) {
   p.out = a.out; p.estride_w = a.expert_stride_w; p.estride_s = a.expert_stride_s;
   p.K = a.K; p.ld_out = a.ld_out; p.M = a.M; p.out_f32 = a.out_f32;
   p.gs128 = a.group_size == 128 ? 1u : 0u;
+  p.x_bf16 = a.x_bf16 ? 1u : 0u;
   const bool tab = a.chunk_tab != nullptr;
   uint32_t chunks = tab ? a.max_chunks : (a.M + 7) / 8;
   if (chunks == 0) return RMLX_OK;
