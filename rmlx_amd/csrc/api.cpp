@@ -443,8 +443,8 @@ int32_t run_matmul_plain(const rmlx_qweight* qw, const void* x, int32_t x_dtype,
   // cast launch in front of every matmul (same conversion, same bits).
   const bool m1_bf16 = kernel == KERNEL_QMV && !can_q2 && can_m1 && x_dtype == RMLX_DTYPE_BF16 && norm_w == nullptr &&
                        qmv_m1_fuses_norm(M, K, qw->bits);
-  // (so does the 4-bit multi-row GEMV, for every row count it takes)
-  const bool rows_bf16 = x_dtype == RMLX_DTYPE_BF16 && qw->bits == 4 && can_qmv && !can_q2 &&
+  // (so do the multi-row GEMVs, for every row count they take)
+  const bool rows_bf16 = x_dtype == RMLX_DTYPE_BF16 && (qw->bits == 4 || qw->bits == 8) && can_qmv && !can_q2 &&
                          ((kernel == KERNEL_QMV && !can_m1) || (kernel == KERNEL_QMV_ROWS && !can_wt32));
   Scratch cast;
   const void* xk = x;
@@ -471,7 +471,7 @@ int32_t run_matmul_plain(const rmlx_qweight* qw, const void* x, int32_t x_dtype,
   }
   if (kernel == KERNEL_QMV_ROWS) kernel = KERNEL_QMV;
   if (kernel == KERNEL_QMV && qw->bits == 8)
-    return launch_qmv_q8(qw->w, qw->s, qw->b, static_cast<const __half*>(xk), out, M, N, K, qw->group_size, stream);
+    return launch_qmv_q8(qw->w, qw->s, qw->b, static_cast<const __half*>(xk), out, M, N, K, qw->group_size, stream, rows_bf16 ? 1 : 0);
   if (kernel == KERNEL_QMV) {
     QmvArgs a{};
     a.w0 = qw->w; a.s0 = qw->s; a.b0 = qw->b;

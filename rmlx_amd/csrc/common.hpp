@@ -184,7 +184,8 @@ int32_t launch_qmv_wt_combine(const uint32_t* w, const __half* s, const __half* 
 // 8-bit streaming GEMV (qmv_q8.hip): f16 activations [M,K], chunks of 16 rows, group size 64 or 128.
 bool qmv_q8_supported(uint32_t N, uint32_t K, uint32_t group_size);
 int32_t launch_qmv_q8(const uint32_t* w, const __half* s, const __half* b, const __half* x, __half* out, uint32_t M,
-                      uint32_t N, uint32_t K, uint32_t group_size, hipStream_t stream);
+                      uint32_t N, uint32_t K, uint32_t group_size, hipStream_t stream,
+                      int32_t x_bf16 = 0);  // 1: x holds bf16 bits, converted in registers
 // chunk-table mode for the expert projections (expert strides in u32 words / halves as for the 4-bit kernel)
 int32_t launch_qmv_q8_tab(const QmvArgs& a, hipStream_t stream);
 // Single-row GEMV (qmv_m1.hip): 4- or 8-bit weights, group size 32 / 64 / 128, f16 activations; M rows are

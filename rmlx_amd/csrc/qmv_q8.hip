@@ -55,7 +55,21 @@ __device__ __forceinline__ h8 bytes_to_f16_plus_1024(uint32_t w0, uint32_t w1) {
 // TAB: rows come from a device chunk table and the weights from the chunk's expert.  TILES == 2: the
 // workgroup multiplies the same activations with a gate tile and an up tile and writes silu(gate) * up.
 // A pass covers 32 slabs (2048 k); waves whose slabs lie past K sit it out, so K % 256 == 0 is enough.
-template <bool TAB, int TILES, bool GS128>
+// XBF: the activations are bf16 bits, converted to f16 in registers (through f32, rounded to nearest even: what the cast
+// kernel does) once the pass's loads are issued.
+__device__ __forceinline__ u4 bf16x8_to_f16x8(u4 v) {
+  typedef _Float16 h2c __attribute__((ext_vector_type(2)));
+  uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    const float lo = __uint_as_float(w[e] << 16), hi = __uint_as_float(w[e] & 0xFFFF0000u);
+    const h2c pair = {(_Float16)lo, (_Float16)hi};
+    w[e] = __builtin_bit_cast(uint32_t, pair);
+  }
+  return (u4){w[0], w[1], w[2], w[3]};
+}
+
+template <bool TAB, int TILES, bool GS128, bool XBF = false>
 __global__ __launch_bounds__(kThreads) void qmv_q8_kernel(Q8Params p) {
   __shared__ float red[kWaves * TILES * 256];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -126,6 +140,10 @@ __global__ __launch_bounds__(kThreads) void qmv_q8_kernel(Q8Params p) {
 #pragma unroll
       for (int t = 0; t < TILES; ++t) wreg[t][it] = wrow[t][(uint64_t)(sl + it) * 4];
 
+    if constexpr (XBF) {
+#pragma unroll
+      for (int it = 0; it < kSpw; ++it) { xa[it][0] = bf16x8_to_f16x8(xa[it][0]); xa[it][1] = bf16x8_to_f16x8(xa[it][1]); }
+    }
     // ---- sum(x) per (row, slab) on the matrix unit while the weights are in flight ---------------
     f4 xs[kSpw];
 #pragma unroll
@@ -191,7 +209,7 @@ bool qmv_q8_supported(uint32_t N, uint32_t K, uint32_t group_size) {
 }
 
 int32_t launch_qmv_q8(const uint32_t* w, const __half* s, const __half* b, const __half* x, __half* out, uint32_t M,
-                      uint32_t N, uint32_t K, uint32_t group_size, hipStream_t stream) {
+                      uint32_t N, uint32_t K, uint32_t group_size, hipStream_t stream, int32_t x_bf16) {
   if (!qmv_q8_supported(N, K, group_size))
     return fail(RMLX_INVALID_SHAPE, "qmv_q8: N %% 16 and K %% 256 required (N=%u K=%u)", N, K);
   if (M == 0) return RMLX_OK;
@@ -200,7 +218,10 @@ int32_t launch_qmv_q8(const uint32_t* w, const __half* s, const __half* b, const
   // (the group size is a template parameter: as a run-time flag inside the pass loop it cost the 64-wide kernel
   // 13 % on decode-sized expert batches)
   const dim3 grid(N / 16, (M + 15) / 16);
-  if (group_size == 128) hipLaunchKernelGGL((qmv_q8_kernel<false, 1, true>), grid, dim3(kThreads), 0, stream, p);
+  if (x_bf16) {
+    if (group_size == 128) hipLaunchKernelGGL((qmv_q8_kernel<false, 1, true, true>), grid, dim3(kThreads), 0, stream, p);
+    else hipLaunchKernelGGL((qmv_q8_kernel<false, 1, false, true>), grid, dim3(kThreads), 0, stream, p);
+  } else if (group_size == 128) hipLaunchKernelGGL((qmv_q8_kernel<false, 1, true>), grid, dim3(kThreads), 0, stream, p);
   else hipLaunchKernelGGL((qmv_q8_kernel<false, 1, false>), grid, dim3(kThreads), 0, stream, p);
   RMLX_HIP_CHECK(hipGetLastError());
   return RMLX_OK;

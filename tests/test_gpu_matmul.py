@@ -1039,7 +1039,7 @@ def test_bf16_rows_are_converted_inside_the_single_row_kernel(hip, bits, gs, n, 
     rng = np.random.default_rng(bits + gs + n + k)
     words, s, b = make_weight(rng, n, k, bits, gs)
     qw = ops.QuantizedWeight.from_numpy(words, s, b, gs, bits)
-    for m in (1, 2, 3, 8, 13, 16):  # (from three rows on: the multi-row GEMV, which converts 4-bit matmuls' rows inside as well)
+    for m in (1, 2, 3, 8, 13, 16):  # (from three rows on: the multi-row GEMVs, which convert inside as well)
         x = make_x(rng, m, k, "bf16")
         x16 = model.bf16_bits_to_f32(x).astype(np.float16)
         got = _run(hip, words, s, b, x, bits, gs=gs, dtype="bf16")
