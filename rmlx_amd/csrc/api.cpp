@@ -441,8 +441,8 @@ int32_t run_matmul_plain(const rmlx_qweight* qw, const void* x, int32_t x_dtype,
   // Activations of the other kernels: f16 (f32 / bf16 are cast first) -- except that the single-row kernel converts bf16
   // activations itself while it stages them, for one or two rows in one pass: a decoding step of a bf16 model pays no
   // cast launch in front of every matmul (same conversion, same bits).
-  const bool m1_bf16 = kernel == KERNEL_QMV && !can_q2 && can_m1 && x_dtype == RMLX_DTYPE_BF16 && norm_w == nullptr &&
-                       qmv_m1_fuses_norm(M, K, qw->bits);
+  const bool m1_bf16 = kernel == KERNEL_QMV && !can_q2 && can_m1 && (x_dtype == RMLX_DTYPE_BF16 || x_dtype == RMLX_DTYPE_F32) &&
+                       norm_w == nullptr && qmv_m1_fuses_norm(M, K, qw->bits);  // (f32 rows likewise)
   // (so do the multi-row GEMVs, for every row count they take)
   const bool rows_bf16 = x_dtype == RMLX_DTYPE_BF16 && (qw->bits == 4 || qw->bits == 8) && can_qmv && !can_q2 &&
                          ((kernel == KERNEL_QMV && !can_m1) || (kernel == KERNEL_QMV_ROWS && !can_wt32));
@@ -459,7 +459,8 @@ int32_t run_matmul_plain(const rmlx_qweight* qw, const void* x, int32_t x_dtype,
   if (kernel == KERNEL_QMV && can_m1) {
     *epi_done = true;
     return launch_qmv_m1(qw->w, qw->s, qw->b, static_cast<const __half*>(xk), out, M, N, K, qw->group_size, qw->bits,
-                         epi.kind, epi.ptr, epi.dtype, norm_w, norm_w != nullptr ? inv_rms : nullptr, stream, m1_bf16 ? 1 : 0);
+                         epi.kind, epi.ptr, epi.dtype, norm_w, norm_w != nullptr ? inv_rms : nullptr, stream,
+                         !m1_bf16 ? 0 : (x_dtype == RMLX_DTYPE_BF16 ? 1 : 2));
   }
   if (kernel == KERNEL_QMV_ROWS && can_wt32) {
     QmvArgs a{};

@@ -194,7 +194,7 @@ bool qmv_m1_supported(uint32_t N, uint32_t K, uint32_t group_size, uint32_t bits
 int32_t launch_qmv_m1(const uint32_t* w, const __half* s, const __half* b, const __half* x, __half* out, uint32_t M,
                       uint32_t N, uint32_t K, uint32_t group_size, uint32_t bits, int epi_kind, const void* epi,
                       int32_t epi_dtype, const __half* norm_w, const float* inv_rms, hipStream_t stream,
-                      int32_t x_bf16 = 0);  // 1: x holds bf16 bits, converted while staged (M <= 2 in one pass, no norm prologue)
+                      int32_t x_bf16 = 0);  // 1: x holds bf16 bits, 2: f32 values; converted while staged (M <= 2 in one pass, no norm prologue)
 bool qmv_m1_fuses_norm(uint32_t M, uint32_t K, uint32_t bits);
 // Single-row GEMV for 2-bit weights (qmv_q2.hip): group size 32 / 64 / 128, f16 activations, one activation row per
 // pass over the weights (grid.y = M), f16 out

@@ -64,7 +64,7 @@ struct M1Params {
   // (gather_div consecutive rows share an index: row m of this launch, which starts at row gather_row0 of the call, takes
   // gather_idx[(gather_row0 + m) / gather_div]; 0 or 1 = an index per row)
   uint32_t gather_div = 1, gather_row0 = 0;
-  int32_t x_bf16 = 0;  // the activations are bf16 bits (kernels built with the conversion prologue only, see launch_r)
+  int32_t x_bf16 = 0;  // 1: the activations are bf16 bits, 2: f32 values (kernels built with the conversion prologues only, see launch_r)
 };
 
 __device__ __forceinline__ h2 as_h2(uint32_t v) { return __builtin_bit_cast(h2, v); }
@@ -135,7 +135,30 @@ __device__ __forceinline__ u4 normalise_unit(const __half* norm_w, const float* 
 
 // Prologue kinds of the activation staging (the NORM template parameter): none, the RMSNorm prologue, bf16 activations
 // converted to f16 on the way (through f32, rounded to nearest even: what the separate cast kernel does).
-constexpr int kPrologueNone = 0, kPrologueNorm = 1, kPrologueBf16 = 2;
+constexpr int kPrologueNone = 0, kPrologueNorm = 1, kPrologueBf16 = 2, kPrologueF32 = 3;  // (f32: rounded to f16 on the way)
+
+// 8 consecutive f32 activations (two 16-byte loads) -> one unit of 8 f16 values, rounded to nearest even
+__device__ __forceinline__ u4 f32_unit_to_f16(u4 lo, u4 hi) {
+  const float f[8] = {__uint_as_float(lo.x), __uint_as_float(lo.y), __uint_as_float(lo.z), __uint_as_float(lo.w),
+                      __uint_as_float(hi.x), __uint_as_float(hi.y), __uint_as_float(hi.z), __uint_as_float(hi.w)};
+  uint32_t w[4];
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    const h2 pair = {(_Float16)f[2 * e], (_Float16)f[2 * e + 1]};
+    w[e] = __builtin_bit_cast(uint32_t, pair);
+  }
+  return (u4){w[0], w[1], w[2], w[3]};
+}
+// unit u of activation row `row` of x (f16 / bf16: 16 bytes; f32: 32 bytes, converted)
+template <int NORM>
+__device__ __forceinline__ u4 load_unit(const __half* x, uint64_t row, uint32_t K, uint32_t u) {
+  if constexpr (NORM == kPrologueF32) {
+    const u4* xg = reinterpret_cast<const u4*>(reinterpret_cast<const float*>(x) + row * K);
+    return f32_unit_to_f16(xg[2 * u], xg[2 * u + 1]);
+  } else {
+    return reinterpret_cast<const u4*>(x + row * K)[u];
+  }
+}
 
 __device__ __forceinline__ u4 bf16_unit_to_f16(u4 v) {
   uint32_t w[4] = {v.x, v.y, v.z, v.w};
@@ -157,15 +180,14 @@ __device__ __forceinline__ void load_activations(const XImage<BITS, MR> g, const
 #pragma unroll
   for (int m = 0; m < MR; ++m) {
     const uint32_t rm = mrow0 + m < M ? mrow0 + m : M - 1;
-    const u4* xg = reinterpret_cast<const u4*>(x + (uint64_t)rm * g.K);
     const uint32_t u0 = (uint32_t)tid < nunits ? (uint32_t)tid : nunits - 1;
-    xv[m][0] = xg[u0];
+    xv[m][0] = load_unit<NORM>(x, rm, g.K, u0);
 #pragma unroll
     for (int i = 1; i < 4; ++i) {
       xv[m][i] = (u4){0u, 0u, 0u, 0u};
       if (nunits > (uint32_t)i * kThreads) {  // uniform; the last round may be partial (clamped, stored under a guard)
         const uint32_t u = tid + i * kThreads;
-        xv[m][i] = xg[u < nunits ? u : nunits - 1];
+        xv[m][i] = load_unit<NORM>(x, rm, g.K, u < nunits ? u : nunits - 1);
       }
     }
   }
@@ -229,7 +251,7 @@ __device__ __forceinline__ void stage_activations(const XImage<BITS, MR> g, cons
 #pragma unroll
     for (int m = 0; m < MR; ++m) {
       const uint32_t rm = mrow0 + m < M ? mrow0 + m : M - 1;
-      u4 v = reinterpret_cast<const u4*>(x + (uint64_t)rm * g.K)[u < nunits ? u : nunits - 1];
+      u4 v = load_unit<NORM>(x, rm, g.K, u < nunits ? u : nunits - 1);
       if constexpr (NORM == kPrologueBf16) v = bf16_unit_to_f16(v);
       if constexpr (NORM == kPrologueNorm) v = normalise_unit(norm_w, inv_rms, rm, u, nunits, v);
       stage_unit(m, u, v);
@@ -963,11 +985,19 @@ void launch_r(const M1Params& p, uint32_t group_size, hipStream_t s) {
       }
       return;
     }
-    if (p.x_bf16) {
+    if (p.x_bf16 == 1) {
       switch (group_size) {
         case 32: launch_k<BITS, 32, R, NT, MR, kPrologueBf16>(p, lds, s); break;
         case 64: launch_k<BITS, 64, R, NT, MR, kPrologueBf16>(p, lds, s); break;
         default: launch_k<BITS, 128, R, NT, MR, kPrologueBf16>(p, lds, s); break;
+      }
+      return;
+    }
+    if (p.x_bf16 == 2) {
+      switch (group_size) {
+        case 32: launch_k<BITS, 32, R, NT, MR, kPrologueF32>(p, lds, s); break;
+        case 64: launch_k<BITS, 64, R, NT, MR, kPrologueF32>(p, lds, s); break;
+        default: launch_k<BITS, 128, R, NT, MR, kPrologueF32>(p, lds, s); break;
       }
       return;
     }

@@ -1031,8 +1031,8 @@ def test_one_and_two_rows_over_short_rows_of_tall_matrices(hip, bits, n, k):
 
 @pytest.mark.parametrize("bits,gs,n,k", [(4, 64, 4096, 4096), (8, 64, 512, 2048), (4, 32, 256, 1152), (4, 128, 4096, 18944), (8, 128, 4096, 2560)])
 def test_bf16_rows_are_converted_inside_the_single_row_kernel(hip, bits, gs, n, k):
-    """One or two bf16 activation rows: the single-row kernel converts them to f16 while it stages them (no cast launch in
-    front of a decoding step's matmuls).  Bit-identical to the same matmul over the rows converted on the host the way
+    """One or two bf16 (or f32) activation rows: the single-row kernel converts them to f16 while it stages them (no cast
+    launch in front of a decoding step's matmuls).  Bit-identical to the same matmul over the rows converted on the host the way
     the cast kernel does (through f32, round to nearest even), and on the oracle; with a fused epilogue as well."""
     from rmlx_amd import ops
     from rmlx_amd.runtime import DeviceBuffer
@@ -1046,6 +1046,11 @@ def test_bf16_rows_are_converted_inside_the_single_row_kernel(hip, bits, gs, n, 
         want = _run(hip, words, s, b, x16, bits, gs=gs)
         assert np.array_equal(got.view(np.uint16), want.view(np.uint16)), (m, n, k)
         assert_close(got, model.qmm(x_as_f64(x, "bf16"), words, s, b, gs, bits), f"bf16 M={m} N={n} K={k} Q{bits} gs={gs}")
+        if m <= 2:  # f32 rows: rounded to f16 inside the single-row kernel, as the cast kernel rounds them
+            x32 = make_x(rng, m, k, "f32")
+            got32 = _run(hip, words, s, b, x32, bits, gs=gs, dtype="f32")
+            want32 = _run(hip, words, s, b, x32.astype(np.float16), bits, gs=gs)
+            assert np.array_equal(got32.view(np.uint16), want32.view(np.uint16)), ("f32", m, n, k)
         e = rng.standard_normal((m, n)).astype(np.float16)
         res = ops.qmm_add_residual(_dev(hip, x, "bf16"), qw, DeviceBuffer.from_numpy(e)).numpy()
         res16 = ops.qmm_add_residual(DeviceBuffer.from_numpy(x16), qw, DeviceBuffer.from_numpy(e)).numpy()
