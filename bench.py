@@ -196,6 +196,30 @@ def bench_moe(ops, rt, timer, rng, T, calls, experts, bits=4):
     return res
 
 
+def bench_moe_shape(ops, rt, timer, rng, T, calls, gate_up, down, gh, dh, E, top_k, D, I):
+    """The routed block over other expert shapes (E experts, top_k picks, hidden D, intermediate I; 4-bit, group 64): time
+    per call, weight bandwidth over the distinct experts of the batch, the first token against the oracle."""
+    from oracle import model
+    x = rng.standard_normal((T, D)).astype(np.float16)
+    logits = rng.standard_normal((T, E)).astype(np.float32)
+    xd, ld = rt.DeviceBuffer.from_numpy(x), rt.DeviceBuffer.from_numpy(logits)
+    out = rt.DeviceBuffer((T, D), rt.F16)
+
+    def run(c):
+        for _ in range(c):
+            ops.moe_forward(gh, None, dh, xd, ld, top_k, stream=timer.stream, out=out)
+
+    ms = timer.run(run, calls, 3, chunk=10)
+    idx, w, _, _ = model.topk_route(logits, top_k)
+    distinct = len(np.unique(idx))
+    nbytes = distinct * (3 * I * D // 2 + 3 * (I * D // 64) * 4)
+    gate, up = tuple(a[:, :I] for a in gate_up), tuple(a[:, I:] for a in gate_up)
+    ref = model.moe_forward(x[:1], idx[:top_k], w[:top_k], gate, up, down, 64, top_k)
+    err = float(np.abs(out.numpy()[:1].astype(np.float64) - ref).max())
+    return {"us": ms * 1e3, "calls": calls, "distinct_experts": distinct, "bytes": nbytes, "gbs": nbytes / (ms * 1e-3) / 1e9,
+            "flops": 2 * top_k * T * 3 * I * D, "max_err": err, "tol": model.tolerance(ref), "pass": bool(err <= model.tolerance(ref))}
+
+
 def bench_gather(ops, rt, timer, rng, batch, mpb, gh, gate_up, calls):
     """gather_qmm over the stacked gate/up weights of the MoE configuration (every batch entry names an expert)."""
     from oracle import model
@@ -406,8 +430,9 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50, help=f"timed steps; a step is a train of {TRAIN} launches")
     ap.add_argument("--warmup", type=int, default=10, help="untimed warm-up steps")
-    ap.add_argument("--only", default="", help="comma-separated sections: headline, floors, qmv, qmm, dequant, gather, moe, moe8, large; moevariants (not in the "
-                                           "default run): the routed block at T = 96 / 128 / 160 under every choice of expert kernels")
+    ap.add_argument("--only", default="", help="comma-separated sections: headline, floors, qmv, qmm, dequant, gather, moe, moe8, large; not in the default "
+                                           "run: moevariants (the routed block at T = 96 / 128 / 160 under every choice of expert kernels), "
+                                           "shapes (dimensions of models in the field that are no multiples of 512)")
     ap.add_argument("--quick", action="store_true", help="headline and floors only, short CPU baseline")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-graph", action="store_true",
@@ -502,6 +527,27 @@ def main():
         r = bench_matmul(ops, rt, timer, rng, 128, 12288, 4096, 8, "bf16", gemm_launches, train_warm, GiB + GiB // 8, gemm_layout=True)
         r["mfma_frac"] = r["tflops"] / MFMA_F16_PEAK_TF
         extra["q8_qmm_bf16_m128_n12288_gemm_layout"] = r
+    if "shapes" in sections:
+        # Dimensions of models in the field that are no multiples of 512 (not BASELINE configurations): dense matmuls with K in
+        # whole blocks of 128 / 64 and short rows of tall matrices, and the routed block over expert shapes with such an
+        # intermediate size.  One line per (shape, rows) / (shape, tokens).
+        progress("shapes")
+        few = max(60, launches // 30)
+        for n, k, ms in ((4096, 11008, (1, 8, 64, 512)), (9728, 896, (1, 2, 24)), (151936, 896, (1,)), (13824, 1152, (16, 512)),
+                         (4096, 2880, (8, 64, 512))):
+            for m in ms:
+                extra[f"shape_q4_n{n}_k{k}_m{m}"] = bench_matmul(ops, rt, timer, rng, m, n, k, 4, "f16", few, 10, GiB // 4, check_rows=256)
+        extra["shape_q4_n4096_k4096_m1_bf16_rows"] = bench_matmul(ops, rt, timer, rng, 1, 4096, 4096, 4, "bf16", launches, warm, GiB + GiB // 8)
+        for name, E, top_k, D, I in (("e128_top8_d2048_i768", 128, 8, 2048, 768), ("e64_top6_d2048_i1408", 64, 6, 2048, 1408),
+                                     ("e16_top2_d4096_i6400", 16, 2, 4096, 6400), ("e32_top4_d2880_i2880", 32, 4, 2880, 2880)):
+            one_gu, one_dn = make_weight(rng, 2 * I, D, 4, lead=(1,)), make_weight(rng, D, I, 4, lead=(1,))
+            gu = tuple(np.ascontiguousarray(np.broadcast_to(a, (E,) + a.shape[1:])) for a in one_gu)  # (one random expert repeated)
+            dn = tuple(np.ascontiguousarray(np.broadcast_to(a, (E,) + a.shape[1:])) for a in one_dn)
+            gq, dq = ops.QuantizedWeight.from_numpy(*gu, 64, 4), ops.QuantizedWeight.from_numpy(*dn, 64, 4)
+            for T in (1, 4, 32, 128, 512, 2048):
+                extra[f"shape_moe_q4_{name}_T{T}"] = bench_moe_shape(ops, rt, timer, np.random.default_rng(700 + T), T, 40 if T <= 128 else 12,
+                                                                     gu, dn, gq, dq, E, top_k, D, I)
+            del gq, dq, gu, dn
     if "dequant" in sections:
         progress("dequant")
         for fmt in ("awq", "gptq"):
