@@ -503,6 +503,7 @@ struct ExpertShapes {
   bool fused;
   bool portable;  // weights the streaming kernels do not take: the portable kernels run the block
   bool gemm;      // the grouped GEMM takes them too (batches with many rows per expert)
+  bool gemm_lds;  // the LDS-staged GEMM's grouped form takes them (dimensions in multiples of 64: what is left without `gemm`)
   uint32_t bits;  // of the gate weight
   bool gemm64;    // group size 64 (the 16-row tile is built for it only)
   uint32_t gemm_min_rows;  // of the gate weight's handle (rmlx_hip_qweight_set_expert_gemm_min_rows)
@@ -586,6 +587,8 @@ int32_t check_expert_weights(const char* who, const rmlx_qweight* gate, const rm
   // the grouped GEMM also takes group sizes the streaming kernels do not (32; 128 at 8 bits)
   sh->gemm = uniform && qmm_rw_grouped_supported(sh->I, sh->D, gate->group_size, gate->bits) &&
              qmm_rw_grouped_supported(sh->D, sh->I, gate->group_size, gate->bits);
+  sh->gemm_lds = uniform && (gate->bits == 4 || gate->bits == 8) && qmm_supported(sh->I, sh->D, gate->group_size, gate->bits) &&
+                 qmm_supported(sh->D, sh->I, gate->group_size, gate->bits);
   return RMLX_OK;
 }
 
@@ -1514,7 +1517,11 @@ int32_t moe_grouped_impl(const rmlx_qweight* gate, const rmlx_qweight* up, const
   // stay on it until the grouped GEMM takes the batch, at every batch size where that does not take the shape either: an
   // expert per assignment on the single-row kernels is far ahead of the portable kernels)
   const uint32_t gemm_rows = expert_gemm_tile_rows(sh, A, sh.E);  // (0: the batch is below the grouped GEMM's threshold)
-  const bool only_single_row = sh.portable && gemm_rows == 0 && A <= kUngroupedOnlyMaxAssignments;
+  // (experts in multiples of 64 that the register-weights grouped GEMM does not take -- a hidden size of 2880: the grouped form
+  // of the LDS-staged GEMM from one row per expert on, where the form without grouping would stream an expert per assignment)
+  const bool lds_gemm = sh.portable && !sh.gemm && sh.gemm_lds && sh.gemm_min_rows != 0 && A >= sh.E &&
+                        !ungrouped_pays(T32, sh.E, (uint32_t)top_k, gate->bits) && A / 64 + sh.E <= 65535;
+  const bool only_single_row = sh.portable && gemm_rows == 0 && !lds_gemm && A <= kUngroupedOnlyMaxAssignments;
   const bool direct = (ungrouped_pays(T32, sh.E, (uint32_t)top_k, gate->bits) || only_single_row) && sh.stream_kernel != 1 &&
                       single_row_experts(gate, up, down, sh) && (route == nullptr || sh.E <= 256);
   // (its down projection adds the weighted expert outputs itself where the wave-per-tile kernel takes the weights)
@@ -1584,6 +1591,59 @@ int32_t moe_grouped_impl(const rmlx_qweight* gate, const rmlx_qweight* up, const
       RMLX_TRY(launch_moe_combine_rows_f16(static_cast<const __half*>(y.ptr), picks, pick_weights, T32, (uint32_t)top_k, sh.D, sh.E,
                                            static_cast<__half*>(out_f16_dev), s));
     }
+    return finish(s);
+  }
+  if (lds_gemm) {
+    // grouping into row tiles of 64 rows of one expert, then per projection: activations to the GEMM's fragment layout (through
+    // the token map for the first), the grouped LDS-staged GEMM, SwiGLU as a pass of its own, and the weighted combine
+    if (!aligned16(xk)) return fail(RMLX_INVALID_SHAPE, "MoeLayer: input must be 16-byte aligned");
+    const uint32_t max_tiles = A / 64 + (A < sh.E ? A : sh.E);
+    const uint32_t per = 32 / gate->bits, gs = gate->group_size;
+    RMLX_TRY(meta.alloc(((size_t)3 * A + 3 * (size_t)max_tiles + 4) * 4, s, arena));
+    uint32_t* sorted = static_cast<uint32_t*>(meta.ptr);
+    uint32_t* sorted_tok = sorted + A;
+    uint32_t* inv = sorted_tok + A;
+    uint32_t* tile_tab = inv + A;
+    uint32_t* n_tiles = tile_tab + 3 * (size_t)max_tiles;
+    RMLX_TRY(launch_moe_sort(expert_indices_dev, A, sh.E, (uint32_t)top_k, sorted, sorted_tok, inv, nullptr, nullptr, tile_tab, n_tiles, 64, s));
+    Scratch ws, gu, y16;
+    const uint32_t kmax = sh.D > sh.I ? sh.D : sh.I;
+    RMLX_TRY(ws.alloc(qmm_grouped_workspace_bytes(max_tiles, kmax), s, arena));
+    RMLX_TRY(gu.alloc((size_t)A * 2 * sh.I * 2, s, arena));
+    RMLX_TRY(h.alloc((size_t)A * sh.I * 2, s, arena));
+    GroupedQmmArgs a{};
+    a.w = gate->w; a.s = gate->s; a.b = gate->b;
+    a.K = sh.D; a.bits = gate->bits; a.group_size = gs;
+    a.x = xk; a.row_map = sorted_tok; a.out_f32 = 0;
+    a.tile_tab = tile_tab; a.n_tiles_dev = n_tiles; a.max_tiles = max_tiles; a.tile_rows = 64;
+    __half* g_out = static_cast<__half*>(gu.ptr);
+    if (sh.fused) {  // one stacked matrix per expert: [A, 2I] = (gate | up)
+      a.N = 2 * sh.I;
+      a.expert_stride_w = (uint64_t)2 * sh.I * (sh.D / per); a.expert_stride_s = (uint64_t)2 * sh.I * (sh.D / gs);
+      a.out = g_out;
+      RMLX_TRY(launch_qmm_grouped(a, ws.ptr, s));
+      RMLX_TRY(launch_silu_gate_strided(g_out, g_out + sh.I, 2 * sh.I, static_cast<__half*>(h.ptr), A, sh.I, s));
+    } else {
+      a.N = sh.I;
+      a.expert_stride_w = (uint64_t)sh.I * (sh.D / per); a.expert_stride_s = (uint64_t)sh.I * (sh.D / gs);
+      a.out = g_out;
+      RMLX_TRY(launch_qmm_grouped(a, ws.ptr, s));
+      a.w = up->w; a.s = up->s; a.b = up->b; a.out = g_out + (size_t)A * sh.I;
+      RMLX_TRY(launch_qmm_grouped(a, ws.ptr, s));
+      RMLX_TRY(launch_silu_gate(g_out, g_out + (size_t)A * sh.I, static_cast<__half*>(h.ptr), (size_t)A * sh.I, s));
+    }
+    RMLX_TRY(y16.alloc((size_t)A * sh.D * 2, s, arena));
+    GroupedQmmArgs d{};
+    d.w = down->w; d.s = down->s; d.b = down->b;
+    d.N = sh.D; d.K = sh.I; d.bits = down->bits; d.group_size = gs;
+    d.expert_stride_w = (uint64_t)sh.D * (sh.I / per); d.expert_stride_s = (uint64_t)sh.D * (sh.I / gs);
+    d.x = static_cast<const __half*>(h.ptr); d.row_map = nullptr; d.out = y16.ptr; d.out_f32 = 0;
+    d.tile_tab = tile_tab; d.n_tiles_dev = n_tiles; d.max_tiles = max_tiles; d.tile_rows = 64;
+    RMLX_TRY(launch_qmm_grouped(d, ws.ptr, s));
+    RMLX_TRY(y.alloc((size_t)A * sh.D * 4, s, arena));
+    RMLX_TRY(launch_cast_f16_to_f32(static_cast<const __half*>(y16.ptr), static_cast<float*>(y.ptr), (size_t)A * sh.D, s));
+    RMLX_TRY(launch_moe_combine(static_cast<const float*>(y.ptr), inv, expert_weights_dev, T32, (uint32_t)top_k, sh.D,
+                                static_cast<__half*>(out_f16_dev), s));
     return finish(s);
   }
   // 2-bit experts: the form without grouping on the 2-bit single-row kernel with a weight matrix per row -- routing,

@@ -37,6 +37,10 @@ struct QmmParams {
   uint32_t M, N, K;
   uint32_t Kx;  // columns of the fragment-major activations: K rounded up to whole unrolled iterations, zeros past K
   uint32_t group_size;
+  // grouped launches (one expert per 64-row tile): table of (expert, first row, rows; bit 31 of the rows: an expert index out of
+  // range, zeros are written) per row tile and its length on the device, expert strides in u32 words / halves
+  const uint32_t* tile_tab; const uint32_t* n_tiles;
+  uint64_t estride_w, estride_s;
 };
 
 
@@ -92,7 +96,9 @@ __device__ __forceinline__ u2 dequant_q8_word_bf16(uint32_t w, float s, float b)
 // and biases are fetched as single halves (a row of them starts on a 2-byte boundary only when K / 64 is odd).
 // GS: the quantisation group size.  A thread's 16 values of a step lie in one group at every size; at 32 and 128 the
 // (scale, bias) of a step is fetched as single halves like in the TAIL form (group 2 * step + quarter / 2, step / 2).
-template <int BM, int BN, int BITS, bool XBF16, bool TAIL, int GS>
+// GROUPED: row tile t of the grid takes its expert and its rows from the tile table; its activations are tile t of the
+// fragment-major workspace (relayout_grouped_kernel), so p.M is the grid's row extent, max_tiles * BM.
+template <int BM, int BN, int BITS, bool XBF16, bool TAIL, int GS, bool GROUPED = false>
 __global__ __launch_bounds__(kThreads) void qmm_kernel(QmmParams p) {
   static_assert(GS == 32 || GS == 64 || GS == 128, "group sizes of the format");
   constexpr bool kHalfLoads = TAIL || GS != 64;
@@ -118,8 +124,24 @@ __global__ __launch_bounds__(kThreads) void qmm_kernel(QmmParams p) {
   const uint32_t tiles_m = (p.M + BM - 1) / BM, tiles_n = p.N / BN;
   const uint32_t total = tiles_m * tiles_n;
   uint32_t id = blockIdx.x;
-  if (total % 8 == 0) id = (id % 8) * (total / 8) + id / 8;
-  const uint32_t m0 = (id % tiles_m) * BM, n0 = (id / tiles_m) * BN;
+  if (!GROUPED && total % 8 == 0) id = (id % 8) * (total / 8) + id / 8;
+  const uint32_t m0 = (GROUPED ? id / tiles_n : id % tiles_m) * BM, n0 = (GROUPED ? id % tiles_n : id / tiles_m) * BN;
+  uint32_t row_lo = 0, row_cnt = 0;
+  uint64_t e_w = 0, e_s = 0;
+  if (GROUPED) {
+    const uint32_t te = m0 / BM;
+    if (te >= *p.n_tiles) return;
+    const uint32_t expert = p.tile_tab[3 * te], c = p.tile_tab[3 * te + 2];
+    row_lo = p.tile_tab[3 * te + 1];
+    row_cnt = c & 0x7FFFFFFFu;
+    if (c >> 31) {  // rows whose expert index is out of range: zeros
+      for (uint32_t i = threadIdx.x; i < row_cnt * BN; i += kThreads)
+        p.out[(uint64_t)(row_lo + i / BN) * p.N + n0 + i % BN] = __float2half(0.f);
+      return;
+    }
+    e_w = expert * p.estride_w;
+    e_s = expert * p.estride_s;
+  }
 
   const uint32_t K = p.K, gpr = K / GS;
   const uint32_t Kx = TAIL ? p.Kx : K;
@@ -128,9 +150,9 @@ __global__ __launch_bounds__(kThreads) void qmm_kernel(QmmParams p) {
 
   // weight staging coordinates
   const int brow = tid >> 2, bq = tid & 3;  // weight row in tile, 16-value quarter of the 64-k step
-  const uint32_t* wptr = p.w + (uint64_t)(n0 + brow) * (K * BITS / 32) + bq * WPT;
-  const __half* sptr = p.s + (uint64_t)(n0 + brow) * gpr;
-  const __half* bptr = p.b + (uint64_t)(n0 + brow) * gpr;
+  const uint32_t* wptr = p.w + e_w + (uint64_t)(n0 + brow) * (K * BITS / 32) + bq * WPT;
+  const __half* sptr = p.s + e_s + (uint64_t)(n0 + brow) * gpr;
+  const __half* bptr = p.b + e_s + (uint64_t)(n0 + brow) * gpr;
 
   // activation fragments: block (16-row tile, 32-wide k chunk) = 64 lanes x 16 bytes, contiguous,
   // already in MFMA operand order.  Tiles past the last one re-read the last tile (their results
@@ -310,7 +332,12 @@ __global__ __launch_bounds__(kThreads) void qmm_kernel(QmmParams p) {
       for (int v = 0; v < 4; ++v) {
         const uint32_t m = m0 + wave * WM + i * 16 + g * 4 + v;
         const uint32_t nn = n0 + j * 16 + r16;
-        if (m < p.M) p.out[(uint64_t)m * p.N + nn] = __float2half(acc[i][j][v]);
+        if (GROUPED) {
+          const uint32_t local = m - m0;
+          if (local < row_cnt) p.out[(uint64_t)(row_lo + local) * p.N + nn] = __float2half(acc[i][j][v]);
+        } else if (m < p.M) {
+          p.out[(uint64_t)m * p.N + nn] = __float2half(acc[i][j][v]);
+        }
       }
 }
 
@@ -375,6 +402,36 @@ __global__ __launch_bounds__(256) void relayout_a_kernel(const void* __restrict_
   }
 }
 
+// The same layout for the row tiles of a grouped launch: tile t (64 rows of one expert: positions first .. first + rows - 1 of
+// the table entry, through the row map where there is one; rows past the entry's repeat its last row) fills fragments
+// 4 t .. 4 t + 3 of the workspace.  f16 activations.
+__global__ __launch_bounds__(256) void relayout_grouped_kernel(const __half* __restrict__ src, const uint32_t* __restrict__ row_map,
+                                                               const uint32_t* __restrict__ tile_tab, const uint32_t* __restrict__ n_tiles,
+                                                               uint32_t max_tiles, u4* __restrict__ dst, uint32_t K, uint32_t Kx) {
+  const uint32_t kchunks = Kx / 32, per_tile = 4 * kchunks * 64, nt = *n_tiles;
+  const uint64_t units = (uint64_t)max_tiles * per_tile;
+  for (uint64_t u = (uint64_t)blockIdx.x * 256 + threadIdx.x; u < units; u += (uint64_t)gridDim.x * 256) {
+    const uint32_t te = (uint32_t)(u / per_tile);
+    if (te >= nt) return;  // (units ascend with the thread's stride)
+    const uint32_t r = (uint32_t)(u % per_tile), lane = r & 63, blk = r >> 6, frag = blk / kchunks, kc = blk % kchunks;
+    const uint32_t cnt = tile_tab[3 * te + 2] & 0x7FFFFFFFu;
+    uint32_t local = frag * 16 + (lane & 15);
+    if (local >= cnt) local = cnt - 1;
+    uint32_t row = tile_tab[3 * te + 1] + local;
+    if (row_map != nullptr) row = row_map[row];
+    u4 o = (u4){0u, 0u, 0u, 0u};
+    if (kc * 32 < K) o = *reinterpret_cast<const u4*>(src + (uint64_t)row * K + kc * 32 + (lane >> 4) * 8);
+    dst[u] = o;
+  }
+}
+
+template <int BITS, int GS>
+void launch_grouped_t(const QmmParams& p, uint32_t max_tiles, hipStream_t s) {
+  const uint32_t tiles = max_tiles * (p.N / 64);
+  if (p.Kx != p.K) hipLaunchKernelGGL((qmm_kernel<64, 64, BITS, false, true, GS, true>), dim3(tiles), dim3(kThreads), 0, s, p);
+  else hipLaunchKernelGGL((qmm_kernel<64, 64, BITS, false, false, GS, true>), dim3(tiles), dim3(kThreads), 0, s, p);
+}
+
 template <int BM, int BITS, bool XBF16>
 void launch_t(const QmmParams& p, hipStream_t s) {
   const uint32_t tiles = ((p.M + BM - 1) / BM) * (p.N / 64);
@@ -403,6 +460,41 @@ bool qmm_supported(uint32_t N, uint32_t K, uint32_t group_size, uint32_t bits) {
 
 size_t qmm_workspace_bytes(uint32_t M, uint32_t K) { return (size_t)((M + 15) / 16) * 16 * padded_k(K) * 2; }
 
+size_t qmm_grouped_workspace_bytes(uint32_t max_tiles, uint32_t K) { return (size_t)max_tiles * 64 * padded_k(K) * 2; }
+
+// Grouped launch over row tiles of 64 rows of one expert each (see GroupedQmmArgs; one weight per launch, f16 output):
+// what the routed block runs on where the register-weights grouped GEMM does not take the shape (dimensions in multiples
+// of 64 that are no multiples of 128).  `workspace`: qmm_grouped_workspace_bytes(max_tiles, K) bytes.
+int32_t launch_qmm_grouped(const GroupedQmmArgs& a, void* workspace, hipStream_t s) {
+  if (!qmm_supported(a.N, a.K, a.group_size, a.bits))
+    return fail(RMLX_INVALID_SHAPE, "grouped qmm: unsupported shape N=%u K=%u bits=%u group_size=%u", a.N, a.K, a.bits, a.group_size);
+  if (a.max_tiles == 0) return RMLX_OK;
+  if (a.w1 != nullptr || a.out_f32 || a.tile_rows != 64 || a.tile_tab == nullptr || a.n_tiles_dev == nullptr || workspace == nullptr)
+    return fail(RMLX_RUNTIME_ERROR, "grouped qmm (LDS-staged): one weight, f16 output, 64-row tiles, a tile table and a workspace");
+  if ((uint64_t)a.max_tiles * (a.N / 64) > 0x7FFFFFFFull) return fail(RMLX_INVALID_SHAPE, "grouped qmm: grid too large");
+  const uint32_t Kx = padded_k(a.K);
+  {
+    const uint64_t units = (uint64_t)a.max_tiles * 4 * (Kx / 32) * 64;
+    uint64_t blocks = (units + 255) / 256;
+    if (blocks > 8192) blocks = 8192;
+    hipLaunchKernelGGL(relayout_grouped_kernel, dim3((unsigned)blocks), dim3(256), 0, s, a.x, a.row_map, a.tile_tab, a.n_tiles_dev,
+                       a.max_tiles, reinterpret_cast<u4*>(workspace), a.K, Kx);
+  }
+  QmmParams p{a.w, a.s, a.b, reinterpret_cast<const uint16_t*>(workspace), static_cast<__half*>(a.out), a.max_tiles * 64, a.N, a.K, Kx,
+              a.group_size, a.tile_tab, a.n_tiles_dev, a.expert_stride_w, a.expert_stride_s};
+  if (a.bits == 4) {
+    if (a.group_size == 32) launch_grouped_t<4, 32>(p, a.max_tiles, s);
+    else if (a.group_size == 128) launch_grouped_t<4, 128>(p, a.max_tiles, s);
+    else launch_grouped_t<4, 64>(p, a.max_tiles, s);
+  } else {
+    if (a.group_size == 32) launch_grouped_t<8, 32>(p, a.max_tiles, s);
+    else if (a.group_size == 128) launch_grouped_t<8, 128>(p, a.max_tiles, s);
+    else launch_grouped_t<8, 64>(p, a.max_tiles, s);
+  }
+  RMLX_HIP_CHECK(hipGetLastError());
+  return RMLX_OK;
+}
+
 int32_t launch_qmm(const QmmArgs& a, hipStream_t s) {
   if (!qmm_supported(a.N, a.K, a.group_size, a.bits))
     return fail(RMLX_INVALID_SHAPE, "qmm: unsupported shape N=%u K=%u bits=%u group_size=%u", a.N, a.K, a.bits, a.group_size);
@@ -418,7 +510,7 @@ int32_t launch_qmm(const QmmArgs& a, hipStream_t s) {
     hipLaunchKernelGGL(relayout_a_kernel, dim3((unsigned)blocks), dim3(256), 0, s, a.x, a.x_dtype,
                        reinterpret_cast<u4*>(a.workspace), a.M, a.K, Kx, want_bf16 ? 1 : 0);
   }
-  QmmParams p{a.w, a.s, a.b, reinterpret_cast<const uint16_t*>(a.workspace), a.out, a.M, a.N, a.K, Kx, a.group_size};
+  QmmParams p{a.w, a.s, a.b, reinterpret_cast<const uint16_t*>(a.workspace), a.out, a.M, a.N, a.K, Kx, a.group_size, nullptr, nullptr, 0, 0};
   // 128-row tiles only when they still give (most of) the CUs a workgroup
   const uint32_t tiles128 = ((a.M + 127) / 128) * (a.N / 64);
   const bool big = a.M > 64 && tiles128 * 4 >= (uint32_t)ctx().num_cus * 3;

@@ -609,6 +609,51 @@ def test_moe_forward_of_bf16_activations(hip, bits, gs, D, I, T):
     assert np.array_equal(got2.view(np.uint16), want.view(np.uint16))
 
 
+@pytest.mark.parametrize("bits,gs,D,I,fused", [(4, 64, 320, 448, True), (4, 64, 2880, 960, True), (8, 64, 576, 320, False),
+                                               (4, 32, 448, 320, True), (4, 128, 384, 640, False)])
+@pytest.mark.parametrize("T", [24, 70, 300])
+def test_moe_forward_on_the_grouped_lds_staged_gemm(hip, bits, gs, D, I, fused, T):
+    """Expert dimensions in multiples of 64 that are no multiples of 128 (a hidden size of 2880): from one row per expert on
+    the block groups the rows into tiles of 64 rows of one expert and multiplies them with the grouped form of the
+    LDS-staged GEMM (activations re-laid through the token map, K padded to whole iterations, SwiGLU and combine as passes
+    of their own).  Stacked and separate gate / up weights, every group size, experts with no rows, with one row and with
+    more than a tile; an expert index out of range gives zeros.  Against the oracle."""
+    from rmlx_amd import ops
+    from rmlx_amd.runtime import DeviceBuffer
+    rng = np.random.default_rng(bits + gs + D + I + T)
+    E, K = 7, 2
+    gu = make_weight(rng, 2 * I, D, bits, gs, lead=(E,))
+    down = make_weight(rng, D, I, bits, gs, lead=(E,))
+    gate, up = tuple(a[:, :I] for a in gu), tuple(np.ascontiguousarray(a[:, I:]) for a in gu)
+    if fused:
+        gh, uh = ops.QuantizedWeight.from_numpy(*gu, gs, bits), None
+    else:
+        gh = ops.QuantizedWeight.from_numpy(*(np.ascontiguousarray(a) for a in gate), gs, bits)
+        uh = ops.QuantizedWeight.from_numpy(*up, gs, bits)
+    dh = ops.QuantizedWeight.from_numpy(*down, gs, bits)
+    x = make_x(rng, T, D)
+    logits = rng.standard_normal((T, E)).astype(np.float32)
+    logits[:, 5] -= 20.0          # expert 5 gets no rows
+    logits[: T // 2, 2] += 4.0    # expert 2 gets half the batch: more than one tile at T = 300
+    idx, w, counts, _ = model.topk_route(logits, K)
+    ref = model.moe_forward(x, idx, w, gate, up, down, gs, K, bits=bits)
+    print(f"grouped LDS GEMM Q{bits} gs{gs} D={D} I={I} fused={fused} T={T} counts={counts.tolist()}", flush=True)
+    xd = DeviceBuffer.from_numpy(x)
+    assert_close(ops.moe_forward(gh, uh, dh, xd, DeviceBuffer.from_numpy(logits), K).numpy(), ref, "moe_forward")
+    out = ops.moe_forward_grouped(gh, uh, dh, xd, DeviceBuffer.from_numpy(idx), DeviceBuffer.from_numpy(w), K).numpy()
+    assert_close(out, ref, "moe_forward_grouped")
+    bad = idx.copy()
+    bad[3] = E + 2
+    w_ref = w.copy()
+    w_ref[3] = 0.0
+    from rmlx_amd.runtime import Stream
+    st = Stream()
+    out = ops.moe_forward_grouped(gh, uh, dh, xd, DeviceBuffer.from_numpy(bad), DeviceBuffer.from_numpy(w), K, stream=st)
+    st.sync()
+    idx_ok = np.where(bad < E, bad, 0).astype(np.uint32)
+    assert_close(out.numpy(), model.moe_forward(x, idx_ok, w_ref, gate, up, down, gs, K, bits=bits), "one pick out of range")
+
+
 @pytest.mark.parametrize("T,K", [(1, 2), (1, 8), (2, 3), (3, 4)])
 def test_moe_forward_grouped_with_repeated_experts(hip, T, K):
     """Caller-supplied picks may name one expert several times for a token; decode-sized batches run kernels
