@@ -699,6 +699,48 @@ bool single_row_experts(const rmlx_qweight* gate, const rmlx_qweight* up, const 
 }
 
 // gate/up + SwiGLU then down, over a device chunk table.  h: f16 [positions, I] scratch.
+// The expert FFN over row tiles of 64 rows of one expert each on the grouped form of the LDS-staged GEMM (expert dimensions in
+// multiples of 64 that the register-weights grouped GEMM does not take): gate / up (one stacked matrix, or two launches), SwiGLU
+// as a pass of its own, down.  x: f16 rows reached through row_map (nullable); y16: f16 [positions, D] in the table's row order.
+int32_t run_expert_ffn_lds(const rmlx_qweight* gate, const rmlx_qweight* up, const rmlx_qweight* down, const ExpertShapes& sh,
+                           const __half* x, const uint32_t* row_map, const uint32_t* tile_tab, const uint32_t* n_tiles,
+                           uint32_t max_tiles, uint32_t positions, __half* y16, hipStream_t s, Arena* arena) {
+  const uint32_t per = 32 / gate->bits, gs = gate->group_size;
+  Scratch ws, gu, h;
+  const uint32_t kmax = sh.D > sh.I ? sh.D : sh.I;
+  RMLX_TRY(ws.alloc(qmm_grouped_workspace_bytes(max_tiles, kmax), s, arena));
+  RMLX_TRY(gu.alloc((size_t)positions * 2 * sh.I * 2, s, arena));
+  RMLX_TRY(h.alloc((size_t)positions * sh.I * 2, s, arena));
+  GroupedQmmArgs a{};
+  a.w = gate->w; a.s = gate->s; a.b = gate->b;
+  a.K = sh.D; a.bits = gate->bits; a.group_size = gs;
+  a.x = x; a.row_map = row_map; a.out_f32 = 0;
+  a.tile_tab = tile_tab; a.n_tiles_dev = n_tiles; a.max_tiles = max_tiles; a.tile_rows = 64;
+  __half* g_out = static_cast<__half*>(gu.ptr);
+  if (sh.fused) {  // one stacked matrix per expert: [positions, 2I] = (gate | up)
+    a.N = 2 * sh.I;
+    a.expert_stride_w = (uint64_t)2 * sh.I * (sh.D / per); a.expert_stride_s = (uint64_t)2 * sh.I * (sh.D / gs);
+    a.out = g_out;
+    RMLX_TRY(launch_qmm_grouped(a, ws.ptr, s));
+    RMLX_TRY(launch_silu_gate_strided(g_out, g_out + sh.I, 2 * sh.I, static_cast<__half*>(h.ptr), positions, sh.I, s));
+  } else {
+    a.N = sh.I;
+    a.expert_stride_w = (uint64_t)sh.I * (sh.D / per); a.expert_stride_s = (uint64_t)sh.I * (sh.D / gs);
+    a.out = g_out;
+    RMLX_TRY(launch_qmm_grouped(a, ws.ptr, s));
+    a.w = up->w; a.s = up->s; a.b = up->b; a.out = g_out + (size_t)positions * sh.I;
+    RMLX_TRY(launch_qmm_grouped(a, ws.ptr, s));
+    RMLX_TRY(launch_silu_gate(g_out, g_out + (size_t)positions * sh.I, static_cast<__half*>(h.ptr), (size_t)positions * sh.I, s));
+  }
+  GroupedQmmArgs d{};
+  d.w = down->w; d.s = down->s; d.b = down->b;
+  d.N = sh.D; d.K = sh.I; d.bits = down->bits; d.group_size = gs;
+  d.expert_stride_w = (uint64_t)sh.D * (sh.I / per); d.expert_stride_s = (uint64_t)sh.D * (sh.I / gs);
+  d.x = static_cast<const __half*>(h.ptr); d.row_map = nullptr; d.out = y16; d.out_f32 = 0;
+  d.tile_tab = tile_tab; d.n_tiles_dev = n_tiles; d.max_tiles = max_tiles; d.tile_rows = 64;
+  return launch_qmm_grouped(d, ws.ptr, s);
+}
+
 int32_t run_expert_ffn(const rmlx_qweight* gate, const rmlx_qweight* up, const rmlx_qweight* down,
                        const ExpertShapes& sh, const __half* x, const uint32_t* row_map,
                        const uint32_t* chunk_tab, const uint32_t* n_chunks, uint32_t max_chunks, __half* h,
@@ -1446,6 +1488,32 @@ int32_t rmlx_hip_expert_group_grouped_forward(const rmlx_qweight* gate, const rm
     RMLX_HIP_CHECK(hipMemcpyAsync(dtab.ptr, expert_of.data(), total * 4, hipMemcpyHostToDevice, s));
     RMLX_HIP_CHECK(hipStreamSynchronize(s));  // `expert_of` is pageable host memory owned by this call
     const uint32_t* experts = static_cast<const uint32_t*>(dtab.ptr);
+    // dimensions in multiples of 64: row tiles of 64 rows of one item on the grouped form of the LDS-staged GEMM, from three rows
+    // per item on (see moe_grouped_impl)
+    if (sh.gemm_lds && sh.gemm_min_rows != 0 && total >= 3 * n_items && aligned16(xk)) {
+      std::vector<uint32_t> tiles;
+      size_t first = 0;
+      for (size_t i = 0; i < n_items; ++i) {
+        for (uint32_t r = 0; r < batch_sizes_host[i]; r += 64) {
+          tiles.push_back(expert_idx_host[i]);
+          tiles.push_back((uint32_t)(first + r));
+          tiles.push_back(batch_sizes_host[i] - r < 64 ? batch_sizes_host[i] - r : 64);
+        }
+        first += batch_sizes_host[i];
+      }
+      const uint32_t n_t = (uint32_t)(tiles.size() / 3);
+      if (n_t <= 65535) {
+        tiles.push_back(n_t);
+        Scratch ttab;
+        RMLX_TRY(ttab.alloc(tiles.size() * 4, s));
+        RMLX_HIP_CHECK(hipMemcpyAsync(ttab.ptr, tiles.data(), tiles.size() * 4, hipMemcpyHostToDevice, s));
+        RMLX_HIP_CHECK(hipStreamSynchronize(s));  // `tiles` is pageable host memory owned by this call
+        const uint32_t* tt = static_cast<const uint32_t*>(ttab.ptr);
+        RMLX_TRY(run_expert_ffn_lds(gate, up, down, sh, xk, nullptr, tt, tt + 3 * (size_t)n_t, n_t, rows,
+                                    static_cast<__half*>(out_f16_dev), s, nullptr));
+        return finish(s);
+      }
+    }
     // where the single-row kernels take the weights (4- / 8-bit, rows in whole 16-byte pieces: a hidden size of 2880), every
     // row multiplies with its own expert on them -- an expert streamed once per row, far ahead of the portable kernels
     if (rows <= kUngroupedOnlyMaxAssignments && sh.stream_kernel != 1 && aligned16(xk) && single_row_experts(gate, up, down, sh)) {
@@ -1519,7 +1587,9 @@ int32_t moe_grouped_impl(const rmlx_qweight* gate, const rmlx_qweight* up, const
   const uint32_t gemm_rows = expert_gemm_tile_rows(sh, A, sh.E);  // (0: the batch is below the grouped GEMM's threshold)
   // (experts in multiples of 64 that the register-weights grouped GEMM does not take -- a hidden size of 2880: the grouped form
   // of the LDS-staged GEMM from one row per expert on, where the form without grouping would stream an expert per assignment)
-  const bool lds_gemm = sh.portable && !sh.gemm && sh.gemm_lds && sh.gemm_min_rows != 0 && A >= sh.E &&
+  // (E = 32, top-4, D = I = 2880: 16 tokens 196 us without grouping against about 300 us, 32 tokens 393 against 307 us: from three
+  // rows per expert on)
+  const bool lds_gemm = sh.portable && !sh.gemm && sh.gemm_lds && sh.gemm_min_rows != 0 && A >= 3 * sh.E &&
                         !ungrouped_pays(T32, sh.E, (uint32_t)top_k, gate->bits) && A / 64 + sh.E <= 65535;
   const bool only_single_row = sh.portable && gemm_rows == 0 && !lds_gemm && A <= kUngroupedOnlyMaxAssignments;
   const bool direct = (ungrouped_pays(T32, sh.E, (uint32_t)top_k, gate->bits) || only_single_row) && sh.stream_kernel != 1 &&
@@ -1598,7 +1668,6 @@ int32_t moe_grouped_impl(const rmlx_qweight* gate, const rmlx_qweight* up, const
     // the token map for the first), the grouped LDS-staged GEMM, SwiGLU as a pass of its own, and the weighted combine
     if (!aligned16(xk)) return fail(RMLX_INVALID_SHAPE, "MoeLayer: input must be 16-byte aligned");
     const uint32_t max_tiles = A / 64 + (A < sh.E ? A : sh.E);
-    const uint32_t per = 32 / gate->bits, gs = gate->group_size;
     RMLX_TRY(meta.alloc(((size_t)3 * A + 3 * (size_t)max_tiles + 4) * 4, s, arena));
     uint32_t* sorted = static_cast<uint32_t*>(meta.ptr);
     uint32_t* sorted_tok = sorted + A;
@@ -1606,40 +1675,9 @@ int32_t moe_grouped_impl(const rmlx_qweight* gate, const rmlx_qweight* up, const
     uint32_t* tile_tab = inv + A;
     uint32_t* n_tiles = tile_tab + 3 * (size_t)max_tiles;
     RMLX_TRY(launch_moe_sort(expert_indices_dev, A, sh.E, (uint32_t)top_k, sorted, sorted_tok, inv, nullptr, nullptr, tile_tab, n_tiles, 64, s));
-    Scratch ws, gu, y16;
-    const uint32_t kmax = sh.D > sh.I ? sh.D : sh.I;
-    RMLX_TRY(ws.alloc(qmm_grouped_workspace_bytes(max_tiles, kmax), s, arena));
-    RMLX_TRY(gu.alloc((size_t)A * 2 * sh.I * 2, s, arena));
-    RMLX_TRY(h.alloc((size_t)A * sh.I * 2, s, arena));
-    GroupedQmmArgs a{};
-    a.w = gate->w; a.s = gate->s; a.b = gate->b;
-    a.K = sh.D; a.bits = gate->bits; a.group_size = gs;
-    a.x = xk; a.row_map = sorted_tok; a.out_f32 = 0;
-    a.tile_tab = tile_tab; a.n_tiles_dev = n_tiles; a.max_tiles = max_tiles; a.tile_rows = 64;
-    __half* g_out = static_cast<__half*>(gu.ptr);
-    if (sh.fused) {  // one stacked matrix per expert: [A, 2I] = (gate | up)
-      a.N = 2 * sh.I;
-      a.expert_stride_w = (uint64_t)2 * sh.I * (sh.D / per); a.expert_stride_s = (uint64_t)2 * sh.I * (sh.D / gs);
-      a.out = g_out;
-      RMLX_TRY(launch_qmm_grouped(a, ws.ptr, s));
-      RMLX_TRY(launch_silu_gate_strided(g_out, g_out + sh.I, 2 * sh.I, static_cast<__half*>(h.ptr), A, sh.I, s));
-    } else {
-      a.N = sh.I;
-      a.expert_stride_w = (uint64_t)sh.I * (sh.D / per); a.expert_stride_s = (uint64_t)sh.I * (sh.D / gs);
-      a.out = g_out;
-      RMLX_TRY(launch_qmm_grouped(a, ws.ptr, s));
-      a.w = up->w; a.s = up->s; a.b = up->b; a.out = g_out + (size_t)A * sh.I;
-      RMLX_TRY(launch_qmm_grouped(a, ws.ptr, s));
-      RMLX_TRY(launch_silu_gate(g_out, g_out + (size_t)A * sh.I, static_cast<__half*>(h.ptr), (size_t)A * sh.I, s));
-    }
+    Scratch y16;
     RMLX_TRY(y16.alloc((size_t)A * sh.D * 2, s, arena));
-    GroupedQmmArgs d{};
-    d.w = down->w; d.s = down->s; d.b = down->b;
-    d.N = sh.D; d.K = sh.I; d.bits = down->bits; d.group_size = gs;
-    d.expert_stride_w = (uint64_t)sh.D * (sh.I / per); d.expert_stride_s = (uint64_t)sh.D * (sh.I / gs);
-    d.x = static_cast<const __half*>(h.ptr); d.row_map = nullptr; d.out = y16.ptr; d.out_f32 = 0;
-    d.tile_tab = tile_tab; d.n_tiles_dev = n_tiles; d.max_tiles = max_tiles; d.tile_rows = 64;
-    RMLX_TRY(launch_qmm_grouped(d, ws.ptr, s));
+    RMLX_TRY(run_expert_ffn_lds(gate, up, down, sh, xk, sorted_tok, tile_tab, n_tiles, max_tiles, A, static_cast<__half*>(y16.ptr), s, arena));
     RMLX_TRY(y.alloc((size_t)A * sh.D * 4, s, arena));
     RMLX_TRY(launch_cast_f16_to_f32(static_cast<const __half*>(y16.ptr), static_cast<float*>(y.ptr), (size_t)A * sh.D, s));
     RMLX_TRY(launch_moe_combine(static_cast<const float*>(y.ptr), inv, expert_weights_dev, T32, (uint32_t)top_k, sh.D,
