@@ -318,7 +318,8 @@ def test_gather_qmm_async_out_of_range_rows_are_zero(hip):
 
 
 @pytest.mark.parametrize("n,k,mpb,gs", [(128, 512, 9, 64), (128, 512, 12, 64), (256, 1024, 17, 64), (384, 1024, 70, 64), (256, 512, 64, 64), (128, 1536, 129, 64),
-                                        (128, 512, 40, 32), (256, 1024, 70, 128), (128, 768, 12, 64), (256, 640, 70, 64), (128, 1408, 40, 32)])
+                                        (128, 512, 40, 32), (256, 1024, 70, 128), (128, 768, 12, 64), (256, 640, 70, 64), (128, 1408, 40, 32),
+                                        (192, 320, 40, 64), (64, 2880, 17, 64), (320, 448, 130, 32)])
 def test_gather_qmm_many_rows_per_entry_on_the_grouped_gemm(hip, n, k, mpb, gs):
     """From 9 rows per batch entry on, gather_qmm multiplies with the grouped MFMA GEMM (row tiles of 16, 32 or 64 rows
     of one expert; the last tile of an entry ragged).  Against the oracle; on a stream, rows of an out-of-range index are zero."""
@@ -334,7 +335,7 @@ def test_gather_qmm_many_rows_per_entry_on_the_grouped_gemm(hip, n, k, mpb, gs):
     out = ops.gather_qmm(xd, wd, sd, bd, DeviceBuffer.from_numpy(idx), batch, mpb, n, k, E, gs).numpy()
     ref = model.gather_qmm(x, words, s, b, idx, gs)
     assert_close(out, ref, "gather_qmm (GEMM)")
-    if gs != 32 or k % 512 == 0:  # (group sizes 64 and 128 on the K-split streaming GEMV, 32 on the wave-per-tile one: whole 512s)
+    if k % 128 == 0 and (gs != 32 or k % 512 == 0):  # (group sizes 64 and 128 on the K-split streaming GEMV, 32 on the wave-per-tile one: whole 512s)
         out_stream = ops.gather_qmm(xd, wd, sd, bd, DeviceBuffer.from_numpy(idx), batch, mpb, n, k, E, gs, kernel=rt.GATHER_STREAM).numpy()
         assert_close(out_stream, ref, "gather_qmm (streaming GEMV)")
     out_port = ops.gather_qmm(xd, wd, sd, bd, DeviceBuffer.from_numpy(idx), batch, mpb, n, k, E, gs, kernel=rt.GATHER_PORTABLE).numpy()
