@@ -611,7 +611,7 @@ def test_moe_forward_of_bf16_activations(hip, bits, gs, D, I, T):
 
 
 @pytest.mark.parametrize("bits,gs,D,I,fused", [(4, 64, 320, 448, True), (4, 64, 2880, 960, True), (8, 64, 576, 320, False),
-                                               (4, 32, 448, 320, True), (4, 128, 384, 640, False)])
+                                               (4, 32, 448, 320, True), (4, 128, 384, 640, False), (4, 64, 768, 320, True), (8, 64, 512, 1088, True)])
 @pytest.mark.parametrize("T", [24, 70, 300])
 def test_moe_forward_on_the_grouped_lds_staged_gemm(hip, bits, gs, D, I, fused, T):
     """Expert dimensions in multiples of 64 that are no multiples of 128 (a hidden size of 2880): from one row per expert on
