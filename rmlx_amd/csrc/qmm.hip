@@ -158,11 +158,14 @@ __global__ __launch_bounds__(kThreads) void qmm_kernel(QmmParams p) {
   // already in MFMA operand order.  Tiles past the last one re-read the last tile (their results
   // are never stored); unconditional loads keep the number of outstanding loads known to the
   // compiler, i.e. exact s_waitcnt vmcnt counts.
+  // A wave of a grouped tile whose rows all lie past the tile's last row (its results are never stored) reads the rows of
+  // wave 0 instead of its own zeros: those lines are in the CU's cache already, so a tile of few rows fetches them once.
   const u4* aptr[TI];
   const uint32_t mt_last = (p.M + 15) / 16 - 1;
+  const uint32_t wrow = GROUPED && (uint32_t)(wave * WM) >= row_cnt ? 0u : (uint32_t)(wave * WM);
 #pragma unroll
   for (int i = 0; i < TI; ++i) {
-    const uint32_t mt = (m0 + wave * WM) / 16 + i;
+    const uint32_t mt = (m0 + wrow) / 16 + i;
     aptr[i] = reinterpret_cast<const u4*>(p.x) + (uint64_t)(mt < mt_last ? mt : mt_last) * (Kx / 32) * 64 + lane;
   }
 
