@@ -704,18 +704,18 @@ bool single_row_experts(const rmlx_qweight* gate, const rmlx_qweight* up, const 
 // as a pass of its own, down.  x: f16 rows reached through row_map (nullable); y16: f16 [positions, D] in the table's row order.
 int32_t run_expert_ffn_lds(const rmlx_qweight* gate, const rmlx_qweight* up, const rmlx_qweight* down, const ExpertShapes& sh,
                            const __half* x, const uint32_t* row_map, const uint32_t* tile_tab, const uint32_t* n_tiles,
-                           uint32_t max_tiles, uint32_t positions, __half* y16, hipStream_t s, Arena* arena) {
+                           uint32_t max_tiles, uint32_t positions, __half* y16, hipStream_t s, Arena* arena, uint32_t tile_rows = 64) {
   const uint32_t per = 32 / gate->bits, gs = gate->group_size;
   Scratch ws, gu, h;
   const uint32_t kmax = sh.D > sh.I ? sh.D : sh.I;
-  RMLX_TRY(ws.alloc(qmm_grouped_workspace_bytes(max_tiles, kmax), s, arena));
+  RMLX_TRY(ws.alloc(qmm_grouped_workspace_bytes(max_tiles, kmax, tile_rows), s, arena));
   RMLX_TRY(gu.alloc((size_t)positions * 2 * sh.I * 2, s, arena));
   RMLX_TRY(h.alloc((size_t)positions * sh.I * 2, s, arena));
   GroupedQmmArgs a{};
   a.w = gate->w; a.s = gate->s; a.b = gate->b;
   a.K = sh.D; a.bits = gate->bits; a.group_size = gs;
   a.x = x; a.row_map = row_map; a.out_f32 = 0;
-  a.tile_tab = tile_tab; a.n_tiles_dev = n_tiles; a.max_tiles = max_tiles; a.tile_rows = 64;
+  a.tile_tab = tile_tab; a.n_tiles_dev = n_tiles; a.max_tiles = max_tiles; a.tile_rows = tile_rows;
   __half* g_out = static_cast<__half*>(gu.ptr);
   if (sh.fused) {  // one stacked matrix per expert: [positions, 2I] = (gate | up)
     a.N = 2 * sh.I;
@@ -737,7 +737,7 @@ int32_t run_expert_ffn_lds(const rmlx_qweight* gate, const rmlx_qweight* up, con
   d.N = sh.D; d.K = sh.I; d.bits = down->bits; d.group_size = gs;
   d.expert_stride_w = (uint64_t)sh.D * (sh.I / per); d.expert_stride_s = (uint64_t)sh.D * (sh.I / gs);
   d.x = static_cast<const __half*>(h.ptr); d.row_map = nullptr; d.out = y16; d.out_f32 = 0;
-  d.tile_tab = tile_tab; d.n_tiles_dev = n_tiles; d.max_tiles = max_tiles; d.tile_rows = 64;
+  d.tile_tab = tile_tab; d.n_tiles_dev = n_tiles; d.max_tiles = max_tiles; d.tile_rows = tile_rows;
   return launch_qmm_grouped(d, ws.ptr, s);
 }
 
@@ -1683,20 +1683,23 @@ int32_t moe_grouped_impl(const rmlx_qweight* gate, const rmlx_qweight* up, const
     return finish(s);
   }
   if (lds_gemm) {
-    // grouping into row tiles of 64 rows of one expert, then per projection: activations to the GEMM's fragment layout (through
+    // grouping into row tiles of 64 (or 128) rows of one expert, then per projection: activations to the GEMM's fragment layout (through
     // the token map for the first), the grouped LDS-staged GEMM, SwiGLU as a pass of its own, and the weighted combine
     if (!aligned16(xk)) return fail(RMLX_INVALID_SHAPE, "MoeLayer: input must be 16-byte aligned");
-    const uint32_t max_tiles = A / 64 + (A < sh.E ? A : sh.E);
+    // (tiles of 128 rows from 64 rows per expert on: E = 32, top-4, D = I = 2880, 512 / 768 / 2048 tokens 483 / 618 / 1231 -> 470 / 491 /
+    // 1023 us; at 32 rows per expert 422 against 350 us)
+    const uint32_t tile_rows = A >= (uint64_t)64 * sh.E ? 128u : 64u;
+    const uint32_t max_tiles = A / tile_rows + (A < sh.E ? A : sh.E);
     RMLX_TRY(meta.alloc(((size_t)3 * A + 3 * (size_t)max_tiles + 4) * 4, s, arena));
     uint32_t* sorted = static_cast<uint32_t*>(meta.ptr);
     uint32_t* sorted_tok = sorted + A;
     uint32_t* inv = sorted_tok + A;
     uint32_t* tile_tab = inv + A;
     uint32_t* n_tiles = tile_tab + 3 * (size_t)max_tiles;
-    RMLX_TRY(launch_moe_sort(expert_indices_dev, A, sh.E, (uint32_t)top_k, sorted, sorted_tok, inv, nullptr, nullptr, tile_tab, n_tiles, 64, s));
+    RMLX_TRY(launch_moe_sort(expert_indices_dev, A, sh.E, (uint32_t)top_k, sorted, sorted_tok, inv, nullptr, nullptr, tile_tab, n_tiles, tile_rows, s));
     Scratch y16;
     RMLX_TRY(y16.alloc((size_t)A * sh.D * 2, s, arena));
-    RMLX_TRY(run_expert_ffn_lds(gate, up, down, sh, xk, sorted_tok, tile_tab, n_tiles, max_tiles, A, static_cast<__half*>(y16.ptr), s, arena));
+    RMLX_TRY(run_expert_ffn_lds(gate, up, down, sh, xk, sorted_tok, tile_tab, n_tiles, max_tiles, A, static_cast<__half*>(y16.ptr), s, arena, tile_rows));
     RMLX_TRY(y.alloc((size_t)A * sh.D * 4, s, arena));
     RMLX_TRY(launch_cast_f16_to_f32(static_cast<const __half*>(y16.ptr), static_cast<float*>(y.ptr), (size_t)A * sh.D, s));
     RMLX_TRY(launch_moe_combine(static_cast<const float*>(y.ptr), inv, expert_weights_dev, T32, (uint32_t)top_k, sh.D,

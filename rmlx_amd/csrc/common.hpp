@@ -281,7 +281,7 @@ struct GroupedQmmArgs {
 bool qmm_rw_grouped_supported(uint32_t N, uint32_t K, uint32_t group_size, uint32_t bits);
 int32_t launch_qmm_rw_grouped(const GroupedQmmArgs& a, hipStream_t s);
 // The LDS-staged GEMM over the same kind of table (tile_rows == 64, one weight, f16 output; shapes: qmm_supported)
-size_t qmm_grouped_workspace_bytes(uint32_t max_tiles, uint32_t K);
+size_t qmm_grouped_workspace_bytes(uint32_t max_tiles, uint32_t K, uint32_t tile_rows = 64);
 int32_t launch_qmm_grouped(const GroupedQmmArgs& a, void* workspace, hipStream_t s);
 
 // MoE helpers

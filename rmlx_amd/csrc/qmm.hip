@@ -405,13 +405,14 @@ __global__ __launch_bounds__(256) void relayout_a_kernel(const void* __restrict_
   }
 }
 
-// The same layout for the row tiles of a grouped launch: tile t (64 rows of one expert: positions first .. first + rows - 1 of
-// the table entry, through the row map where there is one; rows past the entry's repeat its last row) fills fragments
-// 4 t .. 4 t + 3 of the workspace.  f16 activations.
+// The same layout for the row tiles of a grouped launch: tile t (16 * frags rows of one expert: positions first .. first +
+// rows - 1 of the table entry, through the row map where there is one; rows past the entry's repeat its last row) fills
+// fragments frags * t .. frags * t + frags - 1 of the workspace.  f16 activations.
 __global__ __launch_bounds__(256) void relayout_grouped_kernel(const __half* __restrict__ src, const uint32_t* __restrict__ row_map,
                                                                const uint32_t* __restrict__ tile_tab, const uint32_t* __restrict__ n_tiles,
-                                                               uint32_t max_tiles, u4* __restrict__ dst, uint32_t K, uint32_t Kx) {
-  const uint32_t kchunks = Kx / 32, per_tile = 4 * kchunks * 64, nt = *n_tiles;
+                                                               uint32_t max_tiles, u4* __restrict__ dst, uint32_t K, uint32_t Kx,
+                                                               uint32_t frags) {
+  const uint32_t kchunks = Kx / 32, per_tile = frags * kchunks * 64, nt = *n_tiles;
   const uint64_t units = (uint64_t)max_tiles * per_tile;
   for (uint64_t u = (uint64_t)blockIdx.x * 256 + threadIdx.x; u < units; u += (uint64_t)gridDim.x * 256) {
     const uint32_t te = (uint32_t)(u / per_tile);
@@ -429,10 +430,15 @@ __global__ __launch_bounds__(256) void relayout_grouped_kernel(const __half* __r
 }
 
 template <int BITS, int GS>
-void launch_grouped_t(const QmmParams& p, uint32_t max_tiles, hipStream_t s) {
+void launch_grouped_t(const QmmParams& p, uint32_t max_tiles, uint32_t tile_rows, hipStream_t s) {
   const uint32_t tiles = max_tiles * (p.N / 64);
-  if (p.Kx != p.K) hipLaunchKernelGGL((qmm_kernel<64, 64, BITS, false, true, GS, true>), dim3(tiles), dim3(kThreads), 0, s, p);
-  else hipLaunchKernelGGL((qmm_kernel<64, 64, BITS, false, false, GS, true>), dim3(tiles), dim3(kThreads), 0, s, p);
+  if (tile_rows == 128) {
+    if (p.Kx != p.K) hipLaunchKernelGGL((qmm_kernel<128, 64, BITS, false, true, GS, true>), dim3(tiles), dim3(kThreads), 0, s, p);
+    else hipLaunchKernelGGL((qmm_kernel<128, 64, BITS, false, false, GS, true>), dim3(tiles), dim3(kThreads), 0, s, p);
+  } else {
+    if (p.Kx != p.K) hipLaunchKernelGGL((qmm_kernel<64, 64, BITS, false, true, GS, true>), dim3(tiles), dim3(kThreads), 0, s, p);
+    else hipLaunchKernelGGL((qmm_kernel<64, 64, BITS, false, false, GS, true>), dim3(tiles), dim3(kThreads), 0, s, p);
+  }
 }
 
 template <int BM, int BITS, bool XBF16>
@@ -463,36 +469,38 @@ bool qmm_supported(uint32_t N, uint32_t K, uint32_t group_size, uint32_t bits) {
 
 size_t qmm_workspace_bytes(uint32_t M, uint32_t K) { return (size_t)((M + 15) / 16) * 16 * padded_k(K) * 2; }
 
-size_t qmm_grouped_workspace_bytes(uint32_t max_tiles, uint32_t K) { return (size_t)max_tiles * 64 * padded_k(K) * 2; }
+size_t qmm_grouped_workspace_bytes(uint32_t max_tiles, uint32_t K, uint32_t tile_rows) {
+  return (size_t)max_tiles * tile_rows * padded_k(K) * 2;
+}
 
-// Grouped launch over row tiles of 64 rows of one expert each (see GroupedQmmArgs; one weight per launch, f16 output):
+// Grouped launch over row tiles of 64 or 128 rows of one expert each (see GroupedQmmArgs; one weight per launch, f16 output):
 // what the routed block runs on where the register-weights grouped GEMM does not take the shape (dimensions in multiples
-// of 64 that are no multiples of 128).  `workspace`: qmm_grouped_workspace_bytes(max_tiles, K) bytes.
+// of 64 that are no multiples of 128).  `workspace`: qmm_grouped_workspace_bytes(max_tiles, K, tile_rows) bytes.
 int32_t launch_qmm_grouped(const GroupedQmmArgs& a, void* workspace, hipStream_t s) {
   if (!qmm_supported(a.N, a.K, a.group_size, a.bits))
     return fail(RMLX_INVALID_SHAPE, "grouped qmm: unsupported shape N=%u K=%u bits=%u group_size=%u", a.N, a.K, a.bits, a.group_size);
   if (a.max_tiles == 0) return RMLX_OK;
-  if (a.w1 != nullptr || a.out_f32 || a.tile_rows != 64 || a.tile_tab == nullptr || a.n_tiles_dev == nullptr || workspace == nullptr)
-    return fail(RMLX_RUNTIME_ERROR, "grouped qmm (LDS-staged): one weight, f16 output, 64-row tiles, a tile table and a workspace");
+  if (a.w1 != nullptr || a.out_f32 || (a.tile_rows != 64 && a.tile_rows != 128) || a.tile_tab == nullptr || a.n_tiles_dev == nullptr || workspace == nullptr)
+    return fail(RMLX_RUNTIME_ERROR, "grouped qmm (LDS-staged): one weight, f16 output, tiles of 64 or 128 rows, a tile table and a workspace");
   if ((uint64_t)a.max_tiles * (a.N / 64) > 0x7FFFFFFFull) return fail(RMLX_INVALID_SHAPE, "grouped qmm: grid too large");
   const uint32_t Kx = padded_k(a.K);
   {
-    const uint64_t units = (uint64_t)a.max_tiles * 4 * (Kx / 32) * 64;
+    const uint64_t units = (uint64_t)a.max_tiles * (a.tile_rows / 16) * (Kx / 32) * 64;
     uint64_t blocks = (units + 255) / 256;
     if (blocks > 8192) blocks = 8192;
     hipLaunchKernelGGL(relayout_grouped_kernel, dim3((unsigned)blocks), dim3(256), 0, s, a.x, a.row_map, a.tile_tab, a.n_tiles_dev,
-                       a.max_tiles, reinterpret_cast<u4*>(workspace), a.K, Kx);
+                       a.max_tiles, reinterpret_cast<u4*>(workspace), a.K, Kx, a.tile_rows / 16);
   }
-  QmmParams p{a.w, a.s, a.b, reinterpret_cast<const uint16_t*>(workspace), static_cast<__half*>(a.out), a.max_tiles * 64, a.N, a.K, Kx,
+  QmmParams p{a.w, a.s, a.b, reinterpret_cast<const uint16_t*>(workspace), static_cast<__half*>(a.out), a.max_tiles * a.tile_rows, a.N, a.K, Kx,
               a.group_size, a.tile_tab, a.n_tiles_dev, a.expert_stride_w, a.expert_stride_s};
   if (a.bits == 4) {
-    if (a.group_size == 32) launch_grouped_t<4, 32>(p, a.max_tiles, s);
-    else if (a.group_size == 128) launch_grouped_t<4, 128>(p, a.max_tiles, s);
-    else launch_grouped_t<4, 64>(p, a.max_tiles, s);
+    if (a.group_size == 32) launch_grouped_t<4, 32>(p, a.max_tiles, a.tile_rows, s);
+    else if (a.group_size == 128) launch_grouped_t<4, 128>(p, a.max_tiles, a.tile_rows, s);
+    else launch_grouped_t<4, 64>(p, a.max_tiles, a.tile_rows, s);
   } else {
-    if (a.group_size == 32) launch_grouped_t<8, 32>(p, a.max_tiles, s);
-    else if (a.group_size == 128) launch_grouped_t<8, 128>(p, a.max_tiles, s);
-    else launch_grouped_t<8, 64>(p, a.max_tiles, s);
+    if (a.group_size == 32) launch_grouped_t<8, 32>(p, a.max_tiles, a.tile_rows, s);
+    else if (a.group_size == 128) launch_grouped_t<8, 128>(p, a.max_tiles, a.tile_rows, s);
+    else launch_grouped_t<8, 64>(p, a.max_tiles, a.tile_rows, s);
   }
   RMLX_HIP_CHECK(hipGetLastError());
   return RMLX_OK;

@@ -612,13 +612,13 @@ def test_moe_forward_of_bf16_activations(hip, bits, gs, D, I, T):
 
 @pytest.mark.parametrize("bits,gs,D,I,fused", [(4, 64, 320, 448, True), (4, 64, 2880, 960, True), (8, 64, 576, 320, False),
                                                (4, 32, 448, 320, True), (4, 128, 384, 640, False), (4, 64, 768, 320, True), (8, 64, 512, 1088, True)])
-@pytest.mark.parametrize("T", [24, 70, 300])
+@pytest.mark.parametrize("T", [24, 70, 200, 400])
 def test_moe_forward_on_the_grouped_lds_staged_gemm(hip, bits, gs, D, I, fused, T):
     """Expert dimensions in multiples of 64 that are no multiples of 128 (a hidden size of 2880): from one row per expert on
     the block groups the rows into tiles of 64 rows of one expert and multiplies them with the grouped form of the
     LDS-staged GEMM (activations re-laid through the token map, K padded to whole iterations, SwiGLU and combine as passes
     of their own).  Stacked and separate gate / up weights, every group size, experts with no rows, with one row and with
-    more than a tile; an expert index out of range gives zeros.  Against the oracle."""
+    more than a tile (tiles of 128 rows from 64 rows per expert on: T = 400); an expert index out of range gives zeros.  Against the oracle."""
     from rmlx_amd import ops
     from rmlx_amd.runtime import DeviceBuffer
     rng = np.random.default_rng(bits + gs + D + I + T)
@@ -635,7 +635,7 @@ def test_moe_forward_on_the_grouped_lds_staged_gemm(hip, bits, gs, D, I, fused, 
     x = make_x(rng, T, D)
     logits = rng.standard_normal((T, E)).astype(np.float32)
     logits[:, 5] -= 20.0          # expert 5 gets no rows
-    logits[: T // 2, 2] += 4.0    # expert 2 gets half the batch: more than one tile at T = 300
+    logits[: T // 2, 2] += 4.0    # expert 2 gets half the batch: more than one tile at T = 200 and T = 400
     idx, w, counts, _ = model.topk_route(logits, K)
     ref = model.moe_forward(x, idx, w, gate, up, down, gs, K, bits=bits)
     print(f"grouped LDS GEMM Q{bits} gs{gs} D={D} I={I} fused={fused} T={T} counts={counts.tolist()}", flush=True)
