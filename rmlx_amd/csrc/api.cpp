@@ -252,14 +252,19 @@ int32_t run_matmul_plain(const rmlx_qweight* qw, const void* x, int32_t x_dtype,
     // 8-bit: 7.4 / 11.4, 12.6 / 11.4, 19.8 / 11.7; N = 9216, 8-bit: 14.2 / 20.6, 23.0 / 20.6, 36.8 / 21.2).  Over very
     // wide matrices the wave-per-tile kernel has enough tiles to fill the chip and takes 3 to 8 rows (N = 28672, 4-bit,
     // group 32: 22.8 us against 26.9 on the single-row kernel and 25.1 on the GEMM; N = 16384: 21.4 against 17.6 on the GEMM).
-    // With only the LDS-staged GEMM as the alternative (K a multiple of 64 but not of 256, floor 10 to 23 us) the passes keep
-    // up to 16 rows, except over small matrices, where the third pass already costs more than the GEMM (4-bit, 16 rows:
-    // 4864 x 896 13.2 against 10.6 us, 6912 x 1152 16.9 against 12.3; 4096 x 2880 16.2 against 22.8, 5120 x 2880 19.0 against 22.8).
+    // With only the LDS-staged GEMM as the alternative (K a multiple of 64 but not of 128) the passes keep up to 8 rows, and
+    // up to 16 over matrices below 2 MiB; beyond, the fifth pass costs more than the GEMM (4-bit, 16 rows: 4864 x 896 13.2
+    // against 10.6 us, 6912 x 1152 16.9 against 12.3).
     // Short rows make a pass dearer still (a whole-row wave leaves lanes idle below 2048 values): group size 32, 13824 x 1152,
     // 8 / 16 rows 17.5 / 29.9 against 13.0 us, 9728 x 896 at 8 rows 13.7 against 10.8; tiny matrices keep the passes (128 x 896,
     // 16 rows: about 7 against 9.9 us).
+    // With its k loop split over more workgroups (launches of few tiles) the GEMM's floor is 11 to 14 us whatever K: from 9
+    // rows on it wins over every matrix of 2 MiB or more (16 rows: 4096 x 2880 14.9 against 11.6, 8192 x 2880 25.1 against 14.0,
+    // 8-bit 4096 x 2880 15.6 against 11.3; 8 rows: 9.9 against 11.4; but 2048 x 1088, 16 rows: 7.5 against 11.3), and from 5 rows
+    // on over 4-bit matrices of 10 MiB or more (8192 x 2880, 6 rows: 15.1 against 13.6).
     const bool passes_lose = !can_qmv && !can_qmm_rw && can_qmm_lds &&
-                             ((M > 8 && wbytes >= (1ull << 20) && wbytes < (5ull << 20)) || (M > 4 && K < 2048 && wbytes >= (3ull << 20)));
+                             ((M > 8 && wbytes >= (2ull << 20)) || (M > 4 && K < 2048 && wbytes >= (3ull << 20)) ||
+                              (M > 4 && qw->bits == 4 && wbytes >= (10ull << 20) && N <= 8192));
     const bool m1_first = can_m1 && !passes_lose && (can_qmv || !can_qmm_rw || M <= kM1PassRows);
     // One or two rows over short rows of a tall matrix: a wave of the single-row kernel owns a whole row, and a row of fewer
     // than 2048 values leaves part of its lanes without a load (896: 28 of 64), while the multi-row GEMV splits its tiles
@@ -432,9 +437,10 @@ int32_t run_matmul_plain(const rmlx_qweight* qw, const void* x, int32_t x_dtype,
     // f16 weights keep 11 significant bits.  The bf16 MFMA variant (weights rounded to 8 bits)
     // passes the tolerance with little margin, so it has to be asked for explicitly.
     Scratch ws;
-    RMLX_TRY(ws.alloc(qmm_workspace_bytes(M, K), stream));
+    RMLX_TRY(ws.alloc(qmm_workspace_bytes(M, K, N), stream));
     QmmArgs a{qw->w, qw->s, qw->b, x, x_dtype, out, M, N, K, qw->bits, ws.ptr, kernel == KERNEL_QMM_BF16 ? 1 : 0};
     a.group_size = qw->group_size;
+    a.workspace_has_partials = true;
     return launch_qmm(a, stream);
   }
 

@@ -221,7 +221,7 @@ struct QmmArgs {
   int32_t x_dtype;
   __half* out;        // [M,N]
   uint32_t M, N, K, bits;
-  void* workspace;    // qmm_workspace_bytes(M, K) bytes of device scratch (fragment-major activations)
+  void* workspace;    // qmm_workspace_bytes(M, K[, N]) bytes of device scratch (fragment-major activations[, partial sums])
   int bf16_mfma;      // 1: bf16 activations x Q8 weights on the bf16 MFMA (weights rounded to bf16)
   // fused store epilogue (register-weights GEMM; the single-row GEMV takes the same three values): 0 none, 1 out = acc + e, 2 out = silu(e) * acc
   int epi_kind;
@@ -229,11 +229,12 @@ struct QmmArgs {
   int32_t epi_dtype;
   const void* w_packed = nullptr;  // K-split GEMMs: the weights in their tile-contiguous order (gemm_layout_bytes), or null
   uint32_t group_size = 64;        // LDS-staged GEMM (the other GEMMs take it as a launch argument)
+  bool workspace_has_partials = false;  // LDS-staged GEMM: the workspace was sized with N, so a launch of few tiles may split K
 };
 enum { EPI_NONE = 0, EPI_RESIDUAL = 1, EPI_SWIGLU = 2 };
 // out[i] = out[i] + e[i]  /  silu(e[i]) * out[i], in place on f16 out (kernels without a fused epilogue)
 int32_t launch_epilogue(__half* out, int kind, const void* e, int32_t e_dtype, size_t n, hipStream_t s);
-size_t qmm_workspace_bytes(uint32_t M, uint32_t K);
+size_t qmm_workspace_bytes(uint32_t M, uint32_t K, uint32_t N = 0);
 // split-K partial sums of the register-weights GEMM (0 when the launch is not split); pass the buffer in QmmArgs::workspace
 size_t qmm_rw_workspace_bytes(uint32_t M, uint32_t N, uint32_t K, uint32_t group_size, uint32_t bits);
 // 16 x 16 fragments per workgroup (tile rows / 16 x tile columns / 16) of the tile the launcher would pick; 0 = not supported

@@ -41,6 +41,9 @@ struct QmmParams {
   // range, zeros are written) per row tile and its length on the device, expert strides in u32 words / halves
   const uint32_t* tile_tab; const uint32_t* n_tiles;
   uint64_t estride_w, estride_s;
+  // K split (SPLITK launches): workgroup (x, y) runs steps y * Kx / 64 / ksplit .. of tile x and writes f32 partial sums
+  // [ksplit, M, N]; splitk_sum_kernel adds them up
+  float* partial; uint32_t ksplit;
 };
 
 
@@ -98,7 +101,9 @@ __device__ __forceinline__ u2 dequant_q8_word_bf16(uint32_t w, float s, float b)
 // (scale, bias) of a step is fetched as single halves like in the TAIL form (group 2 * step + quarter / 2, step / 2).
 // GROUPED: row tile t of the grid takes its expert and its rows from the tile table; its activations are tile t of the
 // fragment-major workspace (relayout_grouped_kernel), so p.M is the grid's row extent, max_tiles * BM.
-template <int BM, int BN, int BITS, bool XBF16, bool TAIL, int GS, bool GROUPED = false>
+// SPLITK: few tiles (a short batch over a narrow matrix) leave most CUs idle, so the k loop is cut into p.ksplit ranges of
+// whole unrolled iterations, each of which begins before K ends (checked on the host).
+template <int BM, int BN, int BITS, bool XBF16, bool TAIL, int GS, bool GROUPED = false, bool SPLITK = false>
 __global__ __launch_bounds__(kThreads) void qmm_kernel(QmmParams p) {
   static_assert(GS == 32 || GS == 64 || GS == 128, "group sizes of the format");
   constexpr bool kHalfLoads = TAIL || GS != 64;
@@ -145,14 +150,15 @@ __global__ __launch_bounds__(kThreads) void qmm_kernel(QmmParams p) {
 
   const uint32_t K = p.K, gpr = K / GS;
   const uint32_t Kx = TAIL ? p.Kx : K;
-  const int steps = Kx / BK;          // a multiple of kDepth (checked on the host)
-  const int wlast = (int)(K / BK) - 1;  // the last step that has weights
+  const int steps = SPLITK ? (int)(Kx / BK / p.ksplit) : (int)(Kx / BK);  // a multiple of kDepth (checked on the host)
+  const int sbase = SPLITK ? (int)blockIdx.y * steps : 0;                 // the first step of this workgroup's range
+  const int wlast = (int)(K / BK) - 1 - sbase;  // the last step that has weights, counted from sbase (>= 0)
 
   // weight staging coordinates
   const int brow = tid >> 2, bq = tid & 3;  // weight row in tile, 16-value quarter of the 64-k step
-  const uint32_t* wptr = p.w + e_w + (uint64_t)(n0 + brow) * (K * BITS / 32) + bq * WPT;
-  const __half* sptr = p.s + e_s + (uint64_t)(n0 + brow) * gpr;
-  const __half* bptr = p.b + e_s + (uint64_t)(n0 + brow) * gpr;
+  const uint32_t* wptr = p.w + e_w + (uint64_t)(n0 + brow) * (K * BITS / 32) + bq * WPT + (uint32_t)sbase * (BK * BITS / 32);
+  const __half* sptr = p.s + e_s + (uint64_t)(n0 + brow) * gpr + (uint32_t)sbase * BK / GS;
+  const __half* bptr = p.b + e_s + (uint64_t)(n0 + brow) * gpr + (uint32_t)sbase * BK / GS;
 
   // activation fragments: block (16-row tile, 32-wide k chunk) = 64 lanes x 16 bytes, contiguous,
   // already in MFMA operand order.  Tiles past the last one re-read the last tile (their results
@@ -166,7 +172,8 @@ __global__ __launch_bounds__(kThreads) void qmm_kernel(QmmParams p) {
 #pragma unroll
   for (int i = 0; i < TI; ++i) {
     const uint32_t mt = (m0 + wrow) / 16 + i;
-    aptr[i] = reinterpret_cast<const u4*>(p.x) + (uint64_t)(mt < mt_last ? mt : mt_last) * (Kx / 32) * 64 + lane;
+    aptr[i] = reinterpret_cast<const u4*>(p.x) + (uint64_t)(mt < mt_last ? mt : mt_last) * (Kx / 32) * 64 + lane +
+              (uint32_t)sbase * (KK * 64);
   }
 
   // Register ring of kDepth k-steps: global loads run kDepth steps ahead of the MFMAs.  Scales
@@ -338,6 +345,8 @@ __global__ __launch_bounds__(kThreads) void qmm_kernel(QmmParams p) {
         if (GROUPED) {
           const uint32_t local = m - m0;
           if (local < row_cnt) p.out[(uint64_t)(row_lo + local) * p.N + nn] = __float2half(acc[i][j][v]);
+        } else if (SPLITK) {
+          if (m < p.M) p.partial[((uint64_t)blockIdx.y * p.M + m) * p.N + nn] = acc[i][j][v];
         } else if (m < p.M) {
           p.out[(uint64_t)m * p.N + nn] = __float2half(acc[i][j][v]);
         }
@@ -429,6 +438,20 @@ __global__ __launch_bounds__(256) void relayout_grouped_kernel(const __half* __r
   }
 }
 
+// out[m, n] = sum over the K ranges of partial[r, m, n], four columns per thread.
+__global__ __launch_bounds__(256) void splitk_sum_kernel(const float* __restrict__ partial, __half* __restrict__ out, uint64_t quads,
+                                                         uint32_t ksplit) {
+  const uint64_t q = (uint64_t)blockIdx.x * 256 + threadIdx.x;
+  if (q >= quads) return;
+  f4 a = reinterpret_cast<const f4*>(partial)[q];
+  for (uint32_t r = 1; r < ksplit; ++r) {
+    const f4 b = reinterpret_cast<const f4*>(partial)[r * quads + q];
+    a.x += b.x; a.y += b.y; a.z += b.z; a.w += b.w;
+  }
+  const h2 lo = {(_Float16)a.x, (_Float16)a.y}, hi = {(_Float16)a.z, (_Float16)a.w};
+  reinterpret_cast<u2*>(out)[q] = (u2){h2bits(lo), h2bits(hi)};
+}
+
 template <int BITS, int GS>
 void launch_grouped_t(const QmmParams& p, uint32_t max_tiles, uint32_t tile_rows, hipStream_t s) {
   const uint32_t tiles = max_tiles * (p.N / 64);
@@ -467,7 +490,30 @@ bool qmm_supported(uint32_t N, uint32_t K, uint32_t group_size, uint32_t bits) {
          K % group_size == 0 && N > 0 && K >= BK * kDepth;
 }
 
-size_t qmm_workspace_bytes(uint32_t M, uint32_t K) { return (size_t)((M + 15) / 16) * 16 * padded_k(K) * 2; }
+namespace {
+// Into how many K ranges a launch of 64-row tiles is cut, and the padded K that goes with it: few tiles (fewer than half the
+// CUs), K padded to whole unrolled iterations per range, every range at least two iterations long and begun before K ends.
+// Of the splits that qualify, the one with the shortest k loop.  ks = 1: no split.
+struct LdsPlan { uint32_t ks, Kx; };
+LdsPlan lds_plan(uint32_t M, uint32_t N, uint32_t K, bool may_split) {
+  LdsPlan best{1, padded_k(K)};
+  const uint32_t tiles = ((M + 63) / 64) * (N / 64), real = K / BK, cus = (uint32_t)ctx().num_cus;
+  if (!may_split || M > 128 || tiles * 2 > cus) return best;
+  for (uint32_t ks = 2; ks <= 4; ++ks) {
+    const uint32_t unit = ks * BK * kDepth, Kx = (K + unit - 1) / unit * unit, per = Kx / BK / ks;
+    if (per < 2 * kDepth || (ks - 1) * per >= real || tiles * ks > 2 * cus) continue;
+    if (per < best.Kx / BK / best.ks) best = LdsPlan{ks, Kx};
+  }
+  return best;
+}
+size_t relayout_bytes(uint32_t M, uint32_t Kx) { return ((size_t)((M + 15) / 16) * 16 * Kx * 2 + 255) / 256 * 256; }
+}  // namespace
+
+// The fragment-major activations; with N given (f16 multiplies), the partial sums of a K split behind them.
+size_t qmm_workspace_bytes(uint32_t M, uint32_t K, uint32_t N) {
+  const LdsPlan pl = lds_plan(M, N, K, N != 0);
+  return relayout_bytes(M, pl.Kx) + (pl.ks > 1 ? (size_t)pl.ks * M * N * 4 : 0);
+}
 
 size_t qmm_grouped_workspace_bytes(uint32_t max_tiles, uint32_t K, uint32_t tile_rows) {
   return (size_t)max_tiles * tile_rows * padded_k(K) * 2;
@@ -512,8 +558,9 @@ int32_t launch_qmm(const QmmArgs& a, hipStream_t s) {
   if (a.bf16_mfma && a.group_size != 64) return fail(RMLX_INVALID_SHAPE, "qmm: the bf16 MFMA form takes group size 64");
   if (a.M == 0) return RMLX_OK;
   if (a.workspace == nullptr) return fail(RMLX_RUNTIME_ERROR, "qmm: missing activation workspace");
-  const uint32_t Kx = padded_k(a.K);
   const bool want_bf16 = a.bf16_mfma && a.bits == 8 && a.x_dtype == RMLX_DTYPE_BF16;
+  const LdsPlan plan = lds_plan(a.M, a.N, a.K, a.workspace_has_partials && !want_bf16);
+  const uint32_t Kx = plan.Kx, ks = plan.ks;
   {
     const uint64_t units = (uint64_t)((a.M + 15) / 16) * (Kx / 32) * 64;
     uint64_t blocks = (units + 255) / 256;
@@ -522,6 +569,25 @@ int32_t launch_qmm(const QmmArgs& a, hipStream_t s) {
                        reinterpret_cast<u4*>(a.workspace), a.M, a.K, Kx, want_bf16 ? 1 : 0);
   }
   QmmParams p{a.w, a.s, a.b, reinterpret_cast<const uint16_t*>(a.workspace), a.out, a.M, a.N, a.K, Kx, a.group_size, nullptr, nullptr, 0, 0};
+  if (ks > 1) {  // few tiles: the k loop in ks ranges, f32 partial sums behind the activations, one pass that adds them up
+    p.ksplit = ks;
+    p.partial = reinterpret_cast<float*>(static_cast<char*>(a.workspace) + relayout_bytes(a.M, Kx));
+    const dim3 grid(((a.M + 63) / 64) * (a.N / 64), ks);
+    const bool tail = Kx != a.K;
+#define SPLIT_LAUNCH(BITSV, GSV)                                                                                                   \
+  if (tail) hipLaunchKernelGGL((qmm_kernel<64, 64, BITSV, false, true, GSV, false, true>), grid, dim3(kThreads), 0, s, p);         \
+  else hipLaunchKernelGGL((qmm_kernel<64, 64, BITSV, false, false, GSV, false, true>), grid, dim3(kThreads), 0, s, p);
+    if (a.bits == 4) {
+      if (a.group_size == 32) { SPLIT_LAUNCH(4, 32) } else if (a.group_size == 128) { SPLIT_LAUNCH(4, 128) } else { SPLIT_LAUNCH(4, 64) }
+    } else {
+      if (a.group_size == 32) { SPLIT_LAUNCH(8, 32) } else if (a.group_size == 128) { SPLIT_LAUNCH(8, 128) } else { SPLIT_LAUNCH(8, 64) }
+    }
+#undef SPLIT_LAUNCH
+    const uint64_t quads = (uint64_t)a.M * a.N / 4;
+    hipLaunchKernelGGL(splitk_sum_kernel, dim3((unsigned)((quads + 255) / 256)), dim3(256), 0, s, p.partial, a.out, quads, ks);
+    RMLX_HIP_CHECK(hipGetLastError());
+    return RMLX_OK;
+  }
   // 128-row tiles only when they still give (most of) the CUs a workgroup
   const uint32_t tiles128 = ((a.M + 127) / 128) * (a.N / 64);
   const bool big = a.M > 64 && tiles128 * 4 >= (uint32_t)ctx().num_cus * 3;

@@ -960,6 +960,35 @@ def test_staged_gemm_with_k_off_its_unrolled_iteration(hip, bits, dtype, n, k):
     assert_close(_run(hip, words, s2, b2, x, bits, dtype=dtype, kernel=rt.KERNEL_QMM_LDS), ref, "last group zeroed")
 
 
+@pytest.mark.parametrize("bits,gs,n,k", [(bits, gs, n, k) for bits, gs in [(4, 64), (8, 64), (4, 32), (4, 128)]
+                                          for n, k in [(128, 576), (192, 1088), (64, 2880), (256, 4160), (64, 2048), (128, 1536)]
+                                          if k % gs == 0])
+def test_staged_gemm_with_its_k_loop_split(hip, bits, gs, n, k):
+    """A launch of few tiles cuts the k loop of the LDS-staged GEMM into two, three or four ranges of whole unrolled iterations
+    (K padded up to them: 576 -> two ranges of 8 steps, the second with one step of weights; 1088 -> three of 8; 2880 -> four
+    of 12; 4160 -> four of 20; 2048 and 1536 without padding) that leave f32 partial sums, and one pass adds them up.
+    Scales and biases grow along the row, so a range that starts at the wrong group shows; the last row's last group is
+    zeroed in a second run, so a load past the row's end shows.  Against the oracle, from one row to two tiles of rows."""
+    from rmlx_amd import runtime as rt
+    rng = np.random.default_rng(bits * 13 + gs + n + k)
+    words, s, b = make_weight(rng, n, k, bits, gs)
+    ramp = (1.0 + np.arange(k // gs) % 5).astype(np.float16)
+    s = (s * ramp).astype(np.float16)
+    b = (b * ramp[::-1]).astype(np.float16)
+    for m, dtype in ((1, "f16"), (9, "f16"), (64, "bf16"), (100, "f32")):
+        x = make_x(rng, m, k, dtype)
+        ref = model.qmm(x_as_f64(x, dtype), words, s, b, gs, bits)
+        print(f"split staged GEMM Q{bits} gs={gs} {dtype} M={m} N={n} K={k}", flush=True)
+        assert_close(_run(hip, words, s, b, x, bits, gs=gs, dtype=dtype, kernel=rt.KERNEL_QMM_LDS), ref,
+                     f"Q{bits} gs={gs} {dtype} M={m} N={n} K={k}")
+    x = make_x(rng, 33, k, "f16")
+    s2, b2 = s.copy(), b.copy()
+    s2[:, -1] = 0
+    b2[:, -1] = 0
+    ref = model.qmm(x_as_f64(x, "f16"), words, s2, b2, gs, bits)
+    assert_close(_run(hip, words, s2, b2, x, bits, gs=gs, kernel=rt.KERNEL_QMM_LDS), ref, "last group zeroed")
+
+
 @pytest.mark.parametrize("bits", [4, 8])
 @pytest.mark.parametrize("gs", [32, 128])
 @pytest.mark.parametrize("n,k", [(64, 256), (128, 384), (64, 768), (192, 2944), (64, 1280)])
