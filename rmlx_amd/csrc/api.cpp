@@ -1513,16 +1513,17 @@ int32_t rmlx_hip_expert_group_grouped_forward(const rmlx_qweight* gate, const rm
     RMLX_HIP_CHECK(hipMemcpyAsync(dtab.ptr, expert_of.data(), total * 4, hipMemcpyHostToDevice, s));
     RMLX_HIP_CHECK(hipStreamSynchronize(s));  // `expert_of` is pageable host memory owned by this call
     const uint32_t* experts = static_cast<const uint32_t*>(dtab.ptr);
-    // dimensions in multiples of 64: row tiles of 64 rows of one item on the grouped form of the LDS-staged GEMM, from three rows
-    // per item on (see moe_grouped_impl)
+    // dimensions in multiples of 64: row tiles of 64 (or 128) rows of one item on the grouped form of the LDS-staged GEMM, from
+    // three rows per item on (see moe_grouped_impl)
     if (sh.gemm_lds && sh.gemm_min_rows != 0 && total >= 3 * n_items && aligned16(xk)) {
       std::vector<uint32_t> tiles;
       size_t first = 0;
+      const uint32_t tile_rows = total >= 64 * n_items ? 128u : 64u;  // (as in moe_grouped_impl)
       for (size_t i = 0; i < n_items; ++i) {
-        for (uint32_t r = 0; r < batch_sizes_host[i]; r += 64) {
+        for (uint32_t r = 0; r < batch_sizes_host[i]; r += tile_rows) {
           tiles.push_back(expert_idx_host[i]);
           tiles.push_back((uint32_t)(first + r));
-          tiles.push_back(batch_sizes_host[i] - r < 64 ? batch_sizes_host[i] - r : 64);
+          tiles.push_back(batch_sizes_host[i] - r < tile_rows ? batch_sizes_host[i] - r : tile_rows);
         }
         first += batch_sizes_host[i];
       }
@@ -1535,7 +1536,7 @@ int32_t rmlx_hip_expert_group_grouped_forward(const rmlx_qweight* gate, const rm
         RMLX_HIP_CHECK(hipStreamSynchronize(s));  // `tiles` is pageable host memory owned by this call
         const uint32_t* tt = static_cast<const uint32_t*>(ttab.ptr);
         RMLX_TRY(run_expert_ffn_lds(gate, up, down, sh, xk, nullptr, tt, tt + 3 * (size_t)n_t, n_t, rows,
-                                    static_cast<__half*>(out_f16_dev), s, nullptr));
+                                    static_cast<__half*>(out_f16_dev), s, nullptr, tile_rows));
         return finish(s);
       }
     }

@@ -910,7 +910,7 @@ def test_grouped_forward_of_single_rows(hip, E, D, I, fused, n_items):
 def test_grouped_forward_of_shapes_without_a_grouped_kernel(hip, bits, gs, D, I):
     """ExpertGroup over expert dimensions that no chunked or grouped kernel takes (off the multiples of 128, 8-bit at group
     size 32 with short rows): every row multiplies with its own expert on the single-row kernels instead of the portable ones.
-    Items of 1, 5, 17 and 40 rows, an expert named twice.  Against the float64 expert FFN."""
+    Items of 1, 5, 17 and 40 rows, an expert named twice; then items of 1, 150 and 200 rows.  Against the float64 expert FFN."""
     from rmlx_amd import ops
     from rmlx_amd.runtime import DeviceBuffer
     rng = np.random.default_rng(bits + gs + D + I)
@@ -920,13 +920,15 @@ def test_grouped_forward_of_shapes_without_a_grouped_kernel(hip, bits, gs, D, I)
     gate, up = tuple(a[:, :I] for a in gu), tuple(a[:, I:] for a in gu)
     gh, dh = ops.QuantizedWeight.from_numpy(*gu, gs, bits), ops.QuantizedWeight.from_numpy(*down, gs, bits)
     group = ops.ExpertGroup(gh, None, dh)
-    items = [(e, make_x(rng, m, D)) for e, m in ((3, 1), (0, 5), (3, 17), (4, 40))]
-    print(f"ExpertGroup without a grouped kernel Q{bits} gs{gs} D={D} I={I}", flush=True)
-    outs = group.grouped_forward([(e, DeviceBuffer.from_numpy(x)) for e, x in items])
-    for (e, x), (e2, y) in zip(items, outs):
-        assert e == e2
-        ones = np.ones((len(x), 1))
-        assert_close(y, model.moe_forward(x, np.full((len(x), 1), e), ones, gate, up, down, gs, 1, bits=bits), f"expert {e} rows {len(x)}")
+    # (the second set: 64 rows per item and more on average, where dimensions in multiples of 64 take row tiles of 128 rows)
+    for counts in (((3, 1), (0, 5), (3, 17), (4, 40)), ((3, 1), (0, 150), (4, 200))):
+        items = [(e, make_x(rng, m, D)) for e, m in counts]
+        print(f"ExpertGroup without a grouped kernel Q{bits} gs{gs} D={D} I={I} items {counts}", flush=True)
+        outs = group.grouped_forward([(e, DeviceBuffer.from_numpy(x)) for e, x in items])
+        for (e, x), (e2, y) in zip(items, outs):
+            assert e == e2
+            ones = np.ones((len(x), 1))
+            assert_close(y, model.moe_forward(x, np.full((len(x), 1), e), ones, gate, up, down, gs, 1, bits=bits), f"expert {e} rows {len(x)}")
 
 
 @pytest.fixture(scope="module")
