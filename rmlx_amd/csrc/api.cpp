@@ -1707,10 +1707,8 @@ int32_t moe_grouped_impl(const rmlx_qweight* gate, const rmlx_qweight* up, const
     Scratch y16;
     RMLX_TRY(y16.alloc((size_t)A * sh.D * 2, s, arena));
     RMLX_TRY(run_expert_ffn_lds(gate, up, down, sh, xk, sorted_tok, tile_tab, n_tiles, max_tiles, A, static_cast<__half*>(y16.ptr), s, arena, tile_rows));
-    RMLX_TRY(y.alloc((size_t)A * sh.D * 4, s, arena));
-    RMLX_TRY(launch_cast_f16_to_f32(static_cast<const __half*>(y16.ptr), static_cast<float*>(y.ptr), (size_t)A * sh.D, s));
-    RMLX_TRY(launch_moe_combine(static_cast<const float*>(y.ptr), inv, expert_weights_dev, T32, (uint32_t)top_k, sh.D,
-                                static_cast<__half*>(out_f16_dev), s));
+    RMLX_TRY(launch_moe_combine_f16(static_cast<const __half*>(y16.ptr), inv, expert_weights_dev, T32, (uint32_t)top_k, sh.D,
+                                    static_cast<__half*>(out_f16_dev), s));
     return finish(s);
   }
   // 2-bit experts: the form without grouping on the 2-bit single-row kernel with a weight matrix per row -- routing,

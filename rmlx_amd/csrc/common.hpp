@@ -316,6 +316,8 @@ int32_t launch_identity_positions(uint32_t* tok, uint32_t* inv, uint32_t n, uint
 // out[t,:] = sum_k w[t*K+k] * y[inv[t*K+k],:]  (y f32 rows at sorted positions)
 int32_t launch_moe_combine(const float* y, const uint32_t* inv, const float* weights, uint32_t T,
                            uint32_t top_k, uint32_t D, __half* out, hipStream_t s);
+int32_t launch_moe_combine_f16(const __half* y, const uint32_t* inv, const float* weights, uint32_t T, uint32_t top_k,
+                               uint32_t D, __half* out, hipStream_t s);
 // The same over f16 rows in assignment order (row t * top_k + k is pick k of token t); idx: the assignments' experts
 // (outside [0, E): skipped)
 int32_t launch_moe_combine_rows_f16(const __half* y, const uint32_t* idx, const float* weights, uint32_t T, uint32_t top_k,

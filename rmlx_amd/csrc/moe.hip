@@ -324,7 +324,15 @@ __global__ void identity_positions_kernel(uint32_t* __restrict__ tok, uint32_t* 
 // every thread owns four columns, loads its rows of all top_k experts first and sums in order.
 // Assignments whose position is not below n_rows (the grouping kernels mark an expert id outside
 // [0, E) that way) contribute nothing.
-__global__ __launch_bounds__(256) void moe_combine_kernel(const float* __restrict__ y,
+// (YT: the expert outputs as f32, or as f16 where the projection left them so)
+__device__ __forceinline__ float4 load_four(const float* p) { return *reinterpret_cast<const float4*>(p); }
+__device__ __forceinline__ float4 load_four(const __half* p) {
+  const uint2 r = *reinterpret_cast<const uint2*>(p);
+  const float2 lo = __half22float2(*reinterpret_cast<const __half2*>(&r.x)), hi = __half22float2(*reinterpret_cast<const __half2*>(&r.y));
+  return make_float4(lo.x, lo.y, hi.x, hi.y);
+}
+template <typename YT>
+__global__ __launch_bounds__(256) void moe_combine_kernel(const YT* __restrict__ y,
                                                           const uint32_t* __restrict__ inv,
                                                           const float* __restrict__ weights, uint32_t top_k,
                                                           uint32_t D, uint32_t n_rows, __half* __restrict__ out) {
@@ -341,7 +349,7 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(const float* __restric
       const uint32_t pos = inv[(size_t)t * top_k + k];
       if (pos < n_rows) {
         w[k] = weights[(size_t)t * top_k + k];
-        v[k] = *reinterpret_cast<const float4*>(y + (size_t)pos * D + c);
+        v[k] = load_four(y + (size_t)pos * D + c);
       }
     }
   }
@@ -496,7 +504,17 @@ int32_t launch_moe_combine(const float* y, const uint32_t* inv, const float* wei
                            uint32_t D, __half* out, hipStream_t s) {
   if (T == 0) return RMLX_OK;
   if (top_k > 8 || D % 4 != 0) return fail(RMLX_INVALID_SHAPE, "moe_combine: top_k <= 8 and D %% 4 == 0 required (top_k=%u D=%u)", top_k, D);
-  hipLaunchKernelGGL(moe_combine_kernel, dim3(T, (D + 1023) / 1024), dim3(256), 0, s, y, inv, weights, top_k, D, T * top_k, out);
+  hipLaunchKernelGGL(moe_combine_kernel<float>, dim3(T, (D + 1023) / 1024), dim3(256), 0, s, y, inv, weights, top_k, D, T * top_k, out);
+  RMLX_HIP_CHECK(hipGetLastError());
+  return RMLX_OK;
+}
+
+// The same over f16 expert outputs (the products are summed in f32 as above).
+int32_t launch_moe_combine_f16(const __half* y, const uint32_t* inv, const float* weights, uint32_t T, uint32_t top_k,
+                               uint32_t D, __half* out, hipStream_t s) {
+  if (T == 0) return RMLX_OK;
+  if (top_k > 8 || D % 4 != 0) return fail(RMLX_INVALID_SHAPE, "moe_combine: top_k <= 8 and D %% 4 == 0 required (top_k=%u D=%u)", top_k, D);
+  hipLaunchKernelGGL(moe_combine_kernel<__half>, dim3(T, (D + 1023) / 1024), dim3(256), 0, s, y, inv, weights, top_k, D, T * top_k, out);
   RMLX_HIP_CHECK(hipGetLastError());
   return RMLX_OK;
 }
