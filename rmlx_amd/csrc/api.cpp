@@ -1278,20 +1278,21 @@ int32_t rmlx_hip_gather_qmm_select(const rmlx_array* x, const void* w_packed_dev
              qmm_supported(N32, K32, group_size, 4) && aligned16(w) && aligned16(sc) && aligned16(bi) && aligned16(xk) &&
              (uint64_t)B32 * (((uint32_t)m_per_batch + 63) / 64) <= 65535) {
     // many rows per entry over dimensions in multiples of 64 that the register-weights grouped GEMM does not take: row tiles
-    // of 64 rows of one entry on the grouped form of the LDS-staged GEMM
-    const uint32_t per = ((uint32_t)m_per_batch + 63) / 64, n_tiles = B32 * per;
+    // of 64 rows of one entry (128 from 65 rows per entry on) on the grouped form of the LDS-staged GEMM
+    const uint32_t lds_rows = m_per_batch > 64 ? 128u : 64u;
+    const uint32_t per = ((uint32_t)m_per_batch + lds_rows - 1) / lds_rows, n_tiles = B32 * per;
     Scratch tab, ws;
     RMLX_TRY(tab.alloc((size_t)n_tiles * 12 + 4, s));
     uint32_t* t = static_cast<uint32_t*>(tab.ptr);
-    RMLX_TRY(launch_build_gather_chunks(idx, B32, (uint32_t)m_per_batch, E32, 64, t, t + 3 * (size_t)n_tiles, s));
-    RMLX_TRY(ws.alloc(qmm_grouped_workspace_bytes(n_tiles, K32), s));
+    RMLX_TRY(launch_build_gather_chunks(idx, B32, (uint32_t)m_per_batch, E32, lds_rows, t, t + 3 * (size_t)n_tiles, s));
+    RMLX_TRY(ws.alloc(qmm_grouped_workspace_bytes(n_tiles, K32, lds_rows), s));
     GroupedQmmArgs a{};
     a.w = w; a.s = sc; a.b = bi;
     a.N = N32; a.K = K32; a.bits = 4; a.group_size = group_size;
     a.expert_stride_w = (uint64_t)n * (k / 8);
     a.expert_stride_s = (uint64_t)n * gpr;
     a.x = xk; a.out = out_f16_dev;
-    a.tile_tab = t; a.n_tiles_dev = t + 3 * (size_t)n_tiles; a.max_tiles = n_tiles; a.tile_rows = 64;
+    a.tile_tab = t; a.n_tiles_dev = t + 3 * (size_t)n_tiles; a.max_tiles = n_tiles; a.tile_rows = lds_rows;
     RMLX_TRY(launch_qmm_grouped(a, ws.ptr, s));
   } else if (m_per_batch == 1 && kernel == GATHER_AUTO && qmv_m1_supported(N32, K32, group_size, 4) && aligned16(w) &&
              aligned16(sc) && aligned16(bi) && aligned16(xk)) {

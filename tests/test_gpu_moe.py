@@ -321,7 +321,7 @@ def test_gather_qmm_async_out_of_range_rows_are_zero(hip):
                                         (128, 512, 40, 32), (256, 1024, 70, 128), (128, 768, 12, 64), (256, 640, 70, 64), (128, 1408, 40, 32),
                                         (192, 320, 40, 64), (64, 2880, 17, 64), (320, 448, 130, 32)])
 def test_gather_qmm_many_rows_per_entry_on_the_grouped_gemm(hip, n, k, mpb, gs):
-    """From 9 rows per batch entry on, gather_qmm multiplies with the grouped MFMA GEMM (row tiles of 16, 32 or 64 rows
+    """From 9 rows per batch entry on, gather_qmm multiplies with the grouped MFMA GEMMs (row tiles of 16, 32, 64 or 128 rows
     of one expert; the last tile of an entry ragged).  Against the oracle; on a stream, rows of an out-of-range index are zero."""
     from rmlx_amd import ops, runtime as rt
     from rmlx_amd.runtime import DeviceBuffer, Stream
